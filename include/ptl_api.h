@@ -1,0 +1,225 @@
+/*
+ * C ABI of libptl_hip.so: the matmul-based training core of PULP-TrainLib
+ * (Conv2D / pointwise / depthwise / Linear, forward + weight-gradient +
+ * input-gradient, fp32 and IEEE fp16) running as HIP kernels on gfx950.
+ *
+ * Part 1 are the reference's own entry points: same names, same
+ * `void f(void *args)` signature, same argument structs (ptl_structs.h).
+ * Part 2 are the extensions a GPU needs and the reference has no word for:
+ * batched calls, stream/timing control, error reporting.
+ *
+ * Pointers inside the argument structs may be host or device pointers; the
+ * kind is detected per pointer.  Device pointers are used in place and the
+ * call returns after enqueueing on the library stream (ptl_sync() waits).
+ * Host pointers are staged through temporary device buffers and the call
+ * returns with the results already copied back.
+ *
+ * Semantics where the reference is not self-consistent (padding on the
+ * im2col weight/input-gradient path, pointwise input gradient with
+ * Cin != Cout, pad_tensor with pads other than 1): the textbook operation,
+ * i.e. what the reference's naive kernels compute.  matmul_type ids are
+ * accepted and validated but all select the same MFMA kernel family: every
+ * reference variant computes the same product.
+ */
+#ifndef PTL_API_H
+#define PTL_API_H
+
+#include "ptl_structs.h"
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* ------------------------------------------------------------------ */
+/* Part 1: reference entry points                                      */
+/* ------------------------------------------------------------------ */
+
+/* Conv2D, fp32: lib/sources/pulp_conv2d_fp32.c:27, :225, :240, :454 */
+void pulp_conv2d_fp32_fw_cl(void *Conv2D_args);
+void pulp_conv2d_fp32_bw_cl(void *Conv2D_args);
+void pulp_conv2d_fp32_bw_param_grads_cl(void *Conv2D_args);
+void pulp_conv2d_fp32_bw_input_grads_cl(void *Conv2D_args);
+/* Conv2D, fp16: lib/sources/pulp_conv2d_fp16.c:27, :225, :240, :454 */
+void pulp_conv2d_fp16_fw_cl(void *Conv2D_args_fp16);
+void pulp_conv2d_fp16_bw_cl(void *Conv2D_args_fp16);
+void pulp_conv2d_fp16_bw_param_grads_cl(void *Conv2D_args_fp16);
+void pulp_conv2d_fp16_bw_input_grads_cl(void *Conv2D_args_fp16);
+
+/* Pointwise conv: lib/sources/pulp_conv_pw_fp32.c:27, :106, :121, :233 */
+void pulp_conv_pw_fp32_fw_cl(void *PointWise_Conv_args);
+void pulp_conv_pw_fp32_bw_cl(void *PointWise_Conv_args);
+void pulp_conv_pw_fp32_bw_param_grads_cl(void *PointWise_Conv_args);
+void pulp_conv_pw_fp32_bw_input_grads_cl(void *PointWise_Conv_args);
+/* lib/sources/pulp_conv_pw_fp16.c:27, :108, :123, :249 */
+void pulp_conv_pw_fp16_fw_cl(void *PointWise_Conv_args_fp16);
+void pulp_conv_pw_fp16_bw_cl(void *PointWise_Conv_args_fp16);
+void pulp_conv_pw_fp16_bw_param_grads_cl(void *PointWise_Conv_args_fp16);
+void pulp_conv_pw_fp16_bw_input_grads_cl(void *PointWise_Conv_args_fp16);
+
+/* Depthwise conv: lib/sources/pulp_conv_dw_fp32.c:27, :49, :65, :77 */
+void pulp_conv_dw_fp32_fw_cl(void *DepthWise_Conv_args);
+void pulp_conv_dw_fp32_bw_cl(void *DepthWise_Conv_args);
+void pulp_conv_dw_fp32_bw_param_grads_cl(void *DepthWise_Conv_args);
+void pulp_conv_dw_fp32_bw_input_grads_cl(void *DepthWise_Conv_args);
+/* lib/sources/pulp_conv_dw_fp16.c:28, :44, :61, :75 */
+void pulp_conv_dw_fp16_fw_cl(void *DepthWise_Conv_args_fp16);
+void pulp_conv_dw_fp16_bw_cl(void *DepthWise_Conv_args_fp16);
+void pulp_conv_dw_fp16_bw_param_grads_cl(void *DepthWise_Conv_args_fp16);
+void pulp_conv_dw_fp16_bw_input_grads_cl(void *DepthWise_Conv_args_fp16);
+
+/* Linear: lib/sources/pulp_linear_fp32.c:25, :67, :85, :142 */
+void pulp_linear_fp32_fw_cl(void *Linear_args);
+void pulp_linear_fp32_bw_cl(void *Linear_args);
+void pulp_linear_fp32_bw_param_grads_cl(void *Linear_args);
+void pulp_linear_fp32_bw_input_grads_cl(void *Linear_args);
+/* lib/sources/pulp_linear_fp16.c:25, :72, :90, :149 */
+void pulp_linear_fp16_fw_cl(void *Linear_args_fp16);
+void pulp_linear_fp16_bw_cl(void *Linear_args_fp16);
+void pulp_linear_fp16_bw_param_grads_cl(void *Linear_args_fp16);
+void pulp_linear_fp16_bw_input_grads_cl(void *Linear_args_fp16);
+
+/* Matmul kernels and their dispatcher.
+ * mm / mm_M: lib/sources/pulp_matmul_fp32.c:190, :345
+ * mm_fp16 / mm_M_fp16: lib/sources/pulp_matmul_fp16.c:191, :273
+ * mm_manager: lib/sources/pulp_train_utils_fp32.c:1330 (ids 0..23)
+ * mm_manager_fp16: lib/sources/pulp_train_utils_fp16.c:1258 (ids 0..8) */
+void mm(void *matMul_args);
+void mm_M(void *matMul_args);
+void mm_fp16(void *matMul_args_fp16);
+void mm_M_fp16(void *matMul_args_fp16);
+void mm_manager(void *mm_manager_args);
+void mm_manager_fp16(void *mm_manager_args_fp16);
+
+/* Kernels forked by the layer entry points in the reference; exported so
+ * that code which forks them directly keeps linking.
+ * lib/sources/pulp_conv2d_fp32.c:669, :746; pulp_linear_fp32.c:199, :234 */
+void im2col_conv2d_fw_kernel(void *mm_manager_args);
+void im2col_conv2d_param_grad_kernel(void *mm_manager_args);
+void pulp_linear_fp32_fw_cl_kernel(void *mm_manager_args);
+void pulp_linear_fp32_bw_param_grads_cl_kernel(void *mm_manager_args);
+
+/* Direct (naive) convolution kernels on matMul_args, textbook stride/pad:
+ * lib/sources/pulp_conv_naive_fp32.c:198, :302, :410; _fp16.c twins. */
+void naive_conv2d_fw_kernel_CHW(void *matMul_args);
+void naive_conv2d_param_grad_kernel_CHW(void *matMul_args);
+void naive_conv2d_in_grad_kernel_CHW(void *matMul_args);
+void naive_conv2d_fw_kernel_CHW_fp16(void *matMul_args_fp16);
+void naive_conv2d_param_grad_kernel_CHW_fp16(void *matMul_args_fp16);
+void naive_conv2d_in_grad_kernel_CHW_fp16(void *matMul_args_fp16);
+
+/* Depthwise kernels: lib/sources/pulp_conv_naive_fp32.c:29, :113, :153;
+ * lib/sources/pulp_conv_naive_fp16.c:32, :75, :118 */
+void dw_kernel_forward(void *kernel_DW_args);
+void dw_kernel_weight_grad(void *kernel_DW_args);
+void dw_kernel_input_grad(void *kernel_DW_args);
+void dw_kernel_forward_fp16(void *kernel_DW_args_fp16);
+void dw_kernel_weight_grad_fp16(void *kernel_DW_args_fp16);
+void dw_kernel_input_grad_fp16(void *kernel_DW_args_fp16);
+
+/* Materialising patch-matrix builders and the weight block transpose
+ * (index work, bit-exact): lib/sources/pulp_im2col_fp32.c:29, :668, :1020;
+ * lib/sources/pulp_im2col_fp16.c:29, :526, :882.  The layer entry points
+ * above do not call these (their im2col is implicit); they exist for
+ * callers that use the buffers themselves. */
+void pulp_im2row_fp32(void *im2col_args);
+void pulp_im2col_fp32(void *im2col_args);
+void pulp_blocktransp_fp32(void *blocktransp_args);
+void pulp_im2row_fp16(void *im2col_args_fp16);
+void pulp_im2col_fp16(void *im2col_args_fp16);
+void pulp_blocktransp_fp16(void *blocktransp_args_fp16);
+
+/* Layout / transposition / streaming helpers:
+ * lib/sources/pulp_train_utils_fp32.c:39 (transpose_matrix), :79 (transpose),
+ * :186 (copy), :197 (set_to_value), :208 (vect_sum), :809 (cast), :821
+ * (HWC_to_CHW), :875 (CHW_to_HWC), :929 (pad_tensor); fp16 twins in
+ * lib/sources/pulp_train_utils_fp16.c:40-1000. */
+void transpose_matrix(void *transp_args);
+void transpose(void *transp_args);
+void copy(void *copy_args);
+void set_to_value(void *set_to_value_args);
+void vect_sum(void *vect_sum_args);
+void cast_fp16_tensor_to_fp32(void *cast_16t32_args);
+void HWC_to_CHW(void *layout_args);
+void CHW_to_HWC(void *layout_args);
+void pad_tensor(void *pad_args);
+void transpose_matrix_fp16(void *transp_args_fp16);
+void transpose_fp16(void *transp_args_fp16);
+void copy_fp16(void *copy_args_fp16);
+void set_to_value_fp16(void *set_to_value_args_fp16);
+void vect_sum_fp16(void *vect_sum_args_fp16);
+void cast_fp32_tensor_to_fp16(void *cast_32t16_args);
+void HWC_to_CHW_fp16(void *layout_args_fp16);
+void CHW_to_HWC_fp16(void *layout_args_fp16);
+void pad_tensor_fp16(void *pad_args_fp16);
+
+/* ------------------------------------------------------------------ */
+/* Part 2: extensions (no counterpart in the reference)                */
+/* ------------------------------------------------------------------ */
+
+/* Select the device and create the library state.  Returns 0 on success.
+ * Every other call initialises lazily on the current device if needed, and
+ * fails (non-zero, message in ptl_last_error) when no HIP device exists:
+ * there is no CPU fallback. */
+int ptl_init(int device);
+/* Message of the last failed call on this thread ("" if none). */
+const char *ptl_last_error(void);
+/* Status of the last reference-style (void) entry point on this thread:
+ * 0 = ran, 1 = rejected its arguments (message printed, outputs untouched),
+ * 2 = a HIP call failed. */
+int ptl_last_status(void);
+/* Stream on which kernels are enqueued (a hipStream_t); NULL = default. */
+void ptl_set_stream(void *hip_stream);
+int ptl_sync(void);
+/* hipEvent timing on the library stream: begin records, end records,
+ * synchronises and returns the elapsed milliseconds (negative on error). */
+int ptl_timer_begin(void);
+float ptl_timer_end_ms(void);
+
+/* Batched mode: `nsamples` independent samples stored back to back.
+ * input/output blobs describe ONE sample (C,H,W,dim); sample n of a blob
+ * lives at data + n*dim (diff + n*dim).  Forward and input-gradient
+ * results are per sample; the weight gradient written to coeff->diff is
+ * the SUM over the samples (overwriting, like the reference's single-sample
+ * call).  nsamples = 1 is exactly the reference entry point.  Return 0 on
+ * success, non-zero after rejecting the arguments or a HIP failure. */
+int ptl_conv2d_fp32_fw_batched(const struct Conv2D_args *a, int nsamples);
+int ptl_conv2d_fp32_wg_batched(const struct Conv2D_args *a, int nsamples);
+int ptl_conv2d_fp32_ig_batched(const struct Conv2D_args *a, int nsamples);
+int ptl_conv2d_fp16_fw_batched(const struct Conv2D_args_fp16 *a, int nsamples);
+int ptl_conv2d_fp16_wg_batched(const struct Conv2D_args_fp16 *a, int nsamples);
+int ptl_conv2d_fp16_ig_batched(const struct Conv2D_args_fp16 *a, int nsamples);
+
+int ptl_conv_pw_fp32_fw_batched(const struct PointWise_Conv_args *a, int nsamples);
+int ptl_conv_pw_fp32_wg_batched(const struct PointWise_Conv_args *a, int nsamples);
+int ptl_conv_pw_fp32_ig_batched(const struct PointWise_Conv_args *a, int nsamples);
+int ptl_conv_pw_fp16_fw_batched(const struct PointWise_Conv_args_fp16 *a, int nsamples);
+int ptl_conv_pw_fp16_wg_batched(const struct PointWise_Conv_args_fp16 *a, int nsamples);
+int ptl_conv_pw_fp16_ig_batched(const struct PointWise_Conv_args_fp16 *a, int nsamples);
+
+int ptl_conv_dw_fp32_fw_batched(const struct DepthWise_Conv_args *a, int nsamples);
+int ptl_conv_dw_fp32_wg_batched(const struct DepthWise_Conv_args *a, int nsamples);
+int ptl_conv_dw_fp32_ig_batched(const struct DepthWise_Conv_args *a, int nsamples);
+int ptl_conv_dw_fp16_fw_batched(const struct DepthWise_Conv_args_fp16 *a, int nsamples);
+int ptl_conv_dw_fp16_wg_batched(const struct DepthWise_Conv_args_fp16 *a, int nsamples);
+int ptl_conv_dw_fp16_ig_batched(const struct DepthWise_Conv_args_fp16 *a, int nsamples);
+
+int ptl_linear_fp32_fw_batched(const struct Linear_args *a, int nsamples);
+int ptl_linear_fp32_wg_batched(const struct Linear_args *a, int nsamples);
+int ptl_linear_fp32_ig_batched(const struct Linear_args *a, int nsamples);
+int ptl_linear_fp16_fw_batched(const struct Linear_args_fp16 *a, int nsamples);
+int ptl_linear_fp16_wg_batched(const struct Linear_args_fp16 *a, int nsamples);
+int ptl_linear_fp16_ig_batched(const struct Linear_args_fp16 *a, int nsamples);
+
+/* Plain product C[N x M] = A[N x K] * B (B is K x M, or M x K when trans_B),
+ * the contract of the reference's mm family, on raw pointers. */
+int ptl_mm_fp32(const float *A, const float *B, float *C, int N, int M, int K, int trans_B);
+int ptl_mm_fp16(const fp16 *A, const fp16 *B, fp16 *C, int N, int M, int K, int trans_B);
+
+/* Device-to-device copy kernel of `bytes` bytes (multiple of 16), used to
+ * calibrate memory-traffic counters against a known size. */
+int ptl_copy_bytes(const void *src, void *dst, long bytes);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* PTL_API_H */

@@ -1,0 +1,482 @@
+/*
+ * Argument structures of the matmul-based training core, laid out field for
+ * field like the PULP-TrainLib structures they stand in for, so that a caller
+ * compiled against the PULP-TrainLib headers can hand its structs to this
+ * library unchanged.  Every struct names the reference declaration it mirrors.
+ *
+ * Only the data layout is shared with the reference; the code behind the
+ * entry points is HIP for gfx950.
+ */
+#ifndef PTL_STRUCTS_H
+#define PTL_STRUCTS_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* IEEE binary16 storage type.  The reference picks its 16-bit format with a
+ * typedef (lib/include/pulp_train_defines.h:32: float16alt by default, float16
+ * as the documented alternative); this library implements the IEEE `float16`
+ * option, which is what the gfx950 fp16 MFMA consumes.  Host code in this
+ * library never does arithmetic on fp16 values, so a compiler without _Float16
+ * may use a same-sized integer. */
+#if defined(__FLT16_MANT_DIG__)
+typedef _Float16 fp16;
+#else
+typedef uint16_t fp16;
+#endif
+
+/* Step and layer selectors of mm_manager (lib/include/pulp_train_defines.h:51-65). */
+#define LAYER_CONV2D 0
+#define LAYER_DW_CONV 1
+#define LAYER_PW_CONV 2
+#define LAYER_LINEAR 3
+#define STEP_FW 0
+#define STEP_WGT_GRAD 1
+#define STEP_IN_GRAD 2
+
+/* Tensor + gradient handle (lib/include/pulp_train_utils_fp32.h:37-44).
+ * For a weight blob W,H are the kernel size and C the input channels. */
+struct blob {
+    float *data;
+    float *diff;
+    int dim;
+    int W;
+    int H;
+    int C;
+};
+
+/* lib/include/pulp_train_utils_fp16.h:38-45 */
+struct blob_fp16 {
+    fp16 *data;
+    fp16 *diff;
+    int dim;
+    int W;
+    int H;
+    int C;
+};
+
+/* lib/include/pulp_train_utils_fp32.h:63-77 */
+struct im2col_args {
+    struct blob *input;
+    struct blob *c;
+    struct blob *output;
+    float *pBuffer;
+    int Lpad;
+    int Rpad;
+    int Upad;
+    int Dpad;
+    int mod;
+    int stride_w;
+    int stride_h;
+    int HWC;
+    int USE_DMA;
+};
+
+/* lib/include/pulp_train_utils_fp16.h:64-78 */
+struct im2col_args_fp16 {
+    struct blob_fp16 *input;
+    struct blob_fp16 *c;
+    struct blob_fp16 *output;
+    fp16 *pBuffer;
+    int Lpad;
+    int Rpad;
+    int Upad;
+    int Dpad;
+    int mod;
+    int stride_w;
+    int stride_h;
+    int HWC;
+    int USE_DMA;
+};
+
+/* lib/include/pulp_train_utils_fp32.h:91-99 */
+struct transp_args {
+    float *in_matrix;
+    float *out_matrix;
+    int N;
+    int M;
+    int *dim;
+    int *transposed_axes;
+    int n_dim;
+};
+
+/* lib/include/pulp_train_utils_fp16.h:93-101 */
+struct transp_args_fp16 {
+    fp16 *in_matrix;
+    fp16 *out_matrix;
+    int N;
+    int M;
+    int *dim;
+    int *transposed_axes;
+    int n_dim;
+};
+
+/* lib/include/pulp_train_utils_fp32.h:109-114 */
+struct layout_args {
+    struct blob *tensor;
+    float *transp_buffer;
+    int transpose_data;
+    int transpose_grad;
+};
+
+/* lib/include/pulp_train_utils_fp16.h:133-138 */
+struct layout_args_fp16 {
+    struct blob_fp16 *tensor;
+    fp16 *transp_buffer;
+    int transpose_data;
+    int transpose_grad;
+};
+
+/* lib/include/pulp_train_utils_fp32.h:127-135 */
+struct blocktransp_args {
+    float *weights;
+    float *bt_weights;
+    int Cin;
+    int Cout;
+    int Hk;
+    int Wk;
+    int HWC;
+};
+
+/* lib/include/pulp_train_utils_fp16.h:150-158 */
+struct blocktransp_args_fp16 {
+    fp16 *weights;
+    fp16 *bt_weights;
+    int Cin;
+    int Cout;
+    int Hk;
+    int Wk;
+    int HWC;
+};
+
+/* lib/include/pulp_train_utils_fp32.h:144-148 */
+struct copy_args {
+    float *from;
+    float *to;
+    int size;
+};
+
+/* lib/include/pulp_train_utils_fp16.h:167-171 */
+struct copy_args_fp16 {
+    fp16 *from;
+    fp16 *to;
+    int size;
+};
+
+/* lib/include/pulp_train_utils_fp32.h:157-161 */
+struct set_to_value_args {
+    float *to;
+    float value;
+    int size;
+};
+
+/* lib/include/pulp_train_utils_fp16.h:180-184 */
+struct set_to_value_args_fp16 {
+    fp16 *to;
+    fp16 value;
+    int size;
+};
+
+/* lib/include/pulp_train_utils_fp32.h:171-176 */
+struct vect_sum_args {
+    float *op_1;
+    float *op_2;
+    float *dest;
+    int size;
+};
+
+/* lib/include/pulp_train_utils_fp16.h:194-199 */
+struct vect_sum_args_fp16 {
+    fp16 *op_1;
+    fp16 *op_2;
+    fp16 *dest;
+    int size;
+};
+
+/* lib/include/pulp_train_utils_fp32.h:206-210 */
+struct cast_16t32_args {
+    fp16 *source;
+    float *destination;
+    int size;
+};
+
+/* lib/include/pulp_train_utils_fp16.h:208-212 */
+struct cast_32t16_args {
+    float *source;
+    fp16 *destination;
+    int size;
+};
+
+/* lib/include/pulp_train_utils_fp32.h:226-237 (note: RPAD precedes LPAD) */
+struct pad_args {
+    float *source;
+    float *dest;
+    int C;
+    int H;
+    int W;
+    int T_RPAD;
+    int T_LPAD;
+    int T_UPAD;
+    int T_DPAD;
+    int HWC_lay;
+};
+
+/* lib/include/pulp_train_utils_fp16.h:228-239 */
+struct pad_args_fp16 {
+    fp16 *source;
+    fp16 *dest;
+    int C;
+    int H;
+    int W;
+    int T_RPAD;
+    int T_LPAD;
+    int T_UPAD;
+    int T_DPAD;
+    int HWC_lay;
+};
+
+/* GEMM descriptor C[N x M] = A[N x K] * B, with B stored K x M (trans_B = 0)
+ * or M x K (trans_B = 1)  (lib/include/pulp_train_utils_fp32.h:268-297). */
+struct matMul_args {
+    float *A;
+    float *B;
+    float *C;
+    int N;
+    int M;
+    int K;
+    int trans_B;
+
+    int H;
+    int W;
+    int pW;
+    int pH;
+    int pCin;
+    int pCout;
+    int stride_h;
+    int stride_w;
+    int Lpad;
+    int Rpad;
+    int Upad;
+    int Dpad;
+
+    float *bias;
+    int bias_dim;
+    int USE_BIASES;
+    int bias_transposed;
+    int HWC;
+};
+
+/* lib/include/pulp_train_utils_fp16.h:292-321 */
+struct matMul_args_fp16 {
+    fp16 *A;
+    fp16 *B;
+    fp16 *C;
+    int N;
+    int M;
+    int K;
+    int trans_B;
+
+    int H;
+    int W;
+    int pW;
+    int pH;
+    int pCin;
+    int pCout;
+    int stride_h;
+    int stride_w;
+    int Lpad;
+    int Rpad;
+    int Upad;
+    int Dpad;
+
+    fp16 *bias;
+    int bias_dim;
+    int USE_BIASES;
+    int bias_transposed;
+    int HWC;
+};
+
+/* lib/include/pulp_train_utils_fp32.h:338-351 */
+struct kernel_DW_args {
+    struct blob *input;
+    struct blob *weights;
+    struct blob *output;
+    int stride_h;
+    int stride_w;
+    int Lpad;
+    int Rpad;
+    int Upad;
+    int Dpad;
+};
+
+/* lib/include/pulp_train_utils_fp16.h:330-334 */
+struct kernel_DW_args_fp16 {
+    struct blob_fp16 *input;
+    struct blob_fp16 *weights;
+    struct blob_fp16 *output;
+};
+
+struct matMul_DW_args;      /* never dereferenced on this path */
+struct matMul_DW_args_fp16; /* never dereferenced on this path */
+
+/* lib/include/pulp_train_utils_fp32.h:360-366 */
+struct mm_manager_args {
+    struct matMul_args *mm_args;
+    struct matMul_DW_args *mm_dw_args;
+    int layer_type;
+    int step_type;
+    int matmul_type;
+};
+
+/* lib/include/pulp_train_utils_fp16.h:345-351 */
+struct mm_manager_args_fp16 {
+    struct matMul_args_fp16 *mm_args;
+    struct matMul_DW_args_fp16 *mm_dw_args;
+    int layer_type;
+    int step_type;
+    int matmul_type;
+};
+
+/* lib/include/pulp_conv2d_fp32.h:50-72 */
+struct Conv2D_args {
+    struct blob *input;
+    struct blob *coeff;
+    struct blob *bias;
+    struct blob *output;
+    int Lpad;
+    int Rpad;
+    int Upad;
+    int Dpad;
+    int stride_h;
+    int stride_w;
+    float *i2c_buffer;
+    float *bt_buffer;
+    int skip_wg_grad;
+    int skip_in_grad;
+    int HWC;
+    int opt_matmul_type_fw;
+    int opt_matmul_type_wg;
+    int opt_matmul_type_ig;
+    int USE_BIASES;
+    int USE_IM2COL;
+    int USE_DMA_IM2COL;
+};
+
+/* lib/include/pulp_conv2d_fp16.h:51-73 */
+struct Conv2D_args_fp16 {
+    struct blob_fp16 *input;
+    struct blob_fp16 *coeff;
+    struct blob_fp16 *bias;
+    struct blob_fp16 *output;
+    int Lpad;
+    int Rpad;
+    int Upad;
+    int Dpad;
+    int stride_h;
+    int stride_w;
+    fp16 *i2c_buffer;
+    fp16 *bt_buffer;
+    int skip_wg_grad;
+    int skip_in_grad;
+    int HWC;
+    int opt_matmul_type_fw;
+    int opt_matmul_type_wg;
+    int opt_matmul_type_ig;
+    int USE_BIASES;
+    int USE_IM2COL;
+    int USE_DMA_IM2COL;
+};
+
+/* lib/include/pulp_conv_pw_fp32.h:39-50 */
+struct PointWise_Conv_args {
+    struct blob *input;
+    struct blob *coeff;
+    struct blob *output;
+    float *transpose_buffer;
+    int skip_wg_grad;
+    int skip_in_grad;
+    int opt_matmul_type_fw;
+    int opt_matmul_type_wg;
+    int opt_matmul_type_ig;
+    int HWC;
+};
+
+/* lib/include/pulp_conv_pw_fp16.h:40-51 */
+struct PointWise_Conv_args_fp16 {
+    struct blob_fp16 *input;
+    struct blob_fp16 *coeff;
+    struct blob_fp16 *output;
+    fp16 *transpose_buffer;
+    int skip_wg_grad;
+    int skip_in_grad;
+    int opt_matmul_type_fw;
+    int opt_matmul_type_wg;
+    int opt_matmul_type_ig;
+    int HWC;
+};
+
+/* lib/include/pulp_conv_dw_fp32.h:43-60 */
+struct DepthWise_Conv_args {
+    struct blob *input;
+    struct blob *coeff;
+    struct blob *output;
+    int stride_h;
+    int stride_w;
+    int Lpad;
+    int Rpad;
+    int Upad;
+    int Dpad;
+    int skip_wg_grad;
+    int skip_in_grad;
+    int HWC;
+};
+
+/* lib/include/pulp_conv_dw_fp16.h:40-51 (no stride fields) */
+struct DepthWise_Conv_args_fp16 {
+    struct blob_fp16 *input;
+    struct blob_fp16 *coeff;
+    struct blob_fp16 *output;
+    int Lpad;
+    int Rpad;
+    int Upad;
+    int Dpad;
+    int skip_wg_grad;
+    int skip_in_grad;
+    int HWC;
+};
+
+/* lib/include/pulp_linear_fp32.h:39-50 */
+struct Linear_args {
+    struct blob *input;
+    struct blob *coeff;
+    struct blob *bias;
+    struct blob *output;
+    int skip_wg_grad;
+    int skip_in_grad;
+    int opt_matmul_type_fw;
+    int opt_matmul_type_wg;
+    int opt_matmul_type_ig;
+    int use_biases;
+};
+
+/* lib/include/pulp_linear_fp16.h:39-50 */
+struct Linear_args_fp16 {
+    struct blob_fp16 *input;
+    struct blob_fp16 *coeff;
+    struct blob_fp16 *bias;
+    struct blob_fp16 *output;
+    int skip_wg_grad;
+    int skip_in_grad;
+    int opt_matmul_type_fw;
+    int opt_matmul_type_wg;
+    int opt_matmul_type_ig;
+    int use_biases;
+};
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* PTL_STRUCTS_H */

@@ -1,0 +1,112 @@
+"""MI355X-native matmul training core behind PULP-TrainLib's C entry points.
+
+The product is libptl_hip.so (HIP kernels for gfx950 + C entry points with the
+reference's names and argument structs).  This package only loads it and
+mirrors the argument structs for Python callers; it contains no arithmetic
+and no CPU fallback: without the built library `load()` raises.
+"""
+import ctypes
+import os
+
+from . import structs
+from .structs import *  # noqa: F401,F403
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "libptl_hip.so")
+INCLUDE_DIR = os.path.join(os.path.dirname(_HERE), "include")
+
+_lib = None
+
+# Reference-named `void f(void *args)` entry points exported by the library.
+VOID_ENTRY_POINTS = [
+    "pulp_conv2d_fp32_fw_cl", "pulp_conv2d_fp32_bw_cl", "pulp_conv2d_fp32_bw_param_grads_cl",
+    "pulp_conv2d_fp32_bw_input_grads_cl", "pulp_conv2d_fp16_fw_cl", "pulp_conv2d_fp16_bw_cl",
+    "pulp_conv2d_fp16_bw_param_grads_cl", "pulp_conv2d_fp16_bw_input_grads_cl",
+    "pulp_conv_pw_fp32_fw_cl", "pulp_conv_pw_fp32_bw_cl", "pulp_conv_pw_fp32_bw_param_grads_cl",
+    "pulp_conv_pw_fp32_bw_input_grads_cl", "pulp_conv_pw_fp16_fw_cl", "pulp_conv_pw_fp16_bw_cl",
+    "pulp_conv_pw_fp16_bw_param_grads_cl", "pulp_conv_pw_fp16_bw_input_grads_cl",
+    "pulp_conv_dw_fp32_fw_cl", "pulp_conv_dw_fp32_bw_cl", "pulp_conv_dw_fp32_bw_param_grads_cl",
+    "pulp_conv_dw_fp32_bw_input_grads_cl", "pulp_conv_dw_fp16_fw_cl", "pulp_conv_dw_fp16_bw_cl",
+    "pulp_conv_dw_fp16_bw_param_grads_cl", "pulp_conv_dw_fp16_bw_input_grads_cl",
+    "pulp_linear_fp32_fw_cl", "pulp_linear_fp32_bw_cl", "pulp_linear_fp32_bw_param_grads_cl",
+    "pulp_linear_fp32_bw_input_grads_cl", "pulp_linear_fp16_fw_cl", "pulp_linear_fp16_bw_cl",
+    "pulp_linear_fp16_bw_param_grads_cl", "pulp_linear_fp16_bw_input_grads_cl",
+    "mm", "mm_M", "mm_fp16", "mm_M_fp16", "mm_manager", "mm_manager_fp16",
+    "im2col_conv2d_fw_kernel", "im2col_conv2d_param_grad_kernel", "pulp_linear_fp32_fw_cl_kernel",
+    "pulp_linear_fp32_bw_param_grads_cl_kernel",
+    "naive_conv2d_fw_kernel_CHW", "naive_conv2d_param_grad_kernel_CHW", "naive_conv2d_in_grad_kernel_CHW",
+    "naive_conv2d_fw_kernel_CHW_fp16", "naive_conv2d_param_grad_kernel_CHW_fp16",
+    "naive_conv2d_in_grad_kernel_CHW_fp16",
+    "dw_kernel_forward", "dw_kernel_weight_grad", "dw_kernel_input_grad", "dw_kernel_forward_fp16",
+    "dw_kernel_weight_grad_fp16", "dw_kernel_input_grad_fp16",
+    "pulp_im2row_fp32", "pulp_im2col_fp32", "pulp_blocktransp_fp32", "pulp_im2row_fp16", "pulp_im2col_fp16",
+    "pulp_blocktransp_fp16",
+    "transpose_matrix", "transpose", "copy", "set_to_value", "vect_sum", "cast_fp16_tensor_to_fp32", "HWC_to_CHW",
+    "CHW_to_HWC", "pad_tensor", "transpose_matrix_fp16", "transpose_fp16", "copy_fp16", "set_to_value_fp16",
+    "vect_sum_fp16", "cast_fp32_tensor_to_fp16", "HWC_to_CHW_fp16", "CHW_to_HWC_fp16", "pad_tensor_fp16",
+]
+
+# `int f(const args *, int nsamples)` batched launchers.
+BATCHED_ENTRY_POINTS = ["ptl_%s_%s_%s_batched" % (layer, dt, step)
+                        for layer in ("conv2d", "conv_pw", "conv_dw", "linear")
+                        for dt in ("fp32", "fp16") for step in ("fw", "wg", "ig")]
+
+OTHER_ENTRY_POINTS = ["ptl_init", "ptl_last_error", "ptl_last_status", "ptl_set_stream", "ptl_sync",
+                      "ptl_timer_begin", "ptl_timer_end_ms", "ptl_mm_fp32", "ptl_mm_fp16", "ptl_copy_bytes"]
+
+
+def load():
+    """Load libptl_hip.so and declare the signatures.  Raises if the library has not been built."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    if not os.path.exists(LIB_PATH):
+        raise RuntimeError("libptl_hip.so is not built (run `python pulp-trainlib_amd/build.py`); "
+                           "there is no fallback implementation")
+    lib = ctypes.CDLL(LIB_PATH)
+    for name in VOID_ENTRY_POINTS:
+        f = getattr(lib, name)
+        f.argtypes = [ctypes.c_void_p]
+        f.restype = None
+    for name in BATCHED_ENTRY_POINTS:
+        f = getattr(lib, name)
+        f.argtypes = [ctypes.c_void_p, ctypes.c_int]
+        f.restype = ctypes.c_int
+    lib.ptl_init.argtypes = [ctypes.c_int]
+    lib.ptl_init.restype = ctypes.c_int
+    lib.ptl_last_error.argtypes = []
+    lib.ptl_last_error.restype = ctypes.c_char_p
+    lib.ptl_last_status.argtypes = []
+    lib.ptl_last_status.restype = ctypes.c_int
+    lib.ptl_set_stream.argtypes = [ctypes.c_void_p]
+    lib.ptl_set_stream.restype = None
+    lib.ptl_sync.argtypes = []
+    lib.ptl_sync.restype = ctypes.c_int
+    lib.ptl_timer_begin.argtypes = []
+    lib.ptl_timer_begin.restype = ctypes.c_int
+    lib.ptl_timer_end_ms.argtypes = []
+    lib.ptl_timer_end_ms.restype = ctypes.c_float
+    for name in ("ptl_mm_fp32", "ptl_mm_fp16"):
+        f = getattr(lib, name)
+        f.argtypes = [ctypes.c_void_p] * 3 + [ctypes.c_int] * 4
+        f.restype = ctypes.c_int
+    lib.ptl_copy_bytes.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_long]
+    lib.ptl_copy_bytes.restype = ctypes.c_int
+    _lib = lib
+    return lib
+
+
+def call(name, args_struct, nsamples=None):
+    """Call an entry point on a ctypes argument struct and raise on failure.
+
+    `nsamples=None` calls the reference-named `void f(void*)` entry point `name`
+    and checks ptl_last_status(); otherwise `name` is a batched launcher.
+    """
+    lib = load()
+    if nsamples is None:
+        getattr(lib, name)(ctypes.byref(args_struct))
+        rc = lib.ptl_last_status()
+    else:
+        rc = getattr(lib, name)(ctypes.byref(args_struct), int(nsamples))
+    if rc != 0:
+        raise RuntimeError("%s failed (status %d): %s" % (name, rc, lib.ptl_last_error().decode()))

@@ -1,0 +1,52 @@
+// Host-side helpers shared by the entry-point translation units.
+#pragma once
+#include "ptl_common.hpp"
+
+#include <vector>
+
+namespace ptl {
+
+const char *last_error();
+int last_status();
+void set_status(int s);
+int init_device(int device);
+
+// Maps caller pointers to device pointers.  Device pointers pass through;
+// host pointers get a temporary device buffer that is filled before the
+// kernels run (copy_in) and copied back by finish() (copy_out).  finish()
+// synchronises only when something was staged.
+class Stager {
+   public:
+    Stager() = default;
+    ~Stager();
+    Stager(const Stager &) = delete;
+    Stager &operator=(const Stager &) = delete;
+
+    template <typename T>
+    const T *in(const T *p, size_t n) {
+        return static_cast<const T *>(map(p, n * sizeof(T), true, false));
+    }
+    template <typename T>
+    T *out(T *p, size_t n) {
+        return static_cast<T *>(map(p, n * sizeof(T), false, true));
+    }
+    template <typename T>
+    T *inout(T *p, size_t n) {
+        return static_cast<T *>(map(p, n * sizeof(T), true, true));
+    }
+    bool failed() const { return failed_; }
+    int finish(int rc);
+
+   private:
+    struct Item {
+        void *host;
+        void *dev;
+        size_t bytes;
+        bool copy_out;
+    };
+    void *map(const void *p, size_t bytes, bool copy_in, bool copy_out);
+    std::vector<Item> items_;
+    bool failed_ = false;
+};
+
+}  // namespace ptl

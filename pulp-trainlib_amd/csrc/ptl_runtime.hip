@@ -1,0 +1,204 @@
+// Library state, error reporting, workspace and host-pointer staging.
+#include "ptl_common.hpp"
+#include "ptl_host.hpp"
+
+#include <stdarg.h>
+#include <stdio.h>
+#include <string.h>
+
+namespace ptl {
+
+static thread_local char g_err[512] = "";
+static thread_local int g_status = 0;
+
+State &state() {
+    static State s;
+    return s;
+}
+
+void set_error(const char *fmt, ...) {
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(g_err, sizeof(g_err), fmt, ap);
+    va_end(ap);
+}
+
+const char *last_error() { return g_err; }
+int last_status() { return g_status; }
+void set_status(int s) { g_status = s; }
+
+bool hip_ok(hipError_t e, const char *what) {
+    if (e == hipSuccess) return true;
+    set_error("%s: %s", what, hipGetErrorString(e));
+    return false;
+}
+
+int init_device(int device) {
+    State &st = state();
+    int count = 0;
+    hipError_t e = hipGetDeviceCount(&count);
+    if (e != hipSuccess || count == 0) {
+        (void)hipGetLastError();
+        set_error("libptl_hip: no HIP device available (%s); there is no CPU fallback",
+                  e == hipSuccess ? "device count is 0" : hipGetErrorString(e));
+        return 2;
+    }
+    if (device < 0 || device >= count) {
+        set_error("libptl_hip: device %d out of range (0..%d)", device, count - 1);
+        return 1;
+    }
+    if (!hip_ok(hipSetDevice(device), "hipSetDevice")) return 2;
+    if (st.ready && st.device == device) return 0;
+    hipDeviceProp_t prop;
+    if (!hip_ok(hipGetDeviceProperties(&prop, device), "hipGetDeviceProperties")) return 2;
+    st.num_cu = prop.multiProcessorCount > 0 ? prop.multiProcessorCount : 256;
+    if (!st.ev0) {
+        if (!hip_ok(hipEventCreate(&st.ev0), "hipEventCreate")) return 2;
+        if (!hip_ok(hipEventCreate(&st.ev1), "hipEventCreate")) return 2;
+    }
+    st.device = device;
+    st.ready = true;
+    return 0;
+}
+
+bool ensure_init() {
+    State &st = state();
+    if (st.ready) return true;
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess) {
+        (void)hipGetLastError();
+        dev = 0;
+    }
+    return init_device(dev) == 0;
+}
+
+static void *grow(void *&buf, size_t &have, size_t want, const char *what) {
+    if (want <= have) return buf;
+    State &st = state();
+    if (buf) {
+        // kernels enqueued earlier may still read the old buffer
+        if (!hip_ok(hipStreamSynchronize(st.stream), "hipStreamSynchronize")) return nullptr;
+        (void)hipFree(buf);
+        buf = nullptr;
+        have = 0;
+    }
+    size_t sz = want < (size_t)(8u << 20) ? (size_t)(8u << 20) : want + want / 4;
+    if (!hip_ok(hipMalloc(&buf, sz), what)) {
+        buf = nullptr;
+        return nullptr;
+    }
+    have = sz;
+    return buf;
+}
+
+float *workspace(size_t bytes) {
+    State &st = state();
+    void *p = st.ws;
+    p = grow(p, st.ws_bytes, bytes, "hipMalloc(workspace)");
+    st.ws = static_cast<float *>(p);
+    return st.ws;
+}
+
+void *scratch(size_t bytes) {
+    State &st = state();
+    return grow(st.scratch, st.scratch_bytes, bytes, "hipMalloc(scratch)");
+}
+
+// ---------------------------------------------------------------------------
+// Staging of host pointers
+// ---------------------------------------------------------------------------
+static bool is_device_ptr(const void *p) {
+    hipPointerAttribute_t attr;
+    memset(&attr, 0, sizeof(attr));
+    hipError_t e = hipPointerGetAttributes(&attr, p);
+    if (e != hipSuccess) {
+        (void)hipGetLastError();  // plain host memory is reported as an error on some runtimes
+        return false;
+    }
+    return attr.type == hipMemoryTypeDevice || attr.type == hipMemoryTypeManaged;
+}
+
+Stager::~Stager() {
+    for (auto &t : items_)
+        if (t.dev) (void)hipFree(t.dev);
+}
+
+void *Stager::map(const void *host_or_dev, size_t bytes, bool copy_in, bool copy_out) {
+    if (failed_) return nullptr;
+    if (!host_or_dev) {
+        set_error("null tensor pointer");
+        failed_ = true;
+        return nullptr;
+    }
+    if (bytes == 0) return const_cast<void *>(host_or_dev);
+    if (is_device_ptr(host_or_dev)) return const_cast<void *>(host_or_dev);
+    for (auto &t : items_)
+        if (t.host == host_or_dev && t.bytes >= bytes) {
+            t.copy_out = t.copy_out || copy_out;
+            return t.dev;
+        }
+    Item it;
+    it.host = const_cast<void *>(host_or_dev);
+    it.bytes = bytes;
+    it.copy_out = copy_out;
+    it.dev = nullptr;
+    if (!hip_ok(hipMalloc(&it.dev, bytes), "hipMalloc(staging)")) {
+        failed_ = true;
+        return nullptr;
+    }
+    items_.push_back(it);
+    if (copy_in) {
+        if (!hip_ok(hipMemcpyAsync(it.dev, host_or_dev, bytes, hipMemcpyHostToDevice, state().stream),
+                    "hipMemcpy(H2D)")) {
+            failed_ = true;
+            return nullptr;
+        }
+    }
+    return it.dev;
+}
+
+int Stager::finish(int rc) {
+    if (items_.empty()) return failed_ ? 2 : rc;
+    State &st = state();
+    if (!failed_ && rc == 0) {
+        for (auto &t : items_)
+            if (t.copy_out) {
+                if (!hip_ok(hipMemcpyAsync(t.host, t.dev, t.bytes, hipMemcpyDeviceToHost, st.stream),
+                            "hipMemcpy(D2H)"))
+                    failed_ = true;
+            }
+    }
+    if (!hip_ok(hipStreamSynchronize(st.stream), "hipStreamSynchronize")) failed_ = true;
+    return failed_ ? 2 : rc;
+}
+
+}  // namespace ptl
+
+extern "C" {
+
+int ptl_init(int device) { return ptl::init_device(device); }
+const char *ptl_last_error(void) { return ptl::last_error(); }
+int ptl_last_status(void) { return ptl::last_status(); }
+void ptl_set_stream(void *s) { ptl::state().stream = static_cast<hipStream_t>(s); }
+
+int ptl_sync(void) {
+    if (!ptl::ensure_init()) return 2;
+    return ptl::hip_ok(hipStreamSynchronize(ptl::state().stream), "hipStreamSynchronize") ? 0 : 2;
+}
+
+int ptl_timer_begin(void) {
+    if (!ptl::ensure_init()) return 2;
+    return ptl::hip_ok(hipEventRecord(ptl::state().ev0, ptl::state().stream), "hipEventRecord") ? 0 : 2;
+}
+
+float ptl_timer_end_ms(void) {
+    if (!ptl::ensure_init()) return -1.f;
+    ptl::State &st = ptl::state();
+    if (!ptl::hip_ok(hipEventRecord(st.ev1, st.stream), "hipEventRecord")) return -1.f;
+    if (!ptl::hip_ok(hipEventSynchronize(st.ev1), "hipEventSynchronize")) return -1.f;
+    float ms = -1.f;
+    if (!ptl::hip_ok(hipEventElapsedTime(&ms, st.ev0, st.ev1), "hipEventElapsedTime")) return -1.f;
+    return ms;
+}
+
+}  // extern "C"

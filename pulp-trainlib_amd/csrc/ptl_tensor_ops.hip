@@ -1,0 +1,849 @@
+// Bandwidth-bound kernels of the training core: depthwise convolution
+// (forward, weight gradient, input gradient), the materialising patch-matrix
+// builders (im2row / im2col), weight block transpose, matrix and n-d
+// transposition, layout change, padding and the streaming helpers.  All of
+// them are index permutations or short stencils over tensors that are read
+// and written once, so they are organised for coalesced global access (64
+// consecutive lanes touch consecutive addresses on the contiguous side) and
+// measured against HBM bandwidth, not the matrix cores.
+#include "ptl_common.hpp"
+#include "ptl_host.hpp"
+#include "ptl_api.h"
+
+#include <stdio.h>
+
+namespace ptl {
+
+static inline unsigned nblocks(size_t n) { return (unsigned)((n + 255) / 256); }
+
+// ---- Depthwise convolution (CHW planes, one filter per channel) -----------------
+struct DwGeom {
+    int C, H, W, Ho, Wo, Hk, Wk;
+    int Up, Lp, sh, sw;
+};
+
+// Y[b,c,ho,wo] = sum_{hk,wk} W[c,hk,wk] * X[b,c,ho*sh-Up+hk, wo*sw-Lp+wk]
+template <typename T>
+__global__ __launch_bounds__(256) void dw_fw_kernel(const T *__restrict__ X, const T *__restrict__ Wt,
+                                                    T *__restrict__ Y, DwGeom g, size_t total) {
+    size_t idx = (size_t)blockIdx.x * 256 + threadIdx.x;
+    if (idx >= total) return;
+    int wo = (int)(idx % g.Wo);
+    size_t t = idx / g.Wo;
+    int ho = (int)(t % g.Ho);
+    size_t plane = t / g.Ho;  // b*C + c
+    int c = (int)(plane % g.C);
+    const T *xp = X + plane * g.H * g.W;
+    const T *wp = Wt + (size_t)c * g.Hk * g.Wk;
+    int h0 = ho * g.sh - g.Up, w0 = wo * g.sw - g.Lp;
+    float s = 0.f;
+    for (int hk = 0; hk < g.Hk; ++hk) {
+        int h = h0 + hk;
+        if ((unsigned)h >= (unsigned)g.H) continue;
+        for (int wk = 0; wk < g.Wk; ++wk) {
+            int w = w0 + wk;
+            if ((unsigned)w < (unsigned)g.W) s += (float)wp[hk * g.Wk + wk] * (float)xp[h * g.W + w];
+        }
+    }
+    Y[idx] = (T)s;
+}
+
+// dX[b,c,hi,wi] = sum_{hk,wk} W[c,hk,wk] * dY[b,c,ho,wo], ho*sh = hi+Up-hk, wo*sw = wi+Lp-wk
+template <typename T>
+__global__ __launch_bounds__(256) void dw_ig_kernel(const T *__restrict__ dY, const T *__restrict__ Wt,
+                                                    T *__restrict__ dX, DwGeom g, size_t total) {
+    size_t idx = (size_t)blockIdx.x * 256 + threadIdx.x;
+    if (idx >= total) return;
+    int wi = (int)(idx % g.W);
+    size_t t = idx / g.W;
+    int hi = (int)(t % g.H);
+    size_t plane = t / g.H;
+    int c = (int)(plane % g.C);
+    const T *gp = dY + plane * g.Ho * g.Wo;
+    const T *wp = Wt + (size_t)c * g.Hk * g.Wk;
+    float s = 0.f;
+    for (int hk = 0; hk < g.Hk; ++hk) {
+        int hq = hi + g.Up - hk;
+        if (hq < 0 || hq % g.sh != 0) continue;
+        int ho = hq / g.sh;
+        if (ho >= g.Ho) continue;
+        for (int wk = 0; wk < g.Wk; ++wk) {
+            int wq = wi + g.Lp - wk;
+            if (wq < 0 || wq % g.sw != 0) continue;
+            int wo = wq / g.sw;
+            if (wo < g.Wo) s += (float)wp[hk * g.Wk + wk] * (float)gp[ho * g.Wo + wo];
+        }
+    }
+    dX[idx] = (T)s;
+}
+
+// part[chunk][c][tap] = sum over this chunk's (sample, pixel) range of X * dY.
+// grid = (C, chunks); every thread keeps all taps of its channel in registers.
+template <typename T, int MAXT>
+__global__ __launch_bounds__(256) void dw_wg_kernel(const T *__restrict__ X, const T *__restrict__ dY,
+                                                    float *__restrict__ part, DwGeom g, int ns, int per_chunk) {
+    const int c = blockIdx.x;
+    const int P = g.Ho * g.Wo;
+    const size_t n = (size_t)ns * P;
+    size_t i0 = (size_t)blockIdx.y * per_chunk;
+    size_t i1 = i0 + per_chunk < n ? i0 + per_chunk : n;
+    const int taps = g.Hk * g.Wk;
+    float acc[MAXT];
+#pragma unroll
+    for (int t = 0; t < MAXT; ++t) acc[t] = 0.f;
+    for (size_t i = i0 + threadIdx.x; i < i1; i += 256) {
+        int b = (int)(i / P), p = (int)(i % P);
+        int ho = p / g.Wo, wo = p % g.Wo;
+        size_t plane = (size_t)b * g.C + c;
+        float gy = (float)dY[plane * P + p];
+        const T *xp = X + plane * g.H * g.W;
+        int h0 = ho * g.sh - g.Up, w0 = wo * g.sw - g.Lp;
+#pragma unroll
+        for (int t = 0; t < MAXT; ++t) {
+            if (t < taps) {
+                int hk = t / g.Wk, wk = t % g.Wk;
+                int h = h0 + hk, w = w0 + wk;
+                if ((unsigned)h < (unsigned)g.H && (unsigned)w < (unsigned)g.W)
+                    acc[t] += gy * (float)xp[h * g.W + w];
+            }
+        }
+    }
+    __shared__ float red[4][MAXT];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+#pragma unroll
+    for (int t = 0; t < MAXT; ++t) {
+        float v = acc[t];
+#pragma unroll
+        for (int o = 32; o > 0; o >>= 1) v += __shfl_down(v, o, 64);
+        if (lane == 0) red[wave][t] = v;
+    }
+    __syncthreads();
+    if ((int)threadIdx.x < taps) {
+        int t = threadIdx.x;
+        float v = red[0][t] + red[1][t] + red[2][t] + red[3][t];
+        part[((size_t)blockIdx.y * g.C + c) * taps + t] = v;
+    }
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void dw_wg_reduce_kernel(const float *__restrict__ part, T *__restrict__ dW,
+                                                           int n, int chunks) {
+    int i = blockIdx.x * 256 + threadIdx.x;
+    if (i >= n) return;
+    float s = 0.f;
+    for (int z = 0; z < chunks; ++z) s += part[(size_t)z * n + i];
+    dW[i] = (T)s;
+}
+
+template <typename Args>
+static int dw_geom(const Args *a, DwGeom &g, int sh, int sw, const char *fn) {
+    if (!a || !a->input || !a->coeff || !a->output) {
+        printf("[%s] null argument structure\n", fn);
+        set_error("%s: null argument structure", fn);
+        return 1;
+    }
+    g.C = a->input->C;
+    g.H = a->input->H;
+    g.W = a->input->W;
+    g.Ho = a->output->H;
+    g.Wo = a->output->W;
+    g.Hk = a->coeff->H;
+    g.Wk = a->coeff->W;
+    g.Up = a->Upad;
+    g.Lp = a->Lpad;
+    g.sh = sh;
+    g.sw = sw;
+    int nh = g.H - g.Hk + a->Upad + a->Dpad, nw = g.W - g.Wk + a->Lpad + a->Rpad;
+    if (g.C <= 0 || g.H <= 0 || g.W <= 0 || g.Hk <= 0 || g.Wk <= 0 || sh <= 0 || sw <= 0 || nh < 0 || nw < 0 ||
+        a->Upad < 0 || a->Dpad < 0 || a->Lpad < 0 || a->Rpad < 0 || a->output->C != g.C) {
+        printf("[%s] invalid tensor geometry\n", fn);
+        set_error("%s: invalid tensor geometry", fn);
+        return 1;
+    }
+    if (g.Ho != nh / sh + 1 || g.Wo != nw / sw + 1) {
+        printf("[%s] output blob is %dx%d but the geometry gives %dx%d\n", fn, g.Ho, g.Wo, nh / sh + 1,
+               nw / sw + 1);
+        set_error("%s: output blob size does not match the convolution geometry", fn);
+        return 1;
+    }
+    if (g.Hk * g.Wk > 49) {
+        printf("[%s] kernels above 49 taps are not supported\n", fn);
+        set_error("%s: kernels above 49 taps are not supported", fn);
+        return 1;
+    }
+    return 0;
+}
+
+template <typename T, typename Args>
+static int dw_step(const Args *a, int ns, int step, int sh, int sw, const char *fn) {
+    DwGeom g;
+    if (int rc = dw_geom(a, g, sh, sw, fn)) return rc;
+    if (ns <= 0) return 0;
+    if (!ensure_init()) return 2;
+    State &st = state();
+    size_t in_n = (size_t)ns * g.C * g.H * g.W, out_n = (size_t)ns * g.C * g.Ho * g.Wo;
+    size_t w_n = (size_t)g.C * g.Hk * g.Wk;
+    Stager sg;
+    int rc = 0;
+    if (step == STEP_FW) {
+        const T *X = sg.in(reinterpret_cast<const T *>(a->input->data), in_n);
+        const T *Wt = sg.in(reinterpret_cast<const T *>(a->coeff->data), w_n);
+        T *Y = sg.out(reinterpret_cast<T *>(a->output->data), out_n);
+        if (sg.failed()) return 2;
+        hipLaunchKernelGGL((dw_fw_kernel<T>), dim3(nblocks(out_n)), dim3(256), 0, st.stream, X, Wt, Y, g, out_n);
+    } else if (step == STEP_IN_GRAD) {
+        const T *dY = sg.in(reinterpret_cast<const T *>(a->output->diff), out_n);
+        const T *Wt = sg.in(reinterpret_cast<const T *>(a->coeff->data), w_n);
+        T *dX = sg.out(reinterpret_cast<T *>(a->input->diff), in_n);
+        if (sg.failed()) return 2;
+        hipLaunchKernelGGL((dw_ig_kernel<T>), dim3(nblocks(in_n)), dim3(256), 0, st.stream, dY, Wt, dX, g, in_n);
+    } else {
+        const T *X = sg.in(reinterpret_cast<const T *>(a->input->data), in_n);
+        const T *dY = sg.in(reinterpret_cast<const T *>(a->output->diff), out_n);
+        T *dW = sg.out(reinterpret_cast<T *>(a->coeff->diff), w_n);
+        if (sg.failed()) return 2;
+        size_t n = (size_t)ns * g.Ho * g.Wo;
+        // enough chunks for a few workgroups per CU, at least 1024 pixels each
+        int chunks = (int)((4 * (size_t)st.num_cu + g.C - 1) / g.C);
+        size_t maxc = (n + 1023) / 1024;
+        if ((size_t)chunks > maxc) chunks = (int)maxc;
+        if (chunks < 1) chunks = 1;
+        int per = (int)((n + chunks - 1) / chunks);
+        chunks = (int)((n + per - 1) / per);
+        float *part = workspace((size_t)chunks * w_n * sizeof(float));
+        if (!part) return sg.finish(2);
+        int taps = g.Hk * g.Wk;
+        dim3 grid(g.C, chunks);
+        if (taps <= 9)
+            hipLaunchKernelGGL((dw_wg_kernel<T, 9>), grid, dim3(256), 0, st.stream, X, dY, part, g, ns, per);
+        else if (taps <= 25)
+            hipLaunchKernelGGL((dw_wg_kernel<T, 25>), grid, dim3(256), 0, st.stream, X, dY, part, g, ns, per);
+        else
+            hipLaunchKernelGGL((dw_wg_kernel<T, 49>), grid, dim3(256), 0, st.stream, X, dY, part, g, ns, per);
+        hipLaunchKernelGGL((dw_wg_reduce_kernel<T>), dim3(nblocks(w_n)), dim3(256), 0, st.stream, part, dW,
+                           (int)w_n, chunks);
+    }
+    if (!hip_ok(hipGetLastError(), "depthwise launch")) rc = 2;
+    return sg.finish(rc);
+}
+
+// ---- Patch-matrix builders (index work) -------------------------------------------------
+struct PatchGeom {
+    int C;       // channels of the source tensor (Cin for mod 0, Cout for mod 1)
+    int Hs, Ws;  // source extent
+    int Hp, Wp;  // patch grid extent (output pixels for mod 0, input pixels for mod 1)
+    int Hk, Wk;
+    int h_mul, h_add, w_mul, w_add;  // source row = hp*h_mul + h_add + hk
+    int hwc;
+    int col_major;  // 0: buf[p*Q + q] (im2row); 1: buf[q*P + p] (im2col)
+};
+
+// buf(p, q) = src[c, hp*h_mul + h_add + hk, wp*w_mul + w_add + wk] or 0 outside,
+// p = hp*Wp + wp, q = (c,hk,wk) for CHW and (hk,wk,c) for HWC.
+template <typename T>
+__global__ __launch_bounds__(256) void patch_kernel(const T *__restrict__ src, T *__restrict__ buf, PatchGeom g,
+                                                    size_t total) {
+    size_t idx = (size_t)blockIdx.x * 256 + threadIdx.x;
+    if (idx >= total) return;
+    const int Q = g.C * g.Hk * g.Wk, P = g.Hp * g.Wp;
+    int p, q;
+    if (!g.col_major) {
+        p = (int)(idx / Q);
+        q = (int)(idx % Q);
+    } else {
+        q = (int)(idx / P);
+        p = (int)(idx % P);
+    }
+    int hp = p / g.Wp, wp = p % g.Wp;
+    int c, hk, wk;
+    if (!g.hwc) {
+        wk = q % g.Wk;
+        hk = (q / g.Wk) % g.Hk;
+        c = q / (g.Wk * g.Hk);
+    } else {
+        c = q % g.C;
+        wk = (q / g.C) % g.Wk;
+        hk = q / (g.C * g.Wk);
+    }
+    int h = hp * g.h_mul + g.h_add + hk, w = wp * g.w_mul + g.w_add + wk;
+    T v = (T)0;
+    if ((unsigned)h < (unsigned)g.Hs && (unsigned)w < (unsigned)g.Ws) {
+        size_t off = g.hwc ? (((size_t)h * g.Ws + w) * g.C + c) : (((size_t)c * g.Hs + h) * g.Ws + w);
+        v = src[off];
+    }
+    buf[idx] = v;
+}
+
+template <typename T, typename Args>
+static int patch_build(const Args *a, int col_major, const char *fn) {
+    if (!a || !a->input || !a->c || !a->output || !a->pBuffer) {
+        printf("[%s] null argument structure\n", fn);
+        set_error("%s: null argument structure", fn);
+        return 1;
+    }
+    // the reference narrows these fields to 8 bits (lib/sources/pulp_im2col_fp32.c:39-48)
+    const int Lp = (uint8_t)a->Lpad, Rp = (uint8_t)a->Rpad, Up = (uint8_t)a->Upad, Dp = (uint8_t)a->Dpad;
+    const int mod = (uint8_t)a->mod, sh = (uint8_t)a->stride_h, sw = (uint8_t)a->stride_w, hwc = (uint8_t)a->HWC;
+    const int Hin = a->input->H, Win = a->input->W, Cin = a->input->C;
+    const int Hk = a->c->H, Wk = a->c->W, Co = a->output->C;
+    if (hwc != 0 && hwc != 1) {
+        printf("[%s:] Invalid HWC parameter (not 0 or 1)\n", fn);
+        set_error("%s: HWC must be 0 or 1", fn);
+        return 1;
+    }
+    if (Hin <= 0 || Win <= 0 || Cin <= 0 || Hk <= 0 || Wk <= 0) {
+        printf("[%s] invalid tensor geometry\n", fn);
+        set_error("%s: invalid tensor geometry", fn);
+        return 1;
+    }
+    PatchGeom g = {};
+    g.Hk = Hk;
+    g.Wk = Wk;
+    g.hwc = hwc;
+    g.col_major = col_major;
+    const T *src;
+    size_t src_n;
+    if (mod == 0) {
+        if (sh == 0 || sw == 0 || Hin - Hk + Up + Dp < 0 || Win - Wk + Lp + Rp < 0) {
+            printf("[%s] invalid stride or kernel size\n", fn);
+            set_error("%s: invalid stride or kernel size", fn);
+            return 1;
+        }
+        if ((Hin - Hk + Up + Dp + sh) % sh > 0) {
+            printf("\n[%s] Invalid H stride (non multiple H sizes): have H_in=%d, H_ker=%d, U_pad=%d, D_pad=%d, "
+                   "H_stride=%d, remainder=%d",
+                   fn, Hin, Hk, Up, Dp, sh, (Hin - Hk + Up + Dp + sh) % sh);
+            set_error("%s: H stride does not divide the padded extent", fn);
+            return 1;
+        }
+        if ((Win - Wk + Lp + Rp + sw) % sw > 0) {
+            printf("\n[%s] Invalid W stride (non multiple W sizes): have W_in=%d, W_ker=%d, L_pad=%d, R_pad=%d, "
+                   "W_stride=%d, remainder=%d",
+                   fn, Win, Wk, Lp, Rp, sw, (Win - Wk + Lp + Rp + sw) % sw);
+            set_error("%s: W stride does not divide the padded extent", fn);
+            return 1;
+        }
+        g.C = Cin;
+        g.Hs = Hin;
+        g.Ws = Win;
+        g.Hp = (Hin - Hk + Up + Dp + sh) / sh;
+        g.Wp = (Win - Wk + Lp + Rp + sw) / sw;
+        g.h_mul = sh;
+        g.h_add = -Up;
+        g.w_mul = sw;
+        g.w_add = -Lp;
+        src = reinterpret_cast<const T *>(a->input->data);
+        src_n = (size_t)Cin * Hin * Win;
+    } else {
+        // output-gradient patches with full (kernel-1) padding, unit stride
+        g.C = Co;
+        g.Hs = a->output->H;
+        g.Ws = a->output->W;
+        g.Hp = Hin;
+        g.Wp = Win;
+        g.h_mul = 1;
+        g.h_add = -(Hk - 1);
+        g.w_mul = 1;
+        g.w_add = -(Wk - 1);
+        src = reinterpret_cast<const T *>(a->output->diff);
+        src_n = (size_t)Co * g.Hs * g.Ws;
+    }
+    if (!ensure_init()) return 2;
+    size_t total = (size_t)g.Hp * g.Wp * g.C * Hk * Wk;
+    Stager sg;
+    const T *dsrc = sg.in(src, src_n);
+    T *dbuf = sg.out(reinterpret_cast<T *>(a->pBuffer), total);
+    if (sg.failed()) return 2;
+    hipLaunchKernelGGL((patch_kernel<T>), dim3(nblocks(total)), dim3(256), 0, state().stream, dsrc, dbuf, g, total);
+    return sg.finish(hip_ok(hipGetLastError(), "patch launch") ? 0 : 2);
+}
+
+// bt[ci][co][i] = w[co][ci][P-1-i]                        (CHW)
+// bt[ci][hk][wk][co] = w[co][Hk-1-hk][Wk-1-wk][ci]        (HWC)
+template <typename T>
+__global__ __launch_bounds__(256) void blocktransp_kernel(const T *__restrict__ w, T *__restrict__ bt, int Ci, int Co,
+                                                          int Hk, int Wk, int hwc, int total) {
+    int idx = blockIdx.x * 256 + threadIdx.x;
+    if (idx >= total) return;
+    const int P = Hk * Wk;
+    if (!hwc) {
+        int i = idx % P, co = (idx / P) % Co, ci = idx / (P * Co);
+        bt[idx] = w[((size_t)co * Ci + ci) * P + (P - 1 - i)];
+    } else {
+        int co = idx % Co, wk = (idx / Co) % Wk, hk = (idx / (Co * Wk)) % Hk, ci = idx / (Co * P);
+        bt[idx] = w[(((size_t)co * Hk + (Hk - 1 - hk)) * Wk + (Wk - 1 - wk)) * Ci + ci];
+    }
+}
+
+template <typename T, typename Args>
+static int blocktransp(const Args *a, const char *fn) {
+    if (!a || !a->weights || !a->bt_weights) {
+        set_error("%s: null argument", fn);
+        return 1;
+    }
+    int hwc = (uint8_t)a->HWC;
+    if (hwc != 0 && hwc != 1) {
+        printf("[%s.c] Invalid data layout (not 0 or 1)!!\n", fn);
+        set_error("%s: HWC must be 0 or 1", fn);
+        return 1;
+    }
+    if (a->Cin <= 0 || a->Cout <= 0 || a->Hk <= 0 || a->Wk <= 0) {
+        set_error("%s: invalid geometry", fn);
+        return 1;
+    }
+    if (!ensure_init()) return 2;
+    size_t n = (size_t)a->Cin * a->Cout * a->Hk * a->Wk;
+    Stager sg;
+    const T *w = sg.in(reinterpret_cast<const T *>(a->weights), n);
+    T *bt = sg.out(reinterpret_cast<T *>(a->bt_weights), n);
+    if (sg.failed()) return 2;
+    hipLaunchKernelGGL((blocktransp_kernel<T>), dim3(nblocks(n)), dim3(256), 0, state().stream, w, bt, a->Cin,
+                       a->Cout, a->Hk, a->Wk, hwc, (int)n);
+    return sg.finish(hip_ok(hipGetLastError(), "blocktranspose launch") ? 0 : 2);
+}
+
+// ---- Transposition ------------------------------------------------------------------------
+
+// out[j*N + i] = in[i*M + j]; 64x64 tiles through LDS so both sides coalesce.
+template <typename T>
+__global__ __launch_bounds__(256) void transpose2d_kernel(const T *__restrict__ in, T *__restrict__ out, int N, int M) {
+    __shared__ T tile[64][65];
+    int j0 = blockIdx.x * 64, i0 = blockIdx.y * 64;
+    int tx = threadIdx.x & 63, ty = threadIdx.x >> 6;
+    for (int r = ty; r < 64; r += 4) {
+        int i = i0 + r, j = j0 + tx;
+        if (i < N && j < M) tile[r][tx] = in[(size_t)i * M + j];
+    }
+    __syncthreads();
+    for (int r = ty; r < 64; r += 4) {
+        int j = j0 + r, i = i0 + tx;
+        if (i < N && j < M) out[(size_t)j * N + i] = tile[tx][r];
+    }
+}
+
+template <typename T>
+static int transpose2d_dev(const T *in, T *out, int N, int M) {
+    dim3 grid((M + 63) / 64, (N + 63) / 64);
+    hipLaunchKernelGGL((transpose2d_kernel<T>), grid, dim3(256), 0, state().stream, in, out, N, M);
+    return hip_ok(hipGetLastError(), "transpose launch") ? 0 : 2;
+}
+
+constexpr int MAX_ND = 8;
+struct NdPerm {
+    int nd;
+    int out_dim[MAX_ND];    // extent of output axis i
+    int in_stride[MAX_ND];  // input stride of the axis that becomes output axis i
+};
+
+// numpy.transpose semantics: output axis i is input axis axes[i].
+template <typename T>
+__global__ __launch_bounds__(256) void transpose_nd_kernel(const T *__restrict__ in, T *__restrict__ out, NdPerm p,
+                                                           size_t total) {
+    size_t idx = (size_t)blockIdx.x * 256 + threadIdx.x;
+    if (idx >= total) return;
+    size_t t = idx, src = 0;
+    for (int i = p.nd - 1; i >= 0; --i) {
+        src += (t % p.out_dim[i]) * (size_t)p.in_stride[i];
+        t /= p.out_dim[i];
+    }
+    out[idx] = in[src];
+}
+
+template <typename T, typename Args>
+static int transpose_nd(const Args *a, const char *fn) {
+    if (!a || !a->in_matrix || !a->out_matrix || !a->dim || !a->transposed_axes) {
+        set_error("%s: null argument", fn);
+        return 1;
+    }
+    int nd = a->n_dim;
+    if (nd < 1 || nd > MAX_ND) {
+        printf("[%s] unsupported number of dimensions %d (1..%d)\n", fn, nd, MAX_ND);
+        set_error("%s: unsupported number of dimensions", fn);
+        return 1;
+    }
+    int stride[MAX_ND];
+    bool seen[MAX_ND] = {false};
+    size_t total = 1;
+    for (int i = nd - 1; i >= 0; --i) {
+        if (a->dim[i] <= 0) {
+            set_error("%s: non-positive extent", fn);
+            return 1;
+        }
+        stride[i] = (int)total;
+        total *= (size_t)a->dim[i];
+    }
+    NdPerm p = {};
+    p.nd = nd;
+    for (int i = 0; i < nd; ++i) {
+        int ax = a->transposed_axes[i];
+        if (ax < 0 || ax >= nd || seen[ax]) {
+            printf("[%s] transposed_axes is not a permutation\n", fn);
+            set_error("%s: transposed_axes is not a permutation", fn);
+            return 1;
+        }
+        seen[ax] = true;
+        p.out_dim[i] = a->dim[ax];
+        p.in_stride[i] = stride[ax];
+    }
+    if (!ensure_init()) return 2;
+    Stager sg;
+    const T *in = sg.in(reinterpret_cast<const T *>(a->in_matrix), total);
+    T *out = sg.out(reinterpret_cast<T *>(a->out_matrix), total);
+    if (sg.failed()) return 2;
+    int rc;
+    if (nd == 2 && a->transposed_axes[0] == 1) {
+        rc = transpose2d_dev<T>(in, out, a->dim[0], a->dim[1]);
+    } else {
+        hipLaunchKernelGGL((transpose_nd_kernel<T>), dim3(nblocks(total)), dim3(256), 0, state().stream, in, out, p,
+                           total);
+        rc = hip_ok(hipGetLastError(), "transpose launch") ? 0 : 2;
+    }
+    return sg.finish(rc);
+}
+
+template <typename T, typename Args>
+static int transpose_mat(const Args *a, const char *fn) {
+    if (!a || !a->in_matrix || !a->out_matrix) {
+        set_error("%s: null argument", fn);
+        return 1;
+    }
+    if (a->N <= 0 || a->M <= 0) return 0;
+    if (!ensure_init()) return 2;
+    size_t total = (size_t)a->N * a->M;
+    Stager sg;
+    const T *in = sg.in(reinterpret_cast<const T *>(a->in_matrix), total);
+    T *out = sg.out(reinterpret_cast<T *>(a->out_matrix), total);
+    if (sg.failed()) return 2;
+    return sg.finish(transpose2d_dev<T>(in, out, a->N, a->M));
+}
+
+// ---- Streaming helpers ---------------------------------------------------------------------
+
+template <typename T>
+__global__ __launch_bounds__(256) void copy_kernel(const T *__restrict__ a, T *__restrict__ b, size_t n) {
+    size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+    if (i < n) b[i] = a[i];
+}
+
+__global__ __launch_bounds__(256) void copy16_kernel(const uint4 *__restrict__ a, uint4 *__restrict__ b, size_t n) {
+    size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+    size_t stride = (size_t)gridDim.x * 256;
+    for (; i < n; i += stride) b[i] = a[i];
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void fill_kernel(T *__restrict__ a, T v, size_t n) {
+    size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+    if (i < n) a[i] = v;
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void add_kernel(const T *__restrict__ a, const T *__restrict__ b, T *__restrict__ c,
+                                                  size_t n) {
+    size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+    if (i < n) c[i] = a[i] + b[i];
+}
+
+template <typename S, typename D>
+__global__ __launch_bounds__(256) void cast_kernel(const S *__restrict__ a, D *__restrict__ b, size_t n) {
+    size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+    if (i < n) b[i] = (D)a[i];
+}
+
+// dest[c][ht][wt] = source[c][ht-U][wt-L] inside, 0 in the border (CHW; HWC alike)
+template <typename T>
+__global__ __launch_bounds__(256) void pad_kernel(const T *__restrict__ src, T *__restrict__ dst, int C, int H, int W,
+                                                  int L, int U, int Ho, int Wo, int hwc, size_t total) {
+    size_t idx = (size_t)blockIdx.x * 256 + threadIdx.x;
+    if (idx >= total) return;
+    int c, ht, wt;
+    if (!hwc) {
+        wt = (int)(idx % Wo);
+        ht = (int)((idx / Wo) % Ho);
+        c = (int)(idx / ((size_t)Wo * Ho));
+    } else {
+        c = (int)(idx % C);
+        wt = (int)((idx / C) % Wo);
+        ht = (int)(idx / ((size_t)C * Wo));
+    }
+    int h = ht - U, w = wt - L;
+    T v = (T)0;
+    if ((unsigned)h < (unsigned)H && (unsigned)w < (unsigned)W)
+        v = hwc ? src[((size_t)h * W + w) * C + c] : src[((size_t)c * H + h) * W + w];
+    dst[idx] = v;
+}
+
+template <typename T, typename Args>
+static int pad_step(const Args *a, const char *fn) {
+    if (!a || !a->source || !a->dest) {
+        set_error("%s: null argument", fn);
+        return 1;
+    }
+    if (a->HWC_lay != 0 && a->HWC_lay != 1) {
+        printf("[%s] HWC layout not implemented!!", fn);
+        set_error("%s: HWC_lay must be 0 or 1", fn);
+        return 1;
+    }
+    if (a->C <= 0 || a->H <= 0 || a->W <= 0 || a->T_LPAD < 0 || a->T_RPAD < 0 || a->T_UPAD < 0 || a->T_DPAD < 0) {
+        set_error("%s: invalid geometry", fn);
+        return 1;
+    }
+    if (!ensure_init()) return 2;
+    int Ho = a->H + a->T_UPAD + a->T_DPAD, Wo = a->W + a->T_LPAD + a->T_RPAD;
+    size_t total = (size_t)a->C * Ho * Wo;
+    Stager sg;
+    const T *s = sg.in(reinterpret_cast<const T *>(a->source), (size_t)a->C * a->H * a->W);
+    T *d = sg.out(reinterpret_cast<T *>(a->dest), total);
+    if (sg.failed()) return 2;
+    hipLaunchKernelGGL((pad_kernel<T>), dim3(nblocks(total)), dim3(256), 0, state().stream, s, d, a->C, a->H, a->W,
+                       a->T_LPAD, a->T_UPAD, Ho, Wo, a->HWC_lay, total);
+    return sg.finish(hip_ok(hipGetLastError(), "pad launch") ? 0 : 2);
+}
+
+// Layout change of one tensor: transpose [rows x cols] into the caller's buffer,
+// then copy the buffer back over the tensor, as the reference does
+// (lib/sources/pulp_train_utils_fp32.c:821-927).
+template <typename T>
+static int relayout_one(T *tensor, T *buffer, int rows, int cols, Stager &sg) {
+    size_t n = (size_t)rows * cols;
+    T *t = sg.inout(tensor, n);
+    T *b = sg.out(buffer, n);
+    if (sg.failed()) return 2;
+    int rc = transpose2d_dev<T>(t, b, rows, cols);
+    if (rc) return rc;
+    hipLaunchKernelGGL((copy_kernel<T>), dim3(nblocks(n)), dim3(256), 0, state().stream, b, t, n);
+    return hip_ok(hipGetLastError(), "copy launch") ? 0 : 2;
+}
+
+template <typename T, typename Args>
+static int relayout(const Args *a, bool to_hwc, const char *fn) {
+    if (!a || !a->tensor || !a->transp_buffer) {
+        set_error("%s: null argument", fn);
+        return 1;
+    }
+    // the reference narrows C/H/W to 16 bits (lib/sources/pulp_train_utils_fp32.c:825-827)
+    int C = (uint16_t)a->tensor->C, H = (uint16_t)a->tensor->H, W = (uint16_t)a->tensor->W;
+    if (C == 0 || H == 0 || W == 0) return 0;
+    if (!ensure_init()) return 2;
+    int rows = to_hwc ? C : H * W, cols = to_hwc ? H * W : C;
+    Stager sg;
+    int rc = 0;
+    if ((uint8_t)a->transpose_data == 1) {
+        if (!a->tensor->data) {
+            set_error("%s: transpose_data=1 with null data", fn);
+            return 1;
+        }
+        rc = relayout_one<T>(reinterpret_cast<T *>(a->tensor->data), reinterpret_cast<T *>(a->transp_buffer), rows,
+                             cols, sg);
+    }
+    if (rc == 0 && (uint8_t)a->transpose_grad == 1) {
+        if (!a->tensor->diff) {
+            set_error("%s: transpose_grad=1 with null diff", fn);
+            return 1;
+        }
+        rc = relayout_one<T>(reinterpret_cast<T *>(a->tensor->diff), reinterpret_cast<T *>(a->transp_buffer), rows,
+                             cols, sg);
+    }
+    return sg.finish(rc);
+}
+
+template <typename T>
+static int copy_step(const T *from, T *to, int size) {
+    if (size <= 0) return 0;
+    if (!from || !to) {
+        set_error("copy: null argument");
+        return 1;
+    }
+    if (!ensure_init()) return 2;
+    Stager sg;
+    const T *a = sg.in(from, (size_t)size);
+    T *b = sg.out(to, (size_t)size);
+    if (sg.failed()) return 2;
+    hipLaunchKernelGGL((copy_kernel<T>), dim3(nblocks(size)), dim3(256), 0, state().stream, a, b, (size_t)size);
+    return sg.finish(hip_ok(hipGetLastError(), "copy launch") ? 0 : 2);
+}
+
+template <typename T>
+static int fill_step(T *to, T value, int size) {
+    if (size <= 0) return 0;
+    if (!to) {
+        set_error("set_to_value: null argument");
+        return 1;
+    }
+    if (!ensure_init()) return 2;
+    Stager sg;
+    T *b = sg.out(to, (size_t)size);
+    if (sg.failed()) return 2;
+    hipLaunchKernelGGL((fill_kernel<T>), dim3(nblocks(size)), dim3(256), 0, state().stream, b, value, (size_t)size);
+    return sg.finish(hip_ok(hipGetLastError(), "fill launch") ? 0 : 2);
+}
+
+template <typename T>
+static int add_step(const T *x, const T *y, T *z, int size) {
+    if (size <= 0) return 0;
+    if (!x || !y || !z) {
+        set_error("vect_sum: null argument");
+        return 1;
+    }
+    if (!ensure_init()) return 2;
+    Stager sg;
+    const T *a = sg.in(x, (size_t)size);
+    const T *b = sg.in(y, (size_t)size);
+    T *c = sg.out(z, (size_t)size);
+    if (sg.failed()) return 2;
+    hipLaunchKernelGGL((add_kernel<T>), dim3(nblocks(size)), dim3(256), 0, state().stream, a, b, c, (size_t)size);
+    return sg.finish(hip_ok(hipGetLastError(), "add launch") ? 0 : 2);
+}
+
+template <typename S, typename D>
+static int cast_step(const S *x, D *y, int size) {
+    if (size <= 0) return 0;
+    if (!x || !y) {
+        set_error("cast: null argument");
+        return 1;
+    }
+    if (!ensure_init()) return 2;
+    Stager sg;
+    const S *a = sg.in(x, (size_t)size);
+    D *b = sg.out(y, (size_t)size);
+    if (sg.failed()) return 2;
+    hipLaunchKernelGGL((cast_kernel<S, D>), dim3(nblocks(size)), dim3(256), 0, state().stream, a, b, (size_t)size);
+    return sg.finish(hip_ok(hipGetLastError(), "cast launch") ? 0 : 2);
+}
+
+}  // namespace ptl
+
+// ---- C ABI ---------------------------------------------------------------------------------
+using ptl::half_t;
+using ptl::set_status;
+
+extern "C" {
+
+int ptl_conv_dw_fp32_fw_batched(const struct DepthWise_Conv_args *a, int ns) {
+    return ptl::dw_step<float>(a, ns, STEP_FW, a ? a->stride_h : 1, a ? a->stride_w : 1, "pulp_conv_dw_fp32_fw_cl");
+}
+int ptl_conv_dw_fp32_wg_batched(const struct DepthWise_Conv_args *a, int ns) {
+    return ptl::dw_step<float>(a, ns, STEP_WGT_GRAD, a ? a->stride_h : 1, a ? a->stride_w : 1,
+                               "pulp_conv_dw_fp32_bw_param_grads_cl");
+}
+int ptl_conv_dw_fp32_ig_batched(const struct DepthWise_Conv_args *a, int ns) {
+    return ptl::dw_step<float>(a, ns, STEP_IN_GRAD, a ? a->stride_h : 1, a ? a->stride_w : 1,
+                               "pulp_conv_dw_fp32_bw_input_grads_cl");
+}
+int ptl_conv_dw_fp16_fw_batched(const struct DepthWise_Conv_args_fp16 *a, int ns) {
+    return ptl::dw_step<half_t>(a, ns, STEP_FW, 1, 1, "pulp_conv_dw_fp16_fw_cl");
+}
+int ptl_conv_dw_fp16_wg_batched(const struct DepthWise_Conv_args_fp16 *a, int ns) {
+    return ptl::dw_step<half_t>(a, ns, STEP_WGT_GRAD, 1, 1, "pulp_conv_dw_fp16_bw_param_grads_cl");
+}
+int ptl_conv_dw_fp16_ig_batched(const struct DepthWise_Conv_args_fp16 *a, int ns) {
+    return ptl::dw_step<half_t>(a, ns, STEP_IN_GRAD, 1, 1, "pulp_conv_dw_fp16_bw_input_grads_cl");
+}
+
+void pulp_im2row_fp32(void *p) {
+    set_status(ptl::patch_build<float>(static_cast<const struct im2col_args *>(p), 0, "pulp_im2col_fp32"));
+}
+void pulp_im2col_fp32(void *p) {
+    set_status(ptl::patch_build<float>(static_cast<const struct im2col_args *>(p), 1, "pulp_im2col_fp32"));
+}
+void pulp_im2row_fp16(void *p) {
+    set_status(ptl::patch_build<half_t>(static_cast<const struct im2col_args_fp16 *>(p), 0, "pulp_im2col_fp16"));
+}
+void pulp_im2col_fp16(void *p) {
+    set_status(ptl::patch_build<half_t>(static_cast<const struct im2col_args_fp16 *>(p), 1, "pulp_im2col_fp16"));
+}
+void pulp_blocktransp_fp32(void *p) {
+    set_status(ptl::blocktransp<float>(static_cast<const struct blocktransp_args *>(p), "pulp_blocktransp_fp32"));
+}
+void pulp_blocktransp_fp16(void *p) {
+    set_status(
+        ptl::blocktransp<half_t>(static_cast<const struct blocktransp_args_fp16 *>(p), "pulp_blocktransp_fp16"));
+}
+
+void transpose_matrix(void *p) {
+    set_status(ptl::transpose_mat<float>(static_cast<const struct transp_args *>(p), "transpose_matrix"));
+}
+void transpose_matrix_fp16(void *p) {
+    set_status(ptl::transpose_mat<half_t>(static_cast<const struct transp_args_fp16 *>(p), "transpose_matrix_fp16"));
+}
+void transpose(void *p) {
+    set_status(ptl::transpose_nd<float>(static_cast<const struct transp_args *>(p), "transpose"));
+}
+void transpose_fp16(void *p) {
+    set_status(ptl::transpose_nd<half_t>(static_cast<const struct transp_args_fp16 *>(p), "transpose_fp16"));
+}
+
+void copy(void *p) {
+    const struct copy_args *a = static_cast<const struct copy_args *>(p);
+    set_status(a ? ptl::copy_step<float>(a->from, a->to, a->size) : 1);
+}
+void copy_fp16(void *p) {
+    const struct copy_args_fp16 *a = static_cast<const struct copy_args_fp16 *>(p);
+    set_status(a ? ptl::copy_step<half_t>(reinterpret_cast<const half_t *>(a->from),
+                                          reinterpret_cast<half_t *>(a->to), a->size)
+                 : 1);
+}
+void set_to_value(void *p) {
+    const struct set_to_value_args *a = static_cast<const struct set_to_value_args *>(p);
+    set_status(a ? ptl::fill_step<float>(a->to, a->value, a->size) : 1);
+}
+void set_to_value_fp16(void *p) {
+    const struct set_to_value_args_fp16 *a = static_cast<const struct set_to_value_args_fp16 *>(p);
+    set_status(a ? ptl::fill_step<half_t>(reinterpret_cast<half_t *>(a->to), (half_t)a->value, a->size) : 1);
+}
+void vect_sum(void *p) {
+    const struct vect_sum_args *a = static_cast<const struct vect_sum_args *>(p);
+    set_status(a ? ptl::add_step<float>(a->op_1, a->op_2, a->dest, a->size) : 1);
+}
+void vect_sum_fp16(void *p) {
+    const struct vect_sum_args_fp16 *a = static_cast<const struct vect_sum_args_fp16 *>(p);
+    set_status(a ? ptl::add_step<half_t>(reinterpret_cast<const half_t *>(a->op_1),
+                                         reinterpret_cast<const half_t *>(a->op_2),
+                                         reinterpret_cast<half_t *>(a->dest), a->size)
+                 : 1);
+}
+void cast_fp16_tensor_to_fp32(void *p) {
+    const struct cast_16t32_args *a = static_cast<const struct cast_16t32_args *>(p);
+    set_status(a ? ptl::cast_step<half_t, float>(reinterpret_cast<const half_t *>(a->source), a->destination, a->size)
+                 : 1);
+}
+void cast_fp32_tensor_to_fp16(void *p) {
+    const struct cast_32t16_args *a = static_cast<const struct cast_32t16_args *>(p);
+    set_status(a ? ptl::cast_step<float, half_t>(a->source, reinterpret_cast<half_t *>(a->destination), a->size) : 1);
+}
+void HWC_to_CHW(void *p) {
+    set_status(ptl::relayout<float>(static_cast<const struct layout_args *>(p), false, "HWC_to_CHW"));
+}
+void CHW_to_HWC(void *p) {
+    set_status(ptl::relayout<float>(static_cast<const struct layout_args *>(p), true, "CHW_to_HWC"));
+}
+void HWC_to_CHW_fp16(void *p) {
+    set_status(ptl::relayout<half_t>(static_cast<const struct layout_args_fp16 *>(p), false, "HWC_to_CHW_fp16"));
+}
+void CHW_to_HWC_fp16(void *p) {
+    set_status(ptl::relayout<half_t>(static_cast<const struct layout_args_fp16 *>(p), true, "CHW_to_HWC_fp16"));
+}
+void pad_tensor(void *p) {
+    set_status(ptl::pad_step<float>(static_cast<const struct pad_args *>(p), "pad_tensor"));
+}
+void pad_tensor_fp16(void *p) {
+    set_status(ptl::pad_step<half_t>(static_cast<const struct pad_args_fp16 *>(p), "pad_tensor_fp16"));
+}
+
+int ptl_copy_bytes(const void *src, void *dst, long bytes) {
+    if (!src || !dst || bytes < 0 || bytes % 16 != 0) {
+        ptl::set_error("ptl_copy_bytes: size must be a non-negative multiple of 16");
+        return 1;
+    }
+    if (bytes == 0) return 0;
+    if (!ptl::ensure_init()) return 2;
+    size_t n = (size_t)bytes / 16;
+    unsigned blocks = (unsigned)((n + 255) / 256);
+    unsigned cap = (unsigned)ptl::state().num_cu * 16;
+    if (blocks > cap) blocks = cap;
+    hipLaunchKernelGGL(ptl::copy16_kernel, dim3(blocks), dim3(256), 0, ptl::state().stream,
+                       static_cast<const uint4 *>(src), static_cast<uint4 *>(dst), n);
+    return ptl::hip_ok(hipGetLastError(), "copy launch") ? 0 : 2;
+}
+
+}  // extern "C"
