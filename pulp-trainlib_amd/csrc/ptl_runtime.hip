@@ -25,7 +25,10 @@ void set_error(const char *fmt, ...) {
 
 const char *last_error() { return g_err; }
 int last_status() { return g_status; }
-void set_status(int s) { g_status = s; }
+void set_status(int s) {
+    g_status = s;
+    if (s != 0) fflush(stdout);  // make the rejection message visible right away
+}
 
 bool hip_ok(hipError_t e, const char *what) {
     if (e == hipSuccess) return true;

@@ -1,0 +1,128 @@
+"""Shared test helpers: seeded inputs, argument-struct builders, error metrics."""
+import ctypes
+
+import numpy as np
+
+MASK = (1 << 64) - 1
+
+
+def splitmix64(seed, n):
+    """n 64-bit words of the SplitMix64 sequence started at `seed` (vectorised)."""
+    idx = np.arange(1, n + 1, dtype=np.uint64)
+    with np.errstate(over="ignore"):
+        z = np.uint64(seed & MASK) + idx * np.uint64(0x9E3779B97F4A7C15)
+        z = (z ^ (z >> np.uint64(30))) * np.uint64(0xBF58476D1CE4E5B9)
+        z = (z ^ (z >> np.uint64(27))) * np.uint64(0x94D049BB133111EB)
+        z = z ^ (z >> np.uint64(31))
+    return z
+
+
+def uniform(seed, shape, lo=-1.0, hi=1.0, dtype=np.float32):
+    n = int(np.prod(shape))
+    u = (splitmix64(seed, n) >> np.uint64(11)).astype(np.float64) * (1.0 / (1 << 53))
+    return (lo + (hi - lo) * u).reshape(shape).astype(dtype)
+
+
+def normal(seed, shape, sigma=1.0, dtype=np.float32):
+    n = int(np.prod(shape))
+    u1 = ((splitmix64(seed, n) >> np.uint64(11)).astype(np.float64) + 1.0) * (1.0 / ((1 << 53) + 1))
+    u2 = (splitmix64(seed ^ 0xABCDEF, n) >> np.uint64(11)).astype(np.float64) * (1.0 / (1 << 53))
+    z = np.sqrt(-2.0 * np.log(u1)) * np.cos(2.0 * np.pi * u2)
+    return (sigma * z).reshape(shape).astype(dtype)
+
+
+def rel_l2(got, ref):
+    got = np.asarray(got, dtype=np.float64)
+    ref = np.asarray(ref, dtype=np.float64)
+    den = np.linalg.norm(ref)
+    return float(np.linalg.norm(got - ref) / (den if den > 0 else 1.0))
+
+
+def np_dtype(dt):
+    return np.float32 if dt == "fp32" else np.float16
+
+
+def ptr(b):
+    return ctypes.pointer(b)
+
+
+class Keep(list):
+    """Holds the objects an argument struct points to."""
+
+
+def conv2d_args(pkg, x, dx, w, dw, y, dy, Ci, H, W, Co, Hk, Wk, Ho, Wo, pad=(0, 0, 0, 0), stride=(1, 1), hwc=0,
+                im2col=1, bias=None, dbias=None, i2c=None, bt=None):
+    """Conv2D_args over the given tensors; pad = (L, R, U, D), stride = (h, w)."""
+    keep = Keep()
+    bi = pkg.blob(x, dx, Ci, H, W)
+    bw = pkg.blob(w, dw, Ci, Hk, Wk, dim=Co * Ci * Hk * Wk)
+    bo = pkg.blob(y, dy, Co, Ho, Wo)
+    bb = pkg.blob(bias, dbias, 1, 1, Co)
+    keep += [bi, bw, bo, bb, x, dx, w, dw, y, dy, bias, dbias, i2c, bt]
+    a = pkg.Conv2DArgs()
+    a.input, a.coeff, a.output = ptr(bi), ptr(bw), ptr(bo)
+    if bias is not None or dbias is not None:
+        a.bias = ptr(bb)
+        a.USE_BIASES = 1
+    a.Lpad, a.Rpad, a.Upad, a.Dpad = pad
+    a.stride_h, a.stride_w = stride
+    a.i2c_buffer = pkg.addr(i2c)
+    a.bt_buffer = pkg.addr(bt)
+    a.HWC = hwc
+    a.USE_IM2COL = im2col
+    return a, keep
+
+
+def pw_args(pkg, x, dx, w, dw, y, dy, Ci, Co, H, W, hwc=0):
+    keep = Keep()
+    bi = pkg.blob(x, dx, Ci, H, W)
+    bw = pkg.blob(w, dw, Ci, 1, 1, dim=Co * Ci)
+    bo = pkg.blob(y, dy, Co, H, W)
+    keep += [bi, bw, bo, x, dx, w, dw, y, dy]
+    a = pkg.PointWiseConvArgs()
+    a.input, a.coeff, a.output = ptr(bi), ptr(bw), ptr(bo)
+    a.HWC = hwc
+    return a, keep
+
+
+def dw_args(pkg, dt, x, dx, w, dw, y, dy, C, H, W, Hk, Wk, Ho, Wo, pad=(0, 0, 0, 0), stride=(1, 1)):
+    keep = Keep()
+    bi = pkg.blob(x, dx, C, H, W)
+    bw = pkg.blob(w, dw, 1, Hk, Wk, dim=C * Hk * Wk)
+    bo = pkg.blob(y, dy, C, Ho, Wo)
+    keep += [bi, bw, bo, x, dx, w, dw, y, dy]
+    if dt == "fp32":
+        a = pkg.DepthWiseConvArgs()
+        a.stride_h, a.stride_w = stride
+    else:
+        assert tuple(stride) == (1, 1)
+        a = pkg.DepthWiseConvArgsFp16()
+    a.input, a.coeff, a.output = ptr(bi), ptr(bw), ptr(bo)
+    a.Lpad, a.Rpad, a.Upad, a.Dpad = pad
+    return a, keep
+
+
+def linear_args(pkg, x, dx, w, dw, y, dy, n_in, n_out, bias=None, dbias=None):
+    keep = Keep()
+    bi = pkg.blob(x, dx, 1, 1, n_in, dim=n_in)
+    bw = pkg.blob(w, dw, 1, n_out, n_in, dim=n_in * n_out)
+    bo = pkg.blob(y, dy, 1, 1, n_out, dim=n_out)
+    bb = pkg.blob(bias, dbias, 1, 1, n_out)
+    keep += [bi, bw, bo, bb, x, dx, w, dw, y, dy, bias, dbias]
+    a = pkg.LinearArgs()
+    a.input, a.coeff, a.output = ptr(bi), ptr(bw), ptr(bo)
+    if bias is not None or dbias is not None:
+        a.bias = ptr(bb)
+        a.use_biases = 1
+    return a, keep
+
+
+def mm_args(pkg, A, B, Cm, N, M, K, trans_B):
+    a = pkg.MatMulArgs()
+    a.A, a.B, a.C = pkg.addr(A), pkg.addr(B), pkg.addr(Cm)
+    a.N, a.M, a.K, a.trans_B = N, M, K, trans_B
+    return a
+
+
+def conv_out(n, k, p0, p1, s):
+    return (n - k + p0 + p1) // s + 1

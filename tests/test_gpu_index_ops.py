@@ -1,0 +1,182 @@
+"""GPU parity of the index-permutation and streaming helpers: bit-exact against the CPU oracle."""
+import ctypes
+
+import numpy as np
+import pytest
+import torch
+
+import helpers as hp
+from test_oracle_pin import PATCH_CASES, patch_args
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+
+
+def dev(a):
+    return None if a is None else torch.from_numpy(np.ascontiguousarray(a)).to(DEV)
+
+
+def bits(a):
+    a = np.ascontiguousarray(a)
+    return a.view(np.uint32 if a.dtype == np.float32 else np.uint16)
+
+
+def sync(lib):
+    assert lib.ptl_sync() == 0, lib.ptl_last_error().decode()
+
+
+@pytest.mark.parametrize("dt", ["fp32", "fp16"])
+@pytest.mark.parametrize("hwc", [0, 1])
+@pytest.mark.parametrize("pad,stride,mod", PATCH_CASES)
+def test_im2row_im2col(pkg, orc, gpu, dt, hwc, pad, stride, mod):
+    Ci, Co, H, W, Hk, Wk = 5, 4, 13, 11, 3, 3
+    if mod == 0 and ((H - Hk + pad[2] + pad[3]) % stride[0] or (W - Wk + pad[0] + pad[1]) % stride[1]):
+        H += 1
+        W += 1 if (W - Wk + pad[0] + pad[1]) % stride[1] else 0
+    Ho, Wo = (H - Hk + 1, W - Wk + 1) if mod else (hp.conv_out(H, Hk, pad[2], pad[3], stride[0]),
+                                                  hp.conv_out(W, Wk, pad[0], pad[1], stride[1]))
+    nd = hp.np_dtype(dt)
+    x = hp.uniform(1, (Ci * H * W,), dtype=nd)
+    dy = hp.uniform(2, (Co * Ho * Wo,), dtype=nd)
+    n = (H * W * Co if mod else Ho * Wo * Ci) * Hk * Wk
+    for fn in ("im2row", "im2col"):
+        buf = np.full(n, -1, nd)
+        a, keep = patch_args(pkg, dt, x, dy, buf, Ci, H, W, Co, Hk, Wk, Ho, Wo, pad, stride, mod, hwc)
+        orc.call("orc_" + fn, dt, a)
+        gx, gdy, gbuf = dev(x), dev(dy), dev(np.full(n, -2, nd))
+        g, keep2 = patch_args(pkg, dt, gx, gdy, gbuf, Ci, H, W, Co, Hk, Wk, Ho, Wo, pad, stride, mod, hwc)
+        pkg.call("pulp_%s_%s" % (fn, dt), g)
+        sync(gpu)
+        assert np.array_equal(bits(gbuf.cpu().numpy()), bits(buf)), fn
+
+
+@pytest.mark.parametrize("dt", ["fp32", "fp16"])
+@pytest.mark.parametrize("hwc", [0, 1])
+def test_blocktranspose(pkg, orc, gpu, dt, hwc):
+    Ci, Co, Hk, Wk = 16, 32, 3, 3
+    nd = hp.np_dtype(dt)
+    w = hp.uniform(3, (Co * Ci * Hk * Wk,), dtype=nd)
+    ref = np.zeros_like(w)
+    a = pkg.BlocktranspArgs()
+    a.weights, a.bt_weights, a.Cin, a.Cout, a.Hk, a.Wk, a.HWC = pkg.addr(w), pkg.addr(ref), Ci, Co, Hk, Wk, hwc
+    orc.call("orc_blocktransp", dt, a)
+    gw, gbt = dev(w), dev(np.zeros_like(w))
+    g = pkg.BlocktranspArgs()
+    g.weights, g.bt_weights, g.Cin, g.Cout, g.Hk, g.Wk, g.HWC = pkg.addr(gw), pkg.addr(gbt), Ci, Co, Hk, Wk, hwc
+    pkg.call("pulp_blocktransp_" + dt, g)
+    sync(gpu)
+    assert np.array_equal(bits(gbt.cpu().numpy()), bits(ref))
+    if not hwc:  # applying it again with the channel roles swapped restores the weights
+        gback = dev(np.zeros_like(w))
+        g.weights, g.bt_weights, g.Cin, g.Cout = pkg.addr(gbt), pkg.addr(gback), Co, Ci
+        pkg.call("pulp_blocktransp_" + dt, g)
+        sync(gpu)
+        assert np.array_equal(bits(gback.cpu().numpy()), bits(w))
+
+
+@pytest.mark.parametrize("dt", ["fp32", "fp16"])
+@pytest.mark.parametrize("dims,axes", [((3, 4), (1, 0)), ((128, 64), (1, 0)), ((65, 130), (1, 0)),
+                                       ((2, 3, 4), (2, 0, 1)), ((3, 197, 64), (0, 2, 1)), ((2, 3, 4, 5), (3, 1, 0, 2)),
+                                       ((6,), (0,))])
+def test_transpose(pkg, gpu, dt, dims, axes):
+    np.random.seed(42)
+    m = np.random.rand(*dims).astype(hp.np_dtype(dt))
+    gm, gout = dev(m), dev(np.zeros(m.size, m.dtype))
+    d = (ctypes.c_int * len(dims))(*dims)
+    ax = (ctypes.c_int * len(dims))(*axes)
+    a = pkg.TranspArgs()
+    a.in_matrix, a.out_matrix, a.dim, a.transposed_axes, a.n_dim = pkg.addr(gm), pkg.addr(gout), d, ax, len(dims)
+    pkg.call("transpose" if dt == "fp32" else "transpose_fp16", a)
+    sync(gpu)
+    assert np.array_equal(gout.cpu().numpy(), np.transpose(m, axes).reshape(-1))
+    if len(dims) == 2:
+        gout.zero_()
+        a.N, a.M = dims
+        pkg.call("transpose_matrix" if dt == "fp32" else "transpose_matrix_fp16", a)
+        sync(gpu)
+        assert np.array_equal(gout.cpu().numpy(), m.T.reshape(-1))
+
+
+@pytest.mark.parametrize("dt", ["fp32", "fp16"])
+def test_layout_change_round_trip(pkg, gpu, dt):
+    C, H, W = 16, 32, 32
+    nd = hp.np_dtype(dt)
+    t, gr = hp.uniform(4, (C, H, W), dtype=nd), hp.uniform(5, (C, H, W), dtype=nd)
+    gt, gg, gbuf = dev(t), dev(gr), dev(np.zeros(C * H * W, nd))
+    b = pkg.blob(gt, gg, C, H, W)
+    la = pkg.LayoutArgs()
+    la.tensor, la.transp_buffer, la.transpose_data, la.transpose_grad = hp.ptr(b), pkg.addr(gbuf), 1, 1
+    sfx = "" if dt == "fp32" else "_fp16"
+    pkg.call("CHW_to_HWC" + sfx, la)
+    sync(gpu)
+    assert np.array_equal(gt.cpu().numpy().reshape(H, W, C), t.transpose(1, 2, 0))
+    assert np.array_equal(gg.cpu().numpy().reshape(H, W, C), gr.transpose(1, 2, 0))
+    assert np.array_equal(gbuf.cpu().numpy().reshape(H, W, C), gr.transpose(1, 2, 0))  # buffer keeps the last result
+    pkg.call("HWC_to_CHW" + sfx, la)
+    sync(gpu)
+    assert np.array_equal(gt.cpu().numpy(), t) and np.array_equal(gg.cpu().numpy(), gr)
+
+
+@pytest.mark.parametrize("dt", ["fp32", "fp16"])
+@pytest.mark.parametrize("hwc", [0, 1])
+@pytest.mark.parametrize("pads", [(1, 1, 1, 1), (0, 2, 1, 0)])
+def test_pad_tensor(pkg, gpu, dt, hwc, pads):
+    L, R, U, D = pads
+    C, H, W = 5, 9, 7
+    nd = hp.np_dtype(dt)
+    x = hp.uniform(8, (C, H, W), dtype=nd)
+    ref = np.pad(x, ((0, 0), (U, D), (L, R)))
+    src = x.transpose(1, 2, 0) if hwc else x
+    gs, gd = dev(src), dev(np.full(ref.size, -1, nd))
+    a = pkg.PadArgs()
+    a.source, a.dest, a.C, a.H, a.W = pkg.addr(gs), pkg.addr(gd), C, H, W
+    a.T_LPAD, a.T_RPAD, a.T_UPAD, a.T_DPAD, a.HWC_lay = L, R, U, D, hwc
+    pkg.call("pad_tensor" if dt == "fp32" else "pad_tensor_fp16", a)
+    sync(gpu)
+    expect = ref.transpose(1, 2, 0) if hwc else ref
+    assert np.array_equal(gd.cpu().numpy().reshape(expect.shape), expect)
+
+
+def test_streaming_helpers(pkg, gpu):
+    n = 1000003
+    x, y = hp.uniform(1, (n,)), hp.uniform(2, (n,))
+    gx, gy, gz = dev(x), dev(y), dev(np.zeros(n, np.float32))
+    c = pkg.CopyArgs()
+    c.from_, c.to, c.size = pkg.addr(gx), pkg.addr(gz), n
+    pkg.call("copy", c)
+    sync(gpu)
+    assert torch.equal(gz, gx)
+    v = pkg.VectSumArgs()
+    v.op_1, v.op_2, v.dest, v.size = pkg.addr(gx), pkg.addr(gy), pkg.addr(gz), n
+    pkg.call("vect_sum", v)
+    sync(gpu)
+    assert np.array_equal(gz.cpu().numpy(), x + y)
+    s = pkg.SetToValueArgs()
+    s.to, s.value, s.size = pkg.addr(gz), 0.375, n - 3
+    pkg.call("set_to_value", s)
+    sync(gpu)
+    out = gz.cpu().numpy()
+    assert np.all(out[:n - 3] == 0.375) and np.array_equal(out[n - 3:], (x + y)[n - 3:])
+    # fp16 twins and the casts
+    hx, hy = x.astype(np.float16), y.astype(np.float16)
+    ghx, ghy, ghz = dev(hx), dev(hy), dev(np.zeros(n, np.float16))
+    v.op_1, v.op_2, v.dest = pkg.addr(ghx), pkg.addr(ghy), pkg.addr(ghz)
+    pkg.call("vect_sum_fp16", v)
+    sync(gpu)
+    assert np.array_equal(ghz.cpu().numpy(), hx + hy)
+    s16 = pkg.SetToValueArgsFp16()
+    s16.to, s16.value, s16.size = pkg.addr(ghz), int(np.float16(-1.5).view(np.uint16)), 10
+    pkg.call("set_to_value_fp16", s16)
+    c.from_, c.to, c.size = pkg.addr(ghx), pkg.addr(ghy), n
+    pkg.call("copy_fp16", c)
+    sync(gpu)
+    assert np.all(ghz.cpu().numpy()[:10] == np.float16(-1.5)) and torch.equal(ghy, ghx)
+    k = pkg.CastArgs()
+    k.source, k.destination, k.size = pkg.addr(ghx), pkg.addr(gz), n
+    pkg.call("cast_fp16_tensor_to_fp32", k)
+    sync(gpu)
+    assert np.array_equal(gz.cpu().numpy(), hx.astype(np.float32))
+    k.source, k.destination = pkg.addr(gx), pkg.addr(ghz)
+    pkg.call("cast_fp32_tensor_to_fp16", k)
+    sync(gpu)
+    assert np.array_equal(ghz.cpu().numpy(), x.astype(np.float16))

@@ -1,0 +1,298 @@
+"""GPU parity: every entry point of libptl_hip.so against the CPU oracle on the same seeded inputs.
+
+Bars (BASELINE north star): fp32 outputs and gradients within 1e-4 relative L2 of the oracle, fp16 within
+1e-2 of the fp16-accumulating oracle, index work bit-exact.  All calls go through the C ABI; tensors live in
+device memory (torch is only the allocator) unless a test says it passes host pointers.
+"""
+import ctypes
+
+import numpy as np
+import pytest
+import torch
+
+import helpers as hp
+from helpers import rel_l2
+
+pytestmark = pytest.mark.gpu
+
+TOL = {"fp32": 1e-4, "fp16": 1e-2}
+DEV = "cuda:0"
+
+
+def dev(a):
+    return None if a is None else torch.from_numpy(np.ascontiguousarray(a)).to(DEV)
+
+
+def host(t):
+    return t.cpu().numpy()
+
+
+def sync(lib):
+    assert lib.ptl_sync() == 0, lib.ptl_last_error().decode()
+
+
+# ------------------------------------------------------------------------------ Conv2D
+def conv_parity(pkg, orc, lib, dt, Ci, H, W, Co, Hk, Wk, pad, stride, hwc, ns, seed, im2col=1, bias=False,
+                host_ptrs=False, via_batched=None):
+    L, R, U, D = pad
+    Ho, Wo = hp.conv_out(H, Hk, U, D, stride[0]), hp.conv_out(W, Wk, L, R, stride[1])
+    nd = hp.np_dtype(dt)
+    xs = (ns, H, W, Ci) if hwc else (ns, Ci, H, W)
+    ws = (Co, Hk, Wk, Ci) if hwc else (Co, Ci, Hk, Wk)
+    ys = (ns, Ho, Wo, Co) if hwc else (ns, Co, Ho, Wo)
+    x = hp.uniform(seed, xs, dtype=nd)
+    w = hp.uniform(seed + 1, ws, dtype=nd)
+    dy = hp.uniform(seed + 2, ys, dtype=nd)
+    b = hp.uniform(seed + 3, (Co,), dtype=nd) if bias else None
+    # oracle
+    y, dx, dw = np.zeros(ys, nd), np.zeros(xs, nd), np.zeros(ws, nd)
+    db = np.zeros((Co,), nd) if bias else None
+    a, keep = hp.conv2d_args(pkg, x, dx, w, dw, y, dy, Ci, H, W, Co, Hk, Wk, Ho, Wo, pad, stride, hwc, im2col, b, db)
+    for s in ("fw", "wg", "ig"):
+        orc.call("orc_conv2d_" + s, dt, a, ns)
+    # HIP
+    if host_ptrs:
+        gx, gw, gdy, gb = x, w, dy, b
+        gy, gdx, gdw = np.full(ys, 3, nd), np.full(xs, 3, nd), np.full(ws, 3, nd)
+        gdb = np.full((Co,), 3, nd) if bias else None
+    else:
+        gx, gw, gdy, gb = dev(x), dev(w), dev(dy), dev(b)
+        gy, gdx, gdw = dev(np.full(ys, 3, nd)), dev(np.full(xs, 3, nd)), dev(np.full(ws, 3, nd))
+        gdb = dev(np.full((Co,), 3, nd)) if bias else None
+    g, keep2 = hp.conv2d_args(pkg, gx, gdx, gw, gdw, gy, gdy, Ci, H, W, Co, Hk, Wk, Ho, Wo, pad, stride, hwc, im2col,
+                              gb, gdb)
+    if via_batched is None:
+        via_batched = ns != 1
+    if via_batched:
+        for s in ("fw", "wg", "ig"):
+            pkg.call("ptl_conv2d_%s_%s_batched" % (dt, s), g, ns)
+    else:
+        pkg.call("pulp_conv2d_%s_fw_cl" % dt, g)
+        pkg.call("pulp_conv2d_%s_bw_cl" % dt, g)
+    sync(lib)
+    out = [("y", gy, y), ("dw", gdw, dw), ("dx", gdx, dx)]
+    if bias:
+        out.append(("db", gdb, db))
+    errs = {}
+    for name, got, ref in out:
+        got = got if host_ptrs else host(got)
+        errs[name] = rel_l2(got, ref)
+        assert errs[name] <= TOL[dt], (name, errs[name])
+    return errs
+
+
+CONV_CASES = [
+    # Ci, H, W, Co, Hk, Wk, pad(L,R,U,D), stride
+    (16, 32, 32, 32, 3, 3, (1, 1, 1, 1), (1, 1)),  # BASELINE config 1
+    (8, 8, 8, 8, 3, 3, (0, 0, 0, 0), (1, 1)),      # reference test default
+    (3, 17, 13, 5, 3, 3, (1, 1, 1, 1), (2, 2)),
+    (4, 15, 15, 6, 5, 5, (2, 2, 2, 2), (2, 2)),
+    (5, 9, 12, 7, 3, 2, (1, 0, 0, 2), (1, 1)),
+    (16, 12, 12, 16, 1, 1, (0, 0, 0, 0), (1, 1)),
+    (3, 32, 32, 16, 3, 3, (1, 1, 1, 1), (1, 1)),   # ResNet-20 stem geometry
+    (16, 33, 33, 32, 3, 3, (1, 1, 1, 1), (2, 2)),
+]
+
+
+@pytest.mark.parametrize("dt", ["fp32", "fp16"])
+@pytest.mark.parametrize("hwc", [0, 1])
+@pytest.mark.parametrize("case", CONV_CASES)
+def test_conv2d_batch1(pkg, orc, gpu, dt, hwc, case):
+    Ci, H, W, Co, Hk, Wk, pad, stride = case
+    conv_parity(pkg, orc, gpu, dt, Ci, H, W, Co, Hk, Wk, pad, stride, hwc, 1, 0xC0DE0001)
+
+
+@pytest.mark.parametrize("dt", ["fp32", "fp16"])
+@pytest.mark.parametrize("hwc", [0, 1])
+def test_conv2d_batched(pkg, orc, gpu, dt, hwc):
+    conv_parity(pkg, orc, gpu, dt, 16, 32, 32, 32, 3, 3, (1, 1, 1, 1), (1, 1), hwc, 5, 0xC0DE0011)
+    conv_parity(pkg, orc, gpu, dt, 6, 11, 11, 9, 3, 3, (1, 1, 1, 1), (2, 2), hwc, 3, 0xC0DE0012)
+
+
+@pytest.mark.parametrize("dt", ["fp32", "fp16"])
+def test_conv2d_naive_selector_and_bias(pkg, orc, gpu, dt):
+    conv_parity(pkg, orc, gpu, dt, 4, 10, 10, 6, 3, 3, (1, 1, 1, 1), (1, 1), 0, 1, 0xC0DE0021, im2col=0)
+    conv_parity(pkg, orc, gpu, dt, 4, 10, 10, 6, 3, 3, (1, 1, 1, 1), (1, 1), 0, 2, 0xC0DE0022, bias=True)
+
+
+def test_conv2d_host_pointers_are_staged(pkg, orc, gpu):
+    conv_parity(pkg, orc, gpu, "fp32", 4, 10, 10, 6, 3, 3, (1, 1, 1, 1), (1, 1), 0, 1, 0xC0DE0031, host_ptrs=True)
+    conv_parity(pkg, orc, gpu, "fp16", 4, 10, 10, 6, 3, 3, (0, 0, 0, 0), (1, 1), 1, 2, 0xC0DE0032, host_ptrs=True)
+
+
+def test_conv2d_skip_flags(pkg, gpu):
+    x = dev(hp.uniform(1, (3, 6, 6)))
+    w = dev(hp.uniform(2, (4, 3, 3, 3)))
+    dy = dev(hp.uniform(3, (4, 4, 4)))
+    dx, dw = dev(np.full((3, 6, 6), 9, np.float32)), dev(np.full((4, 3, 3, 3), 9, np.float32))
+    g, keep = hp.conv2d_args(pkg, x, dx, w, dw, None, dy, 3, 6, 6, 4, 3, 3, 4, 4)
+    g.skip_wg_grad, g.skip_in_grad = 1, 0
+    pkg.call("pulp_conv2d_fp32_bw_cl", g)
+    sync(gpu)
+    assert torch.all(dw == 9) and not torch.any(dx == 9)
+
+
+# --------------------------------------------------------------------------- pointwise
+def pw_parity(pkg, orc, lib, dt, Ci, Co, H, W, hwc, ns, seed):
+    nd = hp.np_dtype(dt)
+    xs = (ns, H * W, Ci) if hwc else (ns, Ci, H * W)
+    ys = (ns, H * W, Co) if hwc else (ns, Co, H * W)
+    ws = (Ci, Co) if (hwc and dt == "fp32") else (Co, Ci)
+    x, w, dy = hp.uniform(seed, xs, dtype=nd), hp.uniform(seed + 1, ws, dtype=nd), hp.uniform(seed + 2, ys, dtype=nd)
+    y, dx, dw = np.zeros(ys, nd), np.zeros(xs, nd), np.zeros(ws, nd)
+    a, keep = hp.pw_args(pkg, x, dx, w, dw, y, dy, Ci, Co, H, W, hwc)
+    for s in ("fw", "wg", "ig"):
+        orc.call("orc_conv_pw_" + s, dt, a, ns)
+    gx, gw, gdy = dev(x), dev(w), dev(dy)
+    gy, gdx, gdw = dev(np.full(ys, 3, nd)), dev(np.full(xs, 3, nd)), dev(np.full(ws, 3, nd))
+    g, keep2 = hp.pw_args(pkg, gx, gdx, gw, gdw, gy, gdy, Ci, Co, H, W, hwc)
+    if ns == 1:
+        pkg.call("pulp_conv_pw_%s_fw_cl" % dt, g)
+        pkg.call("pulp_conv_pw_%s_bw_cl" % dt, g)
+    else:
+        for s in ("fw", "wg", "ig"):
+            pkg.call("ptl_conv_pw_%s_%s_batched" % (dt, s), g, ns)
+    sync(lib)
+    errs = {}
+    for name, got, ref in (("y", gy, y), ("dw", gdw, dw), ("dx", gdx, dx)):
+        errs[name] = rel_l2(host(got), ref)
+        assert errs[name] <= TOL[dt], (name, errs[name])
+    return errs
+
+
+@pytest.mark.parametrize("dt", ["fp32", "fp16"])
+@pytest.mark.parametrize("hwc", [0, 1])
+@pytest.mark.parametrize("Ci,Co,H,W,ns", [(8, 8, 8, 8, 1), (8, 16, 7, 9, 1), (64, 128, 56, 56, 1), (24, 40, 10, 10, 4)])
+def test_pointwise(pkg, orc, gpu, dt, hwc, Ci, Co, H, W, ns):
+    pw_parity(pkg, orc, gpu, dt, Ci, Co, H, W, hwc, ns, 0xC0DE0003)
+
+
+# --------------------------------------------------------------------------- depthwise
+def dw_parity(pkg, orc, lib, dt, C, H, W, K, pad, stride, ns, seed):
+    L, R, U, D = pad
+    Ho, Wo = hp.conv_out(H, K, U, D, stride[0]), hp.conv_out(W, K, L, R, stride[1])
+    nd = hp.np_dtype(dt)
+    x = hp.uniform(seed, (ns, C, H, W), dtype=nd)
+    w = hp.uniform(seed + 1, (C, K, K), dtype=nd)
+    dy = hp.uniform(seed + 2, (ns, C, Ho, Wo), dtype=nd)
+    y, dx, dw = np.zeros_like(dy), np.zeros_like(x), np.zeros_like(w)
+    a, keep = hp.dw_args(pkg, dt, x, dx, w, dw, y, dy, C, H, W, K, K, Ho, Wo, pad, stride)
+    for s in ("fw", "wg", "ig"):
+        orc.call("orc_conv_dw_" + s, dt, a, ns)
+    gx, gw, gdy = dev(x), dev(w), dev(dy)
+    gy, gdx, gdw = dev(np.full(dy.shape, 3, nd)), dev(np.full(x.shape, 3, nd)), dev(np.full(w.shape, 3, nd))
+    g, keep2 = hp.dw_args(pkg, dt, gx, gdx, gw, gdw, gy, gdy, C, H, W, K, K, Ho, Wo, pad, stride)
+    if ns == 1:
+        pkg.call("pulp_conv_dw_%s_fw_cl" % dt, g)
+        pkg.call("pulp_conv_dw_%s_bw_cl" % dt, g)
+    else:
+        for s in ("fw", "wg", "ig"):
+            pkg.call("ptl_conv_dw_%s_%s_batched" % (dt, s), g, ns)
+    sync(lib)
+    for name, got, ref in (("y", gy, y), ("dw", gdw, dw), ("dx", gdx, dx)):
+        e = rel_l2(host(got), ref)
+        assert e <= TOL[dt], (name, e)
+
+
+@pytest.mark.parametrize("dt", ["fp32", "fp16"])
+@pytest.mark.parametrize("C,H,W,K,pad,ns", [(8, 9, 9, 3, (0, 0, 0, 0), 1), (64, 58, 58, 3, (0, 0, 0, 0), 1),
+                                            (16, 12, 10, 5, (0, 0, 0, 0), 3), (8, 9, 9, 3, (1, 1, 1, 1), 2)])
+def test_depthwise(pkg, orc, gpu, dt, C, H, W, K, pad, ns):
+    dw_parity(pkg, orc, gpu, dt, C, H, W, K, pad, (1, 1), ns, 0xC0DE0103)
+
+
+def test_depthwise_fp32_stride_and_padding(pkg, orc, gpu):
+    dw_parity(pkg, orc, gpu, "fp32", 6, 11, 11, 3, (1, 1, 1, 1), (2, 2), 2, 0xC0DE0104)
+
+
+# ------------------------------------------------------------------------------ Linear
+def linear_parity(pkg, orc, lib, dt, n_in, n_out, ns, seed, bias=False):
+    nd = hp.np_dtype(dt)
+    x = hp.normal(seed, (ns, n_in), 1.0 / np.sqrt(n_in), nd)
+    w = hp.normal(seed + 1, (n_out, n_in), 1.0 / np.sqrt(n_in), nd)
+    dy = hp.uniform(seed + 2, (ns, n_out), dtype=nd)
+    b = hp.uniform(seed + 3, (n_out,), dtype=nd) if bias else None
+    y, dx, dw = np.zeros_like(dy), np.zeros_like(x), np.zeros_like(w)
+    db = np.zeros((n_out,), nd) if bias else None
+    a, keep = hp.linear_args(pkg, x, dx, w, dw, y, dy, n_in, n_out, b, db)
+    for s in ("fw", "wg", "ig"):
+        orc.call("orc_linear_" + s, dt, a, ns)
+    gx, gw, gdy, gb = dev(x), dev(w), dev(dy), dev(b)
+    gy, gdx, gdw = dev(np.full(dy.shape, 3, nd)), dev(np.full(x.shape, 3, nd)), dev(np.full(w.shape, 3, nd))
+    gdb = dev(np.full((n_out,), 3, nd)) if bias else None
+    g, keep2 = hp.linear_args(pkg, gx, gdx, gw, gdw, gy, gdy, n_in, n_out, gb, gdb)
+    if ns == 1:
+        pkg.call("pulp_linear_%s_fw_cl" % dt, g)
+        pkg.call("pulp_linear_%s_bw_cl" % dt, g)
+    else:
+        for s in ("fw", "wg", "ig"):
+            pkg.call("ptl_linear_%s_%s_batched" % (dt, s), g, ns)
+    sync(lib)
+    out = [("y", gy, y), ("dw", gdw, dw), ("dx", gdx, dx)]
+    if bias:
+        out.append(("db", gdb, db))
+    errs = {}
+    for name, got, ref in out:
+        errs[name] = rel_l2(host(got), ref)
+        assert errs[name] <= TOL[dt], (name, errs[name])
+    return errs
+
+
+@pytest.mark.parametrize("dt", ["fp32", "fp16"])
+@pytest.mark.parametrize("n_in,n_out,ns", [(8, 8, 1), (1024, 8, 1), (1024, 1024, 1), (100, 37, 1), (1024, 1024, 512),
+                                           (72, 50, 9)])
+def test_linear(pkg, orc, gpu, dt, n_in, n_out, ns):
+    linear_parity(pkg, orc, gpu, dt, n_in, n_out, ns, 0xC0DE0002)
+
+
+@pytest.mark.parametrize("dt", ["fp32", "fp16"])
+def test_linear_bias(pkg, orc, gpu, dt):
+    linear_parity(pkg, orc, gpu, dt, 64, 48, 1, 0xC0DE0202, bias=True)
+    linear_parity(pkg, orc, gpu, dt, 64, 48, 6, 0xC0DE0203, bias=True)
+
+
+# ---------------------------------------------------------------------- mm / mm_manager
+@pytest.mark.parametrize("dt", ["fp32", "fp16"])
+@pytest.mark.parametrize("N,M,K", [(32, 32, 32), (32, 1024, 144), (32, 144, 1024), (16, 1024, 288), (128, 3136, 64),
+                                   (7, 5, 3), (1, 33, 20), (33, 1, 20), (9, 11, 1), (130, 70, 515)])
+def test_mm_family(pkg, orc, gpu, dt, N, M, K):
+    nd = hp.np_dtype(dt)
+    for tb in (0, 1):
+        A = hp.normal(5, (N, K), 1.0 / np.sqrt(K), nd)
+        B = hp.uniform(6, (M, K) if tb else (K, M), dtype=nd)
+        C = np.zeros((N, M), nd)
+        orc.call("orc_mm", dt, hp.mm_args(pkg, A, B, C, N, M, K, tb))
+        gA, gB, gC = dev(A), dev(B), dev(np.full((N, M), 3, nd))
+        m = hp.mm_args(pkg, gA, gB, gC, N, M, K, tb)
+        name = "mm" if dt == "fp32" else "mm_fp16"
+        pkg.call(name, m)
+        sync(gpu)
+        assert rel_l2(host(gC), C) <= TOL[dt]
+        # through the dispatcher, every id of the list gives the same product
+        man = pkg.MMManagerArgs()
+        man.mm_args = ctypes.pointer(m)
+        for mid in ((0, 1, 10, 23) if dt == "fp32" else (0, 3, 8)):
+            gC.fill_(3)
+            man.layer_type, man.step_type, man.matmul_type = pkg.LAYER_CONV2D, pkg.STEP_FW, mid
+            pkg.call("mm_manager" if dt == "fp32" else "mm_manager_fp16", man)
+            sync(gpu)
+            assert rel_l2(host(gC), C) <= TOL[dt]
+
+
+def test_mm_k0_leaves_output_untouched(pkg, gpu):
+    gA, gB, gC = dev(np.zeros((3, 1), np.float32)), dev(np.zeros((1, 4), np.float32)), dev(np.full((3, 4), 5, np.float32))
+    pkg.call("mm", hp.mm_args(pkg, gA, gB, gC, 3, 4, 0, 0))
+    sync(gpu)
+    assert torch.all(gC == 5)
+
+
+def test_mm_reference_closed_form(pkg, gpu):
+    """A, B of tests/test_matmul (32x32x32, divider 1e8) against numpy float64."""
+    N = K = M = 32
+    i, j = np.meshgrid(np.arange(N), np.arange(K), indexing="ij")
+    A = ((1.0 + (i + j + 0.1)) / 1e8).astype(np.float32)
+    B = (i * j + 0.1).astype(np.float32)
+    gA, gB, gC = dev(A), dev(B), dev(np.zeros((N, M), np.float32))
+    pkg.call("mm", hp.mm_args(pkg, gA, gB, gC, N, M, K, 0))
+    sync(gpu)
+    assert rel_l2(host(gC), A.astype(np.float64) @ B.astype(np.float64)) < 1e-6
