@@ -1,0 +1,255 @@
+"""Benchmark of the matmul training core on one MI355X.
+
+One step = forward + weight gradient + input gradient of the Linear 1024 -> 1024 layer in fp16 (fp32
+accumulation) over a batch of 512 independent samples (BASELINE.json configs[1], batched mode), called through
+the C ABI of libptl_hip.so with every tensor already resident in HBM.  Prints ONE JSON line.
+
+The line also carries
+  * "roofline": the dominant kernel (the MFMA GEMM) priced against the dense fp16 MFMA peak, from HIP events
+    recorded on the library's stream around the timed region;
+  * "cpu_baseline": the CPU oracle (a port of the reference's C loops, OpenMP over the host cores) timed on a
+    bounded sample of the same workload;
+  * "detail": per-step timings of the other BASELINE shapes (batch-1 latency and batched mode) with their own
+    roofline fractions, so the headline is not the only number on record.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+sys.path.insert(0, os.path.join(ROOT, "tests"))
+
+PEAK = {"fp16": 2500.0, "fp32": 157.3}  # dense MFMA TFLOP/s
+HBM_GBS = 8000.0
+METRIC = "Conv2D/Linear FW+WG+IG TFLOP/s & % MFMA peak (fp32/fp16); samples/s"
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--no-detail", action="store_true", help="skip the per-shape detail table")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
+    ap.add_argument("--batch", type=int, default=512, help="samples per step of the headline workload")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build runs on ONE GPU; --gpus %d is not supported "
+              "(the path shards by sample, see DESIGN.md)" % args.gpus, file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+    import __graft_entry__ as ge
+    import helpers as hp
+
+    pkg = ge.load_package()
+    lib = pkg.load()  # raises if libptl_hip.so is not built
+    if not torch.cuda.is_available():
+        raise RuntimeError("bench.py needs a GPU")
+    if lib.ptl_init(0) != 0:
+        raise RuntimeError(lib.ptl_last_error().decode())
+    dev = torch.device("cuda:0")
+
+    def check(rc):
+        if rc != 0:
+            raise RuntimeError(lib.ptl_last_error().decode())
+
+    def to_dev(a):
+        return torch.from_numpy(np.ascontiguousarray(a)).to(dev)
+
+    def timed(fn, iters, warm=5):
+        """Average milliseconds per call of fn, by HIP events on the library stream."""
+        for _ in range(warm):
+            fn()
+        check(lib.ptl_sync())
+        check(lib.ptl_timer_begin())
+        for _ in range(iters):
+            fn()
+        ms = lib.ptl_timer_end_ms()
+        if ms < 0:
+            raise RuntimeError(lib.ptl_last_error().decode())
+        return ms / iters
+
+    # ------------------------------------------------------------------ headline workload
+    n_in = n_out = 1024
+    ns = args.batch
+    dt, nd = "fp16", np.float16
+    seed = 0xC0DE0002
+    x = hp.normal(seed, (ns, n_in), 1.0 / 32.0, nd)
+    w = hp.normal(seed + 1, (n_out, n_in), 1.0 / 32.0, nd)
+    dy = hp.uniform(seed + 2, (ns, n_out), dtype=nd)
+    gx, gw, gdy = to_dev(x), to_dev(w), to_dev(dy)
+    gy = torch.zeros(ns, n_out, dtype=torch.float16, device=dev)
+    gdx = torch.zeros(ns, n_in, dtype=torch.float16, device=dev)
+    gdw = torch.zeros(n_out, n_in, dtype=torch.float16, device=dev)
+    la, keep = hp.linear_args(pkg, gx, gdx, gw, gdw, gy, gdy, n_in, n_out)
+    import ctypes
+    la_ref = ctypes.byref(la)
+    fw, wg, ig = lib.ptl_linear_fp16_fw_batched, lib.ptl_linear_fp16_wg_batched, lib.ptl_linear_fp16_ig_batched
+
+    def step():
+        check(fw(la_ref, ns))
+        check(wg(la_ref, ns))
+        check(ig(la_ref, ns))
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    check(lib.ptl_timer_begin())
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+    ev_ms = lib.ptl_timer_end_ms()
+    torch.cuda.synchronize()
+    t1 = time.perf_counter()
+    ms_per_step = (t1 - t0) * 1e3 / args.steps
+    flops_step = 3 * 2.0 * ns * n_in * n_out
+    tflops = flops_step / (ms_per_step * 1e-3) / 1e12
+    launches = 3 * args.steps
+    launch_ms = ev_ms / launches
+    achieved = (flops_step / 3) / (launch_ms * 1e-3) / 1e12
+
+    result = {
+        "metric": METRIC,
+        "value": round(tflops, 3),
+        "unit": "TFLOP/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 6),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "f16",
+        "data": "synthetic",
+        "samples_per_s": round(ns / (ms_per_step * 1e-3), 1),
+        "config": {"workload": "linear_1024x1024_fp16_FW+WG+IG_batched_N%d" % ns, "in": n_in, "out": n_out,
+                   "batch": ns, "accumulate": "f32", "layout": "W[out][in], X[batch][in]"},
+        "roofline": {"bound": "mfma", "achieved": round(achieved, 3), "peak": PEAK["fp16"], "unit": "TFLOP/s",
+                     "frac": round(achieved / PEAK["fp16"], 5), "traffic": None,
+                     "kernel": "ptl::gemm_kernel<_Float16,...>", "flops_per_launch": flops_step / 3,
+                     "avg_launch_us": round(launch_ms * 1e3, 3)},
+    }
+
+    # ------------------------------------------------------------------------ CPU baseline
+    if not args.no_cpu:
+        orc = ge.load_oracle()
+        olib = orc.load()
+        cores = int(olib.orc_num_threads())
+
+        def cpu_step(m):
+            y = np.zeros((m, n_out), nd)
+            dx = np.zeros((m, n_in), nd)
+            dw_ = np.zeros((n_out, n_in), nd)
+            a, k2 = hp.linear_args(pkg, x[:m].copy(), dx, w, dw_, y, dy[:m].copy(), n_in, n_out)
+            t = time.perf_counter()
+            for s in ("fw", "wg", "ig"):
+                orc.call("orc_linear_" + s, dt, a, m)
+            return time.perf_counter() - t
+
+        cpu_step(2)
+        t_probe = cpu_step(4) / 4
+        m = int(max(4, min(ns, 12.0 / max(t_probe, 1e-6))))
+        t_cpu = cpu_step(m)
+        cpu_tflops = 3 * 2.0 * m * n_in * n_out / t_cpu / 1e12
+        result["cpu_baseline"] = {"value": round(cpu_tflops, 6), "unit": "TFLOP/s", "cores": cores, "kind": "port",
+                                  "sample": "%d of the %d samples, FW+WG+IG once, fp16 with fp16 accumulation "
+                                            "(the reference's arithmetic), %.2f s" % (m, ns, t_cpu)}
+
+    # ------------------------------------------------------------------------------ detail
+    if not args.no_detail:
+        result["detail"] = detail_table(pkg, lib, hp, to_dev, timed, check, torch, dev)
+
+    print(json.dumps(result))
+
+
+def detail_table(pkg, lib, hp, to_dev, timed, check, torch, dev):
+    """Per-step timings of the other BASELINE shapes: batch-1 latency and batched mode."""
+    import ctypes
+    rows = []
+
+    def add(name, dt, ms, flops, nbytes):
+        tf = flops / (ms * 1e-3) / 1e12
+        gbs = nbytes / (ms * 1e-3) / 1e9
+        bound = min(PEAK[dt], flops / max(nbytes, 1) * HBM_GBS / 1e3)  # TFLOP/s
+        rows.append({"workload": name, "dtype": dt, "us": round(ms * 1e3, 2), "TFLOP/s": round(tf, 3),
+                     "GB/s": round(gbs, 1), "bound_TFLOP/s": round(bound, 1), "frac_of_bound": round(tf / bound, 4)})
+
+    def run3(prefix, dt, a, ns, name, flops, bytes3, iters):
+        ref = ctypes.byref(a)
+        for s, nb in zip(("fw", "wg", "ig"), bytes3):
+            f = getattr(lib, "%s_%s_%s_batched" % (prefix, dt, s))
+            ms = timed(lambda: check(f(ref, ns)), iters)
+            add("%s %s N=%d" % (name, s.upper(), ns), dt, ms, flops, nb)
+
+    es = {"fp32": 4, "fp16": 2}
+    tdt = {"fp32": torch.float32, "fp16": torch.float16}
+
+    # config 1: Conv2D 16->32, 32x32, 3x3, pad 1 (fp32 as named; fp16 beside it), batch 1 and 128
+    for dt in ("fp32", "fp16"):
+        for ns in (1, 128):
+            Ci, Co, H, W, K = 16, 32, 32, 32, 3
+            x = torch.rand(ns, Ci, H, W, device=dev).to(tdt[dt]) - 0.5
+            w = torch.rand(Co, Ci, K, K, device=dev).to(tdt[dt]) - 0.5
+            dy = torch.rand(ns, Co, H, W, device=dev).to(tdt[dt]) - 0.5
+            y, dx, dw = torch.zeros_like(dy), torch.zeros_like(x), torch.zeros_like(w)
+            a, keep = hp.conv2d_args(pkg, x, dx, w, dw, y, dy, Ci, H, W, Co, K, K, H, W, (1, 1, 1, 1))
+            flops = 2.0 * ns * Co * Ci * K * K * H * W
+            nb = (x.numel() + w.numel() + y.numel()) * es[dt]
+            run3("ptl_conv2d", dt, a, ns, "conv2d 16->32 32x32 k3 p1", flops, (nb, nb, nb), 200 if ns == 1 else 50)
+
+    # ResNet-20 stage-3 conv (64->64, 8x8) and stage-1 conv (16->16, 32x32), fp16, batch 128
+    for (Ci, Co, H) in ((16, 16, 32), (64, 64, 8)):
+        ns, K, dt = 128, 3, "fp16"
+        x = torch.rand(ns, Ci, H, H, device=dev).to(tdt[dt]) - 0.5
+        w = torch.rand(Co, Ci, K, K, device=dev).to(tdt[dt]) - 0.5
+        dy = torch.rand(ns, Co, H, H, device=dev).to(tdt[dt]) - 0.5
+        y, dx, dw = torch.zeros_like(dy), torch.zeros_like(x), torch.zeros_like(w)
+        a, keep = hp.conv2d_args(pkg, x, dx, w, dw, y, dy, Ci, H, H, Co, K, K, H, H, (1, 1, 1, 1))
+        flops = 2.0 * ns * Co * Ci * K * K * H * H
+        nb = (x.numel() + w.numel() + y.numel()) * es[dt]
+        run3("ptl_conv2d", dt, a, ns, "conv2d %d->%d %dx%d k3 p1" % (Ci, Co, H, H), flops, (nb, nb, nb), 50)
+
+    # config 2: Linear 1024x1024, batch 1 (both types) and 512 (fp32; fp16 is the headline)
+    for dt, ns in (("fp32", 1), ("fp16", 1), ("fp32", 512), ("fp16", 8192)):
+        n = 1024
+        x = (torch.randn(ns, n, device=dev) / 32).to(tdt[dt])
+        w = (torch.randn(n, n, device=dev) / 32).to(tdt[dt])
+        dy = (torch.rand(ns, n, device=dev) - 0.5).to(tdt[dt])
+        y, dx, dw = torch.zeros_like(dy), torch.zeros_like(x), torch.zeros_like(w)
+        a, keep = hp.linear_args(pkg, x, dx, w, dw, y, dy, n, n)
+        flops = 2.0 * ns * n * n
+        nb = (n * n + 2 * ns * n) * es[dt]
+        run3("ptl_linear", dt, a, ns, "linear 1024x1024", flops, (nb, nb, nb), 200 if ns <= 512 else 20)
+
+    # config 3: depthwise 3x3 on 64x56x56 (pre-padded 58x58) and pointwise 64->128, fp16, batch 1 and 64
+    for ns in (1, 64):
+        dt = "fp16"
+        C, Hp, Ho, K = 64, 58, 56, 3
+        x = (torch.rand(ns, C, Hp, Hp, device=dev) - 0.5).to(tdt[dt])
+        w = (torch.rand(C, K, K, device=dev) - 0.5).to(tdt[dt])
+        dy = (torch.rand(ns, C, Ho, Ho, device=dev) - 0.5).to(tdt[dt])
+        y, dx, dw = torch.zeros_like(dy), torch.zeros_like(x), torch.zeros_like(w)
+        a, keep = hp.dw_args(pkg, dt, x, dx, w, dw, y, dy, C, Hp, Hp, K, K, Ho, Ho)
+        flops = 2.0 * ns * C * K * K * Ho * Ho
+        nb = (x.numel() + y.numel() + w.numel()) * 2
+        run3("ptl_conv_dw", dt, a, ns, "depthwise 3x3 64x56x56", flops, (nb, nb, nb), 100 if ns == 1 else 30)
+        Ci, Co, H = 64, 128, 56
+        x = (torch.rand(ns, Ci, H * H, device=dev) - 0.5).to(tdt[dt])
+        w = (torch.rand(Co, Ci, device=dev) - 0.5).to(tdt[dt])
+        dy = (torch.rand(ns, Co, H * H, device=dev) - 0.5).to(tdt[dt])
+        y, dx, dw = torch.zeros_like(dy), torch.zeros_like(x), torch.zeros_like(w)
+        a, keep = hp.pw_args(pkg, x, dx, w, dw, y, dy, Ci, Co, H, H)
+        flops = 2.0 * ns * Co * Ci * H * H
+        nb = (x.numel() + y.numel() + w.numel()) * 2
+        run3("ptl_conv_pw", dt, a, ns, "pointwise 64->128 56x56", flops, (nb, nb, nb), 100 if ns == 1 else 30)
+    return rows
+
+
+if __name__ == "__main__":
+    main()
