@@ -170,6 +170,10 @@ int ptl_last_status(void);
 /* Stream on which kernels are enqueued (a hipStream_t); NULL = default. */
 void ptl_set_stream(void *hip_stream);
 int ptl_sync(void);
+/* GEMM kernel selection: 0 (default) = the LDS-DMA pipelined kernel wherever
+ * the problem fits it, the register-staged kernel otherwise; 1 = the
+ * register-staged kernel only.  Both compute the same products. */
+void ptl_set_gemm_path(int path);
 /* hipEvent timing on the library stream: begin records, end records,
  * synchronises and returns the elapsed milliseconds (negative on error). */
 int ptl_timer_begin(void);

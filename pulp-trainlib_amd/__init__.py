@@ -51,7 +51,7 @@ BATCHED_ENTRY_POINTS = ["ptl_%s_%s_%s_batched" % (layer, dt, step)
                         for layer in ("conv2d", "conv_pw", "conv_dw", "linear")
                         for dt in ("fp32", "fp16") for step in ("fw", "wg", "ig")]
 
-OTHER_ENTRY_POINTS = ["ptl_init", "ptl_last_error", "ptl_last_status", "ptl_set_stream", "ptl_sync",
+OTHER_ENTRY_POINTS = ["ptl_init", "ptl_last_error", "ptl_last_status", "ptl_set_stream", "ptl_sync", "ptl_set_gemm_path",
                       "ptl_timer_begin", "ptl_timer_end_ms", "ptl_mm_fp32", "ptl_mm_fp16", "ptl_copy_bytes"]
 
 
@@ -80,6 +80,8 @@ def load():
     lib.ptl_last_status.restype = ctypes.c_int
     lib.ptl_set_stream.argtypes = [ctypes.c_void_p]
     lib.ptl_set_stream.restype = None
+    lib.ptl_set_gemm_path.argtypes = [ctypes.c_int]
+    lib.ptl_set_gemm_path.restype = None
     lib.ptl_sync.argtypes = []
     lib.ptl_sync.restype = ctypes.c_int
     lib.ptl_timer_begin.argtypes = []

@@ -89,10 +89,23 @@ inline AxisMap axis_two(int n, int d0, int s1, int s0, int base = 0) {
 }
 
 __host__ __device__ inline void axis_decode(const AxisMap &a, int idx, int &off, int &h, int &w) {
-    int q0 = idx % a.d0;
-    int t = idx / a.d0;
-    int q1 = t % a.d1;
-    int q2 = t / a.d1;
+    // One- and two-digit maps are the common case; skip the divisions they do not need
+    // (the branches are uniform across a wave).
+    int q0, q1, q2;
+    if (a.d0 >= a.n) {
+        q0 = idx;
+        q1 = 0;
+        q2 = 0;
+    } else if (a.d1 >= (1 << 30)) {
+        q1 = idx / a.d0;
+        q0 = idx - q1 * a.d0;
+        q2 = 0;
+    } else {
+        int t = idx / a.d0;
+        q0 = idx - t * a.d0;
+        q2 = t / a.d1;
+        q1 = t - q2 * a.d1;
+    }
     off = q2 * a.o2 + q1 * a.o1 + q0 * a.o0 + a.ob;
     h = q2 * a.h2 + q1 * a.h1 + q0 * a.h0 + a.hb;
     w = q2 * a.w2 + q1 * a.w1 + q0 * a.w0 + a.wb;
@@ -111,6 +124,8 @@ struct State {
     size_t scratch_bytes = 0;
     hipEvent_t ev0 = nullptr, ev1 = nullptr;
     int num_cu = 256;
+    void *zeros = nullptr;  // 256 zero bytes: source of elements that do not exist
+    int gemm_path = 0;      // 0: pipelined kernel where it fits; 1: staged kernel only
 };
 
 State &state();
@@ -122,6 +137,10 @@ void *scratch(size_t bytes);
 
 template <typename T>
 int gemm(const GemmArgs &g);  // returns 0 on success
+
+// Pipelined LDS-DMA kernel: 0 = launched, -1 = problem does not fit, 2 = HIP failure.
+template <typename T>
+int gemm_async(GemmArgs &g);
 
 // GEMV / outer-product kernels for products with a unit dimension.
 template <typename T>

@@ -399,17 +399,11 @@ static void launch_cfg(GemmArgs &g, hipStream_t s) {
     hipLaunchKernelGGL((gemm_kernel<T, BM, BN, WMv, WNv>), grid, dim3(256), 0, s, g);
 }
 
+// Tile shape, split selection and launch of the staged kernel.
 template <typename T>
-int gemm(const GemmArgs &gin) {
-    if (!ensure_init()) return 2;
-    GemmArgs g = gin;
-    if (g.N <= 0 || g.M <= 0 || g.K <= 0) return 0;
+static int launch_staged(GemmArgs &g) {
     State &st = state();
     constexpr int BKE = Traits<T>::BKE;
-
-    g.a.mode = choose_mode<T>(g.a, g.A, g.N, g.K);
-    g.b.mode = choose_mode<T>(g.b, g.B, g.M, g.K);
-
     // Tile shape: skinny outputs get a 32-row (or 32-column) tile; otherwise the
     // largest square tile that still yields at least one workgroup per CU.
     int cfg;
@@ -446,14 +440,32 @@ int gemm(const GemmArgs &gin) {
         g.ws = workspace((size_t)g.splits * g.N * g.M * sizeof(float));
         if (!g.ws) return 2;
     }
-
     switch (cfg) {
         case 0: launch_cfg<T, 128, 128, 2, 2>(g, st.stream); break;
         case 1: launch_cfg<T, 64, 64, 2, 2>(g, st.stream); break;
         case 2: launch_cfg<T, 32, 128, 1, 4>(g, st.stream); break;
         default: launch_cfg<T, 128, 32, 4, 1>(g, st.stream); break;
     }
-    if (!hip_ok(hipGetLastError(), "gemm launch")) return 2;
+    return hip_ok(hipGetLastError(), "gemm launch") ? 0 : 2;
+}
+
+template <typename T>
+int gemm(const GemmArgs &gin) {
+    if (!ensure_init()) return 2;
+    GemmArgs g = gin;
+    if (g.N <= 0 || g.M <= 0 || g.K <= 0) return 0;
+    State &st = state();
+
+    g.a.mode = choose_mode<T>(g.a, g.A, g.N, g.K);
+    g.b.mode = choose_mode<T>(g.b, g.B, g.M, g.K);
+
+    int rc = -1;
+    if (st.gemm_path == 0) rc = gemm_async<T>(g);
+    if (rc > 0) return rc;
+    if (rc < 0) {
+        rc = launch_staged<T>(g);
+        if (rc) return rc;
+    }
     if (g.splits > 1) {
         size_t total = (size_t)g.N * g.M;
         hipLaunchKernelGGL((splitk_reduce_kernel<T>), dim3((unsigned)((total + 255) / 256)), dim3(256), 0,

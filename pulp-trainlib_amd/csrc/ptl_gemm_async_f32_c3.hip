@@ -1,0 +1,7 @@
+// Pipelined GEMM, f32, 128x32 tile, 512 threads (waves 4x1x2): all sixteen operand fill-mode pairs.
+#include "ptl_gemm_async.hpp"
+#include "ptl_gemm_async.inc"
+
+namespace ptl {
+template int launch_async<float, 128, 32, 512, 4, 1, 2>(GemmArgs &, const void *, hipStream_t);
+}

@@ -1,0 +1,64 @@
+// Tile-shape and split selection of the pipelined GEMM.
+#include "ptl_gemm_async.hpp"
+
+namespace ptl {
+
+// Pipelined GEMM.  Returns 0 on success, 2 on a HIP failure, -1 when the problem
+// does not fit this kernel (caller falls back to the staged kernel).
+// `g.a.mode` / `g.b.mode` must already be chosen; on success g.splits / g.ws say
+// whether a split-K reduction has to follow.
+template <typename T>
+int gemm_async(GemmArgs &g) {
+    State &st = state();
+    const void *zero = st.zeros;
+    if (!zero) return -1;
+    constexpr int SK = 128 / (int)sizeof(T);  // k elements per slab (128 bytes per row)
+    auto tiles = [&](int bm, int bn) { return (long)((g.N + bm - 1) / bm) * ((g.M + bn - 1) / bn); };
+    int cfg;
+    if (g.N <= 32)
+        cfg = 2;
+    else if (g.M <= 32)
+        cfg = 3;
+    else if (tiles(128, 128) >= st.num_cu)
+        cfg = 0;
+    else
+        cfg = 1;
+    long nt = cfg == 0 ? tiles(128, 128) : cfg == 1 ? tiles(64, 64) : cfg == 2 ? tiles(32, 128) : tiles(128, 32);
+
+    g.splits = 1;
+    g.kchunk = ((g.K + SK - 1) / SK) * SK;
+    int want = 1;
+    if (nt * 4 <= st.num_cu) want = (int)((st.num_cu + nt - 1) / nt);
+    int need = (g.K + ASYNC_KWMAX - 1) / ASYNC_KWMAX;  // the k look-up table holds ASYNC_KWMAX entries
+    if (want < need) want = need;
+    if (want > 1) {
+        int min_chunk = 4 * SK;
+        int max_splits = (g.K + min_chunk - 1) / min_chunk;
+        int sp = want < max_splits ? want : max_splits;
+        if (sp > 1) {
+            int chunk = (g.K + sp - 1) / sp;
+            chunk = ((chunk + SK - 1) / SK) * SK;
+            sp = (g.K + chunk - 1) / chunk;
+            g.splits = sp;
+            g.kchunk = chunk;
+        }
+    }
+    if (g.kchunk > ASYNC_KWMAX) return -1;
+    if (g.splits > 1) {
+        size_t bytes = (size_t)g.splits * g.N * g.M * sizeof(float);
+        if (bytes > ((size_t)1 << 30)) return -1;
+        g.ws = workspace(bytes);
+        if (!g.ws) return 2;
+    }
+    switch (cfg) {
+        case 0: return launch_async<T, 128, 128, 512, 2, 2, 2>(g, zero, st.stream);
+        case 1: return launch_async<T, 64, 64, 1024, 2, 2, 4>(g, zero, st.stream);
+        case 2: return launch_async<T, 32, 128, 512, 1, 4, 2>(g, zero, st.stream);
+        default: return launch_async<T, 128, 32, 512, 4, 1, 2>(g, zero, st.stream);
+    }
+}
+
+template int gemm_async<float>(GemmArgs &);
+template int gemm_async<half_t>(GemmArgs &);
+
+}  // namespace ptl

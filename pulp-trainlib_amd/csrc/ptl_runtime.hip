@@ -59,6 +59,10 @@ int init_device(int device) {
         if (!hip_ok(hipEventCreate(&st.ev0), "hipEventCreate")) return 2;
         if (!hip_ok(hipEventCreate(&st.ev1), "hipEventCreate")) return 2;
     }
+    if (!st.zeros) {
+        if (!hip_ok(hipMalloc(&st.zeros, 256), "hipMalloc(zeros)")) return 2;
+        if (!hip_ok(hipMemset(st.zeros, 0, 256), "hipMemset(zeros)")) return 2;
+    }
     st.device = device;
     st.ready = true;
     return 0;
@@ -183,6 +187,8 @@ int ptl_init(int device) { return ptl::init_device(device); }
 const char *ptl_last_error(void) { return ptl::last_error(); }
 int ptl_last_status(void) { return ptl::last_status(); }
 void ptl_set_stream(void *s) { ptl::state().stream = static_cast<hipStream_t>(s); }
+
+void ptl_set_gemm_path(int path) { ptl::state().gemm_path = path; }
 
 int ptl_sync(void) {
     if (!ptl::ensure_init()) return 2;
