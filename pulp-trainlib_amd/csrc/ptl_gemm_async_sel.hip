@@ -29,7 +29,9 @@ int gemm_async(GemmArgs &g) {
     g.kchunk = ((g.K + SK - 1) / SK) * SK;
     int want = 1;
     if (nt * 4 <= st.num_cu) want = (int)((st.num_cu + nt - 1) / nt);
-    int need = (g.K + ASYNC_KWMAX - 1) / ASYNC_KWMAX;  // the k look-up table holds ASYNC_KWMAX entries
+    // Operands that are not on the look-up-free path index k through a table of ASYNC_KWMAX entries.
+    const bool need_lut = !(plain_operand<T>(g.a, g.kchunk, g.K) && plain_operand<T>(g.b, g.kchunk, g.K));
+    int need = need_lut ? (g.K + ASYNC_KWMAX - 1) / ASYNC_KWMAX : 1;
     if (want < need) want = need;
     if (want > 1) {
         int min_chunk = 4 * SK;
@@ -43,7 +45,9 @@ int gemm_async(GemmArgs &g) {
             g.kchunk = chunk;
         }
     }
-    if (g.kchunk > ASYNC_KWMAX) return -1;
+    if (g.kchunk > ASYNC_KWMAX &&
+        !(plain_operand<T>(g.a, g.kchunk, g.K) && plain_operand<T>(g.b, g.kchunk, g.K)))
+        return -1;
     if (g.splits > 1) {
         size_t bytes = (size_t)g.splits * g.N * g.M * sizeof(float);
         if (bytes > ((size_t)1 << 30)) return -1;
