@@ -521,6 +521,41 @@ __global__ __launch_bounds__(256) void gemv_coldot_kernel(const T *__restrict__ 
     part[(size_t)blockIdx.y * M + m] = s;
 }
 
+// Same product with 16-byte loads: a workgroup owns CV*VEC consecutive columns and a
+// slice of k; thread (kl, cv) sums rows k0+kl, k0+kl+32, ... of column vector cv, the
+// 32 row-lanes are then folded through LDS.
+template <typename T>
+__global__ __launch_bounds__(256) void gemv_coldot_vec_kernel(const T *__restrict__ x, const T *__restrict__ Mx,
+                                                              float *__restrict__ part, int K, int M, int kchunk) {
+    constexpr int VEC = Traits<T>::VEC, CV = 8, KL = 256 / CV;
+    const int cv = threadIdx.x % CV, kl = threadIdx.x / CV;
+    const int col = (blockIdx.x * CV + cv) * VEC;
+    const int k0 = blockIdx.y * kchunk, k1 = min(K, k0 + kchunk);
+    float acc[VEC];
+#pragma unroll
+    for (int i = 0; i < VEC; ++i) acc[i] = 0.f;
+    if (col < M) {
+        for (int k = k0 + kl; k < k1; k += KL) {
+            Stage<T> v;
+            v.v[0] = *reinterpret_cast<const uint4 *>(Mx + (size_t)k * M + col);
+            float xv = (float)x[k];
+#pragma unroll
+            for (int i = 0; i < VEC; ++i) acc[i] += xv * (float)v.e[i];
+        }
+    }
+    __shared__ float red[KL][CV * VEC + 1];
+#pragma unroll
+    for (int i = 0; i < VEC; ++i) red[kl][cv * VEC + i] = acc[i];
+    __syncthreads();
+    if (threadIdx.x < CV * VEC) {
+        float s = 0.f;
+#pragma unroll 8
+        for (int r = 0; r < KL; ++r) s += red[r][threadIdx.x];
+        int c = blockIdx.x * CV * VEC + threadIdx.x;
+        if (c < M) part[(size_t)blockIdx.y * M + c] = s;
+    }
+}
+
 template <typename T>
 __global__ __launch_bounds__(256) void colsum_reduce_kernel(const float *__restrict__ part, T *__restrict__ y,
                                                             int M, int splits) {
@@ -566,6 +601,23 @@ int mm_dispatch(const T *A, const T *B, T *C, int N, int M, int K, int trans_B) 
     }
     if (M == 1) return gemv_rowdot<T>(A, B, C, N, K);  // B is K x 1 or 1 x K: the same vector
     if (N == 1 && trans_B) return gemv_rowdot<T>(B, A, C, M, K);
+    constexpr int VECW = Traits<T>::VEC;
+    if (N == 1 && M % VECW == 0 && reinterpret_cast<uintptr_t>(B) % 16 == 0) {
+        const int colblk = 8 * VECW;
+        int blocks_m = (M + colblk - 1) / colblk;
+        int splits = (2 * st.num_cu + blocks_m - 1) / blocks_m;
+        if (splits > (K + 31) / 32) splits = (K + 31) / 32;
+        if (splits < 1) splits = 1;
+        int kchunk = (K + splits - 1) / splits;
+        splits = (K + kchunk - 1) / kchunk;
+        float *part = workspace((size_t)splits * M * sizeof(float));
+        if (!part) return 2;
+        hipLaunchKernelGGL((gemv_coldot_vec_kernel<T>), dim3(blocks_m, splits), dim3(256), 0, st.stream, A, B, part,
+                           K, M, kchunk);
+        hipLaunchKernelGGL((colsum_reduce_kernel<T>), dim3((M + 255) / 256), dim3(256), 0, st.stream, part, C, M,
+                           splits);
+        return hip_ok(hipGetLastError(), "gemv launch") ? 0 : 2;
+    }
     if (N == 1) {
         int splits = (st.num_cu * 256 + M - 1) / M;  // about one thread-column per lane of the chip
         if (splits > K / 8) splits = K / 8;

@@ -135,6 +135,156 @@ __global__ __launch_bounds__(256) void dw_wg_reduce_kernel(const float *__restri
     dW[i] = (T)s;
 }
 
+
+// ---- Depthwise fast path: unit stride, KxK with K = 3 or 5, rows at least 32 wide ------
+// Lanes run along a row (consecutive lanes = consecutive columns, so every global access
+// of a wave is one contiguous run); each thread owns a column strip of RB output rows and
+// walks down the input rows once, keeping the K horizontally shifted values of the current
+// input row in registers.  Per output element this is (RB+K-1)*K/RB loads instead of K*K.
+constexpr int DW_RB = 8;  // output rows per thread
+
+// out[p][r][c] = sum_{i,j} wt[ch][i][j] * in[p][r + i - pu][c + j - pl], zero outside the source.
+// FLIP uses wt[K-1-i][K-1-j]: with pu = K-1-Up, pl = K-1-Lp and the output gradient as
+// source this is the input gradient.
+template <typename T, int K, bool FLIP>
+__global__ __launch_bounds__(256) void dw_rows_kernel(const T *__restrict__ src, const T *__restrict__ Wt,
+                                                      T *__restrict__ dst, int C, int Hs, int Ws, int Hd, int Wd,
+                                                      int pu, int pl, int row_blocks, int col_chunks, long total_waves) {
+    long wave = (long)blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (wave >= total_waves) return;
+    const int lane = threadIdx.x & 63;
+    int cc = (int)(wave % col_chunks);
+    long t = wave / col_chunks;
+    int rb = (int)(t % row_blocks);
+    long plane = t / row_blocks;
+    const int ch = (int)(plane % C);
+    const int c = cc * 64 + lane;
+    const int r0 = rb * DW_RB;
+    float w[K][K];
+#pragma unroll
+    for (int i = 0; i < K; ++i)
+#pragma unroll
+        for (int j = 0; j < K; ++j)
+            w[i][j] = (float)Wt[(size_t)ch * K * K + (FLIP ? (K - 1 - i) * K + (K - 1 - j) : i * K + j)];
+    float acc[DW_RB];
+#pragma unroll
+    for (int q = 0; q < DW_RB; ++q) acc[q] = 0.f;
+    const T *sp = src + (size_t)plane * Hs * Ws;
+    bool colok[K];
+#pragma unroll
+    for (int j = 0; j < K; ++j) colok[j] = (unsigned)(c + j - pl) < (unsigned)Ws;
+#pragma unroll
+    for (int rr = 0; rr < DW_RB + K - 1; ++rr) {
+        const int h = r0 + rr - pu;  // source row (wave-uniform)
+        float v[K];
+        const bool rowok = (unsigned)h < (unsigned)Hs;
+#pragma unroll
+        for (int j = 0; j < K; ++j) v[j] = (rowok && colok[j]) ? (float)sp[(size_t)h * Ws + (c + j - pl)] : 0.f;
+#pragma unroll
+        for (int i = 0; i < K; ++i) {
+            const int q = rr - i;  // output row (relative) fed by this source row through tap row i
+            if (q >= 0 && q < DW_RB) {
+#pragma unroll
+                for (int j = 0; j < K; ++j) acc[q] += w[i][j] * v[j];
+            }
+        }
+    }
+    if (c < Wd) {
+        T *dp = dst + (size_t)plane * Hd * Wd;
+#pragma unroll
+        for (int q = 0; q < DW_RB; ++q)
+            if (r0 + q < Hd) dp[(size_t)(r0 + q) * Wd + c] = (T)acc[q];
+    }
+}
+
+// Weight gradient, same walk: part[wave][i][j] = sum over this wave's strip of
+// X[r + i - pu][c + j - pl] * dY[r][c]; a wave owns (plane, row block, column chunk).
+// Partials are summed per channel by dw_wg_reduce_kernel2.
+template <typename T, int K>
+__global__ __launch_bounds__(256) void dw_wg_rows_kernel(const T *__restrict__ X, const T *__restrict__ dY,
+                                                         float *__restrict__ part, int C, int H, int W, int Ho, int Wo,
+                                                         int pu, int pl, int row_blocks, int col_chunks, int rows_per,
+                                                         long total_waves) {
+    long wave = (long)blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (wave >= total_waves) return;
+    const int lane = threadIdx.x & 63;
+    int cc = (int)(wave % col_chunks);
+    long t = wave / col_chunks;
+    int rb = (int)(t % row_blocks);
+    long plane = t / row_blocks;
+    const int c = cc * 64 + lane;
+    const int r0 = rb * rows_per;
+    const int r1 = min(Ho, r0 + rows_per);
+    float acc[K][K];
+#pragma unroll
+    for (int i = 0; i < K; ++i)
+#pragma unroll
+        for (int j = 0; j < K; ++j) acc[i][j] = 0.f;
+    const T *xp = X + (size_t)plane * H * W;
+    const T *gp = dY + (size_t)plane * Ho * Wo;
+    bool colok[K];
+#pragma unroll
+    for (int j = 0; j < K; ++j) colok[j] = (unsigned)(c + j - pl) < (unsigned)W;
+    const bool gcol = c < Wo;
+    // sliding window of K source rows (each at K column shifts)
+    float win[K][K];
+#pragma unroll
+    for (int i = 0; i < K - 1; ++i) {
+        const int h = r0 + i - pu;
+        const bool rowok = (unsigned)h < (unsigned)H;
+#pragma unroll
+        for (int j = 0; j < K; ++j) win[i][j] = (rowok && colok[j]) ? (float)xp[(size_t)h * W + (c + j - pl)] : 0.f;
+    }
+    for (int r = r0; r < r1; ++r) {
+        const int h = r + (K - 1) - pu;
+        const bool rowok = (unsigned)h < (unsigned)H;
+#pragma unroll
+        for (int j = 0; j < K; ++j)
+            win[K - 1][j] = (rowok && colok[j]) ? (float)xp[(size_t)h * W + (c + j - pl)] : 0.f;
+        const float g = gcol ? (float)gp[(size_t)r * Wo + c] : 0.f;
+#pragma unroll
+        for (int i = 0; i < K; ++i)
+#pragma unroll
+            for (int j = 0; j < K; ++j) acc[i][j] += win[i][j] * g;
+#pragma unroll
+        for (int i = 0; i < K - 1; ++i)
+#pragma unroll
+            for (int j = 0; j < K; ++j) win[i][j] = win[i + 1][j];
+    }
+#pragma unroll
+    for (int i = 0; i < K; ++i)
+#pragma unroll
+        for (int j = 0; j < K; ++j) {
+            float v = acc[i][j];
+#pragma unroll
+            for (int o = 32; o > 0; o >>= 1) v += __shfl_down(v, o, 64);
+            if (lane == 0) part[(size_t)wave * K * K + i * K + j] = v;
+        }
+}
+
+// dW[ch][tap] = sum over samples b and strips s of part[(b*C + ch)*strips + s][tap]
+template <typename T>
+__global__ __launch_bounds__(256) void dw_wg_reduce_kernel2(const float *__restrict__ part, T *__restrict__ dW, int ns,
+                                                            int C, int strips, int taps) {
+    const int ch = blockIdx.x;
+    __shared__ float red[256];
+    for (int tap = 0; tap < taps; ++tap) {
+        float s = 0.f;
+        for (long i = threadIdx.x; i < (long)ns * strips; i += 256) {
+            long b = i / strips, st = i % strips;
+            s += part[(((size_t)b * C + ch) * strips + st) * taps + tap];
+        }
+        red[threadIdx.x] = s;
+        __syncthreads();
+        for (int o = 128; o > 0; o >>= 1) {
+            if ((int)threadIdx.x < o) red[threadIdx.x] += red[threadIdx.x + o];
+            __syncthreads();
+        }
+        if (threadIdx.x == 0) dW[(size_t)ch * taps + tap] = (T)red[0];
+        __syncthreads();
+    }
+}
+
 template <typename Args>
 static int dw_geom(const Args *a, DwGeom &g, int sh, int sw, const char *fn) {
     if (!a || !a->input || !a->coeff || !a->output) {
@@ -185,18 +335,71 @@ static int dw_step(const Args *a, int ns, int step, int sh, int sw, const char *
     size_t w_n = (size_t)g.C * g.Hk * g.Wk;
     Stager sg;
     int rc = 0;
+    // row-walking kernels: unit stride, square 3x3 / 5x5 kernel, rows wide enough to fill a wave
+    const bool rows_path = sh == 1 && sw == 1 && g.Hk == g.Wk && (g.Hk == 3 || g.Hk == 5) && g.Wo >= 32 && g.W >= 32;
+    const long planes = (long)ns * g.C;
     if (step == STEP_FW) {
         const T *X = sg.in(reinterpret_cast<const T *>(a->input->data), in_n);
         const T *Wt = sg.in(reinterpret_cast<const T *>(a->coeff->data), w_n);
         T *Y = sg.out(reinterpret_cast<T *>(a->output->data), out_n);
         if (sg.failed()) return 2;
-        hipLaunchKernelGGL((dw_fw_kernel<T>), dim3(nblocks(out_n)), dim3(256), 0, st.stream, X, Wt, Y, g, out_n);
+        if (rows_path) {
+            int rbs = (g.Ho + DW_RB - 1) / DW_RB, ccs = (g.Wo + 63) / 64;
+            long waves = planes * rbs * ccs;
+            dim3 grid((unsigned)((waves + 3) / 4));
+            if (g.Hk == 3)
+                hipLaunchKernelGGL((dw_rows_kernel<T, 3, false>), grid, dim3(256), 0, st.stream, X, Wt, Y, g.C, g.H,
+                                   g.W, g.Ho, g.Wo, g.Up, g.Lp, rbs, ccs, waves);
+            else
+                hipLaunchKernelGGL((dw_rows_kernel<T, 5, false>), grid, dim3(256), 0, st.stream, X, Wt, Y, g.C, g.H,
+                                   g.W, g.Ho, g.Wo, g.Up, g.Lp, rbs, ccs, waves);
+        } else {
+            hipLaunchKernelGGL((dw_fw_kernel<T>), dim3(nblocks(out_n)), dim3(256), 0, st.stream, X, Wt, Y, g, out_n);
+        }
     } else if (step == STEP_IN_GRAD) {
         const T *dY = sg.in(reinterpret_cast<const T *>(a->output->diff), out_n);
         const T *Wt = sg.in(reinterpret_cast<const T *>(a->coeff->data), w_n);
         T *dX = sg.out(reinterpret_cast<T *>(a->input->diff), in_n);
         if (sg.failed()) return 2;
-        hipLaunchKernelGGL((dw_ig_kernel<T>), dim3(nblocks(in_n)), dim3(256), 0, st.stream, dY, Wt, dX, g, in_n);
+        if (rows_path) {
+            int rbs = (g.H + DW_RB - 1) / DW_RB, ccs = (g.W + 63) / 64;
+            long waves = planes * rbs * ccs;
+            dim3 grid((unsigned)((waves + 3) / 4));
+            if (g.Hk == 3)
+                hipLaunchKernelGGL((dw_rows_kernel<T, 3, true>), grid, dim3(256), 0, st.stream, dY, Wt, dX, g.C,
+                                   g.Ho, g.Wo, g.H, g.W, g.Hk - 1 - g.Up, g.Wk - 1 - g.Lp, rbs, ccs, waves);
+            else
+                hipLaunchKernelGGL((dw_rows_kernel<T, 5, true>), grid, dim3(256), 0, st.stream, dY, Wt, dX, g.C,
+                                   g.Ho, g.Wo, g.H, g.W, g.Hk - 1 - g.Up, g.Wk - 1 - g.Lp, rbs, ccs, waves);
+        } else {
+            hipLaunchKernelGGL((dw_ig_kernel<T>), dim3(nblocks(in_n)), dim3(256), 0, st.stream, dY, Wt, dX, g, in_n);
+        }
+    } else if (rows_path) {
+        const T *X = sg.in(reinterpret_cast<const T *>(a->input->data), in_n);
+        const T *dY = sg.in(reinterpret_cast<const T *>(a->output->diff), out_n);
+        T *dW = sg.out(reinterpret_cast<T *>(a->coeff->diff), w_n);
+        if (sg.failed()) return 2;
+        // strips of rows: enough waves to fill the chip, at least 8 rows each
+        int ccs = (g.Wo + 63) / 64;
+        long want = 8L * st.num_cu * 4;
+        int rbs = (int)((want + planes * ccs - 1) / (planes * ccs));
+        if (rbs > (g.Ho + 7) / 8) rbs = (g.Ho + 7) / 8;
+        if (rbs < 1) rbs = 1;
+        int rows_per = (g.Ho + rbs - 1) / rbs;
+        rbs = (g.Ho + rows_per - 1) / rows_per;
+        long waves = planes * rbs * ccs;
+        int taps = g.Hk * g.Wk;
+        float *part = workspace((size_t)waves * taps * sizeof(float));
+        if (!part) return sg.finish(2);
+        dim3 grid((unsigned)((waves + 3) / 4));
+        if (g.Hk == 3)
+            hipLaunchKernelGGL((dw_wg_rows_kernel<T, 3>), grid, dim3(256), 0, st.stream, X, dY, part, g.C, g.H, g.W,
+                               g.Ho, g.Wo, g.Up, g.Lp, rbs, ccs, rows_per, waves);
+        else
+            hipLaunchKernelGGL((dw_wg_rows_kernel<T, 5>), grid, dim3(256), 0, st.stream, X, dY, part, g.C, g.H, g.W,
+                               g.Ho, g.Wo, g.Up, g.Lp, rbs, ccs, rows_per, waves);
+        hipLaunchKernelGGL((dw_wg_reduce_kernel2<T>), dim3(g.C), dim3(256), 0, st.stream, part, dW, ns, g.C,
+                           rbs * ccs, taps);
     } else {
         const T *X = sg.in(reinterpret_cast<const T *>(a->input->data), in_n);
         const T *dY = sg.in(reinterpret_cast<const T *>(a->output->diff), out_n);
