@@ -37,6 +37,9 @@ def main():
     ap.add_argument("--no-detail", action="store_true", help="skip the per-shape detail table")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
     ap.add_argument("--batch", type=int, default=512, help="samples per step of the headline workload")
+    ap.add_argument("--copy-calib", action="store_true",
+                    help="also run a 64 MiB device copy five times (a kernel of known traffic, to scale the "
+                         "FETCH_SIZE / WRITE_SIZE counters of a rocprofv3 --pmc run)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on ONE GPU; --gpus %d is not supported "
@@ -74,6 +77,14 @@ def main():
         if ms < 0:
             raise RuntimeError(lib.ptl_last_error().decode())
         return ms / iters
+
+    if args.copy_calib:
+        nbytes = 64 << 20
+        src = torch.ones(nbytes // 4, dtype=torch.float32, device=dev)
+        dst = torch.zeros_like(src)
+        for _ in range(5):
+            check(lib.ptl_copy_bytes(src.data_ptr(), dst.data_ptr(), nbytes))
+        check(lib.ptl_sync())
 
     # ------------------------------------------------------------------ headline workload
     n_in = n_out = 1024
@@ -135,6 +146,20 @@ def main():
                      "kernel": "ptl::gemm_kernel<_Float16,...>", "flops_per_launch": flops_step / 3,
                      "avg_launch_us": round(launch_ms * 1e3, 3)},
     }
+
+    # The same step handed over as host buffers (the library stages them: allocate, copy in, run, copy out).
+    # Reported beside the headline, never as the headline.
+    hy, hdx, hdw = np.zeros((ns, n_out), nd), np.zeros((ns, n_in), nd), np.zeros((n_out, n_in), nd)
+    ha, hkeep = hp.linear_args(pkg, x, hdx, w, hdw, hy, dy, n_in, n_out)
+    ha_ref = ctypes.byref(ha)
+    for _ in range(2):
+        check(fw(ha_ref, ns)); check(wg(ha_ref, ns)); check(ig(ha_ref, ns))
+    t0 = time.perf_counter()
+    for _ in range(5):
+        check(fw(ha_ref, ns)); check(wg(ha_ref, ns)); check(ig(ha_ref, ns))
+    host_ms = (time.perf_counter() - t0) * 1e3 / 5
+    result["host_staged"] = {"ms_per_step": round(host_ms, 4), "TFLOP/s": round(flops_step / (host_ms * 1e-3) / 1e12, 3),
+                             "note": "same step with host pointers: per call hipMalloc + H2D + kernel + D2H + sync"}
 
     # ------------------------------------------------------------------------ CPU baseline
     if not args.no_cpu:
