@@ -16,6 +16,10 @@ int launch_async(GemmArgs &g, const void *zero, hipStream_t s);
 // Look-up-free loads need: no coordinates, a single-digit k axis with a
 // non-negative stride, non-negative row offsets below 2^31 bytes, and a k range
 // made of whole slabs (there is no zero fill on this path).
+// Lean kernel for the case that both operands are plain (plain_operand() != 0).
+template <typename T, int BM, int BN, int NT, int WMv, int WNv, int WKv, int NS>
+int launch_plain(GemmArgs &g, hipStream_t s);
+
 template <typename T>
 inline int plain_operand(const OperandMap &om, int kchunk, int K) {
     constexpr int SK = 128 / (int)sizeof(T);

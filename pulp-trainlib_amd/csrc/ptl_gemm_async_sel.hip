@@ -54,12 +54,24 @@ int gemm_async(GemmArgs &g) {
         g.ws = workspace(bytes);
         if (!g.ws) return 2;
     }
-    switch (cfg) {
-        case 0: return launch_async<T, 128, 128, 512, 2, 2, 2>(g, zero, st.stream);
-        case 1: return launch_async<T, 64, 64, 1024, 2, 2, 4>(g, zero, st.stream);
-        case 2: return launch_async<T, 32, 128, 512, 1, 4, 2>(g, zero, st.stream);
-        default: return launch_async<T, 128, 32, 512, 4, 1, 2>(g, zero, st.stream);
+    if (plain_operand<T>(g.a, g.kchunk, g.K) && plain_operand<T>(g.b, g.kchunk, g.K)) {
+        switch (cfg) {
+            case 0: return launch_plain<T, 128, 128, 512, 2, 2, 2, 3>(g, st.stream);
+            case 1: return launch_plain<T, 64, 64, 1024, 2, 2, 4, 3>(g, st.stream);
+            case 2: return launch_plain<T, 32, 128, 512, 1, 4, 2, 3>(g, st.stream);
+            default: return launch_plain<T, 128, 32, 512, 4, 1, 2, 3>(g, st.stream);
+        }
     }
+    int rc = -1;
+    switch (cfg) {
+        case 0: rc = launch_async<T, 128, 128, 512, 2, 2, 2>(g, zero, st.stream); break;
+        case 1: break;
+        case 2: rc = launch_async<T, 32, 128, 512, 1, 4, 2>(g, zero, st.stream); break;
+        default: rc = launch_async<T, 128, 32, 512, 4, 1, 2>(g, zero, st.stream); break;
+    }
+    // The small tile also takes the cases whose ring does not fit LDS with a larger one.
+    if (rc == -1) rc = launch_async<T, 64, 64, 1024, 2, 2, 4>(g, zero, st.stream);
+    return rc;
 }
 
 template int gemm_async<float>(GemmArgs &);
