@@ -386,6 +386,15 @@ static int choose_mode(const OperandMap &om, const void *base, int rows, int K) 
             mult(om.row, VEC, false) && mult(om.k, VEC, true))
             return FILL_VEC_R;
     }
+    // Element gather: consecutive lanes walk the axis whose unit-stride runs are longer (for an
+    // implicit im2col that is the pixel axis: a row of the image against a row of the filter).
+    auto run = [](const AxisMap &a) {
+        int s = a.o0 < 0 ? -a.o0 : a.o0;
+        int len = a.d0 < a.n ? a.d0 : a.n;
+        return s == 1 ? len : 0;
+    };
+    int rk = run(om.k), rr = run(om.row);
+    if (rk != rr) return rk > rr ? FILL_ELEM_K : FILL_ELEM_R;
     int ak = om.k.o0 < 0 ? -om.k.o0 : om.k.o0;
     int ar = om.row.o0 < 0 ? -om.row.o0 : om.row.o0;
     return ak <= ar ? FILL_ELEM_K : FILL_ELEM_R;

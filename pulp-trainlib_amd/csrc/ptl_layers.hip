@@ -10,6 +10,7 @@
 // the sum over samples happens in the fp32 accumulator.
 #include "ptl_common.hpp"
 #include "ptl_host.hpp"
+#include "ptl_conv_tile.hpp"
 #include "ptl_api.h"
 #include "ptl_internal.h"
 
@@ -237,6 +238,21 @@ static int conv2d_fw(const Args *a, int ns, const char *fn) {
     }
     if (sg.failed()) return 2;
 
+    int rc = -1;
+    if (!g.hwc && state().gemm_path == 0) {
+        ConvTileDesc d = {};
+        d.batch = ns; d.Cin = g.Ci; d.Hin = g.H; d.Win = g.W;
+        d.Cout = g.Co; d.Ho = g.Ho; d.Wo = g.Wo;
+        d.KH = g.Hk; d.KW = g.Wk; d.sh = g.sh; d.sw = g.sw;
+        d.padU = g.Up; d.padD = g.Dp; d.padL = g.Lp; d.padR = g.Rp;
+        d.x_sb = (long long)g.Ci * g.H * g.W; d.x_sc = (long long)g.H * g.W; d.x_sy = g.W;
+        d.w_base = 0; d.w_sm = K; d.w_sc = g.Hk * g.Wk; d.w_sy = g.Wk; d.w_sx = 1;
+        OutMap c;
+        c.n = axis_two(ns * P, P, g.Co * P, 1);
+        c.m = axis_plain(g.Co, P);
+        rc = conv_tile<T>(d, X, Wt, Y, c);
+        if (rc > 0) return sg.finish(rc);
+    }
     GemmArgs q = {};
     q.K = K;
     OperandMap wmap = {}, pmap = {};
@@ -267,7 +283,7 @@ static int conv2d_fw(const Args *a, int ns, const char *fn) {
         q.c.m = axis_plain(g.Co, 1);
     }
     q.C = Y;
-    int rc = gemm<T>(q);
+    if (rc < 0) rc = gemm<T>(q);
     if (rc == 0 && bias) {
         hipLaunchKernelGGL((bias_add_kernel<T>), dim3(blocks_for(out_n)), dim3(256), 0, state().stream, Y, bias,
                            out_n, g.Co, g.hwc ? 1 : P);
@@ -375,6 +391,21 @@ static int conv2d_ig(const Args *a, int ns, const char *fn) {
     gmap.row.w0 = 1;
     gmap.row.wb = g.Lp;
     gmap.k.n = K;
+    if (!g.hwc && state().gemm_path == 0) {
+        ConvTileDesc d = {};
+        d.batch = ns; d.Cin = g.Co; d.Hin = Hd; d.Win = Wd;
+        d.Cout = g.Ci; d.Ho = g.H; d.Wo = g.W;
+        d.KH = g.Hk; d.KW = g.Wk; d.sh = 1; d.sw = 1;
+        d.padU = g.Hk - 1 - g.Up; d.padL = g.Wk - 1 - g.Lp;
+        d.padD = g.H + g.Hk - 1 - Hd - d.padU; d.padR = g.W + g.Wk - 1 - Wd - d.padL;
+        d.x_sb = (long long)g.Co * Hd * Wd; d.x_sc = (long long)Hd * Wd; d.x_sy = Wd;
+        d.w_base = Pk - 1; d.w_sm = Pk; d.w_sc = g.Ci * Pk; d.w_sy = -g.Wk; d.w_sx = -1;
+        OutMap c;
+        c.n = axis_two(ns * g.H * g.W, g.H * g.W, g.Ci * g.H * g.W, 1);
+        c.m = axis_plain(g.Ci, g.H * g.W);
+        int rc = conv_tile<T>(d, dY, Wt, dX, c);
+        if (rc >= 0) return sg.finish(rc);
+    }
     GemmArgs q = {};
     q.K = K;
     q.C = dX;
