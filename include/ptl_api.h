@@ -170,10 +170,16 @@ int ptl_last_status(void);
 /* Stream on which kernels are enqueued (a hipStream_t); NULL = default. */
 void ptl_set_stream(void *hip_stream);
 int ptl_sync(void);
-/* GEMM kernel selection: 0 (default) = the LDS-DMA pipelined kernel wherever
- * the problem fits it, the register-staged kernel otherwise; 1 = the
- * register-staged kernel only.  Both compute the same products. */
+/* Kernel selection: 0 (default) = the fastest kernel that fits the problem
+ * (direct convolution for large channel-major Conv2D forward / input-gradient
+ * calls, the LDS-DMA pipelined GEMM elsewhere, the register-staged GEMM as the
+ * last resort); 1 = the register-staged GEMM only; 2 = as 0, but the direct
+ * convolution kernel is taken whenever the geometry fits it, however small the
+ * call.  All routes compute the same products.
+ * ptl_last_conv_direct() tells whether the last Conv2D forward or
+ * input-gradient call ran the direct kernel (1) or a GEMM route (0). */
 void ptl_set_gemm_path(int path);
+int ptl_last_conv_direct(void);
 /* hipEvent timing on the library stream: begin records, end records,
  * synchronises and returns the elapsed milliseconds (negative on error). */
 int ptl_timer_begin(void);

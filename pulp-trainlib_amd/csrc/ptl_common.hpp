@@ -125,7 +125,8 @@ struct State {
     hipEvent_t ev0 = nullptr, ev1 = nullptr;
     int num_cu = 256;
     void *zeros = nullptr;  // 256 zero bytes: source of elements that do not exist
-    int gemm_path = 0;      // 0: pipelined kernel where it fits; 1: staged kernel only
+    int gemm_path = 0;      // 0: fastest kernel that fits; 1: staged GEMM only; 2: direct convolution whenever it fits
+    int last_conv_direct = 0;  // 1 if the last Conv2D forward / input-gradient call ran the direct kernel
 };
 
 State &state();

@@ -220,7 +220,7 @@ int conv_tile(const ConvTileDesc &d, const void *X, const void *Wt, void *Y, con
     // used when there are pixel tiles enough to give every CU a few workgroups.
     const int bn = d.Cout <= 32 ? 32 : d.Cout <= 64 ? 64 : 128;
     const long mt = (d.Cout + bn - 1) / bn;
-    if (((long)(a.g.N + BM - 1) / BM) * mt < 2L * st.num_cu) return -1;
+    if (st.gemm_path != 2 && ((long)(a.g.N + BM - 1) / BM) * mt < 2L * st.num_cu) return -1;
 
     // Raw rows of a tile: the output rows it spans, the image seams inside it, plus the filter height.
     const int PP = d.Ho * d.Wo;
@@ -239,9 +239,12 @@ int conv_tile(const ConvTileDesc &d, const void *X, const void *Wt, void *Y, con
     a.magic_perm = magic_of(d.KH * d.KW * (a.CinP / VEC));
     a.magic_cb = magic_of(a.CinP / VEC);
     a.magic_kw = magic_of(d.KW);
-    if (bn == 32) return launch_conv_tile<T, BM, 32, 1>(a, st.stream);
-    if (bn == 64) return launch_conv_tile<T, BM, 64, 1>(a, st.stream);
-    return launch_conv_tile<T, BM, 128, 1>(a, st.stream);
+    // a filter tile that does not fit LDS is halved (more column tiles, each re-reading the pixels)
+    int rc = -1;
+    if (bn == 128) rc = launch_conv_tile<T, BM, 128, 1>(a, st.stream);
+    if (rc == -1 && bn >= 64) rc = launch_conv_tile<T, BM, 64, 1>(a, st.stream);
+    if (rc == -1) rc = launch_conv_tile<T, BM, 32, 1>(a, st.stream);
+    return rc;
 }
 
 template int conv_tile<float>(const ConvTileDesc &, const void *, const void *, void *, const OutMap &);

@@ -469,7 +469,7 @@ int gemm(const GemmArgs &gin) {
     g.b.mode = choose_mode<T>(g.b, g.B, g.M, g.K);
 
     int rc = -1;
-    if (st.gemm_path == 0) rc = gemm_async<T>(g);
+    if (st.gemm_path != 1) rc = gemm_async<T>(g);
     if (rc > 0) return rc;
     if (rc < 0) {
         rc = launch_staged<T>(g);

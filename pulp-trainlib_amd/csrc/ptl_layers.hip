@@ -239,7 +239,8 @@ static int conv2d_fw(const Args *a, int ns, const char *fn) {
     if (sg.failed()) return 2;
 
     int rc = -1;
-    if (!g.hwc && state().gemm_path == 0) {
+    state().last_conv_direct = 0;
+    if (!g.hwc && state().gemm_path != 1) {
         ConvTileDesc d = {};
         d.batch = ns; d.Cin = g.Ci; d.Hin = g.H; d.Win = g.W;
         d.Cout = g.Co; d.Ho = g.Ho; d.Wo = g.Wo;
@@ -252,6 +253,7 @@ static int conv2d_fw(const Args *a, int ns, const char *fn) {
         c.m = axis_plain(g.Co, P);
         rc = conv_tile<T>(d, X, Wt, Y, c);
         if (rc > 0) return sg.finish(rc);
+        if (rc == 0) state().last_conv_direct = 1;
     }
     GemmArgs q = {};
     q.K = K;
@@ -391,7 +393,8 @@ static int conv2d_ig(const Args *a, int ns, const char *fn) {
     gmap.row.w0 = 1;
     gmap.row.wb = g.Lp;
     gmap.k.n = K;
-    if (!g.hwc && state().gemm_path == 0) {
+    state().last_conv_direct = 0;
+    if (!g.hwc && state().gemm_path != 1) {
         ConvTileDesc d = {};
         d.batch = ns; d.Cin = g.Co; d.Hin = Hd; d.Win = Wd;
         d.Cout = g.Ci; d.Ho = g.H; d.Wo = g.W;
@@ -404,6 +407,7 @@ static int conv2d_ig(const Args *a, int ns, const char *fn) {
         c.n = axis_two(ns * g.H * g.W, g.H * g.W, g.Ci * g.H * g.W, 1);
         c.m = axis_plain(g.Ci, g.H * g.W);
         int rc = conv_tile<T>(d, dY, Wt, dX, c);
+        if (rc == 0) state().last_conv_direct = 1;
         if (rc >= 0) return sg.finish(rc);
     }
     GemmArgs q = {};

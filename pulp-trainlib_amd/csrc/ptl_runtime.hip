@@ -189,6 +189,7 @@ int ptl_last_status(void) { return ptl::last_status(); }
 void ptl_set_stream(void *s) { ptl::state().stream = static_cast<hipStream_t>(s); }
 
 void ptl_set_gemm_path(int path) { ptl::state().gemm_path = path; }
+int ptl_last_conv_direct(void) { return ptl::state().last_conv_direct; }
 
 int ptl_sync(void) {
     if (!ptl::ensure_init()) return 2;

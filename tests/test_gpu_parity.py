@@ -109,6 +109,69 @@ def test_conv2d_batched(pkg, orc, gpu, dt, hwc):
     conv_parity(pkg, orc, gpu, dt, 6, 11, 11, 9, 3, 3, (1, 1, 1, 1), (2, 2), hwc, 3, 0xC0DE0012)
 
 
+# The direct convolution kernel (channel-major forward and input gradient) normally takes only calls with
+# many pixel tiles; selection 2 sends every call whose geometry fits through it, so that small cases the
+# oracle finishes in seconds cover its tile logic: tiles that start mid-row, span several images, hang over
+# the end, strides, asymmetric pads, channel counts off the MFMA step, several filter tiles.
+DIRECT_CASES = [
+    # Ci, H, W, Co, Hk, Wk, pad(L,R,U,D), stride, ns
+    (16, 32, 32, 32, 3, 3, (1, 1, 1, 1), (1, 1), 3),
+    (3, 17, 13, 5, 3, 3, (1, 1, 1, 1), (2, 2), 7),
+    (4, 15, 15, 6, 5, 5, (2, 2, 2, 2), (2, 2), 5),
+    (5, 9, 12, 7, 3, 2, (1, 0, 0, 2), (1, 1), 9),
+    (16, 12, 12, 16, 1, 1, (0, 0, 0, 0), (1, 1), 4),
+    (20, 6, 6, 40, 3, 3, (1, 1, 1, 1), (1, 1), 11),    # tiles span several images
+    (33, 40, 7, 130, 3, 3, (1, 1, 1, 1), (1, 1), 2),    # narrow rows, channels off the k step, several filter tiles
+    (8, 20, 70, 9, 3, 3, (0, 1, 2, 0), (1, 2), 2),      # rows wider than a wave
+    (6, 11, 11, 9, 3, 3, (1, 1, 1, 1), (2, 2), 3),
+    (2, 5, 5, 3, 5, 5, (2, 2, 2, 2), (1, 1), 30),       # filter as large as the image
+]
+
+
+@pytest.mark.parametrize("dt", ["fp32", "fp16"])
+@pytest.mark.parametrize("case", DIRECT_CASES)
+def test_conv2d_direct_kernel(pkg, orc, gpu, dt, case):
+    Ci, H, W, Co, Hk, Wk, pad, stride, ns = case
+    gpu.ptl_set_gemm_path(2)
+    try:
+        conv_parity(pkg, orc, gpu, dt, Ci, H, W, Co, Hk, Wk, pad, stride, 0, ns, 0xC0DE0041, via_batched=True)
+        # the last call of conv_parity is the input gradient (130 fp32 channels exceed LDS: GEMM route)
+        assert gpu.ptl_last_conv_direct() == (0 if (Co == 130 and dt == "fp32") else 1)
+        nd = hp.np_dtype(dt)
+        Ho, Wo = hp.conv_out(H, Hk, pad[2], pad[3], stride[0]), hp.conv_out(W, Wk, pad[0], pad[1], stride[1])
+        x, w = dev(np.zeros((ns, Ci, H, W), nd)), dev(np.zeros((Co, Ci, Hk, Wk), nd))
+        y = dev(np.zeros((ns, Co, Ho, Wo), nd))
+        a, keep = hp.conv2d_args(pkg, x, None, w, None, y, None, Ci, H, W, Co, Hk, Wk, Ho, Wo, pad, stride)
+        pkg.call("ptl_conv2d_%s_fw_batched" % dt, a, ns)
+        assert gpu.ptl_last_conv_direct() == 1
+    finally:
+        gpu.ptl_set_gemm_path(0)
+
+
+def test_conv2d_direct_and_gemm_routes_agree(pkg, gpu):
+    """Same forward / input gradient through the direct kernel and through the GEMM route."""
+    for dt, tol in (("fp32", 1e-5), ("fp16", 2e-3)):
+        nd = hp.np_dtype(dt)
+        ns, Ci, Co, H = 160, 16, 32, 32
+        x = dev(hp.uniform(7, (ns, Ci, H, H), dtype=nd))
+        w = dev(hp.uniform(8, (Co, Ci, 3, 3), dtype=nd))
+        dy = dev(hp.uniform(9, (ns, Co, H, H), dtype=nd))
+        res = []
+        for path in (0, 1):
+            gpu.ptl_set_gemm_path(path)
+            y, dx, dw = torch.zeros_like(dy), torch.zeros_like(x), torch.zeros_like(w)
+            a, keep = hp.conv2d_args(pkg, x, dx, w, dw, y, dy, Ci, H, H, Co, 3, 3, H, H, (1, 1, 1, 1))
+            pkg.call("ptl_conv2d_%s_fw_batched" % dt, a, ns)
+            assert gpu.ptl_last_conv_direct() == (1 if path == 0 else 0)
+            pkg.call("ptl_conv2d_%s_ig_batched" % dt, a, ns)
+            assert gpu.ptl_last_conv_direct() == (1 if path == 0 else 0)
+            sync(gpu)
+            res.append((host(y), host(dx)))
+        gpu.ptl_set_gemm_path(0)
+        assert rel_l2(res[0][0], res[1][0]) <= tol
+        assert rel_l2(res[0][1], res[1][1]) <= tol
+
+
 @pytest.mark.parametrize("dt", ["fp32", "fp16"])
 def test_conv2d_naive_selector_and_bias(pkg, orc, gpu, dt):
     conv_parity(pkg, orc, gpu, dt, 4, 10, 10, 6, 3, 3, (1, 1, 1, 1), (1, 1), 0, 1, 0xC0DE0021, im2col=0)
