@@ -44,8 +44,6 @@ struct ConvTileArgs {
     int c_mode;
 };
 
-// n / d through the reciprocal magic = ceil(2^32 / d); magic 0 stands for d == 1.
-__device__ inline int fast_div(int n, unsigned magic) { return magic ? (int)__umulhi((unsigned)n, magic) : n; }
 
 template <typename T, int BM, int BN, int WAVES_K>
 __global__ __launch_bounds__((BM / 32) * WAVES_K * 64) void conv_tile_kernel(const ConvTileArgs a) {
@@ -157,7 +155,6 @@ __global__ __launch_bounds__((BM / 32) * WAVES_K * 64) void conv_tile_kernel(con
     }
 }
 
-static unsigned magic_of(int dv) { return dv <= 1 ? 0u : (unsigned)((((unsigned long long)1 << 32) + dv - 1) / dv); }
 
 template <typename T, int BM, int BN, int WAVES_K>
 static int launch_conv_tile(ConvTileArgs &a, hipStream_t s) {

@@ -24,3 +24,21 @@ template <typename T>
 int conv_tile(const ConvTileDesc &d, const void *X, const void *Wt, void *Y, const OutMap &c);
 
 }  // namespace ptl
+
+namespace ptl {
+
+// Quotients by a divisor fixed per launch: magic = ceil(2^32 / d) gives exact n / d for
+// n, d < 2^16; magic 0 stands for d == 1.
+inline unsigned magic_of(int dv) { return dv <= 1 ? 0u : (unsigned)((((unsigned long long)1 << 32) + dv - 1) / dv); }
+#if defined(__HIPCC__)
+__device__ inline int fast_div(int n, unsigned magic) { return magic ? (int)__umulhi((unsigned)n, magic) : n; }
+#endif
+
+// Weight gradient of the same convolution:
+//   dW(co, ci, ky, kx) = sum_{b, y, x} dY(b, co, y, x) * in(b, ci, y*sh + ky - padU, x*sw + kx - padL)
+// with dY channel-major [b][Cout][Ho*Wo] and dW dense [Cout][Cin][KH][KW].  Returns 0, a positive
+// status on a HIP error, or -1 when the geometry does not fit the kernel.
+template <typename T>
+int conv_tile_wg(const ConvTileDesc &d, const void *X, const void *dY, void *dW);
+
+}  // namespace ptl

@@ -320,6 +320,19 @@ static int conv2d_wg(const Args *a, int ns, const char *fn) {
     }
     if (sg.failed()) return 2;
 
+    int rc = -1;
+    state().last_conv_direct = 0;
+    if (!g.hwc && state().gemm_path != 1) {
+        ConvTileDesc d = {};
+        d.batch = ns; d.Cin = g.Ci; d.Hin = g.H; d.Win = g.W;
+        d.Cout = g.Co; d.Ho = g.Ho; d.Wo = g.Wo;
+        d.KH = g.Hk; d.KW = g.Wk; d.sh = g.sh; d.sw = g.sw;
+        d.padU = g.Up; d.padD = g.Dp; d.padL = g.Lp; d.padR = g.Rp;
+        d.x_sb = (long long)g.Ci * g.H * g.W; d.x_sc = (long long)g.H * g.W; d.x_sy = g.W;
+        rc = conv_tile_wg<T>(d, X, dY, dW);
+        if (rc > 0) return sg.finish(rc);
+        if (rc == 0) state().last_conv_direct = 1;
+    }
     GemmArgs q = {};
     q.A = dY;
     q.B = X;
@@ -341,7 +354,7 @@ static int conv2d_wg(const Args *a, int ns, const char *fn) {
     q.b.WL = g.W;
     q.c.n = axis_plain(g.Co, K);
     q.c.m = axis_plain(K, 1);
-    int rc = gemm<T>(q);
+    if (rc < 0) rc = gemm<T>(q);
     if (rc == 0 && db) {
         hipLaunchKernelGGL((bias_grad_kernel<T>), dim3(g.Co), dim3(256), 0, state().stream, dY, db, ns, g.Co, P,
                            g.hwc);

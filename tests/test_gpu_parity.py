@@ -148,6 +148,38 @@ def test_conv2d_direct_kernel(pkg, orc, gpu, dt, case):
         gpu.ptl_set_gemm_path(0)
 
 
+# The direct weight-gradient kernel needs unit column stride and row lengths that are multiples of the
+# 16-byte vector (8 halves / 4 floats).
+DIRECT_WG_CASES = [
+    # Ci, H, W, Co, Hk, Wk, pad(L,R,U,D), stride, ns
+    (16, 32, 32, 32, 3, 3, (1, 1, 1, 1), (1, 1), 3),
+    (5, 9, 16, 7, 3, 3, (1, 1, 1, 1), (2, 1), 6),       # row stride 2
+    (20, 6, 8, 40, 3, 3, (1, 1, 1, 1), (1, 1), 11),     # tiles span several images; two channel slabs
+    (33, 12, 24, 70, 3, 3, (1, 1, 1, 1), (1, 1), 2),    # two channel slabs, two row tiles
+    (12, 12, 24, 70, 5, 3, (1, 1, 2, 2), (1, 1), 2),    # 15 taps
+    (8, 10, 8, 9, 1, 1, (0, 0, 0, 0), (1, 1), 5),       # single tap
+    (3, 9, 40, 4, 3, 5, (2, 2, 0, 2), (1, 1), 2),       # pads on three sides, 5 columns of taps
+]
+
+
+@pytest.mark.parametrize("dt", ["fp32", "fp16"])
+@pytest.mark.parametrize("case", DIRECT_WG_CASES)
+def test_conv2d_direct_weight_gradient(pkg, orc, gpu, dt, case):
+    Ci, H, W, Co, Hk, Wk, pad, stride, ns = case
+    gpu.ptl_set_gemm_path(2)
+    try:
+        conv_parity(pkg, orc, gpu, dt, Ci, H, W, Co, Hk, Wk, pad, stride, 0, ns, 0xC0DE0051, via_batched=True)
+        nd = hp.np_dtype(dt)
+        Ho, Wo = hp.conv_out(H, Hk, pad[2], pad[3], stride[0]), hp.conv_out(W, Wk, pad[0], pad[1], stride[1])
+        x, dw = dev(np.zeros((ns, Ci, H, W), nd)), dev(np.zeros((Co, Ci, Hk, Wk), nd))
+        dy = dev(np.zeros((ns, Co, Ho, Wo), nd))
+        a, keep = hp.conv2d_args(pkg, x, None, None, dw, None, dy, Ci, H, W, Co, Hk, Wk, Ho, Wo, pad, stride)
+        pkg.call("ptl_conv2d_%s_wg_batched" % dt, a, ns)
+        assert gpu.ptl_last_conv_direct() == 1
+    finally:
+        gpu.ptl_set_gemm_path(0)
+
+
 def test_conv2d_direct_and_gemm_routes_agree(pkg, gpu):
     """Same forward / input gradient through the direct kernel and through the GEMM route."""
     for dt, tol in (("fp32", 1e-5), ("fp16", 2e-3)):
@@ -165,11 +197,13 @@ def test_conv2d_direct_and_gemm_routes_agree(pkg, gpu):
             assert gpu.ptl_last_conv_direct() == (1 if path == 0 else 0)
             pkg.call("ptl_conv2d_%s_ig_batched" % dt, a, ns)
             assert gpu.ptl_last_conv_direct() == (1 if path == 0 else 0)
+            pkg.call("ptl_conv2d_%s_wg_batched" % dt, a, ns)
+            assert gpu.ptl_last_conv_direct() == (1 if path == 0 else 0)
             sync(gpu)
-            res.append((host(y), host(dx)))
+            res.append((host(y), host(dx), host(dw)))
         gpu.ptl_set_gemm_path(0)
-        assert rel_l2(res[0][0], res[1][0]) <= tol
-        assert rel_l2(res[0][1], res[1][1]) <= tol
+        for got, ref in zip(res[0], res[1]):
+            assert rel_l2(got, ref) <= tol
 
 
 @pytest.mark.parametrize("dt", ["fp32", "fp16"])
