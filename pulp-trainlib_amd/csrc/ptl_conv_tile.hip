@@ -6,18 +6,20 @@
 // memory, Hk*Wk times per input element and one lane-load each.  Here a workgroup
 // owns BM consecutive output pixels (raster order over sample, row, column) and BN
 // output channels, and
-//   * loads the input rows those pixels touch ONCE into LDS, as [channel block][row][col]
+//   * gets the input rows those pixels touch ONCE into LDS, as [channel block][row][col]
 //     chunks of 16 bytes that hold VEC consecutive channels of one input position, the
-//     padding halo written as zeros (raw tile).  A chunk is gathered with VEC strided
-//     element loads, which a wave coalesces along the columns;
+//     padding halo as zeros (raw tile).  A first kernel re-lays the channel-major input in
+//     exactly these chunks ([sample][channel block][row][col]), so the raw tile is filled
+//     by LDS-DMA: one 16-byte lane-load per chunk, halo chunks read a zero buffer, nothing
+//     passes through registers;
 //   * loads its BN filters into LDS as [filter][tap][channel] (rows padded to an odd
 //     multiple of 16 bytes, which spreads sixteen consecutive filters over all 64 banks),
 //     once per workgroup: a workgroup then walks several pixel tiles;
 //   * runs the contraction tap by tap, channel blocks innermost: the A fragment of a lane
 //     (one pixel, VEC channels) is ONE ds_read_b128 at rawoff(pixel) + tapoff(hk, wk), the
 //     B fragment another, i.e. the im2col matrix never exists, not even in LDS;
-//   * parks the accumulators in LDS and stores whole lines along the pixel axis
-//     (shared tile epilogue).
+//   * stores straight from the accumulators: filters are the MFMA rows and pixels the
+//     columns, so the 32 lanes of a half-wave write 32 consecutive pixels of one filter.
 // Workgroups are small (BM/32 waves) and use little LDS, so several are resident per CU
 // and hide each other's load, barrier and store phases.
 #include "ptl_gemm_async.hpp"
@@ -40,6 +42,11 @@ struct ConvTileArgs {
     int b_pitch;  // bytes per filter row in LDS
     int b_bytes;  // LDS bytes of the filter tile (the raw tile follows)
     int tiles;    // pixel tiles; a workgroup walks tiles blockIdx.x, blockIdx.x + gridDim.x, ...
+    const void *zero;  // at least 16 readable zero bytes
+    int fast_pix;      // 1: pixel coordinates by reciprocal multiplication (tile-relative quotients below 2^16)
+    int nfast;         // 1: the output's pixel axis is (sample, pixel-in-sample) with the sample size as radix
+    unsigned magic_pp, magic_wo, magic_thp;
+    int raw_chunks;    // chunks of one raw slab (two channel blocks) rounded up to whole waves
     unsigned magic_tw, magic_rr, magic_perm, magic_cb, magic_kw;  // ceil(2^32 / d): exact for n, d < 2^16
     int c_mode;
 };
@@ -51,20 +58,55 @@ __global__ __launch_bounds__((BM / 32) * WAVES_K * 64) void conv_tile_kernel(con
     constexpr int ES = (int)sizeof(T), VEC = 16 / ES, KSTEP = 2 * VEC, FN = BN / 32;
     extern __shared__ __attribute__((aligned(16))) char smem[];
     char *bl = smem;                                          // filters [BN][b_pitch]
-    uint4 *raw = reinterpret_cast<uint4 *>(smem + a.b_bytes);  // raw tile [channel block][row][col] of VEC channels
-    __shared__ int2 rowinfo[64];  // per raw row: element offset of its column 0 in X, valid flag
+    uint4 *raw = reinterpret_cast<uint4 *>(smem + a.b_bytes);  // two raw tiles [channel block][row][col] of VEC channels
+    __shared__ int mlut[BN];      // per filter: output offset
 
     const ConvTileDesc &d = a.d;
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const int wk = wave % WAVES_K, wm = wave / WAVES_K;
+    static_assert(WAVES_K == 1, "one wave per 32 pixels");
+    const int wm = wave;
     const int m0 = blockIdx.y * BN;
     const int PP = d.Ho * d.Wo;
-    const T *__restrict__ X = reinterpret_cast<const T *>(a.X);
+    const uint4 *__restrict__ Xb = reinterpret_cast<const uint4 *>(a.X);  // blocked input
     const T *__restrict__ Wt = reinterpret_cast<const T *>(a.Wt);
     const int kg = lane >> 5, lr = lane & 31;
     const int cblocks = a.CinP / VEC;
 
+    // Software pipeline over the workgroup's slabs.  A slab is one pixel tile times one k step
+    // of channels (two channel blocks, all taps); a tile's slabs accumulate into the same
+    // registers.  The LDS-DMA of the next slab is enqueued into the other raw buffer before the
+    // current one is computed, so its latency hides behind the MFMAs and stores; one barrier per
+    // slab (it has landed for every wave, and every wave is done with the previous one, whose
+    // buffer is refilled next).  Nothing crosses threads except the raw tile itself: each lane
+    // derives its own addresses.
+    const unsigned raw_lds = (unsigned)(uintptr_t)(lds_char *)raw;
+    const int plane_in = d.Hin * d.Win;
+    auto enqueue = [&](int tile, int cs, int buf) {
+        const int n0 = tile * BM;
+        const int b0 = n0 / PP, y0 = (n0 - b0 * PP) / d.Wo;
+        const int t0 = y0 * d.sh;  // first raw row, counted inside the padded image of sample b0
+        for (int c0 = wave * 64; c0 < a.raw_chunks; c0 += NT) {
+            const int c = c0 + lane;
+            const int row = fast_div(c, a.magic_tw), tx = c - row * a.TW;
+            const int half = fast_div(row, a.magic_rr), rr = row - half * a.RR;
+            const int t = t0 + rr, db = fast_div(t, a.magic_thp);  // (t < THP + RR: small quotient)
+            const int b = b0 + db, iy = t - db * a.THP - d.padU, ix = tx - d.padL;
+            const bool ok = half < 2 && b < d.batch && iy >= 0 && iy < d.Hin && ix >= 0 && ix < d.Win;
+            const int cb = cs * 2 + half;
+            const char *src = ok ? reinterpret_cast<const char *>(Xb + (((b * cblocks + cb) * d.Hin + iy) * d.Win + ix))
+                                 : reinterpret_cast<const char *>(a.zero);
+            lds_dma<16>(src, raw_lds + (unsigned)(buf * a.raw_chunks + c0) * 16u);
+        }
+    };
+
+    if ((int)blockIdx.x < a.tiles) enqueue(blockIdx.x, 0, 0);
+
+    for (int i = tid; i < BN; i += NT) {
+        int off = 0, h, w;
+        if (m0 + i < a.g.M) axis_decode(a.g.c.m, m0 + i, off, h, w);
+        mlut[i] = off;
+    }
     // ---- filters, once per workgroup: one 16-byte chunk = VEC consecutive channels of (filter, tap)
     {
         const int taps = d.KH * d.KW, per_m = taps * cblocks, chunks = BN * per_m;
@@ -85,87 +127,118 @@ __global__ __launch_bounds__((BM / 32) * WAVES_K * 64) void conv_tile_kernel(con
         }
     }
 
-    for (int tile = blockIdx.x; tile < a.tiles; tile += gridDim.x) {
-        const int n0 = tile * BM;
-        const int b0 = n0 / PP, y0 = (n0 - b0 * PP) / d.Wo;
-        const int g0 = b0 * a.THP + y0 * d.sh;  // first raw row, counted over padded images
-        if (tid < a.RR) {
-            const int gr = g0 + tid, b = gr / a.THP, iy = gr - b * a.THP - d.padU;
-            int2 e;
-            e.y = (b < d.batch && iy >= 0 && iy < d.Hin) ? 1 : 0;
-            e.x = e.y ? (int)((long long)b * d.x_sb + (long long)iy * d.x_sy) - d.padL : 0;
-            rowinfo[tid] = e;
-        }
-        __syncthreads();  // (also: the previous tile's epilogue is done with the raw area)
-
-        // ---- raw tile: chunk c = (cb * RR + rr) * TW + tx holds VEC channels of one input position
-        {
-            const int chunks = cblocks * a.PLANE;
-            for (int c = tid; c < chunks; c += NT) {
-                const int row = fast_div(c, a.magic_tw), tx = c - row * a.TW;
-                const int cb = fast_div(row, a.magic_rr), rr = row - cb * a.RR;
-                const int2 ri = rowinfo[rr];
-                const int ix = tx - d.padL;
-                const bool ok = ri.y && ix >= 0 && ix < d.Win;
-                const T *src = X + (long long)(cb * VEC) * d.x_sc + ri.x + tx;
-                union {
-                    uint4 v;
-                    T e[VEC];
-                } u;
+    // Accumulator element v of block j is filter j*32 + 8*(v/4) + 4*kg + v%4 (MFMA rows) at this
+    // lane's pixel (MFMA column lr).
+    T pend[FN][16];
+    T *pend_out = nullptr;
+    auto flush = [&]() {
+        if (pend_out) {
 #pragma unroll
-                for (int e = 0; e < VEC; ++e) u.e[e] = (ok && cb * VEC + e < d.Cin) ? src[(long long)e * d.x_sc] : (T)0;
-                raw[c] = u.v;
-            }
+            for (int j = 0; j < FN; ++j)
+#pragma unroll
+                for (int v = 0; v < 16; ++v) {
+                    const int ml = j * 32 + 8 * (v >> 2) + 4 * kg + (v & 3);
+                    if (m0 + ml < a.g.M) pend_out[mlut[ml]] = pend[j][v];
+                }
         }
-        __syncthreads();
+    };
+    const int csteps = a.CinP / KSTEP;
+    int buf = 0;
+    for (int tile = blockIdx.x; tile < a.tiles; tile += gridDim.x) {
+        // this lane's pixel: window corner in the raw tile, output offset
+        const int n0 = tile * BM;
+        const int b0 = n0 / PP, pix0 = n0 - b0 * PP, y0 = pix0 / d.Wo;
+        const int p = min(n0 + wm * 32 + lr, a.g.N - 1);  // overhang pixels repeat the last one; never stored
+        int pb, prem, py;
+        if (a.fast_pix) {  // small quotients: pixel index relative to the tile's first sample
+            const int q = pix0 + (p - n0), db = fast_div(q, a.magic_pp);
+            pb = b0 + db;
+            prem = q - db * PP;
+            py = fast_div(prem, a.magic_wo);
+        } else {
+            pb = p / PP;
+            prem = p - pb * PP;
+            py = prem / d.Wo;
+        }
+        const int px = prem - py * d.Wo;
+        const int corner = ((pb - b0) * a.THP + (py - y0) * d.sh) * a.TW + px * d.sw;
+        int offn, h, w;
+        if (a.nfast)
+            offn = pb * a.g.c.n.o1 + prem * a.g.c.n.o0 + a.g.c.n.ob;
+        else
+            axis_decode(a.g.c.n, p, offn, h, w);
 
-        // ---- contraction: tap by tap, channel blocks innermost
-        int p = n0 + wm * 32 + lr;
-        if (p >= a.g.N) p = a.g.N - 1;  // overhang pixels repeat the last one; they are never stored
-        const int pb = p / PP, prem = p - pb * PP, py = prem / d.Wo, px = prem - py * d.Wo;
-        const uint4 *arow = raw + (pb * a.THP + py * d.sh - g0) * a.TW + px * d.sw + kg * a.PLANE;
-        const char *brow = bl + lr * a.b_pitch + kg * VEC * ES;
-
-        f32x16 acc[1][FN];
+        f32x16 acc[FN];
 #pragma unroll
         for (int j = 0; j < FN; ++j)
 #pragma unroll
-            for (int v = 0; v < 16; ++v) acc[0][j][v] = 0.f;
+            for (int v = 0; v < 16; ++v) acc[j][v] = 0.f;
 
-        const int csteps = a.CinP / KSTEP;
-        int it = 0;
-        for (int ky = 0; ky < d.KH; ++ky)
-            for (int kx = 0; kx < d.KW; ++kx) {
-                const uint4 *ap = arow + ky * a.TW + kx;
-                const char *bp = brow + (ky * d.KW + kx) * a.CinP * ES;
-                for (int cs = 0; cs < csteps; ++cs, ++it) {
-                    if (WAVES_K > 1 && (it % WAVES_K) != wk) continue;
-                    const uint4 af = ap[cs * 2 * a.PLANE];
-                    uint4 bf[FN];
+        for (int cs = 0; cs < csteps; ++cs, buf ^= 1) {
+            wait_vmcnt<0>();
+            __syncthreads();
+            if (cs + 1 < csteps)
+                enqueue(tile, cs + 1, buf ^ 1);
+            else if (tile + (int)gridDim.x < a.tiles)
+                enqueue(tile + gridDim.x, 0, buf ^ 1);
+            if (cs == 0) flush();  // the previous tile's results
+
+            // Contraction, tap by tap.  Filters are the MFMA rows, pixels the columns: a lane ends
+            // up with 16 filters of ONE pixel per block, so the 32 lanes of a half-wave store 32
+            // consecutive pixels of a filter.
+            const uint4 *prow = raw + buf * a.raw_chunks + corner + kg * a.PLANE;
+            const char *frow = bl + lr * a.b_pitch + (cs * KSTEP + kg * VEC) * ES;
+            for (int ky = 0; ky < d.KH; ++ky)
+                for (int kx = 0; kx < d.KW; ++kx) {
+                    const uint4 pf = prow[ky * a.TW + kx];
+                    const char *fp = frow + (ky * d.KW + kx) * a.CinP * ES;
+                    uint4 ff[FN];
 #pragma unroll
-                    for (int j = 0; j < FN; ++j)
-                        bf[j] = *reinterpret_cast<const uint4 *>(bp + j * 32 * a.b_pitch + cs * KSTEP * ES);
+                    for (int j = 0; j < FN; ++j) ff[j] = *reinterpret_cast<const uint4 *>(fp + j * 32 * a.b_pitch);
 #pragma unroll
-                    for (int j = 0; j < FN; ++j) mfma_step<T>(acc[0][j], af, bf[j]);
+                    for (int j = 0; j < FN; ++j) mfma_step<T>(acc[j], ff[j], pf);
                 }
-            }
-        __syncthreads();
-        tile_epilogue<T, BM, BN, NT, BM / 32, 1, WAVES_K, 1, FN>(acc, a.g, reinterpret_cast<float *>(raw), a.c_mode, n0,
-                                                                  m0, 0, tid, wm, 0, wk);
+        }
+
+        // ---- results wait in registers until the next tile's loads are on their way (stores
+        // count in vmcnt like loads: issued here, the wait at the top of the next iteration
+        // would sit out their whole latency)
+        pend_out = (n0 + wm * 32 + lr < a.g.N) ? reinterpret_cast<T *>(a.g.C) + offn : nullptr;
+#pragma unroll
+        for (int j = 0; j < FN; ++j)
+#pragma unroll
+            for (int v = 0; v < 16; ++v) pend[j][v] = (T)acc[j][v];
     }
+    flush();
 }
 
+// Channel-major [sample][channel][pixel] -> [sample][channel block][pixel] chunks of VEC channels
+// (channels beyond the tensor are zeros).  One thread per chunk: its VEC element loads are
+// coalesced along the pixels, its store is 16 bytes.
+template <typename T>
+__global__ __launch_bounds__(256) void chw_to_blocked_kernel(const T *__restrict__ in, uint4 *__restrict__ out, int C,
+                                                             int cblocks, int HW, long long in_sb, long long in_sc,
+                                                             long long total) {
+    constexpr int VEC = 16 / (int)sizeof(T);
+    const long long i = (long long)blockIdx.x * 256 + threadIdx.x;
+    if (i >= total) return;
+    const long long bc = i / HW;
+    const int pix = (int)(i - bc * HW);
+    const int b = (int)(bc / cblocks), cb = (int)(bc - (long long)b * cblocks);
+    const T *src = in + b * in_sb + (long long)(cb * VEC) * in_sc + pix;
+    union {
+        uint4 v;
+        T e[VEC];
+    } u;
+#pragma unroll
+    for (int e = 0; e < VEC; ++e) u.e[e] = (cb * VEC + e < C) ? src[e * in_sc] : (T)0;
+    out[i] = u.v;
+}
 
 template <typename T, int BM, int BN, int WAVES_K>
-static int launch_conv_tile(ConvTileArgs &a, hipStream_t s) {
+static int launch_conv_tile(ConvTileArgs &a, size_t lds, hipStream_t s) {
     constexpr int NT = (BM / 32) * WAVES_K * 64;
     auto kern = conv_tile_kernel<T, BM, BN, WAVES_K>;
-    const size_t red = red_bytes<BM, BN, WAVES_K>();
-    a.b_bytes = BN * a.b_pitch;
-    const size_t raw_bytes = (size_t)(a.CinP / (16 / (int)sizeof(T))) * a.PLANE * 16;
-    const size_t lds = (size_t)a.b_bytes + (raw_bytes > red ? raw_bytes : red);
-    if (lds > 150 * 1024) return -1;
-    if ((long)BN * a.d.KH * a.d.KW * (a.CinP / (16 / (int)sizeof(T))) >= 65536) return -1;
     static bool attr_set = false;
     if (!attr_set) {
         if (!hip_ok(hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
@@ -178,7 +251,7 @@ static int launch_conv_tile(ConvTileArgs &a, hipStream_t s) {
     // slots), each walking an equal share of the tiles with its filters resident.
     a.tiles = (a.g.N + BM - 1) / BM;
     const int mt = (a.g.M + BN - 1) / BN;
-    int occ = (int)((160 * 1024) / (lds + 1024));
+    int occ = (int)((160 * 1024) / (lds + 2048));
     const int by_waves = 32 / (NT / 64);
     if (occ > by_waves) occ = by_waves;
     if (occ < 1) occ = 1;
@@ -195,9 +268,9 @@ int conv_tile(const ConvTileDesc &d, const void *X, const void *Wt, void *Y, con
     State &st = state();
     constexpr int ES = (int)sizeof(T), VEC = 16 / ES, KSTEP = 2 * VEC, BM = 128;
     ConvTileArgs a = {};
-    a.X = X;
     a.Wt = Wt;
     a.d = d;
+    a.zero = st.zeros;
     a.g.C = Y;
     a.g.c = c;
     a.g.N = d.batch * d.Ho * d.Wo;
@@ -208,16 +281,12 @@ int conv_tile(const ConvTileDesc &d, const void *X, const void *Wt, void *Y, con
     a.CinP = ((d.Cin + KSTEP - 1) / KSTEP) * KSTEP;
     a.THP = d.Hin + d.padU + d.padD;
     a.TW = d.Win + d.padL + d.padR;
-    if (d.padU < 0 || d.padD < 0 || d.padL < 0 || d.padR < 0) return -1;
+    if (!a.zero || d.padU < 0 || d.padD < 0 || d.padL < 0 || d.padR < 0 || d.x_sy != d.Win) return -1;
     // every output pixel's window must lie inside the padded image
     if ((d.Ho - 1) * d.sh + d.KH > a.THP || (d.Wo - 1) * d.sw + d.KW > a.TW) return -1;
-
-    // Filters per workgroup: the narrowest of 32/64/128 that covers them (or 128 with several
-    // column tiles).  The kernel pays a per-workgroup price for its filter tile, so it is only
-    // used when there are pixel tiles enough to give every CU a few workgroups.
-    const int bn = d.Cout <= 32 ? 32 : d.Cout <= 64 ? 64 : 128;
-    const long mt = (d.Cout + bn - 1) / bn;
-    if (st.gemm_path != 2 && ((long)(a.g.N + BM - 1) / BM) * mt < 2L * st.num_cu) return -1;
+    const int cblocks = a.CinP / VEC;
+    const long long in_chunks = (long long)d.batch * cblocks * d.Hin * d.Win;
+    if (in_chunks >= ((long long)1 << 31)) return -1;
 
     // Raw rows of a tile: the output rows it spans, the image seams inside it, plus the filter height.
     const int PP = d.Ho * d.Wo;
@@ -227,21 +296,49 @@ int conv_tile(const ConvTileDesc &d, const void *X, const void *Wt, void *Y, con
     a.RR = (rows_spanned - 1) * d.sh + seams * seam_rows + d.KH;
     if (a.RR > 64) return -1;
     a.PLANE = a.RR * a.TW;
-    if ((long)(a.CinP / VEC) * a.PLANE >= 65536 || a.TW >= 65536) return -1;
+    a.raw_chunks = (2 * a.PLANE + 63) & ~63;  // one slab: two channel blocks
+    if (a.raw_chunks >= 65536 || a.TW >= 65536) return -1;
     int pitch16 = (d.KH * d.KW * a.CinP * ES + 15) / 16;
     if ((pitch16 & 1) == 0) ++pitch16;
     a.b_pitch = pitch16 * 16;
+
+    // Filters per workgroup: the narrowest of 32/64/128 that covers them (or 128 with several
+    // column tiles), halved while the filter tile does not fit LDS (more column tiles, each
+    // re-reading the pixels).  The kernel pays a per-workgroup price for its filter tile, so it
+    // is only used when there are pixel tiles enough to give every CU a few workgroups.
+    int bn = d.Cout <= 32 ? 32 : d.Cout <= 64 ? 64 : 128;
+    size_t lds = 0;
+    for (;; bn /= 2) {
+        lds = (size_t)bn * a.b_pitch + 2 * (size_t)a.raw_chunks * 16;  // filters + two raw buffers
+        if (lds <= 150 * 1024 && (long)bn * d.KH * d.KW * cblocks < 65536) break;
+        if (bn == 32) return -1;
+    }
+    a.b_bytes = bn * a.b_pitch;
+    const long mt = (d.Cout + bn - 1) / bn;
+    if (st.gemm_path != 2 && ((long)(a.g.N + BM - 1) / BM) * mt < 2L * st.num_cu) return -1;
+
     a.magic_tw = magic_of(a.TW);
     a.magic_rr = magic_of(a.RR);
-    a.magic_perm = magic_of(d.KH * d.KW * (a.CinP / VEC));
-    a.magic_cb = magic_of(a.CinP / VEC);
+    a.magic_perm = magic_of(d.KH * d.KW * cblocks);
+    a.magic_cb = magic_of(cblocks);
     a.magic_kw = magic_of(d.KW);
-    // a filter tile that does not fit LDS is halved (more column tiles, each re-reading the pixels)
-    int rc = -1;
-    if (bn == 128) rc = launch_conv_tile<T, BM, 128, 1>(a, st.stream);
-    if (rc == -1 && bn >= 64) rc = launch_conv_tile<T, BM, 64, 1>(a, st.stream);
-    if (rc == -1) rc = launch_conv_tile<T, BM, 32, 1>(a, st.stream);
-    return rc;
+    a.fast_pix = (PP + BM < 65536 && d.Wo < 65536) ? 1 : 0;
+    a.magic_pp = magic_of(PP);
+    a.magic_wo = magic_of(d.Wo);
+    a.magic_thp = magic_of(a.THP);
+    if (a.THP + a.RR >= 65536) return -1;
+    a.nfast = (c.n.d0 == PP && c.n.d1 >= (1 << 30)) ? 1 : 0;
+
+    // re-lay the input in chunks of VEC channels
+    uint4 *xb = reinterpret_cast<uint4 *>(workspace((size_t)in_chunks * 16));
+    if (!xb) return 2;
+    hipLaunchKernelGGL((chw_to_blocked_kernel<T>), dim3((unsigned)((in_chunks + 255) / 256)), dim3(256), 0, st.stream,
+                       reinterpret_cast<const T *>(X), xb, d.Cin, cblocks, d.Hin * d.Win, d.x_sb, d.x_sc, in_chunks);
+    if (!hip_ok(hipGetLastError(), "blocked layout launch")) return 2;
+    a.X = xb;
+    if (bn == 128) return launch_conv_tile<T, BM, 128, 1>(a, lds, st.stream);
+    if (bn == 64) return launch_conv_tile<T, BM, 64, 1>(a, lds, st.stream);
+    return launch_conv_tile<T, BM, 32, 1>(a, lds, st.stream);
 }
 
 template int conv_tile<float>(const ConvTileDesc &, const void *, const void *, void *, const OutMap &);
