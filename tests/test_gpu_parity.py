@@ -135,8 +135,9 @@ def test_conv2d_direct_kernel(pkg, orc, gpu, dt, case):
     gpu.ptl_set_gemm_path(2)
     try:
         conv_parity(pkg, orc, gpu, dt, Ci, H, W, Co, Hk, Wk, pad, stride, 0, ns, 0xC0DE0041, via_batched=True)
-        # the last call of conv_parity is the input gradient
-        assert gpu.ptl_last_conv_direct() == 1
+        # the last call of conv_parity is the input gradient (32 filters of 130 fp32 channels and 9 taps
+        # exceed LDS: GEMM route)
+        assert gpu.ptl_last_conv_direct() == (0 if (Co == 130 and dt == "fp32") else 1)
         nd = hp.np_dtype(dt)
         Ho, Wo = hp.conv_out(H, Hk, pad[2], pad[3], stride[0]), hp.conv_out(W, Wk, pad[0], pad[1], stride[1])
         x, w = dev(np.zeros((ns, Ci, H, W), nd)), dev(np.zeros((Co, Ci, Hk, Wk), nd))
