@@ -219,6 +219,11 @@ int ptl_linear_fp32_ig_batched(const struct Linear_args *a, int nsamples);
 int ptl_linear_fp16_fw_batched(const struct Linear_args_fp16 *a, int nsamples);
 int ptl_linear_fp16_wg_batched(const struct Linear_args_fp16 *a, int nsamples);
 int ptl_linear_fp16_ig_batched(const struct Linear_args_fp16 *a, int nsamples);
+/* Weight and input gradient of a batch in ONE call, as pulp_linear_fp32_bw_cl /
+ * pulp_linear_fp16_bw_cl do for one sample (lib/sources/pulp_linear_fp32.c:67-83,
+ * lib/sources/pulp_linear_fp16.c); both products share a launch where they fit. */
+int ptl_linear_fp32_bw_batched(const struct Linear_args *a, int nsamples);
+int ptl_linear_fp16_bw_batched(const struct Linear_args_fp16 *a, int nsamples);
 
 /* Plain product C[N x M] = A[N x K] * B (B is K x M, or M x K when trans_B),
  * the contract of the reference's mm family, on raw pointers. */

@@ -49,7 +49,8 @@ VOID_ENTRY_POINTS = [
 # `int f(const args *, int nsamples)` batched launchers.
 BATCHED_ENTRY_POINTS = ["ptl_%s_%s_%s_batched" % (layer, dt, step)
                         for layer in ("conv2d", "conv_pw", "conv_dw", "linear")
-                        for dt in ("fp32", "fp16") for step in ("fw", "wg", "ig")]
+                        for dt in ("fp32", "fp16") for step in ("fw", "wg", "ig")] + [
+                            "ptl_linear_fp32_bw_batched", "ptl_linear_fp16_bw_batched"]
 
 OTHER_ENTRY_POINTS = ["ptl_init", "ptl_last_error", "ptl_last_status", "ptl_set_stream", "ptl_sync", "ptl_set_gemm_path",
                       "ptl_last_conv_direct", "ptl_timer_begin", "ptl_timer_end_ms", "ptl_mm_fp32", "ptl_mm_fp16", "ptl_copy_bytes"]

@@ -143,6 +143,13 @@ int gemm(const GemmArgs &g);  // returns 0 on success
 template <typename T>
 int gemm_async(GemmArgs &g);
 
+// Two independent products; one launch where both fit the look-up-free kernel with the same
+// tile shape, else one after the other.
+template <typename T>
+int gemm_pair(const GemmArgs &g0, const GemmArgs &g1);
+template <typename T>
+int gemm_async_pair(GemmArgs &g0, GemmArgs &g1);
+
 // GEMV / outer-product kernels for products with a unit dimension.
 template <typename T>
 int mm_dispatch(const T *A, const T *B, T *C, int N, int M, int K, int trans_B);

@@ -484,6 +484,24 @@ int gemm(const GemmArgs &gin) {
     return 0;
 }
 
+template <typename T>
+int gemm_pair(const GemmArgs &g0in, const GemmArgs &g1in) {
+    if (!ensure_init()) return 2;
+    GemmArgs g0 = g0in, g1 = g1in;
+    if (state().gemm_path == 0 && g0.N > 0 && g0.M > 0 && g0.K > 0 && g1.N > 0 && g1.M > 0 && g1.K > 0) {
+        g0.a.mode = choose_mode<T>(g0.a, g0.A, g0.N, g0.K);
+        g0.b.mode = choose_mode<T>(g0.b, g0.B, g0.M, g0.K);
+        g1.a.mode = choose_mode<T>(g1.a, g1.A, g1.N, g1.K);
+        g1.b.mode = choose_mode<T>(g1.b, g1.B, g1.M, g1.K);
+        int rc = gemm_async_pair<T>(g0, g1);
+        if (rc >= 0) return rc;
+    }
+    int rc = gemm<T>(g0in);
+    return rc ? rc : gemm<T>(g1in);
+}
+
+template int gemm_pair<float>(const GemmArgs &, const GemmArgs &);
+template int gemm_pair<half_t>(const GemmArgs &, const GemmArgs &);
 template int gemm<float>(const GemmArgs &);
 template int gemm<half_t>(const GemmArgs &);
 

@@ -20,6 +20,9 @@ int launch_async(GemmArgs &g, const void *zero, hipStream_t s);
 template <typename T, int BM, int BN, int NT, int WMv, int WNv, int WKv, int NS>
 int launch_plain(GemmArgs &g, hipStream_t s);
 
+template <typename T, int BM, int BN, int NT, int WMv, int WNv, int WKv, int NS>
+int launch_plain_pair(GemmArgs &g0, GemmArgs &g1, hipStream_t s);
+
 template <typename T>
 inline int plain_operand(const OperandMap &om, int kchunk, int K) {
     constexpr int SK = 128 / (int)sizeof(T);

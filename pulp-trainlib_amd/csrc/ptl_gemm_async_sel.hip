@@ -74,6 +74,31 @@ int gemm_async(GemmArgs &g) {
     return rc;
 }
 
+// Both products in one launch when they are look-up free, need no k split and agree on the
+// tile shape; -1 otherwise (the caller then runs them one after the other).
+template <typename T>
+int gemm_async_pair(GemmArgs &g0, GemmArgs &g1) {
+    State &st = state();
+    constexpr int SK = 128 / (int)sizeof(T);
+    GemmArgs *gs[2] = {&g0, &g1};
+    int cfg[2];
+    for (int i = 0; i < 2; ++i) {
+        GemmArgs &g = *gs[i];
+        g.splits = 1;
+        g.kchunk = g.K;
+        if (g.K % SK || !plain_operand<T>(g.a, g.kchunk, g.K) || !plain_operand<T>(g.b, g.kchunk, g.K)) return -1;
+        auto tiles = [&](int bm, int bn) { return (long)((g.N + bm - 1) / bm) * ((g.M + bn - 1) / bn); };
+        if (g.N <= 32 || g.M <= 32) return -1;
+        cfg[i] = tiles(128, 128) >= st.num_cu ? 0 : 1;
+        if (cfg[i] == 1 && tiles(64, 64) * 4 <= st.num_cu) return -1;  // would want a k split
+    }
+    if (cfg[0] != cfg[1]) return -1;
+    if (cfg[0] == 0) return launch_plain_pair<T, 128, 128, 512, 2, 2, 2, 3>(g0, g1, st.stream);
+    return launch_plain_pair<T, 64, 64, 1024, 2, 2, 4, 3>(g0, g1, st.stream);
+}
+
+template int gemm_async_pair<float>(GemmArgs &, GemmArgs &);
+template int gemm_async_pair<half_t>(GemmArgs &, GemmArgs &);
 template int gemm_async<float>(GemmArgs &);
 template int gemm_async<half_t>(GemmArgs &);
 

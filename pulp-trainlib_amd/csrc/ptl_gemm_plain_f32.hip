@@ -7,4 +7,6 @@ template int launch_plain<float, 128, 128, 512, 2, 2, 2, 3>(GemmArgs &, hipStrea
 template int launch_plain<float, 64, 64, 1024, 2, 2, 4, 3>(GemmArgs &, hipStream_t);
 template int launch_plain<float, 32, 128, 512, 1, 4, 2, 3>(GemmArgs &, hipStream_t);
 template int launch_plain<float, 128, 32, 512, 4, 1, 2, 3>(GemmArgs &, hipStream_t);
+template int launch_plain_pair<float, 128, 128, 512, 2, 2, 2, 3>(GemmArgs &, GemmArgs &, hipStream_t);
+template int launch_plain_pair<float, 64, 64, 1024, 2, 2, 4, 3>(GemmArgs &, GemmArgs &, hipStream_t);
 }

@@ -11,6 +11,8 @@
 #include "ptl_common.hpp"
 #include "ptl_host.hpp"
 #include "ptl_conv_tile.hpp"
+
+#define STEP_BW_BOTH 3  // weight and input gradient together (library-internal step code)
 #include "ptl_api.h"
 #include "ptl_internal.h"
 
@@ -665,6 +667,48 @@ static int linear_step(const Args *a, int ns, int step, const char *fn) {
                                bias, total, out);
             if (!hip_ok(hipGetLastError(), "bias add launch")) rc = 2;
         }
+    } else if (step == STEP_BW_BOTH) {
+        // weight and input gradient of a batch in one launch
+        const T *X = sg.in(reinterpret_cast<const T *>(a->input->data), (size_t)ns * in);
+        const T *Wt = sg.in(reinterpret_cast<const T *>(a->coeff->data), (size_t)out * in);
+        const T *dY = sg.in(reinterpret_cast<const T *>(a->output->diff), (size_t)ns * out);
+        T *dW = sg.out(reinterpret_cast<T *>(a->coeff->diff), (size_t)out * in);
+        T *dX = sg.out(reinterpret_cast<T *>(a->input->diff), (size_t)ns * in);
+        T *db = use_bias ? sg.out(reinterpret_cast<T *>(a->bias->diff), (size_t)out) : nullptr;
+        if (sg.failed()) return 2;
+        GemmArgs q = {}, r = {};
+        q.A = dY;  // dW[o][i] = sum_b dY[b][o] * X[b][i]
+        q.B = X;
+        q.C = dW;
+        q.N = out;
+        q.M = in;
+        q.K = ns;
+        q.a.row = axis_plain(out, 1);
+        q.a.k = axis_plain(ns, out);
+        q.b.row = axis_plain(in, 1);
+        q.b.k = axis_plain(ns, in);
+        q.a.HL = q.a.WL = q.b.HL = q.b.WL = 1;
+        q.c.n = axis_plain(out, in);
+        q.c.m = axis_plain(in, 1);
+        r.A = dY;  // dX[b][i] = sum_o dY[b][o] * W[o][i]
+        r.B = Wt;
+        r.C = dX;
+        r.N = ns;
+        r.M = in;
+        r.K = out;
+        r.a.row = axis_plain(ns, out);
+        r.a.k = axis_plain(out, 1);
+        r.b.row = axis_plain(in, 1);
+        r.b.k = axis_plain(out, in);
+        r.a.HL = r.a.WL = r.b.HL = r.b.WL = 1;
+        r.c.n = axis_plain(ns, in);
+        r.c.m = axis_plain(in, 1);
+        rc = gemm_pair<T>(q, r);
+        if (rc == 0 && db) {
+            hipLaunchKernelGGL((bias_grad_kernel<T>), dim3(out), dim3(256), 0, state().stream, dY, db, ns, out, 1,
+                               1);
+            if (!hip_ok(hipGetLastError(), "bias grad launch")) rc = 2;
+        }
     } else if (step == STEP_WGT_GRAD) {
         const T *X = sg.in(reinterpret_cast<const T *>(a->input->data), (size_t)ns * in);
         const T *dY = sg.in(reinterpret_cast<const T *>(a->output->diff), (size_t)ns * out);
@@ -813,6 +857,30 @@ int ptl_linear_fp16_fw_batched(const struct Linear_args_fp16 *a, int ns) {
 }
 int ptl_linear_fp16_wg_batched(const struct Linear_args_fp16 *a, int ns) {
     return ptl::linear_step<half_t>(a, ns, STEP_WGT_GRAD, "pulp_linear_fp16_bw_param_grads_cl");
+}
+int ptl_linear_fp32_bw_batched(const struct Linear_args *a, int ns) {
+    if (a && (a->skip_wg_grad || a->skip_in_grad || ns == 1)) {  // one of the two, or one sample: the single steps
+        int rc = a->skip_wg_grad ? 0 : ptl::linear_step<float>(a, ns, STEP_WGT_GRAD, "pulp_linear_fp32_bw_cl");
+        if (rc == 0 && !a->skip_in_grad) rc = ptl::linear_step<float>(a, ns, STEP_IN_GRAD, "pulp_linear_fp32_bw_cl");
+        return rc;
+    }
+    if (ns == 1) {
+        int rc = ptl::linear_step<float>(a, 1, STEP_WGT_GRAD, "pulp_linear_fp32_bw_cl");
+        return rc ? rc : ptl::linear_step<float>(a, 1, STEP_IN_GRAD, "pulp_linear_fp32_bw_cl");
+    }
+    return ptl::linear_step<float>(a, ns, STEP_BW_BOTH, "pulp_linear_fp32_bw_cl");
+}
+int ptl_linear_fp16_bw_batched(const struct Linear_args_fp16 *a, int ns) {
+    if (a && (a->skip_wg_grad || a->skip_in_grad || ns == 1)) {  // one of the two, or one sample: the single steps
+        int rc = a->skip_wg_grad ? 0 : ptl::linear_step<half_t>(a, ns, STEP_WGT_GRAD, "pulp_linear_fp16_bw_cl");
+        if (rc == 0 && !a->skip_in_grad) rc = ptl::linear_step<half_t>(a, ns, STEP_IN_GRAD, "pulp_linear_fp16_bw_cl");
+        return rc;
+    }
+    if (ns == 1) {
+        int rc = ptl::linear_step<half_t>(a, 1, STEP_WGT_GRAD, "pulp_linear_fp16_bw_cl");
+        return rc ? rc : ptl::linear_step<half_t>(a, 1, STEP_IN_GRAD, "pulp_linear_fp16_bw_cl");
+    }
+    return ptl::linear_step<half_t>(a, ns, STEP_BW_BOTH, "pulp_linear_fp16_bw_cl");
 }
 int ptl_linear_fp16_ig_batched(const struct Linear_args_fp16 *a, int ns) {
     return ptl::linear_step<half_t>(a, ns, STEP_IN_GRAD, "pulp_linear_fp16_bw_input_grads_cl");

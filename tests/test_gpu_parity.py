@@ -351,6 +351,40 @@ def test_linear_bias(pkg, orc, gpu, dt):
 
 # ---------------------------------------------------------------------- mm / mm_manager
 @pytest.mark.parametrize("dt", ["fp32", "fp16"])
+@pytest.mark.parametrize("n_in,n_out,ns", [(1024, 1024, 512), (256, 384, 640), (100, 37, 9), (64, 64, 1)])
+def test_linear_bw_batched_matches_separate_steps(pkg, gpu, dt, n_in, n_out, ns):
+    """ptl_linear_*_bw_batched (weight + input gradient in one call) against the two single steps."""
+    nd = hp.np_dtype(dt)
+    x = dev(hp.normal(11, (ns, n_in), 1.0 / 16.0, nd))
+    w = dev(hp.normal(12, (n_out, n_in), 1.0 / 16.0, nd))
+    dy = dev(hp.uniform(13, (ns, n_out), dtype=nd))
+    res = []
+    for both in (False, True):
+        y = torch.zeros(ns, n_out, dtype=x.dtype, device=DEV)
+        dx, dw = torch.full_like(x, 3), torch.full_like(w, 3)
+        a, keep = hp.linear_args(pkg, x, dx, w, dw, y, dy, n_in, n_out)
+        if both:
+            pkg.call("ptl_linear_%s_bw_batched" % dt, a, ns)
+        else:
+            pkg.call("ptl_linear_%s_wg_batched" % dt, a, ns)
+            pkg.call("ptl_linear_%s_ig_batched" % dt, a, ns)
+        sync(gpu)
+        res.append((host(dw), host(dx)))
+    tol = 1e-6 if dt == "fp32" else 2e-3
+    assert rel_l2(res[1][0], res[0][0]) <= tol
+    assert rel_l2(res[1][1], res[0][1]) <= tol
+    # skip flags select one of the two
+    dx, dw = torch.full_like(x, 3), torch.full_like(w, 3)
+    y = torch.zeros(ns, n_out, dtype=x.dtype, device=DEV)
+    a, keep = hp.linear_args(pkg, x, dx, w, dw, y, dy, n_in, n_out)
+    a.skip_in_grad = 1
+    pkg.call("ptl_linear_%s_bw_batched" % dt, a, ns)
+    sync(gpu)
+    assert rel_l2(host(dw), res[0][0]) <= tol
+    assert np.all(host(dx) == 3)
+
+
+@pytest.mark.parametrize("dt", ["fp32", "fp16"])
 @pytest.mark.parametrize("N,M,K", [(32, 32, 32), (32, 1024, 144), (32, 144, 1024), (16, 1024, 288), (128, 3136, 64),
                                    (7, 5, 3), (1, 33, 20), (33, 1, 20), (9, 11, 1), (130, 70, 515)])
 def test_mm_family(pkg, orc, gpu, dt, N, M, K):
