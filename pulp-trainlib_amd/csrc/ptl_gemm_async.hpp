@@ -17,10 +17,10 @@ int launch_async(GemmArgs &g, const void *zero, hipStream_t s);
 // non-negative stride, non-negative row offsets below 2^31 bytes, and a k range
 // made of whole slabs (there is no zero fill on this path).
 // Lean kernel for the case that both operands are plain (plain_operand() != 0).
-template <typename T, int BM, int BN, int NT, int WMv, int WNv, int WKv, int NS>
+template <typename T, int BM, int BN, int NT, int WMv, int WNv, int WKv, int NS, int G>
 int launch_plain(GemmArgs &g, hipStream_t s);
 
-template <typename T, int BM, int BN, int NT, int WMv, int WNv, int WKv, int NS>
+template <typename T, int BM, int BN, int NT, int WMv, int WNv, int WKv, int NS, int G>
 int launch_plain_pair(GemmArgs &g0, GemmArgs &g1, hipStream_t s);
 
 template <typename T>

@@ -56,10 +56,12 @@ int gemm_async(GemmArgs &g) {
     }
     if (plain_operand<T>(g.a, g.kchunk, g.K) && plain_operand<T>(g.b, g.kchunk, g.K)) {
         switch (cfg) {
-            case 0: return launch_plain<T, 128, 128, 512, 2, 2, 2, 3>(g, st.stream);
-            case 1: return launch_plain<T, 64, 64, 1024, 2, 2, 4, 3>(g, st.stream);
-            case 2: return launch_plain<T, 32, 128, 512, 1, 4, 2, 3>(g, st.stream);
-            default: return launch_plain<T, 128, 32, 512, 4, 1, 2, 3>(g, st.stream);
+            case 0: return launch_plain<T, 128, 128, 512, 2, 2, 2, 3, 1>(g, st.stream);
+            case 1:  // small tile: two slabs per wait-and-barrier when the slab count is even
+                if (g.splits == 1 && (g.K / SK) % 2 == 0 && g.K >= 4 * SK) return launch_plain<T, 64, 64, 1024, 2, 2, 4, 3, 2>(g, st.stream);
+                return launch_plain<T, 64, 64, 1024, 2, 2, 4, 3, 1>(g, st.stream);
+            case 2: return launch_plain<T, 32, 128, 512, 1, 4, 2, 3, 1>(g, st.stream);
+            default: return launch_plain<T, 128, 32, 512, 4, 1, 2, 3, 1>(g, st.stream);
         }
     }
     int rc = -1;
@@ -93,8 +95,8 @@ int gemm_async_pair(GemmArgs &g0, GemmArgs &g1) {
         if (cfg[i] == 1 && tiles(64, 64) * 4 <= st.num_cu) return -1;  // would want a k split
     }
     if (cfg[0] != cfg[1]) return -1;
-    if (cfg[0] == 0) return launch_plain_pair<T, 128, 128, 512, 2, 2, 2, 3>(g0, g1, st.stream);
-    return launch_plain_pair<T, 64, 64, 1024, 2, 2, 4, 3>(g0, g1, st.stream);
+    if (cfg[0] == 0) return launch_plain_pair<T, 128, 128, 512, 2, 2, 2, 3, 1>(g0, g1, st.stream);
+    return launch_plain_pair<T, 64, 64, 1024, 2, 2, 4, 3, 1>(g0, g1, st.stream);
 }
 
 template int gemm_async_pair<float>(GemmArgs &, GemmArgs &);

@@ -3,10 +3,11 @@
 #include "ptl_gemm_plain.inc"
 
 namespace ptl {
-template int launch_plain<float, 128, 128, 512, 2, 2, 2, 3>(GemmArgs &, hipStream_t);
-template int launch_plain<float, 64, 64, 1024, 2, 2, 4, 3>(GemmArgs &, hipStream_t);
-template int launch_plain<float, 32, 128, 512, 1, 4, 2, 3>(GemmArgs &, hipStream_t);
-template int launch_plain<float, 128, 32, 512, 4, 1, 2, 3>(GemmArgs &, hipStream_t);
-template int launch_plain_pair<float, 128, 128, 512, 2, 2, 2, 3>(GemmArgs &, GemmArgs &, hipStream_t);
-template int launch_plain_pair<float, 64, 64, 1024, 2, 2, 4, 3>(GemmArgs &, GemmArgs &, hipStream_t);
+template int launch_plain<float, 128, 128, 512, 2, 2, 2, 3, 1>(GemmArgs &, hipStream_t);
+template int launch_plain<float, 64, 64, 1024, 2, 2, 4, 3, 1>(GemmArgs &, hipStream_t);
+template int launch_plain<float, 32, 128, 512, 1, 4, 2, 3, 1>(GemmArgs &, hipStream_t);
+template int launch_plain<float, 128, 32, 512, 4, 1, 2, 3, 1>(GemmArgs &, hipStream_t);
+template int launch_plain_pair<float, 128, 128, 512, 2, 2, 2, 3, 1>(GemmArgs &, GemmArgs &, hipStream_t);
+template int launch_plain_pair<float, 64, 64, 1024, 2, 2, 4, 3, 1>(GemmArgs &, GemmArgs &, hipStream_t);
+template int launch_plain<float, 64, 64, 1024, 2, 2, 4, 3, 2>(GemmArgs &, hipStream_t);
 }
