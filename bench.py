@@ -145,7 +145,11 @@ def main():
         "config": {"workload": "linear_1024x1024_fp16_FW+WG+IG_batched_N%d" % ns, "in": n_in, "out": n_out,
                    "batch": ns, "accumulate": "f32", "layout": "W[out][in], X[batch][in]"},
         "roofline": {"bound": "mfma", "achieved": round(achieved, 3), "peak": PEAK["fp16"], "unit": "TFLOP/s",
-                     "frac": round(achieved / PEAK["fp16"], 5), "traffic": None,
+                     "frac": round(achieved / PEAK["fp16"], 5),
+                     # HBM bytes per launch (mean of the two launches of a step) from the FETCH_SIZE and
+                     # WRITE_SIZE runs summarised in profiles/gemm_plain_f16_linear1024_N512.md; it holds for
+                     # the default batch only
+                     "traffic": 13.3e6 if ns == 512 else None,
                      "kernel": "ptl::gemm_plain_kernel / gemm_plain_pair_kernel<_Float16, 64x64 tile, 1024 threads>",
                      "flops_per_launch": flops_step / 2, "launches_per_step": 2,
                      "avg_launch_us": round(launch_ms * 1e3, 3)},
