@@ -188,11 +188,12 @@ def main():
         cpu_step(2)
         t_probe = cpu_step(4) / 4
         m = int(max(4, min(ns, 12.0 / max(t_probe, 1e-6))))
-        t_cpu = cpu_step(m)
-        cpu_tflops = 3 * 2.0 * m * n_in * n_out / t_cpu / 1e12
+        reps = int(max(1, min(50, round(10.0 / max(t_probe * m, 1e-6)))))  # about 10 s of CPU work
+        t_cpu = sum(cpu_step(m) for _ in range(reps))
+        cpu_tflops = reps * 3 * 2.0 * m * n_in * n_out / t_cpu / 1e12
         result["cpu_baseline"] = {"value": round(cpu_tflops, 6), "unit": "TFLOP/s", "cores": cores, "kind": "port",
-                                  "sample": "%d of the %d samples, FW+WG+IG once, fp16 with fp16 accumulation "
-                                            "(the reference's arithmetic), %.2f s" % (m, ns, t_cpu)}
+                                  "sample": "%d of the %d samples, FW+WG+IG %d times, fp16 with fp16 accumulation "
+                                            "(the reference's arithmetic), %.2f s" % (m, ns, reps, t_cpu)}
 
     # ------------------------------------------------------------------------------ detail
     if not args.no_detail:
