@@ -57,7 +57,14 @@ int gemm_async(GemmArgs &g) {
     if (plain_operand<T>(g.a, g.kchunk, g.K) && plain_operand<T>(g.b, g.kchunk, g.K)) {
         switch (cfg) {
             case 0: return launch_plain<T, 128, 128, 512, 2, 2, 2, 3, 1>(g, st.stream);
-            case 1:  // small tile: two slabs per wait-and-barrier when the slab count is even
+            case 1:
+                // fp32 MFMAs are slow enough to matter at this size: when 64x64 tiles leave half the CUs
+                // idle, 64x32 tiles put a workgroup on every CU
+                if constexpr (sizeof(T) == 4) {
+                    if (g.splits == 1 && tiles(64, 64) * 2 <= st.num_cu && g.M % 32 == 0)
+                        return launch_plain<T, 64, 32, 512, 2, 1, 4, 3, 1>(g, st.stream);
+                }
+                // small tile: two slabs per wait-and-barrier when the slab count is even
                 if (g.splits == 1 && (g.K / SK) % 2 == 0 && g.K >= 4 * SK) return launch_plain<T, 64, 64, 1024, 2, 2, 4, 3, 2>(g, st.stream);
                 return launch_plain<T, 64, 64, 1024, 2, 2, 4, 3, 1>(g, st.stream);
             case 2: return launch_plain<T, 32, 128, 512, 1, 4, 2, 3, 1>(g, st.stream);
