@@ -8,10 +8,11 @@
 // output channels, and
 //   * gets the input rows those pixels touch ONCE into LDS, as [channel block][row][col]
 //     chunks of 16 bytes that hold VEC consecutive channels of one input position, the
-//     padding halo as zeros (raw tile).  A first kernel re-lays the channel-major input in
-//     exactly these chunks ([sample][channel block][row][col]), so the raw tile is filled
-//     by LDS-DMA: one 16-byte lane-load per chunk, halo chunks read a zero buffer, nothing
-//     passes through registers;
+//     padding halo as zeros (raw tile).  Where input rows are whole aligned 16-byte groups
+//     (the usual case) the rows come in pixel-major by LDS-DMA straight from the tensor into
+//     a staging buffer and are re-laid LDS to LDS; otherwise a first kernel re-lays the whole
+//     input in exactly these chunks ([sample][channel block][row][col]) and the raw tile is
+//     filled by LDS-DMA from that copy (halo chunks read a zero buffer);
 //   * loads its BN filters into LDS as [filter][tap][channel] (rows padded to an odd
 //     multiple of 16 bytes, which spreads sixteen consecutive filters over all 64 banks),
 //     once per workgroup: a workgroup then walks several pixel tiles;
@@ -47,28 +48,34 @@ struct ConvTileArgs {
     int nfast;         // 1: the output's pixel axis is (sample, pixel-in-sample) with the sample size as radix
     unsigned magic_pp, magic_wo, magic_thp;
     int raw_chunks;    // chunks of one raw slab (two channel blocks) rounded up to whole waves
+    int stage_chunks;  // chunks of one staging slab (KSTEP channels x RR rows x whole input rows), whole waves
+    int xg;            // 16-byte groups per input row
+    unsigned magic_xg, magic_rrxg;
     unsigned magic_tw, magic_rr, magic_perm, magic_cb, magic_kw;  // ceil(2^32 / d): exact for n, d < 2^16
     int c_mode;
 };
 
 
-template <typename T, int BM, int BN, int WAVES_K>
-__global__ __launch_bounds__((BM / 32) * WAVES_K * 64) void conv_tile_kernel(const ConvTileArgs a) {
-    constexpr int NT = (BM / 32) * WAVES_K * 64;
+template <typename T, int BM, int BN, bool STAGED>
+__global__ __launch_bounds__((BM / 32) * 64) void conv_tile_kernel(const ConvTileArgs a) {
+    constexpr int NT = (BM / 32) * 64;
     constexpr int ES = (int)sizeof(T), VEC = 16 / ES, KSTEP = 2 * VEC, FN = BN / 32;
     extern __shared__ __attribute__((aligned(16))) char smem[];
     char *bl = smem;                                          // filters [BN][b_pitch]
-    uint4 *raw = reinterpret_cast<uint4 *>(smem + a.b_bytes);  // two raw tiles [channel block][row][col] of VEC channels
+    // raw slab(s) [channel block][row][col] of VEC channels: two when they are filled from the
+    // blocked copy of the input, one when they are built from the staging buffers that follow
+    uint4 *raw = reinterpret_cast<uint4 *>(smem + a.b_bytes);
+    T *stage = reinterpret_cast<T *>(raw + a.raw_chunks);  // STAGED: two pixel-major slabs [channel][row][col]
     __shared__ int mlut[BN];      // per filter: output offset
 
     const ConvTileDesc &d = a.d;
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    static_assert(WAVES_K == 1, "one wave per 32 pixels");
     const int wm = wave;
     const int m0 = blockIdx.y * BN;
     const int PP = d.Ho * d.Wo;
-    const uint4 *__restrict__ Xb = reinterpret_cast<const uint4 *>(a.X);  // blocked input
+    const uint4 *__restrict__ Xb = reinterpret_cast<const uint4 *>(a.X);  // blocked input (not STAGED)
+    const T *__restrict__ X = reinterpret_cast<const T *>(a.X);           // channel-major input (STAGED)
     const T *__restrict__ Wt = reinterpret_cast<const T *>(a.Wt);
     const int kg = lane >> 5, lr = lane & 31;
     const int cblocks = a.CinP / VEC;
@@ -82,10 +89,28 @@ __global__ __launch_bounds__((BM / 32) * WAVES_K * 64) void conv_tile_kernel(con
     // derives its own addresses.
     const unsigned raw_lds = (unsigned)(uintptr_t)(lds_char *)raw;
     const int plane_in = d.Hin * d.Win;
+    const unsigned stage_lds = (unsigned)(uintptr_t)(lds_char *)stage;
     auto enqueue = [&](int tile, int cs, int buf) {
         const int n0 = tile * BM;
         const int b0 = n0 / PP, y0 = (n0 - b0 * PP) / d.Wo;
         const int t0 = y0 * d.sh;  // first raw row, counted inside the padded image of sample b0
+        if (STAGED) {
+            // pixel-major staging slab straight from the tensor: chunk c = (channel * RR + row) * XG + group of
+            // VEC columns; rows outside the image and channels beyond the tensor read the zero buffer
+            const int rrxg = a.RR * a.xg;
+            for (int c0 = wave * 64; c0 < a.stage_chunks; c0 += NT) {
+                const int c = c0 + lane;
+                const int ch = fast_div(c, a.magic_rrxg), r = c - ch * rrxg;
+                const int rr = fast_div(r, a.magic_xg), xg = r - rr * a.xg;
+                const int t = t0 + rr, db = fast_div(t, a.magic_thp);
+                const int b = b0 + db, iy = t - db * a.THP - d.padU, chn = cs * KSTEP + ch;
+                const bool ok = ch < KSTEP && chn < d.Cin && b < d.batch && iy >= 0 && iy < d.Hin;
+                const int idx = b * (int)d.x_sb + chn * (int)d.x_sc + iy * d.Win + xg * VEC;
+                const char *src = ok ? reinterpret_cast<const char *>(X + idx) : reinterpret_cast<const char *>(a.zero);
+                lds_dma<16>(src, stage_lds + (unsigned)(buf * a.stage_chunks + c0) * 16u);
+            }
+            return;
+        }
         for (int c0 = wave * 64; c0 < a.raw_chunks; c0 += NT) {
             const int c = c0 + lane;
             const int row = fast_div(c, a.magic_tw), tx = c - row * a.TW;
@@ -97,6 +122,29 @@ __global__ __launch_bounds__((BM / 32) * WAVES_K * 64) void conv_tile_kernel(con
             const char *src = ok ? reinterpret_cast<const char *>(Xb + (((b * cblocks + cb) * d.Hin + iy) * d.Win + ix))
                                  : reinterpret_cast<const char *>(a.zero);
             lds_dma<16>(src, raw_lds + (unsigned)(buf * a.raw_chunks + c0) * 16u);
+        }
+    };
+    // STAGED: staging slab -> raw slab.  One thread per chunk gathers the VEC channels of an input
+    // position (consecutive lanes read consecutive columns) and writes them as 16 bytes; halo
+    // columns become zeros.
+    auto transpose = [&](int sbuf) {
+        const T *sp = stage + (size_t)sbuf * a.stage_chunks * VEC;
+        const int rw = a.RR * d.Win;
+        for (int c = tid; c < 2 * a.PLANE; c += NT) {
+            const int row = fast_div(c, a.magic_tw), tx = c - row * a.TW;
+            const int half = fast_div(row, a.magic_rr), rr = row - half * a.RR;
+            const int ix = tx - d.padL;
+            union {
+                uint4 v;
+                T e[VEC];
+            } u;
+            u.v = make_uint4(0, 0, 0, 0);
+            if (ix >= 0 && ix < d.Win) {
+                const T *q = sp + (half * VEC) * rw + rr * d.Win + ix;
+#pragma unroll
+                for (int e = 0; e < VEC; ++e) u.e[e] = q[e * rw];
+            }
+            raw[c] = u.v;
         }
     };
 
@@ -182,11 +230,15 @@ __global__ __launch_bounds__((BM / 32) * WAVES_K * 64) void conv_tile_kernel(con
             else if (tile + (int)gridDim.x < a.tiles)
                 enqueue(tile + gridDim.x, 0, buf ^ 1);
             if (cs == 0) flush();  // the previous tile's results
+            if (STAGED) {
+                transpose(buf);
+                __syncthreads();
+            }
 
             // Contraction, tap by tap.  Filters are the MFMA rows, pixels the columns: a lane ends
             // up with 16 filters of ONE pixel per block, so the 32 lanes of a half-wave store 32
             // consecutive pixels of a filter.
-            const uint4 *prow = raw + buf * a.raw_chunks + corner + kg * a.PLANE;
+            const uint4 *prow = raw + (STAGED ? 0 : buf * a.raw_chunks) + corner + kg * a.PLANE;
             const char *frow = bl + lr * a.b_pitch + (cs * KSTEP + kg * VEC) * ES;
             for (int ky = 0; ky < d.KH; ++ky)
                 for (int kx = 0; kx < d.KW; ++kx) {
@@ -235,10 +287,10 @@ __global__ __launch_bounds__(256) void chw_to_blocked_kernel(const T *__restrict
     out[i] = u.v;
 }
 
-template <typename T, int BM, int BN, int WAVES_K>
+template <typename T, int BM, int BN, bool STAGED>
 static int launch_conv_tile(ConvTileArgs &a, size_t lds, hipStream_t s) {
-    constexpr int NT = (BM / 32) * WAVES_K * 64;
-    auto kern = conv_tile_kernel<T, BM, BN, WAVES_K>;
+    constexpr int NT = (BM / 32) * 64;
+    auto kern = conv_tile_kernel<T, BM, BN, STAGED>;
     static bool attr_set = false;
     if (!attr_set) {
         if (!hip_ok(hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
@@ -302,6 +354,22 @@ int conv_tile(const ConvTileDesc &d, const void *X, const void *Wt, void *Y, con
     if ((pitch16 & 1) == 0) ++pitch16;
     a.b_pitch = pitch16 * 16;
 
+    // Staged route: the kernel copies pixel-major rows straight from the tensor and re-lays them in
+    // LDS; it needs rows that are whole, aligned 16-byte groups.  Otherwise a first kernel writes
+    // a blocked copy of the whole input.
+    a.xg = d.Win / VEC;
+    a.stage_chunks = (KSTEP * a.RR * a.xg + 63) & ~63;
+    // It pays while slabs are small (one more barrier and an LDS-to-LDS pass per slab, and three
+    // slab buffers instead of two: measured 12 against 15 us on 32x32 images with 16 channels,
+    // 189 against 104 us on 56x56 with 32), so it is taken when a workgroup's slabs stay
+    // below 40 KB.
+    const bool staged = d.Win % VEC == 0 && d.x_sc % VEC == 0 && d.x_sb % VEC == 0 &&
+                        reinterpret_cast<uintptr_t>(X) % 16 == 0 && a.stage_chunks < 65536 &&
+                        (long long)d.batch * d.x_sb < ((long long)1 << 31) &&
+                        ((size_t)a.raw_chunks + 2 * (size_t)a.stage_chunks) * 16 <= 40 * 1024;
+    a.magic_xg = magic_of(a.xg);
+    a.magic_rrxg = magic_of(a.RR * a.xg);
+
     // Filters per workgroup: the narrowest of 32/64/128 that covers them (or 128 with several
     // column tiles), halved while the filter tile does not fit LDS (more column tiles, each
     // re-reading the pixels).  The kernel pays a per-workgroup price for its filter tile, so it
@@ -309,7 +377,9 @@ int conv_tile(const ConvTileDesc &d, const void *X, const void *Wt, void *Y, con
     int bn = d.Cout <= 32 ? 32 : d.Cout <= 64 ? 64 : 128;
     size_t lds = 0;
     for (;; bn /= 2) {
-        lds = (size_t)bn * a.b_pitch + 2 * (size_t)a.raw_chunks * 16;  // filters + two raw buffers
+        // filters + (one raw slab and two staging slabs | two raw slabs)
+        lds = (size_t)bn * a.b_pitch +
+              (staged ? (size_t)a.raw_chunks * 16 + 2 * (size_t)a.stage_chunks * 16 : 2 * (size_t)a.raw_chunks * 16);
         if (lds <= 150 * 1024 && (long)bn * d.KH * d.KW * cblocks < 65536) break;
         if (bn == 32) return -1;
     }
@@ -329,6 +399,12 @@ int conv_tile(const ConvTileDesc &d, const void *X, const void *Wt, void *Y, con
     if (a.THP + a.RR >= 65536) return -1;
     a.nfast = (c.n.d0 == PP && c.n.d1 >= (1 << 30)) ? 1 : 0;
 
+    if (staged) {
+        a.X = X;
+        if (bn == 128) return launch_conv_tile<T, BM, 128, true>(a, lds, st.stream);
+        if (bn == 64) return launch_conv_tile<T, BM, 64, true>(a, lds, st.stream);
+        return launch_conv_tile<T, BM, 32, true>(a, lds, st.stream);
+    }
     // re-lay the input in chunks of VEC channels
     uint4 *xb = reinterpret_cast<uint4 *>(workspace((size_t)in_chunks * 16));
     if (!xb) return 2;
@@ -336,9 +412,9 @@ int conv_tile(const ConvTileDesc &d, const void *X, const void *Wt, void *Y, con
                        reinterpret_cast<const T *>(X), xb, d.Cin, cblocks, d.Hin * d.Win, d.x_sb, d.x_sc, in_chunks);
     if (!hip_ok(hipGetLastError(), "blocked layout launch")) return 2;
     a.X = xb;
-    if (bn == 128) return launch_conv_tile<T, BM, 128, 1>(a, lds, st.stream);
-    if (bn == 64) return launch_conv_tile<T, BM, 64, 1>(a, lds, st.stream);
-    return launch_conv_tile<T, BM, 32, 1>(a, lds, st.stream);
+    if (bn == 128) return launch_conv_tile<T, BM, 128, false>(a, lds, st.stream);
+    if (bn == 64) return launch_conv_tile<T, BM, 64, false>(a, lds, st.stream);
+    return launch_conv_tile<T, BM, 32, false>(a, lds, st.stream);
 }
 
 template int conv_tile<float>(const ConvTileDesc &, const void *, const void *, void *, const OutMap &);
