@@ -340,12 +340,9 @@ int conv_tile(const ConvTileDesc &d, const void *X, const void *Wt, void *Y, con
     const long long in_chunks = (long long)d.batch * cblocks * d.Hin * d.Win;
     if (in_chunks >= ((long long)1 << 31)) return -1;
 
-    // Raw rows of a tile: the output rows it spans, the image seams inside it, plus the filter height.
+    // Raw rows of a tile: the output rows it spans (image seams included) plus the filter height.
     const int PP = d.Ho * d.Wo;
-    const int rows_spanned = (BM - 1 + d.Wo - 1) / d.Wo + 1;
-    const int seams = (BM - 1 + PP - 1) / PP;
-    const int seam_rows = a.THP - d.Ho * d.sh > 0 ? a.THP - d.Ho * d.sh : 0;
-    a.RR = (rows_spanned - 1) * d.sh + seams * seam_rows + d.KH;
+    a.RR = conv_raw_rows(BM, d.Ho, d.Wo, d.sh, d.KH, a.THP, a.g.N);
     if (a.RR > 64) return -1;
     a.PLANE = a.RR * a.TW;
     a.raw_chunks = (2 * a.PLANE + 63) & ~63;  // one slab: two channel blocks

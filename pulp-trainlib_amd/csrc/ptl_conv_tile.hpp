@@ -34,6 +34,37 @@ inline unsigned magic_of(int dv) { return dv <= 1 ? 0u : (unsigned)((((unsigned 
 __device__ inline int fast_div(int n, unsigned magic) { return magic ? (int)__umulhi((unsigned)n, magic) : n; }
 #endif
 
+// Raw input rows (counted over padded images laid end to end) that a tile of `bm` consecutive
+// output pixels touches, maximised over all tiles: exact, from one period of the tile / image
+// pattern, remembered for the last geometry asked.
+inline int conv_raw_rows(int bm, int Ho, int Wo, int sh, int KH, int THP, long long npix) {
+    static int key[6] = {0, 0, 0, 0, 0, 0}, val = 0;
+    static long long key_n = 0;
+    if (key[0] == bm && key[1] == Ho && key[2] == Wo && key[3] == sh && key[4] == KH && key[5] == THP && key_n == npix)
+        return val;
+    const long long PP = (long long)Ho * Wo;
+    long long a = PP, b = bm;
+    while (b) {
+        long long t = a % b;
+        a = b;
+        b = t;
+    }
+    long long period_tiles = PP / a;  // tiles until the (tile start mod image) pattern repeats
+    const long long tiles = (npix + bm - 1) / bm;
+    if (period_tiles > tiles) period_tiles = tiles;
+    int best = 0;
+    for (long long t = 0; t < period_tiles; ++t) {
+        const long long p0 = t * bm, p1 = (p0 + bm - 1 < npix - 1) ? p0 + bm - 1 : npix - 1;
+        const long long g0 = (p0 / PP) * THP + ((p0 % PP) / Wo) * sh, g1 = (p1 / PP) * THP + ((p1 % PP) / Wo) * sh;
+        if ((int)(g1 - g0) > best) best = (int)(g1 - g0);
+    }
+    // the last tile of the tensor may be cut short; it never needs more than a full one
+    val = best + KH;
+    key[0] = bm; key[1] = Ho; key[2] = Wo; key[3] = sh; key[4] = KH; key[5] = THP;
+    key_n = npix;
+    return val;
+}
+
 // Weight gradient of the same convolution:
 //   dW(co, ci, ky, kx) = sum_{b, y, x} dY(b, co, y, x) * in(b, ci, y*sh + ky - padU, x*sw + kx - padL)
 // with dY channel-major [b][Cout][Ho*Wo] and dW dense [Cout][Cin][KH][KW].  Returns 0, a positive

@@ -261,11 +261,8 @@ int conv_tile_wg(const ConvTileDesc &d, const void *X, const void *dY, void *dW)
     a.tiles = (a.N + 127) / 128;
     if (st.gemm_path != 2 && a.tiles < st.num_cu) return -1;
 
-    const int PP = d.Ho * d.Wo, taps = d.KH * d.KW;
-    const int rows_spanned = (127 + d.Wo - 1) / d.Wo + 1;
-    const int seams = (127 + PP - 1) / PP;
-    const int seam_rows = a.THP - d.Ho * d.sh > 0 ? a.THP - d.Ho * d.sh : 0;
-    a.RR = (rows_spanned - 1) * d.sh + seams * seam_rows + d.KH;
+    const int taps = d.KH * d.KW;
+    a.RR = conv_raw_rows(128, d.Ho, d.Wo, d.sh, d.KH, a.THP, a.N);
     if (a.RR > 64) return -1;
     a.PLANE = a.RR * a.TW;
     a.CT = d.Cin <= 16 ? 16 : 32;
