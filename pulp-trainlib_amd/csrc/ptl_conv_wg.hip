@@ -7,7 +7,9 @@
 //   * copies the dY rows of its output channels into LDS ([co][pixel], 16-byte loads);
 //   * copies the input rows the tile touches into LDS as [ci][row][col] with a zero halo,
 //     16 bytes at a time (the halo makes the destination 2-byte aligned only; LDS takes
-//     unaligned 16-byte stores and loads);
+//     unaligned 16-byte stores and loads).  Both copies are register-staged prefetches: the
+//     loads of tile t+1 are issued before tile t is computed and parked in the other of two
+//     LDS buffers afterwards, one barrier per tile;
 //   * feeds the MFMAs: the dY fragment of a lane is one aligned ds_read_b128 (8 pixels of one
 //     output channel), the input fragment one unaligned ds_read_b128 at
 //     coloff(ci, tap) + pixoff(pixel group) -- 8 consecutive pixels of a row shifted by the
@@ -38,7 +40,7 @@ struct ConvWgArgs {
     int raw_bytes;
     int cblocks;  // 32-wide column blocks of (ci, tap) per workgroup
     int xg;       // 16-byte groups per input row
-    unsigned magic_xg, magic_rr, magic_taps, magic_kw;
+    unsigned magic_xg, magic_rr, magic_taps, magic_kw, magic_thp;
 };
 
 template <typename T, int RB, int CBW>
@@ -46,10 +48,9 @@ __global__ __launch_bounds__(512) void conv_wg_kernel(const ConvWgArgs a) {
     constexpr int NT = 512, KT = 128;
     constexpr int ES = (int)sizeof(T), VEC = 16 / ES, KSTEP = 2 * VEC, KSTEPS = KT / KSTEP, GROUPS = KT / VEC;
     extern __shared__ __attribute__((aligned(16))) char smem[];
-    char *at = smem;                                    // dY tile [32*RB][pitch_a]
-    T *raw = reinterpret_cast<T *>(smem + a.a_bytes);   // input tile [CT][RR][TW]
-    __shared__ int2 rowinfo[64];                        // per raw row: element offset in X, valid flag
-    __shared__ int pixoff[GROUPS];                      // per pixel group: raw offset of its first pixel
+    // two buffers, each: dY tile [32*RB][pitch_a] followed by the input tile [CT][RR][TW]
+    const int buf_bytes = a.a_bytes + a.raw_bytes;
+    __shared__ int pixoff[2][GROUPS];  // per pixel group: raw offset of its first pixel
 
     const ConvTileDesc &d = a.d;
     const int tid = threadIdx.x, lane = tid & 63;
@@ -81,61 +82,95 @@ __global__ __launch_bounds__(512) void conv_wg_kernel(const ConvWgArgs a) {
 #pragma unroll
             for (int v = 0; v < 16; ++v) acc[r][jj][v] = 0.f;
 
-    for (int tile = blockIdx.x; tile < a.tiles; tile += gridDim.x) {
+    // Both input tiles start as zeros: the halo columns are never written again, everything
+    // else is rewritten for every tile (rows outside the image and channels beyond the tensor
+    // as zeros).
+    for (int b = 0; b < 2; ++b)
+        for (int c = tid; c < a.raw_bytes / 16; c += NT)
+            reinterpret_cast<uint4 *>(smem + b * buf_bytes + a.a_bytes)[c] = make_uint4(0, 0, 0, 0);
+    __syncthreads();
+
+    // Register-staged prefetch: the global loads of tile t+1 are issued before tile t is
+    // computed and stored to the other LDS buffer afterwards; one barrier per tile.
+    constexpr int A_CHUNKS = 32 * RB * (KT / VEC);
+    constexpr int A_PER = (A_CHUNKS + NT - 1) / NT;  // dY chunks per thread
+    const int units = a.CT * a.RR * a.xg;            // (ci, raw row, group of VEC columns)
+    constexpr int U_MAX = 4;                         // input units per thread the registers hold (host checks)
+    uint4 regA[A_PER], regU[U_MAX];
+
+    auto fetch = [&](int tile) {
         const int n0 = tile * KT;
         const int b0 = n0 / PP, pix0 = n0 - b0 * PP, y0 = pix0 / d.Wo;
-        const int g0 = b0 * a.THP + y0 * d.sh;
-        __syncthreads();  // the previous tile's reads are done
-        if (tid < a.RR) {
-            const int gr = g0 + tid, b = gr / a.THP, iy = gr - b * a.THP - d.padU;
-            int2 e;
-            e.y = (b < d.batch && iy >= 0 && iy < d.Hin) ? 1 : 0;
-            e.x = e.y ? (int)((long long)b * d.x_sb + (long long)iy * d.x_sy) : 0;
-            rowinfo[tid] = e;
-        }
-        if (tid >= 64 && tid < 64 + GROUPS) {
-            const int g = tid - 64;
-            int p = n0 + g * VEC, off = 0;
-            if (p < a.N) {
-                const int b = p / PP, rem = p - b * PP, y = rem / d.Wo, x = rem - y * d.Wo;
-                off = (b * a.THP + y * d.sh - g0) * a.TW + x;
-            }
-            pixoff[g] = off;
-        }
-        // zero the raw tile (halo, rows outside the image, channels beyond the tensor)
-        for (int c = tid; c < a.raw_bytes / 16; c += NT) reinterpret_cast<uint4 *>(raw)[c] = make_uint4(0, 0, 0, 0);
-        // dY tile: chunk (row, pixel group); pixels beyond the tensor are zeros
-        for (int c = tid; c < 32 * RB * (KT / VEC); c += NT) {
+        const int t0 = y0 * d.sh;
+#pragma unroll
+        for (int i = 0; i < A_PER; ++i) {
+            const int c = tid + i * NT;
             const int row = c / (KT / VEC), g = c % (KT / VEC);
             int q = pix0 + g * VEC, b = b0;
             while (q >= PP) {
                 q -= PP;
                 ++b;
             }
-            uint4 v = make_uint4(0, 0, 0, 0);
-            if (n0 + g * VEC < a.N && r0 + row < d.Cout)
-                v = *reinterpret_cast<const uint4 *>(dY + ((long long)b * d.Cout + r0 + row) * PP + q);
-            *reinterpret_cast<uint4 *>(at + row * a.pitch_a + g * 16) = v;
+            regA[i] = make_uint4(0, 0, 0, 0);
+            if (c < A_CHUNKS && n0 + g * VEC < a.N && r0 + row < d.Cout)
+                regA[i] = *reinterpret_cast<const uint4 *>(dY + ((long long)b * d.Cout + r0 + row) * PP + q);
         }
-        __syncthreads();
-        // input rows: unit (ci, rr, group of VEC columns)
-        {
-            const int units = a.CT * a.RR * a.xg;
-            for (int u = tid; u < units; u += NT) {
+#pragma unroll
+        for (int i = 0; i < U_MAX; ++i) {
+            const int u = tid + i * NT;
+            regU[i] = make_uint4(0, 0, 0, 0);
+            if (u < units) {
                 const int row = fast_div(u, a.magic_xg), xg = u - row * a.xg;
                 const int ci = fast_div(row, a.magic_rr), rr = row - ci * a.RR;
-                const int2 ri = rowinfo[rr];
-                if (ri.y && c0 + ci < d.Cin) {
-                    const uint4 v = *reinterpret_cast<const uint4 *>(X + (long long)(c0 + ci) * d.x_sc + ri.x + xg * VEC);
-                    u4raw w = {v.x, v.y, v.z, v.w};
-                    *reinterpret_cast<u4_unaligned *>(raw + ci * a.PLANE + rr * a.TW + d.padL + xg * VEC) = w;
-                }
+                const int t = t0 + rr, db = fast_div(t, a.magic_thp);
+                const int b = b0 + db, iy = t - db * a.THP - d.padU;
+                if (b < d.batch && iy >= 0 && iy < d.Hin && c0 + ci < d.Cin)
+                    regU[i] = *reinterpret_cast<const uint4 *>(X + (long long)b * d.x_sb + (long long)(c0 + ci) * d.x_sc +
+                                                               (long long)iy * d.x_sy + xg * VEC);
             }
         }
-        __syncthreads();
+    };
+    auto park = [&](int tile, int buf) {
+        char *at = smem + buf * buf_bytes;
+        T *raw = reinterpret_cast<T *>(at + a.a_bytes);
+#pragma unroll
+        for (int i = 0; i < A_PER; ++i) {
+            const int c = tid + i * NT;
+            if (c < A_CHUNKS) *reinterpret_cast<uint4 *>(at + (c / (KT / VEC)) * a.pitch_a + (c % (KT / VEC)) * 16) = regA[i];
+        }
+#pragma unroll
+        for (int i = 0; i < U_MAX; ++i) {
+            const int u = tid + i * NT;
+            if (u < units) {
+                const int row = fast_div(u, a.magic_xg), xg = u - row * a.xg;
+                const int ci = fast_div(row, a.magic_rr), rr = row - ci * a.RR;
+                u4raw w = {regU[i].x, regU[i].y, regU[i].z, regU[i].w};
+                *reinterpret_cast<u4_unaligned *>(raw + ci * a.PLANE + rr * a.TW + d.padL + xg * VEC) = w;
+            }
+        }
+        if (tid < GROUPS) {
+            const int n0 = tile * KT;
+            const int b0 = n0 / PP, y0 = (n0 - b0 * PP) / d.Wo;
+            const int g0 = b0 * a.THP + y0 * d.sh;
+            int p = n0 + tid * VEC, off = 0;
+            if (p < a.N) {
+                const int b = p / PP, rem = p - b * PP, y = rem / d.Wo, x = rem - y * d.Wo;
+                off = (b * a.THP + y * d.sh - g0) * a.TW + x;
+            }
+            pixoff[buf][tid] = off;
+        }
+    };
 
+    int buf = 0;
+    if ((int)blockIdx.x < a.tiles) fetch(blockIdx.x);
+    for (int tile = blockIdx.x; tile < a.tiles; tile += gridDim.x, buf ^= 1) {
+        park(tile, buf);
+        __syncthreads();  // tile parked; every wave is done with the tile before the previous one (same buffer)
+        if (tile + (int)gridDim.x < a.tiles) fetch(tile + gridDim.x);
+        const char *at = smem + buf * buf_bytes;
+        const T *raw = reinterpret_cast<const T *>(at + a.a_bytes);
         for (int ks = wk; ks < KSTEPS; ks += 2) {
-            const int po = pixoff[ks * 2 + kg];
+            const int po = pixoff[buf][ks * 2 + kg];
             uint4 af[RB];
 #pragma unroll
             for (int r = 0; r < RB; ++r)
@@ -212,7 +247,8 @@ static int launch_conv_wg(ConvWgArgs &a, int gy, int gz, void *dW, hipStream_t s
     a.a_bytes = 32 * RB * a.pitch_a;
     a.raw_bytes = (int)((((size_t)a.CT * a.PLANE * ES + 32) + 15) & ~(size_t)15);  // slack: a fragment may start at the last element
     const size_t red = (size_t)4 * RB * CBW * 16 * 64 * 4;
-    size_t lds = (size_t)a.a_bytes + a.raw_bytes;
+    if ((long)a.CT * a.RR * a.xg > 4L * 512) return -1;  // input units per thread that the prefetch registers hold
+    size_t lds = 2 * ((size_t)a.a_bytes + a.raw_bytes);
     if (lds < red) lds = red;
     if (lds > 150 * 1024) return -1;
     static bool attr_set = false;
@@ -273,6 +309,8 @@ int conv_tile_wg(const ConvTileDesc &d, const void *X, const void *dY, void *dW)
     a.magic_rr = magic_of(a.RR);
     a.magic_taps = magic_of(taps);
     a.magic_kw = magic_of(d.KW);
+    a.magic_thp = magic_of(a.THP);
+    if (a.THP + a.RR >= 65536) return -1;
     const int gy = (d.Cin + a.CT - 1) / a.CT;
     const int cbw = (a.cblocks + 3) / 4;  // column blocks per wave
     if (cbw > 3) return -1;
