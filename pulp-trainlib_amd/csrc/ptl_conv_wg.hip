@@ -220,21 +220,33 @@ __global__ __launch_bounds__(512) void conv_wg_kernel(const ConvWgArgs a) {
     }
 }
 
-// dW[i] = sum over parts of ws[part][i]: 32 outputs per workgroup, 8 part groups in parallel.
+// dW[i] = sum over parts of ws[part][i]: 64 outputs per workgroup, 16 part groups in parallel,
+// eight loads in flight per thread (the partials are a few MB spread over hundreds of parts:
+// the kernel lives on memory-level parallelism, not on arithmetic).
 template <typename T>
-__global__ __launch_bounds__(256) void conv_wg_reduce_kernel(const float *__restrict__ ws, T *__restrict__ dW, int total,
-                                                             int parts) {
-    __shared__ float part_sum[8][32];
-    const int o = threadIdx.x & 31, pg = threadIdx.x >> 5;
-    const int i = blockIdx.x * 32 + o;
+__global__ __launch_bounds__(1024) void conv_wg_reduce_kernel(const float *__restrict__ ws, T *__restrict__ dW, int total,
+                                                              int parts) {
+    __shared__ float part_sum[16][64];
+    const int o = threadIdx.x & 63, pg = threadIdx.x >> 6;
+    const int i = blockIdx.x * 64 + o;
     float s = 0.f;
-    if (i < total)
-        for (int p = pg; p < parts; p += 8) s += ws[(size_t)p * total + i];
+    if (i < total) {
+        const float *src = ws + i;
+        int p = pg;
+        for (; p + 7 * 16 < parts; p += 8 * 16) {
+            float v[8];
+#pragma unroll
+            for (int u = 0; u < 8; ++u) v[u] = src[(size_t)(p + u * 16) * total];
+#pragma unroll
+            for (int u = 0; u < 8; ++u) s += v[u];
+        }
+        for (; p < parts; p += 16) s += src[(size_t)p * total];
+    }
     part_sum[pg][o] = s;
     __syncthreads();
     if (pg == 0 && i < total) {
 #pragma unroll
-        for (int q = 1; q < 8; ++q) s += part_sum[q][o];
+        for (int q = 1; q < 16; ++q) s += part_sum[q][o];
         dW[i] = (T)s;
     }
 }
@@ -272,7 +284,7 @@ static int launch_conv_wg(ConvWgArgs &a, int gy, int gz, void *dW, hipStream_t s
     // partial is complete, otherwise every (slab, row tile) pair writes a disjoint part of it
     hipLaunchKernelGGL(kern, dim3((unsigned)parts, gy, gz), dim3(512), lds, s, a);
     if (!hip_ok(hipGetLastError(), "conv wg launch")) return 2;
-    hipLaunchKernelGGL((conv_wg_reduce_kernel<T>), dim3((total + 31) / 32), dim3(256), 0, s, a.ws,
+    hipLaunchKernelGGL((conv_wg_reduce_kernel<T>), dim3((total + 63) / 64), dim3(1024), 0, s, a.ws,
                        reinterpret_cast<T *>(dW), total, (int)parts);
     return hip_ok(hipGetLastError(), "conv wg reduce launch") ? 0 : 2;
 }
