@@ -342,15 +342,33 @@ __global__ __launch_bounds__(256) void gemm_kernel(const GemmArgs g) {
     }
 }
 
-// Sum split-K partials in split order and scatter through the output map.
+// Sum split-K partials (fixed order) and scatter through the output map: 64 outputs per
+// workgroup, four split groups in parallel, four loads in flight per thread -- with few outputs
+// and many splits the kernel lives on memory-level parallelism.
 template <typename T>
 __global__ __launch_bounds__(256) void splitk_reduce_kernel(const float *__restrict__ ws, T *__restrict__ C,
                                                             OutMap c, int N, int M, int splits) {
-    size_t total = (size_t)N * M;
-    size_t idx = (size_t)blockIdx.x * 256 + threadIdx.x;
-    if (idx >= total) return;
+    __shared__ float part[4][64];
+    const size_t total = (size_t)N * M;
+    const int o = threadIdx.x & 63, sg = threadIdx.x >> 6;
+    const size_t idx = (size_t)blockIdx.x * 64 + o;
     float s = 0.f;
-    for (int z = 0; z < splits; ++z) s += ws[(size_t)z * total + idx];
+    if (idx < total) {
+        const float *src = ws + idx;
+        int z = sg;
+        for (; z + 3 * 4 < splits; z += 4 * 4) {
+            float v[4];
+#pragma unroll
+            for (int u = 0; u < 4; ++u) v[u] = src[(size_t)(z + u * 4) * total];
+#pragma unroll
+            for (int u = 0; u < 4; ++u) s += v[u];
+        }
+        for (; z < splits; z += 4) s += src[(size_t)z * total];
+    }
+    part[sg][o] = s;
+    __syncthreads();
+    if (sg != 0 || idx >= total) return;
+    s += part[1][o] + part[2][o] + part[3][o];
     int n = (int)(idx / M), m = (int)(idx % M);
     int on, om, h, w;
     axis_decode(c.n, n, on, h, w);
@@ -477,7 +495,7 @@ int gemm(const GemmArgs &gin) {
     }
     if (g.splits > 1) {
         size_t total = (size_t)g.N * g.M;
-        hipLaunchKernelGGL((splitk_reduce_kernel<T>), dim3((unsigned)((total + 255) / 256)), dim3(256), 0,
+        hipLaunchKernelGGL((splitk_reduce_kernel<T>), dim3((unsigned)((total + 63) / 64)), dim3(256), 0,
                            st.stream, g.ws, reinterpret_cast<T *>(g.C), g.c, g.N, g.M, g.splits);
         if (!hip_ok(hipGetLastError(), "split-k reduce launch")) return 2;
     }
