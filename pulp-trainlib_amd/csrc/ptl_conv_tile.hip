@@ -382,7 +382,9 @@ int conv_tile(const ConvTileDesc &d, const void *X, const void *Wt, void *Y, con
     }
     a.b_bytes = bn * a.b_pitch;
     const long mt = (d.Cout + bn - 1) / bn;
-    if (st.gemm_path != 2 && ((long)(a.g.N + BM - 1) / BM) * mt < 2L * st.num_cu) return -1;
+    // ... or when the filter tile is small enough (20 KB) for that price not to matter: measured
+    // 6.7 against 8.2 us for one 16->32 channel 32x32 sample, 19 against 8 us for eight 64->64 8x8 ones.
+    if (st.gemm_path != 2 && ((long)(a.g.N + BM - 1) / BM) * mt < 2L * st.num_cu && a.b_bytes > 20 * 1024) return -1;
 
     a.magic_tw = magic_of(a.TW);
     a.magic_rr = magic_of(a.RR);
