@@ -601,6 +601,57 @@ __global__ __launch_bounds__(256) void gemv_coldot_vec_kernel(const T *__restric
     }
 }
 
+// The same product in ONE launch for moderate K: a workgroup owns 4*VEC consecutive columns and
+// ALL rows; thread (kl, cv) sums rows kl, kl+64, ... of column vector cv with eight loads in
+// flight, the 64 row-lanes are folded through LDS.  (A cross-workgroup "last arriver adds the
+// partials" variant was tried: the device-scope fences it needs write back the whole L2 per
+// workgroup and made it twice as slow as two launches.)
+template <typename T>
+__global__ __launch_bounds__(256) void gemv_coldot_whole_kernel(const T *__restrict__ x, const T *__restrict__ Mx,
+                                                                T *__restrict__ y, int K, int M) {
+    constexpr int VEC = Traits<T>::VEC, CV = 4, KL = 256 / CV;
+    const int cv = threadIdx.x % CV, kl = threadIdx.x / CV;
+    const int col = (blockIdx.x * CV + cv) * VEC;
+    float acc[VEC];
+#pragma unroll
+    for (int i = 0; i < VEC; ++i) acc[i] = 0.f;
+    if (col < M) {
+        const T *p = Mx + col;
+        int k = kl;
+        for (; k + 7 * KL < K; k += 8 * KL) {
+            Stage<T> v[8];
+            float xv[8];
+#pragma unroll
+            for (int u = 0; u < 8; ++u) {
+                v[u].v[0] = *reinterpret_cast<const uint4 *>(p + (size_t)(k + u * KL) * M);
+                xv[u] = (float)x[k + u * KL];
+            }
+#pragma unroll
+            for (int u = 0; u < 8; ++u)
+#pragma unroll
+                for (int i = 0; i < VEC; ++i) acc[i] += xv[u] * (float)v[u].e[i];
+        }
+        for (; k < K; k += KL) {
+            Stage<T> v;
+            v.v[0] = *reinterpret_cast<const uint4 *>(p + (size_t)k * M);
+            const float xv = (float)x[k];
+#pragma unroll
+            for (int i = 0; i < VEC; ++i) acc[i] += xv * (float)v.e[i];
+        }
+    }
+    __shared__ float red[KL][CV * VEC + 1];
+#pragma unroll
+    for (int i = 0; i < VEC; ++i) red[kl][cv * VEC + i] = acc[i];
+    __syncthreads();
+    if (threadIdx.x < CV * VEC) {
+        float s = 0.f;
+#pragma unroll 8
+        for (int r = 0; r < KL; ++r) s += red[r][threadIdx.x];
+        const int c = blockIdx.x * CV * VEC + threadIdx.x;
+        if (c < M) y[c] = (T)s;
+    }
+}
+
 template <typename T>
 __global__ __launch_bounds__(256) void colsum_reduce_kernel(const float *__restrict__ part, T *__restrict__ y,
                                                             int M, int splits) {
@@ -657,6 +708,11 @@ int mm_dispatch(const T *A, const T *B, T *C, int N, int M, int K, int trans_B) 
         splits = (K + kchunk - 1) / kchunk;
         float *part = workspace((size_t)splits * M * sizeof(float));
         if (!part) return 2;
+        if (K <= 4096) {  // one launch: each workgroup sums whole columns
+            hipLaunchKernelGGL((gemv_coldot_whole_kernel<T>), dim3((M + 4 * VECW - 1) / (4 * VECW)), dim3(256), 0,
+                               st.stream, A, B, C, K, M);
+            return hip_ok(hipGetLastError(), "gemv launch") ? 0 : 2;
+        }
         hipLaunchKernelGGL((gemv_coldot_vec_kernel<T>), dim3(blocks_m, splits), dim3(256), 0, st.stream, A, B, part,
                            K, M, kchunk);
         hipLaunchKernelGGL((colsum_reduce_kernel<T>), dim3((M + 255) / 256), dim3(256), 0, st.stream, part, C, M,
