@@ -673,6 +673,29 @@ __global__ __launch_bounds__(256) void outer_kernel(const T *__restrict__ a, con
     C[idx] = (T)((float)a[n] * (float)b[m]);
 }
 
+// Same with 16-byte stores (M a multiple of the vector, b and C 16-byte aligned): a thread owns VEC
+// consecutive columns of four consecutive rows.
+template <typename T>
+__global__ __launch_bounds__(256) void outer_vec_kernel(const T *__restrict__ a, const T *__restrict__ b,
+                                                        T *__restrict__ C, int N, int M) {
+    constexpr int VEC = Traits<T>::VEC;
+    const int mv = M / VEC;
+    const size_t idx = (size_t)blockIdx.x * 256 + threadIdx.x;
+    const size_t total = (size_t)((N + 3) / 4) * mv;
+    if (idx >= total) return;
+    const int n0 = (int)(idx / mv) * 4, m = (int)(idx % mv) * VEC;
+    Stage<T> bv, out;
+    bv.v[0] = *reinterpret_cast<const uint4 *>(b + m);
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+        if (n0 + r >= N) break;
+        const float av = (float)a[n0 + r];
+#pragma unroll
+        for (int i = 0; i < VEC; ++i) out.e[i] = (T)(av * (float)bv.e[i]);
+        *reinterpret_cast<uint4 *>(C + (size_t)(n0 + r) * M + m) = out.v[0];
+    }
+}
+
 template <typename T>
 static int gemv_rowdot(const T *Mx, const T *x, T *y, int R, int K) {
     constexpr int VEC = Traits<T>::VEC;
@@ -691,6 +714,13 @@ int mm_dispatch(const T *A, const T *B, T *C, int N, int M, int K, int trans_B) 
     State &st = state();
     if (K == 1) {
         size_t total = (size_t)N * M;
+        constexpr int VO = Traits<T>::VEC;
+        if (M % VO == 0 && reinterpret_cast<uintptr_t>(B) % 16 == 0 && reinterpret_cast<uintptr_t>(C) % 16 == 0) {
+            size_t units = (size_t)((N + 3) / 4) * (M / VO);
+            hipLaunchKernelGGL((outer_vec_kernel<T>), dim3((unsigned)((units + 255) / 256)), dim3(256), 0, st.stream,
+                               A, B, C, N, M);
+            return hip_ok(hipGetLastError(), "outer launch") ? 0 : 2;
+        }
         hipLaunchKernelGGL((outer_kernel<T>), dim3((unsigned)((total + 255) / 256)), dim3(256), 0, st.stream, A,
                            B, C, N, M);
         return hip_ok(hipGetLastError(), "outer launch") ? 0 : 2;
