@@ -19,6 +19,8 @@ int gemm_async(GemmArgs &g) {
         cfg = 2;
     else if (g.M <= 32)
         cfg = 3;
+    else if (g.N <= 64 || g.M <= 64)  // a 128-wide tile would be half padding
+        cfg = 1;
     else if (tiles(128, 128) >= st.num_cu)
         cfg = 0;
     else
@@ -56,7 +58,11 @@ int gemm_async(GemmArgs &g) {
     }
     if (plain_operand<T>(g.a, g.kchunk, g.K) && plain_operand<T>(g.b, g.kchunk, g.K)) {
         switch (cfg) {
-            case 0: return launch_plain<T, 128, 128, 512, 2, 2, 2, 3, 1>(g, st.stream);
+            case 0:
+                // one or two slabs deep (pointwise layers): four waves without a k split need half the
+                // LDS for the parked tile, so two workgroups share a CU and overlap load, MFMA and store
+                if (g.splits == 1 && g.K <= 2 * SK) return launch_plain<T, 128, 128, 256, 2, 2, 1, 2, 1>(g, st.stream);
+                return launch_plain<T, 128, 128, 512, 2, 2, 2, 3, 1>(g, st.stream);
             case 1:
                 // fp32 MFMAs are slow enough to matter at this size: when 64x64 tiles leave half the CUs
                 // idle, 64x32 tiles put a workgroup on every CU

@@ -11,4 +11,5 @@ template int launch_plain_pair<float, 128, 128, 512, 2, 2, 2, 3, 1>(GemmArgs &, 
 template int launch_plain_pair<float, 64, 64, 1024, 2, 2, 4, 3, 1>(GemmArgs &, GemmArgs &, hipStream_t);
 template int launch_plain<float, 64, 64, 1024, 2, 2, 4, 3, 2>(GemmArgs &, hipStream_t);
 template int launch_plain<float, 64, 32, 512, 2, 1, 4, 3, 1>(GemmArgs &, hipStream_t);
+template int launch_plain<float, 128, 128, 256, 2, 2, 1, 2, 1>(GemmArgs &, hipStream_t);
 }
