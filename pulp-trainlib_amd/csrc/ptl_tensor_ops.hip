@@ -143,6 +143,25 @@ __global__ __launch_bounds__(256) void dw_wg_reduce_kernel(const float *__restri
 // input row in registers.  Per output element this is (RB+K-1)*K/RB loads instead of K*K.
 constexpr int DW_RB = 8;  // output rows per thread
 
+// The K column shifts of one source row for this lane's column c: v[j] = row[c + j - pl] (zero
+// outside the row).  One load of the lane's own column, the shifts come from the neighbouring
+// lanes; only lanes at the edge of the wave's 64-column chunk load their missing neighbours.
+template <typename T, int K>
+__device__ inline void dw_row_shifts(const T *__restrict__ row, bool rowok, int c, int lane, int pl, int Ws,
+                                     const bool (&colok)[K], float (&v)[K]) {
+    const float own = (rowok && (unsigned)c < (unsigned)Ws) ? (float)row[c] : 0.f;
+#pragma unroll
+    for (int j = 0; j < K; ++j) {
+        const int d = j - pl;
+        const float nb = __shfl(own, lane + d, 64);
+        const bool in_wave = (unsigned)(lane + d) < 64u;
+        float val = in_wave ? nb : 0.f;
+        if (!in_wave && rowok && colok[j]) val = (float)row[c + d];
+        v[j] = (d == 0) ? own : val;
+    }
+}
+
+
 // out[p][r][c] = sum_{i,j} wt[ch][i][j] * in[p][r + i - pu][c + j - pl], zero outside the source.
 // FLIP uses wt[K-1-i][K-1-j]: with pu = K-1-Up, pl = K-1-Lp and the output gradient as
 // source this is the input gradient.
@@ -178,8 +197,7 @@ __global__ __launch_bounds__(256) void dw_rows_kernel(const T *__restrict__ src,
         const int h = r0 + rr - pu;  // source row (wave-uniform)
         float v[K];
         const bool rowok = (unsigned)h < (unsigned)Hs;
-#pragma unroll
-        for (int j = 0; j < K; ++j) v[j] = (rowok && colok[j]) ? (float)sp[(size_t)h * Ws + (c + j - pl)] : 0.f;
+        dw_row_shifts<T, K>(sp + (size_t)(rowok ? h : 0) * Ws, rowok, c, lane, pl, Ws, colok, v);
 #pragma unroll
         for (int i = 0; i < K; ++i) {
             const int q = rr - i;  // output row (relative) fed by this source row through tap row i
@@ -232,15 +250,12 @@ __global__ __launch_bounds__(256) void dw_wg_rows_kernel(const T *__restrict__ X
     for (int i = 0; i < K - 1; ++i) {
         const int h = r0 + i - pu;
         const bool rowok = (unsigned)h < (unsigned)H;
-#pragma unroll
-        for (int j = 0; j < K; ++j) win[i][j] = (rowok && colok[j]) ? (float)xp[(size_t)h * W + (c + j - pl)] : 0.f;
+        dw_row_shifts<T, K>(xp + (size_t)(rowok ? h : 0) * W, rowok, c, lane, pl, W, colok, win[i]);
     }
     for (int r = r0; r < r1; ++r) {
         const int h = r + (K - 1) - pu;
         const bool rowok = (unsigned)h < (unsigned)H;
-#pragma unroll
-        for (int j = 0; j < K; ++j)
-            win[K - 1][j] = (rowok && colok[j]) ? (float)xp[(size_t)h * W + (c + j - pl)] : 0.f;
+        dw_row_shifts<T, K>(xp + (size_t)(rowok ? h : 0) * W, rowok, c, lane, pl, W, colok, win[K - 1]);
         const float g = gcol ? (float)gp[(size_t)r * Wo + c] : 0.f;
 #pragma unroll
         for (int i = 0; i < K; ++i)
