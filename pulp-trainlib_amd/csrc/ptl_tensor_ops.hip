@@ -281,22 +281,25 @@ __global__ __launch_bounds__(256) void dw_wg_rows_kernel(const T *__restrict__ X
 template <typename T>
 __global__ __launch_bounds__(256) void dw_wg_reduce_kernel2(const float *__restrict__ part, T *__restrict__ dW, int ns,
                                                             int C, int strips, int taps) {
+    // thread = (tap, slice): consecutive threads read the consecutive taps of one partial; the
+    // slices of a tap are folded through LDS in one pass (taps <= 25)
     const int ch = blockIdx.x;
     __shared__ float red[256];
-    for (int tap = 0; tap < taps; ++tap) {
-        float s = 0.f;
-        for (long i = threadIdx.x; i < (long)ns * strips; i += 256) {
+    const int slices = 256 / taps;
+    const int tap = threadIdx.x % taps, slice = threadIdx.x / taps;
+    float s = 0.f;
+    if (slice < slices) {
+        for (long i = slice; i < (long)ns * strips; i += slices) {
             long b = i / strips, st = i % strips;
             s += part[(((size_t)b * C + ch) * strips + st) * taps + tap];
         }
-        red[threadIdx.x] = s;
-        __syncthreads();
-        for (int o = 128; o > 0; o >>= 1) {
-            if ((int)threadIdx.x < o) red[threadIdx.x] += red[threadIdx.x + o];
-            __syncthreads();
-        }
-        if (threadIdx.x == 0) dW[(size_t)ch * taps + tap] = (T)red[0];
-        __syncthreads();
+    }
+    red[threadIdx.x] = s;
+    __syncthreads();
+    if ((int)threadIdx.x < taps) {
+        float t = 0.f;
+        for (int k = 0; k < slices; ++k) t += red[k * taps + threadIdx.x];
+        dW[(size_t)ch * taps + threadIdx.x] = (T)t;
     }
 }
 
