@@ -47,6 +47,9 @@ struct ConvTileArgs {
     int fast_pix;      // 1: pixel coordinates by reciprocal multiplication (tile-relative quotients below 2^16)
     int nfast;         // 1: the output's pixel axis is (sample, pixel-in-sample) with the sample size as radix
     unsigned magic_pp, magic_wo, magic_thp;
+    int in_sb, in_scb, in_sy, in_sx;  // chunk strides of the chunked input: sample, channel block, row, column
+    int in_cblocks;    // channel blocks that exist in it (the rest of CinP is zeros)
+    int m_unit;        // 1: consecutive filters are consecutive output elements (4-element stores)
     int raw_chunks;    // chunks of one raw slab (two channel blocks) rounded up to whole waves
     int stage_chunks;  // chunks of one staging slab (KSTEP channels x RR rows x whole input rows), whole waves
     int xg;            // 16-byte groups per input row
@@ -88,7 +91,6 @@ __global__ __launch_bounds__((BM / 32) * 64) void conv_tile_kernel(const ConvTil
     // buffer is refilled next).  Nothing crosses threads except the raw tile itself: each lane
     // derives its own addresses.
     const unsigned raw_lds = (unsigned)(uintptr_t)(lds_char *)raw;
-    const int plane_in = d.Hin * d.Win;
     const unsigned stage_lds = (unsigned)(uintptr_t)(lds_char *)stage;
     auto enqueue = [&](int tile, int cs, int buf) {
         const int n0 = tile * BM;
@@ -117,9 +119,9 @@ __global__ __launch_bounds__((BM / 32) * 64) void conv_tile_kernel(const ConvTil
             const int half = fast_div(row, a.magic_rr), rr = row - half * a.RR;
             const int t = t0 + rr, db = fast_div(t, a.magic_thp);  // (t < THP + RR: small quotient)
             const int b = b0 + db, iy = t - db * a.THP - d.padU, ix = tx - d.padL;
-            const bool ok = half < 2 && b < d.batch && iy >= 0 && iy < d.Hin && ix >= 0 && ix < d.Win;
             const int cb = cs * 2 + half;
-            const char *src = ok ? reinterpret_cast<const char *>(Xb + (((b * cblocks + cb) * d.Hin + iy) * d.Win + ix))
+            const bool ok = half < 2 && cb < a.in_cblocks && b < d.batch && iy >= 0 && iy < d.Hin && ix >= 0 && ix < d.Win;
+            const char *src = ok ? reinterpret_cast<const char *>(Xb + (b * a.in_sb + cb * a.in_scb + iy * a.in_sy + ix * a.in_sx))
                                  : reinterpret_cast<const char *>(a.zero);
             lds_dma<16>(src, raw_lds + (unsigned)(buf * a.raw_chunks + c0) * 16u);
         }
@@ -180,15 +182,32 @@ __global__ __launch_bounds__((BM / 32) * 64) void conv_tile_kernel(const ConvTil
     T pend[FN][16];
     T *pend_out = nullptr;
     auto flush = [&]() {
-        if (pend_out) {
+        if (!pend_out) return;
+        if (a.m_unit) {  // four consecutive filters of this pixel are four consecutive elements
 #pragma unroll
             for (int j = 0; j < FN; ++j)
 #pragma unroll
-                for (int v = 0; v < 16; ++v) {
-                    const int ml = j * 32 + 8 * (v >> 2) + 4 * kg + (v & 3);
-                    if (m0 + ml < a.g.M) pend_out[mlut[ml]] = pend[j][v];
+                for (int q = 0; q < 4; ++q) {
+                    const int ml = j * 32 + 8 * q + 4 * kg;
+                    if (m0 + ml + 3 < a.g.M) {
+                        typedef T t4 __attribute__((ext_vector_type(4)));
+                        t4 o = {pend[j][4 * q], pend[j][4 * q + 1], pend[j][4 * q + 2], pend[j][4 * q + 3]};
+                        *reinterpret_cast<t4 *>(pend_out + mlut[ml]) = o;
+                    } else {
+#pragma unroll
+                        for (int e = 0; e < 4; ++e)
+                            if (m0 + ml + e < a.g.M) pend_out[mlut[ml + e]] = pend[j][4 * q + e];
+                    }
                 }
+            return;
         }
+#pragma unroll
+        for (int j = 0; j < FN; ++j)
+#pragma unroll
+            for (int v = 0; v < 16; ++v) {
+                const int ml = j * 32 + 8 * (v >> 2) + 4 * kg + (v & 3);
+                if (m0 + ml < a.g.M) pend_out[mlut[ml]] = pend[j][v];
+            }
     };
     const int csteps = a.CinP / KSTEP;
     int buf = 0;
@@ -333,7 +352,8 @@ int conv_tile(const ConvTileDesc &d, const void *X, const void *Wt, void *Y, con
     a.CinP = ((d.Cin + KSTEP - 1) / KSTEP) * KSTEP;
     a.THP = d.Hin + d.padU + d.padD;
     a.TW = d.Win + d.padL + d.padR;
-    if (!a.zero || d.padU < 0 || d.padD < 0 || d.padL < 0 || d.padR < 0 || d.x_sy != d.Win) return -1;
+    if (!a.zero || d.padU < 0 || d.padD < 0 || d.padL < 0 || d.padR < 0) return -1;
+    if (d.in_hwc ? (d.Cin % VEC != 0 || reinterpret_cast<uintptr_t>(X) % 16 != 0) : d.x_sy != d.Win) return -1;
     // every output pixel's window must lie inside the padded image
     if ((d.Ho - 1) * d.sh + d.KH > a.THP || (d.Wo - 1) * d.sw + d.KW > a.TW) return -1;
     const int cblocks = a.CinP / VEC;
@@ -360,7 +380,7 @@ int conv_tile(const ConvTileDesc &d, const void *X, const void *Wt, void *Y, con
     // slab buffers instead of two: measured 12 against 15 us on 32x32 images with 16 channels,
     // 189 against 104 us on 56x56 with 32), so it is taken when a workgroup's slabs stay
     // below 40 KB.
-    const bool staged = d.Win % VEC == 0 && d.x_sc % VEC == 0 && d.x_sb % VEC == 0 &&
+    const bool staged = !d.in_hwc && d.Win % VEC == 0 && d.x_sc % VEC == 0 && d.x_sb % VEC == 0 &&
                         reinterpret_cast<uintptr_t>(X) % 16 == 0 && a.stage_chunks < 65536 &&
                         (long long)d.batch * d.x_sb < ((long long)1 << 31) &&
                         ((size_t)a.raw_chunks + 2 * (size_t)a.stage_chunks) * 16 <= 40 * 1024;
@@ -398,6 +418,28 @@ int conv_tile(const ConvTileDesc &d, const void *X, const void *Wt, void *Y, con
     if (a.THP + a.RR >= 65536) return -1;
     a.nfast = (c.n.d0 == PP && c.n.d1 >= (1 << 30)) ? 1 : 0;
 
+    // 4-element stores along the filters: unit stride there, and every pixel's run 4-element aligned
+    a.m_unit = (c.m.d0 >= c.m.n && c.m.o0 == 1 && (c.m.ob & 3) == 0 && c.n.d0 >= c.n.n && (c.n.o0 & 3) == 0 &&
+                (c.n.ob & 3) == 0 && reinterpret_cast<uintptr_t>(Y) % (4 * sizeof(T)) == 0)
+                   ? 1
+                   : 0;
+    if (d.in_hwc) {  // the tensor itself is the chunked input
+        a.X = X;
+        a.in_cblocks = d.Cin / VEC;
+        a.in_sx = a.in_cblocks;
+        a.in_sy = d.Win * a.in_cblocks;
+        a.in_sb = d.Hin * a.in_sy;
+        a.in_scb = 1;
+        if ((long long)d.batch * a.in_sb >= ((long long)1 << 31)) return -1;
+        if (bn == 128) return launch_conv_tile<T, BM, 128, false>(a, lds, st.stream);
+        if (bn == 64) return launch_conv_tile<T, BM, 64, false>(a, lds, st.stream);
+        return launch_conv_tile<T, BM, 32, false>(a, lds, st.stream);
+    }
+    a.in_cblocks = cblocks;
+    a.in_sx = 1;
+    a.in_sy = d.Win;
+    a.in_scb = d.Hin * d.Win;
+    a.in_sb = cblocks * a.in_scb;
     if (staged) {
         a.X = X;
         if (bn == 128) return launch_conv_tile<T, BM, 128, true>(a, lds, st.stream);

@@ -15,6 +15,9 @@ struct ConvTileDesc {
     long long x_sb, x_sc;
     int x_sy;
     int w_base, w_sm, w_sc, w_sy, w_sx;
+    // 1: the input is channel-minor, in(b, ci, iy, ix) at X[((b*Hin + iy)*Win + ix)*Cin + ci] (x_s* unused);
+    // with Cin a multiple of the 16-byte vector it already consists of the chunks the kernel wants
+    int in_hwc;
 };
 
 // Launches the direct kernel; the output is written through `c` (n = pixel index over

@@ -242,17 +242,24 @@ static int conv2d_fw(const Args *a, int ns, const char *fn) {
 
     int rc = -1;
     state().last_conv_direct = 0;
-    if (!g.hwc && state().gemm_path != 1) {
+    if (state().gemm_path != 1) {
         ConvTileDesc d = {};
         d.batch = ns; d.Cin = g.Ci; d.Hin = g.H; d.Win = g.W;
         d.Cout = g.Co; d.Ho = g.Ho; d.Wo = g.Wo;
         d.KH = g.Hk; d.KW = g.Wk; d.sh = g.sh; d.sw = g.sw;
         d.padU = g.Up; d.padD = g.Dp; d.padL = g.Lp; d.padR = g.Rp;
         d.x_sb = (long long)g.Ci * g.H * g.W; d.x_sc = (long long)g.H * g.W; d.x_sy = g.W;
-        d.w_base = 0; d.w_sm = K; d.w_sc = g.Hk * g.Wk; d.w_sy = g.Wk; d.w_sx = 1;
         OutMap c;
-        c.n = axis_two(ns * P, P, g.Co * P, 1);
-        c.m = axis_plain(g.Co, P);
+        if (!g.hwc) {
+            d.w_base = 0; d.w_sm = K; d.w_sc = g.Hk * g.Wk; d.w_sy = g.Wk; d.w_sx = 1;
+            c.n = axis_two(ns * P, P, g.Co * P, 1);
+            c.m = axis_plain(g.Co, P);
+        } else {  // X[b][h][w][ci], W[co][hk][wk][ci], Y[b][pix][co]
+            d.in_hwc = 1;
+            d.w_base = 0; d.w_sm = K; d.w_sc = 1; d.w_sy = g.Wk * g.Ci; d.w_sx = g.Ci;
+            c.n = axis_plain(ns * P, g.Co);
+            c.m = axis_plain(g.Co, 1);
+        }
         rc = conv_tile<T>(d, X, Wt, Y, c);
         if (rc > 0) return sg.finish(rc);
         if (rc == 0) state().last_conv_direct = 1;
@@ -409,7 +416,7 @@ static int conv2d_ig(const Args *a, int ns, const char *fn) {
     gmap.row.wb = g.Lp;
     gmap.k.n = K;
     state().last_conv_direct = 0;
-    if (!g.hwc && state().gemm_path != 1) {
+    if (state().gemm_path != 1) {
         ConvTileDesc d = {};
         d.batch = ns; d.Cin = g.Co; d.Hin = Hd; d.Win = Wd;
         d.Cout = g.Ci; d.Ho = g.H; d.Wo = g.W;
@@ -417,10 +424,17 @@ static int conv2d_ig(const Args *a, int ns, const char *fn) {
         d.padU = g.Hk - 1 - g.Up; d.padL = g.Wk - 1 - g.Lp;
         d.padD = g.H + g.Hk - 1 - Hd - d.padU; d.padR = g.W + g.Wk - 1 - Wd - d.padL;
         d.x_sb = (long long)g.Co * Hd * Wd; d.x_sc = (long long)Hd * Wd; d.x_sy = Wd;
-        d.w_base = Pk - 1; d.w_sm = Pk; d.w_sc = g.Ci * Pk; d.w_sy = -g.Wk; d.w_sx = -1;
         OutMap c;
-        c.n = axis_two(ns * g.H * g.W, g.H * g.W, g.Ci * g.H * g.W, 1);
-        c.m = axis_plain(g.Ci, g.H * g.W);
+        if (!g.hwc) {
+            d.w_base = Pk - 1; d.w_sm = Pk; d.w_sc = g.Ci * Pk; d.w_sy = -g.Wk; d.w_sx = -1;
+            c.n = axis_two(ns * g.H * g.W, g.H * g.W, g.Ci * g.H * g.W, 1);
+            c.m = axis_plain(g.Ci, g.H * g.W);
+        } else {  // dY[b][pix][co], W[co][hk][wk][ci], dX[b][pix][ci]
+            d.in_hwc = 1;
+            d.w_base = (Pk - 1) * g.Ci; d.w_sm = 1; d.w_sc = Pk * g.Ci; d.w_sy = -g.Wk * g.Ci; d.w_sx = -g.Ci;
+            c.n = axis_plain(ns * g.H * g.W, g.Ci);
+            c.m = axis_plain(g.Ci, 1);
+        }
         int rc = conv_tile<T>(d, dY, Wt, dX, c);
         if (rc == 0) state().last_conv_direct = 1;
         if (rc >= 0) return sg.finish(rc);

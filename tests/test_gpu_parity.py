@@ -149,6 +149,31 @@ def test_conv2d_direct_kernel(pkg, orc, gpu, dt, case):
         gpu.ptl_set_gemm_path(0)
 
 
+# Channel-minor (HWC) tensors already consist of the 16-byte channel chunks the direct kernel works on:
+# forward and input gradient read them in place (channel counts that are multiples of the vector).
+DIRECT_HWC_CASES = [
+    (16, 32, 32, 32, 3, 3, (1, 1, 1, 1), (1, 1), 3),
+    (8, 9, 12, 7, 3, 2, (1, 0, 0, 2), (1, 1), 9),
+    (24, 6, 6, 40, 3, 3, (1, 1, 1, 1), (1, 1), 11),
+    (16, 17, 13, 12, 3, 3, (1, 1, 1, 1), (2, 2), 7),
+    (40, 10, 10, 130, 1, 1, (0, 0, 0, 0), (1, 1), 4),
+]
+
+
+@pytest.mark.parametrize("dt", ["fp32", "fp16"])
+@pytest.mark.parametrize("case", DIRECT_HWC_CASES)
+def test_conv2d_direct_kernel_hwc(pkg, orc, gpu, dt, case):
+    Ci, H, W, Co, Hk, Wk, pad, stride, ns = case
+    gpu.ptl_set_gemm_path(2)
+    try:
+        conv_parity(pkg, orc, gpu, dt, Ci, H, W, Co, Hk, Wk, pad, stride, 1, ns, 0xC0DE0061, via_batched=True)
+        # the last call of conv_parity is the input gradient: its input has Co channels
+        vec = 8 if dt == "fp16" else 4
+        assert gpu.ptl_last_conv_direct() == (1 if Co % vec == 0 else 0)
+    finally:
+        gpu.ptl_set_gemm_path(0)
+
+
 # The direct weight-gradient kernel needs unit column stride and row lengths that are multiples of the
 # 16-byte vector (8 halves / 4 floats).
 DIRECT_WG_CASES = [
