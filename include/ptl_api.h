@@ -78,6 +78,18 @@ void pulp_linear_fp16_bw_cl(void *Linear_args_fp16);
 void pulp_linear_fp16_bw_param_grads_cl(void *Linear_args_fp16);
 void pulp_linear_fp16_bw_input_grads_cl(void *Linear_args_fp16);
 
+/* Multi-head self-attention training step, fp32: lib/sources/pulp_mhsa_fp32.c:20 (forward), :648 (backward).
+ * Forward fills q, k, v, softmax_buffer, attention_map and output; backward reads them and fills every
+ * `diff` (input->diff is added to, as the reference's closing vector sums do, :1634-1745).
+ * Softmax uses the reference's approximate exponential (fastexp_gist, lib/sources/pulp_train_utils_fp32.c:1223)
+ * and the projection biases are per feature (row of the F x L matrices). */
+void pulp_mhsa_fp32_fw_cl(void *Mhsa_args);
+void pulp_mhsa_fp32_bw_cl(void *Mhsa_args);
+/* Row-wise softmax with the approximate exponential and its backward pass:
+ * lib/sources/pulp_act_fp32.c:187, :335. */
+void pulp_softmax_fp32_fw_cl(void *softmax_args);
+void pulp_softmax_fp32_bw_cl(void *softmax_args);
+
 /* Matmul kernels and their dispatcher.
  * mm / mm_M: lib/sources/pulp_matmul_fp32.c:190, :345
  * mm_fp16 / mm_M_fp16: lib/sources/pulp_matmul_fp16.c:191, :273
@@ -224,6 +236,12 @@ int ptl_linear_fp16_ig_batched(const struct Linear_args_fp16 *a, int nsamples);
  * lib/sources/pulp_linear_fp16.c); both products share a launch where they fit. */
 int ptl_linear_fp32_bw_batched(const struct Linear_args *a, int nsamples);
 int ptl_linear_fp16_bw_batched(const struct Linear_args_fp16 *a, int nsamples);
+
+/* Batched attention step: sample b of every activation blob (input, q, k, v, attention_map,
+ * softmax_buffer, output; data and diff) starts b * (rows x columns of that blob) elements in; weights
+ * are shared and their gradients are summed over the samples. */
+int ptl_mhsa_fp32_fw_batched(const struct Mhsa_args *a, int nsamples);
+int ptl_mhsa_fp32_bw_batched(const struct Mhsa_args *a, int nsamples);
 
 /* Plain product C[N x M] = A[N x K] * B (B is K x M, or M x K when trans_B),
  * the contract of the reference's mm family, on raw pointers. */

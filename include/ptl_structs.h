@@ -476,6 +476,64 @@ struct Linear_args_fp16 {
     int use_biases;
 };
 
+/* Row-wise softmax (lib/include/pulp_act_fp32.h:53-66).  H rows of W elements;
+ * `maxes` and `sums` are H-element scratch rows the forward pass fills. */
+struct softmax_args {
+    float *input_data;
+    float *input_diff;
+    float *output_data;
+    float *output_diff;
+    int H;
+    int W;
+    int L;
+    int n_heads;
+    float *global_max;
+    float *partial_exp_sum;
+    float *maxes;
+    float *sums;
+};
+
+/* Multi-head self-attention (lib/include/pulp_mhsa_fp32.h:52-83).
+ * With L = input->H (sequence length), E = input->W (token size),
+ * F = attention_map->W (heads x head size):
+ *   input, output            E x L   (tokens are columns)
+ *   coeff_in_q/k/v  data     E x F   (transposed projection weights), diff F x E
+ *   bias_in_q/k/v   data     F
+ *   coeff_out                E x F   (data and diff)
+ *   q, k, v, attention_map   F x L   (data and diff)
+ *   softmax_buffer           n_heads x L x L, row = query, column = key (data and diff)
+ * temp_buffer, grad, sums, maxes, head_buffer, input_bn, bias_out, global_max and
+ * partial_exp_sum are scratch or unused on this path. */
+struct Mhsa_args {
+    struct blob *input;
+    struct blob *input_bn;
+    int n_heads;
+    int opt_matmul_type_fw;
+    int opt_matmul_type_wg;
+    int opt_matmul_type_ig;
+    struct blob *output;
+    struct blob *coeff_in_q;
+    struct blob *coeff_in_k;
+    struct blob *coeff_in_v;
+    struct blob *bias_in_q;
+    struct blob *bias_in_k;
+    struct blob *bias_in_v;
+    struct blob *coeff_out;
+    struct blob *bias_out;
+    struct blob *q;
+    struct blob *k;
+    struct blob *v;
+    struct blob *attention_map;
+    float *temp_buffer;
+    float *grad;
+    struct blob *head_buffer;
+    struct blob *softmax_buffer;
+    float *global_max;
+    float *partial_exp_sum;
+    float *maxes;
+    float *sums;
+};
+
 #ifdef __cplusplus
 }
 #endif

@@ -38,6 +38,18 @@ def load():
         f = getattr(lib, "orc_vect_sum_%s" % dt)
         f.argtypes = [ctypes.c_void_p] * 3 + [ctypes.c_int]
         f.restype = None
+    for n in ("orc_mhsa_fw_fp32", "orc_mhsa_bw_fp32"):
+        f = getattr(lib, n)
+        f.argtypes = [ctypes.c_void_p, ctypes.c_int]
+        f.restype = None
+    for n in ("orc_softmax_fw_fp32", "orc_softmax_bw_fp32"):
+        f = getattr(lib, n)
+        f.argtypes = [ctypes.c_void_p]
+        f.restype = None
+    for n in ("orc_fastexp_gist", "orc_q_rsqrt"):
+        f = getattr(lib, n)
+        f.argtypes = [ctypes.c_float]
+        f.restype = ctypes.c_float
     lib.orc_num_threads.restype = ctypes.c_int
     lib.orc_set_num_threads.argtypes = [ctypes.c_int]
     _lib = lib

@@ -44,13 +44,15 @@ VOID_ENTRY_POINTS = [
     "transpose_matrix", "transpose", "copy", "set_to_value", "vect_sum", "cast_fp16_tensor_to_fp32", "HWC_to_CHW",
     "CHW_to_HWC", "pad_tensor", "transpose_matrix_fp16", "transpose_fp16", "copy_fp16", "set_to_value_fp16",
     "vect_sum_fp16", "cast_fp32_tensor_to_fp16", "HWC_to_CHW_fp16", "CHW_to_HWC_fp16", "pad_tensor_fp16",
+    "pulp_mhsa_fp32_fw_cl", "pulp_mhsa_fp32_bw_cl", "pulp_softmax_fp32_fw_cl", "pulp_softmax_fp32_bw_cl",
 ]
 
 # `int f(const args *, int nsamples)` batched launchers.
 BATCHED_ENTRY_POINTS = ["ptl_%s_%s_%s_batched" % (layer, dt, step)
                         for layer in ("conv2d", "conv_pw", "conv_dw", "linear")
                         for dt in ("fp32", "fp16") for step in ("fw", "wg", "ig")] + [
-                            "ptl_linear_fp32_bw_batched", "ptl_linear_fp16_bw_batched"]
+                            "ptl_linear_fp32_bw_batched", "ptl_linear_fp16_bw_batched",
+                            "ptl_mhsa_fp32_fw_batched", "ptl_mhsa_fp32_bw_batched"]
 
 OTHER_ENTRY_POINTS = ["ptl_init", "ptl_last_error", "ptl_last_status", "ptl_set_stream", "ptl_sync", "ptl_set_gemm_path",
                       "ptl_last_conv_direct", "ptl_timer_begin", "ptl_timer_end_ms", "ptl_mm_fp32", "ptl_mm_fp16", "ptl_copy_bytes"]

@@ -15,6 +15,8 @@ int ptl_internal_bias_add_fp16(fp16 *mat, const fp16 *bias, int N, int M, int pe
 /* out[i] = sum_k mat[i*K + k] */
 int ptl_internal_rowsum_fp32(const float *mat, float *out, int N, int K);
 int ptl_internal_rowsum_fp16(const fp16 *mat, fp16 *out, int N, int K);
+/* Row softmax with the approximate exponential (backward = 0) or its gradient (backward = 1). */
+int ptl_internal_softmax_fp32(const struct softmax_args *a, int backward);
 #ifdef __cplusplus
 }
 #endif

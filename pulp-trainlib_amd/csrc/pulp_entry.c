@@ -446,3 +446,11 @@ void naive_conv2d_in_grad_kernel_CHW_fp16(void *p) {
     in.diff = m->A; w.data = m->B; out.diff = m->C;
     ptl_internal_set_status(ptl_conv2d_fp16_ig_batched(&a, 1));
 }
+
+/* ---- Multi-head self-attention (lib/sources/pulp_mhsa_fp32.c:20, :648) and the row softmax
+ * (lib/sources/pulp_act_fp32.c:187, :335) ------------------------------------------------- */
+
+void pulp_mhsa_fp32_fw_cl(void *p) { ptl_internal_set_status(ptl_mhsa_fp32_fw_batched(p, 1)); }
+void pulp_mhsa_fp32_bw_cl(void *p) { ptl_internal_set_status(ptl_mhsa_fp32_bw_batched(p, 1)); }
+void pulp_softmax_fp32_fw_cl(void *p) { ptl_internal_set_status(ptl_internal_softmax_fp32(p, 0)); }
+void pulp_softmax_fp32_bw_cl(void *p) { ptl_internal_set_status(ptl_internal_softmax_fp32(p, 1)); }

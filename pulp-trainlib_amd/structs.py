@@ -113,6 +113,20 @@ class LinearArgs(C.Structure):
                 ("opt_matmul_type_ig", I), ("use_biases", I)]
 
 
+class SoftmaxArgs(C.Structure):
+    _fields_ = [("input_data", P), ("input_diff", P), ("output_data", P), ("output_diff", P), ("H", I), ("W", I),
+                ("L", I), ("n_heads", I), ("global_max", P), ("partial_exp_sum", P), ("maxes", P), ("sums", P)]
+
+
+class MhsaArgs(C.Structure):
+    _fields_ = [("input", BlobP), ("input_bn", BlobP), ("n_heads", I), ("opt_matmul_type_fw", I),
+                ("opt_matmul_type_wg", I), ("opt_matmul_type_ig", I), ("output", BlobP), ("coeff_in_q", BlobP),
+                ("coeff_in_k", BlobP), ("coeff_in_v", BlobP), ("bias_in_q", BlobP), ("bias_in_k", BlobP),
+                ("bias_in_v", BlobP), ("coeff_out", BlobP), ("bias_out", BlobP), ("q", BlobP), ("k", BlobP),
+                ("v", BlobP), ("attention_map", BlobP), ("temp_buffer", P), ("grad", P), ("head_buffer", BlobP),
+                ("softmax_buffer", BlobP), ("global_max", P), ("partial_exp_sum", P), ("maxes", P), ("sums", P)]
+
+
 LAYER_CONV2D, LAYER_DW_CONV, LAYER_PW_CONV, LAYER_LINEAR = 0, 1, 2, 3
 STEP_FW, STEP_WGT_GRAD, STEP_IN_GRAD = 0, 1, 2
 

@@ -126,3 +126,49 @@ def mm_args(pkg, A, B, Cm, N, M, K, trans_B):
 
 def conv_out(n, k, p0, p1, s):
     return (n - k + p0 + p1) // s + 1
+
+
+MHSA_TENSORS = ("x", "wq", "wk", "wv", "bq", "bk", "bv", "wo", "q", "k", "v", "att", "p", "y")
+
+
+def mhsa_shapes(ns, L, E, F, heads):
+    """Shapes of the attention tensors (data and diff alike; weight gradients of wq/wk/wv are F x E)."""
+    return {"x": (ns, E, L), "wq": (E, F), "wk": (E, F), "wv": (E, F), "bq": (F,), "bk": (F,), "bv": (F,),
+            "wo": (E, F), "q": (ns, F, L), "k": (ns, F, L), "v": (ns, F, L), "att": (ns, F, L),
+            "p": (ns, heads, L, L), "y": (ns, E, L)}
+
+
+def mhsa_args(pkg, data, diff, L, E, F, heads):
+    """Mhsa_args over dicts of tensors keyed like MHSA_TENSORS (missing entries -> NULL), blob geometry as in
+    tests/test_mhsa_fp32/net.c of the reference (input H = L, W = E; attention_map W = F)."""
+    keep = Keep()
+    geo = {"x": (1, L, E), "wq": (1, F, E), "wk": (1, F, E), "wv": (1, F, E), "bq": (1, 1, F), "bk": (1, 1, F),
+           "bv": (1, 1, F), "wo": (1, E, F), "q": (1, L, F), "k": (1, L, F), "v": (1, L, F), "att": (1, L, F),
+           "p": (1, heads, L * L), "y": (1, L, E)}
+    blobs = {}
+    for n in MHSA_TENSORS:
+        c, h, w = geo[n]
+        blobs[n] = pkg.blob(data.get(n), diff.get(n), c, h, w)
+        keep += [blobs[n], data.get(n), diff.get(n)]
+    a = pkg.MhsaArgs()
+    a.input, a.output = ptr(blobs["x"]), ptr(blobs["y"])
+    a.n_heads = heads
+    a.coeff_in_q, a.coeff_in_k, a.coeff_in_v = ptr(blobs["wq"]), ptr(blobs["wk"]), ptr(blobs["wv"])
+    a.bias_in_q, a.bias_in_k, a.bias_in_v = ptr(blobs["bq"]), ptr(blobs["bk"]), ptr(blobs["bv"])
+    a.coeff_out = ptr(blobs["wo"])
+    a.q, a.k, a.v = ptr(blobs["q"]), ptr(blobs["k"]), ptr(blobs["v"])
+    a.attention_map, a.softmax_buffer = ptr(blobs["att"]), ptr(blobs["p"])
+    return a, keep
+
+
+def mhsa_inputs(seed, ns, L, E, F, heads):
+    """Seeded inputs: tokens N(0,1), Xavier-uniform weights, small biases, output gradient U[-1,1]."""
+    sh = mhsa_shapes(ns, L, E, F, heads)
+    lim = float(np.sqrt(6.0 / (E + F)))
+    d = {"x": normal(seed, sh["x"])}
+    for i, n in enumerate(("wq", "wk", "wv", "wo")):
+        d[n] = uniform(seed + 1 + i, sh[n], -lim, lim)
+    for i, n in enumerate(("bq", "bk", "bv")):
+        d[n] = uniform(seed + 11 + i, sh[n], -0.1, 0.1)
+    dy = uniform(seed + 21, sh["y"])
+    return d, dy
