@@ -17,6 +17,8 @@
 #include <float.h>
 
 #include "ptl_api.h"
+#include "ptl_gemm_async.hpp"
+#include "ptl_gemm_async.inc"
 #include "ptl_host.hpp"
 #include "ptl_internal.h"
 #include "ptl_structs.h"
@@ -146,6 +148,221 @@ __device__ inline void mix_from_lds(const float *__restrict__ V, const float *S,
     }
 }
 
+// ---------------------------------------------------------------------------------------------------------
+// Tile loader: element (i, j), i < nrows, j < ncols (a multiple of 4), comes from g[i*gstride + j] when
+// i < rvalid and j < cvalid and is zero otherwise; it lands at lds[i*pitch + j].  Each lane moves four
+// consecutive columns with one 16-byte LDS-DMA load (global addresses need only 4-byte alignment, so rows of
+// odd length are fine); a vector that straddles the end of a row is left to tile_edge_load/store, so
+// nothing is ever read outside [0, rvalid) x [0, cvalid).  Two shapes: 32-column tiles stored with pitch 32
+// (eight rows per instruction) and long rows (up to 256 columns per instruction, any pitch that is a multiple
+// of 4).  Work is dealt to the NW waves of the workgroup; completion = the caller's vmcnt wait + barrier.
+template <int NW>
+__device__ inline void tile_dma(const float *__restrict__ g, long long gstride, int nrows, int ncols, int rvalid,
+                                int cvalid, float *lds, int pitch, const float *zero, int wave, int lane) {
+    const unsigned lds_addr = (unsigned)(uintptr_t)(lds_char *)lds;
+    int ninstr, rows_per, lanes_per_row, segs;
+    if (ncols == 32 && pitch == 32) {
+        rows_per = 8;
+        lanes_per_row = 8;
+        segs = 1;
+        ninstr = (nrows + 7) >> 3;
+    } else {
+        rows_per = 1;
+        lanes_per_row = 64;
+        segs = (ncols + 255) >> 8;
+        ninstr = nrows * segs;
+    }
+    for (int j = wave; j < ninstr; j += NW) {
+        int i, col;
+        unsigned m0;
+        if (rows_per == 8) {
+            i = j * 8 + (lane >> 3);
+            col = (lane & 7) * 4;
+            m0 = lds_addr + (unsigned)j * 1024u;
+        } else {
+            const int seg = j % segs;
+            i = j / segs;
+            col = seg * 256 + lane * 4;
+            m0 = lds_addr + ((unsigned)i * pitch + seg * 256) * 4u;
+        }
+        if (i >= nrows || col >= ncols) continue;
+        const bool row_ok = i < rvalid;
+        const bool full = row_ok && col + 4 <= cvalid;
+        if (row_ok && !full && col < cvalid) continue;  // straddles the end of the row: second pass
+        lds_dma<16>(full ? g + (long long)i * gstride + col : zero, m0);
+    }
+}
+
+// The vector of a tile row that straddles the end of the valid columns (at most one per row): thread `tid`
+// of the workgroup loads the one of row `tid` with element loads, and stores it once every tile of the volley
+// has been enqueued, so that all these loads are in flight together.  Tiles have at most 256 rows.
+struct TileEdge {
+    float4 v;
+    float *dst;
+};
+
+__device__ inline TileEdge tile_edge_load(const float *__restrict__ g, long long gstride, int nrows, int ncols,
+                                          int rvalid, int cvalid, float *lds, int pitch, int tid) {
+    TileEdge e;
+    e.dst = nullptr;
+    e.v = make_float4(0.f, 0.f, 0.f, 0.f);
+    const int pcol = cvalid & ~3;
+    if ((cvalid & 3) && pcol < ncols && tid < nrows && tid < rvalid) {
+        const float *src = g + (long long)tid * gstride + pcol;
+        e.v.x = src[0];
+        if (pcol + 1 < cvalid) e.v.y = src[1];
+        if (pcol + 2 < cvalid) e.v.z = src[2];
+        e.dst = lds + (size_t)tid * pitch + pcol;
+    }
+    return e;
+}
+
+__device__ inline void tile_edge_store(const TileEdge &e) {
+    if (e.dst) *reinterpret_cast<float4 *>(e.dst) = e.v;
+}
+
+// ---------------------------------------------------------------------------------------------------------
+// Panel product for the projections and their gradients.
+//
+//   C[n][m] (+)= bias[n] + sum over terms t, samples b (gradient mode) and k of A_t(n,k) * B_t(m,k)
+//
+// where A_t(n,k) sits at A_t + b*a_s + n*a_n + k*a_k (B alike) and one of the two strides of each operand
+// is 1.  The whole 32-row x <=200-deep panel of each operand goes from global memory to LDS in one volley of
+// LDS-DMA loads, all in flight together: one trip to memory per panel.  The four waves split the contraction
+// in groups of eight k and meet in LDS.  LDS layouts: [k][32 rows] when rows are contiguous in memory
+// (fragment = four 4-byte reads, lanes along rows), [row][k] with a pitch of 204 floats (an odd number of
+// 16-byte units) when k is (fragment = one 16-byte read); both are free of bank conflicts.
+constexpr int PG_KC = 200;          // contraction depth of a panel (multiple of 8)
+constexpr int PG_P = PG_KC + 4;     // pitch of the [row][k] layout
+constexpr int PG_PANEL = 32 * PG_P; // floats per operand panel (the [k][32] layout needs 32 * PG_KC)
+
+struct PanelArgs {
+    const float *A[3], *B[3];  // operands of term t (fan-in) or output o (fan-out)
+    float *C[3];
+    const float *bias[3];
+    const float *zero;         // source of elements that do not exist
+    float *part;               // partial sums [nout][groups][N][M] when groups > 1
+    int nout, nterm;
+    int N, M, K;
+    int a_n, a_k, b_m, b_k;
+    long long a_s, b_s, c_s;   // per-sample element strides
+    int c_n;                   // output row stride (columns contiguous)
+    int ns;
+    int sum_samples;           // 1: the contraction also runs over the samples (weight gradients)
+    int spg, groups;           // samples per workgroup and number of sample groups in that mode
+    int accumulate;            // 1: add to what C holds
+};
+
+// Panel of rows [r0, r0+32) x k [k0, k0+PG_KC) of an operand with row stride s_r and k stride s_k.
+template <bool KMAJ>
+__device__ inline TileEdge panel_load(const float *g, int s_r, int s_k, int r0, int R, int k0, int K, float *lds,
+                                      const float *zero, int tid, int wave, int lane) {
+    if (KMAJ) {
+        const float *t = g + (long long)r0 * s_r + k0;
+        tile_dma<4>(t, s_r, 32, PG_KC, R - r0, K - k0, lds, PG_P, zero, wave, lane);
+        return tile_edge_load(t, s_r, 32, PG_KC, R - r0, K - k0, lds, PG_P, tid);
+    }
+    const float *t = g + (long long)k0 * s_k + r0;
+    tile_dma<4>(t, s_k, PG_KC, 32, K - k0, R - r0, lds, 32, zero, wave, lane);
+    return tile_edge_load(t, s_k, PG_KC, 32, K - k0, R - r0, lds, 32, tid);
+}
+
+// The four k values [k4, k4+4) of row r.
+template <bool KMAJ>
+__device__ inline float4 panel_frag(const float *lds, int r, int k4) {
+    if (KMAJ) return *reinterpret_cast<const float4 *>(lds + r * PG_P + k4);
+    float4 v;
+    v.x = lds[k4 * 32 + r];
+    v.y = lds[(k4 + 1) * 32 + r];
+    v.z = lds[(k4 + 2) * 32 + r];
+    v.w = lds[(k4 + 3) * 32 + r];
+    return v;
+}
+
+__device__ inline void mfma4(mh_f32x16 &acc, const float4 &a, const float4 &b) {
+    acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a.x, b.x, acc, 0, 0, 0);
+    acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a.y, b.y, acc, 0, 0, 0);
+    acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a.z, b.z, acc, 0, 0, 0);
+    acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a.w, b.w, acc, 0, 0, 0);
+}
+
+template <bool A_KMAJ, bool B_KMAJ>
+__global__ __launch_bounds__(ATT_NT) void panel_gemm_kernel(PanelArgs a) {
+    extern __shared__ __attribute__((aligned(16))) float pg_lds[];
+    float *As = pg_lds, *Bs = pg_lds + PG_PANEL;
+    const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int l32 = lane & 31, half = lane >> 5;
+    const int m0 = blockIdx.x * 32, n0 = blockIdx.y * 32;
+    int o, b_first, b_count, grp = 0;
+    if (a.sum_samples) {
+        o = blockIdx.z / a.groups;
+        grp = blockIdx.z % a.groups;
+        b_first = grp * a.spg;
+        b_count = min(a.spg, a.ns - b_first);
+    } else {
+        o = blockIdx.z / a.ns;
+        b_first = blockIdx.z % a.ns;
+        b_count = 1;
+    }
+    mh_f32x16 acc = {0};
+    for (int bi = 0; bi < b_count; ++bi)
+        for (int t = 0; t < a.nterm; ++t) {
+            const float *Ag = a.A[o * a.nterm + t] + (long long)(b_first + bi) * a.a_s;
+            const float *Bg = a.B[o * a.nterm + t] + (long long)(b_first + bi) * a.b_s;
+            for (int k0 = 0; k0 < a.K; k0 += PG_KC) {
+                __syncthreads();  // the previous panels have been consumed
+                const TileEdge ea = panel_load<A_KMAJ>(Ag, a.a_n, a.a_k, n0, a.N, k0, a.K, As, a.zero, tid, wave, lane);
+                const TileEdge eb = panel_load<B_KMAJ>(Bg, a.b_m, a.b_k, m0, a.M, k0, a.K, Bs, a.zero, tid, wave, lane);
+                tile_edge_store(ea);
+                tile_edge_store(eb);
+                wait_vmcnt<0>();
+                __syncthreads();
+                // groups of eight k (beyond the valid depth the panels hold zeros), dealt to the waves in runs;
+                // within a group the lower half-wave takes k 0..3 and the upper 4..7
+                const int ngroups = (min(PG_KC, a.K - k0) + 7) >> 3;
+                const int per = (ngroups + 3) >> 2;
+                const int g_end = min(ngroups, (wave + 1) * per);
+                for (int gq = wave * per; gq < g_end; ++gq) {
+                    const int k4 = gq * 8 + half * 4;
+                    mfma4(acc, panel_frag<A_KMAJ>(As, l32, k4), panel_frag<B_KMAJ>(Bs, l32, k4));
+                }
+            }
+        }
+    __syncthreads();
+    float *red = pg_lds;
+#pragma unroll
+    for (int v = 0; v < 16; ++v) red[(wave * 32 + 8 * (v / 4) + 4 * half + (v % 4)) * ATT_RP + l32] = acc[v];
+    __syncthreads();
+    const bool partial = a.sum_samples && a.groups > 1;
+    float *Cb = partial ? a.part + ((size_t)o * a.groups + grp) * a.N * a.M
+                        : a.C[o] + (a.sum_samples ? 0 : (long long)b_first * a.c_s);
+    const int c_n = partial ? a.M : a.c_n;
+    const float *bias = partial ? nullptr : a.bias[o];
+    for (int idx = tid; idx < 1024; idx += ATT_NT) {
+        const int n = idx >> 5, m = idx & 31;
+        float v = ((red[n * ATT_RP + m] + red[(32 + n) * ATT_RP + m]) + red[(64 + n) * ATT_RP + m]) +
+                  red[(96 + n) * ATT_RP + m];
+        if (n0 + n < a.N && m0 + m < a.M) {
+            float *dst = Cb + (size_t)(n0 + n) * c_n + m0 + m;
+            if (bias) v = v + bias[n0 + n];
+            if (a.accumulate && !partial) v = *dst + v;
+            *dst = v;
+        }
+    }
+}
+
+// C_o[i] = sum over groups of part[o][g][i]   (+ what C holds when accumulate)
+__global__ __launch_bounds__(256) void panel_reduce_kernel(PanelArgs a) {
+    const size_t nm = (size_t)a.N * a.M, i = (size_t)blockIdx.x * 256 + threadIdx.x;
+    if (i >= nm) return;
+    const int o = blockIdx.y;
+    const float *p = a.part + (size_t)o * a.groups * nm + i;
+    float s = 0.f;
+    for (int g = 0; g < a.groups; ++g) s += p[(size_t)g * nm];
+    float *dst = a.C[o] + (i / a.M) * a.c_n + (i % a.M);
+    *dst = a.accumulate ? *dst + s : s;
+}
+
 struct AttnArgs {
     const float *q, *k, *v;  // [ns][F][L]
     const float *p;          // probabilities [ns][heads][L][L]   (backward)
@@ -153,6 +370,7 @@ struct AttnArgs {
     const float *dp;         // probability gradient               (backward II)
     const float *rs;         // row sums of dP.P [ns][heads][L]    (backward II)
     float *o0, *o1, *o2;     // kernel outputs (see each kernel)
+    const float *zero;       // 256 zero bytes: source of elements that do not exist
     int L, H, heads, F, LP;
     float scale;
 };
@@ -321,24 +539,280 @@ __global__ __launch_bounds__(ATT_NT) void attn_bw_key_kernel(AttnArgs a) {
     }
 }
 
-// mat[b][f][l] += bias[f] for the three projections at once (mm_bias_add_transposed, per-row branch,
-// lib/sources/pulp_train_utils_fp32.c:1286; lib/sources/pulp_mhsa_fp32.c:150-325).
-__global__ __launch_bounds__(256) void mhsa_bias3_kernel(float *q, float *k, float *v, const float *bq,
-                                                          const float *bk, const float *bv, size_t total, int F,
-                                                          int L) {
-    size_t idx = (size_t)blockIdx.x * 256 + threadIdx.x;
-    if (idx >= total) return;
-    const int f = (int)((idx / L) % F);
-    float *m = blockIdx.y == 0 ? q : blockIdx.y == 1 ? k : v;
-    const float *bias = blockIdx.y == 0 ? bq : blockIdx.y == 1 ? bk : bv;
-    if (bias) m[idx] = m[idx] + bias[f];
+// ---------------------------------------------------------------------------------------------------------
+// Resident variants for sequences of at most 200 tokens and head sizes of 33..64 (ViT geometry): everything a
+// workgroup needs comes in by LDS-DMA in one volley at its start (a single trip to memory instead of one per
+// phase), and all fragments are read from LDS.  Eight waves per workgroup (one workgroup per CU: the panels
+// take 150 KB), so that every SIMD has a second wave to run while one waits.
+constexpr int RS_NW = 8;            // waves
+constexpr int RS_NT = RS_NW * 64;   // threads
+constexpr int RS_RPW = 32 / RS_NW;  // score rows per wave
+constexpr int RS_KS = RS_NW / 2;    // contraction ranges of the token-contracting products
+constexpr int RS_LC = 224;  // key columns covered: 7 blocks of 32
+constexpr int RS_KD = 200;  // contraction depth over tokens (25 groups of 8)
+constexpr int RS_KP = 232;  // pitch of a [d][token] panel read with lanes along tokens (4 rows apart = 32 banks)
+constexpr int RS_VP = 204;  // pitch of a [d][token] panel read as 16-byte fragments along tokens
+constexpr int RS_SP = 228;  // pitch of the [32][token] score tile (16-byte fragments along tokens)
+constexpr int RS_FW_FLOATS = 64 * 32 + 64 * RS_KP + 64 * RS_VP + 32 * RS_SP;
+constexpr int RS_KEY_FLOATS = 2 * 64 * RS_VP + 2 * RS_KD * 32 + RS_KD;
+static_assert(RS_NW * 32 * ATT_RP <= 64 * 32 + 64 * RS_KP, "parked accumulators fit the first two panels");
+
+// S[r][c] = scale * sum_d Rs[d][r] * Cs[d][c]: Rs is [64][32], Cs [64][RS_KP], both in LDS; one 32-column
+// block per wave.
+__device__ inline void scores_resident(const float *Rs, const float *Cs, int CB, float scale, float *S, int wave,
+                                       int l32, int half) {
+    for (int cb = wave; cb < CB; cb += RS_NW) {
+        mh_f32x16 acc = {0};
+#pragma unroll
+        for (int g = 0; g < 8; ++g) {
+            const int d4 = g * 8 + half * 4;
+            float4 x, y;
+            x.x = Rs[d4 * 32 + l32];
+            x.y = Rs[(d4 + 1) * 32 + l32];
+            x.z = Rs[(d4 + 2) * 32 + l32];
+            x.w = Rs[(d4 + 3) * 32 + l32];
+            const float *cp = Cs + d4 * RS_KP + cb * 32 + l32;
+            y.x = cp[0];
+            y.y = cp[RS_KP];
+            y.z = cp[2 * RS_KP];
+            y.w = cp[3 * RS_KP];
+            mfma4(acc, x, y);
+        }
+#pragma unroll
+        for (int v = 0; v < 16; ++v) S[(8 * (v / 4) + 4 * half + (v % 4)) * RS_SP + cb * 32 + l32] = acc[v] * scale;
+    }
 }
 
-// dx += tq + tk + tv in the reference's order (lib/sources/pulp_mhsa_fp32.c:1634-1745).
-__global__ __launch_bounds__(256) void mhsa_sum3_kernel(float *dx, const float *t, size_t n) {
-    size_t idx = (size_t)blockIdx.x * 256 + threadIdx.x;
-    if (idx >= n) return;
-    dx[idx] = ((dx[idx] + t[idx]) + t[n + idx]) + t[2 * n + idx];
+// Parked partial tiles of the RS_KS contraction ranges -> out[d][x0 + x] (d < H, x0 + x < L).
+__device__ inline void mix_store(const float *red, int L, int H, int x0, float *__restrict__ out, int tid) {
+    for (int idx = tid; idx < 64 * 32; idx += RS_NT) {
+        const int d = idx >> 5, xx = idx & 31;
+        float s = 0.f;
+#pragma unroll
+        for (int k2 = 0; k2 < RS_KS; ++k2) s += red[((2 * k2 + (d >> 5)) * 32 + (d & 31)) * ATT_RP + xx];
+        if (d < H && x0 + xx < L) out[(size_t)d * L + x0 + xx] = s;
+    }
+}
+
+// out[d][r0 + r] = sum_c Vs[d][c] * S[r][c] (d < H): Vs [64][RS_VP] and S [32][RS_SP] in LDS, S zero beyond L.
+// Waves: (block of 32 d) x (range of the contraction); the ranges meet in `red`.
+__device__ inline void mix_resident(const float *Vs, const float *S, int L, int H, int r0, float *__restrict__ out,
+                                    float *red, int tid, int wave, int l32, int half) {
+    const int db = wave & 1, ks = wave >> 1;
+    const int ngroups = (L + 7) >> 3, per = (ngroups + RS_KS - 1) / RS_KS;
+    const int g_end = min(ngroups, (ks + 1) * per);
+    mh_f32x16 acc = {0};
+    for (int g = ks * per; g < g_end; ++g) {
+        const int k4 = g * 8 + half * 4;
+        mfma4(acc, *reinterpret_cast<const float4 *>(Vs + (db * 32 + l32) * RS_VP + k4),
+              *reinterpret_cast<const float4 *>(S + l32 * RS_SP + k4));
+    }
+#pragma unroll
+    for (int v = 0; v < 16; ++v) red[(wave * 32 + 8 * (v / 4) + 4 * half + (v % 4)) * ATT_RP + l32] = acc[v];
+    __syncthreads();
+    mix_store(red, L, H, r0, out, tid);
+}
+
+__global__ __launch_bounds__(RS_NT) void attn_fw_res_kernel(AttnArgs a) {
+    extern __shared__ __attribute__((aligned(16))) float att_lds[];
+    float *Qs = att_lds, *Ks = Qs + 64 * 32, *Vs = Ks + 64 * RS_KP, *S = Vs + 64 * RS_VP, *red = att_lds;
+    const int r0 = blockIdx.x * 32, h = blockIdx.y, b = blockIdx.z, L = a.L;
+    const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int l32 = lane & 31, half = lane >> 5;
+    const size_t hoff = ((size_t)b * a.F + (size_t)h * a.H) * L;
+    tile_dma<RS_NW>(a.q + hoff + r0, L, 64, 32, a.H, L - r0, Qs, 32, a.zero, wave, lane);
+    tile_dma<RS_NW>(a.k + hoff, L, 64, RS_LC, a.H, L, Ks, RS_KP, a.zero, wave, lane);
+    tile_dma<RS_NW>(a.v + hoff, L, 64, RS_KD, a.H, L, Vs, RS_VP, a.zero, wave, lane);
+    const TileEdge e0 = tile_edge_load(a.q + hoff + r0, L, 64, 32, a.H, L - r0, Qs, 32, tid);
+    const TileEdge e1 = tile_edge_load(a.k + hoff, L, 64, RS_LC, a.H, L, Ks, RS_KP, tid);
+    const TileEdge e2 = tile_edge_load(a.v + hoff, L, 64, RS_KD, a.H, L, Vs, RS_VP, tid);
+    tile_edge_store(e0);
+    tile_edge_store(e1);
+    tile_edge_store(e2);
+    wait_vmcnt<0>();
+    __syncthreads();
+    scores_resident(Qs, Ks, (L + 31) >> 5, a.scale, S, wave, l32, half);
+    __syncthreads();
+    // softmax of this wave's rows over the keys (lib/sources/pulp_act_fp32.c:187-225): max, approximate
+    // exponential of the difference, sum, division; the rows' reductions run side by side
+    float *P = a.o0 + ((size_t)b * a.heads + h) * L * L;
+    float sv[RS_RPW][4], mx[RS_RPW], sum[RS_RPW];
+#pragma unroll
+    for (int i = 0; i < RS_RPW; ++i) {
+        const float *srow = S + (wave * RS_RPW + i) * RS_SP;
+        mx[i] = -FLT_MAX;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const int c = lane + 64 * j;
+            sv[i][j] = c < L ? srow[c] : -FLT_MAX;
+            mx[i] = fmaxf(mx[i], sv[i][j]);
+        }
+    }
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1)
+#pragma unroll
+        for (int i = 0; i < RS_RPW; ++i) mx[i] = fmaxf(mx[i], __shfl_xor(mx[i], o));
+#pragma unroll
+    for (int i = 0; i < RS_RPW; ++i) {
+        sum[i] = 0.f;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const int c = lane + 64 * j;
+            sv[i][j] = c < L ? fastexp_gist(sv[i][j] - mx[i]) : 0.f;
+            sum[i] += sv[i][j];
+        }
+    }
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1)
+#pragma unroll
+        for (int i = 0; i < RS_RPW; ++i) sum[i] += __shfl_xor(sum[i], o);
+#pragma unroll
+    for (int i = 0; i < RS_RPW; ++i) {
+        const int row = wave * RS_RPW + i;
+        float *srow = S + row * RS_SP;
+        const bool live = r0 + row < L;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const int c = lane + 64 * j;
+            if (c < RS_LC) {
+                const float pv = c < L ? sv[i][j] / sum[i] : 0.f;
+                srow[c] = pv;
+                if (live && c < L) P[(size_t)(r0 + row) * L + c] = pv;
+            }
+        }
+    }
+    __syncthreads();
+    mix_resident(Vs, S, L, a.H, r0, a.o1 + hoff, red, tid, wave, l32, half);
+}
+
+__global__ __launch_bounds__(RS_NT) void attn_bw_query_res_kernel(AttnArgs a) {
+    extern __shared__ __attribute__((aligned(16))) float att_lds[];
+    float *Qs = att_lds, *Ks = Qs + 64 * 32, *Vs = Ks + 64 * RS_KP, *S = Vs + 64 * RS_VP, *red = att_lds;
+    const int r0 = blockIdx.x * 32, h = blockIdx.y, b = blockIdx.z, L = a.L;
+    const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int l32 = lane & 31, half = lane >> 5;
+    const size_t hoff = ((size_t)b * a.F + (size_t)h * a.H) * L;
+    const size_t poff = ((size_t)b * a.heads + h) * L * L;
+    tile_dma<RS_NW>(a.da + hoff + r0, L, 64, 32, a.H, L - r0, Qs, 32, a.zero, wave, lane);
+    tile_dma<RS_NW>(a.v + hoff, L, 64, RS_LC, a.H, L, Ks, RS_KP, a.zero, wave, lane);
+    tile_dma<RS_NW>(a.k + hoff, L, 64, RS_KD, a.H, L, Vs, RS_VP, a.zero, wave, lane);
+    const TileEdge e0 = tile_edge_load(a.da + hoff + r0, L, 64, 32, a.H, L - r0, Qs, 32, tid);
+    const TileEdge e1 = tile_edge_load(a.v + hoff, L, 64, RS_LC, a.H, L, Ks, RS_KP, tid);
+    const TileEdge e2 = tile_edge_load(a.k + hoff, L, 64, RS_KD, a.H, L, Vs, RS_VP, tid);
+    // this wave's probability rows ride along in registers
+    float pr[RS_RPW][4];
+#pragma unroll
+    for (int i = 0; i < RS_RPW; ++i)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const int row = r0 + wave * RS_RPW + i, c = lane + 64 * j;
+            pr[i][j] = (row < L && c < L) ? a.p[poff + (size_t)row * L + c] : 0.f;
+        }
+    tile_edge_store(e0);
+    tile_edge_store(e1);
+    tile_edge_store(e2);
+    wait_vmcnt<0>();
+    __syncthreads();
+    // dP[query][key] = sum_d dA[d][query] v[d][key]   (lib/sources/pulp_mhsa_fp32.c:958-1060)
+    scores_resident(Qs, Ks, (L + 31) >> 5, 1.0f, S, wave, l32, half);
+    __syncthreads();
+    // softmax backward (lib/sources/pulp_act_fp32.c:335-390) and the scaling (:1176-1183)
+    float gv[RS_RPW][4], sum[RS_RPW];
+#pragma unroll
+    for (int i = 0; i < RS_RPW; ++i) {
+        const float *srow = S + (wave * RS_RPW + i) * RS_SP;
+        sum[i] = 0.f;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const int c = lane + 64 * j;
+            gv[i][j] = c < L ? srow[c] : 0.f;
+            sum[i] += gv[i][j] * pr[i][j];
+        }
+    }
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1)
+#pragma unroll
+        for (int i = 0; i < RS_RPW; ++i) sum[i] += __shfl_xor(sum[i], o);
+#pragma unroll
+    for (int i = 0; i < RS_RPW; ++i) {
+        const int row = wave * RS_RPW + i;
+        float *srow = S + row * RS_SP;
+        const bool live = r0 + row < L;
+        float *dprow = a.o0 + poff + (size_t)(r0 + row) * L;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const int c = lane + 64 * j;
+            if (c < RS_LC) {
+                if (live && c < L) dprow[c] = gv[i][j];
+                srow[c] = c < L ? ((gv[i][j] - sum[i]) * pr[i][j]) * a.scale : 0.f;
+            }
+        }
+        if (live && lane == 0) a.o2[((size_t)b * a.heads + h) * L + r0 + row] = sum[i];
+    }
+    __syncthreads();
+    // dq[d][query] = sum_key k[d][key] dS[query][key]   (:1342-1360)
+    mix_resident(Vs, S, L, a.H, r0, a.o1 + hoff, red, tid, wave, l32, half);
+}
+
+// Key side: tile of 32 keys; dA and q ([d][query], 16-byte fragments along the queries) and the key columns
+// of P and dP ([query][32 keys]) are resident; dS replaces dP in place before the products.
+//   dv[d][key] = sum_query dA[d][query] P[query][key]                         (:884-902)
+//   dk[d][key] = sum_query q[d][query] dS[query][key], dS = (dP - rs) P scale  (:1244-1330)
+__global__ __launch_bounds__(RS_NT) void attn_bw_key_res_kernel(AttnArgs a) {
+    extern __shared__ __attribute__((aligned(16))) float att_lds[];
+    float *dAs = att_lds, *Qs = dAs + 64 * RS_VP, *Pp = Qs + 64 * RS_VP, *Gp = Pp + RS_KD * 32, *rsl = Gp + RS_KD * 32;
+    float *red = att_lds;
+    const int c0 = blockIdx.x * 32, h = blockIdx.y, b = blockIdx.z, L = a.L, H = a.H;
+    const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int l32 = lane & 31, half = lane >> 5;
+    const size_t hoff = ((size_t)b * a.F + (size_t)h * H) * L;
+    const size_t poff = ((size_t)b * a.heads + h) * L * L;
+    tile_dma<RS_NW>(a.da + hoff, L, 64, RS_KD, H, L, dAs, RS_VP, a.zero, wave, lane);
+    tile_dma<RS_NW>(a.q + hoff, L, 64, RS_KD, H, L, Qs, RS_VP, a.zero, wave, lane);
+    tile_dma<RS_NW>(a.p + poff + c0, L, RS_KD, 32, L, L - c0, Pp, 32, a.zero, wave, lane);
+    tile_dma<RS_NW>(a.dp + poff + c0, L, RS_KD, 32, L, L - c0, Gp, 32, a.zero, wave, lane);
+    const TileEdge e0 = tile_edge_load(a.da + hoff, L, 64, RS_KD, H, L, dAs, RS_VP, tid);
+    const TileEdge e1 = tile_edge_load(a.q + hoff, L, 64, RS_KD, H, L, Qs, RS_VP, tid);
+    const TileEdge e2 = tile_edge_load(a.p + poff + c0, L, RS_KD, 32, L, L - c0, Pp, 32, tid);
+    const TileEdge e3 = tile_edge_load(a.dp + poff + c0, L, RS_KD, 32, L, L - c0, Gp, 32, tid);
+    const float rsv = (tid < RS_KD && tid < L) ? a.rs[((size_t)b * a.heads + h) * L + tid] : 0.f;
+    tile_edge_store(e0);
+    tile_edge_store(e1);
+    tile_edge_store(e2);
+    tile_edge_store(e3);
+    if (tid < RS_KD) rsl[tid] = rsv;
+    wait_vmcnt<0>();
+    __syncthreads();
+    for (int idx = tid; idx < RS_KD * 32; idx += RS_NT) Gp[idx] = ((Gp[idx] - rsl[idx >> 5]) * Pp[idx]) * a.scale;
+    __syncthreads();
+    const int db = wave & 1, ks = wave >> 1;
+    const int ngroups = (L + 7) >> 3, per = (ngroups + RS_KS - 1) / RS_KS;
+    const int g_end = min(ngroups, (ks + 1) * per);
+    mh_f32x16 accv = {0}, acck = {0};
+    for (int g = ks * per; g < g_end; ++g) {
+        const int k4 = g * 8 + half * 4;
+        float4 pb, sb;
+        pb.x = Pp[k4 * 32 + l32];
+        pb.y = Pp[(k4 + 1) * 32 + l32];
+        pb.z = Pp[(k4 + 2) * 32 + l32];
+        pb.w = Pp[(k4 + 3) * 32 + l32];
+        sb.x = Gp[k4 * 32 + l32];
+        sb.y = Gp[(k4 + 1) * 32 + l32];
+        sb.z = Gp[(k4 + 2) * 32 + l32];
+        sb.w = Gp[(k4 + 3) * 32 + l32];
+        mfma4(accv, *reinterpret_cast<const float4 *>(dAs + (db * 32 + l32) * RS_VP + k4), pb);
+        mfma4(acck, *reinterpret_cast<const float4 *>(Qs + (db * 32 + l32) * RS_VP + k4), sb);
+    }
+    float *outs[2] = {a.o0 + hoff, a.o1 + hoff};
+#pragma unroll
+    for (int which = 0; which < 2; ++which) {
+        __syncthreads();
+#pragma unroll
+        for (int v = 0; v < 16; ++v)
+            red[(wave * 32 + 8 * (v / 4) + 4 * half + (v % 4)) * ATT_RP + l32] = which ? acck[v] : accv[v];
+        __syncthreads();
+        mix_store(red, L, H, c0, outs[which], tid);
+    }
 }
 
 // Row softmax over H rows of W (one wave per row).
@@ -431,49 +905,120 @@ static int launch_attn(int which, AttnArgs &a, int ns) {
 }
 
 static int launch_attn_any(int which, AttnArgs &a, int ns) {
+    if (a.L <= RS_KD && a.H > 32 && a.H <= 64) {
+        a.zero = static_cast<const float *>(state().zeros);
+        if (!a.zero) return 2;
+        void (*kern)(AttnArgs) =
+            which == 0 ? attn_fw_res_kernel : which == 1 ? attn_bw_query_res_kernel : attn_bw_key_res_kernel;
+        const size_t lds = (size_t)(which == 2 ? RS_KEY_FLOATS : RS_FW_FLOATS) * sizeof(float);
+        static bool attr_set[3] = {false, false, false};
+        if (!attr_set[which]) {
+            if (!hip_ok(hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
+                                            hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024),
+                        "hipFuncSetAttribute"))
+                return 2;
+            attr_set[which] = true;
+        }
+        dim3 grid((a.L + 31) / 32, a.heads, ns);
+        hipLaunchKernelGGL(kern, grid, dim3(RS_NT), lds, state().stream, a);
+        return hip_ok(hipGetLastError(), "attention launch") ? 0 : 2;
+    }
     if (a.H <= 32) return launch_attn<32>(which, a, ns);
     if (a.H <= 64) return launch_attn<64>(which, a, ns);
     return launch_attn<128>(which, a, ns);
 }
 
-// C[b][n][l] = sum_k A(n,k) * B[b][k][l]: a weight matrix (element (n,k) at n*a_n + k*a_k) against a batch of
-// [K][L] activations.
-static int weight_times_acts(const float *A, int a_n, int a_k, const float *B, float *C, int N, int K, int L,
-                             int ns) {
-    GemmArgs g = {};
-    g.a.HL = g.a.WL = g.b.HL = g.b.WL = 1;
-    g.A = A;
-    g.B = B;
-    g.C = C;
-    g.N = N;
-    g.M = ns * L;
-    g.K = K;
-    g.a.row = axis_plain(N, a_n);
-    g.a.k = axis_plain(K, a_k);
-    g.b.row = axis_two(ns * L, L, K * L, 1);
-    g.b.k = axis_plain(K, L);
-    g.c.n = axis_plain(N, L);
-    g.c.m = axis_two(ns * L, L, N * L, 1);
-    return gemm<float>(g);
+// Sample groups the gradient mode of the panel product uses for `nout` N x M outputs: enough workgroups to
+// fill the chip a few times over.
+static int panel_groups(int nout, int N, int M, int ns) {
+    const long tiles = (long)((N + 31) / 32) * ((M + 31) / 32) * nout;
+    long groups = (4L * state().num_cu + tiles - 1) / tiles;
+    if (groups > ns) groups = ns;
+    return groups < 1 ? 1 : (int)groups;
 }
 
-// C[n][m] = sum over samples and tokens of A[b][n][l] * B[b][m][l] (weight gradients).
-static int acts_times_acts(const float *A, const float *B, float *C, int N, int M, int L, int ns) {
-    GemmArgs g = {};
-    g.a.HL = g.a.WL = g.b.HL = g.b.WL = 1;
-    g.A = A;
-    g.B = B;
-    g.C = C;
-    g.N = N;
-    g.M = M;
-    g.K = ns * L;
-    g.a.row = axis_plain(N, L);
-    g.a.k = axis_two(ns * L, L, N * L, 1);
-    g.b.row = axis_plain(M, L);
-    g.b.k = axis_two(ns * L, L, M * L, 1);
-    g.c.n = axis_plain(N, M);
-    g.c.m = axis_plain(M, 1);
-    return gemm<float>(g);
+static size_t panel_part_floats(int nout, int N, int M, int ns) {
+    const int g = panel_groups(nout, N, M, ns);
+    return g > 1 ? (size_t)nout * g * N * M : 0;
+}
+
+// Launches the panel product; `p` carries operands, strides and sizes, this fills in the rest.  In gradient
+// mode (sum_samples) the partial sums of the sample groups go to `part` and a second kernel adds them.
+static int launch_panel(PanelArgs &p, float *part) {
+    State &st = state();
+    p.zero = static_cast<const float *>(st.zeros);
+    if (!p.zero) return 2;
+    if ((p.a_k != 1 && p.a_n != 1) || (p.b_k != 1 && p.b_m != 1)) {
+        set_error("panel product: operand without a unit stride");
+        return 1;
+    }
+    const bool ak = p.a_k == 1, bk = p.b_k == 1;
+    p.groups = 1;
+    p.spg = p.ns;
+    p.part = nullptr;
+    if (p.sum_samples) {
+        const int groups = panel_groups(p.nout, p.N, p.M, p.ns);
+        if (groups > 1) {
+            p.spg = (p.ns + groups - 1) / groups;
+            p.groups = (p.ns + p.spg - 1) / p.spg;
+            p.part = part;
+            if (!part) return 2;
+        }
+    }
+    void (*kern)(PanelArgs) = ak ? (bk ? panel_gemm_kernel<true, true> : panel_gemm_kernel<true, false>)
+                                 : (bk ? panel_gemm_kernel<false, true> : panel_gemm_kernel<false, false>);
+    const size_t lds = (size_t)2 * PG_PANEL * sizeof(float);  // 52 KB: three workgroups per CU
+    dim3 grid((p.M + 31) / 32, (p.N + 31) / 32, p.sum_samples ? p.nout * p.groups : p.nout * p.ns);
+    if (grid.y > 65535u || grid.z > 65535u) {
+        set_error("panel product: grid too large");
+        return 1;
+    }
+    hipLaunchKernelGGL(kern, grid, dim3(ATT_NT), lds, st.stream, p);
+    if (!hip_ok(hipGetLastError(), "panel product launch")) return 2;
+    if (p.groups > 1) {
+        hipLaunchKernelGGL(panel_reduce_kernel, dim3((unsigned)(((size_t)p.N * p.M + 255) / 256), p.nout), dim3(256),
+                           0, st.stream, p);
+        if (!hip_ok(hipGetLastError(), "panel reduce launch")) return 2;
+    }
+    return 0;
+}
+
+// out[b][N x L] = Wt(N x K) . act[b][K x L]: a weight matrix with element (n,k) at n*a_n + k*a_k against a
+// batch of activations (tokens contiguous).
+static PanelArgs weights_times_acts(int N, int K, int L, int ns, int a_n, int a_k) {
+    PanelArgs p = {};
+    p.nout = p.nterm = 1;
+    p.N = N;
+    p.M = L;
+    p.K = K;
+    p.a_n = a_n;
+    p.a_k = a_k;
+    p.b_m = 1;
+    p.b_k = L;
+    p.b_s = (long long)K * L;
+    p.c_s = (long long)N * L;
+    p.c_n = L;
+    p.ns = ns;
+    return p;
+}
+
+// out[N x M] = sum over samples and tokens of A[b][N x L] . B[b][M x L]^T  (weight gradients).
+static PanelArgs acts_times_acts(int N, int M, int L, int ns) {
+    PanelArgs p = {};
+    p.nout = p.nterm = 1;
+    p.N = N;
+    p.M = M;
+    p.K = L;
+    p.a_n = L;
+    p.a_k = 1;
+    p.a_s = (long long)N * L;
+    p.b_m = L;
+    p.b_k = 1;
+    p.b_s = (long long)M * L;
+    p.c_n = M;
+    p.ns = ns;
+    p.sum_samples = 1;
+    return p;
 }
 
 static bool mhsa_fits(const MhsaDims &m, int ns) {
@@ -511,12 +1056,17 @@ static int mhsa_fw(const Mhsa_args *a, int ns, const char *fn) {
     float *Y = sg.out(a->output->data, xe);
     if (sg.failed()) return 2;
     int rc = 0;
-    // q/k/v[F x L] = W^T . X + bias (weights stored E x F: lib/sources/pulp_mhsa_fp32.c:70-127)
-    for (int j = 0; j < 3 && rc == 0; ++j) rc = weight_times_acts(W[j], 1, F, X, QKV[j], F, E, L, ns);
-    if (rc == 0 && (bias[0] || bias[1] || bias[2])) {
-        hipLaunchKernelGGL(mhsa_bias3_kernel, dim3((unsigned)((fe + 255) / 256), 3), dim3(256), 0, state().stream,
-                           QKV[0], QKV[1], QKV[2], bias[0], bias[1], bias[2], fe, F, L);
-        if (!hip_ok(hipGetLastError(), "bias launch")) rc = 2;
+    {
+        // q/k/v[F x L] = W^T . X + bias in one launch (weights stored E x F: lib/sources/pulp_mhsa_fp32.c:70-325)
+        PanelArgs p = weights_times_acts(F, E, L, ns, 1, F);
+        p.nout = 3;
+        for (int j = 0; j < 3; ++j) {
+            p.A[j] = W[j];
+            p.B[j] = X;
+            p.C[j] = QKV[j];
+            p.bias[j] = bias[j];
+        }
+        rc = launch_panel(p, nullptr);
     }
     if (rc == 0) {
         AttnArgs t = {};
@@ -533,8 +1083,14 @@ static int mhsa_fw(const Mhsa_args *a, int ns, const char *fn) {
         t.scale = q_rsqrt_host((float)m.H);
         rc = launch_attn_any(0, t, ns);
     }
-    // output[E x L] = Wout[E x F] . attention_map (:599-609)
-    if (rc == 0) rc = weight_times_acts(Wo, F, 1, att, Y, E, F, L, ns);
+    if (rc == 0) {
+        // output[E x L] = Wout[E x F] . attention_map (:599-609)
+        PanelArgs p = weights_times_acts(E, F, L, ns, F, 1);
+        p.A[0] = Wo;
+        p.B[0] = att;
+        p.C[0] = Y;
+        rc = launch_panel(p, nullptr);
+    }
     return sg.finish(rc);
 }
 
@@ -571,13 +1127,27 @@ static int mhsa_bw(const Mhsa_args *a, int ns, const char *fn) {
     const float *P = sg.in(a->softmax_buffer->data, pe);
     float *dP = sg.out(a->softmax_buffer->diff, pe);
     if (sg.failed()) return 2;
-    float *tmp = static_cast<float *>(scratch((3 * xe + rows) * sizeof(float)));
-    if (!tmp) return 2;
-    float *rs = tmp + 3 * xe;
+    const size_t p1 = panel_part_floats(1, E, F, ns), p3 = panel_part_floats(3, F, E, ns);
+    float *rs = static_cast<float *>(scratch((rows + (p1 > p3 ? p1 : p3)) * sizeof(float)));
+    if (!rs) return 2;
+    float *part = rs + rows;
     int rc = 0;
-    // dWout[E x F] = dY . att^T (:742-760); datt[F x L] = Wout^T . dY (:816-834)
-    rc = acts_times_acts(dY, att, dWo, E, F, L, ns);
-    if (rc == 0) rc = weight_times_acts(Wo, 1, F, dY, datt, F, E, L, ns);
+    {
+        // dWout[E x F] = sum over samples of dY . att^T (:742-760)
+        PanelArgs p = acts_times_acts(E, F, L, ns);
+        p.A[0] = dY;
+        p.B[0] = att;
+        p.C[0] = dWo;
+        rc = launch_panel(p, part);
+    }
+    if (rc == 0) {
+        // datt[F x L] = Wout^T . dY (:816-834)
+        PanelArgs p = weights_times_acts(F, E, L, ns, 1, F);
+        p.A[0] = Wo;
+        p.B[0] = dY;
+        p.C[0] = datt;
+        rc = launch_panel(p, nullptr);
+    }
     AttnArgs t = {};
     t.q = QKV[0];
     t.k = QKV[1];
@@ -604,15 +1174,28 @@ static int mhsa_bw(const Mhsa_args *a, int ns, const char *fn) {
         t.o2 = nullptr;
         rc = launch_attn_any(2, t, ns);
     }
-    for (int j = 0; j < 3 && rc == 0; ++j) {
-        // dW[F x E] = d{q,k,v} . X^T (:1425-1560); temp[E x L] = W . d{q,k,v} (:1589-1744)
-        rc = acts_times_acts(dQKV[j], X, dW[j], F, E, L, ns);
-        if (rc == 0) rc = weight_times_acts(W[j], F, 1, dQKV[j], tmp + j * xe, E, F, L, ns);
+    if (rc == 0) {
+        // dW_{q,k,v}[F x E] = sum over samples of d{q,k,v} . X^T, one launch (:1425-1560)
+        PanelArgs p = acts_times_acts(F, E, L, ns);
+        p.nout = 3;
+        for (int j = 0; j < 3; ++j) {
+            p.A[j] = dQKV[j];
+            p.B[j] = X;
+            p.C[j] = dW[j];
+        }
+        rc = launch_panel(p, part);
     }
     if (rc == 0) {
-        hipLaunchKernelGGL(mhsa_sum3_kernel, dim3((unsigned)((xe + 255) / 256)), dim3(256), 0, state().stream, dX,
-                           tmp, xe);
-        if (!hip_ok(hipGetLastError(), "sum launch")) rc = 2;
+        // dX[E x L] += W_q . dq + W_k . dk + W_v . dv, one launch (:1589-1745)
+        PanelArgs p = weights_times_acts(E, F, L, ns, F, 1);
+        p.nterm = 3;
+        for (int j = 0; j < 3; ++j) {
+            p.A[j] = W[j];
+            p.B[j] = dQKV[j];
+        }
+        p.C[0] = dX;
+        p.accumulate = 1;
+        rc = launch_panel(p, nullptr);
     }
     return sg.finish(rc);
 }
