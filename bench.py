@@ -282,6 +282,41 @@ def detail_table(pkg, lib, hp, to_dev, timed, check, torch, dev):
         flops = 2.0 * ns * Co * Ci * H * H
         nb = (x.numel() + y.numel() + w.numel()) * 2
         run3("ptl_conv_pw", dt, a, ns, "pointwise 64->128 56x56", flops, (nb, nb, nb), 100 if ns == 1 else 30)
+
+    # larger convolutions, fp16, batched (ResNet-18/50 style layers)
+    for (ns, Ci, Co, H) in ((256, 32, 64, 56), (128, 64, 64, 56), (128, 128, 128, 28), (128, 256, 256, 14)):
+        K, dt = 3, "fp16"
+        x = torch.rand(ns, Ci, H, H, device=dev).to(tdt[dt]) - 0.5
+        w = torch.rand(Co, Ci, K, K, device=dev).to(tdt[dt]) - 0.5
+        dy = torch.rand(ns, Co, H, H, device=dev).to(tdt[dt]) - 0.5
+        y, dx, dw = torch.zeros_like(dy), torch.zeros_like(x), torch.zeros_like(w)
+        a, keep = hp.conv2d_args(pkg, x, dx, w, dw, y, dy, Ci, H, H, Co, K, K, H, H, (1, 1, 1, 1))
+        flops = 2.0 * ns * Co * Ci * K * K * H * H
+        nb = (x.numel() + w.numel() + y.numel()) * es[dt]
+        run3("ptl_conv2d", dt, a, ns, "conv2d %d->%d %dx%d k3 p1" % (Ci, Co, H, H), flops, (nb, nb, nb), 10)
+        del x, w, dy, y, dx, dw
+
+    # config 4: multi-head self-attention step, fp32, L=197 E=192, 3 heads of 64, batch 1 and 32
+    import numpy as np
+    L, E, F, heads = 197, 192, 192, 3
+    for ns in (1, 32):
+        sh = hp.mhsa_shapes(ns, L, E, F, heads)
+        d, dyh = hp.mhsa_inputs(0xC0DE0004, ns, L, E, F, heads)
+        data = {n: to_dev(v) for n, v in d.items()}
+        for n in ("q", "k", "v", "att", "p", "y"):
+            data[n] = torch.zeros(sh[n], device=dev)
+        diff = {n: torch.zeros(sh[n], device=dev) for n in ("x", "q", "k", "v", "att", "p", "wo")}
+        for n in ("wq", "wk", "wv"):
+            diff[n] = torch.zeros((F, E), device=dev)
+        diff["y"] = to_dev(dyh)
+        a, keep = hp.mhsa_args(pkg, data, diff, L, E, F, heads)
+        ref = ctypes.byref(a)
+        f_fw = ns * (4 * 2.0 * F * E * L + heads * 2 * 2.0 * L * L * (F // heads))
+        act = ns * (2 * E * L + 4 * F * L + heads * L * L) * 4 + 4 * E * F * 4  # every tensor of the step once
+        ms = timed(lambda: check(lib.ptl_mhsa_fp32_fw_batched(ref, ns)), 50)
+        add("mhsa L197 E192 3x64 FW N=%d" % ns, "fp32", ms, f_fw, act)
+        ms = timed(lambda: check(lib.ptl_mhsa_fp32_bw_batched(ref, ns)), 50)
+        add("mhsa L197 E192 3x64 BW N=%d" % ns, "fp32", ms, 2 * f_fw, 2 * act)
     return rows
 
 
