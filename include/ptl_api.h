@@ -90,6 +90,41 @@ void pulp_mhsa_fp32_bw_cl(void *Mhsa_args);
 void pulp_softmax_fp32_fw_cl(void *softmax_args);
 void pulp_softmax_fp32_bw_cl(void *softmax_args);
 
+/* Layers around the matmul core in a ResNet-style step.
+ * ReLU: lib/sources/pulp_act_fp32.c:83-129, pulp_act_fp16.c (same structure). */
+void pulp_relu_fp32_fw_cl(void *act_args);
+void pulp_relu_fp32_bw_cl(void *act_args);
+void relu_core_fw_fp32(void *act_args);
+void relu_core_bw_fp32(void *act_args);
+void pulp_relu_fp16_fw_cl(void *act_args_fp16);
+void pulp_relu_fp16_bw_cl(void *act_args_fp16);
+void relu_core_fw_fp16(void *act_args_fp16);
+void relu_core_bw_fp16(void *act_args_fp16);
+/* Residual connection: lib/sources/pulp_residual_fp32.c:26 (output = skip + lout), :59 (skip->diff +=
+ * output->diff unless skip_in_grad), :92 (lout->diff = output->diff); pulp_residual_fp16.c:30, :67, :100. */
+void pulp_residualconn_fp32_fw(void *SkipConn_args);
+void pulp_sumnode_fp32_bw(void *SkipConn_args);
+void pulp_residualconn_fp32_bw(void *SkipConn_args);
+void pulp_residualconn_fp16_fw(void *SkipConn_args_fp16);
+void pulp_sumnode_fp16_bw(void *SkipConn_args_fp16);
+void pulp_residualconn_fp16_bw(void *SkipConn_args_fp16);
+/* Average pooling: lib/sources/pulp_pooling_fp32.c:24, :69; pulp_pooling_fp16.c:24, :69. */
+void pulp_avgpool_fp32_fw_cl(void *pool_args);
+void pulp_avgpool_fp32_bw_cl(void *pool_args);
+void pulp_avgpool_fp16_fw_cl(void *pool_args_fp16);
+void pulp_avgpool_fp16_bw_cl(void *pool_args_fp16);
+/* Cross-entropy over raw logits: lib/sources/pulp_losses_fp32.c:26, :91; pulp_losses_fp16.c:26, :88. */
+void pulp_CrossEntropyLoss(void *loss_args);
+void pulp_CrossEntropyLoss_backward(void *loss_args);
+void pulp_CrossEntropyLoss_fp16(void *loss_args_fp16);
+void pulp_CrossEntropyLoss_backward_fp16(void *loss_args_fp16);
+/* Gradient descent with optional weight decay: lib/sources/pulp_optimizers_fp32.c:26, pulp_optimizers_fp16.c:26. */
+void pulp_gradient_descent_fp32(void *optim_args);
+void pulp_gradient_descent_fp16(void *optim_args_fp16);
+/* Batch normalisation forward: lib/sources/pulp_batchnorm_fp32.c:28-114 (the reference has no backward). */
+void pulp_batch_norm_fp32_fw_cl(void *BatchNorm_args_fp32);
+void pulp_batch_norm_parallelized_fp32_fw_cl(void *BatchNorm_args_fp32);
+
 /* Matmul kernels and their dispatcher.
  * mm / mm_M: lib/sources/pulp_matmul_fp32.c:190, :345
  * mm_fp16 / mm_M_fp16: lib/sources/pulp_matmul_fp16.c:191, :273
@@ -242,6 +277,21 @@ int ptl_linear_fp16_bw_batched(const struct Linear_args_fp16 *a, int nsamples);
  * are shared and their gradients are summed over the samples. */
 int ptl_mhsa_fp32_fw_batched(const struct Mhsa_args *a, int nsamples);
 int ptl_mhsa_fp32_bw_batched(const struct Mhsa_args *a, int nsamples);
+
+/* Batched forms of the layers above: sample b of every activation blob starts b * blob->dim elements
+ * in; the loss takes nsamples target vectors and writes nsamples losses.  step: 0 forward, 1 backward;
+ * for the residual connection 0 forward, 1 sum node backward, 2 residual backward. */
+int ptl_relu_fp32_batched(const struct act_args *a, int nsamples, int step);
+int ptl_relu_fp16_batched(const struct act_args_fp16 *a, int nsamples, int step);
+int ptl_residual_fp32_batched(const struct SkipConn_args *a, int nsamples, int step);
+int ptl_residual_fp16_batched(const struct SkipConn_args_fp16 *a, int nsamples, int step);
+int ptl_avgpool_fp32_batched(const struct pool_args *a, int nsamples, int step);
+int ptl_avgpool_fp16_batched(const struct pool_args_fp16 *a, int nsamples, int step);
+int ptl_cross_entropy_fp32_batched(const struct loss_args *a, int nsamples, int step);
+int ptl_cross_entropy_fp16_batched(const struct loss_args_fp16 *a, int nsamples, int step);
+int ptl_gradient_descent_fp32(const struct optim_args *a);
+int ptl_gradient_descent_fp16(const struct optim_args_fp16 *a);
+int ptl_batch_norm_fp32_fw(const struct BatchNorm_args_fp32 *a);
 
 /* Plain product C[N x M] = A[N x K] * B (B is K x M, or M x K when trans_B),
  * the contract of the reference's mm family, on raw pointers. */

@@ -534,6 +534,106 @@ struct Mhsa_args {
     float *sums;
 };
 
+/* ---- Layers around the matmul core in a ResNet-style training step ---- */
+
+/* Activation (lib/include/pulp_act_fp32.h:27-32, pulp_act_fp16.h:28-33): input->dim elements. */
+struct act_args {
+    struct blob *input;
+    struct blob *output;
+    int H;
+    int W;
+};
+struct act_args_fp16 {
+    struct blob_fp16 *input;
+    struct blob_fp16 *output;
+    int H;
+    int W;
+};
+
+/* Residual connection (lib/include/pulp_residual_fp32.h:50-55, pulp_residual_fp16.h:50-55). */
+struct SkipConn_args {
+    struct blob *skip;
+    struct blob *lout;
+    struct blob *output;
+    int skip_in_grad;
+};
+struct SkipConn_args_fp16 {
+    struct blob_fp16 *skip;
+    struct blob_fp16 *lout;
+    struct blob_fp16 *output;
+    int skip_in_grad;
+};
+
+/* Pooling (lib/include/pulp_pooling_fp32.h:34-41, pulp_pooling_fp16.h:34-41). */
+struct pool_args {
+    struct blob *input;
+    struct blob *output;
+    int Hker;
+    int Wker;
+    int Hstride;
+    int Wstride;
+};
+struct pool_args_fp16 {
+    struct blob_fp16 *input;
+    struct blob_fp16 *output;
+    int Hker;
+    int Wker;
+    int Hstride;
+    int Wstride;
+};
+
+/* Loss (lib/include/pulp_losses_fp32.h:32-36, pulp_losses_fp16.h:33-37): output->data are the logits,
+ * output->diff receives their gradient, target is a one-hot (or soft) vector of output->dim classes. */
+struct loss_args {
+    struct blob *output;
+    float *target;
+    float *wr_loss;
+};
+struct loss_args_fp16 {
+    struct blob_fp16 *output;
+    fp16 *target;
+    fp16 *wr_loss;
+};
+
+/* Gradient descent (lib/include/pulp_optimizers_fp32.h:34-40, pulp_optimizers_fp16.h:35-41). */
+struct optim_args {
+    struct blob *weights;
+    struct blob *biases;
+    float learning_rate;
+    float weight_decay_lambda;
+    int use_biases;
+};
+struct optim_args_fp16 {
+    struct blob_fp16 *weights;
+    struct blob_fp16 *biases;
+    fp16 learning_rate;
+    fp16 weight_decay_lambda;
+    int use_biases;
+};
+
+/* Batch normalisation, forward only (lib/include/pulp_batchnorm_fp32.h:40-66): statistics per channel
+ * over B x H x W; the forward pass reads input, output, weight_data, bias_data, eps and B, C, H, W. */
+struct BatchNorm_args_fp32 {
+    struct blob *input;
+    struct blob *output;
+    struct blob *coeff;
+    struct blob *bias;
+    int batch_size;
+    float *running_mean;
+    float *running_var;
+    float *running_stdev;
+    int freeze_running_params;
+    int skip_wg_grad;
+    int skip_in_grad;
+    float *weight_data;
+    float *bias_data;
+    float *eps;
+    int B;
+    int C;
+    int H;
+    int W;
+};
+
 #ifdef __cplusplus
 }
 #endif

@@ -19,7 +19,7 @@ FLAGS = ["-O3", "-fPIC", "-shared", "-std=gnu99", "-march=x86-64-v3", "-ffp-cont
 
 
 def build():
-    cmd = [CLANG] + FLAGS + [os.path.join(HERE, "ptl_oracle.c"), os.path.join(HERE, "ptl_oracle_mhsa.c"), "-o", LIB,
+    cmd = [CLANG] + FLAGS + [os.path.join(HERE, "ptl_oracle.c"), os.path.join(HERE, "ptl_oracle_mhsa.c"), os.path.join(HERE, "ptl_oracle_glue.c"), "-o", LIB,
                              "-Wl,-rpath,/opt/rocm/lib/llvm/lib", "-lm"]
     res = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
     if res.returncode != 0:

@@ -50,6 +50,16 @@ def load():
         f = getattr(lib, n)
         f.argtypes = [ctypes.c_float]
         f.restype = ctypes.c_float
+    for dt in ("fp32", "fp16"):
+        for n in ("orc_relu", "orc_residual", "orc_avgpool", "orc_cross_entropy"):
+            f = getattr(lib, "%s_%s" % (n, dt))
+            f.argtypes = [ctypes.c_void_p, ctypes.c_int, ctypes.c_int]
+            f.restype = None
+        f = getattr(lib, "orc_gradient_descent_%s" % dt)
+        f.argtypes = [ctypes.c_void_p]
+        f.restype = None
+    lib.orc_batch_norm_fw_fp32.argtypes = [ctypes.c_void_p]
+    lib.orc_batch_norm_fw_fp32.restype = None
     lib.orc_num_threads.restype = ctypes.c_int
     lib.orc_set_num_threads.argtypes = [ctypes.c_int]
     _lib = lib

@@ -45,7 +45,21 @@ VOID_ENTRY_POINTS = [
     "CHW_to_HWC", "pad_tensor", "transpose_matrix_fp16", "transpose_fp16", "copy_fp16", "set_to_value_fp16",
     "vect_sum_fp16", "cast_fp32_tensor_to_fp16", "HWC_to_CHW_fp16", "CHW_to_HWC_fp16", "pad_tensor_fp16",
     "pulp_mhsa_fp32_fw_cl", "pulp_mhsa_fp32_bw_cl", "pulp_softmax_fp32_fw_cl", "pulp_softmax_fp32_bw_cl",
+    "pulp_relu_fp32_fw_cl", "pulp_relu_fp32_bw_cl", "relu_core_fw_fp32", "relu_core_bw_fp32",
+    "pulp_relu_fp16_fw_cl", "pulp_relu_fp16_bw_cl", "relu_core_fw_fp16", "relu_core_bw_fp16",
+    "pulp_residualconn_fp32_fw", "pulp_sumnode_fp32_bw", "pulp_residualconn_fp32_bw",
+    "pulp_residualconn_fp16_fw", "pulp_sumnode_fp16_bw", "pulp_residualconn_fp16_bw",
+    "pulp_avgpool_fp32_fw_cl", "pulp_avgpool_fp32_bw_cl", "pulp_avgpool_fp16_fw_cl", "pulp_avgpool_fp16_bw_cl",
+    "pulp_CrossEntropyLoss", "pulp_CrossEntropyLoss_backward", "pulp_CrossEntropyLoss_fp16",
+    "pulp_CrossEntropyLoss_backward_fp16", "pulp_gradient_descent_fp32", "pulp_gradient_descent_fp16",
+    "pulp_batch_norm_fp32_fw_cl", "pulp_batch_norm_parallelized_fp32_fw_cl",
 ]
+
+# `int f(const args *, int nsamples, int step)` batched launchers of the layers around the matmul core.
+STEP_ENTRY_POINTS = ["ptl_%s_%s_batched" % (n, dt) for n in ("relu", "residual", "avgpool", "cross_entropy")
+                     for dt in ("fp32", "fp16")]
+# `int f(const args *)`
+PLAIN_ENTRY_POINTS = ["ptl_gradient_descent_fp32", "ptl_gradient_descent_fp16", "ptl_batch_norm_fp32_fw"]
 
 # `int f(const args *, int nsamples)` batched launchers.
 BATCHED_ENTRY_POINTS = ["ptl_%s_%s_%s_batched" % (layer, dt, step)
@@ -74,6 +88,14 @@ def load():
     for name in BATCHED_ENTRY_POINTS:
         f = getattr(lib, name)
         f.argtypes = [ctypes.c_void_p, ctypes.c_int]
+        f.restype = ctypes.c_int
+    for name in STEP_ENTRY_POINTS:
+        f = getattr(lib, name)
+        f.argtypes = [ctypes.c_void_p, ctypes.c_int, ctypes.c_int]
+        f.restype = ctypes.c_int
+    for name in PLAIN_ENTRY_POINTS:
+        f = getattr(lib, name)
+        f.argtypes = [ctypes.c_void_p]
         f.restype = ctypes.c_int
     lib.ptl_init.argtypes = [ctypes.c_int]
     lib.ptl_init.restype = ctypes.c_int

@@ -1,0 +1,384 @@
+// Layers around the matmul core in a ResNet-style training step: ReLU, residual connection, average
+// pooling, cross-entropy loss, gradient descent, batch normalisation (forward).  All are bandwidth-bound
+// element or small-reduction kernels; fp16 tensors are read as IEEE half, computed in fp32 and rounded once.
+#include <float.h>
+
+#include "ptl_api.h"
+#include "ptl_host.hpp"
+#include "ptl_structs.h"
+
+namespace ptl {
+
+static inline unsigned glue_blocks(size_t n) { return (unsigned)((n + 255) / 256); }
+
+static int glue_bad(const char *fn, const char *what) {
+    printf("[%s] %s\n", fn, what);
+    set_error("%s: %s", fn, what);
+    return 1;
+}
+
+// ---- ReLU (lib/sources/pulp_act_fp32.c:95-129) ------------------------------------------------------
+template <typename T>
+__global__ __launch_bounds__(256) void relu_fw_kernel(const T *__restrict__ x, T *__restrict__ y, size_t n) {
+    size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+    if (i < n) y[i] = (float)x[i] > 0.f ? x[i] : (T)0.f;
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void relu_bw_kernel(const T *__restrict__ x, const T *__restrict__ dy,
+                                                      T *__restrict__ dx, size_t n) {
+    size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+    if (i < n) dx[i] = (float)x[i] > 0.f ? dy[i] : (T)0.f;
+}
+
+template <typename T, typename Args>
+static int relu_step(const Args *a, int ns, int step, const char *fn) {
+    if (!a || !a->input || !a->output || a->input->dim <= 0) return glue_bad(fn, "invalid arguments");
+    if (ns <= 0) return 0;
+    if (!ensure_init()) return 2;
+    const size_t n = (size_t)ns * a->input->dim;
+    Stager sg;
+    const T *x = sg.in(reinterpret_cast<const T *>(a->input->data), n);
+    if (step == 0) {
+        T *y = sg.out(reinterpret_cast<T *>(a->output->data), n);
+        if (sg.failed() || !x || !y) return sg.failed() ? 2 : glue_bad(fn, "null buffer");
+        hipLaunchKernelGGL((relu_fw_kernel<T>), dim3(glue_blocks(n)), dim3(256), 0, state().stream, x, y, n);
+    } else {
+        const T *dy = sg.in(reinterpret_cast<const T *>(a->output->diff), n);
+        T *dx = sg.out(reinterpret_cast<T *>(a->input->diff), n);
+        if (sg.failed() || !x || !dy || !dx) return sg.failed() ? 2 : glue_bad(fn, "null buffer");
+        hipLaunchKernelGGL((relu_bw_kernel<T>), dim3(glue_blocks(n)), dim3(256), 0, state().stream, x, dy, dx, n);
+    }
+    return sg.finish(hip_ok(hipGetLastError(), "relu launch") ? 0 : 2);
+}
+
+// ---- Residual connection (lib/sources/pulp_residual_fp32.c:26-113) ----------------------------------
+template <typename T>
+__global__ __launch_bounds__(256) void add_kernel(const T *__restrict__ a, const T *__restrict__ b, T *__restrict__ c,
+                                                  size_t n) {
+    size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+    if (i < n) c[i] = (T)((float)a[i] + (float)b[i]);
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void copy_elems_kernel(const T *__restrict__ a, T *__restrict__ c, size_t n) {
+    size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+    if (i < n) c[i] = a[i];
+}
+
+template <typename T, typename Args>
+static int residual_step(const Args *a, int ns, int step, const char *fn) {
+    if (!a || !a->skip || !a->lout || !a->output) return glue_bad(fn, "invalid arguments");
+    const int dim = a->output->dim;
+    if (step == 0 && (a->skip->dim != a->lout->dim || a->lout->dim != dim))
+        return glue_bad(fn, "Sizes of input and output activations not matching!!");
+    if (step == 1 && a->skip_in_grad == 0 && a->skip->dim != dim)
+        return glue_bad(fn, "Sizes of input and output activations not matching!!");
+    if (step == 2 && a->lout->dim != dim) return glue_bad(fn, "Sizes of input and output activations not matching!!");
+    if (ns <= 0 || dim <= 0) return 0;
+    if (step == 1 && a->skip_in_grad != 0) return 0;
+    if (!ensure_init()) return 2;
+    const size_t n = (size_t)ns * dim;
+    Stager sg;
+    if (step == 0) {
+        const T *s = sg.in(reinterpret_cast<const T *>(a->skip->data), n);
+        const T *l = sg.in(reinterpret_cast<const T *>(a->lout->data), n);
+        T *o = sg.out(reinterpret_cast<T *>(a->output->data), n);
+        if (sg.failed() || !s || !l || !o) return sg.failed() ? 2 : glue_bad(fn, "null buffer");
+        hipLaunchKernelGGL((add_kernel<T>), dim3(glue_blocks(n)), dim3(256), 0, state().stream, s, l, o, n);
+    } else if (step == 1) {
+        const T *g = sg.in(reinterpret_cast<const T *>(a->output->diff), n);
+        T *s = sg.inout(reinterpret_cast<T *>(a->skip->diff), n);
+        if (sg.failed() || !g || !s) return sg.failed() ? 2 : glue_bad(fn, "null buffer");
+        hipLaunchKernelGGL((add_kernel<T>), dim3(glue_blocks(n)), dim3(256), 0, state().stream, g, s, s, n);
+    } else {
+        const T *g = sg.in(reinterpret_cast<const T *>(a->output->diff), n);
+        T *l = sg.out(reinterpret_cast<T *>(a->lout->diff), n);
+        if (sg.failed() || !g || !l) return sg.failed() ? 2 : glue_bad(fn, "null buffer");
+        hipLaunchKernelGGL((copy_elems_kernel<T>), dim3(glue_blocks(n)), dim3(256), 0, state().stream, g, l, n);
+    }
+    return sg.finish(hip_ok(hipGetLastError(), "residual launch") ? 0 : 2);
+}
+
+// ---- Average pooling (lib/sources/pulp_pooling_fp32.c:24-122) ---------------------------------------
+struct PoolGeom {
+    int C, H, W, Ho, Wo, Hk, Wk, Hs, Ws, Hact, Wact;
+};
+
+// One wave per output element: lanes stride over the window.
+template <typename T>
+__global__ __launch_bounds__(256) void avgpool_fw_kernel(const T *__restrict__ x, T *__restrict__ y, PoolGeom g,
+                                                         size_t nout) {
+    const size_t o = (size_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+    const int lane = threadIdx.x & 63;
+    if (o >= nout) return;
+    const int wa = (int)(o % g.Wact), ha = (int)((o / g.Wact) % g.Hact);
+    const size_t plane = o / ((size_t)g.Wact * g.Hact);  // sample * C + channel
+    const T *src = x + plane * g.H * g.W;
+    float s = 0.f;
+    for (int e = lane; e < g.Hk * g.Wk; e += 64) {
+        const int hk = e / g.Wk, wk = e - hk * g.Wk;
+        s += (float)src[(size_t)(ha * g.Hs + hk) * g.W + wa * g.Ws + wk];
+    }
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) s += __shfl_xor(s, off);
+    if (lane == 0) y[plane * g.Ho * g.Wo + (size_t)ha * g.Wo + wa] = (T)(s / (float)(g.Hk * g.Wk));
+}
+
+// One thread per input element: sums the output gradients of the windows that contain it.
+template <typename T>
+__global__ __launch_bounds__(256) void avgpool_bw_kernel(const T *__restrict__ dy, T *__restrict__ dx, PoolGeom g,
+                                                         size_t nin) {
+    const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+    if (i >= nin) return;
+    const int w = (int)(i % g.W), h = (int)((i / g.W) % g.H);
+    const size_t plane = i / ((size_t)g.W * g.H);
+    const T *src = dy + plane * g.Ho * g.Wo;
+    float s = 0.f;
+    for (int ho = 0; ho < g.Ho; ++ho) {
+        const int hk = h - ho * g.Hs;
+        if (hk < 0 || hk >= g.Hk) continue;
+        for (int wo = 0; wo < g.Wo; ++wo) {
+            const int wk = w - wo * g.Ws;
+            if (wk < 0 || wk >= g.Wk) continue;
+            s += (float)src[(size_t)ho * g.Wo + wo] / (float)(g.Hk * g.Wk);
+        }
+    }
+    dx[i] = (T)s;
+}
+
+template <typename T, typename Args>
+static int avgpool_step(const Args *a, int ns, int step, const char *fn) {
+    if (!a || !a->input || !a->output) return glue_bad(fn, "invalid arguments");
+    PoolGeom g;
+    g.C = a->input->C;
+    g.H = a->input->H;
+    g.W = a->input->W;
+    g.Ho = a->output->H;
+    g.Wo = a->output->W;
+    g.Hk = a->Hker;
+    g.Wk = a->Wker;
+    g.Hs = a->Hstride;
+    g.Ws = a->Wstride;
+    if (g.C <= 0 || g.H <= 0 || g.W <= 0 || g.Hk <= 0 || g.Wk <= 0 || g.Hs <= 0 || g.Ws <= 0 || g.Hk > g.H ||
+        g.Wk > g.W)
+        return glue_bad(fn, "invalid pooling geometry");
+    g.Hact = (g.H - g.Hk + g.Hs) / g.Hs;
+    g.Wact = (g.W - g.Wk + g.Ws) / g.Ws;
+    if (g.Hact != g.Ho || g.Wact != g.Wo) return glue_bad(fn, "Invalid pooling kernel size or output size!");
+    if (ns <= 0) return 0;
+    if (!ensure_init()) return 2;
+    const size_t nin = (size_t)ns * g.C * g.H * g.W, nout = (size_t)ns * g.C * g.Ho * g.Wo;
+    Stager sg;
+    if (step == 0) {
+        const T *x = sg.in(reinterpret_cast<const T *>(a->input->data), nin);
+        T *y = sg.out(reinterpret_cast<T *>(a->output->data), nout);
+        if (sg.failed() || !x || !y) return sg.failed() ? 2 : glue_bad(fn, "null buffer");
+        hipLaunchKernelGGL((avgpool_fw_kernel<T>), dim3((unsigned)((nout + 3) / 4)), dim3(256), 0, state().stream, x,
+                           y, g, nout);
+    } else {
+        const T *dy = sg.in(reinterpret_cast<const T *>(a->output->diff), nout);
+        T *dx = sg.out(reinterpret_cast<T *>(a->input->diff), nin);
+        if (sg.failed() || !dy || !dx) return sg.failed() ? 2 : glue_bad(fn, "null buffer");
+        hipLaunchKernelGGL((avgpool_bw_kernel<T>), dim3(glue_blocks(nin)), dim3(256), 0, state().stream, dy, dx, g,
+                           nin);
+    }
+    return sg.finish(hip_ok(hipGetLastError(), "pooling launch") ? 0 : 2);
+}
+
+// ---- Cross-entropy over raw logits (lib/sources/pulp_losses_fp32.c:26-138) ---------------------------
+// One wave per sample; lanes stride over the classes.
+template <typename T>
+__global__ __launch_bounds__(256) void cross_entropy_kernel(const T *__restrict__ logits, const T *__restrict__ target,
+                                                            T *__restrict__ loss, T *__restrict__ grad, int ncls,
+                                                            int ns, int backward) {
+    const int b = blockIdx.x * 4 + (threadIdx.x >> 6), lane = threadIdx.x & 63;
+    if (b >= ns) return;
+    const T *z = logits + (size_t)b * ncls, *y = target + (size_t)b * ncls;
+    float mx = -FLT_MAX;
+    for (int i = lane; i < ncls; i += 64) mx = fmaxf(mx, (float)z[i]);
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) mx = fmaxf(mx, __shfl_xor(mx, off));
+    float se = 0.f, dot = 0.f, sy = 0.f;
+    for (int i = lane; i < ncls; i += 64) {
+        se += expf((float)z[i] - mx);
+        dot += (float)y[i] * (float)z[i];
+        sy += (float)y[i];
+    }
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) {
+        se += __shfl_xor(se, off);
+        dot += __shfl_xor(dot, off);
+        sy += __shfl_xor(sy, off);
+    }
+    if (!backward) {
+        if (sizeof(T) == 4 && sy == 0.f) sy = 1.0f;  // only the fp32 forward guards this (pulp_losses_fp32.c:66-69)
+        if (lane == 0) loss[b] = (T)(-(dot - (logf(se) + mx) * sy));
+    } else {
+        if (sy == 0.f) sy = 1.0f;
+        const float inv = 1.0f / se;
+        for (int i = lane; i < ncls; i += 64)
+            grad[(size_t)b * ncls + i] = (T)((expf((float)z[i] - mx) * inv) * sy - (float)y[i]);
+    }
+}
+
+template <typename T, typename Args>
+static int cross_entropy_step(const Args *a, int ns, int step, const char *fn) {
+    if (!a || !a->output || !a->target || a->output->dim <= 0) return glue_bad(fn, "invalid arguments");
+    if (ns <= 0) return 0;
+    if (!ensure_init()) return 2;
+    const int ncls = a->output->dim;
+    const size_t n = (size_t)ns * ncls;
+    Stager sg;
+    const T *z = sg.in(reinterpret_cast<const T *>(a->output->data), n);
+    const T *y = sg.in(reinterpret_cast<const T *>(a->target), n);
+    T *loss = nullptr, *grad = nullptr;
+    if (step == 0)
+        loss = sg.out(reinterpret_cast<T *>(a->wr_loss), (size_t)ns);
+    else
+        grad = sg.out(reinterpret_cast<T *>(a->output->diff), n);
+    if (sg.failed() || !z || !y || (step == 0 ? !loss : !grad)) return sg.failed() ? 2 : glue_bad(fn, "null buffer");
+    hipLaunchKernelGGL((cross_entropy_kernel<T>), dim3((ns + 3) / 4), dim3(256), 0, state().stream, z, y, loss, grad,
+                       ncls, ns, step);
+    return sg.finish(hip_ok(hipGetLastError(), "loss launch") ? 0 : 2);
+}
+
+// ---- Gradient descent (lib/sources/pulp_optimizers_fp32.c:26-104) ------------------------------------
+template <typename T>
+__global__ __launch_bounds__(256) void sgd_kernel(T *__restrict__ w, T *__restrict__ g, size_t n, float lr,
+                                                  float lambda) {
+    size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+    if (i >= n) return;
+    float gi = (float)g[i], wi = (float)w[i];
+    if (lambda != 0.f) {
+        gi = gi + lambda * wi;
+        g[i] = (T)gi;
+        gi = (float)(T)gi;
+    }
+    w[i] = (T)(wi - lr * gi);
+}
+
+template <typename T, typename Args>
+static int sgd_step(const Args *a, const char *fn) {
+    if (!a || !a->weights) return glue_bad(fn, "invalid arguments");
+    if (a->use_biases == 1 && !a->biases) return glue_bad(fn, "use_biases=1 with a null bias blob");
+    if (!ensure_init()) return 2;
+    const float lr = (float)a->learning_rate, lambda = (float)a->weight_decay_lambda;
+    Stager sg;
+    const struct { void *data, *diff; int dim; } parts[2] = {
+        {a->weights->data, a->weights->diff, a->weights->dim},
+        {a->use_biases == 1 ? (void *)a->biases->data : nullptr, a->use_biases == 1 ? (void *)a->biases->diff : nullptr,
+         a->use_biases == 1 ? a->biases->dim : 0}};
+    for (const auto &p : parts) {
+        if (p.dim <= 0) continue;
+        if (!p.data || !p.diff) return glue_bad(fn, "null buffer");
+        T *w = sg.inout(reinterpret_cast<T *>(p.data), (size_t)p.dim);
+        T *g = lambda != 0.f ? sg.inout(reinterpret_cast<T *>(p.diff), (size_t)p.dim)
+                             : const_cast<T *>(sg.in(reinterpret_cast<const T *>(p.diff), (size_t)p.dim));
+        if (sg.failed()) return 2;
+        hipLaunchKernelGGL((sgd_kernel<T>), dim3(glue_blocks((size_t)p.dim)), dim3(256), 0, state().stream, w, g,
+                           (size_t)p.dim, lr, lambda);
+        if (!hip_ok(hipGetLastError(), "optimizer launch")) return sg.finish(2);
+    }
+    return sg.finish(0);
+}
+
+// ---- Batch normalisation forward (lib/sources/pulp_batchnorm_fp32.c:34-114) ---------------------------
+// One workgroup per channel: sums of x and x^2 over B x H x W, then the affine map.
+__global__ __launch_bounds__(256) void batch_norm_fw_kernel(const float *__restrict__ x, float *__restrict__ y,
+                                                            const float *__restrict__ weight,
+                                                            const float *__restrict__ bias, const float *eps, int B,
+                                                            int C, int HW) {
+    __shared__ float red[2][4];
+    const int c = blockIdx.x, tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const size_t n = (size_t)B * HW;
+    float s1 = 0.f, s2 = 0.f;
+    for (size_t e = tid; e < n; e += 256) {
+        const size_t b = e / HW, hw = e - b * HW;
+        const float v = x[(b * C + c) * HW + hw];
+        s1 += v;
+        s2 += v * v;
+    }
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) {
+        s1 += __shfl_xor(s1, off);
+        s2 += __shfl_xor(s2, off);
+    }
+    if (lane == 0) {
+        red[0][wave] = s1;
+        red[1][wave] = s2;
+    }
+    __syncthreads();
+    s1 = (red[0][0] + red[0][1]) + (red[0][2] + red[0][3]);
+    s2 = (red[1][0] + red[1][1]) + (red[1][2] + red[1][3]);
+    const float cnt = (float)n;
+    const float mean = s1 / cnt;
+    const float sd = sqrtf(((s2 - 2 * s1 * mean) / cnt) + (mean * mean) + eps[0]);
+    const float w = weight[c], bb = bias[c];
+    for (size_t e = tid; e < n; e += 256) {
+        const size_t b = e / HW, hw = e - b * HW;
+        const size_t idx = (b * C + c) * HW + hw;
+        y[idx] = ((x[idx] - mean) / sd) * w + bb;
+    }
+}
+
+static int batch_norm_fw(const BatchNorm_args_fp32 *a, const char *fn) {
+    if (!a || !a->input || !a->output || !a->weight_data || !a->bias_data || !a->eps)
+        return glue_bad(fn, "invalid arguments");
+    if (a->B <= 0 || a->C <= 0 || a->H <= 0 || a->W <= 0) return glue_bad(fn, "invalid tensor geometry");
+    if (!ensure_init()) return 2;
+    const size_t n = (size_t)a->B * a->C * a->H * a->W;
+    Stager sg;
+    const float *x = sg.in(a->input->data, n);
+    float *y = sg.out(a->output->data, n);
+    const float *w = sg.in(a->weight_data, (size_t)a->C);
+    const float *b = sg.in(a->bias_data, (size_t)a->C);
+    const float *eps = sg.in(a->eps, (size_t)1);
+    if (sg.failed() || !x || !y) return sg.failed() ? 2 : glue_bad(fn, "null buffer");
+    hipLaunchKernelGGL(batch_norm_fw_kernel, dim3(a->C), dim3(256), 0, state().stream, x, y, w, b, eps, a->B, a->C,
+                       a->H * a->W);
+    return sg.finish(hip_ok(hipGetLastError(), "batch norm launch") ? 0 : 2);
+}
+
+}  // namespace ptl
+
+extern "C" {
+
+int ptl_relu_fp32_batched(const struct act_args *a, int ns, int step) {
+    return ptl::relu_step<float>(a, ns, step, step ? "pulp_relu_fp32_bw_cl" : "pulp_relu_fp32_fw_cl");
+}
+int ptl_relu_fp16_batched(const struct act_args_fp16 *a, int ns, int step) {
+    return ptl::relu_step<ptl::half_t>(a, ns, step, step ? "pulp_relu_fp16_bw_cl" : "pulp_relu_fp16_fw_cl");
+}
+int ptl_residual_fp32_batched(const struct SkipConn_args *a, int ns, int step) {
+    return ptl::residual_step<float>(
+        a, ns, step, step == 0 ? "pulp_residualconn_fp32_fw" : step == 1 ? "pulp_sumnode_fp32_bw" : "pulp_residualconn_fp32_bw");
+}
+int ptl_residual_fp16_batched(const struct SkipConn_args_fp16 *a, int ns, int step) {
+    return ptl::residual_step<ptl::half_t>(
+        a, ns, step, step == 0 ? "pulp_residualconn_fp16_fw" : step == 1 ? "pulp_sumnode_fp16_bw" : "pulp_residualconn_fp16_bw");
+}
+int ptl_avgpool_fp32_batched(const struct pool_args *a, int ns, int step) {
+    return ptl::avgpool_step<float>(a, ns, step, step ? "pulp_avgpool_fp32_bw_cl" : "pulp_avgpool_fp32_fw_cl");
+}
+int ptl_avgpool_fp16_batched(const struct pool_args_fp16 *a, int ns, int step) {
+    return ptl::avgpool_step<ptl::half_t>(a, ns, step, step ? "pulp_avgpool_fp16_bw_cl" : "pulp_avgpool_fp16_fw_cl");
+}
+int ptl_cross_entropy_fp32_batched(const struct loss_args *a, int ns, int step) {
+    return ptl::cross_entropy_step<float>(a, ns, step, step ? "pulp_CrossEntropyLoss_backward" : "pulp_CrossEntropyLoss");
+}
+int ptl_cross_entropy_fp16_batched(const struct loss_args_fp16 *a, int ns, int step) {
+    return ptl::cross_entropy_step<ptl::half_t>(a, ns, step,
+                                                step ? "pulp_CrossEntropyLoss_backward_fp16" : "pulp_CrossEntropyLoss_fp16");
+}
+int ptl_gradient_descent_fp32(const struct optim_args *a) {
+    return ptl::sgd_step<float>(a, "pulp_gradient_descent_fp32");
+}
+int ptl_gradient_descent_fp16(const struct optim_args_fp16 *a) {
+    return ptl::sgd_step<ptl::half_t>(a, "pulp_gradient_descent_fp16");
+}
+int ptl_batch_norm_fp32_fw(const struct BatchNorm_args_fp32 *a) {
+    return ptl::batch_norm_fw(a, "pulp_batch_norm_fp32_fw_cl");
+}
+
+}  // extern "C"

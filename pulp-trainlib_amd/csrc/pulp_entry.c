@@ -454,3 +454,39 @@ void pulp_mhsa_fp32_fw_cl(void *p) { ptl_internal_set_status(ptl_mhsa_fp32_fw_ba
 void pulp_mhsa_fp32_bw_cl(void *p) { ptl_internal_set_status(ptl_mhsa_fp32_bw_batched(p, 1)); }
 void pulp_softmax_fp32_fw_cl(void *p) { ptl_internal_set_status(ptl_internal_softmax_fp32(p, 0)); }
 void pulp_softmax_fp32_bw_cl(void *p) { ptl_internal_set_status(ptl_internal_softmax_fp32(p, 1)); }
+
+/* ---- Layers around the matmul core (lib/sources/pulp_act_fp32.c:83-129, pulp_residual_fp32.c:26-113,
+ * pulp_pooling_fp32.c:24-122, pulp_losses_fp32.c:26-138, pulp_optimizers_fp32.c:26, pulp_batchnorm_fp32.c:28
+ * and their fp16 twins) --------------------------------------------------------------------------- */
+
+void pulp_relu_fp32_fw_cl(void *p) { ptl_internal_set_status(ptl_relu_fp32_batched(p, 1, 0)); }
+void pulp_relu_fp32_bw_cl(void *p) { ptl_internal_set_status(ptl_relu_fp32_batched(p, 1, 1)); }
+void relu_core_fw_fp32(void *p) { ptl_internal_set_status(ptl_relu_fp32_batched(p, 1, 0)); }
+void relu_core_bw_fp32(void *p) { ptl_internal_set_status(ptl_relu_fp32_batched(p, 1, 1)); }
+void pulp_relu_fp16_fw_cl(void *p) { ptl_internal_set_status(ptl_relu_fp16_batched(p, 1, 0)); }
+void pulp_relu_fp16_bw_cl(void *p) { ptl_internal_set_status(ptl_relu_fp16_batched(p, 1, 1)); }
+void relu_core_fw_fp16(void *p) { ptl_internal_set_status(ptl_relu_fp16_batched(p, 1, 0)); }
+void relu_core_bw_fp16(void *p) { ptl_internal_set_status(ptl_relu_fp16_batched(p, 1, 1)); }
+
+void pulp_residualconn_fp32_fw(void *p) { ptl_internal_set_status(ptl_residual_fp32_batched(p, 1, 0)); }
+void pulp_sumnode_fp32_bw(void *p) { ptl_internal_set_status(ptl_residual_fp32_batched(p, 1, 1)); }
+void pulp_residualconn_fp32_bw(void *p) { ptl_internal_set_status(ptl_residual_fp32_batched(p, 1, 2)); }
+void pulp_residualconn_fp16_fw(void *p) { ptl_internal_set_status(ptl_residual_fp16_batched(p, 1, 0)); }
+void pulp_sumnode_fp16_bw(void *p) { ptl_internal_set_status(ptl_residual_fp16_batched(p, 1, 1)); }
+void pulp_residualconn_fp16_bw(void *p) { ptl_internal_set_status(ptl_residual_fp16_batched(p, 1, 2)); }
+
+void pulp_avgpool_fp32_fw_cl(void *p) { ptl_internal_set_status(ptl_avgpool_fp32_batched(p, 1, 0)); }
+void pulp_avgpool_fp32_bw_cl(void *p) { ptl_internal_set_status(ptl_avgpool_fp32_batched(p, 1, 1)); }
+void pulp_avgpool_fp16_fw_cl(void *p) { ptl_internal_set_status(ptl_avgpool_fp16_batched(p, 1, 0)); }
+void pulp_avgpool_fp16_bw_cl(void *p) { ptl_internal_set_status(ptl_avgpool_fp16_batched(p, 1, 1)); }
+
+void pulp_CrossEntropyLoss(void *p) { ptl_internal_set_status(ptl_cross_entropy_fp32_batched(p, 1, 0)); }
+void pulp_CrossEntropyLoss_backward(void *p) { ptl_internal_set_status(ptl_cross_entropy_fp32_batched(p, 1, 1)); }
+void pulp_CrossEntropyLoss_fp16(void *p) { ptl_internal_set_status(ptl_cross_entropy_fp16_batched(p, 1, 0)); }
+void pulp_CrossEntropyLoss_backward_fp16(void *p) { ptl_internal_set_status(ptl_cross_entropy_fp16_batched(p, 1, 1)); }
+
+void pulp_gradient_descent_fp32(void *p) { ptl_internal_set_status(ptl_gradient_descent_fp32(p)); }
+void pulp_gradient_descent_fp16(void *p) { ptl_internal_set_status(ptl_gradient_descent_fp16(p)); }
+
+void pulp_batch_norm_fp32_fw_cl(void *p) { ptl_internal_set_status(ptl_batch_norm_fp32_fw(p)); }
+void pulp_batch_norm_parallelized_fp32_fw_cl(void *p) { ptl_internal_set_status(ptl_batch_norm_fp32_fw(p)); }

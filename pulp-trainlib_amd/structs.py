@@ -127,6 +127,39 @@ class MhsaArgs(C.Structure):
                 ("softmax_buffer", BlobP), ("global_max", P), ("partial_exp_sum", P), ("maxes", P), ("sums", P)]
 
 
+class ActArgs(C.Structure):
+    _fields_ = [("input", BlobP), ("output", BlobP), ("H", I), ("W", I)]
+
+
+class SkipConnArgs(C.Structure):
+    _fields_ = [("skip", BlobP), ("lout", BlobP), ("output", BlobP), ("skip_in_grad", I)]
+
+
+class PoolArgs(C.Structure):
+    _fields_ = [("input", BlobP), ("output", BlobP), ("Hker", I), ("Wker", I), ("Hstride", I), ("Wstride", I)]
+
+
+class LossArgs(C.Structure):
+    _fields_ = [("output", BlobP), ("target", P), ("wr_loss", P)]
+
+
+class OptimArgs(C.Structure):
+    _fields_ = [("weights", BlobP), ("biases", BlobP), ("learning_rate", C.c_float),
+                ("weight_decay_lambda", C.c_float), ("use_biases", I)]
+
+
+class OptimArgsFp16(C.Structure):
+    _fields_ = [("weights", BlobP), ("biases", BlobP), ("learning_rate", C.c_uint16),
+                ("weight_decay_lambda", C.c_uint16), ("use_biases", I)]
+
+
+class BatchNormArgs(C.Structure):
+    _fields_ = [("input", BlobP), ("output", BlobP), ("coeff", BlobP), ("bias", BlobP), ("batch_size", I),
+                ("running_mean", P), ("running_var", P), ("running_stdev", P), ("freeze_running_params", I),
+                ("skip_wg_grad", I), ("skip_in_grad", I), ("weight_data", P), ("bias_data", P), ("eps", P),
+                ("B", I), ("C", I), ("H", I), ("W", I)]
+
+
 LAYER_CONV2D, LAYER_DW_CONV, LAYER_PW_CONV, LAYER_LINEAR = 0, 1, 2, 3
 STEP_FW, STEP_WGT_GRAD, STEP_IN_GRAD = 0, 1, 2
 

@@ -172,3 +172,74 @@ def mhsa_inputs(seed, ns, L, E, F, heads):
         d[n] = uniform(seed + 11 + i, sh[n], -0.1, 0.1)
     dy = uniform(seed + 21, sh["y"])
     return d, dy
+
+
+def act_args(pkg, x, dx, y, dy, dim):
+    keep = Keep()
+    bi, bo = pkg.blob(x, dx, 1, 1, dim, dim=dim), pkg.blob(y, dy, 1, 1, dim, dim=dim)
+    keep += [bi, bo, x, dx, y, dy]
+    a = pkg.ActArgs()
+    a.input, a.output = ptr(bi), ptr(bo)
+    return a, keep
+
+
+def skip_args(pkg, skip, dskip, lout, dlout, out, dout, dim, skip_in_grad=0):
+    keep = Keep()
+    bs, bl, bo = (pkg.blob(skip, dskip, 1, 1, dim, dim=dim), pkg.blob(lout, dlout, 1, 1, dim, dim=dim),
+                  pkg.blob(out, dout, 1, 1, dim, dim=dim))
+    keep += [bs, bl, bo, skip, dskip, lout, dlout, out, dout]
+    a = pkg.SkipConnArgs()
+    a.skip, a.lout, a.output = ptr(bs), ptr(bl), ptr(bo)
+    a.skip_in_grad = skip_in_grad
+    return a, keep
+
+
+def pool_args(pkg, x, dx, y, dy, C, H, W, Ho, Wo, Hk, Wk, Hs, Ws):
+    keep = Keep()
+    bi, bo = pkg.blob(x, dx, C, H, W), pkg.blob(y, dy, C, Ho, Wo)
+    keep += [bi, bo, x, dx, y, dy]
+    a = pkg.PoolArgs()
+    a.input, a.output = ptr(bi), ptr(bo)
+    a.Hker, a.Wker, a.Hstride, a.Wstride = Hk, Wk, Hs, Ws
+    return a, keep
+
+
+def loss_args(pkg, logits, dlogits, target, loss, ncls):
+    keep = Keep()
+    bo = pkg.blob(logits, dlogits, 1, 1, ncls, dim=ncls)
+    keep += [bo, logits, dlogits, target, loss]
+    a = pkg.LossArgs()
+    a.output = ptr(bo)
+    a.target, a.wr_loss = pkg.addr(target), pkg.addr(loss)
+    return a, keep
+
+
+def optim_args(pkg, dt, w, dw, b, db, lr, lam):
+    keep = Keep()
+    bw = pkg.blob(w, dw, 1, 1, int(np.prod(w.shape)), dim=int(np.prod(w.shape)))
+    keep += [bw, w, dw, b, db]
+    a = pkg.OptimArgs() if dt == "fp32" else pkg.OptimArgsFp16()
+    a.weights = ptr(bw)
+    if b is not None:
+        bb = pkg.blob(b, db, 1, 1, int(np.prod(b.shape)), dim=int(np.prod(b.shape)))
+        keep.append(bb)
+        a.biases = ptr(bb)
+        a.use_biases = 1
+    if dt == "fp32":
+        a.learning_rate, a.weight_decay_lambda = lr, lam
+    else:
+        a.learning_rate = int(np.float16(lr).view(np.uint16))
+        a.weight_decay_lambda = int(np.float16(lam).view(np.uint16))
+    return a, keep
+
+
+def batch_norm_args(pkg, x, y, w, b, eps, B, C, H, W):
+    keep = Keep()
+    bi, bo = pkg.blob(x, None, C, H, W), pkg.blob(y, None, C, H, W)
+    keep += [bi, bo, x, y, w, b, eps]
+    a = pkg.BatchNormArgs()
+    a.input, a.output = ptr(bi), ptr(bo)
+    a.weight_data, a.bias_data, a.eps = pkg.addr(w), pkg.addr(b), pkg.addr(eps)
+    a.B, a.C, a.H, a.W = B, C, H, W
+    a.batch_size = B
+    return a, keep

@@ -29,7 +29,8 @@ def test_library_exports_every_declared_symbol(pkg):
     missing = [n for n in names if not hasattr(lib, n)]
     assert not missing, missing
     # and the Python lists name nothing the header does not declare
-    listed = set(pkg.VOID_ENTRY_POINTS + pkg.BATCHED_ENTRY_POINTS + pkg.OTHER_ENTRY_POINTS)
+    listed = set(pkg.VOID_ENTRY_POINTS + pkg.BATCHED_ENTRY_POINTS + pkg.OTHER_ENTRY_POINTS + pkg.STEP_ENTRY_POINTS +
+                 pkg.PLAIN_ENTRY_POINTS)
     assert listed == set(names)
 
 
@@ -44,6 +45,10 @@ STRUCTS = {
     "Conv2D_args_fp16": "Conv2DArgs", "PointWise_Conv_args": "PointWiseConvArgs",
     "PointWise_Conv_args_fp16": "PointWiseConvArgs", "DepthWise_Conv_args": "DepthWiseConvArgs",
     "DepthWise_Conv_args_fp16": "DepthWiseConvArgsFp16", "Linear_args": "LinearArgs", "Linear_args_fp16": "LinearArgs",
+    "softmax_args": "SoftmaxArgs", "Mhsa_args": "MhsaArgs", "act_args": "ActArgs", "act_args_fp16": "ActArgs",
+    "SkipConn_args": "SkipConnArgs", "SkipConn_args_fp16": "SkipConnArgs", "pool_args": "PoolArgs",
+    "pool_args_fp16": "PoolArgs", "loss_args": "LossArgs", "loss_args_fp16": "LossArgs", "optim_args": "OptimArgs",
+    "optim_args_fp16": "OptimArgsFp16", "BatchNorm_args_fp32": "BatchNormArgs",
 }
 
 

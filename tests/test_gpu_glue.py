@@ -1,0 +1,242 @@
+"""GPU parity of the layers around the matmul core (ReLU, residual connection, average pooling, cross-entropy,
+gradient descent, batch-norm forward) against the CPU oracle, and one residual-block training step assembled
+from the library's entry points against torch autograd."""
+import ctypes
+
+import numpy as np
+import pytest
+import torch
+import torch.nn.functional as F
+
+import helpers as hp
+
+pytestmark = pytest.mark.gpu
+
+TOL = {"fp32": 1e-4, "fp16": 1e-2}
+
+
+def dev(a):
+    return torch.from_numpy(np.ascontiguousarray(a)).cuda()
+
+
+def host(t):
+    return t.cpu().numpy() if hasattr(t, "cpu") else t
+
+
+@pytest.mark.parametrize("device", [True, False])
+@pytest.mark.parametrize("dt", ["fp32", "fp16"])
+def test_relu_residual(pkg, orc, gpu, dt, device):
+    olib, npd = orc.load(), hp.np_dtype(dt)
+    mk = dev if device else (lambda z: z.copy())
+    ns, dim = 5, 1000
+    x = hp.uniform(0x7E01, (ns, dim)).astype(npd)
+    g = hp.uniform(0x7E02, (ns, dim)).astype(npd)
+    ry, rdx = np.zeros_like(x), np.zeros_like(x)
+    a, k = hp.act_args(pkg, x, rdx, ry, g, dim)
+    for step in (0, 1):
+        getattr(olib, "orc_relu_" + dt)(ctypes.byref(a), ns, step)
+    y, dx = mk(np.full_like(x, 7)), mk(np.full_like(x, 7))
+    b, k2 = hp.act_args(pkg, mk(x), dx, y, mk(g), dim)
+    for step in (0, 1):
+        assert getattr(gpu, "ptl_relu_%s_batched" % dt)(ctypes.byref(b), ns, step) == 0
+    gpu.ptl_sync()
+    assert np.array_equal(host(y), ry) and np.array_equal(host(dx), rdx)
+    # residual connection
+    s, l = hp.uniform(0x7E03, (ns, dim)).astype(npd), hp.uniform(0x7E04, (ns, dim)).astype(npd)
+    ds0 = hp.uniform(0x7E05, (ns, dim)).astype(npd)
+    rds, rdl, ro = ds0.copy(), np.zeros_like(s), np.zeros_like(s)
+    c, k3 = hp.skip_args(pkg, s, rds, l, rdl, ro, g, dim)
+    for step in (0, 1, 2):
+        getattr(olib, "orc_residual_" + dt)(ctypes.byref(c), ns, step)
+    ds, dl, o = mk(ds0), mk(np.full_like(s, 7)), mk(np.full_like(s, 7))
+    d, k4 = hp.skip_args(pkg, mk(s), ds, mk(l), dl, o, mk(g), dim)
+    for step in (0, 1, 2):
+        assert getattr(gpu, "ptl_residual_%s_batched" % dt)(ctypes.byref(d), ns, step) == 0
+    gpu.ptl_sync()
+    assert np.array_equal(host(o), ro) and np.array_equal(host(ds), rds) and np.array_equal(host(dl), rdl)
+    # skip_in_grad leaves the skip gradient alone
+    d.skip_in_grad = 1
+    assert getattr(gpu, "ptl_residual_%s_batched" % dt)(ctypes.byref(d), ns, 1) == 0
+    gpu.ptl_sync()
+    assert np.array_equal(host(ds), rds)
+
+
+@pytest.mark.parametrize("dt", ["fp32", "fp16"])
+@pytest.mark.parametrize("geo", [(64, 8, 8, 8, 8, 8, 8), (3, 9, 7, 3, 2, 2, 1), (16, 32, 32, 2, 2, 2, 2)])
+def test_avgpool(pkg, orc, gpu, dt, geo):
+    olib, npd = orc.load(), hp.np_dtype(dt)
+    C, H, W, Hk, Wk, Hs, Ws = geo
+    ns = 3
+    Ho, Wo = (H - Hk + Hs) // Hs, (W - Wk + Ws) // Ws
+    x = hp.uniform(0x7E10 + H, (ns, C, H, W)).astype(npd)
+    g = hp.uniform(0x7E11 + H, (ns, C, Ho, Wo)).astype(npd)
+    ry, rdx = np.zeros((ns, C, Ho, Wo), npd), np.zeros((ns, C, H, W), npd)
+    a, k = hp.pool_args(pkg, x, rdx, ry, g, C, H, W, Ho, Wo, Hk, Wk, Hs, Ws)
+    for step in (0, 1):
+        getattr(olib, "orc_avgpool_" + dt)(ctypes.byref(a), ns, step)
+    y, dx = dev(np.full_like(ry, 7)), dev(np.full_like(rdx, 7))
+    b, k2 = hp.pool_args(pkg, dev(x), dx, y, dev(g), C, H, W, Ho, Wo, Hk, Wk, Hs, Ws)
+    for step in (0, 1):
+        assert getattr(gpu, "ptl_avgpool_%s_batched" % dt)(ctypes.byref(b), ns, step) == 0
+    gpu.ptl_sync()
+    assert hp.rel_l2(host(y), ry) <= TOL[dt]
+    assert hp.rel_l2(host(dx), rdx) <= TOL[dt]
+    # a window that does not match the output size is rejected and leaves the output alone
+    b.Hker = Hk + 1
+    assert getattr(gpu, "ptl_avgpool_%s_batched" % dt)(ctypes.byref(b), ns, 0) == 1
+
+
+@pytest.mark.parametrize("dt", ["fp32", "fp16"])
+@pytest.mark.parametrize("ncls", [10, 200])
+def test_cross_entropy(pkg, orc, gpu, dt, ncls):
+    olib, npd = orc.load(), hp.np_dtype(dt)
+    ns = 37
+    z = (3 * hp.normal(0x7E20, (ns, ncls))).astype(npd)
+    y = np.zeros((ns, ncls), npd)
+    y[np.arange(ns), (7 * np.arange(ns)) % ncls] = 1
+    y[5] = npd(1.0 / ncls)
+    rl, rdz = np.zeros(ns, npd), np.zeros((ns, ncls), npd)
+    a, k = hp.loss_args(pkg, z, rdz, y, rl, ncls)
+    for step in (0, 1):
+        getattr(olib, "orc_cross_entropy_" + dt)(ctypes.byref(a), ns, step)
+    loss, dz = np.full(ns, 7, npd), np.full((ns, ncls), 7, npd)
+    b, k2 = hp.loss_args(pkg, z, dz, y, loss, ncls)  # host pointers
+    for step in (0, 1):
+        assert getattr(gpu, "ptl_cross_entropy_%s_batched" % dt)(ctypes.byref(b), ns, step) == 0
+    assert hp.rel_l2(loss, rl) <= TOL[dt]
+    assert hp.rel_l2(dz, rdz) <= TOL[dt]
+
+
+@pytest.mark.parametrize("dt", ["fp32", "fp16"])
+@pytest.mark.parametrize("lam", [0.0, 0.05])
+def test_gradient_descent(pkg, orc, gpu, dt, lam):
+    olib, npd = orc.load(), hp.np_dtype(dt)
+    w0, g0 = hp.uniform(0x7E30, (64, 27)).astype(npd), hp.uniform(0x7E31, (64, 27)).astype(npd)
+    b0, gb0 = hp.uniform(0x7E32, (64,)).astype(npd), hp.uniform(0x7E33, (64,)).astype(npd)
+    rw, rg, rb, rgb = w0.copy(), g0.copy(), b0.copy(), gb0.copy()
+    a, k = hp.optim_args(pkg, dt, rw, rg, rb, rgb, 0.01, lam)
+    getattr(olib, "orc_gradient_descent_" + dt)(ctypes.byref(a))
+    w, g, b, gb = dev(w0), dev(g0), dev(b0), dev(gb0)
+    c, k2 = hp.optim_args(pkg, dt, w, g, b, gb, 0.01, lam)
+    getattr(gpu, "pulp_gradient_descent_" + dt)(ctypes.byref(c))
+    assert gpu.ptl_last_status() == 0, gpu.ptl_last_error().decode()
+    gpu.ptl_sync()
+    for got, ref in ((w, rw), (g, rg), (b, rb), (gb, rgb)):
+        assert hp.rel_l2(host(got), ref) <= (1e-6 if dt == "fp32" else 2e-3)
+
+
+def test_batch_norm_forward(pkg, orc, gpu):
+    B, C, H, W = 8, 16, 9, 11
+    x = (2 * hp.normal(0x7E40, (B, C, H, W)) + 0.5).astype(np.float32)
+    w, b = hp.uniform(0x7E41, (C,), 0.5, 1.5), hp.uniform(0x7E42, (C,))
+    eps = np.array([1e-5], np.float32)
+    ry = np.zeros_like(x)
+    a, k = hp.batch_norm_args(pkg, x, ry, w, b, eps, B, C, H, W)
+    orc.load().orc_batch_norm_fw_fp32(ctypes.byref(a))
+    y = np.full_like(x, 7)
+    c, k2 = hp.batch_norm_args(pkg, x, y, w, b, eps, B, C, H, W)
+    gpu.pulp_batch_norm_fp32_fw_cl(ctypes.byref(c))
+    assert gpu.ptl_last_status() == 0, gpu.ptl_last_error().decode()
+    assert hp.rel_l2(y, ry) <= 1e-5
+
+
+def test_reference_named_single_sample_entry_points(pkg, orc, gpu):
+    dim = 300
+    x, g = hp.uniform(0x7E50, (dim,)), hp.uniform(0x7E51, (dim,))
+    y, dx = np.zeros_like(x), np.zeros_like(x)
+    a, k = hp.act_args(pkg, x, dx, y, g, dim)
+    gpu.pulp_relu_fp32_fw_cl(ctypes.byref(a))
+    gpu.relu_core_bw_fp32(ctypes.byref(a))
+    assert gpu.ptl_last_status() == 0
+    assert np.array_equal(y, np.maximum(x, 0)) and np.array_equal(dx, np.where(x > 0, g, 0))
+    z = hp.normal(0x7E52, (10,))
+    t = np.zeros(10, np.float32)
+    t[3] = 1
+    loss, dz = np.zeros(1, np.float32), np.zeros(10, np.float32)
+    b, k2 = hp.loss_args(pkg, z, dz, t, loss, 10)
+    gpu.pulp_CrossEntropyLoss(ctypes.byref(b))
+    gpu.pulp_CrossEntropyLoss_backward(ctypes.byref(b))
+    zt = torch.tensor(z.astype(np.float64), requires_grad=True)
+    lt = F.cross_entropy(zt[None], torch.tensor([3]))
+    lt.backward()
+    assert abs(loss[0] - lt.item()) < 1e-5 and hp.rel_l2(dz, zt.grad.numpy()) < 1e-5
+
+
+@pytest.mark.parametrize("dt", ["fp32", "fp16"])
+def test_residual_block_training_step(pkg, gpu, dt):
+    """conv3x3 -> ReLU -> conv3x3 -> (+ input) -> ReLU -> global average pool -> linear -> cross-entropy, the
+    backward pass through all of it and one SGD update, from the library's entry points, against torch autograd
+    in float64 on the same (rounded) inputs."""
+    npd = hp.np_dtype(dt)
+    # fp16: every activation and gradient tensor of the chain is stored in half precision (the pooled gradient is
+    # divided by 64 and sits near the subnormal range), so the deepest gradients carry a few percent of rounding
+    tol = {"fp32": 1e-4, "fp16": 6e-2}[dt]
+    ns, C, H, ncls, lr = 6, 16, 8, 10, 0.05
+    x0 = hp.uniform(0x7E60, (ns, C, H, H)).astype(npd)
+    w1 = (hp.uniform(0x7E61, (C, C, 3, 3)) * 0.2).astype(npd)
+    w2 = (hp.uniform(0x7E62, (C, C, 3, 3)) * 0.2).astype(npd)
+    wl = (hp.uniform(0x7E63, (ncls, C)) * 0.5).astype(npd)
+    tgt = np.zeros((ns, ncls), npd)
+    tgt[np.arange(ns), np.arange(ns) % ncls] = 1
+    z = lambda *s: torch.zeros(*s, dtype=torch.float16 if dt == "fp16" else torch.float32, device="cuda")
+    X0, W1, W2, WL, T = dev(x0), dev(w1), dev(w2), dev(wl), dev(tgt)
+    dX0, dW1, dW2, dWL = z(ns, C, H, H), z(C, C, 3, 3), z(C, C, 3, 3), z(ncls, C)
+    A1, dA1, R1, dR1 = z(ns, C, H, H), z(ns, C, H, H), z(ns, C, H, H), z(ns, C, H, H)
+    A2, dA2, S, dS, R2, dR2 = (z(ns, C, H, H) for _ in range(6))
+    Pl, dPl, Z, dZ, loss = z(ns, C), z(ns, C), z(ns, ncls), z(ns, ncls), z(ns)
+    dim = C * H * H
+    c1, k1 = hp.conv2d_args(pkg, X0, dX0, W1, dW1, A1, dA1, C, H, H, C, 3, 3, H, H, (1, 1, 1, 1))
+    r1, k2 = hp.act_args(pkg, A1, dA1, R1, dR1, dim)
+    c2, k3 = hp.conv2d_args(pkg, R1, dR1, W2, dW2, A2, dA2, C, H, H, C, 3, 3, H, H, (1, 1, 1, 1))
+    sk, k4 = hp.skip_args(pkg, X0, dX0, A2, dA2, S, dS, dim)
+    r2, k5 = hp.act_args(pkg, S, dS, R2, dR2, dim)
+    pl, k6 = hp.pool_args(pkg, R2, dR2, Pl, dPl, C, H, H, 1, 1, H, H, H, H)
+    ln, k7 = hp.linear_args(pkg, Pl, dPl, WL, dWL, Z, dZ, C, ncls)
+    ls, k8 = hp.loss_args(pkg, Z, dZ, T, loss, ncls)
+    ok = lambda rc: (rc == 0) or pytest.fail(gpu.ptl_last_error().decode())
+    ref = ctypes.byref
+    L = lambda name: getattr(gpu, name.replace("DT", dt))
+    # forward
+    ok(L("ptl_conv2d_DT_fw_batched")(ref(c1), ns))
+    ok(L("ptl_relu_DT_batched")(ref(r1), ns, 0))
+    ok(L("ptl_conv2d_DT_fw_batched")(ref(c2), ns))
+    ok(L("ptl_residual_DT_batched")(ref(sk), ns, 0))
+    ok(L("ptl_relu_DT_batched")(ref(r2), ns, 0))
+    ok(L("ptl_avgpool_DT_batched")(ref(pl), ns, 0))
+    ok(L("ptl_linear_DT_fw_batched")(ref(ln), ns))
+    ok(L("ptl_cross_entropy_DT_batched")(ref(ls), ns, 0))
+    # backward
+    ok(L("ptl_cross_entropy_DT_batched")(ref(ls), ns, 1))
+    ok(L("ptl_linear_DT_bw_batched")(ref(ln), ns))
+    ok(L("ptl_avgpool_DT_batched")(ref(pl), ns, 1))
+    ok(L("ptl_relu_DT_batched")(ref(r2), ns, 1))
+    ok(L("ptl_residual_DT_batched")(ref(sk), ns, 2))  # dA2 = dS
+    ok(L("ptl_conv2d_DT_wg_batched")(ref(c2), ns))
+    ok(L("ptl_conv2d_DT_ig_batched")(ref(c2), ns))
+    ok(L("ptl_relu_DT_batched")(ref(r1), ns, 1))
+    ok(L("ptl_conv2d_DT_wg_batched")(ref(c1), ns))
+    ok(L("ptl_conv2d_DT_ig_batched")(ref(c1), ns))   # dX0 = conv path
+    ok(L("ptl_residual_DT_batched")(ref(sk), ns, 1))  # dX0 += dS (skip path)
+    gpu.ptl_sync()
+    grads = {n: host(t).astype(np.float64) for n, t in (("w1", dW1), ("w2", dW2), ("wl", dWL), ("x", dX0))}
+    # update
+    for Wt, dWt in ((W1, dW1), (W2, dW2), (WL, dWL)):
+        o, ko = hp.optim_args(pkg, dt, Wt, dWt, None, None, lr, 0.0)
+        ok(L("ptl_gradient_descent_DT")(ref(o)))
+    gpu.ptl_sync()
+    # torch float64
+    xt = torch.tensor(x0.astype(np.float64), requires_grad=True)
+    p = [torch.tensor(v.astype(np.float64), requires_grad=True) for v in (w1, w2, wl)]
+    a1 = F.relu(F.conv2d(xt, p[0], padding=1))
+    s = F.conv2d(a1, p[1], padding=1) + xt
+    pooled = F.relu(s).mean((2, 3))
+    logits = pooled @ p[2].t()
+    lt = F.cross_entropy(logits, torch.tensor(tgt.astype(np.float64)), reduction="none")
+    lt.sum().backward()
+    assert hp.rel_l2(host(loss), lt.detach().numpy()) <= tol
+    assert hp.rel_l2(host(Z), logits.detach().numpy()) <= tol
+    for n, t in (("w1", p[0]), ("w2", p[1]), ("wl", p[2]), ("x", xt)):
+        assert hp.rel_l2(grads[n], t.grad.numpy()) <= tol, n
+    lr_ = float(npd(lr))
+    for Wt, t in ((W1, p[0]), (W2, p[1]), (WL, p[2])):
+        assert hp.rel_l2(host(Wt), (t.detach() - lr_ * t.grad).numpy()) <= tol
