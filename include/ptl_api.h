@@ -222,9 +222,11 @@ int ptl_sync(void);
  * calls, the LDS-DMA pipelined GEMM elsewhere, the register-staged GEMM as the
  * last resort); 1 = the register-staged GEMM only; 2 = as 0, but the direct
  * convolution kernel is taken whenever the geometry fits it, however small the
- * call.  All routes compute the same products.
- * ptl_last_conv_direct() tells whether the last Conv2D forward or
- * input-gradient call ran the direct kernel (1) or a GEMM route (0). */
+ * call; 3 = as 0, but the sum-over-filter-taps route (unit-stride layers whose
+ * channel counts fill whole 128-byte slabs) is taken whenever the geometry fits
+ * it.  All routes compute the same products.
+ * ptl_last_conv_direct() tells whether the last Conv2D call ran one of the
+ * convolution kernels (1) or the implicit-im2col GEMM (0). */
 void ptl_set_gemm_path(int path);
 int ptl_last_conv_direct(void);
 /* hipEvent timing on the library stream: begin records, end records,

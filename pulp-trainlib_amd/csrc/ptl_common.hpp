@@ -64,6 +64,14 @@ struct GemmArgs {
     int splits;
     int kchunk;    // K range per split (multiple of the k tile)
     int tiles_n, tiles_m;
+    // Convolution as a sum over filter taps (look-up-free kernel only): k runs over (tap, channel); after the
+    // `slabs_per_tap` slabs of a tap the A pointer jumps to the next tap of the padded, channel-blocked input:
+    // by tap_jump_x bytes within a filter row, by tap_jump_y at the end of one.  taps <= 1: an ordinary product.
+    int taps, slabs_per_tap, tap_kw;
+    long long tap_jump_x, tap_jump_y;
+    // Weight gradient over taps: grid.y enumerates (tap, k split), tap_splits splits per tap; tap (ky, kx) reads
+    // B shifted by ky*tap_jump_y + kx*tap_jump_x bytes and writes its own partial sums.  0: off.
+    int tap_splits;
 };
 
 inline AxisMap axis_plain(int n, int stride, int base = 0) {
@@ -125,7 +133,7 @@ struct State {
     hipEvent_t ev0 = nullptr, ev1 = nullptr;
     int num_cu = 256;
     void *zeros = nullptr;  // 256 zero bytes: source of elements that do not exist
-    int gemm_path = 0;      // 0: fastest kernel that fits; 1: staged GEMM only; 2: direct convolution whenever it fits
+    int gemm_path = 0;      // 0: fastest kernel that fits; 1: staged GEMM only; 2: direct convolution whenever it fits; 3: tap-sum route whenever it fits
     int last_conv_direct = 0;  // 1 if the last Conv2D forward / input-gradient call ran the direct kernel
 };
 

@@ -1,0 +1,265 @@
+// Convolution as a sum over filter taps on the look-up-free pipelined GEMM (unit stride, channel-major
+// tensors, channel counts that are multiples of a 128-byte slab: 64 halves / 32 floats).
+//
+//   Y[(b,y,x)][co] = sum over taps (ky,kx) and channels c of  Xp[b][c][y+ky][x+kx] * W[co][c][ky][kx]
+//
+// Two small passes prepare the operands in the library's scratch memory:
+//   * the input, zero-padded and channel-blocked as [c/VEC][b][y][x][VEC] (16-byte chunks = VEC consecutive
+//     channels of one position).  For a fixed tap this IS a plain [pixel][channel] matrix: pixel (b,y,x) starts
+//     at a fixed offset, chunk j of a slab sits j channel-block planes further, and moving to another tap adds
+//     one constant to every address - no border tests, no im2col;
+//   * the filters as [co][tap][c], so that k = (tap, c) is contiguous.
+// The GEMM kernel then runs its ordinary slab loop over k = taps x channels with one pointer jump per tap.
+// The input gradient is the same product over the (padded) output gradient with flipped, transposed filters;
+// the filter pass reads them through the strides of the descriptor.
+#include "ptl_conv_tile.hpp"
+#include "ptl_gemm_async.hpp"
+
+namespace ptl {
+
+// in: [b][C][H][W] (strides sb, sc; rows contiguous) -> out: [C/VEC][B][Hp][Wp] chunks, zero halo.
+template <typename T>
+__global__ __launch_bounds__(256) void chw_to_blocked_padded_kernel(const T *__restrict__ in, uint4 *__restrict__ out,
+                                                                    int B, int H, int W, int Hp, int Wp, int padU,
+                                                                    int padL, long long sb, long long sc,
+                                                                    int cblocks, long long total) {
+    constexpr int VEC = 16 / (int)sizeof(T);
+    const long long i = (long long)blockIdx.x * 256 + threadIdx.x;
+    if (i >= total) return;
+    const int xp = (int)(i % Wp);
+    long long r = i / Wp;
+    const int yp = (int)(r % Hp);
+    r /= Hp;
+    const int b = (int)(r % B), cb = (int)(r / B);
+    const int y = yp - padU, x = xp - padL;
+    union {
+        uint4 v;
+        T e[VEC];
+    } u;
+    if (cb < cblocks && y >= 0 && y < H && x >= 0 && x < W) {  // beyond the last block: zero margin
+        const T *src = in + b * sb + (long long)(cb * VEC) * sc + (long long)y * W + x;
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) u.e[e] = src[e * sc];
+    } else {
+        u.v = make_uint4(0, 0, 0, 0);
+    }
+    out[i] = u.v;
+}
+
+// out[m][tap][c] = W[base + m*sm + c*sc + ky*sy + kx*sx]
+template <typename T>
+__global__ __launch_bounds__(256) void filters_tap_major_kernel(const T *__restrict__ w, T *__restrict__ out, int C,
+                                                                int KW, int taps, long long base, long long sm,
+                                                                long long sc, long long sy, long long sx,
+                                                                long long total) {
+    const long long i = (long long)blockIdx.x * 256 + threadIdx.x;
+    if (i >= total) return;
+    const int c = (int)(i % C);
+    const long long r = i / C;
+    const int t = (int)(r % taps);
+    const long long m = r / taps;
+    out[i] = w[base + m * sm + c * sc + (t / KW) * sy + (t % KW) * sx];
+}
+
+template <typename T>
+int conv_taps(const ConvTileDesc &d, const void *X, const void *Wt, void *Y, const OutMap &c) {
+    State &st = state();
+    constexpr int ES = (int)sizeof(T), VEC = 16 / ES, SK = 128 / ES;
+    if (d.in_hwc || d.sh != 1 || d.sw != 1 || d.Cin % SK || d.x_sy != d.Win) return -1;
+    const int Hp = d.Hin + d.padU + d.padD, Wp = d.Win + d.padL + d.padR, taps = d.KH * d.KW;
+    if (d.Ho != Hp - d.KH + 1 || d.Wo != Wp - d.KW + 1 || taps < 2) return -1;
+    const int cblocks = d.Cin / VEC;
+    const long long plane = (long long)Hp * Wp * VEC;            // elements of one (channel block, sample) plane
+    const long long xb_elems = (long long)cblocks * d.batch * plane;
+    const long long wr_elems = (long long)d.Cout * taps * d.Cin;
+    const long long npix = (long long)d.batch * d.Ho * d.Wo;
+    if (xb_elems * ES >= ((long long)1 << 31) || npix >= ((long long)1 << 31) || wr_elems >= ((long long)1 << 31))
+        return -1;
+    // worth it only when the pixel tiles fill the chip: the passes above cost two extra launches
+    if (st.gemm_path == 2) return -1;
+    if (st.gemm_path != 3 && npix / 128 * ((d.Cout + 127) / 128) < st.num_cu) return -1;
+    char *buf = static_cast<char *>(scratch((size_t)(xb_elems + wr_elems) * ES + 256));
+    if (!buf) return 2;
+    uint4 *xb = reinterpret_cast<uint4 *>(buf);
+    T *wr = reinterpret_cast<T *>(buf + (((size_t)xb_elems * ES + 255) & ~(size_t)255));
+    const long long chunks = xb_elems / VEC;
+    hipLaunchKernelGGL((chw_to_blocked_padded_kernel<T>), dim3((unsigned)((chunks + 255) / 256)), dim3(256), 0,
+                       st.stream, reinterpret_cast<const T *>(X), xb, d.batch, d.Hin, d.Win, Hp, Wp, d.padU, d.padL,
+                       d.x_sb, d.x_sc, cblocks, chunks);
+    if (!hip_ok(hipGetLastError(), "blocked layout launch")) return 2;
+    hipLaunchKernelGGL((filters_tap_major_kernel<T>), dim3((unsigned)((wr_elems + 255) / 256)), dim3(256), 0,
+                       st.stream, reinterpret_cast<const T *>(Wt), wr, d.Cin, d.KW, taps, d.w_base, d.w_sm, d.w_sc,
+                       d.w_sy, d.w_sx, wr_elems);
+    if (!hip_ok(hipGetLastError(), "filter layout launch")) return 2;
+
+    GemmArgs q = {};
+    q.A = xb;
+    q.B = wr;
+    q.C = Y;
+    q.N = (int)npix;
+    q.M = d.Cout;
+    q.K = taps * d.Cin;
+    q.a.HL = q.a.WL = q.b.HL = q.b.WL = 1;
+    // pixel (b, y, x) of the padded, blocked input; a 16-byte chunk further along k is one block plane on
+    q.a.row = {};
+    q.a.row.n = q.N;
+    q.a.row.d1 = d.Ho;
+    q.a.row.d0 = d.Wo;
+    q.a.row.o2 = (int)plane;
+    q.a.row.o1 = Wp * VEC;
+    q.a.row.o0 = VEC;
+    const long long kstride = (long long)d.batch * plane / VEC;  // per channel, so that VEC channels = one plane
+    if (kstride >= ((long long)1 << 31) || plane >= ((long long)1 << 31)) return -1;
+    q.a.k = axis_plain(q.K, (int)kstride);
+    q.a.mode = FILL_VEC_K;
+    q.b.row = axis_plain(d.Cout, q.K);
+    q.b.k = axis_plain(q.K, 1);
+    q.b.mode = FILL_VEC_K;
+    q.c = c;
+    q.taps = taps;
+    q.slabs_per_tap = d.Cin / SK;
+    q.tap_kw = d.KW;
+    const long long tap_span = (long long)q.slabs_per_tap * SK * kstride * ES;  // what the slabs of a tap advance A by
+    q.tap_jump_x = (long long)VEC * ES - tap_span;
+    q.tap_jump_y = (long long)(Wp - (d.KW - 1)) * VEC * ES - tap_span;
+    return gemm_async<T>(q);
+}
+
+
+// ---------------------------------------------------------------------------------------------------------
+// Weight gradient the same way: for every tap (ky,kx)
+//   dW[co][c][ky][kx] = sum over padded positions pp of all samples of  dYp[co][pp] * Xp[c][pp + ky*Wp + kx]
+// with dYp the output gradient embedded in the padded grid (zero where no output pixel sits) and Xp the
+// blocked, padded input: per tap a [co][pp] x [pp][c] product whose second operand is the SAME matrix
+// shifted by a constant.  One launch covers all taps and k splits (grid.y), one kernel adds the partial sums.
+
+// out[co][k], k = (b, yp, xp) flattened and padded to Kr: dY[b][co][yp][xp] inside the output, else zero.
+template <typename T>
+__global__ __launch_bounds__(256) void embed_gradient_kernel(const T *__restrict__ dy, T *__restrict__ out, int B,
+                                                             int Cout, int Ho, int Wo, int Hp, int Wp, long long Kr,
+                                                             long long total) {
+    const long long i = (long long)blockIdx.x * 256 + threadIdx.x;
+    if (i >= total) return;
+    const long long k = i % Kr;
+    const int co = (int)(i / Kr);
+    const int xp = (int)(k % Wp);
+    const long long r = k / Wp;
+    const int yp = (int)(r % Hp);
+    const long long b = r / Hp;
+    T v = (T)0;
+    if (b < B && yp < Ho && xp < Wo) v = dy[((b * Cout + co) * Ho + yp) * (long long)Wo + xp];
+    out[i] = v;
+}
+
+// dW[(n*M + m)*taps + tap] = sum over the splits of ws[tap][split][n][m]; 64 outputs x 4 split groups per
+// workgroup, four loads in flight per thread.
+template <typename T>
+__global__ __launch_bounds__(256) void taps_wg_reduce_kernel(const float *__restrict__ ws, T *__restrict__ dW,
+                                                             long long total, int splits, int taps) {
+    __shared__ float part[4][64];
+    const int o = threadIdx.x & 63, sg = threadIdx.x >> 6, tap = blockIdx.y;
+    const long long idx = (long long)blockIdx.x * 64 + o;
+    float s = 0.f;
+    if (idx < total) {
+        const float *src = ws + (long long)tap * splits * total + idx;
+        int z = sg;
+        for (; z + 12 < splits; z += 16) {
+            float v[4];
+#pragma unroll
+            for (int u = 0; u < 4; ++u) v[u] = src[(long long)(z + u * 4) * total];
+#pragma unroll
+            for (int u = 0; u < 4; ++u) s += v[u];
+        }
+        for (; z < splits; z += 4) s += src[(long long)z * total];
+    }
+    part[sg][o] = s;
+    __syncthreads();
+    if (sg != 0 || idx >= total) return;
+    s += part[1][o] + part[2][o] + part[3][o];
+    dW[idx * taps + tap] = (T)s;
+}
+
+template <typename T>
+int conv_taps_wg(const ConvTileDesc &d, const void *X, const void *dY, void *dW) {
+    State &st = state();
+    constexpr int ES = (int)sizeof(T), VEC = 16 / ES, SK = 128 / ES;
+    if (d.in_hwc || d.sh != 1 || d.sw != 1 || d.Cin % VEC || d.x_sy != d.Win) return -1;
+    if (st.gemm_path == 2) return -1;
+    if (st.gemm_path != 3 && (d.Cin < 128 || d.Cout < 128)) return -1;  // measured: below that the direct kernel wins
+    const int Hp = d.Hin + d.padU + d.padD, Wp = d.Win + d.padL + d.padR, taps = d.KH * d.KW;
+    if (d.Ho != Hp - d.KH + 1 || d.Wo != Wp - d.KW + 1) return -1;
+    const int cblocks = d.Cin / VEC;
+    const long long plane = (long long)Hp * Wp * VEC;
+    const long long Kp = (long long)d.batch * Hp * Wp;              // padded positions of all samples
+    const long long Kr = (Kp + SK - 1) / SK * SK;
+    const long long margin = (Kr - Kp) + (long long)(d.KH - 1) * Wp + d.KW + SK;  // positions read past the end
+    const long long xb_chunks = (long long)cblocks * d.batch * Hp * Wp + margin;
+    const long long gy_elems = (long long)d.Cout * Kr;
+    if (xb_chunks * 16 >= ((long long)1 << 31) || gy_elems * ES >= ((long long)1 << 31) || Kr >= ((long long)1 << 31))
+        return -1;
+    const int bm = (d.Cout >= 128 && d.Cin >= 128) ? 128 : 64;
+    const long long tiles = (long long)((d.Cout + bm - 1) / bm) * ((d.Cin + bm - 1) / bm);
+    long long S = (2LL * st.num_cu + tiles * taps - 1) / (tiles * taps);
+    const long long max_s = Kr / (4 * SK) > 0 ? Kr / (4 * SK) : 1;
+    if (S > max_s) S = max_s;
+    if (S < 1) S = 1;
+    long long kchunk = ((Kr + S - 1) / S + SK - 1) / SK * SK;
+    S = (Kr + kchunk - 1) / kchunk;
+    const size_t ws_bytes = (size_t)taps * S * d.Cout * d.Cin * sizeof(float);
+    if (ws_bytes > ((size_t)1 << 30)) return -1;
+    char *buf = static_cast<char *>(scratch((size_t)xb_chunks * 16 + 256 + (size_t)gy_elems * ES));
+    if (!buf) return 2;
+    uint4 *xb = reinterpret_cast<uint4 *>(buf);
+    T *gy = reinterpret_cast<T *>(buf + (((size_t)xb_chunks * 16 + 255) & ~(size_t)255));
+    float *ws = workspace(ws_bytes);
+    if (!ws) return 2;
+    hipLaunchKernelGGL((chw_to_blocked_padded_kernel<T>), dim3((unsigned)((xb_chunks + 255) / 256)), dim3(256), 0,
+                       st.stream, reinterpret_cast<const T *>(X), xb, d.batch, d.Hin, d.Win, Hp, Wp, d.padU, d.padL,
+                       d.x_sb, d.x_sc, cblocks, xb_chunks);
+    if (!hip_ok(hipGetLastError(), "blocked layout launch")) return 2;
+    hipLaunchKernelGGL((embed_gradient_kernel<T>), dim3((unsigned)((gy_elems + 255) / 256)), dim3(256), 0, st.stream,
+                       reinterpret_cast<const T *>(dY), gy, d.batch, d.Cout, d.Ho, d.Wo, Hp, Wp, Kr, gy_elems);
+    if (!hip_ok(hipGetLastError(), "gradient layout launch")) return 2;
+
+    GemmArgs q = {};
+    q.A = gy;
+    q.B = xb;
+    q.C = dW;
+    q.ws = ws;
+    q.N = d.Cout;
+    q.M = d.Cin;
+    q.K = (int)Kr;
+    q.a.HL = q.a.WL = q.b.HL = q.b.WL = 1;
+    q.a.row = axis_plain(d.Cout, (int)Kr);
+    q.a.k = axis_plain((int)Kr, 1);
+    q.a.mode = FILL_VEC_K;
+    const long long cb_stride = (long long)d.batch * plane;
+    if (cb_stride >= ((long long)1 << 31)) return -1;
+    q.b.row = axis_two(d.Cin, VEC, (int)cb_stride, 1);
+    q.b.k = axis_plain((int)Kr, VEC);
+    q.b.mode = FILL_VEC_R;
+    q.c.n = axis_plain(d.Cout, d.Cin * taps);
+    q.c.m = axis_plain(d.Cin, taps);
+    q.kchunk = (int)kchunk;
+    q.splits = (int)(taps * S);
+    q.tap_splits = (int)S;
+    q.tap_kw = d.KW;
+    q.tap_jump_x = (long long)VEC * ES;
+    q.tap_jump_y = (long long)Wp * VEC * ES;
+    if (!plain_operand<T>(q.a, q.kchunk, q.K) || !plain_operand<T>(q.b, q.kchunk, q.K)) return -1;
+    int rc = bm == 128 ? launch_plain<T, 128, 128, 512, 2, 2, 2, 3, 1>(q, st.stream)
+                       : launch_plain<T, 64, 64, 1024, 2, 2, 4, 3, 1>(q, st.stream);
+    if (rc != 0 || q.splits == 1) return rc;  // a single 1x1 tap without k split wrote dW itself
+    const long long total = (long long)d.Cout * d.Cin;
+    hipLaunchKernelGGL((taps_wg_reduce_kernel<T>), dim3((unsigned)((total + 63) / 64), taps), dim3(256), 0, st.stream,
+                       ws, reinterpret_cast<T *>(dW), total, (int)S, taps);
+    return hip_ok(hipGetLastError(), "tap reduce launch") ? 0 : 2;
+}
+
+template int conv_taps_wg<float>(const ConvTileDesc &, const void *, const void *, void *);
+template int conv_taps_wg<half_t>(const ConvTileDesc &, const void *, const void *, void *);
+
+template int conv_taps<float>(const ConvTileDesc &, const void *, const void *, void *, const OutMap &);
+template int conv_taps<half_t>(const ConvTileDesc &, const void *, const void *, void *, const OutMap &);
+
+}  // namespace ptl

@@ -72,6 +72,15 @@ inline int conv_raw_rows(int bm, int Ho, int Wo, int sh, int KH, int THP, long l
 //   dW(co, ci, ky, kx) = sum_{b, y, x} dY(b, co, y, x) * in(b, ci, y*sh + ky - padU, x*sw + kx - padL)
 // with dY channel-major [b][Cout][Ho*Wo] and dW dense [Cout][Cin][KH][KW].  Returns 0, a positive
 // status on a HIP error, or -1 when the geometry does not fit the kernel.
+// The same convolution as a sum over filter taps on the look-up-free GEMM (unit stride, channel-major input,
+// channels a multiple of a slab); -1 when the geometry does not fit.  Input and filters are re-laid in scratch.
+template <typename T>
+int conv_taps(const ConvTileDesc &d, const void *X, const void *Wt, void *Y, const OutMap &c);
+
+// Weight gradient over filter taps on the same GEMM (partial sums per tap and k split + one reduction).
+template <typename T>
+int conv_taps_wg(const ConvTileDesc &d, const void *X, const void *dY, void *dW);
+
 template <typename T>
 int conv_tile_wg(const ConvTileDesc &d, const void *X, const void *dY, void *dW);
 

@@ -35,6 +35,10 @@ int gemm_async(GemmArgs &g) {
     const bool need_lut = !(plain_operand<T>(g.a, g.kchunk, g.K) && plain_operand<T>(g.b, g.kchunk, g.K));
     int need = need_lut ? (g.K + ASYNC_KWMAX - 1) / ASYNC_KWMAX : 1;
     if (want < need) want = need;
+    if (g.taps > 1) {  // a sum over filter taps runs on the look-up-free kernel in one piece
+        if (need_lut) return -1;
+        want = 1;
+    }
     if (want > 1) {
         int min_chunk = 4 * SK;
         int max_splits = (g.K + min_chunk - 1) / min_chunk;

@@ -260,7 +260,8 @@ static int conv2d_fw(const Args *a, int ns, const char *fn) {
             c.n = axis_plain(ns * P, g.Co);
             c.m = axis_plain(g.Co, 1);
         }
-        rc = conv_tile<T>(d, X, Wt, Y, c);
+        rc = conv_taps<T>(d, X, Wt, Y, c);
+        if (rc < 0) rc = conv_tile<T>(d, X, Wt, Y, c);
         if (rc > 0) return sg.finish(rc);
         if (rc == 0) state().last_conv_direct = 1;
     }
@@ -338,7 +339,8 @@ static int conv2d_wg(const Args *a, int ns, const char *fn) {
         d.KH = g.Hk; d.KW = g.Wk; d.sh = g.sh; d.sw = g.sw;
         d.padU = g.Up; d.padD = g.Dp; d.padL = g.Lp; d.padR = g.Rp;
         d.x_sb = (long long)g.Ci * g.H * g.W; d.x_sc = (long long)g.H * g.W; d.x_sy = g.W;
-        rc = conv_tile_wg<T>(d, X, dY, dW);
+        rc = conv_taps_wg<T>(d, X, dY, dW);
+        if (rc < 0) rc = conv_tile_wg<T>(d, X, dY, dW);
         if (rc > 0) return sg.finish(rc);
         if (rc == 0) state().last_conv_direct = 1;
     }
@@ -435,7 +437,9 @@ static int conv2d_ig(const Args *a, int ns, const char *fn) {
             c.n = axis_plain(ns * g.H * g.W, g.Ci);
             c.m = axis_plain(g.Ci, 1);
         }
-        int rc = conv_tile<T>(d, dY, Wt, dX, c);
+        // (the zero-stuffed gradient of a strided layer lives in the scratch buffer the tap route would reuse)
+        int rc = (g.sh == 1 && g.sw == 1) ? conv_taps<T>(d, dY, Wt, dX, c) : -1;
+        if (rc < 0) rc = conv_tile<T>(d, dY, Wt, dX, c);
         if (rc == 0) state().last_conv_direct = 1;
         if (rc >= 0) return sg.finish(rc);
     }

@@ -174,6 +174,71 @@ def test_conv2d_direct_kernel_hwc(pkg, orc, gpu, dt, case):
         gpu.ptl_set_gemm_path(0)
 
 
+# Unit-stride layers whose channel counts are multiples of a 128-byte slab (64 halves / 32 floats) run as a sum
+# over filter taps on the look-up-free GEMM (padded, channel-blocked copy of the input): forward when Ci fits,
+# input gradient when Co does.  Cases: square and ragged images, asymmetric padding, 5x5 and 2x3 filters, tile
+# counts that leave a ragged last tile, channel counts of one and several slabs.
+TAP_CASES = [
+    # Ci, H, W, Co, Hk, Wk, pad(L,R,U,D), ns
+    (64, 14, 14, 64, 3, 3, (1, 1, 1, 1), 4),
+    (128, 9, 11, 64, 3, 3, (1, 1, 1, 1), 3),
+    (64, 12, 10, 130, 3, 3, (0, 2, 1, 0), 2),
+    (64, 8, 8, 192, 5, 5, (2, 2, 2, 2), 2),
+    (192, 7, 9, 64, 2, 3, (1, 1, 0, 1), 5),
+    (64, 6, 6, 64, 3, 3, (0, 0, 0, 0), 1),
+]
+
+
+@pytest.mark.parametrize("dt", ["fp32", "fp16"])
+@pytest.mark.parametrize("case", TAP_CASES)
+def test_conv2d_tap_sum_route(pkg, orc, gpu, dt, case):
+    Ci, H, W, Co, Hk, Wk, pad, ns = case
+    slab = 64 if dt == "fp16" else 32
+    gpu.ptl_set_gemm_path(3)
+    try:
+        conv_parity(pkg, orc, gpu, dt, Ci, H, W, Co, Hk, Wk, pad, (1, 1), 0, ns, 0xC0DE0071, via_batched=True)
+        # the last call of conv_parity is the input gradient, whose "input" channels are Co
+        assert gpu.ptl_last_conv_direct() == (1 if Co % slab == 0 else gpu.ptl_last_conv_direct())
+        # forward and weight gradient alone: both take a convolution kernel
+        nd = hp.np_dtype(dt)
+        Ho, Wo = hp.conv_out(H, Hk, pad[2], pad[3], 1), hp.conv_out(W, Wk, pad[0], pad[1], 1)
+        x, w = dev(hp.uniform(1, (ns, Ci, H, W), dtype=nd)), dev(hp.uniform(2, (Co, Ci, Hk, Wk), dtype=nd))
+        dy = dev(hp.uniform(3, (ns, Co, Ho, Wo), dtype=nd))
+        y, dw = dev(np.zeros((ns, Co, Ho, Wo), nd)), dev(np.zeros((Co, Ci, Hk, Wk), nd))
+        a, keep = hp.conv2d_args(pkg, x, None, w, dw, y, dy, Ci, H, W, Co, Hk, Wk, Ho, Wo, pad, (1, 1))
+        for s in ("fw", "wg"):
+            pkg.call("ptl_conv2d_%s_%s_batched" % (dt, s), a, ns)
+            assert gpu.ptl_last_conv_direct() == 1, s
+    finally:
+        gpu.ptl_set_gemm_path(0)
+
+
+def test_conv2d_routes_agree_on_large_channels(pkg, gpu):
+    """The tap-sum route, the direct kernels and the implicit-im2col GEMM give the same forward, weight gradient
+    and input gradient (fp16, 64 -> 64 channels)."""
+    Ci = Co = 64
+    H = W = 14
+    ns = 6
+    nd = np.float16
+    x, w = dev(hp.uniform(11, (ns, Ci, H, W), dtype=nd)), dev(hp.uniform(12, (Co, Ci, 3, 3), dtype=nd))
+    dy = dev(hp.uniform(13, (ns, Co, H, W), dtype=nd))
+    res = {}
+    for path in (1, 2, 3):
+        y, dx, dw = (dev(np.zeros(s, nd)) for s in ((ns, Co, H, W), (ns, Ci, H, W), (Co, Ci, 3, 3)))
+        a, keep = hp.conv2d_args(pkg, x, dx, w, dw, y, dy, Ci, H, W, Co, 3, 3, H, W, (1, 1, 1, 1), (1, 1))
+        gpu.ptl_set_gemm_path(path)
+        try:
+            for s in ("fw", "wg", "ig"):
+                pkg.call("ptl_conv2d_fp16_%s_batched" % s, a, ns)
+        finally:
+            gpu.ptl_set_gemm_path(0)
+        sync(gpu)
+        res[path] = [host(t).astype(np.float64) for t in (y, dw, dx)]
+    for path in (2, 3):
+        for got, ref in zip(res[path], res[1]):
+            assert rel_l2(got, ref) <= 2e-3
+
+
 # The direct weight-gradient kernel needs unit column stride and row lengths that are multiples of the
 # 16-byte vector (8 halves / 4 floats).
 DIRECT_WG_CASES = [
