@@ -46,6 +46,19 @@ __global__ __launch_bounds__(256) void chw_to_blocked_padded_kernel(const T *__r
     out[i] = u.v;
 }
 
+// Launches the padded, blocked copy of X ([b][C][H][W]) with `margin` zero chunks after it.
+template <typename T>
+static int blocked_padded_copy(const T *X, uint4 *xb, const ConvTileDesc &d, int Hp, int Wp, long long margin) {
+    State &st = state();
+    constexpr int VEC = 16 / (int)sizeof(T);
+    const int cblocks = d.Cin / VEC;
+    const long long planes = (long long)cblocks * d.batch, chunks = planes * Hp * Wp;
+    hipLaunchKernelGGL((chw_to_blocked_padded_kernel<T>), dim3((unsigned)((chunks + margin + 255) / 256)), dim3(256),
+                       0, st.stream, X, xb, d.batch, d.Hin, d.Win, Hp, Wp, d.padU, d.padL, d.x_sb, d.x_sc, cblocks,
+                       chunks + margin);
+    return hip_ok(hipGetLastError(), "blocked layout launch") ? 0 : 2;
+}
+
 // out[m][tap][c] = W[base + m*sm + c*sc + ky*sy + kx*sx]
 template <typename T>
 __global__ __launch_bounds__(256) void filters_tap_major_kernel(const T *__restrict__ w, T *__restrict__ out, int C,
@@ -82,11 +95,7 @@ int conv_taps(const ConvTileDesc &d, const void *X, const void *Wt, void *Y, con
     if (!buf) return 2;
     uint4 *xb = reinterpret_cast<uint4 *>(buf);
     T *wr = reinterpret_cast<T *>(buf + (((size_t)xb_elems * ES + 255) & ~(size_t)255));
-    const long long chunks = xb_elems / VEC;
-    hipLaunchKernelGGL((chw_to_blocked_padded_kernel<T>), dim3((unsigned)((chunks + 255) / 256)), dim3(256), 0,
-                       st.stream, reinterpret_cast<const T *>(X), xb, d.batch, d.Hin, d.Win, Hp, Wp, d.padU, d.padL,
-                       d.x_sb, d.x_sc, cblocks, chunks);
-    if (!hip_ok(hipGetLastError(), "blocked layout launch")) return 2;
+    if (int rc = blocked_padded_copy<T>(reinterpret_cast<const T *>(X), xb, d, Hp, Wp, 0)) return rc;
     hipLaunchKernelGGL((filters_tap_major_kernel<T>), dim3((unsigned)((wr_elems + 255) / 256)), dim3(256), 0,
                        st.stream, reinterpret_cast<const T *>(Wt), wr, d.Cin, d.KW, taps, d.w_base, d.w_sm, d.w_sc,
                        d.w_sy, d.w_sx, wr_elems);
@@ -134,21 +143,37 @@ int conv_taps(const ConvTileDesc &d, const void *X, const void *Wt, void *Y, con
 // shifted by a constant.  One launch covers all taps and k splits (grid.y), one kernel adds the partial sums.
 
 // out[co][k], k = (b, yp, xp) flattened and padded to Kr: dY[b][co][yp][xp] inside the output, else zero.
+// One thread per 16 bytes of the destination.
 template <typename T>
-__global__ __launch_bounds__(256) void embed_gradient_kernel(const T *__restrict__ dy, T *__restrict__ out, int B,
+__global__ __launch_bounds__(256) void embed_gradient_kernel(const T *__restrict__ dy, uint4 *__restrict__ out, int B,
                                                              int Cout, int Ho, int Wo, int Hp, int Wp, long long Kr,
                                                              long long total) {
+    constexpr int VEC = 16 / (int)sizeof(T);
     const long long i = (long long)blockIdx.x * 256 + threadIdx.x;
     if (i >= total) return;
-    const long long k = i % Kr;
-    const int co = (int)(i / Kr);
-    const int xp = (int)(k % Wp);
-    const long long r = k / Wp;
-    const int yp = (int)(r % Hp);
-    const long long b = r / Hp;
-    T v = (T)0;
-    if (b < B && yp < Ho && xp < Wo) v = dy[((b * Cout + co) * Ho + yp) * (long long)Wo + xp];
-    out[i] = v;
+    const long long kv = Kr / VEC;
+    const long long k0 = (i % kv) * VEC;
+    const int co = (int)(i / kv);
+    int xp = (int)(k0 % Wp);
+    long long r = k0 / Wp;
+    int yp = (int)(r % Hp);
+    long long b = r / Hp;
+    union {
+        uint4 v;
+        T e[VEC];
+    } u;
+#pragma unroll
+    for (int e = 0; e < VEC; ++e) {
+        u.e[e] = (b < B && yp < Ho && xp < Wo) ? dy[((b * Cout + co) * Ho + yp) * (long long)Wo + xp] : (T)0;
+        if (++xp == Wp) {
+            xp = 0;
+            if (++yp == Hp) {
+                yp = 0;
+                ++b;
+            }
+        }
+    }
+    out[i] = u.v;
 }
 
 // dW[(n*M + m)*taps + tap] = sum over the splits of ws[tap][split][n][m]; 64 outputs x 4 split groups per
@@ -213,12 +238,10 @@ int conv_taps_wg(const ConvTileDesc &d, const void *X, const void *dY, void *dW)
     T *gy = reinterpret_cast<T *>(buf + (((size_t)xb_chunks * 16 + 255) & ~(size_t)255));
     float *ws = workspace(ws_bytes);
     if (!ws) return 2;
-    hipLaunchKernelGGL((chw_to_blocked_padded_kernel<T>), dim3((unsigned)((xb_chunks + 255) / 256)), dim3(256), 0,
-                       st.stream, reinterpret_cast<const T *>(X), xb, d.batch, d.Hin, d.Win, Hp, Wp, d.padU, d.padL,
-                       d.x_sb, d.x_sc, cblocks, xb_chunks);
-    if (!hip_ok(hipGetLastError(), "blocked layout launch")) return 2;
-    hipLaunchKernelGGL((embed_gradient_kernel<T>), dim3((unsigned)((gy_elems + 255) / 256)), dim3(256), 0, st.stream,
-                       reinterpret_cast<const T *>(dY), gy, d.batch, d.Cout, d.Ho, d.Wo, Hp, Wp, Kr, gy_elems);
+    if (int rc = blocked_padded_copy<T>(reinterpret_cast<const T *>(X), xb, d, Hp, Wp, margin)) return rc;
+    hipLaunchKernelGGL((embed_gradient_kernel<T>), dim3((unsigned)((gy_elems / VEC + 255) / 256)), dim3(256), 0,
+                       st.stream, reinterpret_cast<const T *>(dY), reinterpret_cast<uint4 *>(gy), d.batch, d.Cout, d.Ho,
+                       d.Wo, Hp, Wp, Kr, gy_elems / VEC);
     if (!hip_ok(hipGetLastError(), "gradient layout launch")) return 2;
 
     GemmArgs q = {};
