@@ -90,7 +90,8 @@ int conv_taps(const ConvTileDesc &d, const void *X, const void *Wt, void *Y, con
         return -1;
     // worth it only when the pixel tiles fill the chip: the passes above cost two extra launches
     if (st.gemm_path == 2) return -1;
-    if (st.gemm_path != 3 && npix / 128 * ((d.Cout + 127) / 128) < st.num_cu) return -1;
+    // (and only with at least 64 filters: narrower products fall to the GEMM's slim tiles, where the direct kernel wins)
+    if (st.gemm_path != 3 && (d.Cout < 64 || npix / 128 * ((d.Cout + 127) / 128) < st.num_cu)) return -1;
     char *buf = static_cast<char *>(scratch((size_t)(xb_elems + wr_elems) * ES + 256));
     if (!buf) return 2;
     uint4 *xb = reinterpret_cast<uint4 *>(buf);
