@@ -1,0 +1,169 @@
+"""A ResNet-20-shaped (CIFAR geometry) training step assembled from the library's entry points, the way a
+generated `net.c` of the reference strings its layer calls together: 3x3 stem, three stages of three residual
+blocks (16/32/64 channels, stride-2 1x1 projection shortcuts), ReLU, global average pooling, a linear
+classifier, cross-entropy and one gradient-descent update.  No normalisation layers: the reference has no
+batch-norm backward.  Used by the GPU parity test and by the benchmark's detail table."""
+import ctypes
+
+import numpy as np
+
+import helpers as hp
+
+
+def resnet20_spec(num_classes=10):
+    """[(name, cin, cout, k, stride)] of every convolution, in forward order, plus the block structure."""
+    convs = [("stem", 3, 16, 3, 1)]
+    blocks = []
+    cin = 16
+    for stage, cout in enumerate((16, 32, 64)):
+        for b in range(3):
+            stride = 2 if (stage > 0 and b == 0) else 1
+            n = "s%db%d" % (stage, b)
+            convs.append((n + "c1", cin, cout, 3, stride))
+            convs.append((n + "c2", cout, cout, 3, 1))
+            proj = None
+            if stride != 1 or cin != cout:
+                proj = n + "sc"
+                convs.append((proj, cin, cout, 1, stride))
+            blocks.append((n, cin, cout, stride, proj))
+            cin = cout
+    return convs, blocks, num_classes
+
+
+def init_weights(seed, dt):
+    convs, blocks, ncls = resnet20_spec()
+    w = {}
+    for i, (n, ci, co, k, s) in enumerate(convs):
+        lim = float(np.sqrt(6.0 / (ci * k * k)))
+        w[n] = hp.uniform(seed + i, (co, ci, k, k), -lim, lim).astype(hp.np_dtype(dt))
+    w["fc"] = hp.uniform(seed + 99, (ncls, 64), -0.3, 0.3).astype(hp.np_dtype(dt))
+    return w
+
+
+class ResNetStep:
+    """Device buffers, argument structs and the call sequence of one training step on `ns` samples."""
+
+    def __init__(self, pkg, lib, torch, dt, ns, weights, lr=0.01):
+        self.pkg, self.lib, self.dt, self.ns, self.lr = pkg, lib, dt, ns, lr
+        tdt = torch.float16 if dt == "fp16" else torch.float32
+        dev = lambda a: torch.from_numpy(np.ascontiguousarray(a)).cuda()
+        z = lambda *s: torch.zeros(*s, dtype=tdt, device="cuda")
+        convs, blocks, ncls = resnet20_spec()
+        self.W = {n: dev(v) for n, v in weights.items()}
+        self.dW = {n: z(*v.shape) for n, v in weights.items()}
+        self.keep = []
+        self.fw, self.bw = [], []  # lists of (function name, struct, extra args)
+        spec = {n: (ci, co, k, s) for n, ci, co, k, s in convs}
+        L = lambda name: name.replace("DT", dt)
+
+        def conv(name, x, dx, H):
+            ci, co, k, s = spec[name]
+            Ho = (H + 2 * (k // 2) - k) // s + 1
+            y, dy = z(ns, co, Ho, Ho), z(ns, co, Ho, Ho)
+            p = k // 2
+            # strided layers: 32 + 2 - 3 is odd, which the reference's im2col route rejects; its naive-kernel route
+            # (USE_IM2COL = 0, lib/sources/pulp_conv_naive_fp32.c:520) takes any stride, and so does this library's
+            a, kp = hp.conv2d_args(pkg, x, dx, self.W[name], self.dW[name], y, dy, ci, H, H, co, k, k, Ho, Ho,
+                                   (p, p, p, p), (s, s), 0, 1 if s == 1 else 0)
+            self.keep.append(kp)
+            return a, y, dy, Ho
+
+        def relu(x, dx):
+            y, dy = z(*x.shape), z(*x.shape)
+            a, kp = hp.act_args(pkg, x, dx, y, dy, int(np.prod(x.shape[1:])))
+            self.keep.append(kp)
+            return a, y, dy
+
+        self.x, self.dx0 = z(ns, 3, 32, 32), None
+        a, t, dt_, H = conv("stem", self.x, None, 32)
+        self.fw.append((L("ptl_conv2d_DT_fw_batched"), a, (ns,)))
+        first_bw = [(L("ptl_conv2d_DT_wg_batched"), a, (ns,))]  # the stem needs no input gradient
+        ra, t, dt_ = relu(t, dt_)
+        self.fw.append((L("ptl_relu_DT_batched"), ra, (ns, 0)))
+        first_bw.insert(0, (L("ptl_relu_DT_batched"), ra, (ns, 1)))
+        bw_blocks = []
+        for (n, ci, co, stride, proj) in blocks:
+            xin, dxin, Hin = t, dt_, H
+            c1, y1, dy1, H = conv(n + "c1", xin, dxin, Hin)
+            r1, a1, da1 = relu(y1, dy1)
+            c2, y2, dy2, H = conv(n + "c2", a1, da1, H)
+            seq = [(L("ptl_conv2d_DT_fw_batched"), c1, (ns,)), (L("ptl_relu_DT_batched"), r1, (ns, 0)),
+                   (L("ptl_conv2d_DT_fw_batched"), c2, (ns,))]
+            if proj:
+                # the projection's input gradient must be ADDED to the main branch's: it gets its own buffer
+                dproj = z(*xin.shape)
+                cs, ys, dys, _ = conv(proj, xin, dproj, Hin)
+                seq.append((L("ptl_conv2d_DT_fw_batched"), cs, (ns,)))
+                skip, dskip = ys, dys
+            else:
+                skip, dskip = xin, dxin
+            s_, ds_ = z(*y2.shape), z(*y2.shape)
+            sk, kp = hp.skip_args(pkg, skip, dskip, y2, dy2, s_, ds_, int(np.prod(y2.shape[1:])))
+            self.keep.append(kp)
+            r2, t, dt_ = relu(s_, ds_)
+            seq += [(L("ptl_residual_DT_batched"), sk, (ns, 0)), (L("ptl_relu_DT_batched"), r2, (ns, 0))]
+            self.fw += seq
+            b = [(L("ptl_relu_DT_batched"), r2, (ns, 1)),            # ds = relu'(s) * dt
+                 (L("ptl_residual_DT_batched"), sk, (ns, 2)),         # dy2 = ds
+                 (L("ptl_conv2d_DT_wg_batched"), c2, (ns,)), (L("ptl_conv2d_DT_ig_batched"), c2, (ns,)),
+                 (L("ptl_relu_DT_batched"), r1, (ns, 1)),
+                 (L("ptl_conv2d_DT_wg_batched"), c1, (ns,)), (L("ptl_conv2d_DT_ig_batched"), c1, (ns,))]  # dxin = main
+            if proj:
+                add, kp = hp.skip_args(pkg, dxin, dxin, dproj, dproj, dproj, dproj, int(np.prod(xin.shape[1:])))
+                self.keep.append(kp)
+                # dys = ds (copy through a residual-backward call on a view of the projection output)
+                cp, kp2 = hp.skip_args(pkg, ys, dys, ys, dys, s_, ds_, int(np.prod(y2.shape[1:])))
+                self.keep.append(kp2)
+                b += [(L("ptl_residual_DT_batched"), cp, (ns, 2)),     # dys = ds
+                      (L("ptl_conv2d_DT_wg_batched"), cs, (ns,)), (L("ptl_conv2d_DT_ig_batched"), cs, (ns,)),
+                      self._vect_sum(dxin, dproj)]                     # dxin += dproj
+            else:
+                b.append((L("ptl_residual_DT_batched"), sk, (ns, 1)))  # dxin += ds (identity shortcut)
+            bw_blocks.append(b)
+        pooled, dpooled = z(ns, 64), z(ns, 64)
+        pa, kp = hp.pool_args(pkg, t, dt_, pooled, dpooled, 64, H, H, 1, 1, H, H, H, H)
+        self.keep.append(kp)
+        self.logits, dlogits = z(ns, ncls), z(ns, ncls)
+        la, kp = hp.linear_args(pkg, pooled, dpooled, self.W["fc"], self.dW["fc"], self.logits, dlogits, 64, ncls)
+        self.keep.append(kp)
+        self.target, self.loss = z(ns, ncls), z(ns)
+        ca, kp = hp.loss_args(pkg, self.logits, dlogits, self.target, self.loss, ncls)
+        self.keep.append(kp)
+        self.fw += [(L("ptl_avgpool_DT_batched"), pa, (ns, 0)), (L("ptl_linear_DT_fw_batched"), la, (ns,)),
+                    (L("ptl_cross_entropy_DT_batched"), ca, (ns, 0))]
+        self.bw = [(L("ptl_cross_entropy_DT_batched"), ca, (ns, 1)), (L("ptl_linear_DT_bw_batched"), la, (ns,)),
+                   (L("ptl_avgpool_DT_batched"), pa, (ns, 1))]
+        for b in reversed(bw_blocks):
+            self.bw += b
+        self.bw += first_bw
+        self.opt = []
+        for n in self.W:
+            o, kp = hp.optim_args(pkg, dt, self.W[n], self.dW[n], None, None, lr, 0.0)
+            self.keep.append(kp)
+            self.opt.append((L("ptl_gradient_descent_DT"), o, ()))
+
+    def _vect_sum(self, acc, term):
+        """acc += term through the reference-named vect_sum entry point (lib/sources/pulp_train_utils_fp32.c:208)."""
+        a = self.pkg.VectSumArgs()
+        a.op_1, a.op_2, a.dest, a.size = self.pkg.addr(acc), self.pkg.addr(term), self.pkg.addr(acc), acc.numel()
+        self.keep.append((acc, term))
+        return ("vect_sum" if self.dt == "fp32" else "vect_sum_fp16", a, None)
+
+    def _run(self, seq):
+        for name, a, extra in seq:
+            if extra is None:  # reference-named void entry point
+                getattr(self.lib, name)(ctypes.byref(a))
+                rc = self.lib.ptl_last_status()
+            else:
+                rc = getattr(self.lib, name)(ctypes.byref(a), *extra)
+            if rc != 0:
+                raise RuntimeError("%s failed: %s" % (name, self.lib.ptl_last_error().decode()))
+
+    def step(self, update=True):
+        self._run(self.fw)
+        self._run(self.bw)
+        if update:
+            self._run(self.opt)
+
+    def launches(self):
+        return len(self.fw) + len(self.bw) + len(self.opt)
