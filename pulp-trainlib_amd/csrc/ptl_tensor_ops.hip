@@ -391,39 +391,46 @@ __global__ __launch_bounds__(256) void dw_plane_kernel(const T *__restrict__ src
     }
 }
 
-// part[plane][i][j] = sum over the plane of X[r + i - pu][c + j - pl] * dY[r][c]
+// part[group][ch][i][j] = sum over the planes (b, ch) of the samples b of a group of
+// X[r + i - pu][c + j - pl] * dY[r][c].  A workgroup owns (channel, sample group), walks the group's planes with
+// per-thread sums in registers and reduces once at the end.
 template <typename T, int K>
 __global__ __launch_bounds__(256) void dw_wg_plane_kernel(const T *__restrict__ X, const T *__restrict__ dY,
-                                                          float *__restrict__ part, int H, int W, int Ho, int Wo,
-                                                          int pu, int pl, int x_vecs) {
+                                                          float *__restrict__ part, int C, int ns, int per_group,
+                                                          int H, int W, int Ho, int Wo, int pu, int pl, int x_vecs) {
     extern __shared__ uint4 dw_img[];
     __shared__ float red[4][K * K];
-    const size_t plane = blockIdx.x;
+    const int ch = blockIdx.x, grp = blockIdx.y;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    const T *ximg = dw_load_plane<T>(X + plane * H * W, H * W, dw_img, tid);
-    const T *gimg = dw_load_plane<T>(dY + plane * Ho * Wo, Ho * Wo, dw_img + x_vecs, tid);
-    __syncthreads();
     float acc[K][K];
 #pragma unroll
     for (int i = 0; i < K; ++i)
 #pragma unroll
         for (int j = 0; j < K; ++j) acc[i][j] = 0.f;
     const int groups = (Wo + 7) >> 3;
-    for (int item = tid; item < Ho * groups; item += 256) {
-        const int r = item / groups, c0 = (item - r * groups) * 8;
-        float gy[8];
+    const int b_end = min(ns, (grp + 1) * per_group);
+    for (int b = grp * per_group; b < b_end; ++b) {
+        const size_t plane = (size_t)b * C + ch;
+        __syncthreads();  // the previous plane has been consumed
+        const T *ximg = dw_load_plane<T>(X + plane * H * W, H * W, dw_img, tid);
+        const T *gimg = dw_load_plane<T>(dY + plane * Ho * Wo, Ho * Wo, dw_img + x_vecs, tid);
+        __syncthreads();
+        for (int item = tid; item < Ho * groups; item += 256) {
+            const int r = item / groups, c0 = (item - r * groups) * 8;
+            float gy[8];
 #pragma unroll
-        for (int q = 0; q < 8; ++q) gy[q] = c0 + q < Wo ? (float)gimg[r * Wo + c0 + q] : 0.f;
+            for (int q = 0; q < 8; ++q) gy[q] = c0 + q < Wo ? (float)gimg[r * Wo + c0 + q] : 0.f;
 #pragma unroll
-        for (int i = 0; i < K; ++i) {
-            const int h = r + i - pu;
-            if ((unsigned)h >= (unsigned)H) continue;
-            float v[8 + K - 1];
-            dw_plane_row<T, K>(ximg, h, W, c0, pl, v);
+            for (int i = 0; i < K; ++i) {
+                const int h = r + i - pu;
+                if ((unsigned)h >= (unsigned)H) continue;
+                float v[8 + K - 1];
+                dw_plane_row<T, K>(ximg, h, W, c0, pl, v);
 #pragma unroll
-            for (int j = 0; j < K; ++j)
+                for (int j = 0; j < K; ++j)
 #pragma unroll
-                for (int q = 0; q < 8; ++q) acc[i][j] += v[q + j] * gy[q];
+                    for (int q = 0; q < 8; ++q) acc[i][j] += v[q + j] * gy[q];
+            }
         }
     }
 #pragma unroll
@@ -436,7 +443,8 @@ __global__ __launch_bounds__(256) void dw_wg_plane_kernel(const T *__restrict__ 
             if (lane == 0) red[wave][i * K + j] = v;
         }
     __syncthreads();
-    if (tid < K * K) part[plane * K * K + tid] = (red[0][tid] + red[1][tid]) + (red[2][tid] + red[3][tid]);
+    if (tid < K * K)
+        part[((size_t)grp * C + ch) * K * K + tid] = (red[0][tid] + red[1][tid]) + (red[2][tid] + red[3][tid]);
 }
 
 template <typename Args>
@@ -548,23 +556,31 @@ static int dw_step(const Args *a, int ns, int step, int sh, int sw, const char *
         } else {
             hipLaunchKernelGGL((dw_ig_kernel<T>), dim3(nblocks(in_n)), dim3(256), 0, st.stream, dY, Wt, dX, g, in_n);
         }
-    } else if (plane_path && sizeof(T) == 2) {
+    } else if (plane_path) {
         const T *X = sg.in(reinterpret_cast<const T *>(a->input->data), in_n);
         const T *dY = sg.in(reinterpret_cast<const T *>(a->output->diff), out_n);
         T *dW = sg.out(reinterpret_cast<T *>(a->coeff->diff), w_n);
         if (sg.failed()) return 2;
         const int taps = g.Hk * g.Wk;
-        float *part = workspace((size_t)planes * taps * sizeof(float));
+        // sample groups: about four workgroups per CU
+        int sgroups = (int)((4L * st.num_cu + g.C - 1) / g.C);
+        if (sgroups > ns) sgroups = ns;
+        if (sgroups < 1) sgroups = 1;
+        const int per_group = (ns + sgroups - 1) / sgroups;
+        sgroups = (ns + per_group - 1) / per_group;
+        float *part = workspace((size_t)sgroups * g.C * taps * sizeof(float));
         if (!part) return sg.finish(2);
         const int x_vecs = (int)((in_img + 15) / 16);
         const size_t lds = (size_t)x_vecs * 16 + out_img;
+        dim3 grid(g.C, sgroups);
         if (g.Hk == 3)
-            hipLaunchKernelGGL((dw_wg_plane_kernel<T, 3>), dim3((unsigned)planes), dim3(256), lds, st.stream, X, dY, part,
-                               g.H, g.W, g.Ho, g.Wo, g.Up, g.Lp, x_vecs);
+            hipLaunchKernelGGL((dw_wg_plane_kernel<T, 3>), grid, dim3(256), lds, st.stream, X, dY, part, g.C, ns,
+                               per_group, g.H, g.W, g.Ho, g.Wo, g.Up, g.Lp, x_vecs);
         else
-            hipLaunchKernelGGL((dw_wg_plane_kernel<T, 5>), dim3((unsigned)planes), dim3(256), lds, st.stream, X, dY, part,
-                               g.H, g.W, g.Ho, g.Wo, g.Up, g.Lp, x_vecs);
-        hipLaunchKernelGGL((dw_wg_reduce_kernel2<T>), dim3(g.C), dim3(256), 0, st.stream, part, dW, ns, g.C, 1, taps);
+            hipLaunchKernelGGL((dw_wg_plane_kernel<T, 5>), grid, dim3(256), lds, st.stream, X, dY, part, g.C, ns,
+                               per_group, g.H, g.W, g.Ho, g.Wo, g.Up, g.Lp, x_vecs);
+        hipLaunchKernelGGL((dw_wg_reduce_kernel2<T>), dim3(g.C), dim3(256), 0, st.stream, part, dW, sgroups, g.C, 1,
+                           taps);
     } else if (rows_path) {
         const T *X = sg.in(reinterpret_cast<const T *>(a->input->data), in_n);
         const T *dY = sg.in(reinterpret_cast<const T *>(a->output->diff), out_n);
