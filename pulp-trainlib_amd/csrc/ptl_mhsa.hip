@@ -254,16 +254,16 @@ struct PanelArgs {
 };
 
 // Panel of rows [r0, r0+32) x k [k0, k0+PG_KC) of an operand with row stride s_r and k stride s_k.
-template <bool KMAJ>
+template <bool KMAJ, int NW>
 __device__ inline TileEdge panel_load(const float *g, int s_r, int s_k, int r0, int R, int k0, int K, float *lds,
                                       const float *zero, int tid, int wave, int lane) {
     if (KMAJ) {
         const float *t = g + (long long)r0 * s_r + k0;
-        tile_dma<4>(t, s_r, 32, PG_KC, R - r0, K - k0, lds, PG_P, zero, wave, lane);
+        tile_dma<NW>(t, s_r, 32, PG_KC, R - r0, K - k0, lds, PG_P, zero, wave, lane);
         return tile_edge_load(t, s_r, 32, PG_KC, R - r0, K - k0, lds, PG_P, tid);
     }
     const float *t = g + (long long)k0 * s_k + r0;
-    tile_dma<4>(t, s_k, PG_KC, 32, K - k0, R - r0, lds, 32, zero, wave, lane);
+    tile_dma<NW>(t, s_k, PG_KC, 32, K - k0, R - r0, lds, 32, zero, wave, lane);
     return tile_edge_load(t, s_k, PG_KC, 32, K - k0, R - r0, lds, 32, tid);
 }
 
@@ -286,13 +286,16 @@ __device__ inline void mfma4(mh_f32x16 &acc, const float4 &a, const float4 &b) {
     acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a.w, b.w, acc, 0, 0, 0);
 }
 
-template <bool A_KMAJ, bool B_KMAJ>
-__global__ __launch_bounds__(ATT_NT) void panel_gemm_kernel(PanelArgs a) {
+// NB row blocks of 32 per workgroup share one B panel; each block has its own four waves.
+template <bool A_KMAJ, bool B_KMAJ, int NB>
+__global__ __launch_bounds__(ATT_NT * NB) void panel_gemm_kernel(PanelArgs a) {
     extern __shared__ __attribute__((aligned(16))) float pg_lds[];
-    float *As = pg_lds, *Bs = pg_lds + PG_PANEL;
+    constexpr int NW = 4 * NB, NT = ATT_NT * NB;
+    float *Bs = pg_lds, *As = pg_lds + PG_PANEL;  // As: NB panels
     const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int l32 = lane & 31, half = lane >> 5;
-    const int m0 = blockIdx.x * 32, n0 = blockIdx.y * 32;
+    const int nb = wave >> 2, ks = wave & 3;
+    const int m0 = blockIdx.x * 32, n0 = blockIdx.y * (32 * NB);
     int o, b_first, b_count, grp = 0;
     if (a.sum_samples) {
         o = blockIdx.z / a.groups;
@@ -311,20 +314,32 @@ __global__ __launch_bounds__(ATT_NT) void panel_gemm_kernel(PanelArgs a) {
             const float *Bg = a.B[o * a.nterm + t] + (long long)(b_first + bi) * a.b_s;
             for (int k0 = 0; k0 < a.K; k0 += PG_KC) {
                 __syncthreads();  // the previous panels have been consumed
-                const TileEdge ea = panel_load<A_KMAJ>(Ag, a.a_n, a.a_k, n0, a.N, k0, a.K, As, a.zero, tid, wave, lane);
-                const TileEdge eb = panel_load<B_KMAJ>(Bg, a.b_m, a.b_k, m0, a.M, k0, a.K, Bs, a.zero, tid, wave, lane);
-                tile_edge_store(ea);
+                TileEdge ea[NB];
+#pragma unroll
+                for (int j = 0; j < NB; ++j) {
+                    ea[j].dst = nullptr;
+                    if (n0 + 32 * j < a.N)
+                        ea[j] = panel_load<A_KMAJ, NW>(Ag, a.a_n, a.a_k, n0 + 32 * j, a.N, k0, a.K, As + j * PG_PANEL,
+                                                       a.zero, tid, wave, lane);
+                }
+                const TileEdge eb = panel_load<B_KMAJ, NW>(Bg, a.b_m, a.b_k, m0, a.M, k0, a.K, Bs, a.zero, tid, wave,
+                                                           lane);
+#pragma unroll
+                for (int j = 0; j < NB; ++j) tile_edge_store(ea[j]);
                 tile_edge_store(eb);
                 wait_vmcnt<0>();
                 __syncthreads();
-                // groups of eight k (beyond the valid depth the panels hold zeros), dealt to the waves in runs;
-                // within a group the lower half-wave takes k 0..3 and the upper 4..7
-                const int ngroups = (min(PG_KC, a.K - k0) + 7) >> 3;
-                const int per = (ngroups + 3) >> 2;
-                const int g_end = min(ngroups, (wave + 1) * per);
-                for (int gq = wave * per; gq < g_end; ++gq) {
-                    const int k4 = gq * 8 + half * 4;
-                    mfma4(acc, panel_frag<A_KMAJ>(As, l32, k4), panel_frag<B_KMAJ>(Bs, l32, k4));
+                // groups of eight k (beyond the valid depth the panels hold zeros), dealt to the four waves of a
+                // row block in runs; within a group the lower half-wave takes k 0..3 and the upper 4..7
+                if (n0 + 32 * nb < a.N) {
+                    const float *Aw = As + nb * PG_PANEL;
+                    const int ngroups = (min(PG_KC, a.K - k0) + 7) >> 3;
+                    const int per = (ngroups + 3) >> 2;
+                    const int g_end = min(ngroups, (ks + 1) * per);
+                    for (int gq = ks * per; gq < g_end; ++gq) {
+                        const int k4 = gq * 8 + half * 4;
+                        mfma4(acc, panel_frag<A_KMAJ>(Aw, l32, k4), panel_frag<B_KMAJ>(Bs, l32, k4));
+                    }
                 }
             }
         }
@@ -338,10 +353,10 @@ __global__ __launch_bounds__(ATT_NT) void panel_gemm_kernel(PanelArgs a) {
                         : a.C[o] + (a.sum_samples ? 0 : (long long)b_first * a.c_s);
     const int c_n = partial ? a.M : a.c_n;
     const float *bias = partial ? nullptr : a.bias[o];
-    for (int idx = tid; idx < 1024; idx += ATT_NT) {
-        const int n = idx >> 5, m = idx & 31;
-        float v = ((red[n * ATT_RP + m] + red[(32 + n) * ATT_RP + m]) + red[(64 + n) * ATT_RP + m]) +
-                  red[(96 + n) * ATT_RP + m];
+    for (int idx = tid; idx < 1024 * NB; idx += NT) {
+        const int n = idx >> 5, m = idx & 31;  // n in [0, 32*NB)
+        const float *r = red + ((n >> 5) * 128 + (n & 31)) * ATT_RP + m;
+        float v = ((r[0] + r[32 * ATT_RP]) + r[64 * ATT_RP]) + r[96 * ATT_RP];
         if (n0 + n < a.N && m0 + m < a.M) {
             float *dst = Cb + (size_t)(n0 + n) * c_n + m0 + m;
             if (bias) v = v + bias[n0 + n];
@@ -965,15 +980,36 @@ static int launch_panel(PanelArgs &p, float *part) {
             if (!part) return 2;
         }
     }
-    void (*kern)(PanelArgs) = ak ? (bk ? panel_gemm_kernel<true, true> : panel_gemm_kernel<true, false>)
-                                 : (bk ? panel_gemm_kernel<false, true> : panel_gemm_kernel<false, false>);
-    const size_t lds = (size_t)2 * PG_PANEL * sizeof(float);  // 52 KB: three workgroups per CU
-    dim3 grid((p.M + 31) / 32, (p.N + 31) / 32, p.sum_samples ? p.nout * p.groups : p.nout * p.ns);
+    // Two row blocks per workgroup (the B panel is fetched once for both) when single blocks would already
+    // queue up behind each other on the CUs.
+    const size_t zdim = p.sum_samples ? (size_t)p.nout * p.groups : (size_t)p.nout * p.ns;
+    const size_t single = (size_t)((p.M + 31) / 32) * ((p.N + 31) / 32) * zdim;
+    const int nb = (p.N > 32 && single > (size_t)3 * st.num_cu) ? 2 : 1;
+    void (*kern)(PanelArgs);
+    if (nb == 2)
+        kern = ak ? (bk ? panel_gemm_kernel<true, true, 2> : panel_gemm_kernel<true, false, 2>)
+                  : (bk ? panel_gemm_kernel<false, true, 2> : panel_gemm_kernel<false, false, 2>);
+    else
+        kern = ak ? (bk ? panel_gemm_kernel<true, true, 1> : panel_gemm_kernel<true, false, 1>)
+                  : (bk ? panel_gemm_kernel<false, true, 1> : panel_gemm_kernel<false, false, 1>);
+    const size_t lds = (size_t)(1 + nb) * PG_PANEL * sizeof(float);  // 52 KB or 78 KB
+    if (nb == 2) {
+        static bool attr_set[4] = {false, false, false, false};
+        const int which = (ak ? 2 : 0) + (bk ? 1 : 0);
+        if (!attr_set[which]) {
+            if (!hip_ok(hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
+                                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds),
+                        "hipFuncSetAttribute"))
+                return 2;
+            attr_set[which] = true;
+        }
+    }
+    dim3 grid((p.M + 31) / 32, (p.N + 32 * nb - 1) / (32 * nb), (unsigned)zdim);
     if (grid.y > 65535u || grid.z > 65535u) {
         set_error("panel product: grid too large");
         return 1;
     }
-    hipLaunchKernelGGL(kern, grid, dim3(ATT_NT), lds, st.stream, p);
+    hipLaunchKernelGGL(kern, grid, dim3(ATT_NT * nb), lds, st.stream, p);
     if (!hip_ok(hipGetLastError(), "panel product launch")) return 2;
     if (p.groups > 1) {
         hipLaunchKernelGGL(panel_reduce_kernel, dim3((unsigned)(((size_t)p.N * p.M + 255) / 256), p.nout), dim3(256),
