@@ -10,6 +10,7 @@ namespace ptl {
 template <typename T>
 int gemm_async(GemmArgs &g) {
     State &st = state();
+    st.last_gemm_streamed = 0;
     const void *zero = st.zeros;
     if (!zero) return -1;
     constexpr int SK = 128 / (int)sizeof(T);  // k elements per slab (128 bytes per row)
@@ -61,6 +62,24 @@ int gemm_async(GemmArgs &g) {
         if (!g.ws) return 2;
     }
     if (plain_operand<T>(g.a, g.kchunk, g.K) && plain_operand<T>(g.b, g.kchunk, g.K)) {
+        // few rows, a shallow contraction and many columns: resident A panel, streamed column tiles
+        if (g.splits == 1 && g.taps <= 1 && g.K % SK == 0 && g.K <= 4 * SK && (g.N == 64 || g.N % 128 == 0) &&
+            g.N <= 256 && g.M % 64 == 0 && (long)(g.M / 64) * ((g.N + 127) / 128) >= 4L * st.num_cu) {
+            const int ks = g.K / SK;
+            int rc = -1;
+            if (g.N == 64)
+                rc = ks == 1   ? launch_stream<T, 64, 64, 1>(g, st.num_cu, st.stream)
+                     : ks == 2 ? launch_stream<T, 64, 64, 2>(g, st.num_cu, st.stream)
+                     : ks == 4 ? launch_stream<T, 64, 64, 4>(g, st.num_cu, st.stream)
+                               : -1;
+            else
+                rc = ks == 1   ? launch_stream<T, 128, 64, 1>(g, st.num_cu, st.stream)
+                     : ks == 2 ? launch_stream<T, 128, 64, 2>(g, st.num_cu, st.stream)
+                     : ks == 4 ? launch_stream<T, 128, 64, 4>(g, st.num_cu, st.stream)
+                               : -1;
+            if (rc == 0) st.last_gemm_streamed = 1;
+            if (rc != -1) return rc;
+        }
         switch (cfg) {
             case 0:
                 // one or two slabs deep (pointwise layers): four waves without a k split need half the

@@ -12,4 +12,10 @@ template int launch_plain_pair<float, 64, 64, 1024, 2, 2, 4, 3, 1>(GemmArgs &, G
 template int launch_plain<float, 64, 64, 1024, 2, 2, 4, 3, 2>(GemmArgs &, hipStream_t);
 template int launch_plain<float, 64, 32, 512, 2, 1, 4, 3, 1>(GemmArgs &, hipStream_t);
 template int launch_plain<float, 128, 128, 256, 2, 2, 1, 2, 1>(GemmArgs &, hipStream_t);
+template int launch_stream<float, 128, 64, 1>(GemmArgs &, int, hipStream_t);
+template int launch_stream<float, 128, 64, 2>(GemmArgs &, int, hipStream_t);
+template int launch_stream<float, 128, 64, 4>(GemmArgs &, int, hipStream_t);
+template int launch_stream<float, 64, 64, 1>(GemmArgs &, int, hipStream_t);
+template int launch_stream<float, 64, 64, 2>(GemmArgs &, int, hipStream_t);
+template int launch_stream<float, 64, 64, 4>(GemmArgs &, int, hipStream_t);
 }
