@@ -391,6 +391,93 @@ __global__ __launch_bounds__(256) void dw_plane_kernel(const T *__restrict__ src
     }
 }
 
+// fp16 planes whose rows can be read two elements at a time (even row length, even column offset, plane start
+// 4-byte aligned): a row segment comes from LDS as dwords = pairs of neighbours, and a filter row meets it as
+// two-element dot products with fp32 accumulation (v_dot2_f32_f16) plus one mixed-precision FMA for the odd tap -
+// about half the vector instructions of the element-wise form, which is what bounds these kernels.
+typedef _Float16 dw_h2 __attribute__((ext_vector_type(2)));
+
+// Dwords P[m] = elements (cf + 2m, cf + 2m + 1) of row h, m < NP; zero outside the row.
+template <int NP>
+__device__ inline void dw_row_pairs(const half_t *img, int h, int Ws, int cf, unsigned (&P)[NP]) {
+    const unsigned *row = reinterpret_cast<const unsigned *>(img + h * Ws + cf);
+    if (cf >= 0 && cf + 2 * NP <= Ws) {
+#pragma unroll
+        for (int m = 0; m < NP; ++m) P[m] = row[m];
+    } else {
+#pragma unroll
+        for (int m = 0; m < NP; ++m) P[m] = (unsigned)(cf + 2 * m) < (unsigned)Ws ? row[m] : 0u;
+    }
+}
+
+// acc[q] += sum_j w[j] * x[q + j] for q < 8, x = the elements of P.  we[m] = (w[2m], w[2m+1]),
+// wo[m] = (w[2m+1], w[2m+2]); wf = the taps in fp32.
+template <int K>
+__device__ inline void dw_row_taps(const unsigned (&P)[(8 + K) / 2], const dw_h2 (&we)[K / 2], const dw_h2 (&wo)[K / 2],
+                                   const float (&wf)[K], float (&acc)[8]) {
+#pragma unroll
+    for (int q = 0; q < 8; ++q) {
+        float a = acc[q];
+        if ((q & 1) == 0) {
+#pragma unroll
+            for (int m = 0; m < K / 2; ++m)
+                a = __builtin_amdgcn_fdot2(__builtin_bit_cast(dw_h2, P[q / 2 + m]), we[m], a, false);
+            if (K & 1) a = fmaf((float)__builtin_bit_cast(dw_h2, P[(q + K - 1) / 2]).x, wf[K - 1], a);
+        } else {
+            a = fmaf((float)__builtin_bit_cast(dw_h2, P[(q - 1) / 2]).y, wf[0], a);
+#pragma unroll
+            for (int m = 0; m < (K - 1) / 2; ++m)
+                a = __builtin_amdgcn_fdot2(__builtin_bit_cast(dw_h2, P[(q + 1) / 2 + m]), wo[m], a, false);
+            if (!(K & 1)) a = fmaf((float)__builtin_bit_cast(dw_h2, P[(q + K - 1) / 2]).x, wf[K - 1], a);
+        }
+        acc[q] = a;
+    }
+}
+
+template <int K, bool FLIP>
+__global__ __launch_bounds__(256) void dw_plane_pairs_kernel(const half_t *__restrict__ src,
+                                                             const half_t *__restrict__ Wt, half_t *__restrict__ dst,
+                                                             int C, int Hs, int Ws, int Hd, int Wd, int pu, int pl) {
+    extern __shared__ uint4 dw_img[];
+    const size_t plane = blockIdx.x;
+    const int ch = (int)(plane % C), tid = threadIdx.x;
+    const half_t *img = dw_load_plane<half_t>(src + plane * Hs * Ws, Hs * Ws, dw_img, tid);
+    dw_h2 we[K][K / 2], wo[K][K / 2];
+    float wf[K][K];
+#pragma unroll
+    for (int i = 0; i < K; ++i) {
+        half_t wr[K];
+#pragma unroll
+        for (int j = 0; j < K; ++j) {
+            wr[j] = Wt[(size_t)ch * K * K + (FLIP ? (K - 1 - i) * K + (K - 1 - j) : i * K + j)];
+            wf[i][j] = (float)wr[j];
+        }
+#pragma unroll
+        for (int m = 0; m < K / 2; ++m) {
+            we[i][m] = dw_h2{wr[2 * m], wr[2 * m + 1]};
+            wo[i][m] = dw_h2{wr[2 * m + 1], wr[(2 * m + 2 < K) ? 2 * m + 2 : K - 1]};
+        }
+    }
+    __syncthreads();
+    const int groups = (Wd + 7) >> 3;
+    half_t *dp = dst + plane * Hd * Wd;
+    for (int item = tid; item < Hd * groups; item += 256) {
+        const int r = item / groups, c0 = (item - r * groups) * 8;
+        float acc[8];
+#pragma unroll
+        for (int q = 0; q < 8; ++q) acc[q] = 0.f;
+#pragma unroll
+        for (int i = 0; i < K; ++i) {
+            const int h = r + i - pu;
+            if ((unsigned)h >= (unsigned)Hs) continue;
+            unsigned P[(8 + K) / 2];
+            dw_row_pairs<(8 + K) / 2>(img, h, Ws, c0 - pl, P);
+            dw_row_taps<K>(P, we[i], wo[i], wf[i], acc);
+        }
+        dw_store8<half_t>(dp + (size_t)r * Wd + c0, acc, min(8, Wd - c0));
+    }
+}
+
 // part[group][ch][i][j] = sum over the planes (b, ch) of the samples b of a group of
 // X[r + i - pu][c + j - pl] * dY[r][c].  A workgroup owns (channel, sample group), walks the group's planes with
 // per-thread sums in registers and reduces once at the end.
@@ -486,6 +573,23 @@ static int dw_geom(const Args *a, DwGeom &g, int sh, int sw, const char *fn) {
     return 0;
 }
 
+// Plane-resident depthwise product (forward, or input gradient with FLIP).
+template <typename T, int K, bool FLIP>
+static void launch_dw_plane(const T *src, const T *Wt, T *dst, int C, int Hs, int Ws, int Hd, int Wd, int pu, int pl,
+                            long planes, hipStream_t stream) {
+    const size_t src_img = (size_t)Hs * Ws * sizeof(T) + 32;
+    if constexpr (sizeof(T) == 2) {
+        // rows readable as pairs: see dw_plane_pairs_kernel
+        if (Ws % 2 == 0 && pl % 2 == 0 && reinterpret_cast<uintptr_t>(src) % 4 == 0) {
+            hipLaunchKernelGGL((dw_plane_pairs_kernel<K, FLIP>), dim3((unsigned)planes), dim3(256), src_img, stream, src,
+                               Wt, dst, C, Hs, Ws, Hd, Wd, pu, pl);
+            return;
+        }
+    }
+    hipLaunchKernelGGL((dw_plane_kernel<T, K, FLIP>), dim3((unsigned)planes), dim3(256), src_img, stream, src, Wt, dst,
+                       C, Hs, Ws, Hd, Wd, pu, pl);
+}
+
 template <typename T, typename Args>
 static int dw_step(const Args *a, int ns, int step, int sh, int sw, const char *fn) {
     DwGeom g;
@@ -513,11 +617,9 @@ static int dw_step(const Args *a, int ns, int step, int sh, int sw, const char *
         if (sg.failed()) return 2;
         if (plane_path) {
             if (g.Hk == 3)
-                hipLaunchKernelGGL((dw_plane_kernel<T, 3, false>), dim3((unsigned)planes), dim3(256), in_img, st.stream,
-                                   X, Wt, Y, g.C, g.H, g.W, g.Ho, g.Wo, g.Up, g.Lp);
+                launch_dw_plane<T, 3, false>(X, Wt, Y, g.C, g.H, g.W, g.Ho, g.Wo, g.Up, g.Lp, planes, st.stream);
             else
-                hipLaunchKernelGGL((dw_plane_kernel<T, 5, false>), dim3((unsigned)planes), dim3(256), in_img, st.stream,
-                                   X, Wt, Y, g.C, g.H, g.W, g.Ho, g.Wo, g.Up, g.Lp);
+                launch_dw_plane<T, 5, false>(X, Wt, Y, g.C, g.H, g.W, g.Ho, g.Wo, g.Up, g.Lp, planes, st.stream);
         } else if (rows_path) {
             int rbs = (g.Ho + DW_RB - 1) / DW_RB, ccs = (g.Wo + 63) / 64;
             long waves = planes * rbs * ccs;
@@ -538,11 +640,11 @@ static int dw_step(const Args *a, int ns, int step, int sh, int sw, const char *
         if (sg.failed()) return 2;
         if (plane_path) {
             if (g.Hk == 3)
-                hipLaunchKernelGGL((dw_plane_kernel<T, 3, true>), dim3((unsigned)planes), dim3(256), out_img, st.stream,
-                                   dY, Wt, dX, g.C, g.Ho, g.Wo, g.H, g.W, g.Hk - 1 - g.Up, g.Wk - 1 - g.Lp);
+                launch_dw_plane<T, 3, true>(dY, Wt, dX, g.C, g.Ho, g.Wo, g.H, g.W, g.Hk - 1 - g.Up, g.Wk - 1 - g.Lp,
+                                            planes, st.stream);
             else
-                hipLaunchKernelGGL((dw_plane_kernel<T, 5, true>), dim3((unsigned)planes), dim3(256), out_img, st.stream,
-                                   dY, Wt, dX, g.C, g.Ho, g.Wo, g.H, g.W, g.Hk - 1 - g.Up, g.Wk - 1 - g.Lp);
+                launch_dw_plane<T, 5, true>(dY, Wt, dX, g.C, g.Ho, g.Wo, g.H, g.W, g.Hk - 1 - g.Up, g.Wk - 1 - g.Lp,
+                                            planes, st.stream);
         } else if (rows_path) {
             int rbs = (g.H + DW_RB - 1) / DW_RB, ccs = (g.W + 63) / 64;
             long waves = planes * rbs * ccs;

@@ -405,6 +405,16 @@ def test_depthwise(pkg, orc, gpu, dt, C, H, W, K, pad, ns):
     dw_parity(pkg, orc, gpu, dt, C, H, W, K, pad, (1, 1), ns, 0xC0DE0103)
 
 
+# Batches with at least two planes per CU run the plane-resident kernels: even and odd row lengths (fp16 rows of
+# even length are read as pairs of neighbours), 3x3 and 5x5, and padded fp32 planes.
+@pytest.mark.parametrize("dt,C,H,W,K,pad,ns", [("fp16", 64, 36, 36, 3, (0, 0, 0, 0), 8), ("fp16", 64, 35, 37, 3, (0, 0, 0, 0), 8),
+                                               ("fp16", 32, 38, 40, 5, (0, 0, 0, 0), 16), ("fp16", 32, 37, 39, 5, (0, 0, 0, 0), 16),
+                                               ("fp32", 64, 36, 36, 3, (0, 0, 0, 0), 8), ("fp32", 64, 35, 37, 3, (1, 1, 1, 1), 8),
+                                               ("fp32", 32, 38, 38, 5, (2, 2, 2, 2), 16)])
+def test_depthwise_plane_resident(pkg, orc, gpu, dt, C, H, W, K, pad, ns):
+    dw_parity(pkg, orc, gpu, dt, C, H, W, K, pad, (1, 1), ns, 0xC0DE0105)
+
+
 def test_depthwise_fp32_stride_and_padding(pkg, orc, gpu):
     dw_parity(pkg, orc, gpu, "fp32", 6, 11, 11, 3, (1, 1, 1, 1), (2, 2), 2, 0xC0DE0104)
 
