@@ -534,6 +534,76 @@ __global__ __launch_bounds__(256) void dw_wg_plane_kernel(const T *__restrict__ 
         part[((size_t)grp * C + ch) * K * K + tid] = (red[0][tid] + red[1][tid]) + (red[2][tid] + red[3][tid]);
 }
 
+// The weight-gradient kernel above for fp16 planes readable as pairs (even row lengths, even left pad, 4-byte
+// aligned tensors): the eight output-gradient values of an item are four pairs G, a source row segment is the
+// pairs P (and, for the odd taps, the pairs U that start one element later, made with one funnel shift each), and
+// tap (i, j) gathers four two-element dot products per item and row.
+template <int K>
+__global__ __launch_bounds__(256) void dw_wg_plane_pairs_kernel(const half_t *__restrict__ X,
+                                                                const half_t *__restrict__ dY,
+                                                                float *__restrict__ part, int C, int ns, int per_group,
+                                                                int H, int W, int Ho, int Wo, int pu, int pl,
+                                                                int x_vecs) {
+    constexpr int NP = (8 + K) / 2;
+    extern __shared__ uint4 dw_img[];
+    __shared__ float red[4][K * K];
+    const int ch = blockIdx.x, grp = blockIdx.y;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    float acc[K][K];
+#pragma unroll
+    for (int i = 0; i < K; ++i)
+#pragma unroll
+        for (int j = 0; j < K; ++j) acc[i][j] = 0.f;
+    const int groups = (Wo + 7) >> 3;
+    const int b_end = min(ns, (grp + 1) * per_group);
+    for (int b = grp * per_group; b < b_end; ++b) {
+        const size_t plane = (size_t)b * C + ch;
+        __syncthreads();  // the previous plane has been consumed
+        const half_t *ximg = dw_load_plane<half_t>(X + plane * H * W, H * W, dw_img, tid);
+        const half_t *gimg = dw_load_plane<half_t>(dY + plane * Ho * Wo, Ho * Wo, dw_img + x_vecs, tid);
+        __syncthreads();
+        for (int item = tid; item < Ho * groups; item += 256) {
+            const int r = item / groups, c0 = (item - r * groups) * 8;
+            dw_h2 G[4];
+            {
+                const unsigned *grow = reinterpret_cast<const unsigned *>(gimg + r * Wo + c0);
+#pragma unroll
+                for (int m = 0; m < 4; ++m) G[m] = __builtin_bit_cast(dw_h2, c0 + 2 * m < Wo ? grow[m] : 0u);
+            }
+#pragma unroll
+            for (int i = 0; i < K; ++i) {
+                const int h = r + i - pu;
+                if ((unsigned)h >= (unsigned)H) continue;
+                unsigned P[NP];
+                dw_row_pairs<NP>(ximg, h, W, c0 - pl, P);
+#pragma unroll
+                for (int j = 0; j < K; ++j) {
+                    float a = acc[i][j];
+#pragma unroll
+                    for (int m = 0; m < 4; ++m) {
+                        const unsigned x2 = (j & 1) ? __builtin_amdgcn_alignbit(P[m + j / 2 + 1], P[m + j / 2], 16)
+                                                    : P[m + j / 2];
+                        a = __builtin_amdgcn_fdot2(__builtin_bit_cast(dw_h2, x2), G[m], a, false);
+                    }
+                    acc[i][j] = a;
+                }
+            }
+        }
+    }
+#pragma unroll
+    for (int i = 0; i < K; ++i)
+#pragma unroll
+        for (int j = 0; j < K; ++j) {
+            float v = acc[i][j];
+#pragma unroll
+            for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
+            if (lane == 0) red[wave][i * K + j] = v;
+        }
+    __syncthreads();
+    if (tid < K * K)
+        part[((size_t)grp * C + ch) * K * K + tid] = (red[0][tid] + red[1][tid]) + (red[2][tid] + red[3][tid]);
+}
+
 template <typename Args>
 static int dw_geom(const Args *a, DwGeom &g, int sh, int sw, const char *fn) {
     if (!a || !a->input || !a->coeff || !a->output) {
@@ -675,7 +745,21 @@ static int dw_step(const Args *a, int ns, int step, int sh, int sw, const char *
         const int x_vecs = (int)((in_img + 15) / 16);
         const size_t lds = (size_t)x_vecs * 16 + out_img;
         dim3 grid(g.C, sgroups);
-        if (g.Hk == 3)
+        bool pairs = false;
+        if constexpr (sizeof(T) == 2) {
+            pairs = g.W % 2 == 0 && g.Wo % 2 == 0 && g.Lp % 2 == 0 && reinterpret_cast<uintptr_t>(X) % 4 == 0 &&
+                    reinterpret_cast<uintptr_t>(dY) % 4 == 0;
+            if (pairs) {
+                if (g.Hk == 3)
+                    hipLaunchKernelGGL((dw_wg_plane_pairs_kernel<3>), grid, dim3(256), lds, st.stream, X, dY, part, g.C,
+                                       ns, per_group, g.H, g.W, g.Ho, g.Wo, g.Up, g.Lp, x_vecs);
+                else
+                    hipLaunchKernelGGL((dw_wg_plane_pairs_kernel<5>), grid, dim3(256), lds, st.stream, X, dY, part, g.C,
+                                       ns, per_group, g.H, g.W, g.Ho, g.Wo, g.Up, g.Lp, x_vecs);
+            }
+        }
+        if (pairs) {
+        } else if (g.Hk == 3)
             hipLaunchKernelGGL((dw_wg_plane_kernel<T, 3>), grid, dim3(256), lds, st.stream, X, dY, part, g.C, ns,
                                per_group, g.H, g.W, g.Ho, g.Wo, g.Up, g.Lp, x_vecs);
         else
