@@ -67,6 +67,10 @@ struct GemmArgs {
     // Convolution as a sum over filter taps (look-up-free kernel only): k runs over (tap, channel); after the
     // `slabs_per_tap` slabs of a tap the A pointer jumps to the next tap of the padded, channel-blocked input:
     // by tap_jump_x bytes within a filter row, by tap_jump_y at the end of one.  taps <= 1: an ordinary product.
+    // Lean kernel, k in runs: after every seg_slabs slabs the slab pointers of A / B jump by these bytes (k
+    // made of an outer digit and a contiguous inner one, e.g. (sample, pixel)); 0 = k is one run.
+    int seg_slabs;
+    long long a_seg_jump, b_seg_jump;
     int taps, slabs_per_tap, tap_kw;
     long long tap_jump_x, tap_jump_y;
     // Weight gradient over taps: grid.y enumerates (tap, k split), tap_splits splits per tap; tap (ky, kx) reads

@@ -14,6 +14,30 @@ int gemm_async(GemmArgs &g) {
     const void *zero = st.zeros;
     if (!zero) return -1;
     constexpr int SK = 128 / (int)sizeof(T);  // k elements per slab (128 bytes per row)
+    // k = (outer, inner) with the inner digit contiguous in both operands and a whole number of slabs long
+    // (the weight gradient of a pointwise layer over a batch: k = (sample, pixel)): the lean kernel walks it as
+    // one flat axis whose slab pointers jump at the end of every inner run.
+    bool runs = false;
+    {
+        auto two_digit = [](const AxisMap &k) {
+            return k.d0 < k.n && k.d1 >= (1 << 30) && k.o0 == 1 && k.o1 >= k.d0 && k.ob >= 0 && k.h1 == 0 && k.h0 == 0 &&
+                   k.hb == 0 && k.w1 == 0 && k.w0 == 0 && k.wb == 0;
+        };
+        const AxisMap &ka = g.a.k, &kb = g.b.k;
+        if (g.taps <= 1 && g.a.mode == FILL_VEC_K && g.b.mode == FILL_VEC_K && two_digit(ka) && two_digit(kb) &&
+            ka.d0 == kb.d0 && ka.d0 % SK == 0 && g.K % SK == 0) {
+            GemmArgs flat = g;
+            flat.a.k = axis_plain(g.K, 1, ka.ob);
+            flat.b.k = axis_plain(g.K, 1, kb.ob);
+            flat.seg_slabs = ka.d0 / SK;
+            flat.a_seg_jump = ((long long)ka.o1 - ka.d0) * (long long)sizeof(T);
+            flat.b_seg_jump = ((long long)kb.o1 - kb.d0) * (long long)sizeof(T);
+            if (plain_operand<T>(flat.a, SK, g.K) && plain_operand<T>(flat.b, SK, g.K)) {
+                g = flat;
+                runs = true;
+            }
+        }
+    }
     auto tiles = [&](int bm, int bn) { return (long)((g.N + bm - 1) / bm) * ((g.M + bn - 1) / bn); };
     int cfg;
     if (g.N <= 32)
@@ -27,11 +51,17 @@ int gemm_async(GemmArgs &g) {
     else
         cfg = 1;
     long nt = cfg == 0 ? tiles(128, 128) : cfg == 1 ? tiles(64, 64) : cfg == 2 ? tiles(32, 128) : tiles(128, 32);
+    // k in runs with 128 rows or more and at most 64 columns: a 128x64 tile reads the narrow operand once
+    const bool tall = runs && cfg == 1 && g.N % 128 == 0 && g.M > 32;
+    if (tall) nt = tiles(128, 64);
 
     g.splits = 1;
     g.kchunk = ((g.K + SK - 1) / SK) * SK;
     int want = 1;
     if (nt * 4 <= st.num_cu) want = (int)((st.num_cu + nt - 1) / nt);
+    // a long stream of k is bound by memory, not by the number of workgroups: half as many splits stream
+    // as fast and leave half as many partial sums to add
+    if (runs && want > 1) want = (want + 1) / 2;
     // Operands that are not on the look-up-free path index k through a table of ASYNC_KWMAX entries.
     const bool need_lut = !(plain_operand<T>(g.a, g.kchunk, g.K) && plain_operand<T>(g.b, g.kchunk, g.K));
     int need = need_lut ? (g.K + ASYNC_KWMAX - 1) / ASYNC_KWMAX : 1;
@@ -93,6 +123,7 @@ int gemm_async(GemmArgs &g) {
                     if (g.splits == 1 && tiles(64, 64) * 2 <= st.num_cu && g.M % 32 == 0)
                         return launch_plain<T, 64, 32, 512, 2, 1, 4, 3, 1>(g, st.stream);
                 }
+                if (tall) return launch_plain<T, 128, 64, 512, 2, 2, 2, 3, 1>(g, st.stream);
                 // small tile: two slabs per wait-and-barrier when the slab count is even
                 if (g.splits == 1 && (g.K / SK) % 2 == 0 && g.K >= 4 * SK) return launch_plain<T, 64, 64, 1024, 2, 2, 4, 3, 2>(g, st.stream);
                 return launch_plain<T, 64, 64, 1024, 2, 2, 4, 3, 1>(g, st.stream);

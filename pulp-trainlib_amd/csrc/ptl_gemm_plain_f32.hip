@@ -18,4 +18,5 @@ template int launch_stream<float, 128, 64, 4>(GemmArgs &, int, hipStream_t);
 template int launch_stream<float, 64, 64, 1>(GemmArgs &, int, hipStream_t);
 template int launch_stream<float, 64, 64, 2>(GemmArgs &, int, hipStream_t);
 template int launch_stream<float, 64, 64, 4>(GemmArgs &, int, hipStream_t);
+template int launch_plain<float, 128, 64, 512, 2, 2, 2, 3, 1>(GemmArgs &, hipStream_t);
 }
