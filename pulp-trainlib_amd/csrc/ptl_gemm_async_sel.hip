@@ -115,6 +115,12 @@ int gemm_async(GemmArgs &g) {
                 // one or two slabs deep (pointwise layers): four waves without a k split need half the
                 // LDS for the parked tile, so two workgroups share a CU and overlap load, MFMA and store
                 if (g.splits == 1 && g.K <= 2 * SK) return launch_plain<T, 128, 128, 256, 2, 2, 1, 2, 1>(g, st.stream);
+                // fp16 products large enough to give every CU a 256x128 tile: a third less L2 -> LDS traffic per
+                // MFMA than 128x128, which is what bounds that tile (+15-20 % measured from 4096^3 up)
+                if constexpr (sizeof(T) == 2) {
+                    if (g.splits == 1 && tiles(256, 128) >= st.num_cu)
+                        return launch_plain<T, 256, 128, 512, 4, 2, 1, 3, 1>(g, st.stream);
+                }
                 return launch_plain<T, 128, 128, 512, 2, 2, 2, 3, 1>(g, st.stream);
             case 1:
                 // fp32 MFMAs are slow enough to matter at this size: when 64x64 tiles leave half the CUs

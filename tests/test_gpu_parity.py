@@ -527,6 +527,21 @@ def test_mm_family(pkg, orc, gpu, dt, N, M, K):
             assert rel_l2(host(gC), C) <= TOL[dt]
 
 
+@pytest.mark.parametrize("N,M,K", [(4096, 2048, 256), (4000, 2040, 192)])
+def test_mm_fp16_large_tile(pkg, gpu, N, M, K):
+    """fp16 products that give every CU a 256x128 tile, whole and ragged, against torch in float32."""
+    g = torch.Generator(device="cpu").manual_seed(17)
+    A = (torch.randn(N, K, generator=g) / 8).half().to(DEV)
+    for tb in (0, 1):
+        B = (torch.randn((M, K) if tb else (K, M), generator=g) / 8).half().to(DEV)
+        C = torch.full((N, M), 3, dtype=torch.float16, device=DEV)
+        pkg.call("mm_fp16", hp.mm_args(pkg, A, B, C, N, M, K, tb))
+        sync(gpu)
+        ref = A.float() @ (B.float().t() if tb else B.float())
+        assert float((C.float() - ref).norm() / ref.norm()) <= 1e-3
+        assert float((C.float() - ref).abs().max()) <= 2e-2
+
+
 def test_mm_k0_leaves_output_untouched(pkg, gpu):
     gA, gB, gC = dev(np.zeros((3, 1), np.float32)), dev(np.zeros((1, 4), np.float32)), dev(np.full((3, 4), 5, np.float32))
     pkg.call("mm", hp.mm_args(pkg, gA, gB, gC, 3, 4, 0, 0))
