@@ -527,9 +527,10 @@ def test_mm_family(pkg, orc, gpu, dt, N, M, K):
             assert rel_l2(host(gC), C) <= TOL[dt]
 
 
-@pytest.mark.parametrize("N,M,K", [(4096, 2048, 256), (4000, 2040, 192)])
-def test_mm_fp16_large_tile(pkg, gpu, N, M, K):
-    """fp16 products that give every CU a 256x128 tile, whole and ragged, against torch in float32."""
+@pytest.mark.parametrize("N,M,K", [(4096, 2048, 256), (4000, 2040, 192), (66000, 64, 128), (65536, 48, 192)])
+def test_mm_fp16_large_and_tall_tiles(pkg, gpu, N, M, K):
+    """fp16 products that give every CU a 256x128 tile, and narrow ones on the 128x64 tile; whole and ragged,
+    against torch in float32."""
     g = torch.Generator(device="cpu").manual_seed(17)
     A = (torch.randn(N, K, generator=g) / 8).half().to(DEV)
     for tb in (0, 1):
