@@ -299,6 +299,14 @@ int ptl_cross_entropy_fp16_batched(const struct loss_args_fp16 *a, int nsamples,
 int ptl_gradient_descent_fp32(const struct optim_args *a);
 int ptl_gradient_descent_fp16(const struct optim_args_fp16 *a);
 int ptl_batch_norm_fp32_fw(const struct BatchNorm_args_fp32 *a);
+/* No counterpart in the reference (its batch normalisation has a forward pass only, in fp32): the backward pass
+ * of that forward and both passes in fp16, for a training step that contains the layer.  Backward reads
+ * input->data, output->diff, weight_data and eps, writes input->diff (unless skip_in_grad) and, unless
+ * skip_wg_grad, the C gradients of the scale into coeff->diff and of the shift into bias->diff (either blob
+ * may be NULL). */
+int ptl_batch_norm_fp32_bw(const struct BatchNorm_args_fp32 *a);
+int ptl_batch_norm_fp16_fw(const struct BatchNorm_args_fp16 *a);
+int ptl_batch_norm_fp16_bw(const struct BatchNorm_args_fp16 *a);
 
 /* Plain product C[N x M] = A[N x K] * B (B is K x M, or M x K when trans_B),
  * the contract of the reference's mm family, on raw pointers. */

@@ -634,6 +634,29 @@ struct BatchNorm_args_fp32 {
     int W;
 };
 
+/* The same in fp16 (no counterpart in the reference, which normalises in fp32 only): tensors, affine
+ * parameters and eps in fp16, statistics in fp32. */
+struct BatchNorm_args_fp16 {
+    struct blob_fp16 *input;
+    struct blob_fp16 *output;
+    struct blob_fp16 *coeff;
+    struct blob_fp16 *bias;
+    int batch_size;
+    float *running_mean;
+    float *running_var;
+    float *running_stdev;
+    int freeze_running_params;
+    int skip_wg_grad;
+    int skip_in_grad;
+    fp16 *weight_data;
+    fp16 *bias_data;
+    fp16 *eps;
+    int B;
+    int C;
+    int H;
+    int W;
+};
+
 #ifdef __cplusplus
 }
 #endif

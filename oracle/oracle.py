@@ -58,8 +58,9 @@ def load():
         f = getattr(lib, "orc_gradient_descent_%s" % dt)
         f.argtypes = [ctypes.c_void_p]
         f.restype = None
-    lib.orc_batch_norm_fw_fp32.argtypes = [ctypes.c_void_p]
-    lib.orc_batch_norm_fw_fp32.restype = None
+    for name in ("orc_batch_norm_fw_fp32", "orc_batch_norm_bw_fp32", "orc_batch_norm_fw_fp16", "orc_batch_norm_bw_fp16"):
+        getattr(lib, name).argtypes = [ctypes.c_void_p]
+        getattr(lib, name).restype = None
     lib.orc_num_threads.restype = ctypes.c_int
     lib.orc_set_num_threads.argtypes = [ctypes.c_int]
     _lib = lib

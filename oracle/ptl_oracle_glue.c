@@ -113,24 +113,66 @@ GLUE(float, fp32, struct blob, struct act_args, struct SkipConn_args, struct poo
 GLUE(_Float16, fp16, struct blob_fp16, struct act_args_fp16, struct SkipConn_args_fp16, struct pool_args_fp16,
      struct loss_args_fp16, struct optim_args_fp16)
 
-void orc_batch_norm_fw_fp32(const struct BatchNorm_args_fp32 *a) {
-    const float *in = a->input->data;
-    float *out = a->output->data;
-    const int B = a->B, C = a->C, HW = a->H * a->W, n = B * HW;
-    for (int c = 0; c < C; ++c) {
-        float s1 = 0.0f, s2 = 0.0f;
-        for (int b = 0; b < B; ++b)
-            for (int hw = 0; hw < HW; ++hw) {
-                const int idx = b * C * HW + c * HW + hw;
-                s1 += in[idx];
-                s2 += in[idx] * in[idx];
-            }
-        const float mean = s1 / n;
-        const float sd = sqrt(((s2 - 2 * s1 * mean) / n) + (mean * mean) + a->eps[0]);
-        for (int b = 0; b < B; ++b)
-            for (int hw = 0; hw < HW; ++hw) {
-                const int idx = b * C * HW + c * HW + hw;
-                out[idx] = ((in[idx] - mean) / sd) * a->weight_data[c] + a->bias_data[c];
-            }
+/* Batch normalisation.  Forward: lib/sources/pulp_batchnorm_fp32.c:34-114 (sums of x and x^2 per channel over
+ * B x H x W, deviation = sqrt((s2 - 2 s1 mean) / n + mean^2 + eps)).  The reference has no backward pass and no
+ * fp16 variant; those restate the textbook gradient of that forward,
+ *   xh = (x - mean) / sd, dbeta = sum dy, dgamma = sum dy xh, dx = gamma / sd (dy - dbeta / n - xh dgamma / n),
+ * with fp32 sums, and are pinned against torch autograd in float64 by tests/test_oracle_glue.py. */
+#define BATCH_NORM(T, SFX, ARGS)                                                                          \
+    static void bn_stats_##SFX(const ARGS *a, int c, float *mean, float *sd) {                            \
+        const T *in = a->input->data;                                                                     \
+        const int B = a->B, C = a->C, HW = a->H * a->W, n = B * HW;                                        \
+        float s1 = 0.0f, s2 = 0.0f;                                                                       \
+        for (int b = 0; b < B; ++b)                                                                       \
+            for (int hw = 0; hw < HW; ++hw) {                                                             \
+                const float v = (float)in[b * C * HW + c * HW + hw];                                      \
+                s1 += v;                                                                                  \
+                s2 += v * v;                                                                              \
+            }                                                                                             \
+        *mean = s1 / n;                                                                                   \
+        *sd = sqrtf(((s2 - 2 * s1 * *mean) / n) + (*mean * *mean) + (float)a->eps[0]);                    \
+    }                                                                                                     \
+    void orc_batch_norm_fw_##SFX(const ARGS *a) {                                                         \
+        const T *in = a->input->data;                                                                     \
+        T *out = a->output->data;                                                                         \
+        const int B = a->B, C = a->C, HW = a->H * a->W;                                                    \
+        for (int c = 0; c < C; ++c) {                                                                     \
+            float mean, sd;                                                                               \
+            bn_stats_##SFX(a, c, &mean, &sd);                                                             \
+            for (int b = 0; b < B; ++b)                                                                   \
+                for (int hw = 0; hw < HW; ++hw) {                                                         \
+                    const int idx = b * C * HW + c * HW + hw;                                             \
+                    out[idx] = (T)((((float)in[idx] - mean) / sd) * (float)a->weight_data[c] +            \
+                                   (float)a->bias_data[c]);                                               \
+                }                                                                                         \
+        }                                                                                                 \
+    }                                                                                                     \
+    void orc_batch_norm_bw_##SFX(const ARGS *a) {                                                         \
+        const T *in = a->input->data, *dy = a->output->diff;                                              \
+        const int B = a->B, C = a->C, HW = a->H * a->W, n = B * HW;                                        \
+        for (int c = 0; c < C; ++c) {                                                                     \
+            float mean, sd, db = 0.0f, dg = 0.0f;                                                         \
+            bn_stats_##SFX(a, c, &mean, &sd);                                                             \
+            for (int b = 0; b < B; ++b)                                                                   \
+                for (int hw = 0; hw < HW; ++hw) {                                                         \
+                    const int idx = b * C * HW + c * HW + hw;                                             \
+                    db += (float)dy[idx];                                                                 \
+                    dg += (float)dy[idx] * (((float)in[idx] - mean) / sd);                                \
+                }                                                                                         \
+            if (!a->skip_wg_grad) {                                                                       \
+                if (a->coeff) a->coeff->diff[c] = (T)dg;                                                  \
+                if (a->bias) a->bias->diff[c] = (T)db;                                                    \
+            }                                                                                             \
+            if (a->skip_in_grad) continue;                                                                \
+            for (int b = 0; b < B; ++b)                                                                   \
+                for (int hw = 0; hw < HW; ++hw) {                                                         \
+                    const int idx = b * C * HW + c * HW + hw;                                             \
+                    const float xh = ((float)in[idx] - mean) / sd;                                        \
+                    a->input->diff[idx] =                                                                 \
+                        (T)(((float)a->weight_data[c] / sd) * ((float)dy[idx] - db / n - xh * dg / n));   \
+                }                                                                                         \
+        }                                                                                                 \
     }
-}
+
+BATCH_NORM(float, fp32, struct BatchNorm_args_fp32)
+BATCH_NORM(_Float16, fp16, struct BatchNorm_args_fp16)

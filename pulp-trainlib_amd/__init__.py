@@ -59,7 +59,8 @@ VOID_ENTRY_POINTS = [
 STEP_ENTRY_POINTS = ["ptl_%s_%s_batched" % (n, dt) for n in ("relu", "residual", "avgpool", "cross_entropy")
                      for dt in ("fp32", "fp16")]
 # `int f(const args *)`
-PLAIN_ENTRY_POINTS = ["ptl_gradient_descent_fp32", "ptl_gradient_descent_fp16", "ptl_batch_norm_fp32_fw"]
+PLAIN_ENTRY_POINTS = ["ptl_gradient_descent_fp32", "ptl_gradient_descent_fp16", "ptl_batch_norm_fp32_fw",
+                      "ptl_batch_norm_fp32_bw", "ptl_batch_norm_fp16_fw", "ptl_batch_norm_fp16_bw"]
 
 # `int f(const args *, int nsamples)` batched launchers.
 BATCHED_ENTRY_POINTS = ["ptl_%s_%s_%s_batched" % (layer, dt, step)

@@ -283,60 +283,126 @@ static int sgd_step(const Args *a, const char *fn) {
     return sg.finish(0);
 }
 
-// ---- Batch normalisation forward (lib/sources/pulp_batchnorm_fp32.c:34-114) ---------------------------
-// One workgroup per channel: sums of x and x^2 over B x H x W, then the affine map.
-__global__ __launch_bounds__(256) void batch_norm_fw_kernel(const float *__restrict__ x, float *__restrict__ y,
-                                                            const float *__restrict__ weight,
-                                                            const float *__restrict__ bias, const float *eps, int B,
-                                                            int C, int HW) {
-    __shared__ float red[2][4];
-    const int c = blockIdx.x, tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    const size_t n = (size_t)B * HW;
-    float s1 = 0.f, s2 = 0.f;
-    for (size_t e = tid; e < n; e += 256) {
-        const size_t b = e / HW, hw = e - b * HW;
-        const float v = x[(b * C + c) * HW + hw];
-        s1 += v;
-        s2 += v * v;
+// ---- Batch normalisation (forward: lib/sources/pulp_batchnorm_fp32.c:34-114) ---------------------------
+// Statistics per channel over B x H x W, in two launches so that a few channels still fill the chip:
+//   1. partial sums per (channel, group of samples): forward x and x^2; backward also dy and dy*x;
+//   2. every workgroup of the second kernel owns one (sample, channel) plane, adds the channel's partials in a
+//      fixed order, forms mean and deviation the way the reference does and maps its plane.
+// The backward pass (the reference has none; the usual one for the forward above):
+//   xh = (x - mean) / sd,  dbeta = sum dy,  dgamma = sum dy * xh = (sum dy*x - mean * sum dy) / sd,
+//   dx = gamma / sd * (dy - dbeta / n - xh * dgamma / n).
+constexpr int BN_SUMS = 4;
+
+template <typename T, bool BW>
+__global__ __launch_bounds__(256) void bn_sums_kernel(const T *__restrict__ x, const T *__restrict__ dy,
+                                                      float *__restrict__ part, int B, int C, int HW, int per_group) {
+    __shared__ float red[BN_SUMS][4];
+    const int c = blockIdx.x, grp = blockIdx.y, tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int b0 = grp * per_group, b1 = min(B, b0 + per_group);
+    float s[BN_SUMS] = {0.f, 0.f, 0.f, 0.f};
+    for (int b = b0; b < b1; ++b) {
+        const size_t base = ((size_t)b * C + c) * HW;
+        for (int e = tid; e < HW; e += 256) {
+            const float v = (float)x[base + e];
+            s[0] += v;
+            s[1] += v * v;
+            if (BW) {
+                const float g = (float)dy[base + e];
+                s[2] += g;
+                s[3] += g * v;
+            }
+        }
     }
 #pragma unroll
-    for (int off = 32; off > 0; off >>= 1) {
-        s1 += __shfl_xor(s1, off);
-        s2 += __shfl_xor(s2, off);
-    }
-    if (lane == 0) {
-        red[0][wave] = s1;
-        red[1][wave] = s2;
+    for (int k = 0; k < (BW ? 4 : 2); ++k) {
+#pragma unroll
+        for (int off = 32; off > 0; off >>= 1) s[k] += __shfl_xor(s[k], off);
+        if (lane == 0) red[k][wave] = s[k];
     }
     __syncthreads();
-    s1 = (red[0][0] + red[0][1]) + (red[0][2] + red[0][3]);
-    s2 = (red[1][0] + red[1][1]) + (red[1][2] + red[1][3]);
-    const float cnt = (float)n;
-    const float mean = s1 / cnt;
-    const float sd = sqrtf(((s2 - 2 * s1 * mean) / cnt) + (mean * mean) + eps[0]);
-    const float w = weight[c], bb = bias[c];
-    for (size_t e = tid; e < n; e += 256) {
-        const size_t b = e / HW, hw = e - b * HW;
-        const size_t idx = (b * C + c) * HW + hw;
-        y[idx] = ((x[idx] - mean) / sd) * w + bb;
+    if (tid < (BW ? 4 : 2))
+        part[((size_t)c * gridDim.y + grp) * BN_SUMS + tid] = (red[tid][0] + red[tid][1]) + (red[tid][2] + red[tid][3]);
+}
+
+template <typename T, bool BW>
+__global__ __launch_bounds__(256) void bn_apply_kernel(const T *__restrict__ x, const T *__restrict__ dy,
+                                                       T *__restrict__ out, const T *__restrict__ weight,
+                                                       const T *__restrict__ bias, const T *__restrict__ eps,
+                                                       const float *__restrict__ part, T *__restrict__ dgamma,
+                                                       T *__restrict__ dbeta, int B, int C, int HW, int groups,
+                                                       int write_dx) {
+    const int plane = blockIdx.x, c = plane % C, tid = threadIdx.x;
+    float s[BN_SUMS] = {0.f, 0.f, 0.f, 0.f};
+    for (int g = 0; g < groups; ++g)
+#pragma unroll
+        for (int k = 0; k < (BW ? 4 : 2); ++k) s[k] += part[((size_t)c * groups + g) * BN_SUMS + k];
+    const float cnt = (float)B * (float)HW;
+    const float mean = s[0] / cnt;
+    const float sd = sqrtf(((s[1] - 2 * s[0] * mean) / cnt) + (mean * mean) + (float)eps[0]);
+    const float w = (float)weight[c];
+    const size_t base = (size_t)plane * HW;
+    if (!BW) {
+        const float bb = (float)bias[c];
+        for (int e = tid; e < HW; e += 256) out[base + e] = (T)((((float)x[base + e] - mean) / sd) * w + bb);
+    } else {
+        const float db = s[2], dg = (s[3] - mean * s[2]) / sd;
+        if (plane < C && tid == 0) {  // the planes of the first sample also write the channel's gradients
+            if (dgamma) dgamma[c] = (T)dg;
+            if (dbeta) dbeta[c] = (T)db;
+        }
+        if (write_dx) {
+            const float k0 = w / sd, k1 = db / cnt, k2 = dg / cnt;
+            for (int e = tid; e < HW; e += 256) {
+                const float xh = ((float)x[base + e] - mean) / sd;
+                out[base + e] = (T)(k0 * ((float)dy[base + e] - k1 - xh * k2));
+            }
+        }
     }
 }
 
-static int batch_norm_fw(const BatchNorm_args_fp32 *a, const char *fn) {
-    if (!a || !a->input || !a->output || !a->weight_data || !a->bias_data || !a->eps)
+template <typename T, typename Args>
+static int batch_norm_step(const Args *a, int bw, const char *fn) {
+    if (!a || !a->input || !a->output || !a->weight_data || !a->eps || (!bw && !a->bias_data))
         return glue_bad(fn, "invalid arguments");
     if (a->B <= 0 || a->C <= 0 || a->H <= 0 || a->W <= 0) return glue_bad(fn, "invalid tensor geometry");
     if (!ensure_init()) return 2;
-    const size_t n = (size_t)a->B * a->C * a->H * a->W;
+    State &st = state();
+    const int B = a->B, C = a->C, HW = a->H * a->W;
+    const size_t n = (size_t)B * C * HW;
+    if ((size_t)B * C >= ((size_t)1 << 31)) return glue_bad(fn, "too many planes");
+    // groups of samples: about four workgroups per CU in the first kernel
+    int groups = (4 * st.num_cu + C - 1) / C;
+    if (groups > B) groups = B;
+    const int per_group = (B + groups - 1) / groups;
+    groups = (B + per_group - 1) / per_group;
+    float *part = workspace((size_t)C * groups * BN_SUMS * sizeof(float));
+    if (!part) return 2;
     Stager sg;
-    const float *x = sg.in(a->input->data, n);
-    float *y = sg.out(a->output->data, n);
-    const float *w = sg.in(a->weight_data, (size_t)a->C);
-    const float *b = sg.in(a->bias_data, (size_t)a->C);
-    const float *eps = sg.in(a->eps, (size_t)1);
-    if (sg.failed() || !x || !y) return sg.failed() ? 2 : glue_bad(fn, "null buffer");
-    hipLaunchKernelGGL(batch_norm_fw_kernel, dim3(a->C), dim3(256), 0, state().stream, x, y, w, b, eps, a->B, a->C,
-                       a->H * a->W);
+    const T *x = sg.in(reinterpret_cast<const T *>(a->input->data), n);
+    const T *w = sg.in(reinterpret_cast<const T *>(a->weight_data), (size_t)C);
+    const T *eps = sg.in(reinterpret_cast<const T *>(a->eps), (size_t)1);
+    if (!x) return glue_bad(fn, "null buffer");
+    if (!bw) {
+        T *y = sg.out(reinterpret_cast<T *>(a->output->data), n);
+        const T *b = sg.in(reinterpret_cast<const T *>(a->bias_data), (size_t)C);
+        if (sg.failed() || !y) return sg.failed() ? 2 : glue_bad(fn, "null buffer");
+        hipLaunchKernelGGL((bn_sums_kernel<T, false>), dim3(C, groups), dim3(256), 0, st.stream, x, (const T *)nullptr,
+                           part, B, C, HW, per_group);
+        hipLaunchKernelGGL((bn_apply_kernel<T, false>), dim3((unsigned)(B * C)), dim3(256), 0, st.stream, x,
+                           (const T *)nullptr, y, w, b, eps, part, (T *)nullptr, (T *)nullptr, B, C, HW, groups, 1);
+    } else {
+        const T *dy = sg.in(reinterpret_cast<const T *>(a->output->diff), n);
+        const bool want_dx = !a->skip_in_grad, want_dw = !a->skip_wg_grad;
+        T *dx = want_dx ? sg.out(reinterpret_cast<T *>(a->input->diff), n) : nullptr;
+        T *dg = want_dw && a->coeff ? sg.out(reinterpret_cast<T *>(a->coeff->diff), (size_t)C) : nullptr;
+        T *db = want_dw && a->bias ? sg.out(reinterpret_cast<T *>(a->bias->diff), (size_t)C) : nullptr;
+        if (sg.failed() || !dy || (want_dx && !dx)) return sg.failed() ? 2 : glue_bad(fn, "null buffer");
+        hipLaunchKernelGGL((bn_sums_kernel<T, true>), dim3(C, groups), dim3(256), 0, st.stream, x, dy, part, B, C, HW,
+                           per_group);
+        // without an input gradient only the planes of the first sample run (they write dgamma / dbeta)
+        hipLaunchKernelGGL((bn_apply_kernel<T, true>), dim3((unsigned)(want_dx ? B * C : C)), dim3(256), 0, st.stream,
+                           x, dy, dx, w, (const T *)nullptr, eps, part, dg, db, B, C, HW, groups, want_dx ? 1 : 0);
+    }
     return sg.finish(hip_ok(hipGetLastError(), "batch norm launch") ? 0 : 2);
 }
 
@@ -378,7 +444,16 @@ int ptl_gradient_descent_fp16(const struct optim_args_fp16 *a) {
     return ptl::sgd_step<ptl::half_t>(a, "pulp_gradient_descent_fp16");
 }
 int ptl_batch_norm_fp32_fw(const struct BatchNorm_args_fp32 *a) {
-    return ptl::batch_norm_fw(a, "pulp_batch_norm_fp32_fw_cl");
+    return ptl::batch_norm_step<float>(a, 0, "pulp_batch_norm_fp32_fw_cl");
+}
+int ptl_batch_norm_fp32_bw(const struct BatchNorm_args_fp32 *a) {
+    return ptl::batch_norm_step<float>(a, 1, "ptl_batch_norm_fp32_bw");
+}
+int ptl_batch_norm_fp16_fw(const struct BatchNorm_args_fp16 *a) {
+    return ptl::batch_norm_step<ptl::half_t>(a, 0, "ptl_batch_norm_fp16_fw");
+}
+int ptl_batch_norm_fp16_bw(const struct BatchNorm_args_fp16 *a) {
+    return ptl::batch_norm_step<ptl::half_t>(a, 1, "ptl_batch_norm_fp16_bw");
 }
 
 }  // extern "C"

@@ -233,12 +233,14 @@ def optim_args(pkg, dt, w, dw, b, db, lr, lam):
     return a, keep
 
 
-def batch_norm_args(pkg, x, y, w, b, eps, B, C, H, W):
+def batch_norm_args(pkg, x, y, w, b, eps, B, C, H, W, dx=None, dy=None, dw=None, db=None):
     keep = Keep()
-    bi, bo = pkg.blob(x, None, C, H, W), pkg.blob(y, None, C, H, W)
-    keep += [bi, bo, x, y, w, b, eps]
+    bi, bo = pkg.blob(x, dx, C, H, W), pkg.blob(y, dy, C, H, W)
+    bw, bb = pkg.blob(w, dw, C, 1, 1, dim=C), pkg.blob(b, db, C, 1, 1, dim=C)
+    keep += [bi, bo, bw, bb, x, y, w, b, eps, dx, dy, dw, db]
     a = pkg.BatchNormArgs()
     a.input, a.output = ptr(bi), ptr(bo)
+    a.coeff, a.bias = ptr(bw), ptr(bb)
     a.weight_data, a.bias_data, a.eps = pkg.addr(w), pkg.addr(b), pkg.addr(eps)
     a.B, a.C, a.H, a.W = B, C, H, W
     a.batch_size = B

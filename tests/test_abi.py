@@ -48,7 +48,7 @@ STRUCTS = {
     "softmax_args": "SoftmaxArgs", "Mhsa_args": "MhsaArgs", "act_args": "ActArgs", "act_args_fp16": "ActArgs",
     "SkipConn_args": "SkipConnArgs", "SkipConn_args_fp16": "SkipConnArgs", "pool_args": "PoolArgs",
     "pool_args_fp16": "PoolArgs", "loss_args": "LossArgs", "loss_args_fp16": "LossArgs", "optim_args": "OptimArgs",
-    "optim_args_fp16": "OptimArgsFp16", "BatchNorm_args_fp32": "BatchNormArgs",
+    "optim_args_fp16": "OptimArgsFp16", "BatchNorm_args_fp32": "BatchNormArgs", "BatchNorm_args_fp16": "BatchNormArgs",
 }
 
 

@@ -140,6 +140,41 @@ def test_batch_norm_forward(pkg, orc, gpu):
     assert hp.rel_l2(y, ry) <= 1e-5
 
 
+@pytest.mark.parametrize("dt", ["fp32", "fp16"])
+@pytest.mark.parametrize("B,C,H,W", [(8, 16, 9, 11), (128, 16, 32, 32), (3, 70, 8, 8)])
+def test_batch_norm_training_passes(pkg, orc, gpu, dt, B, C, H, W):
+    """Forward and backward in both types against the oracle (whose backward is pinned against torch autograd)."""
+    nd = hp.np_dtype(dt)
+    x = (1.5 * hp.normal(0x7E60, (B, C, H, W)) + 0.25).astype(nd)
+    g = hp.uniform(0x7E61, (B, C, H, W)).astype(nd)
+    w, b = hp.uniform(0x7E62, (C,), 0.5, 1.5).astype(nd), hp.uniform(0x7E63, (C,)).astype(nd)
+    eps = np.array([1e-5], nd)
+    ry, rdx, rdw, rdb = np.zeros_like(x), np.zeros_like(x), np.zeros_like(w), np.zeros_like(b)
+    a, k = hp.batch_norm_args(pkg, x, ry, w, b, eps, B, C, H, W, rdx, g, rdw, rdb)
+    getattr(orc.load(), "orc_batch_norm_fw_" + dt)(ctypes.byref(a))
+    getattr(orc.load(), "orc_batch_norm_bw_" + dt)(ctypes.byref(a))
+    gx, gg, gw, gb, geps = dev(x), dev(g), dev(w), dev(b), dev(eps)
+    y, dx = torch.full_like(gx, 7), torch.full_like(gx, 7)
+    dw, db = torch.full_like(gw, 7), torch.full_like(gb, 7)
+    c, k2 = hp.batch_norm_args(pkg, gx, y, gw, gb, geps, B, C, H, W, dx, gg, dw, db)
+    assert getattr(gpu, "ptl_batch_norm_%s_fw" % dt)(ctypes.byref(c)) == 0, gpu.ptl_last_error().decode()
+    assert getattr(gpu, "ptl_batch_norm_%s_bw" % dt)(ctypes.byref(c)) == 0, gpu.ptl_last_error().decode()
+    gpu.ptl_sync()
+    tol = 1e-4 if dt == "fp32" else 1e-2
+    for got, ref in ((y, ry), (dx, rdx), (dw, rdw), (db, rdb)):
+        assert hp.rel_l2(host(got), ref) <= tol
+    dx.fill_(9), dw.fill_(9), db.fill_(9)
+    c.skip_in_grad = 1
+    assert getattr(gpu, "ptl_batch_norm_%s_bw" % dt)(ctypes.byref(c)) == 0
+    gpu.ptl_sync()
+    assert bool(torch.all(dx == 9)) and hp.rel_l2(host(dw), rdw) <= tol and hp.rel_l2(host(db), rdb) <= tol
+    c.skip_in_grad, c.skip_wg_grad = 0, 1
+    dw.fill_(9), db.fill_(9)
+    assert getattr(gpu, "ptl_batch_norm_%s_bw" % dt)(ctypes.byref(c)) == 0
+    gpu.ptl_sync()
+    assert bool(torch.all(dw == 9)) and bool(torch.all(db == 9)) and hp.rel_l2(host(dx), rdx) <= tol
+
+
 def test_reference_named_single_sample_entry_points(pkg, orc, gpu):
     dim = 300
     x, g = hp.uniform(0x7E50, (dim,)), hp.uniform(0x7E51, (dim,))

@@ -110,3 +110,36 @@ def test_batch_norm_forward(pkg, orc):
     lib.orc_batch_norm_fw_fp32(ctypes.byref(a))
     ref = F.batch_norm(t64(x), None, None, t64(w), t64(b), training=True, eps=1e-5)
     assert hp.rel_l2(y, ref.numpy()) <= 5e-6
+
+
+@pytest.mark.parametrize("dt", ["fp32", "fp16"])
+def test_batch_norm_backward_and_fp16(pkg, orc, dt):
+    """The restated backward pass (and the fp16 forward) against torch batch_norm and its autograd in float64."""
+    lib = orc.load()
+    nd = hp.np_dtype(dt)
+    B, C, H, W = 5, 6, 7, 4
+    x = (1.5 * hp.normal(0x6E50, (B, C, H, W)) + 0.25).astype(nd)
+    g = hp.uniform(0x6E51, (B, C, H, W)).astype(nd)
+    w, b = hp.uniform(0x6E52, (C,), 0.5, 1.5).astype(nd), hp.uniform(0x6E53, (C,)).astype(nd)
+    eps = np.array([1e-5], nd)
+    y, dx = np.zeros_like(x), np.zeros_like(x)
+    dw, db = np.zeros_like(w), np.zeros_like(b)
+    a, keep = hp.batch_norm_args(pkg, x, y, w, b, eps, B, C, H, W, dx, g, dw, db)
+    getattr(lib, "orc_batch_norm_fw_" + dt)(ctypes.byref(a))
+    getattr(lib, "orc_batch_norm_bw_" + dt)(ctypes.byref(a))
+    tx, tw, tb = t64(x).requires_grad_(), t64(w).requires_grad_(), t64(b).requires_grad_()
+    ref = F.batch_norm(tx, None, None, tw, tb, training=True, eps=float(eps[0]))
+    ref.backward(t64(g))
+    tol = 2e-5 if dt == "fp32" else 2e-3
+    assert hp.rel_l2(y, ref.detach().numpy()) <= tol
+    assert hp.rel_l2(dx, tx.grad.numpy()) <= tol
+    assert hp.rel_l2(dw, tw.grad.numpy()) <= tol and hp.rel_l2(db, tb.grad.numpy()) <= tol
+    # the skip flags leave the corresponding outputs alone
+    dx[:], dw[:], db[:] = 9, 9, 9
+    a.skip_in_grad = 1
+    getattr(lib, "orc_batch_norm_bw_" + dt)(ctypes.byref(a))
+    assert np.all(dx == 9) and not np.any(dw == 9)
+    a.skip_in_grad, a.skip_wg_grad = 0, 1
+    dw[:], db[:] = 9, 9
+    getattr(lib, "orc_batch_norm_bw_" + dt)(ctypes.byref(a))
+    assert np.all(dw == 9) and np.all(db == 9) and not np.any(dx == 9)
