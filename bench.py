@@ -318,15 +318,10 @@ def detail_table(pkg, lib, hp, to_dev, timed, check, torch, dev):
         ms = timed(lambda: check(lib.ptl_mhsa_fp32_bw_batched(ref, ns)), 50)
         add("mhsa L197 E192 3x64 BW N=%d" % ns, "fp32", ms, 2 * f_fw, 2 * act)
 
-    # config 5 (without normalisation layers: the reference has no batch-norm backward): ResNet-20-shaped
-    # training step, fp16, batch 128, assembled from the entry points (tests/resnet_step.py)
+    # config 5: ResNet-20 (CIFAR geometry) training step, fp16, batch 128, assembled from the entry points
+    # (tests/resnet_step.py): with batch normalisation after every convolution, and without
     import resnet_step as rs
     ns, dt = 128, "fp16"
-    net = rs.ResNetStep(pkg, lib, torch, dt, ns, rs.init_weights(0x2E5E0, dt), 0.01)
-    net.x.copy_(torch.randn(ns, 3, 32, 32, device=dev).to(tdt[dt]))
-    net.target.zero_()
-    net.target[torch.arange(ns), torch.randint(0, 10, (ns,))] = 1
-    ms = timed(lambda: net.step(update=True), 10, 3)
     convs, blocks, ncls = rs.resnet20_spec()
     macs, H = 3 * 16 * 9 * 32 * 32, 32
     for (n, ci, co, stride, proj) in blocks:
@@ -334,9 +329,17 @@ def detail_table(pkg, lib, hp, to_dev, timed, check, torch, dev):
         macs += (ci * co * 9 + co * co * 9 + (ci * co if proj else 0)) * Ho * Ho
         H = Ho
     flops = 3 * 2.0 * ns * (macs + 64 * ncls)
-    rows.append({"workload": "resnet20-shaped step (no norm) FW+BW+SGD N=%d, %d launches" % (ns, net.launches()),
-                 "dtype": dt, "us": round(ms * 1e3, 1), "TFLOP/s": round(flops / (ms * 1e-3) / 1e12, 3),
-                 "samples/s": round(ns / (ms * 1e-3), 1)})
+    for norm in (True, False):
+        net = rs.ResNetStep(pkg, lib, torch, dt, ns, rs.init_weights(0x2E5E0, dt), 0.01, norm=norm)
+        net.x.copy_(torch.randn(ns, 3, 32, 32, device=dev).to(tdt[dt]))
+        net.target.zero_()
+        net.target[torch.arange(ns), torch.randint(0, 10, (ns,))] = 1
+        ms = timed(lambda: net.step(update=True), 10, 3)
+        rows.append({"workload": "resnet20 step%s FW+BW+SGD N=%d, %d launches"
+                                 % (" with batch norm" if norm else " (no norm)", ns, net.launches()),
+                     "dtype": dt, "us": round(ms * 1e3, 1), "TFLOP/s": round(flops / (ms * 1e-3) / 1e12, 3),
+                     "samples/s": round(ns / (ms * 1e-3), 1)})
+        del net
     return rows
 
 

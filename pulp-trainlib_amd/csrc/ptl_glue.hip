@@ -286,22 +286,49 @@ static int sgd_step(const Args *a, const char *fn) {
 // ---- Batch normalisation (forward: lib/sources/pulp_batchnorm_fp32.c:34-114) ---------------------------
 // Statistics per channel over B x H x W, in two launches so that a few channels still fill the chip:
 //   1. partial sums per (channel, group of samples): forward x and x^2; backward also dy and dy*x;
-//   2. every workgroup of the second kernel owns one (sample, channel) plane, adds the channel's partials in a
-//      fixed order, forms mean and deviation the way the reference does and maps its plane.
+//   2. the workgroups of the second kernel own the same (channel, group of samples) pieces, add the channel's
+//      partials in a fixed order, form mean and deviation the way the reference does and map their planes.
 // The backward pass (the reference has none; the usual one for the forward above):
 //   xh = (x - mean) / sd,  dbeta = sum dy,  dgamma = sum dy * xh = (sum dy*x - mean * sum dy) / sd,
 //   dx = gamma / sd * (dy - dbeta / n - xh * dgamma / n).
 constexpr int BN_SUMS = 4;
 
+template <typename T>
+union BnVec {
+    uint4 raw;
+    T e[16 / sizeof(T)];
+};
+
 template <typename T, bool BW>
 __global__ __launch_bounds__(256) void bn_sums_kernel(const T *__restrict__ x, const T *__restrict__ dy,
-                                                      float *__restrict__ part, int B, int C, int HW, int per_group) {
+                                                      float *__restrict__ part, int B, int C, int HW, int per_group,
+                                                      int vec) {
     __shared__ float red[BN_SUMS][4];
     const int c = blockIdx.x, grp = blockIdx.y, tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int b0 = grp * per_group, b1 = min(B, b0 + per_group);
+    constexpr int VEC = 16 / (int)sizeof(T);
     float s[BN_SUMS] = {0.f, 0.f, 0.f, 0.f};
     for (int b = b0; b < b1; ++b) {
         const size_t base = ((size_t)b * C + c) * HW;
+        if (vec) {  // planes are whole 16-byte vectors
+            for (int e = tid * VEC; e < HW; e += 256 * VEC) {
+                BnVec<T> xv, gv;
+                xv.raw = *reinterpret_cast<const uint4 *>(x + base + e);
+                if (BW) gv.raw = *reinterpret_cast<const uint4 *>(dy + base + e);
+#pragma unroll
+                for (int q = 0; q < VEC; ++q) {
+                    const float v = (float)xv.e[q];
+                    s[0] += v;
+                    s[1] += v * v;
+                    if (BW) {
+                        const float g = (float)gv.e[q];
+                        s[2] += g;
+                        s[3] += g * v;
+                    }
+                }
+            }
+            continue;
+        }
         for (int e = tid; e < HW; e += 256) {
             const float v = (float)x[base + e];
             s[0] += v;
@@ -330,32 +357,60 @@ __global__ __launch_bounds__(256) void bn_apply_kernel(const T *__restrict__ x, 
                                                        const T *__restrict__ bias, const T *__restrict__ eps,
                                                        const float *__restrict__ part, T *__restrict__ dgamma,
                                                        T *__restrict__ dbeta, int B, int C, int HW, int groups,
-                                                       int write_dx) {
-    const int plane = blockIdx.x, c = plane % C, tid = threadIdx.x;
-    float s[BN_SUMS] = {0.f, 0.f, 0.f, 0.f};
-    for (int g = 0; g < groups; ++g)
+                                                       int per_group, int write_dx, int vec) {
+    constexpr int VEC = 16 / (int)sizeof(T);
+    const int c = blockIdx.x, grp = blockIdx.y, tid = threadIdx.x;
+    // the channel's partial sums (at most 64 groups): one lane each, folded by the first wave in a fixed order
+    __shared__ float tot[BN_SUMS];
+    if (tid < 64) {
 #pragma unroll
-        for (int k = 0; k < (BW ? 4 : 2); ++k) s[k] += part[((size_t)c * groups + g) * BN_SUMS + k];
+        for (int k = 0; k < (BW ? 4 : 2); ++k) {
+            float v = tid < groups ? part[((size_t)c * groups + tid) * BN_SUMS + k] : 0.f;
+#pragma unroll
+            for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off);
+            if (tid == 0) tot[k] = v;
+        }
+    }
+    __syncthreads();
+    float s[BN_SUMS] = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int k = 0; k < (BW ? 4 : 2); ++k) s[k] = tot[k];
     const float cnt = (float)B * (float)HW;
     const float mean = s[0] / cnt;
     const float sd = sqrtf(((s[1] - 2 * s[0] * mean) / cnt) + (mean * mean) + (float)eps[0]);
     const float w = (float)weight[c];
-    const size_t base = (size_t)plane * HW;
-    if (!BW) {
-        const float bb = (float)bias[c];
-        for (int e = tid; e < HW; e += 256) out[base + e] = (T)((((float)x[base + e] - mean) / sd) * w + bb);
-    } else {
-        const float db = s[2], dg = (s[3] - mean * s[2]) / sd;
-        if (plane < C && tid == 0) {  // the planes of the first sample also write the channel's gradients
-            if (dgamma) dgamma[c] = (T)dg;
-            if (dbeta) dbeta[c] = (T)db;
+    const float bb = BW ? 0.f : (float)bias[c];
+    const float db = s[2], dg = (s[3] - mean * s[2]) / sd;
+    if (BW && grp == 0 && tid == 0) {
+        if (dgamma) dgamma[c] = (T)dg;
+        if (dbeta) dbeta[c] = (T)db;
+    }
+    if (BW && !write_dx) return;
+    const float k0 = w / sd, k1 = db / cnt, k2 = dg / cnt;
+    auto map = [&](float xv, float gv) {
+        if (!BW) return ((xv - mean) / sd) * w + bb;
+        const float xh = (xv - mean) / sd;
+        return k0 * (gv - k1 - xh * k2);
+    };
+    // the group's planes of this channel as one index range: element i = (sample i / HW, position i % HW)
+    const int b0 = grp * per_group, nb = min(B, b0 + per_group) - b0;
+    const int total = nb * HW;
+    if (vec) {
+        for (int i = tid * VEC; i < total; i += 256 * VEC) {
+            const int bl = i / HW, e = i - bl * HW;
+            const size_t at = ((size_t)(b0 + bl) * C + c) * HW + e;
+            BnVec<T> xv, gv;
+            xv.raw = *reinterpret_cast<const uint4 *>(x + at);
+            if (BW) gv.raw = *reinterpret_cast<const uint4 *>(dy + at);
+#pragma unroll
+            for (int q = 0; q < VEC; ++q) xv.e[q] = (T)map((float)xv.e[q], BW ? (float)gv.e[q] : 0.f);
+            *reinterpret_cast<uint4 *>(out + at) = xv.raw;
         }
-        if (write_dx) {
-            const float k0 = w / sd, k1 = db / cnt, k2 = dg / cnt;
-            for (int e = tid; e < HW; e += 256) {
-                const float xh = ((float)x[base + e] - mean) / sd;
-                out[base + e] = (T)(k0 * ((float)dy[base + e] - k1 - xh * k2));
-            }
+    } else {
+        for (int i = tid; i < total; i += 256) {
+            const int bl = i / HW, e = i - bl * HW;
+            const size_t at = ((size_t)(b0 + bl) * C + c) * HW + e;
+            out[at] = (T)map((float)x[at], BW ? (float)dy[at] : 0.f);
         }
     }
 }
@@ -372,6 +427,7 @@ static int batch_norm_step(const Args *a, int bw, const char *fn) {
     if ((size_t)B * C >= ((size_t)1 << 31)) return glue_bad(fn, "too many planes");
     // groups of samples: about four workgroups per CU in the first kernel
     int groups = (4 * st.num_cu + C - 1) / C;
+    if (groups > 64) groups = 64;  // the second kernel folds them with one wave
     if (groups > B) groups = B;
     const int per_group = (B + groups - 1) / groups;
     groups = (B + per_group - 1) / per_group;
@@ -380,16 +436,20 @@ static int batch_norm_step(const Args *a, int bw, const char *fn) {
     Stager sg;
     const T *x = sg.in(reinterpret_cast<const T *>(a->input->data), n);
     const T *w = sg.in(reinterpret_cast<const T *>(a->weight_data), (size_t)C);
+    auto aligned16 = [](const void *p) { return reinterpret_cast<uintptr_t>(p) % 16 == 0; };
+    const int VEC = 16 / (int)sizeof(T);
     const T *eps = sg.in(reinterpret_cast<const T *>(a->eps), (size_t)1);
     if (!x) return glue_bad(fn, "null buffer");
     if (!bw) {
         T *y = sg.out(reinterpret_cast<T *>(a->output->data), n);
         const T *b = sg.in(reinterpret_cast<const T *>(a->bias_data), (size_t)C);
         if (sg.failed() || !y) return sg.failed() ? 2 : glue_bad(fn, "null buffer");
+        const int vec = HW % VEC == 0 && aligned16(x) && aligned16(y);
         hipLaunchKernelGGL((bn_sums_kernel<T, false>), dim3(C, groups), dim3(256), 0, st.stream, x, (const T *)nullptr,
-                           part, B, C, HW, per_group);
-        hipLaunchKernelGGL((bn_apply_kernel<T, false>), dim3((unsigned)(B * C)), dim3(256), 0, st.stream, x,
-                           (const T *)nullptr, y, w, b, eps, part, (T *)nullptr, (T *)nullptr, B, C, HW, groups, 1);
+                           part, B, C, HW, per_group, vec);
+        hipLaunchKernelGGL((bn_apply_kernel<T, false>), dim3(C, groups), dim3(256), 0, st.stream, x,
+                           (const T *)nullptr, y, w, b, eps, part, (T *)nullptr, (T *)nullptr, B, C, HW, groups,
+                           per_group, 1, vec);
     } else {
         const T *dy = sg.in(reinterpret_cast<const T *>(a->output->diff), n);
         const bool want_dx = !a->skip_in_grad, want_dw = !a->skip_wg_grad;
@@ -397,11 +457,13 @@ static int batch_norm_step(const Args *a, int bw, const char *fn) {
         T *dg = want_dw && a->coeff ? sg.out(reinterpret_cast<T *>(a->coeff->diff), (size_t)C) : nullptr;
         T *db = want_dw && a->bias ? sg.out(reinterpret_cast<T *>(a->bias->diff), (size_t)C) : nullptr;
         if (sg.failed() || !dy || (want_dx && !dx)) return sg.failed() ? 2 : glue_bad(fn, "null buffer");
+        const int vec = HW % VEC == 0 && aligned16(x) && aligned16(dy) && (!dx || aligned16(dx));
         hipLaunchKernelGGL((bn_sums_kernel<T, true>), dim3(C, groups), dim3(256), 0, st.stream, x, dy, part, B, C, HW,
-                           per_group);
-        // without an input gradient only the planes of the first sample run (they write dgamma / dbeta)
-        hipLaunchKernelGGL((bn_apply_kernel<T, true>), dim3((unsigned)(want_dx ? B * C : C)), dim3(256), 0, st.stream,
-                           x, dy, dx, w, (const T *)nullptr, eps, part, dg, db, B, C, HW, groups, want_dx ? 1 : 0);
+                           per_group, vec);
+        // without an input gradient only the first group of every channel runs (it writes dgamma / dbeta)
+        hipLaunchKernelGGL((bn_apply_kernel<T, true>), dim3(C, want_dx ? groups : 1), dim3(256), 0, st.stream, x, dy,
+                           dx, w, (const T *)nullptr, eps, part, dg, db, B, C, HW, groups, per_group, want_dx ? 1 : 0,
+                           vec);
     }
     return sg.finish(hip_ok(hipGetLastError(), "batch norm launch") ? 0 : 2);
 }

@@ -1,8 +1,9 @@
 """A ResNet-20-shaped (CIFAR geometry) training step assembled from the library's entry points, the way a
 generated `net.c` of the reference strings its layer calls together: 3x3 stem, three stages of three residual
 blocks (16/32/64 channels, stride-2 1x1 projection shortcuts), ReLU, global average pooling, a linear
-classifier, cross-entropy and one gradient-descent update.  No normalisation layers: the reference has no
-batch-norm backward.  Used by the GPU parity test and by the benchmark's detail table."""
+classifier, cross-entropy and one gradient-descent update.  With `norm=True` every convolution is followed by
+batch normalisation over the batch (the reference's forward, lib/sources/pulp_batchnorm_fp32.c:34, and this
+library's backward for it).  Used by the GPU parity test and by the benchmark's detail table."""
 import ctypes
 
 import numpy as np
@@ -43,7 +44,7 @@ def init_weights(seed, dt):
 class ResNetStep:
     """Device buffers, argument structs and the call sequence of one training step on `ns` samples."""
 
-    def __init__(self, pkg, lib, torch, dt, ns, weights, lr=0.01):
+    def __init__(self, pkg, lib, torch, dt, ns, weights, lr=0.01, norm=False):
         self.pkg, self.lib, self.dt, self.ns, self.lr = pkg, lib, dt, ns, lr
         tdt = torch.float16 if dt == "fp16" else torch.float32
         dev = lambda a: torch.from_numpy(np.ascontiguousarray(a)).cuda()
@@ -52,6 +53,8 @@ class ResNetStep:
         self.W = {n: dev(v) for n, v in weights.items()}
         self.dW = {n: z(*v.shape) for n, v in weights.items()}
         self.keep = []
+        self.G, self.dG, self.Bt, self.dBt = {}, {}, {}, {}  # scale / shift of the normalisation layers
+        eps = torch.full((1,), 1e-5, dtype=tdt, device="cuda")
         self.fw, self.bw = [], []  # lists of (function name, struct, extra args)
         spec = {n: (ci, co, k, s) for n, ci, co, k, s in convs}
         L = lambda name: name.replace("DT", dt)
@@ -66,7 +69,21 @@ class ResNetStep:
             a, kp = hp.conv2d_args(pkg, x, dx, self.W[name], self.dW[name], y, dy, ci, H, H, co, k, k, Ho, Ho,
                                    (p, p, p, p), (s, s), 0, 1 if s == 1 else 0)
             self.keep.append(kp)
-            return a, y, dy, Ho
+            fw = [(L("ptl_conv2d_DT_fw_batched"), a, (ns,))]
+            bw = [(L("ptl_conv2d_DT_wg_batched"), a, (ns,))]
+            if dx is not None:
+                bw.append((L("ptl_conv2d_DT_ig_batched"), a, (ns,)))
+            if norm:
+                self.G[name], self.Bt[name] = torch.ones(co, dtype=tdt, device="cuda"), z(co)
+                self.dG[name], self.dBt[name] = z(co), z(co)
+                n_, dn_ = z(ns, co, Ho, Ho), z(ns, co, Ho, Ho)
+                na, kp = hp.batch_norm_args(pkg, y, n_, self.G[name], self.Bt[name], eps, ns, co, Ho, Ho, dy, dn_,
+                                            self.dG[name], self.dBt[name])
+                self.keep.append(kp)
+                fw.append((L("ptl_batch_norm_DT_fw"), na, ()))
+                bw.insert(0, (L("ptl_batch_norm_DT_bw"), na, ()))
+                y, dy = n_, dn_
+            return fw, bw, y, dy, Ho
 
         def relu(x, dx):
             y, dy = z(*x.shape), z(*x.shape)
@@ -75,25 +92,23 @@ class ResNetStep:
             return a, y, dy
 
         self.x, self.dx0 = z(ns, 3, 32, 32), None
-        a, t, dt_, H = conv("stem", self.x, None, 32)
-        self.fw.append((L("ptl_conv2d_DT_fw_batched"), a, (ns,)))
-        first_bw = [(L("ptl_conv2d_DT_wg_batched"), a, (ns,))]  # the stem needs no input gradient
+        f, first_bw, t, dt_, H = conv("stem", self.x, None, 32)  # the stem needs no input gradient
+        self.fw += f
         ra, t, dt_ = relu(t, dt_)
         self.fw.append((L("ptl_relu_DT_batched"), ra, (ns, 0)))
         first_bw.insert(0, (L("ptl_relu_DT_batched"), ra, (ns, 1)))
         bw_blocks = []
         for (n, ci, co, stride, proj) in blocks:
             xin, dxin, Hin = t, dt_, H
-            c1, y1, dy1, H = conv(n + "c1", xin, dxin, Hin)
+            f1, b1, y1, dy1, H = conv(n + "c1", xin, dxin, Hin)
             r1, a1, da1 = relu(y1, dy1)
-            c2, y2, dy2, H = conv(n + "c2", a1, da1, H)
-            seq = [(L("ptl_conv2d_DT_fw_batched"), c1, (ns,)), (L("ptl_relu_DT_batched"), r1, (ns, 0)),
-                   (L("ptl_conv2d_DT_fw_batched"), c2, (ns,))]
+            f2, b2, y2, dy2, H = conv(n + "c2", a1, da1, H)
+            seq = f1 + [(L("ptl_relu_DT_batched"), r1, (ns, 0))] + f2
             if proj:
                 # the projection's input gradient must be ADDED to the main branch's: it gets its own buffer
                 dproj = z(*xin.shape)
-                cs, ys, dys, _ = conv(proj, xin, dproj, Hin)
-                seq.append((L("ptl_conv2d_DT_fw_batched"), cs, (ns,)))
+                fs, bs, ys, dys, _ = conv(proj, xin, dproj, Hin)
+                seq += fs
                 skip, dskip = ys, dys
             else:
                 skip, dskip = xin, dxin
@@ -104,19 +119,15 @@ class ResNetStep:
             seq += [(L("ptl_residual_DT_batched"), sk, (ns, 0)), (L("ptl_relu_DT_batched"), r2, (ns, 0))]
             self.fw += seq
             b = [(L("ptl_relu_DT_batched"), r2, (ns, 1)),            # ds = relu'(s) * dt
-                 (L("ptl_residual_DT_batched"), sk, (ns, 2)),         # dy2 = ds
-                 (L("ptl_conv2d_DT_wg_batched"), c2, (ns,)), (L("ptl_conv2d_DT_ig_batched"), c2, (ns,)),
-                 (L("ptl_relu_DT_batched"), r1, (ns, 1)),
-                 (L("ptl_conv2d_DT_wg_batched"), c1, (ns,)), (L("ptl_conv2d_DT_ig_batched"), c1, (ns,))]  # dxin = main
+                 (L("ptl_residual_DT_batched"), sk, (ns, 2))]         # dy2 = ds
+            b += b2 + [(L("ptl_relu_DT_batched"), r1, (ns, 1))] + b1  # ... dxin = main branch
             if proj:
                 add, kp = hp.skip_args(pkg, dxin, dxin, dproj, dproj, dproj, dproj, int(np.prod(xin.shape[1:])))
                 self.keep.append(kp)
                 # dys = ds (copy through a residual-backward call on a view of the projection output)
                 cp, kp2 = hp.skip_args(pkg, ys, dys, ys, dys, s_, ds_, int(np.prod(y2.shape[1:])))
                 self.keep.append(kp2)
-                b += [(L("ptl_residual_DT_batched"), cp, (ns, 2)),     # dys = ds
-                      (L("ptl_conv2d_DT_wg_batched"), cs, (ns,)), (L("ptl_conv2d_DT_ig_batched"), cs, (ns,)),
-                      self._vect_sum(dxin, dproj)]                     # dxin += dproj
+                b += [(L("ptl_residual_DT_batched"), cp, (ns, 2))] + bs + [self._vect_sum(dxin, dproj)]  # dxin += dproj
             else:
                 b.append((L("ptl_residual_DT_batched"), sk, (ns, 1)))  # dxin += ds (identity shortcut)
             bw_blocks.append(b)
@@ -139,6 +150,10 @@ class ResNetStep:
         self.opt = []
         for n in self.W:
             o, kp = hp.optim_args(pkg, dt, self.W[n], self.dW[n], None, None, lr, 0.0)
+            self.keep.append(kp)
+            self.opt.append((L("ptl_gradient_descent_DT"), o, ()))
+        for n in self.G:  # scale and shift of a normalisation layer in one update
+            o, kp = hp.optim_args(pkg, dt, self.G[n], self.dG[n], self.Bt[n], self.dBt[n], lr, 0.0)
             self.keep.append(kp)
             self.opt.append((L("ptl_gradient_descent_DT"), o, ()))
 

@@ -12,14 +12,27 @@ import resnet_step as rs
 pytestmark = pytest.mark.gpu
 
 
-def torch_step(weights, x, target, lr):
+def torch_step(weights, x, target, lr, norm=False, stored=None):
+    """`stored`: the type every tensor that the library materialises is rounded to on the way forward (the
+    rounding passes gradients through unchanged), so that a float64 reference sees the activations - and with
+    them the ReLU masks - that an fp16 run sees."""
+    q = (lambda t: t.to(stored).to(torch.float64)) if stored is not None else (lambda t: t)
     convs, blocks, ncls = rs.resnet20_spec()
     p = {n: torch.tensor(v.astype(np.float64), requires_grad=True) for n, v in weights.items()}
-    t = F.relu(F.conv2d(torch.tensor(x.astype(np.float64)), p["stem"], padding=1))
+    if norm:
+        for n, ci, co, k, s in convs:
+            p["g:" + n] = torch.ones(co, dtype=torch.float64, requires_grad=True)
+            p["b:" + n] = torch.zeros(co, dtype=torch.float64, requires_grad=True)
+
+    def conv(t, n, **kw):
+        y = q(F.conv2d(t, p[n], **kw))
+        return q(F.batch_norm(y, None, None, p["g:" + n], p["b:" + n], training=True, eps=1e-5)) if norm else y
+
+    t = F.relu(conv(torch.tensor(x.astype(np.float64)), "stem", padding=1))
     for (n, ci, co, stride, proj) in blocks:
-        y = F.conv2d(F.relu(F.conv2d(t, p[n + "c1"], stride=stride, padding=1)), p[n + "c2"], padding=1)
-        sc = F.conv2d(t, p[proj], stride=stride) if proj else t
-        t = F.relu(y + sc)
+        y = conv(F.relu(conv(t, n + "c1", stride=stride, padding=1)), n + "c2", padding=1)
+        sc = conv(t, proj, stride=stride) if proj else t
+        t = F.relu(q(y + sc))
     logits = t.mean((2, 3)) @ p["fc"].t()
     loss = F.cross_entropy(logits, torch.tensor(target.astype(np.float64)), reduction="none")
     loss.sum().backward()
@@ -48,3 +61,34 @@ def test_resnet20_training_step(pkg, gpu, dt, ns, tol):
     for n in w:
         assert hp.rel_l2(net.W[n].cpu().numpy(), ref_new[n]) <= tol, n
     assert net.launches() > 150
+
+
+@pytest.mark.parametrize("dt,ns,tol", [("fp32", 6, 1e-3), ("fp16", 8, 1.5e-1)])
+def test_resnet20_training_step_with_batch_norm(pkg, gpu, dt, ns, tol):
+    """The same step with batch normalisation after every convolution (BASELINE's ResNet-20 configuration).
+    fp16: the reference sees fp16-rounded activations; what remains is the rounding of the stored gradients, which
+    twenty normalised layers down are of the order of 1e-4 and keep few significant bits in fp16 (no loss scaling,
+    as in the reference) - 7 to 10 % on the deepest weight gradients."""
+    lr = 0.01
+    w = rs.init_weights(0x2E5F0, dt)
+    x = hp.normal(0x2E5F1, (ns, 3, 32, 32)).astype(hp.np_dtype(dt))
+    tgt = np.zeros((ns, 10), hp.np_dtype(dt))
+    tgt[np.arange(ns), (3 * np.arange(ns)) % 10] = 1
+    net = rs.ResNetStep(pkg, gpu, torch, dt, ns, w, lr, norm=True)
+    net.x.copy_(torch.from_numpy(x))
+    net.target.copy_(torch.from_numpy(tgt))
+    net.step(update=True)
+    assert gpu.ptl_sync() == 0
+    ref_logits, ref_loss, ref_grads, ref_new = torch_step(w, x, tgt, float(hp.np_dtype(dt)(lr)), norm=True,
+                                                          stored=torch.float16 if dt == "fp16" else None)
+    assert hp.rel_l2(net.logits.cpu().numpy(), ref_logits) <= tol
+    assert hp.rel_l2(net.loss.cpu().numpy(), ref_loss) <= tol
+    for n in ("fc", "s2b2c2", "s2b0sc", "s1b0c1", "stem"):
+        assert hp.rel_l2(net.dW[n].cpu().numpy(), ref_grads[n]) <= tol, n
+    for n in ("s2b2c2", "s0b0c1", "stem"):
+        assert hp.rel_l2(net.dG[n].cpu().numpy(), ref_grads["g:" + n]) <= tol, n
+        assert hp.rel_l2(net.dBt[n].cpu().numpy(), ref_grads["b:" + n]) <= tol, n
+        assert hp.rel_l2(net.G[n].cpu().numpy(), ref_new["g:" + n]) <= tol, n
+    for n in w:
+        assert hp.rel_l2(net.W[n].cpu().numpy(), ref_new[n]) <= tol, n
+    assert net.launches() > 200
