@@ -117,7 +117,8 @@ GLUE(_Float16, fp16, struct blob_fp16, struct act_args_fp16, struct SkipConn_arg
  * B x H x W, deviation = sqrt((s2 - 2 s1 mean) / n + mean^2 + eps)).  The reference has no backward pass and no
  * fp16 variant; those restate the textbook gradient of that forward,
  *   xh = (x - mean) / sd, dbeta = sum dy, dgamma = sum dy xh, dx = gamma / sd (dy - dbeta / n - xh dgamma / n),
- * with fp32 sums, and are pinned against torch autograd in float64 by tests/test_oracle_glue.py. */
+ * with fp32 sums: parity unpinned against the reference (it has nothing to compare with), pinned against torch
+ * autograd in float64 by tests/test_oracle_glue.py. */
 #define BATCH_NORM(T, SFX, ARGS)                                                                          \
     static void bn_stats_##SFX(const ARGS *a, int c, float *mean, float *sd) {                            \
         const T *in = a->input->data;                                                                     \
