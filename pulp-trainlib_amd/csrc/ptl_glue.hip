@@ -18,6 +18,54 @@ static int glue_bad(const char *fn, const char *what) {
 }
 
 // ---- ReLU (lib/sources/pulp_act_fp32.c:95-129) ------------------------------------------------------
+// Element-wise maps c = op(a, b) on 16-byte vectors (tensors that are 16-byte aligned; the last n % VEC elements
+// go one by one).  The one-element-per-thread kernels below remain for unaligned tensors.
+struct OpReluFw {
+    __device__ static float map(float a, float) { return a > 0.f ? a : 0.f; }
+};
+struct OpReluBw {
+    __device__ static float map(float x, float dy) { return x > 0.f ? dy : 0.f; }
+};
+struct OpAdd {
+    __device__ static float map(float a, float b) { return a + b; }
+};
+struct OpCopy {
+    __device__ static float map(float a, float) { return a; }
+};
+
+template <typename T, typename Op, bool TWO>
+__global__ __launch_bounds__(256) void ew_vec_kernel(const T *a, const T *b, T *c, size_t n) {  // c may be a or b
+    constexpr int VEC = 16 / (int)sizeof(T);
+    union V {
+        uint4 raw;
+        T e[VEC];
+    };
+    const size_t nvec = n / VEC, v = (size_t)blockIdx.x * 256 + threadIdx.x;
+    if (v < nvec) {
+        V x, y;
+        x.raw = reinterpret_cast<const uint4 *>(a)[v];
+        if (TWO) y.raw = reinterpret_cast<const uint4 *>(b)[v];
+#pragma unroll
+        for (int q = 0; q < VEC; ++q) x.e[q] = (T)Op::map((float)x.e[q], TWO ? (float)y.e[q] : 0.f);
+        reinterpret_cast<uint4 *>(c)[v] = x.raw;
+    }
+    if (blockIdx.x == 0) {
+        const size_t i = nvec * VEC + threadIdx.x;
+        if (i < n) c[i] = (T)Op::map((float)a[i], TWO ? (float)b[i] : 0.f);
+    }
+}
+
+// Launches the vector form when the tensors allow it; false = the caller launches its element kernel.
+template <typename T, typename Op, bool TWO>
+static bool ew_vec_launch(const T *a, const T *b, T *c, size_t n) {
+    constexpr int VEC = 16 / (int)sizeof(T);
+    auto al = [](const void *p) { return reinterpret_cast<uintptr_t>(p) % 16 == 0; };
+    if (n < (size_t)VEC || !al(a) || !al(c) || (TWO && !al(b))) return false;
+    hipLaunchKernelGGL((ew_vec_kernel<T, Op, TWO>), dim3(glue_blocks((n / VEC))), dim3(256), 0, state().stream, a, b, c,
+                       n);
+    return true;
+}
+
 template <typename T>
 __global__ __launch_bounds__(256) void relu_fw_kernel(const T *__restrict__ x, T *__restrict__ y, size_t n) {
     size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
@@ -42,12 +90,14 @@ static int relu_step(const Args *a, int ns, int step, const char *fn) {
     if (step == 0) {
         T *y = sg.out(reinterpret_cast<T *>(a->output->data), n);
         if (sg.failed() || !x || !y) return sg.failed() ? 2 : glue_bad(fn, "null buffer");
-        hipLaunchKernelGGL((relu_fw_kernel<T>), dim3(glue_blocks(n)), dim3(256), 0, state().stream, x, y, n);
+        if (!ew_vec_launch<T, OpReluFw, false>(x, (const T *)nullptr, y, n))
+            hipLaunchKernelGGL((relu_fw_kernel<T>), dim3(glue_blocks(n)), dim3(256), 0, state().stream, x, y, n);
     } else {
         const T *dy = sg.in(reinterpret_cast<const T *>(a->output->diff), n);
         T *dx = sg.out(reinterpret_cast<T *>(a->input->diff), n);
         if (sg.failed() || !x || !dy || !dx) return sg.failed() ? 2 : glue_bad(fn, "null buffer");
-        hipLaunchKernelGGL((relu_bw_kernel<T>), dim3(glue_blocks(n)), dim3(256), 0, state().stream, x, dy, dx, n);
+        if (!ew_vec_launch<T, OpReluBw, true>(x, dy, dx, n))
+            hipLaunchKernelGGL((relu_bw_kernel<T>), dim3(glue_blocks(n)), dim3(256), 0, state().stream, x, dy, dx, n);
     }
     return sg.finish(hip_ok(hipGetLastError(), "relu launch") ? 0 : 2);
 }
@@ -85,17 +135,20 @@ static int residual_step(const Args *a, int ns, int step, const char *fn) {
         const T *l = sg.in(reinterpret_cast<const T *>(a->lout->data), n);
         T *o = sg.out(reinterpret_cast<T *>(a->output->data), n);
         if (sg.failed() || !s || !l || !o) return sg.failed() ? 2 : glue_bad(fn, "null buffer");
-        hipLaunchKernelGGL((add_kernel<T>), dim3(glue_blocks(n)), dim3(256), 0, state().stream, s, l, o, n);
+        if (!ew_vec_launch<T, OpAdd, true>(s, l, o, n))
+            hipLaunchKernelGGL((add_kernel<T>), dim3(glue_blocks(n)), dim3(256), 0, state().stream, s, l, o, n);
     } else if (step == 1) {
         const T *g = sg.in(reinterpret_cast<const T *>(a->output->diff), n);
         T *s = sg.inout(reinterpret_cast<T *>(a->skip->diff), n);
         if (sg.failed() || !g || !s) return sg.failed() ? 2 : glue_bad(fn, "null buffer");
-        hipLaunchKernelGGL((add_kernel<T>), dim3(glue_blocks(n)), dim3(256), 0, state().stream, g, s, s, n);
+        if (!ew_vec_launch<T, OpAdd, true>(g, (const T *)s, s, n))
+            hipLaunchKernelGGL((add_kernel<T>), dim3(glue_blocks(n)), dim3(256), 0, state().stream, g, s, s, n);
     } else {
         const T *g = sg.in(reinterpret_cast<const T *>(a->output->diff), n);
         T *l = sg.out(reinterpret_cast<T *>(a->lout->diff), n);
         if (sg.failed() || !g || !l) return sg.failed() ? 2 : glue_bad(fn, "null buffer");
-        hipLaunchKernelGGL((copy_elems_kernel<T>), dim3(glue_blocks(n)), dim3(256), 0, state().stream, g, l, n);
+        if (!ew_vec_launch<T, OpCopy, false>(g, (const T *)nullptr, l, n))
+            hipLaunchKernelGGL((copy_elems_kernel<T>), dim3(glue_blocks(n)), dim3(256), 0, state().stream, g, l, n);
     }
     return sg.finish(hip_ok(hipGetLastError(), "residual launch") ? 0 : 2);
 }
