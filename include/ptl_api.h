@@ -298,6 +298,10 @@ int ptl_cross_entropy_fp32_batched(const struct loss_args *a, int nsamples, int 
 int ptl_cross_entropy_fp16_batched(const struct loss_args_fp16 *a, int nsamples, int step);
 int ptl_gradient_descent_fp32(const struct optim_args *a);
 int ptl_gradient_descent_fp16(const struct optim_args_fp16 *a);
+/* No counterpart in the reference: the update of pulp_gradient_descent_* for `count` argument structs in one
+ * launch (a training step updates dozens of small tensors). */
+int ptl_gradient_descent_fp32_multi(const struct optim_args *list, int count);
+int ptl_gradient_descent_fp16_multi(const struct optim_args_fp16 *list, int count);
 int ptl_batch_norm_fp32_fw(const struct BatchNorm_args_fp32 *a);
 /* No counterpart in the reference (its batch normalisation has a forward pass only, in fp32): the backward pass
  * of that forward and both passes in fp16, for a training step that contains the layer.  Backward reads

@@ -67,7 +67,9 @@ BATCHED_ENTRY_POINTS = ["ptl_%s_%s_%s_batched" % (layer, dt, step)
                         for layer in ("conv2d", "conv_pw", "conv_dw", "linear")
                         for dt in ("fp32", "fp16") for step in ("fw", "wg", "ig")] + [
                             "ptl_linear_fp32_bw_batched", "ptl_linear_fp16_bw_batched",
-                            "ptl_mhsa_fp32_fw_batched", "ptl_mhsa_fp32_bw_batched"]
+                            "ptl_mhsa_fp32_fw_batched", "ptl_mhsa_fp32_bw_batched",
+                            # (const optim_args *list, int count)
+                            "ptl_gradient_descent_fp32_multi", "ptl_gradient_descent_fp16_multi"]
 
 OTHER_ENTRY_POINTS = ["ptl_init", "ptl_last_error", "ptl_last_status", "ptl_set_stream", "ptl_sync", "ptl_set_gemm_path",
                       "ptl_last_conv_direct", "ptl_last_gemm_streamed", "ptl_timer_begin", "ptl_timer_end_ms", "ptl_mm_fp32", "ptl_mm_fp16", "ptl_copy_bytes"]

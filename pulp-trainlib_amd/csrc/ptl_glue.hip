@@ -336,6 +336,76 @@ static int sgd_step(const Args *a, const char *fn) {
     return sg.finish(0);
 }
 
+// The same update for a list of parameter tensors in one launch: a training step updates dozens of small
+// tensors, and one launch each is two microseconds each.
+constexpr int SGD_MAXT = 48;
+struct SgdTable {
+    void *w[SGD_MAXT], *g[SGD_MAXT];
+    unsigned n[SGD_MAXT], first[SGD_MAXT + 1];  // elements; first workgroup of tensor t (first[count] = grid)
+    float lr[SGD_MAXT], lambda[SGD_MAXT];
+    int count;
+};
+
+template <typename T>
+__global__ __launch_bounds__(256) void sgd_multi_kernel(const SgdTable t) {
+    int k = 0;
+    while (k + 1 < t.count && blockIdx.x >= t.first[k + 1]) ++k;
+    const size_t i = (size_t)(blockIdx.x - t.first[k]) * 256 + threadIdx.x;
+    if (i >= t.n[k]) return;
+    T *w = reinterpret_cast<T *>(t.w[k]), *g = reinterpret_cast<T *>(t.g[k]);
+    const float lr = t.lr[k], lambda = t.lambda[k];
+    float gi = (float)g[i], wi = (float)w[i];
+    if (lambda != 0.f) {
+        gi = gi + lambda * wi;
+        g[i] = (T)gi;
+        gi = (float)(T)gi;
+    }
+    w[i] = (T)(wi - lr * gi);
+}
+
+template <typename T, typename Args>
+static int sgd_multi(const Args *list, int count, const char *fn) {
+    if (count <= 0) return 0;
+    if (!list) return glue_bad(fn, "invalid arguments");
+    if (!ensure_init()) return 2;
+    Stager sg;
+    SgdTable t;
+    t.count = 0;
+    unsigned blocks = 0;
+    auto flush = [&]() {
+        if (t.count == 0) return true;
+        t.first[t.count] = blocks;
+        hipLaunchKernelGGL((sgd_multi_kernel<T>), dim3(blocks), dim3(256), 0, state().stream, t);
+        t.count = 0;
+        blocks = 0;
+        return hip_ok(hipGetLastError(), "optimizer launch");
+    };
+    for (int i = 0; i < count; ++i) {
+        const Args &a = list[i];
+        if (!a.weights) return glue_bad(fn, "invalid arguments");
+        if (a.use_biases == 1 && !a.biases) return glue_bad(fn, "use_biases=1 with a null bias blob");
+        for (int part = 0; part < 2; ++part) {
+            if (part == 1 && a.use_biases != 1) continue;
+            const auto *b = part == 0 ? a.weights : a.biases;
+            if (b->dim <= 0) continue;
+            if (!b->data || !b->diff) return glue_bad(fn, "null buffer");
+            if (t.count == SGD_MAXT && !flush()) return sg.finish(2);
+            const float lam = (float)a.weight_decay_lambda;
+            t.w[t.count] = sg.inout(reinterpret_cast<T *>(b->data), (size_t)b->dim);
+            t.g[t.count] = lam != 0.f ? sg.inout(reinterpret_cast<T *>(b->diff), (size_t)b->dim)
+                                      : const_cast<T *>(sg.in(reinterpret_cast<const T *>(b->diff), (size_t)b->dim));
+            if (sg.failed()) return 2;
+            t.n[t.count] = (unsigned)b->dim;
+            t.first[t.count] = blocks;
+            t.lr[t.count] = (float)a.learning_rate;
+            t.lambda[t.count] = (float)a.weight_decay_lambda;
+            blocks += glue_blocks((size_t)b->dim);
+            ++t.count;
+        }
+    }
+    return sg.finish(flush() ? 0 : 2);
+}
+
 // ---- Batch normalisation (forward: lib/sources/pulp_batchnorm_fp32.c:34-114) ---------------------------
 // Statistics per channel over B x H x W, in two launches so that a few channels still fill the chip:
 //   1. partial sums per (channel, group of samples): forward x and x^2; backward also dy and dy*x;
@@ -557,6 +627,12 @@ int ptl_gradient_descent_fp32(const struct optim_args *a) {
 }
 int ptl_gradient_descent_fp16(const struct optim_args_fp16 *a) {
     return ptl::sgd_step<ptl::half_t>(a, "pulp_gradient_descent_fp16");
+}
+int ptl_gradient_descent_fp32_multi(const struct optim_args *list, int count) {
+    return ptl::sgd_multi<float>(list, count, "ptl_gradient_descent_fp32_multi");
+}
+int ptl_gradient_descent_fp16_multi(const struct optim_args_fp16 *list, int count) {
+    return ptl::sgd_multi<ptl::half_t>(list, count, "ptl_gradient_descent_fp16_multi");
 }
 int ptl_batch_norm_fp32_fw(const struct BatchNorm_args_fp32 *a) {
     return ptl::batch_norm_step<float>(a, 0, "pulp_batch_norm_fp32_fw_cl");

@@ -147,15 +147,18 @@ class ResNetStep:
         for b in reversed(bw_blocks):
             self.bw += b
         self.bw += first_bw
-        self.opt = []
+        # one update call for all parameter tensors (the per-tensor call of the reference, once per struct)
+        opts = []
         for n in self.W:
             o, kp = hp.optim_args(pkg, dt, self.W[n], self.dW[n], None, None, lr, 0.0)
             self.keep.append(kp)
-            self.opt.append((L("ptl_gradient_descent_DT"), o, ()))
-        for n in self.G:  # scale and shift of a normalisation layer in one update
+            opts.append(o)
+        for n in self.G:  # scale and shift of a normalisation layer share a struct
             o, kp = hp.optim_args(pkg, dt, self.G[n], self.dG[n], self.Bt[n], self.dBt[n], lr, 0.0)
             self.keep.append(kp)
-            self.opt.append((L("ptl_gradient_descent_DT"), o, ()))
+            opts.append(o)
+        table = (type(opts[0]) * len(opts))(*opts)
+        self.opt = [(L("ptl_gradient_descent_DT_multi"), table, (len(opts),))]
 
     def _vect_sum(self, acc, term):
         """acc += term through the reference-named vect_sum entry point (lib/sources/pulp_train_utils_fp32.c:208)."""

@@ -275,3 +275,31 @@ def test_residual_block_training_step(pkg, gpu, dt):
     lr_ = float(npd(lr))
     for Wt, t in ((W1, p[0]), (W2, p[1]), (WL, p[2])):
         assert hp.rel_l2(host(Wt), (t.detach() - lr_ * t.grad).numpy()) <= tol
+
+
+@pytest.mark.parametrize("dt", ["fp32", "fp16"])
+def test_gradient_descent_for_a_list_of_tensors(pkg, gpu, dt):
+    """ptl_gradient_descent_*_multi (one launch for many structs) against the per-struct entry point."""
+    nd = hp.np_dtype(dt)
+    dims = [(5,), (300, 7), (1,), (64, 3, 3, 3), (1000,)] * 13  # 65 structs, 98 tensors: more than one table
+    res = []
+    for multi in (False, True):
+        structs, keep, tensors = [], [], []
+        for i, shp in enumerate(dims):
+            w, g = dev(hp.uniform(0x7F00 + i, shp).astype(nd)), dev(hp.uniform(0x7F80 + i, shp).astype(nd))
+            b = gb = None
+            if i % 2:
+                b, gb = dev(hp.uniform(0x7F40 + i, (shp[0],)).astype(nd)), dev(hp.uniform(0x7FC0 + i, (shp[0],)).astype(nd))
+            o, k = hp.optim_args(pkg, dt, w, g, b, gb, 0.05, 0.01 if i % 3 == 0 else 0.0)
+            structs.append(o), keep.append(k), tensors.append((w, g, b, gb))
+        if multi:
+            table = (type(structs[0]) * len(structs))(*structs)
+            assert getattr(gpu, "ptl_gradient_descent_%s_multi" % dt)(ctypes.byref(table), len(structs)) == 0
+        else:
+            for o in structs:
+                assert getattr(gpu, "ptl_gradient_descent_" + dt)(ctypes.byref(o)) == 0
+        gpu.ptl_sync()
+        res.append([[None if t is None else host(t) for t in ts] for ts in tensors])
+    for one, many in zip(*res):
+        for u, v in zip(one, many):
+            assert (u is None and v is None) or np.array_equal(u, v)

@@ -60,7 +60,7 @@ def test_resnet20_training_step(pkg, gpu, dt, ns, tol):
         assert hp.rel_l2(net.dW[n].cpu().numpy(), ref_grads[n]) <= tol, n
     for n in w:
         assert hp.rel_l2(net.W[n].cpu().numpy(), ref_new[n]) <= tol, n
-    assert net.launches() > 150
+    assert net.launches() > 130
 
 
 @pytest.mark.parametrize("dt,ns,tol", [("fp32", 6, 1e-3), ("fp16", 8, 1.5e-1)])
@@ -91,4 +91,4 @@ def test_resnet20_training_step_with_batch_norm(pkg, gpu, dt, ns, tol):
         assert hp.rel_l2(net.G[n].cpu().numpy(), ref_new["g:" + n]) <= tol, n
     for n in w:
         assert hp.rel_l2(net.W[n].cpu().numpy(), ref_new[n]) <= tol, n
-    assert net.launches() > 200
+    assert net.launches() > 170
