@@ -43,7 +43,7 @@ def main():
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on ONE GPU; --gpus %d is not supported "
-              "(the path shards by sample, see DESIGN.md)" % args.gpus, file=sys.stderr)
+              "(the path shards by sample; no multi-GPU figure is produced)" % args.gpus, file=sys.stderr)
         sys.exit(2)
 
     import torch
