@@ -686,11 +686,12 @@ __global__ __launch_bounds__(RS_NT) void attn_fw_res_kernel(AttnArgs a) {
         const int row = wave * RS_RPW + i;
         float *srow = S + row * RS_SP;
         const bool live = r0 + row < L;
+        const float inv = 1.0f / sum[i];  // one division per row; the products differ from quotients by an ulp at most
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
             const int c = lane + 64 * j;
             if (c < RS_LC) {
-                const float pv = c < L ? sv[i][j] / sum[i] : 0.f;
+                const float pv = c < L ? sv[i][j] * inv : 0.f;
                 srow[c] = pv;
                 if (live && c < L) P[(size_t)(r0 + row) * L + c] = pv;
             }
