@@ -484,7 +484,8 @@ __global__ __launch_bounds__(256) void dw_plane_pairs_kernel(const half_t *__res
 template <typename T, int K>
 __global__ __launch_bounds__(256) void dw_wg_plane_kernel(const T *__restrict__ X, const T *__restrict__ dY,
                                                           float *__restrict__ part, int C, int ns, int per_group,
-                                                          int H, int W, int Ho, int Wo, int pu, int pl, int x_vecs) {
+                                                          int H, int W, int Ho, int Wo, int pu, int pl, int x_vecs,
+                                                          T *__restrict__ direct) {
     extern __shared__ uint4 dw_img[];
     __shared__ float red[4][K * K];
     const int ch = blockIdx.x, grp = blockIdx.y;
@@ -530,8 +531,13 @@ __global__ __launch_bounds__(256) void dw_wg_plane_kernel(const T *__restrict__ 
             if (lane == 0) red[wave][i * K + j] = v;
         }
     __syncthreads();
-    if (tid < K * K)
-        part[((size_t)grp * C + ch) * K * K + tid] = (red[0][tid] + red[1][tid]) + (red[2][tid] + red[3][tid]);
+    if (tid < K * K) {
+        const float sum = (red[0][tid] + red[1][tid]) + (red[2][tid] + red[3][tid]);
+        if (direct)  // a single group of samples: this is the gradient itself
+            direct[(size_t)ch * K * K + tid] = (decltype(direct[0] + direct[0]))sum;
+        else
+            part[((size_t)grp * C + ch) * K * K + tid] = sum;
+    }
 }
 
 // The weight-gradient kernel above for fp16 planes readable as pairs (even row lengths, even left pad, 4-byte
@@ -543,7 +549,7 @@ __global__ __launch_bounds__(256) void dw_wg_plane_pairs_kernel(const half_t *__
                                                                 const half_t *__restrict__ dY,
                                                                 float *__restrict__ part, int C, int ns, int per_group,
                                                                 int H, int W, int Ho, int Wo, int pu, int pl,
-                                                                int x_vecs) {
+                                                                int x_vecs, half_t *__restrict__ direct) {
     constexpr int NP = (8 + K) / 2;
     extern __shared__ uint4 dw_img[];
     __shared__ float red[4][K * K];
@@ -600,8 +606,13 @@ __global__ __launch_bounds__(256) void dw_wg_plane_pairs_kernel(const half_t *__
             if (lane == 0) red[wave][i * K + j] = v;
         }
     __syncthreads();
-    if (tid < K * K)
-        part[((size_t)grp * C + ch) * K * K + tid] = (red[0][tid] + red[1][tid]) + (red[2][tid] + red[3][tid]);
+    if (tid < K * K) {
+        const float sum = (red[0][tid] + red[1][tid]) + (red[2][tid] + red[3][tid]);
+        if (direct)  // a single group of samples: this is the gradient itself
+            direct[(size_t)ch * K * K + tid] = (decltype(direct[0] + direct[0]))sum;
+        else
+            part[((size_t)grp * C + ch) * K * K + tid] = sum;
+    }
 }
 
 template <typename Args>
@@ -680,6 +691,8 @@ static int dw_step(const Args *a, int ns, int step, int sh, int sw, const char *
     const size_t in_img = (size_t)g.H * g.W * sizeof(T) + 32, out_img = (size_t)g.Ho * g.Wo * sizeof(T) + 32;
     const bool plane_path = rows_path && in_img <= 40 * 1024 && out_img <= 40 * 1024 && planes >= 2L * st.num_cu &&
                             planes < ((long)1 << 31) && st.gemm_path != 1;
+    // a single sample: one workgroup per channel produces the weight gradient in one launch
+    const bool wg_single = rows_path && ns == 1 && in_img <= 40 * 1024 && out_img <= 40 * 1024 && st.gemm_path != 1;
     if (step == STEP_FW) {
         const T *X = sg.in(reinterpret_cast<const T *>(a->input->data), in_n);
         const T *Wt = sg.in(reinterpret_cast<const T *>(a->coeff->data), w_n);
@@ -728,7 +741,7 @@ static int dw_step(const Args *a, int ns, int step, int sh, int sw, const char *
         } else {
             hipLaunchKernelGGL((dw_ig_kernel<T>), dim3(nblocks(in_n)), dim3(256), 0, st.stream, dY, Wt, dX, g, in_n);
         }
-    } else if (plane_path) {
+    } else if (plane_path || wg_single) {
         const T *X = sg.in(reinterpret_cast<const T *>(a->input->data), in_n);
         const T *dY = sg.in(reinterpret_cast<const T *>(a->output->diff), out_n);
         T *dW = sg.out(reinterpret_cast<T *>(a->coeff->diff), w_n);
@@ -742,6 +755,7 @@ static int dw_step(const Args *a, int ns, int step, int sh, int sw, const char *
         sgroups = (ns + per_group - 1) / per_group;
         float *part = workspace((size_t)sgroups * g.C * taps * sizeof(float));
         if (!part) return sg.finish(2);
+        T *direct = sgroups == 1 ? dW : nullptr;  // one group: the kernel writes the gradient, no second launch
         const int x_vecs = (int)((in_img + 15) / 16);
         const size_t lds = (size_t)x_vecs * 16 + out_img;
         dim3 grid(g.C, sgroups);
@@ -752,21 +766,22 @@ static int dw_step(const Args *a, int ns, int step, int sh, int sw, const char *
             if (pairs) {
                 if (g.Hk == 3)
                     hipLaunchKernelGGL((dw_wg_plane_pairs_kernel<3>), grid, dim3(256), lds, st.stream, X, dY, part, g.C,
-                                       ns, per_group, g.H, g.W, g.Ho, g.Wo, g.Up, g.Lp, x_vecs);
+                                       ns, per_group, g.H, g.W, g.Ho, g.Wo, g.Up, g.Lp, x_vecs, direct);
                 else
                     hipLaunchKernelGGL((dw_wg_plane_pairs_kernel<5>), grid, dim3(256), lds, st.stream, X, dY, part, g.C,
-                                       ns, per_group, g.H, g.W, g.Ho, g.Wo, g.Up, g.Lp, x_vecs);
+                                       ns, per_group, g.H, g.W, g.Ho, g.Wo, g.Up, g.Lp, x_vecs, direct);
             }
         }
         if (pairs) {
         } else if (g.Hk == 3)
             hipLaunchKernelGGL((dw_wg_plane_kernel<T, 3>), grid, dim3(256), lds, st.stream, X, dY, part, g.C, ns,
-                               per_group, g.H, g.W, g.Ho, g.Wo, g.Up, g.Lp, x_vecs);
+                               per_group, g.H, g.W, g.Ho, g.Wo, g.Up, g.Lp, x_vecs, direct);
         else
             hipLaunchKernelGGL((dw_wg_plane_kernel<T, 5>), grid, dim3(256), lds, st.stream, X, dY, part, g.C, ns,
-                               per_group, g.H, g.W, g.Ho, g.Wo, g.Up, g.Lp, x_vecs);
-        hipLaunchKernelGGL((dw_wg_reduce_kernel2<T>), dim3(g.C), dim3(256), 0, st.stream, part, dW, sgroups, g.C, 1,
-                           taps);
+                               per_group, g.H, g.W, g.Ho, g.Wo, g.Up, g.Lp, x_vecs, direct);
+        if (!direct)
+            hipLaunchKernelGGL((dw_wg_reduce_kernel2<T>), dim3(g.C), dim3(256), 0, st.stream, part, dW, sgroups, g.C, 1,
+                               taps);
     } else if (rows_path) {
         const T *X = sg.in(reinterpret_cast<const T *>(a->input->data), in_n);
         const T *dY = sg.in(reinterpret_cast<const T *>(a->output->diff), out_n);
