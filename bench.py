@@ -261,6 +261,18 @@ def detail_table(pkg, lib, hp, to_dev, timed, check, torch, dev):
         nb = (n * n + 2 * ns * n) * es[dt]
         run3("ptl_linear", dt, a, ns, "linear 1024x1024", flops, (nb, nb, nb), 200 if ns <= 512 else 20)
 
+    # the same GEMM kernels on large plain products (the mm entry point): how far the tiles carry once launch and
+    # first-trip latencies are amortised
+    for dt, (N, M, K) in (("fp16", (4096, 4096, 4096)), ("fp32", (4096, 4096, 2048))):
+        A = (torch.randn(N, K, device=dev) / 8).to(tdt[dt])
+        Bm = (torch.randn(M, K, device=dev) / 8).to(tdt[dt])
+        Cm = torch.zeros(N, M, device=dev, dtype=tdt[dt])
+        f = lib.ptl_mm_fp16 if dt == "fp16" else lib.ptl_mm_fp32
+        margs = [ctypes.c_void_p(A.data_ptr()), ctypes.c_void_p(Bm.data_ptr()), ctypes.c_void_p(Cm.data_ptr()), N, M, K, 1]
+        ms = timed(lambda: check(f(*margs)), 10)
+        add("mm %dx%dx%d (B transposed)" % (N, M, K), dt, ms, 2.0 * N * M * K, (N * K + M * K + N * M) * es[dt])
+        del A, Bm, Cm
+
     # config 3: depthwise 3x3 on 64x56x56 (pre-padded 58x58) and pointwise 64->128, fp16, batch 1 and 64
     for ns in (1, 64):
         dt = "fp16"
