@@ -93,20 +93,35 @@ int gemm_async(GemmArgs &g) {
         if (!g.ws) return 2;
     }
     if (plain_operand<T>(g.a, g.kchunk, g.K) && plain_operand<T>(g.b, g.kchunk, g.K)) {
-        // few rows, a shallow contraction and many columns: resident A panel, streamed column tiles
-        if (g.splits == 1 && g.taps <= 1 && g.K % SK == 0 && g.K <= 4 * SK && (g.N == 64 || g.N % 128 == 0) &&
-            g.N <= 256 && g.M % 64 == 0 && (long)(g.M / 64) * ((g.N + 127) / 128) >= 4L * st.num_cu) {
-            const int ks = g.K / SK;
+        // few rows (or few columns: then the product is computed transposed, which changes nothing about its
+        // sums), a shallow contraction and a long other side: resident panel, streamed tiles
+        auto streams = [&](int few, int many) {
+            return (few == 64 || few % 128 == 0) && few <= 256 && many % 64 == 0 &&
+                   (long)(many / 64) * ((few + 127) / 128) >= 4L * st.num_cu;
+        };
+        if (g.splits == 1 && g.taps <= 1 && g.K % SK == 0 && g.K <= 4 * SK && (streams(g.N, g.M) || streams(g.M, g.N))) {
+            GemmArgs gs = g;
+            if (!streams(g.N, g.M)) {
+                gs.A = g.B;
+                gs.B = g.A;
+                gs.a = g.b;
+                gs.b = g.a;
+                gs.N = g.M;
+                gs.M = g.N;
+                gs.c.n = g.c.m;
+                gs.c.m = g.c.n;
+            }
+            const int ks = gs.K / SK;
             int rc = -1;
-            if (g.N == 64)
-                rc = ks == 1   ? launch_stream<T, 64, 64, 1>(g, st.num_cu, st.stream)
-                     : ks == 2 ? launch_stream<T, 64, 64, 2>(g, st.num_cu, st.stream)
-                     : ks == 4 ? launch_stream<T, 64, 64, 4>(g, st.num_cu, st.stream)
+            if (gs.N == 64)
+                rc = ks == 1   ? launch_stream<T, 64, 64, 1>(gs, st.num_cu, st.stream)
+                     : ks == 2 ? launch_stream<T, 64, 64, 2>(gs, st.num_cu, st.stream)
+                     : ks == 4 ? launch_stream<T, 64, 64, 4>(gs, st.num_cu, st.stream)
                                : -1;
             else
-                rc = ks == 1   ? launch_stream<T, 128, 64, 1>(g, st.num_cu, st.stream)
-                     : ks == 2 ? launch_stream<T, 128, 64, 2>(g, st.num_cu, st.stream)
-                     : ks == 4 ? launch_stream<T, 128, 64, 4>(g, st.num_cu, st.stream)
+                rc = ks == 1   ? launch_stream<T, 128, 64, 1>(gs, st.num_cu, st.stream)
+                     : ks == 2 ? launch_stream<T, 128, 64, 2>(gs, st.num_cu, st.stream)
+                     : ks == 4 ? launch_stream<T, 128, 64, 4>(gs, st.num_cu, st.stream)
                                : -1;
             if (rc == 0) st.last_gemm_streamed = 1;
             if (rc != -1) return rc;

@@ -358,16 +358,22 @@ def test_pointwise(pkg, orc, gpu, dt, hwc, Ci, Co, H, W, ns):
 # Batches large enough for the streaming kernel (row panel resident, column tiles streamed): one or two row
 # tiles, contraction depths of one, two and four slabs over the two data types and the two steps.
 @pytest.mark.parametrize("dt", ["fp32", "fp16"])
+@pytest.mark.parametrize("hwc", [0, 1])
 @pytest.mark.parametrize("Ci,Co,H,W,ns", [(64, 128, 32, 32, 64), (128, 64, 32, 32, 64), (64, 256, 16, 16, 256)])
-def test_pointwise_streamed_column_tiles(pkg, orc, gpu, dt, Ci, Co, H, W, ns):
-    pw_parity(pkg, orc, gpu, dt, Ci, Co, H, W, 0, ns, 0xC0DE0043)
-    x, w = dev(hp.uniform(1, (ns, Ci, H * W), dtype=hp.np_dtype(dt))), dev(hp.uniform(2, (Co, Ci), dtype=hp.np_dtype(dt)))
-    y = torch.zeros((ns, Co, H * W), dtype=x.dtype, device=x.device)
-    g, keep = hp.pw_args(pkg, x, None, w, None, y, None, Ci, Co, H, W, 0)
+def test_pointwise_streamed_column_tiles(pkg, orc, gpu, dt, hwc, Ci, Co, H, W, ns):
+    """Channel-major layers stream pixel columns past a resident weight panel; pixel-major (HWC) layers are the
+    same product transposed, stored four channels at a time."""
+    pw_parity(pkg, orc, gpu, dt, Ci, Co, H, W, hwc, ns, 0xC0DE0043)
+    nd = hp.np_dtype(dt)
+    x = dev(hp.uniform(1, (ns, H * W, Ci) if hwc else (ns, Ci, H * W), dtype=nd))
+    w = dev(hp.uniform(2, (Ci, Co) if (hwc and dt == "fp32") else (Co, Ci), dtype=nd))
+    y = torch.zeros((ns, H * W, Co) if hwc else (ns, Co, H * W), dtype=x.dtype, device=x.device)
+    g, keep = hp.pw_args(pkg, x, None, w, None, y, None, Ci, Co, H, W, hwc)
     pkg.call("ptl_conv_pw_%s_fw_batched" % dt, g, ns)
     sync(gpu)
     assert gpu.ptl_last_gemm_streamed() == 1
-    ref = torch.matmul(w.double(), x.double())
+    wm = w.double().t() if (hwc and dt == "fp32") else w.double()  # [Co][Ci]
+    ref = torch.matmul(x.double(), wm.t()) if hwc else torch.matmul(wm, x.double())
     assert float((y.double() - ref).norm() / ref.norm()) <= TOL[dt]
 
 
