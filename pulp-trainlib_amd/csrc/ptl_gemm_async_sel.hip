@@ -53,7 +53,10 @@ int gemm_async(GemmArgs &g) {
     long nt = cfg == 0 ? tiles(128, 128) : cfg == 1 ? tiles(64, 64) : cfg == 2 ? tiles(32, 128) : tiles(128, 32);
     // at most 64 columns and many rows (64 filters over a batch of pixels), or k in runs: a 128x64 tile halves
     // the reads of the narrow operand against 64x64 (+27 % measured on 64 -> 64 channels, 56x56, batch 128)
-    const bool tall = cfg == 1 && g.N >= 128 && g.M > 32 && (runs || tiles(128, 64) >= 2L * st.num_cu);
+    // a long stream of k into a small output: bound by memory in fp16 (fewer, taller workgroups stream as fast
+    // and leave fewer partial sums), by the MFMAs in fp32 (every CU needs its workgroup)
+    const bool long_k = sizeof(T) == 2 && (runs || g.K >= 512 * SK);
+    const bool tall = cfg == 1 && g.N >= 128 && g.M > 32 && (long_k || tiles(128, 64) >= 2L * st.num_cu);
     if (tall) nt = tiles(128, 64);
 
     g.splits = 1;
@@ -62,7 +65,7 @@ int gemm_async(GemmArgs &g) {
     if (nt * 4 <= st.num_cu) want = (int)((st.num_cu + nt - 1) / nt);
     // a long stream of k is bound by memory, not by the number of workgroups: half as many splits stream
     // as fast and leave half as many partial sums to add
-    if (runs && want > 1) want = (want + 1) / 2;
+    if (long_k && want > 1) want = (want + 1) / 2;
     // Operands that are not on the look-up-free path index k through a table of ASYNC_KWMAX entries.
     const bool need_lut = !(plain_operand<T>(g.a, g.kchunk, g.K) && plain_operand<T>(g.b, g.kchunk, g.K));
     int need = need_lut ? (g.K + ASYNC_KWMAX - 1) / ASYNC_KWMAX : 1;
