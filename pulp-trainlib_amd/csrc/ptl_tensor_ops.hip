@@ -316,7 +316,7 @@ __device__ inline const T *dw_load_plane(const T *__restrict__ plane, int elems,
     const int shift = (int)(a0 & 15) / (int)sizeof(T);
     const uint4 *base = reinterpret_cast<const uint4 *>(a0 & ~(uintptr_t)15);
     const int nvec = (shift + elems + VEC - 1) / VEC;
-    for (int v = tid; v < nvec; v += 256) img[v] = base[v];
+    for (int v = tid; v < nvec; v += (int)blockDim.x) img[v] = base[v];
     return reinterpret_cast<const T *>(img) + shift;
 }
 
@@ -434,10 +434,14 @@ __device__ inline void dw_row_taps(const unsigned (&P)[(8 + K) / 2], const dw_h2
     }
 }
 
-template <int K, bool FLIP>
-__global__ __launch_bounds__(256) void dw_plane_pairs_kernel(const half_t *__restrict__ src,
+// One workgroup (two waves) per plane; a thread produces a block of RB rows x 8 columns: an input row segment is
+// read from LDS once and feeds the (up to K) output rows it belongs to, and the index arithmetic is paid once per
+// block instead of once per eight outputs.
+template <int K, bool FLIP, int RB = 4, int NT = 128>
+__global__ __launch_bounds__(NT) void dw_plane_pairs_kernel(const half_t *__restrict__ src,
                                                              const half_t *__restrict__ Wt, half_t *__restrict__ dst,
                                                              int C, int Hs, int Ws, int Hd, int Wd, int pu, int pl) {
+    constexpr int NP = (8 + K) / 2;
     extern __shared__ uint4 dw_img[];
     const size_t plane = blockIdx.x;
     const int ch = (int)(plane % C), tid = threadIdx.x;
@@ -459,22 +463,29 @@ __global__ __launch_bounds__(256) void dw_plane_pairs_kernel(const half_t *__res
         }
     }
     __syncthreads();
-    const int groups = (Wd + 7) >> 3;
+    const int groups = (Wd + 7) >> 3, rblocks = (Hd + RB - 1) / RB;
     half_t *dp = dst + plane * Hd * Wd;
-    for (int item = tid; item < Hd * groups; item += 256) {
-        const int r = item / groups, c0 = (item - r * groups) * 8;
-        float acc[8];
+    for (int item = tid; item < rblocks * groups; item += NT) {
+        const int rb = item / groups, c0 = (item - rb * groups) * 8, r0 = rb * RB;
+        float acc[RB][8];
 #pragma unroll
-        for (int q = 0; q < 8; ++q) acc[q] = 0.f;
+        for (int r = 0; r < RB; ++r)
 #pragma unroll
-        for (int i = 0; i < K; ++i) {
-            const int h = r + i - pu;
+            for (int q = 0; q < 8; ++q) acc[r][q] = 0.f;
+#pragma unroll
+        for (int hr = 0; hr < RB + K - 1; ++hr) {  // source row r0 - pu + hr feeds output rows r0 + hr - i, i < K
+            const int h = r0 + hr - pu;
             if ((unsigned)h >= (unsigned)Hs) continue;
-            unsigned P[(8 + K) / 2];
-            dw_row_pairs<(8 + K) / 2>(img, h, Ws, c0 - pl, P);
-            dw_row_taps<K>(P, we[i], wo[i], wf[i], acc);
+            unsigned P[NP];
+            dw_row_pairs<NP>(img, h, Ws, c0 - pl, P);
+#pragma unroll
+            for (int i = 0; i < K; ++i)
+                if (hr - i >= 0 && hr - i < RB) dw_row_taps<K>(P, we[i], wo[i], wf[i], acc[hr - i]);
         }
-        dw_store8<half_t>(dp + (size_t)r * Wd + c0, acc, min(8, Wd - c0));
+        const int valid = min(8, Wd - c0);
+#pragma unroll
+        for (int r = 0; r < RB; ++r)
+            if (r0 + r < Hd) dw_store8<half_t>(dp + (size_t)(r0 + r) * Wd + c0, acc[r], valid);
     }
 }
 
@@ -662,7 +673,7 @@ static void launch_dw_plane(const T *src, const T *Wt, T *dst, int C, int Hs, in
     if constexpr (sizeof(T) == 2) {
         // rows readable as pairs: see dw_plane_pairs_kernel
         if (Ws % 2 == 0 && pl % 2 == 0 && reinterpret_cast<uintptr_t>(src) % 4 == 0) {
-            hipLaunchKernelGGL((dw_plane_pairs_kernel<K, FLIP>), dim3((unsigned)planes), dim3(256), src_img, stream, src,
+            hipLaunchKernelGGL((dw_plane_pairs_kernel<K, FLIP>), dim3((unsigned)planes), dim3(128), src_img, stream, src,
                                Wt, dst, C, Hs, Ws, Hd, Wd, pu, pl);
             return;
         }
