@@ -561,7 +561,7 @@ __global__ __launch_bounds__(256) void dw_wg_plane_pairs_kernel(const half_t *__
                                                                 float *__restrict__ part, int C, int ns, int per_group,
                                                                 int H, int W, int Ho, int Wo, int pu, int pl,
                                                                 int x_vecs, half_t *__restrict__ direct) {
-    constexpr int NP = (8 + K) / 2;
+    constexpr int NP = (8 + K) / 2, RB = 2;
     extern __shared__ uint4 dw_img[];
     __shared__ float red[4][K * K];
     const int ch = blockIdx.x, grp = blockIdx.y;
@@ -571,7 +571,7 @@ __global__ __launch_bounds__(256) void dw_wg_plane_pairs_kernel(const half_t *__
     for (int i = 0; i < K; ++i)
 #pragma unroll
         for (int j = 0; j < K; ++j) acc[i][j] = 0.f;
-    const int groups = (Wo + 7) >> 3;
+    const int groups = (Wo + 7) >> 3, rblocks = (Ho + RB - 1) / RB;
     const int b_end = min(ns, (grp + 1) * per_group);
     for (int b = grp * per_group; b < b_end; ++b) {
         const size_t plane = (size_t)b * C + ch;
@@ -579,30 +579,38 @@ __global__ __launch_bounds__(256) void dw_wg_plane_pairs_kernel(const half_t *__
         const half_t *ximg = dw_load_plane<half_t>(X + plane * H * W, H * W, dw_img, tid);
         const half_t *gimg = dw_load_plane<half_t>(dY + plane * Ho * Wo, Ho * Wo, dw_img + x_vecs, tid);
         __syncthreads();
-        for (int item = tid; item < Ho * groups; item += 256) {
-            const int r = item / groups, c0 = (item - r * groups) * 8;
-            dw_h2 G[4];
-            {
-                const unsigned *grow = reinterpret_cast<const unsigned *>(gimg + r * Wo + c0);
+        // a thread takes blocks of RB output rows x 8 columns: a source row is read (and its odd-offset pairs made)
+        // once for the up to K gradient rows it meets
+        for (int item = tid; item < rblocks * groups; item += 256) {
+            const int rb = item / groups, c0 = (item - rb * groups) * 8, r0 = rb * RB;
+            dw_h2 G[RB][4];
 #pragma unroll
-                for (int m = 0; m < 4; ++m) G[m] = __builtin_bit_cast(dw_h2, c0 + 2 * m < Wo ? grow[m] : 0u);
+            for (int r = 0; r < RB; ++r) {
+                const unsigned *grow = reinterpret_cast<const unsigned *>(gimg + (r0 + r) * Wo + c0);
+#pragma unroll
+                for (int m = 0; m < 4; ++m)
+                    G[r][m] = __builtin_bit_cast(dw_h2, (r0 + r < Ho && c0 + 2 * m < Wo) ? grow[m] : 0u);
             }
 #pragma unroll
-            for (int i = 0; i < K; ++i) {
-                const int h = r + i - pu;
+            for (int hr = 0; hr < RB + K - 1; ++hr) {  // source row r0 - pu + hr meets gradient rows r0 + hr - i
+                const int h = r0 + hr - pu;
                 if ((unsigned)h >= (unsigned)H) continue;
-                unsigned P[NP];
+                unsigned P[NP], U[NP - 1];
                 dw_row_pairs<NP>(ximg, h, W, c0 - pl, P);
 #pragma unroll
-                for (int j = 0; j < K; ++j) {
-                    float a = acc[i][j];
+                for (int m = 0; m < NP - 1; ++m) U[m] = __builtin_amdgcn_alignbit(P[m + 1], P[m], 16);
 #pragma unroll
-                    for (int m = 0; m < 4; ++m) {
-                        const unsigned x2 = (j & 1) ? __builtin_amdgcn_alignbit(P[m + j / 2 + 1], P[m + j / 2], 16)
-                                                    : P[m + j / 2];
-                        a = __builtin_amdgcn_fdot2(__builtin_bit_cast(dw_h2, x2), G[m], a, false);
+                for (int i = 0; i < K; ++i) {
+                    if (hr - i < 0 || hr - i >= RB) continue;
+#pragma unroll
+                    for (int j = 0; j < K; ++j) {
+                        float a = acc[i][j];
+#pragma unroll
+                        for (int m = 0; m < 4; ++m)
+                            a = __builtin_amdgcn_fdot2(__builtin_bit_cast(dw_h2, (j & 1) ? U[m + j / 2] : P[m + j / 2]),
+                                                       G[hr - i][m], a, false);
+                        acc[i][j] = a;
                     }
-                    acc[i][j] = a;
                 }
             }
         }
