@@ -2,18 +2,23 @@
 //
 // dW[co][ci][tap] = sum over pixels of dY[co][pixel] * X[ci][pixel shifted by tap]: a GEMM whose
 // contraction runs over pixels.  A workgroup owns up to 64 output channels and a slab of CT
-// input channels, walks pixel tiles of 128 (persistent, accumulators stay in registers) and
-// per tile
+// input channels, walks pixel tiles (persistent, accumulators stay in registers) - a tile is
+// R whole output rows of one sample, R the most that stays within 128 pixels, so that the
+// input rows it needs are R + KH - 1 rows of the same sample - and per tile
 //   * copies the dY rows of its output channels into LDS ([co][pixel], 16-byte loads);
-//   * copies the input rows the tile touches into LDS as [ci][row][col] with a zero halo,
-//     16 bytes at a time (the halo makes the destination 2-byte aligned only; LDS takes
-//     unaligned 16-byte stores and loads).  Both copies are register-staged prefetches: the
-//     loads of tile t+1 are issued before tile t is computed and parked in the other of two
-//     LDS buffers afterwards, one barrier per tile;
-//   * feeds the MFMAs: the dY fragment of a lane is one aligned ds_read_b128 (8 pixels of one
-//     output channel), the input fragment one unaligned ds_read_b128 at
-//     coloff(ci, tap) + pixoff(pixel group) -- 8 consecutive pixels of a row shifted by the
-//     tap.  This needs unit column stride and rows whose length is a multiple of the vector.
+//   * copies the input rows the tile touches into LDS as [ci][row][col] with a zero halo.
+//     A thread loads 16 bytes of a row plus the two elements on either side and writes the
+//     chunk once per filter column kx, shifted by kx elements, into a copy of the tile of its
+//     own: every 16-byte store and every fragment load below is then 16-byte aligned (a
+//     misaligned ds_read_b128 runs at a fraction of the aligned rate; measured 2.4x on the MFMA
+//     loop).  When the copies do not fit there is one copy, stored behind the left halo with
+//     unaligned 16-byte stores, and the fragment loads are unaligned.  Both copies are register-staged prefetches: the loads of tile t+1 are issued
+//     before tile t is computed and parked in the other of two LDS buffers afterwards, one
+//     barrier per tile;
+//   * feeds the MFMAs: the dY fragment of a lane is one ds_read_b128 (8 pixels of one output
+//     channel), the input fragment one ds_read_b128 at coloff(ci, tap) + pixoff(pixel group)
+//     -- 8 consecutive pixels of a row shifted by the tap.  This needs unit column stride and
+//     rows whose length is a multiple of the vector.
 // The eight waves split the column blocks (ci, tap) four ways and the pixel groups two ways.
 // Each workgroup leaves one fp32 partial of its dW block; a second kernel adds the partials.
 #include "ptl_gemm_async.hpp"
@@ -32,25 +37,67 @@ struct ConvWgArgs {
     float *ws;  // [parts][Cout][Cin * taps]
     ConvTileDesc d;
     int CT;       // input channels per workgroup
-    int THP, TW, RR, PLANE;
-    int tiles;    // pixel tiles of 128
-    int N;        // pixels
+    int TW, RR, PLANE;  // row pitch, rows and channel pitch of the input tile (elements; pitches multiples of the vector)
+    int TWraw;    // input row with its halo (elements)
+    int copies;   // copies of the input tile: KW (copy kx is shifted by kx elements) or 1
+    int COPY;     // elements per copy
+    int wchunks;  // 16-byte chunks of an input row
+    int R;        // output rows per tile
+    int tpi;      // tiles per sample
+    int tiles;    // tiles of all samples
+    int ksteps;   // MFMA steps that cover the R * Wo pixels of a tile
     int pitch_a;  // bytes per dY row in LDS
-    int a_bytes;  // LDS bytes of the dY tile (the raw tile follows)
+    int a_bytes;  // LDS bytes of the dY tile (the input tile follows)
     int raw_bytes;
     int cblocks;  // 32-wide column blocks of (ci, tap) per workgroup
-    int xg;       // 16-byte groups per input row
-    unsigned magic_xg, magic_rr, magic_taps, magic_kw, magic_thp;
+    int xg;       // 16-byte chunks per row of the input tile
+    unsigned magic_xg, magic_rr, magic_taps, magic_kw, magic_tpi, magic_wo;
 };
 
-template <typename T, int RB, int CBW>
+// Two elements as a pair of dwords (fp16: one dword, the second unused).
+template <typename T>
+__device__ inline uint2 load_two(const T *p) {
+    if constexpr (sizeof(T) == 2) return make_uint2(*reinterpret_cast<const unsigned *>(p), 0u);
+    else return *reinterpret_cast<const uint2 *>(p);
+}
+
+// The 16 bytes that start `shift` elements (-2..2) after the chunk `cur`, given the two elements before
+// and after it.
+template <typename T>
+__device__ inline uint4 shifted_chunk(const uint2 &before, const uint4 &cur, const uint2 &after, int shift) {
+    if constexpr (sizeof(T) == 2) {
+        const unsigned w0 = before.x, w1 = cur.x, w2 = cur.y, w3 = cur.z, w4 = cur.w, w5 = after.x;
+        switch (shift) {
+            case -2: return make_uint4(w0, w1, w2, w3);
+            case -1:
+                return make_uint4(__builtin_amdgcn_alignbit(w1, w0, 16), __builtin_amdgcn_alignbit(w2, w1, 16),
+                                  __builtin_amdgcn_alignbit(w3, w2, 16), __builtin_amdgcn_alignbit(w4, w3, 16));
+            case 1:
+                return make_uint4(__builtin_amdgcn_alignbit(w2, w1, 16), __builtin_amdgcn_alignbit(w3, w2, 16),
+                                  __builtin_amdgcn_alignbit(w4, w3, 16), __builtin_amdgcn_alignbit(w5, w4, 16));
+            case 2: return make_uint4(w2, w3, w4, w5);
+            default: return cur;
+        }
+    } else {
+        switch (shift) {
+            case -2: return make_uint4(before.x, before.y, cur.x, cur.y);
+            case -1: return make_uint4(before.y, cur.x, cur.y, cur.z);
+            case 1: return make_uint4(cur.y, cur.z, cur.w, after.x);
+            case 2: return make_uint4(cur.z, cur.w, after.x, after.y);
+            default: return cur;
+        }
+    }
+}
+
+// SHIFTED: one copy of the input tile per filter column (a.copies > 1).
+template <typename T, int RB, int CBW, bool SHIFTED>
 __global__ __launch_bounds__(512) void conv_wg_kernel(const ConvWgArgs a) {
-    constexpr int NT = 512, KT = 128;
-    constexpr int ES = (int)sizeof(T), VEC = 16 / ES, KSTEP = 2 * VEC, KSTEPS = KT / KSTEP, GROUPS = KT / VEC;
+    constexpr int NT = 512, KT = 128, MAX_COPIES = 5;
+    constexpr int ES = (int)sizeof(T), VEC = 16 / ES, KSTEP = 2 * VEC, GROUPS = KT / VEC;
     extern __shared__ __attribute__((aligned(16))) char smem[];
-    // two buffers, each: dY tile [32*RB][pitch_a] followed by the input tile [CT][RR][TW]
+    // two buffers, each: dY tile [32*RB][pitch_a] followed by the copies of the input tile [copy][CT][RR][TW]
     const int buf_bytes = a.a_bytes + a.raw_bytes;
-    __shared__ int pixoff[2][GROUPS];  // per pixel group: raw offset of its first pixel
+    __shared__ int pixoff[GROUPS];  // per pixel group: offset of its first pixel in the input tile (the same in every tile)
 
     const ConvTileDesc &d = a.d;
     const int tid = threadIdx.x, lane = tid & 63;
@@ -63,7 +110,7 @@ __global__ __launch_bounds__(512) void conv_wg_kernel(const ConvWgArgs a) {
     const T *__restrict__ X = reinterpret_cast<const T *>(a.X);
     const T *__restrict__ dY = reinterpret_cast<const T *>(a.dY);
 
-    // this lane's column in each of its blocks: offset of (ci, tap) inside the raw tile
+    // this lane's column in each of its blocks: offset of (ci, tap) inside the input tile
     int coloff[CBW];
 #pragma unroll
     for (int jj = 0; jj < CBW; ++jj) {
@@ -71,7 +118,7 @@ __global__ __launch_bounds__(512) void conv_wg_kernel(const ConvWgArgs a) {
         if (m >= cols) m = cols - 1;  // surplus columns repeat the last one; never stored
         const int ci = fast_div(m, a.magic_taps), tap = m - ci * taps;
         const int ky = fast_div(tap, a.magic_kw), kx = tap - ky * d.KW;
-        coloff[jj] = ci * a.PLANE + ky * a.TW + kx;
+        coloff[jj] = ci * a.PLANE + ky * a.TW + (SHIFTED ? kx * a.COPY : kx);
     }
 
     f32x16 acc[RB][CBW];
@@ -82,95 +129,122 @@ __global__ __launch_bounds__(512) void conv_wg_kernel(const ConvWgArgs a) {
 #pragma unroll
             for (int v = 0; v < 16; ++v) acc[r][jj][v] = 0.f;
 
-    // Both input tiles start as zeros: the halo columns are never written again, everything
-    // else is rewritten for every tile (rows outside the image and channels beyond the tensor
-    // as zeros).
+    // Both input tiles start as zeros: the padding between rows and channels is never written again,
+    // everything else is rewritten for every tile (rows outside the image, columns of the halo and
+    // channels beyond the tensor as zeros).
     for (int b = 0; b < 2; ++b)
         for (int c = tid; c < a.raw_bytes / 16; c += NT)
             reinterpret_cast<uint4 *>(smem + b * buf_bytes + a.a_bytes)[c] = make_uint4(0, 0, 0, 0);
+    if (tid < GROUPS) {
+        // groups past the tile's pixels (their dY is zero) read the start of the tile
+        const int p = tid * VEC < a.R * d.Wo ? tid * VEC : 0;
+        const int y = fast_div(p, a.magic_wo);
+        pixoff[tid] = y * d.sh * a.TW + (p - y * d.Wo);
+    }
     __syncthreads();
 
     // Register-staged prefetch: the global loads of tile t+1 are issued before tile t is
     // computed and stored to the other LDS buffer afterwards; one barrier per tile.
+    // What a thread copies is the same piece of every tile - the chunk (row, pixel group) of
+    // the dY tile, the unit (ci, tile row, chunk) of the input tile - so its decoding is
+    // done once here; per tile only the sample and the first row change.
     constexpr int A_CHUNKS = 32 * RB * (KT / VEC);
     constexpr int A_PER = (A_CHUNKS + NT - 1) / NT;  // dY chunks per thread
-    const int units = a.CT * a.RR * a.xg;            // (ci, raw row, group of VEC columns)
+    const int units = a.CT * a.RR * a.xg;            // (ci, tile row, chunk of VEC columns)
     constexpr int U_MAX = 4;                         // input units per thread the registers hold (host checks)
     uint4 regA[A_PER], regU[U_MAX];
+    uint2 regP[SHIFTED ? U_MAX : 1], regN[SHIFTED ? U_MAX : 1];  // the two elements before and after the chunk
+    int a_lds[A_PER], a_pix[A_PER];  // LDS byte offset (-1: no chunk), first pixel inside the tile
+    long long a_row[A_PER];          // element offset of the output channel's plane (-1: beyond the tensor)
+    int u_lds[U_MAX], u_rr[U_MAX];   // LDS element offset (-1: no unit), tile row
+    int u_has[U_MAX];                // 1: the chunk lies inside the row, 2: the elements before it, 4: those after it
+    long long u_src[U_MAX];          // element offset of (channel, chunk) (-1: beyond the tensor)
+#pragma unroll
+    for (int i = 0; i < A_PER; ++i) {
+        const int c = tid + i * NT;
+        const int row = c / (KT / VEC), g = c % (KT / VEC);
+        a_lds[i] = c < A_CHUNKS ? row * a.pitch_a + g * 16 : -1;
+        a_pix[i] = g * VEC;
+        a_row[i] = (c < A_CHUNKS && r0 + row < d.Cout) ? (long long)(r0 + row) * PP + g * VEC : -1;
+    }
+#pragma unroll
+    for (int i = 0; i < U_MAX; ++i) {
+        const int u = tid + i * NT;
+        const int row = fast_div(u, a.magic_xg), xg = u - row * a.xg;
+        const int ci = fast_div(row, a.magic_rr), rr = row - ci * a.RR;
+        u_lds[i] = u < units ? ci * a.PLANE + rr * a.TW + xg * VEC : -1;
+        u_rr[i] = rr;
+        u_has[i] = (xg < a.wchunks ? 1 : 0) | (xg >= 1 && xg <= a.wchunks ? 2 : 0) | (xg + 1 < a.wchunks ? 4 : 0);
+        if (!SHIFTED) {  // the chunks of the row go behind the left halo as they are
+            u_has[i] &= 1;
+            u_lds[i] = (u < units && xg < a.wchunks) ? u_lds[i] + d.padL : -1;
+        }
+        u_src[i] = (u < units && c0 + ci < d.Cin) ? (long long)(c0 + ci) * d.x_sc + xg * VEC : -1;
+    }
 
     auto fetch = [&](int tile) {
-        const int n0 = tile * KT;
-        const int b0 = n0 / PP, pix0 = n0 - b0 * PP, y0 = pix0 / d.Wo;
-        const int t0 = y0 * d.sh;
+        const int b0 = fast_div(tile, a.magic_tpi), y0 = (tile - b0 * a.tpi) * a.R;
+        const int rows = d.Ho - y0 < a.R ? d.Ho - y0 : a.R;  // the last tile of a sample may be short
+        const int npx = rows * d.Wo, raw_rows = (rows - 1) * d.sh + d.KH, t0 = y0 * d.sh - d.padU;
+        const T *gy = dY + (long long)b0 * d.Cout * PP + (long long)y0 * d.Wo;
+        const T *gx = X + (long long)b0 * d.x_sb;
 #pragma unroll
         for (int i = 0; i < A_PER; ++i) {
-            const int c = tid + i * NT;
-            const int row = c / (KT / VEC), g = c % (KT / VEC);
-            int q = pix0 + g * VEC, b = b0;
-            while (q >= PP) {
-                q -= PP;
-                ++b;
-            }
             regA[i] = make_uint4(0, 0, 0, 0);
-            if (c < A_CHUNKS && n0 + g * VEC < a.N && r0 + row < d.Cout)
-                regA[i] = *reinterpret_cast<const uint4 *>(dY + ((long long)b * d.Cout + r0 + row) * PP + q);
+            if (a_row[i] >= 0 && a_pix[i] < npx) regA[i] = *reinterpret_cast<const uint4 *>(gy + a_row[i]);
         }
 #pragma unroll
         for (int i = 0; i < U_MAX; ++i) {
-            const int u = tid + i * NT;
             regU[i] = make_uint4(0, 0, 0, 0);
-            if (u < units) {
-                const int row = fast_div(u, a.magic_xg), xg = u - row * a.xg;
-                const int ci = fast_div(row, a.magic_rr), rr = row - ci * a.RR;
-                const int t = t0 + rr, db = fast_div(t, a.magic_thp);
-                const int b = b0 + db, iy = t - db * a.THP - d.padU;
-                if (b < d.batch && iy >= 0 && iy < d.Hin && c0 + ci < d.Cin)
-                    regU[i] = *reinterpret_cast<const uint4 *>(X + (long long)b * d.x_sb + (long long)(c0 + ci) * d.x_sc +
-                                                               (long long)iy * d.x_sy + xg * VEC);
+            if constexpr (SHIFTED) regP[i] = regN[i] = make_uint2(0, 0);
+            const int iy = t0 + u_rr[i];
+            if (u_src[i] >= 0 && u_rr[i] < raw_rows && iy >= 0 && iy < d.Hin) {
+                const T *src = gx + u_src[i] + (long long)iy * d.x_sy;
+                if (u_has[i] & 1) regU[i] = *reinterpret_cast<const uint4 *>(src);
+                if constexpr (SHIFTED) {
+                    if (u_has[i] & 2) regP[i] = load_two<T>(src - 2);
+                    if (u_has[i] & 4) regN[i] = load_two<T>(src + VEC);
+                }
             }
         }
     };
-    auto park = [&](int tile, int buf) {
+    auto park = [&](int buf) {
         char *at = smem + buf * buf_bytes;
         T *raw = reinterpret_cast<T *>(at + a.a_bytes);
 #pragma unroll
-        for (int i = 0; i < A_PER; ++i) {
-            const int c = tid + i * NT;
-            if (c < A_CHUNKS) *reinterpret_cast<uint4 *>(at + (c / (KT / VEC)) * a.pitch_a + (c % (KT / VEC)) * 16) = regA[i];
-        }
+        for (int i = 0; i < A_PER; ++i)
+            if (a_lds[i] >= 0) *reinterpret_cast<uint4 *>(at + a_lds[i]) = regA[i];
+        if constexpr (!SHIFTED) {
 #pragma unroll
-        for (int i = 0; i < U_MAX; ++i) {
-            const int u = tid + i * NT;
-            if (u < units) {
-                const int row = fast_div(u, a.magic_xg), xg = u - row * a.xg;
-                const int ci = fast_div(row, a.magic_rr), rr = row - ci * a.RR;
-                u4raw w = {regU[i].x, regU[i].y, regU[i].z, regU[i].w};
-                *reinterpret_cast<u4_unaligned *>(raw + ci * a.PLANE + rr * a.TW + d.padL + xg * VEC) = w;
+            for (int i = 0; i < U_MAX; ++i)
+                if (u_lds[i] >= 0) {
+                    u4raw w = {regU[i].x, regU[i].y, regU[i].z, regU[i].w};
+                    *reinterpret_cast<u4_unaligned *>(raw + u_lds[i]) = w;
+                }
+        } else {
+#pragma unroll
+            for (int s = 0; s < MAX_COPIES; ++s) {
+                if (s >= a.copies) break;
+                // copy s, position i holds input column i + s - padL
+#pragma unroll
+                for (int i = 0; i < U_MAX; ++i)
+                    if (u_lds[i] >= 0)
+                        *reinterpret_cast<uint4 *>(raw + s * a.COPY + u_lds[i]) =
+                            shifted_chunk<T>(regP[i], regU[i], regN[i], s - d.padL);
             }
-        }
-        if (tid < GROUPS) {
-            const int n0 = tile * KT;
-            const int b0 = n0 / PP, y0 = (n0 - b0 * PP) / d.Wo;
-            const int g0 = b0 * a.THP + y0 * d.sh;
-            int p = n0 + tid * VEC, off = 0;
-            if (p < a.N) {
-                const int b = p / PP, rem = p - b * PP, y = rem / d.Wo, x = rem - y * d.Wo;
-                off = (b * a.THP + y * d.sh - g0) * a.TW + x;
-            }
-            pixoff[buf][tid] = off;
         }
     };
 
     int buf = 0;
     if ((int)blockIdx.x < a.tiles) fetch(blockIdx.x);
     for (int tile = blockIdx.x; tile < a.tiles; tile += gridDim.x, buf ^= 1) {
-        park(tile, buf);
+        park(buf);
         __syncthreads();  // tile parked; every wave is done with the tile before the previous one (same buffer)
         if (tile + (int)gridDim.x < a.tiles) fetch(tile + gridDim.x);
         const char *at = smem + buf * buf_bytes;
         const T *raw = reinterpret_cast<const T *>(at + a.a_bytes);
-        for (int ks = wk; ks < KSTEPS; ks += 2) {
-            const int po = pixoff[buf][ks * 2 + kg];
+        for (int ks = wk; ks < a.ksteps; ks += 2) {
+            const int po = pixoff[ks * 2 + kg];
             uint4 af[RB];
 #pragma unroll
             for (int r = 0; r < RB; ++r)
@@ -187,26 +261,24 @@ __global__ __launch_bounds__(512) void conv_wg_kernel(const ConvWgArgs a) {
     }
     __syncthreads();
 
-    // the two pixel-group halves meet in LDS, then one fp32 partial per workgroup
+    // the two pixel-group halves meet in LDS (one block of 32 output channels at a time, so that the
+    // exchange fits the space of the tiles), then one fp32 partial per workgroup
     float *red = reinterpret_cast<float *>(smem);
-    constexpr int PER = RB * CBW * 16;
-    if (wk == 1) {
-        float *dst = red + (size_t)wc * PER * 64 + lane;
+    constexpr int PER = CBW * 16;
+    const int Kw = d.Cin * taps;
+    const int valid_cols = (d.Cin - c0 < a.CT ? d.Cin - c0 : a.CT) * taps;
+    float *__restrict__ out = a.ws + (size_t)blockIdx.x * d.Cout * Kw + (size_t)c0 * taps;
 #pragma unroll
-        for (int r = 0; r < RB; ++r)
+    for (int r = 0; r < RB; ++r) {
+        float *mine = red + (size_t)wc * PER * 64 + lane;
+        if (wk == 1) {
 #pragma unroll
             for (int jj = 0; jj < CBW; ++jj)
 #pragma unroll
-                for (int v = 0; v < 16; ++v) dst[((r * CBW + jj) * 16 + v) * 64] = acc[r][jj][v];
-    }
-    __syncthreads();
-    if (wk == 0) {
-        const float *src = red + (size_t)wc * PER * 64 + lane;
-        const int Kw = d.Cin * taps;
-        const int valid_cols = (d.Cin - c0 < a.CT ? d.Cin - c0 : a.CT) * taps;
-        float *__restrict__ out = a.ws + (size_t)blockIdx.x * d.Cout * Kw + (size_t)c0 * taps;
-#pragma unroll
-        for (int r = 0; r < RB; ++r)
+                for (int v = 0; v < 16; ++v) mine[(jj * 16 + v) * 64] = acc[r][jj][v];
+        }
+        __syncthreads();
+        if (wk == 0) {
 #pragma unroll
             for (int jj = 0; jj < CBW; ++jj) {
                 const int m = (wc + 4 * jj) * 32 + lr;
@@ -214,9 +286,11 @@ __global__ __launch_bounds__(512) void conv_wg_kernel(const ConvWgArgs a) {
 #pragma unroll
                 for (int v = 0; v < 16; ++v) {
                     const int co = r0 + r * 32 + 8 * (v >> 2) + 4 * kg + (v & 3);
-                    if (co < d.Cout) out[(size_t)co * Kw + m] = acc[r][jj][v] + src[((r * CBW + jj) * 16 + v) * 64];
+                    if (co < d.Cout) out[(size_t)co * Kw + m] = acc[r][jj][v] + mine[(jj * 16 + v) * 64];
                 }
             }
+        }
+        if (r + 1 < RB) __syncthreads();
     }
 }
 
@@ -254,25 +328,42 @@ __global__ __launch_bounds__(1024) void conv_wg_reduce_kernel(const float *__res
 template <typename T, int RB, int CBW>
 static int launch_conv_wg(ConvWgArgs &a, int gy, int gz, void *dW, hipStream_t s) {
     constexpr int ES = (int)sizeof(T), VEC = 16 / ES;
-    auto kern = conv_wg_kernel<T, RB, CBW>;
     a.pitch_a = 128 * ES + 16;
     a.a_bytes = 32 * RB * a.pitch_a;
-    a.raw_bytes = (int)((((size_t)a.CT * a.PLANE * ES + 32) + 15) & ~(size_t)15);  // slack: a fragment may start at the last element
-    const size_t red = (size_t)4 * RB * CBW * 16 * 64 * 4;
+    const size_t red = (size_t)4 * CBW * 16 * 64 * 4;  // exchange of one 32-channel block between the wave pairs
+    // (fp16; an fp32 fragment feeds four MFMAs and the extra registers would cost a workgroup per CU)
+    // one shifted copy of the input tile per filter column when the chunk shifts are within the two elements
+    // a thread holds on either side and both buffers fit (pitches in whole chunks, one odd chunk per channel to
+    // spread the channels over the LDS banks); else one copy with the pitches of the data and unaligned
+    // fragment loads
+    const int KW = a.d.KW, first = -a.d.padL, last = KW - 1 - a.d.padL;
+    size_t lds = 0;
+    for (a.copies = (ES == 2 && KW > 1 && KW <= 5 && first >= -2 && last <= 2) ? KW : 1;; a.copies = 1) {
+        a.TW = a.copies > 1 ? (a.TWraw + VEC - 1) / VEC * VEC : a.TWraw;
+        a.PLANE = a.RR * a.TW + (a.copies > 1 ? VEC : 0);
+        a.COPY = a.CT * a.PLANE;
+        a.xg = a.copies > 1 ? a.TW / VEC : a.wchunks;
+        // slack: an unaligned fragment may start at the last element
+        a.raw_bytes = (int)((((size_t)a.copies * a.COPY * ES + 32) + 15) & ~(size_t)15);
+        lds = 2 * ((size_t)a.a_bytes + a.raw_bytes);
+        if (lds <= 150 * 1024 || a.copies == 1) break;
+    }
+    a.magic_xg = magic_of(a.xg);
     if ((long)a.CT * a.RR * a.xg > 4L * 512) return -1;  // input units per thread that the prefetch registers hold
-    size_t lds = 2 * ((size_t)a.a_bytes + a.raw_bytes);
     if (lds < red) lds = red;
     if (lds > 150 * 1024) return -1;
-    static bool attr_set = false;
-    if (!attr_set) {
+    constexpr bool CAN_SHIFT = ES == 2;
+    auto kern = (CAN_SHIFT && a.copies > 1) ? conv_wg_kernel<T, RB, CBW, CAN_SHIFT> : conv_wg_kernel<T, RB, CBW, false>;
+    static bool attr_set[2] = {false, false};
+    if (!attr_set[a.copies > 1]) {
         if (!hip_ok(hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
                                         hipFuncAttributeMaxDynamicSharedMemorySize, 150 * 1024),
                     "hipFuncSetAttribute"))
             return 2;
-        attr_set = true;
+        attr_set[a.copies > 1] = true;
     }
-    // two workgroups per CU over the whole grid, each walking an equal share of the pixel tiles
-    long parts = 2L * state().num_cu / ((long)gy * gz);
+    // as many workgroups as the CUs hold at once over the whole grid, each walking an equal share of the pixel tiles
+    long parts = (lds <= 80 * 1024 ? 2L : 1L) * state().num_cu / ((long)gy * gz);
     if (parts < 1) parts = 1;
     if (parts > a.tiles) parts = a.tiles;
     const int per = (int)((a.tiles + parts - 1) / parts);
@@ -297,34 +388,36 @@ int conv_tile_wg(const ConvTileDesc &d, const void *X, const void *dY, void *dW)
     a.X = X;
     a.dY = dY;
     a.d = d;
-    a.N = d.batch * d.Ho * d.Wo;
-    a.THP = d.Hin + d.padU + d.padD;
-    a.TW = d.Win + d.padL + d.padR;
+    const int THP = d.Hin + d.padU + d.padD, TWraw = d.Win + d.padL + d.padR;
     if (d.padU < 0 || d.padD < 0 || d.padL < 0 || d.padR < 0) return -1;
-    if ((d.Ho - 1) * d.sh + d.KH > a.THP || (d.Wo - 1) * d.sw + d.KW > a.TW) return -1;
+    if ((d.Ho - 1) * d.sh + d.KH > THP || (d.Wo - 1) * d.sw + d.KW > TWraw) return -1;
     // 8 (4) consecutive pixels of a fragment must be 8 consecutive input columns of one row,
     // and input rows must be copyable 16 bytes at a time
     if (d.sw != 1 || d.Wo % VEC || d.Win % VEC || d.x_sy % VEC || d.x_sc % VEC || d.x_sb % VEC) return -1;
     if (reinterpret_cast<uintptr_t>(X) % 16 || reinterpret_cast<uintptr_t>(dY) % 16) return -1;
-    a.tiles = (a.N + 127) / 128;
+    if (d.Wo > 128) return -1;  // a tile is whole output rows within 128 pixels
+    a.R = 128 / d.Wo < d.Ho ? 128 / d.Wo : d.Ho;
+    a.tpi = (d.Ho + a.R - 1) / a.R;
+    if ((long long)d.batch * a.tpi * a.tpi >= ((long long)1 << 32)) return -1;  // range of the reciprocal division
+    a.tiles = d.batch * a.tpi;
+    a.ksteps = (a.R * d.Wo + 2 * VEC - 1) / (2 * VEC);
     // few pixel tiles: worth it only for small fp16 weight tensors (measured 8.6 against 11.2 us for one
     // 16->32 channel 32x32 sample, 14 against 9.5 us for eight 64->64 8x8 ones)
     if (st.gemm_path != 2 && a.tiles < st.num_cu && !(ES == 2 && (long)d.Cout * d.Cin * d.KH * d.KW <= 8192)) return -1;
 
     const int taps = d.KH * d.KW;
-    a.RR = conv_raw_rows(128, d.Ho, d.Wo, d.sh, d.KH, a.THP, a.N);
+    a.TWraw = TWraw;
+    a.RR = (a.R - 1) * d.sh + d.KH;
     if (a.RR > 64) return -1;
-    a.PLANE = a.RR * a.TW;
     a.CT = d.Cin <= 16 ? 16 : 32;
-    a.xg = d.Win / VEC;
-    if ((long)a.CT * a.RR * a.xg >= 65536 || (long)a.CT * taps >= 65536) return -1;
+    a.wchunks = d.Win / VEC;
+    if ((long)a.CT * a.RR * (TWraw / VEC + 1) >= 65536 || (long)a.CT * taps >= 65536) return -1;
     a.cblocks = (a.CT * taps + 31) / 32;
-    a.magic_xg = magic_of(a.xg);
     a.magic_rr = magic_of(a.RR);
     a.magic_taps = magic_of(taps);
     a.magic_kw = magic_of(d.KW);
-    a.magic_thp = magic_of(a.THP);
-    if (a.THP + a.RR >= 65536) return -1;
+    a.magic_tpi = magic_of(a.tpi);
+    a.magic_wo = magic_of(d.Wo);
     const int gy = (d.Cin + a.CT - 1) / a.CT;
     const int cbw = (a.cblocks + 3) / 4;  // column blocks per wave
     if (cbw > 3) return -1;

@@ -339,8 +339,10 @@ static int conv2d_wg(const Args *a, int ns, const char *fn) {
         d.KH = g.Hk; d.KW = g.Wk; d.sh = g.sh; d.sw = g.sw;
         d.padU = g.Up; d.padD = g.Dp; d.padL = g.Lp; d.padR = g.Rp;
         d.x_sb = (long long)g.Ci * g.H * g.W; d.x_sc = (long long)g.H * g.W; d.x_sy = g.W;
-        rc = conv_taps_wg<T>(d, X, dY, dW);
+        // the resident-tile kernel where rows are whole 16-byte chunks, else (or on request) the sum over taps
+        if (state().gemm_path == 3) rc = conv_taps_wg<T>(d, X, dY, dW);
         if (rc < 0) rc = conv_tile_wg<T>(d, X, dY, dW);
+        if (rc < 0 && state().gemm_path != 3) rc = conv_taps_wg<T>(d, X, dY, dW);
         if (rc > 0) return sg.finish(rc);
         if (rc == 0) state().last_conv_direct = 1;
     }

@@ -250,6 +250,10 @@ DIRECT_WG_CASES = [
     (12, 12, 24, 70, 5, 3, (1, 1, 2, 2), (1, 1), 2),    # 15 taps
     (8, 10, 8, 9, 1, 1, (0, 0, 0, 0), (1, 1), 5),       # single tap
     (3, 9, 40, 4, 3, 5, (2, 2, 0, 2), (1, 1), 2),       # pads on three sides, 5 columns of taps
+    (4, 3, 128, 6, 3, 3, (1, 1, 1, 1), (1, 1), 2),      # one output row per tile
+    (9, 8, 16, 5, 3, 3, (2, 0, 1, 1), (1, 1), 3),       # all the column padding on the left
+    (9, 8, 16, 5, 3, 3, (0, 2, 1, 1), (1, 1), 3),       # ... on the right
+    (40, 8, 8, 33, 3, 3, (1, 1, 1, 1), (1, 1), 5),      # a tile is a whole sample
 ]
 
 
