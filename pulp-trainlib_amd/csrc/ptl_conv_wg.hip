@@ -89,8 +89,9 @@ __device__ inline uint4 shifted_chunk(const uint2 &before, const uint4 &cur, con
     }
 }
 
-// SHIFTED: one copy of the input tile per filter column (a.copies > 1).
-template <typename T, int RB, int CBW, bool SHIFTED>
+// SHIFTED: one copy of the input tile per filter column (a.copies > 1); 2: three filter columns with one column of
+// left padding, the shifts -1, 0, 1 known to the compiler.
+template <typename T, int RB, int CBW, int SHIFTED>
 __global__ __launch_bounds__(512) void conv_wg_kernel(const ConvWgArgs a) {
     constexpr int NT = 512, KT = 128, MAX_COPIES = 5;
     constexpr int ES = (int)sizeof(T), VEC = 16 / ES, KSTEP = 2 * VEC, GROUPS = KT / VEC;
@@ -154,52 +155,61 @@ __global__ __launch_bounds__(512) void conv_wg_kernel(const ConvWgArgs a) {
     constexpr int U_MAX = 4;                         // input units per thread the registers hold (host checks)
     uint4 regA[A_PER], regU[U_MAX];
     uint2 regP[SHIFTED ? U_MAX : 1], regN[SHIFTED ? U_MAX : 1];  // the two elements before and after the chunk
+    // Offsets are 32-bit (the host checks that one sample fits) on top of a base that is the same for
+    // the whole workgroup, so that the loads take the scalar-base form without 64-bit address sums.
     int a_lds[A_PER], a_pix[A_PER];  // LDS byte offset (-1: no chunk), first pixel inside the tile
-    long long a_row[A_PER];          // element offset of the output channel's plane (-1: beyond the tensor)
-    int u_lds[U_MAX], u_rr[U_MAX];   // LDS element offset (-1: no unit), tile row
-    int u_has[U_MAX];                // 1: the chunk lies inside the row, 2: the elements before it, 4: those after it
-    long long u_src[U_MAX];          // element offset of (channel, chunk) (-1: beyond the tensor)
+    unsigned a_row[A_PER];           // element offset of (output channel, pixel group) inside the sample
+    bool a_ok[A_PER];
+    int u_lds[U_MAX], u_rr[U_MAX];   // LDS byte offset (-1: no unit), tile row
+    int u_has[U_MAX];                // 1: the chunk lies inside the row, 2: the elements before it, 4: those after it;
+                                     // 0: channel beyond the tensor
+    unsigned u_src[U_MAX];           // element offset of (channel, tile row, chunk) from the tile's first row
+    const int uslots = (units + NT - 1) / NT;
 #pragma unroll
     for (int i = 0; i < A_PER; ++i) {
         const int c = tid + i * NT;
         const int row = c / (KT / VEC), g = c % (KT / VEC);
         a_lds[i] = c < A_CHUNKS ? row * a.pitch_a + g * 16 : -1;
         a_pix[i] = g * VEC;
-        a_row[i] = (c < A_CHUNKS && r0 + row < d.Cout) ? (long long)(r0 + row) * PP + g * VEC : -1;
+        a_ok[i] = c < A_CHUNKS && r0 + row < d.Cout;
+        a_row[i] = a_ok[i] ? (unsigned)((r0 + row) * PP + g * VEC) : 0u;
     }
 #pragma unroll
     for (int i = 0; i < U_MAX; ++i) {
         const int u = tid + i * NT;
         const int row = fast_div(u, a.magic_xg), xg = u - row * a.xg;
         const int ci = fast_div(row, a.magic_rr), rr = row - ci * a.RR;
-        u_lds[i] = u < units ? ci * a.PLANE + rr * a.TW + xg * VEC : -1;
+        u_lds[i] = u < units ? (ci * a.PLANE + rr * a.TW + xg * VEC) * ES : -1;
         u_rr[i] = rr;
         u_has[i] = (xg < a.wchunks ? 1 : 0) | (xg >= 1 && xg <= a.wchunks ? 2 : 0) | (xg + 1 < a.wchunks ? 4 : 0);
         if (!SHIFTED) {  // the chunks of the row go behind the left halo as they are
             u_has[i] &= 1;
-            u_lds[i] = (u < units && xg < a.wchunks) ? u_lds[i] + d.padL : -1;
+            u_lds[i] = (u < units && xg < a.wchunks) ? u_lds[i] + d.padL * ES : -1;
         }
-        u_src[i] = (u < units && c0 + ci < d.Cin) ? (long long)(c0 + ci) * d.x_sc + xg * VEC : -1;
+        if (u >= units || c0 + ci >= d.Cin) u_has[i] = 0;
+        u_src[i] = u_has[i] ? (unsigned)((c0 + ci) * (int)d.x_sc + rr * (int)d.x_sy + xg * VEC) : 0u;
     }
 
     auto fetch = [&](int tile) {
         const int b0 = fast_div(tile, a.magic_tpi), y0 = (tile - b0 * a.tpi) * a.R;
         const int rows = d.Ho - y0 < a.R ? d.Ho - y0 : a.R;  // the last tile of a sample may be short
         const int npx = rows * d.Wo, raw_rows = (rows - 1) * d.sh + d.KH, t0 = y0 * d.sh - d.padU;
+        // tile rows [lo, hi) lie inside the image and are needed by the tile's pixels
+        const int lo = t0 < 0 ? -t0 : 0, hi = d.Hin - t0 < raw_rows ? d.Hin - t0 : raw_rows;
         const T *gy = dY + (long long)b0 * d.Cout * PP + (long long)y0 * d.Wo;
-        const T *gx = X + (long long)b0 * d.x_sb;
+        const T *gx = X + (long long)b0 * d.x_sb + (long long)t0 * d.x_sy;  // dereferenced for rows of the image only
 #pragma unroll
         for (int i = 0; i < A_PER; ++i) {
             regA[i] = make_uint4(0, 0, 0, 0);
-            if (a_row[i] >= 0 && a_pix[i] < npx) regA[i] = *reinterpret_cast<const uint4 *>(gy + a_row[i]);
+            if (a_ok[i] && a_pix[i] < npx) regA[i] = *reinterpret_cast<const uint4 *>(gy + a_row[i]);
         }
 #pragma unroll
         for (int i = 0; i < U_MAX; ++i) {
+            if (i >= uslots) break;
             regU[i] = make_uint4(0, 0, 0, 0);
             if constexpr (SHIFTED) regP[i] = regN[i] = make_uint2(0, 0);
-            const int iy = t0 + u_rr[i];
-            if (u_src[i] >= 0 && u_rr[i] < raw_rows && iy >= 0 && iy < d.Hin) {
-                const T *src = gx + u_src[i] + (long long)iy * d.x_sy;
+            if (u_has[i] && u_rr[i] >= lo && u_rr[i] < hi) {
+                const T *src = gx + u_src[i];
                 if (u_has[i] & 1) regU[i] = *reinterpret_cast<const uint4 *>(src);
                 if constexpr (SHIFTED) {
                     if (u_has[i] & 2) regP[i] = load_two<T>(src - 2);
@@ -210,27 +220,31 @@ __global__ __launch_bounds__(512) void conv_wg_kernel(const ConvWgArgs a) {
     };
     auto park = [&](int buf) {
         char *at = smem + buf * buf_bytes;
-        T *raw = reinterpret_cast<T *>(at + a.a_bytes);
+        char *raw = at + a.a_bytes;
 #pragma unroll
         for (int i = 0; i < A_PER; ++i)
             if (a_lds[i] >= 0) *reinterpret_cast<uint4 *>(at + a_lds[i]) = regA[i];
         if constexpr (!SHIFTED) {
 #pragma unroll
-            for (int i = 0; i < U_MAX; ++i)
+            for (int i = 0; i < U_MAX; ++i) {
+                if (i >= uslots) break;
                 if (u_lds[i] >= 0) {
                     u4raw w = {regU[i].x, regU[i].y, regU[i].z, regU[i].w};
                     *reinterpret_cast<u4_unaligned *>(raw + u_lds[i]) = w;
                 }
+            }
         } else {
 #pragma unroll
-            for (int s = 0; s < MAX_COPIES; ++s) {
-                if (s >= a.copies) break;
+            for (int s = 0; s < (SHIFTED == 2 ? 3 : MAX_COPIES); ++s) {
+                if (SHIFTED != 2 && s >= a.copies) break;
                 // copy s, position i holds input column i + s - padL
 #pragma unroll
-                for (int i = 0; i < U_MAX; ++i)
+                for (int i = 0; i < U_MAX; ++i) {
+                    if (i >= uslots) break;
                     if (u_lds[i] >= 0)
-                        *reinterpret_cast<uint4 *>(raw + s * a.COPY + u_lds[i]) =
-                            shifted_chunk<T>(regP[i], regU[i], regN[i], s - d.padL);
+                        *reinterpret_cast<uint4 *>(raw + s * a.COPY * ES + u_lds[i]) =
+                            shifted_chunk<T>(regP[i], regU[i], regN[i], SHIFTED == 2 ? s - 1 : s - d.padL);
+                }
             }
         }
     };
@@ -353,17 +367,23 @@ static int launch_conv_wg(ConvWgArgs &a, int gy, int gz, void *dW, hipStream_t s
     if (lds < red) lds = red;
     if (lds > 150 * 1024) return -1;
     constexpr bool CAN_SHIFT = ES == 2;
-    auto kern = (CAN_SHIFT && a.copies > 1) ? conv_wg_kernel<T, RB, CBW, CAN_SHIFT> : conv_wg_kernel<T, RB, CBW, false>;
-    static bool attr_set[2] = {false, false};
-    if (!attr_set[a.copies > 1]) {
+    const int mode = !(CAN_SHIFT && a.copies > 1) ? 0 : (KW == 3 && a.d.padL == 1) ? 2 : 1;
+    auto kern = mode == 2   ? conv_wg_kernel<T, RB, CBW, CAN_SHIFT ? 2 : 0>
+                : mode == 1 ? conv_wg_kernel<T, RB, CBW, CAN_SHIFT ? 1 : 0>
+                            : conv_wg_kernel<T, RB, CBW, 0>;
+    static bool attr_set[3] = {false, false, false};
+    if (!attr_set[mode]) {
         if (!hip_ok(hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
                                         hipFuncAttributeMaxDynamicSharedMemorySize, 150 * 1024),
                     "hipFuncSetAttribute"))
             return 2;
-        attr_set[a.copies > 1] = true;
+        attr_set[mode] = true;
     }
     // as many workgroups as the CUs hold at once over the whole grid, each walking an equal share of the pixel tiles
     long parts = (lds <= 80 * 1024 ? 2L : 1L) * state().num_cu / ((long)gy * gz);
+    // (fp16 with under four tiles per workgroup: half as many partial sums to write and add pay more than the
+    // second workgroup per CU; measured 14.5 against 16.7 us for 16 -> 32 channels, 32x32, batch 128)
+    if (ES == 2 && parts > 1 && a.tiles < 4 * parts) parts = (parts + 1) / 2;
     if (parts < 1) parts = 1;
     if (parts > a.tiles) parts = a.tiles;
     const int per = (int)((a.tiles + parts - 1) / parts);
@@ -396,6 +416,10 @@ int conv_tile_wg(const ConvTileDesc &d, const void *X, const void *dY, void *dW)
     if (d.sw != 1 || d.Wo % VEC || d.Win % VEC || d.x_sy % VEC || d.x_sc % VEC || d.x_sb % VEC) return -1;
     if (reinterpret_cast<uintptr_t>(X) % 16 || reinterpret_cast<uintptr_t>(dY) % 16) return -1;
     if (d.Wo > 128) return -1;  // a tile is whole output rows within 128 pixels
+    // offsets inside one sample are 32-bit
+    if ((long long)d.Cin * d.x_sc + (long long)(d.Hin + d.KH) * d.x_sy >= ((long long)1 << 31) ||
+        (long long)d.Cout * d.Ho * d.Wo >= ((long long)1 << 31) || d.x_sc >= ((long long)1 << 31))
+        return -1;
     a.R = 128 / d.Wo < d.Ho ? 128 / d.Wo : d.Ho;
     a.tpi = (d.Ho + a.R - 1) / a.R;
     if ((long long)d.batch * a.tpi * a.tpi >= ((long long)1 << 32)) return -1;  // range of the reciprocal division
