@@ -41,7 +41,9 @@ struct ConvWgArgs {
     int TWraw;    // input row with its halo (elements)
     int copies;   // copies of the input tile: KW (copy kx is shifted by kx elements) or 1
     int COPY;     // elements per copy
-    int wchunks;  // 16-byte chunks of an input row
+    int wchunks;  // whole 16-byte chunks of an input row
+    int Wp;       // pixels a tile holds per output row: Wo rounded up to the vector
+    int ragged;   // rows are not whole 16-byte chunks (4-byte aligned loads, short last chunk)
     int R;        // output rows per tile
     int tpi;      // tiles per sample
     int tiles;    // tiles of all samples
@@ -51,7 +53,7 @@ struct ConvWgArgs {
     int raw_bytes;
     int cblocks;  // 32-wide column blocks of (ci, tap) per workgroup
     int xg;       // 16-byte chunks per row of the input tile
-    unsigned magic_xg, magic_rr, magic_taps, magic_kw, magic_tpi, magic_wo;
+    unsigned magic_xg, magic_rr, magic_taps, magic_kw, magic_tpi, magic_wp;
 };
 
 // Two elements as a pair of dwords (fp16: one dword, the second unused).
@@ -59,6 +61,20 @@ template <typename T>
 __device__ inline uint2 load_two(const T *p) {
     if constexpr (sizeof(T) == 2) return make_uint2(*reinterpret_cast<const unsigned *>(p), 0u);
     else return *reinterpret_cast<const uint2 *>(p);
+}
+
+// The first `n` (2, 4, 6 or 8) fp16 elements at a 4-byte aligned address, the rest zero.
+__device__ inline uint4 load_upto8(const half_t *p, int n) {
+    if (n == 8) {
+        const u4raw w = *reinterpret_cast<const u4raw __attribute__((aligned(4))) *>(p);
+        return make_uint4(w.x, w.y, w.z, w.w);
+    }
+    const unsigned *q = reinterpret_cast<const unsigned *>(p);
+    uint4 v = make_uint4(0, 0, 0, 0);
+    if (n >= 2) v.x = q[0];
+    if (n >= 4) v.y = q[1];
+    if (n >= 6) v.z = q[2];
+    return v;
 }
 
 // The 16 bytes that start `shift` elements (-2..2) after the chunk `cur`, given the two elements before
@@ -90,11 +106,13 @@ __device__ inline uint4 shifted_chunk(const uint2 &before, const uint4 &cur, con
 }
 
 // SHIFTED: one copy of the input tile per filter column (a.copies > 1); 2: three filter columns with one column of
-// left padding, the shifts -1, 0, 1 known to the compiler.
+// left padding, the shifts -1, 0, 1 known to the compiler; 3: the same for rows that are not whole 16-byte chunks
+// (fp16, even row lengths: a tile holds every output row padded to whole chunks, the pad pixels with zero dY).
 template <typename T, int RB, int CBW, int SHIFTED>
 __global__ __launch_bounds__(512) void conv_wg_kernel(const ConvWgArgs a) {
     constexpr int NT = 512, KT = 128, MAX_COPIES = 5;
     constexpr int ES = (int)sizeof(T), VEC = 16 / ES, KSTEP = 2 * VEC, GROUPS = KT / VEC;
+    constexpr bool RAGGED = SHIFTED == 3, FIXED3 = SHIFTED >= 2;
     extern __shared__ __attribute__((aligned(16))) char smem[];
     // two buffers, each: dY tile [32*RB][pitch_a] followed by the copies of the input tile [copy][CT][RR][TW]
     const int buf_bytes = a.a_bytes + a.raw_bytes;
@@ -138,9 +156,9 @@ __global__ __launch_bounds__(512) void conv_wg_kernel(const ConvWgArgs a) {
             reinterpret_cast<uint4 *>(smem + b * buf_bytes + a.a_bytes)[c] = make_uint4(0, 0, 0, 0);
     if (tid < GROUPS) {
         // groups past the tile's pixels (their dY is zero) read the start of the tile
-        const int p = tid * VEC < a.R * d.Wo ? tid * VEC : 0;
-        const int y = fast_div(p, a.magic_wo);
-        pixoff[tid] = y * d.sh * a.TW + (p - y * d.Wo);
+        const int p = tid * VEC < a.R * a.Wp ? tid * VEC : 0;
+        const int y = fast_div(p, a.magic_wp);
+        pixoff[tid] = y * d.sh * a.TW + (p - y * a.Wp);
     }
     __syncthreads();
 
@@ -157,22 +175,26 @@ __global__ __launch_bounds__(512) void conv_wg_kernel(const ConvWgArgs a) {
     uint2 regP[SHIFTED ? U_MAX : 1], regN[SHIFTED ? U_MAX : 1];  // the two elements before and after the chunk
     // Offsets are 32-bit (the host checks that one sample fits) on top of a base that is the same for
     // the whole workgroup, so that the loads take the scalar-base form without 64-bit address sums.
-    int a_lds[A_PER], a_pix[A_PER];  // LDS byte offset (-1: no chunk), first pixel inside the tile
+    int a_lds[A_PER], a_y[A_PER];    // LDS byte offset (-1: no chunk), output row inside the tile
+    int a_n[RAGGED ? A_PER : 1];     // elements of the chunk that lie inside the row
     unsigned a_row[A_PER];           // element offset of (output channel, pixel group) inside the sample
     bool a_ok[A_PER];
     int u_lds[U_MAX], u_rr[U_MAX];   // LDS byte offset (-1: no unit), tile row
     int u_has[U_MAX];                // 1: the chunk lies inside the row, 2: the elements before it, 4: those after it;
                                      // 0: channel beyond the tensor
     unsigned u_src[U_MAX];           // element offset of (channel, tile row, chunk) from the tile's first row
+    int u_n[RAGGED ? U_MAX : 1];     // elements of the chunk that lie inside the row
     const int uslots = (units + NT - 1) / NT;
 #pragma unroll
     for (int i = 0; i < A_PER; ++i) {
         const int c = tid + i * NT;
         const int row = c / (KT / VEC), g = c % (KT / VEC);
         a_lds[i] = c < A_CHUNKS ? row * a.pitch_a + g * 16 : -1;
-        a_pix[i] = g * VEC;
-        a_ok[i] = c < A_CHUNKS && r0 + row < d.Cout;
-        a_row[i] = a_ok[i] ? (unsigned)((r0 + row) * PP + g * VEC) : 0u;
+        a_y[i] = fast_div(g * VEC, a.magic_wp);
+        const int x = g * VEC - a_y[i] * a.Wp;
+        a_ok[i] = c < A_CHUNKS && r0 + row < d.Cout && x < d.Wo;
+        a_row[i] = a_ok[i] ? (unsigned)((r0 + row) * PP + a_y[i] * d.Wo + x) : 0u;
+        if constexpr (RAGGED) a_n[i] = d.Wo - x < VEC ? d.Wo - x : VEC;
     }
 #pragma unroll
     for (int i = 0; i < U_MAX; ++i) {
@@ -181,19 +203,20 @@ __global__ __launch_bounds__(512) void conv_wg_kernel(const ConvWgArgs a) {
         const int ci = fast_div(row, a.magic_rr), rr = row - ci * a.RR;
         u_lds[i] = u < units ? (ci * a.PLANE + rr * a.TW + xg * VEC) * ES : -1;
         u_rr[i] = rr;
-        u_has[i] = (xg < a.wchunks ? 1 : 0) | (xg >= 1 && xg <= a.wchunks ? 2 : 0) | (xg + 1 < a.wchunks ? 4 : 0);
+        u_has[i] = (xg * VEC < d.Win ? 1 : 0) | (xg >= 1 && xg * VEC - 2 < d.Win ? 2 : 0) | (xg * VEC + VEC < d.Win ? 4 : 0);
         if (!SHIFTED) {  // the chunks of the row go behind the left halo as they are
             u_has[i] &= 1;
             u_lds[i] = (u < units && xg < a.wchunks) ? u_lds[i] + d.padL * ES : -1;
         }
         if (u >= units || c0 + ci >= d.Cin) u_has[i] = 0;
         u_src[i] = u_has[i] ? (unsigned)((c0 + ci) * (int)d.x_sc + rr * (int)d.x_sy + xg * VEC) : 0u;
+        if constexpr (RAGGED) u_n[i] = d.Win - xg * VEC < VEC ? d.Win - xg * VEC : VEC;
     }
 
     auto fetch = [&](int tile) {
         const int b0 = fast_div(tile, a.magic_tpi), y0 = (tile - b0 * a.tpi) * a.R;
         const int rows = d.Ho - y0 < a.R ? d.Ho - y0 : a.R;  // the last tile of a sample may be short
-        const int npx = rows * d.Wo, raw_rows = (rows - 1) * d.sh + d.KH, t0 = y0 * d.sh - d.padU;
+        const int raw_rows = (rows - 1) * d.sh + d.KH, t0 = y0 * d.sh - d.padU;
         // tile rows [lo, hi) lie inside the image and are needed by the tile's pixels
         const int lo = t0 < 0 ? -t0 : 0, hi = d.Hin - t0 < raw_rows ? d.Hin - t0 : raw_rows;
         const T *gy = dY + (long long)b0 * d.Cout * PP + (long long)y0 * d.Wo;
@@ -201,7 +224,10 @@ __global__ __launch_bounds__(512) void conv_wg_kernel(const ConvWgArgs a) {
 #pragma unroll
         for (int i = 0; i < A_PER; ++i) {
             regA[i] = make_uint4(0, 0, 0, 0);
-            if (a_ok[i] && a_pix[i] < npx) regA[i] = *reinterpret_cast<const uint4 *>(gy + a_row[i]);
+            if (a_ok[i] && a_y[i] < rows) {
+                if constexpr (RAGGED) regA[i] = load_upto8(gy + a_row[i], a_n[i]);
+                else regA[i] = *reinterpret_cast<const uint4 *>(gy + a_row[i]);
+            }
         }
 #pragma unroll
         for (int i = 0; i < U_MAX; ++i) {
@@ -210,7 +236,10 @@ __global__ __launch_bounds__(512) void conv_wg_kernel(const ConvWgArgs a) {
             if constexpr (SHIFTED) regP[i] = regN[i] = make_uint2(0, 0);
             if (u_has[i] && u_rr[i] >= lo && u_rr[i] < hi) {
                 const T *src = gx + u_src[i];
-                if (u_has[i] & 1) regU[i] = *reinterpret_cast<const uint4 *>(src);
+                if (u_has[i] & 1) {
+                    if constexpr (RAGGED) regU[i] = load_upto8(src, u_n[i]);
+                    else regU[i] = *reinterpret_cast<const uint4 *>(src);
+                }
                 if constexpr (SHIFTED) {
                     if (u_has[i] & 2) regP[i] = load_two<T>(src - 2);
                     if (u_has[i] & 4) regN[i] = load_two<T>(src + VEC);
@@ -235,15 +264,15 @@ __global__ __launch_bounds__(512) void conv_wg_kernel(const ConvWgArgs a) {
             }
         } else {
 #pragma unroll
-            for (int s = 0; s < (SHIFTED == 2 ? 3 : MAX_COPIES); ++s) {
-                if (SHIFTED != 2 && s >= a.copies) break;
+            for (int s = 0; s < (FIXED3 ? 3 : MAX_COPIES); ++s) {
+                if (!FIXED3 && s >= a.copies) break;
                 // copy s, position i holds input column i + s - padL
 #pragma unroll
                 for (int i = 0; i < U_MAX; ++i) {
                     if (i >= uslots) break;
                     if (u_lds[i] >= 0)
                         *reinterpret_cast<uint4 *>(raw + s * a.COPY * ES + u_lds[i]) =
-                            shifted_chunk<T>(regP[i], regU[i], regN[i], SHIFTED == 2 ? s - 1 : s - d.padL);
+                            shifted_chunk<T>(regP[i], regU[i], regN[i], FIXED3 ? s - 1 : s - d.padL);
                 }
             }
         }
@@ -357,6 +386,7 @@ static int launch_conv_wg(ConvWgArgs &a, int gy, int gz, void *dW, hipStream_t s
         a.PLANE = a.RR * a.TW + (a.copies > 1 ? VEC : 0);
         a.COPY = a.CT * a.PLANE;
         a.xg = a.copies > 1 ? a.TW / VEC : a.wchunks;
+        if (a.ragged && a.copies == 1) return -1;  // short chunks exist in the shifted form only
         // slack: an unaligned fragment may start at the last element
         a.raw_bytes = (int)((((size_t)a.copies * a.COPY * ES + 32) + 15) & ~(size_t)15);
         lds = 2 * ((size_t)a.a_bytes + a.raw_bytes);
@@ -367,11 +397,13 @@ static int launch_conv_wg(ConvWgArgs &a, int gy, int gz, void *dW, hipStream_t s
     if (lds < red) lds = red;
     if (lds > 150 * 1024) return -1;
     constexpr bool CAN_SHIFT = ES == 2;
-    const int mode = !(CAN_SHIFT && a.copies > 1) ? 0 : (KW == 3 && a.d.padL == 1) ? 2 : 1;
-    auto kern = mode == 2   ? conv_wg_kernel<T, RB, CBW, CAN_SHIFT ? 2 : 0>
+    const int mode = !(CAN_SHIFT && a.copies > 1) ? 0 : (KW == 3 && a.d.padL == 1) ? (a.ragged ? 3 : 2) : 1;
+    if (a.ragged && mode != 3) return -1;
+    auto kern = mode == 3   ? conv_wg_kernel<T, RB, CBW, CAN_SHIFT ? 3 : 0>
+                : mode == 2 ? conv_wg_kernel<T, RB, CBW, CAN_SHIFT ? 2 : 0>
                 : mode == 1 ? conv_wg_kernel<T, RB, CBW, CAN_SHIFT ? 1 : 0>
                             : conv_wg_kernel<T, RB, CBW, 0>;
-    static bool attr_set[3] = {false, false, false};
+    static bool attr_set[4] = {false, false, false, false};
     if (!attr_set[mode]) {
         if (!hip_ok(hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
                                         hipFuncAttributeMaxDynamicSharedMemorySize, 150 * 1024),
@@ -413,18 +445,24 @@ int conv_tile_wg(const ConvTileDesc &d, const void *X, const void *dY, void *dW)
     if ((d.Ho - 1) * d.sh + d.KH > THP || (d.Wo - 1) * d.sw + d.KW > TWraw) return -1;
     // 8 (4) consecutive pixels of a fragment must be 8 consecutive input columns of one row,
     // and input rows must be copyable 16 bytes at a time
-    if (d.sw != 1 || d.Wo % VEC || d.Win % VEC || d.x_sy % VEC || d.x_sc % VEC || d.x_sb % VEC) return -1;
-    if (reinterpret_cast<uintptr_t>(X) % 16 || reinterpret_cast<uintptr_t>(dY) % 16) return -1;
-    if (d.Wo > 128) return -1;  // a tile is whole output rows within 128 pixels
+    if (d.sw != 1) return -1;
+    a.ragged = d.Wo % VEC || d.Win % VEC || d.x_sy % VEC || d.x_sc % VEC || d.x_sb % VEC ||
+               reinterpret_cast<uintptr_t>(X) % 16 || reinterpret_cast<uintptr_t>(dY) % 16;
+    // ... or, for fp16 3x3 layers with one column of padding, rows of whole dwords
+    if (a.ragged && (ES != 2 || d.KW != 3 || d.padL != 1 || d.Wo % 2 || d.Win % 2 || d.x_sy % 2 || d.x_sc % 2 ||
+                     d.x_sb % 2 || reinterpret_cast<uintptr_t>(X) % 4 || reinterpret_cast<uintptr_t>(dY) % 4))
+        return -1;
+    a.Wp = (d.Wo + VEC - 1) / VEC * VEC;
+    if (a.Wp > 128) return -1;  // a tile is whole output rows within 128 pixels
     // offsets inside one sample are 32-bit
     if ((long long)d.Cin * d.x_sc + (long long)(d.Hin + d.KH) * d.x_sy >= ((long long)1 << 31) ||
         (long long)d.Cout * d.Ho * d.Wo >= ((long long)1 << 31) || d.x_sc >= ((long long)1 << 31))
         return -1;
-    a.R = 128 / d.Wo < d.Ho ? 128 / d.Wo : d.Ho;
+    a.R = 128 / a.Wp < d.Ho ? 128 / a.Wp : d.Ho;
     a.tpi = (d.Ho + a.R - 1) / a.R;
     if ((long long)d.batch * a.tpi * a.tpi >= ((long long)1 << 32)) return -1;  // range of the reciprocal division
     a.tiles = d.batch * a.tpi;
-    a.ksteps = (a.R * d.Wo + 2 * VEC - 1) / (2 * VEC);
+    a.ksteps = (a.R * a.Wp + 2 * VEC - 1) / (2 * VEC);
     // few pixel tiles: worth it only for small fp16 weight tensors (measured 8.6 against 11.2 us for one
     // 16->32 channel 32x32 sample, 14 against 9.5 us for eight 64->64 8x8 ones)
     if (st.gemm_path != 2 && a.tiles < st.num_cu && !(ES == 2 && (long)d.Cout * d.Cin * d.KH * d.KW <= 8192)) return -1;
@@ -441,7 +479,7 @@ int conv_tile_wg(const ConvTileDesc &d, const void *X, const void *dY, void *dW)
     a.magic_taps = magic_of(taps);
     a.magic_kw = magic_of(d.KW);
     a.magic_tpi = magic_of(a.tpi);
-    a.magic_wo = magic_of(d.Wo);
+    a.magic_wp = magic_of(a.Wp);
     const int gy = (d.Cin + a.CT - 1) / a.CT;
     const int cbw = (a.cblocks + 3) / 4;  // column blocks per wave
     if (cbw > 3) return -1;

@@ -275,6 +275,35 @@ def test_conv2d_direct_weight_gradient(pkg, orc, gpu, dt, case):
         gpu.ptl_set_gemm_path(0)
 
 
+# fp16 3x3 layers with one column of padding also take it when rows are whole dwords but not whole 16-byte
+# chunks (28, 14, 12, 6 columns): the tile pads every output row to whole chunks.
+RAGGED_WG_CASES = [
+    # Ci, H, W, Co, ns
+    (20, 14, 14, 40, 5),     # two tiles per sample, the second short
+    (33, 9, 28, 70, 3),      # two channel slabs, two row tiles
+    (8, 6, 6, 9, 7),         # a tile is a whole sample
+    (16, 10, 12, 16, 3),
+    (4, 5, 26, 6, 2),
+]
+
+
+@pytest.mark.parametrize("case", RAGGED_WG_CASES)
+def test_conv2d_direct_weight_gradient_ragged_rows(pkg, orc, gpu, case):
+    Ci, H, W, Co, ns = case
+    gpu.ptl_set_gemm_path(2)
+    try:
+        conv_parity(pkg, orc, gpu, "fp16", Ci, H, W, Co, 3, 3, (1, 1, 1, 1), (1, 1), 0, ns, 0xC0DE0052,
+                    via_batched=True)
+        nd = np.float16
+        x, dw = dev(np.zeros((ns, Ci, H, W), nd)), dev(np.zeros((Co, Ci, 3, 3), nd))
+        dy = dev(np.zeros((ns, Co, H, W), nd))
+        a, keep = hp.conv2d_args(pkg, x, None, None, dw, None, dy, Ci, H, W, Co, 3, 3, H, W, (1, 1, 1, 1), (1, 1))
+        pkg.call("ptl_conv2d_fp16_wg_batched", a, ns)
+        assert gpu.ptl_last_conv_direct() == 1
+    finally:
+        gpu.ptl_set_gemm_path(0)
+
+
 def test_conv2d_direct_and_gemm_routes_agree(pkg, gpu):
     """Same forward / input gradient through the direct kernel and through the GEMM route."""
     for dt, tol in (("fp32", 1e-5), ("fp16", 2e-3)):
