@@ -368,6 +368,41 @@ __global__ __launch_bounds__(1024) void conv_wg_reduce_kernel(const float *__res
     }
 }
 
+// The same sum for few parts of a large tensor: four consecutive outputs per thread, 16-byte loads, all
+// parts of a thread in flight together.
+template <typename T>
+__global__ __launch_bounds__(256) void conv_wg_reduce_few_kernel(const float *__restrict__ ws, T *__restrict__ dW,
+                                                                 int total, int parts) {
+    const int i = (blockIdx.x * 256 + threadIdx.x) * 4;
+    if (i >= total) return;
+    const float4 *src = reinterpret_cast<const float4 *>(ws + i);
+    const size_t step = (size_t)total / 4;
+    float4 s = make_float4(0.f, 0.f, 0.f, 0.f);
+    int p = 0;
+    for (; p + 8 <= parts; p += 8) {
+        float4 v[8];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) v[u] = src[(size_t)(p + u) * step];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) {
+            s.x += v[u].x;
+            s.y += v[u].y;
+            s.z += v[u].z;
+            s.w += v[u].w;
+        }
+    }
+    for (; p < parts; ++p) {
+        const float4 v = src[(size_t)p * step];
+        s.x += v.x;
+        s.y += v.y;
+        s.z += v.z;
+        s.w += v.w;
+    }
+    typedef T t4 __attribute__((ext_vector_type(4)));
+    const t4 o = {(T)s.x, (T)s.y, (T)s.z, (T)s.w};
+    *reinterpret_cast<t4 *>(dW + i) = o;
+}
+
 template <typename T, int RB, int CBW>
 static int launch_conv_wg(ConvWgArgs &a, int gy, int gz, void *dW, hipStream_t s) {
     constexpr int ES = (int)sizeof(T), VEC = 16 / ES;
@@ -427,8 +462,12 @@ static int launch_conv_wg(ConvWgArgs &a, int gy, int gz, void *dW, hipStream_t s
     // partial is complete, otherwise every (slab, row tile) pair writes a disjoint part of it
     hipLaunchKernelGGL(kern, dim3((unsigned)parts, gy, gz), dim3(512), lds, s, a);
     if (!hip_ok(hipGetLastError(), "conv wg launch")) return 2;
-    hipLaunchKernelGGL((conv_wg_reduce_kernel<T>), dim3((total + 63) / 64), dim3(1024), 0, s, a.ws,
-                       reinterpret_cast<T *>(dW), total, (int)parts);
+    if (parts <= 32 && total % 4 == 0 && total >= 65536 && reinterpret_cast<uintptr_t>(dW) % (4 * sizeof(T)) == 0)
+        hipLaunchKernelGGL((conv_wg_reduce_few_kernel<T>), dim3((total / 4 + 255) / 256), dim3(256), 0, s, a.ws,
+                           reinterpret_cast<T *>(dW), total, (int)parts);
+    else
+        hipLaunchKernelGGL((conv_wg_reduce_kernel<T>), dim3((total + 63) / 64), dim3(1024), 0, s, a.ws,
+                           reinterpret_cast<T *>(dW), total, (int)parts);
     return hip_ok(hipGetLastError(), "conv wg reduce launch") ? 0 : 2;
 }
 

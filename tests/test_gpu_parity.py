@@ -254,6 +254,7 @@ DIRECT_WG_CASES = [
     (9, 8, 16, 5, 3, 3, (2, 0, 1, 1), (1, 1), 3),       # all the column padding on the left
     (9, 8, 16, 5, 3, 3, (0, 2, 1, 1), (1, 1), 3),       # ... on the right
     (40, 8, 8, 33, 3, 3, (1, 1, 1, 1), (1, 1), 5),      # a tile is a whole sample
+    (96, 8, 8, 96, 3, 3, (1, 1, 1, 1), (1, 1), 2),      # large filter tensor, two partial sums (vector reduction)
 ]
 
 
