@@ -45,6 +45,20 @@ __global__ __launch_bounds__(256) void dilate_kernel(const T *__restrict__ src, 
     dst[idx] = v;
 }
 
+// dst[0 .. n) = 0, 16 bytes per thread where the alignment allows.
+template <typename T>
+__global__ __launch_bounds__(256) void zero_kernel(T *__restrict__ dst, size_t n, int vec) {
+    constexpr int VEC = 16 / (int)sizeof(T);
+    const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+    if (vec) {
+        if (i * VEC + VEC <= n) reinterpret_cast<uint4 *>(dst)[i] = make_uint4(0, 0, 0, 0);
+        else
+            for (size_t e = i * VEC; e < n; ++e) dst[e] = (T)0;
+    } else if (i < n) {
+        dst[i] = (T)0;
+    }
+}
+
 // out[b][c][pix] += bias[c] (CHW) or out[b][pix][c] += bias[c] (HWC)
 template <typename T>
 __global__ __launch_bounds__(256) void bias_add_kernel(T *__restrict__ out, const T *__restrict__ bias, size_t total,
@@ -395,6 +409,56 @@ static int conv2d_ig(const Args *a, int ns, const char *fn) {
     const T *dY = sg.in(reinterpret_cast<const T *>(a->output->diff), out_n);
     T *dX = sg.out(reinterpret_cast<T *>(a->input->diff), in_n);
     if (sg.failed()) return 2;
+
+    // A strided single-tap layer without padding (projection shortcut): only the input positions the layer read
+    // get a gradient, dX[ci][sh*u][sw*v] = sum_co W[co][ci] dY[co][u][v] - one plain product written through a
+    // strided output map into the zeroed tensor (the general route below would run a stride-1 pass over a
+    // zero-stuffed gradient four times the size: measured 32 against 11 us for 16 -> 32 channels, 32x32, batch 128).
+    if (Pk == 1 && (g.sh != 1 || g.sw != 1) && g.Up == 0 && g.Lp == 0 && state().gemm_path != 1) {
+        const int vec = reinterpret_cast<uintptr_t>(dX) % 16 == 0;
+        const size_t threads = vec ? (in_n + 16 / sizeof(T) - 1) / (16 / sizeof(T)) : in_n;
+        hipLaunchKernelGGL((zero_kernel<T>), dim3(blocks_for(threads)), dim3(256), 0, state().stream, dX, in_n, vec);
+        if (!hip_ok(hipGetLastError(), "zero launch")) return sg.finish(2);
+        state().last_conv_direct = 0;
+        GemmArgs q = {};
+        q.K = g.Co;
+        q.C = dX;
+        q.a.HL = q.a.WL = q.b.HL = q.b.WL = 1;
+        AxisMap pix = {};  // output pixel (sample, u, v) inside the input tensor
+        pix.n = ns * P;
+        pix.d1 = g.Ho;
+        pix.d0 = g.Wo;
+        if (!g.hwc) {
+            q.A = Wt;
+            q.B = dY;
+            q.N = g.Ci;
+            q.M = ns * P;
+            q.a.row = axis_plain(g.Ci, 1);
+            q.a.k = axis_plain(g.Co, g.Ci);
+            q.b.row = axis_two(q.M, P, g.Co * P, 1);
+            q.b.k = axis_plain(g.Co, P);
+            pix.o2 = g.Ci * g.H * g.W;
+            pix.o1 = g.sh * g.W;
+            pix.o0 = g.sw;
+            q.c.n = axis_plain(g.Ci, g.H * g.W);
+            q.c.m = pix;
+        } else {
+            q.A = dY;
+            q.B = Wt;
+            q.N = ns * P;
+            q.M = g.Ci;
+            q.a.row = axis_plain(q.N, g.Co);
+            q.a.k = axis_plain(g.Co, 1);
+            q.b.row = axis_plain(g.Ci, 1);
+            q.b.k = axis_plain(g.Co, g.Ci);
+            pix.o2 = g.H * g.W * g.Ci;
+            pix.o1 = g.sh * g.W * g.Ci;
+            pix.o0 = g.sw * g.Ci;
+            q.c.n = pix;
+            q.c.m = axis_plain(g.Ci, 1);
+        }
+        return sg.finish(gemm<T>(q));
+    }
 
     // A strided forward is undone by a unit-stride pass over the zero-stuffed gradient.
     if (g.sh != 1 || g.sw != 1) {

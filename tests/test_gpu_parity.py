@@ -109,6 +109,17 @@ def test_conv2d_batched(pkg, orc, gpu, dt, hwc):
     conv_parity(pkg, orc, gpu, dt, 6, 11, 11, 9, 3, 3, (1, 1, 1, 1), (2, 2), hwc, 3, 0xC0DE0012)
 
 
+# Strided single-tap layers (projection shortcuts): the input gradient is one product scattered into the zeroed
+# tensor.  Outputs start as 3s, so positions the layer never read must come back as zeros.
+@pytest.mark.parametrize("dt", ["fp32", "fp16"])
+@pytest.mark.parametrize("hwc", [0, 1])
+@pytest.mark.parametrize("case", [(16, 11, 11, 32, (2, 2), 5), (6, 9, 13, 10, (2, 3), 3), (32, 15, 8, 64, (2, 1), 4)])
+def test_conv2d_strided_single_tap(pkg, orc, gpu, dt, hwc, case):
+    Ci, H, W, Co, stride, ns = case
+    conv_parity(pkg, orc, gpu, dt, Ci, H, W, Co, 1, 1, (0, 0, 0, 0), stride, hwc, ns, 0xC0DE0081,
+                via_batched=True)
+
+
 # The direct convolution kernel (channel-major forward and input gradient) normally takes only calls with
 # many pixel tiles; selection 2 sends every call whose geometry fits through it, so that small cases the
 # oracle finishes in seconds cover its tile logic: tiles that start mid-row, span several images, hang over
