@@ -504,7 +504,11 @@ int conv_tile_wg(const ConvTileDesc &d, const void *X, const void *dY, void *dW)
     a.ksteps = (a.R * a.Wp + 2 * VEC - 1) / (2 * VEC);
     // few pixel tiles: worth it only for small fp16 weight tensors (measured 8.6 against 11.2 us for one
     // 16->32 channel 32x32 sample, 14 against 9.5 us for eight 64->64 8x8 ones)
-    if (st.gemm_path != 2 && a.tiles < st.num_cu && !(ES == 2 && (long)d.Cout * d.Cin * d.KH * d.KW <= 8192)) return -1;
+    // (from 128 channels on the alternative is the sum over taps, which loses from half a tile per CU:
+    // measured 25 against 33 us for 128 -> 128 channels on 8x8 images at batch 128)
+    const bool wide = d.Cin >= 128 && d.Cout >= 128 && 2 * a.tiles >= st.num_cu;
+    if (st.gemm_path != 2 && a.tiles < st.num_cu && !wide && !(ES == 2 && (long)d.Cout * d.Cin * d.KH * d.KW <= 8192))
+        return -1;
 
     const int taps = d.KH * d.KW;
     a.TWraw = TWraw;
