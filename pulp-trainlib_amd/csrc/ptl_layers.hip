@@ -24,25 +24,21 @@ namespace ptl {
 
 // Zero-stuffed copy of an output gradient for strided convolutions:
 // dst[b][c][ho*sh][wo*sw] = src[b][c][ho][wo] (CHW) or the HWC equivalent.
+// One workgroup per plane (CHW: a channel of a sample, HWC: a sample), 32-bit index arithmetic inside it.
 template <typename T>
-__global__ __launch_bounds__(256) void dilate_kernel(const T *__restrict__ src, T *__restrict__ dst, int planes,
-                                                     int Ho, int Wo, int Hd, int Wd, int sh, int sw, int cin) {
+__global__ __launch_bounds__(256) void dilate_kernel(const T *__restrict__ src, T *__restrict__ dst, int Ho, int Wo,
+                                                     int Hd, int Wd, int sh, int sw, int cin) {
     // cin = innermost channel count (1 for CHW planes, C for HWC)
-    size_t total = (size_t)planes * Hd * Wd * cin;
-    size_t idx = (size_t)blockIdx.x * 256 + threadIdx.x;
-    if (idx >= total) return;
-    int c = (int)(idx % cin);
-    size_t t = idx / cin;
-    int wd = (int)(t % Wd);
-    t /= Wd;
-    int hd = (int)(t % Hd);
-    int p = (int)(t / Hd);
-    T v = (T)0;
-    if (hd % sh == 0 && wd % sw == 0) {
-        int ho = hd / sh, wo = wd / sw;
-        v = src[(((size_t)p * Ho + ho) * Wo + wo) * cin + c];
+    const unsigned rowlen = (unsigned)Wd * cin, n = (unsigned)Hd * rowlen;
+    const T *sp = src + (size_t)blockIdx.x * Ho * Wo * cin;
+    T *dp = dst + (size_t)blockIdx.x * n;
+    for (unsigned i = threadIdx.x; i < n; i += 256) {
+        const unsigned hd = i / rowlen, r = i - hd * rowlen;
+        const unsigned wd = cin == 1 ? r : r / cin, c = cin == 1 ? 0 : r - wd * cin;
+        T v = (T)0;
+        if (hd % sh == 0 && wd % sw == 0) v = sp[((hd / sh) * Wo + wd / sw) * cin + c];
+        dp[i] = v;
     }
-    dst[idx] = v;
 }
 
 // dst[0 .. n) = 0, 16 bytes per thread where the alignment allows.
@@ -464,8 +460,8 @@ static int conv2d_ig(const Args *a, int ns, const char *fn) {
     if (g.sh != 1 || g.sw != 1) {
         T *dil = static_cast<T *>(scratch(dil_n * sizeof(T)));
         if (!dil) return 2;
-        hipLaunchKernelGGL((dilate_kernel<T>), dim3(blocks_for(dil_n)), dim3(256), 0, state().stream, dY, dil,
-                           g.hwc ? ns : ns * g.Co, g.Ho, g.Wo, Hd, Wd, g.sh, g.sw, g.hwc ? g.Co : 1);
+        hipLaunchKernelGGL((dilate_kernel<T>), dim3((unsigned)(g.hwc ? ns : ns * g.Co)), dim3(256), 0, state().stream, dY,
+                           dil, g.Ho, g.Wo, Hd, Wd, g.sh, g.sw, g.hwc ? g.Co : 1);
         if (!hip_ok(hipGetLastError(), "dilate launch")) return sg.finish(2);
         dY = dil;
     }
