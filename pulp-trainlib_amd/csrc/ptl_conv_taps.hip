@@ -24,13 +24,14 @@ __global__ __launch_bounds__(256) void chw_to_blocked_padded_kernel(const T *__r
                                                                     int padL, long long sb, long long sc,
                                                                     int cblocks, long long total) {
     constexpr int VEC = 16 / (int)sizeof(T);
-    const long long i = (long long)blockIdx.x * 256 + threadIdx.x;
+    // (the host keeps the copy below 2^31 bytes: 32-bit index arithmetic)
+    const unsigned i = blockIdx.x * 256u + threadIdx.x;
     if (i >= total) return;
-    const int xp = (int)(i % Wp);
-    long long r = i / Wp;
-    const int yp = (int)(r % Hp);
-    r /= Hp;
-    const int b = (int)(r % B), cb = (int)(r / B);
+    unsigned r = i / (unsigned)Wp;
+    const int xp = (int)(i - r * Wp);
+    const unsigned r2 = r / (unsigned)Hp;
+    const int yp = (int)(r - r2 * Hp);
+    const int cb = (int)(r2 / (unsigned)B), b = (int)(r2 - (unsigned)cb * B);
     const int y = yp - padU, x = xp - padL;
     union {
         uint4 v;
@@ -154,15 +155,16 @@ __global__ __launch_bounds__(256) void embed_gradient_kernel(const T *__restrict
                                                              int Cout, int Ho, int Wo, int Hp, int Wp, long long Kr,
                                                              long long total) {
     constexpr int VEC = 16 / (int)sizeof(T);
-    const long long i = (long long)blockIdx.x * 256 + threadIdx.x;
+    // (the host keeps the copy below 2^31 bytes: 32-bit index arithmetic)
+    const unsigned i = blockIdx.x * 256u + threadIdx.x;
     if (i >= total) return;
-    const long long kv = Kr / VEC;
-    const long long k0 = (i % kv) * VEC;
+    const unsigned kv = (unsigned)(Kr / VEC);
     const int co = (int)(i / kv);
-    int xp = (int)(k0 % Wp);
-    long long r = k0 / Wp;
-    int yp = (int)(r % Hp);
-    long long b = r / Hp;
+    const unsigned k0 = (i - (unsigned)co * kv) * VEC;
+    unsigned r = k0 / (unsigned)Wp;
+    int xp = (int)(k0 - r * Wp);
+    long long b = r / (unsigned)Hp;
+    int yp = (int)(r - (unsigned)b * Hp);
     union {
         uint4 v;
         T e[VEC];

@@ -291,11 +291,12 @@ __global__ __launch_bounds__(256) void chw_to_blocked_kernel(const T *__restrict
                                                              int cblocks, int HW, long long in_sb, long long in_sc,
                                                              long long total) {
     constexpr int VEC = 16 / (int)sizeof(T);
-    const long long i = (long long)blockIdx.x * 256 + threadIdx.x;
+    // (the host keeps the chunk count below 2^31: 32-bit index arithmetic)
+    const unsigned i = blockIdx.x * 256u + threadIdx.x;
     if (i >= total) return;
-    const long long bc = i / HW;
+    const unsigned bc = i / (unsigned)HW;
     const int pix = (int)(i - bc * HW);
-    const int b = (int)(bc / cblocks), cb = (int)(bc - (long long)b * cblocks);
+    const int b = (int)(bc / (unsigned)cblocks), cb = (int)(bc - (unsigned)b * cblocks);
     const T *src = in + b * in_sb + (long long)(cb * VEC) * in_sc + pix;
     union {
         uint4 v;
