@@ -19,13 +19,12 @@ namespace ptl {
 
 // in: [b][C][H][W] (strides sb, sc; rows contiguous) -> out: [C/VEC][B][Hp][Wp] chunks, zero halo.
 template <typename T>
-__global__ __launch_bounds__(256) void chw_to_blocked_padded_kernel(const T *__restrict__ in, uint4 *__restrict__ out,
-                                                                    int B, int H, int W, int Hp, int Wp, int padU,
-                                                                    int padL, long long sb, long long sc,
-                                                                    int cblocks, long long total) {
+__device__ inline void chw_to_blocked_padded(unsigned block, const T *__restrict__ in, uint4 *__restrict__ out, int B,
+                                             int H, int W, int Hp, int Wp, int padU, int padL, long long sb,
+                                             long long sc, int cblocks, long long total) {
     constexpr int VEC = 16 / (int)sizeof(T);
     // (the host keeps the copy below 2^31 bytes: 32-bit index arithmetic)
-    const unsigned i = blockIdx.x * 256u + threadIdx.x;
+    const unsigned i = block * 256u + threadIdx.x;
     if (i >= total) return;
     unsigned r = i / (unsigned)Wp;
     const int xp = (int)(i - r * Wp);
@@ -47,6 +46,14 @@ __global__ __launch_bounds__(256) void chw_to_blocked_padded_kernel(const T *__r
     out[i] = u.v;
 }
 
+template <typename T>
+__global__ __launch_bounds__(256) void chw_to_blocked_padded_kernel(const T *__restrict__ in, uint4 *__restrict__ out,
+                                                                    int B, int H, int W, int Hp, int Wp, int padU,
+                                                                    int padL, long long sb, long long sc,
+                                                                    int cblocks, long long total) {
+    chw_to_blocked_padded<T>(blockIdx.x, in, out, B, H, W, Hp, Wp, padU, padL, sb, sc, cblocks, total);
+}
+
 // Launches the padded, blocked copy of X ([b][C][H][W]) with `margin` zero chunks after it.
 template <typename T>
 static int blocked_padded_copy(const T *X, uint4 *xb, const ConvTileDesc &d, int Hp, int Wp, long long margin) {
@@ -62,11 +69,10 @@ static int blocked_padded_copy(const T *X, uint4 *xb, const ConvTileDesc &d, int
 
 // out[m][tap][c] = W[base + m*sm + c*sc + ky*sy + kx*sx]
 template <typename T>
-__global__ __launch_bounds__(256) void filters_tap_major_kernel(const T *__restrict__ w, T *__restrict__ out, int C,
-                                                                int KW, int taps, long long base, long long sm,
-                                                                long long sc, long long sy, long long sx,
-                                                                long long total) {
-    const long long i = (long long)blockIdx.x * 256 + threadIdx.x;
+__device__ inline void filters_tap_major(unsigned block, const T *__restrict__ w, T *__restrict__ out, int C, int KW,
+                                         int taps, long long base, long long sm, long long sc, long long sy,
+                                         long long sx, long long total) {
+    const long long i = (long long)block * 256 + threadIdx.x;
     if (i >= total) return;
     const int c = (int)(i % C);
     const long long r = i / C;
@@ -75,8 +81,31 @@ __global__ __launch_bounds__(256) void filters_tap_major_kernel(const T *__restr
     out[i] = w[base + m * sm + c * sc + (t / KW) * sy + (t % KW) * sx];
 }
 
+// Both layout passes of the forward / input-gradient route in one launch: the first `copy_blocks` workgroups
+// write the padded, blocked input, the rest the tap-major filters.
+struct TapPrepArgs {
+    const void *in;
+    uint4 *xb;
+    int B, H, W, Hp, Wp, padU, padL, cblocks;
+    long long sb, sc, xb_total;
+    unsigned copy_blocks;
+    const void *w;
+    void *wr;
+    int C, KW, taps;
+    long long w_base, w_sm, w_sc, w_sy, w_sx, wr_total;
+};
 template <typename T>
-int conv_taps(const ConvTileDesc &d, const void *X, const void *Wt, void *Y, const OutMap &c, bool flipped) {
+__global__ __launch_bounds__(256) void tap_prepare_kernel(const TapPrepArgs a) {
+    if (blockIdx.x < a.copy_blocks)
+        chw_to_blocked_padded<T>(blockIdx.x, reinterpret_cast<const T *>(a.in), a.xb, a.B, a.H, a.W, a.Hp, a.Wp, a.padU,
+                                 a.padL, a.sb, a.sc, a.cblocks, a.xb_total);
+    else
+        filters_tap_major<T>(blockIdx.x - a.copy_blocks, reinterpret_cast<const T *>(a.w), reinterpret_cast<T *>(a.wr),
+                             a.C, a.KW, a.taps, a.w_base, a.w_sm, a.w_sc, a.w_sy, a.w_sx, a.wr_total);
+}
+
+template <typename T>
+int conv_taps(const ConvTileDesc &d, const void *X, const void *Wt, void *Y, const OutMap &c) {
     State &st = state();
     constexpr int ES = (int)sizeof(T), VEC = 16 / ES, SK = 128 / ES;
     if (d.in_hwc || d.sh != 1 || d.sw != 1 || d.Cin % SK || d.x_sy != d.Win) return -1;
@@ -92,20 +121,33 @@ int conv_taps(const ConvTileDesc &d, const void *X, const void *Wt, void *Y, con
     // worth it only when the pixel tiles fill the chip: the passes above cost two extra launches
     if (st.gemm_path == 2) return -1;
     // (and only with at least 64 filters: narrower products fall to the GEMM's slim tiles, where the direct kernel wins).
-    // Against the gathering GEMM it pays from a quarter of that already when the contraction is long (128 channels)
-    // or runs over flipped filters (input gradient): measured 12.8 against 16.5 us for the input gradient of
-    // 64 -> 64 channels on 8x8 images at batch 128, 16.8 against 27.8 us for 128 -> 128.
-    const long long fill = npix / 128 * ((d.Cout + 127) / 128) * ((flipped || d.Cin >= 128) ? 4 : 1);
+    // Against the gathering GEMM, which takes over below that, it pays from a quarter of a tile per CU: measured
+    // 10.5 against 11.3 us (forward) and 16.5 us (input gradient, flipped filters) for 64 -> 64 channels on 8x8
+    // images at batch 128, 16.8 against 27.8 us for the input gradient of 128 -> 128.
+    const long long fill = npix / 128 * ((d.Cout + 127) / 128) * 4;
     if (st.gemm_path != 3 && (d.Cout < 64 || fill < st.num_cu)) return -1;
     char *buf = static_cast<char *>(scratch((size_t)(xb_elems + wr_elems) * ES + 256));
     if (!buf) return 2;
     uint4 *xb = reinterpret_cast<uint4 *>(buf);
     T *wr = reinterpret_cast<T *>(buf + (((size_t)xb_elems * ES + 255) & ~(size_t)255));
-    if (int rc = blocked_padded_copy<T>(reinterpret_cast<const T *>(X), xb, d, Hp, Wp, 0)) return rc;
-    hipLaunchKernelGGL((filters_tap_major_kernel<T>), dim3((unsigned)((wr_elems + 255) / 256)), dim3(256), 0,
-                       st.stream, reinterpret_cast<const T *>(Wt), wr, d.Cin, d.KW, taps, d.w_base, d.w_sm, d.w_sc,
-                       d.w_sy, d.w_sx, wr_elems);
-    if (!hip_ok(hipGetLastError(), "filter layout launch")) return 2;
+    {
+        TapPrepArgs p = {};
+        p.in = X;
+        p.xb = xb;
+        p.B = d.batch; p.H = d.Hin; p.W = d.Win; p.Hp = Hp; p.Wp = Wp; p.padU = d.padU; p.padL = d.padL;
+        p.cblocks = cblocks;
+        p.sb = d.x_sb; p.sc = d.x_sc;
+        p.xb_total = xb_elems / VEC;
+        p.copy_blocks = (unsigned)((p.xb_total + 255) / 256);
+        p.w = Wt;
+        p.wr = wr;
+        p.C = d.Cin; p.KW = d.KW; p.taps = taps;
+        p.w_base = d.w_base; p.w_sm = d.w_sm; p.w_sc = d.w_sc; p.w_sy = d.w_sy; p.w_sx = d.w_sx;
+        p.wr_total = wr_elems;
+        hipLaunchKernelGGL((tap_prepare_kernel<T>), dim3(p.copy_blocks + (unsigned)((wr_elems + 255) / 256)), dim3(256),
+                           0, st.stream, p);
+        if (!hip_ok(hipGetLastError(), "layout launch")) return 2;
+    }
 
     GemmArgs q = {};
     q.A = xb;
@@ -289,7 +331,7 @@ int conv_taps_wg(const ConvTileDesc &d, const void *X, const void *dY, void *dW)
 template int conv_taps_wg<float>(const ConvTileDesc &, const void *, const void *, void *);
 template int conv_taps_wg<half_t>(const ConvTileDesc &, const void *, const void *, void *);
 
-template int conv_taps<float>(const ConvTileDesc &, const void *, const void *, void *, const OutMap &, bool);
-template int conv_taps<half_t>(const ConvTileDesc &, const void *, const void *, void *, const OutMap &, bool);
+template int conv_taps<float>(const ConvTileDesc &, const void *, const void *, void *, const OutMap &);
+template int conv_taps<half_t>(const ConvTileDesc &, const void *, const void *, void *, const OutMap &);
 
 }  // namespace ptl

@@ -75,7 +75,7 @@ inline int conv_raw_rows(int bm, int Ho, int Wo, int sh, int KH, int THP, long l
 // The same convolution as a sum over filter taps on the look-up-free GEMM (unit stride, channel-major input,
 // channels a multiple of a slab); -1 when the geometry does not fit.  Input and filters are re-laid in scratch.
 template <typename T>
-int conv_taps(const ConvTileDesc &d, const void *X, const void *Wt, void *Y, const OutMap &c, bool flipped);
+int conv_taps(const ConvTileDesc &d, const void *X, const void *Wt, void *Y, const OutMap &c);
 
 // Weight gradient over filter taps on the same GEMM (partial sums per tap and k split + one reduction).
 template <typename T>
