@@ -316,6 +316,32 @@ def test_conv2d_direct_weight_gradient_ragged_rows(pkg, orc, gpu, case):
         gpu.ptl_set_gemm_path(0)
 
 
+# Wide layers at their real image sizes (too large for the CPU oracle in seconds): forward, weight gradient and
+# input gradient against torch's fp32 convolution of the same fp16-rounded tensors, evaluated on the GPU.  The
+# checker is torch; the routes these sizes take are the tap-sum product and the resident-tile weight gradient, with 56-wide
+# rows (28 row tiles per sample), 28- and 14-wide rows (rows padded to whole chunks inside the tile) and several
+# channel slabs.  fp16 outputs are fp32 sums rounded once: 2e-3 relative L2 leaves a factor of five.
+@pytest.mark.parametrize("case", [(64, 64, 56, 16), (32, 64, 56, 16), (128, 128, 28, 16), (256, 256, 14, 16),
+                                  (128, 128, 16, 32), (64, 64, 8, 128)])
+def test_conv2d_wide_layers_against_torch(pkg, gpu, case):
+    Ci, Co, H, ns = case
+    x = dev(hp.uniform(21, (ns, Ci, H, H), dtype=np.float16))
+    w = dev(hp.uniform(22, (Co, Ci, 3, 3), -0.1, 0.1).astype(np.float16))
+    dy = dev(hp.uniform(23, (ns, Co, H, H), dtype=np.float16))
+    y, dx, dw = torch.zeros_like(dy), torch.zeros_like(x), torch.zeros_like(w)
+    a, keep = hp.conv2d_args(pkg, x, dx, w, dw, y, dy, Ci, H, H, Co, 3, 3, H, H, (1, 1, 1, 1), (1, 1))
+    for s in ("fw", "wg", "ig"):
+        pkg.call("ptl_conv2d_fp16_%s_batched" % s, a, ns)
+    sync(gpu)
+    xf, wf, dyf = x.float(), w.float(), dy.float()
+    ref_y = torch.nn.functional.conv2d(xf, wf, padding=1)
+    ref_dw = torch.nn.grad.conv2d_weight(xf, wf.shape, dyf, padding=1)
+    ref_dx = torch.nn.grad.conv2d_input(xf.shape, wf, dyf, padding=1)
+    for name, got, ref in (("y", y, ref_y), ("dw", dw, ref_dw), ("dx", dx, ref_dx)):
+        err = ((got.float() - ref).norm() / ref.norm()).item()
+        assert err <= 2e-3, (name, err)
+
+
 def test_conv2d_direct_and_gemm_routes_agree(pkg, gpu):
     """Same forward / input gradient through the direct kernel and through the GEMM route."""
     for dt, tol in (("fp32", 1e-5), ("fp16", 2e-3)):
