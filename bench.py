@@ -36,6 +36,8 @@ def main():
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--no-detail", action="store_true", help="skip the per-shape detail table")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
+    ap.add_argument("--resnet-only", action="store_true",
+                    help="detail table: only the ResNet-20-shaped step (for a kernel trace of that step alone)")
     ap.add_argument("--batch", type=int, default=512, help="samples per step of the headline workload")
     ap.add_argument("--copy-calib", action="store_true",
                     help="also run a 64 MiB device copy five times (a kernel of known traffic, to scale the "
@@ -196,10 +198,41 @@ def main():
                                             "(the reference's arithmetic), %.2f s" % (m, ns, reps, t_cpu)}
 
     # ------------------------------------------------------------------------------ detail
-    if not args.no_detail:
+    if args.resnet_only:
+        result["detail"] = resnet_rows(pkg, lib, timed, torch, dev)
+    elif not args.no_detail:
         result["detail"] = detail_table(pkg, lib, hp, to_dev, timed, check, torch, dev)
 
     print(json.dumps(result))
+
+
+def resnet_rows(pkg, lib, timed, torch, dev):
+    """The ResNet-20-shaped training step, with and without normalisation layers."""
+    rows = []
+    tdt = {"fp32": torch.float32, "fp16": torch.float16}
+    # config 5: ResNet-20 (CIFAR geometry) training step, fp16, batch 128, assembled from the entry points
+    # (tests/resnet_step.py): with batch normalisation after every convolution, and without
+    import resnet_step as rs
+    ns, dt = 128, "fp16"
+    convs, blocks, ncls = rs.resnet20_spec()
+    macs, H = 3 * 16 * 9 * 32 * 32, 32
+    for (n, ci, co, stride, proj) in blocks:
+        Ho = H // stride
+        macs += (ci * co * 9 + co * co * 9 + (ci * co if proj else 0)) * Ho * Ho
+        H = Ho
+    flops = 3 * 2.0 * ns * (macs + 64 * ncls)
+    for norm in (True, False):
+        net = rs.ResNetStep(pkg, lib, torch, dt, ns, rs.init_weights(0x2E5E0, dt), 0.01, norm=norm)
+        net.x.copy_(torch.randn(ns, 3, 32, 32, device=dev).to(tdt[dt]))
+        net.target.zero_()
+        net.target[torch.arange(ns), torch.randint(0, 10, (ns,))] = 1
+        ms = timed(lambda: net.step(update=True), 10, 3)
+        rows.append({"workload": "resnet20 step%s FW+BW+SGD N=%d, %d launches"
+                                 % (" with batch norm" if norm else " (no norm)", ns, net.launches()),
+                     "dtype": dt, "us": round(ms * 1e3, 1), "TFLOP/s": round(flops / (ms * 1e-3) / 1e12, 3),
+                     "samples/s": round(ns / (ms * 1e-3), 1)})
+        del net
+    return rows
 
 
 def detail_table(pkg, lib, hp, to_dev, timed, check, torch, dev):
@@ -330,28 +363,7 @@ def detail_table(pkg, lib, hp, to_dev, timed, check, torch, dev):
         ms = timed(lambda: check(lib.ptl_mhsa_fp32_bw_batched(ref, ns)), 50)
         add("mhsa L197 E192 3x64 BW N=%d" % ns, "fp32", ms, 2 * f_fw, 2 * act)
 
-    # config 5: ResNet-20 (CIFAR geometry) training step, fp16, batch 128, assembled from the entry points
-    # (tests/resnet_step.py): with batch normalisation after every convolution, and without
-    import resnet_step as rs
-    ns, dt = 128, "fp16"
-    convs, blocks, ncls = rs.resnet20_spec()
-    macs, H = 3 * 16 * 9 * 32 * 32, 32
-    for (n, ci, co, stride, proj) in blocks:
-        Ho = H // stride
-        macs += (ci * co * 9 + co * co * 9 + (ci * co if proj else 0)) * Ho * Ho
-        H = Ho
-    flops = 3 * 2.0 * ns * (macs + 64 * ncls)
-    for norm in (True, False):
-        net = rs.ResNetStep(pkg, lib, torch, dt, ns, rs.init_weights(0x2E5E0, dt), 0.01, norm=norm)
-        net.x.copy_(torch.randn(ns, 3, 32, 32, device=dev).to(tdt[dt]))
-        net.target.zero_()
-        net.target[torch.arange(ns), torch.randint(0, 10, (ns,))] = 1
-        ms = timed(lambda: net.step(update=True), 10, 3)
-        rows.append({"workload": "resnet20 step%s FW+BW+SGD N=%d, %d launches"
-                                 % (" with batch norm" if norm else " (no norm)", ns, net.launches()),
-                     "dtype": dt, "us": round(ms * 1e3, 1), "TFLOP/s": round(flops / (ms * 1e-3) / 1e12, 3),
-                     "samples/s": round(ns / (ms * 1e-3), 1)})
-        del net
+    rows += resnet_rows(pkg, lib, timed, torch, dev)
     return rows
 
 

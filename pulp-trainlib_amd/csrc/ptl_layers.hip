@@ -24,20 +24,21 @@ namespace ptl {
 
 // Zero-stuffed copy of an output gradient for strided convolutions:
 // dst[b][c][ho*sh][wo*sw] = src[b][c][ho][wo] (CHW) or the HWC equivalent.
-// One workgroup per plane (CHW: a channel of a sample, HWC: a sample), 32-bit index arithmetic inside it.
+// One workgroup per plane (CHW: a channel of a sample, HWC: a sample): it clears the plane, then scatters the
+// source elements into it (one division per source element instead of five per destination element).
 template <typename T>
 __global__ __launch_bounds__(256) void dilate_kernel(const T *__restrict__ src, T *__restrict__ dst, int Ho, int Wo,
                                                      int Hd, int Wd, int sh, int sw, int cin) {
     // cin = innermost channel count (1 for CHW planes, C for HWC)
-    const unsigned rowlen = (unsigned)Wd * cin, n = (unsigned)Hd * rowlen;
-    const T *sp = src + (size_t)blockIdx.x * Ho * Wo * cin;
+    const unsigned n = (unsigned)Hd * Wd * cin, m = (unsigned)Ho * Wo * cin, rowlen = (unsigned)Wo * cin;
+    const T *sp = src + (size_t)blockIdx.x * m;
     T *dp = dst + (size_t)blockIdx.x * n;
-    for (unsigned i = threadIdx.x; i < n; i += 256) {
-        const unsigned hd = i / rowlen, r = i - hd * rowlen;
-        const unsigned wd = cin == 1 ? r : r / cin, c = cin == 1 ? 0 : r - wd * cin;
-        T v = (T)0;
-        if (hd % sh == 0 && wd % sw == 0) v = sp[((hd / sh) * Wo + wd / sw) * cin + c];
-        dp[i] = v;
+    for (unsigned i = threadIdx.x; i < n; i += 256) dp[i] = (T)0;
+    __syncthreads();  // orders the two writes of a position within the workgroup
+    for (unsigned i = threadIdx.x; i < m; i += 256) {
+        const unsigned ho = i / rowlen, r = i - ho * rowlen;
+        const unsigned wo = cin == 1 ? r : r / cin, c = cin == 1 ? 0 : r - wo * cin;
+        dp[((ho * sh) * Wd + wo * sw) * cin + c] = sp[i];
     }
 }
 
