@@ -273,10 +273,20 @@ int conv_taps_wg(const ConvTileDesc &d, const void *X, const void *dY, void *dW)
         return -1;
     const int bm = (d.Cout >= 128 && d.Cin >= 128) ? 128 : 64;
     const long long tiles = (long long)((d.Cout + bm - 1) / bm) * ((d.Cin + bm - 1) / bm);
-    long long S = (2LL * st.num_cu + tiles * taps - 1) / (tiles * taps);
+    // k splits: one workgroup of this tile holds a CU (96 KB of ring), so the launch runs in rounds of num_cu
+    // workgroups.  Take the split count with the least rounds x (slabs per workgroup + the fixed cost of a
+    // workgroup's prologue and fp32 partial-sum epilogue, about six slabs' worth).
     const long long max_s = Kr / (4 * SK) > 0 ? Kr / (4 * SK) : 1;
-    if (S > max_s) S = max_s;
-    if (S < 1) S = 1;
+    const long long slabs = Kr / SK, fixed = 6;
+    long long S = 1, best = -1;
+    for (long long s = 1; s <= max_s && s * tiles * taps <= 8LL * st.num_cu; ++s) {
+        const long long rounds = (s * tiles * taps + st.num_cu - 1) / st.num_cu;
+        const long long cost = rounds * ((slabs + s - 1) / s + fixed);
+        if (best < 0 || cost < best) {
+            best = cost;
+            S = s;
+        }
+    }
     long long kchunk = ((Kr + S - 1) / S + SK - 1) / SK * SK;
     S = (Kr + kchunk - 1) / kchunk;
     const size_t ws_bytes = (size_t)taps * S * d.Cout * d.Cin * sizeof(float);

@@ -322,7 +322,7 @@ def test_conv2d_direct_weight_gradient_ragged_rows(pkg, orc, gpu, case):
 # rows (28 row tiles per sample), 28- and 14-wide rows (rows padded to whole chunks inside the tile) and several
 # channel slabs.  fp16 outputs are fp32 sums rounded once: 2e-3 relative L2 leaves a factor of five.
 @pytest.mark.parametrize("case", [(64, 64, 56, 16), (32, 64, 56, 16), (128, 128, 28, 16), (256, 256, 14, 16),
-                                  (128, 128, 16, 32), (64, 64, 8, 128)])
+                                  (128, 128, 16, 32), (64, 64, 8, 128), (128, 256, 14, 32), (512, 512, 7, 32)])
 def test_conv2d_wide_layers_against_torch(pkg, gpu, case):
     Ci, Co, H, ns = case
     x = dev(hp.uniform(21, (ns, Ci, H, H), dtype=np.float16))
@@ -340,6 +340,29 @@ def test_conv2d_wide_layers_against_torch(pkg, gpu, case):
     for name, got, ref in (("y", y, ref_y), ("dw", dw, ref_dw), ("dx", dx, ref_dx)):
         err = ((got.float() - ref).norm() / ref.norm()).item()
         assert err <= 2e-3, (name, err)
+
+
+@pytest.mark.parametrize("case", [(256, 256, 14, 24), (128, 128, 28, 8), (256, 128, 9, 40)])
+def test_conv2d_wide_weight_gradient_routes_against_torch(pkg, gpu, case):
+    """The weight gradient of a wide layer on each of its routes (default choice, resident-tile kernel, sum over
+    taps with its k splits) against torch's fp32 weight gradient of the same fp16-rounded tensors."""
+    Ci, Co, H, ns = case
+    x = dev(hp.uniform(31, (ns, Ci, H, H), dtype=np.float16))
+    dy = dev(hp.uniform(33, (ns, Co, H, H), dtype=np.float16))
+    w = torch.zeros(Co, Ci, 3, 3, device=x.device, dtype=torch.float16)
+    y, dx = torch.zeros_like(dy), torch.zeros_like(x)
+    ref = torch.nn.grad.conv2d_weight(x.float(), w.shape, dy.float(), padding=1)
+    try:
+        for path in (0, 2, 3):
+            gpu.ptl_set_gemm_path(path)
+            dw = torch.full_like(w, 7.0)
+            a, keep = hp.conv2d_args(pkg, x, dx, w, dw, y, dy, Ci, H, H, Co, 3, 3, H, H, (1, 1, 1, 1), (1, 1))
+            pkg.call("ptl_conv2d_fp16_wg_batched", a, ns)
+            sync(gpu)
+            err = ((dw.float() - ref).norm() / ref.norm()).item()
+            assert err <= 2e-3, (path, err)
+    finally:
+        gpu.ptl_set_gemm_path(0)
 
 
 def test_conv2d_direct_and_gemm_routes_agree(pkg, gpu):
