@@ -136,8 +136,13 @@ int gemm_async(GemmArgs &g) {
                 if (g.splits == 1 && g.K <= 2 * SK) return launch_plain<T, 128, 128, 256, 2, 2, 1, 2, 1>(g, st.stream);
                 // fp16 products large enough to give every CU a 256x128 tile: a third less L2 -> LDS traffic per
                 // MFMA than 128x128, which is what bounds that tile (+15-20 % measured from 4096^3 up)
+                // Either tile holds a CU by itself, so a launch runs in rounds of num_cu workgroups and a 256x128
+                // workgroup takes about 1.7 times as long as a 128x128 one: the tall tile also pays where it
+                // saves a half-empty round (196 tall tiles in one round against 392 square ones in two).
                 if constexpr (sizeof(T) == 2) {
-                    if (g.splits == 1 && tiles(256, 128) >= st.num_cu)
+                    const long r_tall = (tiles(256, 128) + st.num_cu - 1) / st.num_cu;
+                    const long r_square = (tiles(128, 128) + st.num_cu - 1) / st.num_cu;
+                    if (g.splits == 1 && g.N >= 256 && 17 * r_tall < 10 * r_square)
                         return launch_plain<T, 256, 128, 512, 4, 2, 1, 3, 1>(g, st.stream);
                 }
                 return launch_plain<T, 128, 128, 512, 2, 2, 2, 3, 1>(g, st.stream);
