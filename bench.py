@@ -329,7 +329,9 @@ def detail_table(pkg, lib, hp, to_dev, timed, check, torch, dev):
         run3("ptl_conv_pw", dt, a, ns, "pointwise 64->128 56x56", flops, (nb, nb, nb), 100 if ns == 1 else 30)
 
     # larger convolutions, fp16, batched (ResNet-18/50 style layers)
-    for (ns, Ci, Co, H) in ((256, 32, 64, 56), (128, 64, 64, 56), (128, 128, 128, 28), (128, 256, 256, 14)):
+    # (the last three rows are a saturating sweep: the same kernels with enough tiles for several full rounds)
+    for (ns, Ci, Co, H) in ((256, 32, 64, 56), (128, 64, 64, 56), (128, 128, 128, 28), (128, 256, 256, 14),
+                            (512, 128, 128, 28), (256, 256, 256, 28), (256, 512, 512, 14)):
         K, dt = 3, "fp16"
         x = torch.rand(ns, Ci, H, H, device=dev).to(tdt[dt]) - 0.5
         w = torch.rand(Co, Ci, K, K, device=dev).to(tdt[dt]) - 0.5
