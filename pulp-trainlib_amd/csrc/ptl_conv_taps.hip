@@ -1,5 +1,5 @@
-// Convolution as a sum over filter taps on the look-up-free pipelined GEMM (unit stride, channel-major
-// tensors, channel counts that are multiples of a 128-byte slab: 64 halves / 32 floats).
+// Convolution as a sum over filter taps on the look-up-free pipelined GEMM (unit stride, channel counts that
+// are multiples of a 128-byte slab: 64 halves / 32 floats; channel-major or channel-minor tensors).
 //
 //   Y[(b,y,x)][co] = sum over taps (ky,kx) and channels c of  Xp[b][c][y+ky][x+kx] * W[co][c][ky][kx]
 //
@@ -10,6 +10,8 @@
 //     one constant to every address - no border tests, no im2col;
 //   * the filters as [co][tap][c], so that k = (tap, c) is contiguous.
 // The GEMM kernel then runs its ordinary slab loop over k = taps x channels with one pointer jump per tap.
+// A channel-minor input [b][y][x][c] only needs its zero halo: [b][yp][xp][c] is the same kind of matrix with
+// the channels of a pixel contiguous (a slab of k is 128 consecutive bytes) and a tap shift of C elements.
 // The input gradient is the same product over the (padded) output gradient with flipped, transposed filters;
 // the filter pass reads them through the strides of the descriptor.
 #include "ptl_conv_tile.hpp"
@@ -67,6 +69,19 @@ static int blocked_padded_copy(const T *X, uint4 *xb, const ConvTileDesc &d, int
     return hip_ok(hipGetLastError(), "blocked layout launch") ? 0 : 2;
 }
 
+// in: [b][H][W][C] as 16-byte chunks (cblocks per pixel) -> out: [b][Hp][Wp][C], zero halo.
+__device__ inline void hwc_to_padded(unsigned block, const uint4 *__restrict__ in, uint4 *__restrict__ out, int H,
+                                     int W, int Hp, int Wp, int padU, int padL, int cblocks, long long total) {
+    const unsigned i = block * 256u + threadIdx.x;
+    if (i >= total) return;
+    const unsigned pix = i / (unsigned)cblocks, cc = i - pix * cblocks;
+    const unsigned r = pix / (unsigned)Wp, b = r / (unsigned)Hp;
+    const int y = (int)(r - b * Hp) - padU, x = (int)(pix - r * Wp) - padL;
+    uint4 v = make_uint4(0, 0, 0, 0);
+    if (y >= 0 && y < H && x >= 0 && x < W) v = in[((b * H + y) * W + x) * cblocks + cc];
+    out[i] = v;
+}
+
 // out[m][tap][c] = W[base + m*sm + c*sc + ky*sy + kx*sx]
 template <typename T>
 __device__ inline void filters_tap_major(unsigned block, const T *__restrict__ w, T *__restrict__ out, int C, int KW,
@@ -86,7 +101,7 @@ __device__ inline void filters_tap_major(unsigned block, const T *__restrict__ w
 struct TapPrepArgs {
     const void *in;
     uint4 *xb;
-    int B, H, W, Hp, Wp, padU, padL, cblocks;
+    int B, H, W, Hp, Wp, padU, padL, cblocks, hwc;
     long long sb, sc, xb_total;
     unsigned copy_blocks;
     const void *w;
@@ -96,7 +111,10 @@ struct TapPrepArgs {
 };
 template <typename T>
 __global__ __launch_bounds__(256) void tap_prepare_kernel(const TapPrepArgs a) {
-    if (blockIdx.x < a.copy_blocks)
+    if (blockIdx.x < a.copy_blocks && a.hwc)
+        hwc_to_padded(blockIdx.x, reinterpret_cast<const uint4 *>(a.in), a.xb, a.H, a.W, a.Hp, a.Wp, a.padU, a.padL,
+                      a.cblocks, a.xb_total);
+    else if (blockIdx.x < a.copy_blocks)
         chw_to_blocked_padded<T>(blockIdx.x, reinterpret_cast<const T *>(a.in), a.xb, a.B, a.H, a.W, a.Hp, a.Wp, a.padU,
                                  a.padL, a.sb, a.sc, a.cblocks, a.xb_total);
     else
@@ -108,7 +126,9 @@ template <typename T>
 int conv_taps(const ConvTileDesc &d, const void *X, const void *Wt, void *Y, const OutMap &c) {
     State &st = state();
     constexpr int ES = (int)sizeof(T), VEC = 16 / ES, SK = 128 / ES;
-    if (d.in_hwc || d.sh != 1 || d.sw != 1 || d.Cin % SK || d.x_sy != d.Win) return -1;
+    const bool hwc = d.in_hwc != 0;
+    if (d.sh != 1 || d.sw != 1 || d.Cin % SK) return -1;
+    if (hwc ? reinterpret_cast<uintptr_t>(X) % 16 != 0 : d.x_sy != d.Win) return -1;
     const int Hp = d.Hin + d.padU + d.padD, Wp = d.Win + d.padL + d.padR, taps = d.KH * d.KW;
     if (d.Ho != Hp - d.KH + 1 || d.Wo != Wp - d.KW + 1 || taps < 2) return -1;
     const int cblocks = d.Cin / VEC;
@@ -136,6 +156,7 @@ int conv_taps(const ConvTileDesc &d, const void *X, const void *Wt, void *Y, con
         p.xb = xb;
         p.B = d.batch; p.H = d.Hin; p.W = d.Win; p.Hp = Hp; p.Wp = Wp; p.padU = d.padU; p.padL = d.padL;
         p.cblocks = cblocks;
+        p.hwc = hwc;
         p.sb = d.x_sb; p.sc = d.x_sc;
         p.xb_total = xb_elems / VEC;
         p.copy_blocks = (unsigned)((p.xb_total + 255) / 256);
@@ -157,16 +178,19 @@ int conv_taps(const ConvTileDesc &d, const void *X, const void *Wt, void *Y, con
     q.M = d.Cout;
     q.K = taps * d.Cin;
     q.a.HL = q.a.WL = q.b.HL = q.b.WL = 1;
-    // pixel (b, y, x) of the padded, blocked input; a 16-byte chunk further along k is one block plane on
+    // row = pixel (b, y, x) of the padded input
     q.a.row = {};
     q.a.row.n = q.N;
     q.a.row.d1 = d.Ho;
     q.a.row.d0 = d.Wo;
-    q.a.row.o2 = (int)plane;
-    q.a.row.o1 = Wp * VEC;
-    q.a.row.o0 = VEC;
-    const long long kstride = (long long)d.batch * plane / VEC;  // per channel, so that VEC channels = one plane
-    if (kstride >= ((long long)1 << 31) || plane >= ((long long)1 << 31)) return -1;
+    // per sample / padded row / pixel; a 16-byte chunk further along k is one block plane on (channel-major) or
+    // the next 16 bytes (channel-minor)
+    const long long sample = (long long)Hp * Wp * d.Cin, pix_shift = hwc ? d.Cin : VEC;
+    const long long kstride = hwc ? 1 : (long long)d.batch * plane / VEC;  // per channel
+    if (kstride >= ((long long)1 << 31) || sample >= ((long long)1 << 31)) return -1;
+    q.a.row.o2 = hwc ? (int)sample : (int)plane;
+    q.a.row.o1 = Wp * (int)pix_shift;
+    q.a.row.o0 = (int)pix_shift;
     q.a.k = axis_plain(q.K, (int)kstride);
     q.a.mode = FILL_VEC_K;
     q.b.row = axis_plain(d.Cout, q.K);
@@ -177,8 +201,8 @@ int conv_taps(const ConvTileDesc &d, const void *X, const void *Wt, void *Y, con
     q.slabs_per_tap = d.Cin / SK;
     q.tap_kw = d.KW;
     const long long tap_span = (long long)q.slabs_per_tap * SK * kstride * ES;  // what the slabs of a tap advance A by
-    q.tap_jump_x = (long long)VEC * ES - tap_span;
-    q.tap_jump_y = (long long)(Wp - (d.KW - 1)) * VEC * ES - tap_span;
+    q.tap_jump_x = pix_shift * ES - tap_span;
+    q.tap_jump_y = (long long)(Wp - (d.KW - 1)) * pix_shift * ES - tap_span;
     return gemm_async<T>(q);
 }
 

@@ -342,6 +342,31 @@ def test_conv2d_wide_layers_against_torch(pkg, gpu, case):
         assert err <= 2e-3, (name, err)
 
 
+@pytest.mark.parametrize("case", [(64, 64, 56, 8), (128, 128, 28, 16), (256, 256, 14, 32), (64, 128, 12, 64),
+                                  (128, 64, 9, 128)])
+def test_conv2d_wide_layers_hwc_against_torch(pkg, gpu, case):
+    """Channel-minor (HWC) wide 3x3 layers, fp16: forward and input gradient on the sum over taps of the padded
+    input, weight gradient on whatever route it takes, against torch's fp32 convolution of the same tensors."""
+    Ci, Co, H, ns = case
+    x = dev(hp.uniform(41, (ns, H, H, Ci), dtype=np.float16))
+    w = dev(hp.uniform(42, (Co, 3, 3, Ci), -0.1, 0.1).astype(np.float16))
+    dy = dev(hp.uniform(43, (ns, H, H, Co), dtype=np.float16))
+    y, dx, dw = torch.full_like(dy, 3.0), torch.full_like(x, 3.0), torch.full_like(w, 3.0)
+    a, keep = hp.conv2d_args(pkg, x, dx, w, dw, y, dy, Ci, H, H, Co, 3, 3, H, H, (1, 1, 1, 1), (1, 1), 1)
+    for s in ("fw", "wg", "ig"):
+        pkg.call("ptl_conv2d_fp16_%s_batched" % s, a, ns)
+        if s != "wg":
+            assert gpu.ptl_last_conv_direct() == 1
+    sync(gpu)
+    xf, wf, dyf = (t.float().permute(0, 3, 1, 2).contiguous() for t in (x, w, dy))
+    ref_y = torch.nn.functional.conv2d(xf, wf, padding=1).permute(0, 2, 3, 1)
+    ref_dw = torch.nn.grad.conv2d_weight(xf, wf.shape, dyf, padding=1).permute(0, 2, 3, 1)
+    ref_dx = torch.nn.grad.conv2d_input(xf.shape, wf, dyf, padding=1).permute(0, 2, 3, 1)
+    for name, got, ref in (("y", y, ref_y), ("dw", dw, ref_dw), ("dx", dx, ref_dx)):
+        err = ((got.float() - ref).norm() / ref.norm()).item()
+        assert err <= 2e-3, (name, err)
+
+
 @pytest.mark.parametrize("case", [(256, 256, 14, 24), (128, 128, 28, 8), (256, 128, 9, 40)])
 def test_conv2d_wide_weight_gradient_routes_against_torch(pkg, gpu, case):
     """The weight gradient of a wide layer on each of its routes (default choice, resident-tile kernel, sum over
