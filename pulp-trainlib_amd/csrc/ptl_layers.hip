@@ -343,8 +343,9 @@ static int conv2d_wg(const Args *a, int ns, const char *fn) {
 
     int rc = -1;
     state().last_conv_direct = 0;
-    if (!g.hwc && state().gemm_path != 1) {
+    if (state().gemm_path != 1) {
         ConvTileDesc d = {};
+        d.in_hwc = g.hwc ? 1 : 0;
         d.batch = ns; d.Cin = g.Ci; d.Hin = g.H; d.Win = g.W;
         d.Cout = g.Co; d.Ho = g.Ho; d.Wo = g.Wo;
         d.KH = g.Hk; d.KW = g.Wk; d.sh = g.sh; d.sw = g.sw;
@@ -355,9 +356,13 @@ static int conv2d_wg(const Args *a, int ns, const char *fn) {
         // (measured at batch 128..512: 82 against 93 us for 256 -> 256 on 14x14, 455 against 533 us on 28x28,
         // 133 against 145 us for 128 -> 256 on 28x28; 128 -> 128 stays with the tile kernel: 87 / 291 against 87 / 317 us)
         const bool taps_first = d.Cin >= 128 && d.Cout >= 128 && (d.Cin >= 256 || d.Cout >= 256);
-        if (state().gemm_path == 3 || (taps_first && state().gemm_path != 2)) rc = conv_taps_wg<T>(d, X, dY, dW);
-        if (rc < 0) rc = conv_tile_wg<T>(d, X, dY, dW);
-        if (rc < 0 && state().gemm_path != 3) rc = conv_taps_wg<T>(d, X, dY, dW);
+        if (g.hwc) {  // channel-minor tensors: the sum over taps from 64 channels on, else the gathering GEMM below
+            rc = conv_taps_wg<T>(d, X, dY, dW);
+        } else {
+            if (state().gemm_path == 3 || (taps_first && state().gemm_path != 2)) rc = conv_taps_wg<T>(d, X, dY, dW);
+            if (rc < 0) rc = conv_tile_wg<T>(d, X, dY, dW);
+            if (rc < 0 && state().gemm_path != 3) rc = conv_taps_wg<T>(d, X, dY, dW);
+        }
         if (rc > 0) return sg.finish(rc);
         if (rc == 0) state().last_conv_direct = 1;
     }
