@@ -343,6 +343,19 @@ def detail_table(pkg, lib, hp, to_dev, timed, check, torch, dev):
         run3("ptl_conv2d", dt, a, ns, "conv2d %d->%d %dx%d k3 p1" % (Ci, Co, H, H), flops, (nb, nb, nb), 10)
         del x, w, dy, y, dx, dw
 
+    # the same wide layers with channel-minor (HWC) tensors: X[b][h][w][ci], W[co][kh][kw][ci], Y[b][h][w][co]
+    for (ns, Ci, Co, H) in ((128, 64, 64, 56), (128, 128, 128, 28), (128, 256, 256, 14)):
+        K, dt = 3, "fp16"
+        x = torch.rand(ns, H, H, Ci, device=dev).to(tdt[dt]) - 0.5
+        w = torch.rand(Co, K, K, Ci, device=dev).to(tdt[dt]) - 0.5
+        dy = torch.rand(ns, H, H, Co, device=dev).to(tdt[dt]) - 0.5
+        y, dx, dw = torch.zeros_like(dy), torch.zeros_like(x), torch.zeros_like(w)
+        a, keep = hp.conv2d_args(pkg, x, dx, w, dw, y, dy, Ci, H, H, Co, K, K, H, H, (1, 1, 1, 1), (1, 1), 1)
+        flops = 2.0 * ns * Co * Ci * K * K * H * H
+        nb = (x.numel() + w.numel() + y.numel()) * es[dt]
+        run3("ptl_conv2d", dt, a, ns, "conv2d HWC %d->%d %dx%d k3 p1" % (Ci, Co, H, H), flops, (nb, nb, nb), 10)
+        del x, w, dy, y, dx, dw
+
     # config 4: multi-head self-attention step, fp32, L=197 E=192, 3 heads of 64, batch 1 and 32
     import numpy as np
     L, E, F, heads = 197, 192, 192, 3
