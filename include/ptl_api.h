@@ -154,6 +154,28 @@ void naive_conv2d_fw_kernel_CHW_fp16(void *matMul_args_fp16);
 void naive_conv2d_param_grad_kernel_CHW_fp16(void *matMul_args_fp16);
 void naive_conv2d_in_grad_kernel_CHW_fp16(void *matMul_args_fp16);
 
+/* The same kernels with the geometry fixed by the name: 3x3 or 5x5 filter, stride 2, padding 1 on every side
+ * (only H, W, pCin, pCout, the pointers and the bias fields of the struct are read):
+ * lib/sources/pulp_conv_naive_fp32.c:520, :581, :643, :702, :762, :825;
+ * lib/sources/pulp_conv_naive_fp16.c:471, :529, :588, :645, :703, :756. */
+void naive_conv2d_fw_kernel_CHW_k3x3_s2_p1(void *matMul_args);
+void naive_conv2d_param_grad_kernel_CHW_k3x3_s2_p1(void *matMul_args);
+void naive_conv2d_in_grad_kernel_CHW_k3x3_s2_p1(void *matMul_args);
+void naive_conv2d_fw_kernel_CHW_k5x5_s2_p1(void *matMul_args);
+void naive_conv2d_param_grad_kernel_CHW_k5x5_s2_p1(void *matMul_args);
+void naive_conv2d_in_grad_kernel_CHW_k5x5_s2_p1(void *matMul_args);
+void naive_conv2d_fw_kernel_CHW_k3x3_s2_p1_fp16(void *matMul_args_fp16);
+void naive_conv2d_param_grad_kernel_CHW_k3x3_s2_p1_fp16(void *matMul_args_fp16);
+void naive_conv2d_in_grad_kernel_CHW_k3x3_s2_p1_fp16(void *matMul_args_fp16);
+void naive_conv2d_fw_kernel_CHW_k5x5_s2_p1_fp16(void *matMul_args_fp16);
+void naive_conv2d_param_grad_kernel_CHW_k5x5_s2_p1_fp16(void *matMul_args_fp16);
+void naive_conv2d_in_grad_kernel_CHW_k5x5_s2_p1_fp16(void *matMul_args_fp16);
+
+/* Bias add on a row-major H x W matrix (t == 0: bias[column], else bias[row]), the epilogue mm_manager runs
+ * when USE_BIASES == 1: lib/sources/pulp_train_utils_fp32.c:1286, lib/include/pulp_train_utils_fp16.h:783. */
+void mm_bias_add_transposed(void *mm_bias_add_args);
+void mm_bias_add_transposed_fp16(void *mm_bias_add_args_fp16);
+
 /* Depthwise kernels: lib/sources/pulp_conv_naive_fp32.c:29, :113, :153;
  * lib/sources/pulp_conv_naive_fp16.c:32, :75, :118 */
 void dw_kernel_forward(void *kernel_DW_args);

@@ -340,6 +340,24 @@ struct mm_manager_args_fp16 {
     int matmul_type;
 };
 
+/* lib/include/pulp_train_utils_fp32.h:569-575 */
+struct mm_bias_add_args {
+    float *mat;
+    float *bias;
+    int H;
+    int W;
+    int t;
+};
+
+/* lib/include/pulp_train_utils_fp16.h:524-530 */
+struct mm_bias_add_args_fp16 {
+    fp16 *mat;
+    fp16 *bias;
+    int H;
+    int W;
+    int t;
+};
+
 /* lib/include/pulp_conv2d_fp32.h:50-72 */
 struct Conv2D_args {
     struct blob *input;

@@ -37,6 +37,9 @@ VOID_ENTRY_POINTS = [
     "naive_conv2d_fw_kernel_CHW", "naive_conv2d_param_grad_kernel_CHW", "naive_conv2d_in_grad_kernel_CHW",
     "naive_conv2d_fw_kernel_CHW_fp16", "naive_conv2d_param_grad_kernel_CHW_fp16",
     "naive_conv2d_in_grad_kernel_CHW_fp16",
+] + ["naive_conv2d_%s_kernel_CHW_k%dx%d_s2_p1%s" % (step, k, k, sfx) for sfx in ("", "_fp16") for k in (3, 5)
+     for step in ("fw", "param_grad", "in_grad")] + [
+    "mm_bias_add_transposed", "mm_bias_add_transposed_fp16",
     "dw_kernel_forward", "dw_kernel_weight_grad", "dw_kernel_input_grad", "dw_kernel_forward_fp16",
     "dw_kernel_weight_grad_fp16", "dw_kernel_input_grad_fp16",
     "pulp_im2row_fp32", "pulp_im2col_fp32", "pulp_blocktransp_fp32", "pulp_im2row_fp16", "pulp_im2col_fp16",

@@ -420,7 +420,10 @@ static int conv2d_ig(const Args *a, int ns, const char *fn) {
     // get a gradient, dX[ci][sh*u][sw*v] = sum_co W[co][ci] dY[co][u][v] - one plain product written through a
     // strided output map into the zeroed tensor (the general route below would run a stride-1 pass over a
     // zero-stuffed gradient four times the size: measured 32 against 11 us for 16 -> 32 channels, 32x32, batch 128).
-    if (Pk == 1 && (g.sh != 1 || g.sw != 1) && g.Up == 0 && g.Lp == 0 && state().gemm_path != 1) {
+    // With bottom / right padding the last output rows or columns sit on padded positions outside the input;
+    // the scatter map has no coordinate test, so such geometries take the general route below.
+    const bool taps_inside = (long long)(g.Ho - 1) * g.sh < g.H && (long long)(g.Wo - 1) * g.sw < g.W;
+    if (Pk == 1 && (g.sh != 1 || g.sw != 1) && g.Up == 0 && g.Lp == 0 && taps_inside && state().gemm_path != 1) {
         const int vec = reinterpret_cast<uintptr_t>(dX) % 16 == 0;
         const size_t threads = vec ? (in_n + 16 / sizeof(T) - 1) / (16 / sizeof(T)) : in_n;
         hipLaunchKernelGGL((zero_kernel<T>), dim3(blocks_for(threads)), dim3(256), 0, state().stream, dX, in_n, vec);

@@ -447,6 +447,51 @@ void naive_conv2d_in_grad_kernel_CHW_fp16(void *p) {
     ptl_internal_set_status(ptl_conv2d_fp16_ig_batched(&a, 1));
 }
 
+/* Fixed-geometry variants: 3x3 or 5x5 filter, stride 2, one row / column of padding on every side
+ * (lib/sources/pulp_conv_naive_fp32.c:520, :581, :643, :702, :762, :825; pulp_conv_naive_fp16.c:471-756).
+ * They read only H, W, pCin, pCout, the pointers and the bias fields of the struct; the geometry is in the name. */
+#define PTL_FIXED_GEOMETRY(NAME, GENERIC, STRUCT, KSIZE)                                   \
+    void NAME(void *p) {                                                                   \
+        struct STRUCT m;                                                                   \
+        if (!p) { ptl_internal_set_status(1); return; }                                    \
+        m = *(const struct STRUCT *)p;                                                     \
+        m.pH = m.pW = (KSIZE);                                                             \
+        m.stride_h = m.stride_w = 2;                                                       \
+        m.Lpad = m.Rpad = m.Upad = m.Dpad = 1;                                             \
+        GENERIC(&m);                                                                       \
+    }
+
+PTL_FIXED_GEOMETRY(naive_conv2d_fw_kernel_CHW_k3x3_s2_p1, naive_conv2d_fw_kernel_CHW, matMul_args, 3)
+PTL_FIXED_GEOMETRY(naive_conv2d_param_grad_kernel_CHW_k3x3_s2_p1, naive_conv2d_param_grad_kernel_CHW, matMul_args, 3)
+PTL_FIXED_GEOMETRY(naive_conv2d_in_grad_kernel_CHW_k3x3_s2_p1, naive_conv2d_in_grad_kernel_CHW, matMul_args, 3)
+PTL_FIXED_GEOMETRY(naive_conv2d_fw_kernel_CHW_k5x5_s2_p1, naive_conv2d_fw_kernel_CHW, matMul_args, 5)
+PTL_FIXED_GEOMETRY(naive_conv2d_param_grad_kernel_CHW_k5x5_s2_p1, naive_conv2d_param_grad_kernel_CHW, matMul_args, 5)
+PTL_FIXED_GEOMETRY(naive_conv2d_in_grad_kernel_CHW_k5x5_s2_p1, naive_conv2d_in_grad_kernel_CHW, matMul_args, 5)
+PTL_FIXED_GEOMETRY(naive_conv2d_fw_kernel_CHW_k3x3_s2_p1_fp16, naive_conv2d_fw_kernel_CHW_fp16, matMul_args_fp16, 3)
+PTL_FIXED_GEOMETRY(naive_conv2d_param_grad_kernel_CHW_k3x3_s2_p1_fp16, naive_conv2d_param_grad_kernel_CHW_fp16,
+                   matMul_args_fp16, 3)
+PTL_FIXED_GEOMETRY(naive_conv2d_in_grad_kernel_CHW_k3x3_s2_p1_fp16, naive_conv2d_in_grad_kernel_CHW_fp16,
+                   matMul_args_fp16, 3)
+PTL_FIXED_GEOMETRY(naive_conv2d_fw_kernel_CHW_k5x5_s2_p1_fp16, naive_conv2d_fw_kernel_CHW_fp16, matMul_args_fp16, 5)
+PTL_FIXED_GEOMETRY(naive_conv2d_param_grad_kernel_CHW_k5x5_s2_p1_fp16, naive_conv2d_param_grad_kernel_CHW_fp16,
+                   matMul_args_fp16, 5)
+PTL_FIXED_GEOMETRY(naive_conv2d_in_grad_kernel_CHW_k5x5_s2_p1_fp16, naive_conv2d_in_grad_kernel_CHW_fp16,
+                   matMul_args_fp16, 5)
+
+/* Bias add on a row-major H x W matrix: t == 0 adds bias[column], otherwise bias[row]
+ * (lib/sources/pulp_train_utils_fp32.c:1286-1324, pulp_train_utils_fp16.c twin). */
+void mm_bias_add_transposed(void *p) {
+    struct mm_bias_add_args *a = (struct mm_bias_add_args *)p;
+    if (!a) { ptl_internal_set_status(1); return; }
+    ptl_internal_set_status(ptl_internal_bias_add_fp32(a->mat, a->bias, a->H, a->W, a->t != 0));
+}
+
+void mm_bias_add_transposed_fp16(void *p) {
+    struct mm_bias_add_args_fp16 *a = (struct mm_bias_add_args_fp16 *)p;
+    if (!a) { ptl_internal_set_status(1); return; }
+    ptl_internal_set_status(ptl_internal_bias_add_fp16(a->mat, a->bias, a->H, a->W, a->t != 0));
+}
+
 /* ---- Multi-head self-attention (lib/sources/pulp_mhsa_fp32.c:20, :648) and the row softmax
  * (lib/sources/pulp_act_fp32.c:187, :335) ------------------------------------------------- */
 

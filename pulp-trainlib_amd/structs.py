@@ -82,6 +82,10 @@ class MMManagerArgs(C.Structure):
                 ("matmul_type", I)]
 
 
+class MMBiasAddArgs(C.Structure):
+    _fields_ = [("mat", P), ("bias", P), ("H", I), ("W", I), ("t", I)]
+
+
 class Conv2DArgs(C.Structure):
     _fields_ = [("input", BlobP), ("coeff", BlobP), ("bias", BlobP), ("output", BlobP),
                 ("Lpad", I), ("Rpad", I), ("Upad", I), ("Dpad", I), ("stride_h", I), ("stride_w", I),

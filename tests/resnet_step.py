@@ -56,6 +56,7 @@ class ResNetStep:
         self.G, self.dG, self.Bt, self.dBt = {}, {}, {}, {}  # scale / shift of the normalisation layers
         eps = torch.full((1,), 1e-5, dtype=tdt, device="cuda")
         self.fw, self.bw = [], []  # lists of (function name, struct, extra args)
+        self.conv_layers, self.norm_layers = [], []  # the tensors each such layer reads and writes (for per-layer checks)
         spec = {n: (ci, co, k, s) for n, ci, co, k, s in convs}
         L = lambda name: name.replace("DT", dt)
 
@@ -69,6 +70,8 @@ class ResNetStep:
             a, kp = hp.conv2d_args(pkg, x, dx, self.W[name], self.dW[name], y, dy, ci, H, H, co, k, k, Ho, Ho,
                                    (p, p, p, p), (s, s), 0, 1 if s == 1 else 0)
             self.keep.append(kp)
+            self.conv_layers.append(dict(name=name, x=x, dx=dx, w=self.W[name], dw=self.dW[name], y=y, dy=dy,
+                                         stride=s, pad=p))
             fw = [(L("ptl_conv2d_DT_fw_batched"), a, (ns,))]
             bw = [(L("ptl_conv2d_DT_wg_batched"), a, (ns,))]
             if dx is not None:
@@ -80,6 +83,8 @@ class ResNetStep:
                 na, kp = hp.batch_norm_args(pkg, y, n_, self.G[name], self.Bt[name], eps, ns, co, Ho, Ho, dy, dn_,
                                             self.dG[name], self.dBt[name])
                 self.keep.append(kp)
+                self.norm_layers.append(dict(name=name, x=y, dx=dy, y=n_, dy=dn_, g=self.G[name], b=self.Bt[name],
+                                             dg=self.dG[name], db=self.dBt[name]))
                 fw.append((L("ptl_batch_norm_DT_fw"), na, ()))
                 bw.insert(0, (L("ptl_batch_norm_DT_bw"), na, ()))
                 y, dy = n_, dn_
@@ -130,11 +135,14 @@ class ResNetStep:
                 b += [(L("ptl_residual_DT_batched"), cp, (ns, 2))] + bs + [self._vect_sum(dxin, dproj)]  # dxin += dproj
             else:
                 b.append((L("ptl_residual_DT_batched"), sk, (ns, 1)))  # dxin += ds (identity shortcut)
+            # what the shortcut adds to the buffer the first convolution's input gradient was written to
+            next(l for l in self.conv_layers if l["name"] == n + "c1")["dx_extra"] = dproj if proj else ds_
             bw_blocks.append(b)
         pooled, dpooled = z(ns, 64), z(ns, 64)
         pa, kp = hp.pool_args(pkg, t, dt_, pooled, dpooled, 64, H, H, 1, 1, H, H, H, H)
         self.keep.append(kp)
         self.logits, dlogits = z(ns, ncls), z(ns, ncls)
+        self.pooled, self.dpooled, self.dlogits = pooled, dpooled, dlogits
         la, kp = hp.linear_args(pkg, pooled, dpooled, self.W["fc"], self.dW["fc"], self.logits, dlogits, 64, ncls)
         self.keep.append(kp)
         self.target, self.loss = z(ns, ncls), z(ns)

@@ -41,7 +41,8 @@ STRUCTS = {
     "set_to_value_args_fp16": "SetToValueArgsFp16", "vect_sum_args": "VectSumArgs", "cast_16t32_args": "CastArgs",
     "cast_32t16_args": "CastArgs", "pad_args": "PadArgs", "pad_args_fp16": "PadArgs", "matMul_args": "MatMulArgs",
     "matMul_args_fp16": "MatMulArgs", "kernel_DW_args": "KernelDWArgs", "kernel_DW_args_fp16": "KernelDWArgsFp16",
-    "mm_manager_args": "MMManagerArgs", "mm_manager_args_fp16": "MMManagerArgs", "Conv2D_args": "Conv2DArgs",
+    "mm_manager_args": "MMManagerArgs", "mm_manager_args_fp16": "MMManagerArgs",
+    "mm_bias_add_args": "MMBiasAddArgs", "mm_bias_add_args_fp16": "MMBiasAddArgs", "Conv2D_args": "Conv2DArgs",
     "Conv2D_args_fp16": "Conv2DArgs", "PointWise_Conv_args": "PointWiseConvArgs",
     "PointWise_Conv_args_fp16": "PointWiseConvArgs", "DepthWise_Conv_args": "DepthWiseConvArgs",
     "DepthWise_Conv_args_fp16": "DepthWiseConvArgsFp16", "Linear_args": "LinearArgs", "Linear_args_fp16": "LinearArgs",

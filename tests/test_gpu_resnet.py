@@ -12,32 +12,32 @@ import resnet_step as rs
 pytestmark = pytest.mark.gpu
 
 
-def torch_step(weights, x, target, lr, norm=False, stored=None):
+def torch_step(weights, x, target, lr, norm=False, stored=None, device="cpu"):
     """`stored`: the type every tensor that the library materialises is rounded to on the way forward (the
     rounding passes gradients through unchanged), so that a float64 reference sees the activations - and with
     them the ReLU masks - that an fp16 run sees."""
     q = (lambda t: t.to(stored).to(torch.float64)) if stored is not None else (lambda t: t)
     convs, blocks, ncls = rs.resnet20_spec()
-    p = {n: torch.tensor(v.astype(np.float64), requires_grad=True) for n, v in weights.items()}
+    p = {n: torch.tensor(v.astype(np.float64), requires_grad=True, device=device) for n, v in weights.items()}
     if norm:
         for n, ci, co, k, s in convs:
-            p["g:" + n] = torch.ones(co, dtype=torch.float64, requires_grad=True)
-            p["b:" + n] = torch.zeros(co, dtype=torch.float64, requires_grad=True)
+            p["g:" + n] = torch.ones(co, dtype=torch.float64, requires_grad=True, device=device)
+            p["b:" + n] = torch.zeros(co, dtype=torch.float64, requires_grad=True, device=device)
 
     def conv(t, n, **kw):
         y = q(F.conv2d(t, p[n], **kw))
         return q(F.batch_norm(y, None, None, p["g:" + n], p["b:" + n], training=True, eps=1e-5)) if norm else y
 
-    t = F.relu(conv(torch.tensor(x.astype(np.float64)), "stem", padding=1))
+    t = F.relu(conv(torch.tensor(x.astype(np.float64), device=device), "stem", padding=1))
     for (n, ci, co, stride, proj) in blocks:
         y = conv(F.relu(conv(t, n + "c1", stride=stride, padding=1)), n + "c2", padding=1)
         sc = conv(t, proj, stride=stride) if proj else t
         t = F.relu(q(y + sc))
     logits = t.mean((2, 3)) @ p["fc"].t()
-    loss = F.cross_entropy(logits, torch.tensor(target.astype(np.float64)), reduction="none")
+    loss = F.cross_entropy(logits, torch.tensor(target.astype(np.float64), device=device), reduction="none")
     loss.sum().backward()
-    return logits.detach().numpy(), loss.detach().numpy(), {n: v.grad.numpy() for n, v in p.items()}, \
-        {n: (v.detach() - lr * v.grad).numpy() for n, v in p.items()}
+    return logits.detach().cpu().numpy(), loss.detach().cpu().numpy(), {n: v.grad.cpu().numpy() for n, v in p.items()}, \
+        {n: (v.detach() - lr * v.grad).cpu().numpy() for n, v in p.items()}
 
 
 @pytest.mark.parametrize("dt,ns,tol", [("fp32", 3, 2e-4), ("fp16", 4, 8e-2)])
