@@ -12,12 +12,13 @@ void set_status(int s);
 int init_device(int device);
 
 // Maps caller pointers to device pointers.  Device pointers pass through;
-// host pointers get a temporary device buffer that is filled before the
-// kernels run (copy_in) and copied back by finish() (copy_out).  finish()
-// synchronises only when something was staged.
+// host pointers get a device buffer from a pool kept between calls, filled
+// before the kernels run (copy_in) and copied back by finish() (copy_out).
+// finish() synchronises only when something was staged.
 class Stager {
    public:
-    Stager() = default;
+    // device_only: host pointers are rejected instead of staged (callers that may not allocate)
+    explicit Stager(bool device_only = false) : device_only_(device_only) {}
     ~Stager();
     Stager(const Stager &) = delete;
     Stager &operator=(const Stager &) = delete;
@@ -35,6 +36,7 @@ class Stager {
         return static_cast<T *>(map(p, n * sizeof(T), true, true));
     }
     bool failed() const { return failed_; }
+    bool rejected() const { return rejected_; }  // failed because of the arguments, not because of HIP
     int finish(int rc);
 
    private:
@@ -43,10 +45,14 @@ class Stager {
         void *dev;
         size_t bytes;
         bool copy_out;
+        bool copied_in;
     };
     void *map(const void *p, size_t bytes, bool copy_in, bool copy_out);
     std::vector<Item> items_;
     bool failed_ = false;
+    bool finished_ = false;
+    bool device_only_ = false;
+    bool rejected_ = false;
 };
 
 }  // namespace ptl

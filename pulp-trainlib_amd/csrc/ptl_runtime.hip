@@ -6,6 +6,8 @@
 #include <stdio.h>
 #include <string.h>
 
+#include <vector>
+
 namespace ptl {
 
 static thread_local char g_err[512] = "";
@@ -83,8 +85,10 @@ static void *grow(void *&buf, size_t &have, size_t want, const char *what) {
     if (want <= have) return buf;
     State &st = state();
     if (buf) {
-        // kernels enqueued earlier may still read the old buffer
-        if (!hip_ok(hipStreamSynchronize(st.stream), "hipStreamSynchronize")) return nullptr;
+        // kernels enqueued earlier - on this stream or on one the caller selected before - may still read the
+        // old buffer
+        (void)st;
+        if (!hip_ok(hipDeviceSynchronize(), "hipDeviceSynchronize")) return nullptr;
         (void)hipFree(buf);
         buf = nullptr;
         have = 0;
@@ -125,43 +129,110 @@ static bool is_device_ptr(const void *p) {
     return attr.type == hipMemoryTypeDevice || attr.type == hipMemoryTypeManaged;
 }
 
+// Device buffers for staged host tensors are kept between calls: a call that stages the same sizes again (a
+// training loop on host arrays) allocates nothing.  A buffer is handed out again only after the call that used
+// it has synchronised its stream (finish(), or the destructor of a Stager that never got there).
+struct StagePool {
+    struct Buf {
+        void *dev;
+        size_t bytes;
+        bool busy;
+    };
+    std::vector<Buf> bufs;
+    size_t total = 0;
+};
+static const size_t STAGE_POOL_LIMIT = (size_t)1 << 30;  // idle buffers beyond this are freed on release
+
+static StagePool &stage_pool() {
+    static StagePool p;
+    return p;
+}
+
+static void *stage_acquire(size_t bytes) {
+    StagePool &p = stage_pool();
+    int best = -1;
+    for (size_t i = 0; i < p.bufs.size(); ++i) {
+        const StagePool::Buf &b = p.bufs[i];
+        if (b.busy || b.bytes < bytes || b.bytes > 2 * bytes + (1u << 20)) continue;
+        if (best < 0 || b.bytes < p.bufs[best].bytes) best = (int)i;
+    }
+    if (best >= 0) {
+        p.bufs[best].busy = true;
+        return p.bufs[best].dev;
+    }
+    void *dev = nullptr;
+    if (!hip_ok(hipMalloc(&dev, bytes), "hipMalloc(staging)")) return nullptr;
+    p.bufs.push_back({dev, bytes, true});
+    p.total += bytes;
+    return dev;
+}
+
+static void stage_release(void *dev) {
+    StagePool &p = stage_pool();
+    for (auto &b : p.bufs)
+        if (b.dev == dev) b.busy = false;
+    // keep the pool bounded: drop idle buffers, largest first
+    while (p.total > STAGE_POOL_LIMIT) {
+        int big = -1;
+        for (size_t i = 0; i < p.bufs.size(); ++i)
+            if (!p.bufs[i].busy && (big < 0 || p.bufs[i].bytes > p.bufs[big].bytes)) big = (int)i;
+        if (big < 0) break;
+        (void)hipFree(p.bufs[big].dev);
+        p.total -= p.bufs[big].bytes;
+        p.bufs.erase(p.bufs.begin() + big);
+    }
+}
+
 Stager::~Stager() {
+    if (items_.empty()) return;
+    // copies or kernels of a call that bailed out early may still be in flight on the buffers
+    if (!finished_) (void)hipStreamSynchronize(state().stream);
     for (auto &t : items_)
-        if (t.dev) (void)hipFree(t.dev);
+        if (t.dev) stage_release(t.dev);
 }
 
 void *Stager::map(const void *host_or_dev, size_t bytes, bool copy_in, bool copy_out) {
     if (failed_) return nullptr;
     if (!host_or_dev) {
         set_error("null tensor pointer");
-        failed_ = true;
+        failed_ = rejected_ = true;
         return nullptr;
     }
     if (bytes == 0) return const_cast<void *>(host_or_dev);
     if (is_device_ptr(host_or_dev)) return const_cast<void *>(host_or_dev);
-    for (auto &t : items_)
-        if (t.host == host_or_dev && t.bytes >= bytes) {
-            t.copy_out = t.copy_out || copy_out;
-            return t.dev;
-        }
-    Item it;
-    it.host = const_cast<void *>(host_or_dev);
-    it.bytes = bytes;
-    it.copy_out = copy_out;
-    it.dev = nullptr;
-    if (!hip_ok(hipMalloc(&it.dev, bytes), "hipMalloc(staging)")) {
-        failed_ = true;
+    if (device_only_) {
+        set_error("host pointer passed to an entry point that may not allocate (staging needs device buffers)");
+        failed_ = rejected_ = true;
         return nullptr;
     }
-    items_.push_back(it);
-    if (copy_in) {
-        if (!hip_ok(hipMemcpyAsync(it.dev, host_or_dev, bytes, hipMemcpyHostToDevice, state().stream),
+    Item *hit = nullptr;
+    for (auto &t : items_)
+        if (t.host == host_or_dev && t.bytes >= bytes) hit = &t;
+    if (!hit) {
+        Item it;
+        it.host = const_cast<void *>(host_or_dev);
+        it.bytes = bytes;
+        it.copy_out = false;
+        it.copied_in = false;
+        it.dev = stage_acquire(bytes);
+        if (!it.dev) {
+            failed_ = true;
+            return nullptr;
+        }
+        items_.push_back(it);
+        hit = &items_.back();
+    }
+    hit->copy_out = hit->copy_out || copy_out;
+    // a tensor first mapped as an output and later as an input still gets its contents
+    if (copy_in && !hit->copied_in) {
+        if (!hip_ok(hipMemcpyAsync(hit->dev, host_or_dev, hit->bytes, hipMemcpyHostToDevice, state().stream),
                     "hipMemcpy(H2D)")) {
             failed_ = true;
             return nullptr;
         }
+        hit->copied_in = true;
     }
-    return it.dev;
+    return hit->dev;
 }
 
 int Stager::finish(int rc) {
@@ -176,6 +247,7 @@ int Stager::finish(int rc) {
             }
     }
     if (!hip_ok(hipStreamSynchronize(st.stream), "hipStreamSynchronize")) failed_ = true;
+    else finished_ = true;
     return failed_ ? 2 : rc;
 }
 
@@ -186,7 +258,14 @@ extern "C" {
 int ptl_init(int device) { return ptl::init_device(device); }
 const char *ptl_last_error(void) { return ptl::last_error(); }
 int ptl_last_status(void) { return ptl::last_status(); }
-void ptl_set_stream(void *s) { ptl::state().stream = static_cast<hipStream_t>(s); }
+// Work already enqueued on the stream being left may still use the library's workspace; the next call would
+// write it from the new stream, so the old stream is drained first (a no-op when it is idle).
+void ptl_set_stream(void *s) {
+    ptl::State &st = ptl::state();
+    hipStream_t next = static_cast<hipStream_t>(s);
+    if (st.ready && next != st.stream) (void)hipStreamSynchronize(st.stream);
+    st.stream = next;
+}
 
 void ptl_set_gemm_path(int path) { ptl::state().gemm_path = path; }
 int ptl_last_conv_direct(void) { return ptl::state().last_conv_direct; }

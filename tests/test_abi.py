@@ -144,3 +144,24 @@ def test_product_does_not_reference_the_oracle():
                     continue
                 text = open(os.path.join(dirpath, f), errors="ignore").read()
                 assert "oracle" not in text.lower() or f == "__init__.py" and "oracle" not in text, (dirpath, f)
+
+
+def test_struct_fields_match_the_reference_headers():
+    """include/ptl_structs.h against tests/golden/struct_fields.json, the (type, name) lists of the reference's
+    own struct declarations (written by tests/golden/make_struct_fields.py from lib/include/*.h): same fields,
+    same order, same types - `fp16` and `float16alt`-style spellings of the 16-bit type aside."""
+    import importlib.util
+    import json
+    spec = importlib.util.spec_from_file_location("make_struct_fields",
+                                                  os.path.join(ROOT, "tests", "golden", "make_struct_fields.py"))
+    mod = importlib.util.module_from_spec(spec)
+    spec.loader.exec_module(mod)
+    mine = mod.struct_fields(open(os.path.join(ROOT, "include", "ptl_structs.h")).read())
+    gold = json.load(open(os.path.join(ROOT, "tests", "golden", "struct_fields.json")))
+    assert set(mine) == set(gold["reference_structs"]) | set(gold["extensions"])
+    assert gold["extensions"] == ["BatchNorm_args_fp16"]
+    norm = lambda t: t.replace("unsigned int", "unsigned").strip()
+    for name, ref in gold["reference_structs"].items():
+        got = [[norm(t), f] for t, f in mine[name]]
+        want = [[norm(t), f] for t, f in ref["fields"]]
+        assert got == want, (name, ref["header"])
