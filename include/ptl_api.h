@@ -289,6 +289,15 @@ int ptl_conv_dw_fp16_fw_batched(const struct DepthWise_Conv_args_fp16 *a, int ns
 int ptl_conv_dw_fp16_wg_batched(const struct DepthWise_Conv_args_fp16 *a, int nsamples);
 int ptl_conv_dw_fp16_ig_batched(const struct DepthWise_Conv_args_fp16 *a, int nsamples);
 
+/* No counterpart in the reference: ptl_conv_dw_fp16_wg_batched for callers that cannot allocate device
+ * memory (code under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc).  Same
+ * arguments, same kernels, same result; the partial sums live in a fixed 1 MiB device array that every call on
+ * a GPU shares (calls that overlap on one GPU race; nothing in it needs clearing between calls).  Every tensor
+ * pointer must be a device pointer, ptl_init() must have run, and a call whose partial sums would not fit
+ * (more than 1 MiB: C x sample groups x taps floats, e.g. 64 x 16 x 9) is rejected with status 1.  Calls no
+ * hipMalloc / hipFree. */
+int ptl_conv_dw_fp16_wg_noalloc(const struct DepthWise_Conv_args_fp16 *a, int nsamples);
+
 int ptl_linear_fp32_fw_batched(const struct Linear_args *a, int nsamples);
 int ptl_linear_fp32_wg_batched(const struct Linear_args *a, int nsamples);
 int ptl_linear_fp32_ig_batched(const struct Linear_args *a, int nsamples);

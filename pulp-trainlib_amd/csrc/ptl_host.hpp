@@ -10,6 +10,7 @@ const char *last_error();
 int last_status();
 void set_status(int s);
 int init_device(int device);
+int dw_noalloc_setup(int device);  // looks up the fixed partial-sum array of the current device
 
 // Maps caller pointers to device pointers.  Device pointers pass through;
 // host pointers get a device buffer from a pool kept between calls, filled

@@ -65,6 +65,7 @@ int init_device(int device) {
         if (!hip_ok(hipMalloc(&st.zeros, 256), "hipMalloc(zeros)")) return 2;
         if (!hip_ok(hipMemset(st.zeros, 0, 256), "hipMemset(zeros)")) return 2;
     }
+    if (int rc = dw_noalloc_setup(device)) return rc;
     st.device = device;
     st.ready = true;
     return 0;

@@ -690,16 +690,48 @@ static void launch_dw_plane(const T *src, const T *Wt, T *dst, int C, int Hs, in
                        C, Hs, Ws, Hd, Wd, pu, pl);
 }
 
+// ---- partial sums of the allocation-free weight-gradient entry point ---------------------------------
+// A fixed array in device memory, one copy per GPU, held until the process ends.  In host code the array's
+// name is only a handle: its device address is looked up once per device (dw_noalloc_setup, called from the
+// library's init) and that pointer is what kernels receive.
+constexpr size_t DW_NOALLOC_BYTES = (size_t)1 << 20;
+constexpr int DW_NOALLOC_MAX_DEVICES = 64;
+static __device__ __align__(256) unsigned char dw_wg_scratch[DW_NOALLOC_BYTES];
+static float *g_dw_wg_scratch_ptr[DW_NOALLOC_MAX_DEVICES] = {};
+
+int dw_noalloc_setup(int device) {
+    if (device < 0 || device >= DW_NOALLOC_MAX_DEVICES) return 0;  // such a device runs the allocating entry points only
+    if (g_dw_wg_scratch_ptr[device]) return 0;
+    void *ptr = nullptr;
+    if (!hip_ok(hipGetSymbolAddress(&ptr, HIP_SYMBOL(dw_wg_scratch)), "hipGetSymbolAddress(dw_wg_scratch)")) return 2;
+    g_dw_wg_scratch_ptr[device] = static_cast<float *>(ptr);
+    return 0;
+}
+
+// `fixed` / `fixed_bytes`: partial sums go to this buffer instead of the growing workspace, tensors must already
+// be in device memory, and the call fails rather than allocate (the allocation-free entry point).
 template <typename T, typename Args>
-static int dw_step(const Args *a, int ns, int step, int sh, int sw, const char *fn) {
+static int dw_step(const Args *a, int ns, int step, int sh, int sw, const char *fn, float *fixed = nullptr,
+                   size_t fixed_bytes = 0) {
     DwGeom g;
     if (int rc = dw_geom(a, g, sh, sw, fn)) return rc;
     if (ns <= 0) return 0;
-    if (!ensure_init()) return 2;
+    if (!fixed && !ensure_init()) return 2;
     State &st = state();
+    bool too_big = false;
+    auto partials = [&](size_t bytes) -> float * {
+        if (!fixed) return workspace(bytes);
+        if (bytes > fixed_bytes) {
+            set_error("%s: the partial sums of this call take %zu bytes, the fixed buffer of the allocation-free "
+                      "entry point holds %zu", fn, bytes, fixed_bytes);
+            too_big = true;
+            return nullptr;
+        }
+        return fixed;
+    };
     size_t in_n = (size_t)ns * g.C * g.H * g.W, out_n = (size_t)ns * g.C * g.Ho * g.Wo;
     size_t w_n = (size_t)g.C * g.Hk * g.Wk;
-    Stager sg;
+    Stager sg(fixed != nullptr);
     int rc = 0;
     // row-walking kernels: unit stride, square 3x3 / 5x5 kernel, rows wide enough to fill a wave
     const bool rows_path = sh == 1 && sw == 1 && g.Hk == g.Wk && (g.Hk == 3 || g.Hk == 5) && g.Wo >= 32 && g.W >= 32;
@@ -716,7 +748,7 @@ static int dw_step(const Args *a, int ns, int step, int sh, int sw, const char *
         const T *X = sg.in(reinterpret_cast<const T *>(a->input->data), in_n);
         const T *Wt = sg.in(reinterpret_cast<const T *>(a->coeff->data), w_n);
         T *Y = sg.out(reinterpret_cast<T *>(a->output->data), out_n);
-        if (sg.failed()) return 2;
+        if (sg.failed()) return sg.rejected() ? 1 : 2;
         if (plane_path) {
             if (g.Hk == 3)
                 launch_dw_plane<T, 3, false>(X, Wt, Y, g.C, g.H, g.W, g.Ho, g.Wo, g.Up, g.Lp, planes, st.stream);
@@ -739,7 +771,7 @@ static int dw_step(const Args *a, int ns, int step, int sh, int sw, const char *
         const T *dY = sg.in(reinterpret_cast<const T *>(a->output->diff), out_n);
         const T *Wt = sg.in(reinterpret_cast<const T *>(a->coeff->data), w_n);
         T *dX = sg.out(reinterpret_cast<T *>(a->input->diff), in_n);
-        if (sg.failed()) return 2;
+        if (sg.failed()) return sg.rejected() ? 1 : 2;
         if (plane_path) {
             if (g.Hk == 3)
                 launch_dw_plane<T, 3, true>(dY, Wt, dX, g.C, g.Ho, g.Wo, g.H, g.W, g.Hk - 1 - g.Up, g.Wk - 1 - g.Lp,
@@ -764,7 +796,7 @@ static int dw_step(const Args *a, int ns, int step, int sh, int sw, const char *
         const T *X = sg.in(reinterpret_cast<const T *>(a->input->data), in_n);
         const T *dY = sg.in(reinterpret_cast<const T *>(a->output->diff), out_n);
         T *dW = sg.out(reinterpret_cast<T *>(a->coeff->diff), w_n);
-        if (sg.failed()) return 2;
+        if (sg.failed()) return sg.rejected() ? 1 : 2;
         const int taps = g.Hk * g.Wk;
         // sample groups: about four workgroups per CU
         int sgroups = (int)((4L * st.num_cu + g.C - 1) / g.C);
@@ -772,8 +804,8 @@ static int dw_step(const Args *a, int ns, int step, int sh, int sw, const char *
         if (sgroups < 1) sgroups = 1;
         const int per_group = (ns + sgroups - 1) / sgroups;
         sgroups = (ns + per_group - 1) / per_group;
-        float *part = workspace((size_t)sgroups * g.C * taps * sizeof(float));
-        if (!part) return sg.finish(2);
+        float *part = partials((size_t)sgroups * g.C * taps * sizeof(float));
+        if (!part) return sg.finish(too_big ? 1 : 2);
         T *direct = sgroups == 1 ? dW : nullptr;  // one group: the kernel writes the gradient, no second launch
         const int x_vecs = (int)((in_img + 15) / 16);
         const size_t lds = (size_t)x_vecs * 16 + out_img;
@@ -805,7 +837,7 @@ static int dw_step(const Args *a, int ns, int step, int sh, int sw, const char *
         const T *X = sg.in(reinterpret_cast<const T *>(a->input->data), in_n);
         const T *dY = sg.in(reinterpret_cast<const T *>(a->output->diff), out_n);
         T *dW = sg.out(reinterpret_cast<T *>(a->coeff->diff), w_n);
-        if (sg.failed()) return 2;
+        if (sg.failed()) return sg.rejected() ? 1 : 2;
         // strips of rows: enough waves to fill the chip, at least 8 rows each
         int ccs = (g.Wo + 63) / 64;
         long want = 8L * st.num_cu * 4;
@@ -816,8 +848,8 @@ static int dw_step(const Args *a, int ns, int step, int sh, int sw, const char *
         rbs = (g.Ho + rows_per - 1) / rows_per;
         long waves = planes * rbs * ccs;
         int taps = g.Hk * g.Wk;
-        float *part = workspace((size_t)waves * taps * sizeof(float));
-        if (!part) return sg.finish(2);
+        float *part = partials((size_t)waves * taps * sizeof(float));
+        if (!part) return sg.finish(too_big ? 1 : 2);
         dim3 grid((unsigned)((waves + 3) / 4));
         if (g.Hk == 3)
             hipLaunchKernelGGL((dw_wg_rows_kernel<T, 3>), grid, dim3(256), 0, st.stream, X, dY, part, g.C, g.H, g.W,
@@ -831,7 +863,7 @@ static int dw_step(const Args *a, int ns, int step, int sh, int sw, const char *
         const T *X = sg.in(reinterpret_cast<const T *>(a->input->data), in_n);
         const T *dY = sg.in(reinterpret_cast<const T *>(a->output->diff), out_n);
         T *dW = sg.out(reinterpret_cast<T *>(a->coeff->diff), w_n);
-        if (sg.failed()) return 2;
+        if (sg.failed()) return sg.rejected() ? 1 : 2;
         size_t n = (size_t)ns * g.Ho * g.Wo;
         // enough chunks for a few workgroups per CU, at least 1024 pixels each
         int chunks = (int)((4 * (size_t)st.num_cu + g.C - 1) / g.C);
@@ -840,8 +872,8 @@ static int dw_step(const Args *a, int ns, int step, int sh, int sw, const char *
         if (chunks < 1) chunks = 1;
         int per = (int)((n + chunks - 1) / chunks);
         chunks = (int)((n + per - 1) / per);
-        float *part = workspace((size_t)chunks * w_n * sizeof(float));
-        if (!part) return sg.finish(2);
+        float *part = partials((size_t)chunks * w_n * sizeof(float));
+        if (!part) return sg.finish(too_big ? 1 : 2);
         int taps = g.Hk * g.Wk;
         dim3 grid(g.C, chunks);
         if (taps <= 9)
@@ -1365,6 +1397,21 @@ int ptl_conv_dw_fp16_fw_batched(const struct DepthWise_Conv_args_fp16 *a, int ns
 }
 int ptl_conv_dw_fp16_wg_batched(const struct DepthWise_Conv_args_fp16 *a, int ns) {
     return ptl::dw_step<half_t>(a, ns, STEP_WGT_GRAD, 1, 1, "pulp_conv_dw_fp16_bw_param_grads_cl");
+}
+
+// Allocation-free twin of ptl_conv_dw_fp16_wg_batched: same kernels, partial sums in the fixed device array.
+int ptl_conv_dw_fp16_wg_noalloc(const struct DepthWise_Conv_args_fp16 *a, int ns) {
+    ptl::State &st = ptl::state();
+    if (!st.ready) {
+        ptl::set_error("ptl_conv_dw_fp16_wg_noalloc: call ptl_init() first (initialisation may allocate, this call may not)");
+        return 1;
+    }
+    float *buf = st.device >= 0 && st.device < ptl::DW_NOALLOC_MAX_DEVICES ? ptl::g_dw_wg_scratch_ptr[st.device] : nullptr;
+    if (!buf) {
+        ptl::set_error("ptl_conv_dw_fp16_wg_noalloc: no fixed buffer on device %d", st.device);
+        return 2;
+    }
+    return ptl::dw_step<half_t>(a, ns, STEP_WGT_GRAD, 1, 1, "ptl_conv_dw_fp16_wg_noalloc", buf, ptl::DW_NOALLOC_BYTES);
 }
 int ptl_conv_dw_fp16_ig_batched(const struct DepthWise_Conv_args_fp16 *a, int ns) {
     return ptl::dw_step<half_t>(a, ns, STEP_IN_GRAD, 1, 1, "pulp_conv_dw_fp16_bw_input_grads_cl");
