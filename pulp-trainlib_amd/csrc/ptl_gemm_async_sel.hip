@@ -134,15 +134,21 @@ int gemm_async(GemmArgs &g) {
                 // one or two slabs deep (pointwise layers): four waves without a k split need half the
                 // LDS for the parked tile, so two workgroups share a CU and overlap load, MFMA and store
                 if (g.splits == 1 && g.K <= 2 * SK) return launch_plain<T, 128, 128, 256, 2, 2, 1, 2, 1>(g, st.stream);
-                // fp16 products large enough to give every CU a 256x128 tile: a third less L2 -> LDS traffic per
-                // MFMA than 128x128, which is what bounds that tile (+15-20 % measured from 4096^3 up)
-                // Either tile holds a CU by itself, so a launch runs in rounds of num_cu workgroups and a 256x128
-                // workgroup takes about 1.7 times as long as a 128x128 one: the tall tile also pays where it
-                // saves a half-empty round (196 tall tiles in one round against 392 square ones in two).
+                // fp16 products large enough to give every CU a larger tile.  Each of these tiles holds a CU by itself,
+                // so a launch runs in rounds of num_cu workgroups; measured per round (4096^3 and 8192^2 x 4096): a
+                // 256x128 workgroup takes 1.7 times as long as a 128x128 one and a 256x256 workgroup 1.8 times as
+                // long as a 256x128 one, for two and four times the work.  The larger tiles move a third / half less
+                // from L2 to LDS and read a quarter less LDS per MFMA (the LDS serves 128 bytes per clock, and fragment
+                // reads alone keep it busy two thirds of the MFMA time on the 128x128 tile); they also pay where they
+                // save a half-empty round (196 tall tiles in one round against 392 square ones in two).
                 if constexpr (sizeof(T) == 2) {
+                    const long r_big = (tiles(256, 256) + st.num_cu - 1) / st.num_cu;
                     const long r_tall = (tiles(256, 128) + st.num_cu - 1) / st.num_cu;
                     const long r_square = (tiles(128, 128) + st.num_cu - 1) / st.num_cu;
-                    if (g.splits == 1 && g.N >= 256 && 17 * r_tall < 10 * r_square)
+                    const long c_big = 306 * r_big, c_tall = 170 * r_tall, c_square = 100 * r_square;
+                    if (g.splits == 1 && g.N >= 256 && g.M >= 256 && c_big < c_tall && c_big < c_square)
+                        return launch_plain<T, 256, 256, 512, 2, 4, 1, 2, 1>(g, st.stream);
+                    if (g.splits == 1 && g.N >= 256 && c_tall < c_square)
                         return launch_plain<T, 256, 128, 512, 4, 2, 1, 3, 1>(g, st.stream);
                 }
                 return launch_plain<T, 128, 128, 512, 2, 2, 2, 3, 1>(g, st.stream);

@@ -19,4 +19,5 @@ template int launch_stream<ptl::half_t, 64, 64, 2>(GemmArgs &, int, hipStream_t)
 template int launch_stream<ptl::half_t, 64, 64, 4>(GemmArgs &, int, hipStream_t);
 template int launch_plain<ptl::half_t, 128, 64, 512, 2, 2, 2, 3, 1>(GemmArgs &, hipStream_t);
 template int launch_plain<ptl::half_t, 256, 128, 512, 4, 2, 1, 3, 1>(GemmArgs &, hipStream_t);
+template int launch_plain<ptl::half_t, 256, 256, 512, 2, 4, 1, 2, 1>(GemmArgs &, hipStream_t);
 }
