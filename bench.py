@@ -36,6 +36,8 @@ def main():
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--no-detail", action="store_true", help="skip the per-shape detail table")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
+    ap.add_argument("--helpers-only", action="store_true",
+                    help="detail table: only the index / streaming helpers (for a counter run of those kernels alone)")
     ap.add_argument("--resnet-only", action="store_true",
                     help="detail table: only the ResNet-20-shaped step (for a kernel trace of that step alone)")
     ap.add_argument("--batch", type=int, default=512, help="samples per step of the headline workload")
@@ -198,7 +200,9 @@ def main():
                                             "(the reference's arithmetic), %.2f s" % (m, ns, reps, t_cpu)}
 
     # ------------------------------------------------------------------------------ detail
-    if args.resnet_only:
+    if args.helpers_only:
+        result["detail"] = helper_rows(pkg, lib, hp, timed, torch, dev)
+    elif args.resnet_only:
         result["detail"] = resnet_rows(pkg, lib, timed, torch, dev)
     elif not args.no_detail:
         result["detail"] = detail_table(pkg, lib, hp, to_dev, timed, check, torch, dev)
@@ -378,7 +382,92 @@ def detail_table(pkg, lib, hp, to_dev, timed, check, torch, dev):
         ms = timed(lambda: check(lib.ptl_mhsa_fp32_bw_batched(ref, ns)), 50)
         add("mhsa L197 E192 3x64 BW N=%d" % ns, "fp32", ms, 2 * f_fw, 2 * act)
 
+    rows += helper_rows(pkg, lib, hp, timed, torch, dev)
     rows += resnet_rows(pkg, lib, timed, torch, dev)
+    return rows
+
+
+def helper_rows(pkg, lib, hp, timed, torch, dev):
+    """The index-permutation and streaming helpers on tensors of 64 MiB and more, priced against HBM: GB/s of the
+    bytes each must read plus the bytes it must write (the layout change is two passes by definition: transpose
+    into the caller's buffer, copy back)."""
+    import ctypes
+    rows = []
+    tdt = {"fp32": torch.float32, "fp16": torch.float16}
+    es = {"fp32": 4, "fp16": 2}
+
+    def add(name, dt, ms, nbytes):
+        gbs = nbytes / (ms * 1e-3) / 1e9
+        rows.append({"workload": name, "dtype": dt, "us": round(ms * 1e3, 2), "GB/s": round(gbs, 1),
+                     "bound_GB/s": HBM_GBS, "frac_of_bound": round(gbs / HBM_GBS, 4)})
+
+    def void_call(name, a):
+        f = getattr(lib, name)
+        ref = ctypes.byref(a)
+
+        def go():
+            f(ref)
+            if lib.ptl_last_status() != 0:
+                raise RuntimeError(lib.ptl_last_error().decode())
+        return go
+
+    for dt, (N, M) in (("fp16", (8192, 4096)), ("fp32", (4096, 4096))):
+        sfx = "" if dt == "fp32" else "_fp16"
+        src = torch.rand(N, M, device=dev).to(tdt[dt])
+        dst = torch.zeros(M, N, device=dev, dtype=tdt[dt])
+        a = pkg.TranspArgs()
+        a.in_matrix, a.out_matrix, a.N, a.M = src.data_ptr(), dst.data_ptr(), N, M
+        ms = timed(void_call("transpose_matrix" + sfx, a), 20)
+        add("transpose_matrix %dx%d" % (N, M), dt, ms, 2 * N * M * es[dt])
+        c = pkg.CopyArgs()
+        c.from_, c.to, c.size = src.data_ptr(), dst.data_ptr(), N * M
+        ms = timed(void_call("copy" + sfx, c), 20)
+        add("copy %d elements" % (N * M), dt, ms, 2 * N * M * es[dt])
+        del src, dst
+    # layout change CHW -> HWC of a 256 x 256 x 512 tensor (64 MiB in fp16): transpose + copy back = 4 x the tensor
+    C, H, W, dt = 256, 256, 512, "fp16"
+    t = torch.rand(C, H, W, device=dev).to(tdt[dt])
+    buf = torch.zeros(C * H * W, device=dev, dtype=tdt[dt])
+    b = pkg.blob(t, None, C, H, W)
+    la = pkg.LayoutArgs()
+    la.tensor, la.transp_buffer, la.transpose_data, la.transpose_grad = hp.ptr(b), buf.data_ptr(), 1, 0
+    ms = timed(void_call("CHW_to_HWC_fp16", la), 10)
+    add("CHW_to_HWC %dx%dx%d (two passes)" % (C, H, W), dt, ms, 4 * C * H * W * es[dt])
+    ms = timed(void_call("HWC_to_CHW_fp16", la), 10)
+    add("HWC_to_CHW %dx%dx%d (two passes)" % (C, H, W), dt, ms, 4 * C * H * W * es[dt])
+    del t, buf
+    # weight block transpose, 2048 x 2048 channels, 3x3 (72 MiB in fp16), both layouts
+    Ci = Co = 2048
+    for hwc in (0, 1):
+        w = torch.rand(Co * Ci * 9, device=dev).to(tdt[dt])
+        bt = torch.zeros_like(w)
+        g = pkg.BlocktranspArgs()
+        g.weights, g.bt_weights, g.Cin, g.Cout, g.Hk, g.Wk, g.HWC = w.data_ptr(), bt.data_ptr(), Ci, Co, 3, 3, hwc
+        ms = timed(void_call("pulp_blocktransp_fp16", g), 10)
+        add("blocktranspose %dx%dx3x3 %s" % (Co, Ci, "HWC" if hwc else "CHW"), dt, ms, 2 * w.numel() * es[dt])
+        del w, bt
+    # im2row of a 64 x 224 x 224 input, 3x3, pad 1 (patch matrix 50176 x 576), fp32 (110 MiB) and fp16
+    for dt in ("fp32", "fp16"):
+        Ci, H, K = 64, 224, 3
+        x = torch.rand(Ci, H, H, device=dev).to(tdt[dt])
+        buf = torch.zeros(H * H * Ci * K * K, device=dev, dtype=tdt[dt])
+        bi, bw, bo = pkg.blob(x, None, Ci, H, H), pkg.blob(None, None, Ci, K, K), pkg.blob(None, None, 1, H, H)
+        a = pkg.Im2colArgs()
+        a.input, a.c, a.output, a.pBuffer = hp.ptr(bi), hp.ptr(bw), hp.ptr(bo), buf.data_ptr()
+        a.Lpad = a.Rpad = a.Upad = a.Dpad = 1
+        a.stride_h = a.stride_w = 1
+        ms = timed(void_call("pulp_im2row_" + dt, a), 10)
+        add("im2row 64x224x224 k3 p1", dt, ms, (x.numel() + buf.numel()) * es[dt])
+        del x, buf
+    # pad_tensor 256 x 360 x 360 by one on every side (63 MiB -> 64 MiB in fp16)
+    C, H, dt = 256, 360, "fp16"
+    srct = torch.rand(C, H, H, device=dev).to(tdt[dt])
+    dstt = torch.zeros(C, H + 2, H + 2, device=dev, dtype=tdt[dt])
+    pa = pkg.PadArgs()
+    pa.source, pa.dest, pa.C, pa.H, pa.W = srct.data_ptr(), dstt.data_ptr(), C, H, H
+    pa.T_RPAD = pa.T_LPAD = pa.T_UPAD = pa.T_DPAD = 1
+    ms = timed(void_call("pad_tensor_fp16", pa), 10)
+    add("pad_tensor %dx%dx%d pad 1" % (C, H, H), dt, ms, (srct.numel() + dstt.numel()) * es[dt])
     return rows
 
 

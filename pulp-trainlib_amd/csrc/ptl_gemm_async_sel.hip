@@ -155,6 +155,8 @@ int gemm_async(GemmArgs &g) {
             case 1:
                 // fp32 MFMAs are slow enough to matter at this size: when 64x64 tiles leave half the CUs
                 // idle, 64x32 tiles put a workgroup on every CU
+                // (fp16: measured no gain on 512 x 1024 x 1024, 15.96 against 16.2 us per step of three such products -
+                // at that size a launch is its fixed latencies, not its MFMAs)
                 if constexpr (sizeof(T) == 4) {
                     if (g.splits == 1 && tiles(64, 64) * 2 <= st.num_cu && g.M % 32 == 0)
                         return launch_plain<T, 64, 32, 512, 2, 1, 4, 3, 1>(g, st.stream);

@@ -16,6 +16,9 @@ namespace ptl {
 
 static inline unsigned nblocks(size_t n) { return (unsigned)((n + 255) / 256); }
 
+// x / d as a multiplication by m = ceil(2^32 / d): exact for x below 2^16.
+__device__ inline unsigned div_magic(unsigned x, unsigned m) { return (unsigned)(((unsigned long long)x * m) >> 32); }
+
 // ---- Depthwise convolution (CHW planes, one filter per channel) -----------------
 struct DwGeom {
     int C, H, W, Ho, Wo, Hk, Wk;
@@ -902,38 +905,215 @@ struct PatchGeom {
 
 // buf(p, q) = src[c, hp*h_mul + h_add + hk, wp*w_mul + w_add + wk] or 0 outside,
 // p = hp*Wp + wp, q = (c,hk,wk) for CHW and (hk,wk,c) for HWC.
-template <typename T>
+// A thread writes PER consecutive elements of the buffer (one 16-byte store when PER elements fill 16 bytes and
+// the buffer is aligned): its first index is decoded with divisions once, the following ones by carrying
+// (wk -> hk -> c -> next row, or wp -> hp -> next column), so the index arithmetic is a handful of additions
+// per element and the write side - nine times the bytes of the read side for a 3x3 filter - moves whole chunks.
+template <typename T, int PER>
 __global__ __launch_bounds__(256) void patch_kernel(const T *__restrict__ src, T *__restrict__ buf, PatchGeom g,
                                                     size_t total) {
-    size_t idx = (size_t)blockIdx.x * 256 + threadIdx.x;
-    if (idx >= total) return;
-    const int Q = g.C * g.Hk * g.Wk, P = g.Hp * g.Wp;
-    int p, q;
+    // (the host keeps the matrix below 2^32 elements: 32-bit index arithmetic)
+    const size_t idx0 = ((size_t)blockIdx.x * 256 + threadIdx.x) * PER;
+    if (idx0 >= total) return;
+    const unsigned Q = (unsigned)(g.C * g.Hk * g.Wk), P = (unsigned)(g.Hp * g.Wp), i32 = (unsigned)idx0;
+    unsigned p, q;
     if (!g.col_major) {
-        p = (int)(idx / Q);
-        q = (int)(idx % Q);
+        p = i32 / Q;
+        q = i32 - p * Q;
     } else {
-        q = (int)(idx / P);
-        p = (int)(idx % P);
+        q = i32 / P;
+        p = i32 - q * P;
     }
-    int hp = p / g.Wp, wp = p % g.Wp;
+    int hp = (int)(p / (unsigned)g.Wp), wp = (int)(p - (unsigned)hp * g.Wp);
     int c, hk, wk;
     if (!g.hwc) {
-        wk = q % g.Wk;
-        hk = (q / g.Wk) % g.Hk;
-        c = q / (g.Wk * g.Hk);
+        const unsigned t = q / (unsigned)g.Wk;
+        wk = (int)(q - t * g.Wk);
+        c = (int)(t / (unsigned)g.Hk);
+        hk = (int)(t - (unsigned)c * g.Hk);
     } else {
-        c = q % g.C;
-        wk = (q / g.C) % g.Wk;
-        hk = q / (g.C * g.Wk);
+        const unsigned t = q / (unsigned)g.C;
+        c = (int)(q - t * g.C);
+        hk = (int)(t / (unsigned)g.Wk);
+        wk = (int)(t - (unsigned)hk * g.Wk);
     }
-    int h = hp * g.h_mul + g.h_add + hk, w = wp * g.w_mul + g.w_add + wk;
-    T v = (T)0;
-    if ((unsigned)h < (unsigned)g.Hs && (unsigned)w < (unsigned)g.Ws) {
-        size_t off = g.hwc ? (((size_t)h * g.Ws + w) * g.C + c) : (((size_t)c * g.Hs + h) * g.Ws + w);
-        v = src[off];
+    T v[PER];
+#pragma unroll
+    for (int e = 0; e < PER; ++e) {
+        const int h = hp * g.h_mul + g.h_add + hk, w = wp * g.w_mul + g.w_add + wk;
+        v[e] = (T)0;
+        if (idx0 + e < total && (unsigned)h < (unsigned)g.Hs && (unsigned)w < (unsigned)g.Ws)
+            v[e] = g.hwc ? src[((size_t)h * g.Ws + w) * g.C + c] : src[((size_t)c * g.Hs + h) * g.Ws + w];
+        // next element of the buffer
+        bool next_q = true, next_p = false;
+        if (g.col_major) {  // p runs fastest
+            next_q = false;
+            next_p = true;
+        }
+        if (next_q) {
+            if (!g.hwc) {
+                if (++wk == g.Wk) {
+                    wk = 0;
+                    if (++hk == g.Hk) {
+                        hk = 0;
+                        if (++c == g.C) {
+                            c = 0;
+                            next_p = true;
+                        }
+                    }
+                }
+            } else {
+                if (++c == g.C) {
+                    c = 0;
+                    if (++wk == g.Wk) {
+                        wk = 0;
+                        if (++hk == g.Hk) {
+                            hk = 0;
+                            next_p = true;
+                        }
+                    }
+                }
+            }
+        }
+        if (next_p) {
+            if (++wp == g.Wp) {
+                wp = 0;
+                if (++hp == g.Hp) {
+                    hp = 0;
+                    if (g.col_major) {  // the column is complete: on to the next q
+                        if (!g.hwc) {
+                            if (++wk == g.Wk) {
+                                wk = 0;
+                                if (++hk == g.Hk) {
+                                    hk = 0;
+                                    ++c;
+                                }
+                            }
+                        } else {
+                            if (++c == g.C) {
+                                c = 0;
+                                if (++wk == g.Wk) {
+                                    wk = 0;
+                                    ++hk;
+                                }
+                            }
+                        }
+                    }
+                }
+            }
+        }
     }
-    buf[idx] = v;
+    if (PER * sizeof(T) == 16 && idx0 + PER <= total) {
+        union {
+            uint4 u;
+            T e[PER];
+        } pack;
+#pragma unroll
+        for (int e = 0; e < PER; ++e) pack.e[e] = v[e];
+        *reinterpret_cast<uint4 *>(buf + idx0) = pack.u;
+    } else {
+#pragma unroll
+        for (int e = 0; e < PER; ++e)
+            if (idx0 + e < total) buf[idx0 + e] = v[e];
+    }
+}
+
+// Row-major patch matrix of a channel-major tensor (im2row, the layout the reference's layers use) through LDS:
+// a workgroup owns R consecutive patch-grid positions of one grid row and CB channels.  It stages the source
+// window those patches cover ([CB][Hk][(R-1)*w_mul + Wk] elements, zero outside the tensor) with coalesced reads -
+// every source element is fetched once per workgroup instead of once per tap - and then writes its part of the
+// R buffer rows as 16-byte chunks, each gathered from LDS.  Divisions by the runtime extents are multiplications
+// by ceil(2^32 / d) (exact for dividends below 2^16).
+template <typename T>
+__global__ __launch_bounds__(256) void patch_rows_kernel(const T *__restrict__ src, T *__restrict__ buf, PatchGeom g, int R,
+                                                         int CB, int LW, unsigned m_cpr, unsigned m_pk, unsigned m_wk) {
+    constexpr int VEC = 16 / (int)sizeof(T);
+    extern __shared__ __attribute__((aligned(16))) char smem[];
+    const int PK = g.Hk * g.Wk, Q = g.C * PK, nq = CB * PK;
+    unsigned short *offs = reinterpret_cast<unsigned short *>(smem);                    // [nq], nq a multiple of VEC
+    T *lds = reinterpret_cast<T *>(smem + (((size_t)nq * 2 + 15) & ~(size_t)15));      // [CB * Hk][LW]
+    const int wp0 = blockIdx.x * R, hp = blockIdx.y, c0 = blockIdx.z * CB;
+    const int nr = min(R, g.Wp - wp0);
+    const int w_first = wp0 * g.w_mul + g.w_add, h_first = hp * g.h_mul + g.h_add;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    // where column q = (channel, filter row, filter column) of a buffer row starts in the staged window
+    for (int q = threadIdx.x; q < nq; q += 256) {
+        const unsigned c_l = div_magic((unsigned)q, m_pk), t = (unsigned)q - c_l * PK;
+        const unsigned hk = div_magic(t, m_wk), wk = t - hk * g.Wk;
+        offs[q] = (unsigned short)((c_l * g.Hk + hk) * LW + wk);
+    }
+    // the window: one wave per (channel, filter row), lanes along the row
+    for (int r = wave; r < CB * g.Hk; r += 4) {
+        const int c_l = r / g.Hk, hk = r - c_l * g.Hk, h = h_first + hk;
+        const bool row_ok = (unsigned)h < (unsigned)g.Hs;
+        const T *row = src + ((size_t)(c0 + c_l) * g.Hs + (row_ok ? h : 0)) * g.Ws;
+        for (int x = lane; x < LW; x += 64) {
+            const int w = w_first + x;
+            lds[r * LW + x] = (row_ok && (unsigned)w < (unsigned)g.Ws) ? row[w] : (T)0;
+        }
+    }
+    __syncthreads();
+    const int cpr = nq / VEC;  // chunks of this workgroup per buffer row
+    T *base = buf + ((size_t)hp * g.Wp + wp0) * Q + (size_t)c0 * PK;
+    for (int item = threadIdx.x; item < nr * cpr; item += 256) {
+        const unsigned p_l = div_magic((unsigned)item, m_cpr), qc = (unsigned)item - p_l * cpr;
+        union {
+            uint4 u;
+            unsigned short o[8];
+        } tab[VEC == 8 ? 1 : 1];
+        union {
+            uint4 u;
+            T e[VEC];
+        } v;
+        const T *win = lds + p_l * g.w_mul;
+        if (VEC == 8) {
+            tab[0].u = *reinterpret_cast<const uint4 *>(offs + qc * 8);
+#pragma unroll
+            for (int e = 0; e < VEC; ++e) v.e[e] = win[tab[0].o[e]];
+        } else {
+            const uint2 t2 = *reinterpret_cast<const uint2 *>(offs + qc * 4);
+            v.e[0] = win[t2.x & 0xffffu];
+            v.e[1] = win[t2.x >> 16];
+            v.e[2] = win[t2.y & 0xffffu];
+            v.e[3] = win[t2.y >> 16];
+        }
+        *reinterpret_cast<uint4 *>(base + (size_t)p_l * Q + qc * VEC) = v.u;
+    }
+}
+
+// 0 = launched; -1 = the geometry does not fit (the caller takes the general kernel).
+template <typename T>
+static int patch_rows(const T *src, T *buf, const PatchGeom &g) {
+    constexpr int VEC = 16 / (int)sizeof(T), ES = (int)sizeof(T);
+    if (g.hwc || g.col_major) return -1;
+    const int PK = g.Hk * g.Wk;
+    const long long Q = (long long)g.C * PK;
+    if (reinterpret_cast<uintptr_t>(buf) % 16 || (Q * ES) % 16 || g.Wp < 16 || Q >= 65536 || g.Hp >= 65536 || g.Wk > 32 ||
+        g.w_mul > 8)
+        return -1;
+    // positions per workgroup: a window row of at most 64 elements (one pass of a wave)
+    int R = (64 - g.Wk) / g.w_mul + 1;
+    if (R > g.Wp) R = g.Wp;
+    // row pitch of the window: an odd number of dwords, so that the rows the lanes of a wave gather from (every
+    // Hk-th one for neighbouring channels) spread over the LDS banks
+    int LW = (R - 1) * g.w_mul + g.Wk;
+    LW = ES == 2 ? (((LW + 1) & ~1) | 2) : (LW | 1);
+    auto bytes = [&](int cb) { return (((size_t)cb * PK * 2 + 15) & ~(size_t)15) + (size_t)cb * g.Hk * LW * ES; };
+    int CB = g.C;
+    while (bytes(CB) > 40 * 1024 && CB % 2 == 0) CB /= 2;
+    // enough workgroups to keep several per CU (their load and store phases overlap only across workgroups), as long
+    // as a workgroup's piece of a buffer row stays a few cache lines long
+    const long long per_z = (long long)((g.Wp + R - 1) / R) * g.Hp;
+    while (per_z * (g.C / CB) < 8LL * state().num_cu && CB % 2 == 0 && (CB / 2) * PK * ES >= 256 && ((CB / 2) * PK) % VEC == 0)
+        CB /= 2;
+    if (bytes(CB) > 64 * 1024 || (CB * PK) % VEC || CB * g.Hk * LW >= 65536 || g.C / CB >= 65536) return -1;
+    const int cpr = CB * PK / VEC;
+    if ((long long)R * cpr >= 65536) return -1;  // (the flat item index stays within the exact range of the reciprocal)
+    auto magic = [](unsigned d) { return (unsigned)((((unsigned long long)1 << 32) + d - 1) / d); };
+    dim3 grid((g.Wp + R - 1) / R, g.Hp, g.C / CB);
+    hipLaunchKernelGGL((patch_rows_kernel<T>), grid, dim3(256), bytes(CB), state().stream, src, buf, g, R, CB, LW, magic(cpr),
+                       magic(PK), magic(g.Wk));
+    return hip_ok(hipGetLastError(), "patch launch") ? 0 : 2;
 }
 
 template <typename T, typename Args>
@@ -1016,7 +1196,18 @@ static int patch_build(const Args *a, int col_major, const char *fn) {
     const T *dsrc = sg.in(src, src_n);
     T *dbuf = sg.out(reinterpret_cast<T *>(a->pBuffer), total);
     if (sg.failed()) return 2;
-    hipLaunchKernelGGL((patch_kernel<T>), dim3(nblocks(total)), dim3(256), 0, state().stream, dsrc, dbuf, g, total);
+    constexpr int VEC = 16 / (int)sizeof(T);
+    if (total >= ((size_t)1 << 32)) {
+        set_error("%s: patch matrix of 2^32 elements or more", fn);
+        return sg.finish(1);
+    }
+    if (int rc = patch_rows<T>(dsrc, dbuf, g); rc >= 0) return sg.finish(rc);
+    if (reinterpret_cast<uintptr_t>(dbuf) % 16 == 0)
+        hipLaunchKernelGGL((patch_kernel<T, VEC>), dim3(nblocks((total + VEC - 1) / VEC)), dim3(256), 0, state().stream,
+                           dsrc, dbuf, g, total);
+    else
+        hipLaunchKernelGGL((patch_kernel<T, 1>), dim3(nblocks(total)), dim3(256), 0, state().stream, dsrc, dbuf, g,
+                           total);
     return sg.finish(hip_ok(hipGetLastError(), "patch launch") ? 0 : 2);
 }
 
@@ -1036,6 +1227,77 @@ __global__ __launch_bounds__(256) void blocktransp_kernel(const T *__restrict__ 
         bt[idx] = w[(((size_t)co * Hk + (Hk - 1 - hk)) * Wk + (Wk - 1 - wk)) * Ci + ci];
     }
 }
+
+// Channel-major weights through an LDS tile of 32 output x 32 input channels x P taps: a workgroup reads, for each
+// of its 32 output channels, the contiguous run of 32 x P elements, and writes, for each of its 32 input channels,
+// the contiguous run of 32 x P elements of the result - both sides of the transposition move whole lines, 16 bytes
+// per thread where VECS says the runs are made of whole aligned chunks.
+template <typename T, bool VECS>
+__global__ __launch_bounds__(256) void blocktransp_tile_kernel(const T *__restrict__ w, T *__restrict__ bt, int Ci,
+                                                               int Co, int P, unsigned m_p) {
+    constexpr int VEC = 16 / (int)sizeof(T);
+    extern __shared__ __attribute__((aligned(16))) char smem[];
+    T *tile = reinterpret_cast<T *>(smem);  // [32 co][32 * P + VEC]: rows start on 16-byte boundaries
+    const int ci0 = blockIdx.x * 32, co0 = blockIdx.y * 32, pitch = 32 * P + VEC;
+    const int nci = min(32, Ci - ci0), nco = min(32, Co - co0);
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    for (int r = wave; r < nco; r += 4) {
+        const T *src = w + ((size_t)(co0 + r) * Ci + ci0) * P;
+        const int n = nci * P;
+        if (VECS) {
+            for (int c = lane; c * VEC < n; c += 64) {
+                if (c * VEC + VEC <= n) {
+                    union {
+                        uint4 u;
+                        T e[VEC];
+                    } v;
+                    v.u = *reinterpret_cast<const uint4 *>(src + c * VEC);
+                    *reinterpret_cast<uint4 *>(tile + r * pitch + c * VEC) = v.u;
+                } else {
+                    for (int e = c * VEC; e < n; ++e) tile[r * pitch + e] = src[e];
+                }
+            }
+        } else {
+            for (int e = lane; e < n; e += 64) tile[r * pitch + e] = src[e];
+        }
+    }
+    __syncthreads();
+    for (int r = wave; r < nci; r += 4) {
+        T *dst = bt + ((size_t)(ci0 + r) * Co + co0) * P;
+        const int n = nco * P;
+        if (VECS) {
+            for (int c = lane; c * VEC < n; c += 64) {
+                unsigned co = div_magic((unsigned)(c * VEC), m_p), i = (unsigned)(c * VEC) - co * P;
+                union {
+                    uint4 u;
+                    T e[VEC];
+                } v;
+#pragma unroll
+                for (int e = 0; e < VEC; ++e) {
+                    v.e[e] = co < (unsigned)nco ? tile[co * pitch + r * P + (P - 1 - i)] : (T)0;
+                    if (++i == (unsigned)P) {
+                        i = 0;
+                        ++co;
+                    }
+                }
+                if (c * VEC + VEC <= n) {
+                    *reinterpret_cast<uint4 *>(dst + c * VEC) = v.u;
+                } else {
+                    for (int e = 0; c * VEC + e < n; ++e) dst[c * VEC + e] = v.e[e];
+                }
+            }
+        } else {
+            for (int e = lane; e < n; e += 64) {
+                const unsigned co = div_magic((unsigned)e, m_p), i = (unsigned)e - co * P;
+                dst[e] = tile[co * pitch + r * P + (P - 1 - i)];
+            }
+        }
+    }
+}
+
+template <typename T>
+static int transpose2d_strided(const T *in, T *out, int N, int M, long long in_rs, long long out_rs, int batch,
+                               long long in_bs, long long out_bs, long long in_base, long long out_base);
 
 template <typename T, typename Args>
 static int blocktransp(const Args *a, const char *fn) {
@@ -1059,35 +1321,135 @@ static int blocktransp(const Args *a, const char *fn) {
     const T *w = sg.in(reinterpret_cast<const T *>(a->weights), n);
     T *bt = sg.out(reinterpret_cast<T *>(a->bt_weights), n);
     if (sg.failed()) return 2;
-    hipLaunchKernelGGL((blocktransp_kernel<T>), dim3(nblocks(n)), dim3(256), 0, state().stream, w, bt, a->Cin,
-                       a->Cout, a->Hk, a->Wk, hwc, (int)n);
-    return sg.finish(hip_ok(hipGetLastError(), "blocktranspose launch") ? 0 : 2);
+    const int P = a->Hk * a->Wk;
+    int rc = 0;
+    if (hwc) {
+        // per tap a strided transposition: in(co, ci) = w[co][P-1-p][ci], out(ci, co) = bt[ci][p][co]
+        rc = transpose2d_strided<T>(w, bt, a->Cout, a->Cin, (long long)P * a->Cin, (long long)P * a->Cout, P,
+                                    -(long long)a->Cin, (long long)a->Cout, (long long)(P - 1) * a->Cin, 0);
+    } else if ((size_t)32 * (32 * P + 16 / sizeof(T)) * sizeof(T) <= 64 * 1024 && n >= 4096) {
+        const size_t lds = (size_t)32 * (32 * P + 16 / sizeof(T)) * sizeof(T);
+        const unsigned m_p = (unsigned)((((unsigned long long)1 << 32) + P - 1) / P);
+        const dim3 grid((a->Cin + 31) / 32, (a->Cout + 31) / 32);
+        // runs of whole 16-byte chunks: every run starts on a chunk (rows of Ci x P and Co x P elements, tiles of 32 x P)
+        const bool vecs = ((size_t)a->Cin * P * sizeof(T)) % 16 == 0 && ((size_t)a->Cout * P * sizeof(T)) % 16 == 0 &&
+                          reinterpret_cast<uintptr_t>(w) % 16 == 0 && reinterpret_cast<uintptr_t>(bt) % 16 == 0;
+        if (vecs)
+            hipLaunchKernelGGL((blocktransp_tile_kernel<T, true>), grid, dim3(256), lds, state().stream, w, bt, a->Cin,
+                               a->Cout, P, m_p);
+        else
+            hipLaunchKernelGGL((blocktransp_tile_kernel<T, false>), grid, dim3(256), lds, state().stream, w, bt, a->Cin,
+                               a->Cout, P, m_p);
+        rc = hip_ok(hipGetLastError(), "blocktranspose launch") ? 0 : 2;
+    } else {
+        if (n >= ((size_t)1 << 31)) {
+            set_error("%s: tensor of 2^31 elements or more", fn);
+            return sg.finish(1);
+        }
+        hipLaunchKernelGGL((blocktransp_kernel<T>), dim3(nblocks(n)), dim3(256), 0, state().stream, w, bt, a->Cin,
+                           a->Cout, a->Hk, a->Wk, hwc, (int)n);
+        rc = hip_ok(hipGetLastError(), "blocktranspose launch") ? 0 : 2;
+    }
+    return sg.finish(rc);
 }
 
 // ---- Transposition ------------------------------------------------------------------------
 
 // out[j*N + i] = in[i*M + j]; 64x64 tiles through LDS so both sides coalesce.
+// General form (blockIdx.z = batch b): in(i, j) = in[in_base + b*in_bs + i*in_rs + j],
+// out(j, i) = out[out_base + b*out_bs + j*out_rs + i].
+struct Transp2D {
+    int N, M;
+    long long in_rs, out_rs, in_bs, out_bs, in_base, out_base;
+};
+
 template <typename T>
-__global__ __launch_bounds__(256) void transpose2d_kernel(const T *__restrict__ in, T *__restrict__ out, int N, int M) {
+__global__ __launch_bounds__(256) void transpose2d_kernel(const T *__restrict__ in, T *__restrict__ out, Transp2D g) {
     __shared__ T tile[64][65];
+    in += g.in_base + (long long)blockIdx.z * g.in_bs;
+    out += g.out_base + (long long)blockIdx.z * g.out_bs;
     int j0 = blockIdx.x * 64, i0 = blockIdx.y * 64;
     int tx = threadIdx.x & 63, ty = threadIdx.x >> 6;
     for (int r = ty; r < 64; r += 4) {
         int i = i0 + r, j = j0 + tx;
-        if (i < N && j < M) tile[r][tx] = in[(size_t)i * M + j];
+        if (i < g.N && j < g.M) tile[r][tx] = in[(long long)i * g.in_rs + j];
     }
     __syncthreads();
     for (int r = ty; r < 64; r += 4) {
         int j = j0 + r, i = i0 + tx;
-        if (i < N && j < M) out[(size_t)j * N + i] = tile[tx][r];
+        if (i < g.N && j < g.M) out[(long long)j * g.out_rs + i] = tile[tx][r];
+    }
+}
+
+// The same with 16-byte global accesses on both sides (rows, row strides, bases and pointers multiples of 16
+// bytes).  The tile is kept as dwords with a pitch of 33 (fp16: two columns per dword) or 65 (fp32), so the
+// column walk of the second phase is conflict free; a thread gathers the VEC elements of its output chunk from
+// VEC tile rows and stores them at once.
+template <typename T>
+__global__ __launch_bounds__(256) void transpose2d_vec_kernel(const T *__restrict__ in, T *__restrict__ out, Transp2D g) {
+    constexpr int VEC = 16 / (int)sizeof(T), CH = 64 / VEC;  // chunks per tile row
+    constexpr int PITCH = sizeof(T) == 2 ? 66 : 65;          // elements
+    __shared__ __attribute__((aligned(16))) T tile[64 * PITCH];
+    in += g.in_base + (long long)blockIdx.z * g.in_bs;
+    out += g.out_base + (long long)blockIdx.z * g.out_bs;
+    const int j0 = blockIdx.x * 64, i0 = blockIdx.y * 64;
+#pragma unroll
+    for (int it = 0; it < 64 * CH / 256; ++it) {
+        const int item = it * 256 + threadIdx.x, r = item / CH, c = item % CH;
+        const int i = i0 + r, j = j0 + c * VEC;
+        if (i < g.N && j < g.M) {  // (M is a multiple of VEC: a chunk is inside or outside)
+            union {
+                uint4 u;
+                T e[VEC];
+                unsigned d[4];
+            } v;
+            v.u = *reinterpret_cast<const uint4 *>(in + (long long)i * g.in_rs + j);
+            if (sizeof(T) == 2) {
+                unsigned *row = reinterpret_cast<unsigned *>(tile + r * PITCH + c * VEC);  // 4-byte aligned
+#pragma unroll
+                for (int k = 0; k < 4; ++k) row[k] = v.d[k];
+            } else {
+#pragma unroll
+                for (int k = 0; k < VEC; ++k) tile[r * PITCH + c * VEC + k] = v.e[k];
+            }
+        }
+    }
+    __syncthreads();
+#pragma unroll
+    for (int it = 0; it < 64 * CH / 256; ++it) {
+        const int item = it * 256 + threadIdx.x, r = item / CH, c = item % CH;  // output row j0 + r, rows i0 + c*VEC ..
+        const int j = j0 + r, i = i0 + c * VEC;
+        if (j < g.M && i < g.N) {
+            union {
+                uint4 u;
+                T e[VEC];
+            } v;
+#pragma unroll
+            for (int k = 0; k < VEC; ++k) v.e[k] = tile[(c * VEC + k) * PITCH + r];
+            *reinterpret_cast<uint4 *>(out + (long long)j * g.out_rs + i) = v.u;
+        }
     }
 }
 
 template <typename T>
-static int transpose2d_dev(const T *in, T *out, int N, int M) {
-    dim3 grid((M + 63) / 64, (N + 63) / 64);
-    hipLaunchKernelGGL((transpose2d_kernel<T>), grid, dim3(256), 0, state().stream, in, out, N, M);
+static int transpose2d_strided(const T *in, T *out, int N, int M, long long in_rs, long long out_rs, int batch,
+                               long long in_bs, long long out_bs, long long in_base, long long out_base) {
+    constexpr int VEC = 16 / (int)sizeof(T);
+    Transp2D g = {N, M, in_rs, out_rs, in_bs, out_bs, in_base, out_base};
+    dim3 grid((M + 63) / 64, (N + 63) / 64, batch);
+    auto mult = [](long long v) { return v % VEC == 0; };
+    const bool vec = mult(N) && mult(M) && mult(in_rs) && mult(out_rs) && mult(in_bs) && mult(out_bs) && mult(in_base) &&
+                     mult(out_base) && reinterpret_cast<uintptr_t>(in) % 16 == 0 && reinterpret_cast<uintptr_t>(out) % 16 == 0;
+    if (vec)
+        hipLaunchKernelGGL((transpose2d_vec_kernel<T>), grid, dim3(256), 0, state().stream, in, out, g);
+    else
+        hipLaunchKernelGGL((transpose2d_kernel<T>), grid, dim3(256), 0, state().stream, in, out, g);
     return hip_ok(hipGetLastError(), "transpose launch") ? 0 : 2;
+}
+
+template <typename T>
+static int transpose2d_dev(const T *in, T *out, int N, int M) {
+    return transpose2d_strided<T>(in, out, N, M, M, N, 1, 0, 0, 0, 0);
 }
 
 constexpr int MAX_ND = 8;
@@ -1187,6 +1549,27 @@ __global__ __launch_bounds__(256) void copy_kernel(const T *__restrict__ a, T *_
     if (i < n) b[i] = a[i];
 }
 
+// 16 bytes per thread (both pointers 16-byte aligned); the last, partial chunk element by element.
+template <typename T>
+__global__ __launch_bounds__(256) void copy_vec_kernel(const T *__restrict__ a, T *__restrict__ b, size_t n) {
+    constexpr int VEC = 16 / (int)sizeof(T);
+    const size_t i = ((size_t)blockIdx.x * 256 + threadIdx.x) * VEC;
+    if (i + VEC <= n) {
+        *reinterpret_cast<uint4 *>(b + i) = *reinterpret_cast<const uint4 *>(a + i);
+    } else {
+        for (size_t e = i; e < n; ++e) b[e] = a[e];
+    }
+}
+
+template <typename T>
+static void launch_copy(const T *a, T *b, size_t n) {
+    constexpr int VEC = 16 / (int)sizeof(T);
+    if (reinterpret_cast<uintptr_t>(a) % 16 == 0 && reinterpret_cast<uintptr_t>(b) % 16 == 0)
+        hipLaunchKernelGGL((copy_vec_kernel<T>), dim3(nblocks((n + VEC - 1) / VEC)), dim3(256), 0, state().stream, a, b, n);
+    else
+        hipLaunchKernelGGL((copy_kernel<T>), dim3(nblocks(n)), dim3(256), 0, state().stream, a, b, n);
+}
+
 __global__ __launch_bounds__(256) void copy16_kernel(const uint4 *__restrict__ a, uint4 *__restrict__ b, size_t n) {
     size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
     size_t stride = (size_t)gridDim.x * 256;
@@ -1212,27 +1595,98 @@ __global__ __launch_bounds__(256) void cast_kernel(const S *__restrict__ a, D *_
     if (i < n) b[i] = (D)a[i];
 }
 
-// dest[c][ht][wt] = source[c][ht-U][wt-L] inside, 0 in the border (CHW; HWC alike)
-template <typename T>
+// dest[c][ht][wt] = source[c][ht-U][wt-L] inside, 0 in the border (CHW; HWC alike).  A thread writes PER
+// consecutive destination elements (one 16-byte store): first index decoded once, the rest by carrying.
+template <typename T, int PER>
 __global__ __launch_bounds__(256) void pad_kernel(const T *__restrict__ src, T *__restrict__ dst, int C, int H, int W,
-                                                  int L, int U, int Ho, int Wo, int hwc, size_t total) {
-    size_t idx = (size_t)blockIdx.x * 256 + threadIdx.x;
-    if (idx >= total) return;
+                                                  int L, int U, int Ho, int Wo, int hwc, size_t total, int src_aligned,
+                                                  size_t src_bytes) {
+    const size_t idx0 = ((size_t)blockIdx.x * 256 + threadIdx.x) * PER;
+    if (idx0 >= total) return;
+    // (the host keeps the tensor below 2^32 elements: 32-bit index arithmetic)
+    const unsigned i32 = (unsigned)idx0;
     int c, ht, wt;
     if (!hwc) {
-        wt = (int)(idx % Wo);
-        ht = (int)((idx / Wo) % Ho);
-        c = (int)(idx / ((size_t)Wo * Ho));
+        const unsigned r = i32 / (unsigned)Wo;
+        wt = (int)(i32 - r * Wo);
+        c = (int)(r / (unsigned)Ho);
+        ht = (int)(r - (unsigned)c * Ho);
     } else {
-        c = (int)(idx % C);
-        wt = (int)((idx / C) % Wo);
-        ht = (int)(idx / ((size_t)C * Wo));
+        const unsigned r = i32 / (unsigned)C;
+        c = (int)(i32 - r * C);
+        ht = (int)(r / (unsigned)Wo);
+        wt = (int)(r - (unsigned)ht * Wo);
     }
-    int h = ht - U, w = wt - L;
-    T v = (T)0;
-    if ((unsigned)h < (unsigned)H && (unsigned)w < (unsigned)W)
-        v = hwc ? src[((size_t)h * W + w) * C + c] : src[((size_t)c * H + h) * W + w];
-    dst[idx] = v;
+    if (PER * sizeof(T) == 16 && src_aligned) {
+        // the whole chunk inside one contiguous run of the source (a row, or the channels of a pixel): two aligned
+        // 16-byte loads around it and a byte shift instead of PER element loads
+        const int h = ht - U, w = wt - L;
+        const bool inside = (unsigned)h < (unsigned)H && (unsigned)w < (unsigned)W && idx0 + PER <= total &&
+                            (hwc ? c + PER <= C : w + PER <= W);
+        if (inside) {
+            const size_t si = hwc ? ((size_t)h * W + w) * C + c : ((size_t)c * H + h) * W + w;
+            const size_t ba = si * sizeof(T), a0 = ba & ~(size_t)15;
+            const unsigned sh = (unsigned)(ba - a0);
+            if (sh == 0 || a0 + 32 <= src_bytes) {
+                const char *sb = reinterpret_cast<const char *>(src);
+                const uint4 lo = *reinterpret_cast<const uint4 *>(sb + a0);
+                uint4 out = lo;
+                if (sh != 0) {
+                    const uint4 hi = *reinterpret_cast<const uint4 *>(sb + a0 + 16);
+                    const unsigned d[8] = {lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
+                    const unsigned o = sh >> 2, bits = (sh & 3u) * 8u;
+                    unsigned t[5];
+#pragma unroll
+                    for (int j = 0; j < 5; ++j) t[j] = o == 0 ? d[j] : o == 1 ? d[j + 1] : o == 2 ? d[j + 2] : d[j + 3];
+                    unsigned r[4];
+#pragma unroll
+                    for (int j = 0; j < 4; ++j)
+                        r[j] = (unsigned)(((((unsigned long long)t[j + 1]) << 32) | t[j]) >> bits);
+                    out = make_uint4(r[0], r[1], r[2], r[3]);
+                }
+                *reinterpret_cast<uint4 *>(dst + idx0) = out;
+                return;
+            }
+        }
+    }
+    T v[PER];
+#pragma unroll
+    for (int e = 0; e < PER; ++e) {
+        const int h = ht - U, w = wt - L;
+        v[e] = (T)0;
+        if (idx0 + e < total && (unsigned)h < (unsigned)H && (unsigned)w < (unsigned)W)
+            v[e] = hwc ? src[((size_t)h * W + w) * C + c] : src[((size_t)c * H + h) * W + w];
+        if (!hwc) {
+            if (++wt == Wo) {
+                wt = 0;
+                if (++ht == Ho) {
+                    ht = 0;
+                    ++c;
+                }
+            }
+        } else {
+            if (++c == C) {
+                c = 0;
+                if (++wt == Wo) {
+                    wt = 0;
+                    ++ht;
+                }
+            }
+        }
+    }
+    if (PER * sizeof(T) == 16 && idx0 + PER <= total) {
+        union {
+            uint4 u;
+            T e[PER];
+        } pack;
+#pragma unroll
+        for (int e = 0; e < PER; ++e) pack.e[e] = v[e];
+        *reinterpret_cast<uint4 *>(dst + idx0) = pack.u;
+    } else {
+#pragma unroll
+        for (int e = 0; e < PER; ++e)
+            if (idx0 + e < total) dst[idx0 + e] = v[e];
+    }
 }
 
 template <typename T, typename Args>
@@ -1253,12 +1707,22 @@ static int pad_step(const Args *a, const char *fn) {
     if (!ensure_init()) return 2;
     int Ho = a->H + a->T_UPAD + a->T_DPAD, Wo = a->W + a->T_LPAD + a->T_RPAD;
     size_t total = (size_t)a->C * Ho * Wo;
+    if (total >= ((size_t)1 << 32)) {
+        set_error("%s: tensor of 2^32 elements or more", fn);
+        return 1;
+    }
     Stager sg;
     const T *s = sg.in(reinterpret_cast<const T *>(a->source), (size_t)a->C * a->H * a->W);
     T *d = sg.out(reinterpret_cast<T *>(a->dest), total);
     if (sg.failed()) return 2;
-    hipLaunchKernelGGL((pad_kernel<T>), dim3(nblocks(total)), dim3(256), 0, state().stream, s, d, a->C, a->H, a->W,
-                       a->T_LPAD, a->T_UPAD, Ho, Wo, a->HWC_lay, total);
+    constexpr int VEC = 16 / (int)sizeof(T);
+    if (reinterpret_cast<uintptr_t>(d) % 16 == 0)
+        hipLaunchKernelGGL((pad_kernel<T, VEC>), dim3(nblocks((total + VEC - 1) / VEC)), dim3(256), 0, state().stream, s, d,
+                           a->C, a->H, a->W, a->T_LPAD, a->T_UPAD, Ho, Wo, a->HWC_lay, total,
+                           reinterpret_cast<uintptr_t>(s) % 16 == 0 ? 1 : 0, (size_t)a->C * a->H * a->W * sizeof(T));
+    else
+        hipLaunchKernelGGL((pad_kernel<T, 1>), dim3(nblocks(total)), dim3(256), 0, state().stream, s, d, a->C, a->H, a->W,
+                           a->T_LPAD, a->T_UPAD, Ho, Wo, a->HWC_lay, total, 0, (size_t)0);
     return sg.finish(hip_ok(hipGetLastError(), "pad launch") ? 0 : 2);
 }
 
@@ -1273,7 +1737,7 @@ static int relayout_one(T *tensor, T *buffer, int rows, int cols, Stager &sg) {
     if (sg.failed()) return 2;
     int rc = transpose2d_dev<T>(t, b, rows, cols);
     if (rc) return rc;
-    hipLaunchKernelGGL((copy_kernel<T>), dim3(nblocks(n)), dim3(256), 0, state().stream, b, t, n);
+    launch_copy<T>(b, t, n);
     return hip_ok(hipGetLastError(), "copy launch") ? 0 : 2;
 }
 
@@ -1321,7 +1785,7 @@ static int copy_step(const T *from, T *to, int size) {
     const T *a = sg.in(from, (size_t)size);
     T *b = sg.out(to, (size_t)size);
     if (sg.failed()) return 2;
-    hipLaunchKernelGGL((copy_kernel<T>), dim3(nblocks(size)), dim3(256), 0, state().stream, a, b, (size_t)size);
+    launch_copy<T>(a, b, (size_t)size);
     return sg.finish(hip_ok(hipGetLastError(), "copy launch") ? 0 : 2);
 }
 

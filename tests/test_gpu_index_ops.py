@@ -180,3 +180,104 @@ def test_streaming_helpers(pkg, gpu):
     pkg.call("cast_fp32_tensor_to_fp16", k)
     sync(gpu)
     assert np.array_equal(ghz.cpu().numpy(), x.astype(np.float16))
+
+
+# ---------------------------------------------------------------- larger and ragged shapes for the chunked kernels
+@pytest.mark.parametrize("dt", ["fp32", "fp16"])
+@pytest.mark.parametrize("N,M", [(256, 512), (72, 200), (1000, 24), (8, 8), (136, 1048), (63, 129)])
+def test_transpose_matrix_tiles(pkg, gpu, dt, N, M):
+    """Whole and ragged 64x64 tiles, sizes that are and are not multiples of a 16-byte chunk."""
+    nd = hp.np_dtype(dt)
+    m = hp.uniform(0x7A05, (N, M), dtype=nd)
+    gm, gout = dev(m), dev(np.full(N * M, 3, nd))
+    a = pkg.TranspArgs()
+    a.in_matrix, a.out_matrix, a.N, a.M = pkg.addr(gm), pkg.addr(gout), N, M
+    pkg.call("transpose_matrix" if dt == "fp32" else "transpose_matrix_fp16", a)
+    sync(gpu)
+    assert np.array_equal(bits(gout.cpu().numpy()), bits(m.T.reshape(-1)))
+
+
+@pytest.mark.parametrize("dt", ["fp32", "fp16"])
+@pytest.mark.parametrize("hwc", [0, 1])
+@pytest.mark.parametrize("Ci,Co,Hk,Wk", [(64, 96, 3, 3), (40, 33, 3, 3), (72, 64, 5, 5), (8, 16, 1, 1), (130, 70, 2, 3)])
+def test_blocktranspose_tiles(pkg, orc, gpu, dt, hwc, Ci, Co, Hk, Wk):
+    nd = hp.np_dtype(dt)
+    w = hp.uniform(0xB7, (Co * Ci * Hk * Wk,), dtype=nd)
+    ref = np.zeros_like(w)
+    a = pkg.BlocktranspArgs()
+    a.weights, a.bt_weights, a.Cin, a.Cout, a.Hk, a.Wk, a.HWC = pkg.addr(w), pkg.addr(ref), Ci, Co, Hk, Wk, hwc
+    orc.call("orc_blocktransp", dt, a)
+    gw, gbt = dev(w), dev(np.full(w.shape, 3, nd))
+    g = pkg.BlocktranspArgs()
+    g.weights, g.bt_weights, g.Cin, g.Cout, g.Hk, g.Wk, g.HWC = pkg.addr(gw), pkg.addr(gbt), Ci, Co, Hk, Wk, hwc
+    pkg.call("pulp_blocktransp_" + dt, g)
+    sync(gpu)
+    assert np.array_equal(bits(gbt.cpu().numpy()), bits(ref))
+
+
+@pytest.mark.parametrize("dt", ["fp32", "fp16"])
+@pytest.mark.parametrize("hwc", [0, 1])
+@pytest.mark.parametrize("Ci,H,W,K,pad,stride,mod", [(16, 32, 32, 3, (1, 1, 1, 1), (1, 1), 0), (7, 19, 23, 3, (1, 1, 1, 1), (2, 2), 0),
+                                                     (6, 14, 9, 5, (2, 2, 2, 2), (1, 1), 0), (5, 12, 12, 3, (0, 0, 0, 0), (1, 1), 1)])
+def test_im2row_im2col_chunked(pkg, orc, gpu, dt, hwc, Ci, H, W, K, pad, stride, mod):
+    """Patch matrices whose rows are not multiples of a 16-byte chunk (chunks straddle rows and columns), BASELINE
+    config 1 among them."""
+    Co = 4
+    Ho, Wo = (H - K + 1, W - K + 1) if mod else (hp.conv_out(H, K, pad[2], pad[3], stride[0]),
+                                                hp.conv_out(W, K, pad[0], pad[1], stride[1]))
+    nd = hp.np_dtype(dt)
+    x = hp.uniform(11, (Ci * H * W,), dtype=nd)
+    dy = hp.uniform(12, (Co * Ho * Wo,), dtype=nd)
+    n = (H * W * Co if mod else Ho * Wo * Ci) * K * K
+    for fn in ("im2row", "im2col"):
+        buf = np.full(n, -1, nd)
+        a, keep = patch_args(pkg, dt, x, dy, buf, Ci, H, W, Co, K, K, Ho, Wo, pad, stride, mod, hwc)
+        orc.call("orc_" + fn, dt, a)
+        gx, gdy, gbuf = dev(x), dev(dy), dev(np.full(n, -2, nd))
+        g, keep2 = patch_args(pkg, dt, gx, gdy, gbuf, Ci, H, W, Co, K, K, Ho, Wo, pad, stride, mod, hwc)
+        pkg.call("pulp_%s_%s" % (fn, dt), g)
+        sync(gpu)
+        assert np.array_equal(bits(gbuf.cpu().numpy()), bits(buf)), fn
+        # an unaligned buffer takes the element-wise kernel: same result one element further
+        gbig = dev(np.full(n + 8, -2, nd))
+        g.pBuffer = pkg.addr(gbig) + gbig.element_size()
+        pkg.call("pulp_%s_%s" % (fn, dt), g)
+        sync(gpu)
+        assert np.array_equal(bits(gbig.cpu().numpy()[1:n + 1]), bits(buf)), fn
+
+
+@pytest.mark.parametrize("dt", ["fp32", "fp16"])
+@pytest.mark.parametrize("hwc", [0, 1])
+@pytest.mark.parametrize("C,H,W,pads", [(16, 32, 32, (1, 1, 1, 1)), (5, 9, 13, (2, 0, 1, 3)), (3, 7, 7, (0, 0, 0, 0))])
+def test_pad_tensor_chunked(pkg, orc, gpu, dt, hwc, C, H, W, pads):
+    nd = hp.np_dtype(dt)
+    R, L, U, D = pads
+    src = hp.uniform(21, (C * H * W,), dtype=nd)
+    n = C * (H + U + D) * (W + L + R)
+    ref = np.full(n, -1, nd)
+    a = pkg.PadArgs()
+    a.source, a.dest, a.C, a.H, a.W = pkg.addr(src), pkg.addr(ref), C, H, W
+    a.T_RPAD, a.T_LPAD, a.T_UPAD, a.T_DPAD, a.HWC_lay = R, L, U, D, hwc
+    orc.call("orc_pad_tensor", dt, a)
+    gs, gd = dev(src), dev(np.full(n, -2, nd))
+    g = pkg.PadArgs()
+    g.source, g.dest, g.C, g.H, g.W = pkg.addr(gs), pkg.addr(gd), C, H, W
+    g.T_RPAD, g.T_LPAD, g.T_UPAD, g.T_DPAD, g.HWC_lay = R, L, U, D, hwc
+    pkg.call("pad_tensor" if dt == "fp32" else "pad_tensor_fp16", g)
+    sync(gpu)
+    assert np.array_equal(bits(gd.cpu().numpy()), bits(ref))
+
+
+@pytest.mark.parametrize("dt", ["fp32", "fp16"])
+@pytest.mark.parametrize("n", [1, 7, 8, 1000, 4099])
+def test_copy_sizes(pkg, gpu, dt, n):
+    nd = hp.np_dtype(dt)
+    src = hp.uniform(31, (n + 4,), dtype=nd)
+    for shift in (0, 1):  # aligned and unaligned source
+        gs, gd = dev(src), dev(np.full(n + 4, 3, nd))
+        c = pkg.CopyArgs()
+        c.from_, c.to, c.size = pkg.addr(gs) + shift * gs.element_size(), pkg.addr(gd), n
+        pkg.call("copy" if dt == "fp32" else "copy_fp16", c)
+        sync(gpu)
+        out = gd.cpu().numpy()
+        assert np.array_equal(bits(out[:n]), bits(src[shift:shift + n])) and np.all(out[n:] == 3)
