@@ -177,6 +177,8 @@ def main():
     if not args.no_cpu:
         orc = ge.load_oracle()
         olib = orc.load()
+        # the reference's own core count (NUM_CORES = 8, tests/test_conv2d_fp32/Makefile:16), clamped to the host
+        olib.orc_set_num_threads(min(8, os.cpu_count() or 8))
         cores = int(olib.orc_num_threads())
 
         def cpu_step(m):
@@ -198,6 +200,7 @@ def main():
         result["cpu_baseline"] = {"value": round(cpu_tflops, 6), "unit": "TFLOP/s", "cores": cores, "kind": "port",
                                   "sample": "%d of the %d samples, FW+WG+IG %d times, fp16 with fp16 accumulation "
                                             "(the reference's arithmetic), %.2f s" % (m, ns, reps, t_cpu)}
+        result["cpu_baseline_detail"] = cpu_rows(pkg, orc, hp, cores)
 
     # ------------------------------------------------------------------------------ detail
     if args.helpers_only:
@@ -208,6 +211,80 @@ def main():
         result["detail"] = detail_table(pkg, lib, hp, to_dev, timed, check, torch, dev)
 
     print(json.dumps(result))
+
+
+def cpu_rows(pkg, orc, hp, cores):
+    """The CPU oracle (a port of the reference's loops, OpenMP over `cores` threads) on the other BASELINE
+    configurations, one sample each where the batched mode is a loop over samples: microseconds and TFLOP/s per
+    step, median of a bounded number of repetitions (about a second per row)."""
+    import ctypes
+    rows = []
+
+    def median_time(fn, budget=0.6, max_reps=21):
+        fn()
+        times = []
+        t_all = time.perf_counter()
+        while len(times) < max_reps and (len(times) < 3 or time.perf_counter() - t_all < budget):
+            t = time.perf_counter()
+            fn()
+            times.append(time.perf_counter() - t)
+        times.sort()
+        return times[len(times) // 2], len(times)
+
+    def add(name, dt, flops, fn):
+        t, reps = median_time(fn)
+        rows.append({"workload": name, "dtype": dt, "us": round(t * 1e6, 1), "TFLOP/s": round(flops / t / 1e12, 6),
+                     "threads": cores, "kind": "port", "sample": "one call, median of %d" % reps})
+
+    for dt in ("fp32", "fp16"):  # config 1
+        nd = hp.np_dtype(dt)
+        Ci, Co, H, K = 16, 32, 32, 3
+        x, w, dy = hp.uniform(1, (Ci, H, H), dtype=nd), hp.uniform(2, (Co, Ci, K, K), dtype=nd), hp.uniform(3, (Co, H, H), dtype=nd)
+        y, dx, dw = np.zeros_like(dy), np.zeros_like(x), np.zeros_like(w)
+        a, keep = hp.conv2d_args(pkg, x, dx, w, dw, y, dy, Ci, H, H, Co, K, K, H, H, (1, 1, 1, 1))
+        for s in ("fw", "wg", "ig"):
+            add("conv2d 16->32 32x32 k3 p1 %s N=1" % s.upper(), dt, 2.0 * Co * Ci * K * K * H * H,
+                lambda s=s: orc.call("orc_conv2d_" + s, dt, a, 1))
+    for dt in ("fp32", "fp16"):  # config 2, one sample (batched mode on the CPU = a loop over samples)
+        nd = hp.np_dtype(dt)
+        n = 1024
+        x, w, dy = hp.normal(4, (n,), 1 / 32.0, nd), hp.normal(5, (n, n), 1 / 32.0, nd), hp.uniform(6, (n,), dtype=nd)
+        y, dx, dw = np.zeros_like(dy), np.zeros_like(x), np.zeros_like(w)
+        a, keep = hp.linear_args(pkg, x, dx, w, dw, y, dy, n, n)
+        for s in ("fw", "wg", "ig"):
+            add("linear 1024x1024 %s N=1" % s.upper(), dt, 2.0 * n * n, lambda s=s: orc.call("orc_linear_" + s, dt, a, 1))
+    dt, nd = "fp16", np.float16  # config 3
+    C, Hp, Ho, K = 64, 58, 56, 3
+    x, w, dy = hp.uniform(7, (C, Hp, Hp), dtype=nd), hp.uniform(8, (C, K, K), dtype=nd), hp.uniform(9, (C, Ho, Ho), dtype=nd)
+    y, dx, dw = np.zeros_like(dy), np.zeros_like(x), np.zeros_like(w)
+    a3, keep3 = hp.dw_args(pkg, dt, x, dx, w, dw, y, dy, C, Hp, Hp, K, K, Ho, Ho)
+    for s in ("fw", "wg", "ig"):
+        add("depthwise 3x3 64x56x56 %s N=1" % s.upper(), dt, 2.0 * C * K * K * Ho * Ho,
+            lambda s=s: orc.call("orc_conv_dw_" + s, dt, a3, 1))
+    Ci, Co, H = 64, 128, 56
+    x, w, dy = hp.uniform(10, (Ci, H * H), dtype=nd), hp.uniform(11, (Co, Ci), dtype=nd), hp.uniform(12, (Co, H * H), dtype=nd)
+    y, dx, dw = np.zeros_like(dy), np.zeros_like(x), np.zeros_like(w)
+    a4, keep4 = hp.pw_args(pkg, x, dx, w, dw, y, dy, Ci, Co, H, H)
+    for s in ("fw", "wg", "ig"):
+        add("pointwise 64->128 56x56 %s N=1" % s.upper(), dt, 2.0 * Co * Ci * H * H,
+            lambda s=s: orc.call("orc_conv_pw_" + s, dt, a4, 1))
+    # config 4: attention step, one sequence
+    L, E, F, heads = 197, 192, 192, 3
+    sh = hp.mhsa_shapes(1, L, E, F, heads)
+    d, dyh = hp.mhsa_inputs(0xC0DE0004, 1, L, E, F, heads)
+    data = dict(d)
+    for n_ in ("q", "k", "v", "att", "p", "y"):
+        data[n_] = np.zeros(sh[n_], np.float32)
+    diff = {n_: np.zeros(sh[n_], np.float32) for n_ in ("x", "q", "k", "v", "att", "p", "wo")}
+    for n_ in ("wq", "wk", "wv"):
+        diff[n_] = np.zeros((F, E), np.float32)
+    diff["y"] = dyh
+    am, keepm = hp.mhsa_args(pkg, data, diff, L, E, F, heads)
+    olib = orc.load()
+    f_fw = 4 * 2.0 * F * E * L + heads * 2 * 2.0 * L * L * (F // heads)
+    add("mhsa L197 E192 3x64 FW N=1", "fp32", f_fw, lambda: olib.orc_mhsa_fw_fp32(ctypes.byref(am), 1))
+    add("mhsa L197 E192 3x64 BW N=1", "fp32", 2 * f_fw, lambda: olib.orc_mhsa_bw_fp32(ctypes.byref(am), 1))
+    return rows
 
 
 def resnet_rows(pkg, lib, timed, torch, dev):
