@@ -331,7 +331,11 @@ int conv_taps_wg(const ConvTileDesc &d, const void *X, const void *dY, void *dW)
     const long long gy_elems = (long long)d.Cout * Kr;
     if (xb_chunks * 16 >= ((long long)1 << 31) || gy_elems * ES >= ((long long)1 << 31) || Kr >= ((long long)1 << 31))
         return -1;
-    const int bm = (d.Cout >= 128 && d.Cin >= 128) ? 128 : 64;
+    // fp16 layers whose channel counts fill 256x256 tiles take those (a quarter less LDS traffic and half the L2 -> LDS
+    // traffic per MFMA of the 128x128 tile, and a quarter of the partial sums)
+    const int bm = (ES == 2 && d.Cout % 256 == 0 && d.Cin % 256 == 0 && st.gemm_path != 4) ? 256
+                   : (d.Cout >= 128 && d.Cin >= 128)                                          ? 128
+                                                                                              : 64;
     const long long tiles = (long long)((d.Cout + bm - 1) / bm) * ((d.Cin + bm - 1) / bm);
     // k splits: one workgroup of this tile holds a CU (96 KB of ring), so the launch runs in rounds of num_cu
     // workgroups.  Take the split count with the least rounds x (slabs per workgroup + the fixed cost of a
@@ -410,8 +414,15 @@ int conv_taps_wg(const ConvTileDesc &d, const void *X, const void *dY, void *dW)
     q.tap_jump_x = (long long)(hwc ? d.Cin : VEC) * ES;  // one padded position further in the second operand
     q.tap_jump_y = (long long)Wp * (hwc ? d.Cin : VEC) * ES;
     if (!plain_operand<T>(q.a, q.kchunk, q.K) || !plain_operand<T>(q.b, q.kchunk, q.K)) return -1;
-    int rc = bm == 128 ? launch_plain<T, 128, 128, 512, 2, 2, 2, 3, 1>(q, st.stream)
+    int rc;
+    if constexpr (ES == 2) {
+        rc = bm == 256   ? launch_plain<T, 256, 256, 512, 2, 4, 1, 2, 1>(q, st.stream)
+             : bm == 128 ? launch_plain<T, 128, 128, 512, 2, 2, 2, 3, 1>(q, st.stream)
+                         : launch_plain<T, 64, 64, 1024, 2, 2, 4, 3, 1>(q, st.stream);
+    } else {
+        rc = bm == 128 ? launch_plain<T, 128, 128, 512, 2, 2, 2, 3, 1>(q, st.stream)
                        : launch_plain<T, 64, 64, 1024, 2, 2, 4, 3, 1>(q, st.stream);
+    }
     if (rc != 0 || q.splits == 1) return rc;  // a single 1x1 tap without k split wrote dW itself
     const long long total = (long long)d.Cout * d.Cin;
     hipLaunchKernelGGL((taps_wg_reduce_kernel<T>), dim3((unsigned)((total + 63) / 64), taps), dim3(256), 0, st.stream,
