@@ -246,16 +246,20 @@ int ptl_sync(void);
  * convolution kernel is taken whenever the geometry fits it, however small the
  * call; 3 = as 0, but the sum-over-filter-taps route (unit-stride layers whose
  * channel counts fill whole 128-byte slabs) is taken whenever the geometry fits
- * it.  All routes compute the same products.
+ * it, on the pipelined GEMM; 5 = the same route with the input tile resident in
+ * LDS for all taps (3x3 fp16 channel-major layers) wherever that kernel fits.
+ * All routes compute the same products.
  * ptl_last_conv_direct() tells whether the last Conv2D call ran one of the
  * convolution kernels (1) or the implicit-im2col GEMM (0);
  * ptl_last_gemm_streamed() whether the last product that went to the pipelined
  * GEMM ran its streaming kernel (resident row panel, column tiles streamed:
  * the route of pointwise layers over a batch) (1) or a tile-per-workgroup
- * kernel (0). */
+ * kernel (0); ptl_last_conv_resident() whether the last Conv2D forward or
+ * input-gradient call that took the tap route kept its input tile in LDS (1). */
 void ptl_set_gemm_path(int path);
 int ptl_last_conv_direct(void);
 int ptl_last_gemm_streamed(void);
+int ptl_last_conv_resident(void);
 /* hipEvent timing on the library stream: begin records, end records,
  * synchronises and returns the elapsed milliseconds (negative on error). */
 int ptl_timer_begin(void);

@@ -76,7 +76,7 @@ BATCHED_ENTRY_POINTS = ["ptl_%s_%s_%s_batched" % (layer, dt, step)
                             "ptl_gradient_descent_fp32_multi", "ptl_gradient_descent_fp16_multi"]
 
 OTHER_ENTRY_POINTS = ["ptl_init", "ptl_last_error", "ptl_last_status", "ptl_set_stream", "ptl_sync", "ptl_set_gemm_path",
-                      "ptl_last_conv_direct", "ptl_last_gemm_streamed", "ptl_timer_begin", "ptl_timer_end_ms", "ptl_mm_fp32", "ptl_mm_fp16", "ptl_copy_bytes"]
+                      "ptl_last_conv_direct", "ptl_last_gemm_streamed", "ptl_last_conv_resident", "ptl_timer_begin", "ptl_timer_end_ms", "ptl_mm_fp32", "ptl_mm_fp16", "ptl_copy_bytes"]
 
 
 def load():
@@ -118,6 +118,8 @@ def load():
     lib.ptl_last_conv_direct.restype = ctypes.c_int
     lib.ptl_last_gemm_streamed.argtypes = []
     lib.ptl_last_gemm_streamed.restype = ctypes.c_int
+    lib.ptl_last_conv_resident.argtypes = []
+    lib.ptl_last_conv_resident.restype = ctypes.c_int
     lib.ptl_sync.argtypes = []
     lib.ptl_sync.restype = ctypes.c_int
     lib.ptl_timer_begin.argtypes = []

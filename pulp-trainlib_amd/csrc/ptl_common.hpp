@@ -137,8 +137,9 @@ struct State {
     hipEvent_t ev0 = nullptr, ev1 = nullptr;
     int num_cu = 256;
     void *zeros = nullptr;  // 256 zero bytes: source of elements that do not exist
-    int gemm_path = 0;      // 0: fastest kernel that fits; 1: staged GEMM only; 2: direct convolution whenever it fits; 3: tap-sum route whenever it fits
+    int gemm_path = 0;      // 0: fastest kernel that fits; 1: staged GEMM only; 2: direct convolution whenever it fits; 3: tap-sum route on the GEMM whenever it fits; 5: tap-sum route, LDS-resident input tile where it fits
     int last_gemm_streamed = 0;  // 1 if the last pipelined GEMM ran the streaming kernel
+    int last_conv_resident = 0;  // 1 if the last Conv2D forward / input-gradient call kept its input tile in LDS for all taps
     int last_conv_direct = 0;  // 1 if the last Conv2D forward / input-gradient call ran the direct kernel
 };
 

@@ -151,11 +151,18 @@ int conv_taps(const ConvTileDesc &d, const void *X, const void *Wt, void *Y, con
     // 10.5 against 11.3 us (forward) and 16.5 us (input gradient, flipped filters) for 64 -> 64 channels on 8x8
     // images at batch 128, 16.8 against 27.8 us for the input gradient of 128 -> 128.
     const long long fill = npix / 128 * ((d.Cout + 127) / 128) * 4;
-    if (st.gemm_path != 3 && (d.Cout < 64 || fill < st.num_cu)) return -1;
-    char *buf = static_cast<char *>(scratch((size_t)(xb_elems + wr_elems) * ES + 256));
+    const bool forced = st.gemm_path == 3 || st.gemm_path == 5;
+    if (!forced && (d.Cout < 64 || fill < st.num_cu)) return -1;
+    // 3x3 fp16 layers keep the input tile in LDS for all nine taps (ptl_conv_halo.hip): the tap-sum GEMM fetches it
+    // once per tap.  Measured at batch 128..512, forward: 64 -> 64 on 56x56 63 against 96 us, 128 -> 128 on 28x28
+    // 52 against 76, 256 -> 256 on 28x28 295 against 372, 512 -> 512 on 14x14 273 against 293.
+    const bool halo = ES == 2 && !hwc && conv_halo_fits(d, Hp, Wp) && (long long)d.batch * Hp * Wp < ((long long)1 << 31) &&
+                      (st.gemm_path == 5 || st.gemm_path == 0);
+    const long long margin = halo ? conv_halo_margin() : 0;  // chunks the resident-tile kernel may read past the end
+    char *buf = static_cast<char *>(scratch((size_t)(xb_elems + margin * VEC + wr_elems) * ES + 256));
     if (!buf) return 2;
     uint4 *xb = reinterpret_cast<uint4 *>(buf);
-    T *wr = reinterpret_cast<T *>(buf + (((size_t)xb_elems * ES + 255) & ~(size_t)255));
+    T *wr = reinterpret_cast<T *>(buf + (((size_t)(xb_elems + margin * VEC) * ES + 255) & ~(size_t)255));
     {
         TapPrepArgs p = {};
         p.in = X;
@@ -164,7 +171,7 @@ int conv_taps(const ConvTileDesc &d, const void *X, const void *Wt, void *Y, con
         p.cblocks = cblocks;
         p.hwc = hwc;
         p.sb = d.x_sb; p.sc = d.x_sc;
-        p.xb_total = xb_elems / VEC;
+        p.xb_total = xb_elems / VEC + margin;
         p.copy_blocks = (unsigned)((p.xb_total + 255) / 256);
         p.w = Wt;
         p.wr = wr;
@@ -175,6 +182,9 @@ int conv_taps(const ConvTileDesc &d, const void *X, const void *Wt, void *Y, con
                            0, st.stream, p);
         if (!hip_ok(hipGetLastError(), "layout launch")) return 2;
     }
+
+    st.last_conv_resident = halo;
+    if (halo) return conv_halo_launch(d, xb, wr, Y, Hp, Wp);
 
     GemmArgs q = {};
     q.A = xb;

@@ -77,6 +77,13 @@ inline int conv_raw_rows(int bm, int Ho, int Wo, int sh, int KH, int THP, long l
 template <typename T>
 int conv_taps(const ConvTileDesc &d, const void *X, const void *Wt, void *Y, const OutMap &c);
 
+// 3x3 unit-stride fp16 channel-major layers with the input tile resident in LDS for all taps (same prepared
+// operands as the tap-sum route: blocked padded input with conv_halo_margin() readable chunks behind it, tap-major
+// filters).  Y is the dense channel-major output [batch][Cout][Ho][Wo].
+bool conv_halo_fits(const ConvTileDesc &d, int Hp, int Wp);
+long long conv_halo_margin();
+int conv_halo_launch(const ConvTileDesc &d, const void *xb, const void *wr, void *Y, int Hp, int Wp);
+
 // Weight gradient over filter taps on the same GEMM (partial sums per tap and k split + one reduction).
 template <typename T>
 int conv_taps_wg(const ConvTileDesc &d, const void *X, const void *dY, void *dW);

@@ -253,6 +253,7 @@ static int conv2d_fw(const Args *a, int ns, const char *fn) {
 
     int rc = -1;
     state().last_conv_direct = 0;
+    state().last_conv_resident = 0;
     if (state().gemm_path != 1) {
         ConvTileDesc d = {};
         d.batch = ns; d.Cin = g.Ci; d.Hin = g.H; d.Win = g.W;
@@ -343,6 +344,7 @@ static int conv2d_wg(const Args *a, int ns, const char *fn) {
 
     int rc = -1;
     state().last_conv_direct = 0;
+    state().last_conv_resident = 0;
     if (state().gemm_path != 1) {
         ConvTileDesc d = {};
         d.in_hwc = g.hwc ? 1 : 0;
@@ -493,6 +495,7 @@ static int conv2d_ig(const Args *a, int ns, const char *fn) {
     gmap.row.wb = g.Lp;
     gmap.k.n = K;
     state().last_conv_direct = 0;
+    state().last_conv_resident = 0;
     if (state().gemm_path != 1) {
         ConvTileDesc d = {};
         d.batch = ns; d.Cin = g.Co; d.Hin = Hd; d.Win = Wd;

@@ -271,6 +271,7 @@ void ptl_set_stream(void *s) {
 void ptl_set_gemm_path(int path) { ptl::state().gemm_path = path; }
 int ptl_last_conv_direct(void) { return ptl::state().last_conv_direct; }
 int ptl_last_gemm_streamed(void) { return ptl::state().last_gemm_streamed; }
+int ptl_last_conv_resident(void) { return ptl::state().last_conv_resident; }
 
 int ptl_sync(void) {
     if (!ptl::ensure_init()) return 2;

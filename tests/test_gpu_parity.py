@@ -235,6 +235,60 @@ def test_conv2d_tap_sum_route(pkg, orc, gpu, dt, case):
         gpu.ptl_set_gemm_path(0)
 
 
+# 3x3 fp16 channel-major layers through the kernel that keeps the input tile in LDS for all nine taps (path 5):
+# forward when Ci and Co are multiples of 64, input gradient likewise.  Cases: one and two channel slabs, 64 and
+# 128 filters per tile, asymmetric padding, the widest image the tile holds, too wide an image (falls back).
+RESIDENT_CASES = [
+    # Ci, H, W, Co, pad(L,R,U,D), ns, resident
+    (64, 14, 14, 64, (1, 1, 1, 1), 4, 1),
+    (128, 9, 11, 64, (1, 1, 1, 1), 3, 1),
+    (64, 12, 10, 128, (0, 2, 1, 0), 2, 1),
+    (64, 7, 61, 64, (1, 1, 1, 1), 1, 1),
+    (64, 5, 62, 64, (1, 1, 1, 1), 1, 0),
+    (192, 6, 6, 256, (0, 0, 0, 0), 2, 1),
+]
+
+
+@pytest.mark.parametrize("case", RESIDENT_CASES)
+def test_conv2d_resident_tile_route(pkg, orc, gpu, case):
+    Ci, H, W, Co, pad, ns, resident = case
+    gpu.ptl_set_gemm_path(5)
+    try:
+        conv_parity(pkg, orc, gpu, "fp16", Ci, H, W, Co, 3, 3, pad, (1, 1), 0, ns, 0xC0DE0075, via_batched=True)
+        assert gpu.ptl_last_conv_resident() == resident  # (the input gradient ran last)
+    finally:
+        gpu.ptl_set_gemm_path(0)
+
+
+def test_conv2d_resident_tile_many_tiles(pkg, gpu):
+    """More position tiles than workgroups (every workgroup walks several tiles, the last one ragged) and two
+    filter tiles: the resident-tile kernel against the tap-sum GEMM and against torch in float32."""
+    import torch.nn.functional as F
+    Ci, Co, H, W, ns = 128, 256, 30, 30, 80
+    nd = np.float16
+    x, w = dev(hp.uniform(21, (ns, Ci, H, W), dtype=nd)), dev(hp.uniform(22, (Co, Ci, 3, 3), dtype=nd) * 0.1)
+    dy = dev(hp.uniform(23, (ns, Co, H, W), dtype=nd))
+    res = {}
+    for path in (3, 5):
+        y, dx = dev(np.zeros((ns, Co, H, W), nd)), dev(np.zeros((ns, Ci, H, W), nd))
+        a, keep = hp.conv2d_args(pkg, x, dx, w, None, y, dy, Ci, H, W, Co, 3, 3, H, W, (1, 1, 1, 1), (1, 1))
+        gpu.ptl_set_gemm_path(path)
+        try:
+            for s in ("fw", "ig"):
+                pkg.call("ptl_conv2d_fp16_%s_batched" % s, a, ns)
+                assert gpu.ptl_last_conv_resident() == (1 if path == 5 else 0)
+        finally:
+            gpu.ptl_set_gemm_path(0)
+        sync(gpu)
+        res[path] = [y.float(), dx.float()]
+    ref_y = F.conv2d(x.float(), w.float(), padding=1)
+    ref_dx = torch.nn.grad.conv2d_input(x.shape, w.float(), dy.float(), padding=1)
+    rel = lambda got, ref: float((got - ref).norm() / ref.norm())
+    for got, other, ref in zip(res[5], res[3], (ref_y, ref_dx)):
+        assert rel(got, ref) <= 1e-3
+        assert rel(got, other) <= 1e-3
+
+
 def test_conv2d_routes_agree_on_large_channels(pkg, gpu):
     """The tap-sum route, the direct kernels and the implicit-im2col GEMM give the same forward, weight gradient
     and input gradient (fp16, 64 -> 64 channels)."""
