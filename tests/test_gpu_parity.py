@@ -237,10 +237,12 @@ def test_conv2d_tap_sum_route(pkg, orc, gpu, dt, case):
 
 # 3x3 fp16 channel-major layers through the kernel that keeps the input tile in LDS for all nine taps (path 5):
 # forward when Ci and Co are multiples of 64, input gradient likewise.  Cases: one and two channel slabs, 64 and
-# 128 filters per tile, asymmetric padding, the widest image the tile holds, too wide an image (falls back).
+# 128 filters per tile, asymmetric padding, images small enough for the bottom rows of the padded grid to be left out
+# (tiles that cross one and two sample boundaries), the widest image the tile holds, too wide an image (falls back).
 RESIDENT_CASES = [
     # Ci, H, W, Co, pad(L,R,U,D), ns, resident
     (64, 14, 14, 64, (1, 1, 1, 1), 4, 1),
+    (64, 28, 28, 64, (1, 1, 1, 1), 3, 1),
     (128, 9, 11, 64, (1, 1, 1, 1), 3, 1),
     (64, 12, 10, 128, (0, 2, 1, 0), 2, 1),
     (64, 7, 61, 64, (1, 1, 1, 1), 1, 1),
