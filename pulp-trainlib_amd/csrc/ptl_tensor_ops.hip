@@ -637,6 +637,189 @@ __global__ __launch_bounds__(256) void dw_wg_plane_pairs_kernel(const half_t *__
     }
 }
 
+// ---- 3x3 fp16 planes straight from global memory -----------------------------------------------------------
+// Rows readable as pairs (see dw_row_pairs).  A lane owns a block of DW_DRB output rows x 8 columns and loads
+// the DW_DRB + 2 source row segments it needs itself (one 16-byte and one 4-byte load per row, 4-byte aligned):
+// no LDS, no barrier, and the blocks of all planes are dealt to the lanes without gaps (a wave may straddle two
+// planes).  Neighbouring lanes overlap by two elements per row and two rows per block, which the L1/L2 absorb:
+// the planes cross the HBM interface once.
+constexpr int DW_DRB = 7;
+
+// P[hr][m] = elements (cf + 2m, cf + 2m + 1) of source row r0 - pu + hr, zero outside the plane.
+template <int ROWS>
+__device__ inline void dw_direct_rows(const half_t *__restrict__ sp, int Hs, int Ws, int h0, int cf,
+                                      unsigned (&P)[ROWS][5]) {
+    const bool inner = cf >= 0 && cf + 10 <= Ws;
+#pragma unroll
+    for (int hr = 0; hr < ROWS; ++hr) {
+        const int h = h0 + hr;
+        const unsigned *row = reinterpret_cast<const unsigned *>(sp + h * Ws + cf);
+        if ((unsigned)h < (unsigned)Hs) {
+            if (inner) {
+#pragma unroll
+                for (int m = 0; m < 5; ++m) P[hr][m] = row[m];
+            } else {
+#pragma unroll
+                for (int m = 0; m < 5; ++m) P[hr][m] = (unsigned)(cf + 2 * m) < (unsigned)Ws ? row[m] : 0u;
+            }
+        } else {
+#pragma unroll
+            for (int m = 0; m < 5; ++m) P[hr][m] = 0u;
+        }
+    }
+}
+
+template <bool FLIP>
+__global__ __launch_bounds__(256) void dw_direct_kernel(const half_t *__restrict__ src, const half_t *__restrict__ Wt,
+                                                        half_t *__restrict__ dst, int C, int Hs, int Ws, int Hd, int Wd,
+                                                        int pu, int pl, int rblocks, int groups, unsigned total) {
+    constexpr int RB = DW_DRB;
+    const unsigned id = blockIdx.x * 256u + threadIdx.x;
+    if (id >= total) return;
+    const unsigned per_plane = (unsigned)(rblocks * groups);
+    const unsigned plane = id / per_plane, blk = id - plane * per_plane;
+    const int rb = (int)(blk / (unsigned)groups), c0 = (int)(blk - (unsigned)rb * groups) * 8, r0 = rb * RB;
+    const int ch = (int)(plane % (unsigned)C);
+    dw_h2 we[3], wo[3];
+    float w0[3], w2[3];
+#pragma unroll
+    for (int i = 0; i < 3; ++i) {
+        half_t wr[3];
+#pragma unroll
+        for (int j = 0; j < 3; ++j) wr[j] = Wt[ch * 9 + (FLIP ? (2 - i) * 3 + (2 - j) : i * 3 + j)];
+        we[i] = dw_h2{wr[0], wr[1]};
+        wo[i] = dw_h2{wr[1], wr[2]};
+        w0[i] = (float)wr[0];
+        w2[i] = (float)wr[2];
+    }
+    unsigned P[RB + 2][5];
+    dw_direct_rows<RB + 2>(src + (size_t)plane * Hs * Ws, Hs, Ws, r0 - pu, c0 - pl, P);
+    float acc[RB][8];
+#pragma unroll
+    for (int r = 0; r < RB; ++r)
+#pragma unroll
+        for (int q = 0; q < 8; ++q) acc[r][q] = 0.f;
+#pragma unroll
+    for (int hr = 0; hr < RB + 2; ++hr) {
+#pragma unroll
+        for (int i = 0; i < 3; ++i) {
+            const int r = hr - i;
+            if (r < 0 || r >= RB) continue;
+#pragma unroll
+            for (int q = 0; q < 8; ++q) {
+                float a = acc[r][q];
+                if ((q & 1) == 0) {
+                    a = __builtin_amdgcn_fdot2(__builtin_bit_cast(dw_h2, P[hr][q / 2]), we[i], a, false);
+                    a = fmaf((float)__builtin_bit_cast(dw_h2, P[hr][q / 2 + 1]).x, w2[i], a);
+                } else {
+                    a = fmaf((float)__builtin_bit_cast(dw_h2, P[hr][q / 2]).y, w0[i], a);
+                    a = __builtin_amdgcn_fdot2(__builtin_bit_cast(dw_h2, P[hr][q / 2 + 1]), wo[i], a, false);
+                }
+                acc[r][q] = a;
+            }
+        }
+    }
+    half_t *dp = dst + (size_t)plane * Hd * Wd;
+    const int valid = min(8, Wd - c0);
+#pragma unroll
+    for (int r = 0; r < RB; ++r) {
+        if (r0 + r >= Hd) continue;
+        half_t *o = dp + (size_t)(r0 + r) * Wd + c0;
+        if (valid == 8) {  // (rows are whole dwords: a 16-byte global store needs no more than 4-byte alignment)
+            typedef unsigned u4a __attribute__((ext_vector_type(4), aligned(4)));
+            union {
+                u4a v;
+                half_t e[8];
+            } u;
+#pragma unroll
+            for (int q = 0; q < 8; ++q) u.e[q] = (half_t)acc[r][q];
+            *reinterpret_cast<u4a *>(o) = u.v;
+        } else {
+#pragma unroll
+            for (int q = 0; q < 8; ++q)
+                if (q < valid) o[q] = (half_t)acc[r][q];
+        }
+    }
+}
+
+// Weight gradient the same way: a wave walks planes (b, ch) of its sample group, a lane takes blocks of DW_DRB
+// gradient rows x 8 columns with the source rows they meet, the nine tap sums stay in registers; one reduction
+// per workgroup at the end.  part[(grp * C + ch) * 9 + tap], or the gradient itself when there is one group.
+__global__ __launch_bounds__(256) void dw_wg_direct_kernel(const half_t *__restrict__ X, const half_t *__restrict__ dY,
+                                                           float *__restrict__ part, int C, int ns, int per_group, int H,
+                                                           int W, int Ho, int Wo, int pu, int pl,
+                                                           half_t *__restrict__ direct) {
+    constexpr int RB = DW_DRB;
+    __shared__ float red[4][9];
+    const int ch = blockIdx.x, grp = blockIdx.y;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    float acc[3][3];
+#pragma unroll
+    for (int i = 0; i < 3; ++i)
+#pragma unroll
+        for (int j = 0; j < 3; ++j) acc[i][j] = 0.f;
+    const int groups = (Wo + 7) >> 3, rblocks = (Ho + RB - 1) / RB;
+    const int b_end = min(ns, (grp + 1) * per_group);
+    for (int b = grp * per_group + wave; b < b_end; b += 4) {
+        const size_t plane = (size_t)b * C + ch;
+        const half_t *xp = X + plane * H * W, *gp = dY + plane * Ho * Wo;
+        for (int item = lane; item < rblocks * groups; item += 64) {
+            const int rb = item / groups, c0 = (item - rb * groups) * 8, r0 = rb * RB;
+            dw_h2 G[RB][4];
+#pragma unroll
+            for (int r = 0; r < RB; ++r) {
+                const unsigned *grow = reinterpret_cast<const unsigned *>(gp + (r0 + r) * Wo + c0);
+                if (r0 + r < Ho && c0 + 8 <= Wo) {
+#pragma unroll
+                    for (int m = 0; m < 4; ++m) G[r][m] = __builtin_bit_cast(dw_h2, grow[m]);
+                } else {
+#pragma unroll
+                    for (int m = 0; m < 4; ++m)
+                        G[r][m] = __builtin_bit_cast(dw_h2, (r0 + r < Ho && c0 + 2 * m < Wo) ? grow[m] : 0u);
+                }
+            }
+            unsigned P[RB + 2][5];
+            dw_direct_rows<RB + 2>(xp, H, W, r0 - pu, c0 - pl, P);
+#pragma unroll
+            for (int hr = 0; hr < RB + 2; ++hr) {  // source row r0 - pu + hr meets gradient rows r0 + hr - i
+                unsigned U[4];
+#pragma unroll
+                for (int m = 0; m < 4; ++m) U[m] = __builtin_amdgcn_alignbit(P[hr][m + 1], P[hr][m], 16);
+#pragma unroll
+                for (int i = 0; i < 3; ++i) {
+                    if (hr - i < 0 || hr - i >= RB) continue;
+#pragma unroll
+                    for (int j = 0; j < 3; ++j) {
+                        float a = acc[i][j];
+#pragma unroll
+                        for (int m = 0; m < 4; ++m)
+                            a = __builtin_amdgcn_fdot2(__builtin_bit_cast(dw_h2, j == 1 ? U[m] : P[hr][m + j / 2]),
+                                                       G[hr - i][m], a, false);
+                        acc[i][j] = a;
+                    }
+                }
+            }
+        }
+    }
+#pragma unroll
+    for (int i = 0; i < 3; ++i)
+#pragma unroll
+        for (int j = 0; j < 3; ++j) {
+            float v = acc[i][j];
+#pragma unroll
+            for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
+            if (lane == 0) red[wave][i * 3 + j] = v;
+        }
+    __syncthreads();
+    if (tid < 9) {
+        const float sum = (red[0][tid] + red[1][tid]) + (red[2][tid] + red[3][tid]);
+        if (direct)
+            direct[(size_t)ch * 9 + tid] = (half_t)sum;
+        else
+            part[((size_t)grp * C + ch) * 9 + tid] = sum;
+    }
+}
+
 template <typename Args>
 static int dw_geom(const Args *a, DwGeom &g, int sh, int sw, const char *fn) {
     if (!a || !a->input || !a->coeff || !a->output) {
@@ -682,6 +865,18 @@ static void launch_dw_plane(const T *src, const T *Wt, T *dst, int C, int Hs, in
                             long planes, hipStream_t stream) {
     const size_t src_img = (size_t)Hs * Ws * sizeof(T) + 32;
     if constexpr (sizeof(T) == 2) {
+        // 3x3 with rows of whole dwords on both sides, forward geometry (every column group full): straight from
+        // global memory
+        if (K == 3 && !FLIP && Ws % 2 == 0 && Wd % 8 == 0 && pl % 2 == 0 && reinterpret_cast<uintptr_t>(src) % 4 == 0 &&
+            reinterpret_cast<uintptr_t>(dst) % 4 == 0) {
+            const int rblocks = (Hd + DW_DRB - 1) / DW_DRB, groups = (Wd + 7) / 8;
+            const long long total = (long long)planes * rblocks * groups;
+            if (total < ((long long)1 << 31)) {
+                hipLaunchKernelGGL((dw_direct_kernel<FLIP>), dim3((unsigned)((total + 255) / 256)), dim3(256), 0, stream,
+                                   src, Wt, dst, C, Hs, Ws, Hd, Wd, pu, pl, rblocks, groups, (unsigned)total);
+                return;
+            }
+        }
         // rows readable as pairs: see dw_plane_pairs_kernel
         if (Ws % 2 == 0 && pl % 2 == 0 && reinterpret_cast<uintptr_t>(src) % 4 == 0) {
             hipLaunchKernelGGL((dw_plane_pairs_kernel<K, FLIP>), dim3((unsigned)planes), dim3(128), src_img, stream, src,
@@ -817,7 +1012,10 @@ static int dw_step(const Args *a, int ns, int step, int sh, int sw, const char *
         if constexpr (sizeof(T) == 2) {
             pairs = g.W % 2 == 0 && g.Wo % 2 == 0 && g.Lp % 2 == 0 && reinterpret_cast<uintptr_t>(X) % 4 == 0 &&
                     reinterpret_cast<uintptr_t>(dY) % 4 == 0;
-            if (pairs) {
+            if (pairs && g.Hk == 3 && ns > 1) {
+                hipLaunchKernelGGL(dw_wg_direct_kernel, grid, dim3(256), 0, st.stream, X, dY, part, g.C, ns, per_group, g.H,
+                                   g.W, g.Ho, g.Wo, g.Up, g.Lp, direct);
+            } else if (pairs) {
                 if (g.Hk == 3)
                     hipLaunchKernelGGL((dw_wg_plane_pairs_kernel<3>), grid, dim3(256), lds, st.stream, X, dY, part, g.C,
                                        ns, per_group, g.H, g.W, g.Ho, g.Wo, g.Up, g.Lp, x_vecs, direct);
