@@ -598,7 +598,10 @@ def test_depthwise(pkg, orc, gpu, dt, C, H, W, K, pad, ns):
 
 # Batches with at least two planes per CU run the plane-resident kernels: even and odd row lengths (fp16 rows of
 # even length are read as pairs of neighbours), 3x3 and 5x5, and padded fp32 planes.
-@pytest.mark.parametrize("dt,C,H,W,K,pad,ns", [("fp16", 64, 36, 36, 3, (0, 0, 0, 0), 8), ("fp16", 64, 35, 37, 3, (0, 0, 0, 0), 8),
+# fp16 3x3 planes whose output rows are whole 16-byte groups load their blocks straight from global memory (forward;
+# the weight gradient whenever rows are whole dwords): full and ragged row blocks, an even left pad.
+@pytest.mark.parametrize("dt,C,H,W,K,pad,ns", [("fp16", 64, 34, 34, 3, (0, 0, 0, 0), 8), ("fp16", 64, 23, 32, 3, (2, 0, 1, 1), 8),
+                                               ("fp16", 64, 36, 36, 3, (0, 0, 0, 0), 8), ("fp16", 64, 35, 37, 3, (0, 0, 0, 0), 8),
                                                ("fp16", 32, 38, 40, 5, (0, 0, 0, 0), 16), ("fp16", 32, 37, 39, 5, (0, 0, 0, 0), 16),
                                                ("fp32", 64, 36, 36, 3, (0, 0, 0, 0), 8), ("fp32", 64, 35, 37, 3, (1, 1, 1, 1), 8),
                                                ("fp32", 32, 38, 38, 5, (2, 2, 2, 2), 16)])
