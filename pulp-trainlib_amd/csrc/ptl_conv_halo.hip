@@ -287,6 +287,198 @@ int launch_halo_pipe(const HaloArgs &a, int grid, hipStream_t stream) {
     return hip_ok(hipGetLastError(), "halo convolution launch") ? 0 : 2;
 }
 
+
+// ---------------------------------------------------------------------------------------------------------
+// Weight gradient on the same layouts:
+//   dW[co][ci][ky][kx] = sum over padded positions p of  gb[p][co] * xb[p + ky*Wp + kx][ci]
+// with gb the output gradient embedded at the top left of the padded grids (zero elsewhere), channel-blocked
+// like xb.  The contraction runs over positions, so both operands sit in LDS as [position][8 channels] chunks
+// and a fragment is two transposing reads (ds_read_b64_tr_b16); a tap is a shift by whole chunks, so every
+// read stays aligned.  A workgroup (4 waves) owns 128 filters x 64 channels x a group of taps (0..4 or 5..8)
+// and a range of positions; it walks units of 128 positions (gradient tile 32 KB + input tile of 256 positions
+// 32 KB, two buffers, the next unit in flight while this one is multiplied) with all accumulators in registers
+// and writes one fp32 partial sum per tap at the end; a second kernel adds the partial sums.
+constexpr int HWG_UNIT = 128;                 // positions per unit
+constexpr int HWG_GP = 132, HWG_XP = 260;     // LDS pitches (chunks) of the gradient / input tiles: == 4 mod 16,
+                                              // so that the 16 rows of a transposing read fall on distinct banks
+constexpr int HWG_GB = 16 * HWG_GP * 16, HWG_XB = 8 * HWG_XP * 16, HWG_BUF = HWG_GB + HWG_XB;
+
+struct HaloWgArgs {
+    const char *xb;    // [Cin/8][Px] chunks, readable 256 chunks past the start of the last unit
+    const char *gb;    // [Cout/8][Pd] chunks, Pd a multiple of HWG_UNIT, zero from the last padded position on
+    float *ws;         // partial sums [tap][smax][Cout][Cin]
+    long long Px, Pd;
+    int Cin, Cout, Wp;
+    int units;         // Pd / HWG_UNIT
+    int tiles_ci;      // Cin / 64
+    int tiles;         // (Cout / 128) * (Cin / 64)
+    int S0, S1, smax;  // position splits of the two tap groups
+};
+
+typedef short hwg_s4 __attribute__((ext_vector_type(4)));
+typedef __attribute__((address_space(3))) hwg_s4 hwg_lds_s4;
+
+__device__ inline uint4 hwg_frag(const char *p) {
+    union {
+        hwg_s4 h[2];
+        uint4 v;
+    } t;
+    t.h[0] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((hwg_lds_s4 *)(lds_char *)p);
+    t.h[1] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((hwg_lds_s4 *)(lds_char *)(p + 64));
+    return t.v;
+}
+
+template <int T0, int NT>
+__device__ inline void halo_wg_body(const HaloWgArgs &a, char *smem, int tile, int split, int S) {
+    const unsigned lds0 = (unsigned)(uintptr_t)(lds_char *)smem;
+    const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int wm = wave & 1, wn = wave >> 1;
+    const int i16 = lane & 15, g16 = (lane >> 4) & 1, kg = lane >> 5;
+    const int co_cb0 = (tile / a.tiles_ci) * 16, ci_cb0 = (tile % a.tiles_ci) * 8;
+    const int u0 = (int)((long long)split * a.units / S), u1 = (int)((long long)(split + 1) * a.units / S);
+    const unsigned voff = (unsigned)lane * 16u;
+
+    auto issue = [&](int u, int buf) {
+        const long long p0 = (long long)u * HWG_UNIT;
+#pragma unroll
+        for (int q = 0; q < 16; ++q) {
+            const int idx = q * 4 + wave;
+            if (q < 8) {  // gradient tile: 16 channel blocks x 2 pieces of 64 positions
+                const int cb = idx >> 1, piece = idx & 1;
+                const char *base = a.gb + ((long long)(co_cb0 + cb) * a.Pd + p0 + piece * 64) * 16;
+                lds_dma16_saddr(voff, base, lds0 + (unsigned)(buf * HWG_BUF + (cb * HWG_GP + piece * 64) * 16));
+            } else {  // input tile: 8 channel blocks x 4 pieces
+                const int j = idx - 32, cb = j >> 2, piece = j & 3;
+                const char *base = a.xb + ((long long)(ci_cb0 + cb) * a.Px + p0 + piece * 64) * 16;
+                lds_dma16_saddr(voff, base,
+                                lds0 + (unsigned)(buf * HWG_BUF + HWG_GB + (cb * HWG_XP + piece * 64) * 16));
+            }
+        }
+    };
+
+    // this lane's piece of a transposing read: position k0 + i16 / 4 of channel block .. + (i16 & 3) / 2,
+    // channels 4 * (i16 & 1) .. + 3 of that block
+    const unsigned ga = (unsigned)((((wm * 8 + 2 * g16 + ((i16 & 3) >> 1)) * HWG_GP + 8 * kg + (i16 >> 2)) * 16) + (i16 & 1) * 8);
+    const unsigned xa = (unsigned)(HWG_GB + (((wn * 4 + 2 * g16 + ((i16 & 3) >> 1)) * HWG_XP + 8 * kg + (i16 >> 2)) * 16) +
+                                   (i16 & 1) * 8);
+    int tapoff[NT];
+#pragma unroll
+    for (int t = 0; t < NT; ++t) tapoff[t] = (((T0 + t) / 3) * a.Wp + (T0 + t) % 3) * 16;
+
+    f32x16 acc[2][NT];
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int t = 0; t < NT; ++t)
+#pragma unroll
+            for (int v = 0; v < 16; ++v) acc[i][t][v] = 0.f;
+
+    if (u0 < u1) issue(u0, 0);
+    for (int u = u0; u < u1; ++u) {
+        const int buf = (u - u0) & 1;
+        wait_vmcnt<0>();
+        __syncthreads();  // unit u has landed for every wave, and every wave has left unit u - 1
+        issue(u + 1 < u1 ? u + 1 : u, buf ^ 1);
+        const char *gt = smem + buf * HWG_BUF + ga, *xt = smem + buf * HWG_BUF + xa;
+        uint4 gf[2][2], xf[2][NT];
+        auto read = [&](int set, int ks) {
+#pragma unroll
+            for (int i = 0; i < 2; ++i) gf[set][i] = hwg_frag(gt + ks * 256 + i * 4 * HWG_GP * 16);
+#pragma unroll
+            for (int t = 0; t < NT; ++t) xf[set][t] = hwg_frag(xt + ks * 256 + tapoff[t]);
+        };
+        read(0, 0);
+        static_for<0, 8>([&](auto KI) {
+            constexpr int ks = decltype(KI)::value, cur = ks & 1;
+            if constexpr (ks + 1 < 8) read(cur ^ 1, ks + 1);
+#pragma unroll
+            for (int i = 0; i < 2; ++i)
+#pragma unroll
+                for (int t = 0; t < NT; ++t) mfma_step<half_t>(acc[i][t], gf[cur][i], xf[cur][t]);
+            if constexpr (ks + 1 < 8) {
+                // 2 * (2 + NT) transposing reads under 2 * NT MFMAs
+#pragma unroll
+                for (int m = 0; m < 4; ++m) {
+                    __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
+                    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+                }
+#pragma unroll
+                for (int m = 4; m < 2 * NT; ++m) {
+                    __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+                    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+                }
+            }
+        });
+    }
+    wait_vmcnt<0>();  // nothing may still be landing in LDS when the workgroup ends
+    if (u0 >= u1) return;
+    // partial sums: lane = channel, four consecutive filters per register group
+    const int co0 = (tile / a.tiles_ci) * 128 + wm * 64 + 4 * kg, ci = (tile % a.tiles_ci) * 64 + wn * 32 + (lane & 31);
+#pragma unroll
+    for (int t = 0; t < NT; ++t) {
+        float *dst = a.ws + (((size_t)(T0 + t) * a.smax + split) * a.Cout + co0) * a.Cin + ci;
+#pragma unroll
+        for (int i = 0; i < 2; ++i)
+#pragma unroll
+            for (int v = 0; v < 16; ++v) dst[(size_t)(i * 32 + 8 * (v >> 2) + (v & 3)) * a.Cin] = acc[i][t][v];
+    }
+}
+
+__global__ __launch_bounds__(HALO_NT) void conv_halo_wg_kernel(const HaloWgArgs a) {
+    extern __shared__ __align__(16) char smem[];
+    const int id = blockIdx.x, n0 = a.tiles * a.S0;
+    if (id < n0)
+        halo_wg_body<0, 5>(a, smem, id / a.S0, id % a.S0, a.S0);
+    else
+        halo_wg_body<5, 4>(a, smem, (id - n0) / a.S1, (id - n0) % a.S1, a.S1);
+}
+
+// dW[idx * 9 + tap] = sum over the splits of the tap's group of ws[tap][split][idx]
+__global__ __launch_bounds__(256) void conv_halo_wg_reduce_kernel(const float *__restrict__ ws, half_t *__restrict__ dW,
+                                                                  long long total, int S0, int S1, int smax) {
+    const long long idx = (long long)blockIdx.x * 256 + threadIdx.x;
+    const int tap = blockIdx.y;
+    if (idx >= total) return;
+    const int S = tap < 5 ? S0 : S1;
+    const float *src = ws + (size_t)tap * smax * total + idx;
+    float s = 0.f;
+    int z = 0;
+    for (; z + 4 <= S; z += 4) {
+        float v[4];
+#pragma unroll
+        for (int k = 0; k < 4; ++k) v[k] = src[(size_t)(z + k) * total];
+        s += (v[0] + v[1]) + (v[2] + v[3]);
+    }
+    for (; z < S; ++z) s += src[(size_t)z * total];
+    dW[idx * 9 + tap] = (half_t)s;
+}
+
+// gb[cb][p] for p < pstride: the gradient dY[b][8 cb .. + 7][y][x] at p = (b, y, x) of the padded grid (y < Ho,
+// x < Wo), zero elsewhere and from the last padded position on.
+__global__ __launch_bounds__(256) void conv_halo_embed_kernel(const half_t *__restrict__ dy, uint4 *__restrict__ out,
+                                                              int B, int Ho, int Wo, int Hp, int Wp, long long sb,
+                                                              long long sc, unsigned P, unsigned pstride,
+                                                              unsigned total) {
+    const unsigned i = blockIdx.x * 256u + threadIdx.x;
+    if (i >= total) return;
+    const unsigned cb = i / pstride, p = i - cb * pstride;
+    union {
+        uint4 v;
+        half_t e[8];
+    } u;
+    u.v = make_uint4(0, 0, 0, 0);
+    if (p < P) {
+        const unsigned r = p / (unsigned)Wp, xp = p - r * (unsigned)Wp;
+        const unsigned b = r / (unsigned)Hp, yp = r - b * (unsigned)Hp;
+        if (yp < (unsigned)Ho && xp < (unsigned)Wo) {
+            const half_t *src = dy + b * sb + (long long)(cb * 8) * sc + (long long)yp * Wo + xp;
+#pragma unroll
+            for (int e = 0; e < 8; ++e) u.e[e] = src[e * sc];
+        }
+    }
+    out[i] = u.v;
+}
+
 }  // namespace
 
 long long conv_halo_margin() { return HALO_BM + HALO_NP; }
@@ -321,6 +513,82 @@ int conv_halo_launch(const ConvTileDesc &d, const void *xb, const void *wr, void
 #endif
     const int grid = a.tiles < st.num_cu ? a.tiles : st.num_cu;
     return bn == 128 ? launch_halo_pipe<128, 4>(a, grid, st.stream) : launch_halo_pipe<64, 6>(a, grid, st.stream);
+}
+
+
+bool conv_halo_wg_fits(const ConvTileDesc &d, int Hp, int Wp) {
+    return !d.in_hwc && d.KH == 3 && d.KW == 3 && d.sh == 1 && d.sw == 1 && d.Cin % 64 == 0 && d.Cout % 128 == 0 &&
+           2 * Wp + 2 <= 128 && d.Ho == Hp - 2 && d.Wo == Wp - 2 && (long long)d.batch * Hp * Wp < ((long long)1 << 31);
+}
+// Measured against the alternatives (fp16, batch 128..512): 128 -> 128 on 28x28 73 / 243 against 87 / 306 us (resident
+// output tile kernel), 256 -> 256 on 14x14 70 against 83 us and on 28x28 384 against 390 us (tap-sum GEMM); 512 -> 512
+// on 14x14 359 against 353 us and 64 -> 128 on 56x56 280 against 274 us stay where they were.
+bool conv_halo_wg_preferred(const ConvTileDesc &d) {
+    const int Hp = d.Hin + d.padU + d.padD, Wp = d.Win + d.padL + d.padR;
+    return conv_halo_wg_fits(d, Hp, Wp) && Wp <= 32 && !(d.Cin >= 512 && d.Cout >= 512) &&
+           (long long)d.batch * Hp * Wp >= 64ll * HWG_UNIT;
+}
+long long conv_halo_wg_margin() { return 2 * HWG_UNIT + 256; }
+long long conv_halo_wg_gradient_stride(const ConvTileDesc &d, int Hp, int Wp) {
+    const long long P = (long long)d.batch * Hp * Wp;
+    return (P + HWG_UNIT - 1) / HWG_UNIT * HWG_UNIT;
+}
+size_t conv_halo_wg_partial_bytes(const ConvTileDesc &d, int Hp, int Wp, int *S0, int *S1) {
+    State &st = state();
+    const int tiles = (d.Cout / 128) * (d.Cin / 64);
+    const long long units = conv_halo_wg_gradient_stride(d, Hp, Wp) / HWG_UNIT;
+    // one workgroup per CU; the two tap groups (five and four taps) get position splits in the ratio 5 : 4 so that
+    // their workgroups finish together
+    long long per_tile = st.num_cu / tiles;
+    if (per_tile < 2) per_tile = 2;
+    long long s0 = (per_tile * 5 + 4) / 9, s1 = per_tile - s0;
+    if (s1 < 1) s1 = 1;
+    if (s0 > units) s0 = units;
+    if (s1 > units) s1 = units;
+    *S0 = (int)s0;
+    *S1 = (int)s1;
+    const long long smax = s0 > s1 ? s0 : s1;
+    return (size_t)9 * smax * d.Cout * d.Cin * sizeof(float);
+}
+
+// gb: room for (Cout / 8) * conv_halo_wg_gradient_stride() chunks; xb as for the forward kernel with
+// conv_halo_wg_margin() readable chunks behind it; ws: conv_halo_wg_partial_bytes().
+int conv_halo_wg_launch(const ConvTileDesc &d, const void *dY, const void *xb, void *gb, float *ws, void *dW, int Hp,
+                        int Wp, int S0, int S1) {
+    State &st = state();
+    const long long P = (long long)d.batch * Hp * Wp, Pd = conv_halo_wg_gradient_stride(d, Hp, Wp);
+    const long long chunks = (long long)(d.Cout / 8) * Pd;
+    if (chunks >= ((long long)1 << 31)) return -1;
+    hipLaunchKernelGGL(conv_halo_embed_kernel, dim3((unsigned)((chunks + 255) / 256)), dim3(256), 0, st.stream,
+                       static_cast<const half_t *>(dY), static_cast<uint4 *>(gb), d.batch, d.Ho, d.Wo, Hp, Wp,
+                       (long long)d.Cout * d.Ho * d.Wo, (long long)d.Ho * d.Wo, (unsigned)P, (unsigned)Pd,
+                       (unsigned)chunks);
+    if (!hip_ok(hipGetLastError(), "gradient layout launch")) return 2;
+    HaloWgArgs a = {};
+    a.xb = static_cast<const char *>(xb);
+    a.gb = static_cast<const char *>(gb);
+    a.ws = ws;
+    a.Px = P;
+    a.Pd = Pd;
+    a.Cin = d.Cin; a.Cout = d.Cout; a.Wp = Wp;
+    a.units = (int)(Pd / HWG_UNIT);
+    a.tiles_ci = d.Cin / 64;
+    a.tiles = (d.Cout / 128) * a.tiles_ci;
+    a.S0 = S0; a.S1 = S1; a.smax = S0 > S1 ? S0 : S1;
+    constexpr int lds = 2 * HWG_BUF;
+    static bool attr = false;
+    if (!attr) {
+        if (!hip_ok(hipFuncSetAttribute((const void *)conv_halo_wg_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, lds),
+                    "halo weight-gradient LDS size"))
+            return 2;
+        attr = true;
+    }
+    hipLaunchKernelGGL(conv_halo_wg_kernel, dim3((unsigned)(a.tiles * (S0 + S1))), dim3(HALO_NT), lds, st.stream, a);
+    if (!hip_ok(hipGetLastError(), "halo weight-gradient launch")) return 2;
+    const long long total = (long long)d.Cout * d.Cin;
+    hipLaunchKernelGGL(conv_halo_wg_reduce_kernel, dim3((unsigned)((total + 255) / 256), 9), dim3(256), 0, st.stream, ws,
+                       static_cast<half_t *>(dW), total, S0, S1, a.smax);
+    return hip_ok(hipGetLastError(), "halo weight-gradient reduce launch") ? 0 : 2;
 }
 
 }  // namespace ptl

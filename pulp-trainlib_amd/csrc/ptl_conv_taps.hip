@@ -316,6 +316,30 @@ int conv_taps_wg(const ConvTileDesc &d, const void *X, const void *dY, void *dW)
     constexpr int ES = (int)sizeof(T), VEC = 16 / ES, SK = 128 / ES;
     const bool hwc = d.in_hwc != 0;
     if (d.sh != 1 || d.sw != 1 || d.Cin % VEC) return -1;
+    if constexpr (ES == 2) {
+        // 3x3 channel-major layers: both operands channel-blocked, tiles resident in LDS for all taps
+        const int Hp = d.Hin + d.padU + d.padD, Wp = d.Win + d.padL + d.padR;
+        if (!hwc && d.x_sy == d.Win && conv_halo_wg_fits(d, Hp, Wp) &&
+            (st.gemm_path == 5 || (st.gemm_path == 0 && conv_halo_wg_preferred(d)))) {
+            const long long P = (long long)d.batch * Hp * Wp, margin = conv_halo_wg_margin();
+            const long long xb_chunks = (long long)(d.Cin / VEC) * P + margin;
+            const long long gb_chunks = (long long)(d.Cout / VEC) * conv_halo_wg_gradient_stride(d, Hp, Wp);
+            int S0 = 1, S1 = 1;
+            const size_t ws_bytes = conv_halo_wg_partial_bytes(d, Hp, Wp, &S0, &S1);
+            if (xb_chunks * 16 < ((long long)1 << 31) && gb_chunks * 16 < ((long long)1 << 31) &&
+                ws_bytes <= ((size_t)1 << 30)) {
+                char *buf = static_cast<char *>(scratch((size_t)(xb_chunks + gb_chunks) * 16 + 256));
+                if (!buf) return 2;
+                float *ws = workspace(ws_bytes);
+                if (!ws) return 2;
+                uint4 *xb = reinterpret_cast<uint4 *>(buf);
+                char *gb = buf + (((size_t)xb_chunks * 16 + 255) & ~(size_t)255);
+                if (int rc = blocked_padded_copy<T>(reinterpret_cast<const T *>(X), xb, d, Hp, Wp, margin)) return rc;
+                st.last_conv_resident = 1;
+                return conv_halo_wg_launch(d, dY, xb, gb, ws, dW, Hp, Wp, S0, S1);
+            }
+        }
+    }
     if (hwc) {  // channel-minor: both operands are [position][channel] matrices read 16 bytes along the channels
         if (d.Cout % VEC || reinterpret_cast<uintptr_t>(X) % 16 || reinterpret_cast<uintptr_t>(dY) % 16) return -1;
         // (no direct kernel for this layout: the alternative is the gathering GEMM, which this route beats from 64

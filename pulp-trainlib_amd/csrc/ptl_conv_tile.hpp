@@ -84,6 +84,16 @@ bool conv_halo_fits(const ConvTileDesc &d, int Hp, int Wp);
 long long conv_halo_margin();
 int conv_halo_launch(const ConvTileDesc &d, const void *xb, const void *wr, void *Y, int Hp, int Wp);
 
+// Weight gradient of the same layers on the same layouts (gradient embedded in the padded grid, channel-blocked):
+// partial sums per tap and position split + one reduction.  See ptl_conv_halo.hip for the buffer sizes.
+bool conv_halo_wg_fits(const ConvTileDesc &d, int Hp, int Wp);
+bool conv_halo_wg_preferred(const ConvTileDesc &d);  // fits, and measured faster than the other weight-gradient routes
+long long conv_halo_wg_margin();
+long long conv_halo_wg_gradient_stride(const ConvTileDesc &d, int Hp, int Wp);
+size_t conv_halo_wg_partial_bytes(const ConvTileDesc &d, int Hp, int Wp, int *S0, int *S1);
+int conv_halo_wg_launch(const ConvTileDesc &d, const void *dY, const void *xb, void *gb, float *ws, void *dW, int Hp,
+                        int Wp, int S0, int S1);
+
 // Weight gradient over filter taps on the same GEMM (partial sums per tap and k split + one reduction).
 template <typename T>
 int conv_taps_wg(const ConvTileDesc &d, const void *X, const void *dY, void *dW);

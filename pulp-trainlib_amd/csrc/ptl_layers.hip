@@ -361,7 +361,9 @@ static int conv2d_wg(const Args *a, int ns, const char *fn) {
         if (g.hwc) {  // channel-minor tensors: the sum over taps from 64 channels on, else the gathering GEMM below
             rc = conv_taps_wg<T>(d, X, dY, dW);
         } else {
-            if (state().gemm_path == 3 || (taps_first && state().gemm_path != 2)) rc = conv_taps_wg<T>(d, X, dY, dW);
+            const bool tiles_resident = sizeof(T) == 2 && state().gemm_path == 0 && conv_halo_wg_preferred(d);
+            if (state().gemm_path == 3 || state().gemm_path == 5 || tiles_resident || (taps_first && state().gemm_path != 2))
+                rc = conv_taps_wg<T>(d, X, dY, dW);
             if (rc < 0) rc = conv_tile_wg<T>(d, X, dY, dW);
             if (rc < 0 && state().gemm_path != 3) rc = conv_taps_wg<T>(d, X, dY, dW);
         }

@@ -262,6 +262,32 @@ def test_conv2d_resident_tile_route(pkg, orc, gpu, case):
         gpu.ptl_set_gemm_path(0)
 
 
+@pytest.mark.parametrize("case", [(64, 12, 10, 128, (0, 2, 1, 0), 2), (192, 6, 6, 256, (0, 0, 0, 0), 2),
+                                  (128, 14, 14, 128, (1, 1, 1, 1), 9)])
+def test_conv2d_resident_tile_weight_gradient(pkg, orc, gpu, case):
+    """The weight gradient on the channel-blocked layouts (path 5; filters a multiple of 128, channels of 64):
+    against the oracle; ragged last unit, one and several channel tiles."""
+    Ci, H, W, Co, pad, ns = case
+    nd = np.float16
+    Ho, Wo = hp.conv_out(H, 3, pad[2], pad[3], 1), hp.conv_out(W, 3, pad[0], pad[1], 1)
+    x, w = hp.uniform(31, (ns, Ci, H, W), dtype=nd), hp.uniform(32, (Co, Ci, 3, 3), dtype=nd)
+    dy = hp.uniform(33, (ns, Co, Ho, Wo), dtype=nd)
+    ref = np.zeros((Co, Ci, 3, 3), nd)
+    a, keep = hp.conv2d_args(pkg, x, None, w, ref, np.zeros((ns, Co, Ho, Wo), nd), dy, Ci, H, W, Co, 3, 3, Ho, Wo, pad, (1, 1))
+    orc.call("orc_conv2d_wg", "fp16", a, ns)
+    gdw = dev(np.full((Co, Ci, 3, 3), 3, nd))
+    g, keep2 = hp.conv2d_args(pkg, dev(x), None, dev(w), gdw, dev(np.zeros((ns, Co, Ho, Wo), nd)), dev(dy), Ci, H, W, Co,
+                              3, 3, Ho, Wo, pad, (1, 1))
+    gpu.ptl_set_gemm_path(5)
+    try:
+        pkg.call("ptl_conv2d_fp16_wg_batched", g, ns)
+        assert gpu.ptl_last_conv_resident() == 1
+    finally:
+        gpu.ptl_set_gemm_path(0)
+    sync(gpu)
+    assert rel_l2(host(gdw), ref) <= TOL["fp16"]
+
+
 def test_conv2d_resident_tile_many_tiles(pkg, gpu):
     """More position tiles than workgroups (every workgroup walks several tiles, the last one ragged) and two
     filter tiles: the resident-tile kernel against the tap-sum GEMM and against torch in float32."""
@@ -273,20 +299,22 @@ def test_conv2d_resident_tile_many_tiles(pkg, gpu):
     res = {}
     for path in (3, 5):
         y, dx = dev(np.zeros((ns, Co, H, W), nd)), dev(np.zeros((ns, Ci, H, W), nd))
-        a, keep = hp.conv2d_args(pkg, x, dx, w, None, y, dy, Ci, H, W, Co, 3, 3, H, W, (1, 1, 1, 1), (1, 1))
+        dw = dev(np.zeros((Co, Ci, 3, 3), nd))
+        a, keep = hp.conv2d_args(pkg, x, dx, w, dw, y, dy, Ci, H, W, Co, 3, 3, H, W, (1, 1, 1, 1), (1, 1))
         gpu.ptl_set_gemm_path(path)
         try:
-            for s in ("fw", "ig"):
+            for s in ("fw", "ig", "wg"):
                 pkg.call("ptl_conv2d_fp16_%s_batched" % s, a, ns)
-                assert gpu.ptl_last_conv_resident() == (1 if path == 5 else 0)
+                assert gpu.ptl_last_conv_resident() == (1 if path == 5 else 0), s
         finally:
             gpu.ptl_set_gemm_path(0)
         sync(gpu)
-        res[path] = [y.float(), dx.float()]
+        res[path] = [y.float(), dx.float(), dw.float()]
     ref_y = F.conv2d(x.float(), w.float(), padding=1)
     ref_dx = torch.nn.grad.conv2d_input(x.shape, w.float(), dy.float(), padding=1)
+    ref_dw = torch.nn.grad.conv2d_weight(x.float(), w.shape, dy.float(), padding=1)
     rel = lambda got, ref: float((got - ref).norm() / ref.norm())
-    for got, other, ref in zip(res[5], res[3], (ref_y, ref_dx)):
+    for got, other, ref in zip(res[5], res[3], (ref_y, ref_dx, ref_dw)):
         assert rel(got, ref) <= 1e-3
         assert rel(got, other) <= 1e-3
 
