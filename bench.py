@@ -29,6 +29,36 @@ HBM_GBS = 8000.0
 METRIC = "Conv2D/Linear FW+WG+IG TFLOP/s & % MFMA peak (fp32/fp16); samples/s"
 
 
+TRAFFIC_PROFILE = os.path.join(ROOT, "profiles", "gemm_plain_f16_linear1024_N512.md")
+TRAFFIC_SOURCES = ["ptl_gemm_plain.inc", "ptl_gemm_async.inc", "ptl_gemm_async_sel.hip", "ptl_gemm_plain_f16.hip"]
+
+
+def kernel_sources_digest():
+    """sha256 over the sources of the headline kernels and their selection."""
+    import hashlib
+    h = hashlib.sha256()
+    for name in TRAFFIC_SOURCES:
+        with open(os.path.join(ROOT, "pulp-trainlib_amd", "csrc", name), "rb") as f:
+            h.update(f.read())
+    return h.hexdigest()[:16]
+
+
+def recorded_traffic(ns):
+    """(bytes per launch, note): the HBM traffic the counter runs measured for the headline launches, as
+    recorded in the profile summary (a line `roofline.traffic: bytes_per_launch=... batch=... sources=...`)."""
+    try:
+        with open(TRAFFIC_PROFILE) as f:
+            lines = [l for l in f if l.startswith("roofline.traffic:")]
+        fields = dict(kv.split("=") for kv in lines[-1].split()[1:])
+        if int(fields["batch"]) != ns:
+            return None, "counters were collected at batch %s" % fields["batch"]
+        if fields["sources"] != kernel_sources_digest():
+            return None, "kernel sources changed since the counter runs (recorded %s)" % fields["sources"]
+        return float(fields["bytes_per_launch"]), None
+    except (OSError, IndexError, KeyError, ValueError) as e:
+        return None, "no usable traffic record (%s)" % type(e).__name__
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -132,6 +162,8 @@ def main():
     launch_ms = ev_ms / launches
     achieved = flops_step / (2 * launch_ms * 1e-3) / 1e12
 
+    traffic, traffic_note = recorded_traffic(ns)
+
     result = {
         "metric": METRIC,
         "value": round(tflops, 3),
@@ -150,14 +182,20 @@ def main():
                    "batch": ns, "accumulate": "f32", "layout": "W[out][in], X[batch][in]"},
         "roofline": {"bound": "mfma", "achieved": round(achieved, 3), "peak": PEAK["fp16"], "unit": "TFLOP/s",
                      "frac": round(achieved / PEAK["fp16"], 5),
-                     # HBM bytes per launch (mean of the two launches of a step) from the FETCH_SIZE and
-                     # WRITE_SIZE runs summarised in profiles/gemm_plain_f16_linear1024_N512.md; it holds for
-                     # the default batch only
-                     "traffic": 13.3e6 if ns == 512 else None,
+                     # HBM bytes per launch (mean of the two launches of a step), from the FETCH_SIZE and
+                     # WRITE_SIZE counter runs recorded in the profile summary of this workload; null when the
+                     # batch differs or the kernel sources have changed since those runs
+                     "traffic": traffic,
                      "kernel": "ptl::gemm_plain_kernel / gemm_plain_pair_kernel<_Float16, 64x64 tile, 1024 threads>",
                      "flops_per_launch": flops_step / 2, "launches_per_step": 2,
                      "avg_launch_us": round(launch_ms * 1e3, 3)},
     }
+
+    if traffic_note:
+        result["roofline"]["traffic_note"] = traffic_note
+    # `value` is wall-clock over the timed steps (launch overhead of the calling thread included);
+    # `roofline.achieved` prices the same steps against HIP event time on the library's stream.
+    result["roofline"]["event_ms_per_step"] = round(ev_ms / args.steps, 6)
 
     # The same step handed over as host buffers (the library stages them: allocate, copy in, run, copy out).
     # Reported beside the headline, never as the headline.
