@@ -1795,10 +1795,13 @@ __global__ __launch_bounds__(256) void cast_kernel(const S *__restrict__ a, D *_
 
 // dest[c][ht][wt] = source[c][ht-U][wt-L] inside, 0 in the border (CHW; HWC alike).  A thread writes PER
 // consecutive destination elements (one 16-byte store): first index decoded once, the rest by carrying.
+// The elements of a chunk that come from the source are consecutive in the source (the end of a row is followed
+// by the start of the next, the end of a channel by the start of the next): a chunk is one 16-byte load from the
+// first of them (at element alignment - the memory system takes unaligned vector accesses) spread over the
+// positions that are not border, also when it straddles rows.
 template <typename T, int PER>
 __global__ __launch_bounds__(256) void pad_kernel(const T *__restrict__ src, T *__restrict__ dst, int C, int H, int W,
-                                                  int L, int U, int Ho, int Wo, int hwc, size_t total, int src_aligned,
-                                                  size_t src_bytes) {
+                                                  int L, int U, int Ho, int Wo, int hwc, size_t total, size_t n_src) {
     const size_t idx0 = ((size_t)blockIdx.x * 256 + threadIdx.x) * PER;
     if (idx0 >= total) return;
     // (the host keeps the tensor below 2^32 elements: 32-bit index arithmetic)
@@ -1815,45 +1818,15 @@ __global__ __launch_bounds__(256) void pad_kernel(const T *__restrict__ src, T *
         ht = (int)(r / (unsigned)Wo);
         wt = (int)(r - (unsigned)ht * Wo);
     }
-    if (PER * sizeof(T) == 16 && src_aligned) {
-        // the whole chunk inside one contiguous run of the source (a row, or the channels of a pixel): two aligned
-        // 16-byte loads around it and a byte shift instead of PER element loads
-        const int h = ht - U, w = wt - L;
-        const bool inside = (unsigned)h < (unsigned)H && (unsigned)w < (unsigned)W && idx0 + PER <= total &&
-                            (hwc ? c + PER <= C : w + PER <= W);
-        if (inside) {
-            const size_t si = hwc ? ((size_t)h * W + w) * C + c : ((size_t)c * H + h) * W + w;
-            const size_t ba = si * sizeof(T), a0 = ba & ~(size_t)15;
-            const unsigned sh = (unsigned)(ba - a0);
-            if (sh == 0 || a0 + 32 <= src_bytes) {
-                const char *sb = reinterpret_cast<const char *>(src);
-                const uint4 lo = *reinterpret_cast<const uint4 *>(sb + a0);
-                uint4 out = lo;
-                if (sh != 0) {
-                    const uint4 hi = *reinterpret_cast<const uint4 *>(sb + a0 + 16);
-                    const unsigned d[8] = {lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
-                    const unsigned o = sh >> 2, bits = (sh & 3u) * 8u;
-                    unsigned t[5];
-#pragma unroll
-                    for (int j = 0; j < 5; ++j) t[j] = o == 0 ? d[j] : o == 1 ? d[j + 1] : o == 2 ? d[j + 2] : d[j + 3];
-                    unsigned r[4];
-#pragma unroll
-                    for (int j = 0; j < 4; ++j)
-                        r[j] = (unsigned)(((((unsigned long long)t[j + 1]) << 32) | t[j]) >> bits);
-                    out = make_uint4(r[0], r[1], r[2], r[3]);
-                }
-                *reinterpret_cast<uint4 *>(dst + idx0) = out;
-                return;
-            }
-        }
-    }
-    T v[PER];
+    unsigned mask = 0;
+    size_t base = 0;
 #pragma unroll
     for (int e = 0; e < PER; ++e) {
         const int h = ht - U, w = wt - L;
-        v[e] = (T)0;
-        if (idx0 + e < total && (unsigned)h < (unsigned)H && (unsigned)w < (unsigned)W)
-            v[e] = hwc ? src[((size_t)h * W + w) * C + c] : src[((size_t)c * H + h) * W + w];
+        if (idx0 + e < total && (unsigned)h < (unsigned)H && (unsigned)w < (unsigned)W) {
+            if (mask == 0) base = hwc ? ((size_t)h * W + w) * C + c : ((size_t)c * H + h) * W + w;
+            mask |= 1u << e;
+        }
         if (!hwc) {
             if (++wt == Wo) {
                 wt = 0;
@@ -1872,18 +1845,40 @@ __global__ __launch_bounds__(256) void pad_kernel(const T *__restrict__ src, T *
             }
         }
     }
-    if (PER * sizeof(T) == 16 && idx0 + PER <= total) {
-        union {
-            uint4 u;
-            T e[PER];
-        } pack;
+    union {
+        uint4 u;
+        T e[PER];
+    } in, out;
+    if (PER * sizeof(T) == 16 && mask != 0 && base + PER <= n_src) {
+        typedef unsigned pad_u4 __attribute__((ext_vector_type(4), aligned(2)));
+        const pad_u4 v = *reinterpret_cast<const pad_u4 *>(src + base);
+        in.u = make_uint4(v.x, v.y, v.z, v.w);
+    } else {
 #pragma unroll
-        for (int e = 0; e < PER; ++e) pack.e[e] = v[e];
-        *reinterpret_cast<uint4 *>(dst + idx0) = pack.u;
+        for (int e = 0; e < PER; ++e) in.e[e] = (mask >> e) != 0 && base + e < n_src ? src[base + e] : (T)0;
+    }
+    if (mask == (1u << PER) - 1u) {
+        out = in;
+    } else {
+        int r = 0;
+#pragma unroll
+        for (int e = 0; e < PER; ++e) {
+            T v = (T)0;
+            if (mask & (1u << e)) {
+#pragma unroll
+                for (int q = 0; q <= e; ++q)
+                    if (q == r) v = in.e[q];
+                ++r;
+            }
+            out.e[e] = v;
+        }
+    }
+    if (PER * sizeof(T) == 16 && idx0 + PER <= total) {
+        *reinterpret_cast<uint4 *>(dst + idx0) = out.u;
     } else {
 #pragma unroll
         for (int e = 0; e < PER; ++e)
-            if (idx0 + e < total) dst[idx0 + e] = v[e];
+            if (idx0 + e < total) dst[idx0 + e] = out.e[e];
     }
 }
 
@@ -1914,13 +1909,13 @@ static int pad_step(const Args *a, const char *fn) {
     T *d = sg.out(reinterpret_cast<T *>(a->dest), total);
     if (sg.failed()) return 2;
     constexpr int VEC = 16 / (int)sizeof(T);
+    const size_t n_src = (size_t)a->C * a->H * a->W;
     if (reinterpret_cast<uintptr_t>(d) % 16 == 0)
         hipLaunchKernelGGL((pad_kernel<T, VEC>), dim3(nblocks((total + VEC - 1) / VEC)), dim3(256), 0, state().stream, s, d,
-                           a->C, a->H, a->W, a->T_LPAD, a->T_UPAD, Ho, Wo, a->HWC_lay, total,
-                           reinterpret_cast<uintptr_t>(s) % 16 == 0 ? 1 : 0, (size_t)a->C * a->H * a->W * sizeof(T));
+                           a->C, a->H, a->W, a->T_LPAD, a->T_UPAD, Ho, Wo, a->HWC_lay, total, n_src);
     else
         hipLaunchKernelGGL((pad_kernel<T, 1>), dim3(nblocks(total)), dim3(256), 0, state().stream, s, d, a->C, a->H, a->W,
-                           a->T_LPAD, a->T_UPAD, Ho, Wo, a->HWC_lay, total, 0, (size_t)0);
+                           a->T_LPAD, a->T_UPAD, Ho, Wo, a->HWC_lay, total, n_src);
     return sg.finish(hip_ok(hipGetLastError(), "pad launch") ? 0 : 2);
 }
 
