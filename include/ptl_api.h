@@ -302,6 +302,13 @@ int ptl_conv_dw_fp16_ig_batched(const struct DepthWise_Conv_args_fp16 *a, int ns
  * hipMalloc / hipFree. */
 int ptl_conv_dw_fp16_wg_noalloc(const struct DepthWise_Conv_args_fp16 *a, int nsamples);
 
+/* Weight and input gradient of a Conv2D batch in ONE call, as pulp_conv2d_fp32_bw_cl / pulp_conv2d_fp16_bw_cl do
+ * for one sample (lib/sources/pulp_conv2d_fp32.c:225-237, lib/sources/pulp_conv2d_fp16.c:225); honours skip_wg_grad /
+ * skip_in_grad.  fp16 channel-major 3x3 "same" layers that run the resident-tile kernels share one channel-blocked
+ * copy of the output gradient between the two steps. */
+int ptl_conv2d_fp32_bw_batched(const struct Conv2D_args *a, int nsamples);
+int ptl_conv2d_fp16_bw_batched(const struct Conv2D_args_fp16 *a, int nsamples);
+
 int ptl_linear_fp32_fw_batched(const struct Linear_args *a, int nsamples);
 int ptl_linear_fp32_wg_batched(const struct Linear_args *a, int nsamples);
 int ptl_linear_fp32_ig_batched(const struct Linear_args *a, int nsamples);

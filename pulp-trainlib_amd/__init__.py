@@ -70,6 +70,7 @@ BATCHED_ENTRY_POINTS = ["ptl_%s_%s_%s_batched" % (layer, dt, step)
                         for layer in ("conv2d", "conv_pw", "conv_dw", "linear")
                         for dt in ("fp32", "fp16") for step in ("fw", "wg", "ig")] + [
                             "ptl_linear_fp32_bw_batched", "ptl_linear_fp16_bw_batched",
+                            "ptl_conv2d_fp32_bw_batched", "ptl_conv2d_fp16_bw_batched",
                             "ptl_mhsa_fp32_fw_batched", "ptl_mhsa_fp32_bw_batched",
                             "ptl_conv_dw_fp16_wg_noalloc",
                             # (const optim_args *list, int count)

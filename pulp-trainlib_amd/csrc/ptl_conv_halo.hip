@@ -453,11 +453,11 @@ __global__ __launch_bounds__(256) void conv_halo_wg_reduce_kernel(const float *_
     dW[idx * 9 + tap] = (half_t)s;
 }
 
-// gb[cb][p] for p < pstride: the gradient dY[b][8 cb .. + 7][y][x] at p = (b, y, x) of the padded grid (y < Ho,
-// x < Wo), zero elsewhere and from the last padded position on.
+// gb[cb][p] for p < pstride: the tensor element t[b][8 cb .. + 7][yp - pu][xp - pl] at p = (b, yp, xp) of the padded
+// grid, zero outside the tensor and from the last padded position on.
 __global__ __launch_bounds__(256) void conv_halo_embed_kernel(const half_t *__restrict__ dy, uint4 *__restrict__ out,
-                                                              int B, int Ho, int Wo, int Hp, int Wp, long long sb,
-                                                              long long sc, unsigned P, unsigned pstride,
+                                                              int B, int Ho, int Wo, int Hp, int Wp, int pu, int pl,
+                                                              long long sb, long long sc, unsigned P, unsigned pstride,
                                                               unsigned total) {
     const unsigned i = blockIdx.x * 256u + threadIdx.x;
     if (i >= total) return;
@@ -469,9 +469,9 @@ __global__ __launch_bounds__(256) void conv_halo_embed_kernel(const half_t *__re
     u.v = make_uint4(0, 0, 0, 0);
     if (p < P) {
         const unsigned r = p / (unsigned)Wp, xp = p - r * (unsigned)Wp;
-        const unsigned b = r / (unsigned)Hp, yp = r - b * (unsigned)Hp;
-        if (yp < (unsigned)Ho && xp < (unsigned)Wo) {
-            const half_t *src = dy + b * sb + (long long)(cb * 8) * sc + (long long)yp * Wo + xp;
+        const unsigned b = r / (unsigned)Hp, yy = r - b * (unsigned)Hp - (unsigned)pu, xx = xp - (unsigned)pl;
+        if (yy < (unsigned)Ho && xx < (unsigned)Wo) {
+            const half_t *src = dy + b * sb + (long long)(cb * 8) * sc + (long long)yy * Wo + xx;
 #pragma unroll
             for (int e = 0; e < 8; ++e) u.e[e] = src[e * sc];
         }
@@ -489,13 +489,13 @@ bool conv_halo_fits(const ConvTileDesc &d, int Hp, int Wp) {
 }
 
 // xb: blocked, padded input with conv_halo_margin() readable chunks after the last block; wr: tap-major filters.
-int conv_halo_launch(const ConvTileDesc &d, const void *xb, const void *wr, void *Y, int Hp, int Wp) {
+int conv_halo_launch(const ConvTileDesc &d, const void *xb, const void *wr, void *Y, int Hp, int Wp, long long pstride) {
     State &st = state();
     HaloArgs a = {};
     a.xb = static_cast<const char *>(xb);
     a.wr = static_cast<const char *>(wr);
     a.y = static_cast<half_t *>(Y);
-    a.P = (long long)d.batch * Hp * Wp;
+    a.P = pstride > 0 ? pstride : (long long)d.batch * Hp * Wp;
     // leave the bottom rows of every padded grid out when a tile that crosses sample boundaries still fits
     const int qs = d.Ho * Wp, crossings = (HALO_BM - 1 + qs - 1) / qs;
     const bool skip = Hp > d.Ho && HALO_BM + (crossings + 1) * (Hp - d.Ho) * Wp + 2 <= HALO_NP;
@@ -551,25 +551,32 @@ size_t conv_halo_wg_partial_bytes(const ConvTileDesc &d, int Hp, int Wp, int *S0
     return (size_t)9 * smax * d.Cout * d.Cin * sizeof(float);
 }
 
-// gb: room for (Cout / 8) * conv_halo_wg_gradient_stride() chunks; xb as for the forward kernel with
-// conv_halo_wg_margin() readable chunks behind it; ws: conv_halo_wg_partial_bytes().
-int conv_halo_wg_launch(const ConvTileDesc &d, const void *dY, const void *xb, void *gb, float *ws, void *dW, int Hp,
-                        int Wp, int S0, int S1) {
+// A channel-major tensor t[batch][C][Hs][Ws] as padded, channel-blocked chunks out[C / 8][pstride] (see
+// conv_halo_embed_kernel): the tensor sits pu rows / pl columns inside each Hp x Wp grid.
+int conv_halo_embed(const void *t, void *out, int batch, int C, int Hs, int Ws, int Hp, int Wp, int pu, int pl,
+                    long long pstride) {
+    State &st = state();
+    const long long P = (long long)batch * Hp * Wp, chunks = (long long)(C / 8) * pstride;
+    if (chunks >= ((long long)1 << 31) || pstride < P) return -1;
+    hipLaunchKernelGGL(conv_halo_embed_kernel, dim3((unsigned)((chunks + 255) / 256)), dim3(256), 0, st.stream,
+                       static_cast<const half_t *>(t), static_cast<uint4 *>(out), batch, Hs, Ws, Hp, Wp, pu, pl,
+                       (long long)C * Hs * Ws, (long long)Hs * Ws, (unsigned)P, (unsigned)pstride, (unsigned)chunks);
+    return hip_ok(hipGetLastError(), "blocked layout launch") ? 0 : 2;
+}
+
+// gb: the blocked, embedded gradient (top left of the grids at gb[cb * gstride + 0]; zero from the last padded
+// position to conv_halo_wg_gradient_stride() positions); xb as for the forward kernel with conv_halo_wg_margin()
+// readable chunks behind it; ws: conv_halo_wg_partial_bytes().
+int conv_halo_wg_launch(const ConvTileDesc &d, const void *xb, const void *gb, long long gstride, float *ws, void *dW,
+                        int Hp, int Wp, int S0, int S1) {
     State &st = state();
     const long long P = (long long)d.batch * Hp * Wp, Pd = conv_halo_wg_gradient_stride(d, Hp, Wp);
-    const long long chunks = (long long)(d.Cout / 8) * Pd;
-    if (chunks >= ((long long)1 << 31)) return -1;
-    hipLaunchKernelGGL(conv_halo_embed_kernel, dim3((unsigned)((chunks + 255) / 256)), dim3(256), 0, st.stream,
-                       static_cast<const half_t *>(dY), static_cast<uint4 *>(gb), d.batch, d.Ho, d.Wo, Hp, Wp,
-                       (long long)d.Cout * d.Ho * d.Wo, (long long)d.Ho * d.Wo, (unsigned)P, (unsigned)Pd,
-                       (unsigned)chunks);
-    if (!hip_ok(hipGetLastError(), "gradient layout launch")) return 2;
     HaloWgArgs a = {};
     a.xb = static_cast<const char *>(xb);
     a.gb = static_cast<const char *>(gb);
     a.ws = ws;
     a.Px = P;
-    a.Pd = Pd;
+    a.Pd = gstride;
     a.Cin = d.Cin; a.Cout = d.Cout; a.Wp = Wp;
     a.units = (int)(Pd / HWG_UNIT);
     a.tiles_ci = d.Cin / 64;

@@ -128,6 +128,11 @@ __global__ __launch_bounds__(256) void tap_prepare_kernel(const TapPrepArgs a) {
                              a.C, a.KW, a.taps, a.w_base, a.w_sm, a.w_sc, a.w_sy, a.w_sx, a.wr_total);
 }
 
+__global__ __launch_bounds__(256) void zero_chunks_kernel(uint4 *__restrict__ p, unsigned n) {
+    const unsigned i = blockIdx.x * 256u + threadIdx.x;
+    if (i < n) p[i] = make_uint4(0, 0, 0, 0);
+}
+
 template <typename T>
 int conv_taps(const ConvTileDesc &d, const void *X, const void *Wt, void *Y, const OutMap &c) {
     State &st = state();
@@ -335,8 +340,10 @@ int conv_taps_wg(const ConvTileDesc &d, const void *X, const void *dY, void *dW)
                 uint4 *xb = reinterpret_cast<uint4 *>(buf);
                 char *gb = buf + (((size_t)xb_chunks * 16 + 255) & ~(size_t)255);
                 if (int rc = blocked_padded_copy<T>(reinterpret_cast<const T *>(X), xb, d, Hp, Wp, margin)) return rc;
+                const long long gstride = conv_halo_wg_gradient_stride(d, Hp, Wp);
+                if (int rc = conv_halo_embed(dY, gb, d.batch, d.Cout, d.Ho, d.Wo, Hp, Wp, 0, 0, gstride)) return rc;
                 st.last_conv_resident = 1;
-                return conv_halo_wg_launch(d, dY, xb, gb, ws, dW, Hp, Wp, S0, S1);
+                return conv_halo_wg_launch(d, xb, gb, gstride, ws, dW, Hp, Wp, S0, S1);
             }
         }
     }
@@ -463,6 +470,70 @@ int conv_taps_wg(const ConvTileDesc &d, const void *X, const void *dY, void *dW)
                        ws, reinterpret_cast<T *>(dW), total, (int)S, taps, d.Cin, hwc ? 1 : 0);
     return hip_ok(hipGetLastError(), "tap reduce launch") ? 0 : 2;
 }
+
+// Backward pass of a 3x3 "same" layer (pads of both sides add up to 2, unit stride, fp16, channel-major): the weight
+// gradient and the input gradient read the SAME channel-blocked copy of the output gradient - the input gradient
+// as its padded input (the gradient sits KH-1-padU rows / KW-1-padL columns inside each grid), the weight gradient
+// that many positions further on as the gradient embedded at the top left of the grid.  One layout pass less than
+// the two calls on their own.
+template <typename T>
+int conv_halo_bw(const ConvTileDesc &fwd, const ConvTileDesc &ig, const void *X, const void *dY, const void *Wt,
+                 void *dW, void *dX) {
+    if constexpr (sizeof(T) != 2) {
+        return -1;
+    } else {
+        State &st = state();
+        constexpr int VEC = 8;
+        const int Hp = fwd.Hin + fwd.padU + fwd.padD, Wp = fwd.Win + fwd.padL + fwd.padR;
+        const int Hpi = ig.Hin + ig.padU + ig.padD, Wpi = ig.Win + ig.padL + ig.padR;
+        if (Hp != Hpi || Wp != Wpi || fwd.x_sy != fwd.Win || ig.x_sy != ig.Win) return -1;
+        if (!conv_halo_fits(ig, Hp, Wp) || !conv_halo_wg_fits(fwd, Hp, Wp) || !conv_halo_wg_preferred(fwd)) return -1;
+        if (!(st.gemm_path == 0 || st.gemm_path == 5)) return -1;
+        const long long P = (long long)fwd.batch * Hp * Wp;
+        const int goff = ig.padU * Wp + ig.padL;  // where the weight gradient's view of the copy starts
+        const long long gstride = conv_halo_wg_gradient_stride(fwd, Hp, Wp) + 128;
+        if (goff > 128) return -1;
+        const long long xmargin = conv_halo_wg_margin(), gmargin = conv_halo_margin() + 128;
+        const long long xb_chunks = (long long)(fwd.Cin / VEC) * P + xmargin;
+        const long long gb_chunks = (long long)(fwd.Cout / VEC) * gstride + gmargin;
+        const long long wr_elems = (long long)ig.Cout * 9 * ig.Cin;
+        int S0 = 1, S1 = 1;
+        const size_t ws_bytes = conv_halo_wg_partial_bytes(fwd, Hp, Wp, &S0, &S1);
+        if (xb_chunks * 16 >= ((long long)1 << 31) || gb_chunks * 16 >= ((long long)1 << 31) ||
+            ws_bytes > ((size_t)1 << 30))
+            return -1;
+        char *buf = static_cast<char *>(scratch((size_t)(xb_chunks + gb_chunks) * 16 + (size_t)wr_elems * 2 + 768));
+        if (!buf) return 2;
+        float *ws = workspace(ws_bytes);
+        if (!ws) return 2;
+        uint4 *xb = reinterpret_cast<uint4 *>(buf);
+        char *gb = buf + (((size_t)xb_chunks * 16 + 255) & ~(size_t)255);
+        T *wr = reinterpret_cast<T *>(gb + (((size_t)gb_chunks * 16 + 255) & ~(size_t)255));
+        // the shared copy of the output gradient (margin included: the input-gradient kernel reads past the end)
+        if (int rc = conv_halo_embed(dY, gb, ig.batch, ig.Cin, ig.Hin, ig.Win, Hp, Wp, ig.padU, ig.padL, gstride)) return rc;
+        {  // the last block's margin, and the flipped, transposed filters of the input gradient
+            hipLaunchKernelGGL(zero_chunks_kernel, dim3((unsigned)((gmargin + 255) / 256)), dim3(256), 0, st.stream,
+                               reinterpret_cast<uint4 *>(gb) + (long long)(fwd.Cout / VEC) * gstride, (unsigned)gmargin);
+            TapPrepArgs p = {};
+            p.copy_blocks = 0;
+            p.w = Wt;
+            p.wr = wr;
+            p.C = ig.Cin; p.KW = 3; p.taps = 9;
+            p.w_base = ig.w_base; p.w_sm = ig.w_sm; p.w_sc = ig.w_sc; p.w_sy = ig.w_sy; p.w_sx = ig.w_sx;
+            p.wr_total = wr_elems;
+            hipLaunchKernelGGL((tap_prepare_kernel<T>), dim3((unsigned)((wr_elems + 255) / 256)), dim3(256), 0, st.stream, p);
+            if (!hip_ok(hipGetLastError(), "layout launch")) return 2;
+        }
+        if (int rc = blocked_padded_copy<T>(reinterpret_cast<const T *>(X), xb, fwd, Hp, Wp, xmargin)) return rc;
+        st.last_conv_resident = 1;
+        if (int rc = conv_halo_wg_launch(fwd, xb, gb + (size_t)goff * 16, gstride, ws, dW, Hp, Wp, S0, S1)) return rc;
+        return conv_halo_launch(ig, gb, wr, dX, Hp, Wp, gstride);
+    }
+}
+template int conv_halo_bw<float>(const ConvTileDesc &, const ConvTileDesc &, const void *, const void *, const void *,
+                                 void *, void *);
+template int conv_halo_bw<half_t>(const ConvTileDesc &, const ConvTileDesc &, const void *, const void *, const void *,
+                                  void *, void *);
 
 template int conv_taps_wg<float>(const ConvTileDesc &, const void *, const void *, void *);
 template int conv_taps_wg<half_t>(const ConvTileDesc &, const void *, const void *, void *);

@@ -82,7 +82,10 @@ int conv_taps(const ConvTileDesc &d, const void *X, const void *Wt, void *Y, con
 // filters).  Y is the dense channel-major output [batch][Cout][Ho][Wo].
 bool conv_halo_fits(const ConvTileDesc &d, int Hp, int Wp);
 long long conv_halo_margin();
-int conv_halo_launch(const ConvTileDesc &d, const void *xb, const void *wr, void *Y, int Hp, int Wp);
+int conv_halo_launch(const ConvTileDesc &d, const void *xb, const void *wr, void *Y, int Hp, int Wp,
+                     long long pstride = 0);  // pstride: positions between channel blocks of xb (0: batch*Hp*Wp)
+int conv_halo_embed(const void *t, void *out, int batch, int C, int Hs, int Ws, int Hp, int Wp, int pu, int pl,
+                    long long pstride);
 
 // Weight gradient of the same layers on the same layouts (gradient embedded in the padded grid, channel-blocked):
 // partial sums per tap and position split + one reduction.  See ptl_conv_halo.hip for the buffer sizes.
@@ -91,8 +94,14 @@ bool conv_halo_wg_preferred(const ConvTileDesc &d);  // fits, and measured faste
 long long conv_halo_wg_margin();
 long long conv_halo_wg_gradient_stride(const ConvTileDesc &d, int Hp, int Wp);
 size_t conv_halo_wg_partial_bytes(const ConvTileDesc &d, int Hp, int Wp, int *S0, int *S1);
-int conv_halo_wg_launch(const ConvTileDesc &d, const void *dY, const void *xb, void *gb, float *ws, void *dW, int Hp,
-                        int Wp, int S0, int S1);
+int conv_halo_wg_launch(const ConvTileDesc &d, const void *xb, const void *gb, long long gstride, float *ws, void *dW,
+                        int Hp, int Wp, int S0, int S1);
+
+// Weight gradient and input gradient of one 3x3 "same" layer sharing one blocked copy of the output gradient;
+// -1 when the layer does not fit both resident-tile kernels.
+template <typename T>
+int conv_halo_bw(const ConvTileDesc &fwd, const ConvTileDesc &ig, const void *X, const void *dY, const void *Wt,
+                 void *dW, void *dX);
 
 // Weight gradient over filter taps on the same GEMM (partial sums per tap and k split + one reduction).
 template <typename T>

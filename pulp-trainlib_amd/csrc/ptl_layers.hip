@@ -607,6 +607,60 @@ static int pw_geom(const Args *a, const char *fn) {
     return 0;
 }
 
+// Weight and input gradient of one call (the batched twin of pulp_conv2d_*_bw_cl): honours skip_wg_grad /
+// skip_in_grad; where both run on the resident-tile kernels they share the blocked copy of the output gradient.
+template <typename T, typename Args>
+static int conv2d_bw(const Args *a, int ns, const char *fn) {
+    if (!a) {
+        set_error("%s: null argument structure", fn);
+        return 1;
+    }
+    const bool wg = a->skip_wg_grad == 0, ig = a->skip_in_grad == 0;
+    if (wg && ig && sizeof(T) == 2 && a->USE_BIASES != 1 && ns > 1 && a->input && a->coeff && a->output) {
+        ConvGeom g;
+        if (int rc = conv_geom(a, g, fn, true)) return rc;
+        const int P = g.Ho * g.Wo, Pk = g.Hk * g.Wk, K = g.Ci * Pk;
+        size_t in_n = (size_t)ns * g.Ci * g.H * g.W, out_n = (size_t)ns * g.Co * P;
+        if (!g.hwc && g.Hk == 3 && g.Wk == 3 && g.sh == 1 && g.sw == 1 && g.Up + g.Dp == 2 && g.Lp + g.Rp == 2 &&
+            fits_int(in_n) && fits_int(out_n) && (state().gemm_path == 0 || state().gemm_path == 5)) {
+            if (!ensure_init()) return 2;
+            ConvTileDesc f = {}, b = {};
+            f.batch = ns; f.Cin = g.Ci; f.Hin = g.H; f.Win = g.W;
+            f.Cout = g.Co; f.Ho = g.Ho; f.Wo = g.Wo;
+            f.KH = 3; f.KW = 3; f.sh = 1; f.sw = 1;
+            f.padU = g.Up; f.padD = g.Dp; f.padL = g.Lp; f.padR = g.Rp;
+            f.x_sb = (long long)g.Ci * g.H * g.W; f.x_sc = (long long)g.H * g.W; f.x_sy = g.W;
+            b.batch = ns; b.Cin = g.Co; b.Hin = g.Ho; b.Win = g.Wo;
+            b.Cout = g.Ci; b.Ho = g.H; b.Wo = g.W;
+            b.KH = 3; b.KW = 3; b.sh = 1; b.sw = 1;
+            b.padU = 2 - g.Up; b.padL = 2 - g.Lp;
+            b.padD = g.H + 2 - g.Ho - b.padU; b.padR = g.W + 2 - g.Wo - b.padL;
+            b.x_sb = (long long)g.Co * P; b.x_sc = P; b.x_sy = g.Wo;
+            b.w_base = Pk - 1; b.w_sm = Pk; b.w_sc = g.Ci * Pk; b.w_sy = -g.Wk; b.w_sx = -1;
+            if (conv_halo_wg_preferred(f)) {
+                Stager sg;
+                const T *X = sg.in(reinterpret_cast<const T *>(a->input->data), in_n);
+                const T *dY = sg.in(reinterpret_cast<const T *>(a->output->diff), out_n);
+                const T *Wt = sg.in(reinterpret_cast<const T *>(a->coeff->data), (size_t)g.Co * K);
+                T *dW = sg.out(reinterpret_cast<T *>(a->coeff->diff), (size_t)g.Co * K);
+                T *dX = sg.out(reinterpret_cast<T *>(a->input->diff), in_n);
+                if (sg.failed()) return 2;
+                state().last_conv_direct = 0;
+                state().last_conv_resident = 0;
+                const int rc = conv_halo_bw<T>(f, b, X, dY, Wt, dW, dX);
+                if (rc >= 0) {
+                    if (rc == 0) state().last_conv_direct = 1;
+                    return sg.finish(rc);
+                }
+                sg.finish(0);
+            }
+        }
+    }
+    int rc = wg ? conv2d_wg<T>(a, ns, fn) : 0;
+    if (rc == 0 && ig) rc = conv2d_ig<T>(a, ns, fn);
+    return rc;
+}
+
 template <typename T, typename Args>
 static int pw_step(const Args *a, int ns, int step, const char *fn) {
     if (int rc = pw_geom(a, fn)) return rc;
@@ -920,6 +974,12 @@ int ptl_conv2d_fp16_wg_batched(const struct Conv2D_args_fp16 *a, int ns) {
 }
 int ptl_conv2d_fp16_ig_batched(const struct Conv2D_args_fp16 *a, int ns) {
     return ptl::conv2d_ig<half_t>(a, ns, "pulp_conv2d_fp16_bw_input_grads_cl");
+}
+int ptl_conv2d_fp32_bw_batched(const struct Conv2D_args *a, int ns) {
+    return ptl::conv2d_bw<float>(a, ns, "pulp_conv2d_fp32_bw_cl");
+}
+int ptl_conv2d_fp16_bw_batched(const struct Conv2D_args_fp16 *a, int ns) {
+    return ptl::conv2d_bw<half_t>(a, ns, "pulp_conv2d_fp16_bw_cl");
 }
 
 int ptl_conv_pw_fp32_fw_batched(const struct PointWise_Conv_args *a, int ns) {

@@ -288,6 +288,45 @@ def test_conv2d_resident_tile_weight_gradient(pkg, orc, gpu, case):
     assert rel_l2(host(gdw), ref) <= TOL["fp16"]
 
 
+@pytest.mark.parametrize("case", [(128, 14, 14, 128, (1, 1, 1, 1), 9, 1), (64, 12, 10, 128, (0, 2, 1, 1), 7, 1),
+                                  (64, 12, 10, 128, (1, 1, 1, 1), 7, 1), (16, 9, 9, 8, (1, 1, 1, 1), 3, 0),
+                                  (64, 12, 10, 128, (0, 0, 0, 0), 7, 0)])
+@pytest.mark.parametrize("skip", [(0, 0), (1, 0), (0, 1)])
+def test_conv2d_backward_in_one_call(pkg, orc, gpu, case, skip):
+    """ptl_conv2d_fp16_bw_batched against the oracle's two steps: layers that share the blocked copy of the output
+    gradient between the resident-tile kernels (symmetric and asymmetric "same" padding), layers that fall back to
+    the two single steps, and the skip flags (a skipped gradient must stay untouched)."""
+    Ci, H, W, Co, pad, ns, shared = case
+    nd = np.float16
+    Ho, Wo = hp.conv_out(H, 3, pad[2], pad[3], 1), hp.conv_out(W, 3, pad[0], pad[1], 1)
+    x, w = hp.uniform(41, (ns, Ci, H, W), dtype=nd), hp.uniform(42, (Co, Ci, 3, 3), dtype=nd)
+    dy = hp.uniform(43, (ns, Co, Ho, Wo), dtype=nd)
+    rdw, rdx = np.zeros((Co, Ci, 3, 3), nd), np.zeros((ns, Ci, H, W), nd)
+    a, keep = hp.conv2d_args(pkg, x, rdx, w, rdw, np.zeros((ns, Co, Ho, Wo), nd), dy, Ci, H, W, Co, 3, 3, Ho, Wo, pad, (1, 1))
+    orc.call("orc_conv2d_wg", "fp16", a, ns)
+    orc.call("orc_conv2d_ig", "fp16", a, ns)
+    gdw, gdx = dev(np.full((Co, Ci, 3, 3), 3, nd)), dev(np.full((ns, Ci, H, W), 3, nd))
+    g, keep2 = hp.conv2d_args(pkg, dev(x), gdx, dev(w), gdw, dev(np.zeros((ns, Co, Ho, Wo), nd)), dev(dy), Ci, H, W, Co,
+                              3, 3, Ho, Wo, pad, (1, 1))
+    g.skip_wg_grad, g.skip_in_grad = skip
+    gpu.ptl_set_gemm_path(5 if shared else 0)
+    try:
+        pkg.call("ptl_conv2d_fp16_bw_batched", g, ns)
+        if skip == (0, 0):
+            assert gpu.ptl_last_conv_resident() == shared
+    finally:
+        gpu.ptl_set_gemm_path(0)
+    sync(gpu)
+    if skip[0]:
+        assert np.all(host(gdw) == 3)
+    else:
+        assert rel_l2(host(gdw), rdw) <= TOL["fp16"]
+    if skip[1]:
+        assert np.all(host(gdx) == 3)
+    else:
+        assert rel_l2(host(gdx), rdx) <= TOL["fp16"]
+
+
 def test_conv2d_resident_tile_many_tiles(pkg, gpu):
     """More position tiles than workgroups (every workgroup walks several tiles, the last one ragged) and two
     filter tiles: the resident-tile kernel against the tap-sum GEMM and against torch in float32."""
