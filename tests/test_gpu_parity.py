@@ -248,6 +248,9 @@ RESIDENT_CASES = [
     (64, 7, 61, 64, (1, 1, 1, 1), 1, 1),
     (64, 5, 62, 64, (1, 1, 1, 1), 1, 0),
     (192, 6, 6, 256, (0, 0, 0, 0), 2, 1),
+    (64, 3, 3, 64, (0, 0, 0, 0), 1, 1),     # one output pixel per sample, a single ragged tile
+    (64, 3, 5, 128, (1, 1, 1, 1), 1, 1),
+    (64, 16, 16, 64, (1, 1, 1, 1), 17, 1),  # tiles that straddle two sample boundaries with the bottom rows left out
 ]
 
 
@@ -263,7 +266,8 @@ def test_conv2d_resident_tile_route(pkg, orc, gpu, case):
 
 
 @pytest.mark.parametrize("case", [(64, 12, 10, 128, (0, 2, 1, 0), 2), (192, 6, 6, 256, (0, 0, 0, 0), 2),
-                                  (128, 14, 14, 128, (1, 1, 1, 1), 9)])
+                                  (128, 14, 14, 128, (1, 1, 1, 1), 9), (64, 3, 3, 128, (0, 0, 0, 0), 1),
+                                  (64, 5, 61, 128, (1, 1, 1, 1), 3)])
 def test_conv2d_resident_tile_weight_gradient(pkg, orc, gpu, case):
     """The weight gradient on the channel-blocked layouts (path 5; filters a multiple of 128, channels of 64):
     against the oracle; ragged last unit, one and several channel tiles."""
