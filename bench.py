@@ -460,6 +460,10 @@ def detail_table(pkg, lib, hp, to_dev, timed, check, torch, dev):
         flops = 2.0 * ns * Co * Ci * K * K * H * H
         nb = (x.numel() + w.numel() + y.numel()) * es[dt]
         run3("ptl_conv2d", dt, a, ns, "conv2d %d->%d %dx%d k3 p1" % (Ci, Co, H, H), flops, (nb, nb, nb), 10)
+        # weight + input gradient in one call (the two kernels share the blocked copy of the output gradient)
+        ref = ctypes.byref(a)
+        ms = timed(lambda: check(lib.ptl_conv2d_fp16_bw_batched(ref, ns)), 10)
+        add("conv2d %d->%d %dx%d k3 p1 WG+IG in one call N=%d" % (Ci, Co, H, H, ns), dt, ms, 2 * flops, 2 * nb)
         del x, w, dy, y, dx, dw
 
     # the same wide layers with channel-minor (HWC) tensors: X[b][h][w][ci], W[co][kh][kw][ci], Y[b][h][w][co]

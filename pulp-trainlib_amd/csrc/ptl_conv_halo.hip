@@ -43,15 +43,7 @@ struct HaloArgs {
     unsigned jump;      // positions skipped per sample boundary: 0 or (Hp - Ho)*Wp
     int Cin, Cout, Hp, Wp, Ho, Wo;
     int tiles, ct_count;  // tile = position tile * ct_count + filter tile
-#ifdef PTL_HALO_ABL
-    int abl;
-#endif
 };
-#ifdef PTL_HALO_ABL
-#define HALO_ABL(bit) (a.abl & (bit))
-#else
-#define HALO_ABL(bit) false
-#endif
 
 template <int I, int N, typename F>
 __device__ inline void static_for(F &&f) {
@@ -128,7 +120,6 @@ __global__ __launch_bounds__(HALO_NT) void conv_halo_pipe_kernel(const HaloArgs 
     auto issue_filters = [&](int tile, int cs, int tap, int slot) {
         const int ct = tile % a.ct_count;
         const char *base = a.wr + ((long long)ct * BN * K9 + (long long)tap * a.Cin + cs * 64) * 2;
-        if (HALO_ABL(2)) return;
 #pragma unroll
         for (int i = 0; i < LB; ++i)
             lds_dma16_saddr(voff_b[i], base, ring_lds + (unsigned)(slot * STAGE + (wave + 4 * i) * 1024));
@@ -138,7 +129,6 @@ __global__ __launch_bounds__(HALO_NT) void conv_halo_pipe_kernel(const HaloArgs 
         const long long p0 = (long long)q0 + (long long)(q0 / a.qimg) * a.jump;
         const int c0 = (q * 4 + wave) * 64, j = c0 / HALO_NP, i0 = c0 - j * HALO_NP;
         const char *base = a.xb + (((long long)(cs * 8 + j)) * a.P + p0 + i0) * 16;
-        if (HALO_ABL(1)) return;
         lds_dma16_saddr(voff_h, base, halo_lds + (unsigned)(hb * HALO_BYTES + c0 * 16));
     };
     auto next_unit = [&](int tile, int cs, int &ntile, int &ncs) {
@@ -239,7 +229,7 @@ __global__ __launch_bounds__(HALO_NT) void conv_halo_pipe_kernel(const HaloArgs 
             if (half == 1) slot = wrap(slot + 1);
         });
         const bool tile_done = cs + 1 == UC;
-        if (tile_done && !HALO_ABL(4)) {
+        if (tile_done) {
             const unsigned q0 = (unsigned)(tile / a.ct_count) * HALO_BM;
             const int co0 = (tile % a.ct_count) * BN;
             const unsigned PO = (unsigned)(a.Ho * a.Wo);
@@ -508,9 +498,6 @@ int conv_halo_launch(const ConvTileDesc &d, const void *xb, const void *wr, void
     const long long ptiles = ((long long)a.Q + HALO_BM - 1) / HALO_BM;
     if (ptiles * a.ct_count >= (1ll << 30)) return -1;
     a.tiles = (int)(ptiles * a.ct_count);
-#ifdef PTL_HALO_ABL
-    a.abl = getenv("PTL_HALO_ABL") ? atoi(getenv("PTL_HALO_ABL")) : 0;
-#endif
     const int grid = a.tiles < st.num_cu ? a.tiles : st.num_cu;
     return bn == 128 ? launch_halo_pipe<128, 4>(a, grid, st.stream) : launch_halo_pipe<64, 6>(a, grid, st.stream);
 }
