@@ -1,0 +1,80 @@
+"""Randomised geometries (fixed seeds) through the fp16 convolution and depthwise kernels whose index arithmetic
+depends on the image size: the resident-tile Conv2D kernels (forward, input gradient, weight gradient, both
+gradients in one call) and the depthwise kernels, against torch in float32.  The oracle checks in
+test_gpu_parity.py pin the arithmetic; these cases sweep row lengths, paddings and batch sizes for ragged tiles,
+sample boundaries inside a tile, partial column groups and plane edges."""
+import ctypes
+import random
+
+import numpy as np
+import pytest
+import torch
+import torch.nn.functional as F
+
+import helpers as hp
+
+pytestmark = pytest.mark.gpu
+
+
+def rel(got, ref):
+    return float((got.float() - ref).norm() / (ref.norm() + 1e-20))
+
+
+@pytest.mark.parametrize("seed", [11, 12, 13])
+def test_conv2d_resident_tile_random_geometries(pkg, gpu, seed):
+    rng = random.Random(seed)
+    for it in range(14):
+        Ci, Co = rng.choice([64, 64, 128, 192]), rng.choice([64, 128, 128, 192, 256])
+        pl, pr, pu, pd = (rng.randint(0, 2) for _ in range(4))
+        W, H = rng.randint(max(3 - pl - pr, 1), 61 - pl - pr), rng.randint(max(3 - pu - pd, 1), 40)
+        ns = rng.choice([1, 2, 3, 5, 8, 17, 40])
+        Ho, Wo = H + pu + pd - 2, W + pl + pr - 2
+        x = (torch.rand(ns, Ci, H, W, device="cuda") - 0.5).half()
+        w = ((torch.rand(Co, Ci, 3, 3, device="cuda") - 0.5) * 0.2).half()
+        dy = (torch.rand(ns, Co, Ho, Wo, device="cuda") - 0.5).half()
+        y, dx, dw = torch.full_like(dy, 3), torch.full_like(x, 3), torch.full_like(w, 3)
+        dx2, dw2 = torch.full_like(x, 3), torch.full_like(w, 3)
+        a, keep = hp.conv2d_args(pkg, x, dx, w, dw, y, dy, Ci, H, W, Co, 3, 3, Ho, Wo, (pl, pr, pu, pd), (1, 1))
+        a2, keep2 = hp.conv2d_args(pkg, x, dx2, w, dw2, y, dy, Ci, H, W, Co, 3, 3, Ho, Wo, (pl, pr, pu, pd), (1, 1))
+        gpu.ptl_set_gemm_path(5)
+        try:
+            for s in ("fw", "ig", "wg"):
+                pkg.call("ptl_conv2d_fp16_%s_batched" % s, a, ns)
+            pkg.call("ptl_conv2d_fp16_bw_batched", a2, ns)
+        finally:
+            gpu.ptl_set_gemm_path(0)
+        gpu.ptl_sync()
+        xp = F.pad(x.float(), (pl, pr, pu, pd))
+        ref_y = F.conv2d(xp, w.float())
+        ref_dx = torch.nn.grad.conv2d_input(xp.shape, w.float(), dy.float())[:, :, pu:pu + H, pl:pl + W]
+        ref_dw = torch.nn.grad.conv2d_weight(xp, w.shape, dy.float())
+        case = (Ci, Co, H, W, (pl, pr, pu, pd), ns)
+        for name, got, ref in (("y", y, ref_y), ("dx", dx, ref_dx), ("dw", dw, ref_dw), ("dx one call", dx2, ref_dx),
+                               ("dw one call", dw2, ref_dw)):
+            assert rel(got, ref) <= 2e-3, (case, name)
+
+
+@pytest.mark.parametrize("seed", [21, 22])
+def test_depthwise_random_geometries(pkg, gpu, seed):
+    rng = random.Random(seed)
+    for it in range(14):
+        C, ns = rng.choice([32, 64, 96]), rng.choice([8, 16, 24])
+        pl, pr, pu, pd = rng.choice([0, 2]), rng.randint(0, 2), rng.randint(0, 2), rng.randint(0, 2)
+        W, H = rng.choice([30, 32, 34, 40, 46, 56, 58, 64]), rng.randint(8, 60)
+        Ho, Wo = H + pu + pd - 2, W + pl + pr - 2
+        x = (torch.rand(ns, C, H, W, device="cuda") - 0.5).half()
+        w = (torch.rand(C, 3, 3, device="cuda") - 0.5).half()
+        dy = (torch.rand(ns, C, Ho, Wo, device="cuda") - 0.5).half()
+        y, dx, dw = torch.full_like(dy, 3), torch.full_like(x, 3), torch.full_like(w, 3)
+        a, keep = hp.dw_args(pkg, "fp16", x, dx, w, dw, y, dy, C, H, W, 3, 3, Ho, Wo, (pl, pr, pu, pd))
+        for s in ("fw", "wg", "ig"):
+            pkg.call("ptl_conv_dw_fp16_%s_batched" % s, a, ns)
+        gpu.ptl_sync()
+        xp = F.pad(x.float(), (pl, pr, pu, pd)).requires_grad_(True)
+        wf = w.float().unsqueeze(1).requires_grad_(True)
+        ref_y = F.conv2d(xp, wf, groups=C)
+        ref_y.backward(dy.float())
+        case = (C, H, W, (pl, pr, pu, pd), ns)
+        assert rel(y, ref_y.detach()) <= 2e-3, (case, "y")
+        assert rel(dw, wf.grad.squeeze(1)) <= 2e-3, (case, "dw")
+        assert rel(dx, xp.grad[:, :, pu:pu + H, pl:pl + W]) <= 2e-3, (case, "dx")
