@@ -507,13 +507,17 @@ bool conv_halo_wg_fits(const ConvTileDesc &d, int Hp, int Wp) {
     return !d.in_hwc && d.KH == 3 && d.KW == 3 && d.sh == 1 && d.sw == 1 && d.Cin % 64 == 0 && d.Cout % 128 == 0 &&
            2 * Wp + 2 <= 128 && d.Ho == Hp - 2 && d.Wo == Wp - 2 && (long long)d.batch * Hp * Wp < ((long long)1 << 31);
 }
-// Measured against the alternatives (fp16, batch 128..512): 128 -> 128 on 28x28 73 / 243 against 87 / 306 us (resident
-// output tile kernel), 256 -> 256 on 14x14 70 against 83 us and on 28x28 384 against 390 us (tap-sum GEMM); 512 -> 512
-// on 14x14 359 against 353 us and 64 -> 128 on 56x56 280 against 274 us stay where they were.
+// Measured against the alternatives (fp16): at batch 128..512, 128 -> 128 on 28x28 73 / 243 against 87 / 306 us
+// (resident output tile kernel), 256 -> 256 on 14x14 70 against 83 us and on 28x28 384 against 390 us, 512 -> 512 on
+// 7x7 69 against 86 us (tap-sum GEMM); from 256 channels it wins from 20 units of positions on (512 -> 512 on 7x7 at
+// batch 32: 38 against 53 us; 256 -> 256 on 14x14 at batch 8, 16 units: 30 against 26 us for the resident output tile
+// kernel), with 128 channels only from about a hundred (128 -> 128 on 14x14 at batch 32: 28
+// against 25 us for the resident output tile kernel).  64 -> 128 on 56x56 (280 against 274 us) stays where it was.
 bool conv_halo_wg_preferred(const ConvTileDesc &d) {
     const int Hp = d.Hin + d.padU + d.padD, Wp = d.Win + d.padL + d.padR;
-    return conv_halo_wg_fits(d, Hp, Wp) && Wp <= 32 && !(d.Cin >= 512 && d.Cout >= 512) &&
-           (long long)d.batch * Hp * Wp >= 64ll * HWG_UNIT;
+    const long long units = ((long long)d.batch * Hp * Wp + HWG_UNIT - 1) / HWG_UNIT;
+    const int cmin = d.Cin < d.Cout ? d.Cin : d.Cout;
+    return conv_halo_wg_fits(d, Hp, Wp) && Wp <= 32 && units >= (cmin >= 256 ? 20 : 96);
 }
 long long conv_halo_wg_margin() { return 2 * HWG_UNIT + 256; }
 long long conv_halo_wg_gradient_stride(const ConvTileDesc &d, int Hp, int Wp) {

@@ -149,20 +149,23 @@ int conv_taps(const ConvTileDesc &d, const void *X, const void *Wt, void *Y, con
     const long long npix = (long long)d.batch * d.Ho * d.Wo;
     if (xb_elems * ES >= ((long long)1 << 31) || npix >= ((long long)1 << 31) || wr_elems >= ((long long)1 << 31))
         return -1;
-    // worth it only when the pixel tiles fill the chip: the passes above cost two extra launches
     if (st.gemm_path == 2) return -1;
-    // (and only with at least 64 filters: narrower products fall to the GEMM's slim tiles, where the direct kernel wins).
-    // Against the gathering GEMM, which takes over below that, it pays from a quarter of a tile per CU: measured
-    // 10.5 against 11.3 us (forward) and 16.5 us (input gradient, flipped filters) for 64 -> 64 channels on 8x8
-    // images at batch 128, 16.8 against 27.8 us for the input gradient of 128 -> 128.
-    const long long fill = npix / 128 * ((d.Cout + 127) / 128) * 4;
+    // (only with at least 64 filters: narrower products fall to the GEMM's slim tiles, where the direct kernel wins)
+    // and from about a thousand output pixels: measured at 128..512 channels, batch 8..32, the two layout passes pay
+    // from 1568 pixels on (12.6 against 24.2 us for 128 -> 128 on 14x14 at batch 8, 35.8 against 74.5 us for
+    // 512 -> 512 on 7x7 at batch 32) and do not at 392 (20.5 against 14.8 us for 256 -> 256 on 7x7 at batch 8).
     const bool forced = st.gemm_path == 3 || st.gemm_path == 5;
-    if (!forced && (d.Cout < 64 || fill < st.num_cu)) return -1;
+    if (!forced && (d.Cout < 64 || npix < 1024)) return -1;
     // 3x3 fp16 layers keep the input tile in LDS for all nine taps (ptl_conv_halo.hip): the tap-sum GEMM fetches it
     // once per tap.  Measured at batch 128..512, forward: 64 -> 64 on 56x56 63 against 96 us, 128 -> 128 on 28x28
-    // 52 against 76, 256 -> 256 on 28x28 295 against 372, 512 -> 512 on 14x14 273 against 293.
+    // 52 against 76, 256 -> 256 on 28x28 295 against 372, 512 -> 512 on 14x14 273 against 293.  Its workgroups are
+    // persistent over whole tiles (256 positions x 64 / 128 filters x all channels), so it needs enough tiles: below
+    // about 48 (32 for a single 64-channel slab) the GEMM, which splits the contraction, is faster (14.0 against
+    // 19.0 us for 128 -> 128 on 28x28 at batch 8, 35.8 against 56.5 us for 512 -> 512 on 7x7 at batch 32).
+    const long long halo_tiles = ((long long)d.batch * Hp * Wp + 255) / 256 * ((d.Cout + 127) / 128);
+    const bool halo_pays = halo_tiles >= 48 || (d.Cin == 64 && halo_tiles >= 32);
     const bool halo = ES == 2 && !hwc && conv_halo_fits(d, Hp, Wp) && (long long)d.batch * Hp * Wp < ((long long)1 << 31) &&
-                      (st.gemm_path == 5 || st.gemm_path == 0);
+                      (st.gemm_path == 5 || (st.gemm_path == 0 && halo_pays));
     const long long margin = halo ? conv_halo_margin() : 0;  // chunks the resident-tile kernel may read past the end
     char *buf = static_cast<char *>(scratch((size_t)(xb_elems + margin * VEC + wr_elems) * ES + 256));
     if (!buf) return 2;
@@ -356,6 +359,10 @@ int conv_taps_wg(const ConvTileDesc &d, const void *X, const void *dY, void *dW)
     } else {
         if (d.x_sy != d.Win) return -1;
         if (st.gemm_path != 3 && (d.Cin < 128 || d.Cout < 128)) return -1;  // measured: below that the direct kernel wins
+        // (and below about 8000 padded positions the gathering GEMM does: 12 against 29 us for eight 256 -> 256 7x7
+        // samples, 25 against 27 us for 128 -> 128 on 14x14 at batch 32)
+        if (st.gemm_path != 3 && (long long)d.batch * (d.Hin + d.padU + d.padD) * (d.Win + d.padL + d.padR) < 8192)
+            return -1;
     }
     if (st.gemm_path == 2) return -1;
     const int Hp = d.Hin + d.padU + d.padD, Wp = d.Win + d.padL + d.padR, taps = d.KH * d.KW;

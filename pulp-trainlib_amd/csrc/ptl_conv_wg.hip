@@ -506,8 +506,13 @@ int conv_tile_wg(const ConvTileDesc &d, const void *X, const void *dY, void *dW)
     // 16->32 channel 32x32 sample, 14 against 9.5 us for eight 64->64 8x8 ones)
     // (from 128 channels on the alternative is the sum over taps, which loses from half a tile per CU:
     // measured 25 against 33 us for 128 -> 128 channels on 8x8 images at batch 128)
+    // (with 256 channels on both sides a tile carries enough work at any count: 12 against 29 us for eight
+    // 256 -> 256 7x7 samples; otherwise from half a tile per CU: 32 against 43 us through the gathering GEMM for
+    // 128 -> 64 channels on 28x28 at batch 32, 21 against 14 us at batch 8)
     const bool wide = d.Cin >= 128 && d.Cout >= 128 && 2 * a.tiles >= st.num_cu;
-    if (st.gemm_path != 2 && a.tiles < st.num_cu && !wide && !(ES == 2 && (long)d.Cout * d.Cin * d.KH * d.KW <= 8192))
+    const bool deep = d.Cin >= 256 && d.Cout >= 256;
+    if (st.gemm_path != 2 && 2 * a.tiles < st.num_cu && !wide && !deep &&
+        !(ES == 2 && (long)d.Cout * d.Cin * d.KH * d.KW <= 8192))
         return -1;
 
     const int taps = d.KH * d.KW;

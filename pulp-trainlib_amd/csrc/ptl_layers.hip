@@ -353,11 +353,12 @@ static int conv2d_wg(const Args *a, int ns, const char *fn) {
         d.KH = g.Hk; d.KW = g.Wk; d.sh = g.sh; d.sw = g.sw;
         d.padU = g.Up; d.padD = g.Dp; d.padL = g.Lp; d.padR = g.Rp;
         d.x_sb = (long long)g.Ci * g.H * g.W; d.x_sc = (long long)g.H * g.W; d.x_sy = g.W;
-        // the resident-tile kernel where rows are whole 16-byte chunks, else (or on request) the sum over taps;
-        // from 256 channels on either side the sum over taps on 128x128 tiles beats the resident-tile kernel
-        // (measured at batch 128..512: 82 against 93 us for 256 -> 256 on 14x14, 455 against 533 us on 28x28,
-        // 133 against 145 us for 128 -> 256 on 28x28; 128 -> 128 stays with the tile kernel: 87 / 291 against 87 / 317 us)
-        const bool taps_first = d.Cin >= 128 && d.Cout >= 128 && (d.Cin >= 256 || d.Cout >= 256);
+        // the kernel with resident channel-blocked tiles where it is preferred; else the resident output tile kernel,
+        // else (or on request) the sum over taps.  From 256 channels on either side and 16384 output pixels the sum
+        // over taps goes before the output tile kernel (measured: 81 against 91 us for 256 -> 256 on 14x14 at batch
+        // 128, 455 against 533 us on 28x28 at batch 256; at batch 8 the output tile kernel takes 26 against 34 us)
+        const bool taps_first = d.Cin >= 128 && d.Cout >= 128 && (d.Cin >= 256 || d.Cout >= 256) &&
+                                (long long)ns * g.Ho * g.Wo >= 16384;
         if (g.hwc) {  // channel-minor tensors: the sum over taps from 64 channels on, else the gathering GEMM below
             rc = conv_taps_wg<T>(d, X, dY, dW);
         } else {
