@@ -355,7 +355,13 @@ int conv_taps_wg(const ConvTileDesc &d, const void *X, const void *dY, void *dW)
         // (no direct kernel for this layout: the alternative is the gathering GEMM, which this route beats from 64
         // channels on and a few hundred positions (measured 11.3 against 7.8 us for one 64-channel 8x8 sample,
         // 11.8 against 13.3 us for eight)
-        if (st.gemm_path != 3 && (d.Cin < 64 || d.Cout < 64 || (long long)d.batch * d.Ho * d.Wo < 512)) return -1;
+        // and about 2e8 multiply-adds per tap: a sweep over 64..512 channels on 7x7..56x56 images at batch 8..128 has
+        // the gathering GEMM ahead below that, e.g. 13.0 against 16.3 us for 64 -> 64 on 28x28 at batch 8 and 23.7
+        // against 34.1 us for 256 -> 256 on 14x14 at batch 8, and this route ahead above, 28.3 against 40.7 us for
+        // 64 -> 128 on 28x28 at batch 32, 41.7 against 69.4 us for 256 -> 256 on 14x14 at batch 32)
+        if (st.gemm_path != 3 &&
+            (d.Cin < 64 || d.Cout < 64 || (double)d.batch * d.Ho * d.Wo * d.Cin * d.Cout < 2e8))
+            return -1;
     } else {
         if (d.x_sy != d.Win) return -1;
         if (st.gemm_path != 3 && (d.Cin < 128 || d.Cout < 128)) return -1;  // measured: below that the direct kernel wins

@@ -491,9 +491,13 @@ def test_conv2d_wide_layers_hwc_against_torch(pkg, gpu, case):
     dy = dev(hp.uniform(43, (ns, H, H, Co), dtype=np.float16))
     y, dx, dw = torch.full_like(dy, 3.0), torch.full_like(x, 3.0), torch.full_like(w, 3.0)
     a, keep = hp.conv2d_args(pkg, x, dx, w, dw, y, dy, Ci, H, H, Co, 3, 3, H, H, (1, 1, 1, 1), (1, 1), 1)
-    for s in ("fw", "wg", "ig"):
-        pkg.call("ptl_conv2d_fp16_%s_batched" % s, a, ns)
-        assert gpu.ptl_last_conv_direct() == 1
+    gpu.ptl_set_gemm_path(3)  # (small batches of narrow layers would otherwise take the gathering GEMM)
+    try:
+        for s in ("fw", "wg", "ig"):
+            pkg.call("ptl_conv2d_fp16_%s_batched" % s, a, ns)
+            assert gpu.ptl_last_conv_direct() == 1
+    finally:
+        gpu.ptl_set_gemm_path(0)
     sync(gpu)
     xf, wf, dyf = (t.float().permute(0, 3, 1, 2).contiguous() for t in (x, w, dy))
     ref_y = torch.nn.functional.conv2d(xf, wf, padding=1).permute(0, 2, 3, 1)
