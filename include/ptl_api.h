@@ -353,6 +353,17 @@ int ptl_batch_norm_fp32_fw(const struct BatchNorm_args_fp32 *a);
 int ptl_batch_norm_fp32_bw(const struct BatchNorm_args_fp32 *a);
 int ptl_batch_norm_fp16_fw(const struct BatchNorm_args_fp16 *a);
 int ptl_batch_norm_fp16_bw(const struct BatchNorm_args_fp16 *a);
+/* No counterpart in the reference: the normalisation layer fused with the element-wise layers a residual block
+ * puts behind it, for training steps in which those would cost a launch each.
+ *   forward:  output->data = [relu]( bn(input->data) [+ f->skip] )
+ *   backward: g = output->diff [+ f->diff2], zeroed where output->data <= 0 when f->relu (output->data must still
+ *             hold the forward result), rounded to the tensor type; g is written to f->skip_diff when that is
+ *             given (the gradient of the skip branch); input->diff, coeff->diff and bias->diff as
+ *             ptl_batch_norm_*_bw computes them from g. */
+int ptl_batch_norm_fused_fp32_fw(const struct BatchNorm_args_fp32 *a, const struct ptl_norm_fusion_fp32 *f);
+int ptl_batch_norm_fused_fp32_bw(const struct BatchNorm_args_fp32 *a, const struct ptl_norm_fusion_fp32 *f);
+int ptl_batch_norm_fused_fp16_fw(const struct BatchNorm_args_fp16 *a, const struct ptl_norm_fusion_fp16 *f);
+int ptl_batch_norm_fused_fp16_bw(const struct BatchNorm_args_fp16 *a, const struct ptl_norm_fusion_fp16 *f);
 
 /* Plain product C[N x M] = A[N x K] * B (B is K x M, or M x K when trans_B),
  * the contract of the reference's mm family, on raw pointers. */

@@ -675,6 +675,21 @@ struct BatchNorm_args_fp16 {
     int W;
 };
 
+/* No counterpart in the reference: what a residual block puts behind a normalisation layer, for the fused calls
+ * ptl_batch_norm_fused_*.  All tensors have the shape of the normalisation's output (B x C x H x W). */
+struct ptl_norm_fusion_fp32 {
+    int relu;          /* 1: ReLU after the (optional) addition */
+    const float *skip; /* forward: tensor added to the normalised input; NULL: none */
+    float *skip_diff;  /* backward: receives the gradient of the sum (= of the skip tensor); NULL: not wanted */
+    const float *diff2; /* backward: a second incoming gradient, added to output->diff; NULL: none */
+};
+struct ptl_norm_fusion_fp16 {
+    int relu;
+    const fp16 *skip;
+    fp16 *skip_diff;
+    const fp16 *diff2;
+};
+
 #ifdef __cplusplus
 }
 #endif

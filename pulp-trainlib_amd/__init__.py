@@ -76,6 +76,9 @@ BATCHED_ENTRY_POINTS = ["ptl_%s_%s_%s_batched" % (layer, dt, step)
                             # (const optim_args *list, int count)
                             "ptl_gradient_descent_fp32_multi", "ptl_gradient_descent_fp16_multi"]
 
+# `int f(const BatchNorm_args *, const ptl_norm_fusion *)`
+FUSED_NORM_ENTRY_POINTS = ["ptl_batch_norm_fused_%s_%s" % (dt, step) for dt in ("fp32", "fp16") for step in ("fw", "bw")]
+
 OTHER_ENTRY_POINTS = ["ptl_init", "ptl_last_error", "ptl_last_status", "ptl_set_stream", "ptl_sync", "ptl_set_gemm_path",
                       "ptl_last_conv_direct", "ptl_last_gemm_streamed", "ptl_last_conv_resident", "ptl_timer_begin", "ptl_timer_end_ms", "ptl_mm_fp32", "ptl_mm_fp16", "ptl_copy_bytes"]
 
@@ -104,6 +107,10 @@ def load():
     for name in PLAIN_ENTRY_POINTS:
         f = getattr(lib, name)
         f.argtypes = [ctypes.c_void_p]
+        f.restype = ctypes.c_int
+    for name in FUSED_NORM_ENTRY_POINTS:
+        f = getattr(lib, name)
+        f.argtypes = [ctypes.c_void_p, ctypes.c_void_p]
         f.restype = ctypes.c_int
     lib.ptl_init.argtypes = [ctypes.c_int]
     lib.ptl_init.restype = ctypes.c_int

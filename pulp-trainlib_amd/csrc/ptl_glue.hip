@@ -2,6 +2,7 @@
 // pooling, cross-entropy loss, gradient descent, batch normalisation (forward).  All are bandwidth-bound
 // element or small-reduction kernels; fp16 tensors are read as IEEE half, computed in fp32 and rounded once.
 #include <float.h>
+#include <type_traits>
 
 #include "ptl_api.h"
 #include "ptl_host.hpp"
@@ -422,10 +423,24 @@ union BnVec {
     T e[16 / sizeof(T)];
 };
 
-template <typename T, bool BW>
+// What a residual block puts behind a normalisation layer, done in the same kernels:
+//   forward   out = [relu](bn(x) [+ skip]);
+//   backward  g = (dy [+ dy2]) [where out > 0, else 0], rounded to T like a tensor an element-wise layer would have
+//             written; g is the gradient of the normalisation's output and of the skip input (stored to gout when
+//             wanted), dx = bn'(g).
+template <typename T>
+struct BnFuse {
+    const T *skip;  // forward: added after the normalisation
+    const T *out;   // backward: the forward result (sign = ReLU mask)
+    const T *dy2;   // backward: second incoming gradient
+    T *gout;        // backward: receives g
+    int relu;
+};
+
+template <typename T, bool BW, bool FUSED = false>
 __global__ __launch_bounds__(256) void bn_sums_kernel(const T *__restrict__ x, const T *__restrict__ dy,
                                                       float *__restrict__ part, int B, int C, int HW, int per_group,
-                                                      int vec) {
+                                                      int vec, const BnFuse<T> f = BnFuse<T>()) {
     __shared__ float red[BN_SUMS][4];
     const int c = blockIdx.x, grp = blockIdx.y, tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int b0 = grp * per_group, b1 = min(B, b0 + per_group);
@@ -438,6 +453,20 @@ __global__ __launch_bounds__(256) void bn_sums_kernel(const T *__restrict__ x, c
                 BnVec<T> xv, gv;
                 xv.raw = *reinterpret_cast<const uint4 *>(x + base + e);
                 if (BW) gv.raw = *reinterpret_cast<const uint4 *>(dy + base + e);
+                if (BW && FUSED) {
+                    BnVec<T> g2, ov;
+                    if (f.dy2) {
+                        g2.raw = *reinterpret_cast<const uint4 *>(f.dy2 + base + e);
+#pragma unroll
+                        for (int q = 0; q < VEC; ++q) gv.e[q] = (T)((float)gv.e[q] + (float)g2.e[q]);
+                    }
+                    if (f.relu) {
+                        ov.raw = *reinterpret_cast<const uint4 *>(f.out + base + e);
+#pragma unroll
+                        for (int q = 0; q < VEC; ++q) gv.e[q] = (float)ov.e[q] > 0.f ? gv.e[q] : (T)0;
+                    }
+                    if (f.gout) *reinterpret_cast<uint4 *>(f.gout + base + e) = gv.raw;
+                }
 #pragma unroll
                 for (int q = 0; q < VEC; ++q) {
                     const float v = (float)xv.e[q];
@@ -457,7 +486,13 @@ __global__ __launch_bounds__(256) void bn_sums_kernel(const T *__restrict__ x, c
             s[0] += v;
             s[1] += v * v;
             if (BW) {
-                const float g = (float)dy[base + e];
+                T gt = dy[base + e];
+                if (FUSED) {
+                    if (f.dy2) gt = (T)((float)gt + (float)f.dy2[base + e]);
+                    if (f.relu && !((float)f.out[base + e] > 0.f)) gt = (T)0;
+                    if (f.gout) f.gout[base + e] = gt;
+                }
+                const float g = (float)gt;
                 s[2] += g;
                 s[3] += g * v;
             }
@@ -474,13 +509,14 @@ __global__ __launch_bounds__(256) void bn_sums_kernel(const T *__restrict__ x, c
         part[((size_t)c * gridDim.y + grp) * BN_SUMS + tid] = (red[tid][0] + red[tid][1]) + (red[tid][2] + red[tid][3]);
 }
 
-template <typename T, bool BW>
+template <typename T, bool BW, bool FUSED = false>
 __global__ __launch_bounds__(256) void bn_apply_kernel(const T *__restrict__ x, const T *__restrict__ dy,
                                                        T *__restrict__ out, const T *__restrict__ weight,
                                                        const T *__restrict__ bias, const T *__restrict__ eps,
                                                        const float *__restrict__ part, T *__restrict__ dgamma,
                                                        T *__restrict__ dbeta, int B, int C, int HW, int groups,
-                                                       int per_group, int write_dx, int vec) {
+                                                       int per_group, int write_dx, int vec,
+                                                       const BnFuse<T> f = BnFuse<T>()) {
     constexpr int VEC = 16 / (int)sizeof(T);
     const int c = blockIdx.x, grp = blockIdx.y, tid = threadIdx.x;
     // the channel's partial sums (at most 64 groups): one lane each, folded by the first wave in a fixed order
@@ -524,23 +560,64 @@ __global__ __launch_bounds__(256) void bn_apply_kernel(const T *__restrict__ x, 
             const size_t at = ((size_t)(b0 + bl) * C + c) * HW + e;
             BnVec<T> xv, gv;
             xv.raw = *reinterpret_cast<const uint4 *>(x + at);
-            if (BW) gv.raw = *reinterpret_cast<const uint4 *>(dy + at);
+            if (BW) {
+                // the gradient the first kernel formed (stored, or formed again the same way)
+                gv.raw = *reinterpret_cast<const uint4 *>((FUSED && f.gout ? f.gout : dy) + at);
+                if (FUSED && !f.gout) {
+                    BnVec<T> g2, ov;
+                    if (f.dy2) {
+                        g2.raw = *reinterpret_cast<const uint4 *>(f.dy2 + at);
 #pragma unroll
-            for (int q = 0; q < VEC; ++q) xv.e[q] = (T)map((float)xv.e[q], BW ? (float)gv.e[q] : 0.f);
+                        for (int q = 0; q < VEC; ++q) gv.e[q] = (T)((float)gv.e[q] + (float)g2.e[q]);
+                    }
+                    if (f.relu) {
+                        ov.raw = *reinterpret_cast<const uint4 *>(f.out + at);
+#pragma unroll
+                        for (int q = 0; q < VEC; ++q) gv.e[q] = (float)ov.e[q] > 0.f ? gv.e[q] : (T)0;
+                    }
+                }
+            }
+            if (!BW && FUSED) {
+                BnVec<T> sv;
+                if (f.skip) sv.raw = *reinterpret_cast<const uint4 *>(f.skip + at);
+#pragma unroll
+                for (int q = 0; q < VEC; ++q) {
+                    float v = map((float)xv.e[q], 0.f);
+                    if (f.skip) v += (float)sv.e[q];
+                    if (f.relu) v = fmaxf(v, 0.f);
+                    xv.e[q] = (T)v;
+                }
+            } else {
+#pragma unroll
+                for (int q = 0; q < VEC; ++q) xv.e[q] = (T)map((float)xv.e[q], BW ? (float)gv.e[q] : 0.f);
+            }
             *reinterpret_cast<uint4 *>(out + at) = xv.raw;
         }
     } else {
         for (int i = tid; i < total; i += 256) {
             const int bl = i / HW, e = i - bl * HW;
             const size_t at = ((size_t)(b0 + bl) * C + c) * HW + e;
-            out[at] = (T)map((float)x[at], BW ? (float)dy[at] : 0.f);
+            if (!BW && FUSED) {
+                float v = map((float)x[at], 0.f);
+                if (f.skip) v += (float)f.skip[at];
+                if (f.relu) v = fmaxf(v, 0.f);
+                out[at] = (T)v;
+                continue;
+            }
+            T gt = BW ? (FUSED && f.gout ? f.gout[at] : dy[at]) : (T)0;
+            if (BW && FUSED && !f.gout) {
+                if (f.dy2) gt = (T)((float)gt + (float)f.dy2[at]);
+                if (f.relu && !((float)f.out[at] > 0.f)) gt = (T)0;
+            }
+            out[at] = (T)map((float)x[at], (float)gt);
         }
     }
 }
 
-template <typename T, typename Args>
-static int batch_norm_step(const Args *a, int bw, const char *fn) {
-    if (!a || !a->input || !a->output || !a->weight_data || !a->eps || (!bw && !a->bias_data))
+template <typename T, typename Args, typename Fusion = void>
+static int batch_norm_step(const Args *a, int bw, const char *fn, const Fusion *fu = nullptr) {
+    constexpr bool FUSED = !std::is_void<Fusion>::value;
+    if (!a || !a->input || !a->output || !a->weight_data || !a->eps || (!bw && !a->bias_data) || (FUSED && !fu))
         return glue_bad(fn, "invalid arguments");
     if (a->B <= 0 || a->C <= 0 || a->H <= 0 || a->W <= 0) return glue_bad(fn, "invalid tensor geometry");
     if (!ensure_init()) return 2;
@@ -567,12 +644,19 @@ static int batch_norm_step(const Args *a, int bw, const char *fn) {
         T *y = sg.out(reinterpret_cast<T *>(a->output->data), n);
         const T *b = sg.in(reinterpret_cast<const T *>(a->bias_data), (size_t)C);
         if (sg.failed() || !y) return sg.failed() ? 2 : glue_bad(fn, "null buffer");
-        const int vec = HW % VEC == 0 && aligned16(x) && aligned16(y);
+        int vec = HW % VEC == 0 && aligned16(x) && aligned16(y);
+        BnFuse<T> f = {};
+        if constexpr (FUSED) {
+            f.relu = fu->relu ? 1 : 0;
+            f.skip = fu->skip ? sg.in(reinterpret_cast<const T *>(fu->skip), n) : nullptr;
+            if (sg.failed()) return 2;
+            vec = vec && aligned16(f.skip);
+        }
         hipLaunchKernelGGL((bn_sums_kernel<T, false>), dim3(C, groups), dim3(256), 0, st.stream, x, (const T *)nullptr,
-                           part, B, C, HW, per_group, vec);
-        hipLaunchKernelGGL((bn_apply_kernel<T, false>), dim3(C, groups), dim3(256), 0, st.stream, x,
+                           part, B, C, HW, per_group, vec, BnFuse<T>());
+        hipLaunchKernelGGL((bn_apply_kernel<T, false, FUSED>), dim3(C, groups), dim3(256), 0, st.stream, x,
                            (const T *)nullptr, y, w, b, eps, part, (T *)nullptr, (T *)nullptr, B, C, HW, groups,
-                           per_group, 1, vec);
+                           per_group, 1, vec, f);
     } else {
         const T *dy = sg.in(reinterpret_cast<const T *>(a->output->diff), n);
         const bool want_dx = !a->skip_in_grad, want_dw = !a->skip_wg_grad;
@@ -580,13 +664,25 @@ static int batch_norm_step(const Args *a, int bw, const char *fn) {
         T *dg = want_dw && a->coeff ? sg.out(reinterpret_cast<T *>(a->coeff->diff), (size_t)C) : nullptr;
         T *db = want_dw && a->bias ? sg.out(reinterpret_cast<T *>(a->bias->diff), (size_t)C) : nullptr;
         if (sg.failed() || !dy || (want_dx && !dx)) return sg.failed() ? 2 : glue_bad(fn, "null buffer");
-        const int vec = HW % VEC == 0 && aligned16(x) && aligned16(dy) && (!dx || aligned16(dx));
-        hipLaunchKernelGGL((bn_sums_kernel<T, true>), dim3(C, groups), dim3(256), 0, st.stream, x, dy, part, B, C, HW,
-                           per_group, vec);
+        int vec = HW % VEC == 0 && aligned16(x) && aligned16(dy) && (!dx || aligned16(dx));
+        BnFuse<T> f = {};
+        if constexpr (FUSED) {
+            f.relu = fu->relu ? 1 : 0;
+            if (f.relu) {
+                if (!a->output->data) return glue_bad(fn, "the ReLU mask needs the forward result in output->data");
+                f.out = sg.in(reinterpret_cast<const T *>(a->output->data), n);
+            }
+            f.dy2 = fu->diff2 ? sg.in(reinterpret_cast<const T *>(fu->diff2), n) : nullptr;
+            f.gout = fu->skip_diff ? sg.out(reinterpret_cast<T *>(fu->skip_diff), n) : nullptr;
+            if (sg.failed()) return 2;
+            vec = vec && aligned16(f.out) && aligned16(f.dy2) && aligned16(f.gout);
+        }
+        hipLaunchKernelGGL((bn_sums_kernel<T, true, FUSED>), dim3(C, groups), dim3(256), 0, st.stream, x, dy, part, B, C,
+                           HW, per_group, vec, f);
         // without an input gradient only the first group of every channel runs (it writes dgamma / dbeta)
-        hipLaunchKernelGGL((bn_apply_kernel<T, true>), dim3(C, want_dx ? groups : 1), dim3(256), 0, st.stream, x, dy,
-                           dx, w, (const T *)nullptr, eps, part, dg, db, B, C, HW, groups, per_group, want_dx ? 1 : 0,
-                           vec);
+        hipLaunchKernelGGL((bn_apply_kernel<T, true, FUSED>), dim3(C, want_dx ? groups : 1), dim3(256), 0, st.stream, x,
+                           dy, dx, w, (const T *)nullptr, eps, part, dg, db, B, C, HW, groups, per_group,
+                           want_dx ? 1 : 0, vec, f);
     }
     return sg.finish(hip_ok(hipGetLastError(), "batch norm launch") ? 0 : 2);
 }
@@ -645,6 +741,18 @@ int ptl_batch_norm_fp16_fw(const struct BatchNorm_args_fp16 *a) {
 }
 int ptl_batch_norm_fp16_bw(const struct BatchNorm_args_fp16 *a) {
     return ptl::batch_norm_step<ptl::half_t>(a, 1, "ptl_batch_norm_fp16_bw");
+}
+int ptl_batch_norm_fused_fp32_fw(const struct BatchNorm_args_fp32 *a, const struct ptl_norm_fusion_fp32 *f) {
+    return ptl::batch_norm_step<float>(a, 0, "ptl_batch_norm_fused_fp32_fw", f);
+}
+int ptl_batch_norm_fused_fp32_bw(const struct BatchNorm_args_fp32 *a, const struct ptl_norm_fusion_fp32 *f) {
+    return ptl::batch_norm_step<float>(a, 1, "ptl_batch_norm_fused_fp32_bw", f);
+}
+int ptl_batch_norm_fused_fp16_fw(const struct BatchNorm_args_fp16 *a, const struct ptl_norm_fusion_fp16 *f) {
+    return ptl::batch_norm_step<ptl::half_t>(a, 0, "ptl_batch_norm_fused_fp16_fw", f);
+}
+int ptl_batch_norm_fused_fp16_bw(const struct BatchNorm_args_fp16 *a, const struct ptl_norm_fusion_fp16 *f) {
+    return ptl::batch_norm_step<ptl::half_t>(a, 1, "ptl_batch_norm_fused_fp16_bw", f);
 }
 
 }  // extern "C"

@@ -164,6 +164,11 @@ class BatchNormArgs(C.Structure):
                 ("B", I), ("C", I), ("H", I), ("W", I)]
 
 
+class NormFusion(C.Structure):
+    """struct ptl_norm_fusion_fp32 / _fp16: what ptl_batch_norm_fused_* does behind the normalisation."""
+    _fields_ = [("relu", I), ("skip", P), ("skip_diff", P), ("diff2", P)]
+
+
 LAYER_CONV2D, LAYER_DW_CONV, LAYER_PW_CONV, LAYER_LINEAR = 0, 1, 2, 3
 STEP_FW, STEP_WGT_GRAD, STEP_IN_GRAD = 0, 1, 2
 

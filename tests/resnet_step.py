@@ -44,8 +44,13 @@ def init_weights(seed, dt):
 class ResNetStep:
     """Device buffers, argument structs and the call sequence of one training step on `ns` samples."""
 
-    def __init__(self, pkg, lib, torch, dt, ns, weights, lr=0.01, norm=False):
+    def __init__(self, pkg, lib, torch, dt, ns, weights, lr=0.01, norm=False, fused=False):
+        """`fused` (with `norm`): ReLU, the residual sum and the sum of a tensor's two incoming gradients run inside
+        the normalisation calls (ptl_batch_norm_fused_*) instead of as element-wise calls of their own."""
         self.pkg, self.lib, self.dt, self.ns, self.lr = pkg, lib, dt, ns, lr
+        if fused:
+            assert norm
+            return self._build_fused(torch, weights)
         tdt = torch.float16 if dt == "fp16" else torch.float32
         dev = lambda a: torch.from_numpy(np.ascontiguousarray(a)).cuda()
         z = lambda *s: torch.zeros(*s, dtype=tdt, device="cuda")
@@ -168,6 +173,121 @@ class ResNetStep:
         table = (type(opts[0]) * len(opts))(*opts)
         self.opt = [(L("ptl_gradient_descent_DT_multi"), table, (len(opts),))]
 
+    def _build_fused(self, torch, weights):
+        pkg, dt, ns = self.pkg, self.dt, self.ns
+        tdt = torch.float16 if dt == "fp16" else torch.float32
+        dev = lambda a: torch.from_numpy(np.ascontiguousarray(a)).cuda()
+        z = lambda *s: torch.zeros(*s, dtype=tdt, device="cuda")
+        convs, blocks, ncls = resnet20_spec()
+        self.W = {n: dev(v) for n, v in weights.items()}
+        self.dW = {n: z(*v.shape) for n, v in weights.items()}
+        self.keep, self.G, self.dG, self.Bt, self.dBt = [], {}, {}, {}, {}
+        self.conv_layers, self.norm_layers = [], []
+        eps = torch.full((1,), 1e-5, dtype=tdt, device="cuda")
+        spec = {n: (ci, co, k, s) for n, ci, co, k, s in convs}
+        L = lambda name: name.replace("DT", dt)
+
+        def conv(name, x, dx, H):
+            """The convolution alone: (forward call, backward calls, output, its gradient, output size)."""
+            ci, co, k, s = spec[name]
+            p = k // 2
+            Ho = (H + 2 * p - k) // s + 1
+            y, dy = z(ns, co, Ho, Ho), z(ns, co, Ho, Ho)
+            a, kp = hp.conv2d_args(pkg, x, dx, self.W[name], self.dW[name], y, dy, ci, H, H, co, k, k, Ho, Ho,
+                                   (p, p, p, p), (s, s), 0, 1 if s == 1 else 0)
+            self.keep.append(kp)
+            bw = [(L("ptl_conv2d_DT_wg_batched"), a, (ns,))]
+            if dx is not None:
+                bw.append((L("ptl_conv2d_DT_ig_batched"), a, (ns,)))
+            return (L("ptl_conv2d_DT_fw_batched"), a, (ns,)), bw, y, dy, Ho
+
+        def norm(name, y, dy, Ho, relu, skip=None, out_diff=None):
+            """out = [relu](bn(y) [+ skip]); returns the calls, out, its gradient buffer and the fusion struct (whose
+            skip_diff / diff2 the caller fills in once the tensors exist)."""
+            co = spec[name][1]
+            self.G[name], self.Bt[name] = torch.ones(co, dtype=tdt, device="cuda"), z(co)
+            self.dG[name], self.dBt[name] = z(co), z(co)
+            out, dout = z(ns, co, Ho, Ho), (out_diff if out_diff is not None else z(ns, co, Ho, Ho))
+            na, kp = hp.batch_norm_args(pkg, y, out, self.G[name], self.Bt[name], eps, ns, co, Ho, Ho, dy, dout,
+                                        self.dG[name], self.dBt[name])
+            f = pkg.NormFusion()
+            f.relu = relu
+            f.skip = pkg.addr(skip)
+            self.keep += [kp, f, skip]
+            return (L("ptl_batch_norm_fused_DT_fw"), na, (f,)), (L("ptl_batch_norm_fused_DT_bw"), na, (f,)), out, dout, f
+
+        self.x = z(ns, 3, 32, 32)
+        cf, cb, y, dy, H = conv("stem", self.x, None, 32)
+        nf, nb, t, dt_, fus = norm("stem", y, dy, H, 1)
+        self.fw = [cf, nf]
+        first_bw = [nb] + cb
+        bw_blocks = []
+        for (n, ci, co, stride, proj) in blocks:
+            xin, dxin, Hin, fus_in = t, dt_, H, fus
+            c1f, c1b, y1, dy1, H = conv(n + "c1", xin, dxin, Hin)
+            n1f, n1b, a1, da1, _ = norm(n + "c1", y1, dy1, H, 1)
+            c2f, c2b, y2, dy2, H = conv(n + "c2", a1, da1, H)
+            seq = [c1f, n1f, c2f]
+            ds_ = z(*y2.shape)  # gradient of the sum = gradient of the shortcut branch
+            if proj:
+                dproj = z(*xin.shape)
+                csf, csb, ysr, dysr, _ = conv(proj, xin, dproj, Hin)
+                # the projection's normalisation (no ReLU, nothing added) reads ds_ as the gradient of its output
+                nsf, nsb, ys, _, _ = norm(proj, ysr, dysr, H, 0, out_diff=ds_)
+                seq += [csf, nsf]
+                skip = ys
+            else:
+                skip = xin
+            n2f, n2b, t, dt_, fus = norm(n + "c2", y2, dy2, H, 1, skip=skip)
+            fus.skip_diff = pkg.addr(ds_)
+            self.keep.append(ds_)
+            seq.append(n2f)
+            self.fw += seq
+            b = [n2b] + c2b + [n1b] + c1b
+            if proj:
+                b += [nsb] + csb
+                fus_in.diff2 = pkg.addr(dproj)  # the block's input gets its gradient from c1 and from the projection
+                self.keep.append(dproj)
+            else:
+                fus_in.diff2 = pkg.addr(ds_)    # ... or from c1 and the identity shortcut
+            bw_blocks.append(b)
+        self._tail(torch, t, dt_, H, bw_blocks, first_bw, ncls)
+
+    def _tail(self, torch, t, dt_, H, bw_blocks, first_bw, ncls):
+        """Global average pooling, classifier, loss, the backward order and the update call."""
+        pkg, dt, ns = self.pkg, self.dt, self.ns
+        tdt = torch.float16 if dt == "fp16" else torch.float32
+        z = lambda *s: torch.zeros(*s, dtype=tdt, device="cuda")
+        L = lambda name: name.replace("DT", dt)
+        pooled, dpooled = z(ns, 64), z(ns, 64)
+        pa, kp = hp.pool_args(pkg, t, dt_, pooled, dpooled, 64, H, H, 1, 1, H, H, H, H)
+        self.keep.append(kp)
+        self.logits, dlogits = z(ns, ncls), z(ns, ncls)
+        self.pooled, self.dpooled, self.dlogits = pooled, dpooled, dlogits
+        la, kp = hp.linear_args(pkg, pooled, dpooled, self.W["fc"], self.dW["fc"], self.logits, dlogits, 64, ncls)
+        self.keep.append(kp)
+        self.target, self.loss = z(ns, ncls), z(ns)
+        ca, kp = hp.loss_args(pkg, self.logits, dlogits, self.target, self.loss, ncls)
+        self.keep.append(kp)
+        self.fw += [(L("ptl_avgpool_DT_batched"), pa, (ns, 0)), (L("ptl_linear_DT_fw_batched"), la, (ns,)),
+                    (L("ptl_cross_entropy_DT_batched"), ca, (ns, 0))]
+        self.bw = [(L("ptl_cross_entropy_DT_batched"), ca, (ns, 1)), (L("ptl_linear_DT_bw_batched"), la, (ns,)),
+                   (L("ptl_avgpool_DT_batched"), pa, (ns, 1))]
+        for b in reversed(bw_blocks):
+            self.bw += b
+        self.bw += first_bw
+        opts = []
+        for n in self.W:
+            o, kp = hp.optim_args(pkg, dt, self.W[n], self.dW[n], None, None, self.lr, 0.0)
+            self.keep.append(kp)
+            opts.append(o)
+        for n in self.G:
+            o, kp = hp.optim_args(pkg, dt, self.G[n], self.dG[n], self.Bt[n], self.dBt[n], self.lr, 0.0)
+            self.keep.append(kp)
+            opts.append(o)
+        table = (type(opts[0]) * len(opts))(*opts)
+        self.opt = [(L("ptl_gradient_descent_DT_multi"), table, (len(opts),))]
+
     def _vect_sum(self, acc, term):
         """acc += term through the reference-named vect_sum entry point (lib/sources/pulp_train_utils_fp32.c:208)."""
         a = self.pkg.VectSumArgs()
@@ -181,7 +301,8 @@ class ResNetStep:
                 getattr(self.lib, name)(ctypes.byref(a))
                 rc = self.lib.ptl_last_status()
             else:
-                rc = getattr(self.lib, name)(ctypes.byref(a), *extra)
+                rc = getattr(self.lib, name)(ctypes.byref(a), *[ctypes.byref(e) if isinstance(e, ctypes.Structure) else e
+                                                                 for e in extra])
             if rc != 0:
                 raise RuntimeError("%s failed: %s" % (name, self.lib.ptl_last_error().decode()))
 

@@ -175,6 +175,59 @@ def test_batch_norm_training_passes(pkg, orc, gpu, dt, B, C, H, W):
     assert bool(torch.all(dw == 9)) and bool(torch.all(db == 9)) and hp.rel_l2(host(dx), rdx) <= tol
 
 
+@pytest.mark.parametrize("dt", ["fp32", "fp16"])
+@pytest.mark.parametrize("B,C,H,W", [(8, 16, 9, 11), (128, 16, 32, 32), (5, 70, 8, 8)])
+@pytest.mark.parametrize("relu,skip,second,keep", [(1, 1, 1, 1), (1, 0, 0, 0), (0, 1, 0, 1), (1, 1, 0, 0), (1, 0, 1, 1)])
+def test_batch_norm_fused_with_residual_and_relu(pkg, gpu, dt, B, C, H, W, relu, skip, second, keep):
+    """out = [relu](bn(x) [+ skip]) and its backward from dy [+ dy2] in one call each, against torch autograd in
+    float64 on the same rounded inputs (tolerances: a few roundings of the result type)."""
+    import torch.nn.functional as F
+    nd = hp.np_dtype(dt)
+    x = (1.5 * hp.normal(0x7F60, (B, C, H, W)) + 0.25).astype(nd)
+    sk = hp.normal(0x7F64, (B, C, H, W)).astype(nd)
+    g1, g2 = hp.uniform(0x7F61, (B, C, H, W)).astype(nd), hp.uniform(0x7F65, (B, C, H, W)).astype(nd)
+    w, b = hp.uniform(0x7F62, (C,), 0.5, 1.5).astype(nd), hp.uniform(0x7F63, (C,)).astype(nd)
+    eps = np.array([1e-5], nd)
+    gx, gsk, gg1, gg2, gw, gb, geps = dev(x), dev(sk), dev(g1), dev(g2), dev(w), dev(b), dev(eps)
+    y, dx, ds = torch.full_like(gx, 7), torch.full_like(gx, 7), torch.full_like(gx, 7)
+    dw, db = torch.full_like(gw, 7), torch.full_like(gb, 7)
+    c, k2 = hp.batch_norm_args(pkg, gx, y, gw, gb, geps, B, C, H, W, dx, gg1, dw, db)
+    f = pkg.NormFusion()
+    f.relu = relu
+    f.skip = pkg.addr(gsk) if skip else None
+    f.skip_diff = pkg.addr(ds) if keep else None
+    f.diff2 = pkg.addr(gg2) if second else None
+    assert getattr(gpu, "ptl_batch_norm_fused_%s_fw" % dt)(ctypes.byref(c), ctypes.byref(f)) == 0, gpu.ptl_last_error().decode()
+    assert getattr(gpu, "ptl_batch_norm_fused_%s_bw" % dt)(ctypes.byref(c), ctypes.byref(f)) == 0, gpu.ptl_last_error().decode()
+    gpu.ptl_sync()
+    # reference
+    tx = torch.tensor(x.astype(np.float64), requires_grad=True)
+    tw, tb = torch.tensor(w.astype(np.float64), requires_grad=True), torch.tensor(b.astype(np.float64), requires_grad=True)
+    pre = F.batch_norm(tx, None, None, tw, tb, training=True, eps=float(eps[0]))
+    if skip:
+        pre = pre + torch.tensor(sk.astype(np.float64))
+    out = torch.relu(pre) if relu else pre
+    gin = g1.astype(np.float64) + (g2.astype(np.float64) if second else 0.0)
+    gin = gin.astype(nd).astype(np.float64)  # the sum is a tensor of the layer's type
+    out.backward(torch.tensor(gin))
+    tol = 2e-5 if dt == "fp32" else 2e-3
+    got_y = host(y).astype(np.float64)
+    assert hp.rel_l2(got_y, out.detach().numpy()) <= tol
+    # the mask the library used is its own rounded forward result; where torch's result is within rounding of 0
+    # the two may differ, so the gradient reference takes the library's sign pattern
+    mask = (got_y > 0) if relu else np.ones_like(got_y, bool)
+    gref = np.where(mask, gin, 0.0)
+    if keep:
+        assert np.array_equal(host(ds).astype(np.float64), gref)
+    tx2 = torch.tensor(x.astype(np.float64), requires_grad=True)
+    tw2, tb2 = torch.tensor(w.astype(np.float64), requires_grad=True), torch.tensor(b.astype(np.float64), requires_grad=True)
+    F.batch_norm(tx2, None, None, tw2, tb2, training=True, eps=float(eps[0])).backward(torch.tensor(gref))
+    for got, ref in ((dx, tx2.grad), (dw, tw2.grad), (db, tb2.grad)):
+        assert hp.rel_l2(host(got).astype(np.float64), ref.numpy()) <= tol
+    if not keep:
+        assert bool(torch.all(ds == 7))
+
+
 def test_reference_named_single_sample_entry_points(pkg, orc, gpu):
     dim = 300
     x, g = hp.uniform(0x7E50, (dim,)), hp.uniform(0x7E51, (dim,))
