@@ -247,7 +247,10 @@ int ptl_sync(void);
  * call; 3 = as 0, but the sum-over-filter-taps route (unit-stride layers whose
  * channel counts fill whole 128-byte slabs) is taken whenever the geometry fits
  * it, on the pipelined GEMM; 5 = the same route with the input tile resident in
- * LDS for all taps (3x3 fp16 channel-major layers) wherever that kernel fits.
+ * LDS for all taps (3x3 fp16 channel-major layers) wherever that kernel fits;
+ * 6 = as 0, but the single-launch kernel for small 3x3 fp16 channel-major
+ * layers (at most 64 channels on either side; by default only up to four
+ * workgroups per compute unit) is taken whenever the geometry fits it.
  * All routes compute the same products.
  * ptl_last_conv_direct() tells whether the last Conv2D call ran one of the
  * convolution kernels (1) or the implicit-im2col GEMM (0);
@@ -255,7 +258,8 @@ int ptl_sync(void);
  * GEMM ran its streaming kernel (resident row panel, column tiles streamed:
  * the route of pointwise layers over a batch) (1) or a tile-per-workgroup
  * kernel (0); ptl_last_conv_resident() whether the last Conv2D forward or
- * input-gradient call that took the tap route kept its input tile in LDS (1). */
+ * input-gradient call that took the tap route kept its input tile in LDS (1),
+ * or ran the small-layer kernel (2). */
 void ptl_set_gemm_path(int path);
 int ptl_last_conv_direct(void);
 int ptl_last_gemm_streamed(void);

@@ -26,6 +26,11 @@ struct ConvTileDesc {
 template <typename T>
 int conv_tile(const ConvTileDesc &d, const void *X, const void *Wt, void *Y, const OutMap &c);
 
+// 3x3 fp16 layers with at most 64 channels on either side, dense channel-major tensors: one launch that reads the
+// caller's tensors directly (ptl_conv_small.hip).  Y is the dense channel-major output [batch][Cout][Ho][Wo].
+// Returns -1 when the layer does not fit or is large enough for the persistent kernels to be ahead.
+int conv_small(const ConvTileDesc &d, const void *X, const void *Wt, void *Y);
+
 }  // namespace ptl
 
 namespace ptl {

@@ -626,7 +626,8 @@ static int batch_norm_step(const Args *a, int bw, const char *fn, const Fusion *
     const size_t n = (size_t)B * C * HW;
     if ((size_t)B * C >= ((size_t)1 << 31)) return glue_bad(fn, "too many planes");
     // groups of samples: about four workgroups per CU in the first kernel
-    int groups = (4 * st.num_cu + C - 1) / C;
+    static const int mult = getenv("PTL_BN_MULT") ? atoi(getenv("PTL_BN_MULT")) : 4;
+    int groups = (mult * st.num_cu + C - 1) / C;
     if (groups > 64) groups = 64;  // the second kernel folds them with one wave
     if (groups > B) groups = B;
     const int per_group = (B + groups - 1) / groups;

@@ -272,7 +272,8 @@ static int conv2d_fw(const Args *a, int ns, const char *fn) {
             c.n = axis_plain(ns * P, g.Co);
             c.m = axis_plain(g.Co, 1);
         }
-        rc = conv_taps<T>(d, X, Wt, Y, c);
+        if (sizeof(T) == 2 && !g.hwc) rc = conv_small(d, X, Wt, Y);
+        if (rc < 0) rc = conv_taps<T>(d, X, Wt, Y, c);
         if (rc < 0) rc = conv_tile<T>(d, X, Wt, Y, c);
         if (rc > 0) return sg.finish(rc);
         if (rc == 0) state().last_conv_direct = 1;
@@ -519,7 +520,8 @@ static int conv2d_ig(const Args *a, int ns, const char *fn) {
             c.m = axis_plain(g.Ci, 1);
         }
         // (the zero-stuffed gradient of a strided layer lives in the scratch buffer the tap route would reuse)
-        int rc = (g.sh == 1 && g.sw == 1) ? conv_taps<T>(d, dY, Wt, dX, c) : -1;
+        int rc = (sizeof(T) == 2 && !g.hwc) ? conv_small(d, dY, Wt, dX) : -1;
+        if (rc < 0 && g.sh == 1 && g.sw == 1) rc = conv_taps<T>(d, dY, Wt, dX, c);
         if (rc < 0) rc = conv_tile<T>(d, dY, Wt, dX, c);
         if (rc == 0) state().last_conv_direct = 1;
         if (rc >= 0) return sg.finish(rc);

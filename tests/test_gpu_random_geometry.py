@@ -54,6 +54,52 @@ def test_conv2d_resident_tile_random_geometries(pkg, gpu, seed):
             assert rel(got, ref) <= 2e-3, (case, name)
 
 
+@pytest.mark.parametrize("seed", [31, 32, 33])
+def test_conv2d_small_layer_kernel_random_geometries(pkg, gpu, seed):
+    """The single-launch kernel for small 3x3 fp16 layers (forced with path 6): channel counts that are not whole
+    blocks (3, 24, 40 ...), strides 1 and 2, paddings 0..2 per side, rows of 8..64 elements, ragged last row tiles."""
+    rng = random.Random(seed)
+    ran = 0
+    for it in range(16):
+        Ci, Co = rng.choice([3, 8, 16, 24, 32, 48, 64]), rng.choice([8, 16, 24, 32, 40, 64])
+        st = rng.choice([1, 1, 2])
+        pl, pr, pu, pd = (rng.randint(0, 2) for _ in range(4))
+        W, H = rng.choice([8, 16, 24, 32, 40, 64]), rng.randint(3, 36)
+        if st == 2:  # the strides must divide the padded extents minus the filter
+            pr += (W + pl + pr - 3) % 2
+            pd += (H + pu + pd - 3) % 2
+        ns = rng.choice([1, 2, 3, 7, 32, 130])
+        Ho, Wo = (H + pu + pd - 3) // st + 1, (W + pl + pr - 3) // st + 1
+        x = (torch.rand(ns, Ci, H, W, device="cuda") - 0.5).half()
+        w = ((torch.rand(Co, Ci, 3, 3, device="cuda") - 0.5) * 0.5).half()
+        dy = (torch.rand(ns, Co, Ho, Wo, device="cuda") - 0.5).half()
+        y, dx, dw = torch.full_like(dy, 3), torch.full_like(x, 3), torch.full_like(w, 3)
+        a, keep = hp.conv2d_args(pkg, x, dx, w, dw, y, dy, Ci, H, W, Co, 3, 3, Ho, Wo, (pl, pr, pu, pd), (st, st))
+        case = (Ci, Co, H, W, (pl, pr, pu, pd), st, ns)
+        gpu.ptl_set_gemm_path(6)
+        try:
+            pkg.call("ptl_conv2d_fp16_fw_batched", a, ns)
+            small_fw = gpu.ptl_last_conv_resident() == 2
+            pkg.call("ptl_conv2d_fp16_ig_batched", a, ns)
+            small_ig = gpu.ptl_last_conv_resident() == 2
+        finally:
+            gpu.ptl_set_gemm_path(0)
+        gpu.ptl_sync()
+        # the kernel fits when the filter tensor is whole 16-byte pieces and one row of every channel block is at most
+        # 32 wave-wide loads; the input gradient of a unit-stride layer sees the output as its input, whose rows must
+        # be whole pieces too
+        blocks = lambda c: (16 if c <= 16 else 32 if c <= 32 else 64) // 8
+        assert small_fw == ((Ci * Co * 9) % 8 == 0 and blocks(Ci) * (W // 8) <= 32), case
+        assert small_ig == (st == 1 and Wo % 8 == 0 and (Ci * Co * 9) % 8 == 0 and blocks(Co) * (Wo // 8) <= 32), case
+        ran += small_fw + small_ig
+        xp = F.pad(x.float(), (pl, pr, pu, pd))
+        ref_y = F.conv2d(xp, w.float(), stride=st)
+        ref_dx = torch.nn.grad.conv2d_input(xp.shape, w.float(), dy.float(), stride=st)[:, :, pu:pu + H, pl:pl + W]
+        assert rel(y, ref_y) <= 2e-3, (case, "y")
+        assert rel(dx, ref_dx) <= 2e-3, (case, "dx")
+    assert ran >= 12
+
+
 @pytest.mark.parametrize("seed", [21, 22])
 def test_depthwise_random_geometries(pkg, gpu, seed):
     rng = random.Random(seed)
