@@ -51,12 +51,11 @@ union Piece {
 };
 
 template <int CINP, int F_MAX>
-__global__ __launch_bounds__(CS_NT) void conv_small_kernel(const ConvSmallArgs a) {
-    extern __shared__ __attribute__((aligned(16))) char smem[];
+__device__ inline void conv_small_block(const ConvSmallArgs &a, int tile, char *smem) {
     char *F = smem;
     half_t *T = reinterpret_cast<half_t *>(smem + a.f_bytes);  // [CINP / 8][POS][8]
     const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const int b = blockIdx.x / a.tiles_per_img, y0 = (blockIdx.x - b * a.tiles_per_img) * a.R;
+    const int b = tile / a.tiles_per_img, y0 = (tile - b * a.tiles_per_img) * a.R;
     const int iy0 = y0 * a.s - a.padU;
 
     // ---- all global loads first
@@ -178,25 +177,214 @@ __global__ __launch_bounds__(CS_NT) void conv_small_kernel(const ConvSmallArgs a
     }
 }
 
+// ---- Weight gradient of the same layers (unit stride, output rows as wide as input rows) -----------------------
+// dW(co, ci, ky, kx) = sum over positions of dY(co, p) * X(ci, p + tap shift): the contraction runs over positions,
+// which are contiguous in both channel-major tensors, so both MFMA operands are 16-byte pieces straight from global
+// memory (rows = filters, columns = channels, k = 8 consecutive output columns per lane half); the three column taps
+// of a filter row are the input piece shifted by whole elements in registers (its neighbours' edge dwords are loaded
+// beside it), rows and columns outside the image read as zeros.  A workgroup owns a range of output rows; its waves are
+// (filter row ky) x (32x32 block of the weight tensor) x (share of the positions); the shares are added through LDS
+// and the workgroup's partial sums go to ws[workgroup][co][ci][tap]; a second launch adds the workgroups.
+struct WgSmallArgs {
+    const half_t *X, *dY;
+    float *ws;
+    int batch, Cin, Cout, Hin, Win, Ho, Wo, padU, padL;
+    int nwg, rows_per_wg;  // workgroups, output rows (sample * Ho + row) per workgroup
+    int Go;                // 8-column groups per output row
+    unsigned magic_go, magic_ho, magic_cin9;
+    int cbi_n, combos, kparts;  // 32-channel blocks, (filter block, channel block) pairs, position shares
+    int total;                  // Cout * Cin * 9
+};
+
+// elements D .. D + 7 of a row of which c holds elements 0..7, p3 elements -2, -1 and n0 elements 8, 9
+template <int D>
+__device__ inline uint4 shifted_piece(const uint4 &c, unsigned p3, unsigned n0) {
+    if constexpr (D == 0) return c;
+    if constexpr (D == -1)
+        return make_uint4(__builtin_amdgcn_alignbyte(c.x, p3, 2), __builtin_amdgcn_alignbyte(c.y, c.x, 2),
+                          __builtin_amdgcn_alignbyte(c.z, c.y, 2), __builtin_amdgcn_alignbyte(c.w, c.z, 2));
+    if constexpr (D == 1)
+        return make_uint4(__builtin_amdgcn_alignbyte(c.y, c.x, 2), __builtin_amdgcn_alignbyte(c.z, c.y, 2),
+                          __builtin_amdgcn_alignbyte(c.w, c.z, 2), __builtin_amdgcn_alignbyte(n0, c.w, 2));
+    if constexpr (D == -2) return make_uint4(p3, c.x, c.y, c.z);
+    return make_uint4(c.y, c.z, c.w, n0);
+}
+
+template <int PADL>
+__device__ inline void wg_small_block(const WgSmallArgs &a, int wg, char *smem) {
+    const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int ky = wave % 3, rest = wave / 3;
+    const int combo = rest % a.combos, kpart = rest / a.combos;
+    const bool active = wave < 15 && kpart < a.kparts;
+    const int cbo = combo / a.cbi_n, cbi = combo - cbo * a.cbi_n;
+    const int lr = lane & 31, kg = lane >> 5;
+    const int co = cbo * 32 + lr, ci = cbi * 32 + lr;
+    // this workgroup's rows of the output (sample * Ho + row), as groups of 8 columns, two groups per k step
+    const int r0 = wg * a.rows_per_wg, nrows = min(a.rows_per_wg, a.batch * a.Ho - r0);
+    const int ngroups = nrows * a.Go, nks = (ngroups + 1) >> 1;
+    f32x16 acc[3];
+#pragma unroll
+    for (int kx = 0; kx < 3; ++kx)
+#pragma unroll
+        for (int v = 0; v < 16; ++v) acc[kx][v] = 0.f;
+    if (active) {
+        // Every load is executed by every lane from an address inside the tensors (filters and channels beyond the
+        // tensors repeat the last one: their rows and columns of the product are never stored; rows above or below
+        // the image are clamped into it), and what must read as zero is masked afterwards: the gradient piece where
+        // the group is beyond the range or the input row is outside the image, the edge dwords at the row ends.
+        const half_t *gy = a.dY + (unsigned)(min(co, a.Cout - 1) * a.Ho * a.Wo);
+        const half_t *gx = a.X + (unsigned)(min(ci, a.Cin - 1) * a.Hin * a.Win);
+        const unsigned ysb = (unsigned)(a.Cout * a.Ho * a.Wo), xsb = (unsigned)(a.Cin * a.Hin * a.Win);
+        constexpr int U = 4;  // k steps whose loads are in flight together
+        for (int ks0 = kpart; ks0 < nks; ks0 += U * a.kparts) {
+            uint4 A[U], C[U];
+            unsigned p3[U], n0[U];
+            bool okA[U], okP[U], okN[U];
+#pragma unroll
+            for (int u = 0; u < U; ++u) {
+                const int gi = min(2 * (ks0 + u * a.kparts) + kg, ngroups - 1);
+                const int lrow = fast_div(gi, a.magic_go), xg = gi - lrow * a.Go;
+                const int gr = r0 + lrow, b = fast_div(gr, a.magic_ho), y = gr - b * a.Ho;
+                const int iy = y + ky - a.padU;
+                okA[u] = 2 * (ks0 + u * a.kparts) + kg < ngroups && iy >= 0 && iy < a.Hin;
+                okP[u] = xg > 0;
+                okN[u] = xg + 1 < a.Go;
+                A[u] = *reinterpret_cast<const uint4 *>(gy + (b * ysb + (unsigned)(y * a.Wo + xg * 8)));
+                const half_t *row = gx + (b * xsb + (unsigned)(min(max(iy, 0), a.Hin - 1) * a.Win + xg * 8));
+                C[u] = *reinterpret_cast<const uint4 *>(row);
+                p3[u] = *reinterpret_cast<const unsigned *>(row - (okP[u] ? 2 : 0));
+                n0[u] = *reinterpret_cast<const unsigned *>(row + (okN[u] ? 8 : 0));
+            }
+#pragma unroll
+            for (int u = 0; u < U; ++u) {
+                if (!okA[u]) A[u] = make_uint4(0, 0, 0, 0);
+                if (!okP[u]) p3[u] = 0;
+                if (!okN[u]) n0[u] = 0;
+                mfma_step<half_t>(acc[0], A[u], shifted_piece<0 - PADL>(C[u], p3[u], n0[u]));
+                mfma_step<half_t>(acc[1], A[u], shifted_piece<1 - PADL>(C[u], p3[u], n0[u]));
+                mfma_step<half_t>(acc[2], A[u], shifted_piece<2 - PADL>(C[u], p3[u], n0[u]));
+            }
+        }
+    }
+    // the shares of one (block, tap) side by side in LDS: [share][block][tap][32 filters][32 channels]
+    float *L = reinterpret_cast<float *>(smem);
+    if (active) {
+#pragma unroll
+        for (int kx = 0; kx < 3; ++kx) {
+            float *t = L + ((kpart * a.combos + combo) * 9 + ky * 3 + kx) * 1024 + lr;
+#pragma unroll
+            for (int v = 0; v < 16; ++v) t[(8 * (v >> 2) + 4 * kg + (v & 3)) * 32] = acc[kx][v];
+        }
+    }
+    __syncthreads();
+    float *out = a.ws + (size_t)wg * a.total;
+    const int cin9 = a.Cin * 9, share = a.combos * 9 * 1024;
+    for (int i = tid; i < a.total; i += CS_NT) {
+        const int o = fast_div(i, a.magic_cin9), rem = i - o * cin9;
+        const int c = (rem * 7282) >> 16, tap = rem - c * 9;  // rem / 9 for rem < 2^15
+        const float *src = L + (((o >> 5) * a.cbi_n + (c >> 5)) * 9 + tap) * 1024 + (o & 31) * 32 + (c & 31);
+        float sum = src[0];
+        for (int kp = 1; kp < a.kparts; ++kp) sum += src[kp * share];
+        out[i] = sum;
+    }
+}
+
+__device__ inline void wg_small_any(const WgSmallArgs &a, int wg, char *smem) {
+    if (a.padL == 1)
+        wg_small_block<1>(a, wg, smem);
+    else if (a.padL == 0)
+        wg_small_block<0>(a, wg, smem);
+    else
+        wg_small_block<2>(a, wg, smem);
+}
+
+__global__ __launch_bounds__(CS_NT) void wg_small_kernel(const WgSmallArgs a) {
+    extern __shared__ __attribute__((aligned(16))) char smem[];
+    wg_small_any(a, blockIdx.x, smem);
+}
+
 template <int CINP, int F_MAX>
-int launch_small(const ConvSmallArgs &a, int tiles, size_t lds, hipStream_t s) {
+__global__ __launch_bounds__(CS_NT) void conv_small_kernel(const ConvSmallArgs a) {
+    extern __shared__ __attribute__((aligned(16))) char smem[];
+    conv_small_block<CINP, F_MAX>(a, blockIdx.x, smem);
+}
+
+// Weight gradient and input gradient of one layer in one launch: the first workgroups take the weight gradient's
+// sample ranges (the longer jobs), the rest the input gradient's tiles.
+template <int CINP, int F_MAX>
+__global__ __launch_bounds__(CS_NT) void conv_small_bw_kernel(const ConvSmallArgs ig, const WgSmallArgs wg) {
+    extern __shared__ __attribute__((aligned(16))) char smem[];
+    if ((int)blockIdx.x < wg.nwg)
+        wg_small_any(wg, blockIdx.x, smem);
+    else
+        conv_small_block<CINP, F_MAX>(ig, blockIdx.x - wg.nwg, smem);
+}
+
+constexpr size_t WG_SMALL_LDS = 4 * 9 * 4096;  // shares x blocks <= 4 tiles of nine taps
+
+template <int CINP, int F_MAX>
+int launch_small(const ConvSmallArgs &a, int tiles, size_t lds, hipStream_t s, const WgSmallArgs *wg) {
     state().last_conv_resident = 2;
-    auto kern = conv_small_kernel<CINP, F_MAX>;
     static bool attr_set = false;
     if (!attr_set) {
-        if (!hip_ok(hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
+        if (!hip_ok(hipFuncSetAttribute(reinterpret_cast<const void *>(conv_small_kernel<CINP, F_MAX>),
+                                        hipFuncAttributeMaxDynamicSharedMemorySize, 150 * 1024),
+                    "hipFuncSetAttribute") ||
+            !hip_ok(hipFuncSetAttribute(reinterpret_cast<const void *>(conv_small_bw_kernel<CINP, F_MAX>),
                                         hipFuncAttributeMaxDynamicSharedMemorySize, 150 * 1024),
                     "hipFuncSetAttribute"))
             return 2;
         attr_set = true;
     }
-    hipLaunchKernelGGL(kern, dim3(tiles), dim3(CS_NT), lds, s, a);
+    if (wg)
+        hipLaunchKernelGGL((conv_small_bw_kernel<CINP, F_MAX>), dim3(tiles + wg->nwg), dim3(CS_NT),
+                           lds > WG_SMALL_LDS ? lds : WG_SMALL_LDS, s, a, *wg);
+    else
+        hipLaunchKernelGGL((conv_small_kernel<CINP, F_MAX>), dim3(tiles), dim3(CS_NT), lds, s, a);
     return hip_ok(hipGetLastError(), "small convolution launch") ? 0 : 2;
 }
 
-}  // namespace
+// dW[i] = sum over workgroups of ws[workgroup][i]: 64 outputs per workgroup of the reduction, 16 groups of
+// partials in parallel.
+__global__ __launch_bounds__(1024) void wg_small_reduce_kernel(const float *__restrict__ ws, half_t *__restrict__ dW,
+                                                               int total, int parts) {
+    __shared__ float part_sum[16][64];
+    const int o = threadIdx.x & 63, pg = threadIdx.x >> 6;
+    const int i = blockIdx.x * 64 + o;
+    float s = 0.f;
+    if (i < total) {  // (eight loads in flight per thread: the kernel lives on memory-level parallelism)
+        const float *src = ws + i;
+        int p = pg;
+        for (; p + 7 * 16 < parts; p += 8 * 16) {
+            float v[8];
+#pragma unroll
+            for (int u = 0; u < 8; ++u) v[u] = src[(size_t)(p + u * 16) * total];
+#pragma unroll
+            for (int u = 0; u < 8; ++u) s += v[u];
+        }
+        float v[8];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) v[u] = p + u * 16 < parts ? src[(size_t)(p + u * 16) * total] : 0.f;
+#pragma unroll
+        for (int u = 0; u < 8; ++u) s += v[u];
+    }
+    part_sum[pg][o] = s;
+    __syncthreads();
+    if (pg == 0 && i < total) {
+#pragma unroll
+        for (int q = 1; q < 16; ++q) s += part_sum[q][o];
+        dW[i] = (half_t)s;
+    }
+}
 
-int conv_small(const ConvTileDesc &d, const void *X, const void *Wt, void *Y) {
+struct SmallPlan {
+    ConvSmallArgs a;
+    int tiles, cinp, per_thread;
+    size_t lds;
+};
+
+// Fills the forward / input-gradient launch for `cu_budget` compute units; -1 when the layer does not fit.
+int plan_small(const ConvTileDesc &d, const void *X, const void *Wt, void *Y, int cu_budget, SmallPlan &p) {
     State &st = state();
     if (st.gemm_path != 0 && st.gemm_path != 6) return -1;  // (the other values select one of the other routes)
     if (d.in_hwc || d.KH != 3 || d.KW != 3 || d.sh != d.sw || d.sh < 1 || d.sh > 2) return -1;
@@ -206,7 +394,8 @@ int conv_small(const ConvTileDesc &d, const void *X, const void *Wt, void *Y) {
     if (reinterpret_cast<uintptr_t>(X) % 16 || reinterpret_cast<uintptr_t>(Wt) % 16) return -1;
     const long long f_elems = (long long)d.Cout * d.Cin * 9;
     if (f_elems % 8 != 0) return -1;
-    ConvSmallArgs a = {};
+    ConvSmallArgs &a = p.a;
+    a = ConvSmallArgs();
     // dense filter tensor [outer][inner][3][3]: forward (filter, channel), or the input gradient's view of it
     if (d.w_base == 0 && d.w_sm == d.Cin * 9 && d.w_sc == 9 && d.w_sy == 3 && d.w_sx == 1) {
         a.f_transposed = 0;
@@ -224,7 +413,7 @@ int conv_small(const ConvTileDesc &d, const void *X, const void *Wt, void *Y) {
     // rows per workgroup: the whole image, halved while that leaves the four waves a job each and the chip is not full
     int R = d.Ho;
     auto jobs_of = [&](int r) { return ((r * d.Wo + 31) / 32) * mblocks; };
-    while ((long long)d.batch * ((d.Ho + R - 1) / R) < st.num_cu && R % 2 == 0 && jobs_of(R / 2) >= 4) R /= 2;
+    while ((long long)d.batch * ((d.Ho + R - 1) / R) < cu_budget && R % 2 == 0 && jobs_of(R / 2) >= 4) R /= 2;
     auto items_of = [&](int r) { return cblocks * (d.Win / 8) * ((((r - 1) * s + 3) + 7) / 8); };
     auto lds_of = [&](int r) { return (size_t)cblocks * ((r - 1) * s + 3) * TW * 16; };
     const int pitch = 9 * cinp * 2 + 16;
@@ -260,22 +449,99 @@ int conv_small(const ConvTileDesc &d, const void *X, const void *Wt, void *Y) {
     a.b_pitch = pitch; a.f_bytes = (int)f_bytes;
     a.pgroups = (R * d.Wo + 31) / 32; a.mshift = mblocks - 1;
     if (f_elems >= 65536 || a.f_inner * 9 >= 65536) return -1;  // (quotients by reciprocal multiplication)
-    const size_t lds = f_bytes + lds_of(R);
-    const int per_thread = (a.f_chunks + CS_NT - 1) / CS_NT;
     if (a.halo_chunks >= 65536 || a.RR * cblocks >= 65536) return -1;
-    if (cinp == 16) {
-        if (per_thread <= 1) return launch_small<16, 1>(a, (int)tiles, lds, st.stream);
-        if (per_thread <= 2) return launch_small<16, 2>(a, (int)tiles, lds, st.stream);
-        return -1;
+    p.tiles = (int)tiles;
+    p.lds = f_bytes + lds_of(R);
+    p.cinp = cinp;
+    p.per_thread = (a.f_chunks + CS_NT - 1) / CS_NT;
+    if (p.per_thread > (cinp == 16 ? 2 : cinp == 32 ? 3 : 5)) return -1;
+    return 0;
+}
+
+int dispatch_small(const SmallPlan &p, const WgSmallArgs *wg) {
+    hipStream_t s = state().stream;
+    if (p.cinp == 16)
+        return p.per_thread <= 1 ? launch_small<16, 1>(p.a, p.tiles, p.lds, s, wg) : launch_small<16, 2>(p.a, p.tiles, p.lds, s, wg);
+    if (p.cinp == 32)
+        return p.per_thread <= 2 ? launch_small<32, 2>(p.a, p.tiles, p.lds, s, wg) : launch_small<32, 3>(p.a, p.tiles, p.lds, s, wg);
+    return p.per_thread <= 3 ? launch_small<64, 3>(p.a, p.tiles, p.lds, s, wg) : launch_small<64, 5>(p.a, p.tiles, p.lds, s, wg);
+}
+
+// Fills the weight-gradient launch of the forward layer `d` (partial sums in the workspace); -1 when it does not fit.
+int plan_wg(const ConvTileDesc &d, const void *X, const void *dY, int max_wg, WgSmallArgs &w) {
+    State &st = state();
+    if (st.gemm_path != 6) return -1;  // (on request only: lane-per-channel loads keep the address unit busy 64 cycles each)
+    if (d.in_hwc || d.KH != 3 || d.KW != 3 || d.sh != 1 || d.sw != 1) return -1;
+    if (d.Cin > 64 || d.Cout > 64 || d.Win % 8 != 0 || d.Wo != d.Win || d.x_sy != d.Win) return -1;
+    if (d.x_sc != (long long)d.Hin * d.Win || d.x_sb != (long long)d.Cin * d.Hin * d.Win) return -1;
+    if (d.padU < 0 || d.padL < 0 || d.padL > 2) return -1;
+    if (reinterpret_cast<uintptr_t>(X) % 16 || reinterpret_cast<uintptr_t>(dY) % 16) return -1;
+    w = WgSmallArgs();
+    w.total = d.Cout * d.Cin * 9;
+    const long long positions = (long long)d.batch * d.Ho * d.Wo;
+    // large calls keep the tiled weight-gradient kernels (measured ahead from about a quarter of a million positions)
+    if (st.gemm_path != 6 && positions > 262144) return -1;
+    // workgroups: as many as keep the partial sums within 2 MB, at most `max_wg`, whole output rows each
+    long long nwg_max = (2LL << 20) / ((long long)w.total * 4);
+    nwg_max = nwg_max < 1 ? 1 : nwg_max > max_wg ? max_wg : nwg_max;
+    const long long rows = (long long)d.batch * d.Ho;
+    w.rows_per_wg = (int)((rows + nwg_max - 1) / nwg_max);
+    w.nwg = (int)((rows + w.rows_per_wg - 1) / w.rows_per_wg);
+    w.Go = d.Wo / 8;
+    if (rows >= 65536 || (long long)w.rows_per_wg * w.Go + 16 >= 65536 || w.total >= 65536) return -1;  // (reciprocal multiplication)
+    w.magic_go = magic_of(w.Go);
+    w.magic_ho = magic_of(d.Ho);
+    w.magic_cin9 = magic_of(d.Cin * 9);
+    w.cbi_n = (d.Cin + 31) / 32;
+    w.combos = w.cbi_n * ((d.Cout + 31) / 32);
+    w.kparts = 4 / w.combos;
+    w.X = reinterpret_cast<const half_t *>(X);
+    w.dY = reinterpret_cast<const half_t *>(dY);
+    w.batch = d.batch; w.Cin = d.Cin; w.Cout = d.Cout; w.Hin = d.Hin; w.Win = d.Win; w.Ho = d.Ho; w.Wo = d.Wo;
+    w.padU = d.padU; w.padL = d.padL;
+    w.ws = workspace((size_t)w.nwg * w.total * sizeof(float));
+    return w.ws ? 0 : 2;
+}
+
+int reduce_wg(const WgSmallArgs &w, void *dW) {
+    hipLaunchKernelGGL(wg_small_reduce_kernel, dim3((w.total + 63) / 64), dim3(1024), 0, state().stream, w.ws,
+                       reinterpret_cast<half_t *>(dW), w.total, w.nwg);
+    return hip_ok(hipGetLastError(), "small weight gradient reduction launch") ? 0 : 2;
+}
+
+}  // namespace
+
+int conv_small(const ConvTileDesc &d, const void *X, const void *Wt, void *Y) {
+    SmallPlan p;
+    if (int rc = plan_small(d, X, Wt, Y, state().num_cu, p)) return rc;
+    return dispatch_small(p, nullptr);
+}
+
+int conv_small_wg(const ConvTileDesc &d, const void *X, const void *dY, void *dW) {
+    WgSmallArgs w;
+    if (int rc = plan_wg(d, X, dY, state().num_cu, w)) return rc;
+    static bool attr_set = false;
+    if (!attr_set) {
+        if (!hip_ok(hipFuncSetAttribute(reinterpret_cast<const void *>(wg_small_kernel),
+                                        hipFuncAttributeMaxDynamicSharedMemorySize, 150 * 1024),
+                    "hipFuncSetAttribute"))
+            return 2;
+        attr_set = true;
     }
-    if (cinp == 32) {
-        if (per_thread <= 2) return launch_small<32, 2>(a, (int)tiles, lds, st.stream);
-        if (per_thread <= 3) return launch_small<32, 3>(a, (int)tiles, lds, st.stream);
-        return -1;
-    }
-    if (per_thread <= 3) return launch_small<64, 3>(a, (int)tiles, lds, st.stream);
-    if (per_thread <= 5) return launch_small<64, 5>(a, (int)tiles, lds, st.stream);
-    return -1;
+    hipLaunchKernelGGL(wg_small_kernel, dim3(w.nwg), dim3(CS_NT), WG_SMALL_LDS, state().stream, w);
+    if (!hip_ok(hipGetLastError(), "small weight gradient launch")) return 2;
+    return reduce_wg(w, dW);
+}
+
+int conv_small_bw(const ConvTileDesc &fwd, const ConvTileDesc &ig, const void *X, const void *dY, const void *Wt,
+                  void *dW, void *dX) {
+    WgSmallArgs w;
+    if (int rc = plan_wg(fwd, X, dY, state().num_cu / 2, w)) return rc;
+    SmallPlan p;
+    const int budget = state().num_cu - w.nwg;
+    if (int rc = plan_small(ig, dY, Wt, dX, budget > 32 ? budget : 32, p)) return rc;
+    if (int rc = dispatch_small(p, &w)) return rc;
+    return reduce_wg(w, dW);
 }
 
 }  // namespace ptl

@@ -30,6 +30,11 @@ int conv_tile(const ConvTileDesc &d, const void *X, const void *Wt, void *Y, con
 // caller's tensors directly (ptl_conv_small.hip).  Y is the dense channel-major output [batch][Cout][Ho][Wo].
 // Returns -1 when the layer does not fit or is large enough for the persistent kernels to be ahead.
 int conv_small(const ConvTileDesc &d, const void *X, const void *Wt, void *Y);
+// Weight gradient of such a layer (unit stride, output as wide as the input), and weight + input gradient with the
+// two products in one launch (`fwd` describes the forward layer, `ig` the input gradient as a forward pass over dY).
+int conv_small_wg(const ConvTileDesc &d, const void *X, const void *dY, void *dW);
+int conv_small_bw(const ConvTileDesc &fwd, const ConvTileDesc &ig, const void *X, const void *dY, const void *Wt,
+                  void *dW, void *dX);
 
 }  // namespace ptl
 

@@ -443,54 +443,58 @@ __global__ __launch_bounds__(256) void bn_sums_kernel(const T *__restrict__ x, c
                                                       int vec, const BnFuse<T> f = BnFuse<T>()) {
     __shared__ float red[BN_SUMS][4];
     const int c = blockIdx.x, grp = blockIdx.y, tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    const int b0 = grp * per_group, b1 = min(B, b0 + per_group);
+    // the group's planes of this channel as one index range: element i = (sample i / HW, position i % HW), so that
+    // small planes still keep every thread busy
+    const int b0 = grp * per_group, nb = min(B, b0 + per_group) - b0;
+    const int total = nb * HW;
     constexpr int VEC = 16 / (int)sizeof(T);
     float s[BN_SUMS] = {0.f, 0.f, 0.f, 0.f};
-    for (int b = b0; b < b1; ++b) {
-        const size_t base = ((size_t)b * C + c) * HW;
-        if (vec) {  // planes are whole 16-byte vectors
-            for (int e = tid * VEC; e < HW; e += 256 * VEC) {
-                BnVec<T> xv, gv;
-                xv.raw = *reinterpret_cast<const uint4 *>(x + base + e);
-                if (BW) gv.raw = *reinterpret_cast<const uint4 *>(dy + base + e);
-                if (BW && FUSED) {
-                    BnVec<T> g2, ov;
-                    if (f.dy2) {
-                        g2.raw = *reinterpret_cast<const uint4 *>(f.dy2 + base + e);
+    if (vec) {  // planes are whole 16-byte vectors
+        for (int i = tid * VEC; i < total; i += 256 * VEC) {
+            const int bl = i / HW, e = i - bl * HW;
+            const size_t at = ((size_t)(b0 + bl) * C + c) * HW + e;
+            BnVec<T> xv, gv;
+            xv.raw = *reinterpret_cast<const uint4 *>(x + at);
+            if (BW) gv.raw = *reinterpret_cast<const uint4 *>(dy + at);
+            if (BW && FUSED) {
+                BnVec<T> g2, ov;
+                if (f.dy2) {
+                    g2.raw = *reinterpret_cast<const uint4 *>(f.dy2 + at);
 #pragma unroll
-                        for (int q = 0; q < VEC; ++q) gv.e[q] = (T)((float)gv.e[q] + (float)g2.e[q]);
-                    }
-                    if (f.relu) {
-                        ov.raw = *reinterpret_cast<const uint4 *>(f.out + base + e);
-#pragma unroll
-                        for (int q = 0; q < VEC; ++q) gv.e[q] = (float)ov.e[q] > 0.f ? gv.e[q] : (T)0;
-                    }
-                    if (f.gout) *reinterpret_cast<uint4 *>(f.gout + base + e) = gv.raw;
+                    for (int q = 0; q < VEC; ++q) gv.e[q] = (T)((float)gv.e[q] + (float)g2.e[q]);
                 }
+                if (f.relu) {
+                    ov.raw = *reinterpret_cast<const uint4 *>(f.out + at);
 #pragma unroll
-                for (int q = 0; q < VEC; ++q) {
-                    const float v = (float)xv.e[q];
-                    s[0] += v;
-                    s[1] += v * v;
-                    if (BW) {
-                        const float g = (float)gv.e[q];
-                        s[2] += g;
-                        s[3] += g * v;
-                    }
+                    for (int q = 0; q < VEC; ++q) gv.e[q] = (float)ov.e[q] > 0.f ? gv.e[q] : (T)0;
+                }
+                if (f.gout) *reinterpret_cast<uint4 *>(f.gout + at) = gv.raw;
+            }
+#pragma unroll
+            for (int q = 0; q < VEC; ++q) {
+                const float v = (float)xv.e[q];
+                s[0] += v;
+                s[1] += v * v;
+                if (BW) {
+                    const float g = (float)gv.e[q];
+                    s[2] += g;
+                    s[3] += g * v;
                 }
             }
-            continue;
         }
-        for (int e = tid; e < HW; e += 256) {
-            const float v = (float)x[base + e];
+    } else {
+        for (int i = tid; i < total; i += 256) {
+            const int bl = i / HW, e = i - bl * HW;
+            const size_t at = ((size_t)(b0 + bl) * C + c) * HW + e;
+            const float v = (float)x[at];
             s[0] += v;
             s[1] += v * v;
             if (BW) {
-                T gt = dy[base + e];
+                T gt = dy[at];
                 if (FUSED) {
-                    if (f.dy2) gt = (T)((float)gt + (float)f.dy2[base + e]);
-                    if (f.relu && !((float)f.out[base + e] > 0.f)) gt = (T)0;
-                    if (f.gout) f.gout[base + e] = gt;
+                    if (f.dy2) gt = (T)((float)gt + (float)f.dy2[at]);
+                    if (f.relu && !((float)f.out[at] > 0.f)) gt = (T)0;
+                    if (f.gout) f.gout[at] = gt;
                 }
                 const float g = (float)gt;
                 s[2] += g;
@@ -626,8 +630,7 @@ static int batch_norm_step(const Args *a, int bw, const char *fn, const Fusion *
     const size_t n = (size_t)B * C * HW;
     if ((size_t)B * C >= ((size_t)1 << 31)) return glue_bad(fn, "too many planes");
     // groups of samples: about four workgroups per CU in the first kernel
-    static const int mult = getenv("PTL_BN_MULT") ? atoi(getenv("PTL_BN_MULT")) : 4;
-    int groups = (mult * st.num_cu + C - 1) / C;
+    int groups = (4 * st.num_cu + C - 1) / C;
     if (groups > 64) groups = 64;  // the second kernel folds them with one wave
     if (groups > B) groups = B;
     const int per_group = (B + groups - 1) / groups;

@@ -362,6 +362,8 @@ static int conv2d_wg(const Args *a, int ns, const char *fn) {
                                 (long long)ns * g.Ho * g.Wo >= 16384;
         if (g.hwc) {  // channel-minor tensors: the sum over taps from 64 channels on, else the gathering GEMM below
             rc = conv_taps_wg<T>(d, X, dY, dW);
+        } else if (sizeof(T) == 2 && (rc = conv_small_wg(d, X, dY, dW)) >= 0) {
+            // (small 3x3 layers: one launch for the partial sums over sample ranges, one to add them)
         } else {
             const bool tiles_resident = sizeof(T) == 2 && state().gemm_path == 0 && conv_halo_wg_preferred(d);
             if (state().gemm_path == 3 || state().gemm_path == 5 || tiles_resident || (taps_first && state().gemm_path != 2))
@@ -619,13 +621,14 @@ static int conv2d_bw(const Args *a, int ns, const char *fn) {
         return 1;
     }
     const bool wg = a->skip_wg_grad == 0, ig = a->skip_in_grad == 0;
-    if (wg && ig && sizeof(T) == 2 && a->USE_BIASES != 1 && ns > 1 && a->input && a->coeff && a->output) {
+    if (wg && ig && sizeof(T) == 2 && a->USE_BIASES != 1 && ns >= 1 && a->input && a->coeff && a->output) {
         ConvGeom g;
         if (int rc = conv_geom(a, g, fn, true)) return rc;
         const int P = g.Ho * g.Wo, Pk = g.Hk * g.Wk, K = g.Ci * Pk;
         size_t in_n = (size_t)ns * g.Ci * g.H * g.W, out_n = (size_t)ns * g.Co * P;
         if (!g.hwc && g.Hk == 3 && g.Wk == 3 && g.sh == 1 && g.sw == 1 && g.Up + g.Dp == 2 && g.Lp + g.Rp == 2 &&
-            fits_int(in_n) && fits_int(out_n) && (state().gemm_path == 0 || state().gemm_path == 5)) {
+            fits_int(in_n) && fits_int(out_n) &&
+            (state().gemm_path == 0 || state().gemm_path == 5 || state().gemm_path == 6)) {
             if (!ensure_init()) return 2;
             ConvTileDesc f = {}, b = {};
             f.batch = ns; f.Cin = g.Ci; f.Hin = g.H; f.Win = g.W;
@@ -640,7 +643,10 @@ static int conv2d_bw(const Args *a, int ns, const char *fn) {
             b.padD = g.H + 2 - g.Ho - b.padU; b.padR = g.W + 2 - g.Wo - b.padL;
             b.x_sb = (long long)g.Co * P; b.x_sc = P; b.x_sy = g.Wo;
             b.w_base = Pk - 1; b.w_sm = Pk; b.w_sc = g.Ci * Pk; b.w_sy = -g.Wk; b.w_sx = -1;
-            if (conv_halo_wg_preferred(f)) {
+            // small layers: both products in one launch; wide layers: one shared copy of the output gradient
+            const bool small = g.Ci <= 64 && g.Co <= 64 && g.W % 8 == 0 && state().gemm_path != 5;
+            const bool wide = ns > 1 && state().gemm_path != 6 && conv_halo_wg_preferred(f);
+            if (small || wide) {
                 Stager sg;
                 const T *X = sg.in(reinterpret_cast<const T *>(a->input->data), in_n);
                 const T *dY = sg.in(reinterpret_cast<const T *>(a->output->diff), out_n);
@@ -650,7 +656,8 @@ static int conv2d_bw(const Args *a, int ns, const char *fn) {
                 if (sg.failed()) return 2;
                 state().last_conv_direct = 0;
                 state().last_conv_resident = 0;
-                const int rc = conv_halo_bw<T>(f, b, X, dY, Wt, dW, dX);
+                int rc = small ? conv_small_bw(f, b, X, dY, Wt, dW, dX) : -1;
+                if (rc < 0 && wide) rc = conv_halo_bw<T>(f, b, X, dY, Wt, dW, dX);
                 if (rc >= 0) {
                     if (rc == 0) state().last_conv_direct = 1;
                     return sg.finish(rc);
