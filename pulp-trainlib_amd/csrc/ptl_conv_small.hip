@@ -179,19 +179,28 @@ __device__ inline void conv_small_block(const ConvSmallArgs &a, int tile, char *
 
 // ---- Weight gradient of the same layers (unit stride, output rows as wide as input rows) -----------------------
 // dW(co, ci, ky, kx) = sum over positions of dY(co, p) * X(ci, p + tap shift): the contraction runs over positions,
-// which are contiguous in both channel-major tensors, so both MFMA operands are 16-byte pieces straight from global
-// memory (rows = filters, columns = channels, k = 8 consecutive output columns per lane half); the three column taps
-// of a filter row are the input piece shifted by whole elements in registers (its neighbours' edge dwords are loaded
-// beside it), rows and columns outside the image read as zeros.  A workgroup owns a range of output rows; its waves are
-// (filter row ky) x (32x32 block of the weight tensor) x (share of the positions); the shares are added through LDS
-// and the workgroup's partial sums go to ws[workgroup][co][ci][tap]; a second launch adds the workgroups.
+// which are contiguous in both channel-major tensors, so the MFMA operands (rows = filters, columns = channels,
+// k = 8 consecutive output columns per lane half) are 16-byte pieces of the tensors as they lie in memory.  A lane per
+// channel reading them from global memory keeps the address unit busy 64 cycles per load (one cache line per lane),
+// so a workgroup first copies its tile - S samples x R output rows, every channel of the gradient and of the input
+// with one row of halo above and below - into LDS with coalesced 16-byte loads, input rows separated by 8 zero
+// elements (the left and right padding of neighbouring rows), rows outside the image as zeros.  Its waves are
+// (filter row ky) x (32x32 block of the weight tensor) x (share of the positions); per k step a wave reads the
+// gradient piece, the input piece and the input's two edge dwords, forms the three column taps by shifting whole
+// elements in registers and issues three MFMAs.  The shares are added through LDS and the workgroup's partial sums go
+// to ws[workgroup][co][ci][tap]; a second launch adds the workgroups.
+constexpr int WG_CHUNKS = 4;  // 16-byte pieces per thread and tensor, at most
+
 struct WgSmallArgs {
     const half_t *X, *dY;
     float *ws;
-    int batch, Cin, Cout, Hin, Win, Ho, Wo, padU, padL;
-    int nwg, rows_per_wg;  // workgroups, output rows (sample * Ho + row) per workgroup
-    int Go;                // 8-column groups per output row
-    unsigned magic_go, magic_ho, magic_cin9;
+    int batch, Cin, Cout, Hin, Win, Ho, padU, padL;
+    int nwg, S, R, tiles_per_img;  // workgroups; samples and output rows per tile (R = Ho when S > 1)
+    int G, RG, R2G;                // 8-column groups per row, per R rows, per R + 2 rows
+    int PY, PX, WP;                // LDS pitches in elements: gradient channel, input channel, input row
+    int groups;                    // S * R * G
+    int y_chunks, x_chunks, pad_chunks, pad_rows;  // pieces to copy; zero pieces (one per input row + one) and rows per channel
+    unsigned magic_g, magic_rg, magic_r2g, magic_ychan, magic_xchan, magic_padrows, magic_cin9;
     int cbi_n, combos, kparts;  // 32-channel blocks, (filter block, channel block) pairs, position shares
     int total;                  // Cout * Cin * 9
 };
@@ -213,59 +222,99 @@ __device__ inline uint4 shifted_piece(const uint4 &c, unsigned p3, unsigned n0) 
 template <int PADL>
 __device__ inline void wg_small_block(const WgSmallArgs &a, int wg, char *smem) {
     const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    half_t *Ys = reinterpret_cast<half_t *>(smem);
+    half_t *Xs = Ys + a.Cout * a.PY;
+    // the tile: samples b0 .. b0 + S - 1, output rows y0 .. y0 + R - 1
+    const int timg = wg / a.tiles_per_img;
+    const int b0 = timg * a.S, y0 = (wg - timg * a.tiles_per_img) * a.R;
+
+    // ---- copy: all loads first, then the LDS writes
+    uint4 yv[WG_CHUNKS], xv[WG_CHUNKS];
+    const int ychan = a.groups, xchan = a.S * a.R2G;  // pieces per channel
+#pragma unroll
+    for (int k = 0; k < WG_CHUNKS; ++k) {
+        const int q = tid + CS_NT * k;
+        yv[k] = xv[k] = make_uint4(0, 0, 0, 0);
+        if (q < a.y_chunks) {
+            const int co = fast_div(q, a.magic_ychan), rem = q - co * ychan;
+            const int s = fast_div(rem, a.magic_rg), r2 = rem - s * a.RG;
+            const int ly = fast_div(r2, a.magic_g), xg = r2 - ly * a.G;
+            if (b0 + s < a.batch && y0 + ly < a.Ho)
+                yv[k] = *reinterpret_cast<const uint4 *>(a.dY + (((size_t)(b0 + s) * a.Cout + co) * a.Ho + y0 + ly) * a.Win + 8 * xg);
+        }
+        if (q < a.x_chunks) {
+            const int ci = fast_div(q, a.magic_xchan), rem = q - ci * xchan;
+            const int s = fast_div(rem, a.magic_r2g), r2 = rem - s * a.R2G;
+            const int ly = fast_div(r2, a.magic_g), xg = r2 - ly * a.G;
+            const int iy = y0 - a.padU + ly;
+            if (b0 + s < a.batch && iy >= 0 && iy < a.Hin)
+                xv[k] = *reinterpret_cast<const uint4 *>(a.X + (((size_t)(b0 + s) * a.Cin + ci) * a.Hin + iy) * a.Win + 8 * xg);
+        }
+    }
+    // zero pieces: in front of every input row and behind the last one; behind the last gradient group
+    for (int q = tid; q < a.pad_chunks; q += CS_NT) {
+        const int ci = fast_div(q, a.magic_padrows), row = q - ci * a.pad_rows;
+        *reinterpret_cast<uint4 *>(Xs + ci * a.PX + row * a.WP) = make_uint4(0, 0, 0, 0);
+    }
+    for (int co = tid; co < a.Cout; co += CS_NT)
+        *reinterpret_cast<uint4 *>(Ys + co * a.PY + a.groups * 8) = make_uint4(0, 0, 0, 0);
+#pragma unroll
+    for (int k = 0; k < WG_CHUNKS; ++k) {
+        const int q = tid + CS_NT * k;
+        if (q < a.y_chunks) {
+            const int co = fast_div(q, a.magic_ychan), rem = q - co * ychan;
+            *reinterpret_cast<uint4 *>(Ys + co * a.PY + rem * 8) = yv[k];
+        }
+        if (q < a.x_chunks) {
+            const int ci = fast_div(q, a.magic_xchan), rem = q - ci * xchan;
+            const int row = fast_div(rem, a.magic_g), xg = rem - row * a.G;  // row = s * (R + 2) + ly
+            *reinterpret_cast<uint4 *>(Xs + ci * a.PX + row * a.WP + 8 + 8 * xg) = xv[k];
+        }
+    }
+    __syncthreads();
+
+    // ---- products
     const int ky = wave % 3, rest = wave / 3;
     const int combo = rest % a.combos, kpart = rest / a.combos;
     const bool active = wave < 15 && kpart < a.kparts;
     const int cbo = combo / a.cbi_n, cbi = combo - cbo * a.cbi_n;
     const int lr = lane & 31, kg = lane >> 5;
-    const int co = cbo * 32 + lr, ci = cbi * 32 + lr;
-    // this workgroup's rows of the output (sample * Ho + row), as groups of 8 columns, two groups per k step
-    const int r0 = wg * a.rows_per_wg, nrows = min(a.rows_per_wg, a.batch * a.Ho - r0);
-    const int ngroups = nrows * a.Go, nks = (ngroups + 1) >> 1;
+    const int nks = (a.groups + 1) >> 1;
     f32x16 acc[3];
 #pragma unroll
     for (int kx = 0; kx < 3; ++kx)
 #pragma unroll
         for (int v = 0; v < 16; ++v) acc[kx][v] = 0.f;
     if (active) {
-        // Every load is executed by every lane from an address inside the tensors (filters and channels beyond the
-        // tensors repeat the last one: their rows and columns of the product are never stored; rows above or below
-        // the image are clamped into it), and what must read as zero is masked afterwards: the gradient piece where
-        // the group is beyond the range or the input row is outside the image, the edge dwords at the row ends.
-        const half_t *gy = a.dY + (unsigned)(min(co, a.Cout - 1) * a.Ho * a.Wo);
-        const half_t *gx = a.X + (unsigned)(min(ci, a.Cin - 1) * a.Hin * a.Win);
-        const unsigned ysb = (unsigned)(a.Cout * a.Ho * a.Wo), xsb = (unsigned)(a.Cin * a.Hin * a.Win);
-        constexpr int U = 4;  // k steps whose loads are in flight together
+        // filters and channels beyond the tensors repeat the last one (their rows and columns are never stored)
+        const half_t *yrow = Ys + min(cbo * 32 + lr, a.Cout - 1) * a.PY;
+        const half_t *xrow = Xs + min(cbi * 32 + lr, a.Cin - 1) * a.PX + ky * a.WP + 8;
+        constexpr int U = 4;  // k steps whose LDS reads are in flight together
         for (int ks0 = kpart; ks0 < nks; ks0 += U * a.kparts) {
             uint4 A[U], C[U];
             unsigned p3[U], n0[U];
-            bool okA[U], okP[U], okN[U];
 #pragma unroll
             for (int u = 0; u < U; ++u) {
-                const int gi = min(2 * (ks0 + u * a.kparts) + kg, ngroups - 1);
-                const int lrow = fast_div(gi, a.magic_go), xg = gi - lrow * a.Go;
-                const int gr = r0 + lrow, b = fast_div(gr, a.magic_ho), y = gr - b * a.Ho;
-                const int iy = y + ky - a.padU;
-                okA[u] = 2 * (ks0 + u * a.kparts) + kg < ngroups && iy >= 0 && iy < a.Hin;
-                okP[u] = xg > 0;
-                okN[u] = xg + 1 < a.Go;
-                A[u] = *reinterpret_cast<const uint4 *>(gy + (b * ysb + (unsigned)(y * a.Wo + xg * 8)));
-                const half_t *row = gx + (b * xsb + (unsigned)(min(max(iy, 0), a.Hin - 1) * a.Win + xg * 8));
-                C[u] = *reinterpret_cast<const uint4 *>(row);
-                p3[u] = *reinterpret_cast<const unsigned *>(row - (okP[u] ? 2 : 0));
-                n0[u] = *reinterpret_cast<const unsigned *>(row + (okN[u] ? 8 : 0));
+                // (steps behind the last one read the zero piece of the gradient)
+                const int gi = min(2 * (ks0 + u * a.kparts) + kg, a.groups);
+                const int gx = min(gi, a.groups - 1);
+                const int s = fast_div(gx, a.magic_rg), r2 = gx - s * a.RG;
+                const int ly = fast_div(r2, a.magic_g), xg = r2 - ly * a.G;
+                const half_t *xp = xrow + (s * (a.R + 2) + ly) * a.WP + 8 * xg;
+                A[u] = *reinterpret_cast<const uint4 *>(yrow + gi * 8);
+                C[u] = *reinterpret_cast<const uint4 *>(xp);
+                p3[u] = *reinterpret_cast<const unsigned *>(xp - 2);
+                n0[u] = *reinterpret_cast<const unsigned *>(xp + 8);
             }
 #pragma unroll
             for (int u = 0; u < U; ++u) {
-                if (!okA[u]) A[u] = make_uint4(0, 0, 0, 0);
-                if (!okP[u]) p3[u] = 0;
-                if (!okN[u]) n0[u] = 0;
                 mfma_step<half_t>(acc[0], A[u], shifted_piece<0 - PADL>(C[u], p3[u], n0[u]));
                 mfma_step<half_t>(acc[1], A[u], shifted_piece<1 - PADL>(C[u], p3[u], n0[u]));
                 mfma_step<half_t>(acc[2], A[u], shifted_piece<2 - PADL>(C[u], p3[u], n0[u]));
             }
         }
     }
+    __syncthreads();  // the tiles are dead: the shares take their place
     // the shares of one (block, tap) side by side in LDS: [share][block][tap][32 filters][32 channels]
     float *L = reinterpret_cast<float *>(smem);
     if (active) {
@@ -468,9 +517,9 @@ int dispatch_small(const SmallPlan &p, const WgSmallArgs *wg) {
 }
 
 // Fills the weight-gradient launch of the forward layer `d` (partial sums in the workspace); -1 when it does not fit.
-int plan_wg(const ConvTileDesc &d, const void *X, const void *dY, int max_wg, WgSmallArgs &w) {
+int plan_wg(const ConvTileDesc &d, const void *X, const void *dY, int max_wg, bool alone, WgSmallArgs &w) {
     State &st = state();
-    if (st.gemm_path != 6) return -1;  // (on request only: lane-per-channel loads keep the address unit busy 64 cycles each)
+    if (st.gemm_path != 0 && st.gemm_path != 6) return -1;  // (the other values select one of the other routes)
     if (d.in_hwc || d.KH != 3 || d.KW != 3 || d.sh != 1 || d.sw != 1) return -1;
     if (d.Cin > 64 || d.Cout > 64 || d.Win % 8 != 0 || d.Wo != d.Win || d.x_sy != d.Win) return -1;
     if (d.x_sc != (long long)d.Hin * d.Win || d.x_sb != (long long)d.Cin * d.Hin * d.Win) return -1;
@@ -478,26 +527,58 @@ int plan_wg(const ConvTileDesc &d, const void *X, const void *dY, int max_wg, Wg
     if (reinterpret_cast<uintptr_t>(X) % 16 || reinterpret_cast<uintptr_t>(dY) % 16) return -1;
     w = WgSmallArgs();
     w.total = d.Cout * d.Cin * 9;
+    if (w.total >= 65536) return -1;
     const long long positions = (long long)d.batch * d.Ho * d.Wo;
-    // large calls keep the tiled weight-gradient kernels (measured ahead from about a quarter of a million positions)
-    if (st.gemm_path != 6 && positions > 262144) return -1;
-    // workgroups: as many as keep the partial sums within 2 MB, at most `max_wg`, whole output rows each
-    long long nwg_max = (2LL << 20) / ((long long)w.total * 4);
-    nwg_max = nwg_max < 1 ? 1 : nwg_max > max_wg ? max_wg : nwg_max;
-    const long long rows = (long long)d.batch * d.Ho;
-    w.rows_per_wg = (int)((rows + nwg_max - 1) / nwg_max);
-    w.nwg = (int)((rows + w.rows_per_wg - 1) / w.rows_per_wg);
-    w.Go = d.Wo / 8;
-    if (rows >= 65536 || (long long)w.rows_per_wg * w.Go + 16 >= 65536 || w.total >= 65536) return -1;  // (reciprocal multiplication)
-    w.magic_go = magic_of(w.Go);
-    w.magic_ho = magic_of(d.Ho);
+    // large calls keep the tiled weight-gradient kernels; so do calls for the weight gradient alone from 32 channels
+    // on (measured 14.7 against 13.7 us for 32 -> 32 on 16x16 at batch 128, 9.7 against 11.5 us for 3 -> 16 on 32x32:
+    // what this kernel buys is the input gradient riding along in the same launch)
+    if (st.gemm_path != 6 && (positions > 262144 || (alone && (d.Cin > 16 || d.Cout > 16 || d.batch < 32)))) return -1;
+    w.G = d.Win / 8;
+    w.WP = d.Win + 8;
+    auto round_pitch = [](int n) { return n + ((8 - n % 64) + 64) % 64; };  // = 8 mod 64: rows 16 bytes apart in the banks
+    auto lds_of = [&](int S, int R) {
+        const int py = round_pitch(S * R * d.Win + 8), px = round_pitch((S * (R + 2) + 1) * w.WP);
+        return ((size_t)d.Cout * py + (size_t)d.Cin * px) * 2;
+    };
+    auto chunks_ok = [&](int S, int R) {
+        return (long long)d.Cout * S * R * w.G <= WG_CHUNKS * CS_NT && (long long)d.Cin * S * (R + 2) * w.G <= WG_CHUNKS * CS_NT &&
+               lds_of(S, R) <= WG_SMALL_LDS;
+    };
+    // tiles: whole samples while the partial sums stay within about 5 MB (S samples each otherwise), rows of a
+    // sample split while that fills more of `max_wg` workgroups and leaves the waves eight k steps each
+    int S = 1, R = d.Ho;
+    while ((long long)((d.batch + S - 1) / S) * w.total * 4 > (5LL << 20) && chunks_ok(S * 2, R)) S *= 2;
+    if (S == 1)
+        while (R % 2 == 0 && (long long)d.batch * (d.Ho / R) * 2 <= max_wg && (R / 2) * w.G >= 16 &&
+               (long long)d.batch * (d.Ho / R) * 2 * w.total * 4 <= (5LL << 20))
+            R /= 2;
+    while (!chunks_ok(S, R) && R % 2 == 0 && S == 1) R /= 2;
+    if (!chunks_ok(S, R)) return -1;
+    w.S = S; w.R = R;
+    w.tiles_per_img = (d.Ho + R - 1) / R;
+    w.nwg = ((d.batch + S - 1) / S) * w.tiles_per_img;
+    w.RG = R * w.G; w.R2G = (R + 2) * w.G;
+    w.groups = S * w.RG;
+    w.PY = round_pitch(w.groups * 8 + 8);
+    w.pad_rows = S * (R + 2) + 1;
+    w.PX = round_pitch(w.pad_rows * w.WP);
+    w.y_chunks = d.Cout * w.groups;
+    w.x_chunks = d.Cin * S * w.R2G;
+    w.pad_chunks = d.Cin * w.pad_rows;
+    if (w.y_chunks >= 65536 || w.x_chunks >= 65536 || w.pad_chunks >= 65536) return -1;  // (reciprocal multiplication)
+    w.magic_g = magic_of(w.G);
+    w.magic_rg = magic_of(w.RG);
+    w.magic_r2g = magic_of(w.R2G);
+    w.magic_ychan = magic_of(w.groups);
+    w.magic_xchan = magic_of(S * w.R2G);
+    w.magic_padrows = magic_of(w.pad_rows);
     w.magic_cin9 = magic_of(d.Cin * 9);
     w.cbi_n = (d.Cin + 31) / 32;
     w.combos = w.cbi_n * ((d.Cout + 31) / 32);
     w.kparts = 4 / w.combos;
     w.X = reinterpret_cast<const half_t *>(X);
     w.dY = reinterpret_cast<const half_t *>(dY);
-    w.batch = d.batch; w.Cin = d.Cin; w.Cout = d.Cout; w.Hin = d.Hin; w.Win = d.Win; w.Ho = d.Ho; w.Wo = d.Wo;
+    w.batch = d.batch; w.Cin = d.Cin; w.Cout = d.Cout; w.Hin = d.Hin; w.Win = d.Win; w.Ho = d.Ho;
     w.padU = d.padU; w.padL = d.padL;
     w.ws = workspace((size_t)w.nwg * w.total * sizeof(float));
     return w.ws ? 0 : 2;
@@ -519,7 +600,7 @@ int conv_small(const ConvTileDesc &d, const void *X, const void *Wt, void *Y) {
 
 int conv_small_wg(const ConvTileDesc &d, const void *X, const void *dY, void *dW) {
     WgSmallArgs w;
-    if (int rc = plan_wg(d, X, dY, state().num_cu, w)) return rc;
+    if (int rc = plan_wg(d, X, dY, state().num_cu, true, w)) return rc;
     static bool attr_set = false;
     if (!attr_set) {
         if (!hip_ok(hipFuncSetAttribute(reinterpret_cast<const void *>(wg_small_kernel),
@@ -536,7 +617,7 @@ int conv_small_wg(const ConvTileDesc &d, const void *X, const void *dY, void *dW
 int conv_small_bw(const ConvTileDesc &fwd, const ConvTileDesc &ig, const void *X, const void *dY, const void *Wt,
                   void *dW, void *dX) {
     WgSmallArgs w;
-    if (int rc = plan_wg(fwd, X, dY, state().num_cu / 2, w)) return rc;
+    if (int rc = plan_wg(fwd, X, dY, state().num_cu / 2, false, w)) return rc;
     SmallPlan p;
     const int budget = state().num_cu - w.nwg;
     if (int rc = plan_small(ig, dY, Wt, dX, budget > 32 ? budget : 32, p)) return rc;

@@ -196,9 +196,8 @@ class ResNetStep:
             a, kp = hp.conv2d_args(pkg, x, dx, self.W[name], self.dW[name], y, dy, ci, H, H, co, k, k, Ho, Ho,
                                    (p, p, p, p), (s, s), 0, 1 if s == 1 else 0)
             self.keep.append(kp)
-            bw = [(L("ptl_conv2d_DT_wg_batched"), a, (ns,))]
-            if dx is not None:
-                bw.append((L("ptl_conv2d_DT_ig_batched"), a, (ns,)))
+            # weight and input gradient in one call (the stem needs no input gradient)
+            bw = [(L("ptl_conv2d_DT_bw_batched"), a, (ns,))] if dx is not None else [(L("ptl_conv2d_DT_wg_batched"), a, (ns,))]
             return (L("ptl_conv2d_DT_fw_batched"), a, (ns,)), bw, y, dy, Ho
 
         def norm(name, y, dy, Ho, relu, skip=None, out_diff=None):

@@ -74,7 +74,9 @@ def test_conv2d_small_layer_kernel_random_geometries(pkg, gpu, seed):
         w = ((torch.rand(Co, Ci, 3, 3, device="cuda") - 0.5) * 0.5).half()
         dy = (torch.rand(ns, Co, Ho, Wo, device="cuda") - 0.5).half()
         y, dx, dw = torch.full_like(dy, 3), torch.full_like(x, 3), torch.full_like(w, 3)
+        dx2, dw2 = torch.full_like(x, 3), torch.full_like(w, 3)
         a, keep = hp.conv2d_args(pkg, x, dx, w, dw, y, dy, Ci, H, W, Co, 3, 3, Ho, Wo, (pl, pr, pu, pd), (st, st))
+        a2, keep2 = hp.conv2d_args(pkg, x, dx2, w, dw2, y, dy, Ci, H, W, Co, 3, 3, Ho, Wo, (pl, pr, pu, pd), (st, st))
         case = (Ci, Co, H, W, (pl, pr, pu, pd), st, ns)
         gpu.ptl_set_gemm_path(6)
         try:
@@ -82,6 +84,9 @@ def test_conv2d_small_layer_kernel_random_geometries(pkg, gpu, seed):
             small_fw = gpu.ptl_last_conv_resident() == 2
             pkg.call("ptl_conv2d_fp16_ig_batched", a, ns)
             small_ig = gpu.ptl_last_conv_resident() == 2
+            # the weight gradient (alone, and with the input gradient in the same launch): whatever route takes it
+            pkg.call("ptl_conv2d_fp16_wg_batched", a, ns)
+            pkg.call("ptl_conv2d_fp16_bw_batched", a2, ns)
         finally:
             gpu.ptl_set_gemm_path(0)
         gpu.ptl_sync()
@@ -95,9 +100,50 @@ def test_conv2d_small_layer_kernel_random_geometries(pkg, gpu, seed):
         xp = F.pad(x.float(), (pl, pr, pu, pd))
         ref_y = F.conv2d(xp, w.float(), stride=st)
         ref_dx = torch.nn.grad.conv2d_input(xp.shape, w.float(), dy.float(), stride=st)[:, :, pu:pu + H, pl:pl + W]
+        ref_dw = torch.nn.grad.conv2d_weight(xp, w.shape, dy.float(), stride=st)
         assert rel(y, ref_y) <= 2e-3, (case, "y")
         assert rel(dx, ref_dx) <= 2e-3, (case, "dx")
+        assert rel(dw, ref_dw) <= 2e-3, (case, "dw")
+        assert rel(dx2, ref_dx) <= 2e-3, (case, "dx, one call")
+        assert rel(dw2, ref_dw) <= 2e-3, (case, "dw, one call")
     assert ran >= 12
+
+
+@pytest.mark.parametrize("seed", [41, 42])
+def test_conv2d_small_layer_weight_gradient_random_geometries(pkg, gpu, seed):
+    """Unit-stride 3x3 fp16 layers whose output is as wide as the input (the geometries the small-layer weight-gradient
+    kernel takes, forced with path 6): weight gradient alone and together with the input gradient, tiles of several
+    samples (64 channels), split rows (few samples), ragged last tiles, all three left paddings."""
+    rng = random.Random(seed)
+    for it in range(14):
+        Ci, Co = rng.choice([3, 8, 16, 24, 32, 64]), rng.choice([8, 16, 32, 40, 64])
+        pl = rng.randint(0, 2)
+        pr, pu, pd = 2 - pl, rng.randint(0, 2), rng.randint(0, 2)
+        W, H = rng.choice([8, 16, 24, 32]), rng.randint(max(3 - pu - pd, 1), 34)
+        ns = rng.choice([1, 2, 5, 9, 32, 130])
+        Ho, Wo = H + pu + pd - 2, W
+        x = (torch.rand(ns, Ci, H, W, device="cuda") - 0.5).half()
+        w = ((torch.rand(Co, Ci, 3, 3, device="cuda") - 0.5) * 0.5).half()
+        dy = (torch.rand(ns, Co, Ho, Wo, device="cuda") - 0.5).half()
+        y, dx, dw = torch.full_like(dy, 3), torch.full_like(x, 3), torch.full_like(w, 3)
+        dx2, dw2 = torch.full_like(x, 3), torch.full_like(w, 3)
+        a, keep = hp.conv2d_args(pkg, x, dx, w, dw, y, dy, Ci, H, W, Co, 3, 3, Ho, Wo, (pl, pr, pu, pd), (1, 1))
+        a2, keep2 = hp.conv2d_args(pkg, x, dx2, w, dw2, y, dy, Ci, H, W, Co, 3, 3, Ho, Wo, (pl, pr, pu, pd), (1, 1))
+        case = (Ci, Co, H, W, (pl, pr, pu, pd), ns)
+        gpu.ptl_set_gemm_path(6)
+        try:
+            pkg.call("ptl_conv2d_fp16_wg_batched", a, ns)
+            pkg.call("ptl_conv2d_fp16_bw_batched", a2, ns)
+            assert gpu.ptl_last_conv_resident() == (2 if (Ci * Co * 9) % 8 == 0 else 0), case
+        finally:
+            gpu.ptl_set_gemm_path(0)
+        gpu.ptl_sync()
+        xp = F.pad(x.float(), (pl, pr, pu, pd))
+        ref_dx = torch.nn.grad.conv2d_input(xp.shape, w.float(), dy.float())[:, :, pu:pu + H, pl:pl + W]
+        ref_dw = torch.nn.grad.conv2d_weight(xp, w.shape, dy.float())
+        assert rel(dw, ref_dw) <= 2e-3, (case, "dw")
+        assert rel(dx2, ref_dx) <= 2e-3, (case, "dx, one call")
+        assert rel(dw2, ref_dw) <= 2e-3, (case, "dw, one call")
 
 
 @pytest.mark.parametrize("seed", [21, 22])

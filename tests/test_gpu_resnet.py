@@ -92,4 +92,4 @@ def test_resnet20_training_step_with_batch_norm(pkg, gpu, dt, ns, tol, fused):
         assert hp.rel_l2(net.G[n].cpu().numpy(), ref_new["g:" + n]) <= tol, n
     for n in w:
         assert hp.rel_l2(net.W[n].cpu().numpy(), ref_new[n]) <= tol, n
-    assert net.launches() > (100 if fused else 170)
+    assert net.launches() > (80 if fused else 170)
