@@ -188,7 +188,7 @@ __device__ inline void conv_small_block(const ConvSmallArgs &a, int tile, char *
 // (filter row ky) x (32x32 block of the weight tensor) x (share of the positions); per k step a wave reads the
 // gradient piece, the input piece and the input's two edge dwords, forms the three column taps by shifting whole
 // elements in registers and issues three MFMAs.  The shares are added through LDS and the workgroup's partial sums go
-// to ws[workgroup][co][ci][tap]; a second launch adds the workgroups.
+// to ws[workgroup][block][tap][filter][channel] (filters and channels a tile really has); a second launch adds the workgroups and writes dW[co][ci][tap].
 constexpr int WG_CHUNKS = 4;  // 16-byte pieces per thread and tensor, at most
 
 struct WgSmallArgs {
@@ -200,9 +200,10 @@ struct WgSmallArgs {
     int PY, PX, WP;                // LDS pitches in elements: gradient channel, input channel, input row
     int groups;                    // S * R * G
     int y_chunks, x_chunks, pad_chunks, pad_rows;  // pieces to copy; zero pieces (one per input row + one) and rows per channel
-    unsigned magic_g, magic_rg, magic_r2g, magic_ychan, magic_xchan, magic_padrows, magic_cin9;
+    unsigned magic_g, magic_rg, magic_r2g, magic_ychan, magic_xchan, magic_padrows, magic_tile, magic_cols;
     int cbi_n, combos, kparts;  // 32-channel blocks, (filter block, channel block) pairs, position shares
     int total;                  // Cout * Cin * 9
+    int rows_kept, cols_kept, part_elems;  // filter rows and channels of a 32x32 tile that are stored; floats per workgroup in ws
 };
 
 // elements D .. D + 7 of a row of which c holds elements 0..7, p3 elements -2, -1 and n0 elements 8, 9
@@ -326,15 +327,28 @@ __device__ inline void wg_small_block(const WgSmallArgs &a, int wg, char *smem) 
         }
     }
     __syncthreads();
-    float *out = a.ws + (size_t)wg * a.total;
-    const int cin9 = a.Cin * 9, share = a.combos * 9 * 1024;
-    for (int i = tid; i < a.total; i += CS_NT) {
-        const int o = fast_div(i, a.magic_cin9), rem = i - o * cin9;
-        const int c = (rem * 7282) >> 16, tap = rem - c * 9;  // rem / 9 for rem < 2^15
-        const float *src = L + (((o >> 5) * a.cbi_n + (c >> 5)) * 9 + tap) * 1024 + (o & 31) * 32 + (c & 31);
+    // partial sums in tile order, [block][tap][filter row][channel] with the rows and channels the tensor has: thread t
+    // (consecutive threads take consecutive elements of a tile: decoding an index of the weight tensor per element
+    // would cost more than the sums, sixteen waves share the integer pipes); the second launch puts the sums where
+    // the weight tensor wants them
+    float *out = a.ws + (size_t)wg * a.part_elems;
+    const int share = a.combos * 9 * 1024, tile_elems = a.rows_kept * a.cols_kept;
+    if (tile_elems == 1024) {  // whole tiles: thread t owns element t of every tile
+        for (int t = 0; t < a.combos * 9; ++t) {
+            const float *src = L + t * 1024 + tid;
+            float sum = src[0];
+            for (int kp = 1; kp < a.kparts; ++kp) sum += src[kp * share];
+            out[t * 1024 + tid] = sum;
+        }
+        return;
+    }
+    for (int e = tid; e < a.part_elems; e += CS_NT) {
+        const int t = fast_div(e, a.magic_tile), r = e - t * tile_elems;
+        const int row = fast_div(r, a.magic_cols), col = r - row * a.cols_kept;
+        const float *src = L + t * 1024 + row * 32 + col;
         float sum = src[0];
         for (int kp = 1; kp < a.kparts; ++kp) sum += src[kp * share];
-        out[i] = sum;
+        out[e] = sum;
     }
 }
 
@@ -393,36 +407,41 @@ int launch_small(const ConvSmallArgs &a, int tiles, size_t lds, hipStream_t s, c
     return hip_ok(hipGetLastError(), "small convolution launch") ? 0 : 2;
 }
 
-// dW[i] = sum over workgroups of ws[workgroup][i]: 64 outputs per workgroup of the reduction, 16 groups of
-// partials in parallel.
+// dW(co, ci, tap) = sum over workgroups of ws[workgroup][block][tap][filter row][channel]: 64 consecutive partial
+// elements per workgroup of the reduction (coalesced reads), 16 groups of partials in parallel, eight loads in flight
+// per thread; the few results are scattered to the weight tensor's order.
 __global__ __launch_bounds__(1024) void wg_small_reduce_kernel(const float *__restrict__ ws, half_t *__restrict__ dW,
-                                                               int total, int parts) {
+                                                               int part_elems, int parts, int rows_kept,
+                                                               int cols_kept, int cbi_n, int Cout, int Cin) {
     __shared__ float part_sum[16][64];
     const int o = threadIdx.x & 63, pg = threadIdx.x >> 6;
     const int i = blockIdx.x * 64 + o;
     float s = 0.f;
-    if (i < total) {  // (eight loads in flight per thread: the kernel lives on memory-level parallelism)
+    if (i < part_elems) {
         const float *src = ws + i;
         int p = pg;
         for (; p + 7 * 16 < parts; p += 8 * 16) {
             float v[8];
 #pragma unroll
-            for (int u = 0; u < 8; ++u) v[u] = src[(size_t)(p + u * 16) * total];
+            for (int u = 0; u < 8; ++u) v[u] = src[(size_t)(p + u * 16) * part_elems];
 #pragma unroll
             for (int u = 0; u < 8; ++u) s += v[u];
         }
         float v[8];
 #pragma unroll
-        for (int u = 0; u < 8; ++u) v[u] = p + u * 16 < parts ? src[(size_t)(p + u * 16) * total] : 0.f;
+        for (int u = 0; u < 8; ++u) v[u] = p + u * 16 < parts ? src[(size_t)(p + u * 16) * part_elems] : 0.f;
 #pragma unroll
         for (int u = 0; u < 8; ++u) s += v[u];
     }
     part_sum[pg][o] = s;
     __syncthreads();
-    if (pg == 0 && i < total) {
+    if (pg == 0 && i < part_elems) {
 #pragma unroll
         for (int q = 1; q < 16; ++q) s += part_sum[q][o];
-        dW[i] = (half_t)s;
+        const int tile = i / (rows_kept * cols_kept), r = i - tile * rows_kept * cols_kept;
+        const int combo = tile / 9, tap = tile - combo * 9;
+        const int co = (combo / cbi_n) * 32 + r / cols_kept, ci = (combo % cbi_n) * 32 + r % cols_kept;
+        if (co < Cout && ci < Cin) dW[(co * Cin + ci) * 9 + tap] = (half_t)s;
     }
 }
 
@@ -529,10 +548,11 @@ int plan_wg(const ConvTileDesc &d, const void *X, const void *dY, int max_wg, bo
     w.total = d.Cout * d.Cin * 9;
     if (w.total >= 65536) return -1;
     const long long positions = (long long)d.batch * d.Ho * d.Wo;
-    // large calls keep the tiled weight-gradient kernels; so do calls for the weight gradient alone from 32 channels
-    // on (measured 14.7 against 13.7 us for 32 -> 32 on 16x16 at batch 128, 9.7 against 11.5 us for 3 -> 16 on 32x32:
-    // what this kernel buys is the input gradient riding along in the same launch)
-    if (st.gemm_path != 6 && (positions > 262144 || (alone && (d.Cin > 16 || d.Cout > 16 || d.batch < 32)))) return -1;
+    // large calls keep the tiled weight-gradient kernels, and so do small calls for the weight gradient alone (measured
+    // 12.0 against 13.7 us for 32 -> 32 on 16x16 at batch 128, 16.7 against 20.0 us for 64 -> 64 on 8x8, but 8.8
+    // against 8.4 us for 16 -> 32 on 32x32 at one sample: below a few thousand positions what this kernel buys is
+    // the input gradient riding along in the same launch)
+    if (st.gemm_path != 6 && (positions > 262144 || (alone && positions < 8192))) return -1;
     w.G = d.Win / 8;
     w.WP = d.Win + 8;
     auto round_pitch = [](int n) { return n + ((8 - n % 64) + 64) % 64; };  // = 8 mod 64: rows 16 bytes apart in the banks
@@ -547,10 +567,11 @@ int plan_wg(const ConvTileDesc &d, const void *X, const void *dY, int max_wg, bo
     // tiles: whole samples while the partial sums stay within about 5 MB (S samples each otherwise), rows of a
     // sample split while that fills more of `max_wg` workgroups and leaves the waves eight k steps each
     int S = 1, R = d.Ho;
-    while ((long long)((d.batch + S - 1) / S) * w.total * 4 > (5LL << 20) && chunks_ok(S * 2, R)) S *= 2;
+    const long long part_bytes = (long long)((d.Cin + 31) / 32) * ((d.Cout + 31) / 32) * 9 * (d.Cout < 32 ? d.Cout : 32) * (d.Cin < 32 ? d.Cin : 32) * 4;
+    while ((long long)((d.batch + S - 1) / S) * part_bytes > (5LL << 20) && chunks_ok(S * 2, R)) S *= 2;
     if (S == 1)
         while (R % 2 == 0 && (long long)d.batch * (d.Ho / R) * 2 <= max_wg && (R / 2) * w.G >= 16 &&
-               (long long)d.batch * (d.Ho / R) * 2 * w.total * 4 <= (5LL << 20))
+               (long long)d.batch * (d.Ho / R) * 2 * part_bytes <= (5LL << 20))
             R /= 2;
     while (!chunks_ok(S, R) && R % 2 == 0 && S == 1) R /= 2;
     if (!chunks_ok(S, R)) return -1;
@@ -572,21 +593,25 @@ int plan_wg(const ConvTileDesc &d, const void *X, const void *dY, int max_wg, bo
     w.magic_ychan = magic_of(w.groups);
     w.magic_xchan = magic_of(S * w.R2G);
     w.magic_padrows = magic_of(w.pad_rows);
-    w.magic_cin9 = magic_of(d.Cin * 9);
     w.cbi_n = (d.Cin + 31) / 32;
     w.combos = w.cbi_n * ((d.Cout + 31) / 32);
     w.kparts = 4 / w.combos;
+    w.rows_kept = d.Cout < 32 ? d.Cout : 32;
+    w.cols_kept = d.Cin < 32 ? d.Cin : 32;
+    w.part_elems = w.combos * 9 * w.rows_kept * w.cols_kept;
+    w.magic_tile = magic_of(w.rows_kept * w.cols_kept);
+    w.magic_cols = magic_of(w.cols_kept);
     w.X = reinterpret_cast<const half_t *>(X);
     w.dY = reinterpret_cast<const half_t *>(dY);
     w.batch = d.batch; w.Cin = d.Cin; w.Cout = d.Cout; w.Hin = d.Hin; w.Win = d.Win; w.Ho = d.Ho;
     w.padU = d.padU; w.padL = d.padL;
-    w.ws = workspace((size_t)w.nwg * w.total * sizeof(float));
+    w.ws = workspace((size_t)w.nwg * w.part_elems * sizeof(float));
     return w.ws ? 0 : 2;
 }
 
 int reduce_wg(const WgSmallArgs &w, void *dW) {
-    hipLaunchKernelGGL(wg_small_reduce_kernel, dim3((w.total + 63) / 64), dim3(1024), 0, state().stream, w.ws,
-                       reinterpret_cast<half_t *>(dW), w.total, w.nwg);
+    hipLaunchKernelGGL(wg_small_reduce_kernel, dim3((w.part_elems + 63) / 64), dim3(1024), 0, state().stream, w.ws,
+                       reinterpret_cast<half_t *>(dW), w.part_elems, w.nwg, w.rows_kept, w.cols_kept, w.cbi_n, w.Cout, w.Cin);
     return hip_ok(hipGetLastError(), "small weight gradient reduction launch") ? 0 : 2;
 }
 
