@@ -30,6 +30,7 @@ struct ConvSmallArgs {
     const half_t *X, *Wt;
     half_t *Y;
     int Cin, Cout, Hin, Win, Ho, Wo, s, padU, padL;
+    int dil;                // 2: the input is read zero-stuffed by two (tile rows and columns count the stuffed image)
     int R, tiles_per_img;   // output rows per workgroup
     int RR, TW, POS;        // input rows of a tile, padded row width, RR * TW
     int items;              // wave-wide load items: (channel block, column group, block of 8 rows)
@@ -41,7 +42,7 @@ struct ConvSmallArgs {
     int b_pitch, f_bytes;   // bytes per filter row in LDS, bytes of the filter tile
     int pgroups, mshift;    // jobs = groups of 32 pixels x (1 << mshift) blocks of 32 filters
     // per item: element offset into the sample (first channel, first tile row, column group), half offset into the
-    // LDS tile, first tile row | first channel << 8
+    // LDS tile, first tile row | first channel << 8 | column group << 16
     int item_g[CS_ITEMS], item_l[CS_ITEMS], item_rc[CS_ITEMS];
 };
 
@@ -67,9 +68,14 @@ __device__ inline void conv_small_block(const ConvSmallArgs &a, int tile, char *
         const int item = wave + CS_WAVES * k;
         xin[k].v = make_uint4(0, 0, 0, 0);
         if (item < a.items) {
-            const int rc = a.item_rc[item], rr = (rc & 255) + lrow, ch = (rc >> 8) + lch, iy = iy0 + rr;
-            if (rr < a.RR && ch < a.Cin && iy >= 0 && iy < a.Hin)
+            const int rc = a.item_rc[item], rr = (rc & 255) + lrow, ch = ((rc >> 8) & 255) + lch, iy = iy0 + rr;
+            if (a.dil == 2) {  // even rows of the stuffed image are rows of the tensor
+                if (rr < a.RR && ch < a.Cin && iy >= 0 && !(iy & 1) && (iy >> 1) < a.Hin)
+                    xin[k].v = *reinterpret_cast<const uint4 *>(
+                        a.X + (((size_t)b * a.Cin + ch) * a.Hin + (iy >> 1)) * a.Win + 8 * (rc >> 16));
+            } else if (rr < a.RR && ch < a.Cin && iy >= 0 && iy < a.Hin) {
                 xin[k].v = *reinterpret_cast<const uint4 *>(xs + a.item_g[item]);
+            }
         }
     }
     Piece fin[F_MAX];
@@ -84,7 +90,11 @@ __device__ inline void conv_small_block(const ConvSmallArgs &a, int tile, char *
         for (int i = tid; i < a.f_bytes / 16; i += CS_NT) reinterpret_cast<uint4 *>(F)[i] = make_uint4(0, 0, 0, 0);
         __syncthreads();
     }
-    // ---- halo columns of the tile: whole chunks of zeros
+    // ---- halo columns of the tile: whole chunks of zeros (a zero-stuffed input: the whole tile first)
+    if (a.dil == 2) {
+        for (int i = tid; i < (CINP / 8) * a.POS; i += CS_NT) reinterpret_cast<uint4 *>(T)[i] = make_uint4(0, 0, 0, 0);
+        __syncthreads();
+    } else
     for (int i = tid; i < a.halo_chunks; i += CS_NT) {
         const int row = fast_div(i, a.magic_halo_w), hc = i - row * a.halo_w;  // row = channel block * RR + tile row
         const int cb = fast_div(row, a.magic_rr), rr = row - cb * a.RR;
@@ -98,8 +108,9 @@ __device__ inline void conv_small_block(const ConvSmallArgs &a, int tile, char *
         const int item = wave + CS_WAVES * k;
         if (item < a.items && (a.item_rc[item] & 255) + lrow < a.RR) {
             half_t *row = tl + a.item_l[item];
+            const int step = 8 * a.dil;
 #pragma unroll
-            for (int j = 0; j < 8; ++j) row[j * 8] = xin[k].e[j];
+            for (int j = 0; j < 8; ++j) row[j * step] = xin[k].e[j];
         }
     }
     // ---- filter pieces -> [filter][tap][channel]: element (outer, inner, tap) of the dense tensor goes to
@@ -474,7 +485,10 @@ int plan_small(const ConvTileDesc &d, const void *X, const void *Wt, void *Y, in
     } else {
         return -1;
     }
-    const int s = d.sh, TW = d.Win + d.padL + d.padR, THP = d.Hin + d.padU + d.padD;
+    const int dil = d.in_dil == 2 ? 2 : 1;
+    if (d.in_dil > 2 || (dil == 2 && d.sh != 1)) return -1;
+    const int Hd = (d.Hin - 1) * dil + 1, Wd = (d.Win - 1) * dil + 1;  // the image the taps walk over
+    const int s = d.sh, TW = Wd + d.padL + d.padR, THP = Hd + d.padU + d.padD;
     if ((d.Wo - 1) * s + 3 > TW || (d.Ho - 1) * s + 3 > THP || d.Wo >= 65536 || d.Ho * d.Wo >= 65536) return -1;
     const int cinp = d.Cin <= 16 ? 16 : d.Cin <= 32 ? 32 : 64, cblocks = cinp / 8;
     const int mblocks = (d.Cout + 31) / 32;
@@ -497,6 +511,7 @@ int plan_small(const ConvTileDesc &d, const void *X, const void *Wt, void *Y, in
     a.Y = reinterpret_cast<half_t *>(Y);
     a.Cin = d.Cin; a.Cout = d.Cout; a.Hin = d.Hin; a.Win = d.Win; a.Ho = d.Ho; a.Wo = d.Wo;
     a.s = s; a.padU = d.padU; a.padL = d.padL;
+    a.dil = dil;
     a.R = R; a.tiles_per_img = (d.Ho + R - 1) / R;
     a.RR = (R - 1) * s + 3; a.TW = TW; a.POS = a.RR * TW;
     const int G = d.Win / 8, RR8 = (a.RR + 7) / 8;
@@ -504,10 +519,10 @@ int plan_small(const ConvTileDesc &d, const void *X, const void *Wt, void *Y, in
     for (int item = 0; item < a.items; ++item) {
         const int rblk = item % RR8, t = item / RR8, g = t % G, cb = t / G;
         a.item_g[item] = (cb * 8 * d.Hin + rblk * 8) * d.Win + 8 * g;
-        a.item_l[item] = ((cb * a.POS + rblk * 8 * TW) + d.padL + 8 * g) * 8;
-        a.item_rc[item] = (rblk * 8) | ((cb * 8) << 8);
+        a.item_l[item] = ((cb * a.POS + rblk * 8 * TW) + d.padL + dil * 8 * g) * 8;
+        a.item_rc[item] = (rblk * 8) | ((cb * 8) << 8) | (g << 16);
     }
-    a.halo_w = TW - d.Win;
+    a.halo_w = dil == 2 ? 1 : TW - d.Win;  // (a zero-stuffed input zeroes its whole tile instead)
     a.halo_chunks = cblocks * a.RR * a.halo_w;
     a.magic_halo_w = magic_of(a.halo_w);
     a.magic_rr = magic_of(a.RR);

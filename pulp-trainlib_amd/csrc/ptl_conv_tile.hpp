@@ -18,6 +18,10 @@ struct ConvTileDesc {
     // 1: the input is channel-minor, in(b, ci, iy, ix) at X[((b*Hin + iy)*Win + ix)*Cin + ci] (x_s* unused);
     // with Cin a multiple of the 16-byte vector it already consists of the chunks the kernel wants
     int in_hwc;
+    // 2: the convolution reads the input zero-stuffed by two (element (y, x) of the tensor at (2y, 2x) of a
+    // (2*Hin - 1) x (2*Win - 1) image, zeros between): the input gradient of a stride-2 layer as a unit-stride pass
+    // over its output gradient.  Only the small-layer kernel takes it; 0 or 1: the tensor as it is.
+    int in_dil;
 };
 
 // Launches the direct kernel; the output is written through `c` (n = pixel index over

@@ -435,6 +435,7 @@ struct BnFuse {
     const T *dy2;   // backward: second incoming gradient
     T *gout;        // backward: receives g
     int relu;
+    unsigned hw_magic;  // ceil(2^32 / HW) when indices and HW are below 2^16 (sample index by multiplication), else 0
 };
 
 template <typename T, bool BW, bool FUSED = false>
@@ -451,7 +452,7 @@ __global__ __launch_bounds__(256) void bn_sums_kernel(const T *__restrict__ x, c
     float s[BN_SUMS] = {0.f, 0.f, 0.f, 0.f};
     if (vec) {  // planes are whole 16-byte vectors
         for (int i = tid * VEC; i < total; i += 256 * VEC) {
-            const int bl = i / HW, e = i - bl * HW;
+            const int bl = f.hw_magic ? (int)__umulhi((unsigned)i, f.hw_magic) : i / HW, e = i - bl * HW;
             const size_t at = ((size_t)(b0 + bl) * C + c) * HW + e;
             BnVec<T> xv, gv;
             xv.raw = *reinterpret_cast<const uint4 *>(x + at);
@@ -484,7 +485,7 @@ __global__ __launch_bounds__(256) void bn_sums_kernel(const T *__restrict__ x, c
         }
     } else {
         for (int i = tid; i < total; i += 256) {
-            const int bl = i / HW, e = i - bl * HW;
+            const int bl = f.hw_magic ? (int)__umulhi((unsigned)i, f.hw_magic) : i / HW, e = i - bl * HW;
             const size_t at = ((size_t)(b0 + bl) * C + c) * HW + e;
             const float v = (float)x[at];
             s[0] += v;
@@ -560,7 +561,7 @@ __global__ __launch_bounds__(256) void bn_apply_kernel(const T *__restrict__ x, 
     const int total = nb * HW;
     if (vec) {
         for (int i = tid * VEC; i < total; i += 256 * VEC) {
-            const int bl = i / HW, e = i - bl * HW;
+            const int bl = f.hw_magic ? (int)__umulhi((unsigned)i, f.hw_magic) : i / HW, e = i - bl * HW;
             const size_t at = ((size_t)(b0 + bl) * C + c) * HW + e;
             BnVec<T> xv, gv;
             xv.raw = *reinterpret_cast<const uint4 *>(x + at);
@@ -599,7 +600,7 @@ __global__ __launch_bounds__(256) void bn_apply_kernel(const T *__restrict__ x, 
         }
     } else {
         for (int i = tid; i < total; i += 256) {
-            const int bl = i / HW, e = i - bl * HW;
+            const int bl = f.hw_magic ? (int)__umulhi((unsigned)i, f.hw_magic) : i / HW, e = i - bl * HW;
             const size_t at = ((size_t)(b0 + bl) * C + c) * HW + e;
             if (!BW && FUSED) {
                 float v = map((float)x[at], 0.f);
@@ -635,6 +636,11 @@ static int batch_norm_step(const Args *a, int bw, const char *fn, const Fusion *
     if (groups > B) groups = B;
     const int per_group = (B + groups - 1) / groups;
     groups = (B + per_group - 1) / per_group;
+    const unsigned hw_magic = (HW > 1 && HW < 65536 && (long long)per_group * HW + 4096 < 65536)
+                                  ? (unsigned)((((unsigned long long)1 << 32) + HW - 1) / HW)
+                                  : 0u;
+    BnFuse<T> f0 = {};
+    f0.hw_magic = hw_magic;
     float *part = workspace((size_t)C * groups * BN_SUMS * sizeof(float));
     if (!part) return 2;
     Stager sg;
@@ -650,6 +656,7 @@ static int batch_norm_step(const Args *a, int bw, const char *fn, const Fusion *
         if (sg.failed() || !y) return sg.failed() ? 2 : glue_bad(fn, "null buffer");
         int vec = HW % VEC == 0 && aligned16(x) && aligned16(y);
         BnFuse<T> f = {};
+        f.hw_magic = hw_magic;
         if constexpr (FUSED) {
             f.relu = fu->relu ? 1 : 0;
             f.skip = fu->skip ? sg.in(reinterpret_cast<const T *>(fu->skip), n) : nullptr;
@@ -657,7 +664,7 @@ static int batch_norm_step(const Args *a, int bw, const char *fn, const Fusion *
             vec = vec && aligned16(f.skip);
         }
         hipLaunchKernelGGL((bn_sums_kernel<T, false>), dim3(C, groups), dim3(256), 0, st.stream, x, (const T *)nullptr,
-                           part, B, C, HW, per_group, vec, BnFuse<T>());
+                           part, B, C, HW, per_group, vec, f0);
         hipLaunchKernelGGL((bn_apply_kernel<T, false, FUSED>), dim3(C, groups), dim3(256), 0, st.stream, x,
                            (const T *)nullptr, y, w, b, eps, part, (T *)nullptr, (T *)nullptr, B, C, HW, groups,
                            per_group, 1, vec, f);
@@ -670,6 +677,7 @@ static int batch_norm_step(const Args *a, int bw, const char *fn, const Fusion *
         if (sg.failed() || !dy || (want_dx && !dx)) return sg.failed() ? 2 : glue_bad(fn, "null buffer");
         int vec = HW % VEC == 0 && aligned16(x) && aligned16(dy) && (!dx || aligned16(dx));
         BnFuse<T> f = {};
+        f.hw_magic = hw_magic;
         if constexpr (FUSED) {
             f.relu = fu->relu ? 1 : 0;
             if (f.relu) {

@@ -477,6 +477,23 @@ static int conv2d_ig(const Args *a, int ns, const char *fn) {
         return sg.finish(gemm<T>(q));
     }
 
+    // Small fp16 stride-2 layers: the small-layer kernel stuffs the zeros while it fills its LDS tile.
+    if (sizeof(T) == 2 && !g.hwc && g.sh == 2 && g.sw == 2 && g.Hk == 3 && g.Wk == 3) {
+        ConvTileDesc d = {};
+        d.batch = ns; d.Cin = g.Co; d.Hin = g.Ho; d.Win = g.Wo; d.in_dil = 2;
+        d.Cout = g.Ci; d.Ho = g.H; d.Wo = g.W;
+        d.KH = 3; d.KW = 3; d.sh = 1; d.sw = 1;
+        d.padU = 2 - g.Up; d.padL = 2 - g.Lp;
+        d.padD = g.H + 2 - Hd - d.padU; d.padR = g.W + 2 - Wd - d.padL;
+        d.x_sb = (long long)g.Co * P; d.x_sc = P; d.x_sy = g.Wo;
+        d.w_base = Pk - 1; d.w_sm = Pk; d.w_sc = g.Ci * Pk; d.w_sy = -g.Wk; d.w_sx = -1;
+        state().last_conv_direct = 0;
+        state().last_conv_resident = 0;
+        const int rc = conv_small(d, dY, Wt, dX);
+        if (rc == 0) state().last_conv_direct = 1;
+        if (rc >= 0) return sg.finish(rc);
+    }
+
     // A strided forward is undone by a unit-stride pass over the zero-stuffed gradient.
     if (g.sh != 1 || g.sw != 1) {
         T *dil = static_cast<T *>(scratch(dil_n * sizeof(T)));
