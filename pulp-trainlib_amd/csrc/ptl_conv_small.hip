@@ -23,17 +23,17 @@ namespace ptl {
 namespace {
 
 constexpr int CS_NT = 1024, CS_WAVES = CS_NT / 64;
-constexpr int CS_ITEMS = 32;                      // wave-wide load items per workgroup, at most
+constexpr int CS_ITEMS = 64;                      // wave-wide load items per workgroup, at most
 constexpr int CS_IN_MAX = CS_ITEMS / CS_WAVES;  // input pieces per thread
 
 struct ConvSmallArgs {
-    const half_t *X, *Wt;
-    half_t *Y;
+    const void *X, *Wt;
+    void *Y;
     int Cin, Cout, Hin, Win, Ho, Wo, s, padU, padL;
     int dil;                // 2: the input is read zero-stuffed by two (tile rows and columns count the stuffed image)
     int R, tiles_per_img;   // output rows per workgroup
     int RR, TW, POS;        // input rows of a tile, padded row width, RR * TW
-    int items;              // wave-wide load items: (channel block, column group, block of 8 rows)
+    int items;              // wave-wide load items: (channel block, column group, block of 64 / VEC rows)
     int halo_chunks, halo_w;  // zero chunks of a tile: channel blocks x rows x halo columns; halo columns per row
     unsigned magic_halo_w, magic_rr;
     int f_chunks, f_inner;  // 16-byte pieces of the filter tensor [outer][inner][9]; inner dimension
@@ -41,28 +41,33 @@ struct ConvSmallArgs {
     unsigned magic_inner9, magic_wo;
     int b_pitch, f_bytes;   // bytes per filter row in LDS, bytes of the filter tile
     int pgroups, mshift;    // jobs = groups of 32 pixels x (1 << mshift) blocks of 32 filters
-    // per item: element offset into the sample (first channel, first tile row, column group), half offset into the
+    // per item: element offset into the sample (first channel, first tile row, column group), element offset into the
     // LDS tile, first tile row | first channel << 8 | column group << 16
     int item_g[CS_ITEMS], item_l[CS_ITEMS], item_rc[CS_ITEMS];
 };
 
+template <typename T>
 union Piece {
     uint4 v;
-    half_t e[8];
+    T e[16 / sizeof(T)];
 };
 
-template <int CINP, int F_MAX>
+// T: element type; VEC = 16 / sizeof(T) elements make a 16-byte piece (8 halves, 4 floats): the channels of an LDS
+// chunk, the columns of a global piece, the k values a lane hands to one MFMA step.
+template <typename T, int CINP, int F_MAX>
 __device__ inline void conv_small_block(const ConvSmallArgs &a, int tile, char *smem) {
+    constexpr int ES = (int)sizeof(T), VEC = 16 / ES, KSTEP = 2 * VEC;
     char *F = smem;
-    half_t *T = reinterpret_cast<half_t *>(smem + a.f_bytes);  // [CINP / 8][POS][8]
+    T *Tl = reinterpret_cast<T *>(smem + a.f_bytes);  // [CINP / VEC][POS][VEC]
+    const T *X = reinterpret_cast<const T *>(a.X);
     const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int b = tile / a.tiles_per_img, y0 = (tile - b * a.tiles_per_img) * a.R;
     const int iy0 = y0 * a.s - a.padU;
 
     // ---- all global loads first
-    Piece xin[CS_IN_MAX];
-    const int lrow = lane >> 3, lch = lane & 7;
-    const half_t *xs = a.X + ((size_t)b * a.Cin + lch) * a.Hin * a.Win + (iy0 + lrow) * a.Win;
+    Piece<T> xin[CS_IN_MAX];
+    const int lrow = lane / VEC, lch = lane % VEC;
+    const T *xs = X + ((size_t)b * a.Cin + lch) * a.Hin * a.Win + (iy0 + lrow) * a.Win;
 #pragma unroll
     for (int k = 0; k < CS_IN_MAX; ++k) {
         const int item = wave + CS_WAVES * k;
@@ -72,13 +77,13 @@ __device__ inline void conv_small_block(const ConvSmallArgs &a, int tile, char *
             if (a.dil == 2) {  // even rows of the stuffed image are rows of the tensor
                 if (rr < a.RR && ch < a.Cin && iy >= 0 && !(iy & 1) && (iy >> 1) < a.Hin)
                     xin[k].v = *reinterpret_cast<const uint4 *>(
-                        a.X + (((size_t)b * a.Cin + ch) * a.Hin + (iy >> 1)) * a.Win + 8 * (rc >> 16));
+                        X + (((size_t)b * a.Cin + ch) * a.Hin + (iy >> 1)) * a.Win + VEC * (rc >> 16));
             } else if (rr < a.RR && ch < a.Cin && iy >= 0 && iy < a.Hin) {
                 xin[k].v = *reinterpret_cast<const uint4 *>(xs + a.item_g[item]);
             }
         }
     }
-    Piece fin[F_MAX];
+    Piece<T> fin[F_MAX];
 #pragma unroll
     for (int k = 0; k < F_MAX; ++k) {
         const int q = tid + CS_NT * k;
@@ -92,46 +97,46 @@ __device__ inline void conv_small_block(const ConvSmallArgs &a, int tile, char *
     }
     // ---- halo columns of the tile: whole chunks of zeros (a zero-stuffed input: the whole tile first)
     if (a.dil == 2) {
-        for (int i = tid; i < (CINP / 8) * a.POS; i += CS_NT) reinterpret_cast<uint4 *>(T)[i] = make_uint4(0, 0, 0, 0);
+        for (int i = tid; i < (CINP / VEC) * a.POS; i += CS_NT) reinterpret_cast<uint4 *>(Tl)[i] = make_uint4(0, 0, 0, 0);
         __syncthreads();
     } else
     for (int i = tid; i < a.halo_chunks; i += CS_NT) {
         const int row = fast_div(i, a.magic_halo_w), hc = i - row * a.halo_w;  // row = channel block * RR + tile row
         const int cb = fast_div(row, a.magic_rr), rr = row - cb * a.RR;
         const int col = hc < a.padL ? hc : a.Win + hc;
-        reinterpret_cast<uint4 *>(T)[cb * a.POS + rr * a.TW + col] = make_uint4(0, 0, 0, 0);
+        reinterpret_cast<uint4 *>(Tl)[cb * a.POS + rr * a.TW + col] = make_uint4(0, 0, 0, 0);
     }
     // ---- input pieces -> [channel block][row][column] chunks
-    half_t *tl = T + lrow * a.TW * 8 + lch;
+    T *tl = Tl + lrow * a.TW * VEC + lch;
 #pragma unroll
     for (int k = 0; k < CS_IN_MAX; ++k) {
         const int item = wave + CS_WAVES * k;
         if (item < a.items && (a.item_rc[item] & 255) + lrow < a.RR) {
-            half_t *row = tl + a.item_l[item];
-            const int step = 8 * a.dil;
+            T *row = tl + a.item_l[item];
+            const int step = VEC * a.dil;
 #pragma unroll
-            for (int j = 0; j < 8; ++j) row[j * step] = xin[k].e[j];
+            for (int j = 0; j < VEC; ++j) row[j * step] = xin[k].e[j];
         }
     }
     // ---- filter pieces -> [filter][tap][channel]: element (outer, inner, tap) of the dense tensor goes to
     // (filter, channel) = (outer, inner), or (inner, outer) with the taps flipped; the address moves with the indices
     {
-        const int step_tap = a.f_transposed ? -CINP * 2 : CINP * 2;
-        const int step_inner = (a.f_transposed ? a.b_pitch : 2) - 9 * step_tap;  // after the ninth tap step: tap 0, inner + 1
-        const int step_outer = (a.f_transposed ? 2 : a.b_pitch) - a.f_inner * (a.f_transposed ? a.b_pitch : 2);
+        const int step_tap = a.f_transposed ? -CINP * ES : CINP * ES;
+        const int step_inner = (a.f_transposed ? a.b_pitch : ES) - 9 * step_tap;  // after the ninth tap step: tap 0, inner + 1
+        const int step_outer = (a.f_transposed ? ES : a.b_pitch) - a.f_inner * (a.f_transposed ? a.b_pitch : ES);
 #pragma unroll
         for (int k = 0; k < F_MAX; ++k) {
             const int q = tid + CS_NT * k;
             if (q < a.f_chunks) {
-                const int e0 = q * 8;
+                const int e0 = q * VEC;
                 const int outer = fast_div(e0, a.magic_inner9), rem = e0 - outer * a.f_inner * 9;
                 int inner = (rem * 7282) >> 16;  // rem / 9 for rem < 2^15
                 int tap = rem - inner * 9;
                 const int m = a.f_transposed ? inner : outer, c = a.f_transposed ? outer : inner;
-                int at = m * a.b_pitch + ((a.f_transposed ? 8 - tap : tap) * CINP + c) * 2;
+                int at = m * a.b_pitch + ((a.f_transposed ? 8 - tap : tap) * CINP + c) * ES;
 #pragma unroll
-                for (int j = 0; j < 8; ++j) {
-                    *reinterpret_cast<half_t *>(F + at) = fin[k].e[j];
+                for (int j = 0; j < VEC; ++j) {
+                    *reinterpret_cast<T *>(F + at) = fin[k].e[j];
                     at += step_tap;
                     if (++tap == 9) {
                         tap = 0;
@@ -150,7 +155,7 @@ __device__ inline void conv_small_block(const ConvSmallArgs &a, int tile, char *
     // ---- jobs: 32 pixels x 32 filters
     const int kg = lane >> 5, lr = lane & 31;
     const int npix = min(a.R, a.Ho - y0) * a.Wo, jobs = a.pgroups << a.mshift;
-    const uint4 *T4 = reinterpret_cast<const uint4 *>(T);
+    const uint4 *T4 = reinterpret_cast<const uint4 *>(Tl);
     const size_t plane = (size_t)a.Ho * a.Wo;
     for (int job = wave; job < jobs; job += CS_NT / 64) {
         const int pg = job >> a.mshift, mb = job - (pg << a.mshift);
@@ -163,7 +168,7 @@ __device__ inline void conv_small_block(const ConvSmallArgs &a, int tile, char *
 #pragma unroll
         for (int v = 0; v < 16; ++v) acc[v] = 0.f;
 #pragma unroll
-        for (int ks = 0; ks < CINP / 16; ++ks) {
+        for (int ks = 0; ks < CINP / KSTEP; ++ks) {
             const uint4 *pk = prow + 2 * ks * a.POS;
 #pragma unroll
             for (int ky = 0; ky < 3; ++ky) {
@@ -171,18 +176,18 @@ __device__ inline void conv_small_block(const ConvSmallArgs &a, int tile, char *
 #pragma unroll
                 for (int kx = 0; kx < 3; ++kx) {
                     const uint4 pf = pr[kx];
-                    const uint4 ff = *reinterpret_cast<const uint4 *>(frow + ((ky * 3 + kx) * CINP + ks * 16) * 2);
-                    mfma_step<half_t>(acc, ff, pf);
+                    const uint4 ff = *reinterpret_cast<const uint4 *>(frow + ((ky * 3 + kx) * CINP + ks * KSTEP) * ES);
+                    mfma_step<T>(acc, ff, pf);
                 }
             }
         }
         if (pg * 32 + lr < npix) {
-            half_t *out = a.Y + (((size_t)b * a.Cout + mb * 32 + 4 * kg) * a.Ho + y0 + py) * a.Wo + px;
+            T *out = reinterpret_cast<T *>(a.Y) + (((size_t)b * a.Cout + mb * 32 + 4 * kg) * a.Ho + y0 + py) * a.Wo + px;
             const int left = a.Cout - mb * 32 - 4 * kg;  // filters from this lane's first one
 #pragma unroll
             for (int v = 0; v < 16; ++v) {
                 const int f = 8 * (v >> 2) + (v & 3);
-                if (f < left) out[f * plane] = (half_t)acc[v];
+                if (f < left) out[f * plane] = (T)acc[v];
             }
         }
     }
@@ -203,11 +208,11 @@ __device__ inline void conv_small_block(const ConvSmallArgs &a, int tile, char *
 constexpr int WG_CHUNKS = 4;  // 16-byte pieces per thread and tensor, at most
 
 struct WgSmallArgs {
-    const half_t *X, *dY;
+    const void *X, *dY;
     float *ws;
     int batch, Cin, Cout, Hin, Win, Ho, padU, padL;
     int nwg, S, R, tiles_per_img;  // workgroups; samples and output rows per tile (R = Ho when S > 1)
-    int G, RG, R2G;                // 8-column groups per row, per R rows, per R + 2 rows
+    int G, RG, R2G;                // 16-byte column groups per row, per R rows, per R + 2 rows
     int PY, PX, WP;                // LDS pitches in elements: gradient channel, input channel, input row
     int groups;                    // S * R * G
     int y_chunks, x_chunks, pad_chunks, pad_rows;  // pieces to copy; zero pieces (one per input row + one) and rows per channel
@@ -217,7 +222,29 @@ struct WgSmallArgs {
     int rows_kept, cols_kept, part_elems;  // filter rows and channels of a 32x32 tile that are stored; floats per workgroup in ws
 };
 
-// elements D .. D + 7 of a row of which c holds elements 0..7, p3 elements -2, -1 and n0 elements 8, 9
+// The two elements before and the two behind a 16-byte piece of a row: one dword of halves, two dwords of floats.
+template <typename T>
+struct EdgePair;
+template <>
+struct EdgePair<half_t> {
+    typedef unsigned type;
+};
+template <>
+struct EdgePair<float> {
+    typedef uint2 type;
+};
+
+// elements D .. D + 3 of a row of floats of which c holds elements 0..3, p elements -2, -1 and n elements 4, 5
+template <int D>
+__device__ inline uint4 shifted_piece(const uint4 &c, const uint2 &p, const uint2 &n) {
+    if constexpr (D == 0) return c;
+    if constexpr (D == -1) return make_uint4(p.y, c.x, c.y, c.z);
+    if constexpr (D == 1) return make_uint4(c.y, c.z, c.w, n.x);
+    if constexpr (D == -2) return make_uint4(p.x, p.y, c.x, c.y);
+    return make_uint4(c.z, c.w, n.x, n.y);
+}
+
+// elements D .. D + 7 of a row of halves of which c holds elements 0..7, p3 elements -2, -1 and n0 elements 8, 9
 template <int D>
 __device__ inline uint4 shifted_piece(const uint4 &c, unsigned p3, unsigned n0) {
     if constexpr (D == 0) return c;
@@ -231,11 +258,14 @@ __device__ inline uint4 shifted_piece(const uint4 &c, unsigned p3, unsigned n0) 
     return make_uint4(c.y, c.z, c.w, n0);
 }
 
-template <int PADL>
+template <typename T, int PADL>
 __device__ inline void wg_small_block(const WgSmallArgs &a, int wg, char *smem) {
+    constexpr int VEC = 16 / (int)sizeof(T);
+    typedef typename EdgePair<T>::type edge_t;
     const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    half_t *Ys = reinterpret_cast<half_t *>(smem);
-    half_t *Xs = Ys + a.Cout * a.PY;
+    T *Ys = reinterpret_cast<T *>(smem);
+    T *Xs = Ys + a.Cout * a.PY;
+    const T *gX = reinterpret_cast<const T *>(a.X), *gY = reinterpret_cast<const T *>(a.dY);
     // the tile: samples b0 .. b0 + S - 1, output rows y0 .. y0 + R - 1
     const int timg = wg / a.tiles_per_img;
     const int b0 = timg * a.S, y0 = (wg - timg * a.tiles_per_img) * a.R;
@@ -252,7 +282,7 @@ __device__ inline void wg_small_block(const WgSmallArgs &a, int wg, char *smem) 
             const int s = fast_div(rem, a.magic_rg), r2 = rem - s * a.RG;
             const int ly = fast_div(r2, a.magic_g), xg = r2 - ly * a.G;
             if (b0 + s < a.batch && y0 + ly < a.Ho)
-                yv[k] = *reinterpret_cast<const uint4 *>(a.dY + (((size_t)(b0 + s) * a.Cout + co) * a.Ho + y0 + ly) * a.Win + 8 * xg);
+                yv[k] = *reinterpret_cast<const uint4 *>(gY + (((size_t)(b0 + s) * a.Cout + co) * a.Ho + y0 + ly) * a.Win + VEC * xg);
         }
         if (q < a.x_chunks) {
             const int ci = fast_div(q, a.magic_xchan), rem = q - ci * xchan;
@@ -260,7 +290,7 @@ __device__ inline void wg_small_block(const WgSmallArgs &a, int wg, char *smem) 
             const int ly = fast_div(r2, a.magic_g), xg = r2 - ly * a.G;
             const int iy = y0 - a.padU + ly;
             if (b0 + s < a.batch && iy >= 0 && iy < a.Hin)
-                xv[k] = *reinterpret_cast<const uint4 *>(a.X + (((size_t)(b0 + s) * a.Cin + ci) * a.Hin + iy) * a.Win + 8 * xg);
+                xv[k] = *reinterpret_cast<const uint4 *>(gX + (((size_t)(b0 + s) * a.Cin + ci) * a.Hin + iy) * a.Win + VEC * xg);
         }
     }
     // zero pieces: in front of every input row and behind the last one; behind the last gradient group
@@ -269,18 +299,18 @@ __device__ inline void wg_small_block(const WgSmallArgs &a, int wg, char *smem) 
         *reinterpret_cast<uint4 *>(Xs + ci * a.PX + row * a.WP) = make_uint4(0, 0, 0, 0);
     }
     for (int co = tid; co < a.Cout; co += CS_NT)
-        *reinterpret_cast<uint4 *>(Ys + co * a.PY + a.groups * 8) = make_uint4(0, 0, 0, 0);
+        *reinterpret_cast<uint4 *>(Ys + co * a.PY + a.groups * VEC) = make_uint4(0, 0, 0, 0);
 #pragma unroll
     for (int k = 0; k < WG_CHUNKS; ++k) {
         const int q = tid + CS_NT * k;
         if (q < a.y_chunks) {
             const int co = fast_div(q, a.magic_ychan), rem = q - co * ychan;
-            *reinterpret_cast<uint4 *>(Ys + co * a.PY + rem * 8) = yv[k];
+            *reinterpret_cast<uint4 *>(Ys + co * a.PY + rem * VEC) = yv[k];
         }
         if (q < a.x_chunks) {
             const int ci = fast_div(q, a.magic_xchan), rem = q - ci * xchan;
             const int row = fast_div(rem, a.magic_g), xg = rem - row * a.G;  // row = s * (R + 2) + ly
-            *reinterpret_cast<uint4 *>(Xs + ci * a.PX + row * a.WP + 8 + 8 * xg) = xv[k];
+            *reinterpret_cast<uint4 *>(Xs + ci * a.PX + row * a.WP + VEC + VEC * xg) = xv[k];
         }
     }
     __syncthreads();
@@ -299,12 +329,12 @@ __device__ inline void wg_small_block(const WgSmallArgs &a, int wg, char *smem) 
         for (int v = 0; v < 16; ++v) acc[kx][v] = 0.f;
     if (active) {
         // filters and channels beyond the tensors repeat the last one (their rows and columns are never stored)
-        const half_t *yrow = Ys + min(cbo * 32 + lr, a.Cout - 1) * a.PY;
-        const half_t *xrow = Xs + min(cbi * 32 + lr, a.Cin - 1) * a.PX + ky * a.WP + 8;
+        const T *yrow = Ys + min(cbo * 32 + lr, a.Cout - 1) * a.PY;
+        const T *xrow = Xs + min(cbi * 32 + lr, a.Cin - 1) * a.PX + ky * a.WP + VEC;
         constexpr int U = 4;  // k steps whose LDS reads are in flight together
         for (int ks0 = kpart; ks0 < nks; ks0 += U * a.kparts) {
             uint4 A[U], C[U];
-            unsigned p3[U], n0[U];
+            edge_t p3[U], n0[U];
 #pragma unroll
             for (int u = 0; u < U; ++u) {
                 // (steps behind the last one read the zero piece of the gradient)
@@ -312,17 +342,17 @@ __device__ inline void wg_small_block(const WgSmallArgs &a, int wg, char *smem) 
                 const int gx = min(gi, a.groups - 1);
                 const int s = fast_div(gx, a.magic_rg), r2 = gx - s * a.RG;
                 const int ly = fast_div(r2, a.magic_g), xg = r2 - ly * a.G;
-                const half_t *xp = xrow + (s * (a.R + 2) + ly) * a.WP + 8 * xg;
-                A[u] = *reinterpret_cast<const uint4 *>(yrow + gi * 8);
+                const T *xp = xrow + (s * (a.R + 2) + ly) * a.WP + VEC * xg;
+                A[u] = *reinterpret_cast<const uint4 *>(yrow + gi * VEC);
                 C[u] = *reinterpret_cast<const uint4 *>(xp);
-                p3[u] = *reinterpret_cast<const unsigned *>(xp - 2);
-                n0[u] = *reinterpret_cast<const unsigned *>(xp + 8);
+                p3[u] = *reinterpret_cast<const edge_t *>(xp - 2);
+                n0[u] = *reinterpret_cast<const edge_t *>(xp + VEC);
             }
 #pragma unroll
             for (int u = 0; u < U; ++u) {
-                mfma_step<half_t>(acc[0], A[u], shifted_piece<0 - PADL>(C[u], p3[u], n0[u]));
-                mfma_step<half_t>(acc[1], A[u], shifted_piece<1 - PADL>(C[u], p3[u], n0[u]));
-                mfma_step<half_t>(acc[2], A[u], shifted_piece<2 - PADL>(C[u], p3[u], n0[u]));
+                mfma_step<T>(acc[0], A[u], shifted_piece<0 - PADL>(C[u], p3[u], n0[u]));
+                mfma_step<T>(acc[1], A[u], shifted_piece<1 - PADL>(C[u], p3[u], n0[u]));
+                mfma_step<T>(acc[2], A[u], shifted_piece<2 - PADL>(C[u], p3[u], n0[u]));
             }
         }
     }
@@ -363,65 +393,68 @@ __device__ inline void wg_small_block(const WgSmallArgs &a, int wg, char *smem) 
     }
 }
 
+template <typename T>
 __device__ inline void wg_small_any(const WgSmallArgs &a, int wg, char *smem) {
     if (a.padL == 1)
-        wg_small_block<1>(a, wg, smem);
+        wg_small_block<T, 1>(a, wg, smem);
     else if (a.padL == 0)
-        wg_small_block<0>(a, wg, smem);
+        wg_small_block<T, 0>(a, wg, smem);
     else
-        wg_small_block<2>(a, wg, smem);
+        wg_small_block<T, 2>(a, wg, smem);
 }
 
+template <typename T>
 __global__ __launch_bounds__(CS_NT) void wg_small_kernel(const WgSmallArgs a) {
     extern __shared__ __attribute__((aligned(16))) char smem[];
-    wg_small_any(a, blockIdx.x, smem);
+    wg_small_any<T>(a, blockIdx.x, smem);
 }
 
-template <int CINP, int F_MAX>
+template <typename T, int CINP, int F_MAX>
 __global__ __launch_bounds__(CS_NT) void conv_small_kernel(const ConvSmallArgs a) {
     extern __shared__ __attribute__((aligned(16))) char smem[];
-    conv_small_block<CINP, F_MAX>(a, blockIdx.x, smem);
+    conv_small_block<T, CINP, F_MAX>(a, blockIdx.x, smem);
 }
 
 // Weight gradient and input gradient of one layer in one launch: the first workgroups take the weight gradient's
 // sample ranges (the longer jobs), the rest the input gradient's tiles.
-template <int CINP, int F_MAX>
+template <typename T, int CINP, int F_MAX>
 __global__ __launch_bounds__(CS_NT) void conv_small_bw_kernel(const ConvSmallArgs ig, const WgSmallArgs wg) {
     extern __shared__ __attribute__((aligned(16))) char smem[];
     if ((int)blockIdx.x < wg.nwg)
-        wg_small_any(wg, blockIdx.x, smem);
+        wg_small_any<T>(wg, blockIdx.x, smem);
     else
-        conv_small_block<CINP, F_MAX>(ig, blockIdx.x - wg.nwg, smem);
+        conv_small_block<T, CINP, F_MAX>(ig, blockIdx.x - wg.nwg, smem);
 }
 
 constexpr size_t WG_SMALL_LDS = 4 * 9 * 4096;  // shares x blocks <= 4 tiles of nine taps
 
-template <int CINP, int F_MAX>
+template <typename T, int CINP, int F_MAX>
 int launch_small(const ConvSmallArgs &a, int tiles, size_t lds, hipStream_t s, const WgSmallArgs *wg) {
     state().last_conv_resident = 2;
     static bool attr_set = false;
     if (!attr_set) {
-        if (!hip_ok(hipFuncSetAttribute(reinterpret_cast<const void *>(conv_small_kernel<CINP, F_MAX>),
+        if (!hip_ok(hipFuncSetAttribute(reinterpret_cast<const void *>(conv_small_kernel<T, CINP, F_MAX>),
                                         hipFuncAttributeMaxDynamicSharedMemorySize, 150 * 1024),
                     "hipFuncSetAttribute") ||
-            !hip_ok(hipFuncSetAttribute(reinterpret_cast<const void *>(conv_small_bw_kernel<CINP, F_MAX>),
+            !hip_ok(hipFuncSetAttribute(reinterpret_cast<const void *>(conv_small_bw_kernel<T, CINP, F_MAX>),
                                         hipFuncAttributeMaxDynamicSharedMemorySize, 150 * 1024),
                     "hipFuncSetAttribute"))
             return 2;
         attr_set = true;
     }
     if (wg)
-        hipLaunchKernelGGL((conv_small_bw_kernel<CINP, F_MAX>), dim3(tiles + wg->nwg), dim3(CS_NT),
+        hipLaunchKernelGGL((conv_small_bw_kernel<T, CINP, F_MAX>), dim3(tiles + wg->nwg), dim3(CS_NT),
                            lds > WG_SMALL_LDS ? lds : WG_SMALL_LDS, s, a, *wg);
     else
-        hipLaunchKernelGGL((conv_small_kernel<CINP, F_MAX>), dim3(tiles), dim3(CS_NT), lds, s, a);
+        hipLaunchKernelGGL((conv_small_kernel<T, CINP, F_MAX>), dim3(tiles), dim3(CS_NT), lds, s, a);
     return hip_ok(hipGetLastError(), "small convolution launch") ? 0 : 2;
 }
 
 // dW(co, ci, tap) = sum over workgroups of ws[workgroup][block][tap][filter row][channel]: 64 consecutive partial
 // elements per workgroup of the reduction (coalesced reads), 16 groups of partials in parallel, eight loads in flight
 // per thread; the few results are scattered to the weight tensor's order.
-__global__ __launch_bounds__(1024) void wg_small_reduce_kernel(const float *__restrict__ ws, half_t *__restrict__ dW,
+template <typename T>
+__global__ __launch_bounds__(1024) void wg_small_reduce_kernel(const float *__restrict__ ws, T *__restrict__ dW,
                                                                int part_elems, int parts, int rows_kept,
                                                                int cols_kept, int cbi_n, int Cout, int Cin) {
     __shared__ float part_sum[16][64];
@@ -452,7 +485,7 @@ __global__ __launch_bounds__(1024) void wg_small_reduce_kernel(const float *__re
         const int tile = i / (rows_kept * cols_kept), r = i - tile * rows_kept * cols_kept;
         const int combo = tile / 9, tap = tile - combo * 9;
         const int co = (combo / cbi_n) * 32 + r / cols_kept, ci = (combo % cbi_n) * 32 + r % cols_kept;
-        if (co < Cout && ci < Cin) dW[(co * Cin + ci) * 9 + tap] = (half_t)s;
+        if (co < Cout && ci < Cin) dW[(co * Cin + ci) * 9 + tap] = (T)s;
     }
 }
 
@@ -463,16 +496,18 @@ struct SmallPlan {
 };
 
 // Fills the forward / input-gradient launch for `cu_budget` compute units; -1 when the layer does not fit.
+template <typename T>
 int plan_small(const ConvTileDesc &d, const void *X, const void *Wt, void *Y, int cu_budget, SmallPlan &p) {
+    constexpr int ES = (int)sizeof(T), VEC = 16 / ES, RPI = 64 / VEC;  // element size, elements per piece, rows per item
     State &st = state();
     if (st.gemm_path != 0 && st.gemm_path != 6) return -1;  // (the other values select one of the other routes)
     if (d.in_hwc || d.KH != 3 || d.KW != 3 || d.sh != d.sw || d.sh < 1 || d.sh > 2) return -1;
-    if (d.Cin > 64 || d.Cout > 64 || d.Win % 8 != 0 || d.x_sy != d.Win) return -1;
+    if (d.Cin > 64 || d.Cout > 64 || d.Win % VEC != 0 || d.x_sy != d.Win) return -1;
     if (d.x_sc != (long long)d.Hin * d.Win || d.x_sb != (long long)d.Cin * d.Hin * d.Win) return -1;
     if (d.padU < 0 || d.padU > 2 || d.padL < 0 || d.padL > 2 || d.padD < 0 || d.padR < 0 || d.padR > 8) return -1;
     if (reinterpret_cast<uintptr_t>(X) % 16 || reinterpret_cast<uintptr_t>(Wt) % 16) return -1;
     const long long f_elems = (long long)d.Cout * d.Cin * 9;
-    if (f_elems % 8 != 0) return -1;
+    if (f_elems % VEC != 0) return -1;
     ConvSmallArgs &a = p.a;
     a = ConvSmallArgs();
     // dense filter tensor [outer][inner][3][3]: forward (filter, channel), or the input gradient's view of it
@@ -490,15 +525,15 @@ int plan_small(const ConvTileDesc &d, const void *X, const void *Wt, void *Y, in
     const int Hd = (d.Hin - 1) * dil + 1, Wd = (d.Win - 1) * dil + 1;  // the image the taps walk over
     const int s = d.sh, TW = Wd + d.padL + d.padR, THP = Hd + d.padU + d.padD;
     if ((d.Wo - 1) * s + 3 > TW || (d.Ho - 1) * s + 3 > THP || d.Wo >= 65536 || d.Ho * d.Wo >= 65536) return -1;
-    const int cinp = d.Cin <= 16 ? 16 : d.Cin <= 32 ? 32 : 64, cblocks = cinp / 8;
+    const int cinp = d.Cin <= 16 ? 16 : d.Cin <= 32 ? 32 : 64, cblocks = cinp / VEC;
     const int mblocks = (d.Cout + 31) / 32;
     // rows per workgroup: the whole image, halved while that leaves the four waves a job each and the chip is not full
     int R = d.Ho;
     auto jobs_of = [&](int r) { return ((r * d.Wo + 31) / 32) * mblocks; };
     while ((long long)d.batch * ((d.Ho + R - 1) / R) < cu_budget && R % 2 == 0 && jobs_of(R / 2) >= 4) R /= 2;
-    auto items_of = [&](int r) { return cblocks * (d.Win / 8) * ((((r - 1) * s + 3) + 7) / 8); };
+    auto items_of = [&](int r) { return cblocks * (d.Win / VEC) * ((((r - 1) * s + 3) + RPI - 1) / RPI); };
     auto lds_of = [&](int r) { return (size_t)cblocks * ((r - 1) * s + 3) * TW * 16; };
-    const int pitch = 9 * cinp * 2 + 16;
+    const int pitch = 9 * cinp * ES + 16;  // (an odd multiple of 16 bytes)
     const size_t f_bytes = (size_t)mblocks * 32 * pitch;
     while (R > 1 && (items_of(R) > CS_ITEMS || f_bytes + lds_of(R) > 150 * 1024)) R = (R + 1) / 2;
     if (items_of(R) > CS_ITEMS || f_bytes + lds_of(R) > 150 * 1024) return -1;
@@ -506,27 +541,28 @@ int plan_small(const ConvTileDesc &d, const void *X, const void *Wt, void *Y, in
     // beyond a few workgroups per CU the persistent kernels (filters loaded once per workgroup) are ahead
     if (st.gemm_path != 6 && tiles > 4LL * st.num_cu) return -1;
     if (tiles >= (1LL << 31) / 256) return -1;
-    a.X = reinterpret_cast<const half_t *>(X);
-    a.Wt = reinterpret_cast<const half_t *>(Wt);
-    a.Y = reinterpret_cast<half_t *>(Y);
+    a.X = X;
+    a.Wt = Wt;
+    a.Y = Y;
     a.Cin = d.Cin; a.Cout = d.Cout; a.Hin = d.Hin; a.Win = d.Win; a.Ho = d.Ho; a.Wo = d.Wo;
     a.s = s; a.padU = d.padU; a.padL = d.padL;
     a.dil = dil;
     a.R = R; a.tiles_per_img = (d.Ho + R - 1) / R;
     a.RR = (R - 1) * s + 3; a.TW = TW; a.POS = a.RR * TW;
-    const int G = d.Win / 8, RR8 = (a.RR + 7) / 8;
-    a.items = cblocks * G * RR8;
+    const int G = d.Win / VEC, RRB = (a.RR + RPI - 1) / RPI;
+    a.items = cblocks * G * RRB;
     for (int item = 0; item < a.items; ++item) {
-        const int rblk = item % RR8, t = item / RR8, g = t % G, cb = t / G;
-        a.item_g[item] = (cb * 8 * d.Hin + rblk * 8) * d.Win + 8 * g;
-        a.item_l[item] = ((cb * a.POS + rblk * 8 * TW) + d.padL + dil * 8 * g) * 8;
-        a.item_rc[item] = (rblk * 8) | ((cb * 8) << 8) | (g << 16);
+        const int rblk = item % RRB, t = item / RRB, g = t % G, cb = t / G;
+        a.item_g[item] = (cb * VEC * d.Hin + rblk * RPI) * d.Win + VEC * g;
+        a.item_l[item] = ((cb * a.POS + rblk * RPI * TW) + d.padL + dil * VEC * g) * VEC;
+        a.item_rc[item] = (rblk * RPI) | ((cb * VEC) << 8) | (g << 16);
     }
+    if (a.RR + RPI > 255) return -1;  // (rows are 8 bits of item_rc)
     a.halo_w = dil == 2 ? 1 : TW - d.Win;  // (a zero-stuffed input zeroes its whole tile instead)
     a.halo_chunks = cblocks * a.RR * a.halo_w;
     a.magic_halo_w = magic_of(a.halo_w);
     a.magic_rr = magic_of(a.RR);
-    a.f_chunks = (int)(f_elems / 8);
+    a.f_chunks = (int)(f_elems / VEC);
     a.magic_inner9 = magic_of(a.f_inner * 9);
     a.magic_wo = magic_of(d.Wo);
     a.b_pitch = pitch; a.f_bytes = (int)f_bytes;
@@ -541,21 +577,24 @@ int plan_small(const ConvTileDesc &d, const void *X, const void *Wt, void *Y, in
     return 0;
 }
 
+template <typename T>
 int dispatch_small(const SmallPlan &p, const WgSmallArgs *wg) {
     hipStream_t s = state().stream;
     if (p.cinp == 16)
-        return p.per_thread <= 1 ? launch_small<16, 1>(p.a, p.tiles, p.lds, s, wg) : launch_small<16, 2>(p.a, p.tiles, p.lds, s, wg);
+        return p.per_thread <= 1 ? launch_small<T, 16, 1>(p.a, p.tiles, p.lds, s, wg) : launch_small<T, 16, 2>(p.a, p.tiles, p.lds, s, wg);
     if (p.cinp == 32)
-        return p.per_thread <= 2 ? launch_small<32, 2>(p.a, p.tiles, p.lds, s, wg) : launch_small<32, 3>(p.a, p.tiles, p.lds, s, wg);
-    return p.per_thread <= 3 ? launch_small<64, 3>(p.a, p.tiles, p.lds, s, wg) : launch_small<64, 5>(p.a, p.tiles, p.lds, s, wg);
+        return p.per_thread <= 2 ? launch_small<T, 32, 2>(p.a, p.tiles, p.lds, s, wg) : launch_small<T, 32, 3>(p.a, p.tiles, p.lds, s, wg);
+    return p.per_thread <= 3 ? launch_small<T, 64, 3>(p.a, p.tiles, p.lds, s, wg) : launch_small<T, 64, 5>(p.a, p.tiles, p.lds, s, wg);
 }
 
 // Fills the weight-gradient launch of the forward layer `d` (partial sums in the workspace); -1 when it does not fit.
+template <typename T>
 int plan_wg(const ConvTileDesc &d, const void *X, const void *dY, int max_wg, bool alone, WgSmallArgs &w) {
+    constexpr int ES = (int)sizeof(T), VEC = 16 / ES;
     State &st = state();
     if (st.gemm_path != 0 && st.gemm_path != 6) return -1;  // (the other values select one of the other routes)
     if (d.in_hwc || d.KH != 3 || d.KW != 3 || d.sh != 1 || d.sw != 1) return -1;
-    if (d.Cin > 64 || d.Cout > 64 || d.Win % 8 != 0 || d.Wo != d.Win || d.x_sy != d.Win) return -1;
+    if (d.Cin > 64 || d.Cout > 64 || d.Win % VEC != 0 || d.Wo != d.Win || d.x_sy != d.Win) return -1;
     if (d.x_sc != (long long)d.Hin * d.Win || d.x_sb != (long long)d.Cin * d.Hin * d.Win) return -1;
     if (d.padU < 0 || d.padL < 0 || d.padL > 2) return -1;
     if (reinterpret_cast<uintptr_t>(X) % 16 || reinterpret_cast<uintptr_t>(dY) % 16) return -1;
@@ -568,12 +607,13 @@ int plan_wg(const ConvTileDesc &d, const void *X, const void *dY, int max_wg, bo
     // against 8.4 us for 16 -> 32 on 32x32 at one sample: below a few thousand positions what this kernel buys is
     // the input gradient riding along in the same launch)
     if (st.gemm_path != 6 && (positions > 262144 || (alone && positions < 8192))) return -1;
-    w.G = d.Win / 8;
-    w.WP = d.Win + 8;
-    auto round_pitch = [](int n) { return n + ((8 - n % 64) + 64) % 64; };  // = 8 mod 64: rows 16 bytes apart in the banks
+    w.G = d.Win / VEC;
+    w.WP = d.Win + VEC;
+    // pitches of 16 bytes mod 128: consecutive channels 16 bytes apart in the banks
+    auto round_pitch = [](int n) { return n + ((VEC - n % (8 * VEC)) + 8 * VEC) % (8 * VEC); };
     auto lds_of = [&](int S, int R) {
-        const int py = round_pitch(S * R * d.Win + 8), px = round_pitch((S * (R + 2) + 1) * w.WP);
-        return ((size_t)d.Cout * py + (size_t)d.Cin * px) * 2;
+        const int py = round_pitch(S * R * d.Win + VEC), px = round_pitch((S * (R + 2) + 1) * w.WP);
+        return ((size_t)d.Cout * py + (size_t)d.Cin * px) * ES;
     };
     auto chunks_ok = [&](int S, int R) {
         return (long long)d.Cout * S * R * w.G <= WG_CHUNKS * CS_NT && (long long)d.Cin * S * (R + 2) * w.G <= WG_CHUNKS * CS_NT &&
@@ -595,7 +635,7 @@ int plan_wg(const ConvTileDesc &d, const void *X, const void *dY, int max_wg, bo
     w.nwg = ((d.batch + S - 1) / S) * w.tiles_per_img;
     w.RG = R * w.G; w.R2G = (R + 2) * w.G;
     w.groups = S * w.RG;
-    w.PY = round_pitch(w.groups * 8 + 8);
+    w.PY = round_pitch(w.groups * VEC + VEC);
     w.pad_rows = S * (R + 2) + 1;
     w.PX = round_pitch(w.pad_rows * w.WP);
     w.y_chunks = d.Cout * w.groups;
@@ -616,53 +656,66 @@ int plan_wg(const ConvTileDesc &d, const void *X, const void *dY, int max_wg, bo
     w.part_elems = w.combos * 9 * w.rows_kept * w.cols_kept;
     w.magic_tile = magic_of(w.rows_kept * w.cols_kept);
     w.magic_cols = magic_of(w.cols_kept);
-    w.X = reinterpret_cast<const half_t *>(X);
-    w.dY = reinterpret_cast<const half_t *>(dY);
+    w.X = X;
+    w.dY = dY;
     w.batch = d.batch; w.Cin = d.Cin; w.Cout = d.Cout; w.Hin = d.Hin; w.Win = d.Win; w.Ho = d.Ho;
     w.padU = d.padU; w.padL = d.padL;
     w.ws = workspace((size_t)w.nwg * w.part_elems * sizeof(float));
     return w.ws ? 0 : 2;
 }
 
+template <typename T>
 int reduce_wg(const WgSmallArgs &w, void *dW) {
-    hipLaunchKernelGGL(wg_small_reduce_kernel, dim3((w.part_elems + 63) / 64), dim3(1024), 0, state().stream, w.ws,
-                       reinterpret_cast<half_t *>(dW), w.part_elems, w.nwg, w.rows_kept, w.cols_kept, w.cbi_n, w.Cout, w.Cin);
+    hipLaunchKernelGGL(wg_small_reduce_kernel<T>, dim3((w.part_elems + 63) / 64), dim3(1024), 0, state().stream, w.ws,
+                       reinterpret_cast<T *>(dW), w.part_elems, w.nwg, w.rows_kept, w.cols_kept, w.cbi_n, w.Cout, w.Cin);
     return hip_ok(hipGetLastError(), "small weight gradient reduction launch") ? 0 : 2;
 }
 
 }  // namespace
 
+template <typename T>
 int conv_small(const ConvTileDesc &d, const void *X, const void *Wt, void *Y) {
     SmallPlan p;
-    if (int rc = plan_small(d, X, Wt, Y, state().num_cu, p)) return rc;
-    return dispatch_small(p, nullptr);
+    if (int rc = plan_small<T>(d, X, Wt, Y, state().num_cu, p)) return rc;
+    return dispatch_small<T>(p, nullptr);
 }
 
+template <typename T>
 int conv_small_wg(const ConvTileDesc &d, const void *X, const void *dY, void *dW) {
     WgSmallArgs w;
-    if (int rc = plan_wg(d, X, dY, state().num_cu, true, w)) return rc;
+    if (int rc = plan_wg<T>(d, X, dY, state().num_cu, true, w)) return rc;
     static bool attr_set = false;
     if (!attr_set) {
-        if (!hip_ok(hipFuncSetAttribute(reinterpret_cast<const void *>(wg_small_kernel),
+        if (!hip_ok(hipFuncSetAttribute(reinterpret_cast<const void *>(wg_small_kernel<T>),
                                         hipFuncAttributeMaxDynamicSharedMemorySize, 150 * 1024),
                     "hipFuncSetAttribute"))
             return 2;
         attr_set = true;
     }
-    hipLaunchKernelGGL(wg_small_kernel, dim3(w.nwg), dim3(CS_NT), WG_SMALL_LDS, state().stream, w);
+    hipLaunchKernelGGL(wg_small_kernel<T>, dim3(w.nwg), dim3(CS_NT), WG_SMALL_LDS, state().stream, w);
     if (!hip_ok(hipGetLastError(), "small weight gradient launch")) return 2;
-    return reduce_wg(w, dW);
+    return reduce_wg<T>(w, dW);
 }
 
+template <typename T>
 int conv_small_bw(const ConvTileDesc &fwd, const ConvTileDesc &ig, const void *X, const void *dY, const void *Wt,
                   void *dW, void *dX) {
     WgSmallArgs w;
-    if (int rc = plan_wg(fwd, X, dY, state().num_cu / 2, false, w)) return rc;
+    if (int rc = plan_wg<T>(fwd, X, dY, state().num_cu / 2, false, w)) return rc;
     SmallPlan p;
     const int budget = state().num_cu - w.nwg;
-    if (int rc = plan_small(ig, dY, Wt, dX, budget > 32 ? budget : 32, p)) return rc;
-    if (int rc = dispatch_small(p, &w)) return rc;
-    return reduce_wg(w, dW);
+    if (int rc = plan_small<T>(ig, dY, Wt, dX, budget > 32 ? budget : 32, p)) return rc;
+    if (int rc = dispatch_small<T>(p, &w)) return rc;
+    return reduce_wg<T>(w, dW);
 }
+
+template int conv_small<half_t>(const ConvTileDesc &, const void *, const void *, void *);
+template int conv_small<float>(const ConvTileDesc &, const void *, const void *, void *);
+template int conv_small_wg<half_t>(const ConvTileDesc &, const void *, const void *, void *);
+template int conv_small_wg<float>(const ConvTileDesc &, const void *, const void *, void *);
+template int conv_small_bw<half_t>(const ConvTileDesc &, const ConvTileDesc &, const void *, const void *, const void *,
+                                   void *, void *);
+template int conv_small_bw<float>(const ConvTileDesc &, const ConvTileDesc &, const void *, const void *, const void *,
+                                  void *, void *);
 
 }  // namespace ptl

@@ -30,13 +30,16 @@ struct ConvTileDesc {
 template <typename T>
 int conv_tile(const ConvTileDesc &d, const void *X, const void *Wt, void *Y, const OutMap &c);
 
-// 3x3 fp16 layers with at most 64 channels on either side, dense channel-major tensors: one launch that reads the
+// 3x3 layers with at most 64 channels on either side, dense channel-major tensors: one launch that reads the
 // caller's tensors directly (ptl_conv_small.hip).  Y is the dense channel-major output [batch][Cout][Ho][Wo].
 // Returns -1 when the layer does not fit or is large enough for the persistent kernels to be ahead.
+template <typename T>
 int conv_small(const ConvTileDesc &d, const void *X, const void *Wt, void *Y);
 // Weight gradient of such a layer (unit stride, output as wide as the input), and weight + input gradient with the
 // two products in one launch (`fwd` describes the forward layer, `ig` the input gradient as a forward pass over dY).
+template <typename T>
 int conv_small_wg(const ConvTileDesc &d, const void *X, const void *dY, void *dW);
+template <typename T>
 int conv_small_bw(const ConvTileDesc &fwd, const ConvTileDesc &ig, const void *X, const void *dY, const void *Wt,
                   void *dW, void *dX);
 

@@ -272,7 +272,7 @@ static int conv2d_fw(const Args *a, int ns, const char *fn) {
             c.n = axis_plain(ns * P, g.Co);
             c.m = axis_plain(g.Co, 1);
         }
-        if (sizeof(T) == 2 && !g.hwc) rc = conv_small(d, X, Wt, Y);
+        if (!g.hwc) rc = conv_small<T>(d, X, Wt, Y);
         if (rc < 0) rc = conv_taps<T>(d, X, Wt, Y, c);
         if (rc < 0) rc = conv_tile<T>(d, X, Wt, Y, c);
         if (rc > 0) return sg.finish(rc);
@@ -362,7 +362,7 @@ static int conv2d_wg(const Args *a, int ns, const char *fn) {
                                 (long long)ns * g.Ho * g.Wo >= 16384;
         if (g.hwc) {  // channel-minor tensors: the sum over taps from 64 channels on, else the gathering GEMM below
             rc = conv_taps_wg<T>(d, X, dY, dW);
-        } else if (sizeof(T) == 2 && (rc = conv_small_wg(d, X, dY, dW)) >= 0) {
+        } else if ((rc = conv_small_wg<T>(d, X, dY, dW)) >= 0) {
             // (small 3x3 layers: one launch for the partial sums over sample ranges, one to add them)
         } else {
             const bool tiles_resident = sizeof(T) == 2 && state().gemm_path == 0 && conv_halo_wg_preferred(d);
@@ -478,7 +478,7 @@ static int conv2d_ig(const Args *a, int ns, const char *fn) {
     }
 
     // Small fp16 stride-2 layers: the small-layer kernel stuffs the zeros while it fills its LDS tile.
-    if (sizeof(T) == 2 && !g.hwc && g.sh == 2 && g.sw == 2 && g.Hk == 3 && g.Wk == 3) {
+    if (!g.hwc && g.sh == 2 && g.sw == 2 && g.Hk == 3 && g.Wk == 3) {
         ConvTileDesc d = {};
         d.batch = ns; d.Cin = g.Co; d.Hin = g.Ho; d.Win = g.Wo; d.in_dil = 2;
         d.Cout = g.Ci; d.Ho = g.H; d.Wo = g.W;
@@ -489,7 +489,7 @@ static int conv2d_ig(const Args *a, int ns, const char *fn) {
         d.w_base = Pk - 1; d.w_sm = Pk; d.w_sc = g.Ci * Pk; d.w_sy = -g.Wk; d.w_sx = -1;
         state().last_conv_direct = 0;
         state().last_conv_resident = 0;
-        const int rc = conv_small(d, dY, Wt, dX);
+        const int rc = conv_small<T>(d, dY, Wt, dX);
         if (rc == 0) state().last_conv_direct = 1;
         if (rc >= 0) return sg.finish(rc);
     }
@@ -539,7 +539,7 @@ static int conv2d_ig(const Args *a, int ns, const char *fn) {
             c.m = axis_plain(g.Ci, 1);
         }
         // (the zero-stuffed gradient of a strided layer lives in the scratch buffer the tap route would reuse)
-        int rc = (sizeof(T) == 2 && !g.hwc) ? conv_small(d, dY, Wt, dX) : -1;
+        int rc = !g.hwc ? conv_small<T>(d, dY, Wt, dX) : -1;
         if (rc < 0 && g.sh == 1 && g.sw == 1) rc = conv_taps<T>(d, dY, Wt, dX, c);
         if (rc < 0) rc = conv_tile<T>(d, dY, Wt, dX, c);
         if (rc == 0) state().last_conv_direct = 1;
@@ -638,7 +638,7 @@ static int conv2d_bw(const Args *a, int ns, const char *fn) {
         return 1;
     }
     const bool wg = a->skip_wg_grad == 0, ig = a->skip_in_grad == 0;
-    if (wg && ig && sizeof(T) == 2 && a->USE_BIASES != 1 && ns >= 1 && a->input && a->coeff && a->output) {
+    if (wg && ig && a->USE_BIASES != 1 && ns >= 1 && a->input && a->coeff && a->output) {
         ConvGeom g;
         if (int rc = conv_geom(a, g, fn, true)) return rc;
         const int P = g.Ho * g.Wo, Pk = g.Hk * g.Wk, K = g.Ci * Pk;
@@ -661,8 +661,8 @@ static int conv2d_bw(const Args *a, int ns, const char *fn) {
             b.x_sb = (long long)g.Co * P; b.x_sc = P; b.x_sy = g.Wo;
             b.w_base = Pk - 1; b.w_sm = Pk; b.w_sc = g.Ci * Pk; b.w_sy = -g.Wk; b.w_sx = -1;
             // small layers: both products in one launch; wide layers: one shared copy of the output gradient
-            const bool small = g.Ci <= 64 && g.Co <= 64 && g.W % 8 == 0 && state().gemm_path != 5;
-            const bool wide = ns > 1 && state().gemm_path != 6 && conv_halo_wg_preferred(f);
+            const bool small = g.Ci <= 64 && g.Co <= 64 && g.W % (16 / (int)sizeof(T)) == 0 && state().gemm_path != 5;
+            const bool wide = sizeof(T) == 2 && ns > 1 && state().gemm_path != 6 && conv_halo_wg_preferred(f);
             if (small || wide) {
                 Stager sg;
                 const T *X = sg.in(reinterpret_cast<const T *>(a->input->data), in_n);
@@ -673,7 +673,7 @@ static int conv2d_bw(const Args *a, int ns, const char *fn) {
                 if (sg.failed()) return 2;
                 state().last_conv_direct = 0;
                 state().last_conv_resident = 0;
-                int rc = small ? conv_small_bw(f, b, X, dY, Wt, dW, dX) : -1;
+                int rc = small ? conv_small_bw<T>(f, b, X, dY, Wt, dW, dX) : -1;
                 if (rc < 0 && wide) rc = conv_halo_bw<T>(f, b, X, dY, Wt, dW, dX);
                 if (rc >= 0) {
                     if (rc == 0) state().last_conv_direct = 1;

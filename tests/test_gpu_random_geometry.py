@@ -17,7 +17,7 @@ pytestmark = pytest.mark.gpu
 
 
 def rel(got, ref):
-    return float((got.float() - ref).norm() / (ref.norm() + 1e-20))
+    return float((got.to(ref.dtype) - ref).norm() / (ref.norm() + 1e-20))
 
 
 @pytest.mark.parametrize("seed", [11, 12, 13])
@@ -54,25 +54,26 @@ def test_conv2d_resident_tile_random_geometries(pkg, gpu, seed):
             assert rel(got, ref) <= 2e-3, (case, name)
 
 
-@pytest.mark.parametrize("seed", [31, 32, 33])
-def test_conv2d_small_layer_kernel_random_geometries(pkg, gpu, seed):
-    """The single-launch kernel for small 3x3 fp16 layers (forced with path 6): channel counts that are not whole
+@pytest.mark.parametrize("dt,seed", [("fp16", 31), ("fp16", 32), ("fp16", 33), ("fp32", 34), ("fp32", 35)])
+def test_conv2d_small_layer_kernel_random_geometries(pkg, gpu, dt, seed):
+    """The single-launch kernels for small 3x3 layers (forced with path 6): channel counts that are not whole
     blocks (3, 24, 40 ...), strides 1 and 2, paddings 0..2 per side, rows of 8..64 elements, ragged last row tiles."""
     rng = random.Random(seed)
+    tdt, tol = (torch.float16, 2e-3) if dt == "fp16" else (torch.float32, 2e-5)
     ran = 0
     for it in range(16):
         Ci, Co = rng.choice([3, 8, 16, 24, 32, 48, 64]), rng.choice([8, 16, 24, 32, 40, 64])
         st = rng.choice([1, 1, 2])
         pl, pr, pu, pd = (rng.randint(0, 2) for _ in range(4))
-        W, H = rng.choice([8, 16, 24, 32, 40, 64]), rng.randint(3, 36)
+        W, H = rng.choice([8, 16, 24, 32, 40, 64] if dt == "fp16" else [8, 12, 16, 20, 32, 40]), rng.randint(3, 36)
         if st == 2:  # the strides must divide the padded extents minus the filter
             pr += (W + pl + pr - 3) % 2
             pd += (H + pu + pd - 3) % 2
         ns = rng.choice([1, 2, 3, 7, 32, 130])
         Ho, Wo = (H + pu + pd - 3) // st + 1, (W + pl + pr - 3) // st + 1
-        x = (torch.rand(ns, Ci, H, W, device="cuda") - 0.5).half()
-        w = ((torch.rand(Co, Ci, 3, 3, device="cuda") - 0.5) * 0.5).half()
-        dy = (torch.rand(ns, Co, Ho, Wo, device="cuda") - 0.5).half()
+        x = (torch.rand(ns, Ci, H, W, device="cuda") - 0.5).to(tdt)
+        w = ((torch.rand(Co, Ci, 3, 3, device="cuda") - 0.5) * 0.5).to(tdt)
+        dy = (torch.rand(ns, Co, Ho, Wo, device="cuda") - 0.5).to(tdt)
         y, dx, dw = torch.full_like(dy, 3), torch.full_like(x, 3), torch.full_like(w, 3)
         dx2, dw2 = torch.full_like(x, 3), torch.full_like(w, 3)
         a, keep = hp.conv2d_args(pkg, x, dx, w, dw, y, dy, Ci, H, W, Co, 3, 3, Ho, Wo, (pl, pr, pu, pd), (st, st))
@@ -80,51 +81,53 @@ def test_conv2d_small_layer_kernel_random_geometries(pkg, gpu, seed):
         case = (Ci, Co, H, W, (pl, pr, pu, pd), st, ns)
         gpu.ptl_set_gemm_path(6)
         try:
-            pkg.call("ptl_conv2d_fp16_fw_batched", a, ns)
+            pkg.call("ptl_conv2d_%s_fw_batched" % dt, a, ns)
             small_fw = gpu.ptl_last_conv_resident() == 2
-            pkg.call("ptl_conv2d_fp16_ig_batched", a, ns)
+            pkg.call("ptl_conv2d_%s_ig_batched" % dt, a, ns)
             small_ig = gpu.ptl_last_conv_resident() == 2
             # the weight gradient (alone, and with the input gradient in the same launch): whatever route takes it
-            pkg.call("ptl_conv2d_fp16_wg_batched", a, ns)
-            pkg.call("ptl_conv2d_fp16_bw_batched", a2, ns)
+            pkg.call("ptl_conv2d_%s_wg_batched" % dt, a, ns)
+            pkg.call("ptl_conv2d_%s_bw_batched" % dt, a2, ns)
         finally:
             gpu.ptl_set_gemm_path(0)
         gpu.ptl_sync()
         # the kernel fits when the filter tensor is whole 16-byte pieces and one row of every channel block is at most
-        # 32 wave-wide loads; the input gradient sees the output gradient as its input (zero-stuffed in the kernel for a
+        # 64 wave-wide loads; the input gradient sees the output gradient as its input (zero-stuffed in the kernel for a
         # stride-2 layer), whose rows must be whole pieces too
         blocks = lambda c: (16 if c <= 16 else 32 if c <= 32 else 64) // 8
-        assert small_fw == ((Ci * Co * 9) % 8 == 0 and blocks(Ci) * (W // 8) <= 32), case
-        assert small_ig == (Wo % 8 == 0 and (Ci * Co * 9) % 8 == 0 and blocks(Co) * (Wo // 8) <= 32), case
+        if dt == "fp16":
+            assert small_fw == ((Ci * Co * 9) % 8 == 0 and blocks(Ci) * (W // 8) <= 64), case
+            assert small_ig == (Wo % 8 == 0 and (Ci * Co * 9) % 8 == 0 and blocks(Co) * (Wo // 8) <= 64), case
         ran += small_fw + small_ig
-        xp = F.pad(x.float(), (pl, pr, pu, pd))
-        ref_y = F.conv2d(xp, w.float(), stride=st)
-        ref_dx = torch.nn.grad.conv2d_input(xp.shape, w.float(), dy.float(), stride=st)[:, :, pu:pu + H, pl:pl + W]
-        ref_dw = torch.nn.grad.conv2d_weight(xp, w.shape, dy.float(), stride=st)
-        assert rel(y, ref_y) <= 2e-3, (case, "y")
-        assert rel(dx, ref_dx) <= 2e-3, (case, "dx")
-        assert rel(dw, ref_dw) <= 2e-3, (case, "dw")
-        assert rel(dx2, ref_dx) <= 2e-3, (case, "dx, one call")
-        assert rel(dw2, ref_dw) <= 2e-3, (case, "dw, one call")
-    assert ran >= 12
+        xp = F.pad(x.double(), (pl, pr, pu, pd))
+        ref_y = F.conv2d(xp, w.double(), stride=st)
+        ref_dx = torch.nn.grad.conv2d_input(xp.shape, w.double(), dy.double(), stride=st)[:, :, pu:pu + H, pl:pl + W]
+        ref_dw = torch.nn.grad.conv2d_weight(xp, w.shape, dy.double(), stride=st)
+        assert rel(y, ref_y) <= tol, (case, "y")
+        assert rel(dx, ref_dx) <= tol, (case, "dx")
+        assert rel(dw, ref_dw) <= tol, (case, "dw")
+        assert rel(dx2, ref_dx) <= tol, (case, "dx, one call")
+        assert rel(dw2, ref_dw) <= tol, (case, "dw, one call")
+    assert ran >= (12 if dt == "fp16" else 8)
 
 
-@pytest.mark.parametrize("seed", [41, 42])
-def test_conv2d_small_layer_weight_gradient_random_geometries(pkg, gpu, seed):
+@pytest.mark.parametrize("dt,seed", [("fp16", 41), ("fp16", 42), ("fp32", 43), ("fp32", 44)])
+def test_conv2d_small_layer_weight_gradient_random_geometries(pkg, gpu, dt, seed):
     """Unit-stride 3x3 fp16 layers whose output is as wide as the input (the geometries the small-layer weight-gradient
     kernel takes, forced with path 6): weight gradient alone and together with the input gradient, tiles of several
     samples (64 channels), split rows (few samples), ragged last tiles, all three left paddings."""
     rng = random.Random(seed)
+    tdt, tol, vec = (torch.float16, 2e-3, 8) if dt == "fp16" else (torch.float32, 2e-5, 4)
     for it in range(14):
         Ci, Co = rng.choice([3, 8, 16, 24, 32, 64]), rng.choice([8, 16, 32, 40, 64])
         pl = rng.randint(0, 2)
         pr, pu, pd = 2 - pl, rng.randint(0, 2), rng.randint(0, 2)
-        W, H = rng.choice([8, 16, 24, 32]), rng.randint(max(3 - pu - pd, 1), 34)
+        W, H = rng.choice([8, 16, 24, 32] if dt == "fp16" else [8, 12, 16, 20, 32]), rng.randint(max(3 - pu - pd, 1), 34)
         ns = rng.choice([1, 2, 5, 9, 32, 130])
         Ho, Wo = H + pu + pd - 2, W
-        x = (torch.rand(ns, Ci, H, W, device="cuda") - 0.5).half()
-        w = ((torch.rand(Co, Ci, 3, 3, device="cuda") - 0.5) * 0.5).half()
-        dy = (torch.rand(ns, Co, Ho, Wo, device="cuda") - 0.5).half()
+        x = (torch.rand(ns, Ci, H, W, device="cuda") - 0.5).to(tdt)
+        w = ((torch.rand(Co, Ci, 3, 3, device="cuda") - 0.5) * 0.5).to(tdt)
+        dy = (torch.rand(ns, Co, Ho, Wo, device="cuda") - 0.5).to(tdt)
         y, dx, dw = torch.full_like(dy, 3), torch.full_like(x, 3), torch.full_like(w, 3)
         dx2, dw2 = torch.full_like(x, 3), torch.full_like(w, 3)
         a, keep = hp.conv2d_args(pkg, x, dx, w, dw, y, dy, Ci, H, W, Co, 3, 3, Ho, Wo, (pl, pr, pu, pd), (1, 1))
@@ -132,18 +135,19 @@ def test_conv2d_small_layer_weight_gradient_random_geometries(pkg, gpu, seed):
         case = (Ci, Co, H, W, (pl, pr, pu, pd), ns)
         gpu.ptl_set_gemm_path(6)
         try:
-            pkg.call("ptl_conv2d_fp16_wg_batched", a, ns)
-            pkg.call("ptl_conv2d_fp16_bw_batched", a2, ns)
-            assert gpu.ptl_last_conv_resident() == (2 if (Ci * Co * 9) % 8 == 0 else 0), case
+            pkg.call("ptl_conv2d_%s_wg_batched" % dt, a, ns)
+            pkg.call("ptl_conv2d_%s_bw_batched" % dt, a2, ns)
+            if dt == "fp16":
+                assert gpu.ptl_last_conv_resident() == (2 if (Ci * Co * 9) % 8 == 0 else 0), case
         finally:
             gpu.ptl_set_gemm_path(0)
         gpu.ptl_sync()
-        xp = F.pad(x.float(), (pl, pr, pu, pd))
-        ref_dx = torch.nn.grad.conv2d_input(xp.shape, w.float(), dy.float())[:, :, pu:pu + H, pl:pl + W]
-        ref_dw = torch.nn.grad.conv2d_weight(xp, w.shape, dy.float())
-        assert rel(dw, ref_dw) <= 2e-3, (case, "dw")
-        assert rel(dx2, ref_dx) <= 2e-3, (case, "dx, one call")
-        assert rel(dw2, ref_dw) <= 2e-3, (case, "dw, one call")
+        xp = F.pad(x.double(), (pl, pr, pu, pd))
+        ref_dx = torch.nn.grad.conv2d_input(xp.shape, w.double(), dy.double())[:, :, pu:pu + H, pl:pl + W]
+        ref_dw = torch.nn.grad.conv2d_weight(xp, w.shape, dy.double())
+        assert rel(dw, ref_dw) <= tol, (case, "dw")
+        assert rel(dx2, ref_dx) <= tol, (case, "dx, one call")
+        assert rel(dw2, ref_dw) <= tol, (case, "dw, one call")
 
 
 @pytest.mark.parametrize("seed", [21, 22])
