@@ -465,6 +465,20 @@ def detail_table(pkg, lib, hp, to_dev, timed, check, torch, dev):
         ref = ctypes.byref(a)
         ms = timed(lambda: check(lib.ptl_conv2d_fp16_bw_batched(ref, ns)), 10)
         add("conv2d %d->%d %dx%d k3 p1 WG+IG in one call N=%d" % (Ci, Co, H, H, ns), dt, ms, 2 * flops, 2 * nb)
+        # the same two calls reading the blocked copy of the input that the forward call left in a caller-owned buffer
+        nbytes = lib.ptl_conv2d_fp16_cache_bytes(ref, ns)
+        if nbytes:
+            kept = torch.empty(nbytes, dtype=torch.uint8, device=dev)
+            cache = pkg.ConvCache()
+            cache.buf, cache.bytes = kept.data_ptr(), nbytes
+            check(lib.ptl_conv2d_fp16_fw_batched_cached(ref, ns, ctypes.byref(cache)))
+            if cache.valid:
+                ms = timed(lambda: check(lib.ptl_conv2d_fp16_wg_batched_cached(ref, ns, ctypes.byref(cache))), 10)
+                add("conv2d %d->%d %dx%d k3 p1 WG, input copy kept by FW N=%d" % (Ci, Co, H, H, ns), dt, ms, flops, nb)
+                ms = timed(lambda: check(lib.ptl_conv2d_fp16_bw_batched_cached(ref, ns, ctypes.byref(cache))), 10)
+                add("conv2d %d->%d %dx%d k3 p1 WG+IG in one call, input copy kept by FW N=%d" % (Ci, Co, H, H, ns), dt,
+                    ms, 2 * flops, 2 * nb)
+            del kept
         del x, w, dy, y, dx, dw
 
     # the same wide layers with channel-minor (HWC) tensors: X[b][h][w][ci], W[co][kh][kw][ci], Y[b][h][w][co]

@@ -348,6 +348,16 @@ int ptl_gradient_descent_fp16(const struct optim_args_fp16 *a);
  * launch (a training step updates dozens of small tensors). */
 int ptl_gradient_descent_fp32_multi(const struct optim_args *list, int count);
 int ptl_gradient_descent_fp16_multi(const struct optim_args_fp16 *list, int count);
+/* No counterpart in the reference: forward, weight-gradient and weight + input-gradient calls of a Conv2D batch that
+ * share the padded, channel-blocked copy of the layer's input through a caller-owned buffer (struct
+ * ptl_conv_cache): the forward call fills it when the layer takes the route that builds such a copy (3x3 fp16
+ * channel-major layers with channel counts in multiples of 64; c->valid says whether it did), the gradient calls
+ * read it instead of copying the input again.  ptl_conv2d_fp16_cache_bytes returns the size the buffer needs
+ * (0: the layer would not use one).  Without a valid cache the calls behave like the plain ones. */
+size_t ptl_conv2d_fp16_cache_bytes(const struct Conv2D_args_fp16 *a, int nsamples);
+int ptl_conv2d_fp16_fw_batched_cached(const struct Conv2D_args_fp16 *a, int nsamples, struct ptl_conv_cache *c);
+int ptl_conv2d_fp16_wg_batched_cached(const struct Conv2D_args_fp16 *a, int nsamples, const struct ptl_conv_cache *c);
+int ptl_conv2d_fp16_bw_batched_cached(const struct Conv2D_args_fp16 *a, int nsamples, const struct ptl_conv_cache *c);
 int ptl_batch_norm_fp32_fw(const struct BatchNorm_args_fp32 *a);
 /* No counterpart in the reference (its batch normalisation has a forward pass only, in fp32): the backward pass
  * of that forward and both passes in fp16, for a training step that contains the layer.  Backward reads

@@ -12,6 +12,8 @@
 
 #include <stdint.h>
 
+#include <stddef.h>
+
 #ifdef __cplusplus
 extern "C" {
 #endif
@@ -673,6 +675,17 @@ struct BatchNorm_args_fp16 {
     int C;
     int H;
     int W;
+};
+
+/* No counterpart in the reference: a caller-owned buffer in which a Conv2D forward call leaves its padded,
+ * channel-blocked copy of the layer's input for the weight-gradient call of the same layer on the same input
+ * (ptl_conv2d_fp16_*_cached).  The caller sets buf and bytes (ptl_conv2d_fp16_cache_bytes) and keeps both alive and
+ * the input unchanged between the two calls; the library writes valid and geometry. */
+struct ptl_conv_cache {
+    void *buf;
+    size_t bytes;
+    int valid;       /* 1: buf holds the copy described by geometry */
+    int geometry[6]; /* batch, channels, padded height and width, top and left padding */
 };
 
 /* No counterpart in the reference: what a residual block puts behind a normalisation layer, for the fused calls

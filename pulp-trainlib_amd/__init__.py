@@ -79,6 +79,9 @@ BATCHED_ENTRY_POINTS = ["ptl_%s_%s_%s_batched" % (layer, dt, step)
 # `int f(const BatchNorm_args *, const ptl_norm_fusion *)`
 FUSED_NORM_ENTRY_POINTS = ["ptl_batch_norm_fused_%s_%s" % (dt, step) for dt in ("fp32", "fp16") for step in ("fw", "bw")]
 
+# `int f(const Conv2D_args_fp16 *, int nsamples, [const] ptl_conv_cache *)` and the size query
+CACHED_ENTRY_POINTS = ["ptl_conv2d_fp16_%s_batched_cached" % s for s in ("fw", "wg", "bw")] + ["ptl_conv2d_fp16_cache_bytes"]
+
 OTHER_ENTRY_POINTS = ["ptl_init", "ptl_last_error", "ptl_last_status", "ptl_set_stream", "ptl_sync", "ptl_set_gemm_path",
                       "ptl_last_conv_direct", "ptl_last_gemm_streamed", "ptl_last_conv_resident", "ptl_timer_begin", "ptl_timer_end_ms", "ptl_mm_fp32", "ptl_mm_fp16", "ptl_copy_bytes"]
 
@@ -112,6 +115,12 @@ def load():
         f = getattr(lib, name)
         f.argtypes = [ctypes.c_void_p, ctypes.c_void_p]
         f.restype = ctypes.c_int
+    for name in CACHED_ENTRY_POINTS[:3]:
+        f = getattr(lib, name)
+        f.argtypes = [ctypes.c_void_p, ctypes.c_int, ctypes.c_void_p]
+        f.restype = ctypes.c_int
+    lib.ptl_conv2d_fp16_cache_bytes.argtypes = [ctypes.c_void_p, ctypes.c_int]
+    lib.ptl_conv2d_fp16_cache_bytes.restype = ctypes.c_size_t
     lib.ptl_init.argtypes = [ctypes.c_int]
     lib.ptl_init.restype = ctypes.c_int
     lib.ptl_last_error.argtypes = []

@@ -16,8 +16,27 @@
 // the filter pass reads them through the strides of the descriptor.
 #include "ptl_conv_tile.hpp"
 #include "ptl_gemm_async.hpp"
+#include "ptl_structs.h"
 
 namespace ptl {
+
+static ::ptl_conv_cache *g_cache_fill = nullptr;
+static const ::ptl_conv_cache *g_cache_use = nullptr;
+void conv_cache_set(::ptl_conv_cache *fill, const ::ptl_conv_cache *use) {
+    g_cache_fill = fill;
+    g_cache_use = use;
+}
+
+// The cached copy, if the call in progress was given one that fits this layer: `chunks` 16-byte pieces (margin
+// included) of the blocked, padded input of `d`.
+static const uint4 *cached_input(const ConvTileDesc &d, int Hp, int Wp, long long chunks) {
+    const ::ptl_conv_cache *c = g_cache_use;
+    if (!c || !c->valid || !c->buf || c->bytes < (size_t)chunks * 16) return nullptr;
+    const int want[6] = {d.batch, d.Cin, Hp, Wp, d.padU, d.padL};
+    for (int i = 0; i < 6; ++i)
+        if (c->geometry[i] != want[i]) return nullptr;
+    return reinterpret_cast<const uint4 *>(c->buf);
+}
 
 // in: [b][C][H][W] (strides sb, sc; rows contiguous) -> out: [C/VEC][B][Hp][Wp] chunks, zero halo.
 template <typename T>
@@ -167,10 +186,20 @@ int conv_taps(const ConvTileDesc &d, const void *X, const void *Wt, void *Y, con
     const bool halo = ES == 2 && !hwc && conv_halo_fits(d, Hp, Wp) && (long long)d.batch * Hp * Wp < ((long long)1 << 31) &&
                       (st.gemm_path == 5 || (st.gemm_path == 0 && halo_pays));
     const long long margin = halo ? conv_halo_margin() : 0;  // chunks the resident-tile kernel may read past the end
-    char *buf = static_cast<char *>(scratch((size_t)(xb_elems + margin * VEC + wr_elems) * ES + 256));
+    // the blocked input goes to the caller's buffer when the call brought one (the weight gradient of the layer
+    // reads the same copy), else to scratch memory like the filters
+    const size_t xb_bytes = (size_t)(xb_elems + margin * VEC) * ES;
+    ::ptl_conv_cache *fill = g_cache_fill;
+    const bool keep = halo && fill && fill->buf && fill->bytes >= xb_bytes && reinterpret_cast<uintptr_t>(fill->buf) % 16 == 0;
+    char *buf = static_cast<char *>(scratch((keep ? 0 : xb_bytes) + (size_t)wr_elems * ES + 512));
     if (!buf) return 2;
-    uint4 *xb = reinterpret_cast<uint4 *>(buf);
-    T *wr = reinterpret_cast<T *>(buf + (((size_t)(xb_elems + margin * VEC) * ES + 255) & ~(size_t)255));
+    uint4 *xb = reinterpret_cast<uint4 *>(keep ? static_cast<char *>(fill->buf) : buf);
+    T *wr = reinterpret_cast<T *>(keep ? buf : buf + ((xb_bytes + 255) & ~(size_t)255));
+    if (keep) {
+        const int geo[6] = {d.batch, d.Cin, Hp, Wp, d.padU, d.padL};
+        for (int i = 0; i < 6; ++i) fill->geometry[i] = geo[i];
+        fill->valid = 1;
+    }
     {
         TapPrepArgs p = {};
         p.in = X;
@@ -342,7 +371,10 @@ int conv_taps_wg(const ConvTileDesc &d, const void *X, const void *dY, void *dW)
                 if (!ws) return 2;
                 uint4 *xb = reinterpret_cast<uint4 *>(buf);
                 char *gb = buf + (((size_t)xb_chunks * 16 + 255) & ~(size_t)255);
-                if (int rc = blocked_padded_copy<T>(reinterpret_cast<const T *>(X), xb, d, Hp, Wp, margin)) return rc;
+                if (const uint4 *kept = cached_input(d, Hp, Wp, xb_chunks))
+                    xb = const_cast<uint4 *>(kept);
+                else if (int rc = blocked_padded_copy<T>(reinterpret_cast<const T *>(X), xb, d, Hp, Wp, margin))
+                    return rc;
                 const long long gstride = conv_halo_wg_gradient_stride(d, Hp, Wp);
                 if (int rc = conv_halo_embed(dY, gb, d.batch, d.Cout, d.Ho, d.Wo, Hp, Wp, 0, 0, gstride)) return rc;
                 st.last_conv_resident = 1;
@@ -537,7 +569,10 @@ int conv_halo_bw(const ConvTileDesc &fwd, const ConvTileDesc &ig, const void *X,
             hipLaunchKernelGGL((tap_prepare_kernel<T>), dim3((unsigned)((wr_elems + 255) / 256)), dim3(256), 0, st.stream, p);
             if (!hip_ok(hipGetLastError(), "layout launch")) return 2;
         }
-        if (int rc = blocked_padded_copy<T>(reinterpret_cast<const T *>(X), xb, fwd, Hp, Wp, xmargin)) return rc;
+        if (const uint4 *kept = cached_input(fwd, Hp, Wp, xb_chunks))
+            xb = const_cast<uint4 *>(kept);
+        else if (int rc = blocked_padded_copy<T>(reinterpret_cast<const T *>(X), xb, fwd, Hp, Wp, xmargin))
+            return rc;
         st.last_conv_resident = 1;
         if (int rc = conv_halo_wg_launch(fwd, xb, gb + (size_t)goff * 16, gstride, ws, dW, Hp, Wp, S0, S1)) return rc;
         return conv_halo_launch(ig, gb, wr, dX, Hp, Wp, gstride);

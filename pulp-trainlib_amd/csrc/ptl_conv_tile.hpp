@@ -2,6 +2,8 @@
 #pragma once
 #include "ptl_common.hpp"
 
+struct ptl_conv_cache;
+
 namespace ptl {
 
 // out(b, m, y, x) = sum_{ci, ky, kx} in(b, ci, y*sh + ky - padU, x*sw + kx - padL) * w(m, ci, ky, kx)
@@ -119,6 +121,11 @@ int conv_halo_wg_launch(const ConvTileDesc &d, const void *xb, const void *gb, l
 template <typename T>
 int conv_halo_bw(const ConvTileDesc &fwd, const ConvTileDesc &ig, const void *X, const void *dY, const void *Wt,
                  void *dW, void *dX);
+
+// The caller-owned copy of a layer's blocked, padded input (struct ptl_conv_cache) for the call in progress: `fill` is
+// written by the forward route that builds such a copy, `use` read by the weight-gradient routes.  Both null outside
+// the *_cached entry points.
+void conv_cache_set(struct ::ptl_conv_cache *fill, const struct ::ptl_conv_cache *use);
 
 // Weight gradient over filter taps on the same GEMM (partial sums per tap and k split + one reduction).
 template <typename T>

@@ -1009,6 +1009,39 @@ int ptl_conv2d_fp16_bw_batched(const struct Conv2D_args_fp16 *a, int ns) {
     return ptl::conv2d_bw<half_t>(a, ns, "pulp_conv2d_fp16_bw_cl");
 }
 
+size_t ptl_conv2d_fp16_cache_bytes(const struct Conv2D_args_fp16 *a, int ns) {
+    ptl::ConvGeom g;
+    if (ns <= 0 || ptl::conv_geom(a, g, "ptl_conv2d_fp16_cache_bytes", false)) return 0;
+    if (g.hwc || g.Hk != 3 || g.Wk != 3 || g.sh != 1 || g.sw != 1 || g.Ci % 64 != 0) return 0;
+    ptl::ConvTileDesc d = {};
+    d.batch = ns; d.Cin = g.Ci; d.Hin = g.H; d.Win = g.W;
+    d.Cout = g.Co; d.Ho = g.Ho; d.Wo = g.Wo;
+    d.KH = 3; d.KW = 3; d.sh = 1; d.sw = 1;
+    d.padU = g.Up; d.padD = g.Dp; d.padL = g.Lp; d.padR = g.Rp;
+    const int Hp = g.H + g.Up + g.Dp, Wp = g.W + g.Lp + g.Rp;
+    if (!ptl::conv_halo_fits(d, Hp, Wp)) return 0;
+    return ((size_t)(g.Ci / 8) * ns * Hp * Wp + (size_t)ptl::conv_halo_margin()) * 16;
+}
+int ptl_conv2d_fp16_fw_batched_cached(const struct Conv2D_args_fp16 *a, int ns, struct ptl_conv_cache *c) {
+    if (c) c->valid = 0;
+    ptl::conv_cache_set(c, nullptr);
+    const int rc = ptl::conv2d_fw<half_t>(a, ns, "pulp_conv2d_fp16_fw_cl");
+    ptl::conv_cache_set(nullptr, nullptr);
+    return rc;
+}
+int ptl_conv2d_fp16_wg_batched_cached(const struct Conv2D_args_fp16 *a, int ns, const struct ptl_conv_cache *c) {
+    ptl::conv_cache_set(nullptr, c);
+    const int rc = ptl::conv2d_wg<half_t>(a, ns, "pulp_conv2d_fp16_bw_param_grads_cl");
+    ptl::conv_cache_set(nullptr, nullptr);
+    return rc;
+}
+int ptl_conv2d_fp16_bw_batched_cached(const struct Conv2D_args_fp16 *a, int ns, const struct ptl_conv_cache *c) {
+    ptl::conv_cache_set(nullptr, c);
+    const int rc = ptl::conv2d_bw<half_t>(a, ns, "pulp_conv2d_fp16_bw_cl");
+    ptl::conv_cache_set(nullptr, nullptr);
+    return rc;
+}
+
 int ptl_conv_pw_fp32_fw_batched(const struct PointWise_Conv_args *a, int ns) {
     return ptl::pw_step<float>(a, ns, STEP_FW, "pulp_conv_pw_fp32_fw_cl");
 }

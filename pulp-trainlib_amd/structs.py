@@ -164,6 +164,11 @@ class BatchNormArgs(C.Structure):
                 ("B", I), ("C", I), ("H", I), ("W", I)]
 
 
+class ConvCache(C.Structure):
+    """struct ptl_conv_cache: the caller-owned copy of a layer's blocked input shared by ptl_conv2d_fp16_*_cached."""
+    _fields_ = [("buf", P), ("bytes", C.c_size_t), ("valid", I), ("geometry", I * 6)]
+
+
 class NormFusion(C.Structure):
     """struct ptl_norm_fusion_fp32 / _fp16: what ptl_batch_norm_fused_* does behind the normalisation."""
     _fields_ = [("relu", I), ("skip", P), ("skip_diff", P), ("diff2", P)]

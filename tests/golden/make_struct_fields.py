@@ -24,9 +24,9 @@ def struct_fields(text):
             decl = " ".join(decl.replace("__restrict__", " ").split())
             if not decl:
                 continue
-            mm = re.match(r"^(.*?)([A-Za-z_]\w*)$", decl)
+            mm = re.match(r"^(.*?)([A-Za-z_]\w*)\s*(\[\w*\])?$", decl)
             typ, name = mm.group(1), mm.group(2)
-            typ = re.sub(r"\s*\*\s*", " *", typ).strip()
+            typ = re.sub(r"\s*\*\s*", " *", typ).strip() + (mm.group(3) or "")
             fields.append([typ, name])
         out[m.group(1)] = fields
     return out

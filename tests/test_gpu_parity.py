@@ -254,6 +254,61 @@ RESIDENT_CASES = [
 ]
 
 
+@pytest.mark.parametrize("case", [(64, 14, 14, 64, (1, 1, 1, 1), 12), (128, 9, 11, 64, (0, 2, 1, 1), 20),
+                                  (64, 28, 28, 128, (1, 1, 1, 1), 5), (32, 16, 16, 64, (1, 1, 1, 1), 8)])
+def test_conv2d_forward_leaves_its_blocked_input_for_the_gradients(pkg, gpu, case):
+    """ptl_conv2d_fp16_*_cached: the forward call fills the caller's buffer with its padded, channel-blocked copy of
+    the input, the weight-gradient and the weight + input-gradient calls read it - same results, bit for bit, as the
+    plain calls; a layer that does not build such a copy (32 channels) leaves the cache invalid and the calls fall
+    back; a cache of another geometry is ignored."""
+    Ci, H, W, Co, pad, ns = case
+    pl, pr, pu, pd = pad
+    Ho, Wo = H + pu + pd - 2, W + pl + pr - 2
+    x = (torch.rand(ns, Ci, H, W, device="cuda") - 0.5).half()
+    w = ((torch.rand(Co, Ci, 3, 3, device="cuda") - 0.5) * 0.2).half()
+    dy = (torch.rand(ns, Co, Ho, Wo, device="cuda") - 0.5).half()
+    outs = []
+    for cached in (False, True):
+        y, dx, dw, dw2 = torch.full_like(dy, 3), torch.full_like(x, 3), torch.full_like(w, 3), torch.full_like(w, 3)
+        a, keep = hp.conv2d_args(pkg, x, dx, w, dw, y, dy, Ci, H, W, Co, 3, 3, Ho, Wo, pad, (1, 1))
+        a2, keep2 = hp.conv2d_args(pkg, x, None, w, dw2, y, dy, Ci, H, W, Co, 3, 3, Ho, Wo, pad, (1, 1))
+        gpu.ptl_set_gemm_path(5)
+        try:
+            if cached:
+                nbytes = gpu.ptl_conv2d_fp16_cache_bytes(ctypes.byref(a), ns)
+                assert (nbytes > 0) == (Ci % 64 == 0)
+                buf = torch.empty(max(nbytes, 16), dtype=torch.uint8, device="cuda")
+                c = pkg.ConvCache()
+                c.buf, c.bytes = buf.data_ptr(), nbytes
+                assert gpu.ptl_conv2d_fp16_fw_batched_cached(ctypes.byref(a), ns, ctypes.byref(c)) == 0
+                assert c.valid == (1 if Ci % 64 == 0 else 0)
+                assert gpu.ptl_conv2d_fp16_bw_batched_cached(ctypes.byref(a), ns, ctypes.byref(c)) == 0
+                assert gpu.ptl_conv2d_fp16_wg_batched_cached(ctypes.byref(a2), ns, ctypes.byref(c)) == 0
+                if c.valid:  # a copy of another layer's geometry must not be used
+                    other = pkg.ConvCache()
+                    other.buf, other.bytes, other.valid = buf.data_ptr(), nbytes, 1
+                    for i, v in enumerate((ns, Ci, H + pu + pd + 1, W + pl + pr, pu, pl)):
+                        other.geometry[i] = v
+                    buf.fill_(0x3c)
+                    dw3 = torch.full_like(w, 3)
+                    a3, keep3 = hp.conv2d_args(pkg, x, None, w, dw3, y, dy, Ci, H, W, Co, 3, 3, Ho, Wo, pad, (1, 1))
+                    assert gpu.ptl_conv2d_fp16_wg_batched_cached(ctypes.byref(a3), ns, ctypes.byref(other)) == 0
+                    gpu.ptl_sync()
+                    assert torch.equal(dw3, dw2)
+            else:
+                pkg.call("ptl_conv2d_fp16_fw_batched", a, ns)
+                pkg.call("ptl_conv2d_fp16_bw_batched", a, ns)
+                pkg.call("ptl_conv2d_fp16_wg_batched", a2, ns)
+        finally:
+            gpu.ptl_set_gemm_path(0)
+        gpu.ptl_sync()
+        outs.append((y, dx, dw, dw2))
+    for plain, kept in zip(*outs):
+        assert torch.equal(plain, kept)
+    ref_dw = torch.nn.grad.conv2d_weight(torch.nn.functional.pad(x.float(), pad), w.shape, dy.float())
+    assert float((outs[1][3].float() - ref_dw).norm() / ref_dw.norm()) <= 2e-3
+
+
 @pytest.mark.parametrize("case", RESIDENT_CASES)
 def test_conv2d_resident_tile_route(pkg, orc, gpu, case):
     Ci, H, W, Co, pad, ns, resident = case
