@@ -538,8 +538,10 @@ int plan_small(const ConvTileDesc &d, const void *X, const void *Wt, void *Y, in
     while (R > 1 && (items_of(R) > CS_ITEMS || f_bytes + lds_of(R) > 150 * 1024)) R = (R + 1) / 2;
     if (items_of(R) > CS_ITEMS || f_bytes + lds_of(R) > 150 * 1024) return -1;
     const long long tiles = (long long)d.batch * ((d.Ho + R - 1) / R);
-    // beyond a few workgroups per CU the persistent kernels (filters loaded once per workgroup) are ahead
-    if (st.gemm_path != 6 && tiles > 4LL * st.num_cu) return -1;
+    // beyond a few workgroups per CU the persistent kernels (filters loaded once per workgroup) are ahead where
+    // both channel counts fill their 64-wide tiles; narrower layers stay ahead here for longer
+    const long long tile_limit = (d.Cin == 64 && d.Cout == 64 ? 4LL : 16LL) * st.num_cu;
+    if (st.gemm_path != 6 && tiles > tile_limit) return -1;
     if (tiles >= (1LL << 31) / 256) return -1;
     a.X = X;
     a.Wt = Wt;
