@@ -16,8 +16,9 @@ namespace ptl {
 
 static inline unsigned nblocks(size_t n) { return (unsigned)((n + 255) / 256); }
 
-// x / d as a multiplication by m = ceil(2^32 / d): exact for x below 2^16.
-__device__ inline unsigned div_magic(unsigned x, unsigned m) { return (unsigned)(((unsigned long long)x * m) >> 32); }
+// x / d as a multiplication by m = ceil(2^32 / d): exact for x below 2^16.  d = 1 gives m = 2^32, which a 32-bit
+// m holds as 0: that value stands for the identity.
+__device__ inline unsigned div_magic(unsigned x, unsigned m) { return m ? __umulhi(x, m) : x; }
 
 // ---- Depthwise convolution (CHW planes, one filter per channel) -----------------
 struct DwGeom {
@@ -1426,68 +1427,101 @@ __global__ __launch_bounds__(256) void blocktransp_kernel(const T *__restrict__ 
     }
 }
 
-// Channel-major weights through an LDS tile of 32 output x 32 input channels x P taps: a workgroup reads, for each
-// of its 32 output channels, the contiguous run of 32 x P elements, and writes, for each of its 32 input channels,
-// the contiguous run of 32 x P elements of the result - both sides of the transposition move whole lines, 16 bytes
-// per thread where VECS says the runs are made of whole aligned chunks.
-template <typename T, bool VECS>
-__global__ __launch_bounds__(256) void blocktransp_tile_kernel(const T *__restrict__ w, T *__restrict__ bt, int Ci,
-                                                               int Co, int P, unsigned m_p) {
-    constexpr int VEC = 16 / (int)sizeof(T);
+// Channel-major weights through an LDS tile of TD output x TD input channels x P taps: a workgroup reads, for each
+// of its TD output channels, the contiguous run of TD x P elements, and writes, for each of its TD input channels,
+// the contiguous run of TD x P elements of the result - both sides of the transposition move whole lines, 16 bytes
+// per thread where VECS says the runs are made of whole aligned chunks.  A thread keeps one chunk position of the
+// run and walks down the rows, so where its elements sit in the tile (a division and a flip per element) is
+// worked out once, before the loop.
+template <typename T, bool VECS, int TD, int NT>
+__global__ __launch_bounds__(NT) void blocktransp_tile_kernel(const T *__restrict__ w, T *__restrict__ bt, int Ci,
+                                                              int Co, int P, unsigned m_p, int pitch) {
+    constexpr int VEC = 16 / (int)sizeof(T), E = VECS ? VEC : 1;
     extern __shared__ __attribute__((aligned(16))) char smem[];
-    T *tile = reinterpret_cast<T *>(smem);  // [32 co][32 * P + VEC]: rows start on 16-byte boundaries
-    const int ci0 = blockIdx.x * 32, co0 = blockIdx.y * 32, pitch = 32 * P + VEC;
-    const int nci = min(32, Ci - ci0), nco = min(32, Co - co0);
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    for (int r = wave; r < nco; r += 4) {
-        const T *src = w + ((size_t)(co0 + r) * Ci + ci0) * P;
-        const int n = nci * P;
-        if (VECS) {
-            for (int c = lane; c * VEC < n; c += 64) {
-                if (c * VEC + VEC <= n) {
-                    union {
-                        uint4 u;
-                        T e[VEC];
-                    } v;
-                    v.u = *reinterpret_cast<const uint4 *>(src + c * VEC);
-                    *reinterpret_cast<uint4 *>(tile + r * pitch + c * VEC) = v.u;
-                } else {
-                    for (int e = c * VEC; e < n; ++e) tile[r * pitch + e] = src[e];
+    T *tile = reinterpret_cast<T *>(smem);  // [TD co][pitch]
+    // Tiles in groups of 2 x 2 that one XCD takes in a row (workgroups go to the eight XCDs in turn): where a tile's
+    // runs end inside a 128-byte line, the neighbour that holds the rest of the line meets it in the same L2.
+    const int tiles_x = (Ci + TD - 1) / TD, tiles_y = (Co + TD - 1) / TD, groups_x = (tiles_x + 1) / 2;
+    const unsigned L = blockIdx.x, slot = L >> 3, group = (L & 7) + 8 * (slot >> 2), m = slot & 3;
+    const int gy = group / groups_x, gx = group - gy * groups_x;
+    const int tx = 2 * gx + (m & 1), ty = 2 * gy + (m >> 1);
+    if (tx >= tiles_x || ty >= tiles_y) return;
+    const int ci0 = tx * TD, co0 = ty * TD;
+    const int nci = min(TD, Ci - ci0), nco = min(TD, Co - co0);
+    const int tid = threadIdx.x;
+    {
+        // (a run longer than the workgroup is walked in several sweeps of c)
+        const int n = nci * P, per_row = (n + E - 1) / E, span = min(per_row, NT), rstep = NT / span;
+        const int row0 = tid / span;
+        const size_t row_elems = (size_t)Ci * P;
+        for (int c = tid - row0 * span; c < per_row && row0 < rstep; c += span) {
+            const T *src = w + ((size_t)co0 * Ci + ci0) * P + row0 * row_elems + c * E;
+            T *dst = tile + row0 * pitch + c * E;
+            if (!VECS || c * E + E <= n) {
+                typedef typename std::conditional<VECS, uint4, T>::type Piece;
+                int row = row0;
+                for (; row + 3 * rstep < nco; row += 4 * rstep) {
+                    Piece v[4];
+#pragma unroll
+                    for (int u = 0; u < 4; ++u) v[u] = *reinterpret_cast<const Piece *>(src + u * rstep * row_elems);
+#pragma unroll
+                    for (int u = 0; u < 4; ++u) *reinterpret_cast<Piece *>(dst + u * rstep * pitch) = v[u];
+                    src += 4 * rstep * row_elems;
+                    dst += 4 * rstep * pitch;
+                }
+                for (; row < nco; row += rstep) {
+                    *reinterpret_cast<Piece *>(dst) = *reinterpret_cast<const Piece *>(src);
+                    src += rstep * row_elems;
+                    dst += rstep * pitch;
+                }
+            } else {
+                for (int row = row0; row < nco; row += rstep) {
+                    for (int e = 0; c * E + e < n; ++e) dst[e] = src[e];
+                    src += rstep * row_elems;
+                    dst += rstep * pitch;
                 }
             }
-        } else {
-            for (int e = lane; e < n; e += 64) tile[r * pitch + e] = src[e];
         }
     }
     __syncthreads();
-    for (int r = wave; r < nci; r += 4) {
-        T *dst = bt + ((size_t)(ci0 + r) * Co + co0) * P;
-        const int n = nco * P;
-        if (VECS) {
-            for (int c = lane; c * VEC < n; c += 64) {
-                unsigned co = div_magic((unsigned)(c * VEC), m_p), i = (unsigned)(c * VEC) - co * P;
-                union {
-                    uint4 u;
-                    T e[VEC];
-                } v;
+    {
+        const int n = nco * P, per_row = (n + E - 1) / E, span = min(per_row, NT), rstep = NT / span;
+        const int row0 = tid / span;
+        for (int c = tid - row0 * span; c < per_row && row0 < rstep; c += span) {
+            int off[E];  // where the chunk's elements sit in row 0 of the tile's view for input channel 0
+            unsigned co = div_magic((unsigned)(c * E), m_p), i = (unsigned)(c * E) - co * P;
 #pragma unroll
-                for (int e = 0; e < VEC; ++e) {
-                    v.e[e] = co < (unsigned)nco ? tile[co * pitch + r * P + (P - 1 - i)] : (T)0;
-                    if (++i == (unsigned)P) {
-                        i = 0;
-                        ++co;
-                    }
-                }
-                if (c * VEC + VEC <= n) {
-                    *reinterpret_cast<uint4 *>(dst + c * VEC) = v.u;
-                } else {
-                    for (int e = 0; c * VEC + e < n; ++e) dst[c * VEC + e] = v.e[e];
+            for (int e = 0; e < E; ++e) {
+                off[e] = min((int)co, nco - 1) * pitch + (P - 1 - (int)i);
+                if (++i == (unsigned)P) {
+                    i = 0;
+                    ++co;
                 }
             }
-        } else {
-            for (int e = lane; e < n; e += 64) {
-                const unsigned co = div_magic((unsigned)e, m_p), i = (unsigned)e - co * P;
-                dst[e] = tile[co * pitch + r * P + (P - 1 - i)];
+            T *dst = bt + ((size_t)ci0 * Co + co0) * P + (size_t)row0 * Co * P + c * E;
+            const T *t = tile + row0 * P;
+            typedef typename std::conditional<VECS, uint4, T>::type Piece;
+            union Chunk {
+                Piece u;
+                T e[E];
+            };
+            if (c * E + E <= n) {
+                for (int row = row0; row < nci; row += rstep) {
+                    Chunk v;
+#pragma unroll
+                    for (int e = 0; e < E; ++e) v.e[e] = t[off[e]];
+                    *reinterpret_cast<Piece *>(dst) = v.u;
+                    dst += (size_t)rstep * Co * P;
+                    t += rstep * P;
+                }
+            } else {  // the run's last, partial chunk (constant indices only: others would send the chunk through memory)
+                for (int row = row0; row < nci; row += rstep) {
+#pragma unroll
+                    for (int e = 0; e < E; ++e)
+                        if (c * E + e < n) dst[e] = t[off[e]];
+                    dst += (size_t)rstep * Co * P;
+                    t += rstep * P;
+                }
             }
         }
     }
@@ -1526,18 +1560,24 @@ static int blocktransp(const Args *a, const char *fn) {
         rc = transpose2d_strided<T>(w, bt, a->Cout, a->Cin, (long long)P * a->Cin, (long long)P * a->Cout, P,
                                     -(long long)a->Cin, (long long)a->Cout, (long long)(P - 1) * a->Cin, 0);
     } else if ((size_t)32 * (32 * P + 16 / sizeof(T)) * sizeof(T) <= 64 * 1024 && n >= 4096) {
-        const size_t lds = (size_t)32 * (32 * P + 16 / sizeof(T)) * sizeof(T);
+        constexpr int VEC = 16 / (int)sizeof(T);
         const unsigned m_p = (unsigned)((((unsigned long long)1 << 32) + P - 1) / P);
-        const dim3 grid((a->Cin + 31) / 32, (a->Cout + 31) / 32);
         // runs of whole 16-byte chunks: every run starts on a chunk (rows of Ci x P and Co x P elements, tiles of 32 x P)
         const bool vecs = ((size_t)a->Cin * P * sizeof(T)) % 16 == 0 && ((size_t)a->Cout * P * sizeof(T)) % 16 == 0 &&
                           reinterpret_cast<uintptr_t>(w) % 16 == 0 && reinterpret_cast<uintptr_t>(bt) % 16 == 0;
+        auto tile_grid = [&](int td) {  // (groups of four tiles, rounded up to eight groups)
+            const long long groups = (long long)(((a->Cin + td - 1) / td + 1) / 2) * (((a->Cout + td - 1) / td + 1) / 2);
+            return (unsigned)(32 * ((groups + 7) / 8));
+        };
+        const int pitch = 32 * P + VEC;  // rows of the tile start on 16-byte boundaries
+        const size_t lds = (size_t)32 * pitch * sizeof(T);
+        const dim3 grid(tile_grid(32));
         if (vecs)
-            hipLaunchKernelGGL((blocktransp_tile_kernel<T, true>), grid, dim3(256), lds, state().stream, w, bt, a->Cin,
-                               a->Cout, P, m_p);
+            hipLaunchKernelGGL((blocktransp_tile_kernel<T, true, 32, 256>), grid, dim3(256), lds, state().stream, w, bt,
+                               a->Cin, a->Cout, P, m_p, pitch);
         else
-            hipLaunchKernelGGL((blocktransp_tile_kernel<T, false>), grid, dim3(256), lds, state().stream, w, bt, a->Cin,
-                               a->Cout, P, m_p);
+            hipLaunchKernelGGL((blocktransp_tile_kernel<T, false, 32, 256>), grid, dim3(256), lds, state().stream, w,
+                               bt, a->Cin, a->Cout, P, m_p, pitch);
         rc = hip_ok(hipGetLastError(), "blocktranspose launch") ? 0 : 2;
     } else {
         if (n >= ((size_t)1 << 31)) {

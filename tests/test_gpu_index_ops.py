@@ -199,7 +199,8 @@ def test_transpose_matrix_tiles(pkg, gpu, dt, N, M):
 
 @pytest.mark.parametrize("dt", ["fp32", "fp16"])
 @pytest.mark.parametrize("hwc", [0, 1])
-@pytest.mark.parametrize("Ci,Co,Hk,Wk", [(64, 96, 3, 3), (40, 33, 3, 3), (72, 64, 5, 5), (8, 16, 1, 1), (130, 70, 2, 3)])
+@pytest.mark.parametrize("Ci,Co,Hk,Wk", [(64, 96, 3, 3), (40, 33, 3, 3), (72, 64, 5, 5), (8, 16, 1, 1), (130, 70, 2, 3),
+                                         (256, 320, 3, 3), (296, 264, 3, 3), (264, 256, 1, 1)])
 def test_blocktranspose_tiles(pkg, orc, gpu, dt, hwc, Ci, Co, Hk, Wk):
     nd = hp.np_dtype(dt)
     w = hp.uniform(0xB7, (Co * Ci * Hk * Wk,), dtype=nd)
@@ -218,7 +219,8 @@ def test_blocktranspose_tiles(pkg, orc, gpu, dt, hwc, Ci, Co, Hk, Wk):
 @pytest.mark.parametrize("dt", ["fp32", "fp16"])
 @pytest.mark.parametrize("hwc", [0, 1])
 @pytest.mark.parametrize("Ci,H,W,K,pad,stride,mod", [(16, 32, 32, 3, (1, 1, 1, 1), (1, 1), 0), (7, 19, 23, 3, (1, 1, 1, 1), (2, 2), 0),
-                                                     (6, 14, 9, 5, (2, 2, 2, 2), (1, 1), 0), (5, 12, 12, 3, (0, 0, 0, 0), (1, 1), 1)])
+                                                     (6, 14, 9, 5, (2, 2, 2, 2), (1, 1), 0), (5, 12, 12, 3, (0, 0, 0, 0), (1, 1), 1),
+                                                     (16, 32, 32, 1, (0, 0, 0, 0), (1, 1), 0), (64, 40, 48, 1, (0, 0, 0, 0), (1, 1), 0)])
 def test_im2row_im2col_chunked(pkg, orc, gpu, dt, hwc, Ci, H, W, K, pad, stride, mod):
     """Patch matrices whose rows are not multiples of a 16-byte chunk (chunks straddle rows and columns), BASELINE
     config 1 among them."""
