@@ -1223,60 +1223,107 @@ __global__ __launch_bounds__(256) void patch_kernel(const T *__restrict__ src, T
 // every source element is fetched once per workgroup instead of once per tap - and then writes its part of the
 // R buffer rows as 16-byte chunks, each gathered from LDS.  Divisions by the runtime extents are multiplications
 // by ceil(2^32 / d) (exact for dividends below 2^16).
-template <typename T>
+// A vector memory instruction occupies the address unit for its 64 lanes whatever each lane moves, so the window
+// is read in as few instructions as the layout allows: WIDE (rows of the tensor start on 16-byte boundaries) takes
+// the aligned 16-byte pieces that cover the window - the window then starts up to a piece early, `shift` elements
+// that the offsets table skips - and otherwise one element per lane, one wave per window row.
+typedef unsigned PatchPiece __attribute__((ext_vector_type(4)));  // (a built-in vector: loads from any address space)
+__device__ const PatchPiece patch_zero = {0u, 0u, 0u, 0u};  // what the window holds outside the tensor
+
+template <typename T, bool WIDE>
 __global__ __launch_bounds__(256) void patch_rows_kernel(const T *__restrict__ src, T *__restrict__ buf, PatchGeom g, int R,
-                                                         int CB, int LW, unsigned m_cpr, unsigned m_pk, unsigned m_wk) {
+                                                         int CB, int LW, unsigned m_pk, unsigned m_wk, unsigned m_hk) {
     constexpr int VEC = 16 / (int)sizeof(T);
+    // (as global-memory pointers: a generic one would load through the flat path, whose waits are shared with LDS)
+    typedef const T __attribute__((address_space(1))) *GlobalT;
+    typedef const PatchPiece __attribute__((address_space(1))) *GlobalPiece;
     extern __shared__ __attribute__((aligned(16))) char smem[];
     const int PK = g.Hk * g.Wk, Q = g.C * PK, nq = CB * PK;
     unsigned short *offs = reinterpret_cast<unsigned short *>(smem);                    // [nq], nq a multiple of VEC
-    T *lds = reinterpret_cast<T *>(smem + (((size_t)nq * 2 + 15) & ~(size_t)15));      // [CB * Hk][LW]
+    T *lds = reinterpret_cast<T *>(smem + (((size_t)nq * 2 + 15) & ~(size_t)15));      // [CB * Hk][LW], one spare slot
     const int wp0 = blockIdx.x * R, hp = blockIdx.y, c0 = blockIdx.z * CB;
     const int nr = min(R, g.Wp - wp0);
     const int w_first = wp0 * g.w_mul + g.w_add, h_first = hp * g.h_mul + g.h_add;
+    const int w_start = WIDE ? (w_first & ~(VEC - 1)) : w_first, shift = w_first - w_start;  // (& rounds down below 0 too)
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     // where column q = (channel, filter row, filter column) of a buffer row starts in the staged window
     for (int q = threadIdx.x; q < nq; q += 256) {
         const unsigned c_l = div_magic((unsigned)q, m_pk), t = (unsigned)q - c_l * PK;
         const unsigned hk = div_magic(t, m_wk), wk = t - hk * g.Wk;
-        offs[q] = (unsigned short)((c_l * g.Hk + hk) * LW + wk);
+        offs[q] = (unsigned short)((c_l * g.Hk + hk) * LW + wk + shift);
     }
-    // the window: one wave per (channel, filter row), lanes along the row
-    for (int r = wave; r < CB * g.Hk; r += 4) {
-        const int c_l = r / g.Hk, hk = r - c_l * g.Hk, h = h_first + hk;
-        const bool row_ok = (unsigned)h < (unsigned)g.Hs;
-        const T *row = src + ((size_t)(c0 + c_l) * g.Hs + (row_ok ? h : 0)) * g.Ws;
-        for (int x = lane; x < LW; x += 64) {
-            const int w = w_first + x;
-            lds[r * LW + x] = (row_ok && (unsigned)w < (unsigned)g.Ws) ? row[w] : (T)0;
+    const int rows = CB * g.Hk, width = (R - 1) * g.w_mul + g.Wk;  // the window: rows, and what the patches reach of one
+    // Every lane always loads and always stores: a load under a condition becomes a branch with a wait of its own,
+    // and the compiler moves a load into the branch that holds its only use.  What lies outside the tensor is read
+    // from a piece of zeros; what lies outside the window is written to the spare slot behind it.
+    if (WIDE) {
+        const int np = (shift + width + VEC - 1) / VEC, items = rows * np;  // pieces per row; LW holds np whole pieces
+        const unsigned m_np = (unsigned)((((unsigned long long)1 << 32) + np - 1) / np);
+        for (int i0 = threadIdx.x; i0 < items; i0 += 4 * 256) {
+            PatchPiece v[4];
+            int at[4];
+#pragma unroll
+            for (int u = 0; u < 4; ++u) {
+                const int item = i0 + u * 256;
+                const int r = (int)div_magic((unsigned)min(item, items - 1), m_np), piece = min(item, items - 1) - r * np;
+                const int c_l = (int)div_magic((unsigned)r, m_hk), h = h_first + (r - c_l * g.Hk), w = w_start + piece * VEC;
+                const bool ok = (unsigned)h < (unsigned)g.Hs && (unsigned)w < (unsigned)g.Ws;  // (a piece is all in or all out)
+                const int off = ((c0 + c_l) * g.Hs + h) * g.Ws + w;  // (below 2^31: the host checks the tensor's size)
+                v[u] = *(ok ? (GlobalPiece)(src + off) : (GlobalPiece)&patch_zero);
+                at[u] = item < items ? r * LW + piece * VEC : rows * LW;
+            }
+#pragma unroll
+            for (int u = 0; u < 4; ++u) {  // (rows start on 4-byte boundaries only: their pitch is an odd number of dwords)
+                unsigned *dst = reinterpret_cast<unsigned *>(lds + at[u]);
+                dst[0] = v[u].x; dst[1] = v[u].y; dst[2] = v[u].z; dst[3] = v[u].w;
+            }
+        }
+    } else {
+        const int w_lane = w_first + lane;
+        const bool col_ok = (unsigned)w_lane < (unsigned)g.Ws && lane < width;
+        for (int r0 = wave; r0 < rows; r0 += 64) {
+            T v[16];
+#pragma unroll
+            for (int u = 0; u < 16; ++u) {
+                const int r = min(r0 + 4 * u, rows - 1);
+                const int c_l = (int)div_magic((unsigned)r, m_hk), h = h_first + (r - c_l * g.Hk);
+                const bool ok = (unsigned)h < (unsigned)g.Hs && col_ok;
+                const int off = ((c0 + c_l) * g.Hs + h) * g.Ws + w_lane;
+                v[u] = *(ok ? (GlobalT)(src + off) : (GlobalT)&patch_zero);
+            }
+#pragma unroll
+            for (int u = 0; u < 16; ++u) lds[lane < width && r0 + 4 * u < rows ? (r0 + 4 * u) * LW + lane : rows * LW] = v[u];
         }
     }
     __syncthreads();
+    // a thread keeps one chunk position of the buffer rows (its table entries stay in registers) and walks down the
+    // positions; a row piece longer than the workgroup takes several sweeps
     const int cpr = nq / VEC;  // chunks of this workgroup per buffer row
+    const int span = min(cpr, 256), pstep = 256 / span, p0 = threadIdx.x / span;
     T *base = buf + ((size_t)hp * g.Wp + wp0) * Q + (size_t)c0 * PK;
-    for (int item = threadIdx.x; item < nr * cpr; item += 256) {
-        const unsigned p_l = div_magic((unsigned)item, m_cpr), qc = (unsigned)item - p_l * cpr;
-        union {
-            uint4 u;
-            unsigned short o[8];
-        } tab[VEC == 8 ? 1 : 1];
-        union {
-            uint4 u;
-            T e[VEC];
-        } v;
-        const T *win = lds + p_l * g.w_mul;
+    for (int qc = threadIdx.x - p0 * span; qc < cpr && p0 < pstep; qc += span) {
+        int o[VEC];
         if (VEC == 8) {
-            tab[0].u = *reinterpret_cast<const uint4 *>(offs + qc * 8);
-#pragma unroll
-            for (int e = 0; e < VEC; ++e) v.e[e] = win[tab[0].o[e]];
+            const uint4 t4 = *reinterpret_cast<const uint4 *>(offs + qc * 8);
+            o[0] = t4.x & 0xffffu; o[1] = t4.x >> 16; o[2] = t4.y & 0xffffu; o[3] = t4.y >> 16;
+            o[4 % VEC] = t4.z & 0xffffu; o[5 % VEC] = t4.z >> 16; o[6 % VEC] = t4.w & 0xffffu; o[7 % VEC] = t4.w >> 16;
         } else {
             const uint2 t2 = *reinterpret_cast<const uint2 *>(offs + qc * 4);
-            v.e[0] = win[t2.x & 0xffffu];
-            v.e[1] = win[t2.x >> 16];
-            v.e[2] = win[t2.y & 0xffffu];
-            v.e[3] = win[t2.y >> 16];
+            o[0] = t2.x & 0xffffu; o[1] = t2.x >> 16; o[2] = t2.y & 0xffffu; o[3] = t2.y >> 16;
         }
-        *reinterpret_cast<uint4 *>(base + (size_t)p_l * Q + qc * VEC) = v.u;
+        const T *win = lds + p0 * g.w_mul;
+        T *dst = base + (size_t)p0 * Q + qc * VEC;
+        for (int p_l = p0; p_l < nr; p_l += pstep) {
+            union {
+                uint4 u;
+                T e[VEC];
+            } v;
+#pragma unroll
+            for (int e = 0; e < VEC; ++e) v.e[e] = win[o[e]];
+            *reinterpret_cast<uint4 *>(dst) = v.u;
+            win += pstep * g.w_mul;
+            dst += (size_t)pstep * Q;
+        }
     }
 }
 
@@ -1288,30 +1335,41 @@ static int patch_rows(const T *src, T *buf, const PatchGeom &g) {
     const int PK = g.Hk * g.Wk;
     const long long Q = (long long)g.C * PK;
     if (reinterpret_cast<uintptr_t>(buf) % 16 || (Q * ES) % 16 || g.Wp < 16 || Q >= 65536 || g.Hp >= 65536 || g.Wk > 32 ||
-        g.w_mul > 8)
+        g.w_mul > 8 || (long long)(g.C + 64) * g.Hs * g.Ws >= ((long long)1 << 31))  // (32-bit element offsets, with slack)
         return -1;
-    // positions per workgroup: a window row of at most 64 elements (one pass of a wave)
+    // rows of the tensor that start on 16-byte boundaries are read as aligned 16-byte pieces
+    const bool wide = ((size_t)g.Ws * ES) % 16 == 0 && reinterpret_cast<uintptr_t>(src) % 16 == 0;
+    // positions per workgroup: a window row of at most 64 elements (one pass of a wave) - half that with pieces,
+    // whose loads are few either way: more and shorter workgroups overlap their load and store phases better -
+    // and then the same number for every workgroup of a grid row
     int R = (64 - g.Wk) / g.w_mul + 1;
+    if (wide && R >= 32) R = (R + 1) / 2;
     if (R > g.Wp) R = g.Wp;
+    R = (g.Wp + (g.Wp + R - 1) / R - 1) / ((g.Wp + R - 1) / R);
     // row pitch of the window: an odd number of dwords, so that the rows the lanes of a wave gather from (every
-    // Hk-th one for neighbouring channels) spread over the LDS banks
+    // Hk-th one for neighbouring channels) spread over the LDS banks; with pieces, room for the whole pieces that
+    // cover a window starting anywhere in its first piece
     int LW = (R - 1) * g.w_mul + g.Wk;
+    if (wide) LW = (VEC - 1 + LW + VEC - 1) / VEC * VEC;
     LW = ES == 2 ? (((LW + 1) & ~1) | 2) : (LW | 1);
-    auto bytes = [&](int cb) { return (((size_t)cb * PK * 2 + 15) & ~(size_t)15) + (size_t)cb * g.Hk * LW * ES; };
+    // (table of column offsets, window, one spare slot)
+    auto bytes = [&](int cb) { return (((size_t)cb * PK * 2 + 15) & ~(size_t)15) + (size_t)cb * g.Hk * LW * ES + 16; };
     int CB = g.C;
     while (bytes(CB) > 40 * 1024 && CB % 2 == 0) CB /= 2;
-    // enough workgroups to keep several per CU (their load and store phases overlap only across workgroups), as long
-    // as a workgroup's piece of a buffer row stays a few cache lines long
+    // whole buffer rows per workgroup (one contiguous run of R x Q elements) unless that leaves CUs idle; a
+    // workgroup's piece of a buffer row stays a few cache lines long
     const long long per_z = (long long)((g.Wp + R - 1) / R) * g.Hp;
-    while (per_z * (g.C / CB) < 8LL * state().num_cu && CB % 2 == 0 && (CB / 2) * PK * ES >= 256 && ((CB / 2) * PK) % VEC == 0)
+    while (per_z * (g.C / CB) < 2LL * state().num_cu && CB % 2 == 0 && (CB / 2) * PK * ES >= 256 && ((CB / 2) * PK) % VEC == 0)
         CB /= 2;
     if (bytes(CB) > 64 * 1024 || (CB * PK) % VEC || CB * g.Hk * LW >= 65536 || g.C / CB >= 65536) return -1;
-    const int cpr = CB * PK / VEC;
-    if ((long long)R * cpr >= 65536) return -1;  // (the flat item index stays within the exact range of the reciprocal)
     auto magic = [](unsigned d) { return (unsigned)((((unsigned long long)1 << 32) + d - 1) / d); };
     dim3 grid((g.Wp + R - 1) / R, g.Hp, g.C / CB);
-    hipLaunchKernelGGL((patch_rows_kernel<T>), grid, dim3(256), bytes(CB), state().stream, src, buf, g, R, CB, LW, magic(cpr),
-                       magic(PK), magic(g.Wk));
+    if (wide)
+        hipLaunchKernelGGL((patch_rows_kernel<T, true>), grid, dim3(256), bytes(CB), state().stream, src, buf, g, R, CB, LW,
+                           magic(PK), magic(g.Wk), magic(g.Hk));
+    else
+        hipLaunchKernelGGL((patch_rows_kernel<T, false>), grid, dim3(256), bytes(CB), state().stream, src, buf, g, R, CB,
+                           LW, magic(PK), magic(g.Wk), magic(g.Hk));
     return hip_ok(hipGetLastError(), "patch launch") ? 0 : 2;
 }
 
