@@ -1980,6 +1980,90 @@ __global__ __launch_bounds__(256) void pad_kernel(const T *__restrict__ src, T *
     }
 }
 
+// The same result with far fewer instructions per chunk, for rows of at least one chunk.  Both layouts are one
+// case: NR = groups x Ho rows of WoE elements, of which rows U .. U+H-1 of a group hold WE source elements from
+// column LE on (channel-major: groups = C, WoE = Wo; channel-last: one group, rows of Wo x C).  The source elements
+// that a run of destination elements takes are consecutive, so a workgroup copies the aligned 16-byte pieces of the
+// source that cover its 256 chunks into LDS (one coalesced load per thread), and a thread picks its chunk out of
+// them: validity is a bit mask built from the two row segments a chunk can touch, and the e-th valid element is the
+// (number of valid elements before it)-th after the chunk's first.  The row and column of a workgroup's first
+// element come from one division per workgroup; a thread's own from reciprocal multiplications on the small rest.
+struct PadRows {
+    int Ho, H, U, WoE, WE, LE;
+    unsigned m_wo, m_ho;  // ceil(2^32 / WoE), ceil(2^32 / Ho)
+};
+
+template <typename T>
+__global__ __launch_bounds__(256) void pad_rows_kernel(const T *__restrict__ src, T *__restrict__ dst, PadRows g,
+                                                       unsigned total, unsigned n_src) {
+    constexpr int PER = 16 / (int)sizeof(T);
+    __shared__ __attribute__((aligned(16))) T span[(256 + 2) * PER];
+    // valid source elements before destination position (group c, row ht, column wt)
+    auto before = [&](unsigned c, int ht, int wt) {
+        const int rows = min(max(ht - g.U, 0), g.H);
+        const int cols = (unsigned)(ht - g.U) < (unsigned)g.H ? min(max(wt - g.LE, 0), g.WE) : 0;
+        return (c * g.H + rows) * (unsigned)g.WE + cols;
+    };
+    const unsigned B = blockIdx.x * (256u * PER);
+    const unsigned r_B = B / (unsigned)g.WoE, wt_B = B - r_B * g.WoE;
+    const unsigned c_B = r_B / (unsigned)g.Ho, ht_B = r_B - c_B * g.Ho;
+    const unsigned s_lo = before(c_B, (int)ht_B, (int)wt_B) & ~(unsigned)(PER - 1);
+    // the pieces of the source this workgroup's chunks can take from: at most 256 x PER elements and two ragged
+    // ends - a piece per thread and two more, both loads on their way before either is waited for (what lies
+    // beyond the source comes from a piece of zeros: a load under a condition would wait on its own)
+    {
+        typedef const PatchPiece __attribute__((address_space(1))) *GlobalPiece;
+        const unsigned at0 = s_lo + threadIdx.x * PER, at1 = s_lo + (256 + threadIdx.x) * PER;
+        const bool more = threadIdx.x < 2;
+        const PatchPiece v0 = *(at0 + PER <= n_src ? (GlobalPiece)(src + at0) : (GlobalPiece)&patch_zero);
+        const PatchPiece v1 = *(more && at1 + PER <= n_src ? (GlobalPiece)(src + at1) : (GlobalPiece)&patch_zero);
+        *reinterpret_cast<PatchPiece *>(span + threadIdx.x * PER) = v0;
+        if (more) *reinterpret_cast<PatchPiece *>(span + (256 + threadIdx.x) * PER) = v1;
+        // (the tensor's last, partial piece, element by element)
+        if (at0 < n_src && at0 + PER > n_src)
+            for (int e = 0; at0 + e < n_src; ++e) span[threadIdx.x * PER + e] = src[at0 + e];
+        if (more && at1 < n_src && at1 + PER > n_src)
+            for (int e = 0; at1 + e < n_src; ++e) span[(256 + threadIdx.x) * PER + e] = src[at1 + e];
+    }
+    __syncthreads();
+    const unsigned idx0 = B + threadIdx.x * PER;
+    if (idx0 >= total) return;
+    // this thread's row and column: a few rows below the workgroup's first
+    const unsigned x = wt_B + threadIdx.x * PER, dr = div_magic(x, g.m_wo);
+    const int wt = (int)(x - dr * g.WoE);
+    const unsigned y = ht_B + dr, dc = div_magic(y, g.m_ho);
+    const int ht = (int)(y - dc * g.Ho);
+    const unsigned c = c_B + dc;
+    // valid positions of the chunk: the rest of this row, then the start of the next
+    const int n1 = min(PER, g.WoE - wt), ht2 = ht + 1 == g.Ho ? 0 : ht + 1;
+    unsigned mask = 0;
+    if ((unsigned)(ht - g.U) < (unsigned)g.H) {
+        const int lo = max(g.LE - wt, 0), hi = min(g.LE + g.WE - wt, n1);
+        if (hi > lo) mask = ((1u << hi) - 1u) & ~((1u << lo) - 1u);
+    }
+    if (n1 < PER && (unsigned)(ht2 - g.U) < (unsigned)g.H) {
+        const int lo = n1 + g.LE, hi = min(n1 + g.LE + g.WE, PER);
+        if (hi > lo) mask |= ((1u << hi) - 1u) & ~((1u << lo) - 1u);
+    }
+    const T *from = span + (before(c, ht, wt) - s_lo);
+    union {
+        uint4 u;
+        T e[PER];
+    } out;
+#pragma unroll
+    for (int e = 0; e < PER; ++e) {
+        const T v = from[__popc(mask & ((1u << e) - 1u))];
+        out.e[e] = (mask >> e) & 1u ? v : (T)0;
+    }
+    if (idx0 + PER <= total) {
+        *reinterpret_cast<uint4 *>(dst + idx0) = out.u;
+    } else {
+#pragma unroll
+        for (int e = 0; e < PER; ++e)
+            if (idx0 + e < total) dst[idx0 + e] = out.e[e];
+    }
+}
+
 template <typename T, typename Args>
 static int pad_step(const Args *a, const char *fn) {
     if (!a || !a->source || !a->dest) {
@@ -2008,7 +2092,20 @@ static int pad_step(const Args *a, const char *fn) {
     if (sg.failed()) return 2;
     constexpr int VEC = 16 / (int)sizeof(T);
     const size_t n_src = (size_t)a->C * a->H * a->W;
-    if (reinterpret_cast<uintptr_t>(d) % 16 == 0)
+    // rows of at least a chunk, short enough for the reciprocal divisions (exact below 2^16) of a row or column
+    // index a workgroup's 256 chunks further on
+    const long long WoE = a->HWC_lay ? (long long)Wo * a->C : Wo;
+    const bool rows_form = reinterpret_cast<uintptr_t>(d) % 16 == 0 && reinterpret_cast<uintptr_t>(s) % 16 == 0 &&
+                           WoE >= VEC && WoE + 256 * VEC < 65536 && Ho + 256 * VEC < 65536 && state().gemm_path != 1;
+    if (rows_form) {
+        PadRows g;
+        g.Ho = Ho; g.H = a->H; g.U = a->T_UPAD;
+        g.WoE = (int)WoE; g.WE = a->HWC_lay ? a->W * a->C : a->W; g.LE = a->HWC_lay ? a->T_LPAD * a->C : a->T_LPAD;
+        g.m_wo = (unsigned)((((unsigned long long)1 << 32) + g.WoE - 1) / g.WoE);
+        g.m_ho = (unsigned)((((unsigned long long)1 << 32) + Ho - 1) / Ho);
+        hipLaunchKernelGGL((pad_rows_kernel<T>), dim3(nblocks((total + VEC - 1) / VEC)), dim3(256), 0, state().stream, s, d,
+                           g, (unsigned)total, (unsigned)n_src);
+    } else if (reinterpret_cast<uintptr_t>(d) % 16 == 0)
         hipLaunchKernelGGL((pad_kernel<T, VEC>), dim3(nblocks((total + VEC - 1) / VEC)), dim3(256), 0, state().stream, s, d,
                            a->C, a->H, a->W, a->T_LPAD, a->T_UPAD, Ho, Wo, a->HWC_lay, total, n_src);
     else

@@ -250,7 +250,9 @@ def test_im2row_im2col_chunked(pkg, orc, gpu, dt, hwc, Ci, H, W, K, pad, stride,
 
 @pytest.mark.parametrize("dt", ["fp32", "fp16"])
 @pytest.mark.parametrize("hwc", [0, 1])
-@pytest.mark.parametrize("C,H,W,pads", [(16, 32, 32, (1, 1, 1, 1)), (5, 9, 13, (2, 0, 1, 3)), (3, 7, 7, (0, 0, 0, 0))])
+@pytest.mark.parametrize("C,H,W,pads", [(16, 32, 32, (1, 1, 1, 1)), (5, 9, 13, (2, 0, 1, 3)), (3, 7, 7, (0, 0, 0, 0)),
+                                         (64, 60, 52, (1, 1, 1, 1)), (7, 130, 37, (3, 2, 0, 5)), (2, 5, 4001, (1, 0, 1, 1)),
+                                         (33, 3, 5, (0, 4, 2, 0)), (3, 700, 9, (1, 2, 300, 1))])
 def test_pad_tensor_chunked(pkg, orc, gpu, dt, hwc, C, H, W, pads):
     nd = hp.np_dtype(dt)
     R, L, U, D = pads
