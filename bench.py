@@ -592,6 +592,9 @@ def helper_rows(pkg, lib, hp, timed, torch, dev):
         a.stride_h = a.stride_w = 1
         ms = timed(void_call("pulp_im2row_" + dt, a), 10)
         add("im2row 64x224x224 k3 p1", dt, ms, (x.numel() + buf.numel()) * es[dt])
+        if dt == "fp16":  # the column-major patch matrix of the same input
+            ms = timed(void_call("pulp_im2col_" + dt, a), 10)
+            add("im2col 64x224x224 k3 p1", dt, ms, (x.numel() + buf.numel()) * es[dt])
         del x, buf
     # pad_tensor 256 x 360 x 360 by one on every side (63 MiB -> 64 MiB in fp16)
     C, H, dt = 256, 360, "fp16"

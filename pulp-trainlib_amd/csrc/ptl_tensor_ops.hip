@@ -1102,6 +1102,9 @@ struct PatchGeom {
     int col_major;  // 0: buf[p*Q + q] (im2row); 1: buf[q*P + p] (im2col)
 };
 
+typedef unsigned PatchPiece __attribute__((ext_vector_type(4)));  // (a built-in vector: loads from any address space)
+__device__ const PatchPiece patch_zero = {0u, 0u, 0u, 0u};  // what the window holds outside the tensor
+
 // buf(p, q) = src[c, hp*h_mul + h_add + hk, wp*w_mul + w_add + wk] or 0 outside,
 // p = hp*Wp + wp, q = (c,hk,wk) for CHW and (hk,wk,c) for HWC.
 // A thread writes PER consecutive elements of the buffer (one 16-byte store when PER elements fill 16 bytes and
@@ -1140,9 +1143,13 @@ __global__ __launch_bounds__(256) void patch_kernel(const T *__restrict__ src, T
 #pragma unroll
     for (int e = 0; e < PER; ++e) {
         const int h = hp * g.h_mul + g.h_add + hk, w = wp * g.w_mul + g.w_add + wk;
-        v[e] = (T)0;
-        if (idx0 + e < total && (unsigned)h < (unsigned)g.Hs && (unsigned)w < (unsigned)g.Ws)
-            v[e] = g.hwc ? src[((size_t)h * g.Ws + w) * g.C + c] : src[((size_t)c * g.Hs + h) * g.Ws + w];
+        // (every lane always loads, what lies outside the tensor from a word of zeros: a load under a condition
+        // becomes a branch with a wait of its own, one trip to memory per element; 32-bit offsets - the host keeps
+        // the source below 2^32 elements)
+        const bool ok = idx0 + e < total && (unsigned)h < (unsigned)g.Hs && (unsigned)w < (unsigned)g.Ws;
+        const unsigned off = g.hwc ? ((unsigned)h * g.Ws + w) * g.C + c : ((unsigned)c * g.Hs + h) * g.Ws + w;
+        typedef const T __attribute__((address_space(1))) *GlobalT;
+        v[e] = *(ok ? (GlobalT)(src + off) : (GlobalT)&patch_zero);
         // next element of the buffer
         bool next_q = true, next_p = false;
         if (g.col_major) {  // p runs fastest
@@ -1227,8 +1234,6 @@ __global__ __launch_bounds__(256) void patch_kernel(const T *__restrict__ src, T
 // is read in as few instructions as the layout allows: WIDE (rows of the tensor start on 16-byte boundaries) takes
 // the aligned 16-byte pieces that cover the window - the window then starts up to a piece early, `shift` elements
 // that the offsets table skips - and otherwise one element per lane, one wave per window row.
-typedef unsigned PatchPiece __attribute__((ext_vector_type(4)));  // (a built-in vector: loads from any address space)
-__device__ const PatchPiece patch_zero = {0u, 0u, 0u, 0u};  // what the window holds outside the tensor
 
 template <typename T, bool WIDE>
 __global__ __launch_bounds__(256) void patch_rows_kernel(const T *__restrict__ src, T *__restrict__ buf, PatchGeom g, int R,
@@ -1325,6 +1330,75 @@ __global__ __launch_bounds__(256) void patch_rows_kernel(const T *__restrict__ s
             dst += (size_t)pstep * Q;
         }
     }
+}
+
+// Column-major patch matrix (im2col) of a channel-major tensor at unit column stride: row q = (c, hk, wk) of the
+// buffer is channel c's plane shifted by the tap, so a 16-byte chunk of it (consecutive grid columns of one grid
+// row, when the grid's width is a whole number of chunks) is one run of consecutive source elements.  A thread
+// loads that run with one 16-byte access at element alignment - from a start moved inside the row where the run
+// would begin before it or end behind it - and shifts the 128 bits by the distance moved, which leaves zeros in
+// exactly the positions that lie outside the row; a run in a row outside the tensor reads a piece of zeros.  One
+// division per workgroup, reciprocal multiplications on the small per-thread rests.
+struct PatchCols {
+    int cpr, wpc;              // chunks per buffer row, chunks per grid row
+    unsigned m_cpr, m_wpc, m_pk, m_wk;
+};
+
+template <typename T>
+__global__ __launch_bounds__(256) void patch_cols_kernel(const T *__restrict__ src, T *__restrict__ buf, PatchGeom g,
+                                                         PatchCols k, unsigned chunks) {
+    constexpr int VEC = 16 / (int)sizeof(T), EB = 8 * (int)sizeof(T);
+    typedef unsigned Run __attribute__((ext_vector_type(4), aligned(2)));  // (element alignment of the narrower type)
+    typedef const Run __attribute__((address_space(1))) *GlobalRun;
+    const unsigned B = blockIdx.x * 256u, i = B + threadIdx.x;
+    if (i >= chunks) return;
+    const int PK = g.Hk * g.Wk;
+    const unsigned q_B = B / (unsigned)k.cpr, r_B = B - q_B * k.cpr;
+    const unsigned c_B = q_B / (unsigned)PK, t_B = q_B - c_B * PK;
+    const unsigned x = r_B + threadIdx.x, dq = div_magic(x, k.m_cpr), r = x - dq * k.cpr;
+    const unsigned t2 = t_B + dq, dc = div_magic(t2, k.m_pk), t3 = t2 - dc * PK;
+    const int c = (int)(c_B + dc), hk = (int)div_magic(t3, k.m_wk), wk = (int)t3 - hk * g.Wk;
+    const int hp = (int)div_magic(r, k.m_wpc), wp0 = ((int)r - hp * k.wpc) * VEC;
+    const int h = hp * g.h_mul + g.h_add + hk, w0 = wp0 + g.w_add + wk;
+    const int w_in = min(max(w0, 0), g.Ws - VEC), d = w0 - w_in;  // d > 0: the run ends behind the row
+    const bool ok = (unsigned)h < (unsigned)g.Hs && d > -VEC && d < VEC;
+    const unsigned off = ((unsigned)c * g.Hs + h) * g.Ws + w_in;
+    Run v = *(ok ? (GlobalRun)(src + off) : (GlobalRun)&patch_zero);
+    const int bits = (d < 0 ? -d : d) * EB;
+    if (d > 0) {  // towards element 0
+        if (bits & 64) v = Run{v.z, v.w, 0u, 0u};
+        if (bits & 32) v = Run{v.y, v.z, v.w, 0u};
+        const unsigned bs = bits & 31;
+        v = Run{__builtin_amdgcn_alignbit(v.y, v.x, bs), __builtin_amdgcn_alignbit(v.z, v.y, bs),
+                __builtin_amdgcn_alignbit(v.w, v.z, bs), v.w >> bs};
+    } else if (d < 0) {
+        if (bits & 64) v = Run{0u, 0u, v.x, v.y};
+        if (bits & 32) v = Run{0u, v.x, v.y, v.z};
+        const unsigned bs = bits & 31;  // (0 or 16: a left shift by 16 is alignbit(hi, lo, 16) one dword up)
+        if (bs) v = Run{v.x << 16, __builtin_amdgcn_alignbit(v.y, v.x, 16), __builtin_amdgcn_alignbit(v.z, v.y, 16),
+                        __builtin_amdgcn_alignbit(v.w, v.z, 16)};
+    }
+    typedef unsigned Chunk __attribute__((ext_vector_type(4)));
+    *reinterpret_cast<Chunk *>(buf + (size_t)i * VEC) = Chunk{v.x, v.y, v.z, v.w};
+}
+
+// 0 = launched; -1 = the geometry does not fit (the caller takes the general kernel).
+template <typename T>
+static int patch_cols(const T *src, T *buf, const PatchGeom &g) {
+    constexpr int VEC = 16 / (int)sizeof(T);
+    if (g.hwc || !g.col_major || g.w_mul != 1 || g.Wp % VEC || g.Ws < VEC || reinterpret_cast<uintptr_t>(buf) % 16)
+        return -1;
+    const long long P = (long long)g.Hp * g.Wp, PK = (long long)g.Hk * g.Wk, chunks = P / VEC * PK * g.C;
+    // (the reciprocal divisions are exact below 2^16: a row or tap index at most a workgroup's 256 chunks further on)
+    if (P / VEC + 256 >= 65536 || PK + 256 >= 65536 || chunks >= ((long long)1 << 32) / 256 * 256) return -1;
+    auto magic = [](unsigned d) { return (unsigned)((((unsigned long long)1 << 32) + d - 1) / d); };
+    PatchCols k;
+    k.cpr = (int)(P / VEC);
+    k.wpc = g.Wp / VEC;
+    k.m_cpr = magic(k.cpr); k.m_wpc = magic(k.wpc); k.m_pk = magic((unsigned)PK); k.m_wk = magic(g.Wk);
+    hipLaunchKernelGGL((patch_cols_kernel<T>), dim3((unsigned)((chunks + 255) / 256)), dim3(256), 0, state().stream, src, buf, g,
+                       k, (unsigned)chunks);
+    return hip_ok(hipGetLastError(), "patch launch") ? 0 : 2;
 }
 
 // 0 = launched; -1 = the geometry does not fit (the caller takes the general kernel).
@@ -1454,11 +1528,12 @@ static int patch_build(const Args *a, int col_major, const char *fn) {
     T *dbuf = sg.out(reinterpret_cast<T *>(a->pBuffer), total);
     if (sg.failed()) return 2;
     constexpr int VEC = 16 / (int)sizeof(T);
-    if (total >= ((size_t)1 << 32)) {
-        set_error("%s: patch matrix of 2^32 elements or more", fn);
+    if (total >= ((size_t)1 << 32) || src_n >= ((size_t)1 << 32)) {
+        set_error("%s: patch matrix or source of 2^32 elements or more", fn);
         return sg.finish(1);
     }
     if (int rc = patch_rows<T>(dsrc, dbuf, g); rc >= 0) return sg.finish(rc);
+    if (int rc = patch_cols<T>(dsrc, dbuf, g); rc >= 0) return sg.finish(rc);
     if (reinterpret_cast<uintptr_t>(dbuf) % 16 == 0)
         hipLaunchKernelGGL((patch_kernel<T, VEC>), dim3(nblocks((total + VEC - 1) / VEC)), dim3(256), 0, state().stream,
                            dsrc, dbuf, g, total);

@@ -220,7 +220,10 @@ def test_blocktranspose_tiles(pkg, orc, gpu, dt, hwc, Ci, Co, Hk, Wk):
 @pytest.mark.parametrize("hwc", [0, 1])
 @pytest.mark.parametrize("Ci,H,W,K,pad,stride,mod", [(16, 32, 32, 3, (1, 1, 1, 1), (1, 1), 0), (7, 19, 23, 3, (1, 1, 1, 1), (2, 2), 0),
                                                      (6, 14, 9, 5, (2, 2, 2, 2), (1, 1), 0), (5, 12, 12, 3, (0, 0, 0, 0), (1, 1), 1),
-                                                     (16, 32, 32, 1, (0, 0, 0, 0), (1, 1), 0), (64, 40, 48, 1, (0, 0, 0, 0), (1, 1), 0)])
+                                                     (16, 32, 32, 1, (0, 0, 0, 0), (1, 1), 0), (64, 40, 48, 1, (0, 0, 0, 0), (1, 1), 0),
+                                                     (8, 20, 24, 5, (2, 2, 2, 2), (1, 1), 0), (4, 19, 16, 3, (1, 1, 1, 1), (2, 1), 0),
+                                                     (3, 8, 8, 3, (1, 1, 1, 1), (1, 1), 0), (6, 10, 16, 3, (0, 0, 0, 0), (1, 1), 1),
+                                                     (2, 70, 136, 3, (1, 1, 1, 1), (1, 1), 0)])
 def test_im2row_im2col_chunked(pkg, orc, gpu, dt, hwc, Ci, H, W, K, pad, stride, mod):
     """Patch matrices whose rows are not multiples of a 16-byte chunk (chunks straddle rows and columns), BASELINE
     config 1 among them."""
