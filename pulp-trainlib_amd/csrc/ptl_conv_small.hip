@@ -210,13 +210,14 @@ constexpr int WG_CHUNKS = 4;  // 16-byte pieces per thread and tensor, at most
 struct WgSmallArgs {
     const void *X, *dY;
     float *ws;
-    int batch, Cin, Cout, Hin, Win, Ho, padU, padL;
+    int batch, Cin, Cout, Hin, Win, Ho, Wo, padU, padL;
+    int stride, rows_in;           // 1 or 2 (both ways); input rows a tile of R output rows meets: (R - 1) * stride + 3
     int nwg, S, R, tiles_per_img;  // workgroups; samples and output rows per tile (R = Ho when S > 1)
-    int G, RG, R2G;                // 16-byte column groups per row, per R rows, per R + 2 rows
+    int G, RG, Gin, R2G;           // 16-byte column groups per gradient row, per R of them; per input row, per rows_in of them
     int PY, PX, WP;                // LDS pitches in elements: gradient channel, input channel, input row
     int groups;                    // S * R * G
     int y_chunks, x_chunks, pad_chunks, pad_rows;  // pieces to copy; zero pieces (one per input row + one) and rows per channel
-    unsigned magic_g, magic_rg, magic_r2g, magic_ychan, magic_xchan, magic_padrows, magic_tile, magic_cols;
+    unsigned magic_g, magic_gin, magic_rg, magic_r2g, magic_ychan, magic_xchan, magic_padrows, magic_tile, magic_cols;
     int cbi_n, combos, kparts;  // 32-channel blocks, (filter block, channel block) pairs, position shares
     int total;                  // Cout * Cin * 9
     int rows_kept, cols_kept, part_elems;  // filter rows and channels of a 32x32 tile that are stored; floats per workgroup in ws
@@ -258,7 +259,11 @@ __device__ inline uint4 shifted_piece(const uint4 &c, unsigned p3, unsigned n0) 
     return make_uint4(c.y, c.z, c.w, n0);
 }
 
-template <typename T, int PADL>
+// STRIDE 2 (one column of left padding): an input row is kept as its even and its odd columns, each half behind a
+// zero piece of its own - the eight input columns 2 x + kx - 1 that meet eight consecutive gradient columns x are
+// then eight consecutive elements again: of the odd half one to the left (kx = 0), of the even half (1), of the odd
+// half (2) - and gradient row y meets input rows 2 y + ky.
+template <typename T, int PADL, int STRIDE>
 __device__ inline void wg_small_block(const WgSmallArgs &a, int wg, char *smem) {
     constexpr int VEC = 16 / (int)sizeof(T);
     typedef typename EdgePair<T>::type edge_t;
@@ -282,21 +287,23 @@ __device__ inline void wg_small_block(const WgSmallArgs &a, int wg, char *smem) 
             const int s = fast_div(rem, a.magic_rg), r2 = rem - s * a.RG;
             const int ly = fast_div(r2, a.magic_g), xg = r2 - ly * a.G;
             if (b0 + s < a.batch && y0 + ly < a.Ho)
-                yv[k] = *reinterpret_cast<const uint4 *>(gY + (((size_t)(b0 + s) * a.Cout + co) * a.Ho + y0 + ly) * a.Win + VEC * xg);
+                yv[k] = *reinterpret_cast<const uint4 *>(gY + (((size_t)(b0 + s) * a.Cout + co) * a.Ho + y0 + ly) * a.Wo + VEC * xg);
         }
         if (q < a.x_chunks) {
             const int ci = fast_div(q, a.magic_xchan), rem = q - ci * xchan;
             const int s = fast_div(rem, a.magic_r2g), r2 = rem - s * a.R2G;
-            const int ly = fast_div(r2, a.magic_g), xg = r2 - ly * a.G;
-            const int iy = y0 - a.padU + ly;
+            const int ly = fast_div(r2, a.magic_gin), xg = r2 - ly * a.Gin;
+            const int iy = y0 * STRIDE - a.padU + ly;
             if (b0 + s < a.batch && iy >= 0 && iy < a.Hin)
                 xv[k] = *reinterpret_cast<const uint4 *>(gX + (((size_t)(b0 + s) * a.Cin + ci) * a.Hin + iy) * a.Win + VEC * xg);
         }
     }
     // zero pieces: in front of every input row and behind the last one; behind the last gradient group
     for (int q = tid; q < a.pad_chunks; q += CS_NT) {
-        const int ci = fast_div(q, a.magic_padrows), row = q - ci * a.pad_rows;
-        *reinterpret_cast<uint4 *>(Xs + ci * a.PX + row * a.WP) = make_uint4(0, 0, 0, 0);
+        const int ci = fast_div(q, a.magic_padrows), j = q - ci * a.pad_rows;
+        // (per row one piece, or one per half; the last one behind the last row)
+        const int at = STRIDE == 1 ? j * a.WP : (j >> 1) * a.WP + (j & 1) * (VEC + a.Win / 2);
+        *reinterpret_cast<uint4 *>(Xs + ci * a.PX + at) = make_uint4(0, 0, 0, 0);
     }
     for (int co = tid; co < a.Cout; co += CS_NT)
         *reinterpret_cast<uint4 *>(Ys + co * a.PY + a.groups * VEC) = make_uint4(0, 0, 0, 0);
@@ -309,8 +316,23 @@ __device__ inline void wg_small_block(const WgSmallArgs &a, int wg, char *smem) 
         }
         if (q < a.x_chunks) {
             const int ci = fast_div(q, a.magic_xchan), rem = q - ci * xchan;
-            const int row = fast_div(rem, a.magic_g), xg = rem - row * a.G;  // row = s * (R + 2) + ly
-            *reinterpret_cast<uint4 *>(Xs + ci * a.PX + row * a.WP + VEC + VEC * xg) = xv[k];
+            const int row = fast_div(rem, a.magic_gin), xg = rem - row * a.Gin;  // row = s * rows_in + ly
+            T *at = Xs + ci * a.PX + row * a.WP + VEC;
+            if constexpr (STRIDE == 1) {
+                *reinterpret_cast<uint4 *>(at + VEC * xg) = xv[k];
+            } else {
+                const uint4 c = xv[k];
+                uint2 even, odd;
+                if constexpr (sizeof(T) == 2) {
+                    even = make_uint2((c.x & 0xffffu) | (c.y << 16), (c.z & 0xffffu) | (c.w << 16));
+                    odd = make_uint2((c.x >> 16) | (c.y & 0xffff0000u), (c.z >> 16) | (c.w & 0xffff0000u));
+                } else {
+                    even = make_uint2(c.x, c.z);
+                    odd = make_uint2(c.y, c.w);
+                }
+                *reinterpret_cast<uint2 *>(at + (VEC / 2) * xg) = even;
+                *reinterpret_cast<uint2 *>(at + VEC + a.Win / 2 + (VEC / 2) * xg) = odd;
+            }
         }
     }
     __syncthreads();
@@ -333,7 +355,7 @@ __device__ inline void wg_small_block(const WgSmallArgs &a, int wg, char *smem) 
         const T *xrow = Xs + min(cbi * 32 + lr, a.Cin - 1) * a.PX + ky * a.WP + VEC;
         constexpr int U = 4;  // k steps whose LDS reads are in flight together
         for (int ks0 = kpart; ks0 < nks; ks0 += U * a.kparts) {
-            uint4 A[U], C[U];
+            uint4 A[U], C[U], D[U];
             edge_t p3[U], n0[U];
 #pragma unroll
             for (int u = 0; u < U; ++u) {
@@ -342,17 +364,31 @@ __device__ inline void wg_small_block(const WgSmallArgs &a, int wg, char *smem) 
                 const int gx = min(gi, a.groups - 1);
                 const int s = fast_div(gx, a.magic_rg), r2 = gx - s * a.RG;
                 const int ly = fast_div(r2, a.magic_g), xg = r2 - ly * a.G;
-                const T *xp = xrow + (s * (a.R + 2) + ly) * a.WP + VEC * xg;
+                const T *xp = xrow + (s * a.rows_in + STRIDE * ly) * a.WP + VEC * xg;
                 A[u] = *reinterpret_cast<const uint4 *>(yrow + gi * VEC);
-                C[u] = *reinterpret_cast<const uint4 *>(xp);
-                p3[u] = *reinterpret_cast<const edge_t *>(xp - 2);
-                n0[u] = *reinterpret_cast<const edge_t *>(xp + VEC);
+                if constexpr (STRIDE == 1) {
+                    C[u] = *reinterpret_cast<const uint4 *>(xp);
+                    p3[u] = *reinterpret_cast<const edge_t *>(xp - 2);
+                    n0[u] = *reinterpret_cast<const edge_t *>(xp + VEC);
+                } else {  // C: the even half's piece; D, with the two elements before it: the odd half's
+                    const T *xo = xp + VEC + a.Win / 2;
+                    C[u] = *reinterpret_cast<const uint4 *>(xp);
+                    D[u] = *reinterpret_cast<const uint4 *>(xo);
+                    p3[u] = *reinterpret_cast<const edge_t *>(xo - 2);
+                    n0[u] = p3[u];
+                }
             }
 #pragma unroll
             for (int u = 0; u < U; ++u) {
-                mfma_step<T>(acc[0], A[u], shifted_piece<0 - PADL>(C[u], p3[u], n0[u]));
-                mfma_step<T>(acc[1], A[u], shifted_piece<1 - PADL>(C[u], p3[u], n0[u]));
-                mfma_step<T>(acc[2], A[u], shifted_piece<2 - PADL>(C[u], p3[u], n0[u]));
+                if constexpr (STRIDE == 1) {
+                    mfma_step<T>(acc[0], A[u], shifted_piece<0 - PADL>(C[u], p3[u], n0[u]));
+                    mfma_step<T>(acc[1], A[u], shifted_piece<1 - PADL>(C[u], p3[u], n0[u]));
+                    mfma_step<T>(acc[2], A[u], shifted_piece<2 - PADL>(C[u], p3[u], n0[u]));
+                } else {
+                    mfma_step<T>(acc[0], A[u], shifted_piece<-1>(D[u], p3[u], n0[u]));
+                    mfma_step<T>(acc[1], A[u], C[u]);
+                    mfma_step<T>(acc[2], A[u], D[u]);
+                }
             }
         }
     }
@@ -395,12 +431,14 @@ __device__ inline void wg_small_block(const WgSmallArgs &a, int wg, char *smem) 
 
 template <typename T>
 __device__ inline void wg_small_any(const WgSmallArgs &a, int wg, char *smem) {
-    if (a.padL == 1)
-        wg_small_block<T, 1>(a, wg, smem);
+    if (a.stride == 2)
+        wg_small_block<T, 1, 2>(a, wg, smem);
+    else if (a.padL == 1)
+        wg_small_block<T, 1, 1>(a, wg, smem);
     else if (a.padL == 0)
-        wg_small_block<T, 0>(a, wg, smem);
+        wg_small_block<T, 0, 1>(a, wg, smem);
     else
-        wg_small_block<T, 2>(a, wg, smem);
+        wg_small_block<T, 2, 1>(a, wg, smem);
 }
 
 template <typename T>
@@ -595,10 +633,15 @@ int plan_wg(const ConvTileDesc &d, const void *X, const void *dY, int max_wg, bo
     constexpr int ES = (int)sizeof(T), VEC = 16 / ES;
     State &st = state();
     if (st.gemm_path != 0 && st.gemm_path != 6) return -1;  // (the other values select one of the other routes)
-    if (d.in_hwc || d.KH != 3 || d.KW != 3 || d.sh != 1 || d.sw != 1) return -1;
-    if (d.Cin > 64 || d.Cout > 64 || d.Win % VEC != 0 || d.Wo != d.Win || d.x_sy != d.Win) return -1;
+    if (d.in_hwc || d.KH != 3 || d.KW != 3 || d.sh != d.sw || d.sh < 1 || d.sh > 2) return -1;
+    const int st2 = d.sh == 2;
+    if (d.Cin > 64 || d.Cout > 64 || d.Win % VEC != 0 || d.Wo % VEC != 0 || d.x_sy != d.Win) return -1;
     if (d.x_sc != (long long)d.Hin * d.Win || d.x_sb != (long long)d.Cin * d.Hin * d.Win) return -1;
     if (d.padU < 0 || d.padL < 0 || d.padL > 2) return -1;
+    // unit stride: a gradient row as long as an input row; stride 2: half as long, one column of left padding, and
+    // the input columns the last gradient column meets inside the row
+    if (!st2 && d.Wo != d.Win) return -1;
+    if (st2 && (d.padL != 1 || d.Win % (2 * VEC) != 0 || d.Wo * 2 != d.Win)) return -1;
     if (reinterpret_cast<uintptr_t>(X) % 16 || reinterpret_cast<uintptr_t>(dY) % 16) return -1;
     w = WgSmallArgs();
     w.total = d.Cout * d.Cin * 9;
@@ -609,16 +652,19 @@ int plan_wg(const ConvTileDesc &d, const void *X, const void *dY, int max_wg, bo
     // against 8.4 us for 16 -> 32 on 32x32 at one sample: below a few thousand positions what this kernel buys is
     // the input gradient riding along in the same launch)
     if (st.gemm_path != 6 && (positions > 262144 || (alone && positions < 8192))) return -1;
-    w.G = d.Win / VEC;
-    w.WP = d.Win + VEC;
+    w.G = d.Wo / VEC;
+    w.Gin = d.Win / VEC;
+    w.stride = d.sh;
+    w.WP = d.Win + (st2 ? 2 : 1) * VEC;
+    auto rows_in = [&](int R) { return (R - 1) * d.sh + 3; };
     // pitches of 16 bytes mod 128: consecutive channels 16 bytes apart in the banks
     auto round_pitch = [](int n) { return n + ((VEC - n % (8 * VEC)) + 8 * VEC) % (8 * VEC); };
     auto lds_of = [&](int S, int R) {
-        const int py = round_pitch(S * R * d.Win + VEC), px = round_pitch((S * (R + 2) + 1) * w.WP);
+        const int py = round_pitch(S * R * d.Wo + VEC), px = round_pitch((S * rows_in(R) + 1) * w.WP);
         return ((size_t)d.Cout * py + (size_t)d.Cin * px) * ES;
     };
     auto chunks_ok = [&](int S, int R) {
-        return (long long)d.Cout * S * R * w.G <= WG_CHUNKS * CS_NT && (long long)d.Cin * S * (R + 2) * w.G <= WG_CHUNKS * CS_NT &&
+        return (long long)d.Cout * S * R * w.G <= WG_CHUNKS * CS_NT && (long long)d.Cin * S * rows_in(R) * w.Gin <= WG_CHUNKS * CS_NT &&
                lds_of(S, R) <= WG_SMALL_LDS;
     };
     // tiles: whole samples while the partial sums stay within about 5 MB (S samples each otherwise), rows of a
@@ -635,16 +681,18 @@ int plan_wg(const ConvTileDesc &d, const void *X, const void *dY, int max_wg, bo
     w.S = S; w.R = R;
     w.tiles_per_img = (d.Ho + R - 1) / R;
     w.nwg = ((d.batch + S - 1) / S) * w.tiles_per_img;
-    w.RG = R * w.G; w.R2G = (R + 2) * w.G;
+    w.rows_in = rows_in(R);
+    w.RG = R * w.G; w.R2G = w.rows_in * w.Gin;
     w.groups = S * w.RG;
     w.PY = round_pitch(w.groups * VEC + VEC);
-    w.pad_rows = S * (R + 2) + 1;
-    w.PX = round_pitch(w.pad_rows * w.WP);
+    w.pad_rows = (st2 ? 2 : 1) * S * w.rows_in + 1;
+    w.PX = round_pitch((S * w.rows_in + 1) * w.WP);
     w.y_chunks = d.Cout * w.groups;
     w.x_chunks = d.Cin * S * w.R2G;
     w.pad_chunks = d.Cin * w.pad_rows;
     if (w.y_chunks >= 65536 || w.x_chunks >= 65536 || w.pad_chunks >= 65536) return -1;  // (reciprocal multiplication)
     w.magic_g = magic_of(w.G);
+    w.magic_gin = magic_of(w.Gin);
     w.magic_rg = magic_of(w.RG);
     w.magic_r2g = magic_of(w.R2G);
     w.magic_ychan = magic_of(w.groups);
@@ -660,7 +708,7 @@ int plan_wg(const ConvTileDesc &d, const void *X, const void *dY, int max_wg, bo
     w.magic_cols = magic_of(w.cols_kept);
     w.X = X;
     w.dY = dY;
-    w.batch = d.batch; w.Cin = d.Cin; w.Cout = d.Cout; w.Hin = d.Hin; w.Win = d.Win; w.Ho = d.Ho;
+    w.batch = d.batch; w.Cin = d.Cin; w.Cout = d.Cout; w.Hin = d.Hin; w.Win = d.Win; w.Ho = d.Ho; w.Wo = d.Wo;
     w.padU = d.padU; w.padL = d.padL;
     w.ws = workspace((size_t)w.nwg * w.part_elems * sizeof(float));
     return w.ws ? 0 : 2;
@@ -694,6 +742,7 @@ int conv_small_wg(const ConvTileDesc &d, const void *X, const void *dY, void *dW
             return 2;
         attr_set = true;
     }
+    state().last_conv_resident = 2;
     hipLaunchKernelGGL(wg_small_kernel<T>, dim3(w.nwg), dim3(CS_NT), WG_SMALL_LDS, state().stream, w);
     if (!hip_ok(hipGetLastError(), "small weight gradient launch")) return 2;
     return reduce_wg<T>(w, dW);

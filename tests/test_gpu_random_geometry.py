@@ -150,6 +150,55 @@ def test_conv2d_small_layer_weight_gradient_random_geometries(pkg, gpu, dt, seed
         assert rel(dw2, ref_dw) <= tol, (case, "dw, one call")
 
 
+@pytest.mark.parametrize("dt,seed", [("fp16", 51), ("fp16", 52), ("fp32", 53)])
+def test_conv2d_small_layer_stride2_gradients_random_geometries(pkg, gpu, dt, seed):
+    """3x3 layers at stride 2 with one column of left padding and an even input width (what the small-layer
+    weight-gradient kernel takes at that stride, forced with path 6): weight gradient alone and both gradients in
+    one call, against torch in float64; the ResNet-20 shapes among them."""
+    rng = random.Random(seed)
+    tdt, tol, vec = (torch.float16, 2e-3, 8) if dt == "fp16" else (torch.float32, 2e-5, 4)
+    fixed = [(16, 32, 32, 32, 1, 0, 128), (32, 64, 16, 16, 1, 0, 128)]
+    for it in range(12):
+        if it < len(fixed) and dt == "fp16":
+            Ci, Co, H, W, pu, pd, ns = fixed[it]
+        else:
+            Ci, Co = rng.choice([3, 8, 16, 24, 32, 64]), rng.choice([8, 16, 32, 40, 64])
+            W = rng.choice([16, 32, 48] if dt == "fp16" else [8, 16, 24, 32])
+            pu = rng.randint(0, 2)
+            H = rng.randint(4, 33)
+            pd = rng.randint(0, 2)
+            if (H + pu + pd - 3) % 2:
+                H += 1
+            ns = rng.choice([1, 2, 5, 9, 32, 130])
+        pl, pr = 1, 0  # (W + 1 + pr - 3) / 2 + 1 = W / 2 output columns with pr = 0 ... (W + pl + pr - 3) must be even
+        if (W + pl + pr - 3) % 2:
+            pr = 1
+        Ho, Wo = (H + pu + pd - 3) // 2 + 1, (W + pl + pr - 3) // 2 + 1
+        x = (torch.rand(ns, Ci, H, W, device="cuda") - 0.5).to(tdt)
+        w = ((torch.rand(Co, Ci, 3, 3, device="cuda") - 0.5) * 0.5).to(tdt)
+        dy = (torch.rand(ns, Co, Ho, Wo, device="cuda") - 0.5).to(tdt)
+        y, dx, dw = torch.full_like(dy, 3), torch.full_like(x, 3), torch.full_like(w, 3)
+        dx2, dw2 = torch.full_like(x, 3), torch.full_like(w, 3)
+        a, keep = hp.conv2d_args(pkg, x, dx, w, dw, y, dy, Ci, H, W, Co, 3, 3, Ho, Wo, (pl, pr, pu, pd), (2, 2))
+        a2, keep2 = hp.conv2d_args(pkg, x, dx2, w, dw2, y, dy, Ci, H, W, Co, 3, 3, Ho, Wo, (pl, pr, pu, pd), (2, 2))
+        case = (Ci, Co, H, W, (pl, pr, pu, pd), ns)
+        gpu.ptl_set_gemm_path(6)
+        try:
+            pkg.call("ptl_conv2d_%s_wg_batched" % dt, a, ns)
+            if it < len(fixed) and dt == "fp16":
+                assert gpu.ptl_last_conv_resident() == 2, case
+            pkg.call("ptl_conv2d_%s_bw_batched" % dt, a2, ns)
+        finally:
+            gpu.ptl_set_gemm_path(0)
+        gpu.ptl_sync()
+        xp = F.pad(x.double(), (pl, pr, pu, pd))
+        ref_dx = torch.nn.grad.conv2d_input(xp.shape, w.double(), dy.double(), stride=2)[:, :, pu:pu + H, pl:pl + W]
+        ref_dw = torch.nn.grad.conv2d_weight(xp, w.shape, dy.double(), stride=2)
+        assert rel(dw, ref_dw) <= tol, (case, "dw")
+        assert rel(dx2, ref_dx) <= tol, (case, "dx, one call")
+        assert rel(dw2, ref_dw) <= tol, (case, "dw, one call")
+
+
 @pytest.mark.parametrize("seed", [21, 22])
 def test_depthwise_random_geometries(pkg, gpu, seed):
     rng = random.Random(seed)
