@@ -38,6 +38,7 @@ struct ConvSmallArgs {
     unsigned magic_halo_w, magic_rr;
     int f_chunks, f_inner;  // 16-byte pieces of the filter tensor [outer][inner][9]; inner dimension
     int f_transposed;       // 0: outer = filter, inner = channel; 1: outer = channel, inner = filter, taps flipped
+    int K;                  // filter extent both ways: 3, or 1 (one tap, kept in the first tap's place of a filter row)
     unsigned magic_inner9, magic_wo;
     int b_pitch, f_bytes;   // bytes per filter row in LDS, bytes of the filter tile
     int pgroups, mshift;    // jobs = groups of 32 pixels x (1 << mshift) blocks of 32 filters
@@ -120,7 +121,25 @@ __device__ inline void conv_small_block(const ConvSmallArgs &a, int tile, char *
     }
     // ---- filter pieces -> [filter][tap][channel]: element (outer, inner, tap) of the dense tensor goes to
     // (filter, channel) = (outer, inner), or (inner, outer) with the taps flipped; the address moves with the indices
-    {
+    if (a.K == 1) {  // [outer][inner]: element (outer, inner) goes to (filter, channel) or (channel, filter), tap place 0
+#pragma unroll
+        for (int k = 0; k < F_MAX; ++k) {
+            const int q = tid + CS_NT * k;
+            if (q < a.f_chunks) {
+                const int e0 = q * VEC;
+                int outer = fast_div(e0, a.magic_inner9), inner = e0 - outer * a.f_inner;
+#pragma unroll
+                for (int j = 0; j < VEC; ++j) {
+                    const int m = a.f_transposed ? inner : outer, c = a.f_transposed ? outer : inner;
+                    *reinterpret_cast<T *>(F + m * a.b_pitch + c * ES) = fin[k].e[j];
+                    if (++inner == a.f_inner) {
+                        inner = 0;
+                        ++outer;
+                    }
+                }
+            }
+        }
+    } else {
         const int step_tap = a.f_transposed ? -CINP * ES : CINP * ES;
         const int step_inner = (a.f_transposed ? a.b_pitch : ES) - 9 * step_tap;  // after the ninth tap step: tap 0, inner + 1
         const int step_outer = (a.f_transposed ? ES : a.b_pitch) - a.f_inner * (a.f_transposed ? a.b_pitch : ES);
@@ -167,6 +186,11 @@ __device__ inline void conv_small_block(const ConvSmallArgs &a, int tile, char *
         f32x16 acc;
 #pragma unroll
         for (int v = 0; v < 16; ++v) acc[v] = 0.f;
+        if (a.K == 1) {
+#pragma unroll
+            for (int ks = 0; ks < CINP / KSTEP; ++ks)
+                mfma_step<T>(acc, *reinterpret_cast<const uint4 *>(frow + ks * KSTEP * ES), prow[2 * ks * a.POS]);
+        } else
 #pragma unroll
         for (int ks = 0; ks < CINP / KSTEP; ++ks) {
             const uint4 *pk = prow + 2 * ks * a.POS;
@@ -211,7 +235,7 @@ struct WgSmallArgs {
     const void *X, *dY;
     float *ws;
     int batch, Cin, Cout, Hin, Win, Ho, Wo, padU, padL;
-    int stride, rows_in;           // 1 or 2 (both ways); input rows a tile of R output rows meets: (R - 1) * stride + 3
+    int stride, rows_in;           // 1 or 2 (both ways); input rows a tile of R output rows meets: (R - 1) * stride + filter rows
     int nwg, S, R, tiles_per_img;  // workgroups; samples and output rows per tile (R = Ho when S > 1)
     int G, RG, Gin, R2G;           // 16-byte column groups per gradient row, per R of them; per input row, per rows_in of them
     int PY, PX, WP;                // LDS pitches in elements: gradient channel, input channel, input row
@@ -219,7 +243,8 @@ struct WgSmallArgs {
     int y_chunks, x_chunks, pad_chunks, pad_rows;  // pieces to copy; zero pieces (one per input row + one) and rows per channel
     unsigned magic_g, magic_gin, magic_rg, magic_r2g, magic_ychan, magic_xchan, magic_padrows, magic_tile, magic_cols;
     int cbi_n, combos, kparts;  // 32-channel blocks, (filter block, channel block) pairs, position shares
-    int total;                  // Cout * Cin * 9
+    int total;                  // Cout * Cin * taps
+    int taps;                   // 9, or 1 for a 1x1 filter
     int rows_kept, cols_kept, part_elems;  // filter rows and channels of a 32x32 tile that are stored; floats per workgroup in ws
 };
 
@@ -263,7 +288,8 @@ __device__ inline uint4 shifted_piece(const uint4 &c, unsigned p3, unsigned n0) 
 // zero piece of its own - the eight input columns 2 x + kx - 1 that meet eight consecutive gradient columns x are
 // then eight consecutive elements again: of the odd half one to the left (kx = 0), of the even half (1), of the odd
 // half (2) - and gradient row y meets input rows 2 y + ky.
-template <typename T, int PADL, int STRIDE>
+// K1: a 1x1 filter - one tap, no padding: every wave takes a share of the positions (no filter rows to split over).
+template <typename T, int PADL, int STRIDE, bool K1 = false>
 __device__ inline void wg_small_block(const WgSmallArgs &a, int wg, char *smem) {
     constexpr int VEC = 16 / (int)sizeof(T);
     typedef typename EdgePair<T>::type edge_t;
@@ -338,9 +364,9 @@ __device__ inline void wg_small_block(const WgSmallArgs &a, int wg, char *smem) 
     __syncthreads();
 
     // ---- products
-    const int ky = wave % 3, rest = wave / 3;
+    const int ky = K1 ? 0 : wave % 3, rest = K1 ? wave : wave / 3;
     const int combo = rest % a.combos, kpart = rest / a.combos;
-    const bool active = wave < 15 && kpart < a.kparts;
+    const bool active = (K1 || wave < 15) && kpart < a.kparts;
     const int cbo = combo / a.cbi_n, cbi = combo - cbo * a.cbi_n;
     const int lr = lane & 31, kg = lane >> 5;
     const int nks = (a.groups + 1) >> 1;
@@ -380,7 +406,9 @@ __device__ inline void wg_small_block(const WgSmallArgs &a, int wg, char *smem) 
             }
 #pragma unroll
             for (int u = 0; u < U; ++u) {
-                if constexpr (STRIDE == 1) {
+                if constexpr (K1) {  // (the even half at stride 2: columns 2 x)
+                    mfma_step<T>(acc[0], A[u], C[u]);
+                } else if constexpr (STRIDE == 1) {
                     mfma_step<T>(acc[0], A[u], shifted_piece<0 - PADL>(C[u], p3[u], n0[u]));
                     mfma_step<T>(acc[1], A[u], shifted_piece<1 - PADL>(C[u], p3[u], n0[u]));
                     mfma_step<T>(acc[2], A[u], shifted_piece<2 - PADL>(C[u], p3[u], n0[u]));
@@ -397,8 +425,8 @@ __device__ inline void wg_small_block(const WgSmallArgs &a, int wg, char *smem) 
     float *L = reinterpret_cast<float *>(smem);
     if (active) {
 #pragma unroll
-        for (int kx = 0; kx < 3; ++kx) {
-            float *t = L + ((kpart * a.combos + combo) * 9 + ky * 3 + kx) * 1024 + lr;
+        for (int kx = 0; kx < (K1 ? 1 : 3); ++kx) {
+            float *t = L + ((kpart * a.combos + combo) * a.taps + ky * 3 + kx) * 1024 + lr;
 #pragma unroll
             for (int v = 0; v < 16; ++v) t[(8 * (v >> 2) + 4 * kg + (v & 3)) * 32] = acc[kx][v];
         }
@@ -409,9 +437,9 @@ __device__ inline void wg_small_block(const WgSmallArgs &a, int wg, char *smem) 
     // would cost more than the sums, sixteen waves share the integer pipes); the second launch puts the sums where
     // the weight tensor wants them
     float *out = a.ws + (size_t)wg * a.part_elems;
-    const int share = a.combos * 9 * 1024, tile_elems = a.rows_kept * a.cols_kept;
+    const int share = a.combos * a.taps * 1024, tile_elems = a.rows_kept * a.cols_kept;
     if (tile_elems == 1024) {  // whole tiles: thread t owns element t of every tile
-        for (int t = 0; t < a.combos * 9; ++t) {
+        for (int t = 0; t < a.combos * a.taps; ++t) {
             const float *src = L + t * 1024 + tid;
             float sum = src[0];
             for (int kp = 1; kp < a.kparts; ++kp) sum += src[kp * share];
@@ -431,7 +459,11 @@ __device__ inline void wg_small_block(const WgSmallArgs &a, int wg, char *smem) 
 
 template <typename T>
 __device__ inline void wg_small_any(const WgSmallArgs &a, int wg, char *smem) {
-    if (a.stride == 2)
+    if (a.taps == 1 && a.stride == 2)
+        wg_small_block<T, 0, 2, true>(a, wg, smem);
+    else if (a.taps == 1)
+        wg_small_block<T, 0, 1, true>(a, wg, smem);
+    else if (a.stride == 2)
         wg_small_block<T, 1, 2>(a, wg, smem);
     else if (a.padL == 1)
         wg_small_block<T, 1, 1>(a, wg, smem);
@@ -494,7 +526,7 @@ int launch_small(const ConvSmallArgs &a, int tiles, size_t lds, hipStream_t s, c
 template <typename T>
 __global__ __launch_bounds__(1024) void wg_small_reduce_kernel(const float *__restrict__ ws, T *__restrict__ dW,
                                                                int part_elems, int parts, int rows_kept,
-                                                               int cols_kept, int cbi_n, int Cout, int Cin) {
+                                                               int cols_kept, int cbi_n, int Cout, int Cin, int taps) {
     __shared__ float part_sum[16][64];
     const int o = threadIdx.x & 63, pg = threadIdx.x >> 6;
     const int i = blockIdx.x * 64 + o;
@@ -521,9 +553,9 @@ __global__ __launch_bounds__(1024) void wg_small_reduce_kernel(const float *__re
 #pragma unroll
         for (int q = 1; q < 16; ++q) s += part_sum[q][o];
         const int tile = i / (rows_kept * cols_kept), r = i - tile * rows_kept * cols_kept;
-        const int combo = tile / 9, tap = tile - combo * 9;
+        const int combo = tile / taps, tap = tile - combo * taps;
         const int co = (combo / cbi_n) * 32 + r / cols_kept, ci = (combo % cbi_n) * 32 + r % cols_kept;
-        if (co < Cout && ci < Cin) dW[(co * Cin + ci) * 9 + tap] = (T)s;
+        if (co < Cout && ci < Cin) dW[(co * Cin + ci) * taps + tap] = (T)s;
     }
 }
 
@@ -539,20 +571,21 @@ int plan_small(const ConvTileDesc &d, const void *X, const void *Wt, void *Y, in
     constexpr int ES = (int)sizeof(T), VEC = 16 / ES, RPI = 64 / VEC;  // element size, elements per piece, rows per item
     State &st = state();
     if (st.gemm_path != 0 && st.gemm_path != 6) return -1;  // (the other values select one of the other routes)
-    if (d.in_hwc || d.KH != 3 || d.KW != 3 || d.sh != d.sw || d.sh < 1 || d.sh > 2) return -1;
+    const int K = d.KH;  // 3x3, or a single tap
+    if (d.in_hwc || d.KH != d.KW || (K != 3 && K != 1) || d.sh != d.sw || d.sh < 1 || d.sh > 2) return -1;
     if (d.Cin > 64 || d.Cout > 64 || d.Win % VEC != 0 || d.x_sy != d.Win) return -1;
     if (d.x_sc != (long long)d.Hin * d.Win || d.x_sb != (long long)d.Cin * d.Hin * d.Win) return -1;
     if (d.padU < 0 || d.padU > 2 || d.padL < 0 || d.padL > 2 || d.padD < 0 || d.padR < 0 || d.padR > 8) return -1;
     if (reinterpret_cast<uintptr_t>(X) % 16 || reinterpret_cast<uintptr_t>(Wt) % 16) return -1;
-    const long long f_elems = (long long)d.Cout * d.Cin * 9;
+    const long long f_elems = (long long)d.Cout * d.Cin * K * K;
     if (f_elems % VEC != 0) return -1;
     ConvSmallArgs &a = p.a;
     a = ConvSmallArgs();
     // dense filter tensor [outer][inner][3][3]: forward (filter, channel), or the input gradient's view of it
-    if (d.w_base == 0 && d.w_sm == d.Cin * 9 && d.w_sc == 9 && d.w_sy == 3 && d.w_sx == 1) {
+    if (d.w_base == 0 && d.w_sm == d.Cin * K * K && d.w_sc == K * K && d.w_sy == K && d.w_sx == 1) {
         a.f_transposed = 0;
         a.f_inner = d.Cin;
-    } else if (d.w_base == 8 && d.w_sm == 9 && d.w_sc == d.Cout * 9 && d.w_sy == -3 && d.w_sx == -1) {
+    } else if (d.w_base == K * K - 1 && d.w_sm == K * K && d.w_sc == d.Cout * K * K && d.w_sy == -K && d.w_sx == -1) {
         a.f_transposed = 1;
         a.f_inner = d.Cout;
     } else {
@@ -562,16 +595,16 @@ int plan_small(const ConvTileDesc &d, const void *X, const void *Wt, void *Y, in
     if (d.in_dil > 2 || (dil == 2 && d.sh != 1)) return -1;
     const int Hd = (d.Hin - 1) * dil + 1, Wd = (d.Win - 1) * dil + 1;  // the image the taps walk over
     const int s = d.sh, TW = Wd + d.padL + d.padR, THP = Hd + d.padU + d.padD;
-    if ((d.Wo - 1) * s + 3 > TW || (d.Ho - 1) * s + 3 > THP || d.Wo >= 65536 || d.Ho * d.Wo >= 65536) return -1;
+    if ((d.Wo - 1) * s + K > TW || (d.Ho - 1) * s + K > THP || d.Wo >= 65536 || d.Ho * d.Wo >= 65536) return -1;
     const int cinp = d.Cin <= 16 ? 16 : d.Cin <= 32 ? 32 : 64, cblocks = cinp / VEC;
     const int mblocks = (d.Cout + 31) / 32;
     // rows per workgroup: the whole image, halved while that leaves the four waves a job each and the chip is not full
     int R = d.Ho;
     auto jobs_of = [&](int r) { return ((r * d.Wo + 31) / 32) * mblocks; };
     while ((long long)d.batch * ((d.Ho + R - 1) / R) < cu_budget && R % 2 == 0 && jobs_of(R / 2) >= 4) R /= 2;
-    auto items_of = [&](int r) { return cblocks * (d.Win / VEC) * ((((r - 1) * s + 3) + RPI - 1) / RPI); };
-    auto lds_of = [&](int r) { return (size_t)cblocks * ((r - 1) * s + 3) * TW * 16; };
-    const int pitch = 9 * cinp * ES + 16;  // (an odd multiple of 16 bytes)
+    auto items_of = [&](int r) { return cblocks * (d.Win / VEC) * ((((r - 1) * s + K) + RPI - 1) / RPI); };
+    auto lds_of = [&](int r) { return (size_t)cblocks * ((r - 1) * s + K) * TW * 16; };
+    const int pitch = K * K * cinp * ES + 16;  // (an odd multiple of 16 bytes)
     const size_t f_bytes = (size_t)mblocks * 32 * pitch;
     while (R > 1 && (items_of(R) > CS_ITEMS || f_bytes + lds_of(R) > 150 * 1024)) R = (R + 1) / 2;
     if (items_of(R) > CS_ITEMS || f_bytes + lds_of(R) > 150 * 1024) return -1;
@@ -588,7 +621,8 @@ int plan_small(const ConvTileDesc &d, const void *X, const void *Wt, void *Y, in
     a.s = s; a.padU = d.padU; a.padL = d.padL;
     a.dil = dil;
     a.R = R; a.tiles_per_img = (d.Ho + R - 1) / R;
-    a.RR = (R - 1) * s + 3; a.TW = TW; a.POS = a.RR * TW;
+    a.RR = (R - 1) * s + K; a.TW = TW; a.POS = a.RR * TW;
+    a.K = K;
     const int G = d.Win / VEC, RRB = (a.RR + RPI - 1) / RPI;
     a.items = cblocks * G * RRB;
     for (int item = 0; item < a.items; ++item) {
@@ -603,7 +637,7 @@ int plan_small(const ConvTileDesc &d, const void *X, const void *Wt, void *Y, in
     a.magic_halo_w = magic_of(a.halo_w);
     a.magic_rr = magic_of(a.RR);
     a.f_chunks = (int)(f_elems / VEC);
-    a.magic_inner9 = magic_of(a.f_inner * 9);
+    a.magic_inner9 = magic_of(a.f_inner * K * K);
     a.magic_wo = magic_of(d.Wo);
     a.b_pitch = pitch; a.f_bytes = (int)f_bytes;
     a.pgroups = (R * d.Wo + 31) / 32; a.mshift = mblocks - 1;
@@ -633,7 +667,8 @@ int plan_wg(const ConvTileDesc &d, const void *X, const void *dY, int max_wg, bo
     constexpr int ES = (int)sizeof(T), VEC = 16 / ES;
     State &st = state();
     if (st.gemm_path != 0 && st.gemm_path != 6) return -1;  // (the other values select one of the other routes)
-    if (d.in_hwc || d.KH != 3 || d.KW != 3 || d.sh != d.sw || d.sh < 1 || d.sh > 2) return -1;
+    const int K = d.KH;  // 3x3, or a single tap
+    if (d.in_hwc || d.KH != d.KW || (K != 3 && K != 1) || d.sh != d.sw || d.sh < 1 || d.sh > 2) return -1;
     const int st2 = d.sh == 2;
     if (d.Cin > 64 || d.Cout > 64 || d.Win % VEC != 0 || d.Wo % VEC != 0 || d.x_sy != d.Win) return -1;
     if (d.x_sc != (long long)d.Hin * d.Win || d.x_sb != (long long)d.Cin * d.Hin * d.Win) return -1;
@@ -641,10 +676,12 @@ int plan_wg(const ConvTileDesc &d, const void *X, const void *dY, int max_wg, bo
     // unit stride: a gradient row as long as an input row; stride 2: half as long, one column of left padding, and
     // the input columns the last gradient column meets inside the row
     if (!st2 && d.Wo != d.Win) return -1;
-    if (st2 && (d.padL != 1 || d.Win % (2 * VEC) != 0 || d.Wo * 2 != d.Win)) return -1;
+    if (st2 && (d.padL != (K == 3 ? 1 : 0) || d.Win % (2 * VEC) != 0 || d.Wo * 2 != d.Win)) return -1;
+    if (K == 1 && d.padL != 0) return -1;
     if (reinterpret_cast<uintptr_t>(X) % 16 || reinterpret_cast<uintptr_t>(dY) % 16) return -1;
     w = WgSmallArgs();
-    w.total = d.Cout * d.Cin * 9;
+    w.taps = K * K;
+    w.total = d.Cout * d.Cin * w.taps;
     if (w.total >= 65536) return -1;
     const long long positions = (long long)d.batch * d.Ho * d.Wo;
     // large calls keep the tiled weight-gradient kernels, and so do small calls for the weight gradient alone (measured
@@ -656,7 +693,7 @@ int plan_wg(const ConvTileDesc &d, const void *X, const void *dY, int max_wg, bo
     w.Gin = d.Win / VEC;
     w.stride = d.sh;
     w.WP = d.Win + (st2 ? 2 : 1) * VEC;
-    auto rows_in = [&](int R) { return (R - 1) * d.sh + 3; };
+    auto rows_in = [&](int R) { return (R - 1) * d.sh + K; };
     // pitches of 16 bytes mod 128: consecutive channels 16 bytes apart in the banks
     auto round_pitch = [](int n) { return n + ((VEC - n % (8 * VEC)) + 8 * VEC) % (8 * VEC); };
     auto lds_of = [&](int S, int R) {
@@ -670,7 +707,7 @@ int plan_wg(const ConvTileDesc &d, const void *X, const void *dY, int max_wg, bo
     // tiles: whole samples while the partial sums stay within about 5 MB (S samples each otherwise), rows of a
     // sample split while that fills more of `max_wg` workgroups and leaves the waves eight k steps each
     int S = 1, R = d.Ho;
-    const long long part_bytes = (long long)((d.Cin + 31) / 32) * ((d.Cout + 31) / 32) * 9 * (d.Cout < 32 ? d.Cout : 32) * (d.Cin < 32 ? d.Cin : 32) * 4;
+    const long long part_bytes = (long long)((d.Cin + 31) / 32) * ((d.Cout + 31) / 32) * w.taps * (d.Cout < 32 ? d.Cout : 32) * (d.Cin < 32 ? d.Cin : 32) * 4;
     while ((long long)((d.batch + S - 1) / S) * part_bytes > (5LL << 20) && chunks_ok(S * 2, R)) S *= 2;
     if (S == 1)
         while (R % 2 == 0 && (long long)d.batch * (d.Ho / R) * 2 <= max_wg && (R / 2) * w.G >= 16 &&
@@ -700,10 +737,10 @@ int plan_wg(const ConvTileDesc &d, const void *X, const void *dY, int max_wg, bo
     w.magic_padrows = magic_of(w.pad_rows);
     w.cbi_n = (d.Cin + 31) / 32;
     w.combos = w.cbi_n * ((d.Cout + 31) / 32);
-    w.kparts = 4 / w.combos;
+    w.kparts = (K == 1 ? 16 : 4) / w.combos;
     w.rows_kept = d.Cout < 32 ? d.Cout : 32;
     w.cols_kept = d.Cin < 32 ? d.Cin : 32;
-    w.part_elems = w.combos * 9 * w.rows_kept * w.cols_kept;
+    w.part_elems = w.combos * w.taps * w.rows_kept * w.cols_kept;
     w.magic_tile = magic_of(w.rows_kept * w.cols_kept);
     w.magic_cols = magic_of(w.cols_kept);
     w.X = X;
@@ -717,7 +754,7 @@ int plan_wg(const ConvTileDesc &d, const void *X, const void *dY, int max_wg, bo
 template <typename T>
 int reduce_wg(const WgSmallArgs &w, void *dW) {
     hipLaunchKernelGGL(wg_small_reduce_kernel<T>, dim3((w.part_elems + 63) / 64), dim3(1024), 0, state().stream, w.ws,
-                       reinterpret_cast<T *>(dW), w.part_elems, w.nwg, w.rows_kept, w.cols_kept, w.cbi_n, w.Cout, w.Cin);
+                       reinterpret_cast<T *>(dW), w.part_elems, w.nwg, w.rows_kept, w.cols_kept, w.cbi_n, w.Cout, w.Cin, w.taps);
     return hip_ok(hipGetLastError(), "small weight gradient reduction launch") ? 0 : 2;
 }
 

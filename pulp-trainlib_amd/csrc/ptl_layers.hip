@@ -477,14 +477,14 @@ static int conv2d_ig(const Args *a, int ns, const char *fn) {
         return sg.finish(gemm<T>(q));
     }
 
-    // Small fp16 stride-2 layers: the small-layer kernel stuffs the zeros while it fills its LDS tile.
-    if (!g.hwc && g.sh == 2 && g.sw == 2 && g.Hk == 3 && g.Wk == 3) {
+    // Small stride-2 layers (3x3 or 1x1): the small-layer kernel stuffs the zeros while it fills its LDS tile.
+    if (!g.hwc && g.sh == 2 && g.sw == 2 && g.Hk == g.Wk && (g.Hk == 3 || g.Hk == 1)) {
         ConvTileDesc d = {};
         d.batch = ns; d.Cin = g.Co; d.Hin = g.Ho; d.Win = g.Wo; d.in_dil = 2;
         d.Cout = g.Ci; d.Ho = g.H; d.Wo = g.W;
-        d.KH = 3; d.KW = 3; d.sh = 1; d.sw = 1;
-        d.padU = 2 - g.Up; d.padL = 2 - g.Lp;
-        d.padD = g.H + 2 - Hd - d.padU; d.padR = g.W + 2 - Wd - d.padL;
+        d.KH = g.Hk; d.KW = g.Wk; d.sh = 1; d.sw = 1;
+        d.padU = g.Hk - 1 - g.Up; d.padL = g.Wk - 1 - g.Lp;
+        d.padD = g.H + g.Hk - 1 - Hd - d.padU; d.padR = g.W + g.Wk - 1 - Wd - d.padL;
         d.x_sb = (long long)g.Co * P; d.x_sc = P; d.x_sy = g.Wo;
         d.w_base = Pk - 1; d.w_sm = Pk; d.w_sc = g.Ci * Pk; d.w_sy = -g.Wk; d.w_sx = -1;
         state().last_conv_direct = 0;
@@ -643,29 +643,29 @@ static int conv2d_bw(const Args *a, int ns, const char *fn) {
         if (int rc = conv_geom(a, g, fn, true)) return rc;
         const int P = g.Ho * g.Wo, Pk = g.Hk * g.Wk, K = g.Ci * Pk;
         size_t in_n = (size_t)ns * g.Ci * g.H * g.W, out_n = (size_t)ns * g.Co * P;
-        const bool unit = g.sh == 1 && g.sw == 1 && g.Up + g.Dp == 2 && g.Lp + g.Rp == 2;
+        const bool unit = g.sh == 1 && g.sw == 1 && g.Up + g.Dp == g.Hk - 1 && g.Lp + g.Rp == g.Wk - 1;
         const bool halving = g.sh == 2 && g.sw == 2;  // (small layers only: the zeros are stuffed on the way into LDS)
-        if (!g.hwc && g.Hk == 3 && g.Wk == 3 && (unit || halving) && fits_int(in_n) && fits_int(out_n) &&
+        if (!g.hwc && g.Hk == g.Wk && (g.Hk == 3 || g.Hk == 1) && (unit || halving) && fits_int(in_n) && fits_int(out_n) &&
             (state().gemm_path == 0 || state().gemm_path == 5 || state().gemm_path == 6)) {
             if (!ensure_init()) return 2;
             ConvTileDesc f = {}, b = {};
             f.batch = ns; f.Cin = g.Ci; f.Hin = g.H; f.Win = g.W;
             f.Cout = g.Co; f.Ho = g.Ho; f.Wo = g.Wo;
-            f.KH = 3; f.KW = 3; f.sh = g.sh; f.sw = g.sw;
+            f.KH = g.Hk; f.KW = g.Wk; f.sh = g.sh; f.sw = g.sw;
             f.padU = g.Up; f.padD = g.Dp; f.padL = g.Lp; f.padR = g.Rp;
             f.x_sb = (long long)g.Ci * g.H * g.W; f.x_sc = (long long)g.H * g.W; f.x_sy = g.W;
             // the input gradient: a unit-stride pass over the output gradient, zero-stuffed where the forward strode
             const int Hd = (g.Ho - 1) * g.sh + 1, Wd = (g.Wo - 1) * g.sw + 1;
             b.batch = ns; b.Cin = g.Co; b.Hin = g.Ho; b.Win = g.Wo; b.in_dil = halving ? 2 : 0;
             b.Cout = g.Ci; b.Ho = g.H; b.Wo = g.W;
-            b.KH = 3; b.KW = 3; b.sh = 1; b.sw = 1;
-            b.padU = 2 - g.Up; b.padL = 2 - g.Lp;
-            b.padD = g.H + 2 - Hd - b.padU; b.padR = g.W + 2 - Wd - b.padL;
+            b.KH = g.Hk; b.KW = g.Wk; b.sh = 1; b.sw = 1;
+            b.padU = g.Hk - 1 - g.Up; b.padL = g.Wk - 1 - g.Lp;
+            b.padD = g.H + g.Hk - 1 - Hd - b.padU; b.padR = g.W + g.Wk - 1 - Wd - b.padL;
             b.x_sb = (long long)g.Co * P; b.x_sc = P; b.x_sy = g.Wo;
             b.w_base = Pk - 1; b.w_sm = Pk; b.w_sc = g.Ci * Pk; b.w_sy = -g.Wk; b.w_sx = -1;
             // small layers: both products in one launch; wide layers: one shared copy of the output gradient
             const bool small = g.Ci <= 64 && g.Co <= 64 && g.W % (16 / (int)sizeof(T)) == 0 && state().gemm_path != 5;
-            const bool wide = unit && sizeof(T) == 2 && ns > 1 && state().gemm_path != 6 && conv_halo_wg_preferred(f);
+            const bool wide = unit && g.Hk == 3 && sizeof(T) == 2 && ns > 1 && state().gemm_path != 6 && conv_halo_wg_preferred(f);
             if (small || wide) {
                 Stager sg;
                 const T *X = sg.in(reinterpret_cast<const T *>(a->input->data), in_n);

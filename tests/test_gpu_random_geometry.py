@@ -199,6 +199,53 @@ def test_conv2d_small_layer_stride2_gradients_random_geometries(pkg, gpu, dt, se
         assert rel(dw2, ref_dw) <= tol, (case, "dw, one call")
 
 
+@pytest.mark.parametrize("dt,seed", [("fp16", 61), ("fp32", 62)])
+def test_conv2d_small_layer_1x1_random_geometries(pkg, gpu, dt, seed):
+    """1x1 layers without padding at stride 1 and 2 (the projection shortcuts of a ResNet: the small-layer kernels
+    take them as a single tap, forced with path 6): forward, both gradients alone and in one call, against torch in
+    float64."""
+    rng = random.Random(seed)
+    tdt, tol, vec = (torch.float16, 2e-3, 8) if dt == "fp16" else (torch.float32, 2e-5, 4)
+    fixed = [(16, 32, 32, 2, 128), (32, 64, 16, 2, 128)]
+    for it in range(12):
+        if it < len(fixed):
+            Ci, Co, H, st, ns = fixed[it]
+            W = H
+        else:
+            Ci, Co = rng.choice([8, 16, 24, 32, 64]), rng.choice([8, 16, 32, 40, 64])
+            st = rng.choice([1, 2])
+            W = rng.choice([16, 32, 48] if dt == "fp16" else [8, 16, 24, 32])
+            H = rng.randint(2, 33)
+            ns = rng.choice([1, 2, 5, 9, 32, 130])
+        Ho, Wo = (H - 1) // st + 1, (W - 1) // st + 1
+        x = (torch.rand(ns, Ci, H, W, device="cuda") - 0.5).to(tdt)
+        w = ((torch.rand(Co, Ci, 1, 1, device="cuda") - 0.5) * 0.5).to(tdt)
+        dy = (torch.rand(ns, Co, Ho, Wo, device="cuda") - 0.5).to(tdt)
+        y, dx, dw = torch.full_like(dy, 3), torch.full_like(x, 3), torch.full_like(w, 3)
+        dx2, dw2 = torch.full_like(x, 3), torch.full_like(w, 3)
+        # (a stride that does not divide the extent: the reference's naive-kernel route, USE_IM2COL = 0, takes it)
+        a, keep = hp.conv2d_args(pkg, x, dx, w, dw, y, dy, Ci, H, W, Co, 1, 1, Ho, Wo, (0, 0, 0, 0), (st, st), 0, 1 if st == 1 else 0)
+        a2, keep2 = hp.conv2d_args(pkg, x, dx2, w, dw2, y, dy, Ci, H, W, Co, 1, 1, Ho, Wo, (0, 0, 0, 0), (st, st), 0, 1 if st == 1 else 0)
+        case = (Ci, Co, H, W, st, ns)
+        gpu.ptl_set_gemm_path(6)
+        try:
+            for step, args in (("fw", a), ("wg", a), ("ig", a), ("bw", a2)):
+                pkg.call("ptl_conv2d_%s_%s_batched" % (dt, step), args, ns)
+                if it < len(fixed):
+                    assert gpu.ptl_last_conv_resident() == 2, (case, step)
+        finally:
+            gpu.ptl_set_gemm_path(0)
+        gpu.ptl_sync()
+        ref_y = F.conv2d(x.double(), w.double(), stride=st)
+        ref_dx = torch.nn.grad.conv2d_input(x.shape, w.double(), dy.double(), stride=st)
+        ref_dw = torch.nn.grad.conv2d_weight(x.double(), w.shape, dy.double(), stride=st)
+        assert rel(y, ref_y) <= tol, (case, "y")
+        assert rel(dw, ref_dw) <= tol, (case, "dw")
+        assert rel(dx, ref_dx) <= tol, (case, "dx")
+        assert rel(dx2, ref_dx) <= tol, (case, "dx, one call")
+        assert rel(dw2, ref_dw) <= tol, (case, "dw, one call")
+
+
 @pytest.mark.parametrize("seed", [21, 22])
 def test_depthwise_random_geometries(pkg, gpu, seed):
     rng = random.Random(seed)
