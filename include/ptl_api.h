@@ -358,6 +358,15 @@ size_t ptl_conv2d_fp16_cache_bytes(const struct Conv2D_args_fp16 *a, int nsample
 int ptl_conv2d_fp16_fw_batched_cached(const struct Conv2D_args_fp16 *a, int nsamples, struct ptl_conv_cache *c);
 int ptl_conv2d_fp16_wg_batched_cached(const struct Conv2D_args_fp16 *a, int nsamples, const struct ptl_conv_cache *c);
 int ptl_conv2d_fp16_bw_batched_cached(const struct Conv2D_args_fp16 *a, int nsamples, const struct ptl_conv_cache *c);
+/* No counterpart in the reference: ptl_conv2d_*_bw_batched with the last launch of a small layer's weight gradient
+ * (the addition of its partial sums) put off and done for all deferred layers at once by ptl_conv2d_*_wg_flush
+ * (struct ptl_wg_batch; a training step with twenty small layers saves twenty launches).  A layer that does not take
+ * the small-layer kernels, or finds the batch full, is completed by the call itself as usual.  The flush returns 0
+ * also for an empty batch. */
+int ptl_conv2d_fp16_bw_batched_deferred(const struct Conv2D_args_fp16 *a, int nsamples, struct ptl_wg_batch *batch);
+int ptl_conv2d_fp32_bw_batched_deferred(const struct Conv2D_args *a, int nsamples, struct ptl_wg_batch *batch);
+int ptl_conv2d_fp16_wg_flush(struct ptl_wg_batch *batch);
+int ptl_conv2d_fp32_wg_flush(struct ptl_wg_batch *batch);
 int ptl_batch_norm_fp32_fw(const struct BatchNorm_args_fp32 *a);
 /* No counterpart in the reference (its batch normalisation has a forward pass only, in fp32): the backward pass
  * of that forward and both passes in fp16, for a training step that contains the layer.  Backward reads

@@ -688,6 +688,24 @@ struct ptl_conv_cache {
     int geometry[6]; /* batch, channels, padded height and width, top and left padding */
 };
 
+/* No counterpart in the reference: the weight gradients of several small Conv2D layers completed by one launch.
+ * A backward call of such a layer is two launches, the second one only adds up the partial sums of the first;
+ * with a batch (ptl_conv2d_*_bw_batched_deferred) the partial sums stay in the caller's buffer and
+ * ptl_conv2d_*_wg_flush adds up those of all layers deferred since the last flush.  The caller sets buf and bytes
+ * (device memory, 16 MiB hold the layers of a ResNet-20 at batch 128) and zeroes used and count once; the library
+ * maintains the rest.  coeff->diff of a deferred layer is valid after the flush, not before. */
+#define PTL_WG_BATCH_MAX 32
+struct ptl_wg_batch {
+    void *buf;
+    size_t bytes;
+    size_t used;      /* bytes of buf in use */
+    int count;        /* layers waiting for the flush */
+    size_t offset[32]; /* per layer: where its partial sums start in buf */
+    void *grad[32];    /* per layer: its coeff->diff */
+    int shape[256];    /* per layer eight numbers: floats per part, parts, filter rows and channels kept of a 32 x 32
+                          tile, channel blocks, filters, channels, taps */
+};
+
 /* No counterpart in the reference: what a residual block puts behind a normalisation layer, for the fused calls
  * ptl_batch_norm_fused_*.  All tensors have the shape of the normalisation's output (B x C x H x W). */
 struct ptl_norm_fusion_fp32 {

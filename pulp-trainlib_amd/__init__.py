@@ -82,6 +82,10 @@ FUSED_NORM_ENTRY_POINTS = ["ptl_batch_norm_fused_%s_%s" % (dt, step) for dt in (
 # `int f(const Conv2D_args_fp16 *, int nsamples, [const] ptl_conv_cache *)` and the size query
 CACHED_ENTRY_POINTS = ["ptl_conv2d_fp16_%s_batched_cached" % s for s in ("fw", "wg", "bw")] + ["ptl_conv2d_fp16_cache_bytes"]
 
+# `int f(const Conv2D_args[_fp16] *, int nsamples, ptl_wg_batch *)` and `int f(ptl_wg_batch *)`
+DEFERRED_ENTRY_POINTS = ["ptl_conv2d_%s_bw_batched_deferred" % dt for dt in ("fp16", "fp32")] + \
+                        ["ptl_conv2d_%s_wg_flush" % dt for dt in ("fp16", "fp32")]
+
 OTHER_ENTRY_POINTS = ["ptl_init", "ptl_last_error", "ptl_last_status", "ptl_set_stream", "ptl_sync", "ptl_set_gemm_path",
                       "ptl_last_conv_direct", "ptl_last_gemm_streamed", "ptl_last_conv_resident", "ptl_timer_begin", "ptl_timer_end_ms", "ptl_mm_fp32", "ptl_mm_fp16", "ptl_copy_bytes"]
 
@@ -118,6 +122,14 @@ def load():
     for name in CACHED_ENTRY_POINTS[:3]:
         f = getattr(lib, name)
         f.argtypes = [ctypes.c_void_p, ctypes.c_int, ctypes.c_void_p]
+        f.restype = ctypes.c_int
+    for name in DEFERRED_ENTRY_POINTS[:2]:
+        f = getattr(lib, name)
+        f.argtypes = [ctypes.c_void_p, ctypes.c_int, ctypes.c_void_p]
+        f.restype = ctypes.c_int
+    for name in DEFERRED_ENTRY_POINTS[2:]:
+        f = getattr(lib, name)
+        f.argtypes = [ctypes.c_void_p]
         f.restype = ctypes.c_int
     lib.ptl_conv2d_fp16_cache_bytes.argtypes = [ctypes.c_void_p, ctypes.c_int]
     lib.ptl_conv2d_fp16_cache_bytes.restype = ctypes.c_size_t

@@ -17,6 +17,7 @@
 #include "ptl_gemm_async.hpp"
 #include "ptl_gemm_async.inc"
 #include "ptl_conv_tile.hpp"
+#include "ptl_structs.h"
 #include "ptl_host.hpp"
 
 namespace ptl {
@@ -524,12 +525,12 @@ int launch_small(const ConvSmallArgs &a, int tiles, size_t lds, hipStream_t s, c
 // elements per workgroup of the reduction (coalesced reads), 16 groups of partials in parallel, eight loads in flight
 // per thread; the few results are scattered to the weight tensor's order.
 template <typename T>
-__global__ __launch_bounds__(1024) void wg_small_reduce_kernel(const float *__restrict__ ws, T *__restrict__ dW,
-                                                               int part_elems, int parts, int rows_kept,
-                                                               int cols_kept, int cbi_n, int Cout, int Cin, int taps) {
+__device__ inline void wg_small_reduce_block(const float *__restrict__ ws, T *__restrict__ dW, int block, int part_elems,
+                                             int parts, int rows_kept, int cols_kept, int cbi_n, int Cout, int Cin,
+                                             int taps) {
     __shared__ float part_sum[16][64];
     const int o = threadIdx.x & 63, pg = threadIdx.x >> 6;
-    const int i = blockIdx.x * 64 + o;
+    const int i = block * 64 + o;
     float s = 0.f;
     if (i < part_elems) {
         const float *src = ws + i;
@@ -557,6 +558,32 @@ __global__ __launch_bounds__(1024) void wg_small_reduce_kernel(const float *__re
         const int co = (combo / cbi_n) * 32 + r / cols_kept, ci = (combo % cbi_n) * 32 + r % cols_kept;
         if (co < Cout && ci < Cin) dW[(co * Cin + ci) * taps + tap] = (T)s;
     }
+}
+
+template <typename T>
+__global__ __launch_bounds__(1024) void wg_small_reduce_kernel(const float *__restrict__ ws, T *__restrict__ dW,
+                                                               int part_elems, int parts, int rows_kept,
+                                                               int cols_kept, int cbi_n, int Cout, int Cin, int taps) {
+    wg_small_reduce_block<T>(ws, dW, blockIdx.x, part_elems, parts, rows_kept, cols_kept, cbi_n, Cout, Cin, taps);
+}
+
+// The same addition for the layers of a deferred batch in one launch: the blocks of all layers in one grid, a block
+// finds its layer by the running block count.
+struct WgFlushArgs {
+    int count;
+    int first_block[PTL_WG_BATCH_MAX + 1];
+    const float *ws[PTL_WG_BATCH_MAX];
+    void *grad[PTL_WG_BATCH_MAX];
+    int shape[PTL_WG_BATCH_MAX][8];
+};
+
+template <typename T>
+__global__ __launch_bounds__(1024) void wg_small_flush_kernel(const WgFlushArgs a) {
+    int layer = 0;
+    while (layer + 1 < a.count && (int)blockIdx.x >= a.first_block[layer + 1]) ++layer;
+    const int *sh = a.shape[layer];
+    wg_small_reduce_block<T>(a.ws[layer], reinterpret_cast<T *>(a.grad[layer]), (int)blockIdx.x - a.first_block[layer], sh[0],
+                             sh[1], sh[2], sh[3], sh[4], sh[5], sh[6], sh[7]);
 }
 
 struct SmallPlan {
@@ -785,6 +812,10 @@ int conv_small_wg(const ConvTileDesc &d, const void *X, const void *dY, void *dW
     return reduce_wg<T>(w, dW);
 }
 
+static ::ptl_wg_batch *g_wg_defer = nullptr;  // where the one-call backward leaves its partial sums, if anywhere
+
+void conv_small_defer_to(::ptl_wg_batch *batch) { g_wg_defer = batch; }
+
 template <typename T>
 int conv_small_bw(const ConvTileDesc &fwd, const ConvTileDesc &ig, const void *X, const void *dY, const void *Wt,
                   void *dW, void *dX) {
@@ -793,9 +824,60 @@ int conv_small_bw(const ConvTileDesc &fwd, const ConvTileDesc &ig, const void *X
     SmallPlan p;
     const int budget = state().num_cu - w.nwg;
     if (int rc = plan_small<T>(ig, dY, Wt, dX, budget > 32 ? budget : 32, p)) return rc;
+    // a deferred layer: its partial sums go to the batch's buffer (if they fit) and wait for the flush
+    ::ptl_wg_batch *b = g_wg_defer;
+    const size_t need = ((size_t)w.nwg * w.part_elems * sizeof(float) + 255) / 256 * 256;
+    const bool defer = b && b->buf && b->count >= 0 && b->count < PTL_WG_BATCH_MAX && b->used % 256 == 0 &&
+                       b->used <= b->bytes && need <= b->bytes - b->used && reinterpret_cast<uintptr_t>(b->buf) % 256 == 0;
+    if (defer) w.ws = reinterpret_cast<float *>(static_cast<char *>(b->buf) + b->used);
     if (int rc = dispatch_small<T>(p, &w)) return rc;
-    return reduce_wg<T>(w, dW);
+    if (!defer) return reduce_wg<T>(w, dW);
+    const int at = b->count++;
+    b->offset[at] = b->used;
+    b->grad[at] = dW;
+    const int shape[8] = {w.part_elems, w.nwg, w.rows_kept, w.cols_kept, w.cbi_n, w.Cout, w.Cin, w.taps};
+    for (int i = 0; i < 8; ++i) b->shape[8 * at + i] = shape[i];
+    b->used += need;
+    return 0;
 }
+
+template <typename T>
+int conv_small_flush(::ptl_wg_batch *b) {
+    if (!b || b->count < 0 || b->count > PTL_WG_BATCH_MAX || (b->count > 0 && !b->buf)) {
+        set_error("weight-gradient flush: invalid batch");
+        return 1;
+    }
+    if (b->count == 0) {
+        b->used = 0;
+        return 0;
+    }
+    if (!ensure_init()) return 2;
+    WgFlushArgs a;
+    a.count = b->count;
+    int blocks = 0;
+    for (int i = 0; i < b->count; ++i) {
+        const int *shape = b->shape + 8 * i;
+        if (b->offset[i] % 4 || b->offset[i] > b->bytes || !b->grad[i] || shape[0] <= 0 || shape[1] <= 0 || shape[2] <= 0 ||
+            shape[3] <= 0 || shape[4] <= 0 || shape[7] <= 0 ||
+            (size_t)shape[0] * shape[1] * sizeof(float) > b->bytes - b->offset[i]) {
+            set_error("weight-gradient flush: layer %d of the batch does not describe partial sums inside its buffer", i);
+            return 1;
+        }
+        a.first_block[i] = blocks;
+        blocks += (shape[0] + 63) / 64;
+        a.ws[i] = reinterpret_cast<const float *>(static_cast<const char *>(b->buf) + b->offset[i]);
+        a.grad[i] = b->grad[i];
+        for (int k = 0; k < 8; ++k) a.shape[i][k] = shape[k];
+    }
+    a.first_block[b->count] = blocks;
+    hipLaunchKernelGGL(wg_small_flush_kernel<T>, dim3(blocks), dim3(1024), 0, state().stream, a);
+    b->count = 0;
+    b->used = 0;
+    return hip_ok(hipGetLastError(), "weight-gradient flush launch") ? 0 : 2;
+}
+
+template int conv_small_flush<half_t>(::ptl_wg_batch *);
+template int conv_small_flush<float>(::ptl_wg_batch *);
 
 template int conv_small<half_t>(const ConvTileDesc &, const void *, const void *, void *);
 template int conv_small<float>(const ConvTileDesc &, const void *, const void *, void *);

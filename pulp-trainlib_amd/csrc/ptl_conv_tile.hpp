@@ -3,6 +3,7 @@
 #include "ptl_common.hpp"
 
 struct ptl_conv_cache;
+struct ptl_wg_batch;
 
 namespace ptl {
 
@@ -126,6 +127,11 @@ int conv_halo_bw(const ConvTileDesc &fwd, const ConvTileDesc &ig, const void *X,
 // written by the forward route that builds such a copy, `use` read by the weight-gradient routes.  Both null outside
 // the *_cached entry points.
 void conv_cache_set(struct ::ptl_conv_cache *fill, const struct ::ptl_conv_cache *use);
+// Where the small-layer weight gradient leaves its partial sums instead of adding them up itself (nullptr: nowhere);
+// the one launch that adds up all the layers a batch holds.
+void conv_small_defer_to(struct ::ptl_wg_batch *batch);
+template <typename T>
+int conv_small_flush(struct ::ptl_wg_batch *batch);
 
 // Weight gradient over filter taps on the same GEMM (partial sums per tap and k split + one reduction).
 template <typename T>

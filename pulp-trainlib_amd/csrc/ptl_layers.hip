@@ -1045,6 +1045,21 @@ int ptl_conv2d_fp16_bw_batched_cached(const struct Conv2D_args_fp16 *a, int ns, 
     return rc;
 }
 
+int ptl_conv2d_fp16_bw_batched_deferred(const struct Conv2D_args_fp16 *a, int ns, struct ptl_wg_batch *batch) {
+    ptl::conv_small_defer_to(batch);
+    const int rc = ptl::conv2d_bw<half_t>(a, ns, "pulp_conv2d_fp16_bw_cl");
+    ptl::conv_small_defer_to(nullptr);
+    return rc;
+}
+int ptl_conv2d_fp32_bw_batched_deferred(const struct Conv2D_args *a, int ns, struct ptl_wg_batch *batch) {
+    ptl::conv_small_defer_to(batch);
+    const int rc = ptl::conv2d_bw<float>(a, ns, "pulp_conv2d_fp32_bw_cl");
+    ptl::conv_small_defer_to(nullptr);
+    return rc;
+}
+int ptl_conv2d_fp16_wg_flush(struct ptl_wg_batch *batch) { return ptl::conv_small_flush<half_t>(batch); }
+int ptl_conv2d_fp32_wg_flush(struct ptl_wg_batch *batch) { return ptl::conv_small_flush<float>(batch); }
+
 int ptl_conv_pw_fp32_fw_batched(const struct PointWise_Conv_args *a, int ns) {
     return ptl::pw_step<float>(a, ns, STEP_FW, "pulp_conv_pw_fp32_fw_cl");
 }

@@ -169,6 +169,12 @@ class ConvCache(C.Structure):
     _fields_ = [("buf", P), ("bytes", C.c_size_t), ("valid", I), ("geometry", I * 6)]
 
 
+class WgBatch(C.Structure):
+    """struct ptl_wg_batch: the partial sums of the small layers whose weight gradients one flush completes."""
+    _fields_ = [("buf", P), ("bytes", C.c_size_t), ("used", C.c_size_t), ("count", I), ("offset", C.c_size_t * 32),
+                ("grad", P * 32), ("shape", I * 256)]
+
+
 class NormFusion(C.Structure):
     """struct ptl_norm_fusion_fp32 / _fp16: what ptl_batch_norm_fused_* does behind the normalisation."""
     _fields_ = [("relu", I), ("skip", P), ("skip_diff", P), ("diff2", P)]

@@ -187,6 +187,10 @@ class ResNetStep:
         spec = {n: (ci, co, k, s) for n, ci, co, k, s in convs}
         L = lambda name: name.replace("DT", dt)
 
+        self.wg_buf = torch.empty(64 << 20, dtype=torch.uint8, device="cuda")
+        self.wg_batch = pkg.WgBatch()
+        self.wg_batch.buf, self.wg_batch.bytes = self.wg_buf.data_ptr(), self.wg_buf.numel()
+
         def conv(name, x, dx, H):
             """The convolution alone: (forward call, backward calls, output, its gradient, output size)."""
             ci, co, k, s = spec[name]
@@ -196,8 +200,9 @@ class ResNetStep:
             a, kp = hp.conv2d_args(pkg, x, dx, self.W[name], self.dW[name], y, dy, ci, H, H, co, k, k, Ho, Ho,
                                    (p, p, p, p), (s, s), 0, 1 if s == 1 else 0)
             self.keep.append(kp)
-            # weight and input gradient in one call (the stem needs no input gradient)
-            bw = [(L("ptl_conv2d_DT_bw_batched"), a, (ns,))] if dx is not None else [(L("ptl_conv2d_DT_wg_batched"), a, (ns,))]
+            # weight and input gradient in one call (the stem needs no input gradient); the additions that complete
+            # the weight gradients of the small layers wait for one flush behind the backward pass
+            bw = [(L("ptl_conv2d_DT_bw_batched_deferred"), a, (ns, self.wg_batch))] if dx is not None else [(L("ptl_conv2d_DT_wg_batched"), a, (ns,))]
             return (L("ptl_conv2d_DT_fw_batched"), a, (ns,)), bw, y, dy, Ho
 
         def norm(name, y, dy, Ho, relu, skip=None, out_diff=None):
@@ -275,6 +280,8 @@ class ResNetStep:
         for b in reversed(bw_blocks):
             self.bw += b
         self.bw += first_bw
+        if hasattr(self, "wg_batch"):
+            self.bw.append((L("ptl_conv2d_DT_wg_flush"), self.wg_batch, ()))
         opts = []
         for n in self.W:
             o, kp = hp.optim_args(pkg, dt, self.W[n], self.dW[n], None, None, self.lr, 0.0)

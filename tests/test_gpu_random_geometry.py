@@ -246,6 +246,53 @@ def test_conv2d_small_layer_1x1_random_geometries(pkg, gpu, dt, seed):
         assert rel(dw2, ref_dw) <= tol, (case, "dw, one call")
 
 
+@pytest.mark.parametrize("dt", ["fp16", "fp32"])
+def test_conv2d_deferred_weight_gradient_sums(pkg, gpu, dt):
+    """Backward calls that leave the addition of their partial sums to one flush: the same bits as the calls that add
+    up themselves, for several layers in one batch (3x3 and 1x1, stride 1 and 2), a layer that does not take the
+    small-layer kernels (completed by its own call), a batch too small for a layer (likewise) and an empty flush."""
+    tdt = torch.float16 if dt == "fp16" else torch.float32
+    layers = [(16, 16, 32, 3, 1, 128), (16, 32, 32, 3, 2, 128), (16, 32, 32, 1, 2, 128), (64, 64, 8, 3, 1, 130),
+              (24, 40, 16, 3, 1, 5), (128, 128, 8, 3, 1, 4)]
+    buf = torch.empty(32 << 20, dtype=torch.uint8, device="cuda")
+    for room in (buf.numel(), 600 << 10):
+        batch = pkg.WgBatch()
+        batch.buf, batch.bytes = buf.data_ptr(), room
+        flush = getattr(gpu, "ptl_conv2d_%s_wg_flush" % dt)
+        assert flush(ctypes.byref(batch)) == 0 and batch.count == 0, gpu.ptl_last_error()
+        keep, pairs = [], []
+        for (Ci, Co, H, k, st, ns) in layers:
+            p = k // 2
+            Ho = (H + 2 * p - k) // st + 1
+            x = (torch.rand(ns, Ci, H, H, device="cuda") - 0.5).to(tdt)
+            w = ((torch.rand(Co, Ci, k, k, device="cuda") - 0.5) * 0.5).to(tdt)
+            dy = (torch.rand(ns, Co, Ho, Ho, device="cuda") - 0.5).to(tdt)
+            y = torch.zeros_like(dy)
+            outs = []
+            for deferred in (False, True):
+                dx, dw = torch.full_like(x, 3), torch.full_like(w, 3)
+                a, kp = hp.conv2d_args(pkg, x, dx, w, dw, y, dy, Ci, H, H, Co, k, k, Ho, Ho, (p, p, p, p), (st, st), 0,
+                                       1 if st == 1 else 0)
+                keep.append((kp, x, w, dy, y))
+                if deferred:
+                    rc = getattr(gpu, "ptl_conv2d_%s_bw_batched_deferred" % dt)(ctypes.byref(a), ns, ctypes.byref(batch))
+                    assert rc == 0, gpu.ptl_last_error()
+                else:
+                    pkg.call("ptl_conv2d_%s_bw_batched" % dt, a, ns)
+                outs.append((dx, dw))
+            pairs.append(outs)
+        waiting = batch.count
+        assert 0 < waiting < len(layers)  # (the 128-channel layer never waits; with little room fewer do)
+        if room == buf.numel():  # (in fp32 a 64-channel tile can be too large for the small-layer kernels)
+            assert waiting >= (len(layers) - 1 if dt == "fp16" else 3)
+        assert flush(ctypes.byref(batch)) == 0, gpu.ptl_last_error()
+        gpu.ptl_sync()
+        assert batch.count == 0 and batch.used == 0
+        for (now, later), layer in zip(pairs, layers):
+            assert torch.equal(now[0], later[0]), (layer, "dx")
+            assert torch.equal(now[1], later[1]), (layer, "dw")
+
+
 @pytest.mark.parametrize("seed", [21, 22])
 def test_depthwise_random_geometries(pkg, gpu, seed):
     rng = random.Random(seed)
