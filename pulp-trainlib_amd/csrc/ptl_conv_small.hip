@@ -716,6 +716,9 @@ int plan_wg(const ConvTileDesc &d, const void *X, const void *dY, int max_wg, bo
     // against 8.4 us for 16 -> 32 on 32x32 at one sample: below a few thousand positions what this kernel buys is
     // the input gradient riding along in the same launch)
     if (st.gemm_path != 6 && (positions > 262144 || (alone && positions < 8192))) return -1;
+    // (a single tap alone: beyond 65536 positions the streaming GEMM with its k split is ahead - 10.0 against 13.6 us
+    // for 32 -> 32 on 16x16 at batch 512)
+    if (st.gemm_path != 6 && K == 1 && alone && positions > 65536) return -1;
     w.G = d.Wo / VEC;
     w.Gin = d.Win / VEC;
     w.stride = d.sh;
