@@ -93,3 +93,50 @@ def test_resnet20_training_step_with_batch_norm(pkg, gpu, dt, ns, tol, fused):
     for n in w:
         assert hp.rel_l2(net.W[n].cpu().numpy(), ref_new[n]) <= tol, n
     assert net.launches() > (80 if fused else 170)
+
+
+@pytest.mark.parametrize("fused", [True, False])
+def test_training_step_replays_as_a_hip_graph(pkg, gpu, fused):
+    """The whole step (92 or 178 library calls) captured once into a HIP graph on a stream of the caller's and
+    replayed: after the warm-up calls the library allocates nothing and records no memset node, so every replay -
+    with eager library work and synchronisations between the replays - leaves bit for bit the parameters that the
+    same steps leave when called one by one."""
+    import ctypes
+    ns, dt = 16, "fp16"
+    side = torch.cuda.Stream()
+    gpu.ptl_set_stream(ctypes.c_void_p(side.cuda_stream))
+    try:
+        with torch.cuda.stream(side):
+            net = rs.ResNetStep(pkg, gpu, torch, dt, ns, rs.init_weights(0x2E600, dt), 0.01, norm=True, fused=fused)
+            net.x.copy_(torch.from_numpy(hp.normal(0x2E601, (ns, 3, 32, 32)).astype(np.float16)))
+            net.target.zero_()
+            net.target[torch.arange(ns), (3 * torch.arange(ns)) % 10] = 1
+            for _ in range(2):  # (workspaces reach their size, kernel attributes are set)
+                net.step()
+            side.synchronize()
+            params = dict(list(net.W.items()) + [("g:" + k, v) for k, v in net.G.items()] +
+                          [("b:" + k, v) for k, v in net.Bt.items()])
+            start = {n: v.clone() for n, v in params.items()}
+            eager = []
+            for _ in range(3):
+                net.step()
+                side.synchronize()
+                eager.append({n: v.clone() for n, v in params.items()})
+            for n in params:
+                params[n].copy_(start[n])
+            side.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph, stream=side):
+            net.step()
+        other = torch.zeros(1 << 16, dtype=torch.float16, device="cuda")
+        for k in range(3):
+            graph.replay()
+            torch.cuda.synchronize()
+            for n in params:
+                assert torch.equal(params[n], eager[k][n]), (k, n)
+            with torch.cuda.stream(side):  # eager work of the library between the replays
+                assert gpu.ptl_copy_bytes(ctypes.c_void_p(net.x.data_ptr()), ctypes.c_void_p(other.data_ptr()), 1 << 16) == 0
+                side.synchronize()
+    finally:
+        gpu.ptl_set_stream(None)
+        assert gpu.ptl_sync() == 0
