@@ -821,14 +821,15 @@ void conv_small_defer_to(::ptl_wg_batch *batch) { g_wg_defer = batch; }
 
 template <typename T>
 int conv_small_bw(const ConvTileDesc &fwd, const ConvTileDesc &ig, const void *X, const void *dY, const void *Wt,
-                  void *dW, void *dX) {
+                  void *dW, void *dX, bool may_defer) {
     WgSmallArgs w;
     if (int rc = plan_wg<T>(fwd, X, dY, state().num_cu / 2, false, w)) return rc;
     SmallPlan p;
     const int budget = state().num_cu - w.nwg;
     if (int rc = plan_small<T>(ig, dY, Wt, dX, budget > 32 ? budget : 32, p)) return rc;
     // a deferred layer: its partial sums go to the batch's buffer (if they fit) and wait for the flush
-    ::ptl_wg_batch *b = g_wg_defer;
+    // (not when dW is a staging copy of a host tensor: the call copies it back when it returns)
+    ::ptl_wg_batch *b = may_defer ? g_wg_defer : nullptr;
     const size_t need = ((size_t)w.nwg * w.part_elems * sizeof(float) + 255) / 256 * 256;
     const bool defer = b && b->buf && b->count >= 0 && b->count < PTL_WG_BATCH_MAX && b->used % 256 == 0 &&
                        b->used <= b->bytes && need <= b->bytes - b->used && reinterpret_cast<uintptr_t>(b->buf) % 256 == 0;
@@ -887,8 +888,8 @@ template int conv_small<float>(const ConvTileDesc &, const void *, const void *,
 template int conv_small_wg<half_t>(const ConvTileDesc &, const void *, const void *, void *);
 template int conv_small_wg<float>(const ConvTileDesc &, const void *, const void *, void *);
 template int conv_small_bw<half_t>(const ConvTileDesc &, const ConvTileDesc &, const void *, const void *, const void *,
-                                   void *, void *);
+                                   void *, void *, bool);
 template int conv_small_bw<float>(const ConvTileDesc &, const ConvTileDesc &, const void *, const void *, const void *,
-                                  void *, void *);
+                                  void *, void *, bool);
 
 }  // namespace ptl

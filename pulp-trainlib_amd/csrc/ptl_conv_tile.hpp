@@ -44,7 +44,7 @@ template <typename T>
 int conv_small_wg(const ConvTileDesc &d, const void *X, const void *dY, void *dW);
 template <typename T>
 int conv_small_bw(const ConvTileDesc &fwd, const ConvTileDesc &ig, const void *X, const void *dY, const void *Wt,
-                  void *dW, void *dX);
+                  void *dW, void *dX, bool may_defer);
 
 }  // namespace ptl
 

@@ -676,7 +676,9 @@ static int conv2d_bw(const Args *a, int ns, const char *fn) {
                 if (sg.failed()) return 2;
                 state().last_conv_direct = 0;
                 state().last_conv_resident = 0;
-                int rc = small ? conv_small_bw<T>(f, b, X, dY, Wt, dW, dX) : -1;
+                // (a host tensor's gradient is a staging copy that this call copies back: its sums cannot wait)
+                const bool on_device = static_cast<const void *>(dW) == static_cast<const void *>(a->coeff->diff);
+                int rc = small ? conv_small_bw<T>(f, b, X, dY, Wt, dW, dX, on_device) : -1;
                 if (rc < 0 && wide) rc = conv_halo_bw<T>(f, b, X, dY, Wt, dW, dX);
                 if (rc >= 0) {
                     if (rc == 0) state().last_conv_direct = 1;

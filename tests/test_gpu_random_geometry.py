@@ -291,6 +291,24 @@ def test_conv2d_deferred_weight_gradient_sums(pkg, gpu, dt):
         for (now, later), layer in zip(pairs, layers):
             assert torch.equal(now[0], later[0]), (layer, "dx")
             assert torch.equal(now[1], later[1]), (layer, "dw")
+    # tensors in host memory: the call works on staging copies that it copies back, so it completes the gradient
+    # itself and leaves the batch alone
+    nd = np.float16 if dt == "fp16" else np.float32
+    Ci, Co, H, ns = 16, 16, 16, 8
+    rng = np.random.default_rng(7)
+    x, w, dy = [(rng.random(sh) - 0.5).astype(nd) for sh in ((ns, Ci, H, H), (Co, Ci, 3, 3), (ns, Co, H, H))]
+    y = np.zeros_like(dy)
+    host = []
+    for deferred in (False, True):
+        dx, dw = np.full_like(x, 3), np.full_like(w, 3)
+        a, kp = hp.conv2d_args(pkg, x, dx, w, dw, y, dy, Ci, H, H, Co, 3, 3, H, H, (1, 1, 1, 1), (1, 1))
+        if deferred:
+            assert getattr(gpu, "ptl_conv2d_%s_bw_batched_deferred" % dt)(ctypes.byref(a), ns, ctypes.byref(batch)) == 0
+            assert batch.count == 0
+        else:
+            pkg.call("ptl_conv2d_%s_bw_batched" % dt, a, ns)
+        host.append((dx, dw))
+    assert np.array_equal(host[0][0], host[1][0]) and np.array_equal(host[0][1], host[1][1])
 
 
 @pytest.mark.parametrize("seed", [21, 22])
