@@ -248,18 +248,20 @@ int ptl_sync(void);
  * channel counts fill whole 128-byte slabs) is taken whenever the geometry fits
  * it, on the pipelined GEMM; 5 = the same route with the input tile resident in
  * LDS for all taps (3x3 fp16 channel-major layers) wherever that kernel fits;
- * 6 = as 0, but the single-launch kernel for small 3x3 fp16 channel-major
- * layers (at most 64 channels on either side; by default only up to four
- * workgroups per compute unit) is taken whenever the geometry fits it.
+ * 6 = as 0, but the kernels for small channel-major layers (3x3 or 1x1 filters,
+ * stride 1 or 2, at most 64 channels on either side, fp16 and fp32; by default
+ * only up to four - for layers narrower than 64 channels sixteen - workgroups
+ * per compute unit, and for the weight gradient only up to 262144 positions)
+ * are taken whenever the geometry fits them.
  * All routes compute the same products.
  * ptl_last_conv_direct() tells whether the last Conv2D call ran one of the
  * convolution kernels (1) or the implicit-im2col GEMM (0);
  * ptl_last_gemm_streamed() whether the last product that went to the pipelined
  * GEMM ran its streaming kernel (resident row panel, column tiles streamed:
  * the route of pointwise layers over a batch) (1) or a tile-per-workgroup
- * kernel (0); ptl_last_conv_resident() whether the last Conv2D forward or
- * input-gradient call that took the tap route kept its input tile in LDS (1),
- * or ran the small-layer kernel (2). */
+ * kernel (0); ptl_last_conv_resident() whether the last Conv2D call that took
+ * the tap route kept its input tile in LDS (1), or ran the small-layer kernels
+ * (2: forward, either gradient, or both gradients in one call). */
 void ptl_set_gemm_path(int path);
 int ptl_last_conv_direct(void);
 int ptl_last_gemm_streamed(void);
