@@ -246,6 +246,8 @@ struct WgSmallArgs {
     int cbi_n, combos, kparts;  // 32-channel blocks, (filter block, channel block) pairs, position shares
     int total;                  // Cout * Cin * taps
     int taps;                   // 9, or 1 for a 1x1 filter
+    int bsplit, kparts_split;   // 1: a workgroup per (tile, block of the weight tensor); the position shares of such a workgroup
+    int tiles;                  // tiles of samples and rows (= nwg, or nwg / combos with bsplit): the parts of the second launch
     int rows_kept, cols_kept, part_elems;  // filter rows and channels of a 32x32 tile that are stored; floats per workgroup in ws
 };
 
@@ -295,12 +297,29 @@ __device__ inline void wg_small_block(const WgSmallArgs &a, int wg, char *smem) 
     constexpr int VEC = 16 / (int)sizeof(T);
     typedef typename EdgePair<T>::type edge_t;
     const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    // Layers of more than 32 channels on a side: a workgroup per 32 x 32 block of the weight tensor (bsplit) - it
+    // copies the 32 gradient and the 32 input channels of its block only, splits the positions over all its waves
+    // and leaves a quarter of the partial sums; `tile` is the tile of samples and rows it shares with its siblings.
+    int tile = wg, co0 = 0, ci0 = 0, Cout = a.Cout, Cin = a.Cin, combos = a.combos, kparts = a.kparts, cbi_n = a.cbi_n;
+    int part_elems = a.part_elems;
+    if (a.bsplit) {
+        tile = wg / a.combos;
+        const int block = wg - tile * a.combos, bo = block / a.cbi_n;
+        co0 = 32 * bo;
+        ci0 = 32 * (block - bo * a.cbi_n);
+        Cout = min(32, a.Cout - co0);
+        Cin = min(32, a.Cin - ci0);
+        combos = cbi_n = 1;
+        kparts = a.kparts_split;
+        part_elems = a.part_elems / a.combos;
+    }
+    const int y_chunks = Cout * a.groups, x_chunks = Cin * a.S * a.R2G, pad_chunks = Cin * a.pad_rows;
     T *Ys = reinterpret_cast<T *>(smem);
-    T *Xs = Ys + a.Cout * a.PY;
+    T *Xs = Ys + Cout * a.PY;
     const T *gX = reinterpret_cast<const T *>(a.X), *gY = reinterpret_cast<const T *>(a.dY);
     // the tile: samples b0 .. b0 + S - 1, output rows y0 .. y0 + R - 1
-    const int timg = wg / a.tiles_per_img;
-    const int b0 = timg * a.S, y0 = (wg - timg * a.tiles_per_img) * a.R;
+    const int timg = tile / a.tiles_per_img;
+    const int b0 = timg * a.S, y0 = (tile - timg * a.tiles_per_img) * a.R;
 
     // ---- copy: all loads first, then the LDS writes
     uint4 yv[WG_CHUNKS], xv[WG_CHUNKS];
@@ -309,39 +328,39 @@ __device__ inline void wg_small_block(const WgSmallArgs &a, int wg, char *smem) 
     for (int k = 0; k < WG_CHUNKS; ++k) {
         const int q = tid + CS_NT * k;
         yv[k] = xv[k] = make_uint4(0, 0, 0, 0);
-        if (q < a.y_chunks) {
+        if (q < y_chunks) {
             const int co = fast_div(q, a.magic_ychan), rem = q - co * ychan;
             const int s = fast_div(rem, a.magic_rg), r2 = rem - s * a.RG;
             const int ly = fast_div(r2, a.magic_g), xg = r2 - ly * a.G;
             if (b0 + s < a.batch && y0 + ly < a.Ho)
-                yv[k] = *reinterpret_cast<const uint4 *>(gY + (((size_t)(b0 + s) * a.Cout + co) * a.Ho + y0 + ly) * a.Wo + VEC * xg);
+                yv[k] = *reinterpret_cast<const uint4 *>(gY + (((size_t)(b0 + s) * a.Cout + co0 + co) * a.Ho + y0 + ly) * a.Wo + VEC * xg);
         }
-        if (q < a.x_chunks) {
+        if (q < x_chunks) {
             const int ci = fast_div(q, a.magic_xchan), rem = q - ci * xchan;
             const int s = fast_div(rem, a.magic_r2g), r2 = rem - s * a.R2G;
             const int ly = fast_div(r2, a.magic_gin), xg = r2 - ly * a.Gin;
             const int iy = y0 * STRIDE - a.padU + ly;
             if (b0 + s < a.batch && iy >= 0 && iy < a.Hin)
-                xv[k] = *reinterpret_cast<const uint4 *>(gX + (((size_t)(b0 + s) * a.Cin + ci) * a.Hin + iy) * a.Win + VEC * xg);
+                xv[k] = *reinterpret_cast<const uint4 *>(gX + (((size_t)(b0 + s) * a.Cin + ci0 + ci) * a.Hin + iy) * a.Win + VEC * xg);
         }
     }
     // zero pieces: in front of every input row and behind the last one; behind the last gradient group
-    for (int q = tid; q < a.pad_chunks; q += CS_NT) {
+    for (int q = tid; q < pad_chunks; q += CS_NT) {
         const int ci = fast_div(q, a.magic_padrows), j = q - ci * a.pad_rows;
         // (per row one piece, or one per half; the last one behind the last row)
         const int at = STRIDE == 1 ? j * a.WP : (j >> 1) * a.WP + (j & 1) * (VEC + a.Win / 2);
         *reinterpret_cast<uint4 *>(Xs + ci * a.PX + at) = make_uint4(0, 0, 0, 0);
     }
-    for (int co = tid; co < a.Cout; co += CS_NT)
+    for (int co = tid; co < Cout; co += CS_NT)
         *reinterpret_cast<uint4 *>(Ys + co * a.PY + a.groups * VEC) = make_uint4(0, 0, 0, 0);
 #pragma unroll
     for (int k = 0; k < WG_CHUNKS; ++k) {
         const int q = tid + CS_NT * k;
-        if (q < a.y_chunks) {
+        if (q < y_chunks) {
             const int co = fast_div(q, a.magic_ychan), rem = q - co * ychan;
             *reinterpret_cast<uint4 *>(Ys + co * a.PY + rem * VEC) = yv[k];
         }
-        if (q < a.x_chunks) {
+        if (q < x_chunks) {
             const int ci = fast_div(q, a.magic_xchan), rem = q - ci * xchan;
             const int row = fast_div(rem, a.magic_gin), xg = rem - row * a.Gin;  // row = s * rows_in + ly
             T *at = Xs + ci * a.PX + row * a.WP + VEC;
@@ -366,9 +385,9 @@ __device__ inline void wg_small_block(const WgSmallArgs &a, int wg, char *smem) 
 
     // ---- products
     const int ky = K1 ? 0 : wave % 3, rest = K1 ? wave : wave / 3;
-    const int combo = rest % a.combos, kpart = rest / a.combos;
-    const bool active = (K1 || wave < 15) && kpart < a.kparts;
-    const int cbo = combo / a.cbi_n, cbi = combo - cbo * a.cbi_n;
+    const int combo = rest % combos, kpart = rest / combos;
+    const bool active = (K1 || wave < 15) && kpart < kparts;
+    const int cbo = combo / cbi_n, cbi = combo - cbo * cbi_n;
     const int lr = lane & 31, kg = lane >> 5;
     const int nks = (a.groups + 1) >> 1;
     f32x16 acc[3];
@@ -378,16 +397,16 @@ __device__ inline void wg_small_block(const WgSmallArgs &a, int wg, char *smem) 
         for (int v = 0; v < 16; ++v) acc[kx][v] = 0.f;
     if (active) {
         // filters and channels beyond the tensors repeat the last one (their rows and columns are never stored)
-        const T *yrow = Ys + min(cbo * 32 + lr, a.Cout - 1) * a.PY;
-        const T *xrow = Xs + min(cbi * 32 + lr, a.Cin - 1) * a.PX + ky * a.WP + VEC;
+        const T *yrow = Ys + min(cbo * 32 + lr, Cout - 1) * a.PY;
+        const T *xrow = Xs + min(cbi * 32 + lr, Cin - 1) * a.PX + ky * a.WP + VEC;
         constexpr int U = 4;  // k steps whose LDS reads are in flight together
-        for (int ks0 = kpart; ks0 < nks; ks0 += U * a.kparts) {
+        for (int ks0 = kpart; ks0 < nks; ks0 += U * kparts) {
             uint4 A[U], C[U], D[U];
             edge_t p3[U], n0[U];
 #pragma unroll
             for (int u = 0; u < U; ++u) {
                 // (steps behind the last one read the zero piece of the gradient)
-                const int gi = min(2 * (ks0 + u * a.kparts) + kg, a.groups);
+                const int gi = min(2 * (ks0 + u * kparts) + kg, a.groups);
                 const int gx = min(gi, a.groups - 1);
                 const int s = fast_div(gx, a.magic_rg), r2 = gx - s * a.RG;
                 const int ly = fast_div(r2, a.magic_g), xg = r2 - ly * a.G;
@@ -427,7 +446,7 @@ __device__ inline void wg_small_block(const WgSmallArgs &a, int wg, char *smem) 
     if (active) {
 #pragma unroll
         for (int kx = 0; kx < (K1 ? 1 : 3); ++kx) {
-            float *t = L + ((kpart * a.combos + combo) * a.taps + ky * 3 + kx) * 1024 + lr;
+            float *t = L + ((kpart * combos + combo) * a.taps + ky * 3 + kx) * 1024 + lr;
 #pragma unroll
             for (int v = 0; v < 16; ++v) t[(8 * (v >> 2) + 4 * kg + (v & 3)) * 32] = acc[kx][v];
         }
@@ -437,23 +456,23 @@ __device__ inline void wg_small_block(const WgSmallArgs &a, int wg, char *smem) 
     // (consecutive threads take consecutive elements of a tile: decoding an index of the weight tensor per element
     // would cost more than the sums, sixteen waves share the integer pipes); the second launch puts the sums where
     // the weight tensor wants them
-    float *out = a.ws + (size_t)wg * a.part_elems;
-    const int share = a.combos * a.taps * 1024, tile_elems = a.rows_kept * a.cols_kept;
+    float *out = a.ws + (size_t)wg * part_elems;
+    const int share = combos * a.taps * 1024, tile_elems = a.rows_kept * a.cols_kept;
     if (tile_elems == 1024) {  // whole tiles: thread t owns element t of every tile
-        for (int t = 0; t < a.combos * a.taps; ++t) {
+        for (int t = 0; t < combos * a.taps; ++t) {
             const float *src = L + t * 1024 + tid;
             float sum = src[0];
-            for (int kp = 1; kp < a.kparts; ++kp) sum += src[kp * share];
+            for (int kp = 1; kp < kparts; ++kp) sum += src[kp * share];
             out[t * 1024 + tid] = sum;
         }
         return;
     }
-    for (int e = tid; e < a.part_elems; e += CS_NT) {
+    for (int e = tid; e < part_elems; e += CS_NT) {
         const int t = fast_div(e, a.magic_tile), r = e - t * tile_elems;
         const int row = fast_div(r, a.magic_cols), col = r - row * a.cols_kept;
         const float *src = L + t * 1024 + row * 32 + col;
         float sum = src[0];
-        for (int kp = 1; kp < a.kparts; ++kp) sum += src[kp * share];
+        for (int kp = 1; kp < kparts; ++kp) sum += src[kp * share];
         out[e] = sum;
     }
 }
@@ -726,12 +745,17 @@ int plan_wg(const ConvTileDesc &d, const void *X, const void *dY, int max_wg, bo
     auto rows_in = [&](int R) { return (R - 1) * d.sh + K; };
     // pitches of 16 bytes mod 128: consecutive channels 16 bytes apart in the banks
     auto round_pitch = [](int n) { return n + ((VEC - n % (8 * VEC)) + 8 * VEC) % (8 * VEC); };
+    // more than one 32 x 32 block of the weight tensor: a workgroup per block (32 channels of either tensor in LDS,
+    // every wave on a share of the positions, a block's worth of partial sums to write)
+    const int blocks = ((d.Cin + 31) / 32) * ((d.Cout + 31) / 32);
+    w.bsplit = blocks > 1;
+    const int co_wg = w.bsplit ? 32 : d.Cout, ci_wg = w.bsplit ? 32 : d.Cin;  // channels a workgroup copies, at most
     auto lds_of = [&](int S, int R) {
         const int py = round_pitch(S * R * d.Wo + VEC), px = round_pitch((S * rows_in(R) + 1) * w.WP);
-        return ((size_t)d.Cout * py + (size_t)d.Cin * px) * ES;
+        return ((size_t)co_wg * py + (size_t)ci_wg * px) * ES;
     };
     auto chunks_ok = [&](int S, int R) {
-        return (long long)d.Cout * S * R * w.G <= WG_CHUNKS * CS_NT && (long long)d.Cin * S * rows_in(R) * w.Gin <= WG_CHUNKS * CS_NT &&
+        return (long long)co_wg * S * R * w.G <= WG_CHUNKS * CS_NT && (long long)ci_wg * S * rows_in(R) * w.Gin <= WG_CHUNKS * CS_NT &&
                lds_of(S, R) <= WG_SMALL_LDS;
     };
     // tiles: whole samples while the partial sums stay within about 5 MB (S samples each otherwise), rows of a
@@ -740,23 +764,24 @@ int plan_wg(const ConvTileDesc &d, const void *X, const void *dY, int max_wg, bo
     const long long part_bytes = (long long)((d.Cin + 31) / 32) * ((d.Cout + 31) / 32) * w.taps * (d.Cout < 32 ? d.Cout : 32) * (d.Cin < 32 ? d.Cin : 32) * 4;
     while ((long long)((d.batch + S - 1) / S) * part_bytes > (5LL << 20) && chunks_ok(S * 2, R)) S *= 2;
     if (S == 1)
-        while (R % 2 == 0 && (long long)d.batch * (d.Ho / R) * 2 <= max_wg && (R / 2) * w.G >= 16 &&
+        while (R % 2 == 0 && (long long)d.batch * (d.Ho / R) * 2 * blocks <= max_wg && (R / 2) * w.G >= 16 &&
                (long long)d.batch * (d.Ho / R) * 2 * part_bytes <= (5LL << 20))
             R /= 2;
     while (!chunks_ok(S, R) && R % 2 == 0 && S == 1) R /= 2;
     if (!chunks_ok(S, R)) return -1;
     w.S = S; w.R = R;
     w.tiles_per_img = (d.Ho + R - 1) / R;
-    w.nwg = ((d.batch + S - 1) / S) * w.tiles_per_img;
+    w.tiles = ((d.batch + S - 1) / S) * w.tiles_per_img;
+    w.nwg = w.tiles * (w.bsplit ? blocks : 1);
     w.rows_in = rows_in(R);
     w.RG = R * w.G; w.R2G = w.rows_in * w.Gin;
     w.groups = S * w.RG;
     w.PY = round_pitch(w.groups * VEC + VEC);
     w.pad_rows = (st2 ? 2 : 1) * S * w.rows_in + 1;
     w.PX = round_pitch((S * w.rows_in + 1) * w.WP);
-    w.y_chunks = d.Cout * w.groups;
-    w.x_chunks = d.Cin * S * w.R2G;
-    w.pad_chunks = d.Cin * w.pad_rows;
+    w.y_chunks = co_wg * w.groups;
+    w.x_chunks = ci_wg * S * w.R2G;
+    w.pad_chunks = ci_wg * w.pad_rows;
     if (w.y_chunks >= 65536 || w.x_chunks >= 65536 || w.pad_chunks >= 65536) return -1;  // (reciprocal multiplication)
     w.magic_g = magic_of(w.G);
     w.magic_gin = magic_of(w.Gin);
@@ -768,6 +793,7 @@ int plan_wg(const ConvTileDesc &d, const void *X, const void *dY, int max_wg, bo
     w.cbi_n = (d.Cin + 31) / 32;
     w.combos = w.cbi_n * ((d.Cout + 31) / 32);
     w.kparts = (K == 1 ? 16 : 4) / w.combos;
+    w.kparts_split = K == 1 ? 16 : 4;
     w.rows_kept = d.Cout < 32 ? d.Cout : 32;
     w.cols_kept = d.Cin < 32 ? d.Cin : 32;
     w.part_elems = w.combos * w.taps * w.rows_kept * w.cols_kept;
@@ -777,14 +803,14 @@ int plan_wg(const ConvTileDesc &d, const void *X, const void *dY, int max_wg, bo
     w.dY = dY;
     w.batch = d.batch; w.Cin = d.Cin; w.Cout = d.Cout; w.Hin = d.Hin; w.Win = d.Win; w.Ho = d.Ho; w.Wo = d.Wo;
     w.padU = d.padU; w.padL = d.padL;
-    w.ws = workspace((size_t)w.nwg * w.part_elems * sizeof(float));
+    w.ws = workspace((size_t)w.tiles * w.part_elems * sizeof(float));
     return w.ws ? 0 : 2;
 }
 
 template <typename T>
 int reduce_wg(const WgSmallArgs &w, void *dW) {
     hipLaunchKernelGGL(wg_small_reduce_kernel<T>, dim3((w.part_elems + 63) / 64), dim3(1024), 0, state().stream, w.ws,
-                       reinterpret_cast<T *>(dW), w.part_elems, w.nwg, w.rows_kept, w.cols_kept, w.cbi_n, w.Cout, w.Cin, w.taps);
+                       reinterpret_cast<T *>(dW), w.part_elems, w.tiles, w.rows_kept, w.cols_kept, w.cbi_n, w.Cout, w.Cin, w.taps);
     return hip_ok(hipGetLastError(), "small weight gradient reduction launch") ? 0 : 2;
 }
 
@@ -830,7 +856,7 @@ int conv_small_bw(const ConvTileDesc &fwd, const ConvTileDesc &ig, const void *X
     // a deferred layer: its partial sums go to the batch's buffer (if they fit) and wait for the flush
     // (not when dW is a staging copy of a host tensor: the call copies it back when it returns)
     ::ptl_wg_batch *b = may_defer ? g_wg_defer : nullptr;
-    const size_t need = ((size_t)w.nwg * w.part_elems * sizeof(float) + 255) / 256 * 256;
+    const size_t need = ((size_t)w.tiles * w.part_elems * sizeof(float) + 255) / 256 * 256;
     const bool defer = b && b->buf && b->count >= 0 && b->count < PTL_WG_BATCH_MAX && b->used % 256 == 0 &&
                        b->used <= b->bytes && need <= b->bytes - b->used && reinterpret_cast<uintptr_t>(b->buf) % 256 == 0;
     if (defer) w.ws = reinterpret_cast<float *>(static_cast<char *>(b->buf) + b->used);
@@ -839,7 +865,7 @@ int conv_small_bw(const ConvTileDesc &fwd, const ConvTileDesc &ig, const void *X
     const int at = b->count++;
     b->offset[at] = b->used;
     b->grad[at] = dW;
-    const int shape[8] = {w.part_elems, w.nwg, w.rows_kept, w.cols_kept, w.cbi_n, w.Cout, w.Cin, w.taps};
+    const int shape[8] = {w.part_elems, w.tiles, w.rows_kept, w.cols_kept, w.cbi_n, w.Cout, w.Cin, w.taps};
     for (int i = 0; i < 8; ++i) b->shape[8 * at + i] = shape[i];
     b->used += need;
     return 0;
