@@ -340,18 +340,19 @@ def resnet_rows(pkg, lib, timed, torch, dev):
         macs += (ci * co * 9 + co * co * 9 + (ci * co if proj else 0)) * Ho * Ho
         H = Ho
     flops = 3 * 2.0 * ns * (macs + 64 * ncls)
-    for norm, fused in ((True, True), (True, False), (False, False)):
-        net = rs.ResNetStep(pkg, lib, torch, dt, ns, rs.init_weights(0x2E5E0, dt), 0.01, norm=norm, fused=fused)
+    for norm, fused, stats in ((True, True, False), (True, True, True), (True, False, False), (False, False, False)):
+        net = rs.ResNetStep(pkg, lib, torch, dt, ns, rs.init_weights(0x2E5E0, dt), 0.01, norm=norm, fused=fused, stats=stats)
         net.x.copy_(torch.randn(ns, 3, 32, 32, device=dev).to(tdt[dt]))
         net.target.zero_()
         net.target[torch.arange(ns), torch.randint(0, 10, (ns,))] = 1
         ms = timed(lambda: net.step(update=True), 10, 3)
         rows.append({"workload": "resnet20 step%s FW+BW+SGD N=%d, %d launches"
-                                 % ((" with batch norm" + (", element-wise layers fused into it" if fused else "")) if norm
+                                 % ((" with batch norm" + (", element-wise layers fused into it" if fused else "") +
+                                     (", its sums formed by the convolutions" if stats else "")) if norm
                                     else " (no norm)", ns, net.launches()),
                      "dtype": dt, "us": round(ms * 1e3, 1), "TFLOP/s": round(flops / (ms * 1e-3) / 1e12, 3),
                      "samples/s": round(ns / (ms * 1e-3), 1)})
-        if norm and fused:
+        if norm and fused and not stats:
             # the same step captured once into a HIP graph on a side stream and replayed (one submission per step
             # instead of 92 calls)
             import ctypes

@@ -389,6 +389,18 @@ int ptl_batch_norm_fused_fp32_fw(const struct BatchNorm_args_fp32 *a, const stru
 int ptl_batch_norm_fused_fp32_bw(const struct BatchNorm_args_fp32 *a, const struct ptl_norm_fusion_fp32 *f);
 int ptl_batch_norm_fused_fp16_fw(const struct BatchNorm_args_fp16 *a, const struct ptl_norm_fusion_fp16 *f);
 int ptl_batch_norm_fused_fp16_bw(const struct BatchNorm_args_fp16 *a, const struct ptl_norm_fusion_fp16 *f);
+/* No counterpart in the reference: the forward convolution that also leaves the sums a batch normalisation of its
+ * output needs (struct ptl_norm_stats; formed from the values as stored, inside the small-layer kernels - other
+ * layers, and layers with USE_BIASES, return with st->valid = 0), and the fused normalisation forward that takes
+ * them: with st->valid and matching channels and count it runs one launch instead of two, else it behaves like
+ * ptl_batch_norm_fused_*_fw (f may be NULL: no fusion).  The sums are added in another order than the
+ * normalisation's own, so results agree to rounding of the statistics, not bit for bit. */
+int ptl_conv2d_fp32_fw_batched_stats(const struct Conv2D_args *a, int nsamples, struct ptl_norm_stats *st);
+int ptl_conv2d_fp16_fw_batched_stats(const struct Conv2D_args_fp16 *a, int nsamples, struct ptl_norm_stats *st);
+int ptl_batch_norm_fused_fp32_fw_stats(const struct BatchNorm_args_fp32 *a, const struct ptl_norm_fusion_fp32 *f,
+                                       const struct ptl_norm_stats *st);
+int ptl_batch_norm_fused_fp16_fw_stats(const struct BatchNorm_args_fp16 *a, const struct ptl_norm_fusion_fp16 *f,
+                                       const struct ptl_norm_stats *st);
 
 /* Plain product C[N x M] = A[N x K] * B (B is K x M, or M x K when trans_B),
  * the contract of the reference's mm family, on raw pointers. */

@@ -706,6 +706,20 @@ struct ptl_wg_batch {
                           tile, channel blocks, filters, channels, taps */
 };
 
+/* No counterpart in the reference: sums of a convolution's output and of its squares per channel, left by
+ * ptl_conv2d_*_fw_batched_stats for the batch normalisation behind it (ptl_batch_norm_fused_*_fw_stats), which then
+ * skips the launch that would read the tensor again for them.  The caller provides part (device memory, 16-byte
+ * aligned; 16 bytes per channel and workgroup of the convolution, 1 MiB hold any layer of a ResNet-20 at batch 128);
+ * the convolution fills the rest and sets valid to 1 when it took a route that forms the sums, else to 0. */
+struct ptl_norm_stats {
+    float *part;    /* [channel][part][4]: sum, sum of squares, two unused */
+    size_t bytes;   /* size of part */
+    size_t count;   /* elements per channel the sums cover (samples x rows x columns) */
+    int parts;      /* partial sums per channel */
+    int channels;
+    int valid;
+};
+
 /* No counterpart in the reference: what a residual block puts behind a normalisation layer, for the fused calls
  * ptl_batch_norm_fused_*.  All tensors have the shape of the normalisation's output (B x C x H x W). */
 struct ptl_norm_fusion_fp32 {

@@ -43,6 +43,11 @@ struct ConvSmallArgs {
     unsigned magic_inner9, magic_wo;
     int b_pitch, f_bytes;   // bytes per filter row in LDS, bytes of the filter tile
     int pgroups, mshift;    // jobs = groups of 32 pixels x (1 << mshift) blocks of 32 filters
+    // Sums of the output (before it is rounded to T) and of its squares per filter, for a normalisation layer behind
+    // the convolution:
+    // stats[(filter * ntiles + tile) * 4 + {0, 1}]; NULL: not wanted.  stats_off: bytes into LDS of the jobs' sums.
+    float *stats;
+    int stats_off, ntiles;
     // per item: element offset into the sample (first channel, first tile row, column group), element offset into the
     // LDS tile, first tile row | first channel << 8 | column group << 16
     int item_g[CS_ITEMS], item_l[CS_ITEMS], item_rc[CS_ITEMS];
@@ -53,6 +58,20 @@ union Piece {
     uint4 v;
     T e[16 / sizeof(T)];
 };
+
+// One halving step of a sum over the 16 lanes of a row: of the 2 * HALF values a lane holds it keeps the upper or the
+// lower HALF (`up`) and adds the partner lane's copy of them, which arrives through the DPP pattern CTRL (a pattern that
+// pairs lanes whose `up` differ).
+template <int HALF, int CTRL>
+__device__ inline void stats_fold(float (&s0)[16], float (&s1)[16], bool up) {
+#pragma unroll
+    for (int j = 0; j < HALF; ++j) {
+        const float keep0 = up ? s0[j + HALF] : s0[j], send0 = up ? s0[j] : s0[j + HALF];
+        const float keep1 = up ? s1[j + HALF] : s1[j], send1 = up ? s1[j] : s1[j + HALF];
+        s0[j] = keep0 + __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(send0), CTRL, 0xF, 0xF, false));
+        s1[j] = keep1 + __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(send1), CTRL, 0xF, 0xF, false));
+    }
+}
 
 // T: element type; VEC = 16 / sizeof(T) elements make a 16-byte piece (8 halves, 4 floats): the channels of an LDS
 // chunk, the columns of a global piece, the k values a lane hands to one MFMA step.
@@ -206,14 +225,53 @@ __device__ inline void conv_small_block(const ConvSmallArgs &a, int tile, char *
                 }
             }
         }
+        const int left = a.Cout - mb * 32 - 4 * kg;  // filters from this lane's first one
         if (pg * 32 + lr < npix) {
             T *out = reinterpret_cast<T *>(a.Y) + (((size_t)b * a.Cout + mb * 32 + 4 * kg) * a.Ho + y0 + py) * a.Wo + px;
-            const int left = a.Cout - mb * 32 - 4 * kg;  // filters from this lane's first one
 #pragma unroll
             for (int v = 0; v < 16; ++v) {
                 const int f = 8 * (v >> 2) + (v & 3);
                 if (f < left) out[f * plane] = (T)acc[v];
             }
+        }
+        if (a.stats) {
+            // Sums over the job's 32 pixels of the results (and of their squares): a lane holds 16 filters of one
+            // pixel.  Four exchanges inside a row of 16 lanes (mirrored row, mirrored half row, lanes 2 and 1 apart: DPP
+            // moves, no LDS traffic) in each of which a lane keeps the half of its values that one bit of its lane
+            // number selects and adds the partner's copy of them leave filter `lane % 16` summed over the row; the
+            // two rows of a half-wave are added last.
+            float s0[16], s1[16];
+            // (lanes beyond the tile's last pixel repeat it and count as zeros; filters the layer does not have come
+            // out as sums nobody reads)
+            const bool pix_ok = pg * 32 + lr < npix;
+#pragma unroll
+            for (int v = 0; v < 16; ++v) s0[v] = pix_ok ? acc[v] : 0.f;
+#pragma unroll
+            for (int v = 0; v < 16; ++v) s1[v] = s0[v] * s0[v];
+            stats_fold<8, 0x140>(s0, s1, (lr & 8) != 0);
+            stats_fold<4, 0x141>(s0, s1, (lr & 4) != 0);
+            stats_fold<2, 0x4E>(s0, s1, (lr & 2) != 0);
+            stats_fold<1, 0xB1>(s0, s1, (lr & 1) != 0);
+            const float o0 = __shfl_xor(s0[0], 16), o1 = __shfl_xor(s1[0], 16);
+            if (lr < 16) {
+                const int f = 8 * (lr >> 2) + (lr & 3) + 4 * kg;  // value index lr of this lane's sixteen
+                float2 *S = reinterpret_cast<float2 *>(smem + a.stats_off);
+                S[job * 32 + f] = make_float2(s0[0] + o0, s1[0] + o1);
+            }
+        }
+    }
+    if (a.stats) {  // the jobs' sums of a filter added in job order: one partial per workgroup and filter
+        __syncthreads();
+        if (tid < a.Cout) {
+            const int mb = tid >> 5, f = tid & 31, npg = min(a.pgroups, (npix + 31) >> 5);
+            const float2 *S = reinterpret_cast<const float2 *>(smem + a.stats_off);
+            float t0 = 0.f, t1 = 0.f;
+            for (int pg = 0; pg < npg; ++pg) {
+                const float2 v = S[((pg << a.mshift) + mb) * 32 + f];
+                t0 += v.x;
+                t1 += v.y;
+            }
+            *reinterpret_cast<float2 *>(a.stats + ((size_t)tid * a.ntiles + tile) * 4) = make_float2(t0, t1);
         }
     }
 }
@@ -816,10 +874,31 @@ int reduce_wg(const WgSmallArgs &w, void *dW) {
 
 }  // namespace
 
+static ::ptl_norm_stats *g_norm_stats = nullptr;  // where the forward pass leaves the sums of its output, if anywhere
+
+void conv_small_stats_to(::ptl_norm_stats *st) { g_norm_stats = st; }
+
 template <typename T>
 int conv_small(const ConvTileDesc &d, const void *X, const void *Wt, void *Y) {
     SmallPlan p;
     if (int rc = plan_small<T>(d, X, Wt, Y, state().num_cu, p)) return rc;
+    if (::ptl_norm_stats *st = g_norm_stats) {
+        // a pair of sums per job (32 pixels x 32 filters) in LDS behind the tile, a partial per workgroup and filter
+        // in the caller's buffer; a layer whose jobs or partials do not fit goes without
+        const size_t off = (p.lds + 15) / 16 * 16, need = (size_t)(p.a.pgroups << p.a.mshift) * 32 * sizeof(float2);
+        const size_t part_bytes = (size_t)d.Cout * p.tiles * 4 * sizeof(float);
+        if (off + need <= 150 * 1024 && st->part && part_bytes <= st->bytes &&
+            reinterpret_cast<uintptr_t>(st->part) % 16 == 0) {
+            p.a.stats = st->part;
+            p.a.stats_off = (int)off;
+            p.a.ntiles = p.tiles;
+            p.lds = off + need;
+            st->parts = p.tiles;
+            st->channels = d.Cout;
+            st->count = (size_t)d.batch * d.Ho * d.Wo;
+            st->valid = 1;
+        }
+    }
     return dispatch_small<T>(p, nullptr);
 }
 

@@ -4,6 +4,7 @@
 
 struct ptl_conv_cache;
 struct ptl_wg_batch;
+struct ptl_norm_stats;
 
 namespace ptl {
 
@@ -132,6 +133,9 @@ void conv_cache_set(struct ::ptl_conv_cache *fill, const struct ::ptl_conv_cache
 void conv_small_defer_to(struct ::ptl_wg_batch *batch);
 template <typename T>
 int conv_small_flush(struct ::ptl_wg_batch *batch);
+// Where the small-layer forward kernel leaves per-workgroup sums of its output and of its squares per filter (struct
+// ptl_norm_stats; nullptr: nowhere).  The call marks the struct valid when it filled it.
+void conv_small_stats_to(struct ::ptl_norm_stats *st);
 
 // Weight gradient over filter taps on the same GEMM (partial sums per tap and k split + one reduction).
 template <typename T>

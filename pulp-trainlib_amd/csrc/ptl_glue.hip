@@ -519,17 +519,18 @@ __global__ __launch_bounds__(256) void bn_apply_kernel(const T *__restrict__ x, 
                                                        T *__restrict__ out, const T *__restrict__ weight,
                                                        const T *__restrict__ bias, const T *__restrict__ eps,
                                                        const float *__restrict__ part, T *__restrict__ dgamma,
-                                                       T *__restrict__ dbeta, int B, int C, int HW, int groups,
+                                                       T *__restrict__ dbeta, int B, int C, int HW, int nparts,
                                                        int per_group, int write_dx, int vec,
                                                        const BnFuse<T> f = BnFuse<T>()) {
     constexpr int VEC = 16 / (int)sizeof(T);
     const int c = blockIdx.x, grp = blockIdx.y, tid = threadIdx.x;
-    // the channel's partial sums (at most 64 groups): one lane each, folded by the first wave in a fixed order
+    // the channel's partial sums (the first kernel's: at most 64, one per lane), folded by the first wave in a fixed order
     __shared__ float tot[BN_SUMS];
     if (tid < 64) {
 #pragma unroll
         for (int k = 0; k < (BW ? 4 : 2); ++k) {
-            float v = tid < groups ? part[((size_t)c * groups + tid) * BN_SUMS + k] : 0.f;
+            float v = 0.f;
+            for (int i = tid; i < nparts; i += 64) v += part[((size_t)c * nparts + i) * BN_SUMS + k];
 #pragma unroll
             for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off);
             if (tid == 0) tot[k] = v;
@@ -619,8 +620,10 @@ __global__ __launch_bounds__(256) void bn_apply_kernel(const T *__restrict__ x, 
     }
 }
 
+// `given`: sums of the input left by the layer before (forward only); used when they cover this tensor.
 template <typename T, typename Args, typename Fusion = void>
-static int batch_norm_step(const Args *a, int bw, const char *fn, const Fusion *fu = nullptr) {
+static int batch_norm_step(const Args *a, int bw, const char *fn, const Fusion *fu = nullptr,
+                           const ::ptl_norm_stats *given = nullptr) {
     constexpr bool FUSED = !std::is_void<Fusion>::value;
     if (!a || !a->input || !a->output || !a->weight_data || !a->eps || (!bw && !a->bias_data) || (FUSED && !fu))
         return glue_bad(fn, "invalid arguments");
@@ -663,11 +666,15 @@ static int batch_norm_step(const Args *a, int bw, const char *fn, const Fusion *
             if (sg.failed()) return 2;
             vec = vec && aligned16(f.skip);
         }
-        hipLaunchKernelGGL((bn_sums_kernel<T, false>), dim3(C, groups), dim3(256), 0, st.stream, x, (const T *)nullptr,
-                           part, B, C, HW, per_group, vec, f0);
+        const bool have = given && given->valid == 1 && given->part && given->channels == C && given->parts > 0 &&
+                          given->count == (size_t)B * HW &&
+                          (size_t)C * given->parts * BN_SUMS * sizeof(float) <= given->bytes;
+        if (!have)
+            hipLaunchKernelGGL((bn_sums_kernel<T, false>), dim3(C, groups), dim3(256), 0, st.stream, x,
+                               (const T *)nullptr, part, B, C, HW, per_group, vec, f0);
         hipLaunchKernelGGL((bn_apply_kernel<T, false, FUSED>), dim3(C, groups), dim3(256), 0, st.stream, x,
-                           (const T *)nullptr, y, w, b, eps, part, (T *)nullptr, (T *)nullptr, B, C, HW, groups,
-                           per_group, 1, vec, f);
+                           (const T *)nullptr, y, w, b, eps, have ? given->part : part, (T *)nullptr, (T *)nullptr, B,
+                           C, HW, have ? given->parts : groups, per_group, 1, vec, f);
     } else {
         const T *dy = sg.in(reinterpret_cast<const T *>(a->output->diff), n);
         const bool want_dx = !a->skip_in_grad, want_dw = !a->skip_wg_grad;
@@ -765,6 +772,16 @@ int ptl_batch_norm_fused_fp16_fw(const struct BatchNorm_args_fp16 *a, const stru
 }
 int ptl_batch_norm_fused_fp16_bw(const struct BatchNorm_args_fp16 *a, const struct ptl_norm_fusion_fp16 *f) {
     return ptl::batch_norm_step<ptl::half_t>(a, 1, "ptl_batch_norm_fused_fp16_bw", f);
+}
+int ptl_batch_norm_fused_fp32_fw_stats(const struct BatchNorm_args_fp32 *a, const struct ptl_norm_fusion_fp32 *f,
+                                       const struct ptl_norm_stats *st) {
+    static const struct ptl_norm_fusion_fp32 none = {};
+    return ptl::batch_norm_step<float>(a, 0, "ptl_batch_norm_fused_fp32_fw_stats", f ? f : &none, st);
+}
+int ptl_batch_norm_fused_fp16_fw_stats(const struct BatchNorm_args_fp16 *a, const struct ptl_norm_fusion_fp16 *f,
+                                       const struct ptl_norm_stats *st) {
+    static const struct ptl_norm_fusion_fp16 none = {};
+    return ptl::batch_norm_step<ptl::half_t>(a, 0, "ptl_batch_norm_fused_fp16_fw_stats", f ? f : &none, st);
 }
 
 }  // extern "C"

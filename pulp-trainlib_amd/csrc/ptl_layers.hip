@@ -967,6 +967,21 @@ static int rowsum_mat(const T *mat, T *out, int N, int K) {
     return sg.finish(hip_ok(hipGetLastError(), "row sum launch") ? 0 : 2);
 }
 
+template <typename T, typename Args>
+static int conv2d_fw_stats(const Args *a, int ns, ::ptl_norm_stats *st, const char *fn) {
+    if (!st) {
+        set_error("%s: null statistics struct", fn);
+        return 1;
+    }
+    st->valid = 0;
+    const bool take = a && a->USE_BIASES != 1;  // (a bias is added by a launch behind the kernel that forms the sums)
+    if (take) conv_small_stats_to(st);
+    const int rc = conv2d_fw<T>(a, ns, fn);
+    conv_small_stats_to(nullptr);
+    if (rc) st->valid = 0;
+    return rc;
+}
+
 }  // namespace ptl
 
 // ---- C ABI -------------------------------------------------------------------------------
@@ -1058,6 +1073,12 @@ int ptl_conv2d_fp32_bw_batched_deferred(const struct Conv2D_args *a, int ns, str
     const int rc = ptl::conv2d_bw<float>(a, ns, "pulp_conv2d_fp32_bw_cl");
     ptl::conv_small_defer_to(nullptr);
     return rc;
+}
+int ptl_conv2d_fp16_fw_batched_stats(const struct Conv2D_args_fp16 *a, int ns, struct ptl_norm_stats *st) {
+    return ptl::conv2d_fw_stats<half_t>(a, ns, st, "pulp_conv2d_fp16_fw_cl");
+}
+int ptl_conv2d_fp32_fw_batched_stats(const struct Conv2D_args *a, int ns, struct ptl_norm_stats *st) {
+    return ptl::conv2d_fw_stats<float>(a, ns, st, "pulp_conv2d_fp32_fw_cl");
 }
 int ptl_conv2d_fp16_wg_flush(struct ptl_wg_batch *batch) { return ptl::conv_small_flush<half_t>(batch); }
 int ptl_conv2d_fp32_wg_flush(struct ptl_wg_batch *batch) { return ptl::conv_small_flush<float>(batch); }

@@ -175,6 +175,11 @@ class WgBatch(C.Structure):
                 ("grad", P * 32), ("shape", I * 256)]
 
 
+class NormStats(C.Structure):
+    """struct ptl_norm_stats: sums of a convolution's output per channel for the normalisation behind it."""
+    _fields_ = [("part", P), ("bytes", C.c_size_t), ("count", C.c_size_t), ("parts", I), ("channels", I), ("valid", I)]
+
+
 class NormFusion(C.Structure):
     """struct ptl_norm_fusion_fp32 / _fp16: what ptl_batch_norm_fused_* does behind the normalisation."""
     _fields_ = [("relu", I), ("skip", P), ("skip_diff", P), ("diff2", P)]

@@ -44,13 +44,18 @@ def init_weights(seed, dt):
 class ResNetStep:
     """Device buffers, argument structs and the call sequence of one training step on `ns` samples."""
 
-    def __init__(self, pkg, lib, torch, dt, ns, weights, lr=0.01, norm=False, fused=False):
+    def __init__(self, pkg, lib, torch, dt, ns, weights, lr=0.01, norm=False, fused=False, stats=False):
         """`fused` (with `norm`): ReLU, the residual sum and the sum of a tensor's two incoming gradients run inside
-        the normalisation calls (ptl_batch_norm_fused_*) instead of as element-wise calls of their own."""
+        the normalisation calls (ptl_batch_norm_fused_*) instead of as element-wise calls of their own and the backward
+        calls defer the additions of their weight gradients to one flush; with `stats` the forward convolutions also
+        leave the sums the normalisation behind them needs (ptl_conv2d_*_fw_batched_stats), which then runs one launch
+        instead of two."""
         self.pkg, self.lib, self.dt, self.ns, self.lr = pkg, lib, dt, ns, lr
         if fused:
             assert norm
+            self.use_stats = stats
             return self._build_fused(torch, weights)
+        assert not stats
         tdt = torch.float16 if dt == "fp16" else torch.float32
         dev = lambda a: torch.from_numpy(np.ascontiguousarray(a)).cuda()
         z = lambda *s: torch.zeros(*s, dtype=tdt, device="cuda")
@@ -187,6 +192,7 @@ class ResNetStep:
         spec = {n: (ci, co, k, s) for n, ci, co, k, s in convs}
         L = lambda name: name.replace("DT", dt)
 
+        self.stats = {}  # per convolution: the struct its forward call fills and its normalisation reads
         self.wg_buf = torch.empty(64 << 20, dtype=torch.uint8, device="cuda")
         self.wg_batch = pkg.WgBatch()
         self.wg_batch.buf, self.wg_batch.bytes = self.wg_buf.data_ptr(), self.wg_buf.numel()
@@ -203,7 +209,15 @@ class ResNetStep:
             # weight and input gradient in one call (the stem needs no input gradient); the additions that complete
             # the weight gradients of the small layers wait for one flush behind the backward pass
             bw = [(L("ptl_conv2d_DT_bw_batched_deferred"), a, (ns, self.wg_batch))] if dx is not None else [(L("ptl_conv2d_DT_wg_batched"), a, (ns,))]
-            return (L("ptl_conv2d_DT_fw_batched"), a, (ns,)), bw, y, dy, Ho
+            if not self.use_stats:
+                return (L("ptl_conv2d_DT_fw_batched"), a, (ns,)), bw, y, dy, Ho
+            # the forward call leaves the sums of its output for the normalisation behind it
+            st = pkg.NormStats()
+            part = torch.zeros(1 << 16, dtype=torch.float32, device="cuda")
+            st.part, st.bytes = part.data_ptr(), part.numel() * 4
+            self.stats[name] = st
+            self.keep.append(part)
+            return (L("ptl_conv2d_DT_fw_batched_stats"), a, (ns, st)), bw, y, dy, Ho
 
         def norm(name, y, dy, Ho, relu, skip=None, out_diff=None):
             """out = [relu](bn(y) [+ skip]); returns the calls, out, its gradient buffer and the fusion struct (whose
@@ -218,7 +232,8 @@ class ResNetStep:
             f.relu = relu
             f.skip = pkg.addr(skip)
             self.keep += [kp, f, skip]
-            return (L("ptl_batch_norm_fused_DT_fw"), na, (f,)), (L("ptl_batch_norm_fused_DT_bw"), na, (f,)), out, dout, f
+            fw = (L("ptl_batch_norm_fused_DT_fw_stats"), na, (f, self.stats[name])) if self.use_stats else (L("ptl_batch_norm_fused_DT_fw"), na, (f,))
+            return fw, (L("ptl_batch_norm_fused_DT_bw"), na, (f,)), out, dout, f
 
         self.x = z(ns, 3, 32, 32)
         cf, cb, y, dy, H = conv("stem", self.x, None, 32)

@@ -311,6 +311,89 @@ def test_conv2d_deferred_weight_gradient_sums(pkg, gpu, dt):
     assert np.array_equal(host[0][0], host[1][0]) and np.array_equal(host[0][1], host[1][1])
 
 
+@pytest.mark.parametrize("dt", ["fp16", "fp32"])
+def test_conv2d_forward_sums_feed_the_normalisation(pkg, gpu, dt):
+    """ptl_conv2d_*_fw_batched_stats: the same output bits as the plain forward call, and per channel the sum of the
+    output and of its squares (over the struct's parts, against the stored tensor summed in float64: the kernel sums
+    its results before they are rounded to the tensor type, so in fp16 the two differ by the rounding noise of the
+    elements, 2^-12 of the root of the sum of squares), for 3x3 and 1x1 layers, both strides, ragged last tiles and
+    channel counts that do not fill a 32-filter block.  ptl_batch_norm_fused_*_fw_stats with them: the result of the
+    call that forms its own sums to the rounding of the statistics.  Layers that cannot leave sums (a wide layer, one
+    with a bias, a buffer that is too small) say so, and the normalisation then forms its own: bit for bit."""
+    tdt = torch.float16 if dt == "fp16" else torch.float32
+    tol_sum, tol_sq, tol_out = (2e-3, 1e-3, 1e-3) if dt == "fp16" else (2e-6, 1e-6, 1e-5)
+    part = torch.empty(1 << 18, dtype=torch.float32, device="cuda")
+    #        ns, Ci, Co, H, K, stride, bias, room in bytes, sums expected
+    cases = [(128, 16, 16, 32, 3, 1, 0, part.numel() * 4, True), (128, 64, 64, 8, 3, 1, 0, part.numel() * 4, dt == "fp16"),
+             (64, 16, 32, 32, 3, 2, 0, part.numel() * 4, True), (64, 16, 32, 32, 1, 2, 0, part.numel() * 4, True),
+             (5, 24, 40, 16, 3, 1, 0, part.numel() * 4, True), (3, 8, 20, 24, 3, 1, 0, part.numel() * 4, True),
+             (2, 3, 16, 32, 3, 1, 0, part.numel() * 4, True), (9, 64, 48, 8, 1, 1, 0, part.numel() * 4, True),
+             (7, 12, 36, 24, 3, 1, 0, part.numel() * 4, True),
+             (4, 128, 128, 8, 3, 1, 0, part.numel() * 4, False), (5, 24, 40, 16, 3, 1, 1, part.numel() * 4, False),
+             (128, 16, 16, 32, 3, 1, 0, 4096, False)]
+    for case in cases:
+        ns, Ci, Co, H, K, s, bias, room, expect = case
+        p = K // 2
+        Ho = (H + 2 * p - K) // s + 1
+        x = (torch.rand(ns, Ci, H, H, device="cuda") - 0.5).to(tdt)
+        w = (torch.rand(Co, Ci, K, K, device="cuda") - 0.5).to(tdt)
+        bs = (torch.rand(Co, device="cuda") - 0.5).to(tdt)
+        y, y2 = torch.full((ns, Co, Ho, Ho), 3.0, device="cuda", dtype=tdt), torch.full((ns, Co, Ho, Ho), 3.0, device="cuda", dtype=tdt)
+        part.fill_(7.0)
+        st = pkg.NormStats()
+        st.part, st.bytes, st.valid = part.data_ptr(), room, 5
+        outs = []
+        for out, with_sums in ((y, True), (y2, False)):
+            a, kp = hp.conv2d_args(pkg, x, None, w, None, out, None, Ci, H, H, Co, K, K, Ho, Ho, (p, p, p, p), (s, s), 0,
+                                   1 if s == 1 else 0, bs if bias else None)
+            if with_sums:
+                rc = getattr(gpu, "ptl_conv2d_%s_fw_batched_stats" % dt)(ctypes.byref(a), ns, ctypes.byref(st))
+                assert rc == 0, gpu.ptl_last_error()
+            else:
+                pkg.call("ptl_conv2d_%s_fw_batched" % dt, a, ns)
+        assert gpu.ptl_sync() == 0
+        assert torch.equal(y, y2), case
+        assert st.valid == (1 if expect else 0), case
+        if st.valid:
+            assert st.channels == Co and st.count == ns * Ho * Ho and st.parts >= 1
+            used = Co * st.parts * 4
+            assert used * 4 <= room and bool((part[used:] == 7.0).all()), case
+            pt = part[:used].view(Co, st.parts, 4).double()
+            s0, s1 = pt[:, :, 0].sum(1), pt[:, :, 1].sum(1)
+            r0, r1 = y.double().sum((0, 2, 3)), (y.double() ** 2).sum((0, 2, 3))
+            assert bool(((s0 - r0).abs() <= tol_sum * r1.sqrt()).all()), case
+            assert bool(((s1 - r1).abs() <= tol_sq * r1).all()), case
+        else:
+            assert bool((part == 7.0).all()), case
+        # the normalisation behind it, with a residual sum and a ReLU
+        g, b = (torch.rand(Co, device="cuda") + 0.5).to(tdt), (torch.rand(Co, device="cuda") - 0.5).to(tdt)
+        eps = torch.tensor([1e-5], device="cuda").to(tdt)
+        skip = (torch.rand(ns, Co, Ho, Ho, device="cuda") - 0.5).to(tdt)
+        o1, o2 = torch.full_like(y, 3), torch.full_like(y, 3)
+        f = pkg.NormFusion()
+        f.relu, f.skip = 1, skip.data_ptr()
+        n1, k1 = hp.batch_norm_args(pkg, y, o1, g, b, eps, ns, Co, Ho, Ho)
+        n2, k2 = hp.batch_norm_args(pkg, y, o2, g, b, eps, ns, Co, Ho, Ho)
+        rc = getattr(gpu, "ptl_batch_norm_fused_%s_fw_stats" % dt)(ctypes.byref(n1), ctypes.byref(f), ctypes.byref(st))
+        assert rc == 0, gpu.ptl_last_error()
+        assert getattr(gpu, "ptl_batch_norm_fused_%s_fw" % dt)(ctypes.byref(n2), ctypes.byref(f)) == 0
+        assert gpu.ptl_sync() == 0
+        if st.valid:
+            assert hp.rel_l2(o1.float().cpu().numpy(), o2.float().cpu().numpy()) <= tol_out, case
+            # sums of another tensor (a count that does not match) are not taken
+            st.count += 1
+            o3 = torch.full_like(y, 3)
+            n3, k3 = hp.batch_norm_args(pkg, y, o3, g, b, eps, ns, Co, Ho, Ho)
+            assert getattr(gpu, "ptl_batch_norm_fused_%s_fw_stats" % dt)(ctypes.byref(n3), None, ctypes.byref(st)) == 0
+            n4, k4 = hp.batch_norm_args(pkg, y, o2, g, b, eps, ns, Co, Ho, Ho)
+            none = pkg.NormFusion()
+            assert getattr(gpu, "ptl_batch_norm_fused_%s_fw" % dt)(ctypes.byref(n4), ctypes.byref(none)) == 0
+            assert gpu.ptl_sync() == 0
+            assert torch.equal(o3, o2), case  # (no fusion struct: nothing behind the normalisation)
+        else:
+            assert torch.equal(o1, o2), case
+
+
 @pytest.mark.parametrize("seed", [21, 22])
 def test_depthwise_random_geometries(pkg, gpu, seed):
     rng = random.Random(seed)

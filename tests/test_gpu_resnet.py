@@ -95,9 +95,46 @@ def test_resnet20_training_step_with_batch_norm(pkg, gpu, dt, ns, tol, fused):
     assert net.launches() > (80 if fused else 170)
 
 
-@pytest.mark.parametrize("fused", [True, False])
+@pytest.mark.parametrize("dt,ns,tol", [("fp32", 6, 1e-3), ("fp16", 16, 5e-3)])
+def test_resnet20_step_with_sums_from_the_convolutions(pkg, gpu, dt, ns, tol):
+    """The fused step whose forward convolutions leave the sums for the normalisation behind them
+    (ptl_conv2d_*_fw_batched_stats / ptl_batch_norm_fused_*_fw_stats) against the fused step whose normalisation
+    layers form their own: every convolution of the network leaves its sums, and the step comes out the same to the
+    rounding of the statistics (fp32: everything the step writes; fp16, where one flipped rounding of an activation
+    moves the deepest gradients by per cent: the forward results)."""
+    w = rs.init_weights(0x2E610, dt)
+    x = hp.normal(0x2E611, (ns, 3, 32, 32)).astype(hp.np_dtype(dt))
+    nets = []
+    for stats in (False, True):
+        net = rs.ResNetStep(pkg, gpu, torch, dt, ns, w, 0.01, norm=True, fused=True, stats=stats)
+        net.x.copy_(torch.from_numpy(x))
+        net.target.zero_()
+        net.target[torch.arange(ns), (3 * torch.arange(ns)) % 10] = 1
+        net.step(update=True)
+        assert gpu.ptl_sync() == 0
+        nets.append(net)
+    own, given = nets
+    # (in fp32 the filters of a 64-channel layer are too large for the small-layer kernels: those layers leave no
+    # sums and their normalisation forms its own)
+    valid = sum(st.valid for st in given.stats.values())
+    assert len(given.stats) == 21 and (valid == 21 if dt == "fp16" else 14 <= valid < 21), valid
+    assert own.launches() == given.launches()
+    rel = lambda a, b: hp.rel_l2(a.float().cpu().numpy(), b.float().cpu().numpy())
+    assert rel(given.logits, own.logits) <= tol
+    assert rel(given.loss, own.loss) <= tol
+    if dt == "fp32":
+        for n in own.dW:
+            assert rel(given.dW[n], own.dW[n]) <= tol, n
+            assert rel(given.W[n], own.W[n]) <= tol, n
+        for n in own.dG:
+            assert rel(given.dG[n], own.dG[n]) <= tol, n
+            assert rel(given.dBt[n], own.dBt[n]) <= tol, n
+
+
+@pytest.mark.parametrize("fused", [True, False, "stats"])
 def test_training_step_replays_as_a_hip_graph(pkg, gpu, fused):
-    """The whole step (92 or 178 library calls) captured once into a HIP graph on a stream of the caller's and
+    """The whole step (92 or 178 library calls; "stats": the 92 with the sums of the convolutions' outputs formed by
+    the convolutions) captured once into a HIP graph on a stream of the caller's and
     replayed: after the warm-up calls the library allocates nothing and records no memset node, so every replay -
     with eager library work and synchronisations between the replays - leaves bit for bit the parameters that the
     same steps leave when called one by one."""
@@ -107,7 +144,8 @@ def test_training_step_replays_as_a_hip_graph(pkg, gpu, fused):
     gpu.ptl_set_stream(ctypes.c_void_p(side.cuda_stream))
     try:
         with torch.cuda.stream(side):
-            net = rs.ResNetStep(pkg, gpu, torch, dt, ns, rs.init_weights(0x2E600, dt), 0.01, norm=True, fused=fused)
+            net = rs.ResNetStep(pkg, gpu, torch, dt, ns, rs.init_weights(0x2E600, dt), 0.01, norm=True, fused=bool(fused),
+                                stats=fused == "stats")
             net.x.copy_(torch.from_numpy(hp.normal(0x2E601, (ns, 3, 32, 32)).astype(np.float16)))
             net.target.zero_()
             net.target[torch.arange(ns), (3 * torch.arange(ns)) % 10] = 1
