@@ -1382,6 +1382,78 @@ __global__ __launch_bounds__(256) void patch_cols_kernel(const T *__restrict__ s
     *reinterpret_cast<Chunk *>(buf + (size_t)i * VEC) = Chunk{v.x, v.y, v.z, v.w};
 }
 
+// The column-major patch matrix at unit strides from the source's side: a row (c, hk, wk) of the matrix is the image
+// plane c shifted by (hk - pad, wk - pad), so one 16-byte piece of a source row - with its left and right neighbours -
+// is all that the K x K pieces at the same place of the K x K shifted copies need.  A thread loads the three aligned
+// pieces once (zeros outside the tensor) and stores K x K pieces: elements VEC + d .. 2 VEC + d - 1 of the three
+// pieces in a row, d = wk - PADL, cut out with compile-time dword selections and 16-bit funnel shifts.  Source rows
+// run from -padU to Hp + K - 2 - padU, so that the matrix rows over the padding are written too.  The write side moves
+// as in a fill kernel and the read side is a ninth of it.
+template <typename T, int K, int PADL>
+__global__ __launch_bounds__(256) void patch_cols_shifted_kernel(const T *__restrict__ src, T *__restrict__ buf,
+                                                                 PatchGeom g, int wpcs, unsigned m_wpcs, int pieces) {
+    constexpr int VEC = 16 / (int)sizeof(T), EPD = 4 / (int)sizeof(T);  // elements per piece, per dword
+    typedef const PatchPiece __attribute__((address_space(1))) *GlobalPiece;
+    const int i = blockIdx.x * 256 + threadIdx.x, c = blockIdx.y;
+    if (i >= pieces) return;
+    const int hv = (int)div_magic((unsigned)i, m_wpcs), wpc = i - hv * wpcs;
+    const int h = hv + g.h_add;  // (h_add = -padU)
+    const bool row_ok = (unsigned)h < (unsigned)g.Hs;
+    const unsigned off = ((unsigned)c * g.Hs + (row_ok ? h : 0)) * g.Ws + wpc * VEC;
+    const bool l_ok = row_ok && wpc > 0, r_ok = row_ok && (wpc + 2) * VEC <= g.Ws;
+    const PatchPiece mine = *(row_ok ? (GlobalPiece)(src + off) : (GlobalPiece)&patch_zero);
+    const PatchPiece left = *(l_ok ? (GlobalPiece)(src + off - VEC) : (GlobalPiece)&patch_zero);
+    const PatchPiece right = *(r_ok ? (GlobalPiece)(src + off + VEC) : (GlobalPiece)&patch_zero);
+    const unsigned win[12] = {left.x, left.y, left.z, left.w, mine.x, mine.y, mine.z, mine.w, right.x, right.y, right.z, right.w};
+    PatchPiece out[K];
+#pragma unroll
+    for (int wk = 0; wk < K; ++wk) {
+        const int s0 = VEC + wk - PADL, dw = s0 / EPD, sub = s0 % EPD;  // (compile-time after unrolling)
+        if (sub == 0)
+            out[wk] = PatchPiece{win[dw], win[dw + 1], win[dw + 2], win[dw + 3]};
+        else
+            out[wk] = PatchPiece{__builtin_amdgcn_alignbit(win[dw + 1], win[dw], 16), __builtin_amdgcn_alignbit(win[dw + 2], win[dw + 1], 16),
+                                 __builtin_amdgcn_alignbit(win[dw + 3], win[dw + 2], 16), __builtin_amdgcn_alignbit(win[dw + 4], win[dw + 3], 16)};
+    }
+    const size_t P = (size_t)g.Hp * g.Wp;
+#pragma unroll
+    for (int hk = 0; hk < K; ++hk) {
+        const int hp = hv - hk;
+        if ((unsigned)hp < (unsigned)g.Hp) {
+            T *row = buf + ((size_t)(c * K + hk) * K) * P + (size_t)hp * g.Wp + wpc * VEC;
+#pragma unroll
+            for (int wk = 0; wk < K; ++wk) *reinterpret_cast<PatchPiece *>(row + wk * P) = out[wk];
+        }
+    }
+}
+
+template <typename T, int K, int PADL>
+static int launch_patch_cols_shifted(const T *src, T *buf, const PatchGeom &g) {
+    constexpr int VEC = 16 / (int)sizeof(T);
+    const int wpcs = g.Wp / VEC, pieces = (g.Hp + K - 1) * wpcs;
+    const unsigned m = (unsigned)((((unsigned long long)1 << 32) + wpcs - 1) / wpcs);
+    hipLaunchKernelGGL((patch_cols_shifted_kernel<T, K, PADL>), dim3((pieces + 255) / 256, g.C), dim3(256), 0, state().stream,
+                       src, buf, g, wpcs, wpcs == 1 ? 0u : m, pieces);
+    return hip_ok(hipGetLastError(), "patch launch") ? 0 : 2;
+}
+
+// 0 = launched; -1 = the geometry does not fit.
+template <typename T>
+static int patch_cols_shifted(const T *src, T *buf, const PatchGeom &g) {
+    constexpr int VEC = 16 / (int)sizeof(T);
+    if (g.hwc || !g.col_major || g.w_mul != 1 || g.h_mul != 1 || g.Hk != g.Wk || g.Wp % VEC || g.Ws % VEC || g.Wp > g.Ws ||
+        g.C > 65535 || reinterpret_cast<uintptr_t>(buf) % 16 || reinterpret_cast<uintptr_t>(src) % 16)
+        return -1;
+    // (32-bit element offsets into the source, quotients by multiplication below 2^16 pieces per plane)
+    if ((long long)g.C * g.Hs * g.Ws >= ((long long)1 << 31) || (long long)(g.Hp + g.Hk) * (g.Wp / VEC) >= 65536) return -1;
+    const int K = g.Hk, padl = -g.w_add;
+    if (K == 3 && padl == 1) return launch_patch_cols_shifted<T, 3, 1>(src, buf, g);
+    if (K == 3 && padl == 0) return launch_patch_cols_shifted<T, 3, 0>(src, buf, g);
+    if (K == 5 && padl == 2) return launch_patch_cols_shifted<T, 5, 2>(src, buf, g);
+    if (K == 7 && padl == 3) return launch_patch_cols_shifted<T, 7, 3>(src, buf, g);
+    return -1;
+}
+
 // 0 = launched; -1 = the geometry does not fit (the caller takes the general kernel).
 template <typename T>
 static int patch_cols(const T *src, T *buf, const PatchGeom &g) {
@@ -1533,6 +1605,7 @@ static int patch_build(const Args *a, int col_major, const char *fn) {
         return sg.finish(1);
     }
     if (int rc = patch_rows<T>(dsrc, dbuf, g); rc >= 0) return sg.finish(rc);
+    if (int rc = patch_cols_shifted<T>(dsrc, dbuf, g); rc >= 0) return sg.finish(rc);
     if (int rc = patch_cols<T>(dsrc, dbuf, g); rc >= 0) return sg.finish(rc);
     if (reinterpret_cast<uintptr_t>(dbuf) % 16 == 0)
         hipLaunchKernelGGL((patch_kernel<T, VEC>), dim3(nblocks((total + VEC - 1) / VEC)), dim3(256), 0, state().stream,

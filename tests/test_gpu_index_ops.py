@@ -223,10 +223,13 @@ def test_blocktranspose_tiles(pkg, orc, gpu, dt, hwc, Ci, Co, Hk, Wk):
                                                      (16, 32, 32, 1, (0, 0, 0, 0), (1, 1), 0), (64, 40, 48, 1, (0, 0, 0, 0), (1, 1), 0),
                                                      (8, 20, 24, 5, (2, 2, 2, 2), (1, 1), 0), (4, 19, 16, 3, (1, 1, 1, 1), (2, 1), 0),
                                                      (3, 8, 8, 3, (1, 1, 1, 1), (1, 1), 0), (6, 10, 16, 3, (0, 0, 0, 0), (1, 1), 1),
-                                                     (2, 70, 136, 3, (1, 1, 1, 1), (1, 1), 0)])
+                                                     (2, 70, 136, 3, (1, 1, 1, 1), (1, 1), 0),
+                                                     (5, 12, 16, 3, (0, 2, 2, 0), (1, 1), 0), (4, 11, 16, 3, (1, 1, 0, 1), (1, 1), 0),
+                                                     (3, 10, 16, 7, (3, 3, 3, 3), (1, 1), 0), (5, 9, 24, 3, (1, 1, 2, 3), (1, 1), 0)])
 def test_im2row_im2col_chunked(pkg, orc, gpu, dt, hwc, Ci, H, W, K, pad, stride, mod):
     """Patch matrices whose rows are not multiples of a 16-byte chunk (chunks straddle rows and columns), BASELINE
-    config 1 among them."""
+    config 1 among them; rows as wide as the image at unit strides (the column-major matrix as shifted copies of the
+    planes: 3x3, 5x5 and 7x7 filters, padding on one side only, more padding above and below than the filter needs)."""
     Co = 4
     Ho, Wo = (H - K + 1, W - K + 1) if mod else (hp.conv_out(H, K, pad[2], pad[3], stride[0]),
                                                 hp.conv_out(W, K, pad[0], pad[1], stride[1]))
