@@ -186,7 +186,7 @@ def main():
                      # WRITE_SIZE counter runs recorded in the profile summary of this workload; null when the
                      # batch differs or the kernel sources have changed since those runs
                      "traffic": traffic,
-                     "kernel": "ptl::gemm_plain_kernel / gemm_plain_pair_kernel<_Float16, 64x64 tile, 1024 threads>",
+                     "kernel": "ptl::gemm_plain_kernel<_Float16, 64x64 tile, 1024 threads> / gemm_plain_pair_mixed_kernel<_Float16> (128x64 and 64x64 tiles)",
                      "flops_per_launch": flops_step / 2, "launches_per_step": 2,
                      "avg_launch_us": round(launch_ms * 1e3, 3)},
     }

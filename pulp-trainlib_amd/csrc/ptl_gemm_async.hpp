@@ -22,6 +22,8 @@ int launch_plain(GemmArgs &g, hipStream_t s);
 
 template <typename T, int BM, int BN, int NT, int WMv, int WNv, int WKv, int NS, int G>
 int launch_plain_pair(GemmArgs &g0, GemmArgs &g1, hipStream_t s);
+template <typename T, int NS, int G>
+int launch_plain_pair_mixed(GemmArgs &g0, GemmArgs &g1, hipStream_t s);
 
 // Streaming kernel (A panel resident, column tiles streamed) for plain operands with K == KS slabs; -1 when
 // the product does not fit it.

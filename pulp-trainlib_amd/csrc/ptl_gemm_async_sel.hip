@@ -201,6 +201,12 @@ int gemm_async_pair(GemmArgs &g0, GemmArgs &g1) {
     }
     if (cfg[0] != cfg[1]) return -1;
     if (cfg[0] == 0) return launch_plain_pair<T, 128, 128, 512, 2, 2, 2, 3, 1>(g0, g1, st.stream);
+    // A first product with at most half the contraction of the second: tiles twice as large for it even the
+    // workgroups out; taken where that brings the launch down to one workgroup per CU.
+    auto tiles_of = [](const GemmArgs &g, int bm, int bn) { return (long)((g.N + bm - 1) / bm) * ((g.M + bn - 1) / bn); };
+    if (g0.K * 2 <= g1.K && g0.N % 128 == 0 && tiles_of(g0, 64, 64) + tiles_of(g1, 64, 64) > st.num_cu &&
+        tiles_of(g0, 128, 64) + tiles_of(g1, 64, 64) <= st.num_cu)
+        return launch_plain_pair_mixed<T, 3, 1>(g0, g1, st.stream);
     return launch_plain_pair<T, 64, 64, 1024, 2, 2, 4, 3, 1>(g0, g1, st.stream);
 }
 
