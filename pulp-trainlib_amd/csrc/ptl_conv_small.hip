@@ -48,6 +48,7 @@ struct ConvSmallArgs {
     // stats[(filter * ntiles + tile) * 4 + {0, 1}]; NULL: not wanted.  stats_off: bytes into LDS of the jobs' sums.
     float *stats;
     int stats_off, ntiles;
+    int ksplit, red_off;    // 1: the three filter rows of a job on three waves; bytes into LDS of their partial sums
     // per item: element offset into the sample (first channel, first tile row, column group), element offset into the
     // LDS tile, first tile row | first channel << 8 | column group << 16
     int item_g[CS_ITEMS], item_l[CS_ITEMS], item_rc[CS_ITEMS];
@@ -196,35 +197,8 @@ __device__ inline void conv_small_block(const ConvSmallArgs &a, int tile, char *
     const int npix = min(a.R, a.Ho - y0) * a.Wo, jobs = a.pgroups << a.mshift;
     const uint4 *T4 = reinterpret_cast<const uint4 *>(Tl);
     const size_t plane = (size_t)a.Ho * a.Wo;
-    for (int job = wave; job < jobs; job += CS_NT / 64) {
-        const int pg = job >> a.mshift, mb = job - (pg << a.mshift);
-        if (pg * 32 >= npix) break;
-        const int p = min(pg * 32 + lr, npix - 1);
-        const int py = fast_div(p, a.magic_wo), px = p - py * a.Wo;
-        const uint4 *prow = T4 + (py * a.TW + px) * a.s + kg * a.POS;
-        const char *frow = F + (mb * 32 + lr) * a.b_pitch + kg * 16;
-        f32x16 acc;
-#pragma unroll
-        for (int v = 0; v < 16; ++v) acc[v] = 0.f;
-        if (a.K == 1) {
-#pragma unroll
-            for (int ks = 0; ks < CINP / KSTEP; ++ks)
-                mfma_step<T>(acc, *reinterpret_cast<const uint4 *>(frow + ks * KSTEP * ES), prow[2 * ks * a.POS]);
-        } else
-#pragma unroll
-        for (int ks = 0; ks < CINP / KSTEP; ++ks) {
-            const uint4 *pk = prow + 2 * ks * a.POS;
-#pragma unroll
-            for (int ky = 0; ky < 3; ++ky) {
-                const uint4 *pr = pk + ky * a.TW;
-#pragma unroll
-                for (int kx = 0; kx < 3; ++kx) {
-                    const uint4 pf = pr[kx];
-                    const uint4 ff = *reinterpret_cast<const uint4 *>(frow + ((ky * 3 + kx) * CINP + ks * KSTEP) * ES);
-                    mfma_step<T>(acc, ff, pf);
-                }
-            }
-        }
+    // what a wave does with the finished sums of a job: store them, and add them up for the normalisation if asked
+    auto finish = [&](const f32x16 &acc, int job, int pg, int mb, int py, int px) {
         const int left = a.Cout - mb * 32 - 4 * kg;  // filters from this lane's first one
         if (pg * 32 + lr < npix) {
             T *out = reinterpret_cast<T *>(a.Y) + (((size_t)b * a.Cout + mb * 32 + 4 * kg) * a.Ho + y0 + py) * a.Wo + px;
@@ -259,6 +233,76 @@ __device__ inline void conv_small_block(const ConvSmallArgs &a, int tile, char *
                 S[job * 32 + f] = make_float2(s0[0] + o0, s1[0] + o1);
             }
         }
+    };
+    if (a.ksplit) {
+        // A single sample: tiles of one or two jobs on many CUs, and the three filter rows of a job on three waves
+        // (three SIMDs), whose sums meet in LDS.  A job's MFMAs keep one SIMD's matrix pipe busy for their whole
+        // length - in fp32, at two k values per instruction, 4 us for 32 channels - so fewer jobs per CU and
+        // a third of a job per SIMD is what shortens such a call (the split alone, with four jobs on a CU's four
+        // SIMDs, changes nothing).  Larger batches keep the order of summation they have at every batch size.
+        const int job = wave / 3, part = wave - 3 * job;
+        const int pg = job >> a.mshift, mb = job - (pg << a.mshift);
+        const bool active = job < jobs && pg * 32 < npix;
+        f32x16 acc;
+#pragma unroll
+        for (int v = 0; v < 16; ++v) acc[v] = 0.f;
+        int py = 0, px = 0;
+        if (active) {
+            const int p = min(pg * 32 + lr, npix - 1);
+            py = fast_div(p, a.magic_wo);
+            px = p - py * a.Wo;
+            const uint4 *prow = T4 + (py * a.TW + px) * a.s + kg * a.POS + part * a.TW;
+            const char *frow = F + (mb * 32 + lr) * a.b_pitch + kg * 16 + part * 3 * CINP * ES;
+#pragma unroll
+            for (int ks = 0; ks < CINP / KSTEP; ++ks) {
+                const uint4 *pr = prow + 2 * ks * a.POS;
+#pragma unroll
+                for (int kx = 0; kx < 3; ++kx)
+                    mfma_step<T>(acc, *reinterpret_cast<const uint4 *>(frow + (kx * CINP + ks * KSTEP) * ES), pr[kx]);
+            }
+        }
+        float *red = reinterpret_cast<float *>(smem + a.red_off);  // [job][filter row 1, 2][value][lane]
+        if (active && part) {
+#pragma unroll
+            for (int v = 0; v < 16; ++v) red[((job * 2 + part - 1) * 16 + v) * 64 + lane] = acc[v];
+        }
+        __syncthreads();
+        if (active && !part) {
+#pragma unroll
+            for (int v = 0; v < 16; ++v) acc[v] += red[(job * 2 * 16 + v) * 64 + lane] + red[((job * 2 + 1) * 16 + v) * 64 + lane];
+            finish(acc, job, pg, mb, py, px);
+        }
+    } else
+    for (int job = wave; job < jobs; job += CS_NT / 64) {
+        const int pg = job >> a.mshift, mb = job - (pg << a.mshift);
+        if (pg * 32 >= npix) break;
+        const int p = min(pg * 32 + lr, npix - 1);
+        const int py = fast_div(p, a.magic_wo), px = p - py * a.Wo;
+        const uint4 *prow = T4 + (py * a.TW + px) * a.s + kg * a.POS;
+        const char *frow = F + (mb * 32 + lr) * a.b_pitch + kg * 16;
+        f32x16 acc;
+#pragma unroll
+        for (int v = 0; v < 16; ++v) acc[v] = 0.f;
+        if (a.K == 1) {
+#pragma unroll
+            for (int ks = 0; ks < CINP / KSTEP; ++ks)
+                mfma_step<T>(acc, *reinterpret_cast<const uint4 *>(frow + ks * KSTEP * ES), prow[2 * ks * a.POS]);
+        } else
+#pragma unroll
+        for (int ks = 0; ks < CINP / KSTEP; ++ks) {
+            const uint4 *pk = prow + 2 * ks * a.POS;
+#pragma unroll
+            for (int ky = 0; ky < 3; ++ky) {
+                const uint4 *pr = pk + ky * a.TW;
+#pragma unroll
+                for (int kx = 0; kx < 3; ++kx) {
+                    const uint4 pf = pr[kx];
+                    const uint4 ff = *reinterpret_cast<const uint4 *>(frow + ((ky * 3 + kx) * CINP + ks * KSTEP) * ES);
+                    mfma_step<T>(acc, ff, pf);
+                }
+            }
+        }
+        finish(acc, job, pg, mb, py, px);
     }
     if (a.stats) {  // the jobs' sums of a filter added in job order: one partial per workgroup and filter
         __syncthreads();
@@ -705,7 +749,9 @@ int plan_small(const ConvTileDesc &d, const void *X, const void *Wt, void *Y, in
     // rows per workgroup: the whole image, halved while that leaves the four waves a job each and the chip is not full
     int R = d.Ho;
     auto jobs_of = [&](int r) { return ((r * d.Wo + 31) / 32) * mblocks; };
-    while ((long long)d.batch * ((d.Ho + R - 1) / R) < cu_budget && R % 2 == 0 && jobs_of(R / 2) >= 4) R /= 2;
+    // (a single sample: down to one job per workgroup, whose three filter rows then go to three waves - see ksplit)
+    const int min_jobs = d.batch == 1 && K == 3 ? 1 : 4;
+    while ((long long)d.batch * ((d.Ho + R - 1) / R) < cu_budget && R % 2 == 0 && jobs_of(R / 2) >= min_jobs) R /= 2;
     auto items_of = [&](int r) { return cblocks * (d.Win / VEC) * ((((r - 1) * s + K) + RPI - 1) / RPI); };
     auto lds_of = [&](int r) { return (size_t)cblocks * ((r - 1) * s + K) * TW * 16; };
     const int pitch = K * K * cinp * ES + 16;  // (an odd multiple of 16 bytes)
@@ -749,6 +795,13 @@ int plan_small(const ConvTileDesc &d, const void *X, const void *Wt, void *Y, in
     if (a.halo_chunks >= 65536 || a.RR * cblocks >= 65536) return -1;
     p.tiles = (int)tiles;
     p.lds = f_bytes + lds_of(R);
+    // a single sample: the filter rows of a job on separate waves, 8 KB of partial sums per job behind the tile
+    const int jobs = a.pgroups << a.mshift;
+    if (d.batch == 1 && K == 3 && 3 * jobs <= CS_WAVES && (p.lds + 15) / 16 * 16 + (size_t)jobs * 2 * 16 * 64 * sizeof(float) <= 150 * 1024) {
+        a.ksplit = 1;
+        a.red_off = (int)((p.lds + 15) / 16 * 16);
+        p.lds = a.red_off + (size_t)jobs * 2 * 16 * 64 * sizeof(float);
+    }
     p.cinp = cinp;
     p.per_thread = (a.f_chunks + CS_NT - 1) / CS_NT;
     if (p.per_thread > (cinp == 16 ? 2 : cinp == 32 ? 3 : 5)) return -1;
