@@ -170,23 +170,19 @@ __device__ inline void conv_small_block(const ConvSmallArgs &a, int tile, char *
             if (q < a.f_chunks) {
                 const int e0 = q * VEC;
                 const int outer = fast_div(e0, a.magic_inner9), rem = e0 - outer * a.f_inner * 9;
-                int inner = (rem * 7282) >> 16;  // rem / 9 for rem < 2^15
-                int tap = rem - inner * 9;
+                const int inner = (rem * 7282) >> 16;  // rem / 9 for rem < 2^15
+                const int tap = rem - inner * 9;
                 const int m = a.f_transposed ? inner : outer, c = a.f_transposed ? outer : inner;
-                int at = m * a.b_pitch + ((a.f_transposed ? 8 - tap : tap) * CINP + c) * ES;
+                const int at0 = m * a.b_pitch + ((a.f_transposed ? 8 - tap : tap) * CINP + c) * ES;
+                // a piece is shorter than the nine taps of a filter plane, so it crosses into the next plane at most
+                // once: its first n1 elements step through the taps from at0, the rest from the next plane's tap 0
+                const int n1 = 9 - tap;
+                const bool last = inner + 1 == a.f_inner;
+                const int next0 = at0 + n1 * step_tap + step_inner + (last ? step_outer : 0);
+                const int rest = next0 - n1 * step_tap;  // (element j >= n1 sits at rest + j * step_tap)
 #pragma unroll
-                for (int j = 0; j < VEC; ++j) {
-                    *reinterpret_cast<T *>(F + at) = fin[k].e[j];
-                    at += step_tap;
-                    if (++tap == 9) {
-                        tap = 0;
-                        at += step_inner;
-                        if (++inner == a.f_inner) {
-                            inner = 0;
-                            at += step_outer;
-                        }
-                    }
-                }
+                for (int j = 0; j < VEC; ++j)
+                    *reinterpret_cast<T *>(F + (j < n1 ? at0 : rest) + j * step_tap) = fin[k].e[j];
             }
         }
     }
