@@ -791,7 +791,7 @@ def test_linear_bias(pkg, orc, gpu, dt):
 
 # ---------------------------------------------------------------------- mm / mm_manager
 @pytest.mark.parametrize("dt", ["fp32", "fp16"])
-@pytest.mark.parametrize("n_in,n_out,ns", [(1024, 1024, 512), (256, 384, 640), (100, 37, 9), (64, 64, 1)])
+@pytest.mark.parametrize("n_in,n_out,ns", [(1024, 1024, 512), (1024, 1024, 384), (1024, 896, 320), (256, 384, 640), (100, 37, 9), (64, 64, 1)])
 def test_linear_bw_batched_matches_separate_steps(pkg, gpu, dt, n_in, n_out, ns):
     """ptl_linear_*_bw_batched (weight + input gradient in one call) against the two single steps."""
     nd = hp.np_dtype(dt)
