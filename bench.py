@@ -2,15 +2,18 @@
 
 One step = forward + weight gradient + input gradient of the Linear 1024 -> 1024 layer in fp16 (fp32
 accumulation) over a batch of 512 independent samples (BASELINE.json configs[1], batched mode), called through
-the C ABI of libptl_hip.so with every tensor already resident in HBM.  Prints ONE JSON line.
+the C ABI of libptl_hip.so with every tensor already resident in HBM.
 
-The line also carries
+The LAST line of stdout is one compact JSON object (a few KB at most) that carries
   * "roofline": the dominant kernel (the MFMA GEMM) priced against the dense fp16 MFMA peak, from HIP events
     recorded on the library's stream around the timed region;
   * "cpu_baseline": the CPU oracle (a port of the reference's C loops, OpenMP over the host cores) timed on a
     bounded sample of the same workload;
-  * "detail": per-step timings of the other BASELINE shapes (batch-1 latency and batched mode) with their own
-    roofline fractions, so the headline is not the only number on record.
+  * "targets": a handful of figures of the other BASELINE shapes (wide convolutions, a large plain product,
+    depthwise / pointwise at batch 64, the ResNet-20 step).
+Everything else -- the per-step timings of every other shape (batch-1 latency and batched mode) with their own
+roofline fractions, and the CPU port on every configuration -- is printed BEFORE it, one JSON object per line
+(`{"detail": {...}}`, `{"cpu_baseline_detail": {...}}`), and with --detail-file also written to a file.
 """
 import argparse
 import json
@@ -66,6 +69,8 @@ def main():
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--no-detail", action="store_true", help="skip the per-shape detail table")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
+    ap.add_argument("--detail-file", default=None,
+                    help="also write the headline, the CPU table and the detail table to this file as one JSON document")
     ap.add_argument("--helpers-only", action="store_true",
                     help="detail table: only the index / streaming helpers (for a counter run of those kernels alone)")
     ap.add_argument("--resnet-only", action="store_true",
@@ -164,6 +169,7 @@ def main():
 
     traffic, traffic_note = recorded_traffic(ns)
 
+    cpu_detail, detail = [], []
     result = {
         "metric": METRIC,
         "value": round(tflops, 3),
@@ -238,17 +244,68 @@ def main():
         result["cpu_baseline"] = {"value": round(cpu_tflops, 6), "unit": "TFLOP/s", "cores": cores, "kind": "port",
                                   "sample": "%d of the %d samples, FW+WG+IG %d times, fp16 with fp16 accumulation "
                                             "(the reference's arithmetic), %.2f s" % (m, ns, reps, t_cpu)}
-        result["cpu_baseline_detail"] = cpu_rows(pkg, orc, hp, cores)
+        cpu_detail = cpu_rows(pkg, orc, hp, cores)
 
     # ------------------------------------------------------------------------------ detail
     if args.helpers_only:
-        result["detail"] = helper_rows(pkg, lib, hp, timed, torch, dev)
+        detail = helper_rows(pkg, lib, hp, timed, torch, dev)
     elif args.resnet_only:
-        result["detail"] = resnet_rows(pkg, lib, timed, torch, dev)
+        detail = resnet_rows(pkg, lib, timed, torch, dev)
     elif not args.no_detail:
-        result["detail"] = detail_table(pkg, lib, hp, to_dev, timed, check, torch, dev)
+        detail = detail_table(pkg, lib, hp, to_dev, timed, check, torch, dev)
 
-    print(json.dumps(result))
+    lines = compose_output(result, cpu_detail, detail)
+    if args.detail_file:
+        with open(args.detail_file, "w") as f:
+            json.dump({"headline": result, "cpu_baseline_detail": cpu_detail, "detail": detail}, f, indent=1)
+    for line in lines:
+        print(line)
+    sys.stdout.flush()
+
+
+# (key of the "targets" block, workload names in the detail table -- matched as prefixes --, field reported)
+TARGET_ROWS = (
+    ("conv512_14x14_N256_FW_WG_IG_frac_of_mfma_peak",
+     ["conv2d 512->512 14x14 k3 p1 %s N=256" % s for s in ("FW", "WG", "IG")], "frac_of_bound"),
+    ("conv256_28x28_N256_FW_WG_IG_frac_of_mfma_peak",
+     ["conv2d 256->256 28x28 k3 p1 %s N=256" % s for s in ("FW", "WG", "IG")], "frac_of_bound"),
+    ("conv128_28x28_N512_FW_WG_IG_frac_of_mfma_peak",
+     ["conv2d 128->128 28x28 k3 p1 %s N=512" % s for s in ("FW", "WG", "IG")], "frac_of_bound"),
+    ("mm_4096x4096x4096_fp16_TFLOP/s", ["mm 4096x4096x4096 (B transposed)"], "TFLOP/s"),
+    ("depthwise_64x56x56_N64_FW_WG_IG_GB/s", ["depthwise 3x3 64x56x56 %s N=64" % s for s in ("FW", "WG", "IG")], "GB/s"),
+    ("pointwise_64to128_56x56_N64_FW_WG_IG_GB/s", ["pointwise 64->128 56x56 %s N=64" % s for s in ("FW", "WG", "IG")], "GB/s"),
+    ("mhsa_L197_E192_N32_FW_BW_us", ["mhsa L197 E192 3x64 %s N=32" % s for s in ("FW", "BW")], "us"),
+    ("resnet20_fp16_N128_step_samples/s",
+     ["resnet20 step with batch norm, element-wise layers fused into it FW+BW+SGD"], "samples/s"),
+)
+MAX_LAST_LINE = 4096
+
+
+def compose_output(result, cpu_detail, detail):
+    """The lines bench.py prints, in order: one JSON object per row of the CPU table and of the detail table, then
+    the headline object LAST, kept under MAX_LAST_LINE bytes so that a reader that only sees the tail of stdout
+    still gets it whole.  Strict JSON throughout (a NaN or an infinity raises)."""
+    lines = []
+    for row in cpu_detail or ():
+        lines.append(json.dumps({"cpu_baseline_detail": row}, allow_nan=False))
+    for row in detail or ():
+        lines.append(json.dumps({"detail": row}, allow_nan=False))
+    head = dict(result)
+    targets = {}
+    for key, names, field in TARGET_ROWS:
+        vals = []
+        for name in names:
+            hit = [row for row in detail or () if row["workload"].startswith(name) and field in row]
+            vals.append(hit[0][field] if hit else None)
+        if any(v is not None for v in vals):
+            targets[key] = vals if len(vals) > 1 else vals[0]
+    if targets:
+        head["targets"] = targets
+    last = json.dumps(head, allow_nan=False)
+    if len(last) >= MAX_LAST_LINE:
+        raise RuntimeError("headline line is %d bytes, limit %d" % (len(last), MAX_LAST_LINE))
+    lines.append(last)
+    return lines
 
 
 def cpu_rows(pkg, orc, hp, cores):

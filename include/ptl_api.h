@@ -134,6 +134,44 @@ void mm(void *matMul_args);
 void mm_M(void *matMul_args);
 void mm_fp16(void *matMul_args_fp16);
 void mm_M_fp16(void *matMul_args_fp16);
+/* The unrolled variants, by name (lib/include/pulp_matmul_fp32.h:72-244; lib/include/pulp_matmul_fp16.h:56-107):
+ * each computes the product of mm / mm_fp16; the reference's matmul harness calls them by name
+ * (tests/test_matmul/net.c:95-186). */
+void mm_u2(void *matMul_args);
+void mm_unroll_1x2(void *matMul_args);
+void mm_unroll_1x4(void *matMul_args);
+void mm_unroll_1x8(void *matMul_args);
+void mm_unroll_2x1(void *matMul_args);
+void mm_unroll_4x1(void *matMul_args);
+void mm_unroll_8x1(void *matMul_args);
+void mm_unroll_2x2(void *matMul_args);
+void mm_unroll_2x4(void *matMul_args);
+void mm_unroll_4x2(void *matMul_args);
+void mm_unroll_4x4(void *matMul_args);
+void mm_M_u2(void *matMul_args);
+void mm_M_unroll_2x1(void *matMul_args);
+void mm_M_unroll_4x1(void *matMul_args);
+void mm_M_unroll_8x1(void *matMul_args);
+void mm_M_unroll_1x2(void *matMul_args);
+void mm_M_unroll_1x4(void *matMul_args);
+void mm_M_unroll_1x8(void *matMul_args);
+void mm_M_unroll_2x2(void *matMul_args);
+void mm_M_unroll_4x2(void *matMul_args);
+void mm_M_unroll_2x4(void *matMul_args);
+void mm_M_unroll_4x4(void *matMul_args);
+void mm_fp16_SIMD_2x4(void *matMul_args_fp16);
+void mm_fp16_SIMD_4x8(void *matMul_args_fp16);
+void mm_fp16_unroll_8x1(void *matMul_args_fp16);
+void mm_fp16_unroll_4x1(void *matMul_args_fp16);
+void mm_fp16_unroll_2x1(void *matMul_args_fp16);
+void mm_M_fp16_SIMD_2x4(void *matMul_args_fp16);
+void mm_M_fp16_SIMD_4x8(void *matMul_args_fp16);
+/* Matrix x vector, C[i] = sum_k A[i*K+k] * B[k] (lib/include/pulp_matmul_fp16.h:118-135;
+ * lib/sources/pulp_matmul_fp16.c:1158): with M > 1 and trans_B set, M is the vector's length; with M > 1 and
+ * trans_B clear the reference stops the program, this library prints the same message and rejects the call. */
+void mv_fp16_SIMD_2x1(void *matMul_args_fp16);
+void mv_fp16_SIMD_4x1(void *matMul_args_fp16);
+void mv_fp16_SIMD_8x1(void *matMul_args_fp16);
 void mm_manager(void *mm_manager_args);
 void mm_manager_fp16(void *mm_manager_args_fp16);
 
@@ -236,8 +274,20 @@ const char *ptl_last_error(void);
  * 0 = ran, 1 = rejected its arguments (message printed, outputs untouched),
  * 2 = a HIP call failed. */
 int ptl_last_status(void);
-/* Stream on which kernels are enqueued (a hipStream_t); NULL = default. */
+/* Stream on which kernels are enqueued (a hipStream_t); NULL = default.  The stream being left is drained first
+ * (its kernels may still use the library's buffers).  Must not be called while that stream is being captured into
+ * a graph: the call is then refused (ptl_last_status() == 1, the stream stays); a drain that fails is reported
+ * with status 2 after the switch. */
 void ptl_set_stream(void *hip_stream);
+/* The library keeps two internal device buffers (partial sums of split contractions; blocked / padded / dilated
+ * copies) that grow when a call needs more - by synchronising the device, freeing and allocating, which is illegal
+ * while a stream is being captured and unwelcome in a steady-state loop.  ptl_reserve grows them to at least the
+ * given sizes now (0 = leave); ptl_reserved reports their present sizes, so a caller can run its shapes once,
+ * read the sizes and reserve them at start-up the next time.  A call that would have to grow a buffer while the
+ * library's stream is being captured fails with status 2 and an error text that names ptl_reserve, and the
+ * capture stays valid.  No counterpart in the reference (its callers own every buffer). */
+int ptl_reserve(size_t workspace_bytes, size_t scratch_bytes);
+void ptl_reserved(size_t *workspace_bytes, size_t *scratch_bytes);
 int ptl_sync(void);
 /* Kernel selection: 0 (default) = the fastest kernel that fits the problem
  * (direct convolution for large channel-major Conv2D forward / input-gradient
@@ -261,11 +311,14 @@ int ptl_sync(void);
  * the route of pointwise layers over a batch) (1) or a tile-per-workgroup
  * kernel (0); ptl_last_conv_resident() whether the last Conv2D call that took
  * the tap route kept its input tile in LDS (1), or ran the small-layer kernels
- * (2: forward, either gradient, or both gradients in one call). */
+ * (2: forward, either gradient, or both gradients in one call);
+ * ptl_last_gemm_tile() the output tile of the last product that ran a tile-per-workgroup kernel of the
+ * look-up-free pipelined GEMM, as rows * 1000 + columns (256256 = 256 x 256, 128064 = 128 x 64). */
 void ptl_set_gemm_path(int path);
 int ptl_last_conv_direct(void);
 int ptl_last_gemm_streamed(void);
 int ptl_last_conv_resident(void);
+int ptl_last_gemm_tile(void);
 /* hipEvent timing on the library stream: begin records, end records,
  * synchronises and returns the elapsed milliseconds (negative on error). */
 int ptl_timer_begin(void);

@@ -17,6 +17,13 @@ INCLUDE_DIR = os.path.join(os.path.dirname(_HERE), "include")
 
 _lib = None
 
+# The reference's hand-unrolled matmul variants (pulp_matmul_fp32.h:72-244, pulp_matmul_fp16.h:56-135), exported by name.
+MM_VARIANTS_FP32 = ["mm_u2"] + ["mm_unroll_%s" % u for u in ("1x2", "1x4", "1x8", "2x1", "4x1", "8x1", "2x2", "2x4", "4x2", "4x4")] + [
+    "mm_M_u2"] + ["mm_M_unroll_%s" % u for u in ("2x1", "4x1", "8x1", "1x2", "1x4", "1x8", "2x2", "4x2", "2x4", "4x4")]
+MM_VARIANTS_FP16 = ["mm_fp16_SIMD_2x4", "mm_fp16_SIMD_4x8", "mm_fp16_unroll_8x1", "mm_fp16_unroll_4x1",
+                    "mm_fp16_unroll_2x1", "mm_M_fp16_SIMD_2x4", "mm_M_fp16_SIMD_4x8"]
+MV_VARIANTS_FP16 = ["mv_fp16_SIMD_2x1", "mv_fp16_SIMD_4x1", "mv_fp16_SIMD_8x1"]
+
 # Reference-named `void f(void *args)` entry points exported by the library.
 VOID_ENTRY_POINTS = [
     "pulp_conv2d_fp32_fw_cl", "pulp_conv2d_fp32_bw_cl", "pulp_conv2d_fp32_bw_param_grads_cl",
@@ -40,6 +47,7 @@ VOID_ENTRY_POINTS = [
 ] + ["naive_conv2d_%s_kernel_CHW_k%dx%d_s2_p1%s" % (step, k, k, sfx) for sfx in ("", "_fp16") for k in (3, 5)
      for step in ("fw", "param_grad", "in_grad")] + [
     "mm_bias_add_transposed", "mm_bias_add_transposed_fp16",
+] + MM_VARIANTS_FP32 + MM_VARIANTS_FP16 + MV_VARIANTS_FP16 + [
     "dw_kernel_forward", "dw_kernel_weight_grad", "dw_kernel_input_grad", "dw_kernel_forward_fp16",
     "dw_kernel_weight_grad_fp16", "dw_kernel_input_grad_fp16",
     "pulp_im2row_fp32", "pulp_im2col_fp32", "pulp_blocktransp_fp32", "pulp_im2row_fp16", "pulp_im2col_fp16",
@@ -57,6 +65,8 @@ VOID_ENTRY_POINTS = [
     "pulp_CrossEntropyLoss_backward_fp16", "pulp_gradient_descent_fp32", "pulp_gradient_descent_fp16",
     "pulp_batch_norm_fp32_fw_cl", "pulp_batch_norm_parallelized_fp32_fw_cl",
 ]
+
+
 
 # `int f(const args *, int nsamples, int step)` batched launchers of the layers around the matmul core.
 STEP_ENTRY_POINTS = ["ptl_%s_%s_batched" % (n, dt) for n in ("relu", "residual", "avgpool", "cross_entropy")
@@ -92,7 +102,8 @@ STATS_ENTRY_POINTS = ["ptl_conv2d_%s_fw_batched_stats" % dt for dt in ("fp16", "
                      ["ptl_batch_norm_fused_%s_fw_stats" % dt for dt in ("fp16", "fp32")]
 
 OTHER_ENTRY_POINTS = ["ptl_init", "ptl_last_error", "ptl_last_status", "ptl_set_stream", "ptl_sync", "ptl_set_gemm_path",
-                      "ptl_last_conv_direct", "ptl_last_gemm_streamed", "ptl_last_conv_resident", "ptl_timer_begin", "ptl_timer_end_ms", "ptl_mm_fp32", "ptl_mm_fp16", "ptl_copy_bytes"]
+                      "ptl_last_conv_direct", "ptl_last_gemm_streamed", "ptl_last_conv_resident", "ptl_last_gemm_tile", "ptl_timer_begin", "ptl_timer_end_ms", "ptl_mm_fp32", "ptl_mm_fp16", "ptl_copy_bytes",
+                      "ptl_reserve", "ptl_reserved"]
 
 
 def load():
@@ -162,6 +173,8 @@ def load():
     lib.ptl_last_gemm_streamed.restype = ctypes.c_int
     lib.ptl_last_conv_resident.argtypes = []
     lib.ptl_last_conv_resident.restype = ctypes.c_int
+    lib.ptl_last_gemm_tile.argtypes = []
+    lib.ptl_last_gemm_tile.restype = ctypes.c_int
     lib.ptl_sync.argtypes = []
     lib.ptl_sync.restype = ctypes.c_int
     lib.ptl_timer_begin.argtypes = []
@@ -174,6 +187,10 @@ def load():
         f.restype = ctypes.c_int
     lib.ptl_copy_bytes.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_long]
     lib.ptl_copy_bytes.restype = ctypes.c_int
+    lib.ptl_reserve.argtypes = [ctypes.c_size_t, ctypes.c_size_t]
+    lib.ptl_reserve.restype = ctypes.c_int
+    lib.ptl_reserved.argtypes = [ctypes.POINTER(ctypes.c_size_t), ctypes.POINTER(ctypes.c_size_t)]
+    lib.ptl_reserved.restype = None
     _lib = lib
     return lib
 

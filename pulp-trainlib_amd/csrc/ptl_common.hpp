@@ -141,6 +141,7 @@ struct State {
     int last_gemm_streamed = 0;  // 1 if the last pipelined GEMM ran the streaming kernel
     int last_conv_resident = 0;  // 1 if the last Conv2D forward / input-gradient call kept its input tile in LDS for all taps
     int last_conv_direct = 0;  // 1 if the last Conv2D forward / input-gradient call ran the direct kernel
+    int last_gemm_tile = 0;    // rows * 1000 + columns of the tile of the last look-up-free pipelined product
 };
 
 State &state();

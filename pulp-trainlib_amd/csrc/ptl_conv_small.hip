@@ -215,7 +215,7 @@ __device__ inline void conv_small_block(const ConvSmallArgs &a, int tile, char *
             // out as sums nobody reads)
             const bool pix_ok = pg * 32 + lr < npix;
 #pragma unroll
-            for (int v = 0; v < 16; ++v) s0[v] = pix_ok ? acc[v] : 0.f;
+            for (int v = 0; v < 16; ++v) s0[v] = pix_ok ? (float)(T)acc[v] : 0.f;  // the value as stored
 #pragma unroll
             for (int v = 0; v < 16; ++v) s1[v] = s0[v] * s0[v];
             stats_fold<8, 0x140>(s0, s1, (lr & 8) != 0);

@@ -39,6 +39,8 @@ class Stager {
     bool failed() const { return failed_; }
     bool rejected() const { return rejected_; }  // failed because of the arguments, not because of HIP
     int finish(int rc);
+    // Gives the staging buffers back without copying anything out (the kernels they were mapped for did not run).
+    void discard();
 
    private:
     struct Item {

@@ -673,7 +673,7 @@ static int conv2d_bw(const Args *a, int ns, const char *fn) {
                 const T *Wt = sg.in(reinterpret_cast<const T *>(a->coeff->data), (size_t)g.Co * K);
                 T *dW = sg.out(reinterpret_cast<T *>(a->coeff->diff), (size_t)g.Co * K);
                 T *dX = sg.out(reinterpret_cast<T *>(a->input->diff), in_n);
-                if (sg.failed()) return 2;
+                if (sg.failed()) return sg.rejected() ? 1 : 2;
                 state().last_conv_direct = 0;
                 state().last_conv_resident = 0;
                 // (a host tensor's gradient is a staging copy that this call copies back: its sums cannot wait)
@@ -684,7 +684,9 @@ static int conv2d_bw(const Args *a, int ns, const char *fn) {
                     if (rc == 0) state().last_conv_direct = 1;
                     return sg.finish(rc);
                 }
-                sg.finish(0);
+                // neither kernel took the layer: nothing was written, so nothing of the staged gradients goes back
+                // to the caller; the two single-step calls below are the only writers
+                sg.discard();
             }
         }
     }

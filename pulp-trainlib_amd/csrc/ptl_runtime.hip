@@ -82,13 +82,28 @@ bool ensure_init() {
     return init_device(dev) == 0;
 }
 
+// True while the library's stream records into a HIP graph: synchronising, freeing and allocating are illegal then
+// (each of them would invalidate the capture).
+static bool stream_is_capturing(hipStream_t s) {
+    hipStreamCaptureStatus status = hipStreamCaptureStatusNone;
+    if (hipStreamIsCapturing(s, &status) != hipSuccess) {
+        (void)hipGetLastError();
+        return false;
+    }
+    return status != hipStreamCaptureStatusNone;
+}
+
 static void *grow(void *&buf, size_t &have, size_t want, const char *what) {
     if (want <= have) return buf;
     State &st = state();
+    if (stream_is_capturing(st.stream)) {
+        set_error("%s: %zu bytes are needed and %zu are there, and the stream is being captured into a graph; call "
+                  "ptl_reserve() or run this shape once before the capture begins", what, want, have);
+        return nullptr;
+    }
     if (buf) {
         // kernels enqueued earlier - on this stream or on one the caller selected before - may still read the
         // old buffer
-        (void)st;
         if (!hip_ok(hipDeviceSynchronize(), "hipDeviceSynchronize")) return nullptr;
         (void)hipFree(buf);
         buf = nullptr;
@@ -236,6 +251,15 @@ void *Stager::map(const void *host_or_dev, size_t bytes, bool copy_in, bool copy
     return hit->dev;
 }
 
+void Stager::discard() {
+    if (items_.empty()) return;
+    // copies into the buffers may still be in flight
+    (void)hipStreamSynchronize(state().stream);
+    for (auto &t : items_)
+        if (t.dev) stage_release(t.dev);
+    items_.clear();
+}
+
 int Stager::finish(int rc) {
     if (items_.empty()) return failed_ ? 2 : rc;
     State &st = state();
@@ -260,18 +284,52 @@ int ptl_init(int device) { return ptl::init_device(device); }
 const char *ptl_last_error(void) { return ptl::last_error(); }
 int ptl_last_status(void) { return ptl::last_status(); }
 // Work already enqueued on the stream being left may still use the library's workspace; the next call would
-// write it from the new stream, so the old stream is drained first (a no-op when it is idle).
+// write it from the new stream, so the old stream is drained first (a no-op when it is idle).  A stream that is
+// being captured cannot be drained: the switch is refused then (status 1, the stream stays), and a drain that
+// fails (a destroyed handle) is reported the same way after the switch.
 void ptl_set_stream(void *s) {
     ptl::State &st = ptl::state();
     hipStream_t next = static_cast<hipStream_t>(s);
-    if (st.ready && next != st.stream) (void)hipStreamSynchronize(st.stream);
+    ptl::set_status(0);
+    if (st.ready && next != st.stream) {
+        if (ptl::stream_is_capturing(st.stream)) {
+            ptl::set_error("ptl_set_stream: the current stream is being captured into a graph; switch streams "
+                           "before the capture begins or after it ends");
+            ptl::set_status(1);
+            return;
+        }
+        hipError_t e = hipStreamSynchronize(st.stream);
+        if (e != hipSuccess) {
+            (void)hipGetLastError();
+            ptl::set_error("ptl_set_stream: draining the previous stream failed (%s)", hipGetErrorString(e));
+            ptl::set_status(2);
+        }
+    }
     st.stream = next;
+}
+
+// Grows the two internal buffers (partial sums; blocked / padded copies) to at least the given sizes now, so that
+// no later call has to: callers that capture the library's launches into a graph, or that may not allocate in
+// their steady state, reserve once after ptl_init.  ptl_reserved reports the present sizes (after a warm-up pass
+// over the caller's shapes they are the sizes those shapes need).
+int ptl_reserve(size_t workspace_bytes, size_t scratch_bytes) {
+    if (!ptl::ensure_init()) return 2;
+    if (workspace_bytes && !ptl::workspace(workspace_bytes)) return 2;
+    if (scratch_bytes && !ptl::scratch(scratch_bytes)) return 2;
+    return 0;
+}
+
+void ptl_reserved(size_t *workspace_bytes, size_t *scratch_bytes) {
+    ptl::State &st = ptl::state();
+    if (workspace_bytes) *workspace_bytes = st.ws_bytes;
+    if (scratch_bytes) *scratch_bytes = st.scratch_bytes;
 }
 
 void ptl_set_gemm_path(int path) { ptl::state().gemm_path = path; }
 int ptl_last_conv_direct(void) { return ptl::state().last_conv_direct; }
 int ptl_last_gemm_streamed(void) { return ptl::state().last_gemm_streamed; }
 int ptl_last_conv_resident(void) { return ptl::state().last_conv_resident; }
+int ptl_last_gemm_tile(void) { return ptl::state().last_gemm_tile; }
 
 int ptl_sync(void) {
     if (!ptl::ensure_init()) return 2;

@@ -238,6 +238,45 @@ void mm_M(void *p) { ptl_internal_set_status(mm32((const struct matMul_args *)p)
 void mm_fp16(void *p) { ptl_internal_set_status(mm16((const struct matMul_args_fp16 *)p)); }
 void mm_M_fp16(void *p) { ptl_internal_set_status(mm16((const struct matMul_args_fp16 *)p)); }
 
+/* The hand-unrolled variants (lib/include/pulp_matmul_fp32.h:72-244, pulp_matmul_fp16.h:56-107): the same
+ * product as mm / mm_fp16, with loops unrolled over rows and columns for the cluster's cores and, in fp16,
+ * two-element SIMD partial sums.  On the GPU they are one product, so every name lands on the same launcher;
+ * the reference's harness calls them by name (tests/test_matmul/net.c:95-186). */
+#define PTL_MM32_ALIAS(name) void name(void *p) { ptl_internal_set_status(mm32((const struct matMul_args *)p)); }
+#define PTL_MM16_ALIAS(name) void name(void *p) { ptl_internal_set_status(mm16((const struct matMul_args_fp16 *)p)); }
+PTL_MM32_ALIAS(mm_u2)
+PTL_MM32_ALIAS(mm_unroll_1x2) PTL_MM32_ALIAS(mm_unroll_1x4) PTL_MM32_ALIAS(mm_unroll_1x8)
+PTL_MM32_ALIAS(mm_unroll_2x1) PTL_MM32_ALIAS(mm_unroll_4x1) PTL_MM32_ALIAS(mm_unroll_8x1)
+PTL_MM32_ALIAS(mm_unroll_2x2) PTL_MM32_ALIAS(mm_unroll_2x4) PTL_MM32_ALIAS(mm_unroll_4x2)
+PTL_MM32_ALIAS(mm_unroll_4x4)
+PTL_MM32_ALIAS(mm_M_u2)
+PTL_MM32_ALIAS(mm_M_unroll_2x1) PTL_MM32_ALIAS(mm_M_unroll_4x1) PTL_MM32_ALIAS(mm_M_unroll_8x1)
+PTL_MM32_ALIAS(mm_M_unroll_1x2) PTL_MM32_ALIAS(mm_M_unroll_1x4) PTL_MM32_ALIAS(mm_M_unroll_1x8)
+PTL_MM32_ALIAS(mm_M_unroll_2x2) PTL_MM32_ALIAS(mm_M_unroll_4x2) PTL_MM32_ALIAS(mm_M_unroll_2x4)
+PTL_MM32_ALIAS(mm_M_unroll_4x4)
+PTL_MM16_ALIAS(mm_fp16_SIMD_2x4) PTL_MM16_ALIAS(mm_fp16_SIMD_4x8)
+PTL_MM16_ALIAS(mm_fp16_unroll_8x1) PTL_MM16_ALIAS(mm_fp16_unroll_4x1) PTL_MM16_ALIAS(mm_fp16_unroll_2x1)
+PTL_MM16_ALIAS(mm_M_fp16_SIMD_2x4) PTL_MM16_ALIAS(mm_M_fp16_SIMD_4x8)
+
+/* Matrix x vector (lib/sources/pulp_matmul_fp16.c:1158-1176 and the 4x1 / 8x1 twins): C[i] = sum_k A[i*K+k] B[k].
+ * With M > 1 the reference takes M as the vector's length when trans_B is set and stops otherwise ("second
+ * tensor is not a vector", exit(1)); here that call is rejected with the same message and C is left alone. */
+static int mv16(const struct matMul_args_fp16 *a) {
+    if (!a) return 1;
+    int K = a->K;
+    if (a->M > 1) {
+        if (!a->trans_B) {
+            printf("\nError: second tensor is not a vector.\n");
+            return 1;
+        }
+        K = a->M;
+    }
+    return ptl_mm_fp16(a->A, a->B, a->C, a->N, 1, K, 1);
+}
+void mv_fp16_SIMD_2x1(void *p) { ptl_internal_set_status(mv16((const struct matMul_args_fp16 *)p)); }
+void mv_fp16_SIMD_4x1(void *p) { ptl_internal_set_status(mv16((const struct matMul_args_fp16 *)p)); }
+void mv_fp16_SIMD_8x1(void *p) { ptl_internal_set_status(mv16((const struct matMul_args_fp16 *)p)); }
+
 /* Selection checks of mm_manager (lib/sources/pulp_train_utils_fp32.c:1347-1669):
  * layer in {CONV2D, PW_CONV, LINEAR}, step in {FW, WGT_GRAD, IN_GRAD}, id within
  * the list.  Returns 0 when a matmul would have been selected. */

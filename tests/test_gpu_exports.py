@@ -183,6 +183,55 @@ def test_mm_M_and_manager_bias_epilogue(pkg, orc, gpu, dt, N, M, K):
             m.C = pkg.addr(gC)
 
 
+def test_every_unrolled_matmul_variant_by_name(pkg, orc, gpu):
+    """The hand-unrolled mm variants the reference's matmul harness forks by name (tests/test_matmul/net.c:95-186;
+    lib/include/pulp_matmul_fp32.h:72-244, pulp_matmul_fp16.h:56-107): on the harness's closed-form operands
+    (tests/test_matmul/utils/GM.py:81-93, 32x32x32) and on a ragged product, both orientations of B, each against the
+    oracle's mm."""
+    for dt, names in (("fp32", ["mm", "mm_M"] + pkg.MM_VARIANTS_FP32), ("fp16", ["mm_fp16", "mm_M_fp16"] + pkg.MM_VARIANTS_FP16)):
+        nd = hp.np_dtype(dt)
+        assert len(names) == (24 if dt == "fp32" else 9)
+        i, j = np.meshgrid(np.arange(32), np.arange(32), indexing="ij")
+        cases = [(((1.0 + (i + j + 0.1)) / 1e3).astype(nd), ((i * j + 0.1) / 64).astype(nd)),
+                 (hp.uniform(0xC0DE0341, (50, 39), dtype=nd), hp.uniform(0xC0DE0342, (39, 70), dtype=nd))]
+        for A, B in cases:
+            (N, K), M = A.shape, B.shape[1]
+            for tb in (0, 1):
+                Bm = np.ascontiguousarray(B.T) if tb else B
+                C = np.zeros((N, M), nd)
+                orc.call("orc_mm", dt, hp.mm_args(pkg, A, Bm, C, N, M, K, tb))
+                assert rel_l2(C, A.astype(np.float64) @ B.astype(np.float64)) <= TOL[dt]
+                gA, gB = dev(A), dev(Bm)
+                for name in names:
+                    gC = dev(np.full((N, M), 3, nd))
+                    pkg.call(name, hp.mm_args(pkg, gA, gB, gC, N, M, K, tb))
+                    sync(gpu)
+                    assert rel_l2(host(gC), C) <= TOL[dt], (name, tb)
+
+
+def test_matrix_vector_variants_by_name(pkg, orc, gpu):
+    """mv_fp16_SIMD_{2,4,8}x1 (lib/sources/pulp_matmul_fp16.c:1158): C[i] = sum_k A[i][k] B[k]; with M > 1 and
+    trans_B set M is the vector's length; with M > 1 and trans_B clear the call is refused and C stays."""
+    N, K = 37, 130
+    A = hp.normal(0xC0DE0343, (N, K), 1.0 / np.sqrt(K), np.float16)
+    B = hp.uniform(0xC0DE0344, (K,), dtype=np.float16)
+    C = np.zeros((N, 1), np.float16)
+    orc.call("orc_mm", "fp16", hp.mm_args(pkg, A, B, C, N, 1, K, 0))
+    assert rel_l2(C[:, 0], A.astype(np.float64) @ B.astype(np.float64)) <= 1e-2
+    gA, gB = dev(A), dev(B)
+    for name in pkg.MV_VARIANTS_FP16:
+        for (M, Kf, tb) in ((1, K, 0), (1, K, 1), (K, 5, 1)):  # (the last: K taken from M)
+            gC = dev(np.full((N,), 3, np.float16))
+            pkg.call(name, hp.mm_args(pkg, gA, gB, gC, N, M, Kf, tb))
+            sync(gpu)
+            assert rel_l2(host(gC), C[:, 0]) <= 1e-2, (name, M, tb)
+        gC = dev(np.full((N,), 3, np.float16))
+        with pytest.raises(RuntimeError):
+            pkg.call(name, hp.mm_args(pkg, gA, gB, gC, N, K, 5, 0))
+        sync(gpu)
+        assert torch.all(gC == 3)
+
+
 @pytest.mark.parametrize("hwc", [0, 1])
 def test_im2col_conv2d_kernels_by_name(pkg, orc, gpu, hwc):
     """im2col_conv2d_fw_kernel = product + per-output-channel bias (rows of C in CHW, columns in HWC);

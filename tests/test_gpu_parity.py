@@ -867,6 +867,23 @@ def test_mm_fp16_large_and_tall_tiles(pkg, gpu, N, M, K):
         assert float((C.float() - ref).abs().max()) <= 2e-2
 
 
+@pytest.mark.parametrize("N,M,K", [(4096, 4096, 512), (4100, 4090, 192)])
+def test_mm_fp16_square_tiles_with_chunked_epilogue(pkg, gpu, N, M, K):
+    """fp16 products with more than 256 tall tiles take the 256x256 tile, whose accumulators are parked and stored
+    in four passes; whole and ragged, both orientations of B, against torch in float32."""
+    g = torch.Generator(device="cpu").manual_seed(23)
+    A = (torch.randn(N, K, generator=g) / 8).half().to(DEV)
+    for tb in (0, 1):
+        B = (torch.randn((M, K) if tb else (K, M), generator=g) / 8).half().to(DEV)
+        C = torch.full((N, M), 3, dtype=torch.float16, device=DEV)
+        pkg.call("mm_fp16", hp.mm_args(pkg, A, B, C, N, M, K, tb))
+        sync(gpu)
+        assert gpu.ptl_last_gemm_tile() == 256 * 1000 + 256, gpu.ptl_last_gemm_tile()
+        ref = A.float() @ (B.float().t() if tb else B.float())
+        assert float((C.float() - ref).norm() / ref.norm()) <= 1e-3
+        assert float((C.float() - ref).abs().max()) <= 2e-2
+
+
 def test_mm_k0_leaves_output_untouched(pkg, gpu):
     gA, gB, gC = dev(np.zeros((3, 1), np.float32)), dev(np.zeros((1, 4), np.float32)), dev(np.full((3, 4), 5, np.float32))
     pkg.call("mm", hp.mm_args(pkg, gA, gB, gC, 3, 4, 0, 0))

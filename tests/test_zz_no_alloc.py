@@ -48,6 +48,32 @@ def test_noalloc_depthwise_weight_gradient_matches_allocating_entry_point(pkg, g
         assert hp.rel_l2(b, ref) <= 1e-3, case
 
 
+def test_noalloc_entry_point_called_first_allocates_no_device_memory(pkg, gpu):
+    """The allocation-free entry point on a geometry that no allocating call has prepared: free device memory is
+    the same before and after, the result is right, and only then the allocating twin runs (bit-identical)."""
+    C, H, W, K, ns = 20, 44, 52, 3, 7
+    Ho, Wo = H - K + 1, W - K + 1
+    x = dev(hp.uniform(0xC0DE0710, (ns, C, H, W), dtype=np.float16))
+    dy = dev(hp.uniform(0xC0DE0711, (ns, C, Ho, Wo), dtype=np.float16))
+    dw = dev(np.full((C, K, K), 3, np.float16))
+    dw2 = dev(np.full((C, K, K), 3, np.float16))
+    ref = torch.nn.grad.conv2d_weight(x.float().reshape(1, ns * C, H, W), (ns * C, 1, K, K),
+                                      dy.float().reshape(1, ns * C, Ho, Wo), groups=ns * C)
+    ref = ref.reshape(ns, C, K, K).sum(0).cpu().numpy()
+    a, keep = hp.dw_args(pkg, "fp16", x, None, None, dw, None, dy, C, H, W, K, K, Ho, Wo)
+    torch.cuda.synchronize()
+    free0, _ = torch.cuda.mem_get_info()
+    pkg.call("ptl_conv_dw_fp16_wg_noalloc", a, ns)
+    assert gpu.ptl_sync() == 0, gpu.ptl_last_error().decode()
+    free1, _ = torch.cuda.mem_get_info()
+    assert free1 == free0, (free0, free1)
+    assert hp.rel_l2(dw.cpu().numpy(), ref) <= 1e-3
+    a2, keep2 = hp.dw_args(pkg, "fp16", x, None, None, dw2, None, dy, C, H, W, K, K, Ho, Wo)
+    pkg.call("ptl_conv_dw_fp16_wg_batched", a2, ns)
+    assert gpu.ptl_sync() == 0
+    assert torch.equal(dw, dw2)
+
+
 def test_noalloc_rejections_leave_the_output_untouched(pkg, gpu):
     C, H, K, ns = 8, 12, 3, 2
     x = hp.uniform(1, (ns, C, H, H), dtype=np.float16)
