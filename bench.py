@@ -277,6 +277,10 @@ TARGET_ROWS = (
     ("mhsa_L197_E192_N32_FW_BW_us", ["mhsa L197 E192 3x64 %s N=32" % s for s in ("FW", "BW")], "us"),
     ("resnet20_fp16_N128_step_samples/s",
      ["resnet20 step with batch norm, element-wise layers fused into it FW+BW+SGD"], "samples/s"),
+    ("mm_4096_fp16_random_then_zero_operands_TFLOP/s",
+     ["power: mm 4096x4096x4096 (B transposed), random", "power: mm 4096x4096x4096 (B transposed), zero"], "TFLOP/s"),
+    ("mm_4096_fp16_random_then_zero_operands_board_W",
+     ["power: mm 4096x4096x4096 (B transposed), random", "power: mm 4096x4096x4096 (B transposed), zero"], "W"),
 )
 MAX_LAST_LINE = 4096
 
@@ -306,6 +310,89 @@ def compose_output(result, cpu_detail, detail):
         raise RuntimeError("headline line is %d bytes, limit %d" % (len(last), MAX_LAST_LINE))
     lines.append(last)
     return lines
+
+
+class PowerSampler:
+    """Board power from the amdgpu hwmon node (microwatts in power1_input / power1_average), read every 10 ms on a
+    thread while a workload runs.  None when the node is not there."""
+
+    def __init__(self):
+        import glob
+        self.path = self.cap = None
+        for h in sorted(glob.glob("/sys/class/drm/card*/device/hwmon/hwmon*")):
+            for n in ("power1_input", "power1_average"):
+                if self.path is None and os.path.exists(os.path.join(h, n)):
+                    self.path = os.path.join(h, n)
+                    try:
+                        self.cap = int(open(os.path.join(h, "power1_cap")).read()) / 1e6
+                    except (OSError, ValueError):
+                        self.cap = None
+
+    def run(self, fn, sync, secs=1.0):
+        """Calls fn back to back for `secs` seconds; returns (microseconds per call, mean watts over the last two
+        thirds of the samples or None)."""
+        import threading
+        for _ in range(3):
+            fn()
+        sync()
+        samples, stop = [], [False]
+
+        def loop():
+            while not stop[0]:
+                try:
+                    samples.append(int(open(self.path).read()) / 1e6)
+                except (OSError, ValueError):
+                    pass
+                time.sleep(0.01)
+        th = threading.Thread(target=loop) if self.path else None
+        if th:
+            th.start()
+        t0, n = time.perf_counter(), 0
+        while time.perf_counter() - t0 < secs:
+            for _ in range(20):
+                fn()
+            sync()
+            n += 20
+        dt = time.perf_counter() - t0
+        stop[0] = True
+        if th:
+            th.join()
+        tail = samples[len(samples) // 3:]
+        return dt / n * 1e6, (sum(tail) / len(tail) if tail else None)
+
+
+def power_rows(pkg, lib, hp, check, torch, dev):
+    """The same launches on random and on all-zero operands, with the board power read beside them.  On random
+    operands the matrix kernels run against the board's power limit (the clock drops until the power fits), on zeros
+    they do not: the difference is what the limit, not the kernel's pipeline, takes."""
+    import ctypes
+    rows = []
+    ps = PowerSampler()
+    sync = torch.cuda.synchronize
+    N = 4096
+    ns, Ci, Co, H = 256, 512, 512, 14
+    for kind in ("random", "zero"):
+        def mk(*shape):
+            if kind == "zero":
+                return torch.zeros(*shape, device=dev, dtype=torch.float16)
+            return (torch.rand(*shape, device=dev) - 0.5).to(torch.float16)
+        A, Bm, Cm = mk(N, N), mk(N, N), torch.zeros(N, N, device=dev, dtype=torch.float16)
+        margs = [ctypes.c_void_p(A.data_ptr()), ctypes.c_void_p(Bm.data_ptr()), ctypes.c_void_p(Cm.data_ptr()), N, N, N, 1]
+        us, w = ps.run(lambda: check(lib.ptl_mm_fp16(*margs)), sync)
+        rows.append({"workload": "power: mm 4096x4096x4096 (B transposed), %s operands" % kind, "dtype": "fp16",
+                     "us": round(us, 2), "TFLOP/s": round(2.0 * N ** 3 / us / 1e6, 1),
+                     "W": None if w is None else round(w), "cap_W": ps.cap})
+        del A, Bm, Cm
+        x, wt = mk(ns, Ci, H, H), mk(Co, Ci, 3, 3)
+        y = torch.zeros(ns, Co, H, H, device=dev, dtype=torch.float16)
+        a, keep = hp.conv2d_args(pkg, x, None, wt, None, y, None, Ci, H, H, Co, 3, 3, H, H, (1, 1, 1, 1))
+        ref = ctypes.byref(a)
+        us, w = ps.run(lambda: check(lib.ptl_conv2d_fp16_fw_batched(ref, ns)), sync)
+        rows.append({"workload": "power: conv2d 512->512 14x14 k3 p1 FW N=256, %s operands" % kind, "dtype": "fp16",
+                     "us": round(us, 2), "TFLOP/s": round(2.0 * ns * Co * Ci * 9 * H * H / us / 1e6, 1),
+                     "W": None if w is None else round(w), "cap_W": ps.cap})
+        del x, wt, y
+    return rows
 
 
 def cpu_rows(pkg, orc, hp, cores):
@@ -597,6 +684,7 @@ def detail_table(pkg, lib, hp, to_dev, timed, check, torch, dev):
 
     rows += helper_rows(pkg, lib, hp, timed, torch, dev)
     rows += resnet_rows(pkg, lib, timed, torch, dev)
+    rows += power_rows(pkg, lib, hp, check, torch, dev)
     return rows
 
 

@@ -867,7 +867,7 @@ def test_mm_fp16_large_and_tall_tiles(pkg, gpu, N, M, K):
         assert float((C.float() - ref).abs().max()) <= 2e-2
 
 
-@pytest.mark.parametrize("N,M,K", [(4096, 4096, 512), (4100, 4090, 192)])
+@pytest.mark.parametrize("N,M,K", [(4096, 4096, 512), (4090, 4000, 192)])
 def test_mm_fp16_square_tiles_with_chunked_epilogue(pkg, gpu, N, M, K):
     """fp16 products with more than 256 tall tiles take the 256x256 tile, whose accumulators are parked and stored
     in four passes; whole and ragged, both orientations of B, against torch in float32."""
