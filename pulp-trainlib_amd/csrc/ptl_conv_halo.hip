@@ -279,6 +279,273 @@ int launch_halo_pipe(const HaloArgs &a, int grid, hipStream_t stream) {
 
 
 // ---------------------------------------------------------------------------------------------------------
+// Channel-minor (HWC) tensors, read in place: X[b][y][x][c] already consists of the 16-byte chunks the kernel
+// wants, the 64 channels of a slab are 128 consecutive bytes of a pixel, and the filters W[co][ky][kx][ci] are
+// tap-major as they lie.  What is missing is the zero border - and that costs nothing here, because every lane
+// of a load gives its own address: the input tile in LDS is a run of positions of a VIRTUAL padded grid with ONE
+// zero row above and ONE zero column left of every sample,
+//     V[b][yv][xv] = X[b][yv - 1][xv - 1]  for yv, xv >= 1,   zero for yv = 0 or xv = 0 or b >= batch,
+// Hv = H + 1 rows of Wv = W + 1 columns: the column right of a row's last pixel is the zero column of the next row,
+// the row below a sample's last row the zero row of the next sample.  Output pixel (b, y, x) is the row of the
+// product at position (b*Hv + y)*Wv + x, its tap (ky, kx) the position ky*Wv + kx further on.  A lane whose
+// position is a zero of the grid loads from a page of zeros.  So a layer is ONE launch - no padded copy, no
+// filter pass (the input gradient needs the flipped, transposed filters: one small pass) - and only one column in
+// Wv (and, where the rows below a sample are not skipped, one row in Hv) is computed and dropped.
+// The tile in LDS is [position][8 chunks] (a wave's load covers 8 positions x 128 bytes: whole cache lines), the
+// chunks of a row XOR-swizzled like the filter rows, so a fragment address is  (row << 7) + ((chunk << 4) ^ swizzle(row))
+// with the tap's shift inside row: three vector instructions per tap and fragment and one per read.
+struct HaloHwcArgs {
+    const char *x;      // [batch][H][W][Cin] halves
+    const char *zeros;  // 128 readable zero bytes
+    const char *wr;     // [Cout][9][Cin] halves
+    half_t *y;          // [batch][H][W][Cout]
+    unsigned Q;         // rows of the product
+    unsigned qimg;      // rows per sample: Hv*Wv, or H*Wv with the row below the sample left out
+    unsigned jump;      // positions skipped per sample boundary: 0 or Wv
+    unsigned maxcross;  // sample boundaries a tile can cross (0 when jump is 0)
+    unsigned m_img, m_row;  // multipliers for position / (Hv*Wv) and / Wv (see fast_div31)
+    int s_img, s_row;
+    int batch, Cin, Cout, H, W, Hv, Wv;
+    int tiles, ct_count;  // tile = position tile * ct_count + filter tile
+};
+
+// n / d for n < 2^31 with m = ceil(2^(31 + s) / d), s = ceil(log2 d) >= 1 (d >= 2)
+__device__ inline unsigned fast_div31(unsigned n, unsigned m, int s) { return __umulhi(n, m) >> (s - 1); }
+
+template <int BN, int NS>
+__global__ __launch_bounds__(HALO_NT) void conv_halo_hwc_kernel(const HaloHwcArgs a) {
+    constexpr int STAGE = BN * 128;      // bytes of a ring slot: one tap x 64 channels x BN filters
+    constexpr int LB = BN / 32;          // filter chunks per thread and stage
+    constexpr int FM = BN / 32, FN = 2;  // fragments per wave: filters x positions (64 positions per wave)
+    constexpr int MID = 1;               // half of a stage in front of which the next stage is certified
+    constexpr int NR = 2 * (FM + FN), NM = 2 * FM * FN;  // fragment reads / MFMAs per half stage (two k-steps)
+    static_assert(NS >= 3 && NS <= 7, "ring depth");
+    static_assert(NR <= NM, "one fragment read per MFMA");
+    extern __shared__ __align__(16) char smem[];
+    const unsigned halo_lds = (unsigned)(uintptr_t)(lds_char *)smem, ring_lds = halo_lds + 2 * HALO_BYTES;
+    const char *const halo = smem, *const ring = smem + 2 * HALO_BYTES;
+    const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int l32 = lane & 31, kg = lane >> 5;
+    const int G = gridDim.x, UC = a.Cin / 64;
+    const long long K9 = 9ll * a.Cin;
+    const int cin2 = a.Cin * 2;
+    const unsigned HvWv = (unsigned)(a.Hv * a.Wv);
+
+    unsigned voff_b[LB];
+#pragma unroll
+    for (int i = 0; i < LB; ++i) {
+        const int row = (wave + 4 * i) * 8 + (lane >> 3);
+        voff_b[i] = (unsigned)(row * K9 * 2) + (unsigned)((((lane & 7) ^ swz(row))) << 4);
+    }
+    unsigned wfrag[4];
+#pragma unroll
+    for (int ks = 0; ks < 4; ++ks) wfrag[ks] = (unsigned)(l32 * 128 + (((2 * ks + kg) ^ swz(l32)) << 4));
+
+    struct Unit {
+        int tile, cs;
+        const char *fb;  // filters of (filter tile, channel slab)
+        unsigned p0;     // virtual position of the tile's first row
+        unsigned rem0;   // row of the tile's first position within its sample's rows
+    };
+    auto make_unit = [&](int tile, int cs) {
+        Unit u;
+        u.tile = tile;
+        u.cs = cs;
+        const unsigned pt = (unsigned)tile / (unsigned)a.ct_count, ct = (unsigned)tile - pt * (unsigned)a.ct_count;
+        const unsigned q0 = pt * HALO_BM, b0 = q0 / a.qimg;
+        u.rem0 = q0 - b0 * a.qimg;
+        u.p0 = q0 + b0 * a.jump;  // (the host keeps batch * Hv * Wv + the tile's reach below 2^31)
+        u.fb = a.wr + ((long long)ct * BN * K9 + cs * 64) * 2;
+        return u;
+    };
+    // tile-local position of the row of this lane's fragment j: its row number plus `jump` per sample boundary
+    // between the tile's first row and its own
+    auto lane_rows = [&](const Unit &u, unsigned (&row)[FN]) {
+#pragma unroll
+        for (int j = 0; j < FN; ++j) {
+            const unsigned r = (unsigned)(64 * wave + 32 * j + l32), v = u.rem0 + r;
+            unsigned skip = 0;
+            for (unsigned k = 1, lim = a.qimg; k <= a.maxcross; ++k, lim += a.qimg) skip += v >= lim ? a.jump : 0u;
+            row[j] = r + skip;
+        }
+    };
+    auto next_unit = [&](const Unit &u) {
+        if (u.cs + 1 < UC) return make_unit(u.tile, u.cs + 1);
+        if (u.tile + G < a.tiles) return make_unit(u.tile + G, 0);
+        return u;  // past the end: the same unit again
+    };
+    auto issue_filter = [&](const Unit &u, int tap, unsigned slot_lds, int i) {
+        lds_dma16_saddr(voff_b[i], u.fb + tap * cin2, slot_lds + (unsigned)((wave + 4 * i) * 1024));
+    };
+    // piece q (0 .. 11) of a unit's input tile: eight positions x the slab's eight chunks per wave
+    auto issue_piece = [&](const Unit &u, unsigned buf_lds, int q) {
+        const unsigned pl = (unsigned)((wave + 4 * q) * 8 + (lane >> 3));  // tile-local position
+        const unsigned pv = u.p0 + pl;
+        const unsigned b = fast_div31(pv, a.m_img, a.s_img), rem = pv - b * HvWv;
+        const unsigned yv = fast_div31(rem, a.m_row, a.s_row), xv = rem - yv * (unsigned)a.Wv;
+        const bool ok = b < (unsigned)a.batch && yv >= 1u && xv >= 1u;
+        const unsigned chunk = (unsigned)(((lane & 7) ^ swz((int)pl)) << 4);
+        const unsigned pix = (b * (unsigned)a.H + yv - 1u) * (unsigned)a.W + xv - 1u;  // < 2^31 / Cin
+        const char *src = ok ? a.x + ((size_t)pix * (unsigned)cin2 + (unsigned)(u.cs * 128) + chunk) : a.zeros + chunk;
+        lds_dma<16>(src, buf_lds + (unsigned)((wave + 4 * q) * 1024));
+    };
+
+    Unit cu = make_unit(blockIdx.x, 0), nu = next_unit(cu);
+    int hb = 0;
+    unsigned slot_off = 0, prev_off = (NS - 1) * STAGE;  // ring slot of the current stage / of the stage before it
+#pragma unroll
+    for (int q = 0; q < 12; ++q) issue_piece(cu, halo_lds, q);
+#pragma unroll
+    for (int s = 0; s < NS - 1; ++s)  // (NS - 1 <= 9 taps: all of the first unit)
+#pragma unroll
+        for (int i = 0; i < LB; ++i) issue_filter(cu, s, ring_lds + s * STAGE, i);
+    wait_vmcnt<(NS - 2) * LB>();
+    __syncthreads();  // stage 0 of the first unit has landed
+
+    // fragment sets (two k-steps of 16 each): the one being multiplied and the one being read
+    uint4 wf[2][2][FM], xf[2][2][FN];
+    unsigned xrow[FN], xrow_next[FN];
+    lane_rows(cu, xrow);
+    lane_rows(nu, xrow_next);
+    // per fragment j of the tap being read: (row << 7) and the swizzle term ((kg << 4) ^ swizzle(row) << 4)
+    unsigned xa[FN], xt[FN];
+    auto tap_addresses = [&](const unsigned (&row)[FN], int shift) {
+#pragma unroll
+        for (int j = 0; j < FN; ++j) {
+            const unsigned rt = row[j] + (unsigned)shift;
+            xa[j] = rt << 7;
+            xt[j] = ((rt << 3) & 0x70u) ^ (unsigned)(kg << 4);
+        }
+    };
+    // read r (0 .. NR - 1) of the fragments of the pair of k-steps `half` of a stage: per k-step the filter fragments,
+    // then the position fragments
+    auto read_frag = [&](int set, const char *wbase, const char *xbuf, int half, int r) {
+        const int h = r / (FM + FN), k = r % (FM + FN), ks = 2 * half + h;
+        if (k < FM)
+            wf[set][h][k] = *reinterpret_cast<const uint4 *>(wbase + wfrag[ks] + k * 32 * 128);
+        else
+            xf[set][h][k - FM] = *reinterpret_cast<const uint4 *>(xbuf + (xa[k - FM] + (xt[k - FM] ^ (unsigned)(ks << 5))));
+    };
+    tap_addresses(xrow, 0);
+#pragma unroll
+    for (int r = 0; r < NR; ++r) read_frag(0, ring, halo, 0, r);
+
+    f32x16 acc[FM][FN];
+    while (true) {
+        if (cu.cs == 0) {
+#pragma unroll
+            for (int i = 0; i < FM; ++i)
+#pragma unroll
+                for (int j = 0; j < FN; ++j)
+#pragma unroll
+                    for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.f;
+        }
+        const char *xbase = halo + hb * HALO_BYTES, *xnext = halo + (hb ^ 1) * HALO_BYTES;
+        const unsigned next_lds = halo_lds + (unsigned)((hb ^ 1) * HALO_BYTES);
+        static_for<0, 18>([&](auto GI) {
+            constexpr int g = decltype(GI)::value, sidx = g / 2, half = g % 2, cur = g & 1;
+            // loads this half stage issues: the filters of stage sidx + NS - 1 into the slot of stage sidx - 1, then
+            // this stage's share of the next unit's input tile
+            constexpr int ahead = sidx + NS - 1;
+            constexpr int np = half == MID ? pipe_pieces<NS>(sidx) : 0, q0 = pipe_piece0<NS>(sidx);
+            constexpr int nd = half == MID ? LB + np : 0;
+            static_assert(nd <= NM, "one load per MFMA");
+            if constexpr (half == MID) {
+                // certify stage sidx + 1; every wave has then left stage sidx - 1
+                wait_vmcnt<pipe_wait<NS, LB>(sidx)>();
+                // (a bare barrier: fragment reads still in flight address slots that nobody refills now)
+                asm volatile("s_barrier" ::: "memory");
+            }
+            // fragments of the next pair of k-steps
+            constexpr int gn = g + 1, sn = (gn / 2) % 9, hn = gn % 2;
+            const unsigned noff = hn == 0 ? (slot_off + STAGE == NS * STAGE ? 0u : slot_off + STAGE) : slot_off;
+            const char *wnext = ring + noff, *xbuf = gn < 18 ? xbase : xnext;
+            if constexpr (hn == 0) {  // a new tap (of the next unit's tile behind the last stage)
+                const int shift = (sn / 3) * a.Wv + sn % 3;
+                if constexpr (gn < 18)
+                    tap_addresses(xrow, shift);
+                else
+                    tap_addresses(xrow_next, shift);
+            }
+            // One fragment read and at most one load behind each MFMA, in exactly this order (nothing may cross a
+            // sched_barrier): the address arithmetic of the loads sits between the MFMAs, not in front of them.
+            static_for<0, NM>([&](auto MI) {
+                constexpr int m = decltype(MI)::value, h = m / (FM * FN), i = (m % (FM * FN)) / FN, j = m % FN;
+                if constexpr (m < NR) read_frag(cur ^ 1, wnext, xbuf, hn, m);
+                mfma_step<half_t>(acc[i][j], wf[cur][h][i], xf[cur][h][j]);
+                if constexpr (m < nd) {
+                    if constexpr (m < LB) {
+                        if constexpr (ahead < 9)
+                            issue_filter(cu, ahead, ring_lds + prev_off, m);
+                        else
+                            issue_filter(nu, ahead - 9, ring_lds + prev_off, m);
+                    } else {
+                        issue_piece(nu, next_lds, q0 + m - LB);
+                    }
+                }
+                __builtin_amdgcn_sched_barrier(0);
+            });
+            if constexpr (half == 1) {
+                prev_off = slot_off;
+                slot_off = slot_off + STAGE == NS * STAGE ? 0u : slot_off + STAGE;
+            }
+        });
+        const bool tile_done = cu.cs + 1 == UC;
+        if (tile_done) {
+            const unsigned q0 = ((unsigned)cu.tile / (unsigned)a.ct_count) * HALO_BM;
+            const int co0 = (cu.tile % a.ct_count) * BN;
+#pragma unroll
+            for (int j = 0; j < FN; ++j) {
+                const unsigned q = q0 + (unsigned)(64 * wave + 32 * j + l32);  // (Q < 2^31 on the host)
+                const unsigned b = q / a.qimg, rem = q - b * a.qimg;
+                const unsigned yy = rem / (unsigned)a.Wv, xx = rem - yy * (unsigned)a.Wv;
+                if (q < a.Q && yy < (unsigned)a.H && xx < (unsigned)a.W) {
+                    // a lane holds runs of four consecutive filters of its position: 8-byte stores
+                    half_t *dst = a.y + ((size_t)(b * (unsigned)a.H + yy) * (unsigned)a.W + xx) * (unsigned)a.Cout + co0 + 4 * kg;
+#pragma unroll
+                    for (int i = 0; i < FM; ++i)
+#pragma unroll
+                        for (int vg = 0; vg < 4; ++vg) {
+                            union {
+                                half_t e[4];
+                                uint2 v;
+                            } o;
+#pragma unroll
+                            for (int e = 0; e < 4; ++e) o.e[e] = (half_t)acc[i][j][4 * vg + e];
+                            *reinterpret_cast<uint2 *>(dst + i * 32 + 8 * vg) = o.v;
+                        }
+                }
+            }
+        }
+        const bool last = tile_done && cu.tile + G >= a.tiles;
+        if (last) break;
+        cu = nu;
+        hb ^= 1;
+        nu = next_unit(cu);
+#pragma unroll
+        for (int j = 0; j < FN; ++j) xrow[j] = xrow_next[j];
+        lane_rows(nu, xrow_next);
+    }
+    wait_vmcnt<0>();  // nothing may still be landing in LDS when the workgroup ends
+}
+
+template <int BN, int NS>
+int launch_halo_hwc(const HaloHwcArgs &a, int grid, hipStream_t stream) {
+    constexpr int lds = 2 * HALO_BYTES + NS * BN * 128;
+    static_assert(lds <= 160 * 1024, "LDS");
+    static bool attr = false;
+    if (!attr) {
+        if (!hip_ok(hipFuncSetAttribute((const void *)conv_halo_hwc_kernel<BN, NS>,
+                                        hipFuncAttributeMaxDynamicSharedMemorySize, lds),
+                    "halo convolution LDS size"))
+            return 2;
+        attr = true;
+    }
+    hipLaunchKernelGGL((conv_halo_hwc_kernel<BN, NS>), dim3((unsigned)grid), dim3(HALO_NT), lds, stream, a);
+    return hip_ok(hipGetLastError(), "halo convolution launch") ? 0 : 2;
+}
+
+// ---------------------------------------------------------------------------------------------------------
 // Weight gradient on the same layouts:
 //   dW[co][ci][ky][kx] = sum over padded positions p of  gb[p][co] * xb[p + ky*Wp + kx][ci]
 // with gb the output gradient embedded at the top left of the padded grids (zero elsewhere), channel-blocked
@@ -502,6 +769,53 @@ int conv_halo_launch(const ConvTileDesc &d, const void *xb, const void *wr, void
     return bn == 128 ? launch_halo_pipe<128, 4>(a, grid, st.stream) : launch_halo_pipe<64, 6>(a, grid, st.stream);
 }
 
+
+// Channel-minor 3x3 "same" layers (one row / column of padding on every side), unit stride, whole 64-channel slabs
+// on both sides, rows short enough for a tile and its reach to fit the LDS buffer, 16-byte aligned tensors.
+bool conv_halo_hwc_fits(const ConvTileDesc &d, const void *X, const void *Y) {
+    const int Wv = d.Win + 1;
+    return d.in_hwc && d.KH == 3 && d.KW == 3 && d.sh == 1 && d.sw == 1 && d.padU == 1 && d.padD == 1 && d.padL == 1 &&
+           d.padR == 1 && d.Ho == d.Hin && d.Wo == d.Win && d.Cin % 64 == 0 && d.Cout % 64 == 0 && d.Cin <= 8192 &&
+           HALO_BM + 2 * Wv + 2 <= HALO_NP && reinterpret_cast<uintptr_t>(X) % 16 == 0 &&
+           reinterpret_cast<uintptr_t>(Y) % 8 == 0 &&
+           (long long)(d.batch + 1) * (d.Hin + 1) * Wv + HALO_NP < ((long long)1 << 31);
+}
+
+static void magic31(unsigned d, unsigned *m, int *s) {  // d >= 2
+    int l = 1;
+    while ((1ull << l) < d) ++l;
+    *s = l;
+    *m = (unsigned)(((1ull << (31 + l)) + d - 1) / d);
+}
+
+// X: [batch][H][W][Cin], wr: tap-major filters [Cout][9][Cin], Y: [batch][H][W][Cout].
+int conv_halo_hwc_launch(const ConvTileDesc &d, const void *X, const void *wr, void *Y) {
+    State &st = state();
+    HaloHwcArgs a = {};
+    a.x = static_cast<const char *>(X);
+    a.zeros = static_cast<const char *>(st.zeros);
+    a.wr = static_cast<const char *>(wr);
+    a.y = static_cast<half_t *>(Y);
+    a.batch = d.batch; a.Cin = d.Cin; a.Cout = d.Cout; a.H = d.Hin; a.W = d.Win;
+    a.Hv = d.Hin + 1; a.Wv = d.Win + 1;
+    // leave the zero row of every sample out of the row enumeration when a tile that crosses sample boundaries and
+    // its reach (two rows and two positions) still fit
+    const int qs = d.Hin * a.Wv, crossings = (HALO_BM - 1 + qs - 1) / qs;
+    const bool skip = HALO_BM + crossings * a.Wv + 2 * a.Wv + 2 <= HALO_NP;
+    a.qimg = (unsigned)(skip ? qs : a.Hv * a.Wv);
+    a.jump = (unsigned)(skip ? a.Wv : 0);
+    a.maxcross = (unsigned)(skip ? crossings : 0);
+    a.Q = (unsigned)((long long)d.batch * a.qimg);
+    magic31((unsigned)(a.Hv * a.Wv), &a.m_img, &a.s_img);
+    magic31((unsigned)a.Wv, &a.m_row, &a.s_row);
+    const int bn = d.Cout % 128 == 0 ? 128 : 64;
+    a.ct_count = d.Cout / bn;
+    const long long ptiles = ((long long)a.Q + HALO_BM - 1) / HALO_BM;
+    if (ptiles * a.ct_count >= (1ll << 30)) return -1;
+    a.tiles = (int)(ptiles * a.ct_count);
+    const int grid = a.tiles < st.num_cu ? a.tiles : st.num_cu;
+    return bn == 128 ? launch_halo_hwc<128, 4>(a, grid, st.stream) : launch_halo_hwc<64, 6>(a, grid, st.stream);
+}
 
 bool conv_halo_wg_fits(const ConvTileDesc &d, int Hp, int Wp) {
     return !d.in_hwc && d.KH == 3 && d.KW == 3 && d.sh == 1 && d.sw == 1 && d.Cin % 64 == 0 && d.Cout % 128 == 0 &&

@@ -183,6 +183,28 @@ int conv_taps(const ConvTileDesc &d, const void *X, const void *Wt, void *Y, con
     // 19.0 us for 128 -> 128 on 28x28 at batch 8, 35.8 against 56.5 us for 512 -> 512 on 7x7 at batch 32).
     const long long halo_tiles = ((long long)d.batch * Hp * Wp + 255) / 256 * ((d.Cout + 127) / 128);
     const bool halo_pays = halo_tiles >= 48 || (d.Cin == 64 && halo_tiles >= 32);
+    // channel-minor tensors: the same kernel reads them in place (no padded copy; the filters too when they are
+    // tap-major as they lie, which the forward pass's are)
+    if (ES == 2 && hwc && conv_halo_hwc_fits(d, X, Y) && (st.gemm_path == 5 || (st.gemm_path == 0 && halo_pays))) {
+        const void *wr = Wt;
+        if (!(d.w_base == 0 && d.w_sc == 1 && d.w_sx == d.Cin && d.w_sy == d.KW * d.Cin && d.w_sm == taps * d.Cin &&
+              reinterpret_cast<uintptr_t>(Wt) % 16 == 0)) {
+            char *buf = static_cast<char *>(scratch((size_t)wr_elems * ES + 256));
+            if (!buf) return 2;
+            TapPrepArgs p = {};
+            p.copy_blocks = 0;
+            p.w = Wt;
+            p.wr = buf;
+            p.C = d.Cin; p.KW = d.KW; p.taps = taps;
+            p.w_base = d.w_base; p.w_sm = d.w_sm; p.w_sc = d.w_sc; p.w_sy = d.w_sy; p.w_sx = d.w_sx;
+            p.wr_total = wr_elems;
+            hipLaunchKernelGGL((tap_prepare_kernel<T>), dim3((unsigned)((wr_elems + 255) / 256)), dim3(256), 0, st.stream, p);
+            if (!hip_ok(hipGetLastError(), "layout launch")) return 2;
+            wr = buf;
+        }
+        st.last_conv_resident = 1;
+        return conv_halo_hwc_launch(d, X, wr, Y);
+    }
     const bool halo = ES == 2 && !hwc && conv_halo_fits(d, Hp, Wp) && (long long)d.batch * Hp * Wp < ((long long)1 << 31) &&
                       (st.gemm_path == 5 || (st.gemm_path == 0 && halo_pays));
     const long long margin = halo ? conv_halo_margin() : 0;  // chunks the resident-tile kernel may read past the end

@@ -105,6 +105,10 @@ bool conv_halo_fits(const ConvTileDesc &d, int Hp, int Wp);
 long long conv_halo_margin();
 int conv_halo_launch(const ConvTileDesc &d, const void *xb, const void *wr, void *Y, int Hp, int Wp,
                      long long pstride = 0);  // pstride: positions between channel blocks of xb (0: batch*Hp*Wp)
+// The same layers with channel-minor tensors read in place (X [batch][H][W][Cin], tap-major filters, Y
+// [batch][H][W][Cout]): one launch, the zero border comes from the addresses of the loads.
+bool conv_halo_hwc_fits(const ConvTileDesc &d, const void *X, const void *Y);
+int conv_halo_hwc_launch(const ConvTileDesc &d, const void *X, const void *wr, void *Y);
 int conv_halo_embed(const void *t, void *out, int batch, int C, int Hs, int Ws, int Hp, int Wp, int pu, int pl,
                     long long pstride);
 

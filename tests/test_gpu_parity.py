@@ -386,6 +386,37 @@ def test_conv2d_backward_in_one_call(pkg, orc, gpu, case, skip):
         assert rel_l2(host(gdx), rdx) <= TOL["fp16"]
 
 
+@pytest.mark.parametrize("case", [(64, 14, 14, 128, 9), (128, 5, 7, 64, 21), (64, 62, 62, 64, 2), (192, 28, 28, 256, 5),
+                                  (64, 3, 61, 128, 4), (128, 1, 1, 128, 300), (64, 30, 9, 192, 3)])
+def test_conv2d_resident_tile_channel_minor_in_place(pkg, gpu, case):
+    """Channel-minor 3x3 "same" layers on the resident-tile kernel that reads X[b][y][x][c] in place (the zero border
+    comes from the addresses of its loads): forward and input gradient against torch in float32; tiles that cross
+    several samples, a single row, the widest row that fits, ragged last tiles, one and several filter tiles and
+    channel slabs."""
+    import torch.nn.functional as F
+    Ci, H, W, Co, ns = case
+    nd = np.float16
+    x = dev(hp.uniform(51, (ns, H, W, Ci), dtype=nd))
+    w = dev(hp.uniform(52, (Co, 3, 3, Ci), dtype=nd) * 0.2)
+    dy = dev(hp.uniform(53, (ns, H, W, Co), dtype=nd))
+    y, dx = dev(np.full((ns, H, W, Co), 3, nd)), dev(np.full((ns, H, W, Ci), 3, nd))
+    a, keep = hp.conv2d_args(pkg, x, dx, w, None, y, dy, Ci, H, W, Co, 3, 3, H, W, (1, 1, 1, 1), (1, 1), 1)
+    gpu.ptl_set_gemm_path(5)
+    try:
+        for s in ("fw", "ig"):
+            pkg.call("ptl_conv2d_fp16_%s_batched" % s, a, ns)
+            assert gpu.ptl_last_conv_resident() == 1, s
+    finally:
+        gpu.ptl_set_gemm_path(0)
+    sync(gpu)
+    xc, wc, dyc = x.float().permute(0, 3, 1, 2), w.float().permute(0, 3, 1, 2), dy.float().permute(0, 3, 1, 2)
+    ref_y = F.conv2d(xc, wc, padding=1).permute(0, 2, 3, 1)
+    ref_dx = torch.nn.grad.conv2d_input(xc.shape, wc, dyc, padding=1).permute(0, 2, 3, 1)
+    rel = lambda got, ref: float((got.float() - ref).norm() / ref.norm())
+    assert rel(y, ref_y) <= 1e-3
+    assert rel(dx, ref_dx) <= 1e-3
+
+
 def test_conv2d_resident_tile_many_tiles(pkg, gpu):
     """More position tiles than workgroups (every workgroup walks several tiles, the last one ragged) and two
     filter tiles: the resident-tile kernel against the tap-sum GEMM and against torch in float32."""
