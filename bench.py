@@ -279,8 +279,9 @@ TARGET_ROWS = (
      ["resnet20 step with batch norm, element-wise layers fused into it FW+BW+SGD"], "samples/s"),
     ("mm_4096_fp16_random_then_zero_operands_TFLOP/s",
      ["power: mm 4096x4096x4096 (B transposed), random", "power: mm 4096x4096x4096 (B transposed), zero"], "TFLOP/s"),
-    ("mm_4096_fp16_random_then_zero_operands_board_W",
-     ["power: mm 4096x4096x4096 (B transposed), random", "power: mm 4096x4096x4096 (B transposed), zero"], "W"),
+    ("mfma_32x32x16_loop_alone_random_then_zero_operands_TFLOP/s",
+     ["power: loop of v_mfma_f32_32x32x16_f16 alone, random operands, 1 wave ",
+      "power: loop of v_mfma_f32_32x32x16_f16 alone, zero operands, 1 wave "], "TFLOP/s"),
 )
 MAX_LAST_LINE = 4096
 
@@ -371,6 +372,19 @@ def power_rows(pkg, lib, hp, check, torch, dev):
     sync = torch.cuda.synchronize
     N = 4096
     ns, Ci, Co, H = 256, 512, 512, 14
+    # what the matrix cores sustain on a loop of nothing but MFMAs (no loads, no LDS): the ceiling on that data
+    for shape in (32, 16):
+        for kind in ("random", "zero"):
+            for waves in (1, 2):
+                tf = ctypes.c_float(0)
+
+                def probe():
+                    check(lib.ptl_probe_mfma_fp16(shape, 1 if kind == "random" else 0, waves, 4000, ctypes.byref(tf)))
+                us, w = ps.run(probe, sync, 0.4)
+                rows.append({"workload": "power: loop of v_mfma_f32_%s_f16 alone, %s operands, %d wave%s per SIMD"
+                                         % ("32x32x16" if shape == 32 else "16x16x32", kind, waves, "s" if waves > 1 else ""),
+                             "dtype": "fp16", "us": round(us, 2), "TFLOP/s": round(tf.value, 1),
+                             "W": None if w is None else round(w), "cap_W": ps.cap})
     for kind in ("random", "zero"):
         def mk(*shape):
             if kind == "zero":

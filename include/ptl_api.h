@@ -319,6 +319,12 @@ int ptl_last_conv_direct(void);
 int ptl_last_gemm_streamed(void);
 int ptl_last_conv_resident(void);
 int ptl_last_gemm_tile(void);
+/* A measurement aid (no counterpart in the reference, not on the training path): the rate, in TFLOP/s, that this
+ * board sustains on a loop of nothing but fp16 MFMAs - shape 32: v_mfma_f32_32x32x16_f16, 16: v_mfma_f32_16x16x32_f16 -
+ * on random (1) or all-zero (0) operands, with one or two waves per SIMD on every compute unit, `iters` x 262144 flops
+ * per wave.  On random operands such a loop runs against the board's power limit; the rate it holds is what a GEMM
+ * or convolution kernel can approach on that data.  Uses the library's scratch buffer and event pair. */
+int ptl_probe_mfma_fp16(int shape, int random_operands, int waves_per_simd, int iters, float *tflops);
 /* hipEvent timing on the library stream: begin records, end records,
  * synchronises and returns the elapsed milliseconds (negative on error). */
 int ptl_timer_begin(void);

@@ -103,7 +103,7 @@ STATS_ENTRY_POINTS = ["ptl_conv2d_%s_fw_batched_stats" % dt for dt in ("fp16", "
 
 OTHER_ENTRY_POINTS = ["ptl_init", "ptl_last_error", "ptl_last_status", "ptl_set_stream", "ptl_sync", "ptl_set_gemm_path",
                       "ptl_last_conv_direct", "ptl_last_gemm_streamed", "ptl_last_conv_resident", "ptl_last_gemm_tile", "ptl_timer_begin", "ptl_timer_end_ms", "ptl_mm_fp32", "ptl_mm_fp16", "ptl_copy_bytes",
-                      "ptl_reserve", "ptl_reserved"]
+                      "ptl_reserve", "ptl_reserved", "ptl_probe_mfma_fp16"]
 
 
 def load():
@@ -191,6 +191,8 @@ def load():
     lib.ptl_reserve.restype = ctypes.c_int
     lib.ptl_reserved.argtypes = [ctypes.POINTER(ctypes.c_size_t), ctypes.POINTER(ctypes.c_size_t)]
     lib.ptl_reserved.restype = None
+    lib.ptl_probe_mfma_fp16.argtypes = [ctypes.c_int] * 4 + [ctypes.POINTER(ctypes.c_float)]
+    lib.ptl_probe_mfma_fp16.restype = ctypes.c_int
     _lib = lib
     return lib
 

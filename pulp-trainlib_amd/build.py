@@ -16,7 +16,7 @@ LIB = os.path.join(HERE, "libptl_hip.so")
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 CLANG = os.environ.get("PTL_CC", "/opt/rocm/lib/llvm/bin/clang")
 
-HIP_SOURCES = ["ptl_runtime.hip", "ptl_gemm.hip", "ptl_gemm_async_sel.hip", "ptl_gemm_plain_f16.hip", "ptl_gemm_plain_f32.hip", "ptl_gemm_async_f16_c0.hip", "ptl_gemm_async_f16_c1.hip", "ptl_gemm_async_f16_c2.hip", "ptl_gemm_async_f16_c3.hip", "ptl_gemm_async_f32_c0.hip", "ptl_gemm_async_f32_c1.hip", "ptl_gemm_async_f32_c2.hip", "ptl_gemm_async_f32_c3.hip", "ptl_layers.hip", "ptl_conv_tile.hip", "ptl_conv_wg.hip", "ptl_conv_taps.hip", "ptl_conv_halo.hip", "ptl_conv_small.hip", "ptl_tensor_ops.hip", "ptl_mhsa.hip", "ptl_glue.hip"]
+HIP_SOURCES = ["ptl_runtime.hip", "ptl_gemm.hip", "ptl_gemm_async_sel.hip", "ptl_gemm_plain_f16.hip", "ptl_gemm_plain_f32.hip", "ptl_gemm_async_f16_c0.hip", "ptl_gemm_async_f16_c1.hip", "ptl_gemm_async_f16_c2.hip", "ptl_gemm_async_f16_c3.hip", "ptl_gemm_async_f32_c0.hip", "ptl_gemm_async_f32_c1.hip", "ptl_gemm_async_f32_c2.hip", "ptl_gemm_async_f32_c3.hip", "ptl_layers.hip", "ptl_conv_tile.hip", "ptl_conv_wg.hip", "ptl_conv_taps.hip", "ptl_conv_halo.hip", "ptl_conv_small.hip", "ptl_tensor_ops.hip", "ptl_mhsa.hip", "ptl_glue.hip", "ptl_probe.hip"]
 C_SOURCES = ["pulp_entry.c"]
 
 # -packed-fp32-ops: keep the compiler from forming packed fp32 VALU ops.

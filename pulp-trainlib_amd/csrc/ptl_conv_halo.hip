@@ -34,14 +34,19 @@ constexpr int HALO_BYTES = HALO_NP * 8 * 16;       // one buffer: 8 channel bloc
 constexpr int HALO_NT = 256;
 
 struct HaloArgs {
-    const char *xb;     // [Cin/8][P] chunks, readable HALO_NP chunks past the last tile's start in every block
+    const char *xb;     // channel-major route: [Cin/8][P] chunks, readable HALO_NP chunks past the last tile's start in
+                        // every block; channel-minor route: the tensor itself, [batch][H][W][Cin] halves
+    const char *zeros;  // channel-minor route: 128 readable zero bytes
     const char *wr;     // [Cout][9][Cin] halves
-    half_t *y;          // [batch][Cout][Ho][Wo]
+    half_t *y;          // [batch][Cout][Ho][Wo], channel-minor route [batch][Ho][Wo][Cout]
     long long P;        // padded positions of all samples (stride between channel blocks of xb)
     unsigned Q;         // rows of the product
-    unsigned qimg;      // rows per sample: Hp*Wp, or Ho*Wp with the bottom rows left out
+    unsigned qimg;      // rows per sample: Hp*Wp, or Ho*Wp with the rows below the sample left out
     unsigned jump;      // positions skipped per sample boundary: 0 or (Hp - Ho)*Wp
-    int Cin, Cout, Hp, Wp, Ho, Wo;
+    unsigned maxcross;  // sample boundaries a tile can cross (0 when jump is 0)
+    unsigned m_img, m_row;  // channel-minor route: multipliers for position / (Hp*Wp) and / Wp (see fast_div31)
+    int s_img, s_row;
+    int batch, Cin, Cout, Hp, Wp, Ho, Wo;
     int tiles, ct_count;  // tile = position tile * ct_count + filter tile
 };
 
@@ -81,20 +86,58 @@ __host__ __device__ constexpr int pipe_wait(int sidx) {
     return n;
 }
 
-template <int BN, int NS>
-__global__ __launch_bounds__(HALO_NT) void conv_halo_pipe_kernel(const HaloArgs a) {
+// The products run on v_mfma_f32_16x16x32_f16: a fragment is 16 rows x 32 k (a lane holds row lane % 16, k group
+// lane / 16 of eight), one ds_read_b128 each as with the 32 x 32 x 16 form and the same bytes from LDS per flop; a
+// lane then holds four consecutive filters of one position.  These kernels run against the board's power limit (on
+// random operands the clock drops until the power fits), and there the 16 x 16 x 32 form sustains more: a loop of
+// nothing but MFMAs 1.9 against 1.7 PFLOP/s, this kernel 4-9 % on 512 -> 512 channels measured on one board in turns.
+__device__ inline void mfma16(f32x4 &acc, const uint4 &a, const uint4 &b) {
+    acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8, a), __builtin_bit_cast(f16x8, b), acc, 0, 0, 0);
+}
+
+// n / d for n < 2^31 with m = ceil(2^(31 + s) / d), s = ceil(log2 d) >= 1 (d >= 2)
+__device__ inline unsigned fast_div31(unsigned n, unsigned m, int s) { return __umulhi(n, m) >> (s - 1); }
+
+// Everything about a unit that the loads of its stages need, worked out once per unit (wave-uniform).
+struct HaloUnit {
+    int tile, cs;
+    const char *fb;   // filters of (filter tile, channel slab): + tap * Cin * 2 per stage, + voff_b per lane
+    const char *hb;   // channel-major: this wave's first input piece (blocks 2 * wave and 2 * wave + 1 of the slab, from
+                      // the tile's first position); channel-minor: the tensor + the slab's byte offset in a pixel
+    unsigned p0;      // position of the tile's first row in the padded grids laid end to end
+    unsigned rem0;    // row of the tile's first position within its sample's rows
+};
+
+// HWC = false: the input arrives zero-padded and channel-blocked (see the head of the file).
+// HWC = true: channel-minor tensors read in place.  X[b][y][x][c] already consists of the 16-byte chunks the
+// kernel wants, the 64 channels of a slab are 128 consecutive bytes of a pixel, and the filters W[co][ky][kx][ci]
+// of the forward pass are tap-major as they lie.  What is missing is the zero border - and that costs nothing,
+// because every lane of a load gives its own address: the input tile in LDS is a run of positions of a VIRTUAL
+// padded grid with ONE zero row above and ONE zero column left of every sample,
+//     V[b][yv][xv] = X[b][yv - 1][xv - 1]  for yv, xv >= 1,   zero for yv = 0 or xv = 0 or b >= batch,
+// Hp = H + 1 rows of Wp = W + 1 columns: the column right of a row's last pixel is the zero column of the next row,
+// the row below a sample's last row the zero row of the next sample.  A lane whose position is a zero of the grid
+// loads from a page of zeros.  So a layer is ONE launch and only one column in Wp (and, where the row below a
+// sample is not skipped, one row in Hp) is computed and dropped.  The tile in LDS is then [position][8 chunks] (a
+// wave's load covers 8 positions x 128 bytes: whole cache lines), the chunks of a row XOR-swizzled like the filter
+// rows, and a fragment address is (row << 7) + ((chunk << 4) ^ swizzle(row)) with the tap's shift inside `row`.
+template <int BN, int NS, bool HWC>
+__global__ __launch_bounds__(HALO_NT) void conv_halo_kernel(const HaloArgs a) {
     constexpr int STAGE = BN * 128;      // bytes of a ring slot: one tap x 64 channels x BN filters
     constexpr int LB = BN / 32;          // filter chunks per thread and stage
-    constexpr int FM = BN / 32, FN = 2;  // fragments per wave: filters x positions (64 positions per wave)
+    constexpr int FM = BN / 16, FN = 4;  // fragments per wave: filters x positions (64 positions per wave)
     constexpr int MID = 1;               // half of a stage in front of which the next stage is certified
+    constexpr int NR = FM + FN, NM = FM * FN;  // fragment reads / MFMAs per half stage (one k-step of 32)
     static_assert(NS >= 3 && NS <= 7, "ring depth");
     extern __shared__ __align__(16) char smem[];
     const unsigned halo_lds = (unsigned)(uintptr_t)(lds_char *)smem, ring_lds = halo_lds + 2 * HALO_BYTES;
     const char *const halo = smem, *const ring = smem + 2 * HALO_BYTES;
     const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const int l32 = lane & 31, kg = lane >> 5;
+    const int l16 = lane & 15, kq = lane >> 4;
     const int G = gridDim.x, UC = a.Cin / 64;
-    const long long K9 = 9ll * a.Cin;
+    const long long K9 = 9ll * a.Cin, P16 = a.P * 16;
+    const int cin2 = a.Cin * 2;
+    const unsigned HpWp = (unsigned)(a.Hp * a.Wp);
 
     unsigned voff_b[LB];
 #pragma unroll
@@ -103,294 +146,64 @@ __global__ __launch_bounds__(HALO_NT) void conv_halo_pipe_kernel(const HaloArgs 
         voff_b[i] = (unsigned)(row * K9 * 2) + (unsigned)((((lane & 7) ^ swz(row))) << 4);
     }
     const unsigned voff_h = (unsigned)lane * 16u;
-    unsigned wfrag[4];
+    unsigned wfrag[2];
 #pragma unroll
-    for (int ks = 0; ks < 4; ++ks) wfrag[ks] = (unsigned)(l32 * 128 + (((2 * ks + kg) ^ swz(l32)) << 4));
-    // byte offset of this lane's two position fragments within a tile whose first row is q0
-    auto lane_offsets = [&](int tile, unsigned (&off)[FN]) {
-        const unsigned q0 = (unsigned)(tile / a.ct_count) * HALO_BM, i0 = q0 / a.qimg;
-#pragma unroll
-        for (int j = 0; j < FN; ++j) {
-            const unsigned r = (unsigned)(64 * wave + 32 * j + l32);
-            const unsigned skip = a.jump ? ((q0 + r) / a.qimg - i0) * a.jump : 0u;
-            off[j] = (unsigned)(kg * HALO_NP + r + skip) * 16u;
-        }
-    };
+    for (int ks = 0; ks < 2; ++ks) wfrag[ks] = (unsigned)(l16 * 128 + (((4 * ks + kq) ^ swz(l16)) << 4));
 
-    auto issue_filters = [&](int tile, int cs, int tap, int slot) {
-        const int ct = tile % a.ct_count;
-        const char *base = a.wr + ((long long)ct * BN * K9 + (long long)tap * a.Cin + cs * 64) * 2;
-#pragma unroll
-        for (int i = 0; i < LB; ++i)
-            lds_dma16_saddr(voff_b[i], base, ring_lds + (unsigned)(slot * STAGE + (wave + 4 * i) * 1024));
-    };
-    auto issue_halo = [&](int tile, int cs, int hb, int q) {
-        const unsigned q0 = (unsigned)(tile / a.ct_count) * HALO_BM;
-        const long long p0 = (long long)q0 + (long long)(q0 / a.qimg) * a.jump;
-        const int c0 = (q * 4 + wave) * 64, j = c0 / HALO_NP, i0 = c0 - j * HALO_NP;
-        const char *base = a.xb + (((long long)(cs * 8 + j)) * a.P + p0 + i0) * 16;
-        lds_dma16_saddr(voff_h, base, halo_lds + (unsigned)(hb * HALO_BYTES + c0 * 16));
-    };
-    auto next_unit = [&](int tile, int cs, int &ntile, int &ncs) {
-        if (cs + 1 < UC) {
-            ntile = tile;
-            ncs = cs + 1;
-        } else if (tile + G < a.tiles) {
-            ntile = tile + G;
-            ncs = 0;
-        } else {  // past the end: the same unit again
-            ntile = tile;
-            ncs = cs;
-        }
-    };
-    auto wrap = [](int s) { return s >= NS ? s - NS : s; };
-
-    int tile = blockIdx.x, cs = 0, hb = 0, slot = 0;  // slot: ring slot of the current stage
-    int ntile, ncs;
-    next_unit(tile, cs, ntile, ncs);
-#pragma unroll
-    for (int q = 0; q < 12; ++q) issue_halo(tile, cs, 0, q);
-#pragma unroll
-    for (int s = 0; s < NS - 1; ++s) issue_filters(tile, cs, s, s);  // (NS - 1 <= 9 taps: all of the first unit)
-    wait_vmcnt<(NS - 2) * LB>();
-    __syncthreads();  // stage 0 of the first unit has landed
-
-    // fragment sets (two k-steps of 16 each): the one being multiplied and the one being read
-    uint4 wf[2][2][FM], xf[2][2][FN];
-    unsigned xoff[FN], xoff_next[FN];
-    lane_offsets(tile, xoff);
-    lane_offsets(ntile, xoff_next);
-    auto read_frags = [&](int set, const char *wbase, const char *xtap, const unsigned (&xo)[FN], int half) {
-#pragma unroll
-        for (int h = 0; h < 2; ++h) {
-            const int ks = 2 * half + h;
-#pragma unroll
-            for (int i = 0; i < FM; ++i)
-                wf[set][h][i] = *reinterpret_cast<const uint4 *>(wbase + wfrag[ks] + i * 32 * 128);
-#pragma unroll
-            for (int j = 0; j < FN; ++j)
-                xf[set][h][j] = *reinterpret_cast<const uint4 *>(xtap + xo[j] + 2 * ks * HALO_NP * 16);
-        }
-    };
-    read_frags(0, ring, halo, xoff, 0);
-
-    f32x16 acc[FM][FN];
-    while (true) {
-        if (cs == 0) {
-#pragma unroll
-            for (int i = 0; i < FM; ++i)
-#pragma unroll
-                for (int j = 0; j < FN; ++j)
-#pragma unroll
-                    for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.f;
-        }
-        const char *xbase = halo + hb * HALO_BYTES, *xnext = halo + (hb ^ 1) * HALO_BYTES;
-        static_for<0, 18>([&](auto GI) {
-            constexpr int g = decltype(GI)::value, sidx = g / 2, half = g % 2, cur = g & 1;
-            if constexpr (half == MID) {
-                // certify stage sidx + 1, then refill the slot of stage sidx - 1 with stage sidx + NS - 1
-                wait_vmcnt<pipe_wait<NS, LB>(sidx)>();
-                // (a bare barrier: fragment reads still in flight address slots that nobody refills now, so they
-                // need not be waited for here)
-                asm volatile("s_barrier" ::: "memory");
-                constexpr int ahead = sidx + NS - 1;
-                const int fslot = wrap(slot + NS - 1);
-                if (ahead < 9)
-                    issue_filters(tile, cs, ahead, fslot);
-                else
-                    issue_filters(ntile, ncs, ahead - 9, fslot);
-                constexpr int np = pipe_pieces<NS>(sidx), q0 = pipe_piece0<NS>(sidx);
-#pragma unroll
-                for (int q = 0; q < np; ++q) issue_halo(ntile, ncs, hb ^ 1, q0 + q);
-            }
-            {  // fragments of the next pair of k-steps
-                constexpr int gn = g + 1, sn = (gn / 2) % 9, hn = gn % 2;
-                const int nslot = hn == 0 ? wrap(slot + 1) : slot;
-                const int tapoff = ((sn / 3) * a.Wp + sn % 3) * 16;
-                if (gn < 18)
-                    read_frags(cur ^ 1, ring + nslot * STAGE, xbase + tapoff, xoff, hn);
-                else
-                    read_frags(cur ^ 1, ring + nslot * STAGE, xnext + tapoff, xoff_next, hn);
-            }
-#pragma unroll
-            for (int h = 0; h < 2; ++h)
-#pragma unroll
-                for (int i = 0; i < FM; ++i)
-#pragma unroll
-                    for (int j = 0; j < FN; ++j) mfma_step<half_t>(acc[i][j], wf[cur][h][i], xf[cur][h][j]);
-            // one fragment read under each of the first MFMAs
-            constexpr int R = 2 * (FM + FN), M = 2 * FM * FN;
-#pragma unroll
-            for (int r = 0; r < R; ++r) {
-                __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
-                __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-            }
-            if constexpr (M > R) __builtin_amdgcn_sched_group_barrier(0x008, M - R, 0);
-            if (half == 1) slot = wrap(slot + 1);
-        });
-        const bool tile_done = cs + 1 == UC;
-        if (tile_done) {
-            const unsigned q0 = (unsigned)(tile / a.ct_count) * HALO_BM;
-            const int co0 = (tile % a.ct_count) * BN;
-            const unsigned PO = (unsigned)(a.Ho * a.Wo);
-#pragma unroll
-            for (int j = 0; j < FN; ++j) {
-                const unsigned q = q0 + (unsigned)(64 * wave + 32 * j + l32);  // (Q < 2^31 on the host)
-                const unsigned b = q / a.qimg, rem = q - b * a.qimg;
-                const unsigned yy = rem / (unsigned)a.Wp, xx = rem - yy * (unsigned)a.Wp;
-                if (q < a.Q && yy < (unsigned)a.Ho && xx < (unsigned)a.Wo) {
-                    half_t *dst = a.y + ((size_t)b * a.Cout + co0 + 4 * kg) * PO + yy * (unsigned)a.Wo + xx;
-#pragma unroll
-                    for (int i = 0; i < FM; ++i)
-#pragma unroll
-                        for (int v = 0; v < 16; ++v)
-                            dst[(size_t)(i * 32 + 8 * (v >> 2) + (v & 3)) * PO] = (half_t)acc[i][j][v];
-                }
-            }
-        }
-        const bool last = tile_done && tile + G >= a.tiles;
-        if (last) break;
-        tile = ntile;
-        cs = ncs;
-        hb ^= 1;
-        next_unit(tile, cs, ntile, ncs);
-#pragma unroll
-        for (int j = 0; j < FN; ++j) xoff[j] = xoff_next[j];
-        lane_offsets(ntile, xoff_next);
-    }
-    wait_vmcnt<0>();  // nothing may still be landing in LDS when the workgroup ends
-}
-
-template <int BN, int NS>
-int launch_halo_pipe(const HaloArgs &a, int grid, hipStream_t stream) {
-    constexpr int lds = 2 * HALO_BYTES + NS * BN * 128;
-    static_assert(lds <= 160 * 1024, "LDS");
-    static bool attr = false;
-    if (!attr) {
-        if (!hip_ok(hipFuncSetAttribute((const void *)conv_halo_pipe_kernel<BN, NS>,
-                                        hipFuncAttributeMaxDynamicSharedMemorySize, lds),
-                    "halo convolution LDS size"))
-            return 2;
-        attr = true;
-    }
-    hipLaunchKernelGGL((conv_halo_pipe_kernel<BN, NS>), dim3((unsigned)grid), dim3(HALO_NT), lds, stream, a);
-    return hip_ok(hipGetLastError(), "halo convolution launch") ? 0 : 2;
-}
-
-
-// ---------------------------------------------------------------------------------------------------------
-// Channel-minor (HWC) tensors, read in place: X[b][y][x][c] already consists of the 16-byte chunks the kernel
-// wants, the 64 channels of a slab are 128 consecutive bytes of a pixel, and the filters W[co][ky][kx][ci] are
-// tap-major as they lie.  What is missing is the zero border - and that costs nothing here, because every lane
-// of a load gives its own address: the input tile in LDS is a run of positions of a VIRTUAL padded grid with ONE
-// zero row above and ONE zero column left of every sample,
-//     V[b][yv][xv] = X[b][yv - 1][xv - 1]  for yv, xv >= 1,   zero for yv = 0 or xv = 0 or b >= batch,
-// Hv = H + 1 rows of Wv = W + 1 columns: the column right of a row's last pixel is the zero column of the next row,
-// the row below a sample's last row the zero row of the next sample.  Output pixel (b, y, x) is the row of the
-// product at position (b*Hv + y)*Wv + x, its tap (ky, kx) the position ky*Wv + kx further on.  A lane whose
-// position is a zero of the grid loads from a page of zeros.  So a layer is ONE launch - no padded copy, no
-// filter pass (the input gradient needs the flipped, transposed filters: one small pass) - and only one column in
-// Wv (and, where the rows below a sample are not skipped, one row in Hv) is computed and dropped.
-// The tile in LDS is [position][8 chunks] (a wave's load covers 8 positions x 128 bytes: whole cache lines), the
-// chunks of a row XOR-swizzled like the filter rows, so a fragment address is  (row << 7) + ((chunk << 4) ^ swizzle(row))
-// with the tap's shift inside row: three vector instructions per tap and fragment and one per read.
-struct HaloHwcArgs {
-    const char *x;      // [batch][H][W][Cin] halves
-    const char *zeros;  // 128 readable zero bytes
-    const char *wr;     // [Cout][9][Cin] halves
-    half_t *y;          // [batch][H][W][Cout]
-    unsigned Q;         // rows of the product
-    unsigned qimg;      // rows per sample: Hv*Wv, or H*Wv with the row below the sample left out
-    unsigned jump;      // positions skipped per sample boundary: 0 or Wv
-    unsigned maxcross;  // sample boundaries a tile can cross (0 when jump is 0)
-    unsigned m_img, m_row;  // multipliers for position / (Hv*Wv) and / Wv (see fast_div31)
-    int s_img, s_row;
-    int batch, Cin, Cout, H, W, Hv, Wv;
-    int tiles, ct_count;  // tile = position tile * ct_count + filter tile
-};
-
-// n / d for n < 2^31 with m = ceil(2^(31 + s) / d), s = ceil(log2 d) >= 1 (d >= 2)
-__device__ inline unsigned fast_div31(unsigned n, unsigned m, int s) { return __umulhi(n, m) >> (s - 1); }
-
-template <int BN, int NS>
-__global__ __launch_bounds__(HALO_NT) void conv_halo_hwc_kernel(const HaloHwcArgs a) {
-    constexpr int STAGE = BN * 128;      // bytes of a ring slot: one tap x 64 channels x BN filters
-    constexpr int LB = BN / 32;          // filter chunks per thread and stage
-    constexpr int FM = BN / 32, FN = 2;  // fragments per wave: filters x positions (64 positions per wave)
-    constexpr int MID = 1;               // half of a stage in front of which the next stage is certified
-    constexpr int NR = 2 * (FM + FN), NM = 2 * FM * FN;  // fragment reads / MFMAs per half stage (two k-steps)
-    static_assert(NS >= 3 && NS <= 7, "ring depth");
-    static_assert(NR <= NM, "one fragment read per MFMA");
-    extern __shared__ __align__(16) char smem[];
-    const unsigned halo_lds = (unsigned)(uintptr_t)(lds_char *)smem, ring_lds = halo_lds + 2 * HALO_BYTES;
-    const char *const halo = smem, *const ring = smem + 2 * HALO_BYTES;
-    const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const int l32 = lane & 31, kg = lane >> 5;
-    const int G = gridDim.x, UC = a.Cin / 64;
-    const long long K9 = 9ll * a.Cin;
-    const int cin2 = a.Cin * 2;
-    const unsigned HvWv = (unsigned)(a.Hv * a.Wv);
-
-    unsigned voff_b[LB];
-#pragma unroll
-    for (int i = 0; i < LB; ++i) {
-        const int row = (wave + 4 * i) * 8 + (lane >> 3);
-        voff_b[i] = (unsigned)(row * K9 * 2) + (unsigned)((((lane & 7) ^ swz(row))) << 4);
-    }
-    unsigned wfrag[4];
-#pragma unroll
-    for (int ks = 0; ks < 4; ++ks) wfrag[ks] = (unsigned)(l32 * 128 + (((2 * ks + kg) ^ swz(l32)) << 4));
-
-    struct Unit {
-        int tile, cs;
-        const char *fb;  // filters of (filter tile, channel slab)
-        unsigned p0;     // virtual position of the tile's first row
-        unsigned rem0;   // row of the tile's first position within its sample's rows
-    };
+    // The divisions that locate a tile and the 64-bit products behind its addresses are about a hundred scalar
+    // instructions: once per unit, not once per load.
     auto make_unit = [&](int tile, int cs) {
-        Unit u;
+        HaloUnit u;
         u.tile = tile;
         u.cs = cs;
         const unsigned pt = (unsigned)tile / (unsigned)a.ct_count, ct = (unsigned)tile - pt * (unsigned)a.ct_count;
         const unsigned q0 = pt * HALO_BM, b0 = q0 / a.qimg;
         u.rem0 = q0 - b0 * a.qimg;
-        u.p0 = q0 + b0 * a.jump;  // (the host keeps batch * Hv * Wv + the tile's reach below 2^31)
+        u.p0 = q0 + b0 * a.jump;  // (the host keeps the positions, a tile's reach included, below 2^31)
         u.fb = a.wr + ((long long)ct * BN * K9 + cs * 64) * 2;
+        u.hb = HWC ? a.xb + cs * 128 : a.xb + ((long long)(cs * 8 + 2 * wave) * a.P + u.p0) * 16;
         return u;
     };
     // tile-local position of the row of this lane's fragment j: its row number plus `jump` per sample boundary
     // between the tile's first row and its own
-    auto lane_rows = [&](const Unit &u, unsigned (&row)[FN]) {
+    auto lane_rows = [&](const HaloUnit &u, unsigned (&row)[FN]) {
 #pragma unroll
         for (int j = 0; j < FN; ++j) {
-            const unsigned r = (unsigned)(64 * wave + 32 * j + l32), v = u.rem0 + r;
+            const unsigned r = (unsigned)(64 * wave + 16 * j + l16), v = u.rem0 + r;
             unsigned skip = 0;
             for (unsigned k = 1, lim = a.qimg; k <= a.maxcross; ++k, lim += a.qimg) skip += v >= lim ? a.jump : 0u;
             row[j] = r + skip;
         }
     };
-    auto next_unit = [&](const Unit &u) {
+    auto next_unit = [&](const HaloUnit &u) {
         if (u.cs + 1 < UC) return make_unit(u.tile, u.cs + 1);
         if (u.tile + G < a.tiles) return make_unit(u.tile + G, 0);
         return u;  // past the end: the same unit again
     };
-    auto issue_filter = [&](const Unit &u, int tap, unsigned slot_lds, int i) {
+    // load i of a filter stage / piece q (0 .. 11) of a unit's input tile
+    auto issue_filter = [&](const HaloUnit &u, int tap, unsigned slot_lds, int i) {
         lds_dma16_saddr(voff_b[i], u.fb + tap * cin2, slot_lds + (unsigned)((wave + 4 * i) * 1024));
     };
-    // piece q (0 .. 11) of a unit's input tile: eight positions x the slab's eight chunks per wave
-    auto issue_piece = [&](const Unit &u, unsigned buf_lds, int q) {
-        const unsigned pl = (unsigned)((wave + 4 * q) * 8 + (lane >> 3));  // tile-local position
-        const unsigned pv = u.p0 + pl;
-        const unsigned b = fast_div31(pv, a.m_img, a.s_img), rem = pv - b * HvWv;
-        const unsigned yv = fast_div31(rem, a.m_row, a.s_row), xv = rem - yv * (unsigned)a.Wv;
-        const bool ok = b < (unsigned)a.batch && yv >= 1u && xv >= 1u;
-        const unsigned chunk = (unsigned)(((lane & 7) ^ swz((int)pl)) << 4);
-        const unsigned pix = (b * (unsigned)a.H + yv - 1u) * (unsigned)a.W + xv - 1u;  // < 2^31 / Cin
-        const char *src = ok ? a.x + ((size_t)pix * (unsigned)cin2 + (unsigned)(u.cs * 128) + chunk) : a.zeros + chunk;
-        lds_dma<16>(src, buf_lds + (unsigned)((wave + 4 * q) * 1024));
+    auto issue_piece = [&](const HaloUnit &u, unsigned buf_lds, int q) {
+        if constexpr (HWC) {
+            // eight positions x the slab's eight chunks per wave and piece
+            const unsigned pl = (unsigned)((wave + 4 * q) * 8 + (lane >> 3));  // tile-local position
+            const unsigned pv = u.p0 + pl;
+            const unsigned b = fast_div31(pv, a.m_img, a.s_img), rem = pv - b * HpWp;
+            const unsigned yv = fast_div31(rem, a.m_row, a.s_row), xv = rem - yv * (unsigned)a.Wp;
+            const bool ok = b < (unsigned)a.batch && yv >= 1u && xv >= 1u;
+            const unsigned chunk = (unsigned)(((lane & 7) ^ swz((int)pl)) << 4);
+            const unsigned pix = (b * (unsigned)a.Ho + yv - 1u) * (unsigned)a.Wo + xv - 1u;  // < 2^31 / Cin
+            const char *src = ok ? u.hb + ((size_t)pix * (unsigned)cin2 + chunk) : a.zeros + chunk;
+            lds_dma<16>(src, buf_lds + (unsigned)((wave + 4 * q) * 1024));
+        } else {
+            // pieces 0..5: block 2 * wave, pieces 6..11: block 2 * wave + 1; 64 positions each
+            const char *base = u.hb + (q >= 6 ? P16 : 0ll) + (q % 6) * 1024;
+            lds_dma16_saddr(voff_h, base, buf_lds + (unsigned)(((2 * wave + q / 6) * HALO_NP + (q % 6) * 64) * 16));
+        }
     };
 
-    Unit cu = make_unit(blockIdx.x, 0), nu = next_unit(cu);
+    HaloUnit cu = make_unit(blockIdx.x, 0), nu = next_unit(cu);
     int hb = 0;
     unsigned slot_off = 0, prev_off = (NS - 1) * STAGE;  // ring slot of the current stage / of the stage before it
 #pragma unroll
@@ -402,35 +215,43 @@ __global__ __launch_bounds__(HALO_NT) void conv_halo_hwc_kernel(const HaloHwcArg
     wait_vmcnt<(NS - 2) * LB>();
     __syncthreads();  // stage 0 of the first unit has landed
 
-    // fragment sets (two k-steps of 16 each): the one being multiplied and the one being read
-    uint4 wf[2][2][FM], xf[2][2][FN];
+    // fragment sets (one k-step of 32 each): the one being multiplied and the one being read
+    uint4 wf[2][FM], xf[2][FN];
     unsigned xrow[FN], xrow_next[FN];
     lane_rows(cu, xrow);
     lane_rows(nu, xrow_next);
-    // per fragment j of the tap being read: (row << 7) and the swizzle term ((kg << 4) ^ swizzle(row) << 4)
+    // per position fragment j of the tap being read: channel-major, the byte offset of (k group, row) in a tile whose
+    // channel blocks are HALO_NP chunks apart; channel-minor, (row << 7) and the swizzle term of the row
     unsigned xa[FN], xt[FN];
     auto tap_addresses = [&](const unsigned (&row)[FN], int shift) {
 #pragma unroll
         for (int j = 0; j < FN; ++j) {
             const unsigned rt = row[j] + (unsigned)shift;
-            xa[j] = rt << 7;
-            xt[j] = ((rt << 3) & 0x70u) ^ (unsigned)(kg << 4);
+            if constexpr (HWC) {
+                xa[j] = rt << 7;
+                xt[j] = ((rt << 3) & 0x70u) ^ (unsigned)(kq << 4);
+            } else {
+                xa[j] = (unsigned)(kq * HALO_NP + rt) * 16u;
+            }
         }
     };
-    // read r (0 .. NR - 1) of the fragments of the pair of k-steps `half` of a stage: per k-step the filter fragments,
-    // then the position fragments
-    auto read_frag = [&](int set, const char *wbase, const char *xbuf, int half, int r) {
-        const int h = r / (FM + FN), k = r % (FM + FN), ks = 2 * half + h;
-        if (k < FM)
-            wf[set][h][k] = *reinterpret_cast<const uint4 *>(wbase + wfrag[ks] + k * 32 * 128);
-        else
-            xf[set][h][k - FM] = *reinterpret_cast<const uint4 *>(xbuf + (xa[k - FM] + (xt[k - FM] ^ (unsigned)(ks << 5))));
+    // read r (0 .. NR - 1) of the fragments of k-step ks of a stage, in the order the MFMAs first need them: the first
+    // filter fragment, the position fragments, the other filter fragments
+    auto read_frag = [&](int set, const char *wbase, const char *xbuf, int ks, int r) {
+        if (r == 0 || r > FN) {
+            const int i = r == 0 ? 0 : r - FN;
+            wf[set][i] = *reinterpret_cast<const uint4 *>(wbase + wfrag[ks] + i * 16 * 128);
+        } else if constexpr (HWC) {
+            xf[set][r - 1] = *reinterpret_cast<const uint4 *>(xbuf + (xa[r - 1] + (xt[r - 1] ^ (unsigned)(ks << 6))));
+        } else {
+            xf[set][r - 1] = *reinterpret_cast<const uint4 *>(xbuf + xa[r - 1] + 4 * ks * HALO_NP * 16);
+        }
     };
     tap_addresses(xrow, 0);
 #pragma unroll
     for (int r = 0; r < NR; ++r) read_frag(0, ring, halo, 0, r);
 
-    f32x16 acc[FM][FN];
+    f32x4 acc[FM][FN];
     while (true) {
         if (cu.cs == 0) {
 #pragma unroll
@@ -438,7 +259,7 @@ __global__ __launch_bounds__(HALO_NT) void conv_halo_hwc_kernel(const HaloHwcArg
 #pragma unroll
                 for (int j = 0; j < FN; ++j)
 #pragma unroll
-                    for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.f;
+                    for (int v = 0; v < 4; ++v) acc[i][j][v] = 0.f;
         }
         const char *xbase = halo + hb * HALO_BYTES, *xnext = halo + (hb ^ 1) * HALO_BYTES;
         const unsigned next_lds = halo_lds + (unsigned)((hb ^ 1) * HALO_BYTES);
@@ -449,38 +270,42 @@ __global__ __launch_bounds__(HALO_NT) void conv_halo_hwc_kernel(const HaloHwcArg
             constexpr int ahead = sidx + NS - 1;
             constexpr int np = half == MID ? pipe_pieces<NS>(sidx) : 0, q0 = pipe_piece0<NS>(sidx);
             constexpr int nd = half == MID ? LB + np : 0;
-            static_assert(nd <= NM, "one load per MFMA");
+            constexpr int dstep = nd > 0 ? (NM - NR) / nd : 1;  // MFMAs between two loads
+            static_assert(dstep >= 1, "fragment reads first, then the loads spread over the other MFMAs");
             if constexpr (half == MID) {
                 // certify stage sidx + 1; every wave has then left stage sidx - 1
                 wait_vmcnt<pipe_wait<NS, LB>(sidx)>();
-                // (a bare barrier: fragment reads still in flight address slots that nobody refills now)
+                // (a bare barrier: fragment reads still in flight address slots that nobody refills now, so they
+                // need not be waited for here)
                 asm volatile("s_barrier" ::: "memory");
             }
-            // fragments of the next pair of k-steps
+            // fragments of the next k-step
             constexpr int gn = g + 1, sn = (gn / 2) % 9, hn = gn % 2;
             const unsigned noff = hn == 0 ? (slot_off + STAGE == NS * STAGE ? 0u : slot_off + STAGE) : slot_off;
             const char *wnext = ring + noff, *xbuf = gn < 18 ? xbase : xnext;
             if constexpr (hn == 0) {  // a new tap (of the next unit's tile behind the last stage)
-                const int shift = (sn / 3) * a.Wv + sn % 3;
+                const int shift = (sn / 3) * a.Wp + sn % 3;
                 if constexpr (gn < 18)
                     tap_addresses(xrow, shift);
                 else
                     tap_addresses(xrow_next, shift);
             }
-            // One fragment read and at most one load behind each MFMA, in exactly this order (nothing may cross a
-            // sched_barrier): the address arithmetic of the loads sits between the MFMAs, not in front of them.
+            // One fragment read behind each of the first MFMAs, then the loads spread over the others, in exactly this
+            // order (nothing may cross a sched_barrier): the address arithmetic of a load sits between two MFMAs
+            // instead of in front of a run of them.
             static_for<0, NM>([&](auto MI) {
-                constexpr int m = decltype(MI)::value, h = m / (FM * FN), i = (m % (FM * FN)) / FN, j = m % FN;
+                constexpr int m = decltype(MI)::value, i = m / FN, j = m % FN;
                 if constexpr (m < NR) read_frag(cur ^ 1, wnext, xbuf, hn, m);
-                mfma_step<half_t>(acc[i][j], wf[cur][h][i], xf[cur][h][j]);
-                if constexpr (m < nd) {
-                    if constexpr (m < LB) {
+                mfma16(acc[i][j], wf[cur][i], xf[cur][j]);
+                if constexpr (m >= NR && (m - NR) % dstep == 0 && (m - NR) / dstep < nd) {
+                    constexpr int d = (m - NR) / dstep;
+                    if constexpr (d < LB) {
                         if constexpr (ahead < 9)
-                            issue_filter(cu, ahead, ring_lds + prev_off, m);
+                            issue_filter(cu, ahead, ring_lds + prev_off, d);
                         else
-                            issue_filter(nu, ahead - 9, ring_lds + prev_off, m);
+                            issue_filter(nu, ahead - 9, ring_lds + prev_off, d);
                     } else {
-                        issue_piece(nu, next_lds, q0 + m - LB);
+                        issue_piece(nu, next_lds, q0 + d - LB);
                     }
                 }
                 __builtin_amdgcn_sched_barrier(0);
@@ -494,26 +319,33 @@ __global__ __launch_bounds__(HALO_NT) void conv_halo_hwc_kernel(const HaloHwcArg
         if (tile_done) {
             const unsigned q0 = ((unsigned)cu.tile / (unsigned)a.ct_count) * HALO_BM;
             const int co0 = (cu.tile % a.ct_count) * BN;
+            const unsigned PO = (unsigned)(a.Ho * a.Wo);
 #pragma unroll
             for (int j = 0; j < FN; ++j) {
-                const unsigned q = q0 + (unsigned)(64 * wave + 32 * j + l32);  // (Q < 2^31 on the host)
+                const unsigned q = q0 + (unsigned)(64 * wave + 16 * j + l16);  // (Q < 2^31 on the host)
                 const unsigned b = q / a.qimg, rem = q - b * a.qimg;
-                const unsigned yy = rem / (unsigned)a.Wv, xx = rem - yy * (unsigned)a.Wv;
-                if (q < a.Q && yy < (unsigned)a.H && xx < (unsigned)a.W) {
-                    // a lane holds runs of four consecutive filters of its position: 8-byte stores
-                    half_t *dst = a.y + ((size_t)(b * (unsigned)a.H + yy) * (unsigned)a.W + xx) * (unsigned)a.Cout + co0 + 4 * kg;
+                const unsigned yy = rem / (unsigned)a.Wp, xx = rem - yy * (unsigned)a.Wp;
+                if (q < a.Q && yy < (unsigned)a.Ho && xx < (unsigned)a.Wo) {
+                    // a lane holds four consecutive filters of its position per filter fragment
+                    if constexpr (HWC) {
+                        half_t *dst = a.y + ((size_t)b * PO + yy * (unsigned)a.Wo + xx) * (unsigned)a.Cout + co0 + 4 * kq;
 #pragma unroll
-                    for (int i = 0; i < FM; ++i)
-#pragma unroll
-                        for (int vg = 0; vg < 4; ++vg) {
+                        for (int i = 0; i < FM; ++i) {
                             union {
                                 half_t e[4];
                                 uint2 v;
                             } o;
 #pragma unroll
-                            for (int e = 0; e < 4; ++e) o.e[e] = (half_t)acc[i][j][4 * vg + e];
-                            *reinterpret_cast<uint2 *>(dst + i * 32 + 8 * vg) = o.v;
+                            for (int v = 0; v < 4; ++v) o.e[v] = (half_t)acc[i][j][v];
+                            *reinterpret_cast<uint2 *>(dst + i * 16) = o.v;
                         }
+                    } else {
+                        half_t *dst = a.y + ((size_t)b * a.Cout + co0 + 4 * kq) * PO + yy * (unsigned)a.Wo + xx;
+#pragma unroll
+                        for (int i = 0; i < FM; ++i)
+#pragma unroll
+                            for (int v = 0; v < 4; ++v) dst[(size_t)(i * 16 + v) * PO] = (half_t)acc[i][j][v];
+                    }
                 }
             }
         }
@@ -529,21 +361,22 @@ __global__ __launch_bounds__(HALO_NT) void conv_halo_hwc_kernel(const HaloHwcArg
     wait_vmcnt<0>();  // nothing may still be landing in LDS when the workgroup ends
 }
 
-template <int BN, int NS>
-int launch_halo_hwc(const HaloHwcArgs &a, int grid, hipStream_t stream) {
+template <int BN, int NS, bool HWC>
+int launch_halo(const HaloArgs &a, int grid, hipStream_t stream) {
     constexpr int lds = 2 * HALO_BYTES + NS * BN * 128;
     static_assert(lds <= 160 * 1024, "LDS");
     static bool attr = false;
     if (!attr) {
-        if (!hip_ok(hipFuncSetAttribute((const void *)conv_halo_hwc_kernel<BN, NS>,
+        if (!hip_ok(hipFuncSetAttribute((const void *)conv_halo_kernel<BN, NS, HWC>,
                                         hipFuncAttributeMaxDynamicSharedMemorySize, lds),
                     "halo convolution LDS size"))
             return 2;
         attr = true;
     }
-    hipLaunchKernelGGL((conv_halo_hwc_kernel<BN, NS>), dim3((unsigned)grid), dim3(HALO_NT), lds, stream, a);
+    hipLaunchKernelGGL((conv_halo_kernel<BN, NS, HWC>), dim3((unsigned)grid), dim3(HALO_NT), lds, stream, a);
     return hip_ok(hipGetLastError(), "halo convolution launch") ? 0 : 2;
 }
+
 
 // ---------------------------------------------------------------------------------------------------------
 // Weight gradient on the same layouts:
@@ -753,22 +586,23 @@ int conv_halo_launch(const ConvTileDesc &d, const void *xb, const void *wr, void
     a.wr = static_cast<const char *>(wr);
     a.y = static_cast<half_t *>(Y);
     a.P = pstride > 0 ? pstride : (long long)d.batch * Hp * Wp;
+    if (a.P + HALO_NP >= ((long long)1 << 31)) return -1;
     // leave the bottom rows of every padded grid out when a tile that crosses sample boundaries still fits
     const int qs = d.Ho * Wp, crossings = (HALO_BM - 1 + qs - 1) / qs;
     const bool skip = Hp > d.Ho && HALO_BM + (crossings + 1) * (Hp - d.Ho) * Wp + 2 <= HALO_NP;
     a.qimg = (unsigned)(skip ? qs : Hp * Wp);
     a.jump = (unsigned)(skip ? (Hp - d.Ho) * Wp : 0);
+    a.maxcross = (unsigned)(skip ? crossings : 0);
     a.Q = (unsigned)((long long)d.batch * a.qimg);
-    a.Cin = d.Cin; a.Cout = d.Cout; a.Hp = Hp; a.Wp = Wp; a.Ho = d.Ho; a.Wo = d.Wo;
+    a.batch = d.batch; a.Cin = d.Cin; a.Cout = d.Cout; a.Hp = Hp; a.Wp = Wp; a.Ho = d.Ho; a.Wo = d.Wo;
     const int bn = d.Cout % 128 == 0 ? 128 : 64;
     a.ct_count = d.Cout / bn;
     const long long ptiles = ((long long)a.Q + HALO_BM - 1) / HALO_BM;
     if (ptiles * a.ct_count >= (1ll << 30)) return -1;
     a.tiles = (int)(ptiles * a.ct_count);
     const int grid = a.tiles < st.num_cu ? a.tiles : st.num_cu;
-    return bn == 128 ? launch_halo_pipe<128, 4>(a, grid, st.stream) : launch_halo_pipe<64, 6>(a, grid, st.stream);
+    return bn == 128 ? launch_halo<128, 4, false>(a, grid, st.stream) : launch_halo<64, 6, false>(a, grid, st.stream);
 }
-
 
 // Channel-minor 3x3 "same" layers (one row / column of padding on every side), unit stride, whole 64-channel slabs
 // on both sides, rows short enough for a tile and its reach to fit the LDS buffer, 16-byte aligned tensors.
@@ -791,30 +625,30 @@ static void magic31(unsigned d, unsigned *m, int *s) {  // d >= 2
 // X: [batch][H][W][Cin], wr: tap-major filters [Cout][9][Cin], Y: [batch][H][W][Cout].
 int conv_halo_hwc_launch(const ConvTileDesc &d, const void *X, const void *wr, void *Y) {
     State &st = state();
-    HaloHwcArgs a = {};
-    a.x = static_cast<const char *>(X);
+    HaloArgs a = {};
+    a.xb = static_cast<const char *>(X);
     a.zeros = static_cast<const char *>(st.zeros);
     a.wr = static_cast<const char *>(wr);
     a.y = static_cast<half_t *>(Y);
-    a.batch = d.batch; a.Cin = d.Cin; a.Cout = d.Cout; a.H = d.Hin; a.W = d.Win;
-    a.Hv = d.Hin + 1; a.Wv = d.Win + 1;
+    a.batch = d.batch; a.Cin = d.Cin; a.Cout = d.Cout; a.Ho = d.Hin; a.Wo = d.Win;
+    a.Hp = d.Hin + 1; a.Wp = d.Win + 1;
     // leave the zero row of every sample out of the row enumeration when a tile that crosses sample boundaries and
     // its reach (two rows and two positions) still fit
-    const int qs = d.Hin * a.Wv, crossings = (HALO_BM - 1 + qs - 1) / qs;
-    const bool skip = HALO_BM + crossings * a.Wv + 2 * a.Wv + 2 <= HALO_NP;
-    a.qimg = (unsigned)(skip ? qs : a.Hv * a.Wv);
-    a.jump = (unsigned)(skip ? a.Wv : 0);
+    const int qs = d.Hin * a.Wp, crossings = (HALO_BM - 1 + qs - 1) / qs;
+    const bool skip = HALO_BM + crossings * a.Wp + 2 * a.Wp + 2 <= HALO_NP;
+    a.qimg = (unsigned)(skip ? qs : a.Hp * a.Wp);
+    a.jump = (unsigned)(skip ? a.Wp : 0);
     a.maxcross = (unsigned)(skip ? crossings : 0);
     a.Q = (unsigned)((long long)d.batch * a.qimg);
-    magic31((unsigned)(a.Hv * a.Wv), &a.m_img, &a.s_img);
-    magic31((unsigned)a.Wv, &a.m_row, &a.s_row);
+    magic31((unsigned)(a.Hp * a.Wp), &a.m_img, &a.s_img);
+    magic31((unsigned)a.Wp, &a.m_row, &a.s_row);
     const int bn = d.Cout % 128 == 0 ? 128 : 64;
     a.ct_count = d.Cout / bn;
     const long long ptiles = ((long long)a.Q + HALO_BM - 1) / HALO_BM;
     if (ptiles * a.ct_count >= (1ll << 30)) return -1;
     a.tiles = (int)(ptiles * a.ct_count);
     const int grid = a.tiles < st.num_cu ? a.tiles : st.num_cu;
-    return bn == 128 ? launch_halo_hwc<128, 4>(a, grid, st.stream) : launch_halo_hwc<64, 6>(a, grid, st.stream);
+    return bn == 128 ? launch_halo<128, 4, true>(a, grid, st.stream) : launch_halo<64, 6, true>(a, grid, st.stream);
 }
 
 bool conv_halo_wg_fits(const ConvTileDesc &d, int Hp, int Wp) {
