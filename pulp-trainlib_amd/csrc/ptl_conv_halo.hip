@@ -575,7 +575,7 @@ long long conv_halo_margin() { return HALO_BM + HALO_NP; }
 
 bool conv_halo_fits(const ConvTileDesc &d, int Hp, int Wp) {
     return !d.in_hwc && d.KH == 3 && d.KW == 3 && d.sh == 1 && d.sw == 1 && d.Cin % 64 == 0 && d.Cout % 64 == 0 &&
-           2 * Wp + 2 <= HALO_NP - HALO_BM && d.Ho == Hp - 2 && d.Wo == Wp - 2;
+           2 * Wp + 2 <= HALO_NP - HALO_BM && conv_output_fits_pads(d) && Hp >= d.Ho && Wp >= d.Wo;
 }
 
 // xb: blocked, padded input with conv_halo_margin() readable chunks after the last block; wr: tap-major filters.
@@ -589,7 +589,9 @@ int conv_halo_launch(const ConvTileDesc &d, const void *xb, const void *wr, void
     if (a.P + HALO_NP >= ((long long)1 << 31)) return -1;
     // leave the bottom rows of every padded grid out when a tile that crosses sample boundaries still fits
     const int qs = d.Ho * Wp, crossings = (HALO_BM - 1 + qs - 1) / qs;
-    const bool skip = Hp > d.Ho && HALO_BM + (crossings + 1) * (Hp - d.Ho) * Wp + 2 <= HALO_NP;
+    // (a tile's positions: its rows, the rows skipped at the boundaries it crosses, and its reach of two rows and two
+    // positions)
+    const bool skip = Hp > d.Ho && HALO_BM + crossings * (Hp - d.Ho) * Wp + 2 * Wp + 2 <= HALO_NP;
     a.qimg = (unsigned)(skip ? qs : Hp * Wp);
     a.jump = (unsigned)(skip ? (Hp - d.Ho) * Wp : 0);
     a.maxcross = (unsigned)(skip ? crossings : 0);
@@ -653,7 +655,8 @@ int conv_halo_hwc_launch(const ConvTileDesc &d, const void *X, const void *wr, v
 
 bool conv_halo_wg_fits(const ConvTileDesc &d, int Hp, int Wp) {
     return !d.in_hwc && d.KH == 3 && d.KW == 3 && d.sh == 1 && d.sw == 1 && d.Cin % 64 == 0 && d.Cout % 128 == 0 &&
-           2 * Wp + 2 <= 128 && d.Ho == Hp - 2 && d.Wo == Wp - 2 && (long long)d.batch * Hp * Wp < ((long long)1 << 31);
+           2 * Wp + 2 <= 128 && conv_output_fits_pads(d) && Hp >= d.Ho && Wp >= d.Wo &&
+           (long long)d.batch * Hp * Wp < ((long long)1 << 31);
 }
 // Measured against the alternatives (fp16): at batch 128..512, 128 -> 128 on 28x28 73 / 243 against 87 / 306 us
 // (resident output tile kernel), 256 -> 256 on 14x14 70 against 83 us and on 28x28 384 against 390 us, 512 -> 512 on
@@ -662,7 +665,8 @@ bool conv_halo_wg_fits(const ConvTileDesc &d, int Hp, int Wp) {
 // kernel), with 128 channels only from about a hundred (128 -> 128 on 14x14 at batch 32: 28
 // against 25 us for the resident output tile kernel).  64 -> 128 on 56x56 (280 against 274 us) stays where it was.
 bool conv_halo_wg_preferred(const ConvTileDesc &d) {
-    const int Hp = d.Hin + d.padU + d.padD, Wp = d.Win + d.padL + d.padR;
+    int Hp, Wp;
+    conv_padded_grid(d, &Hp, &Wp);
     const long long units = ((long long)d.batch * Hp * Wp + HWG_UNIT - 1) / HWG_UNIT;
     const int cmin = d.Cin < d.Cout ? d.Cin : d.Cout;
     return conv_halo_wg_fits(d, Hp, Wp) && Wp <= 32 && units >= (cmin >= 256 ? 20 : 96);

@@ -159,8 +159,10 @@ int conv_taps(const ConvTileDesc &d, const void *X, const void *Wt, void *Y, con
     const bool hwc = d.in_hwc != 0;
     if (d.sh != 1 || d.sw != 1 || d.Cin % SK) return -1;
     if (hwc ? reinterpret_cast<uintptr_t>(X) % 16 != 0 : d.x_sy != d.Win) return -1;
-    const int Hp = d.Hin + d.padU + d.padD, Wp = d.Win + d.padL + d.padR, taps = d.KH * d.KW;
-    if (d.Ho != Hp - d.KH + 1 || d.Wo != Wp - d.KW + 1 || taps < 2) return -1;
+    const int taps = d.KH * d.KW;
+    int Hp, Wp;
+    conv_padded_grid(d, &Hp, &Wp);
+    if (!conv_output_fits_pads(d) || taps < 2) return -1;
     const int cblocks = d.Cin / VEC;
     const long long plane = (long long)Hp * Wp * VEC;            // elements of one (channel block, sample) plane
     const long long xb_elems = (long long)cblocks * d.batch * plane;
@@ -207,7 +209,8 @@ int conv_taps(const ConvTileDesc &d, const void *X, const void *Wt, void *Y, con
     }
     const bool halo = ES == 2 && !hwc && conv_halo_fits(d, Hp, Wp) && (long long)d.batch * Hp * Wp < ((long long)1 << 31) &&
                       (st.gemm_path == 5 || (st.gemm_path == 0 && halo_pays));
-    const long long margin = halo ? conv_halo_margin() : 0;  // chunks the resident-tile kernel may read past the end
+    // chunks read past the end: the resident-tile kernel's reach, or the window of the last sample's last pixels
+    const long long margin = halo ? conv_halo_margin() : ((long long)(d.KH - 1) * Wp + d.KW) * (hwc ? cblocks : 1);
     // the blocked input goes to the caller's buffer when the call brought one (the weight gradient of the layer
     // reads the same copy), else to scratch memory like the filters
     const size_t xb_bytes = (size_t)(xb_elems + margin * VEC) * ES;
@@ -377,7 +380,8 @@ int conv_taps_wg(const ConvTileDesc &d, const void *X, const void *dY, void *dW)
     if (d.sh != 1 || d.sw != 1 || d.Cin % VEC) return -1;
     if constexpr (ES == 2) {
         // 3x3 channel-major layers: both operands channel-blocked, tiles resident in LDS for all taps
-        const int Hp = d.Hin + d.padU + d.padD, Wp = d.Win + d.padL + d.padR;
+        int Hp, Wp;
+        conv_padded_grid(d, &Hp, &Wp);
         if (!hwc && d.x_sy == d.Win && conv_halo_wg_fits(d, Hp, Wp) &&
             (st.gemm_path == 5 || (st.gemm_path == 0 && conv_halo_wg_preferred(d)))) {
             const long long P = (long long)d.batch * Hp * Wp, margin = conv_halo_wg_margin();
@@ -421,12 +425,14 @@ int conv_taps_wg(const ConvTileDesc &d, const void *X, const void *dY, void *dW)
         if (st.gemm_path != 3 && (d.Cin < 128 || d.Cout < 128)) return -1;  // measured: below that the direct kernel wins
         // (and below about 8000 padded positions the gathering GEMM does: 12 against 29 us for eight 256 -> 256 7x7
         // samples, 25 against 27 us for 128 -> 128 on 14x14 at batch 32)
-        if (st.gemm_path != 3 && (long long)d.batch * (d.Hin + d.padU + d.padD) * (d.Win + d.padL + d.padR) < 8192)
+        if (st.gemm_path != 3 && (long long)d.batch * (d.Hin + 2) * (d.Win + 2) < 8192)
             return -1;
     }
     if (st.gemm_path == 2) return -1;
-    const int Hp = d.Hin + d.padU + d.padD, Wp = d.Win + d.padL + d.padR, taps = d.KH * d.KW;
-    if (d.Ho != Hp - d.KH + 1 || d.Wo != Wp - d.KW + 1) return -1;
+    const int taps = d.KH * d.KW;
+    int Hp, Wp;
+    conv_padded_grid(d, &Hp, &Wp);
+    if (!conv_output_fits_pads(d)) return -1;
     const int cblocks = d.Cin / VEC;
     const long long plane = (long long)Hp * Wp * VEC;
     const long long Kp = (long long)d.batch * Hp * Wp;              // padded positions of all samples
@@ -551,8 +557,9 @@ int conv_halo_bw(const ConvTileDesc &fwd, const ConvTileDesc &ig, const void *X,
     } else {
         State &st = state();
         constexpr int VEC = 8;
-        const int Hp = fwd.Hin + fwd.padU + fwd.padD, Wp = fwd.Win + fwd.padL + fwd.padR;
-        const int Hpi = ig.Hin + ig.padU + ig.padD, Wpi = ig.Win + ig.padL + ig.padR;
+        int Hp, Wp, Hpi, Wpi;
+        conv_padded_grid(fwd, &Hp, &Wp);
+        conv_padded_grid(ig, &Hpi, &Wpi);
         if (Hp != Hpi || Wp != Wpi || fwd.x_sy != fwd.Win || ig.x_sy != ig.Win) return -1;
         if (!conv_halo_fits(ig, Hp, Wp) || !conv_halo_wg_fits(fwd, Hp, Wp) || !conv_halo_wg_preferred(fwd)) return -1;
         if (!(st.gemm_path == 0 || st.gemm_path == 5)) return -1;

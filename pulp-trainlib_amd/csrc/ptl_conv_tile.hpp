@@ -98,6 +98,22 @@ inline int conv_raw_rows(int bm, int Ho, int Wo, int sh, int KH, int THP, long l
 template <typename T>
 int conv_taps(const ConvTileDesc &d, const void *X, const void *Wt, void *Y, const OutMap &c);
 
+// The padded grid of the tap-sum and resident-tile routes: every sample takes Hin + max(padU, padD) rows of
+// Win + max(padL, padR) positions, the tensor padU rows / padL columns inside it.  The zero rows above a sample are
+// also the zero rows below the one before it, the zero columns left of a row the ones right of the row before it
+// (a window that runs off a row's end continues at the start of the next row), so a 3x3 "same" layer pads by ONE
+// row and ONE column per sample instead of two: fewer bytes to write and read, and fewer positions that the
+// kernels compute and drop.  Behind the last sample of a channel block the next block's first rows (or the
+// margin behind the last block) are the zeros.
+inline void conv_padded_grid(const ConvTileDesc &d, int *Hp, int *Wp) {
+    *Hp = d.Hin + (d.padU > d.padD ? d.padU : d.padD);
+    *Wp = d.Win + (d.padL > d.padR ? d.padL : d.padR);
+}
+// whether the output is the "valid" convolution of the fully padded input (what these routes compute)
+inline bool conv_output_fits_pads(const ConvTileDesc &d) {
+    return d.Ho == d.Hin + d.padU + d.padD - d.KH + 1 && d.Wo == d.Win + d.padL + d.padR - d.KW + 1;
+}
+
 // 3x3 unit-stride fp16 channel-major layers with the input tile resident in LDS for all taps (same prepared
 // operands as the tap-sum route: blocked padded input with conv_halo_margin() readable chunks behind it, tap-major
 // filters).  Y is the dense channel-major output [batch][Cout][Ho][Wo].

@@ -1040,7 +1040,8 @@ size_t ptl_conv2d_fp16_cache_bytes(const struct Conv2D_args_fp16 *a, int ns) {
     d.Cout = g.Co; d.Ho = g.Ho; d.Wo = g.Wo;
     d.KH = 3; d.KW = 3; d.sh = 1; d.sw = 1;
     d.padU = g.Up; d.padD = g.Dp; d.padL = g.Lp; d.padR = g.Rp;
-    const int Hp = g.H + g.Up + g.Dp, Wp = g.W + g.Lp + g.Rp;
+    int Hp, Wp;
+    ptl::conv_padded_grid(d, &Hp, &Wp);
     if (!ptl::conv_halo_fits(d, Hp, Wp)) return 0;
     return ((size_t)(g.Ci / 8) * ns * Hp * Wp + (size_t)ptl::conv_halo_margin()) * 16;
 }

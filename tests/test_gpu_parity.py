@@ -246,7 +246,8 @@ RESIDENT_CASES = [
     (128, 9, 11, 64, (1, 1, 1, 1), 3, 1),
     (64, 12, 10, 128, (0, 2, 1, 0), 2, 1),
     (64, 7, 61, 64, (1, 1, 1, 1), 1, 1),
-    (64, 5, 62, 64, (1, 1, 1, 1), 1, 0),
+    (64, 5, 62, 64, (1, 1, 1, 1), 1, 1),    # the widest row whose reach (two rows of W + 1 positions + 2) fits
+    (64, 5, 63, 64, (1, 1, 1, 1), 1, 0),
     (192, 6, 6, 256, (0, 0, 0, 0), 2, 1),
     (64, 3, 3, 64, (0, 0, 0, 0), 1, 1),     # one output pixel per sample, a single ragged tile
     (64, 3, 5, 128, (1, 1, 1, 1), 1, 1),
