@@ -48,6 +48,7 @@ struct HaloArgs {
     int s_img, s_row;
     int batch, Cin, Cout, Hp, Wp, Ho, Wo;
     int tiles, ct_count;  // tile = position tile * ct_count + filter tile
+    int xcd_map;          // 1: the grid is a multiple of 8 and a workgroup's first tile follows its XCD
 };
 
 template <int I, int N, typename F>
@@ -203,7 +204,11 @@ __global__ __launch_bounds__(HALO_NT) void conv_halo_kernel(const HaloArgs a) {
         }
     };
 
-    HaloUnit cu = make_unit(blockIdx.x, 0), nu = next_unit(cu);
+    // Workgroups are dealt to the 8 XCDs in turn, each with an L2 of its own: XCD x takes the tiles [x * G/8, (x+1) * G/8)
+    // of every round, so that the filter tiles of one position tile - neighbours in the tile order, readers of the same
+    // input tile - and position tiles that overlap in their reach meet in one L2.
+    const int first_tile = a.xcd_map ? (int)(blockIdx.x & 7) * (G >> 3) + (int)(blockIdx.x >> 3) : (int)blockIdx.x;
+    HaloUnit cu = make_unit(first_tile, 0), nu = next_unit(cu);
     int hb = 0;
     unsigned slot_off = 0, prev_off = (NS - 1) * STAGE;  // ring slot of the current stage / of the stage before it
 #pragma unroll
@@ -270,7 +275,7 @@ __global__ __launch_bounds__(HALO_NT) void conv_halo_kernel(const HaloArgs a) {
             constexpr int ahead = sidx + NS - 1;
             constexpr int np = half == MID ? pipe_pieces<NS>(sidx) : 0, q0 = pipe_piece0<NS>(sidx);
             constexpr int nd = half == MID ? LB + np : 0;
-            constexpr int dstep = nd > 0 ? (NM - NR) / nd : 1;  // MFMAs between two loads
+            constexpr int dstep = (NM - NR) / (nd > 0 ? nd : 1);  // MFMAs between two loads
             static_assert(dstep >= 1, "fragment reads first, then the loads spread over the other MFMAs");
             if constexpr (half == MID) {
                 // certify stage sidx + 1; every wave has then left stage sidx - 1
@@ -403,6 +408,7 @@ struct HaloWgArgs {
     int tiles_ci;      // Cin / 64
     int tiles;         // (Cout / 128) * (Cin / 64)
     int S0, S1, smax;  // position splits of the two tap groups
+    int xcd_map;       // 1: bundles of `tiles` workgroups per XCD (see the kernel)
 };
 
 typedef short hwg_s4 __attribute__((ext_vector_type(4)));
@@ -516,11 +522,27 @@ __device__ inline void halo_wg_body(const HaloWgArgs &a, char *smem, int tile, i
 
 __global__ __launch_bounds__(HALO_NT) void conv_halo_wg_kernel(const HaloWgArgs a) {
     extern __shared__ __align__(16) char smem[];
-    const int id = blockIdx.x, n0 = a.tiles * a.S0;
-    if (id < n0)
-        halo_wg_body<0, 5>(a, smem, id / a.S0, id % a.S0, a.S0);
+    // The workgroups of one (tap group, position split) - one per tile of the weight tensor - stream the same
+    // positions at the same time: the gradient tile is read by the tiles of a filter block, the input tile by the
+    // tiles of a channel block.  Workgroups are dealt to the 8 XCDs in turn, so such a bundle takes every eighth
+    // workgroup: its tiles meet in one L2 (measured on 256 -> 256 channels, 28x28, batch 256: 9.4 M of the kernel's
+    // 14.5 M L2 requests missed with the bundles spread over the XCDs, 3.9 M this way; the run time did not change -
+    // the kernel runs against the board's power limit, not against its memory).
+    int tile, bundle;
+    if (a.xcd_map) {
+        const int xcd = blockIdx.x & 7, j = blockIdx.x >> 3;
+        tile = j % a.tiles;
+        bundle = (j / a.tiles) * 8 + xcd;
+        if (bundle >= a.S0 + a.S1) return;
+    } else {
+        const int id = blockIdx.x, n0 = a.tiles * a.S0;
+        tile = id < n0 ? id / a.S0 : (id - n0) / a.S1;
+        bundle = id < n0 ? id % a.S0 : a.S0 + (id - n0) % a.S1;
+    }
+    if (bundle < a.S0)
+        halo_wg_body<0, 5>(a, smem, tile, bundle, a.S0);
     else
-        halo_wg_body<5, 4>(a, smem, (id - n0) / a.S1, (id - n0) % a.S1, a.S1);
+        halo_wg_body<5, 4>(a, smem, tile, bundle - a.S0, a.S1);
 }
 
 // dW[idx * 9 + tap] = sum over the splits of the tap's group of ws[tap][split][idx]
@@ -603,6 +625,7 @@ int conv_halo_launch(const ConvTileDesc &d, const void *xb, const void *wr, void
     if (ptiles * a.ct_count >= (1ll << 30)) return -1;
     a.tiles = (int)(ptiles * a.ct_count);
     const int grid = a.tiles < st.num_cu ? a.tiles : st.num_cu;
+    a.xcd_map = grid % 8 == 0;
     return bn == 128 ? launch_halo<128, 4, false>(a, grid, st.stream) : launch_halo<64, 6, false>(a, grid, st.stream);
 }
 
@@ -650,6 +673,7 @@ int conv_halo_hwc_launch(const ConvTileDesc &d, const void *X, const void *wr, v
     if (ptiles * a.ct_count >= (1ll << 30)) return -1;
     a.tiles = (int)(ptiles * a.ct_count);
     const int grid = a.tiles < st.num_cu ? a.tiles : st.num_cu;
+    a.xcd_map = grid % 8 == 0;
     return bn == 128 ? launch_halo<128, 4, true>(a, grid, st.stream) : launch_halo<64, 6, true>(a, grid, st.stream);
 }
 
@@ -733,7 +757,9 @@ int conv_halo_wg_launch(const ConvTileDesc &d, const void *xb, const void *gb, l
             return 2;
         attr = true;
     }
-    hipLaunchKernelGGL(conv_halo_wg_kernel, dim3((unsigned)(a.tiles * (S0 + S1))), dim3(HALO_NT), lds, st.stream, a);
+    a.xcd_map = 1;
+    const int bundles = a.xcd_map ? (S0 + S1 + 7) / 8 * 8 : S0 + S1;
+    hipLaunchKernelGGL(conv_halo_wg_kernel, dim3((unsigned)(a.tiles * bundles)), dim3(HALO_NT), lds, st.stream, a);
     if (!hip_ok(hipGetLastError(), "halo weight-gradient launch")) return 2;
     const long long total = (long long)d.Cout * d.Cin;
     hipLaunchKernelGGL(conv_halo_wg_reduce_kernel, dim3((unsigned)((total + 255) / 256), 9), dim3(256), 0, st.stream, ws,
