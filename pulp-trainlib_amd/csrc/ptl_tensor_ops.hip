@@ -679,7 +679,12 @@ __global__ __launch_bounds__(256) void dw_direct_kernel(const half_t *__restrict
     if (id >= total) return;
     const unsigned per_plane = (unsigned)(rblocks * groups);
     const unsigned plane = id / per_plane, blk = id - plane * per_plane;
-    const int rb = (int)(blk / (unsigned)groups), c0 = (int)(blk - (unsigned)rb * groups) * 8, r0 = rb * RB;
+    // (the last column group and the last row block are moved back to end with the plane when it has at least one
+    // full group / block: they then overlap their neighbours, whose values they repeat, and every store is a whole
+    // 16-byte one)
+    const int rb = (int)(blk / (unsigned)groups);
+    const int c0 = Wd >= 8 ? min((int)(blk - (unsigned)rb * groups) * 8, Wd - 8) : 0;
+    const int r0 = Hd >= RB ? min(rb * RB, Hd - RB) : 0;
     const int ch = (int)(plane % (unsigned)C);
     dw_h2 we[3], wo[3];
     float w0[3], w2[3];
@@ -866,9 +871,9 @@ static void launch_dw_plane(const T *src, const T *Wt, T *dst, int C, int Hs, in
                             long planes, hipStream_t stream) {
     const size_t src_img = (size_t)Hs * Ws * sizeof(T) + 32;
     if constexpr (sizeof(T) == 2) {
-        // 3x3 with rows of whole dwords on both sides, forward geometry (every column group full): straight from
-        // global memory
-        if (K == 3 && !FLIP && Ws % 2 == 0 && Wd % 8 == 0 && pl % 2 == 0 && reinterpret_cast<uintptr_t>(src) % 4 == 0 &&
+        // 3x3 with rows of whole dwords on both sides and at least one group of eight columns: straight from global
+        // memory (forward, and the input gradient as the flipped correlation over the output gradient)
+        if (K == 3 && Ws % 2 == 0 && Wd % 2 == 0 && Wd >= 8 && pl % 2 == 0 && reinterpret_cast<uintptr_t>(src) % 4 == 0 &&
             reinterpret_cast<uintptr_t>(dst) % 4 == 0) {
             const int rblocks = (Hd + DW_DRB - 1) / DW_DRB, groups = (Wd + 7) / 8;
             const long long total = (long long)planes * rblocks * groups;
