@@ -429,7 +429,7 @@ __device__ inline void halo_wg_body(const HaloWgArgs &a, char *smem, int tile, i
     const unsigned lds0 = (unsigned)(uintptr_t)(lds_char *)smem;
     const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int wm = wave & 1, wn = wave >> 1;
-    const int i16 = lane & 15, g16 = (lane >> 4) & 1, kg = lane >> 5;
+    const int i16 = lane & 15, kq = lane >> 4;
     const int co_cb0 = (tile / a.tiles_ci) * 16, ci_cb0 = (tile % a.tiles_ci) * 8;
     const int u0 = (int)((long long)split * a.units / S), u1 = (int)((long long)(split + 1) * a.units / S);
     const unsigned voff = (unsigned)lane * 16u;
@@ -452,22 +452,25 @@ __device__ inline void halo_wg_body(const HaloWgArgs &a, char *smem, int tile, i
         }
     };
 
-    // this lane's piece of a transposing read: position k0 + i16 / 4 of channel block .. + (i16 & 3) / 2,
-    // channels 4 * (i16 & 1) .. + 3 of that block
-    const unsigned ga = (unsigned)((((wm * 8 + 2 * g16 + ((i16 & 3) >> 1)) * HWG_GP + 8 * kg + (i16 >> 2)) * 16) + (i16 & 1) * 8);
-    const unsigned xa = (unsigned)(HWG_GB + (((wn * 4 + 2 * g16 + ((i16 & 3) >> 1)) * HWG_XP + 8 * kg + (i16 >> 2)) * 16) +
-                                   (i16 & 1) * 8);
+    // A wave owns 64 filters x 32 channels x NT taps as 16 x 16 blocks (v_mfma_f32_16x16x32_f16: 32 positions per
+    // k-step, a lane holds row lane % 16 and positions 8 * (lane / 16) .. + 7 of the step).  This lane's piece of a
+    // transposing read: position k0 + i16 / 4 of channel block .. + (i16 & 3) / 2, channels 4 * (i16 & 1) .. + 3 of
+    // that block; the second read of a fragment is four positions on.
+    const unsigned ga = (unsigned)((((wm * 8 + ((i16 & 3) >> 1)) * HWG_GP + 8 * kq + (i16 >> 2)) * 16) + (i16 & 1) * 8);
+    const unsigned xa = (unsigned)(HWG_GB + (((wn * 4 + ((i16 & 3) >> 1)) * HWG_XP + 8 * kq + (i16 >> 2)) * 16) + (i16 & 1) * 8);
     int tapoff[NT];
 #pragma unroll
     for (int t = 0; t < NT; ++t) tapoff[t] = (((T0 + t) / 3) * a.Wp + (T0 + t) % 3) * 16;
 
-    f32x16 acc[2][NT];
+    f32x4 acc[4][2][NT];
 #pragma unroll
-    for (int i = 0; i < 2; ++i)
+    for (int i = 0; i < 4; ++i)
 #pragma unroll
-        for (int t = 0; t < NT; ++t)
+        for (int c = 0; c < 2; ++c)
 #pragma unroll
-            for (int v = 0; v < 16; ++v) acc[i][t][v] = 0.f;
+            for (int t = 0; t < NT; ++t)
+#pragma unroll
+                for (int v = 0; v < 4; ++v) acc[i][c][t][v] = 0.f;
 
     if (u0 < u1) issue(u0, 0);
     for (int u = u0; u < u1; ++u) {
@@ -476,30 +479,29 @@ __device__ inline void halo_wg_body(const HaloWgArgs &a, char *smem, int tile, i
         __syncthreads();  // unit u has landed for every wave, and every wave has left unit u - 1
         issue(u + 1 < u1 ? u + 1 : u, buf ^ 1);
         const char *gt = smem + buf * HWG_BUF + ga, *xt = smem + buf * HWG_BUF + xa;
-        uint4 gf[2][2], xf[2][NT];
+        uint4 gf[2][4], xf[2][2][NT];
         auto read = [&](int set, int ks) {
 #pragma unroll
-            for (int i = 0; i < 2; ++i) gf[set][i] = hwg_frag(gt + ks * 256 + i * 4 * HWG_GP * 16);
+            for (int i = 0; i < 4; ++i) gf[set][i] = hwg_frag(gt + ks * 512 + i * 2 * HWG_GP * 16);
 #pragma unroll
-            for (int t = 0; t < NT; ++t) xf[set][t] = hwg_frag(xt + ks * 256 + tapoff[t]);
+            for (int c = 0; c < 2; ++c)
+#pragma unroll
+                for (int t = 0; t < NT; ++t) xf[set][c][t] = hwg_frag(xt + ks * 512 + c * 2 * HWG_XP * 16 + tapoff[t]);
         };
         read(0, 0);
-        static_for<0, 8>([&](auto KI) {
+        static_for<0, 4>([&](auto KI) {
             constexpr int ks = decltype(KI)::value, cur = ks & 1;
-            if constexpr (ks + 1 < 8) read(cur ^ 1, ks + 1);
+            if constexpr (ks + 1 < 4) read(cur ^ 1, ks + 1);
 #pragma unroll
-            for (int i = 0; i < 2; ++i)
+            for (int i = 0; i < 4; ++i)
 #pragma unroll
-                for (int t = 0; t < NT; ++t) mfma_step<half_t>(acc[i][t], gf[cur][i], xf[cur][t]);
-            if constexpr (ks + 1 < 8) {
-                // 2 * (2 + NT) transposing reads under 2 * NT MFMAs
+                for (int c = 0; c < 2; ++c)
 #pragma unroll
-                for (int m = 0; m < 4; ++m) {
-                    __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
-                    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-                }
+                    for (int t = 0; t < NT; ++t) mfma16(acc[i][c][t], gf[cur][i], xf[cur][c][t]);
+            if constexpr (ks + 1 < 4) {
+                // 2 * (4 + 2 * NT) transposing reads under 8 * NT MFMAs: one read behind each of the first MFMAs
 #pragma unroll
-                for (int m = 4; m < 2 * NT; ++m) {
+                for (int m = 0; m < 2 * (4 + 2 * NT); ++m) {
                     __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
                     __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
                 }
@@ -508,15 +510,17 @@ __device__ inline void halo_wg_body(const HaloWgArgs &a, char *smem, int tile, i
     }
     wait_vmcnt<0>();  // nothing may still be landing in LDS when the workgroup ends
     if (u0 >= u1) return;
-    // partial sums: lane = channel, four consecutive filters per register group
-    const int co0 = (tile / a.tiles_ci) * 128 + wm * 64 + 4 * kg, ci = (tile % a.tiles_ci) * 64 + wn * 32 + (lane & 31);
+    // partial sums: lane = channel, four consecutive filters per block
+    const int co0 = (tile / a.tiles_ci) * 128 + wm * 64 + 4 * kq, ci0 = (tile % a.tiles_ci) * 64 + wn * 32 + i16;
 #pragma unroll
     for (int t = 0; t < NT; ++t) {
-        float *dst = a.ws + (((size_t)(T0 + t) * a.smax + split) * a.Cout + co0) * a.Cin + ci;
+        float *dst = a.ws + (((size_t)(T0 + t) * a.smax + split) * a.Cout + co0) * a.Cin + ci0;
 #pragma unroll
-        for (int i = 0; i < 2; ++i)
+        for (int i = 0; i < 4; ++i)
 #pragma unroll
-            for (int v = 0; v < 16; ++v) dst[(size_t)(i * 32 + 8 * (v >> 2) + (v & 3)) * a.Cin] = acc[i][t][v];
+            for (int c = 0; c < 2; ++c)
+#pragma unroll
+                for (int v = 0; v < 4; ++v) dst[(size_t)(i * 16 + v) * a.Cin + c * 16] = acc[i][c][t][v];
     }
 }
 
