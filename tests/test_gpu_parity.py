@@ -296,6 +296,15 @@ def test_conv2d_forward_leaves_its_blocked_input_for_the_gradients(pkg, gpu, cas
                     assert gpu.ptl_conv2d_fp16_wg_batched_cached(ctypes.byref(a3), ns, ctypes.byref(other)) == 0
                     gpu.ptl_sync()
                     assert torch.equal(dw3, dw2)
+                    # ... and a valid cache IS what the gradient reads: with every chunk of the copy (border included)
+                    # overwritten by 0x3c3c = 1.05859375, each filter's gradient is that constant times the sum of its
+                    # output gradient, whatever the tap and channel
+                    dw4 = torch.full_like(w, 3)
+                    a4, keep4 = hp.conv2d_args(pkg, x, None, w, dw4, y, dy, Ci, H, W, Co, 3, 3, Ho, Wo, pad, (1, 1))
+                    assert gpu.ptl_conv2d_fp16_wg_batched_cached(ctypes.byref(a4), ns, ctypes.byref(c)) == 0
+                    gpu.ptl_sync()
+                    want = (1.05859375 * dy.float().sum(dim=(0, 2, 3))).view(Co, 1, 1, 1).expand_as(w)
+                    assert float((dw4.float() - want).norm() / want.norm()) <= 2e-3
             else:
                 pkg.call("ptl_conv2d_fp16_fw_batched", a, ns)
                 pkg.call("ptl_conv2d_fp16_bw_batched", a, ns)
