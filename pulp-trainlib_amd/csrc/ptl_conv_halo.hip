@@ -409,6 +409,11 @@ struct HaloWgArgs {
     int tiles;         // (Cout / 128) * (Cin / 64)
     int S0, S1, smax;  // position splits of the two tap groups
     int xcd_map;       // 1: bundles of `tiles` workgroups per XCD (see the kernel)
+    // channel-minor tensors read in place (HWC = true): xb = X[batch][H][W][Cin], gb = dY[batch][H][W][Cout]
+    const char *zeros;
+    int batch, H, W, Hp;
+    unsigned m_img, m_row;
+    int s_img, s_row;
 };
 
 typedef short hwg_s4 __attribute__((ext_vector_type(4)));
@@ -424,7 +429,14 @@ __device__ inline uint4 hwg_frag(const char *p) {
     return t.v;
 }
 
-template <int T0, int NT>
+// HWC = true: the same tiles filled from channel-minor tensors where they lie.  The positions are those of the
+// virtual grid of the forward kernel (one zero row above and one zero column left of every sample, Hp = H + 1 rows
+// of Wp = W + 1 positions): position (b, yv, xv) of the gradient tile is dY[b][yv][xv] for yv < H and xv < W, of the
+// input tile X[b][yv - 1][xv - 1] for yv, xv >= 1, and a chunk of zeros otherwise.  A wave's load still fills 64
+// consecutive positions of one channel block in LDS; every lane gives its own address (16 bytes of its position's
+// pixel, pixels Cout or Cin elements apart) or that of the zero page, and the eight loads that take the eight blocks
+// of the same 128 bytes of a pixel follow each other in one wave.
+template <int T0, int NT, bool HWC>
 __device__ inline void halo_wg_body(const HaloWgArgs &a, char *smem, int tile, int split, int S) {
     const unsigned lds0 = (unsigned)(uintptr_t)(lds_char *)smem;
     const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -436,6 +448,40 @@ __device__ inline void halo_wg_body(const HaloWgArgs &a, char *smem, int tile, i
 
     auto issue = [&](int u, int buf) {
         const long long p0 = (long long)u * HWG_UNIT;
+        if constexpr (HWC) {
+            const unsigned HpWp = (unsigned)(a.Hp * a.Wp);
+            // this wave's piece of the gradient tile (64 positions from piece wave & 1) and of the input tile (piece wave)
+            const char *gsrc, *xsrc;
+            {
+                const unsigned pv = (unsigned)p0 + (unsigned)((wave & 1) * 64 + lane);
+                const unsigned b = fast_div31(pv, a.m_img, a.s_img), rem = pv - b * HpWp;
+                const unsigned yv = fast_div31(rem, a.m_row, a.s_row), xv = rem - yv * (unsigned)a.Wp;
+                const bool ok = b < (unsigned)a.batch && yv < (unsigned)a.H && xv < (unsigned)a.W;
+                const size_t pix = ((size_t)b * (unsigned)a.H + yv) * (unsigned)a.W + xv;
+                gsrc = ok ? a.gb + (pix * (unsigned)a.Cout + (unsigned)(co_cb0 * 8)) * 2 : nullptr;
+            }
+            {
+                const unsigned pv = (unsigned)p0 + (unsigned)(wave * 64 + lane);
+                const unsigned b = fast_div31(pv, a.m_img, a.s_img), rem = pv - b * HpWp;
+                const unsigned yv = fast_div31(rem, a.m_row, a.s_row), xv = rem - yv * (unsigned)a.Wp;
+                const bool ok = b < (unsigned)a.batch && yv >= 1u && xv >= 1u;
+                const size_t pix = ((size_t)b * (unsigned)a.H + yv - 1u) * (unsigned)a.W + xv - 1u;
+                xsrc = ok ? a.xb + (pix * (unsigned)a.Cin + (unsigned)(ci_cb0 * 8)) * 2 : nullptr;
+            }
+#pragma unroll
+            for (int q = 0; q < 16; ++q) {
+                if (q < 8) {
+                    const int cb = 2 * q + (wave >> 1), piece = wave & 1;
+                    lds_dma<16>(gsrc ? gsrc + cb * 16 : a.zeros,
+                                lds0 + (unsigned)(buf * HWG_BUF + (cb * HWG_GP + piece * 64) * 16));
+                } else {
+                    const int cb = q - 8, piece = wave;
+                    lds_dma<16>(xsrc ? xsrc + cb * 16 : a.zeros,
+                                lds0 + (unsigned)(buf * HWG_BUF + HWG_GB + (cb * HWG_XP + piece * 64) * 16));
+                }
+            }
+            return;
+        }
 #pragma unroll
         for (int q = 0; q < 16; ++q) {
             const int idx = q * 4 + wave;
@@ -524,6 +570,7 @@ __device__ inline void halo_wg_body(const HaloWgArgs &a, char *smem, int tile, i
     }
 }
 
+template <bool HWC>
 __global__ __launch_bounds__(HALO_NT) void conv_halo_wg_kernel(const HaloWgArgs a) {
     extern __shared__ __align__(16) char smem[];
     // The workgroups of one (tap group, position split) - one per tile of the weight tensor - stream the same
@@ -544,14 +591,16 @@ __global__ __launch_bounds__(HALO_NT) void conv_halo_wg_kernel(const HaloWgArgs 
         bundle = id < n0 ? id % a.S0 : a.S0 + (id - n0) % a.S1;
     }
     if (bundle < a.S0)
-        halo_wg_body<0, 5>(a, smem, tile, bundle, a.S0);
+        halo_wg_body<0, 5, HWC>(a, smem, tile, bundle, a.S0);
     else
-        halo_wg_body<5, 4>(a, smem, tile, bundle - a.S0, a.S1);
+        halo_wg_body<5, 4, HWC>(a, smem, tile, bundle - a.S0, a.S1);
 }
 
-// dW[idx * 9 + tap] = sum over the splits of the tap's group of ws[tap][split][idx]
+// dW[idx * 9 + tap] (filters [co][ci][tap]) or, tap-major, dW[((idx / Cin) * 9 + tap) * Cin + idx % Cin] (filters
+// [co][tap][ci]) = sum over the splits of the tap's group of ws[tap][split][idx], idx = co * Cin + ci
 __global__ __launch_bounds__(256) void conv_halo_wg_reduce_kernel(const float *__restrict__ ws, half_t *__restrict__ dW,
-                                                                  long long total, int S0, int S1, int smax) {
+                                                                  long long total, int S0, int S1, int smax,
+                                                                  int tap_major_cin) {
     const long long idx = (long long)blockIdx.x * 256 + threadIdx.x;
     const int tap = blockIdx.y;
     if (idx >= total) return;
@@ -566,7 +615,10 @@ __global__ __launch_bounds__(256) void conv_halo_wg_reduce_kernel(const float *_
         s += (v[0] + v[1]) + (v[2] + v[3]);
     }
     for (; z < S; ++z) s += src[(size_t)z * total];
-    dW[idx * 9 + tap] = (half_t)s;
+    if (tap_major_cin > 0)
+        dW[((idx / tap_major_cin) * 9 + tap) * tap_major_cin + idx % tap_major_cin] = (half_t)s;
+    else
+        dW[idx * 9 + tap] = (half_t)s;
 }
 
 // gb[cb][p] for p < pstride: the tensor element t[b][8 cb .. + 7][yp - pu][xp - pl] at p = (b, yp, xp) of the padded
@@ -699,6 +751,13 @@ bool conv_halo_wg_preferred(const ConvTileDesc &d) {
     const int cmin = d.Cin < d.Cout ? d.Cin : d.Cout;
     return conv_halo_wg_fits(d, Hp, Wp) && Wp <= 32 && units >= (cmin >= 256 ? 20 : 96);
 }
+// Channel-minor: the other route copies both tensors into padded form first (9 + 9 of 66 us on 128 -> 128 28x28 at
+// batch 128), so this one is taken from the same amount of work on whatever the row length.
+bool conv_halo_wg_hwc_preferred(const ConvTileDesc &d) {
+    const long long units = ((long long)d.batch * (d.Hin + 1) * (d.Win + 1) + HWG_UNIT - 1) / HWG_UNIT;
+    const int cmin = d.Cin < d.Cout ? d.Cin : d.Cout;
+    return units >= (cmin >= 256 ? 20 : 96);
+}
 long long conv_halo_wg_margin() { return 2 * HWG_UNIT + 256; }
 long long conv_halo_wg_gradient_stride(const ConvTileDesc &d, int Hp, int Wp) {
     const long long P = (long long)d.batch * Hp * Wp;
@@ -735,12 +794,33 @@ int conv_halo_embed(const void *t, void *out, int batch, int C, int Hs, int Ws, 
     return hip_ok(hipGetLastError(), "blocked layout launch") ? 0 : 2;
 }
 
+template <bool HWC>
+static int halo_wg_run(HaloWgArgs &a, const ConvTileDesc &d, float *ws, void *dW) {
+    State &st = state();
+    constexpr int lds = 2 * HWG_BUF;
+    static bool attr = false;
+    if (!attr) {
+        if (!hip_ok(hipFuncSetAttribute((const void *)conv_halo_wg_kernel<HWC>, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                        lds),
+                    "halo weight-gradient LDS size"))
+            return 2;
+        attr = true;
+    }
+    a.xcd_map = 1;
+    const int bundles = (a.S0 + a.S1 + 7) / 8 * 8;
+    hipLaunchKernelGGL(conv_halo_wg_kernel<HWC>, dim3((unsigned)(a.tiles * bundles)), dim3(HALO_NT), lds, st.stream, a);
+    if (!hip_ok(hipGetLastError(), "halo weight-gradient launch")) return 2;
+    const long long total = (long long)d.Cout * d.Cin;
+    hipLaunchKernelGGL(conv_halo_wg_reduce_kernel, dim3((unsigned)((total + 255) / 256), 9), dim3(256), 0, st.stream, ws,
+                       static_cast<half_t *>(dW), total, a.S0, a.S1, a.smax, HWC ? d.Cin : 0);
+    return hip_ok(hipGetLastError(), "halo weight-gradient reduce launch") ? 0 : 2;
+}
+
 // gb: the blocked, embedded gradient (top left of the grids at gb[cb * gstride + 0]; zero from the last padded
 // position to conv_halo_wg_gradient_stride() positions); xb as for the forward kernel with conv_halo_wg_margin()
 // readable chunks behind it; ws: conv_halo_wg_partial_bytes().
 int conv_halo_wg_launch(const ConvTileDesc &d, const void *xb, const void *gb, long long gstride, float *ws, void *dW,
                         int Hp, int Wp, int S0, int S1) {
-    State &st = state();
     const long long P = (long long)d.batch * Hp * Wp, Pd = conv_halo_wg_gradient_stride(d, Hp, Wp);
     HaloWgArgs a = {};
     a.xb = static_cast<const char *>(xb);
@@ -753,22 +833,38 @@ int conv_halo_wg_launch(const ConvTileDesc &d, const void *xb, const void *gb, l
     a.tiles_ci = d.Cin / 64;
     a.tiles = (d.Cout / 128) * a.tiles_ci;
     a.S0 = S0; a.S1 = S1; a.smax = S0 > S1 ? S0 : S1;
-    constexpr int lds = 2 * HWG_BUF;
-    static bool attr = false;
-    if (!attr) {
-        if (!hip_ok(hipFuncSetAttribute((const void *)conv_halo_wg_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, lds),
-                    "halo weight-gradient LDS size"))
-            return 2;
-        attr = true;
-    }
-    a.xcd_map = 1;
-    const int bundles = a.xcd_map ? (S0 + S1 + 7) / 8 * 8 : S0 + S1;
-    hipLaunchKernelGGL(conv_halo_wg_kernel, dim3((unsigned)(a.tiles * bundles)), dim3(HALO_NT), lds, st.stream, a);
-    if (!hip_ok(hipGetLastError(), "halo weight-gradient launch")) return 2;
-    const long long total = (long long)d.Cout * d.Cin;
-    hipLaunchKernelGGL(conv_halo_wg_reduce_kernel, dim3((unsigned)((total + 255) / 256), 9), dim3(256), 0, st.stream, ws,
-                       static_cast<half_t *>(dW), total, S0, S1, a.smax);
-    return hip_ok(hipGetLastError(), "halo weight-gradient reduce launch") ? 0 : 2;
+    return halo_wg_run<false>(a, d, ws, dW);
+}
+
+// Channel-minor 3x3 "same" layers (as conv_halo_hwc_fits) with whole 128-filter tiles and rows whose reach of two
+// rows and two positions fits the 128 positions behind a unit; both tensors 16-byte aligned.
+bool conv_halo_wg_hwc_fits(const ConvTileDesc &d, const void *X, const void *dY) {
+    const int Wv = d.Win + 1;
+    return d.in_hwc && d.KH == 3 && d.KW == 3 && d.sh == 1 && d.sw == 1 && d.padU == 1 && d.padD == 1 && d.padL == 1 &&
+           d.padR == 1 && d.Ho == d.Hin && d.Wo == d.Win && d.Cin % 64 == 0 && d.Cout % 128 == 0 && 2 * Wv + 2 <= 128 &&
+           reinterpret_cast<uintptr_t>(X) % 16 == 0 && reinterpret_cast<uintptr_t>(dY) % 16 == 0 &&
+           (long long)(d.batch + 1) * (d.Hin + 1) * Wv + 2 * HWG_UNIT + 256 < ((long long)1 << 31);
+}
+
+// X: [batch][H][W][Cin], dY: [batch][H][W][Cout], dW: [Cout][3][3][Cin]; ws: conv_halo_wg_partial_bytes() of the
+// virtual grid (Hp = H + 1, Wp = W + 1).
+int conv_halo_wg_hwc_launch(const ConvTileDesc &d, const void *X, const void *dY, float *ws, void *dW, int S0, int S1) {
+    State &st = state();
+    const int Hp = d.Hin + 1, Wp = d.Win + 1;
+    HaloWgArgs a = {};
+    a.xb = static_cast<const char *>(X);
+    a.gb = static_cast<const char *>(dY);
+    a.zeros = static_cast<const char *>(st.zeros);
+    if (!a.zeros) return 2;
+    a.ws = ws;
+    a.Cin = d.Cin; a.Cout = d.Cout; a.Wp = Wp; a.Hp = Hp; a.H = d.Hin; a.W = d.Win; a.batch = d.batch;
+    a.units = (int)(conv_halo_wg_gradient_stride(d, Hp, Wp) / HWG_UNIT);
+    a.tiles_ci = d.Cin / 64;
+    a.tiles = (d.Cout / 128) * a.tiles_ci;
+    a.S0 = S0; a.S1 = S1; a.smax = S0 > S1 ? S0 : S1;
+    magic31((unsigned)(Hp * Wp), &a.m_img, &a.s_img);
+    magic31((unsigned)Wp, &a.m_row, &a.s_row);
+    return halo_wg_run<true>(a, d, ws, dW);
 }
 
 }  // namespace ptl

@@ -408,6 +408,20 @@ int conv_taps_wg(const ConvTileDesc &d, const void *X, const void *dY, void *dW)
             }
         }
     }
+    if constexpr (ES == 2) {
+        // 3x3 "same" channel-minor layers: the same kernel on the caller's tensors in place
+        if (hwc && conv_halo_wg_hwc_fits(d, X, dY) &&
+            (st.gemm_path == 5 || (st.gemm_path == 0 && conv_halo_wg_hwc_preferred(d)))) {
+            int S0 = 1, S1 = 1;
+            const size_t ws_bytes = conv_halo_wg_partial_bytes(d, d.Hin + 1, d.Win + 1, &S0, &S1);
+            if (ws_bytes <= ((size_t)1 << 30)) {
+                float *ws = workspace(ws_bytes);
+                if (!ws) return 2;
+                st.last_conv_resident = 1;
+                return conv_halo_wg_hwc_launch(d, X, dY, ws, dW, S0, S1);
+            }
+        }
+    }
     if (hwc) {  // channel-minor: both operands are [position][channel] matrices read 16 bytes along the channels
         if (d.Cout % VEC || reinterpret_cast<uintptr_t>(X) % 16 || reinterpret_cast<uintptr_t>(dY) % 16) return -1;
         // (no direct kernel for this layout: the alternative is the gathering GEMM, which this route beats from 64

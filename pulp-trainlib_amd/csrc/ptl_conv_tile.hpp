@@ -135,6 +135,11 @@ bool conv_halo_wg_preferred(const ConvTileDesc &d);  // fits, and measured faste
 long long conv_halo_wg_margin();
 long long conv_halo_wg_gradient_stride(const ConvTileDesc &d, int Hp, int Wp);
 size_t conv_halo_wg_partial_bytes(const ConvTileDesc &d, int Hp, int Wp, int *S0, int *S1);
+// The same kernel on channel-minor tensors read in place (3x3 "same" layers, Cout a multiple of 128): one launch + the
+// addition of the partial sums; ws sized by conv_halo_wg_partial_bytes() for Hp = Hin + 1, Wp = Win + 1.
+bool conv_halo_wg_hwc_fits(const ConvTileDesc &d, const void *X, const void *dY);
+bool conv_halo_wg_hwc_preferred(const ConvTileDesc &d);
+int conv_halo_wg_hwc_launch(const ConvTileDesc &d, const void *X, const void *dY, float *ws, void *dW, int S0, int S1);
 int conv_halo_wg_launch(const ConvTileDesc &d, const void *xb, const void *gb, long long gstride, float *ws, void *dW,
                         int Hp, int Wp, int S0, int S1);
 

@@ -296,15 +296,20 @@ def test_conv2d_forward_leaves_its_blocked_input_for_the_gradients(pkg, gpu, cas
                     assert gpu.ptl_conv2d_fp16_wg_batched_cached(ctypes.byref(a3), ns, ctypes.byref(other)) == 0
                     gpu.ptl_sync()
                     assert torch.equal(dw3, dw2)
-                    # ... and a valid cache IS what the gradient reads: with every chunk of the copy (border included)
-                    # overwritten by 0x3c3c = 1.05859375, each filter's gradient is that constant times the sum of its
-                    # output gradient, whatever the tap and channel
+                    # ... and a valid cache IS what the resident-tile weight gradient reads: with every chunk of the
+                    # copy (border included) overwritten by 0x3c3c = 1.05859375, each filter's gradient is that constant
+                    # times the sum of its output gradient, whatever the tap and channel
                     dw4 = torch.full_like(w, 3)
                     a4, keep4 = hp.conv2d_args(pkg, x, None, w, dw4, y, dy, Ci, H, W, Co, 3, 3, Ho, Wo, pad, (1, 1))
                     assert gpu.ptl_conv2d_fp16_wg_batched_cached(ctypes.byref(a4), ns, ctypes.byref(c)) == 0
+                    took_copy = gpu.ptl_last_conv_resident() == 1  # (the route that reads the copy: 128-filter tiles)
                     gpu.ptl_sync()
-                    want = (1.05859375 * dy.float().sum(dim=(0, 2, 3))).view(Co, 1, 1, 1).expand_as(w)
-                    assert float((dw4.float() - want).norm() / want.norm()) <= 2e-3
+                    assert took_copy == (Co % 128 == 0)
+                    if took_copy:
+                        want = (1.05859375 * dy.float().sum(dim=(0, 2, 3))).view(Co, 1, 1, 1).expand_as(w)
+                        assert float((dw4.float() - want).norm() / want.norm()) <= 2e-3
+                    else:
+                        assert torch.equal(dw4, dw2)
             else:
                 pkg.call("ptl_conv2d_fp16_fw_batched", a, ns)
                 pkg.call("ptl_conv2d_fp16_bw_batched", a, ns)
@@ -425,6 +430,36 @@ def test_conv2d_resident_tile_channel_minor_in_place(pkg, gpu, case):
     rel = lambda got, ref: float((got.float() - ref).norm() / ref.norm())
     assert rel(y, ref_y) <= 1e-3
     assert rel(dx, ref_dx) <= 1e-3
+
+
+@pytest.mark.parametrize("case", [(64, 14, 14, 128, 9), (128, 5, 7, 128, 21), (64, 62, 62, 128, 2), (192, 28, 28, 256, 5),
+                                  (64, 3, 61, 128, 4), (128, 1, 1, 128, 300), (64, 30, 9, 384, 3)])
+def test_conv2d_resident_tile_weight_gradient_channel_minor_in_place(pkg, gpu, case):
+    """The resident-tile weight gradient on channel-minor tensors read in place (whole 128-filter tiles): against
+    torch in float32 and against the tap-sum route; the filter gradient is [Cout][3][3][Cin].  Units that cross
+    several samples, a single row, the widest row that fits, a ragged last unit, several filter and channel tiles."""
+    Ci, H, W, Co, ns = case
+    nd = np.float16
+    x = dev(hp.uniform(61, (ns, H, W, Ci), dtype=nd))
+    w = dev(hp.uniform(62, (Co, 3, 3, Ci), dtype=nd) * 0.2)
+    dy = dev(hp.uniform(63, (ns, H, W, Co), dtype=nd))
+    res = {}
+    for path in (5, 3):
+        dw, y = dev(np.full((Co, 3, 3, Ci), 3, nd)), dev(np.zeros((ns, H, W, Co), nd))
+        a, keep = hp.conv2d_args(pkg, x, None, w, dw, y, dy, Ci, H, W, Co, 3, 3, H, W, (1, 1, 1, 1), (1, 1), 1)
+        gpu.ptl_set_gemm_path(path)
+        try:
+            pkg.call("ptl_conv2d_fp16_wg_batched", a, ns)
+            assert gpu.ptl_last_conv_resident() == (1 if path == 5 else 0)
+        finally:
+            gpu.ptl_set_gemm_path(0)
+        sync(gpu)
+        res[path] = dw
+    xc, dyc = x.float().permute(0, 3, 1, 2), dy.float().permute(0, 3, 1, 2)
+    ref = torch.nn.grad.conv2d_weight(xc, (Co, Ci, 3, 3), dyc, padding=1).permute(0, 2, 3, 1)
+    rel = lambda got, r: float((got.float() - r).norm() / r.norm())
+    assert rel(res[5], ref) <= 1e-3
+    assert rel(res[5], res[3].float()) <= 2e-3
 
 
 def test_conv2d_resident_tile_many_tiles(pkg, gpu):
