@@ -460,6 +460,18 @@ def test_conv2d_resident_tile_weight_gradient_channel_minor_in_place(pkg, gpu, c
     rel = lambda got, r: float((got.float() - r).norm() / r.norm())
     assert rel(res[5], ref) <= 1e-3
     assert rel(res[5], res[3].float()) <= 2e-3
+    # both gradients in one call (the reference's pulp_conv2d_fp16_bw_cl pattern) take the same two kernels
+    dw, dx, y = dev(np.full((Co, 3, 3, Ci), 3, nd)), dev(np.full((ns, H, W, Ci), 3, nd)), dev(np.zeros((ns, H, W, Co), nd))
+    a, keep = hp.conv2d_args(pkg, x, dx, w, dw, y, dy, Ci, H, W, Co, 3, 3, H, W, (1, 1, 1, 1), (1, 1), 1)
+    gpu.ptl_set_gemm_path(5)
+    try:
+        pkg.call("ptl_conv2d_fp16_bw_batched", a, ns)
+    finally:
+        gpu.ptl_set_gemm_path(0)
+    sync(gpu)
+    assert torch.equal(dw, res[5])
+    ref_dx = torch.nn.grad.conv2d_input(xc.shape, w.float().permute(0, 3, 1, 2), dyc, padding=1).permute(0, 2, 3, 1)
+    assert rel(dx, ref_dx) <= 1e-3
 
 
 def test_conv2d_resident_tile_many_tiles(pkg, gpu):
