@@ -419,69 +419,83 @@ struct HaloWgArgs {
 typedef short hwg_s4 __attribute__((ext_vector_type(4)));
 typedef __attribute__((address_space(3))) hwg_s4 hwg_lds_s4;
 
-__device__ inline uint4 hwg_frag(const char *p) {
+// A fragment = two transposing reads, `second` bytes (four positions) apart.
+__device__ inline uint4 hwg_frag(const char *p, int second) {
     union {
         hwg_s4 h[2];
         uint4 v;
     } t;
     t.h[0] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((hwg_lds_s4 *)(lds_char *)p);
-    t.h[1] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((hwg_lds_s4 *)(lds_char *)(p + 64));
+    t.h[1] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((hwg_lds_s4 *)(lds_char *)(p + second));
     return t.v;
 }
 
-// HWC = true: the same tiles filled from channel-minor tensors where they lie.  The positions are those of the
-// virtual grid of the forward kernel (one zero row above and one zero column left of every sample, Hp = H + 1 rows
-// of Wp = W + 1 positions): position (b, yv, xv) of the gradient tile is dY[b][yv][xv] for yv < H and xv < W, of the
-// input tile X[b][yv - 1][xv - 1] for yv, xv >= 1, and a chunk of zeros otherwise.  A wave's load still fills 64
-// consecutive positions of one channel block in LDS; every lane gives its own address (16 bytes of its position's
-// pixel, pixels Cout or Cin elements apart) or that of the zero page, and the eight loads that take the eight blocks
-// of the same 128 bytes of a pixel follow each other in one wave.
-template <int T0, int NT, bool HWC>
+// HWC = true: the tiles filled from channel-minor tensors where they lie.  The positions are those of the virtual
+// grid of the forward kernel (one zero row above and one zero column left of every sample, Hp = H + 1 rows of
+// Wp = W + 1 positions): position (b, yv, xv) of the gradient tile is dY[b][yv][xv] for yv < H and xv < W, of the
+// input tile X[b][yv - 1][xv - 1] for yv, xv >= 1 - the pixel of the gradient tile Wp + 1 positions earlier - and a
+// chunk of zeros otherwise.  So ONE table of 256 pixel indices per unit (-1: zeros), entry e = the gradient-tile
+// pixel of position p0 - (Wp + 1) + e, serves both tiles; a thread works out one entry (two multiply-shift
+// divisions), a unit ahead, into one of two slots behind the tile buffers.  The tiles are [position][chunk] in
+// LDS - a load covers whole 128-byte runs of the tensors: 8 positions x 8 chunks of the input tile, 4 positions x
+// 16 chunks of the gradient tile - with the chunks of a position rotated by two slots per position, which puts
+// the 16 pieces of a transposing read (4 positions x 2 channel blocks x 2 halves) on 16 different 8-byte cells of
+// one 128-byte stripe; a lane's channel block in a load and its offsets in the fragment reads do not depend on
+// the unit, the tap shift is part of the per-tap offset.
+// FI: 16-filter blocks per wave: 4 = 128 filters per workgroup (two tap groups of 5 and 4 taps), 2 = 64 filters
+// (all nine taps in one workgroup).
+template <int T0, int NT, bool HWC, int FI>
 __device__ inline void halo_wg_body(const HaloWgArgs &a, char *smem, int tile, int split, int S) {
     const unsigned lds0 = (unsigned)(uintptr_t)(lds_char *)smem;
     const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int wm = wave & 1, wn = wave >> 1;
     const int i16 = lane & 15, kq = lane >> 4;
-    const int co_cb0 = (tile / a.tiles_ci) * 16, ci_cb0 = (tile % a.tiles_ci) * 8;
+    const int co_cb0 = (tile / a.tiles_ci) * (4 * FI), ci_cb0 = (tile % a.tiles_ci) * 8;
     const int u0 = (int)((long long)split * a.units / S), u1 = (int)((long long)(split + 1) * a.units / S);
     const unsigned voff = (unsigned)lane * 16u;
+    static_assert(HWC || FI == 4, "the channel-major form has 128-filter tiles only");
+
+    // ---- channel-minor: position table and loads
+    int *const tab = reinterpret_cast<int *>(smem + 2 * HWG_BUF);
+    auto fill_table = [&](int u, int slot) {
+        const long long pt = (long long)u * HWG_UNIT - (a.Wp + 1) + tid;
+        int v = -1;
+        if (pt >= 0) {
+            const unsigned pv = (unsigned)pt, HpWp = (unsigned)(a.Hp * a.Wp);
+            const unsigned b = fast_div31(pv, a.m_img, a.s_img), rem = pv - b * HpWp;
+            const unsigned yv = fast_div31(rem, a.m_row, a.s_row), xv = rem - yv * (unsigned)a.Wp;
+            if (b < (unsigned)a.batch && yv < (unsigned)a.H && xv < (unsigned)a.W)
+                v = (int)((b * (unsigned)a.H + yv) * (unsigned)a.W + xv);  // (the host keeps pixel counts below 2^31)
+        }
+        tab[slot * 256 + tid] = v;
+    };
+    // this lane's channel block in every load of the gradient / input tile, as a byte offset within a pixel
+    const unsigned g_chunk = (unsigned)(co_cb0 + (((lane & 15) & 8) | (((lane & 7) - 2 * (lane >> 4)) & 7))) * 16u;
+    const unsigned x_chunk = (unsigned)(ci_cb0 + (((lane & 7) - 2 * (lane >> 3)) & 7)) * 16u;
+    const unsigned cout2 = (unsigned)a.Cout * 2u, cin2 = (unsigned)a.Cin * 2u;
+    auto issue_hwc = [&](int buf, int slot) {
+        const int *t = tab + slot * 256;
+        constexpr int GQ = 2 * FI;  // loads of the gradient tile per wave: 128 positions x 4 * FI chunks
+#pragma unroll
+        for (int q = 0; q < 8; ++q) {
+            if (q < GQ) {
+                // 64 / (4 * FI) positions x 4 * FI chunks per load
+                constexpr int PPL = 16 / FI;  // positions per load
+                const int ig = wave * GQ + q;
+                const int idx = t[ig * PPL + (FI == 4 ? lane >> 4 : lane >> 3) + a.Wp + 1];
+                const unsigned chunk = FI == 4 ? g_chunk : (unsigned)(co_cb0 + (((lane & 7) - 2 * (lane >> 3)) & 7)) * 16u;
+                const char *src = idx >= 0 ? a.gb + ((size_t)(unsigned)idx * cout2 + chunk) : a.zeros;
+                lds_dma<16>(src, lds0 + (unsigned)(buf * HWG_BUF + ig * 1024));
+            }
+            const int ix = wave * 8 + q;
+            const int idx = t[ix * 8 + (lane >> 3)];
+            const char *src = idx >= 0 ? a.xb + ((size_t)(unsigned)idx * cin2 + x_chunk) : a.zeros;
+            lds_dma<16>(src, lds0 + (unsigned)(buf * HWG_BUF + HWG_GB + ix * 1024));
+        }
+    };
 
     auto issue = [&](int u, int buf) {
         const long long p0 = (long long)u * HWG_UNIT;
-        if constexpr (HWC) {
-            const unsigned HpWp = (unsigned)(a.Hp * a.Wp);
-            // this wave's piece of the gradient tile (64 positions from piece wave & 1) and of the input tile (piece wave)
-            const char *gsrc, *xsrc;
-            {
-                const unsigned pv = (unsigned)p0 + (unsigned)((wave & 1) * 64 + lane);
-                const unsigned b = fast_div31(pv, a.m_img, a.s_img), rem = pv - b * HpWp;
-                const unsigned yv = fast_div31(rem, a.m_row, a.s_row), xv = rem - yv * (unsigned)a.Wp;
-                const bool ok = b < (unsigned)a.batch && yv < (unsigned)a.H && xv < (unsigned)a.W;
-                const size_t pix = ((size_t)b * (unsigned)a.H + yv) * (unsigned)a.W + xv;
-                gsrc = ok ? a.gb + (pix * (unsigned)a.Cout + (unsigned)(co_cb0 * 8)) * 2 : nullptr;
-            }
-            {
-                const unsigned pv = (unsigned)p0 + (unsigned)(wave * 64 + lane);
-                const unsigned b = fast_div31(pv, a.m_img, a.s_img), rem = pv - b * HpWp;
-                const unsigned yv = fast_div31(rem, a.m_row, a.s_row), xv = rem - yv * (unsigned)a.Wp;
-                const bool ok = b < (unsigned)a.batch && yv >= 1u && xv >= 1u;
-                const size_t pix = ((size_t)b * (unsigned)a.H + yv - 1u) * (unsigned)a.W + xv - 1u;
-                xsrc = ok ? a.xb + (pix * (unsigned)a.Cin + (unsigned)(ci_cb0 * 8)) * 2 : nullptr;
-            }
-#pragma unroll
-            for (int q = 0; q < 16; ++q) {
-                if (q < 8) {
-                    const int cb = 2 * q + (wave >> 1), piece = wave & 1;
-                    lds_dma<16>(gsrc ? gsrc + cb * 16 : a.zeros,
-                                lds0 + (unsigned)(buf * HWG_BUF + (cb * HWG_GP + piece * 64) * 16));
-                } else {
-                    const int cb = q - 8, piece = wave;
-                    lds_dma<16>(xsrc ? xsrc + cb * 16 : a.zeros,
-                                lds0 + (unsigned)(buf * HWG_BUF + HWG_GB + (cb * HWG_XP + piece * 64) * 16));
-                }
-            }
-            return;
-        }
 #pragma unroll
         for (int q = 0; q < 16; ++q) {
             const int idx = q * 4 + wave;
@@ -498,19 +512,39 @@ __device__ inline void halo_wg_body(const HaloWgArgs &a, char *smem, int tile, i
         }
     };
 
-    // A wave owns 64 filters x 32 channels x NT taps as 16 x 16 blocks (v_mfma_f32_16x16x32_f16: 32 positions per
+    // A wave owns 16 * FI filters x 32 channels x NT taps as 16 x 16 blocks (v_mfma_f32_16x16x32_f16: 32 positions per
     // k-step, a lane holds row lane % 16 and positions 8 * (lane / 16) .. + 7 of the step).  This lane's piece of a
     // transposing read: position k0 + i16 / 4 of channel block .. + (i16 & 3) / 2, channels 4 * (i16 & 1) .. + 3 of
     // that block; the second read of a fragment is four positions on.
-    const unsigned ga = (unsigned)((((wm * 8 + ((i16 & 3) >> 1)) * HWG_GP + 8 * kq + (i16 >> 2)) * 16) + (i16 & 1) * 8);
-    const unsigned xa = (unsigned)(HWG_GB + (((wn * 4 + ((i16 & 3) >> 1)) * HWG_XP + 8 * kq + (i16 >> 2)) * 16) + (i16 & 1) * 8);
-    int tapoff[NT];
+    // Byte offsets of this lane's first read of gradient fragment i / input fragment (c, tap) in k-step 0; a k-step on is
+    // + KSG / KSX bytes, the second read + RDG / RDX.
+    constexpr int GROW = HWC ? (FI == 4 ? 256 : 128) : 16;  // bytes from one position of the gradient tile to the next
+    constexpr int KSG = 32 * GROW, RDG = 4 * GROW, KSX = HWC ? 32 * 128 : 512, RDX = HWC ? 4 * 128 : 64;
+    const int pj = (i16 & 3) >> 1, pq = i16 >> 2, ph = (i16 & 1) * 8;
+    unsigned goff[FI], xoff[2][NT];
 #pragma unroll
-    for (int t = 0; t < NT; ++t) tapoff[t] = (((T0 + t) / 3) * a.Wp + (T0 + t) % 3) * 16;
+    for (int i = 0; i < FI; ++i) {
+        if constexpr (HWC) {
+            const int cb = wm * 2 * FI + 2 * i + pj;  // block within the tile's 4 * FI
+            goff[i] = (unsigned)((8 * kq + pq) * GROW + ((cb & 8) | (((cb & 7) + 2 * pq) & 7)) * 16 + ph);
+        } else {
+            goff[i] = (unsigned)((((wm * 8 + 2 * i + pj) * HWG_GP + 8 * kq + pq) * 16) + ph);
+        }
+    }
+#pragma unroll
+    for (int c = 0; c < 2; ++c)
+#pragma unroll
+        for (int t = 0; t < NT; ++t) {
+            const int sh = ((T0 + t) / 3) * a.Wp + (T0 + t) % 3;
+            if constexpr (HWC)
+                xoff[c][t] = (unsigned)(HWG_GB + (8 * kq + pq + sh) * 128 + ((wn * 4 + 2 * c + pj + 2 * pq + 2 * sh) & 7) * 16 + ph);
+            else
+                xoff[c][t] = (unsigned)(HWG_GB + (((wn * 4 + 2 * c + pj) * HWG_XP + 8 * kq + pq + sh) * 16) + ph);
+        }
 
-    f32x4 acc[4][2][NT];
+    f32x4 acc[FI][2][NT];
 #pragma unroll
-    for (int i = 0; i < 4; ++i)
+    for (int i = 0; i < FI; ++i)
 #pragma unroll
         for (int c = 0; c < 2; ++c)
 #pragma unroll
@@ -518,37 +552,55 @@ __device__ inline void halo_wg_body(const HaloWgArgs &a, char *smem, int tile, i
 #pragma unroll
                 for (int v = 0; v < 4; ++v) acc[i][c][t][v] = 0.f;
 
-    if (u0 < u1) issue(u0, 0);
+    if (u0 < u1) {
+        if constexpr (HWC) {
+            fill_table(u0, 0);
+            __syncthreads();
+            issue_hwc(0, 0);
+            if (u0 + 1 < u1) fill_table(u0 + 1, 1);
+        } else {
+            issue(u0, 0);
+        }
+    }
     for (int u = u0; u < u1; ++u) {
         const int buf = (u - u0) & 1;
         wait_vmcnt<0>();
         __syncthreads();  // unit u has landed for every wave, and every wave has left unit u - 1
-        issue(u + 1 < u1 ? u + 1 : u, buf ^ 1);
-        const char *gt = smem + buf * HWG_BUF + ga, *xt = smem + buf * HWG_BUF + xa;
-        uint4 gf[2][4], xf[2][2][NT];
+        if constexpr (HWC) {
+            // the table of unit u + 1 was written before the barrier; that of unit u + 2 takes the slot of unit u,
+            // whose loads were issued before the barrier
+            if (u + 1 < u1) issue_hwc(buf ^ 1, buf ^ 1);
+            if (u + 2 < u1) fill_table(u + 2, buf);
+        } else {
+            issue(u + 1 < u1 ? u + 1 : u, buf ^ 1);
+        }
+        const char *bt = smem + buf * HWG_BUF;
+        uint4 gf[2][FI], xf[2][2][NT];
         auto read = [&](int set, int ks) {
 #pragma unroll
-            for (int i = 0; i < 4; ++i) gf[set][i] = hwg_frag(gt + ks * 512 + i * 2 * HWG_GP * 16);
+            for (int i = 0; i < FI; ++i) gf[set][i] = hwg_frag(bt + goff[i] + ks * KSG, RDG);
 #pragma unroll
             for (int c = 0; c < 2; ++c)
 #pragma unroll
-                for (int t = 0; t < NT; ++t) xf[set][c][t] = hwg_frag(xt + ks * 512 + c * 2 * HWG_XP * 16 + tapoff[t]);
+                for (int t = 0; t < NT; ++t) xf[set][c][t] = hwg_frag(bt + xoff[c][t] + ks * KSX, RDX);
         };
         read(0, 0);
         static_for<0, 4>([&](auto KI) {
             constexpr int ks = decltype(KI)::value, cur = ks & 1;
             if constexpr (ks + 1 < 4) read(cur ^ 1, ks + 1);
 #pragma unroll
-            for (int i = 0; i < 4; ++i)
+            for (int i = 0; i < FI; ++i)
 #pragma unroll
                 for (int c = 0; c < 2; ++c)
 #pragma unroll
                     for (int t = 0; t < NT; ++t) mfma16(acc[i][c][t], gf[cur][i], xf[cur][c][t]);
             if constexpr (ks + 1 < 4) {
-                // 2 * (4 + 2 * NT) transposing reads under 8 * NT MFMAs: one read behind each of the first MFMAs
+                // 2 * (FI + 2 * NT) transposing reads under 2 * FI * NT MFMAs: one read (two where the reads outnumber
+                // the MFMAs) behind each of the first MFMAs
+                constexpr int RD = 2 * (FI + 2 * NT), MF = 2 * FI * NT, PER = (RD + MF - 1) / MF;
 #pragma unroll
-                for (int m = 0; m < 2 * (4 + 2 * NT); ++m) {
-                    __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+                for (int m = 0; m < (RD + PER - 1) / PER; ++m) {
+                    __builtin_amdgcn_sched_group_barrier(0x100, PER, 0);
                     __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
                 }
             }
@@ -557,12 +609,12 @@ __device__ inline void halo_wg_body(const HaloWgArgs &a, char *smem, int tile, i
     wait_vmcnt<0>();  // nothing may still be landing in LDS when the workgroup ends
     if (u0 >= u1) return;
     // partial sums: lane = channel, four consecutive filters per block
-    const int co0 = (tile / a.tiles_ci) * 128 + wm * 64 + 4 * kq, ci0 = (tile % a.tiles_ci) * 64 + wn * 32 + i16;
+    const int co0 = (tile / a.tiles_ci) * (32 * FI) + wm * (16 * FI) + 4 * kq, ci0 = (tile % a.tiles_ci) * 64 + wn * 32 + i16;
 #pragma unroll
     for (int t = 0; t < NT; ++t) {
         float *dst = a.ws + (((size_t)(T0 + t) * a.smax + split) * a.Cout + co0) * a.Cin + ci0;
 #pragma unroll
-        for (int i = 0; i < 4; ++i)
+        for (int i = 0; i < FI; ++i)
 #pragma unroll
             for (int c = 0; c < 2; ++c)
 #pragma unroll
@@ -570,7 +622,7 @@ __device__ inline void halo_wg_body(const HaloWgArgs &a, char *smem, int tile, i
     }
 }
 
-template <bool HWC>
+template <bool HWC, int FI>
 __global__ __launch_bounds__(HALO_NT) void conv_halo_wg_kernel(const HaloWgArgs a) {
     extern __shared__ __align__(16) char smem[];
     // The workgroups of one (tap group, position split) - one per tile of the weight tensor - stream the same
@@ -590,10 +642,14 @@ __global__ __launch_bounds__(HALO_NT) void conv_halo_wg_kernel(const HaloWgArgs 
         tile = id < n0 ? id / a.S0 : (id - n0) / a.S1;
         bundle = id < n0 ? id % a.S0 : a.S0 + (id - n0) % a.S1;
     }
-    if (bundle < a.S0)
-        halo_wg_body<0, 5, HWC>(a, smem, tile, bundle, a.S0);
-    else
-        halo_wg_body<5, 4, HWC>(a, smem, tile, bundle - a.S0, a.S1);
+    if constexpr (FI == 2) {
+        halo_wg_body<0, 9, HWC, 2>(a, smem, tile, bundle, a.S0);  // (64-filter tiles: one group of nine taps, S1 = 0)
+    } else {
+        if (bundle < a.S0)
+            halo_wg_body<0, 5, HWC, 4>(a, smem, tile, bundle, a.S0);
+        else
+            halo_wg_body<5, 4, HWC, 4>(a, smem, tile, bundle - a.S0, a.S1);
+    }
 }
 
 // dW[idx * 9 + tap] (filters [co][ci][tap]) or, tap-major, dW[((idx / Cin) * 9 + tap) * Cin + idx % Cin] (filters
@@ -765,8 +821,17 @@ long long conv_halo_wg_gradient_stride(const ConvTileDesc &d, int Hp, int Wp) {
 }
 size_t conv_halo_wg_partial_bytes(const ConvTileDesc &d, int Hp, int Wp, int *S0, int *S1) {
     State &st = state();
-    const int tiles = (d.Cout / 128) * (d.Cin / 64);
     const long long units = conv_halo_wg_gradient_stride(d, Hp, Wp) / HWG_UNIT;
+    if (d.Cout % 128) {  // 64-filter tiles (channel-minor only): all nine taps in one workgroup, one split count
+        const int tiles = (d.Cout / 64) * (d.Cin / 64);
+        long long s = st.num_cu / tiles;
+        if (s < 1) s = 1;
+        if (s > units) s = units;
+        *S0 = (int)s;
+        *S1 = (int)s;
+        return (size_t)9 * s * d.Cout * d.Cin * sizeof(float);
+    }
+    const int tiles = (d.Cout / 128) * (d.Cin / 64);
     // one workgroup per CU; the two tap groups (five and four taps) get position splits in the ratio 5 : 4 so that
     // their workgroups finish together
     long long per_tile = st.num_cu / tiles;
@@ -794,25 +859,27 @@ int conv_halo_embed(const void *t, void *out, int batch, int C, int Hs, int Ws, 
     return hip_ok(hipGetLastError(), "blocked layout launch") ? 0 : 2;
 }
 
-template <bool HWC>
+template <bool HWC, int FI>
 static int halo_wg_run(HaloWgArgs &a, const ConvTileDesc &d, float *ws, void *dW) {
     State &st = state();
-    constexpr int lds = 2 * HWG_BUF;
+    constexpr int lds = 2 * HWG_BUF + (HWC ? 2 * 256 * (int)sizeof(int) : 0);  // (+ the two position tables)
     static bool attr = false;
     if (!attr) {
-        if (!hip_ok(hipFuncSetAttribute((const void *)conv_halo_wg_kernel<HWC>, hipFuncAttributeMaxDynamicSharedMemorySize,
-                                        lds),
+        if (!hip_ok(hipFuncSetAttribute((const void *)conv_halo_wg_kernel<HWC, FI>,
+                                        hipFuncAttributeMaxDynamicSharedMemorySize, lds),
                     "halo weight-gradient LDS size"))
             return 2;
         attr = true;
     }
     a.xcd_map = 1;
     const int bundles = (a.S0 + a.S1 + 7) / 8 * 8;
-    hipLaunchKernelGGL(conv_halo_wg_kernel<HWC>, dim3((unsigned)(a.tiles * bundles)), dim3(HALO_NT), lds, st.stream, a);
+    hipLaunchKernelGGL((conv_halo_wg_kernel<HWC, FI>), dim3((unsigned)(a.tiles * bundles)), dim3(HALO_NT), lds, st.stream,
+                       a);
     if (!hip_ok(hipGetLastError(), "halo weight-gradient launch")) return 2;
     const long long total = (long long)d.Cout * d.Cin;
+    // (64-filter tiles: one group of nine taps, every tap has S0 splits)
     hipLaunchKernelGGL(conv_halo_wg_reduce_kernel, dim3((unsigned)((total + 255) / 256), 9), dim3(256), 0, st.stream, ws,
-                       static_cast<half_t *>(dW), total, a.S0, a.S1, a.smax, HWC ? d.Cin : 0);
+                       static_cast<half_t *>(dW), total, a.S0, FI == 2 ? a.S0 : a.S1, a.smax, HWC ? d.Cin : 0);
     return hip_ok(hipGetLastError(), "halo weight-gradient reduce launch") ? 0 : 2;
 }
 
@@ -833,15 +900,15 @@ int conv_halo_wg_launch(const ConvTileDesc &d, const void *xb, const void *gb, l
     a.tiles_ci = d.Cin / 64;
     a.tiles = (d.Cout / 128) * a.tiles_ci;
     a.S0 = S0; a.S1 = S1; a.smax = S0 > S1 ? S0 : S1;
-    return halo_wg_run<false>(a, d, ws, dW);
+    return halo_wg_run<false, 4>(a, d, ws, dW);
 }
 
-// Channel-minor 3x3 "same" layers (as conv_halo_hwc_fits) with whole 128-filter tiles and rows whose reach of two
+// Channel-minor 3x3 "same" layers (as conv_halo_hwc_fits) with whole 64-filter tiles and rows whose reach of two
 // rows and two positions fits the 128 positions behind a unit; both tensors 16-byte aligned.
 bool conv_halo_wg_hwc_fits(const ConvTileDesc &d, const void *X, const void *dY) {
     const int Wv = d.Win + 1;
     return d.in_hwc && d.KH == 3 && d.KW == 3 && d.sh == 1 && d.sw == 1 && d.padU == 1 && d.padD == 1 && d.padL == 1 &&
-           d.padR == 1 && d.Ho == d.Hin && d.Wo == d.Win && d.Cin % 64 == 0 && d.Cout % 128 == 0 && 2 * Wv + 2 <= 128 &&
+           d.padR == 1 && d.Ho == d.Hin && d.Wo == d.Win && d.Cin % 64 == 0 && d.Cout % 64 == 0 && 2 * Wv + 2 <= 128 &&
            reinterpret_cast<uintptr_t>(X) % 16 == 0 && reinterpret_cast<uintptr_t>(dY) % 16 == 0 &&
            (long long)(d.batch + 1) * (d.Hin + 1) * Wv + 2 * HWG_UNIT + 256 < ((long long)1 << 31);
 }
@@ -860,11 +927,12 @@ int conv_halo_wg_hwc_launch(const ConvTileDesc &d, const void *X, const void *dY
     a.Cin = d.Cin; a.Cout = d.Cout; a.Wp = Wp; a.Hp = Hp; a.H = d.Hin; a.W = d.Win; a.batch = d.batch;
     a.units = (int)(conv_halo_wg_gradient_stride(d, Hp, Wp) / HWG_UNIT);
     a.tiles_ci = d.Cin / 64;
-    a.tiles = (d.Cout / 128) * a.tiles_ci;
-    a.S0 = S0; a.S1 = S1; a.smax = S0 > S1 ? S0 : S1;
+    const bool wide = d.Cout % 128 == 0;  // 128-filter tiles in two tap groups, else 64-filter tiles with all nine taps
+    a.tiles = (d.Cout / (wide ? 128 : 64)) * a.tiles_ci;
+    a.S0 = S0; a.S1 = wide ? S1 : 0; a.smax = S0 > a.S1 ? S0 : a.S1;
     magic31((unsigned)(Hp * Wp), &a.m_img, &a.s_img);
     magic31((unsigned)Wp, &a.m_row, &a.s_row);
-    return halo_wg_run<true>(a, d, ws, dW);
+    return wide ? halo_wg_run<true, 4>(a, d, ws, dW) : halo_wg_run<true, 2>(a, d, ws, dW);
 }
 
 }  // namespace ptl

@@ -433,11 +433,14 @@ def test_conv2d_resident_tile_channel_minor_in_place(pkg, gpu, case):
 
 
 @pytest.mark.parametrize("case", [(64, 14, 14, 128, 9), (128, 5, 7, 128, 21), (64, 62, 62, 128, 2), (192, 28, 28, 256, 5),
-                                  (64, 3, 61, 128, 4), (128, 1, 1, 128, 300), (64, 30, 9, 384, 3)])
+                                  (64, 3, 61, 128, 4), (128, 1, 1, 128, 300), (64, 30, 9, 384, 3),
+                                  (64, 14, 14, 64, 9), (128, 5, 7, 192, 21), (64, 62, 62, 64, 2), (64, 1, 1, 64, 300),
+                                  (192, 20, 20, 320, 7)])
 def test_conv2d_resident_tile_weight_gradient_channel_minor_in_place(pkg, gpu, case):
-    """The resident-tile weight gradient on channel-minor tensors read in place (whole 128-filter tiles): against
-    torch in float32 and against the tap-sum route; the filter gradient is [Cout][3][3][Cin].  Units that cross
-    several samples, a single row, the widest row that fits, a ragged last unit, several filter and channel tiles."""
+    """The resident-tile weight gradient on channel-minor tensors read in place (128-filter tiles in two tap groups;
+    64-filter tiles with all nine taps where the filters are no multiple of 128): against torch in float32 and against
+    the tap-sum route; the filter gradient is [Cout][3][3][Cin].  Units that cross several samples, a single row,
+    the widest row that fits, a ragged last unit, several filter and channel tiles."""
     Ci, H, W, Co, ns = case
     nd = np.float16
     x = dev(hp.uniform(61, (ns, H, W, Ci), dtype=nd))

@@ -27,7 +27,7 @@ TABLE = [
     (0, 512, 128, 128, 28, [(1, 1), (1, 1), (1, 1)]),
     (0, 256, 256, 256, 28, [(1, 1), (1, 1), (1, 1)]),
     (0, 256, 512, 512, 14, [(1, 1), (1, 1), (1, 1)]),
-    (1, 128, 64, 64, 56, [(1, 1), (0, 1), (1, 1)]),    # channel-minor, in place; 64 filters: weight gradient as a sum over taps
+    (1, 128, 64, 64, 56, [(1, 1), (1, 1), (1, 1)]),    # channel-minor: all three steps on the caller's tensors in place
     (1, 128, 128, 128, 28, [(1, 1), (1, 1), (1, 1)]),
     (1, 128, 256, 256, 14, [(1, 1), (1, 1), (1, 1)]),
     (0, 8, 128, 128, 28, [(0, 1), (0, 0), (0, 1)]),    # too few tiles for the persistent kernels
