@@ -657,20 +657,28 @@ __global__ __launch_bounds__(HALO_NT) void conv_halo_wg_kernel(const HaloWgArgs 
 __global__ __launch_bounds__(256) void conv_halo_wg_reduce_kernel(const float *__restrict__ ws, half_t *__restrict__ dW,
                                                                   long long total, int S0, int S1, int smax,
                                                                   int tap_major_cin) {
-    const long long idx = (long long)blockIdx.x * 256 + threadIdx.x;
-    const int tap = blockIdx.y;
-    if (idx >= total) return;
+    // 64 outputs x 4 groups of splits per workgroup (a 64 x 64 filter tensor still gives 576 workgroups), four loads
+    // in flight per thread, the four groups added in a fixed order
+    __shared__ float part[4][64];
+    const int o = threadIdx.x & 63, sg = threadIdx.x >> 6, tap = blockIdx.y;
+    const long long idx = (long long)blockIdx.x * 64 + o;
     const int S = tap < 5 ? S0 : S1;
-    const float *src = ws + (size_t)tap * smax * total + idx;
     float s = 0.f;
-    int z = 0;
-    for (; z + 4 <= S; z += 4) {
-        float v[4];
+    if (idx < total) {
+        const float *src = ws + (size_t)tap * smax * total + idx;
+        int z = sg;
+        for (; z + 12 < S; z += 16) {
+            float v[4];
 #pragma unroll
-        for (int k = 0; k < 4; ++k) v[k] = src[(size_t)(z + k) * total];
-        s += (v[0] + v[1]) + (v[2] + v[3]);
+            for (int k = 0; k < 4; ++k) v[k] = src[(size_t)(z + 4 * k) * total];
+            s += (v[0] + v[1]) + (v[2] + v[3]);
+        }
+        for (; z < S; z += 4) s += src[(size_t)z * total];
     }
-    for (; z < S; ++z) s += src[(size_t)z * total];
+    part[sg][o] = s;
+    __syncthreads();
+    if (sg != 0 || idx >= total) return;
+    s = (part[0][o] + part[1][o]) + (part[2][o] + part[3][o]);
     if (tap_major_cin > 0)
         dW[((idx / tap_major_cin) * 9 + tap) * tap_major_cin + idx % tap_major_cin] = (half_t)s;
     else
@@ -878,7 +886,7 @@ static int halo_wg_run(HaloWgArgs &a, const ConvTileDesc &d, float *ws, void *dW
     if (!hip_ok(hipGetLastError(), "halo weight-gradient launch")) return 2;
     const long long total = (long long)d.Cout * d.Cin;
     // (64-filter tiles: one group of nine taps, every tap has S0 splits)
-    hipLaunchKernelGGL(conv_halo_wg_reduce_kernel, dim3((unsigned)((total + 255) / 256), 9), dim3(256), 0, st.stream, ws,
+    hipLaunchKernelGGL(conv_halo_wg_reduce_kernel, dim3((unsigned)((total + 63) / 64), 9), dim3(256), 0, st.stream, ws,
                        static_cast<half_t *>(dW), total, a.S0, FI == 2 ? a.S0 : a.S1, a.smax, HWC ? d.Cin : 0);
     return hip_ok(hipGetLastError(), "halo weight-gradient reduce launch") ? 0 : 2;
 }
