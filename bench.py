@@ -276,7 +276,8 @@ TARGET_ROWS = (
     ("pointwise_64to128_56x56_N64_FW_WG_IG_GB/s", ["pointwise 64->128 56x56 %s N=64" % s for s in ("FW", "WG", "IG")], "GB/s"),
     ("mhsa_L197_E192_N32_FW_BW_us", ["mhsa L197 E192 3x64 %s N=32" % s for s in ("FW", "BW")], "us"),
     ("resnet20_fp16_N128_step_samples/s",
-     ["resnet20 step with batch norm, element-wise layers fused into it FW+BW+SGD"], "samples/s"),
+     ["resnet20 step with batch norm, element-wise layers fused into it, its sums formed by the convolutions"],
+     "samples/s"),
     ("mm_4096_fp16_random_then_zero_operands_TFLOP/s",
      ["power: mm 4096x4096x4096 (B transposed), random", "power: mm 4096x4096x4096 (B transposed), zero"], "TFLOP/s"),
     ("mfma_32x32x16_loop_alone_random_then_zero_operands_TFLOP/s",

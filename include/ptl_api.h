@@ -297,7 +297,9 @@ int ptl_sync(void);
  * call; 3 = as 0, but the sum-over-filter-taps route (unit-stride layers whose
  * channel counts fill whole 128-byte slabs) is taken whenever the geometry fits
  * it, on the pipelined GEMM; 5 = the same route with the input tile resident in
- * LDS for all taps (3x3 fp16 channel-major layers) wherever that kernel fits;
+ * LDS for all taps (3x3 unit-stride fp16 layers with channel counts in multiples
+ * of 64: channel-major on a prepared copy of the input, channel-minor "same"
+ * layers on the caller's tensors in place) wherever that kernel fits;
  * 6 = as 0, but the kernels for small channel-major layers (3x3 or 1x1 filters,
  * stride 1 or 2, at most 64 channels on either side, fp16 and fp32; by default
  * only up to four - for layers narrower than 64 channels sixteen - workgroups
