@@ -407,6 +407,18 @@ def power_rows(pkg, lib, hp, check, torch, dev):
                      "us": round(us, 2), "TFLOP/s": round(2.0 * ns * Co * Ci * 9 * H * H / us / 1e6, 1),
                      "W": None if w is None else round(w), "cap_W": ps.cap})
         del x, wt, y
+    # and on operands shaped like a trained network's: the input a rectified Gaussian (half of it zeros), small
+    # Gaussian filters - between the two above in the power they draw
+    x = torch.relu(torch.randn(ns, Ci, H, H, device=dev)).to(torch.float16)
+    wt = (torch.randn(Co, Ci, 3, 3, device=dev) * 0.03).to(torch.float16)
+    y = torch.zeros(ns, Co, H, H, device=dev, dtype=torch.float16)
+    a, keep = hp.conv2d_args(pkg, x, None, wt, None, y, None, Ci, H, H, Co, 3, 3, H, H, (1, 1, 1, 1))
+    ref = ctypes.byref(a)
+    us, w = ps.run(lambda: check(lib.ptl_conv2d_fp16_fw_batched(ref, ns)), sync)
+    rows.append({"workload": "power: conv2d 512->512 14x14 k3 p1 FW N=256, rectified-Gaussian input, Gaussian filters",
+                 "dtype": "fp16", "us": round(us, 2), "TFLOP/s": round(2.0 * ns * Co * Ci * 9 * H * H / us / 1e6, 1),
+                 "W": None if w is None else round(w), "cap_W": ps.cap})
+    del x, wt, y
     return rows
 
 
