@@ -275,7 +275,9 @@ __global__ __launch_bounds__(HALO_NT) void conv_halo_kernel(const HaloArgs a) {
             constexpr int ahead = sidx + NS - 1;
             constexpr int np = half == MID ? pipe_pieces<NS>(sidx) : 0, q0 = pipe_piece0<NS>(sidx);
             constexpr int nd = half == MID ? LB + np : 0;
-            constexpr int dstep = (NM - NR) / (nd > 0 ? nd : 1);  // MFMAs between two loads
+            // (the 32-filter tile has two MFMAs behind its six fragment reads: its loads go two to an MFMA)
+            constexpr int per = nd > NM - NR ? (nd + NM - NR - 1) / (NM - NR) : 1;  // loads behind one MFMA
+            constexpr int dstep = per > 1 ? 1 : (NM - NR) / (nd > 0 ? nd : 1);     // MFMAs between two loads
             static_assert(dstep >= 1, "fragment reads first, then the loads spread over the other MFMAs");
             if constexpr (half == MID) {
                 // certify stage sidx + 1; every wave has then left stage sidx - 1
@@ -302,16 +304,20 @@ __global__ __launch_bounds__(HALO_NT) void conv_halo_kernel(const HaloArgs a) {
                 constexpr int m = decltype(MI)::value, i = m / FN, j = m % FN;
                 if constexpr (m < NR) read_frag(cur ^ 1, wnext, xbuf, hn, m);
                 mfma16(acc[i][j], wf[cur][i], xf[cur][j]);
-                if constexpr (m >= NR && (m - NR) % dstep == 0 && (m - NR) / dstep < nd) {
-                    constexpr int d = (m - NR) / dstep;
-                    if constexpr (d < LB) {
-                        if constexpr (ahead < 9)
-                            issue_filter(cu, ahead, ring_lds + prev_off, d);
-                        else
-                            issue_filter(nu, ahead - 9, ring_lds + prev_off, d);
-                    } else {
-                        issue_piece(nu, next_lds, q0 + d - LB);
-                    }
+                if constexpr (m >= NR && (m - NR) % dstep == 0) {
+                    static_for<0, per>([&](auto PI) {
+                        constexpr int d = (m - NR) / dstep * per + decltype(PI)::value;
+                        if constexpr (d < nd) {
+                            if constexpr (d < LB) {
+                                if constexpr (ahead < 9)
+                                    issue_filter(cu, ahead, ring_lds + prev_off, d);
+                                else
+                                    issue_filter(nu, ahead - 9, ring_lds + prev_off, d);
+                            } else {
+                                issue_piece(nu, next_lds, q0 + d - LB);
+                            }
+                        }
+                    });
                 }
                 __builtin_amdgcn_sched_barrier(0);
             });
@@ -716,7 +722,7 @@ __global__ __launch_bounds__(256) void conv_halo_embed_kernel(const half_t *__re
 long long conv_halo_margin() { return HALO_BM + HALO_NP; }
 
 bool conv_halo_fits(const ConvTileDesc &d, int Hp, int Wp) {
-    return !d.in_hwc && d.KH == 3 && d.KW == 3 && d.sh == 1 && d.sw == 1 && d.Cin % 64 == 0 && d.Cout % 64 == 0 &&
+    return !d.in_hwc && d.KH == 3 && d.KW == 3 && d.sh == 1 && d.sw == 1 && d.Cin % 64 == 0 && d.Cout % 32 == 0 &&
            2 * Wp + 2 <= HALO_NP - HALO_BM && conv_output_fits_pads(d) && Hp >= d.Ho && Wp >= d.Wo;
 }
 
@@ -739,14 +745,16 @@ int conv_halo_launch(const ConvTileDesc &d, const void *xb, const void *wr, void
     a.maxcross = (unsigned)(skip ? crossings : 0);
     a.Q = (unsigned)((long long)d.batch * a.qimg);
     a.batch = d.batch; a.Cin = d.Cin; a.Cout = d.Cout; a.Hp = Hp; a.Wp = Wp; a.Ho = d.Ho; a.Wo = d.Wo;
-    const int bn = d.Cout % 128 == 0 ? 128 : 64;
+    const int bn = d.Cout % 128 == 0 ? 128 : d.Cout % 64 == 0 ? 64 : 32;
     a.ct_count = d.Cout / bn;
     const long long ptiles = ((long long)a.Q + HALO_BM - 1) / HALO_BM;
     if (ptiles * a.ct_count >= (1ll << 30)) return -1;
     a.tiles = (int)(ptiles * a.ct_count);
     const int grid = a.tiles < st.num_cu ? a.tiles : st.num_cu;
     a.xcd_map = grid % 8 == 0;
-    return bn == 128 ? launch_halo<128, 4, false>(a, grid, st.stream) : launch_halo<64, 6, false>(a, grid, st.stream);
+    return bn == 128  ? launch_halo<128, 4, false>(a, grid, st.stream)
+           : bn == 64 ? launch_halo<64, 6, false>(a, grid, st.stream)
+                      : launch_halo<32, 7, false>(a, grid, st.stream);
 }
 
 // Channel-minor 3x3 "same" layers (one row / column of padding on every side), unit stride, whole 64-channel slabs

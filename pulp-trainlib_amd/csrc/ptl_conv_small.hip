@@ -757,7 +757,10 @@ int plan_small(const ConvTileDesc &d, const void *X, const void *Wt, void *Y, in
     const long long tiles = (long long)d.batch * ((d.Ho + R - 1) / R);
     // beyond a few workgroups per CU the persistent kernels (filters loaded once per workgroup) are ahead where
     // both channel counts fill their 64-wide tiles; narrower layers stay ahead here for longer
-    const long long tile_limit = (d.Cin == 64 && d.Cout == 64 ? 4LL : 16LL) * st.num_cu;
+    // (64 channels into 32 filters - the input gradient of a 32 -> 64 layer - has the resident-tile kernel's 32-filter
+    // tile behind it in fp16 at unit stride)
+    const bool persistent_next = d.Cin == 64 && (d.Cout == 64 || (d.Cout == 32 && ES == 2 && K == 3 && s == 1 && dil == 1));
+    const long long tile_limit = (persistent_next ? 4LL : 16LL) * st.num_cu;
     if (st.gemm_path != 6 && tiles > tile_limit) return -1;
     if (tiles >= (1LL << 31) / 256) return -1;
     a.X = X;

@@ -176,7 +176,9 @@ int conv_taps(const ConvTileDesc &d, const void *X, const void *Wt, void *Y, con
     // from 1568 pixels on (12.6 against 24.2 us for 128 -> 128 on 14x14 at batch 8, 35.8 against 74.5 us for
     // 512 -> 512 on 7x7 at batch 32) and do not at 392 (20.5 against 14.8 us for 256 -> 256 on 7x7 at batch 8).
     const bool forced = st.gemm_path == 3 || st.gemm_path == 5;
-    if (!forced && (d.Cout < 64 || npix < 1024)) return -1;
+    // (32 filters - the input gradient of a layer with 32 channels - only on the resident-tile kernel below)
+    const bool slim = d.Cout < 64 && !(ES == 2 && !hwc && d.Cout % 32 == 0 && conv_halo_fits(d, Hp, Wp));
+    if (!forced && (slim || npix < 1024)) return -1;
     // 3x3 fp16 layers keep the input tile in LDS for all nine taps (ptl_conv_halo.hip): the tap-sum GEMM fetches it
     // once per tap.  Measured at batch 128..512, forward: 64 -> 64 on 56x56 63 against 96 us, 128 -> 128 on 28x28
     // 52 against 76, 256 -> 256 on 28x28 295 against 372, 512 -> 512 on 14x14 273 against 293.  Its workgroups are
@@ -209,6 +211,7 @@ int conv_taps(const ConvTileDesc &d, const void *X, const void *Wt, void *Y, con
     }
     const bool halo = ES == 2 && !hwc && conv_halo_fits(d, Hp, Wp) && (long long)d.batch * Hp * Wp < ((long long)1 << 31) &&
                       (st.gemm_path == 5 || (st.gemm_path == 0 && halo_pays));
+    if (!halo && d.Cout < 64 && st.gemm_path != 3) return -1;  // (the tap-sum GEMM has no tile for fewer than 64 filters)
     // chunks read past the end: the resident-tile kernel's reach, or the window of the last sample's last pixels
     const long long margin = halo ? conv_halo_margin() : ((long long)(d.KH - 1) * Wp + d.KW) * (hwc ? cblocks : 1);
     // the blocked input goes to the caller's buffer when the call brought one (the weight gradient of the layer

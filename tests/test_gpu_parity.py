@@ -477,6 +477,37 @@ def test_conv2d_resident_tile_weight_gradient_channel_minor_in_place(pkg, gpu, c
     assert rel(dx, ref_dx) <= 1e-3
 
 
+@pytest.mark.parametrize("case", [(64, 32, 14, 14, 9), (128, 96, 10, 12, 5), (64, 32, 56, 56, 3), (192, 160, 7, 30, 4)])
+def test_conv2d_resident_tile_32_filter_tiles(pkg, gpu, case):
+    """Filter counts that are multiples of 32 but not of 64 on the resident-tile kernel (32-filter tiles): the forward
+    pass of a layer into such a count and the input gradient of the mirrored layer (channel-major), against torch
+    in float32."""
+    import torch.nn.functional as F
+    Ci, Co, H, W, ns = case
+    nd = np.float16
+    rel = lambda got, ref: float((got.float() - ref).norm() / ref.norm())
+    x = dev(hp.uniform(71, (ns, Ci, H, W), dtype=nd))
+    w = dev(hp.uniform(72, (Co, Ci, 3, 3), dtype=nd) * 0.2)
+    y = dev(np.full((ns, Co, H, W), 3, nd))
+    a, keep = hp.conv2d_args(pkg, x, None, w, None, y, None, Ci, H, W, Co, 3, 3, H, W, (1, 1, 1, 1), (1, 1))
+    # mirrored layer Co -> Ci: its input gradient is a convolution from Ci channels to Co filters
+    w2 = dev(hp.uniform(73, (Ci, Co, 3, 3), dtype=nd) * 0.2)
+    dy2 = dev(hp.uniform(74, (ns, Ci, H, W), dtype=nd))
+    dx2, x2 = dev(np.full((ns, Co, H, W), 3, nd)), dev(np.zeros((ns, Co, H, W), nd))
+    b, keep2 = hp.conv2d_args(pkg, x2, dx2, w2, None, None, dy2, Co, H, W, Ci, 3, 3, H, W, (1, 1, 1, 1), (1, 1))
+    gpu.ptl_set_gemm_path(5)
+    try:
+        pkg.call("ptl_conv2d_fp16_fw_batched", a, ns)
+        assert gpu.ptl_last_conv_resident() == 1
+        pkg.call("ptl_conv2d_fp16_ig_batched", b, ns)
+        assert gpu.ptl_last_conv_resident() == 1
+    finally:
+        gpu.ptl_set_gemm_path(0)
+    sync(gpu)
+    assert rel(y, F.conv2d(x.float(), w.float(), padding=1)) <= 1e-3
+    assert rel(dx2, torch.nn.grad.conv2d_input((ns, Co, H, W), w2.float(), dy2.float(), padding=1)) <= 1e-3
+
+
 def test_conv2d_resident_tile_many_tiles(pkg, gpu):
     """More position tiles than workgroups (every workgroup walks several tiles, the last one ragged) and two
     filter tiles: the resident-tile kernel against the tap-sum GEMM and against torch in float32."""
