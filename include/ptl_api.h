@@ -462,6 +462,26 @@ int ptl_batch_norm_fused_fp32_fw_stats(const struct BatchNorm_args_fp32 *a, cons
                                        const struct ptl_norm_stats *st);
 int ptl_batch_norm_fused_fp16_fw_stats(const struct BatchNorm_args_fp16 *a, const struct ptl_norm_fusion_fp16 *f,
                                        const struct ptl_norm_stats *st);
+/* No counterpart in the reference: the backward twin of the pair above.  The one-call backward of the convolution
+ * BEHIND a normalisation forms, in the epilogue of its input gradient, the gradient g that the normalisation's
+ * backward pass starts from (struct ptl_grad_post: g = (dX [+ add]) [where mask > 0, else 0]) and the sums of g and
+ * g * x per channel; sums->valid says whether it did (the small-layer kernel on device tensors: unit stride, at most
+ * 64 channels and filters; otherwise input->diff is the plain input gradient and valid is 0).  Host tensors are
+ * rejected (status 1).
+ * ptl_batch_norm_fused_*_bw_stats is the normalisation's backward call behind it.  With bw->valid == 1 it takes
+ * output->diff as g - nothing added, nothing masked, f ignored - and, when fw (the forward sums of the
+ * normalisation's input, still in their buffer) is valid too, runs one launch instead of two.  With bw NULL or not
+ * valid it is ptl_batch_norm_fused_*_bw with f: describe the same addition and mask there (f->diff2 = post->add,
+ * f->relu with output->data = post->mask) and let f->skip_diff be output->diff, so that g ends up in output->diff
+ * either way. */
+int ptl_conv2d_fp32_bw_batched_deferred_post(const struct Conv2D_args *a, int nsamples, struct ptl_wg_batch *batch,
+                                             const struct ptl_grad_post *post, struct ptl_norm_stats *sums);
+int ptl_conv2d_fp16_bw_batched_deferred_post(const struct Conv2D_args_fp16 *a, int nsamples, struct ptl_wg_batch *batch,
+                                             const struct ptl_grad_post *post, struct ptl_norm_stats *sums);
+int ptl_batch_norm_fused_fp32_bw_stats(const struct BatchNorm_args_fp32 *a, const struct ptl_norm_fusion_fp32 *f,
+                                       const struct ptl_norm_stats *fw, const struct ptl_norm_stats *bw);
+int ptl_batch_norm_fused_fp16_bw_stats(const struct BatchNorm_args_fp16 *a, const struct ptl_norm_fusion_fp16 *f,
+                                       const struct ptl_norm_stats *fw, const struct ptl_norm_stats *bw);
 
 /* Plain product C[N x M] = A[N x K] * B (B is K x M, or M x K when trans_B),
  * the contract of the reference's mm family, on raw pointers. */

@@ -735,6 +735,19 @@ struct ptl_norm_fusion_fp16 {
     const fp16 *diff2;
 };
 
+/* No counterpart in the reference: what stands between a convolution's input gradient and the backward pass of the
+ * batch normalisation in front of that convolution, done in the convolution's epilogue
+ * (ptl_conv2d_*_bw_batched_deferred_post).  All tensors have the shape of the convolution's input (device memory):
+ *   g = input->diff as the call computes it [+ add], rounded to the tensor type, [zeroed where mask <= 0];
+ * g is what the call stores to input->diff, and the sums of g and of g * x per channel go to a struct
+ * ptl_norm_stats (part[..][0] and [1]).  x is the normalisation's input (its sums need it), mask its output when a
+ * ReLU follows it, add a second incoming gradient (the shortcut's). */
+struct ptl_grad_post {
+    const void *add;  /* NULL: none */
+    const void *mask; /* NULL: no ReLU */
+    const void *x;
+};
+
 #ifdef __cplusplus
 }
 #endif

@@ -48,6 +48,11 @@ struct ConvSmallArgs {
     // stats[(filter * ntiles + tile) * 4 + {0, 1}]; NULL: not wanted.  stats_off: bytes into LDS of the jobs' sums.
     float *stats;
     int stats_off, ntiles;
+    // Gradient epilogue (post != 0; input-gradient launches in front of a normalisation's backward pass): what is stored
+    // is g = (T)(result [+ post_add]) [where post_mask > 0, else 0], and the sums are those of g and of g * post_x.
+    // The three tensors have the shape of Y.
+    const void *post_add, *post_mask, *post_x;
+    int post, post_off;  // post_off: bytes into LDS of the waves' [32 filters][32 pixels] areas (see PostTile)
     int ksplit, red_off;    // 1: the three filter rows of a job on three waves; bytes into LDS of their partial sums
     // per item: element offset into the sample (first channel, first tile row, column group), element offset into the
     // LDS tile, first tile row | first channel << 8 | column group << 16
@@ -76,6 +81,19 @@ __device__ inline void stats_fold(float (&s0)[16], float (&s1)[16], bool up) {
 
 // T: element type; VEC = 16 / sizeof(T) elements make a 16-byte piece (8 halves, 4 floats): the channels of an LDS
 // chunk, the columns of a global piece, the k values a lane hands to one MFMA step.
+// Geometry of the gradient epilogue: a wave's LDS area holds a job's results as [32 filters][32 pixels + VEC] (the pad
+// keeps the two filter groups a wave writes at once on different banks and the rows 16-byte aligned); a lane reads
+// VEC pixels, LPR lanes share a filter, FPR filters make a round.
+template <typename T>
+struct PostTile {
+    static constexpr int VEC = 16 / (int)sizeof(T), LPR = 32 / VEC, FPR = 64 / LPR, ROUNDS = 32 / FPR;
+    static constexpr int PITCH = (32 + VEC) * (int)sizeof(T), BYTES = 32 * PITCH;
+};
+template <typename T>
+struct PostIn {
+    uint4 add[PostTile<T>::ROUNDS], mask[PostTile<T>::ROUNDS], x[PostTile<T>::ROUNDS];
+};
+
 template <typename T, int CINP, int F_MAX>
 __device__ inline void conv_small_block(const ConvSmallArgs &a, int tile, char *smem) {
     constexpr int ES = (int)sizeof(T), VEC = 16 / ES, KSTEP = 2 * VEC;
@@ -193,11 +211,85 @@ __device__ inline void conv_small_block(const ConvSmallArgs &a, int tile, char *
     const int npix = min(a.R, a.Ho - y0) * a.Wo, jobs = a.pgroups << a.mshift;
     const uint4 *T4 = reinterpret_cast<const uint4 *>(Tl);
     const size_t plane = (size_t)a.Ho * a.Wo;
+    // ---- the gradient epilogue (a.post: see ConvSmallArgs).  A job's 32 pixels are consecutive in memory (tiles are
+    // whole rows), so its results, turned through a wave's own LDS area to [filter][pixel], meet the three tensors
+    // in 16-byte pieces: a lane takes VEC pixels of one filter, PT::FPR filters a round.  The pieces of the tensors are
+    // asked for before the job's MFMAs and used behind them.
+    using PT = PostTile<T>;
+    const int pf = lane / PT::LPR, pq = lane % PT::LPR;
+    auto post_at = [&](int pg, int mb, int r, size_t &e) {
+        const int f = mb * 32 + r * PT::FPR + pf, p = pg * 32 + pq * VEC;
+        e = (((size_t)b * a.Cout + f) * a.Ho + y0) * a.Wo + p;
+        return f < a.Cout && p < npix;  // (rows are whole pieces: a piece is inside the tile or outside)
+    };
+    auto post_load = [&](int pg, int mb, PostIn<T> &in) {
+#pragma unroll
+        for (int r = 0; r < PT::ROUNDS; ++r) {
+            size_t e;
+            const bool ok = post_at(pg, mb, r, e);
+            in.add[r] = in.mask[r] = in.x[r] = make_uint4(0, 0, 0, 0);
+            if (ok && a.post_add) in.add[r] = *reinterpret_cast<const uint4 *>(reinterpret_cast<const T *>(a.post_add) + e);
+            if (ok && a.post_mask) in.mask[r] = *reinterpret_cast<const uint4 *>(reinterpret_cast<const T *>(a.post_mask) + e);
+            if (ok) in.x[r] = *reinterpret_cast<const uint4 *>(reinterpret_cast<const T *>(a.post_x) + e);
+        }
+    };
+    auto post_finish = [&](const f32x16 &acc, int job, int pg, int mb, const PostIn<T> &in) {
+        char *area = smem + a.post_off + wave * PT::BYTES;
+#pragma unroll
+        for (int v = 0; v < 16; ++v) {
+            const int f = 8 * (v >> 2) + (v & 3) + 4 * kg;
+            *reinterpret_cast<T *>(area + f * PT::PITCH + lr * ES) = (T)acc[v];
+        }
+        // (the wave's lanes read what other lanes of it wrote: nothing to wait for but the order of the accesses)
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+#pragma unroll
+        for (int r = 0; r < PT::ROUNDS; ++r) {
+            size_t e;
+            const bool ok = post_at(pg, mb, r, e);
+            Piece<T> t, va, vm, vx;
+            t.v = *reinterpret_cast<const uint4 *>(area + (r * PT::FPR + pf) * PT::PITCH + pq * 16);
+            va.v = in.add[r];
+            vm.v = in.mask[r];
+            vx.v = in.x[r];
+            float s0 = 0.f, s1 = 0.f;
+#pragma unroll
+            for (int j = 0; j < VEC; ++j) {
+                T g = t.e[j];
+                if (a.post_add) g = (T)((float)g + (float)va.e[j]);
+                if (a.post_mask && !((float)vm.e[j] > 0.f)) g = (T)0;
+                t.e[j] = g;
+                s0 += (float)g;
+                s1 += (float)g * (float)vx.e[j];
+            }
+            if (ok) *reinterpret_cast<uint4 *>(reinterpret_cast<T *>(a.Y) + e) = t.v;
+            if (a.stats) {
+                if (!ok) s0 = s1 = 0.f;  // (pixels beyond the tile's last one repeat it)
+#pragma unroll
+                for (int off = 1; off < PT::LPR; off <<= 1) {
+                    s0 += __shfl_xor(s0, off);
+                    s1 += __shfl_xor(s1, off);
+                }
+                if (pq == 0)
+                    reinterpret_cast<float2 *>(smem + a.stats_off)[job * 32 + r * PT::FPR + pf] = make_float2(s0, s1);
+            }
+        }
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+    };
     // what a wave does with the finished sums of a job: store them, and add them up for the normalisation if asked
     auto finish = [&](const f32x16 &acc, int job, int pg, int mb, int py, int px) {
+        if (a.post) {
+            PostIn<T> in;
+            post_load(pg, mb, in);
+            post_finish(acc, job, pg, mb, in);
+            return;
+        }
         const int left = a.Cout - mb * 32 - 4 * kg;  // filters from this lane's first one
+        const size_t at = (((size_t)b * a.Cout + mb * 32 + 4 * kg) * a.Ho + y0 + py) * a.Wo + px;
         if (pg * 32 + lr < npix) {
-            T *out = reinterpret_cast<T *>(a.Y) + (((size_t)b * a.Cout + mb * 32 + 4 * kg) * a.Ho + y0 + py) * a.Wo + px;
+            T *out = reinterpret_cast<T *>(a.Y) + at;
 #pragma unroll
             for (int v = 0; v < 16; ++v) {
                 const int f = 8 * (v >> 2) + (v & 3);
@@ -276,6 +368,8 @@ __device__ inline void conv_small_block(const ConvSmallArgs &a, int tile, char *
         const int py = fast_div(p, a.magic_wo), px = p - py * a.Wo;
         const uint4 *prow = T4 + (py * a.TW + px) * a.s + kg * a.POS;
         const char *frow = F + (mb * 32 + lr) * a.b_pitch + kg * 16;
+        PostIn<T> in;
+        if (a.post) post_load(pg, mb, in);
         f32x16 acc;
 #pragma unroll
         for (int v = 0; v < 16; ++v) acc[v] = 0.f;
@@ -298,7 +392,10 @@ __device__ inline void conv_small_block(const ConvSmallArgs &a, int tile, char *
                 }
             }
         }
-        finish(acc, job, pg, mb, py, px);
+        if (a.post)
+            post_finish(acc, job, pg, mb, in);
+        else
+            finish(acc, job, pg, mb, py, px);
     }
     if (a.stats) {  // the jobs' sums of a filter added in job order: one partial per workgroup and filter
         __syncthreads();
@@ -976,6 +1073,15 @@ static ::ptl_wg_batch *g_wg_defer = nullptr;  // where the one-call backward lea
 
 void conv_small_defer_to(::ptl_wg_batch *batch) { g_wg_defer = batch; }
 
+// What the input gradient of the one-call backward does in its epilogue, and where its sums go, if anything
+static const ::ptl_grad_post *g_grad_post = nullptr;
+static ::ptl_norm_stats *g_grad_sums = nullptr;
+
+void conv_small_post_to(const ::ptl_grad_post *post, ::ptl_norm_stats *sums) {
+    g_grad_post = post;
+    g_grad_sums = sums;
+}
+
 template <typename T>
 int conv_small_bw(const ConvTileDesc &fwd, const ConvTileDesc &ig, const void *X, const void *dY, const void *Wt,
                   void *dW, void *dX, bool may_defer) {
@@ -991,7 +1097,36 @@ int conv_small_bw(const ConvTileDesc &fwd, const ConvTileDesc &ig, const void *X
     const bool defer = b && b->buf && b->count >= 0 && b->count < PTL_WG_BATCH_MAX && b->used % 256 == 0 &&
                        b->used <= b->bytes && need <= b->bytes - b->used && reinterpret_cast<uintptr_t>(b->buf) % 256 == 0;
     if (defer) w.ws = reinterpret_cast<float *>(static_cast<char *>(b->buf) + b->used);
-    if (int rc = dispatch_small<T>(p, &w)) return rc;
+    if (g_grad_post && g_grad_sums && may_defer && g_grad_post->x) {
+        // the gradient epilogue: the jobs' sums in LDS behind the tile, a partial per workgroup and channel in the caller's
+        // buffer - like the forward sums; a layer whose jobs or partials do not fit goes without (sums->valid stays 0)
+        ::ptl_norm_stats *st = g_grad_sums;
+        const size_t off = (p.lds + 15) / 16 * 16, need_lds = (size_t)(p.a.pgroups << p.a.mshift) * 32 * sizeof(float2);
+        const size_t part_bytes = (size_t)ig.Cout * p.tiles * 4 * sizeof(float);
+        const size_t off2 = (off + need_lds + 15) / 16 * 16, need2 = (size_t)CS_WAVES * PostTile<T>::BYTES;
+        auto aligned = [](const void *q) { return reinterpret_cast<uintptr_t>(q) % 16 == 0; };
+        if (off2 + need2 <= 150 * 1024 && st->part && part_bytes <= st->bytes && aligned(st->part) && aligned(dX) &&
+            aligned(g_grad_post->add) && aligned(g_grad_post->mask) && aligned(g_grad_post->x) &&
+            ig.Wo % PostTile<T>::VEC == 0) {
+            p.a.post = 1;
+            p.a.post_off = (int)off2;
+            p.a.post_add = g_grad_post->add;
+            p.a.post_mask = g_grad_post->mask;
+            p.a.post_x = g_grad_post->x;
+            p.a.stats = st->part;
+            p.a.stats_off = (int)off;
+            p.a.ntiles = p.tiles;
+            p.lds = off2 + need2;
+            st->parts = p.tiles;
+            st->channels = ig.Cout;
+            st->count = (size_t)ig.batch * ig.Ho * ig.Wo;
+            st->valid = 1;
+        }
+    }
+    if (int rc = dispatch_small<T>(p, &w)) {
+        if (g_grad_sums) g_grad_sums->valid = 0;
+        return rc;
+    }
     if (!defer) return reduce_wg<T>(w, dW);
     const int at = b->count++;
     b->offset[at] = b->used;

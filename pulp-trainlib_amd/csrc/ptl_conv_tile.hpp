@@ -5,6 +5,7 @@
 struct ptl_conv_cache;
 struct ptl_wg_batch;
 struct ptl_norm_stats;
+struct ptl_grad_post;
 
 namespace ptl {
 
@@ -161,6 +162,9 @@ int conv_small_flush(struct ::ptl_wg_batch *batch);
 // Where the small-layer forward kernel leaves per-workgroup sums of its output and of its squares per filter (struct
 // ptl_norm_stats; nullptr: nowhere).  The call marks the struct valid when it filled it.
 void conv_small_stats_to(struct ::ptl_norm_stats *st);
+// What the input gradient of the next one-call backward does in its epilogue (struct ptl_grad_post) and where the sums
+// of the gradient it forms go; sums->valid tells whether it did.  Cleared with (nullptr, nullptr).
+void conv_small_post_to(const struct ::ptl_grad_post *post, struct ::ptl_norm_stats *sums);
 
 // Weight gradient over filter taps on the same GEMM (partial sums per tap and k split + one reduction).
 template <typename T>

@@ -436,6 +436,10 @@ struct BnFuse {
     T *gout;        // backward: receives g
     int relu;
     unsigned hw_magic;  // ceil(2^32 / HW) when indices and HW are below 2^16 (sample index by multiplication), else 0
+    // backward, second kernel: the sums of the gradient and of gradient * input come from here ([channel][part][4],
+    // places 0 and 1) instead of from places 2 and 3 of the first kernel's partials; NULL: from the first kernel
+    const float *part_g;
+    int nparts_g;
 };
 
 template <typename T, bool BW, bool FUSED = false>
@@ -524,16 +528,45 @@ __global__ __launch_bounds__(256) void bn_apply_kernel(const T *__restrict__ x, 
                                                        const BnFuse<T> f = BnFuse<T>()) {
     constexpr int VEC = 16 / (int)sizeof(T);
     const int c = blockIdx.x, grp = blockIdx.y, tid = threadIdx.x;
-    // the channel's partial sums (the first kernel's: at most 64, one per lane), folded by the first wave in a fixed order
+    // the channel's partial sums, four to a part, folded in a fixed order: a part per thread and round, the lanes of a
+    // wave, the four waves
     __shared__ float tot[BN_SUMS];
-    if (tid < 64) {
+    __shared__ float4 wave_tot[4];
+    {
+        float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
+        const float4 *src = reinterpret_cast<const float4 *>(part) + (size_t)c * nparts;
+        for (int i = tid; i < nparts; i += 256) {
+            const float4 p = src[i];
+            v.x += p.x;
+            v.y += p.y;
+            v.z += p.z;
+            v.w += p.w;
+        }
+        if (BW && FUSED && f.part_g) {
+            const float4 *sg = reinterpret_cast<const float4 *>(f.part_g) + (size_t)c * f.nparts_g;
+            v.z = v.w = 0.f;
+            for (int i = tid; i < f.nparts_g; i += 256) {
+                const float4 p = sg[i];
+                v.z += p.x;
+                v.w += p.y;
+            }
+        }
 #pragma unroll
-        for (int k = 0; k < (BW ? 4 : 2); ++k) {
-            float v = 0.f;
-            for (int i = tid; i < nparts; i += 64) v += part[((size_t)c * nparts + i) * BN_SUMS + k];
-#pragma unroll
-            for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off);
-            if (tid == 0) tot[k] = v;
+        for (int off = 32; off > 0; off >>= 1) {
+            v.x += __shfl_xor(v.x, off);
+            v.y += __shfl_xor(v.y, off);
+            if (BW) {
+                v.z += __shfl_xor(v.z, off);
+                v.w += __shfl_xor(v.w, off);
+            }
+        }
+        if ((tid & 63) == 0) wave_tot[tid >> 6] = v;
+        __syncthreads();
+        if (tid == 0) {
+            tot[0] = (wave_tot[0].x + wave_tot[1].x) + (wave_tot[2].x + wave_tot[3].x);
+            tot[1] = (wave_tot[0].y + wave_tot[1].y) + (wave_tot[2].y + wave_tot[3].y);
+            tot[2] = (wave_tot[0].z + wave_tot[1].z) + (wave_tot[2].z + wave_tot[3].z);
+            tot[3] = (wave_tot[0].w + wave_tot[1].w) + (wave_tot[2].w + wave_tot[3].w);
         }
     }
     __syncthreads();
@@ -620,10 +653,12 @@ __global__ __launch_bounds__(256) void bn_apply_kernel(const T *__restrict__ x, 
     }
 }
 
-// `given`: sums of the input left by the layer before (forward only); used when they cover this tensor.
+// `given`: sums of the input left by the convolution before (used when they cover this tensor).
+// `given_g` (backward): sums of the gradient and of gradient * input left by the convolution behind, which has also
+// formed the gradient itself in output->diff; valid ones switch the fusion off (nothing is added or masked again).
 template <typename T, typename Args, typename Fusion = void>
 static int batch_norm_step(const Args *a, int bw, const char *fn, const Fusion *fu = nullptr,
-                           const ::ptl_norm_stats *given = nullptr) {
+                           const ::ptl_norm_stats *given = nullptr, const ::ptl_norm_stats *given_g = nullptr) {
     constexpr bool FUSED = !std::is_void<Fusion>::value;
     if (!a || !a->input || !a->output || !a->weight_data || !a->eps || (!bw && !a->bias_data) || (FUSED && !fu))
         return glue_bad(fn, "invalid arguments");
@@ -635,7 +670,7 @@ static int batch_norm_step(const Args *a, int bw, const char *fn, const Fusion *
     if ((size_t)B * C >= ((size_t)1 << 31)) return glue_bad(fn, "too many planes");
     // groups of samples: about four workgroups per CU in the first kernel
     int groups = (4 * st.num_cu + C - 1) / C;
-    if (groups > 64) groups = 64;  // the second kernel folds them with one wave
+    if (groups > 64) groups = 64;  // (more only lengthens the second kernel's fold)
     if (groups > B) groups = B;
     const int per_group = (B + groups - 1) / groups;
     groups = (B + per_group - 1) / per_group;
@@ -653,6 +688,10 @@ static int batch_norm_step(const Args *a, int bw, const char *fn, const Fusion *
     const int VEC = 16 / (int)sizeof(T);
     const T *eps = sg.in(reinterpret_cast<const T *>(a->eps), (size_t)1);
     if (!x) return glue_bad(fn, "null buffer");
+    auto covers = [&](const ::ptl_norm_stats *g) {
+        return g && g->valid == 1 && g->part && g->channels == C && g->parts > 0 && g->count == (size_t)B * HW &&
+               (size_t)C * g->parts * BN_SUMS * sizeof(float) <= g->bytes && reinterpret_cast<uintptr_t>(g->part) % 16 == 0;
+    };
     if (!bw) {
         T *y = sg.out(reinterpret_cast<T *>(a->output->data), n);
         const T *b = sg.in(reinterpret_cast<const T *>(a->bias_data), (size_t)C);
@@ -666,9 +705,7 @@ static int batch_norm_step(const Args *a, int bw, const char *fn, const Fusion *
             if (sg.failed()) return 2;
             vec = vec && aligned16(f.skip);
         }
-        const bool have = given && given->valid == 1 && given->part && given->channels == C && given->parts > 0 &&
-                          given->count == (size_t)B * HW &&
-                          (size_t)C * given->parts * BN_SUMS * sizeof(float) <= given->bytes;
+        const bool have = covers(given);
         if (!have)
             hipLaunchKernelGGL((bn_sums_kernel<T, false>), dim3(C, groups), dim3(256), 0, st.stream, x,
                                (const T *)nullptr, part, B, C, HW, per_group, vec, f0);
@@ -685,7 +722,19 @@ static int batch_norm_step(const Args *a, int bw, const char *fn, const Fusion *
         int vec = HW % VEC == 0 && aligned16(x) && aligned16(dy) && (!dx || aligned16(dx));
         BnFuse<T> f = {};
         f.hw_magic = hw_magic;
+        const bool formed = FUSED && covers(given_g);  // the gradient in output->diff is final
         if constexpr (FUSED) {
+            if (formed && covers(given)) {
+                // every sum is there: the second kernel alone
+                f.part_g = given_g->part;
+                f.nparts_g = given_g->parts;
+                hipLaunchKernelGGL((bn_apply_kernel<T, true, FUSED>), dim3(C, want_dx ? groups : 1), dim3(256), 0,
+                                   st.stream, x, dy, dx, w, (const T *)nullptr, eps, given->part, dg, db, B, C, HW,
+                                   given->parts, per_group, want_dx ? 1 : 0, vec, f);
+                return sg.finish(hip_ok(hipGetLastError(), "batch norm launch") ? 0 : 2);
+            }
+        }
+        if constexpr (FUSED) if (!formed) {
             f.relu = fu->relu ? 1 : 0;
             if (f.relu) {
                 if (!a->output->data) return glue_bad(fn, "the ReLU mask needs the forward result in output->data");
@@ -782,6 +831,17 @@ int ptl_batch_norm_fused_fp16_fw_stats(const struct BatchNorm_args_fp16 *a, cons
                                        const struct ptl_norm_stats *st) {
     static const struct ptl_norm_fusion_fp16 none = {};
     return ptl::batch_norm_step<ptl::half_t>(a, 0, "ptl_batch_norm_fused_fp16_fw_stats", f ? f : &none, st);
+}
+
+int ptl_batch_norm_fused_fp32_bw_stats(const struct BatchNorm_args_fp32 *a, const struct ptl_norm_fusion_fp32 *f,
+                                       const struct ptl_norm_stats *fw, const struct ptl_norm_stats *bw) {
+    static const struct ptl_norm_fusion_fp32 none = {};
+    return ptl::batch_norm_step<float>(a, 1, "ptl_batch_norm_fused_fp32_bw_stats", f ? f : &none, fw, bw);
+}
+int ptl_batch_norm_fused_fp16_bw_stats(const struct BatchNorm_args_fp16 *a, const struct ptl_norm_fusion_fp16 *f,
+                                       const struct ptl_norm_stats *fw, const struct ptl_norm_stats *bw) {
+    static const struct ptl_norm_fusion_fp16 none = {};
+    return ptl::batch_norm_step<ptl::half_t>(a, 1, "ptl_batch_norm_fused_fp16_bw_stats", f ? f : &none, fw, bw);
 }
 
 }  // extern "C"

@@ -984,6 +984,46 @@ static int conv2d_fw_stats(const Args *a, int ns, ::ptl_norm_stats *st, const ch
     return rc;
 }
 
+// Backward step whose input gradient becomes the gradient a normalisation in front of this layer starts from:
+// input->diff = (dX [+ post->add]) [where post->mask > 0, else 0], rounded to T after the sum like a tensor an
+// element-wise layer would have written, and the sums of that gradient and of its products with post->x in `sums`
+// (valid = 1) - when the small-layer kernel takes the layer.  Any other route leaves the plain input gradient and
+// sums->valid = 0.  Device tensors only.
+template <typename T, typename Args>
+static int conv2d_bw_post(const Args *a, int ns, ::ptl_wg_batch *batch, const ::ptl_grad_post *post,
+                          ::ptl_norm_stats *sums, const char *fn) {
+    if (!post || !sums || !post->x) {
+        set_error("%s: null gradient epilogue or statistics struct", fn);
+        return 1;
+    }
+    sums->valid = 0;
+    if (!a || !a->input || !a->input->diff || a->skip_in_grad) {
+        set_error("%s: the gradient epilogue needs the input gradient", fn);
+        return 1;
+    }
+    if (ns <= 0 || a->input->C <= 0 || a->input->H <= 0 || a->input->W <= 0) {
+        set_error("%s: invalid tensor geometry", fn);
+        return 1;
+    }
+    if (!ensure_init()) return 2;
+    const size_t n = (size_t)ns * a->input->C * a->input->H * a->input->W;
+    {
+        Stager sg(true);  // host tensors are rejected
+        (void)sg.inout(reinterpret_cast<T *>(a->input->diff), n);
+        if (post->add) (void)sg.in(reinterpret_cast<const T *>(post->add), n);
+        if (post->mask) (void)sg.in(reinterpret_cast<const T *>(post->mask), n);
+        (void)sg.in(reinterpret_cast<const T *>(post->x), n);
+        if (sg.failed()) return sg.rejected() ? 1 : 2;
+    }
+    conv_small_defer_to(batch);
+    conv_small_post_to(post, sums);
+    const int rc = conv2d_bw<T>(a, ns, fn);
+    conv_small_post_to(nullptr, nullptr);
+    conv_small_defer_to(nullptr);
+    if (rc) sums->valid = 0;
+    return rc;
+}
+
 }  // namespace ptl
 
 // ---- C ABI -------------------------------------------------------------------------------
@@ -1076,6 +1116,14 @@ int ptl_conv2d_fp32_bw_batched_deferred(const struct Conv2D_args *a, int ns, str
     const int rc = ptl::conv2d_bw<float>(a, ns, "pulp_conv2d_fp32_bw_cl");
     ptl::conv_small_defer_to(nullptr);
     return rc;
+}
+int ptl_conv2d_fp16_bw_batched_deferred_post(const struct Conv2D_args_fp16 *a, int ns, struct ptl_wg_batch *batch,
+                                             const struct ptl_grad_post *post, struct ptl_norm_stats *sums) {
+    return ptl::conv2d_bw_post<half_t>(a, ns, batch, post, sums, "pulp_conv2d_fp16_bw_cl");
+}
+int ptl_conv2d_fp32_bw_batched_deferred_post(const struct Conv2D_args *a, int ns, struct ptl_wg_batch *batch,
+                                             const struct ptl_grad_post *post, struct ptl_norm_stats *sums) {
+    return ptl::conv2d_bw_post<float>(a, ns, batch, post, sums, "pulp_conv2d_fp32_bw_cl");
 }
 int ptl_conv2d_fp16_fw_batched_stats(const struct Conv2D_args_fp16 *a, int ns, struct ptl_norm_stats *st) {
     return ptl::conv2d_fw_stats<half_t>(a, ns, st, "pulp_conv2d_fp16_fw_cl");

@@ -180,6 +180,11 @@ class NormStats(C.Structure):
     _fields_ = [("part", P), ("bytes", C.c_size_t), ("count", C.c_size_t), ("parts", I), ("channels", I), ("valid", I)]
 
 
+class GradPost(C.Structure):
+    """struct ptl_grad_post: what ptl_conv2d_*_bw_batched_deferred_post does to its input gradient."""
+    _fields_ = [("add", P), ("mask", P), ("x", P)]
+
+
 class NormFusion(C.Structure):
     """struct ptl_norm_fusion_fp32 / _fp16: what ptl_batch_norm_fused_* does behind the normalisation."""
     _fields_ = [("relu", I), ("skip", P), ("skip_diff", P), ("diff2", P)]

@@ -44,16 +44,18 @@ def init_weights(seed, dt):
 class ResNetStep:
     """Device buffers, argument structs and the call sequence of one training step on `ns` samples."""
 
-    def __init__(self, pkg, lib, torch, dt, ns, weights, lr=0.01, norm=False, fused=False, stats=False):
+    def __init__(self, pkg, lib, torch, dt, ns, weights, lr=0.01, norm=False, fused=False, stats=False, post=False):
         """`fused` (with `norm`): ReLU, the residual sum and the sum of a tensor's two incoming gradients run inside
         the normalisation calls (ptl_batch_norm_fused_*) instead of as element-wise calls of their own and the backward
         calls defer the additions of their weight gradients to one flush; with `stats` the forward convolutions also
         leave the sums the normalisation behind them needs (ptl_conv2d_*_fw_batched_stats), which then runs one launch
-        instead of two."""
+        instead of two; with `post` (and `stats`) the backward calls of the convolutions also form the gradient the
+        normalisation in front of them starts from, and its sums (ptl_conv2d_*_bw_batched_deferred_post,
+        ptl_batch_norm_fused_*_bw_stats): that normalisation's backward pass is one launch as well."""
         self.pkg, self.lib, self.dt, self.ns, self.lr = pkg, lib, dt, ns, lr
         if fused:
-            assert norm
-            self.use_stats = stats
+            assert norm and (stats or not post)
+            self.use_stats, self.use_post = stats, post
             return self._build_fused(torch, weights)
         assert not stats
         tdt = torch.float16 if dt == "fp16" else torch.float32
@@ -193,12 +195,14 @@ class ResNetStep:
         L = lambda name: name.replace("DT", dt)
 
         self.stats = {}  # per convolution: the struct its forward call fills and its normalisation reads
+        self.grad_stats = {}  # per normalisation: the struct the backward call of the convolution behind it fills
         self.wg_buf = torch.empty(64 << 20, dtype=torch.uint8, device="cuda")
         self.wg_batch = pkg.WgBatch()
         self.wg_batch.buf, self.wg_batch.bytes = self.wg_buf.data_ptr(), self.wg_buf.numel()
 
-        def conv(name, x, dx, H):
-            """The convolution alone: (forward call, backward calls, output, its gradient, output size)."""
+        def conv(name, x, dx, H, post=None):
+            """The convolution alone: (forward call, backward calls, output, its gradient, output size).  `post`:
+            (ptl_grad_post, ptl_norm_stats) of the normalisation in front of it."""
             ci, co, k, s = spec[name]
             p = k // 2
             Ho = (H + 2 * p - k) // s + 1
@@ -209,6 +213,8 @@ class ResNetStep:
             # weight and input gradient in one call (the stem needs no input gradient); the additions that complete
             # the weight gradients of the small layers wait for one flush behind the backward pass
             bw = [(L("ptl_conv2d_DT_bw_batched_deferred"), a, (ns, self.wg_batch))] if dx is not None else [(L("ptl_conv2d_DT_wg_batched"), a, (ns,))]
+            if post is not None:
+                bw = [(L("ptl_conv2d_DT_bw_batched_deferred_post"), a, (ns, self.wg_batch, post[0], post[1]))]
             if not self.use_stats:
                 return (L("ptl_conv2d_DT_fw_batched"), a, (ns,)), bw, y, dy, Ho
             # the forward call leaves the sums of its output for the normalisation behind it
@@ -219,13 +225,15 @@ class ResNetStep:
             self.keep.append(part)
             return (L("ptl_conv2d_DT_fw_batched_stats"), a, (ns, st)), bw, y, dy, Ho
 
-        def norm(name, y, dy, Ho, relu, skip=None, out_diff=None):
+        def norm(name, y, dy, Ho, relu, skip=None, out_diff=None, out=None):
             """out = [relu](bn(y) [+ skip]); returns the calls, out, its gradient buffer and the fusion struct (whose
-            skip_diff / diff2 the caller fills in once the tensors exist)."""
+            skip_diff / diff2 the caller fills in once the tensors exist) - with `post` a triple of that struct, the
+            ptl_grad_post and the ptl_norm_stats for the backward call of the convolution that reads `out`."""
             co = spec[name][1]
             self.G[name], self.Bt[name] = torch.ones(co, dtype=tdt, device="cuda"), z(co)
             self.dG[name], self.dBt[name] = z(co), z(co)
-            out, dout = z(ns, co, Ho, Ho), (out_diff if out_diff is not None else z(ns, co, Ho, Ho))
+            out = out if out is not None else z(ns, co, Ho, Ho)
+            dout = out_diff if out_diff is not None else z(ns, co, Ho, Ho)
             na, kp = hp.batch_norm_args(pkg, y, out, self.G[name], self.Bt[name], eps, ns, co, Ho, Ho, dy, dout,
                                         self.dG[name], self.dBt[name])
             f = pkg.NormFusion()
@@ -233,6 +241,17 @@ class ResNetStep:
             f.skip = pkg.addr(skip)
             self.keep += [kp, f, skip]
             fw = (L("ptl_batch_norm_fused_DT_fw_stats"), na, (f, self.stats[name])) if self.use_stats else (L("ptl_batch_norm_fused_DT_fw"), na, (f,))
+            if self.use_post and out_diff is None:
+                # the gradient of the sum is formed in place, by the convolution behind or (where that one leaves it
+                # to this call) here
+                f.skip_diff = pkg.addr(dout)
+                po, gs = pkg.GradPost(), pkg.NormStats()
+                po.mask, po.x = (pkg.addr(out) if relu else None), pkg.addr(y)
+                part = torch.zeros(1 << 16, dtype=torch.float32, device="cuda")
+                gs.part, gs.bytes = part.data_ptr(), part.numel() * 4
+                self.keep += [po, gs, part]
+                self.grad_stats[name] = gs
+                return fw, (L("ptl_batch_norm_fused_DT_bw_stats"), na, (f, self.stats[name], gs)), out, dout, (f, po, gs)
             return fw, (L("ptl_batch_norm_fused_DT_bw"), na, (f,)), out, dout, f
 
         self.x = z(ns, 3, 32, 32)
@@ -241,34 +260,45 @@ class ResNetStep:
         self.fw = [cf, nf]
         first_bw = [nb] + cb
         bw_blocks = []
+        post = self.use_post
         for (n, ci, co, stride, proj) in blocks:
             xin, dxin, Hin, fus_in = t, dt_, H, fus
-            c1f, c1b, y1, dy1, H = conv(n + "c1", xin, dxin, Hin)
-            n1f, n1b, a1, da1, _ = norm(n + "c1", y1, dy1, H, 1)
-            c2f, c2b, y2, dy2, H = conv(n + "c2", a1, da1, H)
+            c1f, c1b, y1, dy1, H = conv(n + "c1", xin, dxin, Hin, fus_in[1:] if post else None)
+            n1f, n1b, a1, da1, fus1 = norm(n + "c1", y1, dy1, H, 1)
+            c2f, c2b, y2, dy2, H = conv(n + "c2", a1, da1, H, fus1[1:] if post else None)
             seq = [c1f, n1f, c2f]
-            ds_ = z(*y2.shape)  # gradient of the sum = gradient of the shortcut branch
+            # gradient of the sum = gradient of the shortcut branch (in place in the gradient of the block's output
+            # when the convolution behind the block forms it)
+            ds_ = None if post else z(*y2.shape)
             if proj:
                 dproj = z(*xin.shape)
                 csf, csb, ysr, dysr, _ = conv(proj, xin, dproj, Hin)
-                # the projection's normalisation (no ReLU, nothing added) reads ds_ as the gradient of its output
-                nsf, nsb, ys, _, _ = norm(proj, ysr, dysr, H, 0, out_diff=ds_)
-                seq += [csf, nsf]
+                # the projection's normalisation (no ReLU, nothing added) reads the gradient of the sum as the
+                # gradient of its output
+                nsf, nsb, ys = None, None, z(*y2.shape)
                 skip = ys
             else:
                 skip = xin
             n2f, n2b, t, dt_, fus = norm(n + "c2", y2, dy2, H, 1, skip=skip)
-            fus.skip_diff = pkg.addr(ds_)
+            if post:
+                ds_ = dt_
+            else:
+                fus.skip_diff = pkg.addr(ds_)
             self.keep.append(ds_)
+            if proj:
+                nsf, nsb, _, _, _ = norm(proj, ysr, dysr, H, 0, out_diff=ds_, out=ys)
+                seq += [csf, nsf]
             seq.append(n2f)
             self.fw += seq
-            b = [n2b] + c2b + [n1b] + c1b
-            if proj:
-                b += [nsb] + csb
-                fus_in.diff2 = pkg.addr(dproj)  # the block's input gets its gradient from c1 and from the projection
-                self.keep.append(dproj)
+            add = dproj if proj else ds_  # the block's input gets its gradient from c1 and from the shortcut
+            if post:
+                # (the projection's backward pass first: c1's call adds its input gradient)
+                b = [n2b] + c2b + [n1b] + ([nsb] + csb if proj else []) + c1b
+                fus_in[0].diff2 = fus_in[1].add = pkg.addr(add)
             else:
-                fus_in.diff2 = pkg.addr(ds_)    # ... or from c1 and the identity shortcut
+                b = [n2b] + c2b + [n1b] + c1b + ([nsb] + csb if proj else [])
+                fus_in.diff2 = pkg.addr(add)
+            self.keep.append(add)
             bw_blocks.append(b)
         self._tail(torch, t, dt_, H, bw_blocks, first_bw, ncls)
 

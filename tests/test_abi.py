@@ -30,7 +30,8 @@ def test_library_exports_every_declared_symbol(pkg):
     assert not missing, missing
     # and the Python lists name nothing the header does not declare
     listed = set(pkg.VOID_ENTRY_POINTS + pkg.BATCHED_ENTRY_POINTS + pkg.OTHER_ENTRY_POINTS + pkg.STEP_ENTRY_POINTS +
-                 pkg.PLAIN_ENTRY_POINTS + pkg.FUSED_NORM_ENTRY_POINTS + pkg.CACHED_ENTRY_POINTS + pkg.DEFERRED_ENTRY_POINTS + pkg.STATS_ENTRY_POINTS)
+                 pkg.PLAIN_ENTRY_POINTS + pkg.FUSED_NORM_ENTRY_POINTS + pkg.CACHED_ENTRY_POINTS + pkg.DEFERRED_ENTRY_POINTS + pkg.STATS_ENTRY_POINTS +
+                 pkg.GRAD_STATS_ENTRY_POINTS)
     assert listed == set(names)
 
 
@@ -50,7 +51,7 @@ STRUCTS = {
     "SkipConn_args": "SkipConnArgs", "SkipConn_args_fp16": "SkipConnArgs", "pool_args": "PoolArgs",
     "pool_args_fp16": "PoolArgs", "loss_args": "LossArgs", "loss_args_fp16": "LossArgs", "optim_args": "OptimArgs",
     "optim_args_fp16": "OptimArgsFp16", "BatchNorm_args_fp32": "BatchNormArgs", "BatchNorm_args_fp16": "BatchNormArgs",
-    "ptl_norm_fusion_fp32": "NormFusion", "ptl_norm_fusion_fp16": "NormFusion", "ptl_conv_cache": "ConvCache", "ptl_wg_batch": "WgBatch", "ptl_norm_stats": "NormStats",
+    "ptl_norm_fusion_fp32": "NormFusion", "ptl_norm_fusion_fp16": "NormFusion", "ptl_conv_cache": "ConvCache", "ptl_wg_batch": "WgBatch", "ptl_norm_stats": "NormStats", "ptl_grad_post": "GradPost",
 }
 
 
@@ -160,7 +161,7 @@ def test_struct_fields_match_the_reference_headers():
     mine = mod.struct_fields(open(os.path.join(ROOT, "include", "ptl_structs.h")).read())
     gold = json.load(open(os.path.join(ROOT, "tests", "golden", "struct_fields.json")))
     assert set(mine) == set(gold["reference_structs"]) | set(gold["extensions"])
-    assert gold["extensions"] == ["BatchNorm_args_fp16", "ptl_conv_cache", "ptl_norm_fusion_fp16", "ptl_norm_fusion_fp32",
+    assert gold["extensions"] == ["BatchNorm_args_fp16", "ptl_conv_cache", "ptl_grad_post", "ptl_norm_fusion_fp16", "ptl_norm_fusion_fp32",
                                   "ptl_norm_stats", "ptl_wg_batch"]
     norm = lambda t: t.replace("unsigned int", "unsigned").strip()
     for name, ref in gold["reference_structs"].items():

@@ -394,6 +394,124 @@ def test_conv2d_forward_sums_feed_the_normalisation(pkg, gpu, dt):
             assert torch.equal(o1, o2), case
 
 
+@pytest.mark.parametrize("dt", ["fp16", "fp32"])
+def test_conv2d_backward_forms_the_gradient_of_the_normalisation_in_front(pkg, gpu, dt):
+    """ptl_conv2d_*_bw_batched_deferred_post: where the small-layer kernel takes the layer (sums.valid == 1), input->diff
+    is bit for bit what the plain call's input gradient, the addition of a second gradient (rounded to the tensor type)
+    and the ReLU mask give as separate steps, the weight gradient is the plain call's, and the struct's parts add up to
+    the sums of that gradient and of its products with the normalisation's input (float64 sums of the stored tensors;
+    the kernel adds the same values in fp32).  Elsewhere input->diff is the plain input gradient and nothing is
+    written to the buffer.  ptl_batch_norm_fused_*_bw_stats behind it: against ptl_batch_norm_fused_*_bw on the
+    plain gradient with the same addition and mask, to the rounding of the statistics - with the forward sums given
+    (one launch) and without (two), and bit for bit when the convolution left no sums."""
+    tdt = torch.float16 if dt == "fp16" else torch.float32
+    tol = 2e-3 if dt == "fp16" else 2e-5
+    part = torch.empty(1 << 18, dtype=torch.float32, device="cuda")
+    wg_buf = torch.empty(16 << 20, dtype=torch.uint8, device="cuda")
+    #        ns, Ci, Co, H, K, stride, add, mask, room, sums expected (None: either)
+    room = part.numel() * 4
+    cases = [(128, 16, 16, 32, 3, 1, 1, 1, room, True), (64, 32, 32, 16, 3, 1, 0, 1, room, True),
+             (32, 64, 64, 8, 3, 1, 1, 0, room, None), (64, 16, 32, 16, 3, 1, 1, 1, room, True),
+             (5, 24, 40, 16, 3, 1, 1, 1, room, None), (3, 8, 20, 24, 3, 1, 0, 0, room, None),
+             (7, 12, 36, 24, 3, 1, 1, 1, room, None), (64, 16, 32, 32, 3, 2, 1, 1, room, None),
+             (4, 128, 128, 8, 3, 1, 1, 1, room, False), (128, 16, 16, 32, 3, 1, 1, 1, 4096, False)]
+    taken = 0
+    for case in cases:
+        ns, Ci, Co, H, K, s, with_add, with_mask, room, expect = case
+        p = K // 2
+        Ho = (H + 2 * p - K) // s + 1
+        x = (torch.rand(ns, Ci, H, H, device="cuda") - 0.5).to(tdt)
+        w = (torch.rand(Co, Ci, K, K, device="cuda") - 0.5).to(tdt)
+        dy = (torch.rand(ns, Co, Ho, Ho, device="cuda") - 0.5).to(tdt)
+        y = torch.zeros(ns, Co, Ho, Ho, device="cuda", dtype=tdt)
+        add = (torch.rand(ns, Ci, H, H, device="cuda") - 0.5).to(tdt)
+        xn = (torch.rand(ns, Ci, H, H, device="cuda") - 0.3).to(tdt)  # the normalisation's input; x is its output
+        got = []
+        for post_mode in (False, True):
+            dx, dw = torch.full_like(x, 3), torch.full_like(w, 3)
+            a, kp = hp.conv2d_args(pkg, x, dx, w, dw, y, dy, Ci, H, H, Co, K, K, Ho, Ho, (p, p, p, p), (s, s), 0,
+                                   1 if s == 1 else 0)
+            batch = pkg.WgBatch()
+            batch.buf, batch.bytes = wg_buf.data_ptr(), wg_buf.numel()
+            st = pkg.NormStats()
+            part.fill_(7.0)
+            st.part, st.bytes, st.valid = part.data_ptr(), room, 5
+            if post_mode:
+                po = pkg.GradPost()
+                po.add, po.mask, po.x = add.data_ptr() if with_add else None, x.data_ptr() if with_mask else None, xn.data_ptr()
+                rc = getattr(gpu, "ptl_conv2d_%s_bw_batched_deferred_post" % dt)(ctypes.byref(a), ns, ctypes.byref(batch),
+                                                                                ctypes.byref(po), ctypes.byref(st))
+            else:
+                rc = getattr(gpu, "ptl_conv2d_%s_bw_batched_deferred" % dt)(ctypes.byref(a), ns, ctypes.byref(batch))
+            assert rc == 0, gpu.ptl_last_error()
+            assert getattr(gpu, "ptl_conv2d_%s_wg_flush" % dt)(ctypes.byref(batch)) == 0
+            assert gpu.ptl_sync() == 0
+            got.append((dx, dw, st))
+        (dx0, dw0, _), (dx1, dw1, st) = got
+        assert torch.equal(dw0, dw1), case
+        assert st.valid in (0, 1) and (expect is None or st.valid == int(expect)), case
+        g_ref = dx0
+        if with_add:
+            g_ref = (g_ref.float() + add.float()).to(tdt)
+        if with_mask:
+            g_ref = torch.where(x > 0, g_ref, torch.zeros_like(g_ref))
+        if st.valid:
+            taken += 1
+            assert torch.equal(dx1, g_ref), case
+            assert st.channels == Ci and st.count == ns * H * H and st.parts >= 1
+            used = Ci * st.parts * 4
+            assert used * 4 <= room and bool((part[used:] == 7.0).all()), case
+            pt = part[:used].view(Ci, st.parts, 4).double()
+            s0, s1 = pt[:, :, 0].sum(1), pt[:, :, 1].sum(1)
+            gd, xd = g_ref.double(), xn.double()
+            r0, r1 = gd.sum((0, 2, 3)), (gd * xd).sum((0, 2, 3))
+            assert bool(((s0 - r0).abs() <= 1e-5 * gd.abs().sum((0, 2, 3)) + 1e-6).all()), case
+            assert bool(((s1 - r1).abs() <= 1e-5 * (gd * xd).abs().sum((0, 2, 3)) + 1e-6).all()), case
+        else:
+            assert torch.equal(dx1, dx0), case
+            assert bool((part == 7.0).all()), case
+        # the normalisation in front of the convolution: input xn, output x (the mask), gradient of the output dx
+        gm, bt = (torch.rand(Ci, device="cuda") + 0.5).to(tdt), (torch.rand(Ci, device="cuda") - 0.5).to(tdt)
+        eps = torch.tensor([1e-5], device="cuda").to(tdt)
+        fw_part = torch.zeros(Ci, 1, 4, dtype=torch.float32, device="cuda")
+        fw_part[:, 0, 0], fw_part[:, 0, 1] = xn.double().sum((0, 2, 3)).float(), (xn.double() ** 2).sum((0, 2, 3)).float()
+        fw = pkg.NormStats()
+        fw.part, fw.bytes, fw.count, fw.parts, fw.channels, fw.valid = fw_part.data_ptr(), fw_part.numel() * 4, ns * H * H, 1, Ci, 1
+        # the reference: the fused backward call on the plain gradient
+        dyr, dxr, dgr, dbr = dx0.clone(), torch.full_like(x, 3), torch.full_like(gm, 3), torch.full_like(gm, 3)
+        fr = pkg.NormFusion()
+        fr.relu, fr.diff2, fr.skip_diff = with_mask, add.data_ptr() if with_add else None, dyr.data_ptr()
+        nr, kr = hp.batch_norm_args(pkg, xn, x, gm, bt, eps, ns, Ci, H, H, dxr, dyr, dgr, dbr)
+        assert getattr(gpu, "ptl_batch_norm_fused_%s_bw" % dt)(ctypes.byref(nr), ctypes.byref(fr)) == 0
+        assert gpu.ptl_sync() == 0
+        assert torch.equal(dyr, g_ref), case  # (the gradient of the sum, in place)
+        for fw_given in (fw, None):
+            dyn, dxn, dgn, dbn = dx1.clone(), torch.full_like(x, 3), torch.full_like(gm, 3), torch.full_like(gm, 3)
+            fn = pkg.NormFusion()
+            fn.relu, fn.diff2, fn.skip_diff = with_mask, add.data_ptr() if with_add else None, dyn.data_ptr()
+            nn_, kn = hp.batch_norm_args(pkg, xn, x, gm, bt, eps, ns, Ci, H, H, dxn, dyn, dgn, dbn)
+            rc = getattr(gpu, "ptl_batch_norm_fused_%s_bw_stats" % dt)(ctypes.byref(nn_), ctypes.byref(fn),
+                                                                      ctypes.byref(fw_given) if fw_given else None, ctypes.byref(st))
+            assert rc == 0, gpu.ptl_last_error()
+            assert gpu.ptl_sync() == 0
+            assert torch.equal(dyn, g_ref), case
+            if st.valid:
+                assert hp.rel_l2(dxn.float().cpu().numpy(), dxr.float().cpu().numpy()) <= tol, case
+                assert hp.rel_l2(dgn.float().cpu().numpy(), dgr.float().cpu().numpy()) <= tol, case
+                assert hp.rel_l2(dbn.float().cpu().numpy(), dbr.float().cpu().numpy()) <= tol, case
+            else:
+                assert torch.equal(dxn, dxr) and torch.equal(dgn, dgr) and torch.equal(dbn, dbr), case
+    assert taken >= 3
+    # host tensors are rejected
+    xh = np.zeros((2, 16, 8, 8), dtype=hp.np_dtype(dt))
+    wh, yh = np.zeros((16, 16, 3, 3), dtype=xh.dtype), np.zeros((2, 16, 8, 8), dtype=xh.dtype)
+    a, kp = hp.conv2d_args(pkg, xh, xh.copy(), wh, wh.copy(), yh, yh.copy(), 16, 8, 8, 16, 3, 3, 8, 8, (1, 1, 1, 1), (1, 1), 0, 1)
+    po, st = pkg.GradPost(), pkg.NormStats()
+    po.x = xh.ctypes.data
+    rc = getattr(gpu, "ptl_conv2d_%s_bw_batched_deferred_post" % dt)(ctypes.byref(a), 2, None, ctypes.byref(po), ctypes.byref(st))
+    assert rc == 1 and st.valid == 0
+
+
 @pytest.mark.parametrize("seed", [21, 22])
 def test_depthwise_random_geometries(pkg, gpu, seed):
     rng = random.Random(seed)

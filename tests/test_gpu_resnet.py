@@ -131,7 +131,43 @@ def test_resnet20_step_with_sums_from_the_convolutions(pkg, gpu, dt, ns, tol):
             assert rel(given.dBt[n], own.dBt[n]) <= tol, n
 
 
-@pytest.mark.parametrize("fused", [True, False, "stats"])
+@pytest.mark.parametrize("dt,ns,tol", [("fp32", 6, 1e-3), ("fp16", 16, 5e-3)])
+def test_resnet20_step_with_gradient_sums_from_the_convolutions(pkg, gpu, dt, ns, tol):
+    """The step whose backward convolutions also form the gradient of the normalisation in front of them and its sums
+    (ptl_conv2d_*_bw_batched_deferred_post / ptl_batch_norm_fused_*_bw_stats) against the step whose normalisation
+    layers do that themselves: the same forward pass bit for bit, the unit-stride 3x3 layers leave their sums (the
+    normalisation behind a stride-2 layer, a projection's and the last one form their own), and the gradients come
+    out the same to the rounding of the statistics (fp32: everything the step writes; fp16, where one flipped
+    rounding moves the deepest gradients by per cent: the last stage's)."""
+    w = rs.init_weights(0x2E620, dt)
+    x = hp.normal(0x2E621, (ns, 3, 32, 32)).astype(hp.np_dtype(dt))
+    nets = []
+    for post in (False, True):
+        net = rs.ResNetStep(pkg, gpu, torch, dt, ns, w, 0.01, norm=True, fused=True, stats=True, post=post)
+        net.x.copy_(torch.from_numpy(x))
+        net.target.zero_()
+        net.target[torch.arange(ns), (3 * torch.arange(ns)) % 10] = 1
+        net.step(update=True)
+        assert gpu.ptl_sync() == 0
+        nets.append(net)
+    own, given = nets
+    assert torch.equal(own.logits, given.logits) and torch.equal(own.loss, given.loss)
+    # 19 normalisation layers have a convolution behind them; two of those convolutions have stride 2
+    valid = sum(st.valid for st in given.grad_stats.values())
+    assert len(given.grad_stats) == 19 and (valid >= 16 if dt == "fp16" else 10 <= valid <= 18), valid
+    print("gradient sums left by", valid, "of 19")
+    assert own.launches() == given.launches()
+    rel = lambda a, b: hp.rel_l2(a.float().cpu().numpy(), b.float().cpu().numpy())
+    names = list(own.dW) if dt == "fp32" else ["fc", "s2b2c2", "s2b2c1", "s2b1c2"]
+    for n in names:
+        assert rel(given.dW[n], own.dW[n]) <= tol, n
+        assert rel(given.W[n], own.W[n]) <= tol, n
+    for n in (own.dG if dt == "fp32" else ["s2b2c2", "s2b2c1", "s2b1c2"]):
+        assert rel(given.dG[n], own.dG[n]) <= tol, n
+        assert rel(given.dBt[n], own.dBt[n]) <= tol, n
+
+
+@pytest.mark.parametrize("fused", [True, False, "stats", "post"])
 def test_training_step_replays_as_a_hip_graph(pkg, gpu, fused):
     """The whole step (92 or 178 library calls; "stats": the 92 with the sums of the convolutions' outputs formed by
     the convolutions) captured once into a HIP graph on a stream of the caller's and
@@ -145,7 +181,7 @@ def test_training_step_replays_as_a_hip_graph(pkg, gpu, fused):
     try:
         with torch.cuda.stream(side):
             net = rs.ResNetStep(pkg, gpu, torch, dt, ns, rs.init_weights(0x2E600, dt), 0.01, norm=True, fused=bool(fused),
-                                stats=fused == "stats")
+                                stats=fused in ("stats", "post"), post=fused == "post")
             net.x.copy_(torch.from_numpy(hp.normal(0x2E601, (ns, 3, 32, 32)).astype(np.float16)))
             net.target.zero_()
             net.target[torch.arange(ns), (3 * torch.arange(ns)) % 10] = 1
