@@ -313,7 +313,9 @@ int ptl_sync(void);
  * the route of pointwise layers over a batch) (1) or a tile-per-workgroup
  * kernel (0); ptl_last_conv_resident() whether the last Conv2D call that took
  * the tap route kept its input tile in LDS (1), or ran the small-layer kernels
- * (2: forward, either gradient, or both gradients in one call);
+ * (2: forward, either gradient, or both gradients in one call; 3: the forward
+ * kernel that also applied the normalisation in front of the layer, see
+ * ptl_conv2d_*_fw_batched_normed);
  * ptl_last_gemm_tile() the output tile of the last product that ran a tile-per-workgroup kernel of the
  * look-up-free pipelined GEMM, as rows * 1000 + columns (256256 = 256 x 256, 128064 = 128 x 64). */
 void ptl_set_gemm_path(int path);
@@ -462,6 +464,18 @@ int ptl_batch_norm_fused_fp32_fw_stats(const struct BatchNorm_args_fp32 *a, cons
                                        const struct ptl_norm_stats *st);
 int ptl_batch_norm_fused_fp16_fw_stats(const struct BatchNorm_args_fp16 *a, const struct ptl_norm_fusion_fp16 *f,
                                        const struct ptl_norm_stats *st);
+/* No counterpart in the reference: ptl_batch_norm_fused_*_fw_stats(norm, f, norm_st) followed by
+ * ptl_conv2d_*_fw_batched_stats(a, nsamples, st) (st may be NULL: no sums wanted) for a convolution that reads the
+ * normalisation's output (norm->output->data == a->input->data) - same results bit for bit, the normalisation's
+ * output tensor included.  Where the small-layer kernel takes the convolution (device tensors, valid norm_st, every
+ * input row read by the tile that starts at it: unit or double stride with "same" padding) it is one launch: the
+ * kernel normalises its input tile while it loads it and writes the normalisation's output on the way. */
+int ptl_conv2d_fp32_fw_batched_normed(const struct Conv2D_args *a, int nsamples, struct ptl_norm_stats *st,
+                                      const struct BatchNorm_args_fp32 *norm, const struct ptl_norm_fusion_fp32 *f,
+                                      const struct ptl_norm_stats *norm_st);
+int ptl_conv2d_fp16_fw_batched_normed(const struct Conv2D_args_fp16 *a, int nsamples, struct ptl_norm_stats *st,
+                                      const struct BatchNorm_args_fp16 *norm, const struct ptl_norm_fusion_fp16 *f,
+                                      const struct ptl_norm_stats *norm_st);
 /* No counterpart in the reference: the backward twin of the pair above.  The one-call backward of the convolution
  * BEHIND a normalisation forms, in the epilogue of its input gradient, the gradient g that the normalisation's
  * backward pass starts from (struct ptl_grad_post: g = (dX [+ add]) [where mask > 0, else 0]) and the sums of g and

@@ -19,6 +19,7 @@
 #include "ptl_conv_tile.hpp"
 #include "ptl_structs.h"
 #include "ptl_host.hpp"
+#include "ptl_norm_fold.hpp"
 
 namespace ptl {
 namespace {
@@ -53,6 +54,16 @@ struct ConvSmallArgs {
     // The three tensors have the shape of Y.
     const void *post_add, *post_mask, *post_x;
     int post, post_off;  // post_off: bytes into LDS of the waves' [32 filters][32 pixels] areas (see PostTile)
+    // A normalisation in front of the layer, applied while the input is loaded (pre != 0; forward launches): X is the
+    // normalisation's input, pre_part its sums ([channel][part][4], over pre_count elements per channel), and what the
+    // taps see is out = [relu](norm(X) * weight + bias [+ pre_skip]), which the workgroup that owns a row also
+    // writes to pre_out (every input row is owned by the tile whose output rows start at it).  pre_off: bytes into
+    // LDS of the channels' {mean, weight / deviation, bias, -}.
+    const float *pre_part;
+    const void *pre_w, *pre_b, *pre_eps, *pre_skip;
+    void *pre_out;
+    float pre_count;
+    int pre, pre_parts, pre_relu, pre_off;
     int ksplit, red_off;    // 1: the three filter rows of a job on three waves; bytes into LDS of their partial sums
     // per item: element offset into the sample (first channel, first tile row, column group), element offset into the
     // LDS tile, first tile row | first channel << 8 | column group << 16
@@ -129,6 +140,18 @@ __device__ inline void conv_small_block(const ConvSmallArgs &a, int tile, char *
         const int q = tid + CS_NT * k;
         if (q < a.f_chunks) fin[k].v = reinterpret_cast<const uint4 *>(a.Wt)[q];
     }
+    if (a.pre) {  // the statistics of the normalisation in front: a wave per channel
+        float4 *tab = reinterpret_cast<float4 *>(smem + a.pre_off);
+        for (int c = wave; c < a.Cin; c += CS_WAVES) {
+            const float4 v = norm_fold_wave(a.pre_part, a.pre_parts, c, lane);
+            if (lane == 0) {
+                float mean, sd;
+                norm_mean_sd(v.x, v.y, a.pre_count, (float)reinterpret_cast<const T *>(a.pre_eps)[0], mean, sd);
+                tab[c] = make_float4(mean, (float)reinterpret_cast<const T *>(a.pre_w)[c] / sd,
+                                     (float)reinterpret_cast<const T *>(a.pre_b)[c], 0.f);
+            }
+        }
+    }
 
     // channels the tensor does not have must read as zeros on the filter side too (0 x garbage is not 0)
     if (a.Cin < CINP) {
@@ -145,18 +168,6 @@ __device__ inline void conv_small_block(const ConvSmallArgs &a, int tile, char *
         const int cb = fast_div(row, a.magic_rr), rr = row - cb * a.RR;
         const int col = hc < a.padL ? hc : a.Win + hc;
         reinterpret_cast<uint4 *>(Tl)[cb * a.POS + rr * a.TW + col] = make_uint4(0, 0, 0, 0);
-    }
-    // ---- input pieces -> [channel block][row][column] chunks
-    T *tl = Tl + lrow * a.TW * VEC + lch;
-#pragma unroll
-    for (int k = 0; k < CS_IN_MAX; ++k) {
-        const int item = wave + CS_WAVES * k;
-        if (item < a.items && (a.item_rc[item] & 255) + lrow < a.RR) {
-            T *row = tl + a.item_l[item];
-            const int step = VEC * a.dil;
-#pragma unroll
-            for (int j = 0; j < VEC; ++j) row[j * step] = xin[k].e[j];
-        }
     }
     // ---- filter pieces -> [filter][tap][channel]: element (outer, inner, tap) of the dense tensor goes to
     // (filter, channel) = (outer, inner), or (inner, outer) with the taps flipped; the address moves with the indices
@@ -202,6 +213,49 @@ __device__ inline void conv_small_block(const ConvSmallArgs &a, int tile, char *
                 for (int j = 0; j < VEC; ++j)
                     *reinterpret_cast<T *>(F + (j < n1 ? at0 : rest) + j * step_tap) = fin[k].e[j];
             }
+        }
+    }
+    // (asked for only now, with the filter pieces out of their registers)
+    Piece<T> skp[CS_IN_MAX];
+    if (a.pre && a.pre_skip) {
+        const T *ss = reinterpret_cast<const T *>(a.pre_skip) + (xs - X);
+#pragma unroll
+        for (int k = 0; k < CS_IN_MAX; ++k) {
+            const int item = wave + CS_WAVES * k;
+            skp[k].v = make_uint4(0, 0, 0, 0);
+            if (item < a.items) {
+                const int rc = a.item_rc[item], rr = (rc & 255) + lrow, ch = ((rc >> 8) & 255) + lch, iy = iy0 + rr;
+                if (rr < a.RR && ch < a.Cin && iy >= 0 && iy < a.Hin)
+                    skp[k].v = *reinterpret_cast<const uint4 *>(ss + a.item_g[item]);
+            }
+        }
+    }
+    // ---- input pieces -> [channel block][row][column] chunks
+    T *tl = Tl + lrow * a.TW * VEC + lch;
+    if (a.pre) __syncthreads();  // (the channels' statistics are in LDS)
+#pragma unroll
+    for (int k = 0; k < CS_IN_MAX; ++k) {
+        const int item = wave + CS_WAVES * k;
+        if (item < a.items && (a.item_rc[item] & 255) + lrow < a.RR) {
+            if (a.pre) {
+                const int rc = a.item_rc[item], ch = ((rc >> 8) & 255) + lch, iy = iy0 + (rc & 255) + lrow;
+                if (ch < a.Cin && iy >= 0 && iy < a.Hin) {  // (a piece of the tensor, not of the padding)
+                    const float4 t = reinterpret_cast<const float4 *>(smem + a.pre_off)[ch];
+#pragma unroll
+                    for (int j = 0; j < VEC; ++j) {
+                        float v = norm_forward((float)xin[k].e[j], t.x, t.y, t.z);
+                        if (a.pre_skip) v += (float)skp[k].e[j];
+                        if (a.pre_relu) v = fmaxf(v, 0.f);
+                        xin[k].e[j] = (T)v;
+                    }
+                    if (iy >= y0 * a.s && iy < (y0 + a.R) * a.s)
+                        *reinterpret_cast<uint4 *>(reinterpret_cast<T *>(a.pre_out) + (xs - X) + a.item_g[item]) = xin[k].v;
+                }
+            }
+            T *row = tl + a.item_l[item];
+            const int step = VEC * a.dil;
+#pragma unroll
+            for (int j = 0; j < VEC; ++j) row[j * step] = xin[k].e[j];
         }
     }
     __syncthreads();
@@ -1027,10 +1081,45 @@ static ::ptl_norm_stats *g_norm_stats = nullptr;  // where the forward pass leav
 
 void conv_small_stats_to(::ptl_norm_stats *st) { g_norm_stats = st; }
 
+static const ConvPreNorm *g_pre_norm = nullptr;  // the normalisation the next forward call applies, if any
+static bool g_pre_taken = false;
+
+void conv_small_pre_to(const ConvPreNorm *pre) {
+    g_pre_norm = pre;
+    g_pre_taken = false;
+}
+bool conv_small_pre_pending() { return g_pre_norm && !g_pre_taken; }
+
 template <typename T>
 int conv_small(const ConvTileDesc &d, const void *X, const void *Wt, void *Y) {
     SmallPlan p;
-    if (int rc = plan_small<T>(d, X, Wt, Y, state().num_cu, p)) return rc;
+    const ConvPreNorm *pre = g_pre_norm;
+    if (int rc = plan_small<T>(d, X, Wt, Y, state().num_cu, p)) return pre ? CONV_PRE_REFUSED : rc;
+    if (pre) {
+        // the table of the channels' statistics behind the tile; every input row must be a row that some tile both
+        // loads and owns (rows [y0 * s, (y0 + R) * s) of the tile at output row y0)
+        auto aligned = [](const void *q) { return reinterpret_cast<uintptr_t>(q) % 16 == 0; };
+        const size_t off = (p.lds + 15) / 16 * 16, need = (size_t)d.Cin * sizeof(float4);
+        const bool ok = X == pre->out && pre->x && pre->weight && pre->bias && pre->eps && pre->part && pre->parts > 0 &&
+                        aligned(pre->x) && aligned(pre->out) && aligned(pre->skip) && aligned(pre->part) &&
+                        p.a.dil == 1 && d.padU <= d.KH - d.sh && (long long)d.Ho * d.sh >= d.Hin &&
+                        pre->count == (size_t)d.batch * d.Hin * d.Win && off + need <= 150 * 1024;
+        if (!ok) return CONV_PRE_REFUSED;
+        p.a.X = pre->x;
+        p.a.pre = 1;
+        p.a.pre_out = pre->out;
+        p.a.pre_skip = pre->skip;
+        p.a.pre_w = pre->weight;
+        p.a.pre_b = pre->bias;
+        p.a.pre_eps = pre->eps;
+        p.a.pre_part = pre->part;
+        p.a.pre_parts = pre->parts;
+        p.a.pre_relu = pre->relu;
+        p.a.pre_count = (float)d.batch * (float)(d.Hin * d.Win);
+        p.a.pre_off = (int)off;
+        p.lds = off + need;
+        g_pre_taken = true;
+    }
     if (::ptl_norm_stats *st = g_norm_stats) {
         // a pair of sums per job (32 pixels x 32 filters) in LDS behind the tile, a partial per workgroup and filter
         // in the caller's buffer; a layer whose jobs or partials do not fit goes without
@@ -1048,7 +1137,9 @@ int conv_small(const ConvTileDesc &d, const void *X, const void *Wt, void *Y) {
             st->valid = 1;
         }
     }
-    return dispatch_small<T>(p, nullptr);
+    const int rc = dispatch_small<T>(p, nullptr);
+    if (pre && rc == 0) state().last_conv_resident = 3;
+    return rc;
 }
 
 template <typename T>

@@ -162,6 +162,21 @@ int conv_small_flush(struct ::ptl_wg_batch *batch);
 // Where the small-layer forward kernel leaves per-workgroup sums of its output and of its squares per filter (struct
 // ptl_norm_stats; nullptr: nowhere).  The call marks the struct valid when it filled it.
 void conv_small_stats_to(struct ::ptl_norm_stats *st);
+// A normalisation layer that the next forward call of the small-layer kernel applies while it loads its input
+// (nullptr: none).  x: the normalisation's input; out: its output = the convolution's input tensor, written by the
+// call; skip: added after the normalisation (or null); weight, bias, eps: the layer's; part / parts / count: the
+// sums of x ([channel][part][4] floats).  A call that cannot honour it launches nothing and returns CONV_PRE_REFUSED;
+// conv_small_pre_pending() tells a caller that routes elsewhere that it must not.
+struct ConvPreNorm {
+    const void *x, *skip, *weight, *bias, *eps;
+    void *out;
+    const float *part;
+    int parts, relu;
+    size_t count;
+};
+constexpr int CONV_PRE_REFUSED = -3;
+void conv_small_pre_to(const ConvPreNorm *pre);
+bool conv_small_pre_pending();
 // What the input gradient of the next one-call backward does in its epilogue (struct ptl_grad_post) and where the sums
 // of the gradient it forms go; sums->valid tells whether it did.  Cleared with (nullptr, nullptr).
 void conv_small_post_to(const struct ::ptl_grad_post *post, struct ::ptl_norm_stats *sums);

@@ -6,6 +6,7 @@
 
 #include "ptl_api.h"
 #include "ptl_host.hpp"
+#include "ptl_norm_fold.hpp"
 #include "ptl_structs.h"
 
 namespace ptl {
@@ -528,45 +529,20 @@ __global__ __launch_bounds__(256) void bn_apply_kernel(const T *__restrict__ x, 
                                                        const BnFuse<T> f = BnFuse<T>()) {
     constexpr int VEC = 16 / (int)sizeof(T);
     const int c = blockIdx.x, grp = blockIdx.y, tid = threadIdx.x;
-    // the channel's partial sums, four to a part, folded in a fixed order: a part per thread and round, the lanes of a
-    // wave, the four waves
+    // the channel's partial sums, folded by the first wave (the order every kernel that needs them keeps)
     __shared__ float tot[BN_SUMS];
-    __shared__ float4 wave_tot[4];
-    {
-        float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
-        const float4 *src = reinterpret_cast<const float4 *>(part) + (size_t)c * nparts;
-        for (int i = tid; i < nparts; i += 256) {
-            const float4 p = src[i];
-            v.x += p.x;
-            v.y += p.y;
-            v.z += p.z;
-            v.w += p.w;
-        }
+    if (tid < 64) {
+        float4 v = norm_fold_wave(part, nparts, c, tid);
         if (BW && FUSED && f.part_g) {
-            const float4 *sg = reinterpret_cast<const float4 *>(f.part_g) + (size_t)c * f.nparts_g;
-            v.z = v.w = 0.f;
-            for (int i = tid; i < f.nparts_g; i += 256) {
-                const float4 p = sg[i];
-                v.z += p.x;
-                v.w += p.y;
-            }
+            const float4 g = norm_fold_wave(f.part_g, f.nparts_g, c, tid);
+            v.z = g.x;
+            v.w = g.y;
         }
-#pragma unroll
-        for (int off = 32; off > 0; off >>= 1) {
-            v.x += __shfl_xor(v.x, off);
-            v.y += __shfl_xor(v.y, off);
-            if (BW) {
-                v.z += __shfl_xor(v.z, off);
-                v.w += __shfl_xor(v.w, off);
-            }
-        }
-        if ((tid & 63) == 0) wave_tot[tid >> 6] = v;
-        __syncthreads();
         if (tid == 0) {
-            tot[0] = (wave_tot[0].x + wave_tot[1].x) + (wave_tot[2].x + wave_tot[3].x);
-            tot[1] = (wave_tot[0].y + wave_tot[1].y) + (wave_tot[2].y + wave_tot[3].y);
-            tot[2] = (wave_tot[0].z + wave_tot[1].z) + (wave_tot[2].z + wave_tot[3].z);
-            tot[3] = (wave_tot[0].w + wave_tot[1].w) + (wave_tot[2].w + wave_tot[3].w);
+            tot[0] = v.x;
+            tot[1] = v.y;
+            tot[2] = v.z;
+            tot[3] = v.w;
         }
     }
     __syncthreads();
@@ -574,8 +550,8 @@ __global__ __launch_bounds__(256) void bn_apply_kernel(const T *__restrict__ x, 
 #pragma unroll
     for (int k = 0; k < (BW ? 4 : 2); ++k) s[k] = tot[k];
     const float cnt = (float)B * (float)HW;
-    const float mean = s[0] / cnt;
-    const float sd = sqrtf(((s[1] - 2 * s[0] * mean) / cnt) + (mean * mean) + (float)eps[0]);
+    float mean, sd;
+    norm_mean_sd(s[0], s[1], cnt, (float)eps[0], mean, sd);
     const float w = (float)weight[c];
     const float bb = BW ? 0.f : (float)bias[c];
     const float db = s[2], dg = (s[3] - mean * s[2]) / sd;
@@ -585,8 +561,9 @@ __global__ __launch_bounds__(256) void bn_apply_kernel(const T *__restrict__ x, 
     }
     if (BW && !write_dx) return;
     const float k0 = w / sd, k1 = db / cnt, k2 = dg / cnt;
+    const float gain = w / sd;  // (the forward pass's division once per channel, not per element)
     auto map = [&](float xv, float gv) {
-        if (!BW) return ((xv - mean) / sd) * w + bb;
+        if (!BW) return norm_forward(xv, mean, gain, bb);
         const float xh = (xv - mean) / sd;
         return k0 * (gv - k1 - xh * k2);
     };

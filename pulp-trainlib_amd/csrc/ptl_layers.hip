@@ -273,6 +273,8 @@ static int conv2d_fw(const Args *a, int ns, const char *fn) {
             c.m = axis_plain(g.Co, 1);
         }
         if (!g.hwc) rc = conv_small<T>(d, X, Wt, Y);
+        // (a normalisation to apply on the way in is the small-layer kernel's business alone: nothing was launched)
+        if (rc == CONV_PRE_REFUSED || conv_small_pre_pending()) return CONV_PRE_REFUSED;
         if (rc < 0) rc = conv_taps<T>(d, X, Wt, Y, c);
         if (rc < 0) rc = conv_tile<T>(d, X, Wt, Y, c);
         if (rc > 0) return sg.finish(rc);
@@ -984,6 +986,60 @@ static int conv2d_fw_stats(const Args *a, int ns, ::ptl_norm_stats *st, const ch
     return rc;
 }
 
+// The forward call of a normalisation layer and of the convolution that reads its output, in that order - as one
+// launch where the small-layer kernel takes the convolution (it then applies the normalisation to its input tile while
+// it loads it and writes the normalisation's output on the way), as the two calls otherwise.  Same results bit for bit.
+template <typename T, typename Args, typename NormArgs, typename Fusion>
+static int conv2d_fw_normed(const Args *a, int ns, ::ptl_norm_stats *st_out, const NormArgs *n, const Fusion *f,
+                            const ::ptl_norm_stats *st_in, int (*norm_call)(const NormArgs *, const Fusion *,
+                                                                            const ::ptl_norm_stats *),
+                            const char *fn) {
+    if (!a || !n) {
+        set_error("%s: null argument", fn);
+        return 1;
+    }
+    if (st_out) st_out->valid = 0;
+    const bool shapes = a->input && n->input && n->output && n->output->data && n->output->data == a->input->data &&
+                        n->input->data && n->weight_data && n->bias_data && n->eps && ns > 0 && n->B == ns &&
+                        n->C == a->input->C && n->H == a->input->H && n->W == a->input->W && n->C > 0 && n->H > 0 && n->W > 0;
+    const bool sums = st_in && st_in->valid == 1 && st_in->part && st_in->parts > 0 && shapes && st_in->channels == n->C &&
+                      st_in->count == (size_t)ns * n->H * n->W &&
+                      (size_t)n->C * st_in->parts * 4 * sizeof(float) <= st_in->bytes;
+    if (sums && ensure_init() && state().gemm_path != 1) {
+        const size_t cnt = (size_t)ns * n->C * n->H * n->W;
+        bool device;
+        {
+            Stager sg(true);  // (host tensors: the two calls, which stage them)
+            (void)sg.in(reinterpret_cast<const T *>(n->input->data), cnt);
+            (void)sg.out(reinterpret_cast<T *>(n->output->data), cnt);
+            if (f && f->skip) (void)sg.in(reinterpret_cast<const T *>(f->skip), cnt);
+            (void)sg.in(reinterpret_cast<const T *>(n->weight_data), (size_t)n->C);
+            (void)sg.in(reinterpret_cast<const T *>(n->bias_data), (size_t)n->C);
+            (void)sg.in(reinterpret_cast<const T *>(n->eps), (size_t)1);
+            device = !sg.failed();
+        }
+        if (device) {
+            ConvPreNorm pre = {};
+            pre.x = n->input->data;
+            pre.out = n->output->data;
+            pre.skip = f ? f->skip : nullptr;
+            pre.weight = n->weight_data;
+            pre.bias = n->bias_data;
+            pre.eps = n->eps;
+            pre.part = st_in->part;
+            pre.parts = st_in->parts;
+            pre.relu = f && f->relu ? 1 : 0;
+            pre.count = st_in->count;
+            conv_small_pre_to(&pre);
+            const int rc = st_out ? conv2d_fw_stats<T>(a, ns, st_out, fn) : conv2d_fw<T>(a, ns, fn);
+            conv_small_pre_to(nullptr);
+            if (rc != CONV_PRE_REFUSED) return rc;
+        }
+    }
+    if (int rc = norm_call(n, f, st_in)) return rc;
+    return st_out ? conv2d_fw_stats<T>(a, ns, st_out, fn) : conv2d_fw<T>(a, ns, fn);
+}
+
 // Backward step whose input gradient becomes the gradient a normalisation in front of this layer starts from:
 // input->diff = (dX [+ post->add]) [where post->mask > 0, else 0], rounded to T after the sum like a tensor an
 // element-wise layer would have written, and the sums of that gradient and of its products with post->x in `sums`
@@ -1116,6 +1172,18 @@ int ptl_conv2d_fp32_bw_batched_deferred(const struct Conv2D_args *a, int ns, str
     const int rc = ptl::conv2d_bw<float>(a, ns, "pulp_conv2d_fp32_bw_cl");
     ptl::conv_small_defer_to(nullptr);
     return rc;
+}
+int ptl_conv2d_fp16_fw_batched_normed(const struct Conv2D_args_fp16 *a, int ns, struct ptl_norm_stats *st,
+                                      const struct BatchNorm_args_fp16 *norm, const struct ptl_norm_fusion_fp16 *f,
+                                      const struct ptl_norm_stats *norm_st) {
+    return ptl::conv2d_fw_normed<half_t>(a, ns, st, norm, f, norm_st, ptl_batch_norm_fused_fp16_fw_stats,
+                                         "pulp_conv2d_fp16_fw_cl");
+}
+int ptl_conv2d_fp32_fw_batched_normed(const struct Conv2D_args *a, int ns, struct ptl_norm_stats *st,
+                                      const struct BatchNorm_args_fp32 *norm, const struct ptl_norm_fusion_fp32 *f,
+                                      const struct ptl_norm_stats *norm_st) {
+    return ptl::conv2d_fw_normed<float>(a, ns, st, norm, f, norm_st, ptl_batch_norm_fused_fp32_fw_stats,
+                                        "pulp_conv2d_fp32_fw_cl");
 }
 int ptl_conv2d_fp16_bw_batched_deferred_post(const struct Conv2D_args_fp16 *a, int ns, struct ptl_wg_batch *batch,
                                              const struct ptl_grad_post *post, struct ptl_norm_stats *sums) {

@@ -44,18 +44,20 @@ def init_weights(seed, dt):
 class ResNetStep:
     """Device buffers, argument structs and the call sequence of one training step on `ns` samples."""
 
-    def __init__(self, pkg, lib, torch, dt, ns, weights, lr=0.01, norm=False, fused=False, stats=False, post=False):
+    def __init__(self, pkg, lib, torch, dt, ns, weights, lr=0.01, norm=False, fused=False, stats=False, post=False, pre=False):
         """`fused` (with `norm`): ReLU, the residual sum and the sum of a tensor's two incoming gradients run inside
         the normalisation calls (ptl_batch_norm_fused_*) instead of as element-wise calls of their own and the backward
         calls defer the additions of their weight gradients to one flush; with `stats` the forward convolutions also
         leave the sums the normalisation behind them needs (ptl_conv2d_*_fw_batched_stats), which then runs one launch
         instead of two; with `post` (and `stats`) the backward calls of the convolutions also form the gradient the
         normalisation in front of them starts from, and its sums (ptl_conv2d_*_bw_batched_deferred_post,
-        ptl_batch_norm_fused_*_bw_stats): that normalisation's backward pass is one launch as well."""
+        ptl_batch_norm_fused_*_bw_stats): that normalisation's backward pass is one launch as well; with `pre` (and `stats`) the
+        forward call of a convolution also stands for the forward call of the normalisation in front of it
+        (ptl_conv2d_*_fw_batched_normed)."""
         self.pkg, self.lib, self.dt, self.ns, self.lr = pkg, lib, dt, ns, lr
         if fused:
-            assert norm and (stats or not post)
-            self.use_stats, self.use_post = stats, post
+            assert norm and (stats or not (post or pre))
+            self.use_stats, self.use_post, self.use_pre = stats, post, pre
             return self._build_fused(torch, weights)
         assert not stats
         tdt = torch.float16 if dt == "fp16" else torch.float32
@@ -200,9 +202,10 @@ class ResNetStep:
         self.wg_batch = pkg.WgBatch()
         self.wg_batch.buf, self.wg_batch.bytes = self.wg_buf.data_ptr(), self.wg_buf.numel()
 
-        def conv(name, x, dx, H, post=None):
+        def conv(name, x, dx, H, post=None, pre=None):
             """The convolution alone: (forward call, backward calls, output, its gradient, output size).  `post`:
-            (ptl_grad_post, ptl_norm_stats) of the normalisation in front of it."""
+            (ptl_grad_post, ptl_norm_stats) of the normalisation in front of it; `pre`: that normalisation's forward
+            call, which this layer's forward call then includes."""
             ci, co, k, s = spec[name]
             p = k // 2
             Ho = (H + 2 * p - k) // s + 1
@@ -223,6 +226,8 @@ class ResNetStep:
             st.part, st.bytes = part.data_ptr(), part.numel() * 4
             self.stats[name] = st
             self.keep.append(part)
+            if pre is not None:
+                return (L("ptl_conv2d_DT_fw_batched_normed"), a, (ns, st, pre[1], pre[2][0], pre[2][1])), bw, y, dy, Ho
             return (L("ptl_conv2d_DT_fw_batched_stats"), a, (ns, st)), bw, y, dy, Ho
 
         def norm(name, y, dy, Ho, relu, skip=None, out_diff=None, out=None):
@@ -257,16 +262,17 @@ class ResNetStep:
         self.x = z(ns, 3, 32, 32)
         cf, cb, y, dy, H = conv("stem", self.x, None, 32)
         nf, nb, t, dt_, fus = norm("stem", y, dy, H, 1)
-        self.fw = [cf, nf]
+        post, pre = self.use_post, self.use_pre
+        # (pending: the forward call of a normalisation that the next convolution's call will stand for)
+        self.fw, pending = ([cf], nf) if pre else ([cf, nf], None)
         first_bw = [nb] + cb
         bw_blocks = []
-        post = self.use_post
         for (n, ci, co, stride, proj) in blocks:
             xin, dxin, Hin, fus_in = t, dt_, H, fus
-            c1f, c1b, y1, dy1, H = conv(n + "c1", xin, dxin, Hin, fus_in[1:] if post else None)
+            c1f, c1b, y1, dy1, H = conv(n + "c1", xin, dxin, Hin, fus_in[1:] if post else None, pending)
             n1f, n1b, a1, da1, fus1 = norm(n + "c1", y1, dy1, H, 1)
-            c2f, c2b, y2, dy2, H = conv(n + "c2", a1, da1, H, fus1[1:] if post else None)
-            seq = [c1f, n1f, c2f]
+            c2f, c2b, y2, dy2, H = conv(n + "c2", a1, da1, H, fus1[1:] if post else None, n1f if pre else None)
+            seq = [c1f, c2f] if pre else [c1f, n1f, c2f]
             # gradient of the sum = gradient of the shortcut branch (in place in the gradient of the block's output
             # when the convolution behind the block forms it)
             ds_ = None if post else z(*y2.shape)
@@ -288,7 +294,10 @@ class ResNetStep:
             if proj:
                 nsf, nsb, _, _, _ = norm(proj, ysr, dysr, H, 0, out_diff=ds_, out=ys)
                 seq += [csf, nsf]
-            seq.append(n2f)
+            if pre:
+                pending = n2f
+            else:
+                seq.append(n2f)
             self.fw += seq
             add = dproj if proj else ds_  # the block's input gets its gradient from c1 and from the shortcut
             if post:
@@ -300,6 +309,8 @@ class ResNetStep:
                 fus_in.diff2 = pkg.addr(add)
             self.keep.append(add)
             bw_blocks.append(b)
+        if pending is not None:
+            self.fw.append(pending)
         self._tail(torch, t, dt_, H, bw_blocks, first_bw, ncls)
 
     def _tail(self, torch, t, dt_, H, bw_blocks, first_bw, ncls):

@@ -395,6 +395,95 @@ def test_conv2d_forward_sums_feed_the_normalisation(pkg, gpu, dt):
 
 
 @pytest.mark.parametrize("dt", ["fp16", "fp32"])
+def test_conv2d_forward_applies_the_normalisation_in_front(pkg, gpu, dt):
+    """ptl_conv2d_*_fw_batched_normed against the two calls it stands for (ptl_batch_norm_fused_*_fw_stats, then
+    ptl_conv2d_*_fw_batched_stats): the normalisation's output tensor, the convolution's output and the sums it
+    leaves, bit for bit - where the small-layer kernel does both in one launch (ptl_last_conv_resident() == 3: 3x3
+    layers of either stride with "same" padding, with and without ReLU and skip tensor, ragged tiles) and where it
+    cannot and the two calls run (a wide layer, a strided 1x1 layer that does not read every row, no padding,
+    sums that do not cover the tensor, host tensors)."""
+    tdt = torch.float16 if dt == "fp16" else torch.float32
+    part0 = torch.empty(1 << 18, dtype=torch.float32, device="cuda")
+    parts = [torch.empty(1 << 18, dtype=torch.float32, device="cuda") for _ in range(2)]
+    #        ns, Cp, Ci, Co, H, K, stride, pad, relu, skip, sums valid, one launch expected (None: either)
+    cases = [(128, 3, 16, 16, 32, 3, 1, 1, 1, 0, 1, True), (64, 16, 32, 32, 16, 3, 1, 1, 1, 1, 1, True),
+             (32, 16, 16, 32, 32, 3, 2, 1, 1, 1, 1, True), (16, 32, 64, 64, 8, 3, 1, 1, 0, 1, 1, None),
+             (5, 8, 24, 40, 16, 3, 1, 1, 1, 1, 1, None), (3, 8, 20, 12, 24, 3, 1, 1, 0, 0, 1, None),
+             (7, 12, 36, 24, 24, 1, 1, 0, 1, 0, 1, None), (32, 16, 16, 32, 32, 1, 2, 0, 1, 1, 1, False),
+             (8, 16, 16, 16, 16, 3, 1, 0, 1, 0, 1, False), (4, 16, 128, 128, 8, 3, 1, 1, 1, 1, 1, False),
+             (64, 16, 32, 32, 16, 3, 1, 1, 1, 1, 0, False)]
+    fused = 0
+    for case in cases:
+        ns, Cp, Ci, Co, H, K, s, p, relu, with_skip, sums_valid, expect = case
+        Ho = (H + 2 * p - K) // s + 1
+        # the layer in front: a 3x3 convolution whose output the normalisation reads, and its sums
+        xp = (torch.rand(ns, Cp, H, H, device="cuda") - 0.5).to(tdt)
+        wp = (torch.rand(Ci, Cp, 3, 3, device="cuda") - 0.5).to(tdt)
+        y0 = torch.zeros(ns, Ci, H, H, device="cuda", dtype=tdt)
+        a0, k0 = hp.conv2d_args(pkg, xp, None, wp, None, y0, None, Cp, H, H, Ci, 3, 3, H, H, (1, 1, 1, 1), (1, 1), 0, 1)
+        st_in = pkg.NormStats()
+        st_in.part, st_in.bytes = part0.data_ptr(), part0.numel() * 4
+        assert getattr(gpu, "ptl_conv2d_%s_fw_batched_stats" % dt)(ctypes.byref(a0), ns, ctypes.byref(st_in)) == 0
+        if not st_in.valid:  # (a layer in front that leaves no sums: those of the stored tensor, as one part)
+            part0[:Ci * 4].view(Ci, 1, 4)[:, 0, 0] = y0.double().sum((0, 2, 3)).float()
+            part0[:Ci * 4].view(Ci, 1, 4)[:, 0, 1] = (y0.double() ** 2).sum((0, 2, 3)).float()
+            st_in.count, st_in.parts, st_in.channels, st_in.valid = ns * H * H, 1, Ci, 1
+        if not sums_valid:
+            st_in.count += 1
+        gm, bt = (torch.rand(Ci, device="cuda") + 0.5).to(tdt), (torch.rand(Ci, device="cuda") - 0.5).to(tdt)
+        eps = torch.tensor([1e-5], device="cuda").to(tdt)
+        skip = (torch.rand(ns, Ci, H, H, device="cuda") - 0.5).to(tdt)
+        w = (torch.rand(Co, Ci, K, K, device="cuda") - 0.5).to(tdt)
+        f = pkg.NormFusion()
+        f.relu, f.skip = relu, skip.data_ptr() if with_skip else None
+        res = []
+        for one_call in (False, True):
+            out, y = torch.full_like(y0, 3), torch.full((ns, Co, Ho, Ho), 3.0, device="cuda", dtype=tdt)
+            na, kn = hp.batch_norm_args(pkg, y0, out, gm, bt, eps, ns, Ci, H, H)
+            a, kp = hp.conv2d_args(pkg, out, None, w, None, y, None, Ci, H, H, Co, K, K, Ho, Ho, (p, p, p, p), (s, s), 0,
+                                   1 if s == 1 else 0)
+            st = pkg.NormStats()
+            parts[one_call].fill_(7.0)
+            st.part, st.bytes = parts[one_call].data_ptr(), parts[one_call].numel() * 4
+            if one_call:
+                rc = getattr(gpu, "ptl_conv2d_%s_fw_batched_normed" % dt)(ctypes.byref(a), ns, ctypes.byref(st), ctypes.byref(na),
+                                                                         ctypes.byref(f), ctypes.byref(st_in))
+                assert rc == 0, gpu.ptl_last_error()
+                took = gpu.ptl_last_conv_resident() == 3
+            else:
+                assert getattr(gpu, "ptl_batch_norm_fused_%s_fw_stats" % dt)(ctypes.byref(na), ctypes.byref(f), ctypes.byref(st_in)) == 0
+                assert getattr(gpu, "ptl_conv2d_%s_fw_batched_stats" % dt)(ctypes.byref(a), ns, ctypes.byref(st)) == 0
+            assert gpu.ptl_sync() == 0
+            res.append((out, y, st))
+        (out_a, y_a, st_a), (out_b, y_b, st_b) = res
+        assert expect is None or took == expect, case
+        fused += took
+        assert torch.equal(out_a, out_b), case
+        assert torch.equal(y_a, y_b), case
+        assert (st_a.valid, st_a.parts, st_a.channels, st_a.count) == (st_b.valid, st_b.parts, st_b.channels, st_b.count), case
+        assert torch.equal(parts[0], parts[1]), case
+    assert fused >= 4
+    # host tensors: the two calls, staged
+    xh = hp.uniform(5, (2, 16, 8, 8), -0.5, 0.5).astype(hp.np_dtype(dt))
+    wh = hp.uniform(6, (16, 16, 3, 3), -0.5, 0.5).astype(xh.dtype)
+    gh, bh, eh = np.ones(16, xh.dtype), np.zeros(16, xh.dtype), np.full(1, 1e-5, xh.dtype)
+    outs = []
+    for one_call in (False, True):
+        oh, yh = np.zeros_like(xh), np.zeros((2, 16, 8, 8), xh.dtype)
+        na, kn = hp.batch_norm_args(pkg, xh, oh, gh, bh, eh, 2, 16, 8, 8)
+        a, kp = hp.conv2d_args(pkg, oh, None, wh, None, yh, None, 16, 8, 8, 16, 3, 3, 8, 8, (1, 1, 1, 1), (1, 1), 0, 1)
+        none = pkg.NormFusion()
+        if one_call:
+            assert getattr(gpu, "ptl_conv2d_%s_fw_batched_normed" % dt)(ctypes.byref(a), 2, None, ctypes.byref(na), ctypes.byref(none), None) == 0
+        else:
+            assert getattr(gpu, "ptl_batch_norm_fused_%s_fw" % dt)(ctypes.byref(na), ctypes.byref(none)) == 0
+            pkg.call("ptl_conv2d_%s_fw_batched" % dt, a, 2)
+        outs.append((oh, yh))
+    assert np.array_equal(outs[0][0], outs[1][0]) and np.array_equal(outs[0][1], outs[1][1])
+    assert np.abs(outs[0][1]).max() > 0
+
+
+@pytest.mark.parametrize("dt", ["fp16", "fp32"])
 def test_conv2d_backward_forms_the_gradient_of_the_normalisation_in_front(pkg, gpu, dt):
     """ptl_conv2d_*_bw_batched_deferred_post: where the small-layer kernel takes the layer (sums.valid == 1), input->diff
     is bit for bit what the plain call's input gradient, the addition of a second gradient (rounded to the tensor type)

@@ -69,7 +69,9 @@ def test_resnet20_training_step_with_batch_norm(pkg, gpu, dt, ns, tol, fused):
     """The same step with batch normalisation after every convolution (BASELINE's ResNet-20 configuration).
     fp16: the reference sees fp16-rounded activations; what remains is the rounding of the stored gradients, which
     twenty normalised layers down are of the order of 1e-4 and keep few significant bits in fp16 (no loss scaling,
-    as in the reference) - 7 to 10 % on the deepest weight gradients."""
+    as in the reference) - 7 to 10 % on the deepest weight gradients, and around 15 % on the gain and shift gradients
+    of the stem's normalisation, the deepest sums of such values (just under or just over 15 % depending on which of
+    two equivalent orders the normalisation's forward arithmetic takes: they get 20 %)."""
     lr = 0.01
     w = rs.init_weights(0x2E5F0, dt)
     x = hp.normal(0x2E5F1, (ns, 3, 32, 32)).astype(hp.np_dtype(dt))
@@ -87,8 +89,9 @@ def test_resnet20_training_step_with_batch_norm(pkg, gpu, dt, ns, tol, fused):
     for n in ("fc", "s2b2c2", "s2b0sc", "s1b0c1", "stem"):
         assert hp.rel_l2(net.dW[n].cpu().numpy(), ref_grads[n]) <= tol, n
     for n in ("s2b2c2", "s0b0c1", "stem"):
-        assert hp.rel_l2(net.dG[n].cpu().numpy(), ref_grads["g:" + n]) <= tol, n
-        assert hp.rel_l2(net.dBt[n].cpu().numpy(), ref_grads["b:" + n]) <= tol, n
+        tol_n = 2e-1 if dt == "fp16" and n == "stem" else tol
+        assert hp.rel_l2(net.dG[n].cpu().numpy(), ref_grads["g:" + n]) <= tol_n, n
+        assert hp.rel_l2(net.dBt[n].cpu().numpy(), ref_grads["b:" + n]) <= tol_n, n
         assert hp.rel_l2(net.G[n].cpu().numpy(), ref_new["g:" + n]) <= tol, n
     for n in w:
         assert hp.rel_l2(net.W[n].cpu().numpy(), ref_new[n]) <= tol, n
@@ -167,7 +170,33 @@ def test_resnet20_step_with_gradient_sums_from_the_convolutions(pkg, gpu, dt, ns
         assert rel(given.dBt[n], own.dBt[n]) <= tol, n
 
 
-@pytest.mark.parametrize("fused", [True, False, "stats", "post"])
+@pytest.mark.parametrize("dt,ns", [("fp32", 6), ("fp16", 16)])
+def test_resnet20_step_with_the_normalisation_inside_the_forward_convolutions(pkg, gpu, dt, ns):
+    """The step whose forward convolution calls stand for the normalisation in front of them as well
+    (ptl_conv2d_*_fw_batched_normed) against the step that calls the two one after the other: 18 calls fewer, and
+    every tensor the step writes bit for bit the same."""
+    w = rs.init_weights(0x2E630, dt)
+    x = hp.normal(0x2E631, (ns, 3, 32, 32)).astype(hp.np_dtype(dt))
+    nets = []
+    for pre in (False, True):
+        net = rs.ResNetStep(pkg, gpu, torch, dt, ns, w, 0.01, norm=True, fused=True, stats=True, post=True, pre=pre)
+        net.x.copy_(torch.from_numpy(x))
+        net.target.zero_()
+        net.target[torch.arange(ns), (3 * torch.arange(ns)) % 10] = 1
+        net.step(update=True)
+        assert gpu.ptl_sync() == 0
+        nets.append(net)
+    two, one = nets
+    assert two.launches() - one.launches() == 18
+    assert torch.equal(two.logits, one.logits) and torch.equal(two.loss, one.loss)
+    for n in two.dW:
+        assert torch.equal(two.dW[n], one.dW[n]) and torch.equal(two.W[n], one.W[n]), n
+    for n in two.dG:
+        assert torch.equal(two.dG[n], one.dG[n]) and torch.equal(two.dBt[n], one.dBt[n]), n
+        assert torch.equal(two.G[n], one.G[n]) and torch.equal(two.Bt[n], one.Bt[n]), n
+
+
+@pytest.mark.parametrize("fused", [True, False, "stats", "post", "pre"])
 def test_training_step_replays_as_a_hip_graph(pkg, gpu, fused):
     """The whole step (92 or 178 library calls; "stats": the 92 with the sums of the convolutions' outputs formed by
     the convolutions) captured once into a HIP graph on a stream of the caller's and
@@ -181,7 +210,7 @@ def test_training_step_replays_as_a_hip_graph(pkg, gpu, fused):
     try:
         with torch.cuda.stream(side):
             net = rs.ResNetStep(pkg, gpu, torch, dt, ns, rs.init_weights(0x2E600, dt), 0.01, norm=True, fused=bool(fused),
-                                stats=fused in ("stats", "post"), post=fused == "post")
+                                stats=fused in ("stats", "post", "pre"), post=fused in ("post", "pre"), pre=fused == "pre")
             net.x.copy_(torch.from_numpy(hp.normal(0x2E601, (ns, 3, 32, 32)).astype(np.float16)))
             net.target.zero_()
             net.target[torch.arange(ns), (3 * torch.arange(ns)) % 10] = 1
