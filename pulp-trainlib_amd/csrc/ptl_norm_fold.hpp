@@ -9,7 +9,7 @@ namespace ptl {
 // Sums of channel `c` over its parts ([channel][part][4] floats, 16-byte aligned), by one wave: lane i adds parts
 // i, i + 64, ... in that order (four loads in flight at a time; a part that is not there adds zeros), then the lanes'
 // sums meet in a butterfly.  Every lane returns the totals.
-__device__ inline float4 norm_fold_wave(const float *__restrict__ part, int nparts, int c, int lane) {
+__device__ __forceinline__ float4 norm_fold_wave(const float *__restrict__ part, int nparts, int c, int lane) {
     const float4 *src = reinterpret_cast<const float4 *>(part) + (size_t)c * nparts;
     float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
     for (int base = 0; base < nparts; base += 256) {
@@ -40,8 +40,9 @@ __device__ inline float4 norm_fold_wave(const float *__restrict__ part, int npar
 // Mean and deviation the way the reference forms them (lib/sources/pulp_batchnorm_fp32.c:99-109: the variance as
 // the mean of (x - mean)^2 expanded, eps added under the root).
 __device__ inline void norm_mean_sd(float sum, float sum_sq, float count, float eps, float &mean, float &sd) {
+    // (the fused operations spelled out: every kernel that calls this rounds at the same places)
     mean = sum / count;
-    sd = sqrtf(((sum_sq - 2 * sum * mean) / count) + (mean * mean) + eps);
+    sd = sqrtf(fmaf(mean, mean, fmaf(-2.f * sum, mean, sum_sq) / count) + eps);
 }
 
 // One element of the forward pass, before the skip tensor, the ReLU and the rounding: the reference's
