@@ -427,7 +427,8 @@ int ptl_conv2d_fp16_bw_batched_cached(const struct Conv2D_args_fp16 *a, int nsam
  * (the addition of its partial sums) put off and done for all deferred layers at once by ptl_conv2d_*_wg_flush
  * (struct ptl_wg_batch; a training step with twenty small layers saves twenty launches).  A layer that does not take
  * the small-layer kernels, finds the batch full, or has its coeff->diff in host memory (a staging copy that the call
- * copies back) is completed by the call itself as usual.  The flush returns 0 also for an empty batch. */
+ * copies back) is completed by the call itself as usual; with skip_in_grad set the call is the weight-gradient step
+ * alone, deferred the same way.  The flush returns 0 also for an empty batch. */
 int ptl_conv2d_fp16_bw_batched_deferred(const struct Conv2D_args_fp16 *a, int nsamples, struct ptl_wg_batch *batch);
 int ptl_conv2d_fp32_bw_batched_deferred(const struct Conv2D_args *a, int nsamples, struct ptl_wg_batch *batch);
 int ptl_conv2d_fp16_wg_flush(struct ptl_wg_batch *batch);

@@ -1142,10 +1142,36 @@ int conv_small(const ConvTileDesc &d, const void *X, const void *Wt, void *Y) {
     return rc;
 }
 
+static ::ptl_wg_batch *g_wg_defer = nullptr;  // where a backward call leaves its partial sums, if anywhere
+
+void conv_small_defer_to(::ptl_wg_batch *batch) { g_wg_defer = batch; }
+
+// A deferred layer: its partial sums go to the batch's buffer (if they fit) and wait for the flush (not when dW is a
+// staging copy of a host tensor: the call copies it back when it returns).  Returns the batch, or null.
+static ::ptl_wg_batch *defer_slot(WgSmallArgs &w, bool may_defer, size_t &need) {
+    ::ptl_wg_batch *b = may_defer ? g_wg_defer : nullptr;
+    need = ((size_t)w.tiles * w.part_elems * sizeof(float) + 255) / 256 * 256;
+    const bool defer = b && b->buf && b->count >= 0 && b->count < PTL_WG_BATCH_MAX && b->used % 256 == 0 &&
+                       b->used <= b->bytes && need <= b->bytes - b->used && reinterpret_cast<uintptr_t>(b->buf) % 256 == 0;
+    if (!defer) return nullptr;
+    w.ws = reinterpret_cast<float *>(static_cast<char *>(b->buf) + b->used);
+    return b;
+}
+static void defer_record(::ptl_wg_batch *b, const WgSmallArgs &w, void *dW, size_t need) {
+    const int at = b->count++;
+    b->offset[at] = b->used;
+    b->grad[at] = dW;
+    const int shape[8] = {w.part_elems, w.tiles, w.rows_kept, w.cols_kept, w.cbi_n, w.Cout, w.Cin, w.taps};
+    for (int i = 0; i < 8; ++i) b->shape[8 * at + i] = shape[i];
+    b->used += need;
+}
+
 template <typename T>
-int conv_small_wg(const ConvTileDesc &d, const void *X, const void *dY, void *dW) {
+int conv_small_wg(const ConvTileDesc &d, const void *X, const void *dY, void *dW, bool may_defer) {
     WgSmallArgs w;
     if (int rc = plan_wg<T>(d, X, dY, state().num_cu, true, w)) return rc;
+    size_t need;
+    ::ptl_wg_batch *b = defer_slot(w, may_defer, need);
     static bool attr_set = false;
     if (!attr_set) {
         if (!hip_ok(hipFuncSetAttribute(reinterpret_cast<const void *>(wg_small_kernel<T>),
@@ -1157,12 +1183,11 @@ int conv_small_wg(const ConvTileDesc &d, const void *X, const void *dY, void *dW
     state().last_conv_resident = 2;
     hipLaunchKernelGGL(wg_small_kernel<T>, dim3(w.nwg), dim3(CS_NT), WG_SMALL_LDS, state().stream, w);
     if (!hip_ok(hipGetLastError(), "small weight gradient launch")) return 2;
-    return reduce_wg<T>(w, dW);
+    if (!b) return reduce_wg<T>(w, dW);
+    defer_record(b, w, dW, need);
+    return 0;
 }
 
-static ::ptl_wg_batch *g_wg_defer = nullptr;  // where the one-call backward leaves its partial sums, if anywhere
-
-void conv_small_defer_to(::ptl_wg_batch *batch) { g_wg_defer = batch; }
 
 // What the input gradient of the one-call backward does in its epilogue, and where its sums go, if anything
 static const ::ptl_grad_post *g_grad_post = nullptr;
@@ -1181,13 +1206,8 @@ int conv_small_bw(const ConvTileDesc &fwd, const ConvTileDesc &ig, const void *X
     SmallPlan p;
     const int budget = state().num_cu - w.nwg;
     if (int rc = plan_small<T>(ig, dY, Wt, dX, budget > 32 ? budget : 32, p)) return rc;
-    // a deferred layer: its partial sums go to the batch's buffer (if they fit) and wait for the flush
-    // (not when dW is a staging copy of a host tensor: the call copies it back when it returns)
-    ::ptl_wg_batch *b = may_defer ? g_wg_defer : nullptr;
-    const size_t need = ((size_t)w.tiles * w.part_elems * sizeof(float) + 255) / 256 * 256;
-    const bool defer = b && b->buf && b->count >= 0 && b->count < PTL_WG_BATCH_MAX && b->used % 256 == 0 &&
-                       b->used <= b->bytes && need <= b->bytes - b->used && reinterpret_cast<uintptr_t>(b->buf) % 256 == 0;
-    if (defer) w.ws = reinterpret_cast<float *>(static_cast<char *>(b->buf) + b->used);
+    size_t need;
+    ::ptl_wg_batch *b = defer_slot(w, may_defer, need);
     if (g_grad_post && g_grad_sums && may_defer && g_grad_post->x) {
         // the gradient epilogue: the jobs' sums in LDS behind the tile, a partial per workgroup and channel in the caller's
         // buffer - like the forward sums; a layer whose jobs or partials do not fit goes without (sums->valid stays 0)
@@ -1218,13 +1238,8 @@ int conv_small_bw(const ConvTileDesc &fwd, const ConvTileDesc &ig, const void *X
         if (g_grad_sums) g_grad_sums->valid = 0;
         return rc;
     }
-    if (!defer) return reduce_wg<T>(w, dW);
-    const int at = b->count++;
-    b->offset[at] = b->used;
-    b->grad[at] = dW;
-    const int shape[8] = {w.part_elems, w.tiles, w.rows_kept, w.cols_kept, w.cbi_n, w.Cout, w.Cin, w.taps};
-    for (int i = 0; i < 8; ++i) b->shape[8 * at + i] = shape[i];
-    b->used += need;
+    if (!b) return reduce_wg<T>(w, dW);
+    defer_record(b, w, dW, need);
     return 0;
 }
 
@@ -1268,8 +1283,8 @@ template int conv_small_flush<float>(::ptl_wg_batch *);
 
 template int conv_small<half_t>(const ConvTileDesc &, const void *, const void *, void *);
 template int conv_small<float>(const ConvTileDesc &, const void *, const void *, void *);
-template int conv_small_wg<half_t>(const ConvTileDesc &, const void *, const void *, void *);
-template int conv_small_wg<float>(const ConvTileDesc &, const void *, const void *, void *);
+template int conv_small_wg<half_t>(const ConvTileDesc &, const void *, const void *, void *, bool);
+template int conv_small_wg<float>(const ConvTileDesc &, const void *, const void *, void *, bool);
 template int conv_small_bw<half_t>(const ConvTileDesc &, const ConvTileDesc &, const void *, const void *, const void *,
                                    void *, void *, bool);
 template int conv_small_bw<float>(const ConvTileDesc &, const ConvTileDesc &, const void *, const void *, const void *,

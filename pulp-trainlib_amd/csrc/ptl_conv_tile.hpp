@@ -42,8 +42,9 @@ template <typename T>
 int conv_small(const ConvTileDesc &d, const void *X, const void *Wt, void *Y);
 // Weight gradient of such a layer (unit stride, output as wide as the input), and weight + input gradient with the
 // two products in one launch (`fwd` describes the forward layer, `ig` the input gradient as a forward pass over dY).
+// (`may_defer`: dW is the caller's own device tensor, so its sums may wait in a batch given with conv_small_defer_to)
 template <typename T>
-int conv_small_wg(const ConvTileDesc &d, const void *X, const void *dY, void *dW);
+int conv_small_wg(const ConvTileDesc &d, const void *X, const void *dY, void *dW, bool may_defer);
 template <typename T>
 int conv_small_bw(const ConvTileDesc &fwd, const ConvTileDesc &ig, const void *X, const void *dY, const void *Wt,
                   void *dW, void *dX, bool may_defer);

@@ -340,7 +340,7 @@ static int sgd_step(const Args *a, const char *fn) {
 
 // The same update for a list of parameter tensors in one launch: a training step updates dozens of small
 // tensors, and one launch each is two microseconds each.
-constexpr int SGD_MAXT = 48;
+constexpr int SGD_MAXT = 96;  // (3 KB of kernel arguments: the parameter tensors of a ResNet-20 with its normalisation layers are 64)
 struct SgdTable {
     void *w[SGD_MAXT], *g[SGD_MAXT];
     unsigned n[SGD_MAXT], first[SGD_MAXT + 1];  // elements; first workgroup of tensor t (first[count] = grid)

@@ -364,7 +364,8 @@ static int conv2d_wg(const Args *a, int ns, const char *fn) {
                                 (long long)ns * g.Ho * g.Wo >= 16384;
         if (g.hwc) {  // channel-minor tensors: the sum over taps from 64 channels on, else the gathering GEMM below
             rc = conv_taps_wg<T>(d, X, dY, dW);
-        } else if ((rc = conv_small_wg<T>(d, X, dY, dW)) >= 0) {
+        } else if ((rc = conv_small_wg<T>(d, X, dY, dW,
+                                           static_cast<const void *>(dW) == static_cast<const void *>(a->coeff->diff))) >= 0) {
             // (small 3x3 layers: one launch for the partial sums over sample ranges, one to add them)
         } else {
             const bool tiles_resident = sizeof(T) == 2 && state().gemm_path == 0 && conv_halo_wg_preferred(d);

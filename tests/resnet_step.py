@@ -215,7 +215,9 @@ class ResNetStep:
             self.keep.append(kp)
             # weight and input gradient in one call (the stem needs no input gradient); the additions that complete
             # the weight gradients of the small layers wait for one flush behind the backward pass
-            bw = [(L("ptl_conv2d_DT_bw_batched_deferred"), a, (ns, self.wg_batch))] if dx is not None else [(L("ptl_conv2d_DT_wg_batched"), a, (ns,))]
+            # (no input gradient: the backward call with skip_in_grad set is the weight-gradient step alone)
+            a.skip_in_grad = 0 if dx is not None else 1
+            bw = [(L("ptl_conv2d_DT_bw_batched_deferred"), a, (ns, self.wg_batch))]
             if post is not None:
                 bw = [(L("ptl_conv2d_DT_bw_batched_deferred_post"), a, (ns, self.wg_batch, post[0], post[1]))]
             if not self.use_stats:

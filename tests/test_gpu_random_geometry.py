@@ -312,6 +312,38 @@ def test_conv2d_deferred_weight_gradient_sums(pkg, gpu, dt):
 
 
 @pytest.mark.parametrize("dt", ["fp16", "fp32"])
+def test_conv2d_deferred_weight_gradient_alone(pkg, gpu, dt):
+    """A first layer has no input gradient: with skip_in_grad set the deferred backward call is the weight-gradient
+    step alone, its sums wait for the flush like the others', and the result has the bits of ptl_conv2d_*_wg_batched."""
+    tdt = torch.float16 if dt == "fp16" else torch.float32
+    buf = torch.empty(8 << 20, dtype=torch.uint8, device="cuda")
+    for (Ci, Co, H, ns) in ((3, 16, 32, 128), (16, 32, 16, 40)):
+        x = (torch.rand(ns, Ci, H, H, device="cuda") - 0.5).to(tdt)
+        w = (torch.rand(Co, Ci, 3, 3, device="cuda") - 0.5).to(tdt)
+        dy = (torch.rand(ns, Co, H, H, device="cuda") - 0.5).to(tdt)
+        y = torch.zeros_like(dy)
+        outs = []
+        for deferred in (False, True):
+            dx, dw = torch.full_like(x, 3), torch.full_like(w, 3)
+            a, kp = hp.conv2d_args(pkg, x, dx, w, dw, y, dy, Ci, H, H, Co, 3, 3, H, H, (1, 1, 1, 1), (1, 1), 0, 1)
+            a.skip_in_grad = 1
+            if deferred:
+                batch = pkg.WgBatch()
+                batch.buf, batch.bytes = buf.data_ptr(), buf.numel()
+                assert getattr(gpu, "ptl_conv2d_%s_bw_batched_deferred" % dt)(ctypes.byref(a), ns, ctypes.byref(batch)) == 0
+                assert batch.count == 1
+                assert getattr(gpu, "ptl_conv2d_%s_wg_flush" % dt)(ctypes.byref(batch)) == 0
+            else:
+                pkg.call("ptl_conv2d_%s_wg_batched" % dt, a, ns)
+            assert gpu.ptl_sync() == 0
+            assert bool((dx == 3).all())
+            outs.append(dw)
+        assert torch.equal(outs[0], outs[1]), (Ci, Co, H, ns)
+        ref = torch.nn.grad.conv2d_weight(x.double(), w.shape, dy.double(), padding=1)
+        assert rel(outs[1].double(), ref) <= (2e-3 if dt == "fp16" else 1e-5)
+
+
+@pytest.mark.parametrize("dt", ["fp16", "fp32"])
 def test_conv2d_forward_sums_feed_the_normalisation(pkg, gpu, dt):
     """ptl_conv2d_*_fw_batched_stats: the same output bits as the plain forward call, and per channel the sum of the
     output and of its squares (over the struct's parts, against the stored tensor summed in float64: the kernel sums
