@@ -792,27 +792,31 @@ int launch_small(const ConvSmallArgs &a, int tiles, size_t lds, hipStream_t s, c
 // dW(co, ci, tap) = sum over workgroups of ws[workgroup][block][tap][filter row][channel]: 64 consecutive partial
 // elements per workgroup of the reduction (coalesced reads), 16 groups of partials in parallel, eight loads in flight
 // per thread; the few results are scattered to the weight tensor's order.
-template <typename T>
-__device__ inline void wg_small_reduce_block(const float *__restrict__ ws, T *__restrict__ dW, int block, int part_elems,
-                                             int parts, int rows_kept, int cols_kept, int cbi_n, int Cout, int Cin,
-                                             int taps) {
-    __shared__ float part_sum[16][64];
-    const int o = threadIdx.x & 63, pg = threadIdx.x >> 6;
-    const int i = block * 64 + o;
+// PG groups of partials in parallel on 1024 / PG consecutive elements: 16 x 64 where a layer has many workgroups, 4 x 256
+// where it has few (a 64-channel layer has 32 of them and 36 864 elements: with 64 elements a block, 576 blocks of
+// two loads a thread).
+template <typename T, int PG>
+__device__ inline void wg_small_reduce_part(const float *__restrict__ ws, T *__restrict__ dW, int block, int part_elems,
+                                            int parts, int rows_kept, int cols_kept, int cbi_n, int Cout, int Cin,
+                                            int taps) {
+    constexpr int EPB = 1024 / PG;
+    __shared__ float part_sum[PG][EPB];
+    const int o = threadIdx.x % EPB, pg = threadIdx.x / EPB;
+    const int i = block * EPB + o;
     float s = 0.f;
     if (i < part_elems) {
         const float *src = ws + i;
         int p = pg;
-        for (; p + 7 * 16 < parts; p += 8 * 16) {
+        for (; p + 7 * PG < parts; p += 8 * PG) {
             float v[8];
 #pragma unroll
-            for (int u = 0; u < 8; ++u) v[u] = src[(size_t)(p + u * 16) * part_elems];
+            for (int u = 0; u < 8; ++u) v[u] = src[(size_t)(p + u * PG) * part_elems];
 #pragma unroll
             for (int u = 0; u < 8; ++u) s += v[u];
         }
         float v[8];
 #pragma unroll
-        for (int u = 0; u < 8; ++u) v[u] = p + u * 16 < parts ? src[(size_t)(p + u * 16) * part_elems] : 0.f;
+        for (int u = 0; u < 8; ++u) v[u] = p + u * PG < parts ? src[(size_t)(p + u * PG) * part_elems] : 0.f;
 #pragma unroll
         for (int u = 0; u < 8; ++u) s += v[u];
     }
@@ -820,12 +824,25 @@ __device__ inline void wg_small_reduce_block(const float *__restrict__ ws, T *__
     __syncthreads();
     if (pg == 0 && i < part_elems) {
 #pragma unroll
-        for (int q = 1; q < 16; ++q) s += part_sum[q][o];
+        for (int q = 1; q < PG; ++q) s += part_sum[q][o];
         const int tile = i / (rows_kept * cols_kept), r = i - tile * rows_kept * cols_kept;
         const int combo = tile / taps, tap = tile - combo * taps;
         const int co = (combo / cbi_n) * 32 + r / cols_kept, ci = (combo % cbi_n) * 32 + r % cols_kept;
         if (co < Cout && ci < Cin) dW[(co * Cin + ci) * taps + tap] = (T)s;
     }
+}
+
+// (the shape of a layer decides its form, so that a deferred layer's sums have the bits of the immediate call's)
+__host__ __device__ inline int wg_reduce_epb(int parts) { return parts <= 64 ? 256 : 64; }
+
+template <typename T>
+__device__ inline void wg_small_reduce_block(const float *__restrict__ ws, T *__restrict__ dW, int block, int part_elems,
+                                             int parts, int rows_kept, int cols_kept, int cbi_n, int Cout, int Cin,
+                                             int taps) {
+    if (wg_reduce_epb(parts) == 256)
+        wg_small_reduce_part<T, 4>(ws, dW, block, part_elems, parts, rows_kept, cols_kept, cbi_n, Cout, Cin, taps);
+    else
+        wg_small_reduce_part<T, 16>(ws, dW, block, part_elems, parts, rows_kept, cols_kept, cbi_n, Cout, Cin, taps);
 }
 
 template <typename T>
@@ -1070,7 +1087,8 @@ int plan_wg(const ConvTileDesc &d, const void *X, const void *dY, int max_wg, bo
 
 template <typename T>
 int reduce_wg(const WgSmallArgs &w, void *dW) {
-    hipLaunchKernelGGL(wg_small_reduce_kernel<T>, dim3((w.part_elems + 63) / 64), dim3(1024), 0, state().stream, w.ws,
+    hipLaunchKernelGGL(wg_small_reduce_kernel<T>, dim3((w.part_elems + wg_reduce_epb(w.tiles) - 1) / wg_reduce_epb(w.tiles)), dim3(1024), 0,
+                       state().stream, w.ws,
                        reinterpret_cast<T *>(dW), w.part_elems, w.tiles, w.rows_kept, w.cols_kept, w.cbi_n, w.Cout, w.Cin, w.taps);
     return hip_ok(hipGetLastError(), "small weight gradient reduction launch") ? 0 : 2;
 }
@@ -1266,7 +1284,7 @@ int conv_small_flush(::ptl_wg_batch *b) {
             return 1;
         }
         a.first_block[i] = blocks;
-        blocks += (shape[0] + 63) / 64;
+        blocks += (shape[0] + wg_reduce_epb(shape[1]) - 1) / wg_reduce_epb(shape[1]);
         a.ws[i] = reinterpret_cast<const float *>(static_cast<const char *>(b->buf) + b->offset[i]);
         a.grad[i] = b->grad[i];
         for (int k = 0; k < 8; ++k) a.shape[i][k] = shape[k];
