@@ -115,6 +115,11 @@ __device__ inline void conv_small_block(const ConvSmallArgs &a, int tile, char *
     const int b = tile / a.tiles_per_img, y0 = (tile - b * a.tiles_per_img) * a.R;
     const int iy0 = y0 * a.s - a.padU;
 
+    // ---- the partial sums of a normalisation in front: asked for before anything else, added up behind the tile's loads
+    constexpr int FOLD_R = CINP / 16;
+    NormFoldRegs<FOLD_R> fold;
+    if (a.pre) norm_fold_ask<FOLD_R>(fold, a.pre_part, a.pre_parts, 0, a.Cin, wave, lane);
+
     // ---- all global loads first
     Piece<T> xin[CS_IN_MAX];
     const int lrow = lane / VEC, lch = lane % VEC;
@@ -140,13 +145,16 @@ __device__ inline void conv_small_block(const ConvSmallArgs &a, int tile, char *
         const int q = tid + CS_NT * k;
         if (q < a.f_chunks) fin[k].v = reinterpret_cast<const uint4 *>(a.Wt)[q];
     }
-    if (a.pre) {  // the statistics of the normalisation in front: a wave per channel
+    if (a.pre) {  // the statistics of the normalisation in front: a wave per channel and round
         float4 *tab = reinterpret_cast<float4 *>(smem + a.pre_off);
-        for (int c = wave; c < a.Cin; c += CS_WAVES) {
-            const float4 v = norm_fold_wave(a.pre_part, a.pre_parts, c, lane);
-            if (lane == 0) {
+        float2 sums[FOLD_R];
+        norm_fold_take<FOLD_R>(fold, sums);
+#pragma unroll
+        for (int r = 0; r < FOLD_R; ++r) {
+            const int c = wave + 16 * r;
+            if (lane == 0 && c < a.Cin) {
                 float mean, sd;
-                norm_mean_sd(v.x, v.y, a.pre_count, (float)reinterpret_cast<const T *>(a.pre_eps)[0], mean, sd);
+                norm_mean_sd(sums[r].x, sums[r].y, a.pre_count, (float)reinterpret_cast<const T *>(a.pre_eps)[0], mean, sd);
                 tab[c] = make_float4(mean, (float)reinterpret_cast<const T *>(a.pre_w)[c] / sd,
                                      (float)reinterpret_cast<const T *>(a.pre_b)[c], 0.f);
             }
@@ -1121,7 +1129,8 @@ int conv_small(const ConvTileDesc &d, const void *X, const void *Wt, void *Y) {
         const bool ok = X == pre->out && pre->x && pre->weight && pre->bias && pre->eps && pre->part && pre->parts > 0 &&
                         aligned(pre->x) && aligned(pre->out) && aligned(pre->skip) && aligned(pre->part) &&
                         p.a.dil == 1 && d.padU <= d.KH - d.sh && (long long)d.Ho * d.sh >= d.Hin &&
-                        pre->count == (size_t)d.batch * d.Hin * d.Win && off + need <= 150 * 1024;
+                        pre->count == (size_t)d.batch * d.Hin * d.Win && off + need <= 150 * 1024 &&
+                        pre->parts <= NORM_FOLD_MAX_PARTS;
         if (!ok) return CONV_PRE_REFUSED;
         p.a.X = pre->x;
         p.a.pre = 1;

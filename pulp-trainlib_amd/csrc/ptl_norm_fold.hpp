@@ -37,6 +37,49 @@ __device__ __forceinline__ float4 norm_fold_wave(const float *__restrict__ part,
     return v;
 }
 
+// The same sums (places 0 and 1 of a part) in two steps, for a kernel that wants the loads in the air before it issues
+// the loads of its tile and the sums only behind them: channels c0 + wave + 16 r (r < R) of a 16-wave workgroup, at
+// most 256 parts (four per lane).  Bit for bit norm_fold_wave's sums.
+constexpr int NORM_FOLD_MAX_PARTS = 256;
+template <int R>
+struct NormFoldRegs {
+    float2 v[R][4];
+};
+template <int R>
+__device__ __forceinline__ void norm_fold_ask(NormFoldRegs<R> &f, const float *__restrict__ part, int nparts, int c0,
+                                              int nch, int wave, int lane) {
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+        const int c = wave + 16 * r;
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+            const int i = 64 * u + lane;
+            f.v[r][u] = make_float2(0.f, 0.f);
+            if (c < nch && i < nparts) f.v[r][u] = *reinterpret_cast<const float2 *>(part + ((size_t)(c0 + c) * nparts + i) * 4);
+        }
+    }
+}
+template <int R>
+__device__ __forceinline__ void norm_fold_take(const NormFoldRegs<R> &f, float2 (&t)[R]) {
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+        t[r] = make_float2(0.f, 0.f);
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+            t[r].x += f.v[r][u].x;
+            t[r].y += f.v[r][u].y;
+        }
+    }
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) {
+#pragma unroll
+        for (int r = 0; r < R; ++r) {
+            t[r].x += __shfl_xor(t[r].x, off);
+            t[r].y += __shfl_xor(t[r].y, off);
+        }
+    }
+}
+
 // Mean and deviation the way the reference forms them (lib/sources/pulp_batchnorm_fp32.c:99-109: the variance as
 // the mean of (x - mean)^2 expanded, eps added under the root).
 __device__ inline void norm_mean_sd(float sum, float sum_sq, float count, float eps, float &mean, float &sd) {
