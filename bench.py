@@ -277,7 +277,7 @@ TARGET_ROWS = (
     ("mhsa_L197_E192_N32_FW_BW_us", ["mhsa L197 E192 3x64 %s N=32" % s for s in ("FW", "BW")], "us"),
     ("resnet20_fp16_N128_step_samples/s",
      ["resnet20 step with batch norm, element-wise layers fused into it, its sums formed by the convolutions in both passes, "
-      "applied inside the forward convolutions"],
+      "applied inside the forward convolutions, pooling + classifier + loss in one call"],
      "samples/s"),
     ("mm_4096_fp16_random_then_zero_operands_TFLOP/s",
      ["power: mm 4096x4096x4096 (B transposed), random", "power: mm 4096x4096x4096 (B transposed), zero"], "TFLOP/s"),
@@ -512,11 +512,12 @@ def resnet_rows(pkg, lib, timed, torch, dev):
         macs += (ci * co * 9 + co * co * 9 + (ci * co if proj else 0)) * Ho * Ho
         H = Ho
     flops = 3 * 2.0 * ns * (macs + 64 * ncls)
-    for norm, fused, stats, post, pre in ((True, True, False, False, False), (True, True, True, False, False),
-                                          (True, True, True, True, False), (True, True, True, True, True),
-                                          (True, False, False, False, False), (False, False, False, False, False)):
+    for norm, fused, stats, post, pre, head in ((True, True, False, False, False, False), (True, True, True, False, False, False),
+                                                (True, True, True, True, False, False), (True, True, True, True, True, False),
+                                                (True, True, True, True, True, True),
+                                                (True, False, False, False, False, False), (False, False, False, False, False, False)):
         net = rs.ResNetStep(pkg, lib, torch, dt, ns, rs.init_weights(0x2E5E0, dt), 0.01, norm=norm, fused=fused, stats=stats,
-                            post=post, pre=pre)
+                            post=post, pre=pre, head=head)
         net.x.copy_(torch.randn(ns, 3, 32, 32, device=dev).to(tdt[dt]))
         net.target.zero_()
         net.target[torch.arange(ns), torch.randint(0, 10, (ns,))] = 1
@@ -525,13 +526,14 @@ def resnet_rows(pkg, lib, timed, torch, dev):
                                  % ((" with batch norm" + (", element-wise layers fused into it" if fused else "") +
                                      (", its sums formed by the convolutions" if stats else "") +
                                      (" in both passes" if post else "") +
-                                     (", applied inside the forward convolutions" if pre else "")) if norm
+                                     (", applied inside the forward convolutions" if pre else "") +
+                                     (", pooling + classifier + loss in one call" if head else "")) if norm
                                     else " (no norm)", ns, net.launches()),
                      "dtype": dt, "us": round(ms * 1e3, 1), "TFLOP/s": round(flops / (ms * 1e-3) / 1e12, 3),
                      "samples/s": round(ns / (ms * 1e-3), 1)})
-        if pre:
+        if head:
             # the same step captured once into a HIP graph on a side stream and replayed (one submission per step
-            # instead of 74 calls)
+            # instead of 69 calls)
             import ctypes
             side = torch.cuda.Stream()
             lib.ptl_set_stream(ctypes.c_void_p(side.cuda_stream))

@@ -465,6 +465,18 @@ int ptl_batch_norm_fused_fp32_fw_stats(const struct BatchNorm_args_fp32 *a, cons
                                        const struct ptl_norm_stats *st);
 int ptl_batch_norm_fused_fp16_fw_stats(const struct BatchNorm_args_fp16 *a, const struct ptl_norm_fusion_fp16 *f,
                                        const struct ptl_norm_stats *st);
+/* No counterpart in the reference: the tail of a classifier and its way back in one call - ptl_avgpool_*_batched(pool,
+ * n, 0), ptl_linear_*_fw_batched(lin, n), ptl_cross_entropy_*_batched(loss, n, 0) and (loss, n, 1),
+ * ptl_linear_*_bw_batched(lin, n), ptl_avgpool_*_batched(pool, n, 1), every tensor those calls write included.  One
+ * launch when the pooling is global (window = plane), its output blob is the classifier's input and the
+ * classifier's output blob the loss's (same data and diff pointers), at most 32 classes, no bias, both gradients
+ * wanted, device tensors, and `batch` (a struct ptl_wg_batch, see ptl_conv2d_*_bw_batched_deferred) has room: the
+ * classifier's weight gradient is then complete after the flush, like a deferred convolution's.  Results agree with
+ * the six calls to rounding (the dot products are added up in another order).  Anything else: the six calls. */
+int ptl_pool_linear_loss_fp32_batched(const struct pool_args *pool, const struct Linear_args *lin, const struct loss_args *loss,
+                                      int nsamples, struct ptl_wg_batch *batch);
+int ptl_pool_linear_loss_fp16_batched(const struct pool_args_fp16 *pool, const struct Linear_args_fp16 *lin,
+                                      const struct loss_args_fp16 *loss, int nsamples, struct ptl_wg_batch *batch);
 /* No counterpart in the reference: ptl_batch_norm_fused_*_fw_stats(norm, f, norm_st) followed by
  * ptl_conv2d_*_fw_batched_stats(a, nsamples, st) (st may be NULL: no sums wanted) for a convolution that reads the
  * normalisation's output (norm->output->data == a->input->data) - same results bit for bit, the normalisation's

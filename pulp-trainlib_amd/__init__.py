@@ -110,6 +110,9 @@ GRAD_STATS_ENTRY_POINTS = ["ptl_conv2d_%s_bw_batched_deferred_post" % dt for dt 
 #         const ptl_norm_stats *)`
 NORMED_ENTRY_POINTS = ["ptl_conv2d_%s_fw_batched_normed" % dt for dt in ("fp16", "fp32")]
 
+# `int f(const pool_args *, const Linear_args *, const loss_args *, int nsamples, ptl_wg_batch *)`
+HEAD_ENTRY_POINTS = ["ptl_pool_linear_loss_%s_batched" % dt for dt in ("fp16", "fp32")]
+
 OTHER_ENTRY_POINTS = ["ptl_init", "ptl_last_error", "ptl_last_status", "ptl_set_stream", "ptl_sync", "ptl_set_gemm_path",
                       "ptl_last_conv_direct", "ptl_last_gemm_streamed", "ptl_last_conv_resident", "ptl_last_gemm_tile", "ptl_timer_begin", "ptl_timer_end_ms", "ptl_mm_fp32", "ptl_mm_fp16", "ptl_copy_bytes",
                       "ptl_reserve", "ptl_reserved", "ptl_probe_mfma_fp16"]
@@ -175,6 +178,10 @@ def load():
     for name in NORMED_ENTRY_POINTS:
         f = getattr(lib, name)
         f.argtypes = [ctypes.c_void_p, ctypes.c_int, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p]
+        f.restype = ctypes.c_int
+    for name in HEAD_ENTRY_POINTS:
+        f = getattr(lib, name)
+        f.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int, ctypes.c_void_p]
         f.restype = ctypes.c_int
     lib.ptl_conv2d_fp16_cache_bytes.argtypes = [ctypes.c_void_p, ctypes.c_int]
     lib.ptl_conv2d_fp16_cache_bytes.restype = ctypes.c_size_t

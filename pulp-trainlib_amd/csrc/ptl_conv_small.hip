@@ -1193,6 +1193,28 @@ static void defer_record(::ptl_wg_batch *b, const WgSmallArgs &w, void *dW, size
     b->used += need;
 }
 
+float *wg_batch_reserve(::ptl_wg_batch *b, void *dW, int parts, int filters, int channels, int taps) {
+    if (!b || !dW || parts <= 0 || filters <= 0 || filters > 32 || channels <= 0 || taps <= 0) return nullptr;
+    // (one block of filters, the channels in blocks of 32: what the flush's index arithmetic covers)
+    WgSmallArgs w = WgSmallArgs();
+    w.cbi_n = (channels + 31) / 32;
+    w.rows_kept = filters;
+    w.cols_kept = channels < 32 ? channels : 32;
+    w.part_elems = w.cbi_n * taps * w.rows_kept * w.cols_kept;
+    w.tiles = parts;
+    w.Cout = filters;
+    w.Cin = channels;
+    w.taps = taps;
+    ::ptl_wg_batch *saved = g_wg_defer;
+    g_wg_defer = b;
+    size_t need;
+    ::ptl_wg_batch *slot = defer_slot(w, true, need);
+    g_wg_defer = saved;
+    if (!slot) return nullptr;
+    defer_record(slot, w, dW, need);
+    return w.ws;
+}
+
 template <typename T>
 int conv_small_wg(const ConvTileDesc &d, const void *X, const void *dY, void *dW, bool may_defer) {
     WgSmallArgs w;

@@ -178,6 +178,10 @@ struct ConvPreNorm {
 constexpr int CONV_PRE_REFUSED = -3;
 void conv_small_pre_to(const ConvPreNorm *pre);
 bool conv_small_pre_pending();
+// Room in a batch of deferred weight-gradient sums for another layer's partial sums (`parts` of them, `part_elems`
+// floats each, in the order the flush reads: [part][32-channel block][tap][filter row][channel of the block]) that
+// the flush will add up into dW[filter][channel][tap]; nullptr when the batch cannot take it.
+float *wg_batch_reserve(struct ::ptl_wg_batch *b, void *dW, int parts, int filters, int channels, int taps);
 // What the input gradient of the next one-call backward does in its epilogue (struct ptl_grad_post) and where the sums
 // of the gradient it forms go; sums->valid tells whether it did.  Cleared with (nullptr, nullptr).
 void conv_small_post_to(const struct ::ptl_grad_post *post, struct ::ptl_norm_stats *sums);

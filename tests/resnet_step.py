@@ -44,7 +44,7 @@ def init_weights(seed, dt):
 class ResNetStep:
     """Device buffers, argument structs and the call sequence of one training step on `ns` samples."""
 
-    def __init__(self, pkg, lib, torch, dt, ns, weights, lr=0.01, norm=False, fused=False, stats=False, post=False, pre=False):
+    def __init__(self, pkg, lib, torch, dt, ns, weights, lr=0.01, norm=False, fused=False, stats=False, post=False, pre=False, head=False):
         """`fused` (with `norm`): ReLU, the residual sum and the sum of a tensor's two incoming gradients run inside
         the normalisation calls (ptl_batch_norm_fused_*) instead of as element-wise calls of their own and the backward
         calls defer the additions of their weight gradients to one flush; with `stats` the forward convolutions also
@@ -53,11 +53,12 @@ class ResNetStep:
         normalisation in front of them starts from, and its sums (ptl_conv2d_*_bw_batched_deferred_post,
         ptl_batch_norm_fused_*_bw_stats): that normalisation's backward pass is one launch as well; with `pre` (and `stats`) the
         forward call of a convolution also stands for the forward call of the normalisation in front of it
-        (ptl_conv2d_*_fw_batched_normed)."""
+        (ptl_conv2d_*_fw_batched_normed); with `head` pooling, classifier and loss run forward and backward in one
+        call (ptl_pool_linear_loss_*_batched), the classifier's weight gradient deferred like the convolutions'."""
         self.pkg, self.lib, self.dt, self.ns, self.lr = pkg, lib, dt, ns, lr
         if fused:
             assert norm and (stats or not (post or pre))
-            self.use_stats, self.use_post, self.use_pre = stats, post, pre
+            self.use_stats, self.use_post, self.use_pre, self.use_head = stats, post, pre, head
             return self._build_fused(torch, weights)
         assert not stats
         tdt = torch.float16 if dt == "fp16" else torch.float32
@@ -331,10 +332,14 @@ class ResNetStep:
         self.target, self.loss = z(ns, ncls), z(ns)
         ca, kp = hp.loss_args(pkg, self.logits, dlogits, self.target, self.loss, ncls)
         self.keep.append(kp)
-        self.fw += [(L("ptl_avgpool_DT_batched"), pa, (ns, 0)), (L("ptl_linear_DT_fw_batched"), la, (ns,)),
-                    (L("ptl_cross_entropy_DT_batched"), ca, (ns, 0))]
-        self.bw = [(L("ptl_cross_entropy_DT_batched"), ca, (ns, 1)), (L("ptl_linear_DT_bw_batched"), la, (ns,)),
-                   (L("ptl_avgpool_DT_batched"), pa, (ns, 1))]
+        if getattr(self, "use_head", False):
+            self.fw += [(L("ptl_pool_linear_loss_DT_batched"), pa, (la, ca, ns, self.wg_batch))]
+            self.bw = []
+        else:
+            self.fw += [(L("ptl_avgpool_DT_batched"), pa, (ns, 0)), (L("ptl_linear_DT_fw_batched"), la, (ns,)),
+                        (L("ptl_cross_entropy_DT_batched"), ca, (ns, 0))]
+            self.bw = [(L("ptl_cross_entropy_DT_batched"), ca, (ns, 1)), (L("ptl_linear_DT_bw_batched"), la, (ns,)),
+                       (L("ptl_avgpool_DT_batched"), pa, (ns, 1))]
         for b in reversed(bw_blocks):
             self.bw += b
         self.bw += first_bw

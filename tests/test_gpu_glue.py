@@ -356,3 +356,63 @@ def test_gradient_descent_for_a_list_of_tensors(pkg, gpu, dt):
     for one, many in zip(*res):
         for u, v in zip(one, many):
             assert (u is None and v is None) or np.array_equal(u, v)
+
+
+@pytest.mark.parametrize("dt", ["fp16", "fp32"])
+def test_pool_linear_loss_in_one_call(pkg, gpu, dt):
+    """ptl_pool_linear_loss_*_batched against the six calls it stands for (pooling, classifier and cross-entropy forward,
+    then their backward passes): the pooled vector bit for bit (same order of additions), everything behind the
+    classifier's dot products to rounding - logits, loss, the gradients of logits, pooled vector and input, and the
+    classifier's weight gradient after the flush of the batch it was deferred to.  Cases the one launch does not take
+    (a bias, a pooling window smaller than the plane, no batch) run the six calls and give their bits."""
+    import torch
+    tdt = torch.float16 if dt == "fp16" else torch.float32
+    tol = 2e-3 if dt == "fp16" else 1e-5
+    buf = torch.empty(4 << 20, dtype=torch.uint8, device="cuda")
+    #        ns, C, H, classes, bias, window, batch given, one launch expected
+    cases = [(128, 64, 8, 10, 0, 8, 1, True), (7, 40, 5, 3, 0, 5, 1, True), (33, 96, 4, 32, 0, 4, 1, True),
+             (16, 64, 8, 10, 1, 8, 1, False), (16, 64, 8, 10, 0, 4, 1, False), (16, 64, 8, 10, 0, 8, 0, False)]
+    for case in cases:
+        ns, C, H, ncls, bias, win, with_batch, expect = case
+        Ho = H // win
+        g = torch.Generator(device="cuda").manual_seed(ns * 1000 + C)
+        x = (torch.rand(ns, C, H, H, device="cuda", generator=g) - 0.3).to(tdt)
+        w = ((torch.rand(ncls, C * Ho * Ho, device="cuda", generator=g) - 0.5) * 0.5).to(tdt)
+        b = (torch.rand(ncls, device="cuda", generator=g) - 0.5).to(tdt)
+        target = torch.zeros(ns, ncls, device="cuda", dtype=tdt)
+        target[torch.arange(ns), (3 * torch.arange(ns)) % ncls] = 1
+        res = []
+        for one_call in (False, True):
+            dx = torch.full_like(x, 3)
+            pooled, dpooled = torch.full((ns, C * Ho * Ho), 3.0, device="cuda", dtype=tdt), torch.full((ns, C * Ho * Ho), 3.0, device="cuda", dtype=tdt)
+            logits, dlogits = torch.full((ns, ncls), 3.0, device="cuda", dtype=tdt), torch.full((ns, ncls), 3.0, device="cuda", dtype=tdt)
+            loss, dw, db = torch.full((ns,), 3.0, device="cuda", dtype=tdt), torch.full_like(w, 3), torch.full_like(b, 3)
+            pa, k1 = hp.pool_args(pkg, x, dx, pooled, dpooled, C, H, H, Ho, Ho, win, win, win, win)
+            la, k2 = hp.linear_args(pkg, pooled, dpooled, w, dw, logits, dlogits, C * Ho * Ho, ncls, b if bias else None, db if bias else None)
+            ca, k3 = hp.loss_args(pkg, logits, dlogits, target, loss, ncls)
+            batch = pkg.WgBatch()
+            batch.buf, batch.bytes = buf.data_ptr(), buf.numel()
+            if one_call:
+                rc = getattr(gpu, "ptl_pool_linear_loss_%s_batched" % dt)(ctypes.byref(pa), ctypes.byref(la), ctypes.byref(ca), ns,
+                                                                         ctypes.byref(batch) if with_batch else None)
+                assert rc == 0, gpu.ptl_last_error()
+                took = batch.count == 1
+                assert getattr(gpu, "ptl_conv2d_%s_wg_flush" % dt)(ctypes.byref(batch)) == 0
+            else:
+                for name, a, extra in (("ptl_avgpool_%s_batched", pa, (ns, 0)), ("ptl_linear_%s_fw_batched", la, (ns,)),
+                                       ("ptl_cross_entropy_%s_batched", ca, (ns, 0)), ("ptl_cross_entropy_%s_batched", ca, (ns, 1)),
+                                       ("ptl_linear_%s_bw_batched", la, (ns,)), ("ptl_avgpool_%s_batched", pa, (ns, 1))):
+                    assert getattr(gpu, name % dt)(ctypes.byref(a), *extra) == 0, gpu.ptl_last_error()
+            assert gpu.ptl_sync() == 0
+            res.append((pooled, logits, loss, dlogits, dw, dpooled, dx, db))
+        A, B = res
+        assert took == expect, case
+        names = ("pooled", "logits", "loss", "dlogits", "dw", "dpooled", "dx", "db")
+        if not took:
+            for i, nm in enumerate(names):
+                assert torch.equal(A[i], B[i]), (case, nm)
+            continue
+        assert torch.equal(A[0], B[0]), case
+        for i, nm in list(enumerate(names))[1:7]:
+            assert hp.rel_l2(B[i].float().cpu().numpy(), A[i].float().cpu().numpy()) <= tol, (case, nm)
+        assert not bool((B[6] == 3).any()) and not bool((B[4] == 3).all())

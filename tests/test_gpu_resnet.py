@@ -196,7 +196,37 @@ def test_resnet20_step_with_the_normalisation_inside_the_forward_convolutions(pk
         assert torch.equal(two.G[n], one.G[n]) and torch.equal(two.Bt[n], one.Bt[n]), n
 
 
-@pytest.mark.parametrize("fused", [True, False, "stats", "post", "pre"])
+@pytest.mark.parametrize("dt,ns,tol", [("fp32", 6, 1e-3), ("fp16", 16, 5e-3)])
+def test_resnet20_step_with_pooling_classifier_and_loss_in_one_call(pkg, gpu, dt, ns, tol):
+    """The step whose tail is one call (ptl_pool_linear_loss_*_batched) against the step with the six calls: five
+    calls fewer, the same forward results up to the classifier's dot products, and gradients that agree to rounding
+    (fp32: everything the step writes; fp16: the last stage's, as in the tests above)."""
+    w = rs.init_weights(0x2E660, dt)
+    x = hp.normal(0x2E661, (ns, 3, 32, 32)).astype(hp.np_dtype(dt))
+    nets = []
+    for head in (False, True):
+        net = rs.ResNetStep(pkg, gpu, torch, dt, ns, w, 0.01, norm=True, fused=True, stats=True, post=True, pre=True, head=head)
+        net.x.copy_(torch.from_numpy(x))
+        net.target.zero_()
+        net.target[torch.arange(ns), (3 * torch.arange(ns)) % 10] = 1
+        net.step(update=True)
+        assert gpu.ptl_sync() == 0
+        nets.append(net)
+    six, one = nets
+    assert six.launches() - one.launches() == 5
+    rel = lambda a, b: hp.rel_l2(a.float().cpu().numpy(), b.float().cpu().numpy())
+    assert torch.equal(six.pooled, one.pooled)
+    assert rel(one.logits, six.logits) <= tol and rel(one.loss, six.loss) <= tol
+    names = list(six.dW) if dt == "fp32" else ["fc", "s2b2c2", "s2b2c1", "s2b1c2"]
+    for n in names:
+        assert rel(one.dW[n], six.dW[n]) <= tol, n
+        assert rel(one.W[n], six.W[n]) <= tol, n
+    for n in (six.dG if dt == "fp32" else ["s2b2c2", "s2b2c1", "s2b1c2"]):
+        assert rel(one.dG[n], six.dG[n]) <= tol, n
+        assert rel(one.dBt[n], six.dBt[n]) <= tol, n
+
+
+@pytest.mark.parametrize("fused", [True, False, "stats", "post", "pre", "head"])
 def test_training_step_replays_as_a_hip_graph(pkg, gpu, fused):
     """The whole step (92 or 178 library calls; "stats": the 92 with the sums of the convolutions' outputs formed by
     the convolutions) captured once into a HIP graph on a stream of the caller's and
@@ -210,7 +240,8 @@ def test_training_step_replays_as_a_hip_graph(pkg, gpu, fused):
     try:
         with torch.cuda.stream(side):
             net = rs.ResNetStep(pkg, gpu, torch, dt, ns, rs.init_weights(0x2E600, dt), 0.01, norm=True, fused=bool(fused),
-                                stats=fused in ("stats", "post", "pre"), post=fused in ("post", "pre"), pre=fused == "pre")
+                                stats=fused in ("stats", "post", "pre", "head"), post=fused in ("post", "pre", "head"),
+                                pre=fused in ("pre", "head"), head=fused == "head")
             net.x.copy_(torch.from_numpy(hp.normal(0x2E601, (ns, 3, 32, 32)).astype(np.float16)))
             net.target.zero_()
             net.target[torch.arange(ns), (3 * torch.arange(ns)) % 10] = 1
