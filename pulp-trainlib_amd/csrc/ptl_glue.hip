@@ -319,38 +319,66 @@ template <typename T>
 __global__ __launch_bounds__(256) void head_kernel(const HeadArgs a) {
     extern __shared__ float head_lds[];
     float *pooled = head_lds, *dpool = pooled + a.C, *logit = dpool + a.C, *dlog = logit + a.ncls;
+    float *Wl = dlog + a.ncls, *yl = Wl + a.ncls * a.C;  // the classifier's weights and the sample's target
     const int n = blockIdx.x, tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const T *x = reinterpret_cast<const T *>(a.x) + (size_t)n * a.C * a.HW;
-    // pooling forward: a wave per channel, lanes stride over the plane (avgpool_fw_kernel's order)
-    for (int c = wave; c < a.C; c += 4) {
-        float s = 0.f;
-        for (int e = lane; e < a.HW; e += 64) s += (float)x[(size_t)c * a.HW + e];
+    // (everything the later phases read from memory is asked for now, with the planes' loads)
+    for (int i = tid; i < a.ncls * a.C; i += 256) Wl[i] = (float)reinterpret_cast<const T *>(a.w)[i];
+    for (int i = tid; i < a.ncls; i += 256) yl[i] = (float)reinterpret_cast<const T *>(a.target)[(size_t)n * a.ncls + i];
+    // pooling forward: a wave per channel, lanes stride over the plane (avgpool_fw_kernel's order), eight channels of
+    // a wave at a time so that their loads are in the air together and their butterflies side by side
+    for (int c0 = wave; c0 < a.C; c0 += 32) {
+        float s[8];
 #pragma unroll
-        for (int off = 32; off > 0; off >>= 1) s += __shfl_xor(s, off);
-        if (lane == 0) {
-            const T p = (T)(s / (float)a.HW);
-            reinterpret_cast<T *>(a.pooled)[(size_t)n * a.C + c] = p;
-            pooled[c] = (float)p;
+        for (int u = 0; u < 8; ++u) {
+            const int c = c0 + 4 * u;
+            s[u] = 0.f;
+            if (c < a.C)
+                for (int e = lane; e < a.HW; e += 64) s[u] += (float)x[(size_t)c * a.HW + e];
+        }
+#pragma unroll
+        for (int off = 32; off > 0; off >>= 1)
+#pragma unroll
+            for (int u = 0; u < 8; ++u) s[u] += __shfl_xor(s[u], off);
+#pragma unroll
+        for (int u = 0; u < 8; ++u) {
+            const int c = c0 + 4 * u;
+            if (lane == 0 && c < a.C) {
+                const T p = (T)(s[u] / (float)a.HW);
+                reinterpret_cast<T *>(a.pooled)[(size_t)n * a.C + c] = p;
+                pooled[c] = (float)p;
+            }
         }
     }
     __syncthreads();
-    // classifier forward: a wave per class
-    const T *W = reinterpret_cast<const T *>(a.w);
-    for (int k = wave; k < a.ncls; k += 4) {
-        float s = 0.f;
-        for (int c = lane; c < a.C; c += 64) s += pooled[c] * (float)W[(size_t)k * a.C + c];
+    // classifier forward: a wave per class, the (at most eight) classes of a wave side by side
+    {
+        float s[8];
 #pragma unroll
-        for (int off = 32; off > 0; off >>= 1) s += __shfl_xor(s, off);
-        if (lane == 0) {
-            const T z = (T)s;
-            reinterpret_cast<T *>(a.logits)[(size_t)n * a.ncls + k] = z;
-            logit[k] = (float)z;
+        for (int u = 0; u < 8; ++u) {
+            const int k = wave + 4 * u;
+            s[u] = 0.f;
+            if (k < a.ncls)
+                for (int c = lane; c < a.C; c += 64) s[u] += pooled[c] * Wl[k * a.C + c];
+        }
+#pragma unroll
+        for (int off = 32; off > 0; off >>= 1)
+#pragma unroll
+            for (int u = 0; u < 8; ++u) s[u] += __shfl_xor(s[u], off);
+#pragma unroll
+        for (int u = 0; u < 8; ++u) {
+            const int k = wave + 4 * u;
+            if (lane == 0 && k < a.ncls) {
+                const T z = (T)s[u];
+                reinterpret_cast<T *>(a.logits)[(size_t)n * a.ncls + k] = z;
+                logit[k] = (float)z;
+            }
         }
     }
     __syncthreads();
     // loss and its gradient: the first wave (cross_entropy_kernel's arithmetic, both passes)
     if (wave == 0) {
-        const T *y = reinterpret_cast<const T *>(a.target) + (size_t)n * a.ncls;
+        const float *y = yl;
         float mx = -FLT_MAX;
         for (int i = lane; i < a.ncls; i += 64) mx = fmaxf(mx, logit[i]);
 #pragma unroll
@@ -358,8 +386,8 @@ __global__ __launch_bounds__(256) void head_kernel(const HeadArgs a) {
         float se = 0.f, dot = 0.f, sy = 0.f;
         for (int i = lane; i < a.ncls; i += 64) {
             se += expf(logit[i] - mx);
-            dot += (float)y[i] * logit[i];
-            sy += (float)y[i];
+            dot += y[i] * logit[i];
+            sy += y[i];
         }
 #pragma unroll
         for (int off = 32; off > 0; off >>= 1) {
@@ -373,7 +401,7 @@ __global__ __launch_bounds__(256) void head_kernel(const HeadArgs a) {
         if (sy == 0.f) sy = 1.0f;
         const float inv = 1.0f / se;
         for (int i = lane; i < a.ncls; i += 64) {
-            const T g = (T)((expf(logit[i] - mx) * inv) * sy - (float)y[i]);
+            const T g = (T)((expf(logit[i] - mx) * inv) * sy - y[i]);
             reinterpret_cast<T *>(a.dlogits)[(size_t)n * a.ncls + i] = g;
             dlog[i] = (float)g;
         }
@@ -382,7 +410,7 @@ __global__ __launch_bounds__(256) void head_kernel(const HeadArgs a) {
     // classifier backward: the gradient of the pooled vector, and this sample's part of the weight gradient
     for (int c = tid; c < a.C; c += 256) {
         float s = 0.f;
-        for (int k = 0; k < a.ncls; ++k) s += dlog[k] * (float)W[(size_t)k * a.C + c];
+        for (int k = 0; k < a.ncls; ++k) s += dlog[k] * Wl[k * a.C + c];
         const T g = (T)s;
         reinterpret_cast<T *>(a.dpooled)[(size_t)n * a.C + c] = g;
         dpool[c] = (float)g;
@@ -396,7 +424,22 @@ __global__ __launch_bounds__(256) void head_kernel(const HeadArgs a) {
     __syncthreads();
     // pooling backward: every element of a plane gets its channel's share (avgpool_bw_kernel with one window)
     T *dx = reinterpret_cast<T *>(a.dx) + (size_t)n * a.C * a.HW;
-    for (int i = tid; i < a.C * a.HW; i += 256) dx[i] = (T)(dpool[i / a.HW] / (float)a.HW);
+    constexpr int VEC = 16 / (int)sizeof(T);
+    if (a.HW % VEC == 0 && (reinterpret_cast<uintptr_t>(a.dx) % 16) == 0) {  // (planes of whole 16-byte pieces)
+        const int pieces = a.HW / VEC;
+        for (int i = tid; i < a.C * pieces; i += 256) {
+            const T v = (T)(dpool[i / pieces] / (float)a.HW);
+            union {
+                uint4 raw;
+                T e[VEC];
+            } o;
+#pragma unroll
+            for (int j = 0; j < VEC; ++j) o.e[j] = v;
+            reinterpret_cast<uint4 *>(dx)[i] = o.raw;
+        }
+    } else {
+        for (int i = tid; i < a.C * a.HW; i += 256) dx[i] = (T)(dpool[i / a.HW] / (float)a.HW);
+    }
 }
 
 template <typename T, typename Pool, typename Lin, typename Loss>
@@ -411,6 +454,7 @@ static int head_step(const Pool *pa, const Lin *la, const Loss *ca, int ns, ::pt
                  ca->wr_loss && pa->Hker == pa->input->H && pa->Wker == pa->input->W && pa->output->H == 1 &&
                  pa->output->W == 1 && pa->input->C > 0 && pa->input->C <= 1024 && pa->input->H * pa->input->W > 0 &&
                  la->input->dim == pa->input->C && la->output->dim > 0 && la->output->dim <= 32 &&
+                 (long long)la->output->dim * pa->input->C <= 8192 &&  // (the weights are kept in LDS)
                  ca->output->dim == la->output->dim && la->use_biases != 1 && !la->skip_wg_grad && !la->skip_in_grad &&
                  pa->output->data == la->input->data && pa->output->diff == la->input->diff &&
                  la->output->data == ca->output->data && la->output->diff == ca->output->diff && pa->input->data &&
@@ -450,7 +494,7 @@ static int head_step(const Pool *pa, const Lin *la, const Loss *ca, int ns, ::pt
             h.ncls = ncls;
             h.cbi_n = (C + 31) / 32;
             h.cols_kept = C < 32 ? C : 32;
-            const size_t lds = (size_t)(2 * C + 2 * ncls) * sizeof(float);
+            const size_t lds = (size_t)(2 * C + 3 * ncls + ncls * C) * sizeof(float);
             hipLaunchKernelGGL((head_kernel<T>), dim3(ns), dim3(256), lds, state().stream, h);
             return hip_ok(hipGetLastError(), "classifier head launch") ? 0 : 2;
         }
