@@ -801,8 +801,8 @@ int launch_small(const ConvSmallArgs &a, int tiles, size_t lds, hipStream_t s, c
 // elements per workgroup of the reduction (coalesced reads), 16 groups of partials in parallel, eight loads in flight
 // per thread; the few results are scattered to the weight tensor's order.
 // PG groups of partials in parallel on 1024 / PG consecutive elements: 16 x 64 where a layer has many workgroups, 4 x 256
-// where it has few (a 64-channel layer has 32 of them and 36 864 elements: with 64 elements a block, 576 blocks of
-// two loads a thread).
+// up to 128 of them (a 64-channel layer has 32 and 36 864 elements: with 64 elements a block, 576 blocks of two loads a
+// thread; at 128 workgroups the two forms are within half a per cent of each other in a ResNet-20 step's flush).
 template <typename T, int PG>
 __device__ inline void wg_small_reduce_part(const float *__restrict__ ws, T *__restrict__ dW, int block, int part_elems,
                                             int parts, int rows_kept, int cols_kept, int cbi_n, int Cout, int Cin,
@@ -841,7 +841,7 @@ __device__ inline void wg_small_reduce_part(const float *__restrict__ ws, T *__r
 }
 
 // (the shape of a layer decides its form, so that a deferred layer's sums have the bits of the immediate call's)
-__host__ __device__ inline int wg_reduce_epb(int parts) { return parts <= 64 ? 256 : 64; }
+__host__ __device__ inline int wg_reduce_epb(int parts) { return parts <= 128 ? 256 : 64; }
 
 template <typename T>
 __device__ inline void wg_small_reduce_block(const float *__restrict__ ws, T *__restrict__ dW, int block, int part_elems,
