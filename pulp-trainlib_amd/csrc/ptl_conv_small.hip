@@ -148,7 +148,7 @@ __device__ inline void conv_small_block(const ConvSmallArgs &a, int tile, char *
     if (a.pre) {  // the statistics of the normalisation in front: a wave per channel and round
         float4 *tab = reinterpret_cast<float4 *>(smem + a.pre_off);
         float2 sums[FOLD_R];
-        norm_fold_take<FOLD_R>(fold, sums);
+        norm_fold_take<FOLD_R>(fold, sums, a.pre_part, a.pre_parts, 0, a.Cin, wave, lane);
 #pragma unroll
         for (int r = 0; r < FOLD_R; ++r) {
             const int c = wave + 16 * r;
@@ -1129,8 +1129,7 @@ int conv_small(const ConvTileDesc &d, const void *X, const void *Wt, void *Y) {
         const bool ok = X == pre->out && pre->x && pre->weight && pre->bias && pre->eps && pre->part && pre->parts > 0 &&
                         aligned(pre->x) && aligned(pre->out) && aligned(pre->skip) && aligned(pre->part) &&
                         p.a.dil == 1 && d.padU <= d.KH - d.sh && (long long)d.Ho * d.sh >= d.Hin &&
-                        pre->count == (size_t)d.batch * d.Hin * d.Win && off + need <= 150 * 1024 &&
-                        pre->parts <= NORM_FOLD_MAX_PARTS;
+                        pre->count == (size_t)d.batch * d.Hin * d.Win && off + need <= 150 * 1024;
         if (!ok) return CONV_PRE_REFUSED;
         p.a.X = pre->x;
         p.a.pre = 1;

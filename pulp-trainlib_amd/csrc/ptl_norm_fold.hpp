@@ -38,9 +38,9 @@ __device__ __forceinline__ float4 norm_fold_wave(const float *__restrict__ part,
 }
 
 // The same sums (places 0 and 1 of a part) in two steps, for a kernel that wants the loads in the air before it issues
-// the loads of its tile and the sums only behind them: channels c0 + wave + 16 r (r < R) of a 16-wave workgroup, at
-// most 256 parts (four per lane).  Bit for bit norm_fold_wave's sums.
-constexpr int NORM_FOLD_MAX_PARTS = 256;
+// the loads of its tile and the sums only behind them: channels c0 + wave + 16 r (r < R) of a 16-wave workgroup.  The
+// first 256 parts (four per lane) are asked for early, the rest - batches of many hundred samples - is read when the
+// sums are taken.  Bit for bit norm_fold_wave's sums.
 template <int R>
 struct NormFoldRegs {
     float2 v[R][4];
@@ -60,7 +60,8 @@ __device__ __forceinline__ void norm_fold_ask(NormFoldRegs<R> &f, const float *_
     }
 }
 template <int R>
-__device__ __forceinline__ void norm_fold_take(const NormFoldRegs<R> &f, float2 (&t)[R]) {
+__device__ __forceinline__ void norm_fold_take(const NormFoldRegs<R> &f, float2 (&t)[R], const float *__restrict__ part,
+                                               int nparts, int c0, int nch, int wave, int lane) {
 #pragma unroll
     for (int r = 0; r < R; ++r) {
         t[r] = make_float2(0.f, 0.f);
@@ -69,6 +70,13 @@ __device__ __forceinline__ void norm_fold_take(const NormFoldRegs<R> &f, float2 
             t[r].x += f.v[r][u].x;
             t[r].y += f.v[r][u].y;
         }
+        const int c = wave + 16 * r;
+        if (nparts > 256 && c < nch)
+            for (int i = 256 + lane; i < nparts; i += 64) {
+                const float2 p = *reinterpret_cast<const float2 *>(part + ((size_t)(c0 + c) * nparts + i) * 4);
+                t[r].x += p.x;
+                t[r].y += p.y;
+            }
     }
 #pragma unroll
     for (int off = 32; off > 0; off >>= 1) {

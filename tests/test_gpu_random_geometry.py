@@ -433,7 +433,8 @@ def test_conv2d_forward_applies_the_normalisation_in_front(pkg, gpu, dt):
     leaves, bit for bit - where the small-layer kernel does both in one launch (ptl_last_conv_resident() == 3: 3x3
     layers of either stride with "same" padding, with and without ReLU and skip tensor, ragged tiles) and where it
     cannot and the two calls run (a wide layer, a strided 1x1 layer that does not read every row, no padding,
-    sums that do not cover the tensor or come in more than 256 parts, host tensors)."""
+    sums that do not cover the tensor, host tensors); sums in 700 parts, more than a lane asks for early, are folded
+    all the same."""
     tdt = torch.float16 if dt == "fp16" else torch.float32
     part0 = torch.empty(1 << 18, dtype=torch.float32, device="cuda")
     parts = [torch.empty(1 << 18, dtype=torch.float32, device="cuda") for _ in range(2)]
@@ -443,7 +444,7 @@ def test_conv2d_forward_applies_the_normalisation_in_front(pkg, gpu, dt):
              (5, 8, 24, 40, 16, 3, 1, 1, 1, 1, 1, None), (3, 8, 20, 12, 24, 3, 1, 1, 0, 0, 1, None),
              (7, 12, 36, 24, 24, 1, 1, 0, 1, 0, 1, None), (32, 16, 16, 32, 32, 1, 2, 0, 1, 1, 1, False),
              (8, 16, 16, 16, 16, 3, 1, 0, 1, 0, 1, False), (4, 16, 128, 128, 8, 3, 1, 1, 1, 1, 1, False),
-             (64, 16, 32, 32, 16, 3, 1, 1, 1, 1, 0, False), (64, 16, 32, 32, 16, 3, 1, 1, 1, 1, 2, False)]
+             (64, 16, 32, 32, 16, 3, 1, 1, 1, 1, 0, False), (64, 16, 32, 32, 16, 3, 1, 1, 1, 1, 2, True)]
     fused = 0
     for case in cases:
         ns, Cp, Ci, Co, H, K, s, p, relu, with_skip, sums_valid, expect = case
@@ -462,11 +463,15 @@ def test_conv2d_forward_applies_the_normalisation_in_front(pkg, gpu, dt):
             st_in.count, st_in.parts, st_in.channels, st_in.valid = ns * H * H, 1, Ci, 1
         if not sums_valid:
             st_in.count += 1
-        if sums_valid == 2:  # (more parts than the kernel folds: 300, all but one of them zeros)
-            part0[:Ci * 300 * 4] = 0
-            part0[:Ci * 300 * 4].view(Ci, 300, 4)[:, 7, 0] = y0.double().sum((0, 2, 3)).float()
-            part0[:Ci * 300 * 4].view(Ci, 300, 4)[:, 7, 1] = (y0.double() ** 2).sum((0, 2, 3)).float()
-            st_in.count, st_in.parts, st_in.channels, st_in.valid = ns * H * H, 300, Ci, 1
+        if sums_valid == 2:  # (more parts than a lane asks for early: 700, the sums spread over them)
+            np_ = 700
+            sums = torch.stack((y0.double().sum((0, 2, 3)), (y0.double() ** 2).sum((0, 2, 3))), 1)  # [Ci][2]
+            wgt = torch.rand(Ci, np_, 1, device="cuda", dtype=torch.float64)
+            wgt = wgt / wgt.sum(1, keepdim=True)
+            pv = part0[:Ci * np_ * 4].view(Ci, np_, 4)
+            pv.zero_()
+            pv[:, :, :2] = (wgt * sums[:, None, :]).float()
+            st_in.count, st_in.parts, st_in.channels, st_in.valid = ns * H * H, np_, Ci, 1
         gm, bt = (torch.rand(Ci, device="cuda") + 0.5).to(tdt), (torch.rand(Ci, device="cuda") - 0.5).to(tdt)
         eps = torch.tensor([1e-5], device="cuda").to(tdt)
         skip = (torch.rand(ns, Ci, H, H, device="cuda") - 0.5).to(tdt)
