@@ -372,8 +372,18 @@ __global__ __launch_bounds__(256) void panel_reduce_kernel(PanelArgs a) {
     if (i >= nm) return;
     const int o = blockIdx.y;
     const float *p = a.part + (size_t)o * a.groups * nm + i;
+    // eight loads in flight at a time (a serial walk is one trip to memory per group); the sums are added in
+    // the order of the groups either way
     float s = 0.f;
-    for (int g = 0; g < a.groups; ++g) s += p[(size_t)g * nm];
+    int g = 0;
+    for (; g + 8 <= a.groups; g += 8) {
+        float v[8];
+#pragma unroll
+        for (int j = 0; j < 8; ++j) v[j] = p[(size_t)(g + j) * nm];
+#pragma unroll
+        for (int j = 0; j < 8; ++j) s += v[j];
+    }
+    for (; g < a.groups; ++g) s += p[(size_t)g * nm];
     float *dst = a.C[o] + (i / a.M) * a.c_n + (i % a.M);
     *dst = a.accumulate ? *dst + s : s;
 }
