@@ -679,6 +679,25 @@ def detail_table(pkg, lib, hp, to_dev, timed, check, torch, dev):
                 ms = timed(lambda: check(lib.ptl_conv2d_fp16_bw_batched_cached(ref, ns, ctypes.byref(cache))), 10)
                 add("conv2d %d->%d %dx%d k3 p1 WG+IG in one call, input copy kept by FW N=%d" % (Ci, Co, H, H, ns), dt,
                     ms, 2 * flops, 2 * nb)
+                # layers in a row: the forward kernel also writes its output as the blocked copy the next layer reads
+                # (timed here with the layer itself as that next layer: same channels in and out), and the forward call
+                # of a layer that was handed such a copy
+                if Ci == Co:
+                    nxt = torch.empty(nbytes, dtype=torch.uint8, device=dev)
+                    oc = pkg.ConvCache()
+                    oc.buf, oc.bytes = nxt.data_ptr(), nbytes
+                    check(lib.ptl_conv2d_fp16_cache_prepare(ref, ns, ctypes.byref(oc)))
+                    ms = timed(lambda: check(lib.ptl_conv2d_fp16_fw_batched_chained(ref, ns, None, ctypes.byref(oc))), 10)
+                    if oc.valid:
+                        add("conv2d %d->%d %dx%d k3 p1 FW writing the next layer's input copy N=%d" % (Ci, Co, H, H, ns),
+                            dt, ms, flops, nb)
+                    ms = timed(lambda: check(lib.ptl_conv2d_fp16_fw_batched_chained(ref, ns, ctypes.byref(cache), None)), 10)
+                    add("conv2d %d->%d %dx%d k3 p1 FW, input copy left by the layer before N=%d" % (Ci, Co, H, H, ns), dt,
+                        ms, flops, nb)
+                    ms = timed(lambda: check(lib.ptl_conv2d_fp16_fw_batched_chained(ref, ns, ctypes.byref(cache),
+                                                                                     ctypes.byref(oc))), 10)
+                    add("conv2d %d->%d %dx%d k3 p1 FW, copy in and copy out N=%d" % (Ci, Co, H, H, ns), dt, ms, flops, nb)
+                    del nxt
             del kept
         del x, w, dy, y, dx, dw
 

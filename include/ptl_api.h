@@ -423,6 +423,21 @@ size_t ptl_conv2d_fp16_cache_bytes(const struct Conv2D_args_fp16 *a, int nsample
 int ptl_conv2d_fp16_fw_batched_cached(const struct Conv2D_args_fp16 *a, int nsamples, struct ptl_conv_cache *c);
 int ptl_conv2d_fp16_wg_batched_cached(const struct Conv2D_args_fp16 *a, int nsamples, const struct ptl_conv_cache *c);
 int ptl_conv2d_fp16_bw_batched_cached(const struct Conv2D_args_fp16 *a, int nsamples, const struct ptl_conv_cache *c);
+/* No counterpart in the reference: layers in a row.  The forward kernel of such a layer can write its output a second
+ * time, as the padded, channel-blocked copy the NEXT layer's kernels read, so that the next layer's forward and
+ * weight-gradient calls start without their layout pass.  ptl_conv2d_fp16_cache_prepare(reader, ...) sets a cache up
+ * as the input copy of the layer `reader` (the caller sets buf - 16-byte aligned device memory - and bytes >=
+ * ptl_conv2d_fp16_cache_bytes(reader, nsamples)): it zeroes the buffer once, on the library's stream, and records the
+ * geometry; 1 if that layer would not read such a copy.  ptl_conv2d_fp16_fw_batched_chained(a, n, in, out) is the
+ * forward call of a layer with `in` = the copy of ITS input (valid: read instead of copying; not valid: filled, as by
+ * the _cached call; NULL: none) and `out` = a cache prepared for the layer that reads this layer's output (NULL:
+ * none): out->valid says whether the copy was written - the layer must take the resident-tile route, and its output
+ * must be the reader's input tensor (same batch, channels, height and width).  The weight-gradient calls of the
+ * reader take the same cache through the _cached entry points.  The copies belong to the caller; a call that
+ * overlaps another one on the same cache races. */
+int ptl_conv2d_fp16_cache_prepare(const struct Conv2D_args_fp16 *reader, int nsamples, struct ptl_conv_cache *c);
+int ptl_conv2d_fp16_fw_batched_chained(const struct Conv2D_args_fp16 *a, int nsamples, struct ptl_conv_cache *in,
+                                       struct ptl_conv_cache *out);
 /* No counterpart in the reference: ptl_conv2d_*_bw_batched with the last launch of a small layer's weight gradient
  * (the addition of its partial sums) put off and done for all deferred layers at once by ptl_conv2d_*_wg_flush
  * (struct ptl_wg_batch; a training step with twenty small layers saves twenty launches).  A layer that does not take

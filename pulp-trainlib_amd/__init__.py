@@ -92,6 +92,10 @@ FUSED_NORM_ENTRY_POINTS = ["ptl_batch_norm_fused_%s_%s" % (dt, step) for dt in (
 # `int f(const Conv2D_args_fp16 *, int nsamples, [const] ptl_conv_cache *)` and the size query
 CACHED_ENTRY_POINTS = ["ptl_conv2d_fp16_%s_batched_cached" % s for s in ("fw", "wg", "bw")] + ["ptl_conv2d_fp16_cache_bytes"]
 
+# `int f(const Conv2D_args_fp16 *reader, int nsamples, ptl_conv_cache *)` and
+# `int f(const Conv2D_args_fp16 *, int nsamples, ptl_conv_cache *in, ptl_conv_cache *out)`
+CHAINED_ENTRY_POINTS = ["ptl_conv2d_fp16_cache_prepare", "ptl_conv2d_fp16_fw_batched_chained"]
+
 # `int f(const Conv2D_args[_fp16] *, int nsamples, ptl_wg_batch *)` and `int f(ptl_wg_batch *)`
 DEFERRED_ENTRY_POINTS = ["ptl_conv2d_%s_bw_batched_deferred" % dt for dt in ("fp16", "fp32")] + \
                         ["ptl_conv2d_%s_wg_flush" % dt for dt in ("fp16", "fp32")]
@@ -151,6 +155,10 @@ def load():
         f = getattr(lib, name)
         f.argtypes = [ctypes.c_void_p, ctypes.c_int, ctypes.c_void_p]
         f.restype = ctypes.c_int
+    lib.ptl_conv2d_fp16_cache_prepare.argtypes = [ctypes.c_void_p, ctypes.c_int, ctypes.c_void_p]
+    lib.ptl_conv2d_fp16_cache_prepare.restype = ctypes.c_int
+    lib.ptl_conv2d_fp16_fw_batched_chained.argtypes = [ctypes.c_void_p, ctypes.c_int, ctypes.c_void_p, ctypes.c_void_p]
+    lib.ptl_conv2d_fp16_fw_batched_chained.restype = ctypes.c_int
     for name in DEFERRED_ENTRY_POINTS[:2]:
         f = getattr(lib, name)
         f.argtypes = [ctypes.c_void_p, ctypes.c_int, ctypes.c_void_p]

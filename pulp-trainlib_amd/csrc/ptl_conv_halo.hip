@@ -49,6 +49,10 @@ struct HaloArgs {
     int batch, Cin, Cout, Hp, Wp, Ho, Wo;
     int tiles, ct_count;  // tile = position tile * ct_count + filter tile
     int xcd_map;          // 1: the grid is a multiple of 8 and a workgroup's first tile follows its XCD
+    // channel-major route, optional: the output once more as the next layer's blocked, padded input
+    half_t *yblk;           // [Cout/8][yb_P] chunks of eight filters, nullptr: no such copy
+    unsigned yb_P;          // chunks per block of eight filters: batch * yb_Hp * yb_Wp
+    int yb_Hp, yb_Wp, yb_padU, yb_padL;
 };
 
 template <int I, int N, typename F>
@@ -331,14 +335,14 @@ __global__ __launch_bounds__(HALO_NT) void conv_halo_kernel(const HaloArgs a) {
             const unsigned q0 = ((unsigned)cu.tile / (unsigned)a.ct_count) * HALO_BM;
             const int co0 = (cu.tile % a.ct_count) * BN;
             const unsigned PO = (unsigned)(a.Ho * a.Wo);
+            if constexpr (HWC) {
 #pragma unroll
-            for (int j = 0; j < FN; ++j) {
-                const unsigned q = q0 + (unsigned)(64 * wave + 16 * j + l16);  // (Q < 2^31 on the host)
-                const unsigned b = q / a.qimg, rem = q - b * a.qimg;
-                const unsigned yy = rem / (unsigned)a.Wp, xx = rem - yy * (unsigned)a.Wp;
-                if (q < a.Q && yy < (unsigned)a.Ho && xx < (unsigned)a.Wo) {
-                    // a lane holds four consecutive filters of its position per filter fragment
-                    if constexpr (HWC) {
+                for (int j = 0; j < FN; ++j) {
+                    const unsigned q = q0 + (unsigned)(64 * wave + 16 * j + l16);  // (Q < 2^31 on the host)
+                    const unsigned b = q / a.qimg, rem = q - b * a.qimg;
+                    const unsigned yy = rem / (unsigned)a.Wp, xx = rem - yy * (unsigned)a.Wp;
+                    if (q < a.Q && yy < (unsigned)a.Ho && xx < (unsigned)a.Wo) {
+                        // a lane holds four consecutive filters of its position per filter fragment
                         half_t *dst = a.y + ((size_t)b * PO + yy * (unsigned)a.Wo + xx) * (unsigned)a.Cout + co0 + 4 * kq;
 #pragma unroll
                         for (int i = 0; i < FM; ++i) {
@@ -350,12 +354,75 @@ __global__ __launch_bounds__(HALO_NT) void conv_halo_kernel(const HaloArgs a) {
                             for (int v = 0; v < 4; ++v) o.e[v] = (half_t)acc[i][j][v];
                             *reinterpret_cast<uint2 *>(dst + i * 16) = o.v;
                         }
-                    } else {
-                        half_t *dst = a.y + ((size_t)b * a.Cout + co0 + 4 * kq) * PO + yy * (unsigned)a.Wo + xx;
+                    }
+                }
+            } else {
+                // Channel-major output: a row of 16 lanes holds four consecutive filters of 16 positions per fragment,
+                // which as it stands is four 32-byte runs per store.  The four position fragments (registers) and
+                // the four filter groups (rows of lanes) change places - two swaps of lane rows per register, on
+                // the values already rounded to halves and packed in pairs - so that lane l holds position l of
+                // the wave's 64 and every filter of the tile: a store is then one run of 128 bytes, and the copy
+                // for the next layer one 16-byte chunk per lane and eight filters.
+                typedef unsigned pk_t;
+                pk_t pk[FM][FN][2];
+#pragma unroll
+                for (int i = 0; i < FM; ++i)
+#pragma unroll
+                    for (int j = 0; j < FN; ++j)
+#pragma unroll
+                        for (int h = 0; h < 2; ++h) {
+                            union {
+                                half_t e[2];
+                                pk_t u;
+                            } o;
+                            o.e[0] = (half_t)acc[i][j][2 * h];
+                            o.e[1] = (half_t)acc[i][j][2 * h + 1];
+                            pk[i][j][h] = o.u;
+                        }
+                static_assert(FN == 4, "four position fragments against four rows of lanes");
+#pragma unroll
+                for (int i = 0; i < FM; ++i)
+#pragma unroll
+                    for (int h = 0; h < 2; ++h) {
+                        const auto s01 = __builtin_amdgcn_permlane16_swap(pk[i][0][h], pk[i][1][h], false, false);
+                        const auto s23 = __builtin_amdgcn_permlane16_swap(pk[i][2][h], pk[i][3][h], false, false);
+                        const auto t02 = __builtin_amdgcn_permlane32_swap(s01[0], s23[0], false, false);
+                        const auto t13 = __builtin_amdgcn_permlane32_swap(s01[1], s23[1], false, false);
+                        pk[i][0][h] = t02[0];  // now [i][kk][h]: filters i*16 + 4*kk + 2*h, + 1 of position `lane`
+                        pk[i][2][h] = t02[1];
+                        pk[i][1][h] = t13[0];
+                        pk[i][3][h] = t13[1];
+                    }
+                const unsigned q = q0 + (unsigned)(64 * wave + lane);  // (Q < 2^31 on the host)
+                const unsigned b = q / a.qimg, rem = q - b * a.qimg;
+                const unsigned yy = rem / (unsigned)a.Wp, xx = rem - yy * (unsigned)a.Wp;
+                if (q < a.Q && yy < (unsigned)a.Ho && xx < (unsigned)a.Wo) {
+                    half_t *dst = a.y + ((size_t)b * a.Cout + co0) * PO + yy * (unsigned)a.Wo + xx;
+#pragma unroll
+                    for (int i = 0; i < FM; ++i)
+#pragma unroll
+                        for (int kk = 0; kk < 4; ++kk)
+#pragma unroll
+                            for (int h = 0; h < 2; ++h) {
+                                union {
+                                    half_t e[2];
+                                    pk_t u;
+                                } o;
+                                o.u = pk[i][kk][h];
+                                dst[(size_t)(i * 16 + 4 * kk + 2 * h) * PO] = o.e[0];
+                                dst[(size_t)(i * 16 + 4 * kk + 2 * h + 1) * PO] = o.e[1];
+                            }
+                    if (a.yblk) {
+                        const unsigned pos = ((b * (unsigned)a.yb_Hp + yy + (unsigned)a.yb_padU) * (unsigned)a.yb_Wp) + xx +
+                                             (unsigned)a.yb_padL;
 #pragma unroll
                         for (int i = 0; i < FM; ++i)
 #pragma unroll
-                            for (int v = 0; v < 4; ++v) dst[(size_t)(i * 16 + v) * PO] = (half_t)acc[i][j][v];
+                            for (int c = 0; c < 2; ++c) {
+                                const unsigned cb = (unsigned)(co0 + i * 16 + 8 * c) >> 3;
+                                *reinterpret_cast<uint4 *>(a.yblk + ((size_t)cb * a.yb_P + pos) * 8) =
+                                    make_uint4(pk[i][2 * c][0], pk[i][2 * c][1], pk[i][2 * c + 1][0], pk[i][2 * c + 1][1]);
+                            }
                     }
                 }
             }
@@ -727,7 +794,8 @@ bool conv_halo_fits(const ConvTileDesc &d, int Hp, int Wp) {
 }
 
 // xb: blocked, padded input with conv_halo_margin() readable chunks after the last block; wr: tap-major filters.
-int conv_halo_launch(const ConvTileDesc &d, const void *xb, const void *wr, void *Y, int Hp, int Wp, long long pstride) {
+int conv_halo_launch(const ConvTileDesc &d, const void *xb, const void *wr, void *Y, int Hp, int Wp, long long pstride,
+                     const HaloOutCopy *oc) {
     State &st = state();
     HaloArgs a = {};
     a.xb = static_cast<const char *>(xb);
@@ -745,6 +813,16 @@ int conv_halo_launch(const ConvTileDesc &d, const void *xb, const void *wr, void
     a.maxcross = (unsigned)(skip ? crossings : 0);
     a.Q = (unsigned)((long long)d.batch * a.qimg);
     a.batch = d.batch; a.Cin = d.Cin; a.Cout = d.Cout; a.Hp = Hp; a.Wp = Wp; a.Ho = d.Ho; a.Wo = d.Wo;
+    if (oc && oc->buf) {
+        // every output pixel must land inside the copy's grid, and the copy's chunks are counted in 32 bits
+        const long long plane = (long long)d.batch * oc->Hp * oc->Wp;
+        if (oc->padU < 0 || oc->padL < 0 || d.Ho + oc->padU > oc->Hp || d.Wo + oc->padL > oc->Wp || d.Cout % 8 != 0 ||
+            plane * (d.Cout / 8) >= ((long long)1 << 31))
+            return -1;
+        a.yblk = static_cast<half_t *>(oc->buf);
+        a.yb_P = (unsigned)plane;
+        a.yb_Hp = oc->Hp; a.yb_Wp = oc->Wp; a.yb_padU = oc->padU; a.yb_padL = oc->padL;
+    }
     const int bn = d.Cout % 128 == 0 ? 128 : d.Cout % 64 == 0 ? 64 : 32;
     a.ct_count = d.Cout / bn;
     const long long ptiles = ((long long)a.Q + HALO_BM - 1) / HALO_BM;

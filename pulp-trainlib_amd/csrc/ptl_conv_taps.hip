@@ -22,15 +22,21 @@ namespace ptl {
 
 static ::ptl_conv_cache *g_cache_fill = nullptr;
 static const ::ptl_conv_cache *g_cache_use = nullptr;
+static const ::ptl_conv_cache *g_cache_in = nullptr;
+static ::ptl_conv_cache *g_cache_out = nullptr;
 void conv_cache_set(::ptl_conv_cache *fill, const ::ptl_conv_cache *use) {
     g_cache_fill = fill;
     g_cache_use = use;
 }
+void conv_cache_chain(const ::ptl_conv_cache *in, ::ptl_conv_cache *out) {
+    g_cache_in = in;
+    g_cache_out = out;
+}
 
 // The cached copy, if the call in progress was given one that fits this layer: `chunks` 16-byte pieces (margin
 // included) of the blocked, padded input of `d`.
-static const uint4 *cached_input(const ConvTileDesc &d, int Hp, int Wp, long long chunks) {
-    const ::ptl_conv_cache *c = g_cache_use;
+static const uint4 *cached_input(const ConvTileDesc &d, int Hp, int Wp, long long chunks,
+                                 const ::ptl_conv_cache *c = g_cache_use) {
     if (!c || !c->valid || !c->buf || c->bytes < (size_t)chunks * 16) return nullptr;
     const int want[6] = {d.batch, d.Cin, Hp, Wp, d.padU, d.padL};
     for (int i = 0; i < 6; ++i)
@@ -217,12 +223,14 @@ int conv_taps(const ConvTileDesc &d, const void *X, const void *Wt, void *Y, con
     // the blocked input goes to the caller's buffer when the call brought one (the weight gradient of the layer
     // reads the same copy), else to scratch memory like the filters
     const size_t xb_bytes = (size_t)(xb_elems + margin * VEC) * ES;
-    ::ptl_conv_cache *fill = g_cache_fill;
+    // a copy the call was handed (left by the layer that produced the input): nothing to copy
+    const uint4 *given = halo && g_cache_in ? cached_input(d, Hp, Wp, xb_elems / VEC + margin, g_cache_in) : nullptr;
+    ::ptl_conv_cache *fill = given ? nullptr : g_cache_fill;
     const bool keep = halo && fill && fill->buf && fill->bytes >= xb_bytes && reinterpret_cast<uintptr_t>(fill->buf) % 16 == 0;
-    char *buf = static_cast<char *>(scratch((keep ? 0 : xb_bytes) + (size_t)wr_elems * ES + 512));
+    char *buf = static_cast<char *>(scratch(((keep || given) ? 0 : xb_bytes) + (size_t)wr_elems * ES + 512));
     if (!buf) return 2;
-    uint4 *xb = reinterpret_cast<uint4 *>(keep ? static_cast<char *>(fill->buf) : buf);
-    T *wr = reinterpret_cast<T *>(keep ? buf : buf + ((xb_bytes + 255) & ~(size_t)255));
+    uint4 *xb = given ? const_cast<uint4 *>(given) : reinterpret_cast<uint4 *>(keep ? static_cast<char *>(fill->buf) : buf);
+    T *wr = reinterpret_cast<T *>((keep || given) ? buf : buf + ((xb_bytes + 255) & ~(size_t)255));
     if (keep) {
         const int geo[6] = {d.batch, d.Cin, Hp, Wp, d.padU, d.padL};
         for (int i = 0; i < 6; ++i) fill->geometry[i] = geo[i];
@@ -237,7 +245,7 @@ int conv_taps(const ConvTileDesc &d, const void *X, const void *Wt, void *Y, con
         p.hwc = hwc;
         p.sb = d.x_sb; p.sc = d.x_sc;
         p.xb_total = xb_elems / VEC + margin;
-        p.copy_blocks = (unsigned)((p.xb_total + 255) / 256);
+        p.copy_blocks = given ? 0u : (unsigned)((p.xb_total + 255) / 256);
         p.w = Wt;
         p.wr = wr;
         p.C = d.Cin; p.KW = d.KW; p.taps = taps;
@@ -249,7 +257,25 @@ int conv_taps(const ConvTileDesc &d, const void *X, const void *Wt, void *Y, con
     }
 
     st.last_conv_resident = halo;
-    if (halo) return conv_halo_launch(d, xb, wr, Y, Hp, Wp);
+    if (halo) {
+        // the output once more as the next layer's blocked, padded input, when the call brought a prepared buffer
+        // for it (geometry: batch, channels, padded height and width, top and left padding of that layer)
+        ::ptl_conv_cache *out = g_cache_out;
+        HaloOutCopy oc = {};
+        if (out && out->buf && reinterpret_cast<uintptr_t>(out->buf) % 16 == 0 && out->geometry[0] == d.batch &&
+            out->geometry[1] == d.Cout && d.Cout % 8 == 0 && out->geometry[2] > 0 && out->geometry[3] > 0 &&
+            out->bytes >= ((size_t)(d.Cout / 8) * d.batch * out->geometry[2] * out->geometry[3] + (size_t)conv_halo_margin()) * 16) {
+            oc.buf = out->buf;
+            oc.Hp = out->geometry[2]; oc.Wp = out->geometry[3]; oc.padU = out->geometry[4]; oc.padL = out->geometry[5];
+        }
+        int rc = conv_halo_launch(d, xb, wr, Y, Hp, Wp, 0, oc.buf ? &oc : nullptr);
+        if (rc == -1 && oc.buf) {  // (the copy does not fit this layer's output: the layer without it)
+            oc.buf = nullptr;
+            rc = conv_halo_launch(d, xb, wr, Y, Hp, Wp);
+        }
+        if (rc == 0 && oc.buf) out->valid = 1;
+        return rc;
+    }
 
     GemmArgs q = {};
     q.A = xb;

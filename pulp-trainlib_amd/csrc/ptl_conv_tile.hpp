@@ -121,8 +121,15 @@ inline bool conv_output_fits_pads(const ConvTileDesc &d) {
 // filters).  Y is the dense channel-major output [batch][Cout][Ho][Wo].
 bool conv_halo_fits(const ConvTileDesc &d, int Hp, int Wp);
 long long conv_halo_margin();
+// A second copy of the output for the layer that reads it next: channel-blocked and padded for THAT layer,
+// [channels / 8][batch][Hp][Wp] 16-byte chunks with the output pixel (y, x) at (y + padU, x + padL); the kernel
+// writes the pixels, the halo is the caller's (zero) business.
+struct HaloOutCopy {
+    void *buf;
+    int Hp, Wp, padU, padL;
+};
 int conv_halo_launch(const ConvTileDesc &d, const void *xb, const void *wr, void *Y, int Hp, int Wp,
-                     long long pstride = 0);  // pstride: positions between channel blocks of xb (0: batch*Hp*Wp)
+                     long long pstride = 0, const HaloOutCopy *out_copy = nullptr);  // pstride: positions between channel blocks of xb (0: batch*Hp*Wp)
 // The same layers with channel-minor tensors read in place (X [batch][H][W][Cin], tap-major filters, Y
 // [batch][H][W][Cout]): one launch, the zero border comes from the addresses of the loads.
 bool conv_halo_hwc_fits(const ConvTileDesc &d, const void *X, const void *Y);
@@ -155,6 +162,10 @@ int conv_halo_bw(const ConvTileDesc &fwd, const ConvTileDesc &ig, const void *X,
 // written by the forward route that builds such a copy, `use` read by the weight-gradient routes.  Both null outside
 // the *_cached entry points.
 void conv_cache_set(struct ::ptl_conv_cache *fill, const struct ::ptl_conv_cache *use);
+// Layers in a row (the *_chained forward entry point): `in` is a copy of this layer's input that the forward route
+// may read instead of making one (valid: left there by the layer before), `out` a prepared buffer for the copy of
+// this layer's output that the next layer reads.  Both null outside that entry point.
+void conv_cache_chain(const struct ::ptl_conv_cache *in, struct ::ptl_conv_cache *out);
 // Where the small-layer weight gradient leaves its partial sums instead of adding them up itself (nullptr: nowhere);
 // the one launch that adds up all the layers a batch holds.
 void conv_small_defer_to(struct ::ptl_wg_batch *batch);

@@ -1149,6 +1149,47 @@ int ptl_conv2d_fp16_fw_batched_cached(const struct Conv2D_args_fp16 *a, int ns, 
     ptl::conv_cache_set(nullptr, nullptr);
     return rc;
 }
+int ptl_conv2d_fp16_cache_prepare(const struct Conv2D_args_fp16 *reader, int ns, struct ptl_conv_cache *c) {
+    if (!c) {
+        ptl::set_error("ptl_conv2d_fp16_cache_prepare: no cache");
+        return 1;
+    }
+    c->valid = 0;
+    const size_t need = ptl_conv2d_fp16_cache_bytes(reader, ns);
+    ptl::ConvGeom g;
+    if (need == 0 || ptl::conv_geom(reader, g, "ptl_conv2d_fp16_cache_prepare", false)) {
+        ptl::set_error("ptl_conv2d_fp16_cache_prepare: the layer does not read a blocked copy of its input");
+        return 1;
+    }
+    if (!c->buf || c->bytes < need || reinterpret_cast<uintptr_t>(c->buf) % 16 != 0) {
+        ptl::set_error("ptl_conv2d_fp16_cache_prepare: the buffer must be 16-byte aligned device memory of %zu bytes", need);
+        return 1;
+    }
+    if (!ptl::ensure_init()) return 2;
+    // zero halo, zero margin: the producing layer only ever writes the pixels
+    const size_t n = need / 2;  // halves, 8 per thread
+    hipLaunchKernelGGL((ptl::zero_kernel<half_t>), dim3(ptl::blocks_for((n + 7) / 8)), dim3(256), 0, ptl::state().stream,
+                       static_cast<half_t *>(c->buf), n, 8);
+    if (!ptl::hip_ok(hipGetLastError(), "zero launch")) return 2;
+    ptl::ConvTileDesc d = {};
+    d.Hin = g.H; d.Win = g.W; d.padU = g.Up; d.padD = g.Dp; d.padL = g.Lp; d.padR = g.Rp;
+    int Hp, Wp;
+    ptl::conv_padded_grid(d, &Hp, &Wp);
+    const int geo[6] = {ns, g.Ci, Hp, Wp, g.Up, g.Lp};
+    for (int i = 0; i < 6; ++i) c->geometry[i] = geo[i];
+    return 0;
+}
+int ptl_conv2d_fp16_fw_batched_chained(const struct Conv2D_args_fp16 *a, int ns, struct ptl_conv_cache *in,
+                                       struct ptl_conv_cache *out) {
+    if (out) out->valid = 0;
+    const bool have = in && in->valid;
+    ptl::conv_cache_set(have ? nullptr : in, nullptr);
+    ptl::conv_cache_chain(have ? in : nullptr, out);
+    const int rc = ptl::conv2d_fw<half_t>(a, ns, "pulp_conv2d_fp16_fw_cl");
+    ptl::conv_cache_set(nullptr, nullptr);
+    ptl::conv_cache_chain(nullptr, nullptr);
+    return rc;
+}
 int ptl_conv2d_fp16_wg_batched_cached(const struct Conv2D_args_fp16 *a, int ns, const struct ptl_conv_cache *c) {
     ptl::conv_cache_set(nullptr, c);
     const int rc = ptl::conv2d_wg<half_t>(a, ns, "pulp_conv2d_fp16_bw_param_grads_cl");

@@ -31,7 +31,7 @@ def test_library_exports_every_declared_symbol(pkg):
     # and the Python lists name nothing the header does not declare
     listed = set(pkg.VOID_ENTRY_POINTS + pkg.BATCHED_ENTRY_POINTS + pkg.OTHER_ENTRY_POINTS + pkg.STEP_ENTRY_POINTS +
                  pkg.PLAIN_ENTRY_POINTS + pkg.FUSED_NORM_ENTRY_POINTS + pkg.CACHED_ENTRY_POINTS + pkg.DEFERRED_ENTRY_POINTS + pkg.STATS_ENTRY_POINTS +
-                 pkg.GRAD_STATS_ENTRY_POINTS + pkg.NORMED_ENTRY_POINTS +
+                 pkg.GRAD_STATS_ENTRY_POINTS + pkg.NORMED_ENTRY_POINTS + pkg.CHAINED_ENTRY_POINTS +
                  pkg.HEAD_ENTRY_POINTS)
     assert listed == set(names)
 

@@ -255,6 +255,90 @@ RESIDENT_CASES = [
 ]
 
 
+# (channels in, height, width, channels between, channels out, padding of the first layer, of the second, batch)
+CHAIN_CASES = [(64, 14, 14, 64, 64, (1, 1, 1, 1), (1, 1, 1, 1), 12), (64, 9, 11, 128, 64, (1, 1, 1, 1), (0, 2, 1, 1), 20),
+               (128, 28, 28, 64, 128, (1, 1, 1, 1), (1, 1, 1, 1), 5), (64, 12, 10, 192, 64, (1, 1, 1, 1), (1, 1, 0, 0), 9),
+               (32, 16, 16, 64, 64, (1, 1, 1, 1), (1, 1, 1, 1), 8)]
+
+
+@pytest.mark.parametrize("case", CHAIN_CASES)
+def test_conv2d_layers_in_a_row_hand_the_blocked_copy_on(pkg, gpu, case):
+    """ptl_conv2d_fp16_fw_batched_chained: the forward kernel of a layer writes its output a second time as the padded,
+    channel-blocked copy the next layer reads; the next layer's forward and weight-gradient calls take that copy
+    instead of making one.  Same bits as the plain calls everywhere; the copy really is what is read (the tensor
+    itself is overwritten before the second layer runs); a first layer that does not take the resident-tile route
+    (32 channels) leaves the copy invalid and the second layer makes its own."""
+    Ci, H, W, Cm, Co, pad1, pad2, ns = case
+    H1, W1 = H + pad1[2] + pad1[3] - 2, W + pad1[0] + pad1[1] - 2
+    H2, W2 = H1 + pad2[2] + pad2[3] - 2, W1 + pad2[0] + pad2[1] - 2
+    x = (torch.rand(ns, Ci, H, W, device="cuda") - 0.5).half()
+    w1 = ((torch.rand(Cm, Ci, 3, 3, device="cuda") - 0.5) * 0.2).half()
+    w2 = ((torch.rand(Co, Cm, 3, 3, device="cuda") - 0.5) * 0.2).half()
+    dy2 = (torch.rand(ns, Co, H2, W2, device="cuda") - 0.5).half()
+    gpu.ptl_set_gemm_path(5)
+    try:
+        # plain calls
+        y1, y2, dw2 = torch.full((ns, Cm, H1, W1), 3.0, device="cuda").half(), torch.full_like(dy2, 3), torch.full_like(w2, 3)
+        a1, k1 = hp.conv2d_args(pkg, x, None, w1, None, y1, None, Ci, H, W, Cm, 3, 3, H1, W1, pad1, (1, 1))
+        a2, k2 = hp.conv2d_args(pkg, y1, None, w2, dw2, y2, dy2, Cm, H1, W1, Co, 3, 3, H2, W2, pad2, (1, 1))
+        pkg.call("ptl_conv2d_fp16_fw_batched", a1, ns)
+        pkg.call("ptl_conv2d_fp16_fw_batched", a2, ns)
+        pkg.call("ptl_conv2d_fp16_wg_batched", a2, ns)
+        gpu.ptl_sync()
+        # the same two layers with the copy handed on
+        z1, z2, ew2 = torch.full_like(y1, 5), torch.full_like(dy2, 5), torch.full_like(w2, 5)
+        b1, k3 = hp.conv2d_args(pkg, x, None, w1, None, z1, None, Ci, H, W, Cm, 3, 3, H1, W1, pad1, (1, 1))
+        b2, k4 = hp.conv2d_args(pkg, z1, None, w2, ew2, z2, dy2, Cm, H1, W1, Co, 3, 3, H2, W2, pad2, (1, 1))
+        nbytes = gpu.ptl_conv2d_fp16_cache_bytes(ctypes.byref(b2), ns)
+        assert nbytes > 0
+        buf = torch.full((nbytes,), 0x3c, dtype=torch.uint8, device="cuda")
+        c = pkg.ConvCache()
+        c.buf, c.bytes = buf.data_ptr(), nbytes
+        assert gpu.ptl_conv2d_fp16_cache_prepare(ctypes.byref(b2), ns, ctypes.byref(c)) == 0
+        assert gpu.ptl_conv2d_fp16_fw_batched_chained(ctypes.byref(b1), ns, None, ctypes.byref(c)) == 0
+        handed_on = Ci % 64 == 0
+        assert c.valid == (1 if handed_on else 0)
+        gpu.ptl_sync()
+        assert torch.equal(z1, y1)
+        if handed_on:
+            # the copy is the second layer's padded, blocked input: [Cm/8][ns][Hp][Wp][8] with zero halo
+            Hp, Wp = H1 + max(pad2[2], pad2[3]), W1 + max(pad2[0], pad2[1])
+            blk = buf[:Cm // 8 * ns * Hp * Wp * 16].view(torch.float16).view(Cm // 8, ns, Hp, Wp, 8)
+            want = torch.zeros_like(blk)
+            want[:, :, pad2[2]:pad2[2] + H1, pad2[0]:pad2[0] + W1, :] = y1.view(ns, Cm // 8, 8, H1, W1).permute(1, 0, 3, 4, 2)
+            assert torch.equal(blk, want)
+            assert int(buf[Cm // 8 * ns * Hp * Wp * 16:].max()) == 0
+            z1.fill_(7)  # what the second layer must NOT read
+        assert gpu.ptl_conv2d_fp16_fw_batched_chained(ctypes.byref(b2), ns, ctypes.byref(c), None) == 0
+        assert gpu.ptl_last_conv_resident() == 1
+        assert c.valid == 1  # (handed on, or filled by this call)
+        assert gpu.ptl_conv2d_fp16_wg_batched_cached(ctypes.byref(b2), ns, ctypes.byref(c)) == 0
+        gpu.ptl_sync()
+        assert torch.equal(z2, y2)
+        if handed_on and gpu.ptl_last_conv_resident() == 1:  # (the weight-gradient route that reads the copy)
+            assert torch.equal(ew2, dw2)
+        elif not handed_on:
+            assert torch.equal(ew2, dw2)
+        # a cache of another geometry is not read
+        if handed_on:
+            z1.copy_(y1)
+            c.geometry[2] += 1
+            z3 = torch.full_like(dy2, 5)
+            b3, k5 = hp.conv2d_args(pkg, z1, None, w2, None, z3, None, Cm, H1, W1, Co, 3, 3, H2, W2, pad2, (1, 1))
+            buf.fill_(0x3c)
+            assert gpu.ptl_conv2d_fp16_fw_batched_chained(ctypes.byref(b3), ns, ctypes.byref(c), None) == 0
+            gpu.ptl_sync()
+            assert torch.equal(z3, y2)
+        # a reader that would not use a copy: prepare says so
+        small = torch.zeros(ns, 32, 8, 8, device="cuda").half()
+        ws = torch.zeros(64, 32, 3, 3, device="cuda").half()
+        ys = torch.zeros(ns, 64, 8, 8, device="cuda").half()
+        a5, k6 = hp.conv2d_args(pkg, small, None, ws, None, ys, None, 32, 8, 8, 64, 3, 3, 8, 8, (1, 1, 1, 1), (1, 1))
+        assert gpu.ptl_conv2d_fp16_cache_prepare(ctypes.byref(a5), ns, ctypes.byref(c)) == 1
+    finally:
+        gpu.ptl_set_gemm_path(0)
+
+
 @pytest.mark.parametrize("case", [(64, 14, 14, 64, (1, 1, 1, 1), 12), (128, 9, 11, 64, (0, 2, 1, 1), 20),
                                   (64, 28, 28, 128, (1, 1, 1, 1), 5), (32, 16, 16, 64, (1, 1, 1, 1), 8)])
 def test_conv2d_forward_leaves_its_blocked_input_for_the_gradients(pkg, gpu, case):
