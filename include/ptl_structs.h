@@ -686,6 +686,8 @@ struct ptl_conv_cache {
     size_t bytes;
     int valid;       /* 1: buf holds the copy described by geometry */
     int geometry[6]; /* batch, channels, padded height and width, top and left padding */
+    int relu;        /* set by the caller, read by ptl_conv2d_fp16_fw_batched_chained when it writes this cache as the
+                        copy of its OUTPUT: 1 = write max(output, 0), for a reader that sits behind a ReLU */
 };
 
 /* No counterpart in the reference: the weight gradients of several small Conv2D layers completed by one launch.

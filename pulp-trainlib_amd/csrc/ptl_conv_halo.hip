@@ -53,6 +53,7 @@ struct HaloArgs {
     half_t *yblk;           // [Cout/8][yb_P] chunks of eight filters, nullptr: no such copy
     unsigned yb_P;          // chunks per block of eight filters: batch * yb_Hp * yb_Wp
     int yb_Hp, yb_Wp, yb_padU, yb_padL;
+    int yb_relu;            // 1: the copy holds max(output, 0)
 };
 
 template <int I, int N, typename F>
@@ -420,8 +421,16 @@ __global__ __launch_bounds__(HALO_NT) void conv_halo_kernel(const HaloArgs a) {
 #pragma unroll
                             for (int c = 0; c < 2; ++c) {
                                 const unsigned cb = (unsigned)(co0 + i * 16 + 8 * c) >> 3;
-                                *reinterpret_cast<uint4 *>(a.yblk + ((size_t)cb * a.yb_P + pos) * 8) =
-                                    make_uint4(pk[i][2 * c][0], pk[i][2 * c][1], pk[i][2 * c + 1][0], pk[i][2 * c + 1][1]);
+                                uint4 ch = make_uint4(pk[i][2 * c][0], pk[i][2 * c][1], pk[i][2 * c + 1][0], pk[i][2 * c + 1][1]);
+                                if (a.yb_relu) {
+                                    typedef _Float16 h2_t __attribute__((ext_vector_type(2)));
+                                    const h2_t z = {(_Float16)0, (_Float16)0};
+                                    auto pos2 = [&](unsigned u) {
+                                        return __builtin_bit_cast(unsigned, __builtin_elementwise_max(__builtin_bit_cast(h2_t, u), z));
+                                    };
+                                    ch = make_uint4(pos2(ch.x), pos2(ch.y), pos2(ch.z), pos2(ch.w));
+                                }
+                                *reinterpret_cast<uint4 *>(a.yblk + ((size_t)cb * a.yb_P + pos) * 8) = ch;
                             }
                     }
                 }
@@ -822,6 +831,7 @@ int conv_halo_launch(const ConvTileDesc &d, const void *xb, const void *wr, void
         a.yblk = static_cast<half_t *>(oc->buf);
         a.yb_P = (unsigned)plane;
         a.yb_Hp = oc->Hp; a.yb_Wp = oc->Wp; a.yb_padU = oc->padU; a.yb_padL = oc->padL;
+        a.yb_relu = oc->relu;
     }
     const int bn = d.Cout % 128 == 0 ? 128 : d.Cout % 64 == 0 ? 64 : 32;
     a.ct_count = d.Cout / bn;

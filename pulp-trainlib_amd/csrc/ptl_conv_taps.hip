@@ -267,6 +267,7 @@ int conv_taps(const ConvTileDesc &d, const void *X, const void *Wt, void *Y, con
             out->bytes >= ((size_t)(d.Cout / 8) * d.batch * out->geometry[2] * out->geometry[3] + (size_t)conv_halo_margin()) * 16) {
             oc.buf = out->buf;
             oc.Hp = out->geometry[2]; oc.Wp = out->geometry[3]; oc.padU = out->geometry[4]; oc.padL = out->geometry[5];
+            oc.relu = out->relu != 0;
         }
         int rc = conv_halo_launch(d, xb, wr, Y, Hp, Wp, 0, oc.buf ? &oc : nullptr);
         if (rc == -1 && oc.buf) {  // (the copy does not fit this layer's output: the layer without it)

@@ -127,6 +127,7 @@ long long conv_halo_margin();
 struct HaloOutCopy {
     void *buf;
     int Hp, Wp, padU, padL;
+    int relu;  // 1: the copy holds max(output, 0)
 };
 int conv_halo_launch(const ConvTileDesc &d, const void *xb, const void *wr, void *Y, int Hp, int Wp,
                      long long pstride = 0, const HaloOutCopy *out_copy = nullptr);  // pstride: positions between channel blocks of xb (0: batch*Hp*Wp)

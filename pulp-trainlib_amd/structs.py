@@ -166,7 +166,7 @@ class BatchNormArgs(C.Structure):
 
 class ConvCache(C.Structure):
     """struct ptl_conv_cache: the caller-owned copy of a layer's blocked input shared by ptl_conv2d_fp16_*_cached."""
-    _fields_ = [("buf", P), ("bytes", C.c_size_t), ("valid", I), ("geometry", I * 6)]
+    _fields_ = [("buf", P), ("bytes", C.c_size_t), ("valid", I), ("geometry", I * 6), ("relu", I)]
 
 
 class WgBatch(C.Structure):

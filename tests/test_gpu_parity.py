@@ -267,7 +267,8 @@ def test_conv2d_layers_in_a_row_hand_the_blocked_copy_on(pkg, gpu, case):
     channel-blocked copy the next layer reads; the next layer's forward and weight-gradient calls take that copy
     instead of making one.  Same bits as the plain calls everywhere; the copy really is what is read (the tensor
     itself is overwritten before the second layer runs); a first layer that does not take the resident-tile route
-    (32 channels) leaves the copy invalid and the second layer makes its own."""
+    (32 channels) leaves the copy invalid and the second layer makes its own; with `relu` set the copy is the blocked
+    form of the rectified output, for a second layer behind a ReLU."""
     Ci, H, W, Cm, Co, pad1, pad2, ns = case
     H1, W1 = H + pad1[2] + pad1[3] - 2, W + pad1[0] + pad1[1] - 2
     H2, W2 = H1 + pad2[2] + pad2[3] - 2, W1 + pad2[0] + pad2[1] - 2
@@ -329,6 +330,33 @@ def test_conv2d_layers_in_a_row_hand_the_blocked_copy_on(pkg, gpu, case):
             assert gpu.ptl_conv2d_fp16_fw_batched_chained(ctypes.byref(b3), ns, ctypes.byref(c), None) == 0
             gpu.ptl_sync()
             assert torch.equal(z3, y2)
+        # behind a ReLU: the copy holds max(output, 0), i.e. the blocked form of the activation's output
+        if handed_on:
+            c2 = pkg.ConvCache()
+            c2.buf, c2.bytes, c2.relu = buf.data_ptr(), nbytes, 1
+            r1 = torch.relu(y1)
+            z4, z5 = torch.full_like(y1, 5), torch.full_like(dy2, 5)
+            b4, k7 = hp.conv2d_args(pkg, x, None, w1, None, z4, None, Ci, H, W, Cm, 3, 3, H1, W1, pad1, (1, 1))
+            b5, k8 = hp.conv2d_args(pkg, r1, None, w2, None, z5, None, Cm, H1, W1, Co, 3, 3, H2, W2, pad2, (1, 1))
+            y5 = torch.full_like(dy2, 3)
+            a5r, k9 = hp.conv2d_args(pkg, r1, None, w2, None, y5, None, Cm, H1, W1, Co, 3, 3, H2, W2, pad2, (1, 1))
+            pkg.call("ptl_conv2d_fp16_fw_batched", a5r, ns)
+            assert gpu.ptl_conv2d_fp16_cache_prepare(ctypes.byref(b5), ns, ctypes.byref(c2)) == 0
+            assert gpu.ptl_conv2d_fp16_fw_batched_chained(ctypes.byref(b4), ns, None, ctypes.byref(c2)) == 0
+            assert c2.valid == 1
+            gpu.ptl_sync()
+            assert torch.equal(z4, y1)  # the layer's own output is not rectified
+            Hp, Wp = H1 + max(pad2[2], pad2[3]), W1 + max(pad2[0], pad2[1])
+            blk = buf[:Cm // 8 * ns * Hp * Wp * 16].view(torch.float16).view(Cm // 8, ns, Hp, Wp, 8)
+            want = torch.zeros_like(blk)
+            want[:, :, pad2[2]:pad2[2] + H1, pad2[0]:pad2[0] + W1, :] = r1.view(ns, Cm // 8, 8, H1, W1).permute(1, 0, 3, 4, 2)
+            assert torch.equal(blk, want)
+            keep_r1 = r1.clone()
+            r1.fill_(7)
+            assert gpu.ptl_conv2d_fp16_fw_batched_chained(ctypes.byref(b5), ns, ctypes.byref(c2), None) == 0
+            gpu.ptl_sync()
+            assert torch.equal(z5, y5)
+            r1.copy_(keep_r1)
         # a reader that would not use a copy: prepare says so
         small = torch.zeros(ns, 32, 8, 8, device="cuda").half()
         ws = torch.zeros(64, 32, 3, 3, device="cuda").half()
