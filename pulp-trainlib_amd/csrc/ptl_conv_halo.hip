@@ -54,6 +54,12 @@ struct HaloArgs {
     unsigned yb_P;          // chunks per block of eight filters: batch * yb_Hp * yb_Wp
     int yb_Hp, yb_Wp, yb_padU, yb_padL;
     int yb_relu;            // 1: the copy holds max(output, 0)
+    // channel-major route: rows are output pixels (b, y, x < Wo) instead of padded positions (b, y, xp < Wp): no row of
+    // the product is a dropped column, and consecutive rows are consecutive pixels of the output
+    int dense;
+    unsigned m_wo;          // multiplier and shift for / Wo (see fast_div31)
+    int s_wo;
+    unsigned row_lim;       // dense: largest tile-local position a row may have (rows past the end are clamped to it)
 };
 
 template <int I, int N, typename F>
@@ -112,6 +118,7 @@ struct HaloUnit {
                       // the tile's first position); channel-minor: the tensor + the slab's byte offset in a pixel
     unsigned p0;      // position of the tile's first row in the padded grids laid end to end
     unsigned rem0;    // row of the tile's first position within its sample's rows
+    unsigned loc0;    // dense rows: padded position of the tile's first row within its sample's grid
 };
 
 // HWC = false: the input arrives zero-padded and channel-blocked (see the head of the file).
@@ -166,6 +173,12 @@ __global__ __launch_bounds__(HALO_NT) void conv_halo_kernel(const HaloArgs a) {
         const unsigned q0 = pt * HALO_BM, b0 = q0 / a.qimg;
         u.rem0 = q0 - b0 * a.qimg;
         u.p0 = q0 + b0 * a.jump;  // (the host keeps the positions, a tile's reach included, below 2^31)
+        u.loc0 = 0;
+        if (!HWC && a.dense) {
+            const unsigned y0 = u.rem0 / (unsigned)a.Wo, x0 = u.rem0 - y0 * (unsigned)a.Wo;
+            u.loc0 = y0 * (unsigned)a.Wp + x0;
+            u.p0 = b0 * HpWp + u.loc0;
+        }
         u.fb = a.wr + ((long long)ct * BN * K9 + cs * 64) * 2;
         u.hb = HWC ? a.xb + cs * 128 : a.xb + ((long long)(cs * 8 + 2 * wave) * a.P + u.p0) * 16;
         return u;
@@ -176,6 +189,15 @@ __global__ __launch_bounds__(HALO_NT) void conv_halo_kernel(const HaloArgs a) {
 #pragma unroll
         for (int j = 0; j < FN; ++j) {
             const unsigned r = (unsigned)(64 * wave + 16 * j + l16), v = u.rem0 + r;
+            if (!HWC && a.dense) {
+                // pixel (cross samples on, y, x) -> its padded position, from the tile's first one
+                unsigned cross = 0;
+                for (unsigned k = 1, lim = a.qimg; k <= a.maxcross; ++k, lim += a.qimg) cross += v >= lim ? 1u : 0u;
+                const unsigned w = v - cross * a.qimg;
+                const unsigned y = fast_div31(w, a.m_wo, a.s_wo), x = w - y * (unsigned)a.Wo;
+                row[j] = min(cross * HpWp + y * (unsigned)a.Wp + x - u.loc0, a.row_lim);
+                continue;
+            }
             unsigned skip = 0;
             for (unsigned k = 1, lim = a.qimg; k <= a.maxcross; ++k, lim += a.qimg) skip += v >= lim ? a.jump : 0u;
             row[j] = r + skip;
@@ -396,7 +418,8 @@ __global__ __launch_bounds__(HALO_NT) void conv_halo_kernel(const HaloArgs a) {
                     }
                 const unsigned q = q0 + (unsigned)(64 * wave + lane);  // (Q < 2^31 on the host)
                 const unsigned b = q / a.qimg, rem = q - b * a.qimg;
-                const unsigned yy = rem / (unsigned)a.Wp, xx = rem - yy * (unsigned)a.Wp;
+                const unsigned rw = a.dense ? (unsigned)a.Wo : (unsigned)a.Wp;  // rows of the enumeration are this wide
+                const unsigned yy = rem / rw, xx = rem - yy * rw;
                 if (q < a.Q && yy < (unsigned)a.Ho && xx < (unsigned)a.Wo) {
                     half_t *dst = a.y + ((size_t)b * a.Cout + co0) * PO + yy * (unsigned)a.Wo + xx;
 #pragma unroll
@@ -802,6 +825,8 @@ bool conv_halo_fits(const ConvTileDesc &d, int Hp, int Wp) {
            2 * Wp + 2 <= HALO_NP - HALO_BM && conv_output_fits_pads(d) && Hp >= d.Ho && Wp >= d.Wo;
 }
 
+static void magic31(unsigned d, unsigned *m, int *s);
+
 // xb: blocked, padded input with conv_halo_margin() readable chunks after the last block; wr: tap-major filters.
 int conv_halo_launch(const ConvTileDesc &d, const void *xb, const void *wr, void *Y, int Hp, int Wp, long long pstride,
                      const HaloOutCopy *oc) {
@@ -820,6 +845,21 @@ int conv_halo_launch(const ConvTileDesc &d, const void *xb, const void *wr, void
     a.qimg = (unsigned)(skip ? qs : Hp * Wp);
     a.jump = (unsigned)(skip ? (Hp - d.Ho) * Wp : 0);
     a.maxcross = (unsigned)(skip ? crossings : 0);
+    // rows = output pixels where the tile and its reach still fit: a tile's 256 pixels spread over the padded grid by
+    // Wp - Wo per row boundary and by the rows left out per sample boundary
+    for (int leave = 1; leave >= 0 && !a.dense && d.Wo >= 2; --leave) {
+        const int rows = leave ? d.Ho : Hp;  // rows of a sample in the enumeration
+        if (leave && Hp == d.Ho) continue;
+        const int qd = rows * d.Wo, cross = (HALO_BM - 1 + qd - 1) / qd;
+        const int spread = ((d.Wo + HALO_BM - 2) / d.Wo) * (Wp - d.Wo) + cross * (Hp - rows) * Wp;
+        if (HALO_BM + spread + 2 * Wp + 2 > HALO_NP) continue;
+        a.dense = 1;
+        a.qimg = (unsigned)qd;
+        a.jump = 0;
+        a.maxcross = (unsigned)cross;
+        a.row_lim = (unsigned)(HALO_NP - 2 * Wp - 3);
+        magic31((unsigned)d.Wo, &a.m_wo, &a.s_wo);
+    }
     a.Q = (unsigned)((long long)d.batch * a.qimg);
     a.batch = d.batch; a.Cin = d.Cin; a.Cout = d.Cout; a.Hp = Hp; a.Wp = Wp; a.Ho = d.Ho; a.Wo = d.Wo;
     if (oc && oc->buf) {
