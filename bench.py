@@ -271,6 +271,8 @@ TARGET_ROWS = (
      ["conv2d 256->256 28x28 k3 p1 %s N=256" % s for s in ("FW", "WG", "IG")], "frac_of_bound"),
     ("conv128_28x28_N512_FW_WG_IG_frac_of_mfma_peak",
      ["conv2d 128->128 28x28 k3 p1 %s N=512" % s for s in ("FW", "WG", "IG")], "frac_of_bound"),
+    ("conv256_28x28_N256_FW_input_copy_handed_on_frac_of_mfma_peak",
+     ["conv2d 256->256 28x28 k3 p1 FW, input copy left by the layer before N=256"], "frac_of_bound"),
     ("mm_4096x4096x4096_fp16_TFLOP/s", ["mm 4096x4096x4096 (B transposed)"], "TFLOP/s"),
     ("depthwise_64x56x56_N64_FW_WG_IG_GB/s", ["depthwise 3x3 64x56x56 %s N=64" % s for s in ("FW", "WG", "IG")], "GB/s"),
     ("pointwise_64to128_56x56_N64_FW_WG_IG_GB/s", ["pointwise 64->128 56x56 %s N=64" % s for s in ("FW", "WG", "IG")], "GB/s"),
@@ -281,9 +283,6 @@ TARGET_ROWS = (
      "samples/s"),
     ("mm_4096_fp16_random_then_zero_operands_TFLOP/s",
      ["power: mm 4096x4096x4096 (B transposed), random", "power: mm 4096x4096x4096 (B transposed), zero"], "TFLOP/s"),
-    ("mfma_32x32x16_loop_alone_random_then_zero_operands_TFLOP/s",
-     ["power: loop of v_mfma_f32_32x32x16_f16 alone, random operands, 1 wave ",
-      "power: loop of v_mfma_f32_32x32x16_f16 alone, zero operands, 1 wave "], "TFLOP/s"),
 )
 MAX_LAST_LINE = 4096
 
