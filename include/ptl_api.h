@@ -431,7 +431,8 @@ int ptl_conv2d_fp16_bw_batched_cached(const struct Conv2D_args_fp16 *a, int nsam
  * geometry; 1 if that layer would not read such a copy.  ptl_conv2d_fp16_fw_batched_chained(a, n, in, out) is the
  * forward call of a layer with `in` = the copy of ITS input (valid: read instead of copying; not valid: filled, as by
  * the _cached call; NULL: none) and `out` = a cache prepared for the layer that reads this layer's output (NULL:
- * none): out->valid says whether the copy was written - the layer must take the resident-tile route, and its output
+ * none): out->valid says whether the copy was written - the layer must take the resident-tile route and have no
+ * bias (USE_BIASES != 1: the bias is added behind the kernel that would write the copy), and its output
  * must be the reader's input tensor (same batch, channels, height and width), or, with out->relu = 1, the input of
  * the ReLU whose output the reader takes: the copy then holds max(output, 0).  The weight-gradient calls of the
  * reader take the same cache through the _cached entry points.  The copies belong to the caller; a call that

@@ -357,6 +357,18 @@ def test_conv2d_layers_in_a_row_hand_the_blocked_copy_on(pkg, gpu, case):
             gpu.ptl_sync()
             assert torch.equal(z5, y5)
             r1.copy_(keep_r1)
+        # a producing layer with a bias writes no copy (the bias is added behind its kernel)
+        if handed_on:
+            bias = (torch.rand(Cm, device="cuda") - 0.5).half()
+            z6 = torch.full_like(y1, 5)
+            b6, k10 = hp.conv2d_args(pkg, x, None, w1, None, z6, None, Ci, H, W, Cm, 3, 3, H1, W1, pad1, (1, 1), bias=bias)
+            c3 = pkg.ConvCache()
+            c3.buf, c3.bytes = buf.data_ptr(), nbytes
+            assert gpu.ptl_conv2d_fp16_cache_prepare(ctypes.byref(b2), ns, ctypes.byref(c3)) == 0
+            assert gpu.ptl_conv2d_fp16_fw_batched_chained(ctypes.byref(b6), ns, None, ctypes.byref(c3)) == 0
+            gpu.ptl_sync()
+            assert c3.valid == 0
+            assert float((z6.float() - (y1.float() + bias.float().view(1, Cm, 1, 1))).abs().max()) <= 2e-2
         # a reader that would not use a copy: prepare says so
         small = torch.zeros(ns, 32, 8, 8, device="cuda").half()
         ws = torch.zeros(64, 32, 3, 3, device="cuda").half()
