@@ -5,11 +5,13 @@
 // tap-major, wr[co][tap][c].  Rows of the product are PADDED POSITIONS, not output pixels: the value of tap
 // (ky, kx) for the row at position p is the chunk at p + ky*Wp + kx, so every tap is the same LDS tile read at
 // a constant shift and an input element is fetched from memory once per (tile, 64-channel slab) instead of
-// once per tap.  Rows whose position is not an output pixel are computed and dropped: always the last KW-1
-// columns of a padded row (Wp/Wo - 1 extra work); the last KH-1 rows of every padded grid are left out of the
-// row enumeration when the tile still fits (small images: rows are numbered q = (b, y < Ho, xp) and a lane's
-// position is q plus (Hp - Ho)*Wp per sample boundary between the tile's first row and its own), else they
-// are computed and dropped as well.
+// once per tap.  Rows whose position is not an output pixel are computed and dropped: the last KW-1 columns of a
+// padded row (Wp/Wo - 1 extra work); the last KH-1 rows of every padded grid are left out of the row enumeration
+// when the tile still fits (small images: rows are numbered q = (b, y < Ho, xp) and a lane's position is q plus
+// (Hp - Ho)*Wp per sample boundary between the tile's first row and its own), else they are computed and dropped
+// as well.  On narrow images, where the dropped columns are at least 1/32 of the rows, the channel-major route
+// numbers its rows by OUTPUT PIXEL instead, q = (b, y, x < Wo): a lane works out its tile-local position from its
+// pixel once per unit (the tile spreads over the padded grid by Wp - Wo per row boundary), nothing else changes.
 //
 // A workgroup (4 waves, one per SIMD) is persistent: it walks tiles of 256 rows x BN filters.  Its work is a
 // sequence of units = (tile, slab of 64 channels); a unit needs the positions of its tile plus 2*Wp + 2 for 8
