@@ -136,6 +136,30 @@ def test_no_device_fails_loudly(pkg):
     assert np.all(C == 0)
 
 
+def test_cache_prepare_rejects_before_any_device_work(pkg):
+    """ptl_conv2d_fp16_cache_prepare: no cache, a layer that reads no blocked copy, a buffer that is too small - all
+    reported as argument errors (1) without touching a device."""
+    lib = pkg.load()
+    x = np.zeros((64, 8, 8), np.float16)
+    w = np.zeros((64, 64, 3, 3), np.float16)
+    y = np.zeros((64, 8, 8), np.float16)
+    a, keep = hp.conv2d_args(pkg, x, None, w, None, y, None, 64, 8, 8, 64, 3, 3, 8, 8, (1, 1, 1, 1))
+    assert lib.ptl_conv2d_fp16_cache_prepare(ctypes.byref(a), 4, None) == 1
+    need = lib.ptl_conv2d_fp16_cache_bytes(ctypes.byref(a), 4)
+    assert need == (64 // 8 * 4 * 9 * 9 + 256 + 384) * 16  # blocked, padded copy of four samples + the kernel's reach
+    c = pkg.ConvCache()
+    c.valid = 1
+    c.buf, c.bytes = 16, need - 16
+    assert lib.ptl_conv2d_fp16_cache_prepare(ctypes.byref(a), 4, ctypes.byref(c)) == 1
+    assert c.valid == 0 and b"16-byte aligned" in lib.ptl_last_error()
+    x32 = np.zeros((32, 8, 8), np.float16)
+    w32 = np.zeros((64, 32, 3, 3), np.float16)
+    a32, keep32 = hp.conv2d_args(pkg, x32, None, w32, None, y, None, 32, 8, 8, 64, 3, 3, 8, 8, (1, 1, 1, 1))
+    c.bytes = 1 << 20
+    assert lib.ptl_conv2d_fp16_cache_prepare(ctypes.byref(a32), 4, ctypes.byref(c)) == 1
+    assert b"does not read a blocked copy" in lib.ptl_last_error()
+
+
 def test_product_does_not_reference_the_oracle():
     """Nothing under the package or include/ names the oracle."""
     for base in ("pulp-trainlib_amd", "include"):
