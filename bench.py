@@ -697,6 +697,40 @@ def detail_table(pkg, lib, hp, to_dev, timed, check, torch, dev):
                                                                                      ctypes.byref(oc))), 10)
                     add("conv2d %d->%d %dx%d k3 p1 FW, copy in and copy out N=%d" % (Ci, Co, H, H, ns), dt, ms, flops, nb)
                     del nxt
+                    # two such layers in a row, forward and backward: plain calls against the copies handed on and kept
+                    if (ns, Ci, H) in ((256, 256, 28), (512, 128, 28)):
+                        y2, dx2, dw2 = torch.zeros_like(dy), torch.zeros_like(x), torch.zeros_like(w)
+                        a2, keep2 = hp.conv2d_args(pkg, y, dx2, w, dw2, y2, dy, Ci, H, H, Co, K, K, H, H, (1, 1, 1, 1))
+                        a1, keep1 = hp.conv2d_args(pkg, x, dx, w, dw, y, dx2, Ci, H, H, Co, K, K, H, H, (1, 1, 1, 1))
+                        r1, r2 = ctypes.byref(a1), ctypes.byref(a2)
+
+                        def plain_pair():
+                            check(lib.ptl_conv2d_fp16_fw_batched(r1, ns))
+                            check(lib.ptl_conv2d_fp16_fw_batched(r2, ns))
+                            check(lib.ptl_conv2d_fp16_bw_batched(r2, ns))
+                            check(lib.ptl_conv2d_fp16_bw_batched(r1, ns))
+
+                        k1 = torch.empty(nbytes, dtype=torch.uint8, device=dev)
+                        k2 = torch.empty(nbytes, dtype=torch.uint8, device=dev)
+                        c1, c2 = pkg.ConvCache(), pkg.ConvCache()
+                        c1.buf, c1.bytes = k1.data_ptr(), nbytes
+                        c2.buf, c2.bytes = k2.data_ptr(), nbytes
+                        check(lib.ptl_conv2d_fp16_cache_prepare(r2, ns, ctypes.byref(c2)))
+
+                        def chained_pair():
+                            c1.valid = 0
+                            check(lib.ptl_conv2d_fp16_fw_batched_chained(r1, ns, ctypes.byref(c1), ctypes.byref(c2)))
+                            check(lib.ptl_conv2d_fp16_fw_batched_chained(r2, ns, ctypes.byref(c2), None))
+                            check(lib.ptl_conv2d_fp16_bw_batched_cached(r2, ns, ctypes.byref(c2)))
+                            check(lib.ptl_conv2d_fp16_bw_batched_cached(r1, ns, ctypes.byref(c1)))
+
+                        ms = timed(plain_pair, 5)
+                        add("conv2d %d->%d %dx%d k3 p1 two layers in a row, FW + WG + IG, plain calls N=%d" % (Ci, Co, H, H, ns),
+                            dt, ms, 6 * flops, 6 * nb)
+                        ms = timed(chained_pair, 5)
+                        add("conv2d %d->%d %dx%d k3 p1 two layers in a row, FW + WG + IG, copies handed on and kept N=%d"
+                            % (Ci, Co, H, H, ns), dt, ms, 6 * flops, 6 * nb)
+                        del k1, k2, y2, dx2, dw2
             del kept
         del x, w, dy, y, dx, dw
 
