@@ -286,25 +286,26 @@ __device__ inline void mfma4(mh_f32x16 &acc, const float4 &a, const float4 &b) {
     acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a.w, b.w, acc, 0, 0, 0);
 }
 
-// NB row blocks of 32 per workgroup share one B panel; each block has its own four waves.
+// NB row blocks of 32 per workgroup share one B panel; each block has its own four waves.  (bx, by, bz): the
+// workgroup's place in the product's grid of (column blocks, row blocks, outputs x samples or sample groups).
 template <bool A_KMAJ, bool B_KMAJ, int NB>
-__global__ __launch_bounds__(ATT_NT * NB) void panel_gemm_kernel(PanelArgs a) {
+__device__ __forceinline__ void panel_gemm_body(const PanelArgs &a, unsigned bx, unsigned by, unsigned bz) {
     extern __shared__ __attribute__((aligned(16))) float pg_lds[];
     constexpr int NW = 4 * NB, NT = ATT_NT * NB;
     float *Bs = pg_lds, *As = pg_lds + PG_PANEL;  // As: NB panels
     const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int l32 = lane & 31, half = lane >> 5;
     const int nb = wave >> 2, ks = wave & 3;
-    const int m0 = blockIdx.x * 32, n0 = blockIdx.y * (32 * NB);
+    const int m0 = (int)bx * 32, n0 = (int)by * (32 * NB);
     int o, b_first, b_count, grp = 0;
     if (a.sum_samples) {
-        o = blockIdx.z / a.groups;
-        grp = blockIdx.z % a.groups;
+        o = (int)bz / a.groups;
+        grp = (int)bz % a.groups;
         b_first = grp * a.spg;
         b_count = min(a.spg, a.ns - b_first);
     } else {
-        o = blockIdx.z / a.ns;
-        b_first = blockIdx.z % a.ns;
+        o = (int)bz / a.ns;
+        b_first = (int)bz % a.ns;
         b_count = 1;
     }
     mh_f32x16 acc = {0};
@@ -366,11 +367,44 @@ __global__ __launch_bounds__(ATT_NT * NB) void panel_gemm_kernel(PanelArgs a) {
     }
 }
 
+template <bool A_KMAJ, bool B_KMAJ, int NB>
+__global__ __launch_bounds__(ATT_NT * NB) void panel_gemm_kernel(PanelArgs a) {
+    panel_gemm_body<A_KMAJ, B_KMAJ, NB>(a, blockIdx.x, blockIdx.y, blockIdx.z);
+}
+
+// Two independent products in one launch (both read what the launch before them wrote, neither reads the other):
+// the first n0 workgroups are the first product's grid (gx0 x gy0 x gz0, x fastest), the rest the second's.  The
+// block is as large as the larger of the two needs; the waves a product does not use leave at once.
+struct PanelPairGrid {
+    unsigned n0, gx0, gy0, gx1, gy1;
+    int nb0, nb1;
+};
+
+template <bool AK0, bool BK0, bool AK1, bool BK1>
+__global__ __launch_bounds__(ATT_NT * 2) void panel_gemm_pair_kernel(PanelArgs a, PanelArgs b, PanelPairGrid g) {
+    unsigned id = blockIdx.x;
+    if (id < g.n0) {
+        if ((int)threadIdx.x >= ATT_NT * g.nb0) return;
+        const unsigned bx = id % g.gx0, r = id / g.gx0;
+        if (g.nb0 == 2)
+            panel_gemm_body<AK0, BK0, 2>(a, bx, r % g.gy0, r / g.gy0);
+        else
+            panel_gemm_body<AK0, BK0, 1>(a, bx, r % g.gy0, r / g.gy0);
+    } else {
+        id -= g.n0;
+        if ((int)threadIdx.x >= ATT_NT * g.nb1) return;
+        const unsigned bx = id % g.gx1, r = id / g.gx1;
+        if (g.nb1 == 2)
+            panel_gemm_body<AK1, BK1, 2>(b, bx, r % g.gy1, r / g.gy1);
+        else
+            panel_gemm_body<AK1, BK1, 1>(b, bx, r % g.gy1, r / g.gy1);
+    }
+}
+
 // C_o[i] = sum over groups of part[o][g][i]   (+ what C holds when accumulate)
-__global__ __launch_bounds__(256) void panel_reduce_kernel(PanelArgs a) {
+__device__ __forceinline__ void panel_reduce_body(const PanelArgs &a, int o) {
     const size_t nm = (size_t)a.N * a.M, i = (size_t)blockIdx.x * 256 + threadIdx.x;
     if (i >= nm) return;
-    const int o = blockIdx.y;
     const float *p = a.part + (size_t)o * a.groups * nm + i;
     // eight loads in flight at a time (a serial walk is one trip to memory per group); the sums are added in
     // the order of the groups either way
@@ -386,6 +420,16 @@ __global__ __launch_bounds__(256) void panel_reduce_kernel(PanelArgs a) {
     for (; g < a.groups; ++g) s += p[(size_t)g * nm];
     float *dst = a.C[o] + (i / a.M) * a.c_n + (i % a.M);
     *dst = a.accumulate ? *dst + s : s;
+}
+
+__global__ __launch_bounds__(256) void panel_reduce_kernel(PanelArgs a) { panel_reduce_body(a, blockIdx.y); }
+
+// ... of two products at once: blockIdx.y runs over the outputs of the first, then of the second
+__global__ __launch_bounds__(256) void panel_reduce_pair_kernel(PanelArgs a, PanelArgs b) {
+    if ((int)blockIdx.y < a.nout)
+        panel_reduce_body(a, blockIdx.y);
+    else
+        panel_reduce_body(b, (int)blockIdx.y - a.nout);
 }
 
 struct AttnArgs {
@@ -970,7 +1014,17 @@ static size_t panel_part_floats(int nout, int N, int M, int ns) {
 
 // Launches the panel product; `p` carries operands, strides and sizes, this fills in the rest.  In gradient
 // mode (sum_samples) the partial sums of the sample groups go to `part` and a second kernel adds them.
-static int launch_panel(PanelArgs &p, float *part) {
+// What a launch of the panel product needs besides its arguments.
+struct PanelPlan {
+    bool ak, bk;
+    int nb;
+    dim3 grid;
+    size_t lds;
+};
+
+// Fills in the fields of `p` the caller leaves open (zero page, sample groups, partial sums) and works out the
+// launch.  0, or the error code.
+static int panel_plan(PanelArgs &p, float *part, PanelPlan &pl) {
     State &st = state();
     p.zero = static_cast<const float *>(st.zeros);
     if (!p.zero) return 2;
@@ -978,7 +1032,8 @@ static int launch_panel(PanelArgs &p, float *part) {
         set_error("panel product: operand without a unit stride");
         return 1;
     }
-    const bool ak = p.a_k == 1, bk = p.b_k == 1;
+    pl.ak = p.a_k == 1;
+    pl.bk = p.b_k == 1;
     p.groups = 1;
     p.spg = p.ns;
     p.part = nullptr;
@@ -995,39 +1050,99 @@ static int launch_panel(PanelArgs &p, float *part) {
     // queue up behind each other on the CUs.
     const size_t zdim = p.sum_samples ? (size_t)p.nout * p.groups : (size_t)p.nout * p.ns;
     const size_t single = (size_t)((p.M + 31) / 32) * ((p.N + 31) / 32) * zdim;
-    const int nb = (p.N > 32 && single > (size_t)3 * st.num_cu) ? 2 : 1;
+    pl.nb = (p.N > 32 && single > (size_t)3 * st.num_cu) ? 2 : 1;
+    pl.lds = (size_t)(1 + pl.nb) * PG_PANEL * sizeof(float);  // 52 KB or 78 KB
+    pl.grid = dim3((p.M + 31) / 32, (p.N + 32 * pl.nb - 1) / (32 * pl.nb), (unsigned)zdim);
+    if (pl.grid.y > 65535u || zdim > 65535u) {
+        set_error("panel product: grid too large");
+        return 1;
+    }
+    return 0;
+}
+
+static int launch_panel_reduce(PanelArgs &p) {
+    if (p.groups <= 1) return 0;
+    hipLaunchKernelGGL(panel_reduce_kernel, dim3((unsigned)(((size_t)p.N * p.M + 255) / 256), p.nout), dim3(256), 0,
+                       state().stream, p);
+    p.groups = 0;  // (added up: a later call finds nothing to do)
+    return hip_ok(hipGetLastError(), "panel reduce launch") ? 0 : 2;
+}
+
+// The additions of two products' sample groups in one launch.
+static int launch_panel_reduce_pair(PanelArgs &p0, PanelArgs &p1) {
+    if (p0.groups <= 1) return launch_panel_reduce(p1);
+    if (p1.groups <= 1) return launch_panel_reduce(p0);
+    const size_t nm0 = (size_t)p0.N * p0.M, nm1 = (size_t)p1.N * p1.M, nm = nm0 > nm1 ? nm0 : nm1;
+    hipLaunchKernelGGL(panel_reduce_pair_kernel, dim3((unsigned)((nm + 255) / 256), p0.nout + p1.nout), dim3(256), 0,
+                       state().stream, p0, p1);
+    p0.groups = p1.groups = 0;
+    return hip_ok(hipGetLastError(), "panel reduce launch") ? 0 : 2;
+}
+
+// Launches the panel product; `p` carries operands, strides and sizes, this fills in the rest.  In gradient
+// mode (sum_samples) the partial sums of the sample groups go to `part` and a second kernel adds them.
+static int launch_panel(PanelArgs &p, float *part) {
+    State &st = state();
+    PanelPlan pl;
+    if (int rc = panel_plan(p, part, pl)) return rc;
+    const bool ak = pl.ak, bk = pl.bk;
     void (*kern)(PanelArgs);
-    if (nb == 2)
+    if (pl.nb == 2)
         kern = ak ? (bk ? panel_gemm_kernel<true, true, 2> : panel_gemm_kernel<true, false, 2>)
                   : (bk ? panel_gemm_kernel<false, true, 2> : panel_gemm_kernel<false, false, 2>);
     else
         kern = ak ? (bk ? panel_gemm_kernel<true, true, 1> : panel_gemm_kernel<true, false, 1>)
                   : (bk ? panel_gemm_kernel<false, true, 1> : panel_gemm_kernel<false, false, 1>);
-    const size_t lds = (size_t)(1 + nb) * PG_PANEL * sizeof(float);  // 52 KB or 78 KB
-    if (nb == 2) {
+    if (pl.nb == 2) {
         static bool attr_set[4] = {false, false, false, false};
         const int which = (ak ? 2 : 0) + (bk ? 1 : 0);
         if (!attr_set[which]) {
             if (!hip_ok(hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
-                                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds),
+                                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)pl.lds),
                         "hipFuncSetAttribute"))
                 return 2;
             attr_set[which] = true;
         }
     }
-    dim3 grid((p.M + 31) / 32, (p.N + 32 * nb - 1) / (32 * nb), (unsigned)zdim);
-    if (grid.y > 65535u || grid.z > 65535u) {
-        set_error("panel product: grid too large");
-        return 1;
-    }
-    hipLaunchKernelGGL(kern, grid, dim3(ATT_NT * nb), lds, st.stream, p);
+    hipLaunchKernelGGL(kern, pl.grid, dim3(ATT_NT * pl.nb), pl.lds, st.stream, p);
     if (!hip_ok(hipGetLastError(), "panel product launch")) return 2;
-    if (p.groups > 1) {
-        hipLaunchKernelGGL(panel_reduce_kernel, dim3((unsigned)(((size_t)p.N * p.M + 255) / 256), p.nout), dim3(256),
-                           0, st.stream, p);
-        if (!hip_ok(hipGetLastError(), "panel reduce launch")) return 2;
+    return launch_panel_reduce(p);
+}
+
+// Two independent panel products in one launch (the two the backward pass has twice: the gradient of the output
+// weights with the gradient of the attention map, and the gradients of the input weights with the gradient of the
+// input), each followed by the addition of its sample groups where it has any.  `PAIR` names the orientations.
+template <bool AK0, bool BK0, bool AK1, bool BK1>
+static int launch_panel_pair(PanelArgs &p0, float *part0, PanelArgs &p1, float *part1, bool add_now = true) {
+    State &st = state();
+    PanelPlan l0, l1;
+    if (int rc = panel_plan(p0, part0, l0)) return rc;
+    if (int rc = panel_plan(p1, part1, l1)) return rc;
+    const size_t n0 = (size_t)l0.grid.x * l0.grid.y * l0.grid.z, n1 = (size_t)l1.grid.x * l1.grid.y * l1.grid.z;
+    if (l0.ak != AK0 || l0.bk != BK0 || l1.ak != AK1 || l1.bk != BK1 || n0 + n1 >= ((size_t)1 << 31) ||
+        st.gemm_path == 7) {  // (not this pair, or one product at a time asked for)
+        if (int rc = launch_panel(p0, part0)) return rc;
+        return launch_panel(p1, part1);
     }
-    return 0;
+    void (*kern)(PanelArgs, PanelArgs, PanelPairGrid) = panel_gemm_pair_kernel<AK0, BK0, AK1, BK1>;
+    const size_t lds = l0.lds > l1.lds ? l0.lds : l1.lds;
+    static bool attr_set = false;
+    if (!attr_set) {
+        if (!hip_ok(hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                        (int)(3 * PG_PANEL * sizeof(float))),
+                    "hipFuncSetAttribute"))
+            return 2;
+        attr_set = true;
+    }
+    PanelPairGrid g;
+    g.n0 = (unsigned)n0;
+    g.gx0 = l0.grid.x; g.gy0 = l0.grid.y;
+    g.gx1 = l1.grid.x; g.gy1 = l1.grid.y;
+    g.nb0 = l0.nb; g.nb1 = l1.nb;
+    const int nbmax = l0.nb > l1.nb ? l0.nb : l1.nb;
+    hipLaunchKernelGGL(kern, dim3((unsigned)(n0 + n1)), dim3(ATT_NT * nbmax), lds, st.stream, p0, p1, g);
+    if (!hip_ok(hipGetLastError(), "panel product pair launch")) return 2;
+    return add_now ? launch_panel_reduce_pair(p0, p1) : 0;  // (else the caller adds the groups up later)
 }
 
 // out[b][N x L] = Wt(N x K) . act[b][K x L]: a weight matrix with element (n,k) at n*a_n + k*a_k against a
@@ -1175,25 +1290,22 @@ static int mhsa_bw(const Mhsa_args *a, int ns, const char *fn) {
     float *dP = sg.out(a->softmax_buffer->diff, pe);
     if (sg.failed()) return 2;
     const size_t p1 = panel_part_floats(1, E, F, ns), p3 = panel_part_floats(3, F, E, ns);
-    float *rs = static_cast<float *>(scratch((rows + (p1 > p3 ? p1 : p3)) * sizeof(float)));
+    float *rs = static_cast<float *>(scratch((rows + p1 + p3) * sizeof(float)));
     if (!rs) return 2;
-    float *part = rs + rows;
+    float *part_o = rs + rows, *part_i = part_o + p1;  // sample-group sums of the output / the input weights' gradients
     int rc = 0;
+    // dWout[E x F] = sum over samples of dY . att^T (:742-760) and datt[F x L] = Wout^T . dY (:816-834), one launch;
+    // the sample groups of dWout are added up at the end, together with those of the input weights' gradients
+    PanelArgs pwo = acts_times_acts(E, F, L, ns);
     {
-        // dWout[E x F] = sum over samples of dY . att^T (:742-760)
-        PanelArgs p = acts_times_acts(E, F, L, ns);
-        p.A[0] = dY;
-        p.B[0] = att;
-        p.C[0] = dWo;
-        rc = launch_panel(p, part);
-    }
-    if (rc == 0) {
-        // datt[F x L] = Wout^T . dY (:816-834)
-        PanelArgs p = weights_times_acts(F, E, L, ns, 1, F);
-        p.A[0] = Wo;
-        p.B[0] = dY;
-        p.C[0] = datt;
-        rc = launch_panel(p, nullptr);
+        pwo.A[0] = dY;
+        pwo.B[0] = att;
+        pwo.C[0] = dWo;
+        PanelArgs q = weights_times_acts(F, E, L, ns, 1, F);
+        q.A[0] = Wo;
+        q.B[0] = dY;
+        q.C[0] = datt;
+        rc = launch_panel_pair<true, true, false, false>(pwo, part_o, q, nullptr, false);
     }
     AttnArgs t = {};
     t.q = QKV[0];
@@ -1222,7 +1334,8 @@ static int mhsa_bw(const Mhsa_args *a, int ns, const char *fn) {
         rc = launch_attn_any(2, t, ns);
     }
     if (rc == 0) {
-        // dW_{q,k,v}[F x E] = sum over samples of d{q,k,v} . X^T, one launch (:1425-1560)
+        // dW_{q,k,v}[F x E] = sum over samples of d{q,k,v} . X^T (:1425-1560) and
+        // dX[E x L] += W_q . dq + W_k . dk + W_v . dv (:1589-1745), one launch
         PanelArgs p = acts_times_acts(F, E, L, ns);
         p.nout = 3;
         for (int j = 0; j < 3; ++j) {
@@ -1230,19 +1343,16 @@ static int mhsa_bw(const Mhsa_args *a, int ns, const char *fn) {
             p.B[j] = X;
             p.C[j] = dW[j];
         }
-        rc = launch_panel(p, part);
-    }
-    if (rc == 0) {
-        // dX[E x L] += W_q . dq + W_k . dk + W_v . dv, one launch (:1589-1745)
-        PanelArgs p = weights_times_acts(E, F, L, ns, F, 1);
-        p.nterm = 3;
+        PanelArgs q = weights_times_acts(E, F, L, ns, F, 1);
+        q.nterm = 3;
         for (int j = 0; j < 3; ++j) {
-            p.A[j] = W[j];
-            p.B[j] = dQKV[j];
+            q.A[j] = W[j];
+            q.B[j] = dQKV[j];
         }
-        p.C[0] = dX;
-        p.accumulate = 1;
-        rc = launch_panel(p, nullptr);
+        q.C[0] = dX;
+        q.accumulate = 1;
+        rc = launch_panel_pair<true, true, true, false>(p, part_i, q, nullptr, false);
+        if (rc == 0) rc = launch_panel_reduce_pair(pwo, p);
     }
     return sg.finish(rc);
 }
