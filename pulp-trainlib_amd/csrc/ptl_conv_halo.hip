@@ -792,30 +792,13 @@ __global__ __launch_bounds__(256) void conv_halo_wg_reduce_kernel(const float *_
         dW[idx * 9 + tap] = (half_t)s;
 }
 
-// gb[cb][p] for p < pstride: the tensor element t[b][8 cb .. + 7][yp - pu][xp - pl] at p = (b, yp, xp) of the padded
-// grid, zero outside the tensor and from the last padded position on.
+// gb[cb][p] for p < pstride (see halo_embed_chunk).
 __global__ __launch_bounds__(256) void conv_halo_embed_kernel(const half_t *__restrict__ dy, uint4 *__restrict__ out,
                                                               int B, int Ho, int Wo, int Hp, int Wp, int pu, int pl,
                                                               long long sb, long long sc, unsigned P, unsigned pstride,
                                                               unsigned total) {
     const unsigned i = blockIdx.x * 256u + threadIdx.x;
-    if (i >= total) return;
-    const unsigned cb = i / pstride, p = i - cb * pstride;
-    union {
-        uint4 v;
-        half_t e[8];
-    } u;
-    u.v = make_uint4(0, 0, 0, 0);
-    if (p < P) {
-        const unsigned r = p / (unsigned)Wp, xp = p - r * (unsigned)Wp;
-        const unsigned b = r / (unsigned)Hp, yy = r - b * (unsigned)Hp - (unsigned)pu, xx = xp - (unsigned)pl;
-        if (yy < (unsigned)Ho && xx < (unsigned)Wo) {
-            const half_t *src = dy + b * sb + (long long)(cb * 8) * sc + (long long)yy * Wo + xx;
-#pragma unroll
-            for (int e = 0; e < 8; ++e) u.e[e] = src[e * sc];
-        }
-    }
-    out[i] = u.v;
+    if (i < total) halo_embed_chunk(i, dy, out, Ho, Wo, Hp, Wp, pu, pl, sb, sc, P, pstride);
 }
 
 }  // namespace

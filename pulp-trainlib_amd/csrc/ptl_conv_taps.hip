@@ -139,17 +139,41 @@ struct TapPrepArgs {
     void *wr;
     int C, KW, taps;
     long long w_base, w_sm, w_sc, w_sy, w_sx, wr_total;
+    // the backward pass's two other passes, in front of the first: the blocked copy of the output gradient
+    // (embed_blocks workgroups, see halo_embed_chunk) and zero_n chunks of zeros at zero_at (zero_blocks workgroups)
+    const void *e_in;
+    uint4 *e_out;
+    int e_Ho, e_Wo, e_Hp, e_Wp, e_pu, e_pl;
+    long long e_sb, e_sc;
+    unsigned e_P, e_pstride, e_total, embed_blocks;
+    uint4 *zero_at;
+    unsigned zero_n, zero_blocks;
 };
 template <typename T>
 __global__ __launch_bounds__(256) void tap_prepare_kernel(const TapPrepArgs a) {
-    if (blockIdx.x < a.copy_blocks && a.hwc)
-        hwc_to_padded(blockIdx.x, reinterpret_cast<const uint4 *>(a.in), a.xb, a.B, a.H, a.W, a.Hp, a.Wp, a.padU, a.padL,
+    unsigned bid = blockIdx.x;
+    if (bid < a.embed_blocks) {
+        const unsigned i = bid * 256u + threadIdx.x;
+        if (i < a.e_total)
+            halo_embed_chunk(i, reinterpret_cast<const half_t *>(a.e_in), a.e_out, a.e_Ho, a.e_Wo, a.e_Hp, a.e_Wp, a.e_pu,
+                             a.e_pl, a.e_sb, a.e_sc, a.e_P, a.e_pstride);
+        return;
+    }
+    bid -= a.embed_blocks;
+    if (bid < a.zero_blocks) {
+        const unsigned i = bid * 256u + threadIdx.x;
+        if (i < a.zero_n) a.zero_at[i] = make_uint4(0, 0, 0, 0);
+        return;
+    }
+    bid -= a.zero_blocks;
+    if (bid < a.copy_blocks && a.hwc)
+        hwc_to_padded(bid, reinterpret_cast<const uint4 *>(a.in), a.xb, a.B, a.H, a.W, a.Hp, a.Wp, a.padU, a.padL,
                       a.cblocks, a.xb_total);
-    else if (blockIdx.x < a.copy_blocks)
-        chw_to_blocked_padded<T>(blockIdx.x, reinterpret_cast<const T *>(a.in), a.xb, a.B, a.H, a.W, a.Hp, a.Wp, a.padU,
+    else if (bid < a.copy_blocks)
+        chw_to_blocked_padded<T>(bid, reinterpret_cast<const T *>(a.in), a.xb, a.B, a.H, a.W, a.Hp, a.Wp, a.padU,
                                  a.padL, a.sb, a.sc, a.cblocks, a.xb_total);
     else
-        filters_tap_major<T>(blockIdx.x - a.copy_blocks, reinterpret_cast<const T *>(a.w), reinterpret_cast<T *>(a.wr),
+        filters_tap_major<T>(bid - a.copy_blocks, reinterpret_cast<const T *>(a.w), reinterpret_cast<T *>(a.wr),
                              a.C, a.KW, a.taps, a.w_base, a.w_sm, a.w_sc, a.w_sy, a.w_sx, a.wr_total);
 }
 
@@ -627,25 +651,48 @@ int conv_halo_bw(const ConvTileDesc &fwd, const ConvTileDesc &ig, const void *X,
         uint4 *xb = reinterpret_cast<uint4 *>(buf);
         char *gb = buf + (((size_t)xb_chunks * 16 + 255) & ~(size_t)255);
         T *wr = reinterpret_cast<T *>(gb + (((size_t)gb_chunks * 16 + 255) & ~(size_t)255));
-        // the shared copy of the output gradient (margin included: the input-gradient kernel reads past the end)
-        if (int rc = conv_halo_embed(dY, gb, ig.batch, ig.Cin, ig.Hin, ig.Win, Hp, Wp, ig.padU, ig.padL, gstride)) return rc;
-        {  // the last block's margin, and the flipped, transposed filters of the input gradient
-            hipLaunchKernelGGL(zero_chunks_kernel, dim3((unsigned)((gmargin + 255) / 256)), dim3(256), 0, st.stream,
-                               reinterpret_cast<uint4 *>(gb) + (long long)(fwd.Cout / VEC) * gstride, (unsigned)gmargin);
+        // One launch for the layout passes, all independent of each other: the shared copy of the output gradient, the
+        // zero margin behind its last block (the input-gradient kernel reads past the end), the blocked copy of the
+        // input unless the call was handed one, the flipped, transposed filters of the input gradient.
+        const uint4 *kept = cached_input(fwd, Hp, Wp, xb_chunks);
+        {
+            const long long Pg = (long long)ig.batch * Hp * Wp, e_chunks = (long long)(ig.Cin / VEC) * gstride;
+            if (e_chunks >= ((long long)1 << 31) || gstride < Pg) return -1;
             TapPrepArgs p = {};
-            p.copy_blocks = 0;
+            p.e_in = dY;
+            p.e_out = reinterpret_cast<uint4 *>(gb);
+            p.e_Ho = ig.Hin; p.e_Wo = ig.Win; p.e_Hp = Hp; p.e_Wp = Wp; p.e_pu = ig.padU; p.e_pl = ig.padL;
+            p.e_sb = (long long)ig.Cin * ig.Hin * ig.Win;
+            p.e_sc = (long long)ig.Hin * ig.Win;
+            p.e_P = (unsigned)Pg;
+            p.e_pstride = (unsigned)gstride;
+            p.e_total = (unsigned)e_chunks;
+            p.embed_blocks = (unsigned)((e_chunks + 255) / 256);
+            p.zero_at = reinterpret_cast<uint4 *>(gb) + (long long)(fwd.Cout / VEC) * gstride;
+            p.zero_n = (unsigned)gmargin;
+            p.zero_blocks = (unsigned)((gmargin + 255) / 256);
+            if (!kept) {
+                const int cblocks = fwd.Cin / VEC;
+                p.in = X;
+                p.xb = xb;
+                p.B = fwd.batch; p.H = fwd.Hin; p.W = fwd.Win; p.Hp = Hp; p.Wp = Wp; p.padU = fwd.padU; p.padL = fwd.padL;
+                p.cblocks = cblocks;
+                p.sb = fwd.x_sb; p.sc = fwd.x_sc;
+                p.xb_total = (long long)cblocks * fwd.batch * Hp * Wp + xmargin;
+                p.copy_blocks = (unsigned)((p.xb_total + 255) / 256);
+            }
             p.w = Wt;
             p.wr = wr;
             p.C = ig.Cin; p.KW = 3; p.taps = 9;
             p.w_base = ig.w_base; p.w_sm = ig.w_sm; p.w_sc = ig.w_sc; p.w_sy = ig.w_sy; p.w_sx = ig.w_sx;
             p.wr_total = wr_elems;
-            hipLaunchKernelGGL((tap_prepare_kernel<T>), dim3((unsigned)((wr_elems + 255) / 256)), dim3(256), 0, st.stream, p);
+            const unsigned long long blocks = (unsigned long long)p.embed_blocks + p.zero_blocks + p.copy_blocks +
+                                              (unsigned long long)((wr_elems + 255) / 256);
+            if (blocks >= (1ull << 31)) return -1;
+            hipLaunchKernelGGL((tap_prepare_kernel<T>), dim3((unsigned)blocks), dim3(256), 0, st.stream, p);
             if (!hip_ok(hipGetLastError(), "layout launch")) return 2;
         }
-        if (const uint4 *kept = cached_input(fwd, Hp, Wp, xb_chunks))
-            xb = const_cast<uint4 *>(kept);
-        else if (int rc = blocked_padded_copy<T>(reinterpret_cast<const T *>(X), xb, fwd, Hp, Wp, xmargin))
-            return rc;
+        if (kept) xb = const_cast<uint4 *>(kept);
         st.last_conv_resident = 1;
         if (int rc = conv_halo_wg_launch(fwd, xb, gb + (size_t)goff * 16, gstride, ws, dW, Hp, Wp, S0, S1)) return rc;
         return conv_halo_launch(ig, gb, wr, dX, Hp, Wp, gstride);

@@ -121,6 +121,30 @@ inline bool conv_output_fits_pads(const ConvTileDesc &d) {
 // filters).  Y is the dense channel-major output [batch][Cout][Ho][Wo].
 bool conv_halo_fits(const ConvTileDesc &d, int Hp, int Wp);
 long long conv_halo_margin();
+// Chunk i of gb[cb][p], p < pstride: the tensor element t[b][8 cb .. + 7][yp - pu][xp - pl] at p = (b, yp, xp) of the
+// padded grid, zero outside the tensor and from the last padded position on (the blocked copy of an output gradient
+// that the resident-tile weight- and input-gradient kernels read).
+__device__ inline void halo_embed_chunk(unsigned i, const half_t *__restrict__ dy, uint4 *__restrict__ out, int Ho,
+                                        int Wo, int Hp, int Wp, int pu, int pl, long long sb, long long sc, unsigned P,
+                                        unsigned pstride) {
+    const unsigned cb = i / pstride, p = i - cb * pstride;
+    union {
+        uint4 v;
+        half_t e[8];
+    } u;
+    u.v = make_uint4(0, 0, 0, 0);
+    if (p < P) {
+        const unsigned r = p / (unsigned)Wp, xp = p - r * (unsigned)Wp;
+        const unsigned b = r / (unsigned)Hp, yy = r - b * (unsigned)Hp - (unsigned)pu, xx = xp - (unsigned)pl;
+        if (yy < (unsigned)Ho && xx < (unsigned)Wo) {
+            const half_t *src = dy + b * sb + (long long)(cb * 8) * sc + (long long)yy * Wo + xx;
+#pragma unroll
+            for (int e = 0; e < 8; ++e) u.e[e] = src[e * sc];
+        }
+    }
+    out[i] = u.v;
+}
+
 // A second copy of the output for the layer that reads it next: channel-blocked and padded for THAT layer,
 // [channels / 8][batch][Hp][Wp] 16-byte chunks with the output pixel (y, x) at (y + padU, x + padL); the kernel
 // writes the pixels, the halo is the caller's (zero) business.
