@@ -451,12 +451,36 @@ int conv_taps_wg(const ConvTileDesc &d, const void *X, const void *dY, void *dW)
                 if (!ws) return 2;
                 uint4 *xb = reinterpret_cast<uint4 *>(buf);
                 char *gb = buf + (((size_t)xb_chunks * 16 + 255) & ~(size_t)255);
-                if (const uint4 *kept = cached_input(d, Hp, Wp, xb_chunks))
-                    xb = const_cast<uint4 *>(kept);
-                else if (int rc = blocked_padded_copy<T>(reinterpret_cast<const T *>(X), xb, d, Hp, Wp, margin))
-                    return rc;
+                // both layout passes in one launch (the blocked copy of the output gradient, and that of the input
+                // unless the call was handed one)
                 const long long gstride = conv_halo_wg_gradient_stride(d, Hp, Wp);
-                if (int rc = conv_halo_embed(dY, gb, d.batch, d.Cout, d.Ho, d.Wo, Hp, Wp, 0, 0, gstride)) return rc;
+                const uint4 *kept = cached_input(d, Hp, Wp, xb_chunks);
+                if (gstride < P) return -1;
+                {
+                    TapPrepArgs p = {};
+                    p.e_in = dY;
+                    p.e_out = reinterpret_cast<uint4 *>(gb);
+                    p.e_Ho = d.Ho; p.e_Wo = d.Wo; p.e_Hp = Hp; p.e_Wp = Wp;
+                    p.e_sb = (long long)d.Cout * d.Ho * d.Wo;
+                    p.e_sc = (long long)d.Ho * d.Wo;
+                    p.e_P = (unsigned)P;
+                    p.e_pstride = (unsigned)gstride;
+                    p.e_total = (unsigned)gb_chunks;
+                    p.embed_blocks = (unsigned)((gb_chunks + 255) / 256);
+                    if (!kept) {
+                        p.in = X;
+                        p.xb = xb;
+                        p.B = d.batch; p.H = d.Hin; p.W = d.Win; p.Hp = Hp; p.Wp = Wp; p.padU = d.padU; p.padL = d.padL;
+                        p.cblocks = d.Cin / VEC;
+                        p.sb = d.x_sb; p.sc = d.x_sc;
+                        p.xb_total = xb_chunks;
+                        p.copy_blocks = (unsigned)((xb_chunks + 255) / 256);
+                    }
+                    hipLaunchKernelGGL((tap_prepare_kernel<T>), dim3(p.embed_blocks + p.copy_blocks), dim3(256), 0, st.stream,
+                                       p);
+                    if (!hip_ok(hipGetLastError(), "layout launch")) return 2;
+                }
+                if (kept) xb = const_cast<uint4 *>(kept);
                 st.last_conv_resident = 1;
                 return conv_halo_wg_launch(d, xb, gb, gstride, ws, dW, Hp, Wp, S0, S1);
             }
