@@ -92,3 +92,61 @@ def test_growth_and_stream_switch_are_refused_under_capture_and_reserve_makes_th
         gpu.ptl_set_gemm_path(0)
         gpu.ptl_set_stream(None)
         assert gpu.ptl_sync() == 0
+
+
+def test_layers_in_a_row_with_the_copy_handed_on_replay_as_a_hip_graph(pkg, gpu):
+    """Two 3x3 layers with the blocked copy handed from the first layer's forward kernel to the second layer's forward
+    and weight-gradient calls (ptl_conv2d_fp16_cache_prepare, _fw_batched_chained, _wg_batched_cached), captured once
+    on a stream of the caller's: every replay, with the outputs and the copy overwritten in between, reproduces the
+    eager result bit for bit."""
+    Ci, H, Cm, Co, ns = 64, 14, 128, 64, 12
+    pad = (1, 1, 1, 1)
+    g = torch.Generator(device="cpu").manual_seed(11)
+    x = (torch.rand(ns, Ci, H, H, generator=g) - 0.5).half().to(DEV)
+    w1 = ((torch.rand(Cm, Ci, 3, 3, generator=g) - 0.5) * 0.2).half().to(DEV)
+    w2 = ((torch.rand(Co, Cm, 3, 3, generator=g) - 0.5) * 0.2).half().to(DEV)
+    dy2 = (torch.rand(ns, Co, H, H, generator=g) - 0.5).half().to(DEV)
+    y1 = torch.zeros(ns, Cm, H, H, device=DEV).half()
+    y2, dw2 = torch.zeros_like(dy2), torch.zeros_like(w2)
+    a1, k1 = hp.conv2d_args(pkg, x, None, w1, None, y1, None, Ci, H, H, Cm, 3, 3, H, H, pad, (1, 1))
+    a2, k2 = hp.conv2d_args(pkg, y1, None, w2, dw2, y2, dy2, Cm, H, H, Co, 3, 3, H, H, pad, (1, 1))
+    nbytes = gpu.ptl_conv2d_fp16_cache_bytes(ctypes.byref(a2), ns)
+    assert nbytes > 0
+    buf = torch.full((nbytes,), 0x3c, dtype=torch.uint8, device=DEV)
+    c = pkg.ConvCache()
+    c.buf, c.bytes = buf.data_ptr(), nbytes
+
+    def step():
+        assert gpu.ptl_conv2d_fp16_cache_prepare(ctypes.byref(a2), ns, ctypes.byref(c)) == 0
+        assert gpu.ptl_conv2d_fp16_fw_batched_chained(ctypes.byref(a1), ns, None, ctypes.byref(c)) == 0
+        assert c.valid == 1
+        assert gpu.ptl_conv2d_fp16_fw_batched_chained(ctypes.byref(a2), ns, ctypes.byref(c), None) == 0
+        assert gpu.ptl_conv2d_fp16_wg_batched_cached(ctypes.byref(a2), ns, ctypes.byref(c)) == 0
+
+    side = torch.cuda.Stream()
+    gpu.ptl_set_gemm_path(5)
+    gpu.ptl_set_stream(ctypes.c_void_p(side.cuda_stream))
+    try:
+        with torch.cuda.stream(side):
+            step()  # (eager: the result to reproduce, and the library's buffers at their size)
+            side.synchronize()
+        eager = [t.clone() for t in (y1, y2, dw2)]
+        ref = torch.nn.functional.conv2d(torch.nn.functional.conv2d(x.double(), w1.double(), padding=1).half().double(),
+                                         w2.double(), padding=1)
+        assert float((eager[1].double() - ref).norm() / ref.norm()) <= 2e-3
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph, stream=side):
+            step()
+        for k in range(3):
+            for t in (y1, y2, dw2):
+                t.fill_(float(k + 2))
+            buf.fill_(0x3c + k)
+            torch.cuda.synchronize()
+            graph.replay()
+            torch.cuda.synchronize()
+            for t, e in zip((y1, y2, dw2), eager):
+                assert torch.equal(t, e)
+    finally:
+        gpu.ptl_set_gemm_path(0)
+        gpu.ptl_set_stream(None)
+        assert gpu.ptl_sync() == 0
