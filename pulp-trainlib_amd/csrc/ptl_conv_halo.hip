@@ -498,7 +498,8 @@ int launch_halo(const HaloArgs &a, int grid, hipStream_t stream) {
 // and a fragment is two transposing reads (ds_read_b64_tr_b16); a tap is a shift by whole chunks, so every
 // read stays aligned.  A workgroup (4 waves) owns 128 filters x 64 channels x a group of taps (0..4 or 5..8)
 // and a range of positions; it walks units of 128 positions (gradient tile 32 KB + input tile of 256 positions
-// 32 KB, two buffers, the next unit in flight while this one is multiplied) with all accumulators in registers
+// 32 KB - of which only the 192 positions that the taps reach are loaded when the rows are at most 31 wide -, two
+// buffers, the next unit in flight while this one is multiplied) with all accumulators in registers
 // and writes one fp32 partial sum per tap at the end; a second kernel adds the partial sums.
 constexpr int HWG_UNIT = 128;                 // positions per unit
 constexpr int HWG_GP = 132, HWG_XP = 260;     // LDS pitches (chunks) of the gradient / input tiles: == 4 mod 16,
@@ -516,6 +517,7 @@ struct HaloWgArgs {
     int tiles;         // (Cout / 128) * (Cin / 64)
     int S0, S1, smax;  // position splits of the two tap groups
     int xcd_map;       // 1: bundles of `tiles` workgroups per XCD (see the kernel)
+    int x_pieces;      // 64-position pieces of the input tile that the taps can reach: 3 when 2 * Wp + 2 <= 64, else 4
     // channel-minor tensors read in place (HWC = true): xb = X[batch][H][W][Cin], gb = dY[batch][H][W][Cout]
     const char *zeros;
     int batch, H, W, Hp;
@@ -594,10 +596,12 @@ __device__ inline void halo_wg_body(const HaloWgArgs &a, char *smem, int tile, i
                 const char *src = idx >= 0 ? a.gb + ((size_t)(unsigned)idx * cout2 + chunk) : a.zeros;
                 lds_dma<16>(src, lds0 + (unsigned)(buf * HWG_BUF + ig * 1024));
             }
-            const int ix = wave * 8 + q;
-            const int idx = t[ix * 8 + (lane >> 3)];
-            const char *src = idx >= 0 ? a.xb + ((size_t)(unsigned)idx * cin2 + x_chunk) : a.zeros;
-            lds_dma<16>(src, lds0 + (unsigned)(buf * HWG_BUF + HWG_GB + ix * 1024));
+            if (wave < a.x_pieces) {  // (wave w loads positions 64 w .. 64 w + 63 of the input tile)
+                const int ix = wave * 8 + q;
+                const int idx = t[ix * 8 + (lane >> 3)];
+                const char *src = idx >= 0 ? a.xb + ((size_t)(unsigned)idx * cin2 + x_chunk) : a.zeros;
+                lds_dma<16>(src, lds0 + (unsigned)(buf * HWG_BUF + HWG_GB + ix * 1024));
+            }
         }
     };
 
@@ -610,7 +614,7 @@ __device__ inline void halo_wg_body(const HaloWgArgs &a, char *smem, int tile, i
                 const int cb = idx >> 1, piece = idx & 1;
                 const char *base = a.gb + ((long long)(co_cb0 + cb) * a.Pd + p0 + piece * 64) * 16;
                 lds_dma16_saddr(voff, base, lds0 + (unsigned)(buf * HWG_BUF + (cb * HWG_GP + piece * 64) * 16));
-            } else {  // input tile: 8 channel blocks x 4 pieces
+            } else if (wave < a.x_pieces) {  // input tile: 8 channel blocks x 4 pieces, piece = wave
                 const int j = idx - 32, cb = j >> 2, piece = j & 3;
                 const char *base = a.xb + ((long long)(ci_cb0 + cb) * a.Px + p0 + piece * 64) * 16;
                 lds_dma16_saddr(voff, base,
@@ -1003,6 +1007,8 @@ static int halo_wg_run(HaloWgArgs &a, const ConvTileDesc &d, float *ws, void *dW
         attr = true;
     }
     a.xcd_map = 1;
+    // the last tap reads positions up to 127 + 2 * Wp + 2 of the input tile: within its first 192 for rows up to 31 wide
+    a.x_pieces = 2 * a.Wp + 2 <= 64 ? 3 : 4;
     const int bundles = (a.S0 + a.S1 + 7) / 8 * 8;
     hipLaunchKernelGGL((conv_halo_wg_kernel<HWC, FI>), dim3((unsigned)(a.tiles * bundles)), dim3(HALO_NT), lds, st.stream,
                        a);
