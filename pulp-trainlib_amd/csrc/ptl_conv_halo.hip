@@ -497,14 +497,21 @@ int launch_halo(const HaloArgs &a, int grid, hipStream_t stream) {
 // like xb.  The contraction runs over positions, so both operands sit in LDS as [position][8 channels] chunks
 // and a fragment is two transposing reads (ds_read_b64_tr_b16); a tap is a shift by whole chunks, so every
 // read stays aligned.  A workgroup (4 waves) owns 128 filters x 64 channels x a group of taps (0..4 or 5..8)
-// and a range of positions; it walks units of 128 positions (gradient tile 32 KB + input tile of 256 positions
-// 32 KB - of which only the 192 positions that the taps reach are loaded when the rows are at most 31 wide -, two
-// buffers, the next unit in flight while this one is multiplied) with all accumulators in registers
+// and a range of positions; it walks units of 128 positions (gradient tile 32 KB, two buffers; input tile of the
+// 192 positions that the taps reach when the rows are at most 31 wide, else 256, of which consecutive units share
+// all but 128: a ring, see HWG_RING; the next unit in flight while this one is multiplied) with all accumulators in
+// registers
 // and writes one fp32 partial sum per tap at the end; a second kernel adds the partial sums.
 constexpr int HWG_UNIT = 128;                 // positions per unit
 constexpr int HWG_GP = 132, HWG_XP = 260;     // LDS pitches (chunks) of the gradient / input tiles: == 4 mod 16,
                                               // so that the 16 rows of a transposing read fall on distinct banks
 constexpr int HWG_GB = 16 * HWG_GP * 16, HWG_XB = 8 * HWG_XP * 16, HWG_BUF = HWG_GB + HWG_XB;
+// Channel-major form: the input tiles of consecutive units overlap (unit u reads positions 128 u .. 128 u + 64 R - 1,
+// R = 3 or 4 pieces of 64), so they live in ONE ring of six 64-position slots per channel block, piece j in slot
+// j % 6, behind the two gradient buffers; a unit brings in two new pieces.  Slots 6 and 7 repeat slots 0 and 1 (a
+// piece that lands in slot 0, or in slot 1 when R = 4, is loaded a second time there), so the reads of a unit, which
+// start at slot 0, 2 or 4, never wrap.
+constexpr int HWG_RP = 8 * 64 + 4, HWG_RB = 8 * HWG_RP * 16, HWG_RING = 2 * HWG_GB;
 
 struct HaloWgArgs {
     const char *xb;    // [Cin/8][Px] chunks, readable 256 chunks past the start of the last unit
@@ -605,20 +612,36 @@ __device__ inline void halo_wg_body(const HaloWgArgs &a, char *smem, int tile, i
         }
     };
 
-    auto issue = [&](int u, int buf) {
+    // 64 positions of input channel block cb, from position pos on, into slot `slot` of the ring
+    auto issue_x = [&](long long pos, int cb, int slot) __attribute__((always_inline)) {
+        const char *base = a.xb + ((long long)(ci_cb0 + cb) * a.Px + pos) * 16;
+        lds_dma16_saddr(voff, base, lds0 + (unsigned)(HWG_RING + (cb * HWG_RP + slot * 64) * 16));
+    };
+    // the gradient tile of unit u into buffer buf and, first = true: the R pieces of its input tile into slots 0 ..
+    // R - 1 (wave w loads piece w); else, k3 = (u - 1 - u0) % 3: its two last pieces, (u - u0) * 2 + R - 2 and the next
+    auto issue = [&](int u, int buf, bool first, int k3) __attribute__((always_inline)) {
         const long long p0 = (long long)u * HWG_UNIT;
 #pragma unroll
-        for (int q = 0; q < 16; ++q) {
-            const int idx = q * 4 + wave;
-            if (q < 8) {  // gradient tile: 16 channel blocks x 2 pieces of 64 positions
-                const int cb = idx >> 1, piece = idx & 1;
-                const char *base = a.gb + ((long long)(co_cb0 + cb) * a.Pd + p0 + piece * 64) * 16;
-                lds_dma16_saddr(voff, base, lds0 + (unsigned)(buf * HWG_BUF + (cb * HWG_GP + piece * 64) * 16));
-            } else if (wave < a.x_pieces) {  // input tile: 8 channel blocks x 4 pieces, piece = wave
-                const int j = idx - 32, cb = j >> 2, piece = j & 3;
-                const char *base = a.xb + ((long long)(ci_cb0 + cb) * a.Px + p0 + piece * 64) * 16;
-                lds_dma16_saddr(voff, base,
-                                lds0 + (unsigned)(buf * HWG_BUF + HWG_GB + (cb * HWG_XP + piece * 64) * 16));
+        for (int q = 0; q < 8; ++q) {  // gradient tile: 16 channel blocks x 2 pieces of 64 positions
+            const int idx = q * 4 + wave, cb = idx >> 1, piece = idx & 1;
+            const char *base = a.gb + ((long long)(co_cb0 + cb) * a.Pd + p0 + piece * 64) * 16;
+            lds_dma16_saddr(voff, base, lds0 + (unsigned)(buf * HWG_GB + (cb * HWG_GP + piece * 64) * 16));
+        }
+        if (first) {
+            if (wave < a.x_pieces) {
+#pragma unroll
+                for (int cb = 0; cb < 8; ++cb) issue_x(p0 + wave * 64, cb, wave);
+            }
+        } else {
+            const int R = a.x_pieces, pc = wave & 1;
+            int slot = 2 * k3 + R + pc;
+            slot = slot >= 6 ? slot - 6 : slot;
+            const long long pos = p0 + (R - 2 + pc) * 64;
+#pragma unroll
+            for (int q = 0; q < 4; ++q) issue_x(pos, q * 2 + (wave >> 1), slot);
+            if (slot < R - 2) {
+#pragma unroll
+                for (int q = 0; q < 4; ++q) issue_x(pos, q * 2 + (wave >> 1), slot + 6);
             }
         }
     };
@@ -650,7 +673,7 @@ __device__ inline void halo_wg_body(const HaloWgArgs &a, char *smem, int tile, i
             if constexpr (HWC)
                 xoff[c][t] = (unsigned)(HWG_GB + (8 * kq + pq + sh) * 128 + ((wn * 4 + 2 * c + pj + 2 * pq + 2 * sh) & 7) * 16 + ph);
             else
-                xoff[c][t] = (unsigned)(HWG_GB + (((wn * 4 + 2 * c + pj) * HWG_XP + 8 * kq + pq + sh) * 16) + ph);
+                xoff[c][t] = (unsigned)(HWG_RING + (((wn * 4 + 2 * c + pj) * HWG_RP + 8 * kq + pq + sh) * 16) + ph);
         }
 
     f32x4 acc[FI][2][NT];
@@ -670,9 +693,10 @@ __device__ inline void halo_wg_body(const HaloWgArgs &a, char *smem, int tile, i
             issue_hwc(0, 0);
             if (u0 + 1 < u1) fill_table(u0 + 1, 1);
         } else {
-            issue(u0, 0);
+            issue(u0, 0, true, 0);
         }
     }
+    int k3 = 0;  // (u - u0) % 3: the unit's input tile starts at slot 2 * k3 of the ring
     for (int u = u0; u < u1; ++u) {
         const int buf = (u - u0) & 1;
         wait_vmcnt<0>();
@@ -683,9 +707,11 @@ __device__ inline void halo_wg_body(const HaloWgArgs &a, char *smem, int tile, i
             if (u + 1 < u1) issue_hwc(buf ^ 1, buf ^ 1);
             if (u + 2 < u1) fill_table(u + 2, buf);
         } else {
-            issue(u + 1 < u1 ? u + 1 : u, buf ^ 1);
+            if (u + 1 < u1) issue(u + 1, buf ^ 1, false, k3);
         }
-        const char *bt = smem + buf * HWG_BUF;
+        const char *bt = smem + buf * (HWC ? HWG_BUF : HWG_GB);
+        const char *xt = HWC ? bt : smem + k3 * (2 * 64 * 16);
+        k3 = k3 == 2 ? 0 : k3 + 1;
         uint4 gf[2][FI], xf[2][2][NT];
         auto read = [&](int set, int ks) {
 #pragma unroll
@@ -693,7 +719,7 @@ __device__ inline void halo_wg_body(const HaloWgArgs &a, char *smem, int tile, i
 #pragma unroll
             for (int c = 0; c < 2; ++c)
 #pragma unroll
-                for (int t = 0; t < NT; ++t) xf[set][c][t] = hwg_frag(bt + xoff[c][t] + ks * KSX, RDX);
+                for (int t = 0; t < NT; ++t) xf[set][c][t] = hwg_frag(xt + xoff[c][t] + ks * KSX, RDX);
         };
         read(0, 0);
         static_for<0, 4>([&](auto KI) {
@@ -997,7 +1023,8 @@ int conv_halo_embed(const void *t, void *out, int batch, int C, int Hs, int Ws, 
 template <bool HWC, int FI>
 static int halo_wg_run(HaloWgArgs &a, const ConvTileDesc &d, float *ws, void *dW) {
     State &st = state();
-    constexpr int lds = 2 * HWG_BUF + (HWC ? 2 * 256 * (int)sizeof(int) : 0);  // (+ the two position tables)
+    // channel-minor: two buffers of both tiles + the two position tables; channel-major: two gradient buffers + the ring
+    constexpr int lds = HWC ? 2 * HWG_BUF + 2 * 256 * (int)sizeof(int) : HWG_RING + HWG_RB;
     static bool attr = false;
     if (!attr) {
         if (!hip_ok(hipFuncSetAttribute((const void *)conv_halo_wg_kernel<HWC, FI>,
