@@ -870,6 +870,55 @@ __global__ __launch_bounds__(256) void conv_halo_wg_reduce4_kernel(const float *
     }
 }
 
+// Channel-major filters [co][ci][tap], many outputs: the nine taps of an output are nine 2-byte stores 18 bytes apart
+// from nine workgroups in the kernels above (21 M such stores for 512 x 512 filters: 8 of the 14 us of that
+// addition).  Here a workgroup adds all nine taps of 256 consecutive outputs - the same sums in the same order, a
+// thread's loads of the nine taps in flight together - and writes their 4608 bytes in 16-byte pieces.
+// total % 256 == 0.
+__global__ __launch_bounds__(256) void conv_halo_wg_reduce9_kernel(const float *__restrict__ ws, half_t *__restrict__ dW,
+                                                                   long long total, int S0, int S1, int smax) {
+    __shared__ float4 part[9][4][64];
+    __shared__ __align__(16) half_t outv[256 * 9];
+    const int o = threadIdx.x & 63, sg = threadIdx.x >> 6;
+    const long long idx = ((long long)blockIdx.x * 64 + o) * 4;
+    float4 s[9];
+#pragma unroll
+    for (int tap = 0; tap < 9; ++tap) {
+        const int S = tap < 5 ? S0 : S1;
+        const float *src = ws + (size_t)tap * smax * total + idx;
+        auto ld = [&](int z) { return *reinterpret_cast<const float4 *>(src + (size_t)z * total); };
+        s[tap] = make_float4(0.f, 0.f, 0.f, 0.f);
+        int z = sg;
+        for (; z + 12 < S; z += 16) {
+            float4 v[4];
+#pragma unroll
+            for (int k = 0; k < 4; ++k) v[k] = ld(z + 4 * k);
+            s[tap].x += (v[0].x + v[1].x) + (v[2].x + v[3].x);
+            s[tap].y += (v[0].y + v[1].y) + (v[2].y + v[3].y);
+            s[tap].z += (v[0].z + v[1].z) + (v[2].z + v[3].z);
+            s[tap].w += (v[0].w + v[1].w) + (v[2].w + v[3].w);
+        }
+        for (; z < S; z += 4) {
+            const float4 v = ld(z);
+            s[tap].x += v.x; s[tap].y += v.y; s[tap].z += v.z; s[tap].w += v.w;
+        }
+    }
+#pragma unroll
+    for (int tap = 0; tap < 9; ++tap) part[tap][sg][o] = s[tap];
+    __syncthreads();
+    // wave sg: taps sg, sg + 4 (and 8 for wave 0) of the quads
+    for (int tap = sg; tap < 9; tap += 4) {
+        const float4 p0 = part[tap][0][o], p1 = part[tap][1][o], p2 = part[tap][2][o], p3 = part[tap][3][o];
+        const float r[4] = {(p0.x + p1.x) + (p2.x + p3.x), (p0.y + p1.y) + (p2.y + p3.y), (p0.z + p1.z) + (p2.z + p3.z),
+                            (p0.w + p1.w) + (p2.w + p3.w)};
+#pragma unroll
+        for (int k = 0; k < 4; ++k) outv[(o * 4 + k) * 9 + tap] = (half_t)r[k];
+    }
+    __syncthreads();
+    uint4 *dst = reinterpret_cast<uint4 *>(dW + (long long)blockIdx.x * 256 * 9);
+    for (int j = threadIdx.x; j < 256 * 9 * 2 / 16; j += 256) dst[j] = reinterpret_cast<const uint4 *>(outv)[j];
+}
+
 // gb[cb][p] for p < pstride (see halo_embed_chunk).
 __global__ __launch_bounds__(256) void conv_halo_embed_kernel(const half_t *__restrict__ dy, uint4 *__restrict__ out,
                                                               int B, int Ho, int Wo, int Hp, int Wp, int pu, int pl,
@@ -1093,7 +1142,11 @@ static int halo_wg_run(HaloWgArgs &a, const ConvTileDesc &d, float *ws, void *dW
     // four outputs per thread from 128 x 128 filters on (same sums; in turns in one process 58.0 -> 56.3 us per call on
     // 256 -> 256 14x14 batch 128 channel-minor, 57.3 -> 56.5 channel-major, equal at batch 256); a 64 x 64 filter tensor
     // would be 144 workgroups that way (52.8 -> 54.6 us)
-    if (total >= 128 * 128)
+    // (in turns in one process: 278.9 -> 275.9 us per call on 512 -> 512 14x14 batch 256; from 1024 workgroups on)
+    if (!HWC && total >= 1024 * 256 && total % 256 == 0 && (uintptr_t)dW % 16 == 0)
+        hipLaunchKernelGGL(conv_halo_wg_reduce9_kernel, dim3((unsigned)(total / 256)), dim3(256), 0, st.stream, ws,
+                           static_cast<half_t *>(dW), total, a.S0, a.S1, a.smax);
+    else if (total >= 128 * 128)
         hipLaunchKernelGGL(conv_halo_wg_reduce4_kernel, dim3((unsigned)((total + 255) / 256), 9), dim3(256), 0, st.stream,
                            ws, static_cast<half_t *>(dW), total, a.S0, FI == 2 ? a.S0 : a.S1, a.smax, HWC ? d.Cin : 0);
     else

@@ -781,6 +781,31 @@ def test_conv2d_wide_layers_against_torch(pkg, gpu, case):
         assert err <= 2e-3, (name, err)
 
 
+def test_conv2d_weight_gradient_of_512_filters_adds_its_partial_sums_the_same_both_ways(pkg, gpu):
+    """512 -> 512 on 14x14: the resident-tile weight gradient; its partial sums are added by the kernel that writes the
+    nine taps of an output together when dW is 16-byte aligned, by the one that writes them tap by tap when it is
+    not - same sums, same bits - and both against torch's fp32 weight gradient."""
+    Ci = Co = 512
+    H, ns = 14, 16
+    x = dev(hp.uniform(31, (ns, Ci, H, H), dtype=np.float16))
+    dy = dev(hp.uniform(33, (ns, Co, H, H), dtype=np.float16))
+    w = torch.zeros(Co, Ci, 3, 3, device="cuda").half()
+    flat = torch.zeros(Co * Ci * 9 + 8, device="cuda").half()
+    got = []
+    for off in (0, 1):  # (a torch allocation is 256-byte aligned; one element on it is 2-byte aligned)
+        dw = flat[off:off + Co * Ci * 9].view(Co, Ci, 3, 3)
+        assert dw.data_ptr() % 16 == (0 if off == 0 else 2)
+        dw.fill_(3.0)
+        a, keep = hp.conv2d_args(pkg, x, None, w, dw, None, dy, Ci, H, H, Co, 3, 3, H, H, (1, 1, 1, 1), (1, 1))
+        pkg.call("ptl_conv2d_fp16_wg_batched", a, ns)
+        assert gpu.ptl_last_conv_resident() == 1
+        sync(gpu)
+        got.append(dw.clone())
+    assert torch.equal(got[0], got[1])
+    ref = torch.nn.grad.conv2d_weight(x.float(), w.shape, dy.float(), padding=1)
+    assert float((got[0].float() - ref).norm() / ref.norm()) <= 2e-3
+
+
 @pytest.mark.parametrize("case", [(64, 64, 56, 8), (128, 128, 28, 16), (256, 256, 14, 32), (64, 128, 12, 64),
                                   (128, 64, 9, 128)])
 def test_conv2d_wide_layers_hwc_against_torch(pkg, gpu, case):
