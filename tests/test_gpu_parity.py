@@ -781,6 +781,30 @@ def test_conv2d_wide_layers_against_torch(pkg, gpu, case):
         assert err <= 2e-3, (name, err)
 
 
+@pytest.mark.parametrize("case", [(256, 256, 32, 32, 16), (128, 256, 20, 45, 24), (256, 128, 30, 30, 40)])
+def test_conv2d_resident_tile_weight_gradient_walks_many_units(pkg, gpu, case):
+    """The resident-tile weight gradient with eight and more units of 128 positions per workgroup, so that the ring of
+    input-tile pieces in LDS goes round several times: rows 33 and 46 wide (the taps reach four 64-position pieces,
+    both repeated slots of the ring are read) and 31 wide (three pieces, the widest such row), against torch's fp32
+    weight gradient of the same tensors."""
+    Ci, Co, H, W, ns = case
+    x = dev(hp.uniform(51, (ns, Ci, H, W), dtype=np.float16))
+    dy = dev(hp.uniform(53, (ns, Co, H, W), dtype=np.float16))
+    w = torch.zeros(Co, Ci, 3, 3, device="cuda").half()
+    dw = torch.full_like(w, 3.0)
+    a, keep = hp.conv2d_args(pkg, x, None, w, dw, None, dy, Ci, H, W, Co, 3, 3, H, W, (1, 1, 1, 1), (1, 1))
+    gpu.ptl_set_gemm_path(5)
+    try:
+        pkg.call("ptl_conv2d_fp16_wg_batched", a, ns)
+        assert gpu.ptl_last_conv_resident() == 1
+    finally:
+        gpu.ptl_set_gemm_path(0)
+    sync(gpu)
+    ref = torch.nn.grad.conv2d_weight(x.float(), w.shape, dy.float(), padding=1)
+    assert float((dw.float() - ref).norm() / ref.norm()) <= 2e-3
+    assert float((dw.float() - ref).abs().max() / ref.abs().max()) <= 5e-3
+
+
 def test_conv2d_weight_gradient_of_512_filters_adds_its_partial_sums_the_same_both_ways(pkg, gpu):
     """512 -> 512 on 14x14: the resident-tile weight gradient; its partial sums are added by the kernel that writes the
     nine taps of an output together when dW is 16-byte aligned, by the one that writes them tap by tap when it is
