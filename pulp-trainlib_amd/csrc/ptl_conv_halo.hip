@@ -1063,7 +1063,14 @@ bool conv_halo_wg_preferred(const ConvTileDesc &d) {
     conv_padded_grid(d, &Hp, &Wp);
     const long long units = ((long long)d.batch * Hp * Wp + HWG_UNIT - 1) / HWG_UNIT;
     const int cmin = d.Cin < d.Cout ? d.Cin : d.Cout;
-    return conv_halo_wg_fits(d, Hp, Wp) && Wp <= 32 && units >= (cmin >= 256 ? 20 : 96);
+    // Rows 33 to 63 wide (four pieces of the input tile per unit; the ring made them cheaper), against the routes they
+    // took before, in turns in one process: 128 -> 128 on 56x56 at batch 128 205 against 237 us (batch 8: 30.0 / 32.2),
+    // 128 -> 256 on 56x56 at batch 64 178 / 233, on 48x48 at batch 128 267 / 355, 256 -> 256 on 32x32 at batch 128
+    // 202 / 222 (batch 16: 40.6 / 56.0, batch 4: equal), on 56x56 at batch 64 319 / 330, 128 -> 128 on 40x40 at
+    // batch 256 207 / 223 (batch 8: 24.9 / 30.7); with 64 channels 64 -> 128 on 56x56 at batch 128 132 / 137, at
+    // batch 16 equal, at batch 4 23.4 against 20.6: those only from 1600 units on.
+    const bool wide_ok = Wp <= 32 || cmin >= 128 || units >= 1600;
+    return conv_halo_wg_fits(d, Hp, Wp) && wide_ok && units >= (cmin >= 256 ? 20 : 96);
 }
 // Channel-minor: the other route copies both tensors into padded form first (9 + 9 of 66 us on 128 -> 128 28x28 at
 // batch 128), so this one is taken from the same amount of work on whatever the row length.

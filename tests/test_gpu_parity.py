@@ -805,6 +805,33 @@ def test_conv2d_resident_tile_weight_gradient_walks_many_units(pkg, gpu, case):
     assert float((dw.float() - ref).abs().max() / ref.abs().max()) <= 5e-3
 
 
+@pytest.mark.parametrize("case", [(128, 128, 56, 8), (128, 256, 40, 8), (64, 128, 56, 64)])
+def test_conv2d_wide_rows_take_the_resident_tile_gradients_by_default(pkg, gpu, case):
+    """Rows 41 and 57 wide, filters a multiple of 128: the weight gradient and the one-call backward choose the
+    resident-tile kernels by themselves (64 input channels only from 1600 units of positions on); both against
+    torch's fp32 gradients of the same tensors, and the one-call backward bit for bit against the two steps."""
+    Ci, Co, H, ns = case
+    x = dev(hp.uniform(61, (ns, Ci, H, H), dtype=np.float16))
+    w = dev(hp.uniform(62, (Co, Ci, 3, 3), -0.1, 0.1).astype(np.float16))
+    dy = dev(hp.uniform(63, (ns, Co, H, H), dtype=np.float16))
+    dw, dx = torch.full_like(w, 3.0), torch.full_like(x, 3.0)
+    a, keep = hp.conv2d_args(pkg, x, dx, w, dw, None, dy, Ci, H, H, Co, 3, 3, H, H, (1, 1, 1, 1), (1, 1))
+    pkg.call("ptl_conv2d_fp16_wg_batched", a, ns)
+    assert gpu.ptl_last_conv_resident() == 1
+    pkg.call("ptl_conv2d_fp16_ig_batched", a, ns)
+    sync(gpu)
+    ref_dw = torch.nn.grad.conv2d_weight(x.float(), w.shape, dy.float(), padding=1)
+    ref_dx = torch.nn.grad.conv2d_input(x.shape, w.float(), dy.float(), padding=1)
+    assert float((dw.float() - ref_dw).norm() / ref_dw.norm()) <= 2e-3
+    assert float((dx.float() - ref_dx).norm() / ref_dx.norm()) <= 2e-3
+    dw2, dx2 = torch.full_like(w, 5.0), torch.full_like(x, 5.0)
+    b, keep2 = hp.conv2d_args(pkg, x, dx2, w, dw2, None, dy, Ci, H, H, Co, 3, 3, H, H, (1, 1, 1, 1), (1, 1))
+    pkg.call("ptl_conv2d_fp16_bw_batched", b, ns)
+    assert gpu.ptl_last_conv_resident() == 1
+    sync(gpu)
+    assert torch.equal(dw2, dw) and torch.equal(dx2, dx)
+
+
 def test_conv2d_weight_gradient_of_512_filters_adds_its_partial_sums_the_same_both_ways(pkg, gpu):
     """512 -> 512 on 14x14: the resident-tile weight gradient; its partial sums are added by the kernel that writes the
     nine taps of an output together when dW is 16-byte aligned, by the one that writes them tap by tap when it is
