@@ -1070,7 +1070,14 @@ bool conv_halo_wg_preferred(const ConvTileDesc &d) {
     // batch 256 207 / 223 (batch 8: 24.9 / 30.7); with 64 channels 64 -> 128 on 56x56 at batch 128 132 / 137, at
     // batch 16 equal, at batch 4 23.4 against 20.6: those only from 1600 units on.
     const bool wide_ok = Wp <= 32 || cmin >= 128 || units >= 1600;
-    return conv_halo_wg_fits(d, Hp, Wp) && wide_ok && units >= (cmin >= 256 ? 20 : 96);
+    // Where it starts to pay, in units of 128 positions (this route against the one chosen without it, in turns in one
+    // process): 512 -> 512 on 14x14 from 14 (batch 8: 35.5 against 39.8 us; batch 4, 7 units: 34.3 / 30.2); 256 -> 256
+    // from 20 (14x14 at batch 8, 14 units: 30.7 / 25.7); 128 channels on a side from 48 (128 -> 128 on 28x28 at batch
+    // 8, 52 units: 24.3 / 28.6; batch 4, 26 units: 21.5 / 15.0), from 28 with four and more tiles of the filter tensor
+    // (128 -> 256 on 14x14 at batch 16: 26.1 / 35.8).
+    const int tiles = (d.Cout / 128) * (d.Cin / 64);
+    const long long need = cmin >= 512 ? 14 : cmin >= 256 ? 20 : cmin >= 128 ? (tiles >= 4 ? 28 : 48) : 96;
+    return conv_halo_wg_fits(d, Hp, Wp) && wide_ok && units >= need;
 }
 // Channel-minor: the other route copies both tensors into padded form first (9 + 9 of 66 us on 128 -> 128 28x28 at
 // batch 128), so this one is taken from the same amount of work on whatever the row length.

@@ -30,7 +30,8 @@ TABLE = [
     (1, 128, 64, 64, 56, [(1, 1), (1, 1), (1, 1)]),    # channel-minor: all three steps on the caller's tensors in place
     (1, 128, 128, 128, 28, [(1, 1), (1, 1), (1, 1)]),
     (1, 128, 256, 256, 14, [(1, 1), (1, 1), (1, 1)]),
-    (0, 8, 128, 128, 28, [(0, 1), (0, 0), (0, 1)]),    # too few tiles for the persistent kernels
+    (0, 8, 128, 128, 28, [(0, 1), (1, 1), (0, 1)]),    # too few tiles for the persistent forward kernel; the weight
+                                                       # gradient's resident-tile kernel pays from 48 units of positions
     (1, 8, 128, 128, 28, [(0, 1), (0, 0), (0, 1)]),
 ]
 
