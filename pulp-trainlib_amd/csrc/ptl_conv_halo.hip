@@ -1084,7 +1084,11 @@ bool conv_halo_wg_preferred(const ConvTileDesc &d) {
 bool conv_halo_wg_hwc_preferred(const ConvTileDesc &d) {
     const long long units = ((long long)d.batch * (d.Hin + 1) * (d.Win + 1) + HWG_UNIT - 1) / HWG_UNIT;
     const int cmin = d.Cin < d.Cout ? d.Cin : d.Cout;
-    return units >= (cmin >= 256 ? 20 : 96);
+    // the same starting points as for the channel-major form, measured the same way: 512 -> 512 on 14x14 at batch 8
+    // 33.4 against 51.0 us, 128 -> 128 on 28x28 at batch 8 / 12 22.9 / 23.5 against 26.9 / 35.5 (batch 4: 18.3 / 14.5),
+    // 128 -> 256 on 14x14 at batch 16 24.8 / 26.6, 256 -> 256 on 14x14 at batch 8 (14 units) 27.8 / 23.6
+    const int tiles = ((d.Cout + 127) / 128) * (d.Cin / 64);
+    return units >= (cmin >= 512 ? 14 : cmin >= 256 ? 20 : cmin >= 128 ? (tiles >= 4 ? 28 : 48) : 96);
 }
 long long conv_halo_wg_margin() { return 2 * HWG_UNIT + 256; }
 long long conv_halo_wg_gradient_stride(const ConvTileDesc &d, int Hp, int Wp) {

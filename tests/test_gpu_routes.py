@@ -32,7 +32,7 @@ TABLE = [
     (1, 128, 256, 256, 14, [(1, 1), (1, 1), (1, 1)]),
     (0, 8, 128, 128, 28, [(0, 1), (1, 1), (0, 1)]),    # too few tiles for the persistent forward kernel; the weight
                                                        # gradient's resident-tile kernel pays from 48 units of positions
-    (1, 8, 128, 128, 28, [(0, 1), (0, 0), (0, 1)]),
+    (1, 8, 128, 128, 28, [(0, 1), (1, 1), (0, 1)]),
 ]
 
 
