@@ -1057,7 +1057,8 @@ bool conv_halo_wg_fits(const ConvTileDesc &d, int Hp, int Wp) {
 // 7x7 69 against 86 us (tap-sum GEMM); from 256 channels it wins from 20 units of positions on (512 -> 512 on 7x7 at
 // batch 32: 38 against 53 us; 256 -> 256 on 14x14 at batch 8, 16 units: 30 against 26 us for the resident output tile
 // kernel), with 128 channels only from about a hundred (128 -> 128 on 14x14 at batch 32: 28
-// against 25 us for the resident output tile kernel).  64 -> 128 on 56x56 (280 against 274 us) stays where it was.
+// against 25 us for the resident output tile kernel).  (Measured before the input tiles of consecutive units shared a
+// ring; the starting points below are from after.)
 bool conv_halo_wg_preferred(const ConvTileDesc &d) {
     int Hp, Wp;
     conv_padded_grid(d, &Hp, &Wp);
