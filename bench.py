@@ -650,8 +650,9 @@ def detail_table(pkg, lib, hp, to_dev, timed, check, torch, dev):
 
     # larger convolutions, fp16, batched (ResNet-18/50 style layers)
     # (the last three rows are a saturating sweep: the same kernels with enough tiles for several full rounds)
-    for (ns, Ci, Co, H) in ((256, 32, 64, 56), (128, 64, 64, 56), (128, 128, 128, 28), (128, 256, 256, 14),
-                            (512, 128, 128, 28), (256, 256, 256, 28), (256, 512, 512, 14)):
+    # (128 -> 128 on 56x56: rows 57 wide, whose gradients take the resident-tile kernels since their input tiles share a ring)
+    for (ns, Ci, Co, H) in ((256, 32, 64, 56), (128, 64, 64, 56), (64, 128, 128, 56), (128, 128, 128, 28),
+                            (128, 256, 256, 14), (512, 128, 128, 28), (256, 256, 256, 28), (256, 512, 512, 14)):
         K, dt = 3, "fp16"
         x = torch.rand(ns, Ci, H, H, device=dev).to(tdt[dt]) - 0.5
         w = torch.rand(Co, Ci, K, K, device=dev).to(tdt[dt]) - 0.5
