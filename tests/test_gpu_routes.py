@@ -22,6 +22,7 @@ TABLE = [
     (0, 128, 64, 64, 8, [(2, 1), (2, 1), (2, 1)]),     # ResNet-20 stage 3
     (0, 256, 32, 64, 56, [(2, 1), (0, 1), (1, 1)]),    # input gradient: 64 channels into 32-filter resident tiles
     (0, 128, 64, 64, 56, [(1, 1), (0, 1), (1, 1)]),    # 64 filters: the weight gradient's resident-tile kernel needs 128
+    (0, 64, 128, 128, 56, [(1, 1), (1, 1), (1, 1)]),   # rows 57 wide: four pieces of the input tile per unit of the weight gradient
     (0, 128, 128, 128, 28, [(1, 1), (1, 1), (1, 1)]),
     (0, 128, 256, 256, 14, [(1, 1), (1, 1), (1, 1)]),
     (0, 512, 128, 128, 28, [(1, 1), (1, 1), (1, 1)]),
