@@ -655,6 +655,13 @@ int conv_halo_bw(const ConvTileDesc &fwd, const ConvTileDesc &ig, const void *X,
         if (Hp != Hpi || Wp != Wpi || fwd.x_sy != fwd.Win || ig.x_sy != ig.Win) return -1;
         if (!conv_halo_fits(ig, Hp, Wp) || !conv_halo_wg_fits(fwd, Hp, Wp) || !conv_halo_wg_preferred(fwd)) return -1;
         if (!(st.gemm_path == 0 || st.gemm_path == 5)) return -1;
+        // The input gradient's persistent kernel needs enough tiles (256 positions x 128 filters): with fewer than
+        // about 40 the two single steps, whose input gradient then goes another way, are faster than the pair
+        // (in turns in one process, pair against two calls: 128 -> 128 on 28x28 at batch 8, 27 tiles, 40.4 / 36.8 us;
+        // 512 -> 512 on 14x14 at batch 8, 32 tiles, 91.5 / 73.7; 256 -> 256 on 32x32 at batch 4, 36 tiles, 55.0 / 46.5;
+        // 128 -> 128 on 28x28 at batch 12, 40 tiles, 41.1 / 44.9; 256 -> 256 on 14x14 at batch 24, 44 tiles, 57.9 / 62.6).
+        const long long ig_tiles = ((long long)ig.batch * Hp * Wp + 255) / 256 * ((ig.Cout + 127) / 128);
+        if (st.gemm_path == 0 && ig_tiles < 40) return -1;
         const long long P = (long long)fwd.batch * Hp * Wp;
         const int goff = ig.padU * Wp + ig.padL;  // where the weight gradient's view of the copy starts
         const long long gstride = conv_halo_wg_gradient_stride(fwd, Hp, Wp) + 128;
