@@ -60,3 +60,31 @@ def test_default_route_of_bench_shapes(pkg, gpu, row):
     cm = (lambda t: t.permute(0, 3, 1, 2)) if hwc else (lambda t: t)
     ref = torch.nn.functional.conv2d(cm(x[:n].float()), cm(w.float()), padding=1)
     assert float((cm(y[:n].float()) - ref).norm() / ref.norm()) <= 1e-3
+
+
+@pytest.mark.parametrize("case", [(8, 512, 512, 14, 0), (24, 256, 256, 14, 1), (8, 128, 128, 28, 0), (12, 128, 128, 28, 1)])
+def test_one_call_backward_takes_the_pair_only_with_tiles_enough(pkg, gpu, case):
+    """ptl_conv2d_fp16_bw_batched: weight and input gradient share the blocked copy of the output gradient between the
+    two resident-tile kernels only where the input gradient's persistent kernel has 40 tiles and more; below that the
+    call does the two single steps (the last of which, the input gradient, is then no resident-tile launch).  Same
+    bits as the two single calls either way."""
+    ns, Ci, Co, H, pair = case
+    g = torch.Generator(device="cpu").manual_seed(5)
+    x = (torch.rand(ns, Ci, H, H, generator=g) - 0.5).half().to(DEV)
+    w = ((torch.rand(Co, Ci, 3, 3, generator=g) - 0.5) * 0.2).half().to(DEV)
+    dy = (torch.rand(ns, Co, H, H, generator=g) - 0.5).half().to(DEV)
+    dx, dw = torch.zeros_like(x), torch.zeros_like(w)
+    a, keep = hp.conv2d_args(pkg, x, dx, w, dw, None, dy, Ci, H, H, Co, 3, 3, H, H, (1, 1, 1, 1), (1, 1))
+    gpu.ptl_set_gemm_path(0)
+    assert gpu.ptl_conv2d_fp16_bw_batched(ctypes.byref(a), ns) == 0, gpu.ptl_last_error().decode()
+    assert gpu.ptl_last_conv_resident() == pair
+    assert gpu.ptl_sync() == 0
+    dx2, dw2 = torch.zeros_like(x), torch.zeros_like(w)
+    b, keep2 = hp.conv2d_args(pkg, x, dx2, w, dw2, None, dy, Ci, H, H, Co, 3, 3, H, H, (1, 1, 1, 1), (1, 1))
+    assert gpu.ptl_conv2d_fp16_wg_batched(ctypes.byref(b), ns) == 0
+    assert gpu.ptl_conv2d_fp16_ig_batched(ctypes.byref(b), ns) == 0
+    assert gpu.ptl_sync() == 0
+    assert torch.equal(dw2, dw)
+    ref = torch.nn.grad.conv2d_input(x.shape, w.float(), dy.float(), padding=1)
+    for t in (dx, dx2):
+        assert float((t.float() - ref).norm() / ref.norm()) <= 2e-3
